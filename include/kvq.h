@@ -1,0 +1,213 @@
+/*
+ * kvq.h -- C ABI of the MI355X (gfx950) int8 KV-cache attention library.
+ *
+ * Conventions (all entry points):
+ *   - extern "C", plain pointers and sizes; every pointer is DEVICE memory
+ *     unless the comment says host.  The caller owns every buffer.
+ *   - work is enqueued on `stream` (a hipStream_t passed as void*; NULL is the
+ *     default stream) and the call returns without synchronising.
+ *   - return value: 0 on success, a negative errno-style code otherwise
+ *     (KVQ_EINVAL for rejected arguments, KVQ_EHIP for a HIP runtime error).
+ *     kvq_last_error() returns a thread-local, human-readable reason.
+ *   - no entry point allocates or frees device memory; scratch comes in as a
+ *     caller-provided workspace whose size the *_workspace_bytes() helpers give.
+ *   - stateless, thread-safe; strides are taken from the caller, never assumed.
+ *
+ * Each declaration cites the interface of MetaX-MACA/vLLM-metax it stands in
+ * for (file:line relative to that tree).
+ */
+#ifndef KVQ_H_
+#define KVQ_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define KVQ_ABI_VERSION 1
+
+#define KVQ_OK 0
+#define KVQ_EINVAL (-22)
+#define KVQ_EHIP (-5)
+#define KVQ_ENOSYS (-38)
+
+/* element types of activations (query / key / value / output) */
+#define KVQ_F32 0
+#define KVQ_BF16 1
+#define KVQ_F16 2
+
+typedef void* kvq_stream_t;
+
+#if defined(__GNUC__)
+#define KVQ_API __attribute__((visibility("default")))
+#else
+#define KVQ_API
+#endif
+
+/*
+ * Byte geometry of the paged int8 cache with inline per-(token, head) scales.
+ * One (block, slot, head) record is [K codes (head_size) | K scale fp32 |
+ * V codes (head_size) | V scale fp32]; the four offsets locate those pieces
+ * relative to the cache base for block 0 / slot 0 / head 0, the three strides
+ * step to the next block / slot / head.  This is exactly the information the
+ * reference's typed views carry: key_cache / value_cache =
+ * kv_cache.transpose(1, 2).split(D + 4, -1) and the fp32 as_strided scale views
+ * (vllm_metax/v1/attention/backends/triton_attn.py:418-479, 729-739), for either
+ * physical order returned by get_kv_cache_stride_order (:350-372).
+ */
+typedef struct kvq_cache_geom {
+  int64_t k_off, v_off, ks_off, vs_off;           /* bytes */
+  int64_t stride_block, stride_slot, stride_head; /* bytes */
+  int32_t num_kv_heads, head_size, block_size;
+  int32_t reserved;
+} kvq_cache_geom;
+
+/* Byte geometry of the int8 MLA latent cache: per block, block_size code rows
+ * of (kv_lora_rank + rope_dim) bytes followed by block_size fp32 scales. */
+typedef struct kvq_mla_geom {
+  int64_t stride_block, stride_row, scale_off; /* bytes */
+  int32_t kv_lora_rank, rope_dim, block_size;
+  int32_t reserved;
+} kvq_mla_geom;
+
+KVQ_API int kvq_abi_version(void);
+KVQ_API const char* kvq_last_error(void);
+
+/* Number of compute units of the current device (host query, cached). */
+KVQ_API int kvq_device_num_cus(void);
+
+/*
+ * Quantise-on-write of new K/V tokens into the paged cache.
+ * Stands in for triton_reshape_and_cache_flash_per_token_head_quant(key, value,
+ * key_cache, value_cache, k_scale_cache, v_scale_cache, slot_mapping,
+ * kv_quant_mode=INT8_PER_TOKEN_HEAD), called at
+ * vllm_metax/v1/attention/backends/triton_attn.py:805-814; native sibling op
+ * reshape_and_cache_flash, csrc/libtorch_stable/torch_bindings.cpp:834-840 and
+ * cache_kernels.cu:309-395, 828-897.
+ *
+ * key/value: [>= num_tokens, num_kv_heads, head_size] of `src_dtype`, strides in
+ * elements (last dim contiguous).  num_tokens is slot_mapping's length (key may
+ * be longer: padding).  Tokens with slot < 0 are skipped.  Per (token, head):
+ * amax = max|x| floored at `eps`, scale = amax / 127, code =
+ * clamp(rint(x / scale), -128, 127); codes and scale are bit-exact.
+ */
+KVQ_API int kvq_reshape_and_cache_int8(const void* key, const void* value, int src_dtype,
+                               int64_t key_stride_t, int64_t key_stride_h,
+                               int64_t value_stride_t, int64_t value_stride_h, void* cache,
+                               const kvq_cache_geom* geom, const int64_t* slot_mapping,
+                               int64_t num_tokens, float eps, kvq_stream_t stream);
+
+/*
+ * Workspace for kvq_paged_attn_int8: split-K partial states.  Depends on the
+ * device (number of resident workgroups), so it is a host query; the value is
+ * an upper bound for any batch of at most max_num_seqs sequences.
+ * Counterpart of the reference's pre-sized split-softmax scratch,
+ * vllm_metax/v1/attention/backends/triton_attn.py:155-176.
+ */
+KVQ_API size_t kvq_paged_attn_workspace_bytes(int max_num_seqs, int num_q_heads, int head_size);
+
+/*
+ * Varlen paged attention over the int8 cache: decode rows and chunked-prefill
+ * rows in one call.  Stands in for unified_attention(q, k=key_cache,
+ * v=value_cache, out, cu_seqlens_q, max_seqlen_q, seqused_k, max_seqlen_k,
+ * softmax_scale, causal, ..., block_table, ..., kv_quant_mode, k_scale_cache,
+ * v_scale_cache) at vllm_metax/v1/attention/backends/triton_attn.py:688-725.
+ *
+ * q / out: [num_tokens, num_q_heads, head_size], strides in elements.
+ * Sequence i owns rows cu_seqlens_q[i] .. cu_seqlens_q[i+1]-1 and attends keys
+ * 0 .. seq_lens[i]-1 (bottom-right causal when `causal`), gathered through
+ * block_table[i * bt_stride + pos / block_size].  K = code * k_scale,
+ * V = code * v_scale, softmax in fp32.  max_query_len (host) selects the tiles:
+ * rows of single-token sequences go to the bandwidth-bound split-K tile, longer
+ * query runs to the MFMA prefill tile.  lse (optional, [num_tokens, num_q_heads]
+ * fp32, natural log) may be NULL.
+ */
+KVQ_API int kvq_paged_attn_int8(void* out, int out_dtype, int64_t out_stride_t, int64_t out_stride_h,
+                        const void* q, int q_dtype, int64_t q_stride_t, int64_t q_stride_h,
+                        const void* cache, const kvq_cache_geom* geom,
+                        const int32_t* block_table, int64_t bt_stride, const int32_t* seq_lens,
+                        const int32_t* cu_seqlens_q, int num_seqs, int num_q_heads,
+                        int max_query_len, float scale, int causal, float* lse,
+                        void* workspace, size_t workspace_bytes, kvq_stream_t stream);
+
+/*
+ * Fixed-partition split-K decode + reduce (one query row per sequence).
+ * Stands in for paged_attention_v2(out, exp_sums, max_logits, tmp_out, query,
+ * key_cache, value_cache, num_kv_heads, scale, block_tables, seq_lens,
+ * block_size, max_seq_len, ...), csrc/libtorch_stable/torch_bindings.cpp:631-641,
+ * paged_attention_v2.cu:44-135: partition j of `partition_size` tokens stores a
+ * locally normalised tmp_out[b, h, j, :], max_logits[b, h, j] and
+ * exp_sums[b, h, j] (all fp32 here); the reduce then writes out.
+ * max_num_partitions = ceil(max_seq_len / partition_size).
+ */
+KVQ_API int kvq_paged_attn_v2_int8(void* out, int out_dtype, float* exp_sums, float* max_logits,
+                           float* tmp_out, const void* q, int q_dtype, int64_t q_stride_t,
+                           int64_t q_stride_h, const void* cache, const kvq_cache_geom* geom,
+                           const int32_t* block_table, int64_t bt_stride,
+                           const int32_t* seq_lens, int num_seqs, int num_q_heads, float scale,
+                           int partition_size, int max_num_partitions, kvq_stream_t stream);
+
+/*
+ * The reduce stage on its own.  Stands in for paged_attention_v2_reduce_kernel,
+ * csrc/libtorch_stable/attention/attention_kernels.cuh:556-661 (and the Triton
+ * stage 2, vllm_metax/v1/attention/ops/triton_decode_attention.py:582-646):
+ * w_j = exp_sums_j * exp(max_logits_j - max), out = sum_j w_j tmp_out_j / sum_j w_j;
+ * a single partition is copied through.  lse (optional) = max + log(sum_j w_j).
+ */
+KVQ_API int kvq_splitk_reduce(void* out, int out_dtype, float* lse, const float* exp_sums,
+                      const float* max_logits, const float* tmp_out, const int32_t* seq_lens,
+                      int num_seqs, int num_q_heads, int head_size, int partition_size,
+                      int max_num_partitions, kvq_stream_t stream);
+
+/*
+ * LSE merge of two partial attention states.  Stands in for merge_attn_states,
+ * csrc/libtorch_stable/attention/merge_attn_states.cu:17-192, 246-320 (python
+ * chooser vllm_metax/v1/attention/ops/merge_attn_states.py:82-114).
+ * outputs [num_tokens, num_heads, head_size] of `dtype` (contiguous);
+ * lse tensors [num_heads, num_tokens] fp32; output_lse may be NULL.  +inf LSE is
+ * read as -inf; both -inf emits the prefix.  Rows >= prefix_num_tokens copy the
+ * suffix.
+ */
+KVQ_API int kvq_merge_attn_states(void* output, float* output_lse, const void* prefix_output,
+                          const float* prefix_lse, const void* suffix_output,
+                          const float* suffix_lse, int dtype, int64_t num_tokens, int num_heads,
+                          int head_size, int64_t prefix_num_tokens, kvq_stream_t stream);
+
+/*
+ * MLA latent quantise-on-write.  Stands in for concat_and_cache_mla(kv_c, k_pe,
+ * kv_cache, slot_mapping, kv_cache_dtype, scale),
+ * csrc/libtorch_stable/torch_bindings.cpp:843-848, cache_kernels.cu:397-439,
+ * 924-985, with the int8 per-token-scale entry this build defines (the
+ * reference has none; nearest precedents cache_kernels.cu:441-542, 593-604).
+ * kv_c [T, kv_lora_rank], k_pe [T, rope_dim] of `src_dtype` (row strides in
+ * elements); one absmax over the whole concatenated row.
+ */
+KVQ_API int kvq_concat_and_cache_mla_int8(const void* kv_c, const void* k_pe, int src_dtype,
+                                  int64_t kv_c_stride, int64_t k_pe_stride, void* cache,
+                                  const kvq_mla_geom* geom, const int64_t* slot_mapping,
+                                  int64_t num_tokens, float eps, kvq_stream_t stream);
+
+KVQ_API size_t kvq_mla_decode_workspace_bytes(int max_num_seqs, int num_heads, int kv_lora_rank);
+
+/*
+ * MLA decode over the int8 latent cache.  Stands in for
+ * TritonMLAImpl.forward_mqa -> decode_attention_fwd(q, k_buffer, v_buffer, o,
+ * lse, block_table, seq_lens, attn_logits, num_kv_splits, sm_scale, page_size,
+ * ..., is_mla=True), vllm_metax/v1/attention/backends/mla/triton_mla.py:226-295,
+ * vllm_metax/v1/attention/ops/triton_decode_attention.py:763-825.
+ * q [B, H, kv_lora_rank + rope_dim] (absorbed), out [B, H, kv_lora_rank],
+ * lse [B, H] fp32 natural log (may be NULL).
+ */
+KVQ_API int kvq_mla_decode_int8(void* out, int out_dtype, float* lse, const void* q, int q_dtype,
+                        int64_t q_stride_b, int64_t q_stride_h, const void* cache,
+                        const kvq_mla_geom* geom, const int32_t* block_table,
+                        int64_t bt_stride, const int32_t* seq_lens, int num_seqs,
+                        int num_heads, float scale, void* workspace, size_t workspace_bytes,
+                        kvq_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* KVQ_H_ */

@@ -1,0 +1,311 @@
+"""CPU oracle for the int8 KV-cache attention path.  TEST INFRASTRUCTURE ONLY.
+
+Only ``tests/``, ``__graft_entry__.smoke()`` and the ``cpu_baseline`` leg of
+``bench.py`` may import this package; the product (``vllm_metax_amd``) never
+does.  It wraps ``kvq_oracle.c`` (a plain-C restatement of the reference
+algorithm, every function citing the reference file:line it follows) through
+ctypes, and takes CPU torch tensors purely as typed memory.
+
+``torch_ref.py`` next to this file restates the reference's tests/kernels
+torch ops in their as-written numeric form; it is what the CPU baseline times
+and what the C oracle is cross-checked against.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+import subprocess
+from dataclasses import dataclass
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "libkvq_oracle.so")
+_lib = None
+
+
+def build(force: bool = False) -> str:
+    """Compile kvq_oracle.c with gcc (a second or two)."""
+    if force and os.path.exists(_LIB_PATH):
+        os.remove(_LIB_PATH)
+    subprocess.run(["make", "-s", "-C", _HERE, "libkvq_oracle.so"], check=True)
+    return _LIB_PATH
+
+
+def lib() -> ctypes.CDLL:
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            build()
+        _lib = ctypes.CDLL(_LIB_PATH)
+        for name in (
+            "kvq_oracle_quant_rows",
+            "kvq_oracle_cache_write",
+            "kvq_oracle_paged_attn",
+            "kvq_oracle_paged_attn_partition",
+            "kvq_oracle_splitk_reduce",
+            "kvq_oracle_merge_attn_states",
+            "kvq_oracle_mla_cache_write",
+            "kvq_oracle_mla_decode",
+            "kvq_oracle_num_threads",
+        ):
+            getattr(_lib, name).restype = ctypes.c_int
+    return _lib
+
+
+def num_threads() -> int:
+    return int(lib().kvq_oracle_num_threads())
+
+
+@dataclass(frozen=True)
+class RecordLayout:
+    """Byte geometry of the paged cache: where the K codes, V codes and the two
+    fp32 scales of a (block, slot, head) record sit relative to the storage base."""
+
+    k_off: int
+    v_off: int
+    ks_off: int
+    vs_off: int
+    stride_block: int
+    stride_slot: int
+    stride_head: int
+    head_size: int
+    block_size: int
+    num_kv_heads: int
+
+    @staticmethod
+    def from_views(kv_cache, key_cache, value_cache, k_scale_cache, v_scale_cache):
+        """Derive the geometry from the typed views alone (data_ptr differences
+        and strides), independent of how the views were constructed.
+
+        key_cache/value_cache: (num_blocks, block_size, Hkv, D + 4) int8 views;
+        scale caches: (num_blocks, block_size, Hkv) fp32 views."""
+        base = kv_cache.data_ptr()
+        nb, bs, hkv, padded = key_cache.shape
+        assert key_cache.element_size() == 1 and k_scale_cache.dtype == torch.float32
+        sb, ss, sh, se = key_cache.stride()
+        assert se == 1
+        assert tuple(4 * s for s in k_scale_cache.stride()) == (sb, ss, sh)
+        assert tuple(4 * s for s in v_scale_cache.stride()) == (sb, ss, sh)
+        assert value_cache.stride() == key_cache.stride()
+        return RecordLayout(
+            k_off=key_cache.data_ptr() - base,
+            v_off=value_cache.data_ptr() - base,
+            ks_off=k_scale_cache.data_ptr() - base,
+            vs_off=v_scale_cache.data_ptr() - base,
+            stride_block=sb,
+            stride_slot=ss,
+            stride_head=sh,
+            head_size=padded - 4,
+            block_size=bs,
+            num_kv_heads=hkv,
+        )
+
+
+def _p(t):
+    return ctypes.c_void_p(t.data_ptr()) if t is not None else ctypes.c_void_p(0)
+
+
+def _f32c(t):
+    assert t.device.type == "cpu"
+    return t.detach().to(torch.float32).contiguous()
+
+
+def _i32c(t):
+    return t.detach().to("cpu", torch.int32).contiguous()
+
+
+def _i64(v):
+    return ctypes.c_int64(int(v))
+
+
+def _check(rc, name):
+    if rc != 0:
+        raise RuntimeError(f"{name} failed with status {rc}")
+
+
+def eps_for(dtype: torch.dtype, eps: float = 1e-10) -> float:
+    """The absmax floor as the reference's op sees it: ``clamp(min=eps)`` is applied
+    in the SOURCE dtype before the cast to fp32 (tests/kernels/quant_utils.py:212-213)."""
+    return float(torch.tensor(eps, dtype=torch.float64).to(dtype).to(torch.float32))
+
+
+def quant_rows(x: torch.Tensor, eps: float | None = None):
+    """x [..., D] (fp32/bf16/fp16, CPU) -> (codes int8 [..., D], scales fp32 [...])."""
+    if eps is None:
+        eps = eps_for(x.dtype)
+    xf = _f32c(x)
+    D = xf.shape[-1]
+    rows = xf.numel() // D
+    codes = torch.empty(xf.shape, dtype=torch.int8)
+    scales = torch.empty(xf.shape[:-1], dtype=torch.float32)
+    _check(
+        lib().kvq_oracle_quant_rows(_p(xf), _i64(rows), _i64(D), ctypes.c_float(eps), _p(codes), _p(scales)),
+        "kvq_oracle_quant_rows",
+    )
+    return codes, scales
+
+
+def cache_write(key, value, kv_cache, lay: RecordLayout, slot_mapping, eps: float | None = None):
+    """Quantise key/value [T', Hkv, D] into kv_cache (CPU int8 storage) in place."""
+    if eps is None:
+        eps = eps_for(key.dtype)
+    kf, vf = _f32c(key), _f32c(value)
+    sm = slot_mapping.detach().to("cpu", torch.int64).contiguous()
+    T = sm.shape[0]
+    assert kf.shape[0] >= T and kf.shape[1] == lay.num_kv_heads and kf.shape[2] == lay.head_size
+    _check(
+        lib().kvq_oracle_cache_write(
+            _p(kf), _p(vf), _p(kv_cache),
+            _i64(lay.k_off), _i64(lay.v_off), _i64(lay.ks_off), _i64(lay.vs_off),
+            _i64(lay.stride_block), _i64(lay.stride_slot), _i64(lay.stride_head),
+            _p(sm), _i64(T), ctypes.c_int(lay.num_kv_heads), ctypes.c_int(lay.head_size),
+            ctypes.c_int(lay.block_size), ctypes.c_float(eps),
+        ),
+        "kvq_oracle_cache_write",
+    )
+
+
+def paged_attn(q, kv_cache, lay: RecordLayout, block_table, seq_lens, cu_seqlens_q,
+               scale: float, causal: bool = True, return_lse: bool = False):
+    """q [N, Hq, D] -> out fp32 [N, Hq, D] (and lse fp32 [N, Hq])."""
+    qf = _f32c(q)
+    N, Hq, D = qf.shape
+    bt, sl, cu = _i32c(block_table), _i32c(seq_lens), _i32c(cu_seqlens_q)
+    B = sl.shape[0]
+    out = torch.empty((N, Hq, D), dtype=torch.float32)
+    lse = torch.empty((N, Hq), dtype=torch.float32) if return_lse else None
+    _check(
+        lib().kvq_oracle_paged_attn(
+            _p(out), _p(lse), _p(qf), _p(kv_cache),
+            _i64(lay.k_off), _i64(lay.v_off), _i64(lay.ks_off), _i64(lay.vs_off),
+            _i64(lay.stride_block), _i64(lay.stride_slot), _i64(lay.stride_head),
+            _p(bt), _i64(bt.stride(0)), _p(sl), _p(cu),
+            ctypes.c_int(B), ctypes.c_int(Hq), ctypes.c_int(lay.num_kv_heads), ctypes.c_int(D),
+            ctypes.c_int(lay.block_size), ctypes.c_float(scale), ctypes.c_int(1 if causal else 0),
+        ),
+        "kvq_oracle_paged_attn",
+    )
+    return (out, lse) if return_lse else out
+
+
+def paged_attn_partition(q, kv_cache, lay: RecordLayout, block_table, seq_lens, scale: float,
+                         partition_size: int, max_parts: int):
+    """Decode rows only.  Returns (tmp_out [B,Hq,P,D], max_logits [B,Hq,P], exp_sums [B,Hq,P])."""
+    qf = _f32c(q)
+    B, Hq, D = qf.shape
+    bt, sl = _i32c(block_table), _i32c(seq_lens)
+    tmp = torch.zeros((B, Hq, max_parts, D), dtype=torch.float32)
+    ml = torch.zeros((B, Hq, max_parts), dtype=torch.float32)
+    es = torch.zeros((B, Hq, max_parts), dtype=torch.float32)
+    _check(
+        lib().kvq_oracle_paged_attn_partition(
+            _p(tmp), _p(ml), _p(es), _p(qf), _p(kv_cache),
+            _i64(lay.k_off), _i64(lay.v_off), _i64(lay.ks_off), _i64(lay.vs_off),
+            _i64(lay.stride_block), _i64(lay.stride_slot), _i64(lay.stride_head),
+            _p(bt), _i64(bt.stride(0)), _p(sl),
+            ctypes.c_int(B), ctypes.c_int(Hq), ctypes.c_int(lay.num_kv_heads), ctypes.c_int(D),
+            ctypes.c_int(lay.block_size), ctypes.c_float(scale), ctypes.c_int(partition_size),
+            ctypes.c_int(max_parts),
+        ),
+        "kvq_oracle_paged_attn_partition",
+    )
+    return tmp, ml, es
+
+
+def splitk_reduce(tmp_out, max_logits, exp_sums, seq_lens, partition_size: int, return_lse: bool = False):
+    tmp, ml, es = _f32c(tmp_out), _f32c(max_logits), _f32c(exp_sums)
+    B, Hq, P, D = tmp.shape
+    sl = _i32c(seq_lens)
+    out = torch.empty((B, Hq, D), dtype=torch.float32)
+    lse = torch.empty((B, Hq), dtype=torch.float32) if return_lse else None
+    _check(
+        lib().kvq_oracle_splitk_reduce(
+            _p(out), _p(lse), _p(tmp), _p(ml), _p(es), _p(sl),
+            ctypes.c_int(B), ctypes.c_int(Hq), ctypes.c_int(D), ctypes.c_int(partition_size), ctypes.c_int(P),
+        ),
+        "kvq_oracle_splitk_reduce",
+    )
+    return (out, lse) if return_lse else out
+
+
+def merge_attn_states(prefix_output, prefix_lse, suffix_output, suffix_lse, prefix_num_tokens=None):
+    """outputs [T, H, D]; lse [H, T].  Returns (output fp32, output_lse fp32)."""
+    po, so = _f32c(prefix_output), _f32c(suffix_output)
+    pl, sl = _f32c(prefix_lse), _f32c(suffix_lse)
+    T, H, D = po.shape
+    if prefix_num_tokens is None:
+        prefix_num_tokens = T
+    out = torch.empty((T, H, D), dtype=torch.float32)
+    lse = torch.empty((H, T), dtype=torch.float32)
+    _check(
+        lib().kvq_oracle_merge_attn_states(
+            _p(out), _p(lse), _p(po), _p(pl), _p(so), _p(sl),
+            _i64(T), ctypes.c_int(H), ctypes.c_int(D), _i64(prefix_num_tokens),
+        ),
+        "kvq_oracle_merge_attn_states",
+    )
+    return out, lse
+
+
+@dataclass(frozen=True)
+class MlaLayout:
+    """Byte geometry of the int8 latent cache: code rows and the per-token fp32
+    scale region of a block."""
+
+    stride_block: int
+    stride_row: int
+    scale_off: int
+    block_size: int
+    kv_lora_rank: int
+    rope_dim: int
+
+    @staticmethod
+    def from_views(cache, codes_view, scales_view, kv_lora_rank):
+        base = cache.data_ptr()
+        nb, bs, W = codes_view.shape
+        assert codes_view.data_ptr() == base and codes_view.stride(2) == 1
+        assert scales_view.stride(1) == 1 and 4 * scales_view.stride(0) == codes_view.stride(0)
+        return MlaLayout(
+            stride_block=codes_view.stride(0),
+            stride_row=codes_view.stride(1),
+            scale_off=scales_view.data_ptr() - base,
+            block_size=bs,
+            kv_lora_rank=kv_lora_rank,
+            rope_dim=W - kv_lora_rank,
+        )
+
+
+def mla_cache_write(kv_c, k_pe, cache, lay: MlaLayout, slot_mapping, eps: float | None = None):
+    if eps is None:
+        eps = eps_for(kv_c.dtype)
+    a, b = _f32c(kv_c), _f32c(k_pe)
+    sm = slot_mapping.detach().to("cpu", torch.int64).contiguous()
+    _check(
+        lib().kvq_oracle_mla_cache_write(
+            _p(a), _p(b), _p(cache), _i64(lay.stride_block), _i64(lay.stride_row), _i64(lay.scale_off),
+            _p(sm), _i64(sm.shape[0]), ctypes.c_int(lay.kv_lora_rank), ctypes.c_int(lay.rope_dim),
+            ctypes.c_int(lay.block_size), ctypes.c_float(eps),
+        ),
+        "kvq_oracle_mla_cache_write",
+    )
+
+
+def mla_decode(q, cache, lay: MlaLayout, block_table, seq_lens, scale: float):
+    """q [B, H, R+P] -> (out fp32 [B, H, R], lse fp32 [B, H])."""
+    qf = _f32c(q)
+    B, H, W = qf.shape
+    assert W == lay.kv_lora_rank + lay.rope_dim
+    bt, sl = _i32c(block_table), _i32c(seq_lens)
+    out = torch.empty((B, H, lay.kv_lora_rank), dtype=torch.float32)
+    lse = torch.empty((B, H), dtype=torch.float32)
+    _check(
+        lib().kvq_oracle_mla_decode(
+            _p(out), _p(lse), _p(qf), _p(cache), _i64(lay.stride_block), _i64(lay.stride_row),
+            _i64(lay.scale_off), _p(bt), _i64(bt.stride(0)), _p(sl),
+            ctypes.c_int(B), ctypes.c_int(H), ctypes.c_int(lay.kv_lora_rank), ctypes.c_int(lay.rope_dim),
+            ctypes.c_int(lay.block_size), ctypes.c_float(scale),
+        ),
+        "kvq_oracle_mla_decode",
+    )
+    return out, lse

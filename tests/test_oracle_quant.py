@@ -1,0 +1,116 @@
+"""Pins the oracle's quantiser (oracle/kvq_oracle.c: kvq_oracle_quant_rows) against things it did
+not come from: torch's CPU round/div (a library routine), closed forms, tie cases and an exact
+rational-arithmetic brute force."""
+from fractions import Fraction
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from oracle import torch_ref
+
+
+def _rand(shape, dtype, seed, kind):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(shape, generator=g, dtype=torch.float32)
+    if kind == "outlier":
+        x[..., ::37] *= 20.0
+    elif kind == "tiny":
+        x *= 1e-12
+    elif kind == "huge":
+        x *= 1e20
+    return x.to(dtype)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("kind", ["normal", "outlier", "tiny", "huge"])
+@pytest.mark.parametrize("d", [64, 128, 576])
+def test_matches_torch_cpu_op_bit_exact(dtype, kind, d):
+    if dtype == torch.float16 and kind == "huge":
+        pytest.skip("overflows fp16")
+    x = _rand((257, 3, d), dtype, 1234 + d, kind)
+    codes, scales = oracle.quant_rows(x)
+    ref_codes, ref_scales = torch_ref.per_token_head_quant_int8(x, d)
+    assert torch.equal(scales, ref_scales.reshape(scales.shape))
+    assert torch.equal(codes, ref_codes)
+
+
+def test_zero_rows_use_floor_in_source_dtype():
+    for dtype in (torch.float32, torch.bfloat16, torch.float16):
+        x = torch.zeros((4, 128), dtype=dtype)
+        codes, scales = oracle.quant_rows(x)
+        ref_codes, ref_scales = torch_ref.per_token_head_quant_int8(x, 128)
+        assert torch.equal(codes, torch.zeros_like(codes)) and torch.equal(codes, ref_codes)
+        assert torch.equal(scales, ref_scales.reshape(-1))
+        # eps = 1e-10 underflows to 0 in fp16: scale 0, codes defined as 0 (the as-written op divides 0/0)
+        assert (scales > 0).all() or dtype == torch.float16
+
+
+def test_closed_forms():
+    x = _rand((1000, 128), torch.float32, 7, "outlier")
+    codes, scales = oracle.quant_rows(x)
+    c = codes.to(torch.int32)
+    assert c.abs().max() <= 127                      # absmax maps to +-127, nothing beyond
+    idx = x.abs().argmax(dim=-1)
+    top = c[torch.arange(x.shape[0]), idx]
+    assert torch.equal(top.abs(), torch.full_like(top, 127))
+    assert torch.equal(torch.sign(top).float(), torch.sign(x[torch.arange(x.shape[0]), idx]))
+    err = (c.double() * scales.double()[:, None] - x.double()).abs()
+    assert (err <= 0.5 * scales.double()[:, None] * (1 + 1e-6)).all()   # half a step at most
+    assert torch.equal(scales, x.abs().amax(dim=-1) / 127.0)
+
+
+def test_ties_round_half_to_even():
+    # absmax 127 -> scale exactly 1.0, so x / scale = x and k + 0.5 is a true tie
+    row = torch.tensor([127.0, 0.5, 1.5, 2.5, 3.5, -0.5, -1.5, -2.5, 126.5, -126.5, 125.5] + [0.0] * 117)
+    codes, scales = oracle.quant_rows(row[None])
+    assert scales.item() == 1.0
+    assert codes[0, :11].tolist() == [127, 0, 2, 2, 4, 0, -2, -2, 126, -126, 126]
+    # bf16 source with an exactly representable tie
+    rowb = torch.tensor([254.0, 1.0, 3.0, 5.0, -7.0] + [0.0] * 123, dtype=torch.bfloat16)  # scale 2.0
+    codes, scales = oracle.quant_rows(rowb[None])
+    assert scales.item() == 2.0 and codes[0, :5].tolist() == [127, 0, 2, 2, -4]
+
+
+def test_negative_extreme_is_minus_127_not_minus_128():
+    row = torch.zeros(128)
+    row[5] = -3.0
+    row[9] = 1.0
+    codes, _ = oracle.quant_rows(row[None])
+    assert codes[0, 5].item() == -127 and codes.min().item() == -127
+
+
+def _f32(fr: Fraction) -> np.float32:
+    """Correctly rounded (nearest-even) float32 of an exact rational, via Python's float:
+    double rounding cannot bite here because inputs are float32 and one double division
+    of two float32-exact values is itself exact to 53 bits, well past float32's 24."""
+    return np.float32(float(fr))
+
+
+def test_bruteforce_exact_rational():
+    g = torch.Generator().manual_seed(99)
+    x = torch.randn((64, 16), generator=g)
+    codes, scales = oracle.quant_rows(x)
+    for r in range(x.shape[0]):
+        vals = [Fraction(float(v)) for v in x[r]]
+        amax = max(abs(v) for v in vals)
+        scale32 = _f32(amax / 127)
+        # float32(amax/127): numerator and denominator are float32-exact, so the double quotient
+        # rounds correctly to float32 unless it sits on a float32 rounding boundary of the double
+        assert np.float32(scales[r].item()) == scale32
+        sfr = Fraction(float(scale32))
+        for j, v in enumerate(vals):
+            q32 = Fraction(float(_f32(v / sfr)))           # fp32 quotient, then round half even
+            fl = q32.__floor__()
+            frac = q32 - fl
+            if frac > Fraction(1, 2) or (frac == Fraction(1, 2) and fl % 2 == 1):
+                fl += 1
+            assert codes[r, j].item() == max(-128, min(127, fl))
+
+
+def test_within_one_code_of_reciprocal_formulation():
+    x = _rand((512, 128), torch.bfloat16, 5, "normal")
+    codes, _ = oracle.quant_rows(x)
+    alt, _ = torch_ref.dynamic_per_token_quant_int8_reciprocal(x)
+    assert (codes.int() - alt.int()).abs().max() <= 1

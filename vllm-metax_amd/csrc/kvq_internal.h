@@ -1,0 +1,73 @@
+// Shared host/device helpers of the gfx950 int8 KV-cache kernels.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "kvq.h"
+
+namespace kvq {
+
+// ---- host side -------------------------------------------------------------
+int fail(int code, const char* fmt, ...);  // records kvq_last_error(), returns code
+int check_hip(hipError_t e, const char* what);
+int num_cus();
+inline hipStream_t as_stream(kvq_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
+
+#define KVQ_REQUIRE(cond, ...)                      \
+  do {                                              \
+    if (!(cond)) return ::kvq::fail(KVQ_EINVAL, __VA_ARGS__); \
+  } while (0)
+
+// ---- device side -----------------------------------------------------------
+typedef _Float16 half_t;
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+// The cache records are only 4-byte aligned (a record is 2*(D+4) bytes), so wide
+// loads from them carry an explicit 4-byte alignment.
+typedef uint32_t u32x2_a4 __attribute__((ext_vector_type(2), aligned(4)));
+typedef uint32_t u32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));
+
+constexpr int kWave = 64;
+
+__device__ __forceinline__ float bf16_bits_to_f32(uint16_t b) {
+  return __builtin_bit_cast(float, (uint32_t)b << 16);
+}
+
+// fp32 -> bf16, round to nearest even (NaN kept quiet).
+__device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
+  uint32_t u = __builtin_bit_cast(uint32_t, f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40u);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (uint16_t)(u >> 16);
+}
+
+template <int DT>
+__device__ __forceinline__ float load_act(const void* p, int64_t i) {
+  if constexpr (DT == KVQ_F32) return reinterpret_cast<const float*>(p)[i];
+  if constexpr (DT == KVQ_BF16) return bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(p)[i]);
+  return (float)reinterpret_cast<const half_t*>(p)[i];
+}
+
+template <int DT>
+__device__ __forceinline__ void store_act(void* p, int64_t i, float v) {
+  if constexpr (DT == KVQ_F32) reinterpret_cast<float*>(p)[i] = v;
+  else if constexpr (DT == KVQ_BF16) reinterpret_cast<uint16_t*>(p)[i] = f32_to_bf16_bits(v);
+  else reinterpret_cast<half_t*>(p)[i] = (half_t)v;
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = 32; o >= 1; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, kWave));
+  return v;
+}
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o >= 1; o >>= 1) v += __shfl_xor(v, o, kWave);
+  return v;
+}
+
+}  // namespace kvq

@@ -1,0 +1,82 @@
+// kvq_paged_attn_int8: the varlen entry point (decode rows + chunked-prefill rows).
+//
+// The host never looks at device data: max_query_len (a host integer the caller's
+// metadata already carries) decides which tiles are launched, and each kernel skips
+// the sequences that are not its kind by reading cu_seqlens_q on the device.
+#include "kvq_attn_core.cuh"
+
+namespace kvq {
+
+
+int launch_decode_streamk(const StreamKArgs& a, int q_dtype, int out_dtype, hipStream_t s);
+size_t streamk_workspace_bytes(int max_num_seqs, int num_q_heads, int head_size, int num_wg);
+int decode_streamk_num_wg(int num_kv_heads);
+int launch_prefill(const AttnIO& io, const int32_t* seq_lens, const int32_t* cu_seqlens_q, int num_seqs,
+                   int max_query_len, int causal, int q_dtype, int out_dtype, hipStream_t s);
+
+}  // namespace kvq
+
+extern "C" int kvq_paged_attn_int8(void* out, int out_dtype, int64_t out_stride_t, int64_t out_stride_h,
+                                   const void* q, int q_dtype, int64_t q_stride_t, int64_t q_stride_h,
+                                   const void* cache, const kvq_cache_geom* geom, const int32_t* block_table,
+                                   int64_t bt_stride, const int32_t* seq_lens, const int32_t* cu_seqlens_q,
+                                   int num_seqs, int num_q_heads, int max_query_len, float scale, int causal,
+                                   float* lse, void* workspace, size_t workspace_bytes, kvq_stream_t stream) {
+  using namespace kvq;
+  const char* op = "paged_attn_int8";
+  KVQ_REQUIRE(geom != nullptr, "%s: geom is NULL", op);
+  KVQ_REQUIRE(out && q && cache && block_table && seq_lens, "%s: NULL pointer", op);
+  KVQ_REQUIRE(num_seqs > 0 && num_q_heads > 0, "%s: num_seqs and num_q_heads must be positive", op);
+  KVQ_REQUIRE(max_query_len >= 1, "%s: max_query_len must be >= 1", op);
+  KVQ_REQUIRE(max_query_len == 1 || cu_seqlens_q != nullptr, "%s: cu_seqlens_q is required when max_query_len > 1", op);
+  const kvq_cache_geom& g = *geom;
+  KVQ_REQUIRE(g.num_kv_heads > 0 && num_q_heads % g.num_kv_heads == 0,
+              "%s: num_q_heads %d is not a multiple of num_kv_heads %d", op, num_q_heads, g.num_kv_heads);
+  KVQ_REQUIRE(num_q_heads / g.num_kv_heads <= 16, "%s: more than 16 q heads per kv head is not supported", op);
+  KVQ_REQUIRE(g.head_size == 64 || g.head_size == 128 || g.head_size == 256,
+              "%s: head_size %d not supported (64, 128, 256)", op, g.head_size);
+  KVQ_REQUIRE(g.block_size > 0 && g.block_size % 16 == 0, "%s: block_size %d must be a multiple of 16", op,
+              g.block_size);
+  KVQ_REQUIRE((g.k_off | g.v_off | g.ks_off | g.vs_off | g.stride_block | g.stride_slot | g.stride_head) % 4 == 0 &&
+                  ((uintptr_t)cache % 4) == 0,
+              "%s: cache offsets/strides must be 4-byte aligned", op);
+  const int osz = out_dtype == KVQ_F32 ? 4 : 2;
+  KVQ_REQUIRE(((uintptr_t)out % 4) == 0 && (out_stride_t * osz) % 4 == 0 && (out_stride_h * osz) % 4 == 0,
+              "%s: out rows must be 4-byte aligned", op);
+  const int num_wg = decode_streamk_num_wg(g.num_kv_heads);
+  KVQ_REQUIRE(num_wg > 0, "%s: no HIP device", op);
+  const size_t need = streamk_workspace_bytes(num_seqs, num_q_heads, g.head_size, num_wg);
+  KVQ_REQUIRE(workspace != nullptr && workspace_bytes >= need && ((uintptr_t)workspace % 16) == 0,
+              "%s: workspace of %zu bytes (16-byte aligned) required, got %zu", op, need, workspace_bytes);
+
+  StreamKArgs a{};
+  a.io.q = q;
+  a.io.q_stride_t = q_stride_t;
+  a.io.q_stride_h = q_stride_h;
+  a.io.out = out;
+  a.io.out_stride_t = out_stride_t;
+  a.io.out_stride_h = out_stride_h;
+  a.io.lse = lse;
+  a.io.cache = static_cast<const uint8_t*>(cache);
+  a.io.g = g;
+  a.io.block_table = block_table;
+  a.io.bt_stride = bt_stride;
+  a.io.num_q_heads = num_q_heads;
+  a.io.group = num_q_heads / g.num_kv_heads;
+  a.io.scale_log2 = scale * kLog2e;
+  a.seq_lens = seq_lens;
+  a.cu_seqlens_q = cu_seqlens_q;
+  a.num_seqs = num_seqs;
+  a.num_wg = num_wg;
+  const size_t slots = (size_t)num_wg + (size_t)num_seqs;
+  a.part_o = static_cast<float*>(workspace);
+  a.part_ml = a.part_o + slots * (size_t)num_q_heads * (size_t)g.head_size;
+
+  hipStream_t s = as_stream(stream);
+  int rc = launch_decode_streamk(a, q_dtype, out_dtype, s);
+  if (rc) return rc;
+  if (max_query_len > 1) {
+    rc = launch_prefill(a.io, seq_lens, cu_seqlens_q, num_seqs, max_query_len, causal, q_dtype, out_dtype, s);
+  }
+  return rc;
+}

@@ -1,0 +1,139 @@
+// Quantise-on-write of new K/V tokens into the paged int8 cache (gfx950).
+//
+// One wavefront owns one (token, kv head, K-or-V) row: the row is read once with
+// coalesced loads, the absmax is reduced across the 64 lanes, and codes plus the
+// fp32 scale go straight into the (block, slot, head) record.  The arithmetic is
+// the bit-exact contract: scale = max(absmax, eps) / 127 (IEEE fp32 division),
+// code = clamp(rint(x / scale), -128, 127) with round-half-to-even.
+#include "kvq_internal.h"
+
+namespace kvq {
+
+template <int DT, int VEC>  // VEC = head_size / 64 when that is 1, 2 or 4; 0 = any head size
+__global__ __launch_bounds__(256) void quant_write_kernel(
+    const void* __restrict__ key, const void* __restrict__ value, int64_t key_stride_t,
+    int64_t key_stride_h, int64_t value_stride_t, int64_t value_stride_h,
+    uint8_t* __restrict__ cache, kvq_cache_geom g, const int64_t* __restrict__ slot_mapping,
+    int64_t num_rows /* T * Hkv * 2 */, float eps) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int64_t row = (int64_t)blockIdx.x * (blockDim.x / kWave) + (threadIdx.x / kWave);
+  if (row >= num_rows) return;
+  const int is_v = (int)(row & 1);
+  const int64_t th = row >> 1;
+  const int h = (int)(th % g.num_kv_heads);
+  const int64_t t = th / g.num_kv_heads;
+  const int64_t slot = slot_mapping[t];
+  if (slot < 0) return;  // padding token
+  const int64_t blk = slot / g.block_size;
+  const int64_t off = slot - blk * g.block_size;
+  const int D = g.head_size;
+
+  const void* src = is_v ? value : key;
+  const int64_t src_base = is_v ? (t * value_stride_t + h * value_stride_h)
+                                : (t * key_stride_t + h * key_stride_h);
+  uint8_t* rec = cache + blk * g.stride_block + off * g.stride_slot + (int64_t)h * g.stride_head;
+  int8_t* codes = reinterpret_cast<int8_t*>(rec + (is_v ? g.v_off : g.k_off));
+  float* scale_ptr = reinterpret_cast<float*>(rec + (is_v ? g.vs_off : g.ks_off));
+
+  if constexpr (VEC > 0) {
+    float x[VEC];
+    float amax = 0.f;
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) {
+      x[i] = load_act<DT>(src, src_base + lane * VEC + i);
+      amax = fmaxf(amax, fabsf(x[i]));
+    }
+    amax = fmaxf(wave_max(amax), eps);  // eps may be 0 for fp16 sources (1e-10 underflows)
+    const float scale = amax / 127.0f;
+    int8_t c[VEC];
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) {
+      float r = scale > 0.f ? rintf(x[i] / scale) : 0.f;  // scale == 0: all-zero fp16 row
+      r = fminf(fmaxf(r, -128.f), 127.f);
+      c[i] = (int8_t)(int)r;
+    }
+    if constexpr (VEC == 1) {
+      codes[lane] = c[0];
+    } else if constexpr (VEC == 2) {
+      uint16_t pk = (uint16_t)(uint8_t)c[0] | ((uint16_t)(uint8_t)c[1] << 8);
+      reinterpret_cast<uint16_t*>(codes)[lane] = pk;  // records are 4-byte aligned
+    } else {
+      uint32_t pk = (uint32_t)(uint8_t)c[0] | ((uint32_t)(uint8_t)c[1] << 8) |
+                    ((uint32_t)(uint8_t)c[2] << 16) | ((uint32_t)(uint8_t)c[3] << 24);
+      reinterpret_cast<uint32_t*>(codes)[lane] = pk;
+    }
+    if (lane == 0) *scale_ptr = scale;
+  } else {
+    float amax = 0.f;
+    for (int d = lane; d < D; d += kWave) amax = fmaxf(amax, fabsf(load_act<DT>(src, src_base + d)));
+    amax = fmaxf(wave_max(amax), eps);  // eps may be 0 for fp16 sources (1e-10 underflows)
+    const float scale = amax / 127.0f;
+    for (int d = lane; d < D; d += kWave) {
+      float r = scale > 0.f ? rintf(load_act<DT>(src, src_base + d) / scale) : 0.f;
+      r = fminf(fmaxf(r, -128.f), 127.f);
+      codes[d] = (int8_t)(int)r;
+    }
+    if (lane == 0) *scale_ptr = scale;
+  }
+}
+
+template <int DT>
+static int launch_quant_write(const void* key, const void* value, int64_t kst, int64_t ksh,
+                              int64_t vst, int64_t vsh, uint8_t* cache, const kvq_cache_geom& g,
+                              const int64_t* slot_mapping, int64_t T, float eps, hipStream_t s) {
+  const int64_t rows = T * g.num_kv_heads * 2;
+  const int64_t blocks = (rows + 3) / 4;
+  if (blocks > 0x7fffffffLL) return fail(KVQ_EINVAL, "reshape_and_cache_int8: too many tokens");
+  dim3 grid((unsigned)blocks), block(256);
+#define KVQ_LAUNCH(V)                                                                     \
+  hipLaunchKernelGGL((quant_write_kernel<DT, V>), grid, block, 0, s, key, value, kst, ksh, \
+                     vst, vsh, cache, g, slot_mapping, rows, eps)
+  switch (g.head_size) {
+    case 64: KVQ_LAUNCH(1); break;
+    case 128: KVQ_LAUNCH(2); break;
+    case 256: KVQ_LAUNCH(4); break;
+    default: KVQ_LAUNCH(0); break;
+  }
+#undef KVQ_LAUNCH
+  return check_hip(hipGetLastError(), "reshape_and_cache_int8 launch");
+}
+
+}  // namespace kvq
+
+extern "C" int kvq_reshape_and_cache_int8(const void* key, const void* value, int src_dtype,
+                                          int64_t key_stride_t, int64_t key_stride_h,
+                                          int64_t value_stride_t, int64_t value_stride_h,
+                                          void* cache, const kvq_cache_geom* geom,
+                                          const int64_t* slot_mapping, int64_t num_tokens,
+                                          float eps, kvq_stream_t stream) {
+  using namespace kvq;
+  KVQ_REQUIRE(geom != nullptr, "reshape_and_cache_int8: geom is NULL");
+  KVQ_REQUIRE(num_tokens >= 0, "reshape_and_cache_int8: negative num_tokens");
+  if (num_tokens == 0) return KVQ_OK;
+  KVQ_REQUIRE(key && value && cache && slot_mapping, "reshape_and_cache_int8: NULL pointer");
+  const kvq_cache_geom& g = *geom;
+  KVQ_REQUIRE(g.num_kv_heads > 0 && g.head_size > 0 && g.block_size > 0,
+              "reshape_and_cache_int8: bad geometry (heads=%d head_size=%d block_size=%d)",
+              g.num_kv_heads, g.head_size, g.block_size);
+  KVQ_REQUIRE(g.head_size % 4 == 0, "reshape_and_cache_int8: head_size %d must be a multiple of 4",
+              g.head_size);
+  KVQ_REQUIRE((g.k_off | g.v_off | g.ks_off | g.vs_off | g.stride_block | g.stride_slot |
+               g.stride_head) % 4 == 0 && ((uintptr_t)cache % 4) == 0,
+              "reshape_and_cache_int8: cache offsets/strides must be 4-byte aligned");
+  KVQ_REQUIRE(eps >= 0.f, "reshape_and_cache_int8: eps must not be negative");
+  hipStream_t s = as_stream(stream);
+  uint8_t* c = static_cast<uint8_t*>(cache);
+  switch (src_dtype) {
+    case KVQ_F32:
+      return launch_quant_write<KVQ_F32>(key, value, key_stride_t, key_stride_h, value_stride_t,
+                                         value_stride_h, c, g, slot_mapping, num_tokens, eps, s);
+    case KVQ_BF16:
+      return launch_quant_write<KVQ_BF16>(key, value, key_stride_t, key_stride_h, value_stride_t,
+                                          value_stride_h, c, g, slot_mapping, num_tokens, eps, s);
+    case KVQ_F16:
+      return launch_quant_write<KVQ_F16>(key, value, key_stride_t, key_stride_h, value_stride_t,
+                                         value_stride_h, c, g, slot_mapping, num_tokens, eps, s);
+    default:
+      return fail(KVQ_EINVAL, "reshape_and_cache_int8: unknown src_dtype %d", src_dtype);
+  }
+}

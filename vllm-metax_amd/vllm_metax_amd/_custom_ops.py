@@ -1,0 +1,381 @@
+"""Python op layer: thin functions that validate torch tensors and call the C ABI.
+
+Same convention as the reference's op layer (vllm_metax/_custom_ops.py:5-17,
+137-166: a python function per op that forwards to the native library): ops return
+``None``, mutate their output arguments in place, take strides from the tensors,
+run on the current torch stream, and raise ``RuntimeError`` on bad arguments
+(csrc/libtorch_stable/cache_kernels.cu:884-889).  torch is only the owner of device
+memory and of the stream here; all arithmetic happens in libkvq_hip.so.
+"""
+from __future__ import annotations
+
+import ctypes
+
+import torch
+
+from . import _C
+from .kv_cache_interface import KVQuantMode
+from .layout import QUANT_EPS, CacheGeometry, MlaGeometry, geometry_from_views, mla_geometry
+
+_DTYPE_CODE = {torch.float32: _C.KVQ_F32, torch.bfloat16: _C.KVQ_BF16, torch.float16: _C.KVQ_F16}
+
+
+def _dtype_code(t: torch.Tensor, what: str) -> int:
+    try:
+        return _DTYPE_CODE[t.dtype]
+    except KeyError:
+        raise RuntimeError(f"{what}: unsupported dtype {t.dtype}") from None
+
+
+def _require_cuda(*tensors: torch.Tensor) -> torch.device:
+    dev = None
+    for t in tensors:
+        if t is None:
+            continue
+        if not t.is_cuda:
+            raise RuntimeError("int8 KV-cache ops need GPU tensors (there is no CPU path)")
+        if dev is None:
+            dev = t.device
+        elif t.device != dev:
+            raise RuntimeError(f"tensors on different devices: {dev} vs {t.device}")
+    return dev
+
+
+def _stream(dev: torch.device) -> ctypes.c_void_p:
+    return ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+
+
+def _ptr(t) -> ctypes.c_void_p:
+    return ctypes.c_void_p(t.data_ptr() if t is not None else 0)
+
+
+def eps_for_dtype(dtype: torch.dtype) -> float:
+    """absmax floor as the reference's quantiser applies it: ``clamp(min=1e-10)`` in the
+    SOURCE dtype, before the cast to fp32 (tests/kernels/quant_utils.py:212-213)."""
+    return float(torch.tensor(QUANT_EPS, dtype=torch.float64).to(dtype).to(torch.float32))
+
+
+def device_num_cus() -> int:
+    return int(_C.load().kvq_device_num_cus())
+
+
+# ---------------------------------------------------------------------------------------------
+# quantise-on-write
+# ---------------------------------------------------------------------------------------------
+
+def reshape_and_cache_flash_per_token_head_quant(
+    key: torch.Tensor,
+    value: torch.Tensor,
+    key_cache: torch.Tensor,
+    value_cache: torch.Tensor,
+    k_scale_cache: torch.Tensor,
+    v_scale_cache: torch.Tensor,
+    slot_mapping: torch.Tensor,
+    kv_quant_mode: KVQuantMode = KVQuantMode.INT8_PER_TOKEN_HEAD,
+    geometry: CacheGeometry | None = None,
+) -> None:
+    """Drop-in for ``triton_reshape_and_cache_flash_per_token_head_quant`` as called at
+    vllm_metax/v1/attention/backends/triton_attn.py:805-814.
+
+    key/value ``[>= T, Hkv, D]``; key_cache/value_cache ``(nb, bs, Hkv, D+4)`` int8 views and
+    k/v_scale_cache ``(nb, bs, Hkv)`` fp32 views of one cache; slot_mapping ``[T]`` int64
+    (negative = padding, skipped).  ``geometry`` may carry the precomputed byte geometry of
+    the four views so the per-step call does no view arithmetic."""
+    if kv_quant_mode != KVQuantMode.INT8_PER_TOKEN_HEAD:
+        raise NotImplementedError(f"kv_quant_mode {kv_quant_mode!r}: only INT8_PER_TOKEN_HEAD is built")
+    dev = _require_cuda(key, value, key_cache, value_cache, k_scale_cache, v_scale_cache, slot_mapping)
+    geom = geometry or geometry_from_views(key_cache, value_cache, k_scale_cache, v_scale_cache)
+    if key.dim() != 3 or value.shape != key.shape or key.dtype != value.dtype:
+        raise RuntimeError("key/value must be [num_tokens, num_kv_heads, head_size] of one dtype")
+    if key.shape[1] != geom.num_kv_heads or key.shape[2] != geom.head_size:
+        raise RuntimeError(f"key shape {tuple(key.shape)} does not match cache (Hkv={geom.num_kv_heads}, D={geom.head_size})")
+    if key.stride(2) != 1 or value.stride(2) != 1:
+        raise RuntimeError("key/value head dim must be contiguous")
+    if slot_mapping.dtype != torch.int64 or slot_mapping.dim() != 1 or not slot_mapping.is_contiguous():
+        raise RuntimeError("slot_mapping must be a contiguous 1-D int64 tensor")
+    num_tokens = slot_mapping.shape[0]
+    if num_tokens > key.shape[0]:
+        raise RuntimeError("slot_mapping is longer than key")
+    lib = _C.load()
+    g = geom.as_struct()
+    with torch.cuda.device(dev):
+        rc = lib.kvq_reshape_and_cache_int8(
+            _ptr(key), _ptr(value), _dtype_code(key, "key"), key.stride(0), key.stride(1), value.stride(0),
+            value.stride(1), ctypes.c_void_p(geom.base_ptr), ctypes.byref(g), _ptr(slot_mapping), num_tokens,
+            eps_for_dtype(key.dtype), _stream(dev))
+    _C.check(rc, "reshape_and_cache_flash_per_token_head_quant")
+
+
+# name used at the reference's call site
+triton_reshape_and_cache_flash_per_token_head_quant = reshape_and_cache_flash_per_token_head_quant
+
+
+# ---------------------------------------------------------------------------------------------
+# attention
+# ---------------------------------------------------------------------------------------------
+
+def paged_attn_workspace_bytes(max_num_seqs: int, num_q_heads: int, head_size: int) -> int:
+    return int(_C.load().kvq_paged_attn_workspace_bytes(max_num_seqs, num_q_heads, head_size))
+
+
+_ws_cache: dict = {}
+
+
+def _default_workspace(dev: torch.device, nbytes: int) -> torch.Tensor:
+    """Grow-only per-device scratch for callers that did not bring their own (tests, eager use).
+    The backend's metadata builder pre-sizes its own instead, so a captured step never lands here."""
+    cur = _ws_cache.get(dev)
+    if cur is None or cur.numel() < nbytes:
+        cur = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=dev)
+        _ws_cache[dev] = cur
+    return cur
+
+
+def unified_attention(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    out: torch.Tensor,
+    cu_seqlens_q: torch.Tensor,
+    max_seqlen_q: int,
+    seqused_k: torch.Tensor,
+    max_seqlen_k: int,
+    softmax_scale: float,
+    causal: bool,
+    window_size=(-1, -1),
+    block_table: torch.Tensor | None = None,
+    softcap: float = 0.0,
+    q_descale=None,
+    k_descale=None,
+    v_descale=None,
+    alibi_slopes=None,
+    use_alibi_sqrt: bool = False,
+    sinks=None,
+    output_scale=None,
+    mm_prefix_range=None,
+    kv_quant_mode: KVQuantMode = KVQuantMode.INT8_PER_TOKEN_HEAD,
+    k_scale_cache: torch.Tensor | None = None,
+    v_scale_cache: torch.Tensor | None = None,
+    workspace: torch.Tensor | None = None,
+    geometry: CacheGeometry | None = None,
+    lse: torch.Tensor | None = None,
+    **unused,
+) -> None:
+    """Drop-in for ``unified_attention`` as called at
+    vllm_metax/v1/attention/backends/triton_attn.py:688-725 with an int8 per-token-head cache.
+
+    q/out ``[N, Hq, D]``; k/v are the ``(nb, bs, Hkv, D+4)`` int8 cache views; ``seqused_k`` ``[B]``
+    int32 context lengths; ``cu_seqlens_q`` ``[B+1]`` int32; ``block_table`` ``[B, max_blocks]``
+    int32.  Extra keyword arguments of the reference's call that only steer its Triton launch
+    (``seq_threshold_3D``, ``softmax_segm_*``, ``use_td`` ...) are accepted and ignored; features
+    this path does not build raise ``NotImplementedError``."""
+    if kv_quant_mode != KVQuantMode.INT8_PER_TOKEN_HEAD:
+        raise NotImplementedError(f"kv_quant_mode {kv_quant_mode!r}: only INT8_PER_TOKEN_HEAD is built")
+    if alibi_slopes is not None or sinks is not None or output_scale is not None or mm_prefix_range is not None:
+        raise NotImplementedError("alibi, sinks, fused output quantisation and mm-prefix ranges are not built")
+    if softcap not in (0, 0.0, None):
+        raise NotImplementedError("logits soft cap is not built")
+    if tuple(window_size) != (-1, -1):
+        raise NotImplementedError("sliding window is not built")
+    if q_descale is not None:
+        raise NotImplementedError("quantised query input is not built")
+    if unused.get("rswa_window") is not None or unused.get("chunk_lookback", -1) not in (-1, None):
+        raise NotImplementedError("rswa / chunk_lookback are not built")
+    if block_table is None or k_scale_cache is None or v_scale_cache is None:
+        raise RuntimeError("block_table, k_scale_cache and v_scale_cache are required")
+    dev = _require_cuda(q, k, v, out, cu_seqlens_q, seqused_k, block_table, k_scale_cache, v_scale_cache, workspace, lse)
+    geom = geometry or geometry_from_views(k, v, k_scale_cache, v_scale_cache)
+    if q.dim() != 3 or out.shape != q.shape or q.shape[2] != geom.head_size:
+        raise RuntimeError("q/out must be [num_tokens, num_q_heads, head_size] matching the cache head size")
+    if q.stride(2) != 1 or out.stride(2) != 1:
+        raise RuntimeError("q/out head dim must be contiguous")
+    num_seqs = seqused_k.shape[0]
+    if seqused_k.dtype != torch.int32 or cu_seqlens_q.dtype != torch.int32 or block_table.dtype != torch.int32:
+        raise RuntimeError("seqused_k, cu_seqlens_q and block_table must be int32")
+    if cu_seqlens_q.shape[0] != num_seqs + 1 or block_table.shape[0] < num_seqs or block_table.stride(1) != 1:
+        raise RuntimeError("cu_seqlens_q must have num_seqs+1 entries and block_table num_seqs contiguous rows")
+    if not seqused_k.is_contiguous() or not cu_seqlens_q.is_contiguous():
+        raise RuntimeError("seqused_k and cu_seqlens_q must be contiguous")
+    if num_seqs == 0 or q.shape[0] == 0:
+        return
+    num_q_heads = q.shape[1]
+    lib = _C.load()
+    need = paged_attn_workspace_bytes(num_seqs, num_q_heads, geom.head_size)
+    if workspace is None:
+        workspace = _default_workspace(dev, need)
+    if lse is not None and (lse.dtype != torch.float32 or not lse.is_contiguous()
+                            or tuple(lse.shape) != (q.shape[0], num_q_heads)):
+        raise RuntimeError("lse must be a contiguous float32 [num_tokens, num_q_heads] tensor")
+    g = geom.as_struct()
+    with torch.cuda.device(dev):
+        rc = lib.kvq_paged_attn_int8(
+            _ptr(out), _dtype_code(out, "out"), out.stride(0), out.stride(1),
+            _ptr(q), _dtype_code(q, "q"), q.stride(0), q.stride(1),
+            ctypes.c_void_p(geom.base_ptr), ctypes.byref(g), _ptr(block_table), block_table.stride(0),
+            _ptr(seqused_k), _ptr(cu_seqlens_q), num_seqs, num_q_heads, int(max_seqlen_q),
+            float(softmax_scale), 1 if causal else 0, _ptr(lse), _ptr(workspace),
+            workspace.numel() * workspace.element_size(), _stream(dev))
+    _C.check(rc, "unified_attention")
+
+
+def paged_attention_v2(
+    out: torch.Tensor,
+    exp_sums: torch.Tensor,
+    max_logits: torch.Tensor,
+    tmp_out: torch.Tensor,
+    query: torch.Tensor,
+    key_cache: torch.Tensor,
+    value_cache: torch.Tensor,
+    num_kv_heads: int,
+    scale: float,
+    block_tables: torch.Tensor,
+    seq_lens: torch.Tensor,
+    block_size: int,
+    max_seq_len: int,
+    alibi_slopes=None,
+    kv_cache_dtype: str = "int8_per_token_head",
+    k_scale: torch.Tensor | None = None,
+    v_scale: torch.Tensor | None = None,
+    partition_size: int = 512,
+    **unused,
+) -> None:
+    """Fixed-partition split-K decode, argument order of ``paged_attention_v2``
+    (csrc/libtorch_stable/torch_bindings.cpp:631-641).  key_cache/value_cache are the int8 cache
+    views and k_scale/v_scale the per-(token, head) fp32 scale views; exp_sums / max_logits
+    ``[B, Hq, P]`` and tmp_out ``[B, Hq, P, D]`` are fp32, P = ceil(max_seq_len / partition_size)."""
+    if kv_cache_dtype != "int8_per_token_head":
+        raise NotImplementedError(f"kv_cache_dtype {kv_cache_dtype!r}: only int8_per_token_head is built")
+    if alibi_slopes is not None:
+        raise NotImplementedError("alibi is not built")
+    if k_scale is None or v_scale is None:
+        raise RuntimeError("k_scale / v_scale (the per-token-head scale views) are required")
+    dev = _require_cuda(out, exp_sums, max_logits, tmp_out, query, key_cache, value_cache, block_tables, seq_lens, k_scale, v_scale)
+    geom = geometry_from_views(key_cache, value_cache, k_scale, v_scale)
+    if geom.num_kv_heads != num_kv_heads or geom.block_size != block_size:
+        raise RuntimeError("num_kv_heads / block_size do not match the cache views")
+    B, Hq, D = query.shape
+    P = (max_seq_len + partition_size - 1) // partition_size
+    for t, shape, name in ((exp_sums, (B, Hq, P), "exp_sums"), (max_logits, (B, Hq, P), "max_logits"),
+                           (tmp_out, (B, Hq, P, D), "tmp_out")):
+        if t.dtype != torch.float32 or tuple(t.shape) != shape or not t.is_contiguous():
+            raise RuntimeError(f"{name} must be a contiguous float32 tensor of shape {shape}")
+    if tuple(out.shape) != (B, Hq, D) or not out.is_contiguous() or query.stride(2) != 1:
+        raise RuntimeError("out must be contiguous [B, Hq, D]; query head dim contiguous")
+    if seq_lens.dtype != torch.int32 or block_tables.dtype != torch.int32 or block_tables.stride(1) != 1:
+        raise RuntimeError("seq_lens and block_tables must be int32 (rows contiguous)")
+    g = geom.as_struct()
+    with torch.cuda.device(dev):
+        rc = _C.load().kvq_paged_attn_v2_int8(
+            _ptr(out), _dtype_code(out, "out"), _ptr(exp_sums), _ptr(max_logits), _ptr(tmp_out), _ptr(query),
+            _dtype_code(query, "query"), query.stride(0), query.stride(1), ctypes.c_void_p(geom.base_ptr),
+            ctypes.byref(g), _ptr(block_tables), block_tables.stride(0), _ptr(seq_lens), B, Hq, float(scale),
+            int(partition_size), int(P), _stream(dev))
+    _C.check(rc, "paged_attention_v2")
+
+
+def splitk_reduce(out: torch.Tensor, exp_sums: torch.Tensor, max_logits: torch.Tensor, tmp_out: torch.Tensor,
+                  seq_lens: torch.Tensor, partition_size: int = 512, lse: torch.Tensor | None = None) -> None:
+    """The reduce stage alone (csrc/libtorch_stable/attention/attention_kernels.cuh:556-661)."""
+    dev = _require_cuda(out, exp_sums, max_logits, tmp_out, seq_lens, lse)
+    B, Hq, P, D = tmp_out.shape
+    for t, name in ((exp_sums, "exp_sums"), (max_logits, "max_logits"), (tmp_out, "tmp_out")):
+        if t.dtype != torch.float32 or not t.is_contiguous():
+            raise RuntimeError(f"{name} must be contiguous float32")
+    if tuple(out.shape) != (B, Hq, D) or not out.is_contiguous() or seq_lens.dtype != torch.int32:
+        raise RuntimeError("out must be contiguous [B, Hq, D] and seq_lens int32")
+    with torch.cuda.device(dev):
+        rc = _C.load().kvq_splitk_reduce(_ptr(out), _dtype_code(out, "out"), _ptr(lse), _ptr(exp_sums),
+                                         _ptr(max_logits), _ptr(tmp_out), _ptr(seq_lens), B, Hq, D,
+                                         int(partition_size), P, _stream(dev))
+    _C.check(rc, "splitk_reduce")
+
+
+def merge_attn_states(output: torch.Tensor, prefix_output: torch.Tensor, prefix_lse: torch.Tensor,
+                      suffix_output: torch.Tensor, suffix_lse: torch.Tensor,
+                      output_lse: torch.Tensor | None = None, prefill_tokens_with_context: int | None = None) -> None:
+    """LSE merge, signature of vllm_metax/v1/attention/ops/merge_attn_states.py:10-114.
+    outputs ``[T, H, D]`` (one dtype, contiguous), lse ``[H, T]`` fp32."""
+    dev = _require_cuda(output, prefix_output, prefix_lse, suffix_output, suffix_lse, output_lse)
+    T, H, D = output.shape
+    if prefix_output.shape != output.shape or suffix_output.shape != output.shape:
+        raise RuntimeError("prefix/suffix/output shapes differ")
+    if prefix_output.dtype != output.dtype or suffix_output.dtype != output.dtype:
+        raise RuntimeError("prefix/suffix/output dtypes differ")
+    for t in (output, prefix_output, suffix_output, prefix_lse, suffix_lse):
+        if not t.is_contiguous():
+            raise RuntimeError("merge_attn_states needs contiguous tensors")
+    if prefix_lse.dtype != torch.float32 or suffix_lse.dtype != torch.float32 or tuple(prefix_lse.shape) != (H, T):
+        raise RuntimeError("lse tensors must be float32 [num_heads, num_tokens]")
+    n_prefix = T if prefill_tokens_with_context is None else int(prefill_tokens_with_context)
+    with torch.cuda.device(dev):
+        rc = _C.load().kvq_merge_attn_states(_ptr(output), _ptr(output_lse), _ptr(prefix_output), _ptr(prefix_lse),
+                                             _ptr(suffix_output), _ptr(suffix_lse), _dtype_code(output, "output"),
+                                             T, H, D, n_prefix, _stream(dev))
+    _C.check(rc, "merge_attn_states")
+
+
+# ---------------------------------------------------------------------------------------------
+# MLA latent cache
+# ---------------------------------------------------------------------------------------------
+
+def concat_and_cache_mla(kv_c: torch.Tensor, k_pe: torch.Tensor, kv_cache: torch.Tensor,
+                         slot_mapping: torch.Tensor, kv_cache_dtype: str = "int8_per_token",
+                         scale: torch.Tensor | None = None, geometry: MlaGeometry | None = None) -> None:
+    """Argument order of ``concat_and_cache_mla`` (csrc/libtorch_stable/torch_bindings.cpp:843-848).
+    kv_c ``[T, R]``, k_pe ``[T, P]``; kv_cache is the int8 latent cache ``(nb, bs, R+P+4)``."""
+    if kv_cache_dtype != "int8_per_token":
+        raise NotImplementedError(f"kv_cache_dtype {kv_cache_dtype!r}: only int8_per_token is built")
+    dev = _require_cuda(kv_c, k_pe, kv_cache, slot_mapping)
+    geom = geometry or mla_geometry(kv_cache, kv_c.shape[-1])
+    if kv_c.dim() != 2 or k_pe.dim() != 2 or kv_c.dtype != k_pe.dtype:
+        raise RuntimeError("kv_c [T, R] and k_pe [T, P] must be 2-D of one dtype")
+    if kv_c.shape[1] != geom.kv_lora_rank or k_pe.shape[1] != geom.rope_dim:
+        raise RuntimeError("kv_c / k_pe widths do not match the cache entry")
+    if kv_c.stride(1) != 1 or k_pe.stride(1) != 1:
+        raise RuntimeError("kv_c / k_pe rows must be contiguous")
+    if slot_mapping.dtype != torch.int64 or not slot_mapping.is_contiguous():
+        raise RuntimeError("slot_mapping must be contiguous int64")
+    T = slot_mapping.shape[0]
+    if T > kv_c.shape[0] or T > k_pe.shape[0]:
+        raise RuntimeError("slot_mapping is longer than kv_c / k_pe")
+    g = geom.as_struct()
+    with torch.cuda.device(dev):
+        rc = _C.load().kvq_concat_and_cache_mla_int8(_ptr(kv_c), _ptr(k_pe), _dtype_code(kv_c, "kv_c"),
+                                                     kv_c.stride(0), k_pe.stride(0), ctypes.c_void_p(geom.base_ptr),
+                                                     ctypes.byref(g), _ptr(slot_mapping), T,
+                                                     eps_for_dtype(kv_c.dtype), _stream(dev))
+    _C.check(rc, "concat_and_cache_mla")
+
+
+def mla_decode_workspace_bytes(max_num_seqs: int, num_heads: int, kv_lora_rank: int) -> int:
+    return int(_C.load().kvq_mla_decode_workspace_bytes(max_num_seqs, num_heads, kv_lora_rank))
+
+
+def mla_decode_int8(q: torch.Tensor, kv_cache: torch.Tensor, o: torch.Tensor, lse: torch.Tensor | None,
+                    block_table: torch.Tensor, seq_lens: torch.Tensor, sm_scale: float, kv_lora_rank: int,
+                    workspace: torch.Tensor | None = None, geometry: MlaGeometry | None = None) -> None:
+    """MLA decode over the int8 latent cache: the job of ``decode_attention_fwd(..., is_mla=True)``
+    (vllm_metax/v1/attention/ops/triton_decode_attention.py:763-825).  q ``[B, H, R+P]``,
+    o ``[B, H, R]``, lse ``[B, H]`` fp32 or None."""
+    dev = _require_cuda(q, kv_cache, o, lse, block_table, seq_lens, workspace)
+    geom = geometry or mla_geometry(kv_cache, kv_lora_rank)
+    B, H, W = q.shape
+    if W != geom.kv_lora_rank + geom.rope_dim or tuple(o.shape) != (B, H, geom.kv_lora_rank):
+        raise RuntimeError("q must be [B, H, R+P] and o [B, H, R]")
+    if q.stride(2) != 1 or not o.is_contiguous():
+        raise RuntimeError("q head dim must be contiguous and o contiguous")
+    if seq_lens.dtype != torch.int32 or block_table.dtype != torch.int32 or block_table.stride(1) != 1:
+        raise RuntimeError("seq_lens and block_table must be int32")
+    if lse is not None and (lse.dtype != torch.float32 or tuple(lse.shape) != (B, H) or not lse.is_contiguous()):
+        raise RuntimeError("lse must be contiguous float32 [B, H]")
+    need = mla_decode_workspace_bytes(B, H, geom.kv_lora_rank)
+    if workspace is None:
+        workspace = _default_workspace(dev, need)
+    g = geom.as_struct()
+    with torch.cuda.device(dev):
+        rc = _C.load().kvq_mla_decode_int8(_ptr(o), _dtype_code(o, "o"), _ptr(lse), _ptr(q), _dtype_code(q, "q"),
+                                           q.stride(0), q.stride(1), ctypes.c_void_p(geom.base_ptr), ctypes.byref(g),
+                                           _ptr(block_table), block_table.stride(0), _ptr(seq_lens), B, H,
+                                           float(sm_scale), _ptr(workspace),
+                                           workspace.numel() * workspace.element_size(), _stream(dev))
+    _C.check(rc, "mla_decode_int8")
