@@ -1,0 +1,152 @@
+"""GPU parity of paged decode attention over the int8 cache (balanced split-K kernel + reduce and
+the fixed-partition entry point), through the C ABI, against the oracle: atol 2e-2 / rtol 1e-2 on
+bf16 outputs (the north-star tolerance), tighter on fp32 outputs."""
+import math
+
+import pytest
+import torch
+
+import kvq_testlib as T
+import oracle
+from vllm_metax_amd import _custom_ops as ops
+from vllm_metax_amd import layout as L
+
+pytestmark = pytest.mark.gpu
+
+
+def build_case(ctx_lens, hq, hkv, d, bs, layout, seed, num_blocks=None, poison=True, outlier=False,
+               q_std=1.0, q_dtype=torch.bfloat16):
+    g = torch.Generator().manual_seed(seed)
+    nb = num_blocks or (sum((c + bs - 1) // bs for c in ctx_lens) + 5)
+    kv, views, lay = T.cpu_cache(nb, bs, hkv, d, layout)
+    if poison:
+        T.storage_bytes(kv).fill_(0xFF)     # NaN scales / -1 codes wherever nothing is written
+    bt = T.make_block_tables(ctx_lens, bs, nb, g)
+    mk = (lambda c: T.outlier_sources((c, hkv, d), g, torch.bfloat16)) if outlier else \
+         (lambda c: torch.randn((c, hkv, d), generator=g).to(torch.bfloat16))
+    ks = [mk(c) for c in ctx_lens]
+    vs = [mk(c) for c in ctx_lens]
+    T.fill_cache_from_sources(kv, lay, bt, ctx_lens, bs, ks, vs)
+    q = (torch.randn((len(ctx_lens), hq, d), generator=g) * q_std).to(q_dtype)
+    sl = torch.tensor(ctx_lens, dtype=torch.int32)
+    cu = torch.arange(len(ctx_lens) + 1, dtype=torch.int32)
+    return kv, lay, bt, q, sl, cu
+
+
+def run_unified(dev, kv_cpu, layout, bt, q, sl, cu, scale, out_dtype=torch.bfloat16, want_lse=False):
+    kv = T.to_device_cache(kv_cpu, dev, layout)
+    k, v = L.key_value_views(kv)
+    ks, vs = L.scale_views(kv)
+    out = torch.full(q.shape, float("nan"), dtype=out_dtype, device=dev)
+    lse = torch.full(q.shape[:2], float("nan"), dtype=torch.float32, device=dev) if want_lse else None
+    ops.unified_attention(q.to(dev), k, v, out, cu.to(dev), 1, sl.to(dev), int(sl.max()), scale, True,
+                          block_table=bt.to(dev), k_scale_cache=ks, v_scale_cache=vs, lse=lse)
+    torch.cuda.synchronize()
+    return (out, lse) if want_lse else out
+
+
+@pytest.mark.parametrize("layout", ["NHD", "HND"])
+def test_config1_shape(gpu_device, layout):
+    """32 q heads / 8 kv heads, head 128, block 16, batch 4, ctx 512 each, 128-block pool."""
+    ctx = [512] * 4
+    kv, lay, bt, q, sl, cu = build_case(ctx, 32, 8, 128, 16, layout, 0, num_blocks=129)
+    scale = 1 / math.sqrt(128)
+    want, want_lse = oracle.paged_attn(q, T.storage_bytes(kv), lay, bt, sl, cu, scale, return_lse=True)
+    got, lse = run_unified(gpu_device, kv, layout, bt, q, sl, cu, scale, want_lse=True)
+    T.assert_close_attn(got, want, what="config 1")
+    torch.testing.assert_close(lse.cpu(), want_lse, atol=2e-3, rtol=1e-3)
+
+
+@pytest.mark.parametrize("ctx", [[1], [31, 32, 33], [15, 16, 17, 1, 2], [1000, 3, 517, 64, 4097], [700] * 70])
+def test_ragged_lengths_fp32_out(gpu_device, ctx):
+    """Ragged and tiny contexts, sequence boundaries falling inside workgroup ranges, more
+    sequences than one wave scans at once; fp32 output isolates kernel error from bf16 rounding."""
+    kv, lay, bt, q, sl, cu = build_case(ctx, 32, 8, 128, 16, "NHD", len(ctx))
+    scale = 1 / math.sqrt(128)
+    want = oracle.paged_attn(q, T.storage_bytes(kv), lay, bt, sl, cu, scale)
+    got = run_unified(gpu_device, kv, "NHD", bt, q, sl, cu, scale, out_dtype=torch.float32)
+    T.assert_close_attn(got, want, atol=2e-3, rtol=2e-3, what=f"ctx={ctx[:5]}")
+
+
+@pytest.mark.parametrize("hq,hkv,d,bs", [(28, 4, 128, 16), (8, 8, 128, 16), (16, 1, 128, 32), (8, 2, 64, 16),
+                                         (4, 2, 256, 16), (32, 16, 128, 64)])
+def test_head_and_block_shapes(gpu_device, hq, hkv, d, bs):
+    ctx = [200, 77, 1025, 48]
+    kv, lay, bt, q, sl, cu = build_case(ctx, hq, hkv, d, bs, "NHD", hq + d)
+    scale = d ** -0.5
+    want = oracle.paged_attn(q, T.storage_bytes(kv), lay, bt, sl, cu, scale)
+    got = run_unified(gpu_device, kv, "NHD", bt, q, sl, cu, scale)
+    T.assert_close_attn(got, want, what=f"hq={hq} hkv={hkv} d={d} bs={bs}")
+
+
+def test_outlier_heavy_sources_and_peaked_softmax(gpu_device):
+    """1 % of channels x20 (stresses the scales) and a large |q| (nearly one-hot softmax)."""
+    ctx = [3000, 513]
+    kv, lay, bt, q, sl, cu = build_case(ctx, 32, 8, 128, 16, "NHD", 9, outlier=True, q_std=3.0)
+    scale = 1 / math.sqrt(128)
+    want = oracle.paged_attn(q, T.storage_bytes(kv), lay, bt, sl, cu, scale)
+    got = run_unified(gpu_device, kv, "NHD", bt, q, sl, cu, scale)
+    T.assert_close_attn(got, want, what="outliers")
+
+
+def test_empty_sequence_and_untouched_padding_rows(gpu_device):
+    ctx = [40, 0, 9]
+    kv, lay, bt, q, sl, cu = build_case([40, 1, 9], 8, 2, 128, 16, "NHD", 10)
+    sl = torch.tensor(ctx, dtype=torch.int32)
+    scale = 0.1
+    want = oracle.paged_attn(q, T.storage_bytes(kv), lay, bt, sl, cu, scale)
+    got = run_unified(gpu_device, kv, "NHD", bt, q, sl, cu, scale)
+    assert (got[1] == 0).all()
+    T.assert_close_attn(got, want, what="empty sequence")
+
+
+def test_fixed_partitions_v2_contract(gpu_device):
+    """512-token partitions: tmp_out / max_logits / exp_sums per partition match the oracle's
+    stage 1, and the reduce matches unsplit attention."""
+    dev = gpu_device
+    ctx = [1500, 512, 513, 30, 2048]
+    hq, hkv, d, bs = 32, 8, 128, 16
+    kv_cpu, lay, bt, q, sl, cu = build_case(ctx, hq, hkv, d, bs, "NHD", 12)
+    scale = d ** -0.5
+    P = (max(ctx) + 511) // 512
+    kv = T.to_device_cache(kv_cpu, dev, "NHD")
+    k, v = L.key_value_views(kv)
+    ks, vs = L.scale_views(kv)
+    B = len(ctx)
+    out = torch.empty((B, hq, d), dtype=torch.bfloat16, device=dev)
+    es = torch.zeros((B, hq, P), dtype=torch.float32, device=dev)
+    ml = torch.zeros((B, hq, P), dtype=torch.float32, device=dev)
+    tmp = torch.zeros((B, hq, P, d), dtype=torch.float32, device=dev)
+    ops.paged_attention_v2(out, es, ml, tmp, q.to(dev), k, v, hkv, scale, bt.to(dev), sl.to(dev), bs, max(ctx),
+                           k_scale=ks, v_scale=vs)
+    torch.cuda.synchronize()
+    base = T.storage_bytes(kv_cpu)
+    wtmp, wml, wes = oracle.paged_attn_partition(q, base, lay, bt, sl, scale, 512, P)
+    for i, c in enumerate(ctx):
+        n = (c + 511) // 512
+        T.assert_close_attn(tmp[i, :, :n], wtmp[i, :, :n], atol=2e-3, rtol=2e-3, what="tmp_out")
+        torch.testing.assert_close(ml[i, :, :n].cpu(), wml[i, :, :n], atol=2e-3, rtol=1e-3)
+        torch.testing.assert_close(es[i, :, :n].cpu(), wes[i, :, :n], atol=1e-3, rtol=5e-3)
+    want = oracle.paged_attn(q, base, lay, bt, sl, cu, scale)
+    T.assert_close_attn(out, want, what="v2 reduce")
+    # the reduce entry point alone, on the oracle's stage-1 output, with lse
+    out2 = torch.empty((B, hq, d), dtype=torch.float32, device=dev)
+    lse = torch.empty((B, hq), dtype=torch.float32, device=dev)
+    ops.splitk_reduce(out2, wes.to(dev), wml.to(dev), wtmp.to(dev), sl.to(dev), 512, lse=lse)
+    w2, wl2 = oracle.splitk_reduce(wtmp, wml, wes, sl, 512, return_lse=True)
+    torch.testing.assert_close(out2.cpu(), w2, atol=1e-5, rtol=1e-4)
+    torch.testing.assert_close(lse.cpu(), wl2, atol=1e-4, rtol=1e-5)
+
+
+def test_block_permutation_invariance_on_device(gpu_device):
+    dev = gpu_device
+    ctx = [333, 1200]
+    kv_cpu, lay, bt, q, sl, cu = build_case(ctx, 32, 8, 128, 16, "NHD", 13, poison=False)
+    scale = 0.09
+    a = run_unified(dev, kv_cpu, "NHD", bt, q, sl, cu, scale, out_dtype=torch.float32)
+    nb = kv_cpu.shape[0]
+    perm = torch.randperm(nb, generator=torch.Generator().manual_seed(1))
+    kv2, _, _ = T.cpu_cache(nb, 16, 8, 128, "NHD")
+    T.storage_bytes(kv2).view(nb, -1)[perm] = T.storage_bytes(kv_cpu).view(nb, -1)
+    b = run_unified(dev, kv2, "NHD", perm[bt.long()].to(torch.int32), q, sl, cu, scale, out_dtype=torch.float32)
+    assert torch.equal(a, b)

@@ -57,7 +57,7 @@ def test_closed_forms():
     assert torch.equal(top.abs(), torch.full_like(top, 127))
     assert torch.equal(torch.sign(top).float(), torch.sign(x[torch.arange(x.shape[0]), idx]))
     err = (c.double() * scales.double()[:, None] - x.double()).abs()
-    assert (err <= 0.5 * scales.double()[:, None] * (1 + 1e-6)).all()   # half a step at most
+    assert (err <= 0.5 * scales.double()[:, None] * (1 + 1e-4)).all()   # half a step (+ fp32 rounding of x/scale)
     assert torch.equal(scales, x.abs().amax(dim=-1) / 127.0)
 
 

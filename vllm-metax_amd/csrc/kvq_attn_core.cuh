@@ -334,7 +334,7 @@ struct DecodeTile {
     if constexpr (ODT == KVQ_F32) {
       float* o = reinterpret_cast<float*>(io.out) + base;
 #pragma unroll
-      for (int i = 0; i < D / 4; i += 4) *reinterpret_cast<floatx4*>(o + i) = (floatx4){v[i], v[i + 1], v[i + 2], v[i + 3]};
+      for (int i = 0; i < D / 4; i += 4) *reinterpret_cast<floatx4_a4*>(o + i) = (floatx4){v[i], v[i + 1], v[i + 2], v[i + 3]};
     } else {
       uint16_t* o = reinterpret_cast<uint16_t*>(io.out) + base;
 #pragma unroll

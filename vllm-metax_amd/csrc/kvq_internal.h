@@ -30,6 +30,7 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 // loads from them carry an explicit 4-byte alignment.
 typedef uint32_t u32x2_a4 __attribute__((ext_vector_type(2), aligned(4)));
 typedef uint32_t u32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));
+typedef float floatx4_a4 __attribute__((ext_vector_type(4), aligned(4)));
 
 constexpr int kWave = 64;
 

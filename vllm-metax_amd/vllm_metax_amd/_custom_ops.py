@@ -196,6 +196,8 @@ def unified_attention(
         raise RuntimeError("cu_seqlens_q must have num_seqs+1 entries and block_table num_seqs contiguous rows")
     if not seqused_k.is_contiguous() or not cu_seqlens_q.is_contiguous():
         raise RuntimeError("seqused_k and cu_seqlens_q must be contiguous")
+    if block_table.shape[1] * geom.block_size < int(max_seqlen_k):
+        raise RuntimeError("block_table rows are too short for max_seqlen_k")
     if num_seqs == 0 or q.shape[0] == 0:
         return
     num_q_heads = q.shape[1]
