@@ -1,0 +1,243 @@
+#!/usr/bin/env python3
+"""Benchmark of the int8 KV-cache decode path on one MI355X.
+
+A "step" is one layer's worth of the hot path on one decode batch: quantise-on-write of the
+batch's new tokens into the paged int8 cache, then paged decode attention over the whole
+context.  Steps rotate over several layer caches (same block table, different cache tensor, as
+in a real model) so that a step's KV bytes come from HBM and not from what the previous step
+left in the last-level cache.  All inputs are resident in HBM before the timed region.
+
+Prints ONE JSON line (see the keys below).  `value` is the algorithmic HBM bytes of a step
+divided by the step time; `roofline` is the same for the decode attention launch alone, timed
+with events on the launch stream; `cpu_baseline` times the as-written torch restatement of the
+reference's tests/kernels ops on a bounded sample of the same batch on the host cores.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(ROOT, "vllm-metax_amd"))
+sys.path.insert(0, ROOT)
+
+import torch  # noqa: E402
+
+HBM_PEAK_GBPS = 8000.0
+METRIC = "int8-KV paged decode: achieved HBM GB/s (% peak), µs/layer @B=64 ctx=8k"
+
+
+def make_batch(workload: str, seed: int = 0):
+    """Context lengths and pool size of the named workload (BASELINE.json configs)."""
+    g = torch.Generator().manual_seed(seed)
+    if workload == "llama3_8b_decode_b64_ctx1k-8k":      # configs[1]
+        ctx = torch.randint(1024, 8193, (64,), generator=g).tolist()
+        return dict(hq=32, hkv=8, d=128, bs=16, ctx=ctx, pool=40000)
+    if workload == "llama3_8b_decode_b64_ctx8k_fixed":   # the headline's fixed-context variant
+        return dict(hq=32, hkv=8, d=128, bs=16, ctx=[8192] * 64, pool=40000)
+    if workload == "longctx_splitk_b8_32k-128k":         # configs[2]
+        ctx = torch.randint(32768, 131073, (8,), generator=g).tolist()
+        return dict(hq=32, hkv=8, d=128, bs=16, ctx=ctx, pool=66000)
+    if workload == "config1_b4_ctx512":                  # configs[0]
+        return dict(hq=32, hkv=8, d=128, bs=16, ctx=[512] * 4, pool=129)
+    raise SystemExit(f"unknown workload {workload}")
+
+
+def algorithmic_bytes(cfg, include_write=True):
+    """Bytes the decode step must move once: every context token's K+V codes and both scales for
+    all kv heads, Q and output rows, the block-table entries and seq_lens; plus, for the write,
+    the new tokens' bf16 K/V rows in and their int8 records out."""
+    hq, hkv, d, bs = cfg["hq"], cfg["hkv"], cfg["d"], cfg["bs"]
+    ctx = cfg["ctx"]
+    B = len(ctx)
+    attn = sum(ctx) * hkv * 2 * (d + 4) + 2 * B * hq * d * 2 + sum((c + bs - 1) // bs for c in ctx) * 4 + 4 * B
+    write = B * hkv * (2 * d * 2 + 2 * (d + 4)) if include_write else 0
+    return attn, write
+
+
+def build_device_state(cfg, dev, layers, seed=0, layout="NHD", permute=True):
+    from vllm_metax_amd import _custom_ops as ops
+    from vllm_metax_amd import layout as L
+
+    hq, hkv, d, bs, ctx, pool = cfg["hq"], cfg["hkv"], cfg["d"], cfg["bs"], cfg["ctx"], cfg["pool"]
+    B = len(ctx)
+    g = torch.Generator().manual_seed(seed)
+    need = [(c + bs - 1) // bs for c in ctx]
+    perm = torch.randperm(pool - 1, generator=g)[: sum(need)] + 1          # block 0 stays the null block
+    if not permute:
+        perm = torch.arange(sum(need)) + 1
+    bt = torch.zeros((B, max(need)), dtype=torch.int32)
+    o = 0
+    for i, n in enumerate(need):
+        bt[i, :n] = perm[o:o + n].to(torch.int32)
+        o += n
+    bt_d = bt.to(dev)
+    sl_d = torch.tensor(ctx, dtype=torch.int32, device=dev)
+    cu_d = torch.arange(B + 1, dtype=torch.int32, device=dev)
+    # slot of the newest token of every sequence (the one this step writes) and of all the others
+    last = torch.tensor([int(bt[i, (c - 1) // bs]) * bs + (c - 1) % bs for i, c in enumerate(ctx)], dtype=torch.int64)
+    caches = []
+    torch.manual_seed(seed)
+    for _ in range(layers):
+        kv = L.allocate_kv_cache(pool, bs, hkv, d, device=dev, layout=layout, fill=0)
+        k, v = L.key_value_views(kv)
+        ks, vs = L.scale_views(kv)
+        ks.fill_(1.0)
+        vs.fill_(1.0)
+        geom = L.geometry_from_views(k, v, ks, vs)
+        # fill the context with N(0,1) bf16 sources through the quantise-on-write kernel itself
+        for i, c in enumerate(ctx):
+            pos = torch.arange(c, device=dev)
+            slots = bt_d[i, pos // bs].to(torch.int64) * bs + pos % bs
+            for s0 in range(0, c, 32768):
+                n = min(32768, c - s0)
+                ksrc = torch.randn((n, hkv, d), device=dev, dtype=torch.float32).to(torch.bfloat16)
+                vsrc = torch.randn((n, hkv, d), device=dev, dtype=torch.float32).to(torch.bfloat16)
+                ops.reshape_and_cache_flash_per_token_head_quant(ksrc, vsrc, k, v, ks, vs, slots[s0:s0 + n], geometry=geom)
+        caches.append(dict(kv=kv, k=k, v=v, ks=ks, vs=vs, geom=geom))
+    q = torch.randn((B, hq, d), device=dev, dtype=torch.float32).to(torch.bfloat16)
+    new_k = torch.randn((B, hkv, d), device=dev, dtype=torch.float32).to(torch.bfloat16)
+    new_v = torch.randn((B, hkv, d), device=dev, dtype=torch.float32).to(torch.bfloat16)
+    out = torch.empty_like(q)
+    ws = torch.empty(ops.paged_attn_workspace_bytes(B, hq, d), dtype=torch.uint8, device=dev)
+    torch.cuda.synchronize()
+    return dict(bt=bt, bt_d=bt_d, sl_d=sl_d, cu_d=cu_d, slots_new=last.to(dev), caches=caches, q=q, new_k=new_k,
+                new_v=new_v, out=out, ws=ws, scale=1.0 / math.sqrt(d), max_ctx=max(ctx))
+
+
+def run_step(st, layer, ops, write=True, attn=True):
+    c = st["caches"][layer]
+    if write:
+        ops.reshape_and_cache_flash_per_token_head_quant(st["new_k"], st["new_v"], c["k"], c["v"], c["ks"], c["vs"],
+                                                         st["slots_new"], geometry=c["geom"])
+    if attn:
+        ops.unified_attention(st["q"], c["k"], c["v"], st["out"], st["cu_d"], 1, st["sl_d"], st["max_ctx"], st["scale"],
+                              True, block_table=st["bt_d"], k_scale_cache=c["ks"], v_scale_cache=c["vs"],
+                              workspace=st["ws"], geometry=c["geom"])
+
+
+def cpu_baseline(cfg, st, seconds_target=15.0):
+    """The reference's CPU path (as-written torch ops, bf16 Q.K / fp32 softmax / bf16 P.V) on a
+    bounded sample of the batch: dequantise the sampled sequences' blocks, then ref_paged_attn."""
+    from oracle import torch_ref
+
+    hq, hkv, d, bs, ctx = cfg["hq"], cfg["hkv"], cfg["d"], cfg["bs"], cfg["ctx"]
+    c0 = st["caches"][0]
+    order = sorted(range(len(ctx)), key=lambda i: ctx[i])
+    sample = [order[len(order) // 2]]                      # start with the median-length sequence
+    k_cpu_views = None
+    q_cpu = st["q"].cpu()
+    threads = torch.get_num_threads()
+    done_bytes, t_total, reps = 0, 0.0, 0
+    idx = 0
+    cand = [order[len(order) // 2]] + [i for i in order if i != order[len(order) // 2]]
+    while t_total < seconds_target and idx < len(cand):
+        i = cand[idx]
+        idx += 1
+        n = (ctx[i] + bs - 1) // bs
+        blocks = st["bt"][i, :n].long()
+        # gather this sequence's blocks to the host (not timed: the reference's cache would already live there)
+        kb = c0["k"][blocks.to(c0["k"].device)].cpu()
+        vb = c0["v"][blocks.to(c0["k"].device)].cpu()
+        ksb = c0["ks"][blocks.to(c0["k"].device)].cpu()
+        vsb = c0["vs"][blocks.to(c0["k"].device)].cpu()
+        local_bt = torch.arange(n, dtype=torch.int32)[None]
+        t0 = time.perf_counter()
+        kd, vd = torch_ref.dequant_cache(kb, vb, ksb, vsb, d, torch.bfloat16)
+        torch_ref.paged_attn(q_cpu[i:i + 1], kd, vd, [1], [ctx[i]], local_bt, st["scale"])
+        t_total += time.perf_counter() - t0
+        done_bytes += ctx[i] * hkv * 2 * (d + 4) + 2 * hq * d * 2 + n * 4 + 4
+        reps += 1
+    return dict(value=done_bytes / t_total / 1e9, unit="GB/s", cores=threads, kind="port",
+                sample=f"{reps} sequence(s) of the batch ({done_bytes / 1e6:.1f} MB of algorithmic bytes), "
+                       f"oracle/torch_ref.py dequant_cache + paged_attn (bf16, as-written), {t_total:.1f} s, "
+                       f"torch threads={threads}, os.cpu_count()={os.cpu_count()}",
+                us_per_layer_extrapolated=t_total / done_bytes * algorithmic_bytes(cfg, False)[0] * 1e6)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=400)
+    ap.add_argument("--warmup", type=int, default=40)
+    ap.add_argument("--workload", default="llama3_8b_decode_b64_ctx1k-8k")
+    ap.add_argument("--layers", type=int, default=4, help="distinct layer caches the steps rotate over")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-seconds", type=float, default=15.0)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        raise SystemExit("bench.py: this build runs on ONE GPU (no collectives, no sharding); use --gpus 1")
+    if not torch.cuda.is_available():
+        raise SystemExit("bench.py: no GPU visible; the HIP kernels have no CPU fallback")
+    from vllm_metax_amd import _custom_ops as ops
+
+    dev = torch.device("cuda:0")
+    cfg = make_batch(args.workload)
+    st = build_device_state(cfg, dev, args.layers)
+    attn_bytes, write_bytes = algorithmic_bytes(cfg)
+    L = args.layers
+
+    for i in range(args.warmup):
+        run_step(st, i % L, ops)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        run_step(st, i % L, ops)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    ms_per_step = dt / args.steps * 1e3
+    value = (attn_bytes + write_bytes) / (dt / args.steps) / 1e9
+
+    # the decode attention launch alone, events on the launch stream (torch's current stream)
+    n_ev = min(args.steps, 200)
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n_ev)]
+    wevs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n_ev)]
+    for i in range(n_ev):
+        wevs[i][0].record()
+        run_step(st, i % L, ops, write=True, attn=False)
+        wevs[i][1].record()
+        evs[i][0].record()
+        run_step(st, i % L, ops, write=False, attn=True)
+        evs[i][1].record()
+    torch.cuda.synchronize()
+    attn_ms = sum(a.elapsed_time(b) for a, b in evs) / n_ev
+    write_ms = sum(a.elapsed_time(b) for a, b in wevs) / n_ev
+    achieved = attn_bytes / (attn_ms * 1e-3) / 1e9
+
+    res = {
+        "metric": METRIC,
+        "value": round(value, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "int8 KV codes, fp16 MFMA operands, fp32 softmax/accumulate, bf16 Q/out",
+        "data": "synthetic",
+        "config": {"workload": args.workload, "batch": len(cfg["ctx"]), "sum_ctx": sum(cfg["ctx"]),
+                   "q_heads": cfg["hq"], "kv_heads": cfg["hkv"], "head_dim": cfg["d"], "block_size": cfg["bs"],
+                   "pool_blocks": cfg["pool"], "layer_caches_rotated": L, "kv_layout": "NHD"},
+        "pct_hbm_peak": round(100 * value / HBM_PEAK_GBPS, 2),
+        "us_per_layer": round(ms_per_step * 1e3, 2),
+        "decode_tokens_per_s": round(len(cfg["ctx"]) / (dt / args.steps), 1),
+        "attn_launch_us": round(attn_ms * 1e3, 2),
+        "write_launch_us": round(write_ms * 1e3, 2),
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "kernel": "paged decode attention launch (split-K main kernel + reduce)",
+                     "algorithmic_bytes_per_launch": attn_bytes},
+    }
+    if not args.no_cpu_baseline:
+        res["cpu_baseline"] = cpu_baseline(cfg, st, args.cpu_seconds)
+    print(json.dumps(res))
+
+
+if __name__ == "__main__":
+    main()

@@ -29,15 +29,18 @@ __device__ __forceinline__ uint32_t perm(uint32_t hi, uint32_t lo, uint32_t sel)
   return __builtin_amdgcn_perm(hi, lo, sel);
 }
 
-// Two biased code bytes (byte b0 and b0+1 of x, already ^0x80) -> two exact fp16 codes.
+// Codes enter the MFMA as code + 1152: 0x6400 | (code ^ 0x80) is the fp16 number
+// 1024 + (code + 128), exact, built by one byte permute per two codes.  The constant is taken
+// out again exactly: the QK accumulator starts at -1152 * sum(q), and the PV accumulator is
+// corrected with 1152 * sum(P~), which one extra MFMA against a row of ones keeps in step.
+constexpr float kCodeBias = 1152.0f;
+
+// Two biased code bytes of x (already ^0x80) -> two fp16 values code + 1152.
 __device__ __forceinline__ uint32_t bytes_to_half2(uint32_t x, bool upper) {
-  const uint32_t magic = 0x64646464u;
-  uint32_t h = perm(magic, x, upper ? 0x04030402u : 0x04010400u);  // 1024 + (code + 128)
-  half2_t v = __builtin_bit_cast(half2_t, h) - (half2_t){(half_t)1152.0f, (half_t)1152.0f};
-  return __builtin_bit_cast(uint32_t, v);
+  return perm(0x64646464u, x, upper ? 0x04030402u : 0x04010400u);
 }
 
-// 8 consecutive code bytes (two dwords) -> 8 fp16 codes, the A/B operand of one MFMA k-step.
+// 8 consecutive code bytes (two dwords) -> 8 fp16 (code + 1152), one MFMA k-step operand.
 __device__ __forceinline__ half8_t dequant8(uint32_t lo, uint32_t hi) {
   lo ^= 0x80808080u;
   hi ^= 0x80808080u;
@@ -76,30 +79,52 @@ struct AttnIO {
   int num_q_heads;
   int group;  // q heads per kv head
   float scale_log2;  // softmax scale * log2(e)
+  uint32_t bs_magic;  // ceil(2^32 / block_size): x / block_size == umulhi(x, bs_magic) for x < 2^22
 };
 
 // One lane's share of a 32-token tile, as loaded.
 template <int D>
 struct KVTile {
-  static constexpr int KQ = D / 64;  // dwordx4 loads per M-tile for K (lane holds D/4 bytes)
+  static constexpr int KQ = D / 64;  // 16-byte chunks per M-tile for K (lane holds D/4 bytes)
   static constexpr int VW = D / 64;  // dwords per token for V (lane holds D/16 bytes)
   u32x4 k[2][KQ];
   uint32_t v[8][VW];
-  float sc;  // lanes 0-31: K scale of token lane; lanes 32-63: V scale of token lane-32
+  // scale of token (lane & 15) read through each half's window; the lane keeps the one of its own
+  // half (lanes 0-31: K scales, 32-63: V scales) when the tile is consumed, not when it is loaded,
+  // so that nothing has to wait on the load here
+  uint32_t sc0, sc1;
 };
 
 template <int D>
 struct DecodeState {
   static constexpr int DT = D / 16;  // M-tiles of the O^T accumulator
-  floatx4 o[DT];
-  float m;  // running max, log2 domain (uniform across the 4 lane groups of a head)
-  float l;  // lane-local partial sum
+  floatx4 o[DT];   // sum_t P~[t] * (code + 1152)
+  floatx4 psum;    // sum_t P~[t] (every register the same), to take the 1152 out again
+  float m;         // running max, log2 domain (uniform across the 4 lane groups of a head)
+  float l;         // lane-local partial sum of p
 };
 
-// Block ids of one sequence, 64 table entries at a time held one per lane.
-struct BlockIds {
-  int32_t v;
-  int base;  // first table entry held, multiple of 64; -1 = nothing loaded
+// Physical blocks of the two 16-token halves of a tile.  They are read with scalar loads
+// (uniform address, constant address space), which do not share a counter with the vector
+// loads of the KV stream, and well ahead of their use, so the pointer chase through the
+// block table never drains the prefetched tiles.
+struct TileBlocks {
+  int32_t b0, b1;
+  int32_t s1_same;  // 1: the second half lies past the sequence end and rereads the first
+};
+
+typedef const __attribute__((address_space(4))) int32_t* const_i32_ptr;
+
+__device__ __forceinline__ int32_t scalar_load_i32(const int32_t* p, int64_t i) {
+  return reinterpret_cast<const_i32_ptr>(reinterpret_cast<uintptr_t>(p))[i];
+}
+
+// Loop-invariant per-lane byte offsets into a (block, slot0, head) window of the cache, so a
+// tile's loads are "uniform base + fixed 32-bit lane offset" and cost no vector address math.
+struct LaneOffsets {
+  uint32_t k;   // r*stride_slot + k_off + g*16
+  uint32_t v;   // 4g*stride_slot + v_off + r*VB
+  uint32_t sc;  // (lane&15)*stride_slot + (lane<32 ? ks_off : vs_off)
 };
 
 template <int D, int QDT, int ODT>
@@ -110,85 +135,155 @@ struct DecodeTile {
   using Tile = KVTile<D>;
   using State = DecodeState<D>;
 
-  // ---- Q as the MFMA B operand: lane (c = head in group, g) holds dims g*D/4 + kk*8 + j ----
-  __device__ static void load_q(const AttnIO& io, int64_t row, int hkv, int lane, half8_t (&qb)[KSTEPS]) {
+  __device__ static LaneOffsets lane_offsets(const kvq_cache_geom& G, int lane) {
+    const int r = lane & 15, g = lane >> 4;
+    LaneOffsets o;
+    o.k = (uint32_t)(r * G.stride_slot + G.k_off + g * 16);
+    o.v = (uint32_t)(4 * g * G.stride_slot + G.v_off + r * VB);
+    o.sc = (uint32_t)((lane & 15) * G.stride_slot + (lane < 32 ? G.ks_off : G.vs_off));
+    return o;
+  }
+
+  // ---- Q as the MFMA B operand --------------------------------------------------------------
+  // Lane (c = head in group, g) holds, for k-step kk, dims (kk>>1)*64 + g*16 + (kk&1)*8 + j:
+  // the same dim order in which a K lane holds its code bytes.  Lanes past the group reread
+  // head 0 and are zeroed.  Returns -1152 * sum(q) of the lane's head: the QK accumulator's
+  // start value that cancels the code bias.
+  __device__ static float load_q(const AttnIO& io, int64_t row, int hkv, int lane, half8_t (&qb)[KSTEPS]) {
     const int c = lane & 15, g = lane >> 4;
     const bool valid = c < io.group;
-    const int64_t base = row * io.q_stride_t + (int64_t)(hkv * io.group + (valid ? c : 0)) * io.q_stride_h +
-                         g * (D / 4);
+    const int64_t base = row * io.q_stride_t + (int64_t)(hkv * io.group + (valid ? c : 0)) * io.q_stride_h + g * 16;
+    float f[D / 4];
 #pragma unroll
-    for (int kk = 0; kk < KSTEPS; ++kk) {
-      u32x4 r;
-      float f[8];
+    for (int ch = 0; ch < D / 64; ++ch) {
+      if constexpr (QDT == KVQ_F32) {
+        const float* p = reinterpret_cast<const float*>(io.q) + base + ch * 64;
 #pragma unroll
-      for (int j = 0; j < 8; ++j) f[j] = valid ? clamp_half_range(load_act<QDT>(io.q, base + kk * 8 + j)) : 0.f;
-      r.x = pack_half2(f[0], f[1]);
-      r.y = pack_half2(f[2], f[3]);
-      r.z = pack_half2(f[4], f[5]);
-      r.w = pack_half2(f[6], f[7]);
-      qb[kk] = __builtin_bit_cast(half8_t, r);
-    }
-  }
-
-  __device__ static int block_id(const AttnIO& io, const int32_t* bt_row, BlockIds& ids, int entry,
-                                 int num_entries, int lane) {
-    const int base = entry & ~63;
-    if (base != ids.base) {
-      const int e = base + lane;
-      ids.v = (e < num_entries) ? bt_row[e] : 0;
-      ids.base = base;
-    }
-    return __builtin_amdgcn_readlane(ids.v, entry & 63);
-  }
-
-  // Issue the global loads of tile `t` (tokens 32t .. 32t+31) of a sequence of `len` tokens.
-  __device__ static void load_tile(const AttnIO& io, const int32_t* bt_row, BlockIds& ids, int len, int t,
-                                   int hkv, int lane, Tile& kv) {
-    const kvq_cache_geom& G = io.g;
-    const int r = lane & 15, g = lane >> 4;
-    const int num_entries = (len + G.block_size - 1) / G.block_size;
-    const int tok0 = t * kTile;
-    // a 16-token M-tile never straddles a block (block_size is a multiple of 16)
-    int e0 = tok0 / G.block_size;
-    int e1 = (tok0 + 16) / G.block_size;
-    e1 = e1 < num_entries ? e1 : num_entries - 1;  // second half may lie past the end: reread, masked later
-    const int64_t b0 = block_id(io, bt_row, ids, e0, num_entries, lane);
-    const int64_t b1 = (e1 == e0) ? b0 : (int64_t)block_id(io, bt_row, ids, e1, num_entries, lane);
-    const int s0 = tok0 % G.block_size;
-    const int s1 = (e1 == (tok0 + 16) / G.block_size) ? (tok0 + 16) % G.block_size : s0;
-    const uint8_t* p0 = io.cache + b0 * G.stride_block + (int64_t)s0 * G.stride_slot + (int64_t)hkv * G.stride_head;
-    const uint8_t* p1 = io.cache + b1 * G.stride_block + (int64_t)s1 * G.stride_slot + (int64_t)hkv * G.stride_head;
-    // K: lane (r, g) reads bytes [g*D/4, (g+1)*D/4) of token r / 16 + r
-    {
-      const uint8_t* k0 = p0 + (int64_t)r * G.stride_slot + G.k_off + g * (D / 4);
-      const uint8_t* k1 = p1 + (int64_t)r * G.stride_slot + G.k_off + g * (D / 4);
+        for (int i = 0; i < 16; i += 4) {
+          const floatx4 v = *reinterpret_cast<const floatx4_a4*>(p + i);
+          f[ch * 16 + i] = v.x; f[ch * 16 + i + 1] = v.y; f[ch * 16 + i + 2] = v.z; f[ch * 16 + i + 3] = v.w;
+        }
+      } else {
+        const uint16_t* p = reinterpret_cast<const uint16_t*>(io.q) + base + ch * 64;
 #pragma unroll
-      for (int i = 0; i < Tile::KQ; ++i) {
-        kv.k[0][i] = *reinterpret_cast<const u32x4_a4*>(k0 + 16 * i);
-        kv.k[1][i] = *reinterpret_cast<const u32x4_a4*>(k1 + 16 * i);
+        for (int i = 0; i < 16; i += 8) {
+          const u32x4 v = *reinterpret_cast<const u32x4_a4*>(p + i);
+#pragma unroll
+          for (int w = 0; w < 4; ++w) {
+            if constexpr (QDT == KVQ_BF16) {
+              f[ch * 16 + i + 2 * w] = __builtin_bit_cast(float, v[w] << 16);
+              f[ch * 16 + i + 2 * w + 1] = __builtin_bit_cast(float, v[w] & 0xffff0000u);
+            } else {
+              const half2_t h = __builtin_bit_cast(half2_t, v[w]);
+              f[ch * 16 + i + 2 * w] = (float)h.x;
+              f[ch * 16 + i + 2 * w + 1] = (float)h.y;
+            }
+          }
+        }
       }
     }
-    // V: lane (r, g) reads bytes [r*VB, (r+1)*VB) of tokens 4g+j (j<4) and 16+4g+(j-4)
+    float qsum = 0.f;
+#pragma unroll
+    for (int kk = 0; kk < KSTEPS; ++kk) {
+      half8_t h;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const float x = valid ? clamp_half_range(f[(kk >> 1) * 16 + (kk & 1) * 8 + j]) : 0.f;
+        h[j] = (half_t)x;
+        qsum += (float)h[j];  // the sum of what the MFMA will actually see
+      }
+      qb[kk] = h;
+    }
+    qsum += __shfl_xor(qsum, 16, kWave);
+    qsum += __shfl_xor(qsum, 32, kWave);
+    return -kCodeBias * qsum;
+  }
+
+  // Token index -> block-table entry / slot, by multiplication (scalar ALU, no divide).
+  __device__ static int div_bs(const AttnIO& io, int x) { return (int)__umulhi((uint32_t)x, io.bs_magic); }
+  __device__ static int mod_bs(const AttnIO& io, int x) { return x - div_bs(io, x) * io.g.block_size; }
+
+  // Block-table entries of tile `t` (clamped into the sequence so the read is always valid).
+  __device__ static TileBlocks fetch_blocks(const AttnIO& io, const int32_t* bt_row, int len, int t) {
+    const int num_entries = div_bs(io, len + io.g.block_size - 1);
+    const int tok0 = t * kTile;
+    int e0 = div_bs(io, tok0);
+    e0 = e0 < num_entries ? e0 : num_entries - 1;
+    const int e1raw = div_bs(io, tok0 + 16);
+    const int e1 = e1raw < num_entries ? e1raw : num_entries - 1;
+    TileBlocks tb;
+    tb.b0 = scalar_load_i32(bt_row, e0);
+    tb.b1 = scalar_load_i32(bt_row, e1);
+    tb.s1_same = e1raw < num_entries ? 0 : 1;
+    return tb;
+  }
+
+  // Buffer resources (scalar registers) of the two 16-token halves of tile `t` for kv head
+  // `hkv`: every load of the tile is "resource + fixed 32-bit lane offset + scalar offset", so
+  // the stream costs no vector address arithmetic and no address registers.
+  struct Window {
+    __amdgpu_buffer_rsrc_t r0, r1;
+  };
+  __device__ static Window window(const AttnIO& io, const TileBlocks& tb, int t, int hkv) {
+    const kvq_cache_geom& G = io.g;
+    const int tok0 = t * kTile;
+    // a 16-token M-tile never straddles a block (block_size is a multiple of 16); a second half
+    // past the end of the sequence rereads the first half and is masked in compute
+    const int s0 = mod_bs(io, tok0);
+    const int s1 = tb.s1_same ? s0 : mod_bs(io, tok0 + 16);
+    const uint8_t* p0 = io.cache + (int64_t)tb.b0 * G.stride_block + (int64_t)s0 * G.stride_slot + (int64_t)hkv * G.stride_head;
+    const uint8_t* p1 = io.cache + (int64_t)tb.b1 * G.stride_block + (int64_t)s1 * G.stride_slot + (int64_t)hkv * G.stride_head;
+    Window w;
+    w.r0 = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(p0), 0, 0x7fffffff, 0x00020000);
+    w.r1 = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(p1), 0, 0x7fffffff, 0x00020000);
+    return w;
+  }
+
+  // K codes and the 64 scales of a tile.  K: lane (r, g) reads 16-byte chunks [i*64 + g*16, +16)
+  // of token r (M-tile 0) / 16 + r (M-tile 1), so the four lanes of a token cover 64 contiguous
+  // bytes per load.  Scales: lanes 0-31 K scale of token lane, lanes 32-63 V scale of token lane-32.
+  __device__ static void load_k(const Window& w, const LaneOffsets& lo, int lane, Tile& kv) {
+#pragma unroll
+    for (int i = 0; i < Tile::KQ; ++i) {
+      kv.k[0][i] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(w.r0, lo.k, 64 * i, 0));
+      kv.k[1][i] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(w.r1, lo.k, 64 * i, 0));
+    }
+    kv.sc0 = __builtin_amdgcn_raw_buffer_load_b32(w.r0, lo.sc, 0, 0);
+    kv.sc1 = __builtin_amdgcn_raw_buffer_load_b32(w.r1, lo.sc, 0, 0);
+  }
+
+  // V codes of a tile: lane (r, g) reads bytes [r*VB, (r+1)*VB) of tokens 4g+j (j<4) and
+  // 16+4g+(j-4); sixteen lanes cover one token's 16*VB contiguous bytes.
+  __device__ static void load_v(const AttnIO& io, const Window& w, const LaneOffsets& lo, Tile& kv) {
+    const int ss = (int)io.g.stride_slot;
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
-      const uint8_t* pv = (j < 4 ? p0 : p1) + (int64_t)(4 * g + (j & 3)) * G.stride_slot + G.v_off + r * VB;
-#pragma unroll
-      for (int w = 0; w < Tile::VW; ++w) kv.v[j][w] = *reinterpret_cast<const uint32_t*>(pv + 4 * w);
-    }
-    // scales: lanes 0-31 K scale of token lane, lanes 32-63 V scale of token lane-32
-    {
-      const int tk = lane & 31;
-      const uint8_t* ps = (tk < 16 ? p0 : p1) + (int64_t)(tk & 15) * G.stride_slot + (lane < 32 ? G.ks_off : G.vs_off);
-      kv.sc = *reinterpret_cast<const float*>(ps);
+      const __amdgpu_buffer_rsrc_t r = j < 4 ? w.r0 : w.r1;
+      const int soff = (j & 3) * ss;
+      if constexpr (Tile::VW == 1) {
+        kv.v[j][0] = __builtin_amdgcn_raw_buffer_load_b32(r, lo.v, soff, 0);
+      } else if constexpr (Tile::VW == 2) {
+        const u32x2 x = __builtin_bit_cast(u32x2, __builtin_amdgcn_raw_buffer_load_b64(r, lo.v, soff, 0));
+        kv.v[j][0] = x.x;
+        kv.v[j][1] = x.y;
+      } else {
+        const u32x4 x = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(r, lo.v, soff, 0));
+        kv.v[j][0] = x.x; kv.v[j][1] = x.y; kv.v[j][2] = x.z; kv.v[j][3] = x.w;
+      }
     }
   }
 
-  // Consume one loaded tile.  `sc_lds` is this wave's 64-float staging area.
-  __device__ static void compute_tile(const AttnIO& io, const Tile& kv, const half8_t (&qb)[KSTEPS], int len,
-                                      int t, int lane, float* sc_lds, State& st) {
+  // Phase 1 of a tile: scales through LDS, S^T = K . Q^T on the MFMA, online softmax.
+  // Consumes kv.k and kv.sc (both free for the next prefetch afterwards) and returns P~^T as
+  // the MFMA B operand.  `sc_lds` is this wave's 64-float staging area; `sc_mul` is the lane's
+  // staging multiplier (softmax scale * log2e for the K-scale lanes, 2^8 for the V-scale lanes).
+  // MASK: the tile holds the end of the sequence (tokens >= len must not contribute).
+  template <bool MASK>
+  __device__ static half8_t qk_softmax(const Tile& kv, const half8_t (&qb)[KSTEPS], float s_init, float sc_mul,
+                                       int len, int t, int lane, float* sc_lds, State& st) {
     const int g = lane >> 4;
-    // --- scales: transpose lane<->token through LDS (wave-private, no barrier needed) ---
-    sc_lds[lane] = kv.sc;
+    // K scales come out pre-multiplied by scale*log2e, V scales by 2^8 (capped so P~ stays finite)
+    sc_lds[lane] = fminf(__builtin_bit_cast(float, (lane & 16) ? kv.sc1 : kv.sc0) * sc_mul, 65504.f);
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
@@ -198,11 +293,11 @@ struct DecodeTile {
     const floatx4 vs1 = *reinterpret_cast<const floatx4*>(sc_lds + 48 + 4 * g);
     __builtin_amdgcn_wave_barrier();
 
-    // --- S^T = K . Q^T : two 16-token M-tiles, KSTEPS k-steps each ---
+    // two 16-token M-tiles, KSTEPS k-steps each; accumulators start at -1152 * sum(q)
     floatx4 s[2];
 #pragma unroll
     for (int mt = 0; mt < 2; ++mt) {
-      s[mt] = (floatx4){0.f, 0.f, 0.f, 0.f};
+      s[mt] = (floatx4){s_init, s_init, s_init, s_init};
 #pragma unroll
       for (int kk = 0; kk < KSTEPS; ++kk) {
         const u32x4& w = kv.k[mt][kk >> 1];
@@ -211,7 +306,7 @@ struct DecodeTile {
       }
     }
 
-    // --- softmax (log2 domain); lane holds tokens 32t + mt*16 + 4g + i of head (lane & 15) ---
+    // softmax in the log2 domain; lane holds tokens 32t + mt*16 + 4g + i of head (lane & 15)
     float logit[8];
     const int tok_base = t * kTile + 4 * g;
     float mloc = -INFINITY;
@@ -219,9 +314,8 @@ struct DecodeTile {
     for (int mt = 0; mt < 2; ++mt) {
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const float ks = (mt ? ks1 : ks0)[i];
-        const bool ok = (tok_base + mt * 16 + i) < len;
-        const float x = ok ? s[mt][i] * (ks * io.scale_log2) : -INFINITY;
+        float x = s[mt][i] * (mt ? ks1 : ks0)[i];
+        if constexpr (MASK) x = ((tok_base + mt * 16 + i) < len) ? x : -INFINITY;
         logit[mt * 4 + i] = x;
         mloc = fmaxf(mloc, x);
       }
@@ -233,6 +327,7 @@ struct DecodeTile {
       const float alpha = __builtin_amdgcn_exp2f(st.m - m_new);  // st.m = -inf -> 0
       st.m = m_new;
       st.l *= alpha;
+      st.psum *= alpha;
 #pragma unroll
       for (int dt = 0; dt < DT; ++dt) st.o[dt] *= alpha;
     }
@@ -244,9 +339,9 @@ struct DecodeTile {
         const int j = mt * 4 + i;
         const float p = __builtin_amdgcn_exp2f(logit[j] - st.m);  // masked: exp2(-inf) = 0
         st.l += p;
-        const float vs = (mt ? vs1 : vs0)[i];
-        const bool ok = (tok_base + mt * 16 + i) < len;
-        pt[j] = ok ? clamp_half_range(p * (vs * kPScale)) : 0.f;  // garbage scales of masked tokens never enter
+        float x = p * (mt ? vs1 : vs0)[i];
+        if constexpr (MASK) x = ((tok_base + mt * 16 + i) < len) ? x : 0.f;  // garbage scales never enter
+        pt[j] = x;
       }
     }
     u32x4 pb;
@@ -254,9 +349,17 @@ struct DecodeTile {
     pb.y = pack_half2(pt[2], pt[3]);
     pb.z = pack_half2(pt[4], pt[5]);
     pb.w = pack_half2(pt[6], pt[7]);
-    const half8_t p_op = __builtin_bit_cast(half8_t, pb);
+    return __builtin_bit_cast(half8_t, pb);
+  }
 
-    // --- O^T += V^T . P~^T : in-register 8x(VB) byte transpose, then one MFMA per dim tile ---
+  // Phase 2 of a tile: O^T += (V + 1152)^T . P~^T with an in-register 8 x VB byte transpose
+  // (one MFMA per 16-dim tile), and sum(P~) against a row of ones.  Consumes kv.v.
+  __device__ static void pv(const Tile& kv, half8_t p_op, State& st) {
+    {
+      const half_t one = (half_t)1.0f;
+      const half8_t ones = {one, one, one, one, one, one, one, one};
+      st.psum = __builtin_amdgcn_mfma_f32_16x16x32_f16(ones, p_op, st.psum, 0, 0, 0);
+    }
 #pragma unroll
     for (int w = 0; w < Tile::VW; ++w) {
       uint32_t x0[4], x1[4];  // per token pair a: bytes (b0,b1) and (b2,b3) of both tokens, interleaved
@@ -281,27 +384,115 @@ struct DecodeTile {
     }
   }
 
+  // Keeps the instruction scheduler from moving work across the phase boundaries of the
+  // stream loop: a refill must be issued where it is written (right after the registers it
+  // overwrites were consumed), and a tile's V conversion must not drift up into the QK phase,
+  // where it would wait on the newest loads instead of the oldest.
+  __device__ static __forceinline__ void phase_fence() { __builtin_amdgcn_sched_barrier(0); }
+
   // Run tiles [t_begin, t_end) of one sequence for kv head `hkv`; leaves the state in `st`.
+  // Two register buffers, refilled in halves: as soon as a tile's K codes (or V codes) have
+  // gone into the MFMA, the same registers take the K (or V) of the tile two ahead, so about
+  // two tiles of loads per wave are in flight at any time.
   __device__ static void run(const AttnIO& io, int seq, int64_t row, int len, int t_begin, int t_end, int hkv,
                              int lane, float* sc_lds, State& st) {
     half8_t qb[KSTEPS];
-    load_q(io, row, hkv, lane, qb);
+    const float s_init = load_q(io, row, hkv, lane, qb);
+    const LaneOffsets lo = lane_offsets(io.g, lane);
+    const float sc_mul = lane < 32 ? io.scale_log2 : kPScale;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) st.o[dt] = (floatx4){0.f, 0.f, 0.f, 0.f};
+    st.psum = (floatx4){0.f, 0.f, 0.f, 0.f};
     st.m = -INFINITY;
     st.l = 0.f;
     const int32_t* bt_row = io.block_table + (int64_t)seq * io.bt_stride;
-    BlockIds ids{0, -1};
     Tile a, b;
-    load_tile(io, bt_row, ids, len, t_begin, hkv, lane, a);
-    for (int t = t_begin; t < t_end; t += 2) {
-      const bool has_b = (t + 1) < t_end;
-      if (has_b) load_tile(io, bt_row, ids, len, t + 1, hkv, lane, b);
-      compute_tile(io, a, qb, len, t, lane, sc_lds, st);
-      if (has_b) {
-        if ((t + 2) < t_end) load_tile(io, bt_row, ids, len, t + 2, hkv, lane, a);
-        compute_tile(io, b, qb, len, t + 1, lane, sc_lds, st);
+    int t = t_begin;
+    // block ids run ahead of the loads that use them (fetch_blocks clamps past the end)
+    TileBlocks ba = fetch_blocks(io, bt_row, len, t);
+    TileBlocks bb = fetch_blocks(io, bt_row, len, t + 1);
+    if (t + 3 < t_end) {
+      // long run.  The prologue issues its loads in exactly the order of the steady state and
+      // without conditions, so that inside the loop every wait is for the oldest loads only.
+      {
+        const Window w = window(io, ba, t, hkv);
+        load_k(w, lo, lane, a);
+        phase_fence();
+        load_v(io, w, lo, a);
+        phase_fence();
+        ba = fetch_blocks(io, bt_row, len, t + 2);
       }
+      {
+        const Window w = window(io, bb, t + 1, hkv);
+        load_k(w, lo, lane, b);
+        phase_fence();
+        load_v(io, w, lo, b);
+        phase_fence();
+        bb = fetch_blocks(io, bt_row, len, t + 3);
+      }
+      // steady state: two tiles per trip; tiles t+2 and t+3 exist, so every load is
+      // unconditional and none of the tiles computed here ends the sequence
+      do {
+        {
+          const Window w = window(io, ba, t + 2, hkv);
+          const half8_t p = qk_softmax<false>(a, qb, s_init, sc_mul, len, t, lane, sc_lds, st);
+          phase_fence();
+          load_k(w, lo, lane, a);
+          phase_fence();
+          pv(a, p, st);
+          phase_fence();
+          load_v(io, w, lo, a);
+          phase_fence();
+          ba = fetch_blocks(io, bt_row, len, t + 4);
+        }
+        {
+          const Window w = window(io, bb, t + 3, hkv);
+          const half8_t p = qk_softmax<false>(b, qb, s_init, sc_mul, len, t + 1, lane, sc_lds, st);
+          phase_fence();
+          load_k(w, lo, lane, b);
+          phase_fence();
+          pv(b, p, st);
+          phase_fence();
+          load_v(io, w, lo, b);
+          phase_fence();
+          bb = fetch_blocks(io, bt_row, len, t + 5);
+        }
+        t += 2;
+      } while (t + 3 < t_end);
+    } else {
+      // short run (at most three tiles)
+      {
+        const Window w = window(io, ba, t, hkv);
+        load_k(w, lo, lane, a);
+        load_v(io, w, lo, a);
+      }
+      ba = fetch_blocks(io, bt_row, len, t + 2);
+      if (t + 1 < t_end) {
+        const Window w = window(io, bb, t + 1, hkv);
+        load_k(w, lo, lane, b);
+        load_v(io, w, lo, b);
+      }
+    }
+    // tail: 1..3 tiles left; a holds t, b holds t+1 (if any); ba = blocks of t+2
+    const int rem = t_end - t;
+    {
+      const bool more = rem >= 3;
+      const Window w = window(io, ba, t + 2, hkv);
+      const half8_t p = ((t + 1) * kTile > len) ? qk_softmax<true>(a, qb, s_init, sc_mul, len, t, lane, sc_lds, st)
+                                                : qk_softmax<false>(a, qb, s_init, sc_mul, len, t, lane, sc_lds, st);
+      if (more) load_k(w, lo, lane, a);
+      pv(a, p, st);
+      if (more) load_v(io, w, lo, a);
+    }
+    if (rem >= 2) {
+      const half8_t p = ((t + 2) * kTile > len) ? qk_softmax<true>(b, qb, s_init, sc_mul, len, t + 1, lane, sc_lds, st)
+                                                : qk_softmax<false>(b, qb, s_init, sc_mul, len, t + 1, lane, sc_lds, st);
+      pv(b, p, st);
+    }
+    if (rem >= 3) {
+      const half8_t p = ((t + 3) * kTile > len) ? qk_softmax<true>(a, qb, s_init, sc_mul, len, t + 2, lane, sc_lds, st)
+                                                : qk_softmax<false>(a, qb, s_init, sc_mul, len, t + 2, lane, sc_lds, st);
+      pv(a, p, st);
     }
   }
 
@@ -314,12 +505,13 @@ struct DecodeTile {
   }
 
   // Lane (c, g) holds O[head c][dim (4g+i)*VB + dt], i = 0..3, dt = 0..DT-1: D/4 contiguous
-  // dims starting at g*D/4.  Gather them in order, scaled by `mul`.
+  // dims starting at g*D/4.  Gather them in order, code bias removed, scaled by `mul`.
   __device__ static void gather_row(const State& st, float mul, float (&v)[D / 4]) {
+    const float corr = kCodeBias * st.psum[0];
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
-      for (int dt = 0; dt < DT; ++dt) v[i * VB + dt] = st.o[dt][i] * mul;
+      for (int dt = 0; dt < DT; ++dt) v[i * VB + dt] = (st.o[dt][i] - corr) * mul;
   }
 
   // Whole sequence handled by this wave: normalise and write the output row (and lse).

@@ -64,6 +64,7 @@ extern "C" int kvq_paged_attn_int8(void* out, int out_dtype, int64_t out_stride_
   a.io.num_q_heads = num_q_heads;
   a.io.group = num_q_heads / g.num_kv_heads;
   a.io.scale_log2 = scale * kLog2e;
+  a.io.bs_magic = (uint32_t)((0x100000000ull + (uint64_t)geom->block_size - 1) / (uint64_t)geom->block_size);
   a.seq_lens = seq_lens;
   a.cu_seqlens_q = cu_seqlens_q;
   a.num_seqs = num_seqs;

@@ -45,7 +45,7 @@ __global__ __launch_bounds__(WPW * 64) void paged_decode_streamk_kernel(StreamKA
   __shared__ __align__(16) float sc_lds[WPW][64];
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
-  const int hkv = blockIdx.y * WPW + wave;
+  const int hkv = __builtin_amdgcn_readfirstlane(blockIdx.y * WPW + wave);
   if (hkv >= a.io.g.num_kv_heads) return;  // no workgroup barriers below
   const int w = blockIdx.x;
   const int B = a.num_seqs;
@@ -179,7 +179,7 @@ __global__ __launch_bounds__(WPW * 64) void paged_decode_v2_kernel(V2Args a) {
   using DTile = DecodeTile<D, QDT, KVQ_F32>;
   __shared__ __align__(16) float sc_lds[WPW][64];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int hkv = blockIdx.z * WPW + wave;
+  const int hkv = __builtin_amdgcn_readfirstlane(blockIdx.z * WPW + wave);
   if (hkv >= a.io.g.num_kv_heads) return;
   const int part = blockIdx.x, seq = blockIdx.y;
   const int len = a.seq_lens[seq];
@@ -394,6 +394,7 @@ int kvq_paged_attn_v2_int8(void* out, int out_dtype, float* exp_sums, float* max
   a.io.num_q_heads = num_q_heads;
   a.io.group = num_q_heads / geom->num_kv_heads;
   a.io.scale_log2 = scale * kLog2e;
+  a.io.bs_magic = (uint32_t)((0x100000000ull + (uint64_t)geom->block_size - 1) / (uint64_t)geom->block_size);
   a.seq_lens = seq_lens;
   a.tmp_out = tmp_out;
   a.max_logits = max_logits;
