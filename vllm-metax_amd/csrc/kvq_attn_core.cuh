@@ -1,18 +1,22 @@
 // Core of the bandwidth-bound int8 paged decode tile (gfx950, wave64, MFMA f16).
 //
-// One wavefront owns one KV head and streams that head's records for a run of
-// 32-token tiles.  Per tile it
-//   * loads the K codes (lane = token x quarter-of-head, 16-byte loads), the V codes
-//     (lane = dim-octet x 8 tokens, 8-byte loads) and the 64 fp32 scales, all straight
-//     from HBM into registers, double-buffered one tile ahead;
-//   * turns codes into exact fp16 integers in registers with the byte-permute magic
-//     number trick (0x6400 | (code ^ 0x80) = 1024 + code + 128, minus 1152);
-//   * S^T[token, head] = K . Q^T on the MFMA (the GQA group's heads are the N dim, so
-//     the KV stream is read once for all of them), softmax in fp32 with the per-token
-//     K scale applied to the logits;
+// One wavefront owns one KV head and streams that head's (token, head) records --
+// [K codes | K scale | V codes | V scale], 2*(D+4) bytes each -- for a run of 32-token tiles.
+// Per tile it
+//   * reads the 32 records as flat 16-byte chunks, consecutive lanes taking consecutive chunks
+//     of one record, so every quarter-wave touches 256 contiguous bytes of HBM; the chunks land
+//     in registers, two tiles ahead of the tile being computed;
+//   * drops the chunks into a wave-private LDS window (one record per row, 16-byte aligned,
+//     bank-conflict-free pitch) and reads them back in MFMA operand order: the transposition
+//     between "how memory is laid out" and "how the matrix core wants it" happens in LDS;
+//   * turns codes into exact fp16 numbers code + 1152 with one byte permute per two codes
+//     (0x6400 | (code ^ 0x80)); the constant is removed exactly afterwards;
+//   * S^T[token, head] = K . Q^T on the MFMA (the GQA group's heads are the N dim, so the KV
+//     stream is read once for all of them), softmax in fp32 with the per-token K scale applied
+//     to the logits;
 //   * O^T[dim, head] += V^T . P~^T on the MFMA, P~ = p * v_scale rounded to fp16.
-// The S accumulator layout (lane = head, registers = tokens) is exactly the B-operand
-// layout P~^T needs, and the running max / sum / rescale of a head stay lane-local.
+// The S accumulator layout (lane = head, registers = tokens) is exactly the B-operand layout
+// P~^T needs, and the running max / sum / rescale of a head stay lane-local.
 #pragma once
 
 #include "kvq_internal.h"
@@ -82,17 +86,13 @@ struct AttnIO {
   uint32_t bs_magic;  // ceil(2^32 / block_size): x / block_size == umulhi(x, bs_magic) for x < 2^22
 };
 
-// One lane's share of a 32-token tile, as loaded.
+// One lane's share of a 32-token tile as it arrives from HBM: raw 16-byte chunks of records.
 template <int D>
 struct KVTile {
-  static constexpr int KQ = D / 64;  // 16-byte chunks per M-tile for K (lane holds D/4 bytes)
-  static constexpr int VW = D / 64;  // dwords per token for V (lane holds D/16 bytes)
-  u32x4 k[2][KQ];
-  uint32_t v[8][VW];
-  // scale of token (lane & 15) read through each half's window; the lane keeps the one of its own
-  // half (lanes 0-31: K scales, 32-63: V scales) when the tile is consumed, not when it is loaded,
-  // so that nothing has to wait on the load here
-  uint32_t sc0, sc1;
+  static constexpr int NCH = D / 8;        // full 16-byte chunks per record (2*D bytes)
+  static constexpr int NLD = NCH / 4;      // wave-wide chunk loads per 16-token half
+  u32x4 c[2][NLD];                         // chunk (n*64 + lane) of half 0 / half 1
+  u32x2 tail0, tail1;                      // last 8 bytes of record (lane & 15) of half 0 / half 1
 };
 
 template <int D>
@@ -119,12 +119,15 @@ __device__ __forceinline__ int32_t scalar_load_i32(const int32_t* p, int64_t i) 
   return reinterpret_cast<const_i32_ptr>(reinterpret_cast<uintptr_t>(p))[i];
 }
 
-// Loop-invariant per-lane byte offsets into a (block, slot0, head) window of the cache, so a
-// tile's loads are "uniform base + fixed 32-bit lane offset" and cost no vector address math.
+// Loop-invariant per-lane offsets.
 struct LaneOffsets {
-  uint32_t k;   // r*stride_slot + k_off + g*16
-  uint32_t v;   // 4g*stride_slot + v_off + r*VB
-  uint32_t sc;  // (lane&15)*stride_slot + (lane<32 ? ks_off : vs_off)
+  uint32_t g_chunk;   // HBM: (lane / NCH)*stride_slot + 16*(lane % NCH), chunk `lane` of a half
+  uint32_t g_tail;    // HBM: (lane & 15)*stride_slot + 2*D, the record's last 8 bytes
+  uint32_t l_chunk;   // LDS: (lane / NCH)*PITCH + 16*(lane % NCH)
+  uint32_t l_tail;    // LDS: (lane & 31)*PITCH + 2*D
+  uint32_t l_k;       // LDS: r*PITCH + g*16, K operand chunk of token r
+  uint32_t l_v;       // LDS: 4g*PITCH + (D+4) + r*VB, V operand bytes of token 4g
+  uint32_t l_sc;      // LDS: (lane & 31)*PITCH + (lane < 32 ? D : 2*D+4), the lane's scale
 };
 
 template <int D, int QDT, int ODT>
@@ -135,12 +138,23 @@ struct DecodeTile {
   using Tile = KVTile<D>;
   using State = DecodeState<D>;
 
+  static constexpr int R = 2 * (D + 4);      // record bytes
+  static constexpr int PITCH = R + 8;        // LDS row pitch: 16-byte aligned rows, conflict-free operand reads
+  static constexpr int NCH = Tile::NCH;
+  static constexpr int NLD = Tile::NLD;
+  static constexpr int LDS_TILE = kTile * PITCH;          // bytes of the record window
+  static constexpr int LDS_WAVE = LDS_TILE + 64 * 4;      // + 64 staged scales
+
   __device__ static LaneOffsets lane_offsets(const kvq_cache_geom& G, int lane) {
     const int r = lane & 15, g = lane >> 4;
     LaneOffsets o;
-    o.k = (uint32_t)(r * G.stride_slot + G.k_off + g * 16);
-    o.v = (uint32_t)(4 * g * G.stride_slot + G.v_off + r * VB);
-    o.sc = (uint32_t)((lane & 15) * G.stride_slot + (lane < 32 ? G.ks_off : G.vs_off));
+    o.g_chunk = (uint32_t)((lane / NCH) * G.stride_slot + 16 * (lane % NCH));
+    o.g_tail = (uint32_t)((lane & 15) * G.stride_slot + 2 * D);
+    o.l_chunk = (uint32_t)((lane / NCH) * PITCH + 16 * (lane % NCH));
+    o.l_tail = (uint32_t)((lane & 31) * PITCH + 2 * D);
+    o.l_k = (uint32_t)(r * PITCH + g * 16);
+    o.l_v = (uint32_t)(4 * g * PITCH + (D + 4) + r * VB);
+    o.l_sc = (uint32_t)((lane & 31) * PITCH + (lane < 32 ? D : 2 * D + 4));
     return o;
   }
 
@@ -219,79 +233,69 @@ struct DecodeTile {
   }
 
   // Buffer resources (scalar registers) of the two 16-token halves of tile `t` for kv head
-  // `hkv`: every load of the tile is "resource + fixed 32-bit lane offset + scalar offset", so
-  // the stream costs no vector address arithmetic and no address registers.
+  // `hkv`, based at the first record of each half: every load of the tile is "resource + fixed
+  // 32-bit lane offset + scalar offset", no vector address arithmetic, no address registers.
   struct Window {
     __amdgpu_buffer_rsrc_t r0, r1;
   };
   __device__ static Window window(const AttnIO& io, const TileBlocks& tb, int t, int hkv) {
     const kvq_cache_geom& G = io.g;
     const int tok0 = t * kTile;
-    // a 16-token M-tile never straddles a block (block_size is a multiple of 16); a second half
+    // a 16-token half never straddles a block (block_size is a multiple of 16); a second half
     // past the end of the sequence rereads the first half and is masked in compute
     const int s0 = mod_bs(io, tok0);
     const int s1 = tb.s1_same ? s0 : mod_bs(io, tok0 + 16);
-    const uint8_t* p0 = io.cache + (int64_t)tb.b0 * G.stride_block + (int64_t)s0 * G.stride_slot + (int64_t)hkv * G.stride_head;
-    const uint8_t* p1 = io.cache + (int64_t)tb.b1 * G.stride_block + (int64_t)s1 * G.stride_slot + (int64_t)hkv * G.stride_head;
+    const uint8_t* p0 = io.cache + G.k_off + (int64_t)tb.b0 * G.stride_block + (int64_t)s0 * G.stride_slot + (int64_t)hkv * G.stride_head;
+    const uint8_t* p1 = io.cache + G.k_off + (int64_t)tb.b1 * G.stride_block + (int64_t)s1 * G.stride_slot + (int64_t)hkv * G.stride_head;
     Window w;
     w.r0 = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(p0), 0, 0x7fffffff, 0x00020000);
     w.r1 = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(p1), 0, 0x7fffffff, 0x00020000);
     return w;
   }
 
-  // K codes and the 64 scales of a tile.  K: lane (r, g) reads 16-byte chunks [i*64 + g*16, +16)
-  // of token r (M-tile 0) / 16 + r (M-tile 1), so the four lanes of a token cover 64 contiguous
-  // bytes per load.  Scales: lanes 0-31 K scale of token lane, lanes 32-63 V scale of token lane-32.
-  __device__ static void load_k(const Window& w, const LaneOffsets& lo, int lane, Tile& kv) {
+  // Issue the HBM loads of one tile: 2*NLD chunk loads (lane n*64+l takes chunk (n*64+l) % NCH of
+  // record (n*64+l) / NCH of the half) and the two 8-byte record tails.
+  __device__ static void load_tile(const AttnIO& io, const Window& w, const LaneOffsets& lo, Tile& kv) {
+    const int step = (64 / NCH) * (int)io.g.stride_slot;  // records advanced per wave-wide load
 #pragma unroll
-    for (int i = 0; i < Tile::KQ; ++i) {
-      kv.k[0][i] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(w.r0, lo.k, 64 * i, 0));
-      kv.k[1][i] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(w.r1, lo.k, 64 * i, 0));
+    for (int n = 0; n < NLD; ++n) {
+      kv.c[0][n] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(w.r0, lo.g_chunk, n * step, 0));
+      kv.c[1][n] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(w.r1, lo.g_chunk, n * step, 0));
     }
-    kv.sc0 = __builtin_amdgcn_raw_buffer_load_b32(w.r0, lo.sc, 0, 0);
-    kv.sc1 = __builtin_amdgcn_raw_buffer_load_b32(w.r1, lo.sc, 0, 0);
+    kv.tail0 = __builtin_bit_cast(u32x2, __builtin_amdgcn_raw_buffer_load_b64(w.r0, lo.g_tail, 0, 0));
+    kv.tail1 = __builtin_bit_cast(u32x2, __builtin_amdgcn_raw_buffer_load_b64(w.r1, lo.g_tail, 0, 0));
   }
 
-  // V codes of a tile: lane (r, g) reads bytes [r*VB, (r+1)*VB) of tokens 4g+j (j<4) and
-  // 16+4g+(j-4); sixteen lanes cover one token's 16*VB contiguous bytes.
-  __device__ static void load_v(const AttnIO& io, const Window& w, const LaneOffsets& lo, Tile& kv) {
-    const int ss = (int)io.g.stride_slot;
+  // Drop a loaded tile into the wave's LDS window, one record per PITCH-byte row, then stage the
+  // 64 scales (K scales pre-multiplied by scale*log2e, V scales by 2^8, capped so P~ stays finite).
+  // After this the tile's registers are free for the next prefetch.
+  __device__ static void stage(const Tile& kv, const LaneOffsets& lo, float sc_mul, int lane, uint8_t* lds) {
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const __amdgpu_buffer_rsrc_t r = j < 4 ? w.r0 : w.r1;
-      const int soff = (j & 3) * ss;
-      if constexpr (Tile::VW == 1) {
-        kv.v[j][0] = __builtin_amdgcn_raw_buffer_load_b32(r, lo.v, soff, 0);
-      } else if constexpr (Tile::VW == 2) {
-        const u32x2 x = __builtin_bit_cast(u32x2, __builtin_amdgcn_raw_buffer_load_b64(r, lo.v, soff, 0));
-        kv.v[j][0] = x.x;
-        kv.v[j][1] = x.y;
-      } else {
-        const u32x4 x = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(r, lo.v, soff, 0));
-        kv.v[j][0] = x.x; kv.v[j][1] = x.y; kv.v[j][2] = x.z; kv.v[j][3] = x.w;
-      }
+    for (int n = 0; n < NLD; ++n) {
+      *reinterpret_cast<u32x4*>(lds + lo.l_chunk + n * (64 / NCH) * PITCH) = kv.c[0][n];
+      *reinterpret_cast<u32x4*>(lds + lo.l_chunk + (16 + n * (64 / NCH)) * PITCH) = kv.c[1][n];
     }
-  }
-
-  // Phase 1 of a tile: scales through LDS, S^T = K . Q^T on the MFMA, online softmax.
-  // Consumes kv.k and kv.sc (both free for the next prefetch afterwards) and returns P~^T as
-  // the MFMA B operand.  `sc_lds` is this wave's 64-float staging area; `sc_mul` is the lane's
-  // staging multiplier (softmax scale * log2e for the K-scale lanes, 2^8 for the V-scale lanes).
-  // MASK: the tile holds the end of the sequence (tokens >= len must not contribute).
-  template <bool MASK>
-  __device__ static half8_t qk_softmax(const Tile& kv, const half8_t (&qb)[KSTEPS], float s_init, float sc_mul,
-                                       int len, int t, int lane, float* sc_lds, State& st) {
-    const int g = lane >> 4;
-    // K scales come out pre-multiplied by scale*log2e, V scales by 2^8 (capped so P~ stays finite)
-    sc_lds[lane] = fminf(__builtin_bit_cast(float, (lane & 16) ? kv.sc1 : kv.sc0) * sc_mul, 65504.f);
+    if (lane < 32) *reinterpret_cast<u32x2*>(lds + lo.l_tail) = (lane & 16) ? kv.tail1 : kv.tail0;
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    const float sc = *reinterpret_cast<const float*>(lds + lo.l_sc);
+    reinterpret_cast<float*>(lds + LDS_TILE)[lane] = fminf(sc * sc_mul, 65504.f);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  }
+
+  // Phase 1 of a tile: S^T = K . Q^T on the MFMA from the LDS window, online softmax.  Returns
+  // P~^T as the MFMA B operand.  MASK: the tile holds the end of the sequence (tokens >= len must
+  // not contribute).
+  template <bool MASK>
+  __device__ static half8_t qk_softmax(const LaneOffsets& lo, const half8_t (&qb)[KSTEPS], float s_init, int len,
+                                       int t, int lane, const uint8_t* lds, State& st) {
+    const int g = lane >> 4;
+    const float* sc_lds = reinterpret_cast<const float*>(lds + LDS_TILE);
     const floatx4 ks0 = *reinterpret_cast<const floatx4*>(sc_lds + 4 * g);
     const floatx4 ks1 = *reinterpret_cast<const floatx4*>(sc_lds + 16 + 4 * g);
-    const floatx4 vs0 = *reinterpret_cast<const floatx4*>(sc_lds + 32 + 4 * g);
-    const floatx4 vs1 = *reinterpret_cast<const floatx4*>(sc_lds + 48 + 4 * g);
-    __builtin_amdgcn_wave_barrier();
 
     // two 16-token M-tiles, KSTEPS k-steps each; accumulators start at -1152 * sum(q)
     floatx4 s[2];
@@ -299,10 +303,10 @@ struct DecodeTile {
     for (int mt = 0; mt < 2; ++mt) {
       s[mt] = (floatx4){s_init, s_init, s_init, s_init};
 #pragma unroll
-      for (int kk = 0; kk < KSTEPS; ++kk) {
-        const u32x4& w = kv.k[mt][kk >> 1];
-        const half8_t a = (kk & 1) ? dequant8(w.z, w.w) : dequant8(w.x, w.y);
-        s[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, qb[kk], s[mt], 0, 0, 0);
+      for (int i = 0; i < KSTEPS / 2; ++i) {
+        const u32x4 w = *reinterpret_cast<const u32x4*>(lds + lo.l_k + mt * 16 * PITCH + i * 64);
+        s[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(dequant8(w.x, w.y), qb[2 * i], s[mt], 0, 0, 0);
+        s[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(dequant8(w.z, w.w), qb[2 * i + 1], s[mt], 0, 0, 0);
       }
     }
 
@@ -331,6 +335,8 @@ struct DecodeTile {
 #pragma unroll
       for (int dt = 0; dt < DT; ++dt) st.o[dt] *= alpha;
     }
+    const floatx4 vs0 = *reinterpret_cast<const floatx4*>(sc_lds + 32 + 4 * g);
+    const floatx4 vs1 = *reinterpret_cast<const floatx4*>(sc_lds + 48 + 4 * g);
     float pt[8];
 #pragma unroll
     for (int mt = 0; mt < 2; ++mt) {
@@ -352,21 +358,24 @@ struct DecodeTile {
     return __builtin_bit_cast(half8_t, pb);
   }
 
-  // Phase 2 of a tile: O^T += (V + 1152)^T . P~^T with an in-register 8 x VB byte transpose
-  // (one MFMA per 16-dim tile), and sum(P~) against a row of ones.  Consumes kv.v.
-  __device__ static void pv(const Tile& kv, half8_t p_op, State& st) {
+  // Phase 2 of a tile: O^T += (V + 1152)^T . P~^T.  Lane (r, g) reads bytes [r*VB, (r+1)*VB) of
+  // tokens 4g+j (j<4) and 16+4g+(j-4) from the LDS window, transposes the 8 x VB byte block in
+  // registers (byte permutes), one MFMA per 16-dim tile; sum(P~) comes from a row of ones.
+  __device__ static void pv(const LaneOffsets& lo, half8_t p_op, const uint8_t* lds, State& st) {
     {
       const half_t one = (half_t)1.0f;
       const half8_t ones = {one, one, one, one, one, one, one, one};
       st.psum = __builtin_amdgcn_mfma_f32_16x16x32_f16(ones, p_op, st.psum, 0, 0, 0);
     }
+    constexpr int VW = VB / 4;
 #pragma unroll
-    for (int w = 0; w < Tile::VW; ++w) {
+    for (int w = 0; w < VW; ++w) {
       uint32_t x0[4], x1[4];  // per token pair a: bytes (b0,b1) and (b2,b3) of both tokens, interleaved
 #pragma unroll
       for (int a = 0; a < 4; ++a) {
-        const uint32_t ta = kv.v[2 * a][w] ^ 0x80808080u;
-        const uint32_t tb = kv.v[2 * a + 1][w] ^ 0x80808080u;
+        const int ja = 2 * a, jb = 2 * a + 1;
+        const uint32_t ta = *reinterpret_cast<const uint32_t*>(lds + lo.l_v + ((ja & 3) + (ja >> 2) * 16) * PITCH + 4 * w) ^ 0x80808080u;
+        const uint32_t tb = *reinterpret_cast<const uint32_t*>(lds + lo.l_v + ((jb & 3) + (jb >> 2) * 16) * PITCH + 4 * w) ^ 0x80808080u;
         x0[a] = perm(tb, ta, 0x05010400u);
         x1[a] = perm(tb, ta, 0x07030602u);
       }
@@ -384,6 +393,18 @@ struct DecodeTile {
     }
   }
 
+  template <bool MASK>
+  __device__ static void compute(const LaneOffsets& lo, const half8_t (&qb)[KSTEPS], float s_init, int len, int t,
+                                 int lane, const uint8_t* lds, State& st) {
+    const half8_t p = qk_softmax<MASK>(lo, qb, s_init, len, t, lane, lds, st);
+    pv(lo, p, lds, st);
+  }
+  __device__ static void compute_any(const LaneOffsets& lo, const half8_t (&qb)[KSTEPS], float s_init, int len, int t,
+                                     int lane, const uint8_t* lds, State& st) {
+    if ((t + 1) * kTile > len) compute<true>(lo, qb, s_init, len, t, lane, lds, st);
+    else compute<false>(lo, qb, s_init, len, t, lane, lds, st);
+  }
+
   // Keeps the instruction scheduler from moving work across the phase boundaries of the
   // stream loop: a refill must be issued where it is written (right after the registers it
   // overwrites were consumed), and a tile's V conversion must not drift up into the QK phase,
@@ -391,11 +412,11 @@ struct DecodeTile {
   __device__ static __forceinline__ void phase_fence() { __builtin_amdgcn_sched_barrier(0); }
 
   // Run tiles [t_begin, t_end) of one sequence for kv head `hkv`; leaves the state in `st`.
-  // Two register buffers, refilled in halves: as soon as a tile's K codes (or V codes) have
-  // gone into the MFMA, the same registers take the K (or V) of the tile two ahead, so about
-  // two tiles of loads per wave are in flight at any time.
+  // Two register buffers: as soon as a tile has been dropped into LDS its registers take the
+  // tile two ahead, so two tiles of loads per wave are in flight while one is computed.
+  // `lds` is this wave's private LDS_WAVE-byte window.
   __device__ static void run(const AttnIO& io, int seq, int64_t row, int len, int t_begin, int t_end, int hkv,
-                             int lane, float* sc_lds, State& st) {
+                             int lane, uint8_t* lds, State& st) {
     half8_t qb[KSTEPS];
     const float s_init = load_q(io, row, hkv, lane, qb);
     const LaneOffsets lo = lane_offsets(io.g, lane);
@@ -414,85 +435,55 @@ struct DecodeTile {
     if (t + 3 < t_end) {
       // long run.  The prologue issues its loads in exactly the order of the steady state and
       // without conditions, so that inside the loop every wait is for the oldest loads only.
-      {
-        const Window w = window(io, ba, t, hkv);
-        load_k(w, lo, lane, a);
-        phase_fence();
-        load_v(io, w, lo, a);
-        phase_fence();
-        ba = fetch_blocks(io, bt_row, len, t + 2);
-      }
-      {
-        const Window w = window(io, bb, t + 1, hkv);
-        load_k(w, lo, lane, b);
-        phase_fence();
-        load_v(io, w, lo, b);
-        phase_fence();
-        bb = fetch_blocks(io, bt_row, len, t + 3);
-      }
+      load_tile(io, window(io, ba, t, hkv), lo, a);
+      phase_fence();
+      ba = fetch_blocks(io, bt_row, len, t + 2);
+      load_tile(io, window(io, bb, t + 1, hkv), lo, b);
+      phase_fence();
+      bb = fetch_blocks(io, bt_row, len, t + 3);
       // steady state: two tiles per trip; tiles t+2 and t+3 exist, so every load is
       // unconditional and none of the tiles computed here ends the sequence
       do {
         {
           const Window w = window(io, ba, t + 2, hkv);
-          const half8_t p = qk_softmax<false>(a, qb, s_init, sc_mul, len, t, lane, sc_lds, st);
+          stage(a, lo, sc_mul, lane, lds);
           phase_fence();
-          load_k(w, lo, lane, a);
-          phase_fence();
-          pv(a, p, st);
-          phase_fence();
-          load_v(io, w, lo, a);
+          load_tile(io, w, lo, a);
           phase_fence();
           ba = fetch_blocks(io, bt_row, len, t + 4);
+          compute<false>(lo, qb, s_init, len, t, lane, lds, st);
+          phase_fence();
         }
         {
           const Window w = window(io, bb, t + 3, hkv);
-          const half8_t p = qk_softmax<false>(b, qb, s_init, sc_mul, len, t + 1, lane, sc_lds, st);
+          stage(b, lo, sc_mul, lane, lds);
           phase_fence();
-          load_k(w, lo, lane, b);
-          phase_fence();
-          pv(b, p, st);
-          phase_fence();
-          load_v(io, w, lo, b);
+          load_tile(io, w, lo, b);
           phase_fence();
           bb = fetch_blocks(io, bt_row, len, t + 5);
+          compute<false>(lo, qb, s_init, len, t + 1, lane, lds, st);
+          phase_fence();
         }
         t += 2;
       } while (t + 3 < t_end);
     } else {
       // short run (at most three tiles)
-      {
-        const Window w = window(io, ba, t, hkv);
-        load_k(w, lo, lane, a);
-        load_v(io, w, lo, a);
-      }
+      load_tile(io, window(io, ba, t, hkv), lo, a);
       ba = fetch_blocks(io, bt_row, len, t + 2);
-      if (t + 1 < t_end) {
-        const Window w = window(io, bb, t + 1, hkv);
-        load_k(w, lo, lane, b);
-        load_v(io, w, lo, b);
-      }
+      if (t + 1 < t_end) load_tile(io, window(io, bb, t + 1, hkv), lo, b);
     }
     // tail: 1..3 tiles left; a holds t, b holds t+1 (if any); ba = blocks of t+2
     const int rem = t_end - t;
-    {
-      const bool more = rem >= 3;
-      const Window w = window(io, ba, t + 2, hkv);
-      const half8_t p = ((t + 1) * kTile > len) ? qk_softmax<true>(a, qb, s_init, sc_mul, len, t, lane, sc_lds, st)
-                                                : qk_softmax<false>(a, qb, s_init, sc_mul, len, t, lane, sc_lds, st);
-      if (more) load_k(w, lo, lane, a);
-      pv(a, p, st);
-      if (more) load_v(io, w, lo, a);
-    }
+    stage(a, lo, sc_mul, lane, lds);
+    if (rem >= 3) load_tile(io, window(io, ba, t + 2, hkv), lo, a);
+    compute_any(lo, qb, s_init, len, t, lane, lds, st);
     if (rem >= 2) {
-      const half8_t p = ((t + 2) * kTile > len) ? qk_softmax<true>(b, qb, s_init, sc_mul, len, t + 1, lane, sc_lds, st)
-                                                : qk_softmax<false>(b, qb, s_init, sc_mul, len, t + 1, lane, sc_lds, st);
-      pv(b, p, st);
+      stage(b, lo, sc_mul, lane, lds);
+      compute_any(lo, qb, s_init, len, t + 1, lane, lds, st);
     }
     if (rem >= 3) {
-      const half8_t p = ((t + 3) * kTile > len) ? qk_softmax<true>(a, qb, s_init, sc_mul, len, t + 2, lane, sc_lds, st)
-                                                : qk_softmax<false>(a, qb, s_init, sc_mul, len, t + 2, lane, sc_lds, st);
-      pv(a, p, st);
+      stage(a, lo, sc_mul, lane, lds);
+      compute_any(lo, qb, s_init, len, t + 2, lane, lds, st);
     }
   }
 

@@ -42,7 +42,7 @@ __device__ __forceinline__ int64_t wg_tile_begin(int w, int64_t total, int num_w
 template <int D, int QDT, int ODT, int WPW>
 __global__ __launch_bounds__(WPW * 64) void paged_decode_streamk_kernel(StreamKArgs a) {
   using DTile = DecodeTile<D, QDT, ODT>;
-  __shared__ __align__(16) float sc_lds[WPW][64];
+  __shared__ __align__(16) uint8_t lds[WPW][DTile::LDS_WAVE];
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int hkv = __builtin_amdgcn_readfirstlane(blockIdx.y * WPW + wave);
@@ -95,7 +95,7 @@ __global__ __launch_bounds__(WPW * 64) void paged_decode_streamk_kernel(StreamKA
     const int64_t rem = hi - seq_start;
     const int t_end = __builtin_amdgcn_readfirstlane(rem < ntiles ? (int)rem : ntiles);
     typename DTile::State st;
-    DTile::run(a.io, seq, row, len, t_begin, t_end, hkv, lane, sc_lds[wave], st);
+    DTile::run(a.io, seq, row, len, t_begin, t_end, hkv, lane, lds[wave], st);
     if (t_begin == 0 && t_end == ntiles) {
       DTile::emit_final(a.io, row, hkv, lane, st);
     } else {
@@ -177,7 +177,7 @@ struct V2Args {
 template <int D, int QDT, int WPW>
 __global__ __launch_bounds__(WPW * 64) void paged_decode_v2_kernel(V2Args a) {
   using DTile = DecodeTile<D, QDT, KVQ_F32>;
-  __shared__ __align__(16) float sc_lds[WPW][64];
+  __shared__ __align__(16) uint8_t lds[WPW][DTile::LDS_WAVE];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int hkv = __builtin_amdgcn_readfirstlane(blockIdx.z * WPW + wave);
   if (hkv >= a.io.g.num_kv_heads) return;
@@ -188,7 +188,7 @@ __global__ __launch_bounds__(WPW * 64) void paged_decode_v2_kernel(V2Args a) {
   if (t_begin >= ntiles) return;
   const int t_end = min(ntiles, t_begin + a.partition_tiles);
   typename DTile::State st;
-  DTile::run(a.io, seq, seq, len, t_begin, t_end, hkv, lane, sc_lds[wave], st);
+  DTile::run(a.io, seq, seq, len, t_begin, t_end, hkv, lane, lds[wave], st);
   DTile::emit_v2(a.io, a.tmp_out, a.max_logits, a.exp_sums, seq, part, a.max_parts, hkv, lane, st);
 }
 
