@@ -412,79 +412,44 @@ struct DecodeTile {
   __device__ static __forceinline__ void phase_fence() { __builtin_amdgcn_sched_barrier(0); }
 
   // Run tiles [t_begin, t_end) of one sequence for kv head `hkv`; leaves the state in `st`.
-  // Two register buffers: as soon as a tile has been dropped into LDS its registers take the
-  // tile two ahead, so two tiles of loads per wave are in flight while one is computed.
+  // One register buffer: as soon as a tile has been dropped into LDS its registers take the
+  // next tile, so one tile of loads per wave is in flight while one is computed (measured on
+  // MI355X: a second tile in flight per wave lowers the achieved HBM bandwidth).
   // `lds` is this wave's private LDS_WAVE-byte window.
   __device__ static void run(const AttnIO& io, int seq, int64_t row, int len, int t_begin, int t_end, int hkv,
                              int lane, uint8_t* lds, State& st) {
+    const LaneOffsets lo = lane_offsets(io.g, lane);
+    const int32_t* bt_row = io.block_table + (int64_t)seq * io.bt_stride;
+    Tile a;
+    int t = t_begin;
+    // the first tile's loads go out before anything else of the run is touched
+    TileBlocks nb = fetch_blocks(io, bt_row, len, t);
+    load_tile(io, window(io, nb, t, hkv), lo, a);
+    phase_fence();
+    nb = fetch_blocks(io, bt_row, len, t + 1);  // block ids run one tile ahead of the loads
     half8_t qb[KSTEPS];
     const float s_init = load_q(io, row, hkv, lane, qb);
-    const LaneOffsets lo = lane_offsets(io.g, lane);
     const float sc_mul = lane < 32 ? io.scale_log2 : kPScale;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) st.o[dt] = (floatx4){0.f, 0.f, 0.f, 0.f};
     st.psum = (floatx4){0.f, 0.f, 0.f, 0.f};
     st.m = -INFINITY;
     st.l = 0.f;
-    const int32_t* bt_row = io.block_table + (int64_t)seq * io.bt_stride;
-    Tile a, b;
-    int t = t_begin;
-    // block ids run ahead of the loads that use them (fetch_blocks clamps past the end)
-    TileBlocks ba = fetch_blocks(io, bt_row, len, t);
-    TileBlocks bb = fetch_blocks(io, bt_row, len, t + 1);
-    if (t + 3 < t_end) {
-      // long run.  The prologue issues its loads in exactly the order of the steady state and
-      // without conditions, so that inside the loop every wait is for the oldest loads only.
-      load_tile(io, window(io, ba, t, hkv), lo, a);
-      phase_fence();
-      ba = fetch_blocks(io, bt_row, len, t + 2);
-      load_tile(io, window(io, bb, t + 1, hkv), lo, b);
-      phase_fence();
-      bb = fetch_blocks(io, bt_row, len, t + 3);
-      // steady state: two tiles per trip; tiles t+2 and t+3 exist, so every load is
-      // unconditional and none of the tiles computed here ends the sequence
-      do {
-        {
-          const Window w = window(io, ba, t + 2, hkv);
-          stage(a, lo, sc_mul, lane, lds);
-          phase_fence();
-          load_tile(io, w, lo, a);
-          phase_fence();
-          ba = fetch_blocks(io, bt_row, len, t + 4);
-          compute<false>(lo, qb, s_init, len, t, lane, lds, st);
-          phase_fence();
-        }
-        {
-          const Window w = window(io, bb, t + 3, hkv);
-          stage(b, lo, sc_mul, lane, lds);
-          phase_fence();
-          load_tile(io, w, lo, b);
-          phase_fence();
-          bb = fetch_blocks(io, bt_row, len, t + 5);
-          compute<false>(lo, qb, s_init, len, t + 1, lane, lds, st);
-          phase_fence();
-        }
-        t += 2;
-      } while (t + 3 < t_end);
-    } else {
-      // short run (at most three tiles)
-      load_tile(io, window(io, ba, t, hkv), lo, a);
-      ba = fetch_blocks(io, bt_row, len, t + 2);
-      if (t + 1 < t_end) load_tile(io, window(io, bb, t + 1, hkv), lo, b);
-    }
-    // tail: 1..3 tiles left; a holds t, b holds t+1 (if any); ba = blocks of t+2
-    const int rem = t_end - t;
-    stage(a, lo, sc_mul, lane, lds);
-    if (rem >= 3) load_tile(io, window(io, ba, t + 2, hkv), lo, a);
-    compute_any(lo, qb, s_init, len, t, lane, lds, st);
-    if (rem >= 2) {
-      stage(b, lo, sc_mul, lane, lds);
-      compute_any(lo, qb, s_init, len, t + 1, lane, lds, st);
-    }
-    if (rem >= 3) {
+    // steady state: tile t+1 exists, so the refill is unconditional and tile t does not end the
+    // sequence
+    while (t + 1 < t_end) {
+      const Window w = window(io, nb, t + 1, hkv);
       stage(a, lo, sc_mul, lane, lds);
-      compute_any(lo, qb, s_init, len, t + 2, lane, lds, st);
+      phase_fence();
+      load_tile(io, w, lo, a);
+      phase_fence();
+      nb = fetch_blocks(io, bt_row, len, t + 2);
+      compute<false>(lo, qb, s_init, len, t, lane, lds, st);
+      phase_fence();
+      ++t;
     }
+    stage(a, lo, sc_mul, lane, lds);
+    compute_any(lo, qb, s_init, len, t, lane, lds, st);
   }
 
   // Sum of the lane-local l over the 4 lane groups of a head.
