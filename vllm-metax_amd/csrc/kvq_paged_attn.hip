@@ -40,6 +40,10 @@ extern "C" int kvq_paged_attn_int8(void* out, int out_dtype, int64_t out_stride_
   KVQ_REQUIRE((g.k_off | g.v_off | g.ks_off | g.vs_off | g.stride_block | g.stride_slot | g.stride_head) % 4 == 0 &&
                   ((uintptr_t)cache % 4) == 0,
               "%s: cache offsets/strides must be 4-byte aligned", op);
+  KVQ_REQUIRE(g.ks_off - g.k_off == g.head_size && g.v_off - g.k_off == g.head_size + 4 &&
+                  g.vs_off - g.k_off == 2 * g.head_size + 4,
+              "%s: a cache record must be [K codes | K scale | V codes | V scale]", op);
+  KVQ_REQUIRE(g.stride_slot > 0 && g.stride_slot <= 0x7fffffff / 64, "%s: stride_slot out of range", op);
   const int osz = out_dtype == KVQ_F32 ? 4 : 2;
   KVQ_REQUIRE(((uintptr_t)out % 4) == 0 && (out_stride_t * osz) % 4 == 0 && (out_stride_h * osz) % 4 == 0,
               "%s: out rows must be 4-byte aligned", op);

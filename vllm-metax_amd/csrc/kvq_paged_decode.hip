@@ -139,21 +139,34 @@ __global__ __launch_bounds__(256) void paged_decode_streamk_reduce_kernel(Stream
   const int w_last = (int)(((start + ntiles) * P - 1) / total);
   if (w_first == w_last) return;  // written directly by the main kernel
 
+  // pass 1: every lane takes one workgroup's (m, l); the wave agrees on the max and the weights
+  // pass 2: weighted sum of the partial outputs, all loads independent of each other
   float m = -INFINITY, l = 0.f, acc[V];
 #pragma unroll
   for (int i = 0; i < V; ++i) acc[i] = 0.f;
-  for (int w = w_first; w <= w_last; ++w) {
-    if (wg_tile_begin(w, total, P) >= wg_tile_begin(w + 1, total, P)) continue;  // empty workgroup
+  for (int wb = w_first; wb <= w_last; wb += kWave) {
+    const int w = wb + lane;
+    const bool live = w <= w_last && wg_tile_begin(w, total, P) < wg_tile_begin(w + 1, total, P);
     const int64_t slot = (int64_t)w + seq;
-    const float mj = a.part_ml[(slot * a.io.num_q_heads + head) * 2 + 0];
-    const float lj = a.part_ml[(slot * a.io.num_q_heads + head) * 2 + 1];
-    const float m_new = fmaxf(m, mj);
-    const float ca = __builtin_amdgcn_exp2f(m - m_new), cb = __builtin_amdgcn_exp2f(mj - m_new);
-    const float* po = a.part_o + (slot * a.io.num_q_heads + head) * (int64_t)D + lane * V;
-    l = l * ca + lj * cb;
+    const float mj = live ? a.part_ml[(slot * a.io.num_q_heads + head) * 2 + 0] : -INFINITY;
+    const float lj = live ? a.part_ml[(slot * a.io.num_q_heads + head) * 2 + 1] : 0.f;
+    const float m_new = fmaxf(m, wave_max(mj));
+    const float ca = __builtin_amdgcn_exp2f(m - m_new);  // first chunk: exp2(-inf) = 0
+    const float ej = __builtin_amdgcn_exp2f(mj - m_new);  // dead lanes: exp2(-inf) = 0
+    l = l * ca + wave_sum(lj * ej);
 #pragma unroll
-    for (int i = 0; i < V; ++i) acc[i] = acc[i] * ca + po[i] * cb;
+    for (int i = 0; i < V; ++i) acc[i] *= ca;
     m = m_new;
+    const uint64_t mask = __builtin_amdgcn_ballot_w64(live);
+    const int count = min(kWave, w_last - wb + 1);
+#pragma unroll 4
+    for (int k = 0; k < count; ++k) {
+      if (!((mask >> k) & 1)) continue;
+      const float wk = __shfl(ej, k, kWave);  // the partial outputs are unnormalised sums
+      const float* po = a.part_o + (((int64_t)(wb + k) + seq) * a.io.num_q_heads + head) * (int64_t)D + lane * V;
+#pragma unroll
+      for (int i = 0; i < V; ++i) acc[i] += po[i] * wk;
+    }
   }
   const float inv = 1.0f / l;
 #pragma unroll
@@ -260,6 +273,10 @@ static int validate_common(const char* op, const void* q, const void* cache, con
   KVQ_REQUIRE((g.k_off | g.v_off | g.ks_off | g.vs_off | g.stride_block | g.stride_slot | g.stride_head) % 4 == 0 &&
                   ((uintptr_t)cache % 4) == 0,
               "%s: cache offsets/strides must be 4-byte aligned", op);
+  KVQ_REQUIRE(g.ks_off - g.k_off == g.head_size && g.v_off - g.k_off == g.head_size + 4 &&
+                  g.vs_off - g.k_off == 2 * g.head_size + 4,
+              "%s: a cache record must be [K codes | K scale | V codes | V scale]", op);
+  KVQ_REQUIRE(g.stride_slot > 0 && g.stride_slot <= 0x7fffffff / 64, "%s: stride_slot out of range", op);
   return KVQ_OK;
 }
 
