@@ -79,6 +79,16 @@ def test_head_and_block_shapes(gpu_device, hq, hkv, d, bs):
     T.assert_close_attn(got, want, what=f"hq={hq} hkv={hkv} d={d} bs={bs}")
 
 
+@pytest.mark.parametrize("q_dtype", [torch.float16, torch.float32])
+def test_query_dtypes(gpu_device, q_dtype):
+    ctx = [130, 700]
+    kv, lay, bt, q, sl, cu = build_case(ctx, 32, 8, 128, 16, "NHD", 21, q_dtype=q_dtype)
+    scale = 128 ** -0.5
+    want = oracle.paged_attn(q, T.storage_bytes(kv), lay, bt, sl, cu, scale)
+    got = run_unified(gpu_device, kv, "NHD", bt, q, sl, cu, scale, out_dtype=q_dtype)
+    T.assert_close_attn(got, want, atol=5e-3, rtol=5e-3, what=f"q dtype {q_dtype}")
+
+
 def test_outlier_heavy_sources_and_peaked_softmax(gpu_device):
     """1 % of channels x20 (stresses the scales) and a large |q| (nearly one-hot softmax)."""
     ctx = [3000, 513]

@@ -1,0 +1,95 @@
+"""GPU parity of the LSE merge kernel and of the MLA latent quantise-on-write, through the C ABI."""
+import pytest
+import torch
+
+import kvq_testlib as T
+import oracle
+from vllm_metax_amd import _custom_ops as ops
+from vllm_metax_amd import layout as L
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("tokens,heads,d", [(613, 8, 128), (37, 5, 64), (256, 16, 512)])
+def test_merge_attn_states(gpu_device, dtype, tokens, heads, d):
+    dev = gpu_device
+    g = torch.Generator().manual_seed(tokens + heads)
+    po = torch.randn((tokens, heads, d), generator=g).to(dtype)
+    so = torch.randn((tokens, heads, d), generator=g).to(dtype)
+    pl = torch.randn((heads, tokens), generator=g) * 5
+    sl = torch.randn((heads, tokens), generator=g) * 5
+    sel = torch.rand((heads, tokens), generator=g)
+    pl[sel < 0.05] = float("inf")                      # the reference's test injects +inf LSEs
+    sl[(sel > 0.05) & (sel < 0.10)] = float("inf")
+    pl[(sel > 0.10) & (sel < 0.12)] = float("-inf")
+    both = (sel > 0.12) & (sel < 0.14)
+    pl[both] = float("-inf")
+    sl[both] = float("-inf")
+    want, want_lse = oracle.merge_attn_states(po, pl, so, sl)
+    out = torch.empty_like(po, device=dev)
+    lse = torch.empty((heads, tokens), dtype=torch.float32, device=dev)
+    ops.merge_attn_states(out, po.to(dev), pl.to(dev), so.to(dev), sl.to(dev), output_lse=lse)
+    torch.cuda.synchronize()
+    tol = dict(atol=1e-5, rtol=1e-5) if dtype == torch.float32 else dict(atol=1e-3, rtol=1e-2)
+    torch.testing.assert_close(out.float().cpu(), want, **tol)
+    torch.testing.assert_close(lse.cpu(), want_lse, atol=1e-5, rtol=1e-5)
+    # rows at or beyond the prefix count copy the suffix bit for bit
+    out2 = torch.empty_like(po, device=dev)
+    ops.merge_attn_states(out2, po.to(dev), pl.to(dev), so.to(dev), sl.to(dev), prefill_tokens_with_context=10)
+    torch.cuda.synchronize()
+    assert torch.equal(out2[10:].cpu(), so[10:]) and torch.equal(out2[:10].cpu(), out[:10].cpu())
+
+
+def test_merge_is_the_splitk_algebra(gpu_device):
+    """Merging the two halves of a context reproduces attention over the whole context."""
+    dev = gpu_device
+    g = torch.Generator().manual_seed(3)
+    Tn, H, D, n = 5, 4, 64, 200
+    q = torch.randn((Tn, H, D), generator=g)
+    k = torch.randn((n, H, D), generator=g)
+    v = torch.randn((n, H, D), generator=g)
+    def attend(ks, vs):
+        s = torch.einsum("thd,nhd->htn", q, ks) * 0.125
+        return torch.einsum("htn,nhd->thd", torch.softmax(s, -1), vs).contiguous(), torch.logsumexp(s, -1).contiguous()
+    o1, l1 = attend(k[:77], v[:77])
+    o2, l2 = attend(k[77:], v[77:])
+    full, lf = attend(k, v)
+    out = torch.empty((Tn, H, D), device=dev)
+    lse = torch.empty((H, Tn), device=dev)
+    ops.merge_attn_states(out, o1.to(dev), l1.contiguous().to(dev), o2.to(dev), l2.contiguous().to(dev), output_lse=lse)
+    torch.testing.assert_close(out.cpu(), full, atol=1e-5, rtol=1e-5)
+    torch.testing.assert_close(lse.cpu(), lf, atol=1e-5, rtol=1e-5)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.float16])
+@pytest.mark.parametrize("bs", [16, 64])
+def test_mla_cache_write_bit_exact(gpu_device, dtype, bs):
+    dev = gpu_device
+    R, P, nb, Tn = 512, 64, 9, 150
+    g = torch.Generator().manual_seed(bs)
+    kv_c = torch.randn((Tn + 3, R), generator=g).to(dtype)
+    k_pe = (torch.randn((Tn + 3, P), generator=g) * 4).to(dtype)
+    kv_c[7] = 0
+    k_pe[7] = 0                                                # an all-zero row
+    slots = torch.randperm(nb * bs, generator=g)[:Tn].to(torch.int64)
+    slots[::17] = -1
+    cpu = L.allocate_mla_cache(nb, bs, R + P, device="cpu", fill=0x33)
+    codes, scales = L.mla_cache_views(cpu)
+    lay = oracle.MlaLayout.from_views(cpu, codes, scales, R)
+    oracle.mla_cache_write(kv_c, k_pe, cpu, lay, slots)
+    gpu = L.allocate_mla_cache(nb, bs, R + P, device=dev, fill=0x33)
+    ops.concat_and_cache_mla(kv_c.to(dev), k_pe.to(dev), gpu, slots.to(dev))
+    torch.cuda.synchronize()
+    assert torch.equal(gpu.cpu(), cpu), "latent cache bytes differ from the oracle"
+
+
+def test_mla_write_errors(gpu_device):
+    dev = gpu_device
+    cache = L.allocate_mla_cache(2, 16, 576, device=dev)
+    kv_c = torch.zeros((4, 512), device=dev, dtype=torch.bfloat16)
+    k_pe = torch.zeros((4, 64), device=dev, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError):
+        ops.concat_and_cache_mla(kv_c, k_pe[:, :32], cache, torch.zeros(4, device=dev, dtype=torch.int64))
+    with pytest.raises(NotImplementedError):
+        ops.concat_and_cache_mla(kv_c, k_pe, cache, torch.zeros(4, device=dev, dtype=torch.int64), kv_cache_dtype="fp8")

@@ -185,10 +185,11 @@ struct DecodeTile {
 #pragma unroll
           for (int w = 0; w < 4; ++w) {
             if constexpr (QDT == KVQ_BF16) {
-              f[ch * 16 + i + 2 * w] = __builtin_bit_cast(float, v[w] << 16);
-              f[ch * 16 + i + 2 * w + 1] = __builtin_bit_cast(float, v[w] & 0xffff0000u);
+              f[ch * 16 + i + 2 * w] = as_f32(v[w] << 16);
+              f[ch * 16 + i + 2 * w + 1] = as_f32(v[w] & 0xffff0000u);
             } else {
-              const half2_t h = __builtin_bit_cast(half2_t, v[w]);
+              const uint32_t e = v[w];  // copy the element out first: bit_cast must not see a vector element lvalue
+              const half2_t h = __builtin_bit_cast(half2_t, e);
               f[ch * 16 + i + 2 * w] = (float)h.x;
               f[ch * 16 + i + 2 * w + 1] = (float)h.y;
             }

@@ -34,6 +34,12 @@ typedef float floatx4_a4 __attribute__((ext_vector_type(4), aligned(4)));
 
 constexpr int kWave = 64;
 
+// Bit reinterpretation through by-value scalars.  __builtin_bit_cast applied directly to a
+// vector ELEMENT expression (v.y, v[i]) reads element 0 of the vector on this compiler, so
+// elements are always copied into a scalar parameter first.
+__device__ __forceinline__ float as_f32(uint32_t u) { return __builtin_bit_cast(float, u); }
+__device__ __forceinline__ uint32_t as_u32(float f) { return __builtin_bit_cast(uint32_t, f); }
+
 __device__ __forceinline__ float bf16_bits_to_f32(uint16_t b) {
   return __builtin_bit_cast(float, (uint32_t)b << 16);
 }

@@ -1,23 +1,84 @@
-// MLA latent cache: int8 quantise-on-write and decode (placeholder until the kernels land).
+// MLA latent cache, int8 codes with one fp32 scale per token: quantise-on-write (gfx950).
+//
+// One wavefront owns one token: the kv_c row (kv_lora_rank wide) and the k_pe row (rope_dim
+// wide) are read once with lane-strided coalesced loads, their joint absmax is reduced across
+// the 64 lanes, and the concatenated row is written as int8 codes into the block's row region,
+// the scale into the block's scale region.  Same arithmetic as the per-(token, head) writer:
+// scale = max(absmax, eps) / 127 (IEEE division), code = clamp(rint(x / scale), -128, 127).
 #include "kvq_internal.h"
 
-extern "C" {
+namespace kvq {
 
-int kvq_concat_and_cache_mla_int8(const void*, const void*, int, int64_t, int64_t, void*, const kvq_mla_geom*,
-                                  const int64_t*, int64_t, float, kvq_stream_t) {
-  return kvq::fail(KVQ_ENOSYS, "concat_and_cache_mla_int8: not built yet");
+template <int DT>
+__global__ __launch_bounds__(256) void mla_quant_write_kernel(const void* __restrict__ kv_c,
+                                                              const void* __restrict__ k_pe, int64_t kv_c_stride,
+                                                              int64_t k_pe_stride, uint8_t* __restrict__ cache,
+                                                              kvq_mla_geom g, const int64_t* __restrict__ slot_mapping,
+                                                              int64_t num_tokens, float eps) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int64_t t = (int64_t)blockIdx.x * (blockDim.x / kWave) + (threadIdx.x / kWave);
+  if (t >= num_tokens) return;
+  const int64_t slot = slot_mapping[t];
+  if (slot < 0) return;  // padding token
+  const int64_t blk = slot / g.block_size;
+  const int64_t off = slot - blk * g.block_size;
+  const int R = g.kv_lora_rank, W = g.kv_lora_rank + g.rope_dim;
+  constexpr int kMaxPerLane = 16;  // rows up to 1024 wide stay in registers
+  float x[kMaxPerLane];
+  float amax = 0.f;
+#pragma unroll
+  for (int i = 0; i < kMaxPerLane; ++i) {
+    const int d = lane + kWave * i;
+    x[i] = 0.f;
+    if (d < W) x[i] = d < R ? load_act<DT>(kv_c, t * kv_c_stride + d) : load_act<DT>(k_pe, t * k_pe_stride + (d - R));
+    amax = fmaxf(amax, fabsf(x[i]));
+  }
+  amax = fmaxf(wave_max(amax), eps);
+  const float scale = amax / 127.0f;
+  int8_t* row = reinterpret_cast<int8_t*>(cache + blk * g.stride_block + off * g.stride_row);
+#pragma unroll
+  for (int i = 0; i < kMaxPerLane; ++i) {
+    const int d = lane + kWave * i;
+    if (d < W) {
+      float r = scale > 0.f ? rintf(x[i] / scale) : 0.f;
+      r = fminf(fmaxf(r, -128.f), 127.f);
+      row[d] = (int8_t)(int)r;
+    }
+  }
+  if (lane == 0) *reinterpret_cast<float*>(cache + blk * g.stride_block + g.scale_off + off * 4) = scale;
 }
 
-size_t kvq_mla_decode_workspace_bytes(int, int, int) { return 0; }
+}  // namespace kvq
 
-int kvq_mla_decode_int8(void*, int, float*, const void*, int, int64_t, int64_t, const void*, const kvq_mla_geom*,
-                        const int32_t*, int64_t, const int32_t*, int, int, float, void*, size_t, kvq_stream_t) {
-  return kvq::fail(KVQ_ENOSYS, "mla_decode_int8: not built yet");
+extern "C" int kvq_concat_and_cache_mla_int8(const void* kv_c, const void* k_pe, int src_dtype,
+                                             int64_t kv_c_stride, int64_t k_pe_stride, void* cache,
+                                             const kvq_mla_geom* geom, const int64_t* slot_mapping,
+                                             int64_t num_tokens, float eps, kvq_stream_t stream) {
+  using namespace kvq;
+  const char* op = "concat_and_cache_mla_int8";
+  KVQ_REQUIRE(geom != nullptr, "%s: geom is NULL", op);
+  KVQ_REQUIRE(num_tokens >= 0, "%s: negative num_tokens", op);
+  if (num_tokens == 0) return KVQ_OK;
+  KVQ_REQUIRE(kv_c && k_pe && cache && slot_mapping, "%s: NULL pointer", op);
+  const kvq_mla_geom& g = *geom;
+  KVQ_REQUIRE(g.kv_lora_rank > 0 && g.rope_dim >= 0 && g.block_size > 0, "%s: bad geometry", op);
+  KVQ_REQUIRE(g.kv_lora_rank + g.rope_dim <= 1024, "%s: rows wider than 1024 are not supported", op);
+  KVQ_REQUIRE((g.stride_block | g.scale_off) % 4 == 0 && ((uintptr_t)cache % 4) == 0,
+              "%s: block stride / scale offset must be 4-byte aligned", op);
+  KVQ_REQUIRE(eps >= 0.f, "%s: eps must not be negative", op);
+  const int64_t blocks = (num_tokens + 3) / 4;
+  KVQ_REQUIRE(blocks <= 0x7fffffffLL, "%s: too many tokens", op);
+  hipStream_t s = as_stream(stream);
+  uint8_t* c = static_cast<uint8_t*>(cache);
+#define KVQ_MLAW(T)                                                                                       \
+  hipLaunchKernelGGL((mla_quant_write_kernel<T>), dim3((unsigned)blocks), dim3(256), 0, s, kv_c, k_pe, \
+                     kv_c_stride, k_pe_stride, c, g, slot_mapping, num_tokens, eps)
+  switch (src_dtype) {
+    case KVQ_F32: KVQ_MLAW(KVQ_F32); break;
+    case KVQ_BF16: KVQ_MLAW(KVQ_BF16); break;
+    case KVQ_F16: KVQ_MLAW(KVQ_F16); break;
+    default: return fail(KVQ_EINVAL, "%s: unknown src_dtype %d", op, src_dtype);
+  }
+#undef KVQ_MLAW
+  return check_hip(hipGetLastError(), "concat_and_cache_mla_int8 launch");
 }
-
-int kvq_merge_attn_states(void*, float*, const void*, const float*, const void*, const float*, int, int64_t, int,
-                          int, int64_t, kvq_stream_t) {
-  return kvq::fail(KVQ_ENOSYS, "merge_attn_states: not built yet");
-}
-
-}  // extern "C"
