@@ -1,0 +1,126 @@
+"""Host-side logic of the backend mirror: capability flags, cache geometry, selection, error
+behaviour, and that the C-ABI library loads and exports every symbol include/kvq.h declares.
+No GPU needed."""
+import os
+import re
+import types
+
+import pytest
+import torch
+
+from vllm_metax_amd import _C, platform as P
+from vllm_metax_amd.kv_cache_interface import KVQuantMode, get_kv_quant_mode, kv_cache_uses_per_token_head_scales
+from vllm_metax_amd.v1.attention.backends.int8_attn import (
+    AttentionType, Int8AttentionBackend, Int8AttentionImpl, Int8AttentionMetadataBuilder, MultipleOf)
+from vllm_metax_amd.v1.attention.backends.mla.int8_mla import Int8MLABackend, Int8MLAImpl, _compute_num_kv_splits
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_library_exports_every_declared_symbol():
+    header = open(os.path.join(ROOT, "include", "kvq.h")).read()
+    declared = set(re.findall(r"KVQ_API\s+[\w\s\*]+?\b(kvq_\w+)\s*\(", header))
+    assert declared == set(_C.SIGNATURES), declared ^ set(_C.SIGNATURES)
+    lib = _C.load()                                   # raises if a symbol is missing
+    assert lib.kvq_abi_version() == _C.ABI_VERSION
+    for name in declared:
+        assert hasattr(lib, name)
+
+
+def test_quant_modes():
+    assert get_kv_quant_mode("int8_per_token_head") == KVQuantMode.INT8_PER_TOKEN_HEAD
+    assert kv_cache_uses_per_token_head_scales("int8_per_token_head")
+    assert not kv_cache_uses_per_token_head_scales("auto")
+    with pytest.raises(ValueError):
+        get_kv_quant_mode("int3")
+
+
+def test_backend_statics_match_the_reference_surface():
+    B = Int8AttentionBackend
+    assert B.get_name() == "TRITON_ATTN" and B.forward_includes_kv_cache_update is False
+    assert "int8_per_token_head" in B.supported_kv_cache_dtypes
+    assert B.get_supported_kernel_block_sizes() == [MultipleOf(16)]
+    assert B.supports_block_size(None) and B.supports_block_size(48) and not B.supports_block_size(24)
+    assert B.get_kv_cache_shape(40000, 16, 8, 128, "int8_per_token_head") == (40000, 8, 16, 264)
+    with pytest.raises(ValueError):
+        B.get_kv_cache_shape(10, 8, 8, 128)
+    os.environ.pop("VLLM_KV_CACHE_LAYOUT", None)
+    assert B.get_kv_cache_stride_order() == (0, 2, 1, 3)
+    os.environ["VLLM_KV_CACHE_LAYOUT"] = "HND"
+    try:
+        assert B.get_kv_cache_stride_order() == (0, 1, 2, 3)
+        assert B.get_kv_cache_stride_order(include_num_layers_dimension=True) == (1, 2, 0, 3, 4)
+    finally:
+        os.environ.pop("VLLM_KV_CACHE_LAYOUT")
+    assert B.use_cascade_attention() is False
+    assert B.get_impl_cls() is Int8AttentionImpl and B.get_builder_cls() is Int8AttentionMetadataBuilder
+    M = Int8MLABackend
+    assert M.get_name() == "TRITON_MLA"
+    assert M.get_kv_cache_shape(100, 64, 1, 576) == (100, 64, 580)
+    assert M.get_kv_cache_stride_order() == (0, 1, 2) and M.get_kv_cache_stride_order(True) == (1, 0, 2, 3)
+
+
+def test_selection_and_reasons():
+    ok = dict(kv_cache_dtype="int8_per_token_head", head_size=128, dtype=torch.bfloat16, block_size=16)
+    assert P.get_attn_backend_cls(**ok) == P.INT8_ATTN_PATH
+    assert P.get_attn_backend_cls("TRITON_ATTN", **ok) == P.INT8_ATTN_PATH
+    assert P.get_attn_backend_cls(use_mla=True, kv_cache_dtype="int8_per_token", dtype=torch.bfloat16,
+                                  block_size=64) == P.INT8_MLA_PATH
+    assert Int8AttentionBackend.validate_configuration(**ok) == []
+    assert Int8AttentionBackend.validate_configuration(**{**ok, "kv_cache_dtype": "fp8"}) == ["kv_cache_dtype not supported"]
+    assert Int8AttentionBackend.validate_configuration(**{**ok, "block_size": 24}) == ["block_size not supported"]
+    with pytest.raises(ValueError, match="not valid for this configuration"):
+        P.get_attn_backend_cls("TRITON_ATTN", **{**ok, "head_size": 80})
+    with pytest.raises(ValueError, match="No valid attention backend"):
+        P.get_attn_backend_cls(**{**ok, "kv_cache_dtype": "auto"})
+    with pytest.raises(ValueError):
+        P.get_attn_backend_cls("FLASH_ATTN", **ok)
+    P.register_attention_backends()                    # no upstream vLLM here: must be a no-op
+
+
+def test_impl_constructor_errors():
+    mk = lambda **kw: Int8AttentionImpl(32, 128, 0.088, 8, **kw)
+    impl = mk()
+    assert impl.num_queries_per_kv == 4 and impl.fused_rope_kvcache_supported() is False
+    for kw in (dict(alibi_slopes=[1.0] * 32), dict(sliding_window=128), dict(logits_soft_cap=30.0),
+               dict(sinks=torch.zeros(32)), dict(attn_type=AttentionType.ENCODER_ONLY)):
+        with pytest.raises(NotImplementedError):
+            mk(**kw)
+    with pytest.raises(ValueError):
+        mk(kv_cache_dtype="auto")
+    with pytest.raises(NotImplementedError):
+        impl.do_rope_and_kv_cache_update()
+    out = torch.ones(3, 32 * 128)
+    assert impl.forward(None, None, None, None, None, None, out) is out and bool((out == 0).all())   # profiling run
+    with pytest.raises(NotImplementedError):
+        impl.forward(None, None, None, None, None, types.SimpleNamespace(), out, output_scale=torch.ones(1))
+    with pytest.raises(NotImplementedError):
+        Int8MLAImpl(128, 576, 0.07, sliding_window=4)
+    with pytest.raises(ValueError):
+        Int8MLAImpl(128, 576, 0.07, kv_cache_dtype="fp8")
+
+
+def test_num_kv_splits_policy():
+    assert _compute_num_kv_splits(4096, 256) == 8
+    assert _compute_num_kv_splits(100, 256) == 1
+    assert _compute_num_kv_splits(1 << 20, 4) == 8
+    assert _compute_num_kv_splits(5000, 256) == 16
+
+
+def test_builder_packs_metadata_without_touching_the_gpu():
+    spec = types.SimpleNamespace(block_size=16, num_kv_heads=8, head_size=128, num_q_heads=32)
+    cfg = types.SimpleNamespace(scheduler_config=types.SimpleNamespace(max_num_seqs=4))
+    b = Int8AttentionMetadataBuilder(spec, ["l0"], cfg, "cpu")
+    c = types.SimpleNamespace(num_reqs=2, num_actual_tokens=2, max_query_len=1, max_seq_len=9,
+                              query_start_loc=torch.tensor([0, 1, 2], dtype=torch.int32),
+                              seq_lens=torch.tensor([9, 4], dtype=torch.int32),
+                              block_table_tensor=torch.zeros((2, 1), dtype=torch.int32),
+                              slot_mapping=torch.tensor([8, 19]), causal=True)
+    md = b.build(0, c)
+    assert md.num_actual_tokens == 2 and md.workspace is None and md.use_cascade is False
+    assert b.build_for_cudagraph_capture(c).seq_lens.tolist() == [1, 1]
+    with pytest.raises(NotImplementedError):
+        b.build(4, c)
+    c.num_reqs = 5
+    with pytest.raises(RuntimeError):
+        b.build(0, c)

@@ -1,0 +1,70 @@
+"""The backend mirror end to end on the GPU, the way the reference's backend tests drive an impl
+without a model runner (tests/v1/attention/test_attention_backends.py:74-183): hand-built paged
+cache and metadata, a mock layer, ``do_kv_cache_update`` then ``forward``, compared with the oracle
+run on the same tokens (the new tokens are quantised first and read back from the cache)."""
+import math
+import types
+
+import pytest
+import torch
+
+import kvq_testlib as T
+import oracle
+from vllm_metax_amd import layout as L
+from vllm_metax_amd.v1.attention.backends.int8_attn import Int8AttentionBackend
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("layout", ["NHD", "HND"])
+def test_decode_step_through_the_backend(gpu_device, layout, monkeypatch):
+    monkeypatch.setenv("VLLM_KV_CACHE_LAYOUT", layout)
+    dev = gpu_device
+    hq, hkv, d, bs, nb = 32, 8, 128, 16, 200
+    ctx = [257, 31, 1024, 5]                       # lengths INCLUDING this step's token
+    B = len(ctx)
+    g = torch.Generator().manual_seed(7)
+    shape = Int8AttentionBackend.get_kv_cache_shape(nb, bs, hkv, d, "int8_per_token_head")
+    order = Int8AttentionBackend.get_kv_cache_stride_order()
+    phys = torch.zeros(tuple(shape[i] for i in order), dtype=torch.int8, device=dev)
+    kv_cache = phys.permute(*[order.index(i) for i in range(4)])      # what the model runner hands over
+    kv_cpu, views, lay = T.cpu_cache(nb, bs, hkv, d, layout)
+    views[2].fill_(1.0)                            # the impl fills the scale views with 1.0 at first use
+    views[3].fill_(1.0)
+    bt = T.make_block_tables(ctx, bs, nb, g)
+    impl = Int8AttentionBackend.get_impl_cls()(hq, d, 1 / math.sqrt(d), hkv, kv_cache_dtype="int8_per_token_head")
+    spec = types.SimpleNamespace(block_size=bs, num_kv_heads=hkv, head_size=d, num_q_heads=hq)
+    cfg = types.SimpleNamespace(scheduler_config=types.SimpleNamespace(max_num_seqs=16))
+    builder = Int8AttentionBackend.get_builder_cls()(spec, ["layer.0"], cfg, dev)
+    layer = types.SimpleNamespace(_k_scale=torch.ones(1, device=dev), _v_scale=torch.ones(1, device=dev))
+    # prefill the context (all but the last token) through the backend's own cache update
+    slots = T.slots_for(bt, ctx, bs)
+    for i, c in enumerate(ctx):
+        if c > 1:
+            k = torch.randn((c - 1, hkv, d), generator=g).to(torch.bfloat16)
+            v = torch.randn((c - 1, hkv, d), generator=g).to(torch.bfloat16)
+            impl.do_kv_cache_update(layer, k.to(dev), v.to(dev), kv_cache, slots[i][:-1].to(dev))
+            oracle.cache_write(k, v, T.storage_bytes(kv_cpu), lay, slots[i][:-1])
+    # the decode step: one new token per sequence, padded batch (2 padding rows, slot -1)
+    pad = 2
+    k_new = torch.randn((B + pad, hkv, d), generator=g).to(torch.bfloat16)
+    v_new = torch.randn((B + pad, hkv, d), generator=g).to(torch.bfloat16)
+    q = torch.randn((B + pad, hq * d), generator=g).to(torch.bfloat16)
+    slot_new = torch.tensor([int(s[-1]) for s in slots] + [-1] * pad, dtype=torch.int64)
+    common = types.SimpleNamespace(
+        num_reqs=B, num_actual_tokens=B, max_query_len=1, max_seq_len=max(ctx),
+        query_start_loc=torch.arange(B + 1, dtype=torch.int32, device=dev),
+        seq_lens=torch.tensor(ctx, dtype=torch.int32, device=dev), block_table_tensor=bt.to(dev),
+        slot_mapping=slot_new.to(dev), causal=True)
+    md = builder.build(0, common)
+    impl.do_kv_cache_update(layer, k_new.to(dev), v_new.to(dev), kv_cache, md.slot_mapping)
+    out = torch.full((B + pad, hq * d), 7.0, dtype=torch.bfloat16, device=dev)
+    ret = impl.forward(layer, q.to(dev), k_new.to(dev), v_new.to(dev), kv_cache, md, out)
+    torch.cuda.synchronize()
+    assert ret is out and bool((out[B:] == 7.0).all()), "rows beyond num_actual_tokens must stay untouched"
+    oracle.cache_write(k_new, v_new, T.storage_bytes(kv_cpu), lay, slot_new)
+    assert torch.equal(T.storage_bytes(kv_cache).cpu(), T.storage_bytes(kv_cpu)), "cache bytes differ"
+    want = oracle.paged_attn(q[:B].view(B, hq, d), T.storage_bytes(kv_cpu), lay, bt,
+                             torch.tensor(ctx, dtype=torch.int32), torch.arange(B + 1, dtype=torch.int32),
+                             1 / math.sqrt(d))
+    T.assert_close_attn(out[:B].view(B, hq, d), want, what=f"backend decode {layout}")

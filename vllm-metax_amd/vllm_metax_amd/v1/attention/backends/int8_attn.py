@@ -1,0 +1,344 @@
+"""Attention backend for the int8 per-token-head KV cache on MI355X.
+
+Host-side mirror of the reference's TRITON_ATTN backend for this path
+(vllm_metax/v1/attention/backends/triton_attn.py): same class triple
+(Backend / MetadataBuilder / Impl), same method names, argument meaning and error behaviour,
+same cache tensor layout and scale views.  Where the reference calls upstream Triton kernels
+(:688-725, :805-814) this calls the HIP kernels through ``_custom_ops``.  The classes are
+duck-typed: they subclass upstream vLLM's base classes only when vLLM is importable, and read
+from ``vllm_config`` / ``kv_cache_spec`` only the attributes the reference reads.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import ClassVar
+
+import torch
+
+from .... import _custom_ops as ops
+from ....kv_cache_interface import KVQuantMode, get_kv_quant_mode, kv_cache_uses_per_token_head_scales
+from ....layout import (
+    geometry_from_views,
+    key_value_views,
+    kv_cache_shape,
+    kv_cache_stride_order,
+    scale_views,
+)
+
+try:  # pragma: no cover - upstream vLLM is not installed in the build container
+    from vllm.v1.attention.backend import (  # type: ignore
+        AttentionBackend as _BackendBase,
+        AttentionImpl as _ImplBase,
+        AttentionMetadataBuilder as _BuilderBase,
+        AttentionType,
+        MultipleOf,
+    )
+except Exception:  # noqa: BLE001
+    _BackendBase = object
+    _ImplBase = object
+    _BuilderBase = object
+
+    class AttentionType:
+        DECODER = "decoder"
+        ENCODER = "encoder"
+        ENCODER_ONLY = "encoder_only"
+        ENCODER_DECODER = "encoder_decoder"
+
+    @dataclass(frozen=True)
+    class MultipleOf:
+        base: int
+
+
+@dataclass
+class Int8AttentionMetadata:
+    """Fields of TritonAttentionMetadata that this path reads
+    (vllm_metax/v1/attention/backends/triton_attn.py:60-99), plus the pre-sized split-K workspace
+    that takes the place of the reference's softmax_segm_* scratch (:155-176)."""
+
+    num_actual_tokens: int
+    max_query_len: int
+    query_start_loc: torch.Tensor
+    max_seq_len: int
+    seq_lens: torch.Tensor
+    block_table: torch.Tensor
+    slot_mapping: torch.Tensor
+    workspace: torch.Tensor | None
+    causal: bool = True
+    use_cascade: bool = False
+    common_prefix_len: int = 0
+
+
+def _first_attr(obj, *names, default=None):
+    for n in names:
+        v = getattr(obj, n, None)
+        if v is not None:
+            return v
+    return default
+
+
+class Int8AttentionMetadataBuilder(_BuilderBase):
+    """Counterpart of TritonAttentionMetadataBuilder
+    (vllm_metax/v1/attention/backends/triton_attn.py:102-269): packs the common metadata and owns
+    the scratch that ``forward`` uses, sized once so a captured decode step never allocates."""
+
+    def __init__(self, kv_cache_spec, layer_names, vllm_config, device):
+        if _BuilderBase is not object:  # pragma: no cover
+            super().__init__(kv_cache_spec, layer_names, vllm_config, device)
+        self.kv_cache_spec = kv_cache_spec
+        self.layer_names = layer_names
+        self.vllm_config = vllm_config
+        self.device = torch.device(device)
+        self.block_size = kv_cache_spec.block_size
+        model_config = getattr(vllm_config, "model_config", None)
+        parallel_config = getattr(vllm_config, "parallel_config", None)
+        if model_config is not None and hasattr(model_config, "get_num_attention_heads"):
+            self.num_heads_q = model_config.get_num_attention_heads(parallel_config)
+            self.num_heads_kv = model_config.get_num_kv_heads(parallel_config)
+            self.headdim = model_config.get_head_size()
+        else:
+            self.num_heads_kv = kv_cache_spec.num_kv_heads
+            self.headdim = kv_cache_spec.head_size
+            self.num_heads_q = _first_attr(kv_cache_spec, "num_q_heads", "num_heads", default=self.num_heads_kv)
+        sched = getattr(vllm_config, "scheduler_config", None)
+        self.max_num_seqs = int(_first_attr(sched, "max_num_seqs", default=256)) if sched is not None else 256
+        self._workspace: torch.Tensor | None = None
+
+    def _get_workspace(self) -> torch.Tensor | None:
+        if self._workspace is None and self.device.type == "cuda":
+            nbytes = ops.paged_attn_workspace_bytes(self.max_num_seqs, self.num_heads_q, self.headdim)
+            self._workspace = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=self.device)
+        return self._workspace
+
+    def build_for_cudagraph_capture(self, common_attn_metadata) -> Int8AttentionMetadata:
+        md = self.build(0, common_attn_metadata)
+        # same trick as the reference (:184-194): capture with length-1 sequences
+        md.seq_lens.fill_(1)
+        return md
+
+    def build(self, common_prefix_len: int, common_attn_metadata, fast_build: bool = False) -> Int8AttentionMetadata:
+        if common_prefix_len > 0:
+            raise NotImplementedError("cascade attention is not supported (the reference disables it too)")
+        c = common_attn_metadata
+        if c.num_reqs > self.max_num_seqs:
+            raise RuntimeError(f"batch of {c.num_reqs} sequences exceeds max_num_seqs={self.max_num_seqs}")
+        return Int8AttentionMetadata(
+            num_actual_tokens=c.num_actual_tokens,
+            max_query_len=c.max_query_len,
+            query_start_loc=c.query_start_loc,
+            max_seq_len=c.max_seq_len,
+            seq_lens=c.seq_lens,
+            block_table=c.block_table_tensor,
+            slot_mapping=c.slot_mapping,
+            workspace=self._get_workspace(),
+            causal=bool(getattr(c, "causal", True)),
+        )
+
+
+class Int8AttentionBackend(_BackendBase):
+    """Capability flags and cache geometry, as MacaTritonAttentionBackend
+    (vllm_metax/v1/attention/backends/triton_attn.py:272-410)."""
+
+    supported_dtypes: ClassVar[list[torch.dtype]] = [torch.float16, torch.bfloat16, torch.float32]
+    supported_kv_cache_dtypes: ClassVar[list[str]] = ["int8_per_token_head"]
+    forward_includes_kv_cache_update: bool = False
+
+    @staticmethod
+    def get_name() -> str:
+        return "TRITON_ATTN"  # the registry slot this backend takes over
+
+    @staticmethod
+    def get_supported_kernel_block_sizes():
+        return [MultipleOf(16)]
+
+    @classmethod
+    def supports_block_size(cls, block_size: int | None) -> bool:
+        return block_size is None or block_size % 16 == 0
+
+    @classmethod
+    def supports_head_size(cls, head_size: int) -> bool:
+        return head_size in (64, 128, 256)
+
+    @classmethod
+    def supports_kv_cache_dtype(cls, kv_cache_dtype: str | None) -> bool:
+        return kv_cache_dtype in cls.supported_kv_cache_dtypes
+
+    @classmethod
+    def supports_dtype(cls, dtype: torch.dtype) -> bool:
+        return dtype in cls.supported_dtypes
+
+    @classmethod
+    def supports_attn_type(cls, attn_type: str) -> bool:
+        return attn_type == AttentionType.DECODER
+
+    @classmethod
+    def supports_non_causal(cls) -> bool:
+        return True
+
+    @classmethod
+    def supports_sliding_window(cls) -> bool:
+        return False
+
+    @classmethod
+    def supports_sink(cls) -> bool:
+        return False
+
+    @classmethod
+    def supports_batch_invariance(cls) -> bool:
+        return False  # the split depends on the batch's total length
+
+    @classmethod
+    def supports_compute_capability(cls, capability) -> bool:
+        return True
+
+    @classmethod
+    def validate_configuration(cls, head_size=None, dtype=None, kv_cache_dtype=None, block_size=None,
+                               use_mla=False, attn_type=AttentionType.DECODER, has_sink=False,
+                               use_sparse=False, **_ignored) -> list[str]:
+        """Reasons this backend cannot serve a configuration (empty list = valid); the selection
+        loop of the reference keeps the first backend with no reasons
+        (vllm_metax/platform.py:386-416, 418-514)."""
+        reasons = []
+        if use_mla:
+            reasons.append("MLA not supported")
+        if use_sparse:
+            reasons.append("sparse attention not supported")
+        if head_size is not None and not cls.supports_head_size(head_size):
+            reasons.append("head_size not supported")
+        if dtype is not None and not cls.supports_dtype(dtype):
+            reasons.append("dtype not supported")
+        if not cls.supports_kv_cache_dtype(kv_cache_dtype):
+            reasons.append("kv_cache_dtype not supported")
+        if not cls.supports_block_size(block_size):
+            reasons.append("block_size not supported")
+        if not cls.supports_attn_type(attn_type):
+            reasons.append("attention type not supported")
+        if has_sink:
+            reasons.append("sink setting not supported")
+        return reasons
+
+    @staticmethod
+    def get_impl_cls():
+        return Int8AttentionImpl
+
+    @staticmethod
+    def get_builder_cls():
+        return Int8AttentionMetadataBuilder
+
+    @staticmethod
+    def get_kv_cache_shape(num_blocks: int, block_size: int, num_kv_heads: int, head_size: int,
+                           cache_dtype_str: str = "int8_per_token_head") -> tuple[int, ...]:
+        return kv_cache_shape(num_blocks, block_size, num_kv_heads, head_size, cache_dtype_str)
+
+    @staticmethod
+    def get_kv_cache_stride_order(include_num_layers_dimension: bool = False) -> tuple[int, ...]:
+        return kv_cache_stride_order(include_num_layers_dimension)
+
+    @staticmethod
+    def use_cascade_attention(*args, **kwargs) -> bool:
+        return False
+
+
+class Int8AttentionImpl(_ImplBase):
+    """Counterpart of TritonAttentionImpl for the per-token-head int8 cache
+    (vllm_metax/v1/attention/backends/triton_attn.py:413-848)."""
+
+    def __init__(self, num_heads: int, head_size: int, scale: float, num_kv_heads: int,
+                 alibi_slopes: list[float] | None = None, sliding_window: int | None = None,
+                 kv_cache_dtype: str = "int8_per_token_head", logits_soft_cap: float | None = None,
+                 attn_type: str = AttentionType.DECODER, kv_sharing_target_layer_name: str | None = None,
+                 sinks: torch.Tensor | None = None, use_alibi_sqrt: bool = False, chunk_lookback: int = -1) -> None:
+        unsupported = {
+            "alibi_slopes": alibi_slopes is not None, "sliding_window": sliding_window is not None,
+            "logits_soft_cap": bool(logits_soft_cap), "sinks": sinks is not None,
+            "kv_sharing_target_layer_name": kv_sharing_target_layer_name is not None,
+            "chunk_lookback": chunk_lookback not in (-1, None),
+        }
+        bad = [k for k, v in unsupported.items() if v]
+        if bad:  # the way TritonMLAImpl refuses features it lacks (mla/triton_mla.py:177-190)
+            raise NotImplementedError(f"Int8AttentionImpl does not support: {', '.join(bad)}")
+        if attn_type != AttentionType.DECODER:
+            raise NotImplementedError("quantized KV cache is not supported for encoder attention")
+        if not kv_cache_uses_per_token_head_scales(kv_cache_dtype) or \
+                get_kv_quant_mode(kv_cache_dtype) != KVQuantMode.INT8_PER_TOKEN_HEAD:
+            raise ValueError(f"Int8AttentionImpl needs kv_cache_dtype 'int8_per_token_head', got {kv_cache_dtype!r}")
+        if num_heads % num_kv_heads:
+            raise ValueError("num_heads must be a multiple of num_kv_heads")
+        self.num_heads = num_heads
+        self.head_size = head_size
+        self.scale = float(scale)
+        self.num_kv_heads = num_kv_heads
+        self.num_queries_per_kv = num_heads // num_kv_heads
+        self.kv_cache_dtype = kv_cache_dtype
+        self.attn_type = attn_type
+        self.sliding_window = (-1, -1)
+        self.logits_soft_cap = 0
+        self._kv_quant_mode = get_kv_quant_mode(kv_cache_dtype)
+        self._is_per_token_head_quant = True
+        # per-cache views and byte geometry, built at first use (one cache tensor per layer)
+        self._views_for: int | None = None
+        self._key_cache = self._value_cache = None
+        self._k_scale_cache = self._v_scale_cache = None
+        self._geometry = None
+
+    def fused_output_quant_supported(self, quant_key) -> bool:
+        return False
+
+    def fused_rope_kvcache_supported(self) -> bool:
+        return False
+
+    # -- cache views ---------------------------------------------------------------------------
+    def _ensure_scale_caches(self, kv_cache: torch.Tensor) -> None:
+        """fp32 strided views over the inline scale bytes, filled with 1.0 at first use, as
+        vllm_metax/v1/attention/backends/triton_attn.py:418-479."""
+        key = (kv_cache.data_ptr(), tuple(kv_cache.shape), tuple(kv_cache.stride()))
+        if self._views_for == key:
+            return
+        self._k_scale_cache, self._v_scale_cache = scale_views(kv_cache)
+        self._k_scale_cache.fill_(1.0)
+        self._v_scale_cache.fill_(1.0)
+        self._key_cache, self._value_cache = key_value_views(kv_cache)
+        self._geometry = geometry_from_views(self._key_cache, self._value_cache, self._k_scale_cache,
+                                             self._v_scale_cache)
+        self._views_for = key
+
+    def _pth_key_value_caches(self, kv_cache: torch.Tensor):
+        """(nb, bs, Hkv, D+4) int8 views of the K and V halves (:729-739)."""
+        self._ensure_scale_caches(kv_cache)
+        return self._key_cache, self._value_cache
+
+    # -- the two per-layer calls ---------------------------------------------------------------
+    def do_kv_cache_update(self, layer, key: torch.Tensor, value: torch.Tensor, kv_cache: torch.Tensor,
+                           slot_mapping: torch.Tensor) -> None:
+        """Quantise-on-write of this step's tokens; mutates ``kv_cache`` in place (:788-815)."""
+        key_cache, value_cache = self._pth_key_value_caches(kv_cache)
+        ops.reshape_and_cache_flash_per_token_head_quant(
+            key, value, key_cache, value_cache, self._k_scale_cache, self._v_scale_cache, slot_mapping,
+            kv_quant_mode=self._kv_quant_mode, geometry=self._geometry)
+
+    def do_rope_and_kv_cache_update(self, *args, **kwargs):
+        raise NotImplementedError("fused rope + cache update is not built (the reference raises here too)")
+
+    def forward(self, layer, query: torch.Tensor, key: torch.Tensor, value: torch.Tensor, kv_cache: torch.Tensor,
+                attn_metadata: Int8AttentionMetadata | None, output: torch.Tensor,
+                output_scale: torch.Tensor | None = None, output_block_scale: torch.Tensor | None = None) -> torch.Tensor:
+        """Paged attention over the int8 cache (:577-727).  ``key`` / ``value`` are not read: this
+        step's tokens are read back from the cache, where ``do_kv_cache_update`` has put them.
+        Writes ``output[:num_actual_tokens]``; rows beyond stay untouched."""
+        if output_scale is not None or output_block_scale is not None:
+            raise NotImplementedError("fused output quantization is not supported")
+        if attn_metadata is None:  # profiling run
+            return output.fill_(0)
+        if attn_metadata.use_cascade:
+            raise NotImplementedError("cascade attention is not supported")
+        n = attn_metadata.num_actual_tokens
+        key_cache, value_cache = self._pth_key_value_caches(kv_cache)
+        q = query[:n].view(n, self.num_heads, self.head_size)
+        out = output[:n].view(n, self.num_heads, self.head_size)
+        ops.unified_attention(
+            q=q, k=key_cache, v=value_cache, out=out, cu_seqlens_q=attn_metadata.query_start_loc,
+            max_seqlen_q=attn_metadata.max_query_len, seqused_k=attn_metadata.seq_lens,
+            max_seqlen_k=attn_metadata.max_seq_len, softmax_scale=self.scale, causal=attn_metadata.causal,
+            window_size=self.sliding_window, block_table=attn_metadata.block_table, softcap=self.logits_soft_cap,
+            kv_quant_mode=self._kv_quant_mode, k_scale_cache=self._k_scale_cache, v_scale_cache=self._v_scale_cache,
+            workspace=attn_metadata.workspace, geometry=self._geometry)
+        return output
