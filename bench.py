@@ -28,6 +28,9 @@ sys.path.insert(0, ROOT)
 import torch  # noqa: E402
 
 HBM_PEAK_GBPS = 8000.0
+# HBM bytes per decode attention launch, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by a plain
+# read / copy kernel of known size (factors 2.000 and 1.000); summaries under profiles/.
+MEASURED_TRAFFIC = {"llama3_8b_decode_b64_ctx1k-8k": 752.3e6}
 METRIC = "int8-KV paged decode: achieved HBM GB/s (% peak), µs/layer @B=64 ctx=8k"
 
 
@@ -230,8 +233,8 @@ def main():
         "attn_launch_us": round(attn_ms * 1e3, 2),
         "write_launch_us": round(write_ms * 1e3, 2),
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
-                     "kernel": "paged decode attention launch (split-K main kernel + reduce)",
+                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": MEASURED_TRAFFIC.get(args.workload),
+                     "kernel": "paged decode attention launch = paged_decode_streamk_kernel + paged_decode_streamk_reduce_kernel",
                      "algorithmic_bytes_per_launch": attn_bytes},
     }
     if not args.no_cpu_baseline:
