@@ -1,0 +1,165 @@
+"""GPU parity of the MLA decode over the int8 latent cache, through the C ABI, against the oracle
+(fp32 + lse contract of the reference's tests/kernels/attention/test_mla_decode_cpu.py:14-41 on the
+dequantised latent rows)."""
+import os
+
+import pytest
+import torch
+
+import kvq_testlib as T
+import oracle
+from vllm_metax_amd import _custom_ops as ops
+from vllm_metax_amd import layout as L
+
+pytestmark = pytest.mark.gpu
+
+R, P = 512, 64
+GOLDEN = os.path.join(os.path.dirname(__file__), "golden", "kvq_golden_small.pt")
+
+
+def _build(ctx, bs, seed, dtype=torch.bfloat16, poison=True, amp=1.0):
+    """A latent cache written by the oracle for sequences of the given lengths, blocks shuffled."""
+    g = torch.Generator().manual_seed(seed)
+    B = len(ctx)
+    per = [(c + bs - 1) // bs for c in ctx]
+    nb = sum(per) + 3
+    order = torch.randperm(nb, generator=g).tolist()
+    cache = L.allocate_mla_cache(nb, bs, R + P, device="cpu", fill=-1 if poison else 0)  # all-ones bytes: unwritten scales read as NaN
+    codes, scales = L.mla_cache_views(cache)
+    lay = oracle.MlaLayout.from_views(cache, codes, scales, R)
+    bt = torch.zeros((B, max(max(per), 1)), dtype=torch.int32)
+    it = iter(order)
+    for i, c in enumerate(ctx):
+        blocks = [next(it) for _ in range(per[i])]
+        bt[i, : per[i]] = torch.tensor(blocks, dtype=torch.int32)
+        if c == 0:
+            continue
+        kv_c = (torch.randn((c, R), generator=g) * amp).to(dtype)
+        k_pe = (torch.randn((c, P), generator=g) * amp).to(dtype)
+        pos = torch.arange(c)
+        slots = (bt[i, pos // bs].long() * bs + pos % bs)
+        oracle.mla_cache_write(kv_c, k_pe, cache, lay, slots)
+    return cache, lay, bt, torch.tensor(ctx, dtype=torch.int32)
+
+
+def _run(q, cache, bt, sl, scale, out_dtype=None, want_lse=True):
+    dev = "cuda:0"
+    B, H, _ = q.shape
+    o = torch.full((B, H, R), float("nan"), dtype=out_dtype or q.dtype, device=dev)
+    lse = torch.full((B, H), float("nan"), dtype=torch.float32, device=dev) if want_lse else None
+    ops.mla_decode_int8(q.to(dev), cache.to(dev), o, lse, bt.to(dev), sl.to(dev), scale, R)
+    torch.cuda.synchronize()
+    return o, lse
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("bs,heads,ctx", [
+    (64, 128, [300, 1, 64, 2049]),
+    (16, 16, [17, 33, 511]),
+    (32, 128, [4096]),
+    (64, 20, [5, 0, 95, 1000, 31, 32]),
+])
+def test_mla_decode_matches_oracle(gpu_device, dtype, bs, heads, ctx):
+    cache, lay, bt, sl = _build(ctx, bs, seed=bs + heads, dtype=torch.bfloat16)
+    g = torch.Generator().manual_seed(7)
+    q = torch.randn((len(ctx), heads, R + P), generator=g).to(dtype)
+    scale = (128 + 64) ** -0.5
+    want, want_lse = oracle.mla_decode(q, cache, lay, bt, sl, scale)
+    got, lse = _run(q, cache, bt, sl, scale)
+    if dtype == torch.float32:
+        T.assert_close_attn(got, want, atol=4e-3, rtol=4e-3, what="mla decode fp32")   # fp16 operand rounding
+    else:
+        T.assert_close_attn(got, want, what="mla decode")
+    live = sl > 0
+    torch.testing.assert_close(lse.cpu()[live], want_lse[live], atol=5e-3, rtol=1e-3)
+    if (~live).any():
+        assert torch.equal(got.float().cpu()[~live], torch.zeros_like(want[~live]))
+        assert torch.isinf(lse.cpu()[~live]).all() and (lse.cpu()[~live] < 0).all()
+
+
+def test_mla_decode_peaked_softmax_and_large_values(gpu_device):
+    """Logits with a large spread (one dominant token) and latent rows with large magnitudes."""
+    ctx = [700, 129]
+    cache, lay, bt, sl = _build(ctx, 64, seed=11, amp=8.0)
+    g = torch.Generator().manual_seed(5)
+    q = (torch.randn((2, 128, R + P), generator=g) * 2).to(torch.bfloat16)
+    scale = 0.3
+    want, want_lse = oracle.mla_decode(q, cache, lay, bt, sl, scale)
+    got, lse = _run(q, cache, bt, sl, scale)
+    T.assert_close_attn(got, want, atol=2e-2 * 8, rtol=1e-2, what="mla decode, peaked")  # atol scaled with |V|
+    torch.testing.assert_close(lse.cpu(), want_lse, atol=5e-2, rtol=1e-3)
+
+
+def test_mla_decode_strided_q_and_no_lse(gpu_device):
+    ctx = [100, 260]
+    cache, lay, bt, sl = _build(ctx, 64, seed=3)
+    g = torch.Generator().manual_seed(9)
+    big = torch.randn((2, 16, 2 * (R + P)), generator=g).to(torch.bfloat16)
+    q = big[:, :, : R + P]                       # head stride 1152, last dim contiguous
+    want, _ = oracle.mla_decode(q, cache, lay, bt, sl, 0.07)
+    dev = gpu_device
+    o = torch.empty((2, 16, R), dtype=torch.bfloat16, device=dev)
+    ops.mla_decode_int8(big.to(dev)[:, :, : R + P], cache.to(dev), o, None, bt.to(dev), sl.to(dev), 0.07, R)
+    torch.cuda.synchronize()
+    T.assert_close_attn(o, want, what="mla decode, strided q")
+
+
+def test_mla_decode_golden(gpu_device):
+    G = torch.load(GOLDEN, weights_only=True)
+    cache = G["mla_cache"]
+    got, lse = _run(G["mla_q"], cache, G["mla_block_table"], G["mla_ctx"], 192 ** -0.5)
+    tol = dict(atol=4e-3, rtol=4e-3) if G["mla_q"].dtype == torch.float32 else {}
+    T.assert_close_attn(got, G["mla_out"], what="golden mla decode", **tol)
+    torch.testing.assert_close(lse.cpu(), G["mla_lse"], atol=5e-3, rtol=1e-3)
+
+
+def test_mla_backend_forward_mqa(gpu_device):
+    from types import SimpleNamespace
+
+    from vllm_metax_amd.v1.attention.backends.mla.int8_mla import Int8MLAImpl
+
+    dev = gpu_device
+    ctx = [77, 513]
+    bs = 64
+    g = torch.Generator().manual_seed(21)
+    H = 16
+    impl = Int8MLAImpl(num_heads=H, head_size=R + P, scale=0.0722, num_kv_heads=1, kv_cache_dtype="int8_per_token",
+                       kv_lora_rank=R, qk_rope_head_dim=P)
+    nb = 16
+    cache = L.allocate_mla_cache(nb, bs, R + P, device=dev)
+    cpu_cache = L.allocate_mla_cache(nb, bs, R + P, device="cpu")
+    codes, scales = L.mla_cache_views(cpu_cache)
+    lay = oracle.MlaLayout.from_views(cpu_cache, codes, scales, R)
+    bt = torch.tensor([[3, 1, 0, 0, 0, 0, 0, 0, 0], [2, 4, 5, 6, 7, 8, 9, 10, 11]], dtype=torch.int32)
+    for i, c in enumerate(ctx):
+        kv_c = torch.randn((c, R), generator=g).to(torch.bfloat16)
+        k_pe = torch.randn((c, 1, P), generator=g).to(torch.bfloat16)
+        pos = torch.arange(c)
+        slots = bt[i, pos // bs].long() * bs + pos % bs
+        impl.do_kv_cache_update(kv_c.to(dev), k_pe.to(dev), cache, slots.to(dev))
+        oracle.mla_cache_write(kv_c, k_pe.reshape(c, P), cpu_cache, lay, slots)
+    torch.cuda.synchronize()
+    assert torch.equal(cache.cpu(), cpu_cache)
+    ql = torch.randn((2, H, R), generator=g).to(torch.bfloat16)
+    qp = torch.randn((2, H, P), generator=g).to(torch.bfloat16)
+    md = SimpleNamespace(decode=SimpleNamespace(block_table=bt.to(dev), seq_lens=torch.tensor(ctx, dtype=torch.int32, device=dev)))
+    o, lse = impl.forward_mqa((ql.to(dev), qp.to(dev)), cache, md)
+    torch.cuda.synchronize()
+    want, want_lse = oracle.mla_decode(torch.cat([ql, qp], -1), cpu_cache, lay, bt, torch.tensor(ctx, dtype=torch.int32), 0.0722)
+    T.assert_close_attn(o, want, what="forward_mqa")
+    torch.testing.assert_close(lse.cpu(), want_lse, atol=5e-3, rtol=1e-3)
+
+
+def test_mla_decode_errors(gpu_device):
+    dev = gpu_device
+    cache = L.allocate_mla_cache(4, 64, R + P, device=dev)
+    q = torch.zeros((1, 8, R + P), dtype=torch.bfloat16, device=dev)
+    o = torch.empty((1, 8, R), dtype=torch.bfloat16, device=dev)
+    bt = torch.zeros((1, 4), dtype=torch.int32, device=dev)
+    sl = torch.tensor([10], dtype=torch.int32, device=dev)
+    with pytest.raises(RuntimeError):
+        ops.mla_decode_int8(q[:, :, :500], cache, o, None, bt, sl, 0.1, R)
+    with pytest.raises(RuntimeError):
+        ops.mla_decode_int8(q, cache, o, None, bt.long(), sl, 0.1, R)
+    with pytest.raises(RuntimeError):
+        ops.mla_decode_int8(q, cache, o, None, bt, sl, 0.1, R, workspace=torch.empty(16, dtype=torch.uint8, device=dev))

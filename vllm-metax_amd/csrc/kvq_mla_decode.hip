@@ -1,13 +1,424 @@
-// MLA decode over the int8 latent cache (placeholder until the MFMA tile lands).
-#include "kvq_internal.h"
+// MLA decode over the int8 latent cache (gfx950, wave64, MFMA 16x16x32 f16).
+//
+// All query heads of a sequence share ONE latent stream (576 int8 codes + one fp32 scale per
+// token), so this is a dense contraction: S^T[token, head] = C . Q^T over 576 dims and
+// O^T[dim, head] = C[:, :512]^T . P~^T, both on the MFMA with the heads as the N dimension.
+//
+// Work item = (sequence, token split); workgroup = 8 waves, wave w owns heads 16w .. 16w+15 of a
+// 128-head group and keeps their absorbed Q (18 k-steps) and their 512 x 16 output tile in
+// registers (a 32-head tile per wave would halve the dequantisation work per flop but needs
+// more than the 512 registers a lane can have).  The workgroup loads each 32-token tile once, as flat 16-byte chunks (every
+// quarter-wave reads 256 contiguous bytes), through registers into a double-buffered LDS window
+// (one barrier per tile); every wave then reads the int8 rows back in MFMA operand order and
+// turns codes into exact fp16 numbers code + 1152 with one byte permute per two codes -- the
+// constant is taken out again through the accumulator start value (QK) and a row of ones (PV).
+// The token splits of a sequence are merged by the reduce kernel with the log-sum-exp algebra
+// (same two-stage shape as the reference's decode_attention_fwd); nothing is allocated here,
+// partials live in the caller's workspace.
+#include "kvq_attn_core.cuh"
+
+namespace kvq {
+
+constexpr int kMlaR = 512, kMlaP = 64, kMlaW = kMlaR + kMlaP;
+constexpr int kMlaPitch = kMlaW + 16;                     // LDS row pitch: 16-byte aligned rows
+constexpr int kMlaTileBytes = kTile * kMlaPitch;          // 32 rows
+constexpr int kMlaBufBytes = kMlaTileBytes + 2 * kTile * 4;  // + 32 K-side and 32 V-side scales
+constexpr int kMlaKSteps = kMlaW / 32;                    // 18
+constexpr int kMlaDT = kMlaR / 16;                        // 32 output row tiles of 16 dims
+constexpr int kMlaVB = kMlaR / 16;                        // 32 V bytes per token per lane
+constexpr int kChunksPerRow = kMlaW / 16;                 // 36
+constexpr int kChunksPerHalf = 16 * kChunksPerRow;        // 576
+constexpr int kMlaThreads = 512;
+
+struct MlaArgs {
+  const void* q;
+  int64_t q_stride_b, q_stride_h;
+  const uint8_t* cache;
+  kvq_mla_geom g;
+  const int32_t* block_table;
+  int64_t bt_stride;
+  const int32_t* seq_lens;
+  float* part_o;    // [B, H, S, 512]
+  float* part_lse;  // [B, H, S] log2-domain lse of the split, -inf for an empty split
+  int num_heads;
+  int num_splits;
+  float scale_log2;
+  uint32_t bs_magic;
+};
+
+// tokens of a sequence per split, a whole number of tiles
+__device__ __forceinline__ int mla_split_len(int len, int num_splits) {
+  const int per = (len + num_splits - 1) / num_splits;
+  return ((per + kTile - 1) / kTile) * kTile;
+}
+
+template <int QDT>
+__global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
+  __shared__ __align__(16) uint8_t lds[2][kMlaBufBytes];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int c = lane & 15, g = lane >> 4;
+  const int seq = blockIdx.y, split = blockIdx.x;
+  const int hbase = blockIdx.z * 128 + wave * 16;
+  const int len = a.seq_lens[seq];
+  const int slen = mla_split_len(len > 0 ? len : 0, a.num_splits);
+  const int tok_begin = split * slen;
+  const int tok_end = min(len, tok_begin + slen);
+  const bool head_ok = (hbase + c) < a.num_heads;
+  const int64_t pidx = ((int64_t)seq * a.num_heads + (hbase + c)) * a.num_splits + split;
+  if (tok_begin >= tok_end) {  // empty split (uniform over the workgroup): mark it and leave
+    if (head_ok && g == 0) a.part_lse[pidx] = -INFINITY;
+    return;
+  }
+  const int t_begin = tok_begin / kTile, t_end = (tok_end + kTile - 1) / kTile;
+  const int bs = a.g.block_size;
+  const int32_t* bt_row = a.block_table + (int64_t)seq * a.bt_stride;
+
+  // ---- cooperative tile load: thread tid takes chunk tid (and tid + 512 for tid < 64) of each
+  //      16-row half; 36 consecutive threads cover one 576-byte row
+  uint32_t goff[2], loff[2];
+#pragma unroll
+  for (int n = 0; n < 2; ++n) {
+    const int qi = tid + kMlaThreads * n;
+    const int row = qi / kChunksPerRow, col = qi % kChunksPerRow;
+    goff[n] = (uint32_t)(row * a.g.stride_row + 16 * col);
+    loff[n] = (uint32_t)(row * kMlaPitch + 16 * col);
+  }
+  const bool second = tid < kChunksPerHalf - kMlaThreads;
+  u32x4 cr[2][2];
+  uint32_t scr[2];
+  auto issue_loads = [&](int t) {
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      int tok = t * kTile + 16 * h;
+      tok = tok < len ? tok : t * kTile;  // a half past the end rereads the first half (masked later)
+      const int e = (int)__umulhi((uint32_t)tok, a.bs_magic);
+      const int s0 = tok - e * bs;
+      const int64_t blk = scalar_load_i32(bt_row, e);
+      const uint8_t* pb = a.cache + blk * a.g.stride_block;
+      const __amdgpu_buffer_rsrc_t rr = __builtin_amdgcn_make_buffer_rsrc(
+          const_cast<uint8_t*>(pb + (int64_t)s0 * a.g.stride_row), 0, 0x7fffffff, 0x00020000);
+      const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
+          const_cast<uint8_t*>(pb + a.g.scale_off + (int64_t)s0 * 4), 0, 0x7fffffff, 0x00020000);
+      cr[h][0] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rr, goff[0], 0, 0));
+      if (second) cr[h][1] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rr, goff[1], 0, 0));
+      scr[h] = __builtin_amdgcn_raw_buffer_load_b32(rs, (uint32_t)((tid & 15) * 4), 0, 0);
+    }
+  };
+  auto stage = [&](uint8_t* buf) {
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      uint8_t* hb = buf + h * 16 * kMlaPitch;
+      *reinterpret_cast<u32x4*>(hb + loff[0]) = cr[h][0];
+      if (second) *reinterpret_cast<u32x4*>(hb + loff[1]) = cr[h][1];
+      if (tid < 16) {
+        float* sc = reinterpret_cast<float*>(buf + kMlaTileBytes);
+        const float v = as_f32(scr[h]);
+        sc[h * 16 + tid] = v * a.scale_log2;                       // K side: scale * log2e folded in
+        sc[kTile + h * 16 + tid] = fminf(v * kPScale, 65504.f);    // V side: 2^8, capped
+      }
+    }
+  };
+
+  issue_loads(t_begin);
+
+  // ---- absorbed Q of this wave's 16 heads as the MFMA B operand: lane (c = head, g) holds, for
+  //      k-step kk, dims 32 kk + 8 g + j
+  half8_t qb[kMlaKSteps];
+  float qsum = 0.f;
+  {
+    const int64_t qbase = (int64_t)seq * a.q_stride_b + (int64_t)(head_ok ? hbase + c : 0) * a.q_stride_h + 8 * g;
+#pragma unroll
+    for (int kk = 0; kk < kMlaKSteps; ++kk) {
+      float f[8];
+      if constexpr (QDT == KVQ_F32) {
+        const float* p = reinterpret_cast<const float*>(a.q) + qbase + 32 * kk;
+        const floatx4 v0 = *reinterpret_cast<const floatx4_a4*>(p), v1 = *reinterpret_cast<const floatx4_a4*>(p + 4);
+        f[0] = v0.x; f[1] = v0.y; f[2] = v0.z; f[3] = v0.w; f[4] = v1.x; f[5] = v1.y; f[6] = v1.z; f[7] = v1.w;
+      } else {
+        const u32x4 v = *reinterpret_cast<const u32x4_a4*>(reinterpret_cast<const uint16_t*>(a.q) + qbase + 32 * kk);
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+          const uint32_t e = v[w];
+          if constexpr (QDT == KVQ_BF16) {
+            f[2 * w] = as_f32(e << 16);
+            f[2 * w + 1] = as_f32(e & 0xffff0000u);
+          } else {
+            const half2_t hh = __builtin_bit_cast(half2_t, e);
+            f[2 * w] = (float)hh.x;
+            f[2 * w + 1] = (float)hh.y;
+          }
+        }
+      }
+      half8_t h8;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        h8[j] = (half_t)(head_ok ? clamp_half_range(f[j]) : 0.f);
+        qsum += (float)h8[j];
+      }
+      qb[kk] = h8;
+    }
+    qsum += __shfl_xor(qsum, 16, kWave);
+    qsum += __shfl_xor(qsum, 32, kWave);
+  }
+  const float s_init = -kCodeBias * qsum;
+
+  floatx4 o[kMlaDT];
+#pragma unroll
+  for (int dt = 0; dt < kMlaDT; ++dt) o[dt] = (floatx4){0.f, 0.f, 0.f, 0.f};
+  floatx4 psum = {0.f, 0.f, 0.f, 0.f};
+  float m = -INFINITY, l = 0.f;
+
+  int buf = 0;
+  for (int t = t_begin; t < t_end; ++t) {
+    stage(lds[buf]);
+    if (t + 1 < t_end) issue_loads(t + 1);
+    __syncthreads();
+    const uint8_t* tile = lds[buf];
+    const float* sck = reinterpret_cast<const float*>(tile + kMlaTileBytes);
+
+    // ---- S^T[32 tokens, 16 heads]: A = code rows, lane (r = token, g): bytes 32 kk + 8 g ..
+    floatx4 s[2];
+#pragma unroll
+    for (int mt = 0; mt < 2; ++mt) {
+      s[mt] = (floatx4){s_init, s_init, s_init, s_init};
+#pragma unroll
+      for (int kk = 0; kk < kMlaKSteps; ++kk) {
+        const u32x2 w = *reinterpret_cast<const u32x2*>(tile + (mt * 16 + c) * kMlaPitch + 32 * kk + 8 * g);
+        s[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(dequant8(w.x, w.y), qb[kk], s[mt], 0, 0, 0);
+      }
+    }
+
+    // ---- softmax, log2 domain; lane (c, g) holds tokens mt*16 + 4g + i of head c
+    float logit[8];
+    float mloc = -INFINITY;
+#pragma unroll
+    for (int mt = 0; mt < 2; ++mt) {
+      const floatx4 ks = *reinterpret_cast<const floatx4*>(sck + 16 * mt + 4 * g);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int tok = t * kTile + 16 * mt + 4 * g + i;
+        float x = s[mt][i] * ks[i];
+        x = tok < tok_end ? x : -INFINITY;
+        logit[4 * mt + i] = x;
+        mloc = fmaxf(mloc, x);
+      }
+    }
+    mloc = fmaxf(mloc, __shfl_xor(mloc, 16, kWave));
+    mloc = fmaxf(mloc, __shfl_xor(mloc, 32, kWave));
+    if (__builtin_amdgcn_ballot_w64(mloc > m) != 0) {
+      const float m_new = fmaxf(m, mloc);
+      const float alpha = __builtin_amdgcn_exp2f(m - m_new);
+      m = m_new;
+      l *= alpha;
+      psum *= alpha;
+#pragma unroll
+      for (int dt = 0; dt < kMlaDT; ++dt) o[dt] *= alpha;
+    }
+    float pt[8];
+#pragma unroll
+    for (int mt = 0; mt < 2; ++mt) {
+      const floatx4 vs = *reinterpret_cast<const floatx4*>(sck + kTile + 16 * mt + 4 * g);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int tok = t * kTile + 16 * mt + 4 * g + i;
+        const float p = __builtin_amdgcn_exp2f(logit[4 * mt + i] - m);
+        l += p;
+        pt[4 * mt + i] = tok < tok_end ? p * vs[i] : 0.f;
+      }
+    }
+    u32x4 pb;
+    pb.x = pack_half2(pt[0], pt[1]);
+    pb.y = pack_half2(pt[2], pt[3]);
+    pb.z = pack_half2(pt[4], pt[5]);
+    pb.w = pack_half2(pt[6], pt[7]);
+    const half8_t p_op = __builtin_bit_cast(half8_t, pb);
+
+    // ---- O^T[512 dims, 16 heads] += (C + 1152)^T . P~^T.  Lane (r, g) supplies bytes
+    //      [32 r, 32 r + 32) of tokens 4g+j (j<4) and 16+4g+(j-4), transposed in registers.
+    {
+      const half_t one = (half_t)1.0f;
+      const half8_t ones = {one, one, one, one, one, one, one, one};
+      psum = __builtin_amdgcn_mfma_f32_16x16x32_f16(ones, p_op, psum, 0, 0, 0);
+    }
+#pragma unroll
+    for (int w = 0; w < kMlaVB / 4; ++w) {
+      uint32_t x0[4], x1[4];
+#pragma unroll
+      for (int pr = 0; pr < 4; ++pr) {
+        const int ja = 2 * pr, jb = 2 * pr + 1;
+        const int ta_tok = (ja & 3) + (ja >> 2) * 16 + 4 * g;
+        const int tb_tok = (jb & 3) + (jb >> 2) * 16 + 4 * g;
+        const uint32_t ta = *reinterpret_cast<const uint32_t*>(tile + ta_tok * kMlaPitch + kMlaVB * c + 4 * w) ^ 0x80808080u;
+        const uint32_t tb = *reinterpret_cast<const uint32_t*>(tile + tb_tok * kMlaPitch + kMlaVB * c + 4 * w) ^ 0x80808080u;
+        x0[pr] = perm(tb, ta, 0x05010400u);
+        x1[pr] = perm(tb, ta, 0x07030602u);
+      }
+#pragma unroll
+      for (int b = 0; b < 4; ++b) {
+        u32x4 av;
+        const uint32_t* x = (b < 2) ? x0 : x1;
+        av.x = bytes_to_half2(x[0], b & 1);
+        av.y = bytes_to_half2(x[1], b & 1);
+        av.z = bytes_to_half2(x[2], b & 1);
+        av.w = bytes_to_half2(x[3], b & 1);
+        const int dt = 4 * w + b;
+        o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, av), p_op, o[dt], 0, 0, 0);
+      }
+    }
+    buf ^= 1;
+  }
+
+  // ---- emit the split's state: locally normalised output and its log2-domain lse.
+  //      Lane (c, g) holds O[head c][dim 32 (4g + i) + dt], dt = 0..31: 32 contiguous dims per i.
+  l += __shfl_xor(l, 16, kWave);
+  l += __shfl_xor(l, 32, kWave);
+  if (!head_ok) return;
+  const float corr = kCodeBias * psum[0];
+  const float inv = 1.0f / (l * kPScale);
+  float* po = a.part_o + pidx * kMlaR;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+#pragma unroll
+    for (int d4 = 0; d4 < kMlaDT / 4; ++d4) {
+      floatx4 v;
+      v.x = (o[4 * d4 + 0][i] - corr) * inv;
+      v.y = (o[4 * d4 + 1][i] - corr) * inv;
+      v.z = (o[4 * d4 + 2][i] - corr) * inv;
+      v.w = (o[4 * d4 + 3][i] - corr) * inv;
+      *reinterpret_cast<floatx4*>(po + 32 * (4 * g + i) + 4 * d4) = v;
+    }
+  }
+  if (g == 0) a.part_lse[pidx] = m + __builtin_amdgcn_logf(l);
+}
+
+// Stage 2: out = sum_j 2^(lse_j - max) o_j / sum_j 2^(lse_j - max); lse = ln 2 * (max + log2 sum).
+// grid (B, ceil(H/4)), one wave per head, lane owns 8 of the 512 dims.
+template <int ODT>
+__global__ __launch_bounds__(256) void mla_reduce_kernel(void* out, float* lse, const float* part_o,
+                                                         const float* part_lse, const int32_t* seq_lens,
+                                                         int num_heads, int num_splits) {
+  const int lane = threadIdx.x & 63;
+  const int head = blockIdx.y * 4 + (threadIdx.x >> 6);
+  const int seq = blockIdx.x;
+  if (head >= num_heads) return;
+  const int64_t base = ((int64_t)seq * num_heads + head) * num_splits;
+  const int64_t obase = ((int64_t)seq * num_heads + head) * kMlaR + lane * 8;
+  float acc[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) acc[i] = 0.f;
+  float mx = -INFINITY;
+  if (seq_lens[seq] > 0)
+    for (int j = 0; j < num_splits; ++j) mx = fmaxf(mx, part_lse[base + j]);
+  if (mx == -INFINITY) {  // nothing attended: defined output
+#pragma unroll
+    for (int i = 0; i < 8; ++i) store_act<ODT>(out, obase + i, 0.f);
+    if (lse != nullptr && lane == 0) lse[(int64_t)seq * num_heads + head] = -INFINITY;
+    return;
+  }
+  float den = 0.f;
+  for (int j = 0; j < num_splits; ++j) {
+    const float lj = part_lse[base + j];
+    if (lj == -INFINITY) continue;
+    const float wj = __builtin_amdgcn_exp2f(lj - mx);
+    den += wj;
+    const float* po = part_o + (base + j) * kMlaR + lane * 8;
+    const floatx4 v0 = *reinterpret_cast<const floatx4*>(po), v1 = *reinterpret_cast<const floatx4*>(po + 4);
+    acc[0] += v0.x * wj; acc[1] += v0.y * wj; acc[2] += v0.z * wj; acc[3] += v0.w * wj;
+    acc[4] += v1.x * wj; acc[5] += v1.y * wj; acc[6] += v1.z * wj; acc[7] += v1.w * wj;
+  }
+  const float inv = 1.0f / den;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) store_act<ODT>(out, obase + i, acc[i] * inv);
+  if (lse != nullptr && lane == 0) lse[(int64_t)seq * num_heads + head] = (mx + __builtin_amdgcn_logf(den)) * kLn2;
+}
+
+// num_kv_splits policy of the reference (vllm_metax/v1/attention/backends/mla/triton_mla.py:45-55),
+// additionally bounded so that (sequences x splits) does not far exceed the resident workgroups.
+static int mla_num_splits(int max_seq_hint, int num_seqs, int num_heads) {
+  (void)max_seq_hint;
+  const int cus = num_cus();
+  const int groups = (num_heads + 127) / 128;
+  int splits = 1;
+  while (splits < 64 && (int64_t)num_seqs * groups * splits * 2 <= (int64_t)cus) splits *= 2;
+  return splits;
+}
+
+}  // namespace kvq
 
 extern "C" {
 
-size_t kvq_mla_decode_workspace_bytes(int, int, int) { return 0; }
+size_t kvq_mla_decode_workspace_bytes(int max_num_seqs, int num_heads, int kv_lora_rank) {
+  if (max_num_seqs <= 0 || num_heads <= 0 || kv_lora_rank <= 0) return 0;
+  // sequences x splits never exceeds max(resident workgroups per head group, sequences)
+  const size_t groups = ((size_t)num_heads + 127) / 128;
+  size_t items = (size_t)kvq::num_cus() / groups;
+  if (items < (size_t)max_num_seqs) items = (size_t)max_num_seqs;
+  return items * (size_t)num_heads * ((size_t)kv_lora_rank + 1) * sizeof(float);
+}
 
-int kvq_mla_decode_int8(void*, int, float*, const void*, int, int64_t, int64_t, const void*, const kvq_mla_geom*,
-                        const int32_t*, int64_t, const int32_t*, int, int, float, void*, size_t, kvq_stream_t) {
-  return kvq::fail(KVQ_ENOSYS, "mla_decode_int8: not built yet");
+int kvq_mla_decode_int8(void* out, int out_dtype, float* lse, const void* q, int q_dtype, int64_t q_stride_b,
+                        int64_t q_stride_h, const void* cache, const kvq_mla_geom* geom,
+                        const int32_t* block_table, int64_t bt_stride, const int32_t* seq_lens, int num_seqs,
+                        int num_heads, float scale, void* workspace, size_t workspace_bytes,
+                        kvq_stream_t stream) {
+  using namespace kvq;
+  const char* op = "mla_decode_int8";
+  KVQ_REQUIRE(geom != nullptr, "%s: geom is NULL", op);
+  KVQ_REQUIRE(out && q && cache && block_table && seq_lens, "%s: NULL pointer", op);
+  KVQ_REQUIRE(num_seqs > 0 && num_seqs <= 65535 && num_heads > 0, "%s: num_seqs / num_heads out of range", op);
+  const kvq_mla_geom& g = *geom;
+  KVQ_REQUIRE(g.kv_lora_rank == kMlaR && g.rope_dim == kMlaP,
+              "%s: only kv_lora_rank 512 + rope 64 is built (got %d + %d)", op, g.kv_lora_rank, g.rope_dim);
+  KVQ_REQUIRE(g.block_size > 0 && g.block_size % 16 == 0, "%s: block_size must be a multiple of 16", op);
+  KVQ_REQUIRE((g.stride_block | g.stride_row | g.scale_off) % 4 == 0 && ((uintptr_t)cache % 4) == 0 &&
+                  g.stride_row >= kMlaW && g.stride_row <= (1 << 20),
+              "%s: cache strides must be 4-byte aligned and rows at least 576 bytes apart", op);
+  const int qsz = q_dtype == KVQ_F32 ? 4 : 2;
+  KVQ_REQUIRE(((uintptr_t)q % 4) == 0 && (q_stride_b * qsz) % 4 == 0 && (q_stride_h * qsz) % 4 == 0,
+              "%s: q rows must be 4-byte aligned", op);
+  const int splits = mla_num_splits(0, num_seqs, num_heads);
+  const size_t need = (size_t)num_seqs * num_heads * splits * ((size_t)kMlaR + 1) * sizeof(float);
+  KVQ_REQUIRE(workspace != nullptr && workspace_bytes >= need && ((uintptr_t)workspace % 16) == 0,
+              "%s: workspace of %zu bytes (16-byte aligned) required, got %zu", op, need, workspace_bytes);
+  MlaArgs a{};
+  a.q = q;
+  a.q_stride_b = q_stride_b;
+  a.q_stride_h = q_stride_h;
+  a.cache = static_cast<const uint8_t*>(cache);
+  a.g = g;
+  a.block_table = block_table;
+  a.bt_stride = bt_stride;
+  a.seq_lens = seq_lens;
+  a.part_o = static_cast<float*>(workspace);
+  a.part_lse = a.part_o + (size_t)num_seqs * num_heads * splits * kMlaR;
+  a.num_heads = num_heads;
+  a.num_splits = splits;
+  a.scale_log2 = scale * kLog2e;
+  a.bs_magic = (uint32_t)((0x100000000ull + (uint64_t)g.block_size - 1) / (uint64_t)g.block_size);
+  hipStream_t s = as_stream(stream);
+  dim3 grid(splits, num_seqs, (num_heads + 127) / 128);
+  switch (q_dtype) {
+    case KVQ_F32: hipLaunchKernelGGL((mla_decode_kernel<KVQ_F32>), grid, dim3(kMlaThreads), 0, s, a); break;
+    case KVQ_BF16: hipLaunchKernelGGL((mla_decode_kernel<KVQ_BF16>), grid, dim3(kMlaThreads), 0, s, a); break;
+    case KVQ_F16: hipLaunchKernelGGL((mla_decode_kernel<KVQ_F16>), grid, dim3(kMlaThreads), 0, s, a); break;
+    default: return fail(KVQ_EINVAL, "%s: unknown q_dtype %d", op, q_dtype);
+  }
+  int rc = check_hip(hipGetLastError(), "mla_decode_int8 launch");
+  if (rc) return rc;
+  dim3 rgrid(num_seqs, (num_heads + 3) / 4);
+#define KVQ_MLAR(T)                                                                                           \
+  hipLaunchKernelGGL((mla_reduce_kernel<T>), rgrid, dim3(256), 0, s, out, lse, a.part_o, a.part_lse, seq_lens, \
+                     num_heads, splits)
+  switch (out_dtype) {
+    case KVQ_F32: KVQ_MLAR(KVQ_F32); break;
+    case KVQ_BF16: KVQ_MLAR(KVQ_BF16); break;
+    case KVQ_F16: KVQ_MLAR(KVQ_F16); break;
+    default: return fail(KVQ_EINVAL, "%s: unknown out_dtype %d", op, out_dtype);
+  }
+#undef KVQ_MLAR
+  return check_hip(hipGetLastError(), "mla_decode_int8 reduce launch");
 }
 
 }  // extern "C"
