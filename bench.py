@@ -47,6 +47,8 @@ def make_batch(workload: str, seed: int = 0):
         return dict(hq=32, hkv=8, d=128, bs=16, ctx=ctx, pool=66000)
     if workload == "config1_b4_ctx512":                  # configs[0]
         return dict(hq=32, hkv=8, d=128, bs=16, ctx=[512] * 4, pool=129)
+    if workload == "mla_decode_b32_h128_ctx4096":        # configs[3]: DeepSeek-V2 MLA decode
+        return dict(mla=True, heads=128, r=512, p=64, bs=64, ctx=[4096] * 32, pool=32 * 64 + 8)
     raise SystemExit(f"unknown workload {workload}")
 
 
@@ -123,6 +125,133 @@ def run_step(st, layer, ops, write=True, attn=True):
                               workspace=st["ws"], geometry=c["geom"])
 
 
+MFMA_F16_PEAK_TFLOPS = 2500.0
+
+
+def mla_algorithmic(cfg):
+    """(bytes, flops) of one MLA decode launch: every context row's 576 codes + fp32 scale, Q in, O and
+    lse out, block table; 2 flops per multiply-add of q.k over 576 dims and p.v over 512 dims."""
+    H, R, P, bs, ctx = cfg["heads"], cfg["r"], cfg["p"], cfg["bs"], cfg["ctx"]
+    B = len(ctx)
+    nbytes = sum(ctx) * (R + P + 4) + B * H * ((R + P) * 2 + R * 2 + 4) + sum((c + bs - 1) // bs for c in ctx) * 4 + 4 * B
+    flops = 2 * sum(ctx) * H * ((R + P) + R)
+    return nbytes, flops
+
+
+def build_mla_state(cfg, dev, layers, seed=0):
+    from vllm_metax_amd import _custom_ops as ops
+    from vllm_metax_amd import layout as L
+
+    H, R, P, bs, ctx, pool = cfg["heads"], cfg["r"], cfg["p"], cfg["bs"], cfg["ctx"], cfg["pool"]
+    B = len(ctx)
+    g = torch.Generator().manual_seed(seed)
+    need = [(c + bs - 1) // bs for c in ctx]
+    perm = torch.randperm(pool - 1, generator=g)[: sum(need)] + 1
+    bt = torch.zeros((B, max(need)), dtype=torch.int32)
+    o = 0
+    for i, n in enumerate(need):
+        bt[i, :n] = perm[o:o + n].to(torch.int32)
+        o += n
+    bt_d = bt.to(dev)
+    sl_d = torch.tensor(ctx, dtype=torch.int32, device=dev)
+    last = torch.tensor([int(bt[i, (c - 1) // bs]) * bs + (c - 1) % bs for i, c in enumerate(ctx)], dtype=torch.int64)
+    torch.manual_seed(seed)
+    caches = []
+    for _ in range(layers):
+        cache = L.allocate_mla_cache(pool, bs, R + P, device=dev)
+        for i, c in enumerate(ctx):
+            pos = torch.arange(c, device=dev)
+            slots = bt_d[i, pos // bs].to(torch.int64) * bs + pos % bs
+            ops.concat_and_cache_mla(torch.randn((c, R), device=dev).to(torch.bfloat16),
+                                     torch.randn((c, P), device=dev).to(torch.bfloat16), cache, slots)
+        caches.append(cache)
+    q = (torch.randn((B, H, R + P), device=dev) * 0.5).to(torch.bfloat16)
+    st = dict(bt=bt, bt_d=bt_d, sl_d=sl_d, caches=caches, q=q, out=torch.empty((B, H, R), dtype=torch.bfloat16, device=dev),
+              lse=torch.empty((B, H), dtype=torch.float32, device=dev), slots_new=last.to(dev),
+              new_c=torch.randn((B, R), device=dev).to(torch.bfloat16), new_pe=torch.randn((B, P), device=dev).to(torch.bfloat16),
+              ws=torch.empty(ops.mla_decode_workspace_bytes(B, H, R), dtype=torch.uint8, device=dev),
+              scale=(128 + P) ** -0.5)
+    torch.cuda.synchronize()
+    return st
+
+
+def run_mla_step(st, layer, ops, cfg, write=True, attn=True):
+    cache = st["caches"][layer]
+    if write:
+        ops.concat_and_cache_mla(st["new_c"], st["new_pe"], cache, st["slots_new"])
+    if attn:
+        ops.mla_decode_int8(st["q"], cache, st["out"], st["lse"], st["bt_d"], st["sl_d"], st["scale"], cfg["r"],
+                            workspace=st["ws"])
+
+
+def mla_cpu_baseline(cfg, st, seconds_target=15.0):
+    """The reference's CPU-runnable MLA decode contract (tests/kernels/attention/test_mla_decode_cpu.py:14-41,
+    as-written torch ops) on dequantised rows of a bounded sample of the batch."""
+    from oracle import torch_ref
+    from vllm_metax_amd import layout as L
+
+    H, R, P, bs, ctx = cfg["heads"], cfg["r"], cfg["p"], cfg["bs"], cfg["ctx"]
+    cache = st["caches"][0]
+    t_total, done, reps = 0.0, 0, 0
+    q_cpu = st["q"].cpu()
+    for i in range(len(ctx)):
+        if t_total >= seconds_target:
+            break
+        n = (ctx[i] + bs - 1) // bs
+        sub = cache[st["bt_d"][i, :n].long()].cpu().contiguous()
+        codes, scales = L.mla_cache_views(sub)
+        t0 = time.perf_counter()
+        latent = (codes.to(torch.float32) * scales[..., None]).to(torch.bfloat16)     # dequantised (n, bs, 576)
+        torch_ref.mla_decode(q_cpu[i:i + 1], latent, st["scale"], torch.arange(n)[None], [ctx[i]], R)
+        t_total += time.perf_counter() - t0
+        done += ctx[i]
+        reps += 1
+    flops = 2 * done * H * (2 * R + P)
+    return dict(value=flops / t_total / 1e12, unit="TFLOP/s", cores=torch.get_num_threads(), kind="port",
+                sample=f"{reps} sequence(s) of the batch ({done} context rows), oracle/torch_ref.py mla_decode "
+                       f"(as-written torch), {t_total:.1f} s, torch threads={torch.get_num_threads()}")
+
+
+def mla_main(args, cfg, dev, ops):
+    st = build_mla_state(cfg, dev, args.layers)
+    nbytes, flops = mla_algorithmic(cfg)
+    L = args.layers
+    for i in range(args.warmup):
+        run_mla_step(st, i % L, ops, cfg)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        run_mla_step(st, i % L, ops, cfg)
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / args.steps
+    n_ev = min(args.steps, 200)
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n_ev)]
+    for i in range(n_ev):
+        run_mla_step(st, i % L, ops, cfg, write=True, attn=False)
+        evs[i][0].record()
+        run_mla_step(st, i % L, ops, cfg, write=False, attn=True)
+        evs[i][1].record()
+    torch.cuda.synchronize()
+    attn_s = sum(a.elapsed_time(b) for a, b in evs) / n_ev * 1e-3
+    res = {
+        "metric": "int8 MLA latent-cache decode: achieved HBM GB/s, µs/layer @B=32 H=128 ctx=4096",
+        "value": round(nbytes / dt / 1e9, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(dt * 1e3, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "int8 latent codes, fp16 MFMA operands, fp32 softmax/accumulate, bf16 Q/out", "data": "synthetic",
+        "config": {"workload": args.workload, "batch": len(cfg["ctx"]), "sum_ctx": sum(cfg["ctx"]), "heads": cfg["heads"],
+                   "kv_lora_rank": cfg["r"], "rope_dim": cfg["p"], "block_size": cfg["bs"], "layer_caches_rotated": L},
+        "us_per_layer": round(dt * 1e6, 2), "attn_launch_us": round(attn_s * 1e6, 2),
+        "roofline": {"bound": "mfma", "achieved": round(flops / attn_s / 1e12, 1), "peak": MFMA_F16_PEAK_TFLOPS,
+                     "unit": "TFLOP/s", "frac": round(flops / attn_s / 1e12 / MFMA_F16_PEAK_TFLOPS, 4), "traffic": None,
+                     "kernel": "MLA decode launch = mla_decode_kernel + mla_reduce_kernel",
+                     "algorithmic_flops_per_launch": flops, "algorithmic_bytes_per_launch": nbytes,
+                     "hbm_frac_of_peak": round(nbytes / attn_s / 1e9 / HBM_PEAK_GBPS, 4)},
+    }
+    if not args.no_cpu_baseline:
+        res["cpu_baseline"] = mla_cpu_baseline(cfg, st, args.cpu_seconds)
+    print(json.dumps(res))
+
+
 def cpu_baseline(cfg, st, seconds_target=15.0):
     """The reference's CPU path (as-written torch ops, bf16 Q.K / fp32 softmax / bf16 P.V) on a
     bounded sample of the batch: dequantise the sampled sequences' blocks, then ref_paged_attn."""
@@ -180,6 +309,8 @@ def main():
 
     dev = torch.device("cuda:0")
     cfg = make_batch(args.workload)
+    if cfg.get("mla"):
+        return mla_main(args, cfg, dev, ops)
     st = build_device_state(cfg, dev, args.layers)
     attn_bytes, write_bytes = algorithmic_bytes(cfg)
     L = args.layers

@@ -29,6 +29,9 @@ constexpr int kMlaVB = kMlaR / 16;                        // 32 V bytes per toke
 constexpr int kChunksPerRow = kMlaW / 16;                 // 36
 constexpr int kChunksPerHalf = 16 * kChunksPerRow;        // 576
 constexpr int kMlaThreads = 512;
+constexpr int kMlaQRegSteps = 4;                          // k-steps of Q kept in registers; the rest in LDS
+constexpr int kMlaQLdsBytes = (kMlaKSteps - kMlaQRegSteps) * kMlaThreads * 16;  // 114688
+constexpr int kMlaLdsBytes = 2 * kMlaBufBytes + kMlaQLdsBytes;                  // 153088 of 163840
 
 struct MlaArgs {
   const void* q;
@@ -38,8 +41,13 @@ struct MlaArgs {
   const int32_t* block_table;
   int64_t bt_stride;
   const int32_t* seq_lens;
-  float* part_o;    // [B, H, S, 512]
-  float* part_lse;  // [B, H, S] log2-domain lse of the split, -inf for an empty split
+  // Split states.  part_o is kept in the order the MFMA leaves it in registers, so that every store
+  // and every load of the reduce is one contiguous KiB per wave: [B, S, ceil(H/16)] blocks of
+  // [32 (= d4 * 4 + i)][64 lanes][4 floats], lane (c, g) holding dims 64 d4 + 16 g + 4 i + (0..3) of
+  // head 16 * block + c.  part_lse: [B, S, 16 * ceil(H/16)] log2-domain, -inf for an empty split.
+  float* part_o;
+  float* part_lse;
+  int head_groups;  // ceil(H / 16)
   int num_heads;
   int num_splits;
   float scale_log2;
@@ -54,7 +62,10 @@ __device__ __forceinline__ int mla_split_len(int len, int num_splits) {
 
 template <int QDT>
 __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
-  __shared__ __align__(16) uint8_t lds[2][kMlaBufBytes];
+  extern __shared__ __align__(16) uint8_t lds_raw[];
+  uint8_t(*lds)[kMlaBufBytes] = reinterpret_cast<uint8_t(*)[kMlaBufBytes]>(lds_raw);
+  // B operands of Q for k-steps >= kMlaQRegSteps: slot [kk][thread], written and read by the same lane
+  u32x4* qlds = reinterpret_cast<u32x4*>(lds_raw + 2 * kMlaBufBytes) + threadIdx.x;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -66,9 +77,11 @@ __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
   const int tok_begin = split * slen;
   const int tok_end = min(len, tok_begin + slen);
   const bool head_ok = (hbase + c) < a.num_heads;
-  const int64_t pidx = ((int64_t)seq * a.num_heads + (hbase + c)) * a.num_splits + split;
+  const int hgroup = blockIdx.z * 8 + wave;
+  const bool wave_ok = hgroup < a.head_groups;    // wave-uniform: this wave owns at least one head
+  const int64_t pblock = ((int64_t)seq * a.num_splits + split) * a.head_groups + hgroup;
   if (tok_begin >= tok_end) {  // empty split (uniform over the workgroup): mark it and leave
-    if (head_ok && g == 0) a.part_lse[pidx] = -INFINITY;
+    if (wave_ok && g == 0) a.part_lse[pblock * 16 + c] = -INFINITY;
     return;
   }
   const int t_begin = tok_begin / kTile, t_end = (tok_end + kTile - 1) / kTile;
@@ -125,10 +138,18 @@ __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
 
   // ---- absorbed Q of this wave's 16 heads as the MFMA B operand: lane (c = head, g) holds, for
   //      k-step kk, dims 32 kk + 8 g + j
-  half8_t qb[kMlaKSteps];
+  half8_t qb[kMlaQRegSteps];
   float qsum = 0.f;
   {
+    const uint32_t okmask = head_ok ? 0xffffffffu : 0u;   // heads past the end contribute zero columns
     const int64_t qbase = (int64_t)seq * a.q_stride_b + (int64_t)(head_ok ? hbase + c : 0) * a.q_stride_h + 8 * g;
+    u32x4 raw[QDT == KVQ_F32 ? 1 : kMlaKSteps];
+    if constexpr (QDT != KVQ_F32) {  // all 18 loads in flight before the first conversion waits
+#pragma unroll
+      for (int kk = 0; kk < kMlaKSteps; ++kk)
+        raw[kk] = *reinterpret_cast<const u32x4_a4*>(reinterpret_cast<const uint16_t*>(a.q) + qbase + 32 * kk);
+      __builtin_amdgcn_sched_barrier(0);
+    }
 #pragma unroll
     for (int kk = 0; kk < kMlaKSteps; ++kk) {
       float f[8];
@@ -137,7 +158,7 @@ __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
         const floatx4 v0 = *reinterpret_cast<const floatx4_a4*>(p), v1 = *reinterpret_cast<const floatx4_a4*>(p + 4);
         f[0] = v0.x; f[1] = v0.y; f[2] = v0.z; f[3] = v0.w; f[4] = v1.x; f[5] = v1.y; f[6] = v1.z; f[7] = v1.w;
       } else {
-        const u32x4 v = *reinterpret_cast<const u32x4_a4*>(reinterpret_cast<const uint16_t*>(a.q) + qbase + 32 * kk);
+        const u32x4 v = raw[kk];
 #pragma unroll
         for (int w = 0; w < 4; ++w) {
           const uint32_t e = v[w];
@@ -151,13 +172,16 @@ __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
           }
         }
       }
-      half8_t h8;
+      u32x4 hb;
+      hb.x = pack_half2(clamp_half_range(f[0]), clamp_half_range(f[1])) & okmask;
+      hb.y = pack_half2(clamp_half_range(f[2]), clamp_half_range(f[3])) & okmask;
+      hb.z = pack_half2(clamp_half_range(f[4]), clamp_half_range(f[5])) & okmask;
+      hb.w = pack_half2(clamp_half_range(f[6]), clamp_half_range(f[7])) & okmask;
+      const half8_t h8 = __builtin_bit_cast(half8_t, hb);
 #pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        h8[j] = (half_t)(head_ok ? clamp_half_range(f[j]) : 0.f);
-        qsum += (float)h8[j];
-      }
-      qb[kk] = h8;
+      for (int j = 0; j < 8; ++j) qsum += (float)h8[j];
+      if (kk < kMlaQRegSteps) qb[kk] = h8;
+      else qlds[(kk - kMlaQRegSteps) * kMlaThreads] = hb;
     }
     qsum += __shfl_xor(qsum, 16, kWave);
     qsum += __shfl_xor(qsum, 32, kWave);
@@ -180,13 +204,17 @@ __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
 
     // ---- S^T[32 tokens, 16 heads]: A = code rows, lane (r = token, g): bytes 32 kk + 8 g ..
     floatx4 s[2];
+    s[0] = (floatx4){s_init, s_init, s_init, s_init};
+    s[1] = s[0];
 #pragma unroll
-    for (int mt = 0; mt < 2; ++mt) {
-      s[mt] = (floatx4){s_init, s_init, s_init, s_init};
+    for (int kk = 0; kk < kMlaKSteps; ++kk) {
+      half8_t qop;
+      if (kk < kMlaQRegSteps) qop = qb[kk];
+      else qop = __builtin_bit_cast(half8_t, qlds[(kk - kMlaQRegSteps) * kMlaThreads]);
 #pragma unroll
-      for (int kk = 0; kk < kMlaKSteps; ++kk) {
+      for (int mt = 0; mt < 2; ++mt) {
         const u32x2 w = *reinterpret_cast<const u32x2*>(tile + (mt * 16 + c) * kMlaPitch + 32 * kk + 8 * g);
-        s[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(dequant8(w.x, w.y), qb[kk], s[mt], 0, 0, 0);
+        s[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(dequant8(w.x, w.y), qop, s[mt], 0, 0, 0);
       }
     }
 
@@ -235,8 +263,10 @@ __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
     pb.w = pack_half2(pt[6], pt[7]);
     const half8_t p_op = __builtin_bit_cast(half8_t, pb);
 
-    // ---- O^T[512 dims, 16 heads] += (C + 1152)^T . P~^T.  Lane (r, g) supplies bytes
-    //      [32 r, 32 r + 32) of tokens 4g+j (j<4) and 16+4g+(j-4), transposed in registers.
+    // ---- O^T[512 dims, 16 heads] += (C + 1152)^T . P~^T.  Lane (r, g) supplies, for w = 0..7, bytes
+    //      [64 w + 4 r, +4) of tokens 4g+j (j<4) and 16+4g+(j-4), transposed in registers: row r of
+    //      output tile 4w+b is dim 64 w + 4 r + b.  (Lanes r = 0..15 read 16 consecutive dwords of a
+    //      row, so the 64 lanes of a read spread over all LDS banks.)
     {
       const half_t one = (half_t)1.0f;
       const half8_t ones = {one, one, one, one, one, one, one, one};
@@ -250,8 +280,8 @@ __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
         const int ja = 2 * pr, jb = 2 * pr + 1;
         const int ta_tok = (ja & 3) + (ja >> 2) * 16 + 4 * g;
         const int tb_tok = (jb & 3) + (jb >> 2) * 16 + 4 * g;
-        const uint32_t ta = *reinterpret_cast<const uint32_t*>(tile + ta_tok * kMlaPitch + kMlaVB * c + 4 * w) ^ 0x80808080u;
-        const uint32_t tb = *reinterpret_cast<const uint32_t*>(tile + tb_tok * kMlaPitch + kMlaVB * c + 4 * w) ^ 0x80808080u;
+        const uint32_t ta = *reinterpret_cast<const uint32_t*>(tile + ta_tok * kMlaPitch + 64 * w + 4 * c) ^ 0x80808080u;
+        const uint32_t tb = *reinterpret_cast<const uint32_t*>(tile + tb_tok * kMlaPitch + 64 * w + 4 * c) ^ 0x80808080u;
         x0[pr] = perm(tb, ta, 0x05010400u);
         x1[pr] = perm(tb, ta, 0x07030602u);
       }
@@ -271,67 +301,79 @@ __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
   }
 
   // ---- emit the split's state: locally normalised output and its log2-domain lse.
-  //      Lane (c, g) holds O[head c][dim 32 (4g + i) + dt], dt = 0..31: 32 contiguous dims per i.
+  //      Lane (c, g) holds O[head c][dim 64 w + 16 g + 4 i + b] in o[4w + b][i].
   l += __shfl_xor(l, 16, kWave);
   l += __shfl_xor(l, 32, kWave);
-  if (!head_ok) return;
+  if (!wave_ok) return;
   const float corr = kCodeBias * psum[0];
   const float inv = 1.0f / (l * kPScale);
-  float* po = a.part_o + pidx * kMlaR;
+  float* po = a.part_o + pblock * (16 * kMlaR) + lane * 4;
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
+  for (int d4 = 0; d4 < kMlaDT / 4; ++d4) {
 #pragma unroll
-    for (int d4 = 0; d4 < kMlaDT / 4; ++d4) {
+    for (int i = 0; i < 4; ++i) {
       floatx4 v;
       v.x = (o[4 * d4 + 0][i] - corr) * inv;
       v.y = (o[4 * d4 + 1][i] - corr) * inv;
       v.z = (o[4 * d4 + 2][i] - corr) * inv;
       v.w = (o[4 * d4 + 3][i] - corr) * inv;
-      *reinterpret_cast<floatx4*>(po + 32 * (4 * g + i) + 4 * d4) = v;
+      *reinterpret_cast<floatx4*>(po + (d4 * 4 + i) * 256) = v;
     }
   }
-  if (g == 0) a.part_lse[pidx] = m + __builtin_amdgcn_logf(l);
+  if (g == 0) a.part_lse[pblock * 16 + c] = m + __builtin_amdgcn_logf(l);
 }
 
 // Stage 2: out = sum_j 2^(lse_j - max) o_j / sum_j 2^(lse_j - max); lse = ln 2 * (max + log2 sum).
-// grid (B, ceil(H/4)), one wave per head, lane owns 8 of the 512 dims.
+// grid (B, ceil(H/16)), 8 waves; wave w combines the d4 = w slice of the block's 16 heads, lane (c, g)
+// as in the split state layout.
 template <int ODT>
-__global__ __launch_bounds__(256) void mla_reduce_kernel(void* out, float* lse, const float* part_o,
+__global__ __launch_bounds__(512) void mla_reduce_kernel(void* out, float* lse, const float* part_o,
                                                          const float* part_lse, const int32_t* seq_lens,
-                                                         int num_heads, int num_splits) {
-  const int lane = threadIdx.x & 63;
-  const int head = blockIdx.y * 4 + (threadIdx.x >> 6);
-  const int seq = blockIdx.x;
-  if (head >= num_heads) return;
-  const int64_t base = ((int64_t)seq * num_heads + head) * num_splits;
-  const int64_t obase = ((int64_t)seq * num_heads + head) * kMlaR + lane * 8;
-  float acc[8];
+                                                         int num_heads, int head_groups, int num_splits) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int c = lane & 15, g = lane >> 4;
+  const int seq = blockIdx.x, hgroup = blockIdx.y;
+  const int head = hgroup * 16 + c;
+  const bool head_ok = head < num_heads;
+  const int64_t lstride = (int64_t)head_groups * 16;                    // part_lse stride between splits
+  const float* pl = part_lse + ((int64_t)seq * num_splits * head_groups + hgroup) * 16 + c;
+  const float* po = part_o + ((int64_t)seq * num_splits * head_groups + hgroup) * (16 * kMlaR) + (wave * 4 * 64 + lane) * 4;
+  const int64_t ostride = (int64_t)head_groups * 16 * kMlaR;            // part_o stride between splits
+  floatx4 acc[4];
 #pragma unroll
-  for (int i = 0; i < 8; ++i) acc[i] = 0.f;
+  for (int r = 0; r < 4; ++r) acc[r] = (floatx4){0.f, 0.f, 0.f, 0.f};
   float mx = -INFINITY;
   if (seq_lens[seq] > 0)
-    for (int j = 0; j < num_splits; ++j) mx = fmaxf(mx, part_lse[base + j]);
-  if (mx == -INFINITY) {  // nothing attended: defined output
-#pragma unroll
-    for (int i = 0; i < 8; ++i) store_act<ODT>(out, obase + i, 0.f);
-    if (lse != nullptr && lane == 0) lse[(int64_t)seq * num_heads + head] = -INFINITY;
-    return;
-  }
+    for (int j = 0; j < num_splits; ++j) mx = fmaxf(mx, pl[j * lstride]);
   float den = 0.f;
-  for (int j = 0; j < num_splits; ++j) {
-    const float lj = part_lse[base + j];
-    if (lj == -INFINITY) continue;
-    const float wj = __builtin_amdgcn_exp2f(lj - mx);
-    den += wj;
-    const float* po = part_o + (base + j) * kMlaR + lane * 8;
-    const floatx4 v0 = *reinterpret_cast<const floatx4*>(po), v1 = *reinterpret_cast<const floatx4*>(po + 4);
-    acc[0] += v0.x * wj; acc[1] += v0.y * wj; acc[2] += v0.z * wj; acc[3] += v0.w * wj;
-    acc[4] += v1.x * wj; acc[5] += v1.y * wj; acc[6] += v1.z * wj; acc[7] += v1.w * wj;
-  }
-  const float inv = 1.0f / den;
+  if (mx != -INFINITY) {
+#pragma unroll 4
+    for (int j = 0; j < num_splits; ++j) {
+      const float lj = pl[j * lstride];
+      const float wj = lj == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(lj - mx);
+      if (__builtin_amdgcn_ballot_w64(wj != 0.f) == 0) continue;       // split empty for the whole block
+      den += wj;
+      const float* pj = po + j * ostride;
 #pragma unroll
-  for (int i = 0; i < 8; ++i) store_act<ODT>(out, obase + i, acc[i] * inv);
-  if (lse != nullptr && lane == 0) lse[(int64_t)seq * num_heads + head] = (mx + __builtin_amdgcn_logf(den)) * kLn2;
+      for (int r = 0; r < 4; ++r) {
+        const floatx4 v = *reinterpret_cast<const floatx4*>(pj + r * 256);
+        acc[r] += (wj != 0.f ? v : (floatx4){0.f, 0.f, 0.f, 0.f}) * wj;
+      }
+    }
+  }
+  if (!head_ok) return;
+  const float inv = den > 0.f ? 1.0f / den : 0.f;                       // nothing attended: zeros
+  const int64_t obase = ((int64_t)seq * num_heads + head) * kMlaR + 16 * g;
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const int64_t o = obase + 64 * wave + 4 * r;
+    store_act<ODT>(out, o + 0, acc[r].x * inv);
+    store_act<ODT>(out, o + 1, acc[r].y * inv);
+    store_act<ODT>(out, o + 2, acc[r].z * inv);
+    store_act<ODT>(out, o + 3, acc[r].w * inv);
+  }
+  if (lse != nullptr && wave == 0 && g == 0)
+    lse[(int64_t)seq * num_heads + head] = den > 0.f ? (mx + __builtin_amdgcn_logf(den)) * kLn2 : -INFINITY;
 }
 
 // num_kv_splits policy of the reference (vllm_metax/v1/attention/backends/mla/triton_mla.py:45-55),
@@ -341,7 +383,7 @@ static int mla_num_splits(int max_seq_hint, int num_seqs, int num_heads) {
   const int cus = num_cus();
   const int groups = (num_heads + 127) / 128;
   int splits = 1;
-  while (splits < 64 && (int64_t)num_seqs * groups * splits * 2 <= (int64_t)cus) splits *= 2;
+  while (splits < 64 && (int64_t)num_seqs * groups * splits < (int64_t)cus) splits *= 2;
   return splits;
 }
 
@@ -351,11 +393,12 @@ extern "C" {
 
 size_t kvq_mla_decode_workspace_bytes(int max_num_seqs, int num_heads, int kv_lora_rank) {
   if (max_num_seqs <= 0 || num_heads <= 0 || kv_lora_rank <= 0) return 0;
-  // sequences x splits never exceeds max(resident workgroups per head group, sequences)
+  // sequences x splits stays below max(2 x resident workgroups per head group, sequences)
   const size_t groups = ((size_t)num_heads + 127) / 128;
-  size_t items = (size_t)kvq::num_cus() / groups;
+  size_t items = 2 * (size_t)kvq::num_cus() / groups;
   if (items < (size_t)max_num_seqs) items = (size_t)max_num_seqs;
-  return items * (size_t)num_heads * ((size_t)kv_lora_rank + 1) * sizeof(float);
+  const size_t heads_padded = ((size_t)num_heads + 15) / 16 * 16;
+  return items * heads_padded * ((size_t)kv_lora_rank + 1) * sizeof(float);
 }
 
 int kvq_mla_decode_int8(void* out, int out_dtype, float* lse, const void* q, int q_dtype, int64_t q_stride_b,
@@ -379,7 +422,8 @@ int kvq_mla_decode_int8(void* out, int out_dtype, float* lse, const void* q, int
   KVQ_REQUIRE(((uintptr_t)q % 4) == 0 && (q_stride_b * qsz) % 4 == 0 && (q_stride_h * qsz) % 4 == 0,
               "%s: q rows must be 4-byte aligned", op);
   const int splits = mla_num_splits(0, num_seqs, num_heads);
-  const size_t need = (size_t)num_seqs * num_heads * splits * ((size_t)kMlaR + 1) * sizeof(float);
+  const int head_groups = (num_heads + 15) / 16;
+  const size_t need = (size_t)num_seqs * head_groups * 16 * splits * ((size_t)kMlaR + 1) * sizeof(float);
   KVQ_REQUIRE(workspace != nullptr && workspace_bytes >= need && ((uintptr_t)workspace % 16) == 0,
               "%s: workspace of %zu bytes (16-byte aligned) required, got %zu", op, need, workspace_bytes);
   MlaArgs a{};
@@ -392,25 +436,41 @@ int kvq_mla_decode_int8(void* out, int out_dtype, float* lse, const void* q, int
   a.bt_stride = bt_stride;
   a.seq_lens = seq_lens;
   a.part_o = static_cast<float*>(workspace);
-  a.part_lse = a.part_o + (size_t)num_seqs * num_heads * splits * kMlaR;
+  a.part_lse = a.part_o + (size_t)num_seqs * head_groups * 16 * splits * kMlaR;
+  a.head_groups = head_groups;
   a.num_heads = num_heads;
   a.num_splits = splits;
   a.scale_log2 = scale * kLog2e;
   a.bs_magic = (uint32_t)((0x100000000ull + (uint64_t)g.block_size - 1) / (uint64_t)g.block_size);
   hipStream_t s = as_stream(stream);
   dim3 grid(splits, num_seqs, (num_heads + 127) / 128);
+#define KVQ_MLAD(T)                                                                                       \
+  do {                                                                                                  \
+    static int lds_ok_dev = -2;  /* the >64 KB dynamic LDS opt-in, once per device */                   \
+    int devid = -1;                                                                                     \
+    if (int e = check_hip(hipGetDevice(&devid), "hipGetDevice")) return e;                              \
+    if (lds_ok_dev != devid) {                                                                          \
+      if (int e = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(&mla_decode_kernel<T>),   \
+                                                hipFuncAttributeMaxDynamicSharedMemorySize, kMlaLdsBytes), \
+                            "hipFuncSetAttribute(mla_decode_kernel)"))                                  \
+        return e;                                                                                       \
+      lds_ok_dev = devid;                                                                               \
+    }                                                                                                   \
+    hipLaunchKernelGGL((mla_decode_kernel<T>), grid, dim3(kMlaThreads), kMlaLdsBytes, s, a);            \
+  } while (0)
   switch (q_dtype) {
-    case KVQ_F32: hipLaunchKernelGGL((mla_decode_kernel<KVQ_F32>), grid, dim3(kMlaThreads), 0, s, a); break;
-    case KVQ_BF16: hipLaunchKernelGGL((mla_decode_kernel<KVQ_BF16>), grid, dim3(kMlaThreads), 0, s, a); break;
-    case KVQ_F16: hipLaunchKernelGGL((mla_decode_kernel<KVQ_F16>), grid, dim3(kMlaThreads), 0, s, a); break;
+    case KVQ_F32: KVQ_MLAD(KVQ_F32); break;
+    case KVQ_BF16: KVQ_MLAD(KVQ_BF16); break;
+    case KVQ_F16: KVQ_MLAD(KVQ_F16); break;
     default: return fail(KVQ_EINVAL, "%s: unknown q_dtype %d", op, q_dtype);
   }
+#undef KVQ_MLAD
   int rc = check_hip(hipGetLastError(), "mla_decode_int8 launch");
   if (rc) return rc;
-  dim3 rgrid(num_seqs, (num_heads + 3) / 4);
+  dim3 rgrid(num_seqs, head_groups);
 #define KVQ_MLAR(T)                                                                                           \
-  hipLaunchKernelGGL((mla_reduce_kernel<T>), rgrid, dim3(256), 0, s, out, lse, a.part_o, a.part_lse, seq_lens, \
-                     num_heads, splits)
+  hipLaunchKernelGGL((mla_reduce_kernel<T>), rgrid, dim3(512), 0, s, out, lse, a.part_o, a.part_lse, seq_lens, \
+                     num_heads, head_groups, splits)
   switch (out_dtype) {
     case KVQ_F32: KVQ_MLAR(KVQ_F32); break;
     case KVQ_BF16: KVQ_MLAR(KVQ_BF16); break;
