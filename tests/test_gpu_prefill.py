@@ -1,0 +1,171 @@
+"""GPU parity of chunked prefill and mixed decode + prefill batches over the int8 cache, through
+the C ABI's varlen entry point, against the oracle (causal attention of a query run of q_len
+tokens that ends at the sequence end; the run's own K/V are already in the cache, as in the
+reference's unified kernel, vllm_metax/v1/attention/ops/triton_unified_attention.py:56-246)."""
+import math
+
+import pytest
+import torch
+
+import kvq_testlib as T
+import oracle
+from vllm_metax_amd import _custom_ops as ops
+from vllm_metax_amd import layout as L
+
+pytestmark = pytest.mark.gpu
+
+
+def build(ctx_lens, q_lens, hq, hkv, d, bs, layout="NHD", seed=0, q_dtype=torch.bfloat16, outlier=False):
+    g = torch.Generator().manual_seed(seed)
+    nb = sum((c + bs - 1) // bs for c in ctx_lens) + 5
+    kv, views, lay = T.cpu_cache(nb, bs, hkv, d, layout)
+    T.storage_bytes(kv).fill_(0xFF)                    # NaN scales wherever nothing is written
+    bt = T.make_block_tables(ctx_lens, bs, nb, g)
+    mk = (lambda c: T.outlier_sources((c, hkv, d), g, torch.bfloat16)) if outlier else \
+         (lambda c: torch.randn((c, hkv, d), generator=g).to(torch.bfloat16))
+    T.fill_cache_from_sources(kv, lay, bt, ctx_lens, bs, [mk(c) for c in ctx_lens], [mk(c) for c in ctx_lens])
+    q = torch.randn((sum(q_lens), hq, d), generator=g).to(q_dtype)
+    sl = torch.tensor(ctx_lens, dtype=torch.int32)
+    cu = torch.tensor([0] + torch.tensor(q_lens).cumsum(0).tolist(), dtype=torch.int32)
+    return kv, lay, bt, q, sl, cu
+
+
+def run(dev, kv_cpu, layout, bt, q, sl, cu, max_q, scale, out_dtype=None, want_lse=False, causal=True):
+    kv = T.to_device_cache(kv_cpu, dev, layout)
+    k, v = L.key_value_views(kv)
+    ks, vs = L.scale_views(kv)
+    out = torch.full(q.shape, float("nan"), dtype=out_dtype or q.dtype, device=dev)
+    lse = torch.full(q.shape[:2], float("nan"), dtype=torch.float32, device=dev) if want_lse else None
+    ops.unified_attention(q.to(dev), k, v, out, cu.to(dev), max_q, sl.to(dev), int(sl.max()), scale, causal,
+                          block_table=bt.to(dev), k_scale_cache=ks, v_scale_cache=vs, lse=lse)
+    torch.cuda.synchronize()
+    return (out, lse) if want_lse else out
+
+
+@pytest.mark.parametrize("hq,hkv,d,bs", [
+    (28, 4, 128, 16),     # Qwen2-7B: 7 q heads per kv head (columns do not fill the MFMA tile evenly)
+    (32, 8, 128, 16),     # Llama-3-8B
+    (8, 8, 64, 32),       # no grouping
+    (16, 1, 128, 16),     # 16 q heads on one kv head
+    (4, 2, 256, 16),
+])
+def test_mixed_batch_matches_oracle(gpu_device, hq, hkv, d, bs):
+    ctx = [700, 33, 129, 64, 257, 5]
+    qls = [1, 33, 100, 1, 17, 5]      # decode rows, a pure prefill, chunks with context, a short full run
+    kv, lay, bt, q, sl, cu = build(ctx, qls, hq, hkv, d, bs, seed=hq + d)
+    scale = 1 / math.sqrt(d)
+    want, want_lse = oracle.paged_attn(q, T.storage_bytes(kv), lay, bt, sl, cu, scale, return_lse=True)
+    got, lse = run(gpu_device, kv, "NHD", bt, q, sl, cu, max(qls), scale, want_lse=True)
+    T.assert_close_attn(got, want, what=f"mixed batch {hq}/{hkv} d{d}")
+    torch.testing.assert_close(lse.cpu(), want_lse, atol=5e-3, rtol=1e-3)
+
+
+@pytest.mark.parametrize("layout", ["NHD", "HND"])
+@pytest.mark.parametrize("q_dtype,out_dtype", [(torch.float32, torch.float32), (torch.float16, torch.float16),
+                                               (torch.bfloat16, torch.float32)])
+def test_prefill_dtypes_and_layouts(gpu_device, layout, q_dtype, out_dtype):
+    ctx, qls = [300, 48], [64, 48]
+    kv, lay, bt, q, sl, cu = build(ctx, qls, 8, 2, 128, 16, layout=layout, seed=4, q_dtype=q_dtype)
+    want = oracle.paged_attn(q, T.storage_bytes(kv), lay, bt, sl, cu, 0.09)
+    got = run(gpu_device, kv, layout, bt, q, sl, cu, 64, 0.09, out_dtype=out_dtype)
+    tol = dict(atol=4e-3, rtol=4e-3) if out_dtype == torch.float32 else {}
+    T.assert_close_attn(got, want, what="prefill dtypes", **tol)
+
+
+def test_long_chunk_with_outliers(gpu_device):
+    """A 2048-token chunk on top of 1000 context tokens, 1 % outlier channels (x20)."""
+    ctx, qls = [3048], [2048]
+    kv, lay, bt, q, sl, cu = build(ctx, qls, 8, 2, 128, 16, seed=9, outlier=True)
+    want = oracle.paged_attn(q, T.storage_bytes(kv), lay, bt, sl, cu, 0.0884)
+    got = run(gpu_device, kv, "NHD", bt, q, sl, cu, 2048, 0.0884, out_dtype=torch.float32)
+    T.assert_close_attn(got, want, atol=2e-2, rtol=1e-2, what="long chunk")
+
+
+def test_causality_first_token_sees_only_itself_and_context(gpu_device):
+    """Changing the K/V records of later tokens of a run must not change earlier rows."""
+    ctx, qls = [96], [40]
+    kv, lay, bt, q, sl, cu = build(ctx, qls, 8, 2, 128, 16, seed=12)
+    dev = gpu_device
+    a = run(dev, kv, "NHD", bt, q, sl, cu, 40, 0.1, out_dtype=torch.float32)
+    # scramble the records of the last 10 tokens of the sequence
+    slots = T.slots_for(bt, ctx, 16)[0][-10:]
+    g = torch.Generator().manual_seed(1)
+    oracle.cache_write(torch.randn((10, 2, 128), generator=g).to(torch.bfloat16) * 3,
+                       torch.randn((10, 2, 128), generator=g).to(torch.bfloat16) * 3, T.storage_bytes(kv), lay, slots)
+    b = run(dev, kv, "NHD", bt, q, sl, cu, 40, 0.1, out_dtype=torch.float32)
+    assert torch.equal(a[:30].cpu(), b[:30].cpu()), "rows before the changed tokens moved"
+    assert not torch.equal(a[30:].cpu(), b[30:].cpu())
+
+
+def test_prefill_golden_mixed_batch(gpu_device):
+    import os
+    G = torch.load(os.path.join(os.path.dirname(__file__), "golden", "kvq_golden_small.pt"), weights_only=True)
+    dev = gpu_device
+    hq, hkv, d, bs, nb = (int(G[k]) for k in ("hq", "hkv", "d", "bs", "nb"))
+    kv = L.allocate_kv_cache(nb, bs, hkv, d, device=dev, layout="NHD")
+    T.storage_bytes(kv).copy_(G["cache_bytes"].to(dev))
+    k, v = L.key_value_views(kv)
+    ks, vs = L.scale_views(kv)
+    out = torch.empty(G["q"].shape, dtype=torch.float32, device=dev)
+    lse = torch.empty(G["q"].shape[:2], dtype=torch.float32, device=dev)
+    ops.unified_attention(G["q"].to(dev), k, v, out, G["cu"].to(dev), 5, G["ctx"].to(dev), int(G["ctx"].max()),
+                          float(G["scale"]), True, block_table=G["block_table"].to(dev), k_scale_cache=ks,
+                          v_scale_cache=vs, lse=lse)
+    torch.cuda.synchronize()
+    T.assert_close_attn(out, G["out"], atol=2e-3, rtol=2e-3, what="golden mixed batch")
+    torch.testing.assert_close(lse.cpu(), G["lse"], atol=5e-3, rtol=1e-3)
+
+
+def test_backend_forward_mixed_batch(gpu_device, monkeypatch):
+    """Through the backend mirror: builder metadata -> do_kv_cache_update of the runs' own tokens ->
+    forward, on a batch holding a decode row, a pure prefill and a chunk with context."""
+    import types
+
+    from vllm_metax_amd.v1.attention.backends.int8_attn import Int8AttentionBackend
+
+    monkeypatch.setenv("VLLM_KV_CACHE_LAYOUT", "NHD")
+    dev = gpu_device
+    hq, hkv, d, bs, nb = 8, 2, 128, 16, 24
+    ctx, qls = [50, 20, 90], [1, 20, 7]
+    B = len(ctx)
+    g = torch.Generator().manual_seed(31)
+    shape = Int8AttentionBackend.get_kv_cache_shape(nb, bs, hkv, d, "int8_per_token_head")
+    order = Int8AttentionBackend.get_kv_cache_stride_order()
+    phys = torch.zeros(tuple(shape[i] for i in order), dtype=torch.int8, device=dev)
+    kv_cache = phys.permute(*[order.index(i) for i in range(4)])
+    kv_cpu, views, lay = T.cpu_cache(nb, bs, hkv, d, "NHD")
+    views[2].fill_(1.0)
+    views[3].fill_(1.0)
+    bt = T.make_block_tables(ctx, bs, nb, g)
+    impl = Int8AttentionBackend.get_impl_cls()(hq, d, 0.0884, hkv, kv_cache_dtype="int8_per_token_head")
+    spec = types.SimpleNamespace(block_size=bs, num_kv_heads=hkv, head_size=d, num_q_heads=hq)
+    cfg = types.SimpleNamespace(scheduler_config=types.SimpleNamespace(max_num_seqs=16))
+    builder = Int8AttentionBackend.get_builder_cls()(spec, ["layer.0"], cfg, dev)
+    layer = types.SimpleNamespace(_k_scale=torch.ones(1, device=dev), _v_scale=torch.ones(1, device=dev))
+    slots = T.slots_for(bt, ctx, bs)
+    ksrc = [torch.randn((c, hkv, d), generator=g).to(torch.bfloat16) for c in ctx]
+    vsrc = [torch.randn((c, hkv, d), generator=g).to(torch.bfloat16) for c in ctx]
+    for i, c in enumerate(ctx):                      # earlier steps: everything before the run
+        n = c - qls[i]
+        if n > 0:
+            impl.do_kv_cache_update(layer, ksrc[i][:n].to(dev), vsrc[i][:n].to(dev), kv_cache, slots[i][:n].to(dev))
+        oracle.cache_write(ksrc[i], vsrc[i], T.storage_bytes(kv_cpu), lay, slots[i])
+    new_k = torch.cat([ksrc[i][ctx[i] - qls[i]:] for i in range(B)])
+    new_v = torch.cat([vsrc[i][ctx[i] - qls[i]:] for i in range(B)])
+    new_slots = torch.cat([slots[i][ctx[i] - qls[i]:] for i in range(B)])
+    n_tok = sum(qls)
+    q = torch.randn((n_tok, hq * d), generator=g).to(torch.bfloat16)
+    cu = torch.tensor([0] + torch.tensor(qls).cumsum(0).tolist(), dtype=torch.int32)
+    common = types.SimpleNamespace(
+        num_reqs=B, num_actual_tokens=n_tok, max_query_len=max(qls), max_seq_len=max(ctx),
+        query_start_loc=cu.to(dev), seq_lens=torch.tensor(ctx, dtype=torch.int32, device=dev),
+        block_table_tensor=bt.to(dev), slot_mapping=new_slots.to(dev), causal=True)
+    md = builder.build(0, common)
+    impl.do_kv_cache_update(layer, new_k.to(dev), new_v.to(dev), kv_cache, md.slot_mapping)
+    out = torch.zeros((n_tok, hq * d), dtype=torch.bfloat16, device=dev)
+    impl.forward(layer, q.to(dev), new_k.to(dev), new_v.to(dev), kv_cache, md, out)
+    torch.cuda.synchronize()
+    assert torch.equal(T.storage_bytes(kv_cache).cpu(), T.storage_bytes(kv_cpu)), "cache bytes differ"
+    want = oracle.paged_attn(q.view(n_tok, hq, d), T.storage_bytes(kv_cpu), lay, bt,
+                             torch.tensor(ctx, dtype=torch.int32), cu, 0.0884)
+    T.assert_close_attn(out.view(n_tok, hq, d), want, what="backend forward, mixed batch")

@@ -164,9 +164,17 @@ struct DecodeTile {
   // head 0 and are zeroed.  Returns -1152 * sum(q) of the lane's head: the QK accumulator's
   // start value that cancels the code bias.
   __device__ static float load_q(const AttnIO& io, int64_t row, int hkv, int lane, half8_t (&qb)[KSTEPS]) {
-    const int c = lane & 15, g = lane >> 4;
+    const int c = lane & 15;
     const bool valid = c < io.group;
-    const int64_t base = row * io.q_stride_t + (int64_t)(hkv * io.group + (valid ? c : 0)) * io.q_stride_h + g * 16;
+    return load_q_row(io, row * io.q_stride_t + (int64_t)(hkv * io.group + (valid ? c : 0)) * io.q_stride_h, valid,
+                      lane, qb);
+  }
+
+  // The same for an arbitrary (row, head) per lane: `elem` is the element offset of the lane's
+  // query row (it must be readable also when !valid; the operand is then zero).
+  __device__ static float load_q_row(const AttnIO& io, int64_t elem, bool valid, int lane, half8_t (&qb)[KSTEPS]) {
+    const int g = lane >> 4;
+    const int64_t base = elem + g * 16;
     float f[D / 4];
 #pragma unroll
     for (int ch = 0; ch < D / 64; ++ch) {
