@@ -47,6 +47,10 @@ def make_batch(workload: str, seed: int = 0):
         return dict(hq=32, hkv=8, d=128, bs=16, ctx=ctx, pool=66000)
     if workload == "config1_b4_ctx512":                  # configs[0]
         return dict(hq=32, hkv=8, d=128, bs=16, ctx=[512] * 4, pool=129)
+    if workload == "qwen2_7b_mixed_4x2048_prefill_60_decode":   # configs[4]
+        dctx = torch.randint(512, 4097, (60,), generator=g).tolist()
+        return dict(mixed=True, hq=28, hkv=4, d=128, bs=16, ctx=[2048, 4096, 6144, 8192] + dctx,
+                    qlens=[2048] * 4 + [1] * 60, pool=12000)
     if workload == "mla_decode_b32_h128_ctx4096":        # configs[3]: DeepSeek-V2 MLA decode
         return dict(mla=True, heads=128, r=512, p=64, bs=64, ctx=[4096] * 32, pool=32 * 64 + 8)
     raise SystemExit(f"unknown workload {workload}")
@@ -252,6 +256,103 @@ def mla_main(args, cfg, dev, ops):
     print(json.dumps(res))
 
 
+def mixed_main(args, cfg, dev, ops):
+    """configs[4]: write all new tokens (quantise-on-write), then ONE varlen attention call over the
+    mixed batch.  ctx here is the sequence length INCLUDING the run's own tokens."""
+    from vllm_metax_amd import layout as L
+
+    hq, hkv, d, bs, ctx, qls, pool = (cfg[k] for k in ("hq", "hkv", "d", "bs", "ctx", "qlens", "pool"))
+    B = len(ctx)
+    g = torch.Generator().manual_seed(0)
+    need = [(c + bs - 1) // bs for c in ctx]
+    perm = torch.randperm(pool - 1, generator=g)[: sum(need)] + 1
+    bt = torch.zeros((B, max(need)), dtype=torch.int32)
+    o = 0
+    for i, n in enumerate(need):
+        bt[i, :n] = perm[o:o + n].to(torch.int32)
+        o += n
+    bt_d = bt.to(dev)
+    sl_d = torch.tensor(ctx, dtype=torch.int32, device=dev)
+    cu = torch.tensor([0] + torch.tensor(qls).cumsum(0).tolist(), dtype=torch.int32)
+    cu_d = cu.to(dev)
+    n_tok = int(cu[-1])
+    torch.manual_seed(0)
+    caches = []
+    new_slots = []
+    for i, c in enumerate(ctx):
+        pos = torch.arange(c - qls[i], c)
+        new_slots.append(bt[i, pos // bs].long() * bs + pos % bs)
+    new_slots = torch.cat(new_slots).to(dev)
+    for _ in range(args.layers):
+        kv = L.allocate_kv_cache(pool, bs, hkv, d, device=dev, layout="NHD", fill=0)
+        k, v = L.key_value_views(kv)
+        ks, vs = L.scale_views(kv)
+        ks.fill_(1.0)
+        vs.fill_(1.0)
+        geom = L.geometry_from_views(k, v, ks, vs)
+        for i, c in enumerate(ctx):
+            pos = torch.arange(c, device=dev)
+            slots = bt_d[i, pos // bs].to(torch.int64) * bs + pos % bs
+            ops.reshape_and_cache_flash_per_token_head_quant(
+                torch.randn((c, hkv, d), device=dev).to(torch.bfloat16), torch.randn((c, hkv, d), device=dev).to(torch.bfloat16),
+                k, v, ks, vs, slots, geometry=geom)
+        caches.append(dict(k=k, v=v, ks=ks, vs=vs, geom=geom, kv=kv))
+    q = torch.randn((n_tok, hq, d), device=dev).to(torch.bfloat16)
+    new_k = torch.randn((n_tok, hkv, d), device=dev).to(torch.bfloat16)
+    new_v = torch.randn((n_tok, hkv, d), device=dev).to(torch.bfloat16)
+    out = torch.empty_like(q)
+    ws = torch.empty(ops.paged_attn_workspace_bytes(B, hq, d), dtype=torch.uint8, device=dev)
+    scale = 1.0 / math.sqrt(d)
+
+    def step(layer, write=True, attn=True):
+        c = caches[layer]
+        if write:
+            ops.reshape_and_cache_flash_per_token_head_quant(new_k, new_v, c["k"], c["v"], c["ks"], c["vs"], new_slots,
+                                                             geometry=c["geom"])
+        if attn:
+            ops.unified_attention(q, c["k"], c["v"], out, cu_d, max(qls), sl_d, max(ctx), scale, True, block_table=bt_d,
+                                  k_scale_cache=c["ks"], v_scale_cache=c["vs"], workspace=ws, geometry=c["geom"])
+
+    Lr = args.layers
+    for i in range(args.warmup):
+        step(i % Lr)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step(i % Lr)
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / args.steps
+    n_ev = min(args.steps, 50)
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n_ev)]
+    for i in range(n_ev):
+        step(i % Lr, write=True, attn=False)
+        evs[i][0].record()
+        step(i % Lr, write=False, attn=True)
+        evs[i][1].record()
+    torch.cuda.synchronize()
+    attn_s = sum(a.elapsed_time(b) for a, b in evs) / n_ev * 1e-3
+    # causal prefill flops: 4 D Hq (q_len * cached + q_len (q_len + 1) / 2); decode rows: 4 D Hq ctx
+    flops = sum(4 * d * hq * (ql * (c - ql) + ql * (ql + 1) // 2) for c, ql in zip(ctx, qls))
+    dec_bytes = sum(c for c, ql in zip(ctx, qls) if ql == 1) * hkv * 2 * (d + 4)
+    pre_bytes = sum(c for c, ql in zip(ctx, qls) if ql > 1) * hkv * 2 * (d + 4) + 2 * n_tok * hq * d * 2
+    write_bytes = n_tok * hkv * (2 * d * 2 + 2 * (d + 4))
+    res = {
+        "metric": "int8-KV mixed batch (4 x 2048-token prefill chunks + 60 decode rows): ms per layer",
+        "value": round((dec_bytes + pre_bytes + write_bytes) / dt / 1e9, 1), "unit": "GB/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(dt * 1e3, 5), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None,
+        "dtype": "int8 KV codes, fp16 MFMA operands, fp32 softmax/accumulate, bf16 Q/out", "data": "synthetic",
+        "config": {"workload": args.workload, "batch": B, "new_tokens": n_tok, "sum_ctx": sum(ctx), "q_heads": hq,
+                   "kv_heads": hkv, "head_dim": d, "block_size": bs, "layer_caches_rotated": Lr},
+        "attn_launch_us": round(attn_s * 1e6, 1),
+        "roofline": {"bound": "mfma", "achieved": round(flops / attn_s / 1e12, 1), "peak": MFMA_F16_PEAK_TFLOPS,
+                     "unit": "TFLOP/s", "frac": round(flops / attn_s / 1e12 / MFMA_F16_PEAK_TFLOPS, 4), "traffic": None,
+                     "kernel": "varlen attention launch = decode stream-K + reduce + paged_prefill_kernel",
+                     "algorithmic_flops_per_launch": flops, "algorithmic_bytes_per_launch": dec_bytes + pre_bytes},
+    }
+    print(json.dumps(res))
+
+
 def cpu_baseline(cfg, st, seconds_target=15.0):
     """The reference's CPU path (as-written torch ops, bf16 Q.K / fp32 softmax / bf16 P.V) on a
     bounded sample of the batch: dequantise the sampled sequences' blocks, then ref_paged_attn."""
@@ -311,6 +412,8 @@ def main():
     cfg = make_batch(args.workload)
     if cfg.get("mla"):
         return mla_main(args, cfg, dev, ops)
+    if cfg.get("mixed"):
+        return mixed_main(args, cfg, dev, ops)
     st = build_device_state(cfg, dev, args.layers)
     attn_bytes, write_bytes = algorithmic_bytes(cfg)
     L = args.layers
