@@ -206,15 +206,18 @@ struct DecodeTile {
       }
     }
     float qsum = 0.f;
+    const uint32_t okmask = valid ? 0xffffffffu : 0u;  // a mask, not a select: no branches around the converts
 #pragma unroll
     for (int kk = 0; kk < KSTEPS; ++kk) {
-      half8_t h;
+      const int b = (kk >> 1) * 16 + (kk & 1) * 8;
+      u32x4 hb;
+      hb.x = pack_half2(clamp_half_range(f[b + 0]), clamp_half_range(f[b + 1])) & okmask;
+      hb.y = pack_half2(clamp_half_range(f[b + 2]), clamp_half_range(f[b + 3])) & okmask;
+      hb.z = pack_half2(clamp_half_range(f[b + 4]), clamp_half_range(f[b + 5])) & okmask;
+      hb.w = pack_half2(clamp_half_range(f[b + 6]), clamp_half_range(f[b + 7])) & okmask;
+      const half8_t h = __builtin_bit_cast(half8_t, hb);
 #pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const float x = valid ? clamp_half_range(f[(kk >> 1) * 16 + (kk & 1) * 8 + j]) : 0.f;
-        h[j] = (half_t)x;
-        qsum += (float)h[j];  // the sum of what the MFMA will actually see
-      }
+      for (int j = 0; j < 8; ++j) qsum += (float)h[j];  // the sum of what the MFMA will actually see
       qb[kk] = h;
     }
     qsum += __shfl_xor(qsum, 16, kWave);

@@ -71,6 +71,13 @@ __device__ __forceinline__ float wave_max(float v) {
   for (int o = 32; o >= 1; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, kWave));
   return v;
 }
+// Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits for every global
+// load in flight (vmcnt(0)), which would drain the tile prefetch issued just before it; here the
+// loads stay in flight and the compiler's own wait before their first use still applies.
+__device__ __forceinline__ void lds_barrier() {
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
 __device__ __forceinline__ int wave_max_i32(int v) {
 #pragma unroll
   for (int o = 32; o >= 1; o >>= 1) v = max(v, __shfl_xor(v, o, kWave));

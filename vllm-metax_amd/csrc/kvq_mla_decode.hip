@@ -198,7 +198,7 @@ __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
   for (int t = t_begin; t < t_end; ++t) {
     stage(lds[buf]);
     if (t + 1 < t_end) issue_loads(t + 1);
-    __syncthreads();
+    lds_barrier();
     const uint8_t* tile = lds[buf];
     const float* sck = reinterpret_cast<const float*>(tile + kMlaTileBytes);
 
