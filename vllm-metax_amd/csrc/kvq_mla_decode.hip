@@ -41,11 +41,12 @@ struct MlaArgs {
   const int32_t* block_table;
   int64_t bt_stride;
   const int32_t* seq_lens;
-  // Split states.  part_o is kept in the order the MFMA leaves it in registers, so that every store
-  // and every load of the reduce is one contiguous KiB per wave: [B, S, ceil(H/16)] blocks of
-  // [32 (= d4 * 4 + i)][64 lanes][4 floats], lane (c, g) holding dims 64 d4 + 16 g + 4 i + (0..3) of
-  // head 16 * block + c.  part_lse: [B, S, 16 * ceil(H/16)] log2-domain, -inf for an empty split.
-  float* part_o;
+  // Split states.  part_o holds the locally normalised outputs as fp16, in the order the MFMA leaves
+  // them in registers, so that every store and every load of the reduce is one contiguous 512 bytes
+  // per wave: [B, S, ceil(H/16)] blocks of [32 (= d4 * 4 + i)][64 lanes][4 halves], lane (c, g) holding
+  // dims 64 d4 + 16 g + 4 i + (0..3) of head 16 * block + c.  part_lse: [B, S, 16 * ceil(H/16)] fp32,
+  // log2 domain, -inf for an empty split.
+  uint16_t* part_o;
   float* part_lse;
   int head_groups;  // ceil(H / 16)
   int num_heads;
@@ -101,19 +102,32 @@ __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
   const bool second = tid < kChunksPerHalf - kMlaThreads;
   u32x4 cr[2][2];
   uint32_t scr[2];
-  auto issue_loads = [&](int t) {
+  // Block ids of the two 16-token halves of tile t (scalar loads); a half past the end of the
+  // sequence rereads its last valid half and is masked in the softmax.
+  struct Blocks {
+    int32_t b[2];
+    int32_t s[2];  // first slot of the half inside its block
+  };
+  auto fetch_blocks = [&](int t) __attribute__((always_inline)) {
+    Blocks r;
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
       int tok = t * kTile + 16 * h;
-      tok = tok < len ? tok : t * kTile;  // a half past the end rereads the first half (masked later)
+      tok = tok < len ? tok : ((len - 1) & ~15);
       const int e = (int)__umulhi((uint32_t)tok, a.bs_magic);
-      const int s0 = tok - e * bs;
-      const int64_t blk = scalar_load_i32(bt_row, e);
-      const uint8_t* pb = a.cache + blk * a.g.stride_block;
+      r.s[h] = tok - e * bs;
+      r.b[h] = scalar_load_i32(bt_row, e);
+    }
+    return r;
+  };
+  auto issue_loads = [&](const Blocks& nb) __attribute__((always_inline)) {
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const uint8_t* pb = a.cache + (int64_t)nb.b[h] * a.g.stride_block;
       const __amdgpu_buffer_rsrc_t rr = __builtin_amdgcn_make_buffer_rsrc(
-          const_cast<uint8_t*>(pb + (int64_t)s0 * a.g.stride_row), 0, 0x7fffffff, 0x00020000);
+          const_cast<uint8_t*>(pb + (int64_t)nb.s[h] * a.g.stride_row), 0, 0x7fffffff, 0x00020000);
       const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
-          const_cast<uint8_t*>(pb + a.g.scale_off + (int64_t)s0 * 4), 0, 0x7fffffff, 0x00020000);
+          const_cast<uint8_t*>(pb + a.g.scale_off + (int64_t)nb.s[h] * 4), 0, 0x7fffffff, 0x00020000);
       cr[h][0] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rr, goff[0], 0, 0));
       if (second) cr[h][1] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rr, goff[1], 0, 0));
       scr[h] = __builtin_amdgcn_raw_buffer_load_b32(rs, (uint32_t)((tid & 15) * 4), 0, 0);
@@ -134,7 +148,8 @@ __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
     }
   };
 
-  issue_loads(t_begin);
+  issue_loads(fetch_blocks(t_begin));
+  Blocks nb = fetch_blocks(t_begin + 1);
 
   // ---- absorbed Q of this wave's 16 heads as the MFMA B operand: lane (c = head, g) holds, for
   //      k-step kk, dims 32 kk + 8 g + j
@@ -197,8 +212,9 @@ __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
   int buf = 0;
   for (int t = t_begin; t < t_end; ++t) {
     stage(lds[buf]);
-    if (t + 1 < t_end) issue_loads(t + 1);
+    issue_loads(nb);  // unconditional: past the split's end it rereads a valid half that is never staged
     lds_barrier();
+    nb = fetch_blocks(t + 2);  // after the barrier, whose wait would otherwise expose these scalar loads
     const uint8_t* tile = lds[buf];
     const float* sck = reinterpret_cast<const float*>(tile + kMlaTileBytes);
 
@@ -307,17 +323,15 @@ __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
   if (!wave_ok) return;
   const float corr = kCodeBias * psum[0];
   const float inv = 1.0f / (l * kPScale);
-  float* po = a.part_o + pblock * (16 * kMlaR) + lane * 4;
+  uint16_t* po = a.part_o + pblock * (16 * kMlaR) + lane * 4;
 #pragma unroll
   for (int d4 = 0; d4 < kMlaDT / 4; ++d4) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      floatx4 v;
-      v.x = (o[4 * d4 + 0][i] - corr) * inv;
-      v.y = (o[4 * d4 + 1][i] - corr) * inv;
-      v.z = (o[4 * d4 + 2][i] - corr) * inv;
-      v.w = (o[4 * d4 + 3][i] - corr) * inv;
-      *reinterpret_cast<floatx4*>(po + (d4 * 4 + i) * 256) = v;
+      u32x2 v;  // a locally normalised output is a convex mix of dequantised rows: within fp16 range
+      v.x = pack_half2(clamp_half_range((o[4 * d4 + 0][i] - corr) * inv), clamp_half_range((o[4 * d4 + 1][i] - corr) * inv));
+      v.y = pack_half2(clamp_half_range((o[4 * d4 + 2][i] - corr) * inv), clamp_half_range((o[4 * d4 + 3][i] - corr) * inv));
+      *reinterpret_cast<u32x2*>(po + (d4 * 4 + i) * 256) = v;
     }
   }
   if (g == 0) a.part_lse[pblock * 16 + c] = m + __builtin_amdgcn_logf(l);
@@ -327,7 +341,7 @@ __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
 // grid (B, ceil(H/16)), 8 waves; wave w combines the d4 = w slice of the block's 16 heads, lane (c, g)
 // as in the split state layout.
 template <int ODT>
-__global__ __launch_bounds__(512) void mla_reduce_kernel(void* out, float* lse, const float* part_o,
+__global__ __launch_bounds__(512) void mla_reduce_kernel(void* out, float* lse, const uint16_t* part_o,
                                                          const float* part_lse, const int32_t* seq_lens,
                                                          int num_heads, int head_groups, int num_splits) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -337,28 +351,37 @@ __global__ __launch_bounds__(512) void mla_reduce_kernel(void* out, float* lse, 
   const bool head_ok = head < num_heads;
   const int64_t lstride = (int64_t)head_groups * 16;                    // part_lse stride between splits
   const float* pl = part_lse + ((int64_t)seq * num_splits * head_groups + hgroup) * 16 + c;
-  const float* po = part_o + ((int64_t)seq * num_splits * head_groups + hgroup) * (16 * kMlaR) + (wave * 4 * 64 + lane) * 4;
+  const uint16_t* po = part_o + ((int64_t)seq * num_splits * head_groups + hgroup) * (16 * kMlaR) + (wave * 4 * 64 + lane) * 4;
   const int64_t ostride = (int64_t)head_groups * 16 * kMlaR;            // part_o stride between splits
   floatx4 acc[4];
 #pragma unroll
   for (int r = 0; r < 4; ++r) acc[r] = (floatx4){0.f, 0.f, 0.f, 0.f};
   float mx = -INFINITY;
-  if (seq_lens[seq] > 0)
-    for (int j = 0; j < num_splits; ++j) mx = fmaxf(mx, pl[j * lstride]);
+  const bool live = seq_lens[seq] > 0;
+#pragma unroll 8
+  for (int j = 0; j < num_splits; ++j) mx = fmaxf(mx, pl[j * lstride]);
+  mx = live ? mx : -INFINITY;
+  const float mref = mx == -INFINITY ? 0.f : mx;
   float den = 0.f;
-  if (mx != -INFINITY) {
-#pragma unroll 4
-    for (int j = 0; j < num_splits; ++j) {
-      const float lj = pl[j * lstride];
-      const float wj = lj == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(lj - mx);
-      if (__builtin_amdgcn_ballot_w64(wj != 0.f) == 0) continue;       // split empty for the whole block
-      den += wj;
-      const float* pj = po + j * ostride;
+  // every load below is unconditional and a split that holds nothing (lse = -inf; its state rows were
+  // never written) is removed with a bit mask on the loaded words: a select on the value would be
+  // turned into a branch around the load, and the loads of successive splits would run one by one
+#pragma unroll 8
+  for (int j = 0; j < num_splits; ++j) {
+    const float lj = pl[j * lstride];
+    const float wj = (live && lj != -INFINITY) ? __builtin_amdgcn_exp2f(lj - mref) : 0.f;
+    const uint32_t keep = wj != 0.f ? 0xffffffffu : 0u;
+    den += wj;
+    const uint16_t* pj = po + j * ostride;
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const floatx4 v = *reinterpret_cast<const floatx4*>(pj + r * 256);
-        acc[r] += (wj != 0.f ? v : (floatx4){0.f, 0.f, 0.f, 0.f}) * wj;
-      }
+    for (int r = 0; r < 4; ++r) {
+      const u32x2 hv = *reinterpret_cast<const u32x2*>(pj + r * 256);
+      const uint32_t h0 = hv.x & keep, h1 = hv.y & keep;
+      const half2_t a0 = __builtin_bit_cast(half2_t, h0), a1 = __builtin_bit_cast(half2_t, h1);
+      acc[r].x += (float)a0.x * wj;
+      acc[r].y += (float)a0.y * wj;
+      acc[r].z += (float)a1.x * wj;
+      acc[r].w += (float)a1.y * wj;
     }
   }
   if (!head_ok) return;
@@ -398,7 +421,7 @@ size_t kvq_mla_decode_workspace_bytes(int max_num_seqs, int num_heads, int kv_lo
   size_t items = 2 * (size_t)kvq::num_cus() / groups;
   if (items < (size_t)max_num_seqs) items = (size_t)max_num_seqs;
   const size_t heads_padded = ((size_t)num_heads + 15) / 16 * 16;
-  return items * heads_padded * ((size_t)kv_lora_rank + 1) * sizeof(float);
+  return items * heads_padded * ((size_t)kv_lora_rank * sizeof(uint16_t) + sizeof(float));
 }
 
 int kvq_mla_decode_int8(void* out, int out_dtype, float* lse, const void* q, int q_dtype, int64_t q_stride_b,
@@ -423,7 +446,8 @@ int kvq_mla_decode_int8(void* out, int out_dtype, float* lse, const void* q, int
               "%s: q rows must be 4-byte aligned", op);
   const int splits = mla_num_splits(0, num_seqs, num_heads);
   const int head_groups = (num_heads + 15) / 16;
-  const size_t need = (size_t)num_seqs * head_groups * 16 * splits * ((size_t)kMlaR + 1) * sizeof(float);
+  const size_t states = (size_t)num_seqs * head_groups * 16 * splits;
+  const size_t need = states * ((size_t)kMlaR * sizeof(uint16_t) + sizeof(float));
   KVQ_REQUIRE(workspace != nullptr && workspace_bytes >= need && ((uintptr_t)workspace % 16) == 0,
               "%s: workspace of %zu bytes (16-byte aligned) required, got %zu", op, need, workspace_bytes);
   MlaArgs a{};
@@ -435,8 +459,8 @@ int kvq_mla_decode_int8(void* out, int out_dtype, float* lse, const void* q, int
   a.block_table = block_table;
   a.bt_stride = bt_stride;
   a.seq_lens = seq_lens;
-  a.part_o = static_cast<float*>(workspace);
-  a.part_lse = a.part_o + (size_t)num_seqs * head_groups * 16 * splits * kMlaR;
+  a.part_lse = static_cast<float*>(workspace);  // fp32 first, so both arrays keep their alignment
+  a.part_o = reinterpret_cast<uint16_t*>(a.part_lse + states);
   a.head_groups = head_groups;
   a.num_heads = num_heads;
   a.num_splits = splits;

@@ -117,9 +117,14 @@ __global__ __launch_bounds__(256) void paged_decode_streamk_reduce_kernel(Stream
   const int seq = blockIdx.x;
   const int B = a.num_seqs;
   if (head >= a.io.num_q_heads) return;
-  if (a.cu_seqlens_q != nullptr && (a.cu_seqlens_q[seq + 1] - a.cu_seqlens_q[seq]) != 1) return;
-  const int64_t row = a.cu_seqlens_q ? (int64_t)a.cu_seqlens_q[seq] : (int64_t)seq;
-  const int ntiles = decode_tiles(a.seq_lens, a.cu_seqlens_q, seq, B);
+  // all the loads that depend on nothing but the arguments go out together, before the first branch
+  const int q0 = a.cu_seqlens_q ? a.cu_seqlens_q[seq] : seq;
+  const int q1 = a.cu_seqlens_q ? a.cu_seqlens_q[seq + 1] : seq + 1;
+  const int len = a.seq_lens[seq];
+  int n_first = decode_tiles(a.seq_lens, a.cu_seqlens_q, lane, B);  // first 64 sequences of the scan
+  if (q1 - q0 != 1) return;
+  const int64_t row = q0;
+  const int ntiles = len > 0 ? (len + kTile - 1) / kTile : 0;
   if (ntiles == 0) {  // empty sequence: defined output (zeros, lse = -inf)
     for (int i = 0; i < V; ++i)
       store_act<ODT>(a.io.out, row * a.io.out_stride_t + (int64_t)head * a.io.out_stride_h + lane * V + i, 0.f);
@@ -128,7 +133,7 @@ __global__ __launch_bounds__(256) void paged_decode_streamk_reduce_kernel(Stream
   }
   int64_t total = 0, start = 0;
   for (int base = 0; base < B; base += kWave) {
-    int n = decode_tiles(a.seq_lens, a.cu_seqlens_q, base + lane, B);
+    int n = base == 0 ? n_first : decode_tiles(a.seq_lens, a.cu_seqlens_q, base + lane, B);
     const int incl = wave_incl_scan(n, lane);
     if (seq >= base && seq < base + kWave) start = total + __builtin_amdgcn_readlane(incl - n, seq - base);
     total += __builtin_amdgcn_readlane(incl, 63);
@@ -147,25 +152,30 @@ __global__ __launch_bounds__(256) void paged_decode_streamk_reduce_kernel(Stream
   for (int wb = w_first; wb <= w_last; wb += kWave) {
     const int w = wb + lane;
     const bool live = w <= w_last && wg_tile_begin(w, total, P) < wg_tile_begin(w + 1, total, P);
-    const int64_t slot = (int64_t)w + seq;
-    const float mj = live ? a.part_ml[(slot * a.io.num_q_heads + head) * 2 + 0] : -INFINITY;
-    const float lj = live ? a.part_ml[(slot * a.io.num_q_heads + head) * 2 + 1] : 0.f;
+    // loads are unconditional (clamped to the sequence's last workgroup) and what they return is
+    // removed with a bit mask where the slot holds nothing: a select on the loaded value becomes a
+    // branch around the load, and the loads of successive slots would then run one after another
+    const int64_t slot = (int64_t)min(w, w_last) + seq;
+    const uint32_t keep = live ? 0xffffffffu : 0u;
+    const float mj_raw = a.part_ml[(slot * a.io.num_q_heads + head) * 2 + 0];
+    const float lj_raw = a.part_ml[(slot * a.io.num_q_heads + head) * 2 + 1];
+    const float mj = live ? as_f32(as_u32(mj_raw) & keep) : -INFINITY;
+    const float lj = as_f32(as_u32(lj_raw) & keep);
     const float m_new = fmaxf(m, wave_max(mj));
     const float ca = __builtin_amdgcn_exp2f(m - m_new);  // first chunk: exp2(-inf) = 0
-    const float ej = __builtin_amdgcn_exp2f(mj - m_new);  // dead lanes: exp2(-inf) = 0
+    const float ej = live ? __builtin_amdgcn_exp2f(mj - m_new) : 0.f;
     l = l * ca + wave_sum(lj * ej);
 #pragma unroll
     for (int i = 0; i < V; ++i) acc[i] *= ca;
     m = m_new;
-    const uint64_t mask = __builtin_amdgcn_ballot_w64(live);
     const int count = min(kWave, w_last - wb + 1);
 #pragma unroll 4
     for (int k = 0; k < count; ++k) {
-      if (!((mask >> k) & 1)) continue;
       const float wk = __shfl(ej, k, kWave);  // the partial outputs are unnormalised sums
+      const uint32_t kk = wk != 0.f ? 0xffffffffu : 0u;
       const float* po = a.part_o + (((int64_t)(wb + k) + seq) * a.io.num_q_heads + head) * (int64_t)D + lane * V;
 #pragma unroll
-      for (int i = 0; i < V; ++i) acc[i] += po[i] * wk;
+      for (int i = 0; i < V; ++i) acc[i] += as_f32(as_u32(po[i]) & kk) * wk;
     }
   }
   const float inv = 1.0f / l;
