@@ -69,7 +69,10 @@ def test_ragged_lengths_fp32_out(gpu_device, ctx):
 
 
 @pytest.mark.parametrize("hq,hkv,d,bs", [(28, 4, 128, 16), (8, 8, 128, 16), (16, 1, 128, 32), (8, 2, 64, 16),
-                                         (4, 2, 256, 16), (32, 16, 128, 64)])
+                                         (4, 2, 256, 16), (32, 16, 128, 64),
+                                         # head counts of the reference's paged-attention grid
+                                         # (tests/kernels/attention/test_attention.py:31-47) at the built head sizes
+                                         (40, 40, 128, 16), (64, 8, 128, 32), (40, 40, 256, 32), (64, 8, 64, 16)])
 def test_head_and_block_shapes(gpu_device, hq, hkv, d, bs):
     ctx = [200, 77, 1025, 48]
     kv, lay, bt, q, sl, cu = build_case(ctx, hq, hkv, d, bs, "NHD", hq + d)
@@ -146,6 +149,43 @@ def test_fixed_partitions_v2_contract(gpu_device):
     w2, wl2 = oracle.splitk_reduce(wtmp, wml, wes, sl, 512, return_lse=True)
     torch.testing.assert_close(out2.cpu(), w2, atol=1e-5, rtol=1e-4)
     torch.testing.assert_close(lse.cpu(), wl2, atol=1e-4, rtol=1e-5)
+
+
+@pytest.mark.parametrize("q_lens", [[1, 1, 1], [1, 5, 129]])
+def test_block_size_does_not_change_the_result(gpu_device, q_lens):
+    """The same tokens paged with 16-, 32-, 64- and 128-token blocks give bit-identical outputs (the
+    page-size self-consistency check of tests/kernels/attention/test_triton_decode_attention.py:12-90),
+    for decode rows and for the reference's mixed batch (query, context) = (1, 1328), (5, 18), (129, 463)
+    (tests/kernels/attention/test_triton_unified_attention.py:81-83)."""
+    dev = gpu_device
+    ctx = [1328, 18, 463]
+    hq, hkv, d = 32, 8, 128
+    g = torch.Generator().manual_seed(77)
+    ks = [torch.randn((c, hkv, d), generator=g).to(torch.bfloat16) for c in ctx]
+    vs = [torch.randn((c, hkv, d), generator=g).to(torch.bfloat16) for c in ctx]
+    q = torch.randn((sum(q_lens), hq, d), generator=g).to(torch.bfloat16)
+    cu = torch.tensor([0] + torch.tensor(q_lens).cumsum(0).tolist(), dtype=torch.int32)
+    sl = torch.tensor(ctx, dtype=torch.int32)
+    outs = []
+    for bs in (16, 32, 64, 128):
+        nb = sum((c + bs - 1) // bs for c in ctx) + 3
+        kv, views, lay = T.cpu_cache(nb, bs, hkv, d, "NHD")
+        T.storage_bytes(kv).fill_(0xFF)
+        bt = T.make_block_tables(ctx, bs, nb, torch.Generator().manual_seed(bs))
+        T.fill_cache_from_sources(kv, lay, bt, ctx, bs, ks, vs)
+        kvd = T.to_device_cache(kv, dev, "NHD")
+        k, v = L.key_value_views(kvd)
+        ksc, vsc = L.scale_views(kvd)
+        out = torch.full(q.shape, float("nan"), dtype=torch.float32, device=dev)
+        ops.unified_attention(q.to(dev), k, v, out, cu.to(dev), max(q_lens), sl.to(dev), max(ctx), 0.0884, True,
+                              block_table=bt.to(dev), k_scale_cache=ksc, v_scale_cache=vsc)
+        torch.cuda.synchronize()
+        outs.append(out.cpu())
+        if bs == 16:
+            want = oracle.paged_attn(q, T.storage_bytes(kv), lay, bt, sl, cu, 0.0884)
+            T.assert_close_attn(out, want, atol=4e-3, rtol=4e-3, what="reference mixed batch")
+    for o in outs[1:]:
+        assert torch.equal(o, outs[0]), "block size changed the result"
 
 
 def test_block_permutation_invariance_on_device(gpu_device):
