@@ -8,6 +8,8 @@
 // window and turned into fp16 operands once per tile, and each operand feeds NT MFMAs.
 // One wavefront = one (sequence, query block, kv head); it streams tiles 0 .. last visible tile
 // with the decode tile's load / stage machinery and applies the causal limit per column.
+#include <type_traits>
+
 #include "kvq_attn_core.cuh"
 
 namespace kvq {
@@ -304,47 +306,89 @@ __global__ __launch_bounds__(WPW * 64) void paged_prefill_kernel(PrefillArgs a) 
 // ---------------------------------------------------------------------------------------------
 // Workgroup-shared tile: the compute-bound shape (long query runs).
 //
-// Four or eight waves share one kv head's 32-token tile.  The records are loaded cooperatively (each
-// wave issues a quarter of the 16-byte chunk loads), dropped raw into LDS, expanded ONCE per
-// workgroup to fp16 -- K as [token][dim], V transposed as [dim][token] in the token order the
-// P~ operand has -- and every wave then feeds its 16 * NT columns straight from the fp16 tile:
-// two 16-byte LDS reads per MFMA group instead of a per-wave byte-permute expansion.  The code
-// bias 1152 is taken out during the expansion (exact in fp16), so no correction terms remain.
-template <int D, int QDT, int ODT, int NT, int WAVES>
-struct FlashPrefill {
+// Four waves share one kv head's 32-token tile.  The records are loaded cooperatively (16-byte
+// chunks, every wave the same loads in the same order, two tiles ahead), dropped raw into LDS,
+// expanded ONCE per workgroup to fp16 -- K as [token][dim], V transposed as [dim][token] in the
+// token order the P~ operand has, the code bias 1152 taken out (exact in fp16) -- and every wave
+// feeds its 32 columns straight from the fp16 tile with MFMA 32x32x16: a 16-byte LDS read per lane
+// is the A operand of 32 Ki flop, and a lane holds 16 tokens of ONE column, so the column maximum
+// needs one cross-lane step.  Raw and fp16 tiles are double-buffered, which leaves one barrier per
+// tile.  Two workgroups fit a CU; they drift apart, so one workgroup's LDS-bound phase runs under
+// the other's ALU- and MFMA-bound phases.
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+template <int D, int QDT, int ODT>
+struct Flash32 {
   using DTile = DecodeTile<D, QDT, ODT>;
-  static constexpr int KSTEPS = D / 32;
-  static constexpr int DT = D / 16;
+  static constexpr int WAVES = 4;
+  static constexpr int KS = D / 16;                      // k-steps of the QK product
+  static constexpr int MT = D / 32;                      // 32-dim row tiles of O^T
   static constexpr int RAW_PITCH = DTile::PITCH;
   static constexpr int RAW_BYTES = kTile * RAW_PITCH;
-  static constexpr int K_PITCH = 2 * D + 16;            // bytes per fp16 K row (token)
+  static constexpr int K_PITCH = 2 * D + 16;
   static constexpr int K_BYTES = kTile * K_PITCH;
-  static constexpr int V_PITCH = 2 * kTile + 16;        // bytes per fp16 V^T row (dim): 32 tokens
+  static constexpr int V_PITCH = 2 * kTile + 16;
   static constexpr int V_BYTES = D * V_PITCH;
-  static constexpr int SC_BYTES = 64 * 4;
-  static constexpr int BUF_BYTES = K_BYTES + V_BYTES + SC_BYTES;
-  static constexpr int LDS_BYTES = 2 * RAW_BYTES + 2 * BUF_BYTES;   // raw and fp16 tiles both double-buffered
-  static constexpr int COLS = 16 * NT * WAVES;           // columns per workgroup
+  static constexpr int BUF_BYTES = K_BYTES + V_BYTES + 64 * 4;
+  static constexpr int LDS_BYTES = 2 * RAW_BYTES + 2 * BUF_BYTES;
+  static constexpr int COLS = 32 * WAVES;
 
-  struct State {
-    floatx4 o[NT][DT];
-    float m[NT], l[NT];
-  };
-
-  // two biased code bytes -> two fp16 codes (bias removed)
-  __device__ static uint32_t to_half2(uint32_t x, bool upper) {
+  __device__ static __forceinline__ uint32_t to_half2(uint32_t x, bool upper) {
     const half2_t bias = {(half_t)kCodeBias, (half_t)kCodeBias};
     const half2_t v = __builtin_bit_cast(half2_t, bytes_to_half2(x, upper)) - bias;
     return __builtin_bit_cast(uint32_t, v);
   }
 
-  // Expand the raw tile into buffer `buf`: thread t converts one 16-code K chunk and one
-  // 4-token x 4-dim V block; wave 0 stages the 64 scales.
+  // Q of the lane's column as the B operand: lane (c = lane & 31, g = lane >> 5) holds, for k-step
+  // ks, dims 16 ks + 8 g + j.
+  __device__ static __forceinline__ void load_q(const AttnIO& io, int64_t elem, bool valid, int lane, half8_t (&qb)[KS]) {
+    const int g = lane >> 5;
+    const uint32_t okmask = valid ? 0xffffffffu : 0u;
+    u32x4 raw[QDT == KVQ_F32 ? 1 : KS];
+    if constexpr (QDT != KVQ_F32) {
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks)
+        raw[ks] = *reinterpret_cast<const u32x4_a4*>(reinterpret_cast<const uint16_t*>(io.q) + elem + 16 * ks + 8 * g);
+    }
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      float f[8];
+      if constexpr (QDT == KVQ_F32) {
+        const float* p = reinterpret_cast<const float*>(io.q) + elem + 16 * ks + 8 * g;
+        const floatx4 v0 = *reinterpret_cast<const floatx4_a4*>(p), v1 = *reinterpret_cast<const floatx4_a4*>(p + 4);
+        f[0] = v0.x; f[1] = v0.y; f[2] = v0.z; f[3] = v0.w; f[4] = v1.x; f[5] = v1.y; f[6] = v1.z; f[7] = v1.w;
+      } else {
+        const u32x4 v = raw[ks];
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+          const uint32_t e = v[w];
+          if constexpr (QDT == KVQ_BF16) {
+            f[2 * w] = as_f32(e << 16);
+            f[2 * w + 1] = as_f32(e & 0xffff0000u);
+          } else {
+            const half2_t hh = __builtin_bit_cast(half2_t, e);
+            f[2 * w] = (float)hh.x;
+            f[2 * w + 1] = (float)hh.y;
+          }
+        }
+      }
+      u32x4 hb;
+      hb.x = pack_half2(clamp_half_range(f[0]), clamp_half_range(f[1])) & okmask;
+      hb.y = pack_half2(clamp_half_range(f[2]), clamp_half_range(f[3])) & okmask;
+      hb.z = pack_half2(clamp_half_range(f[4]), clamp_half_range(f[5])) & okmask;
+      hb.w = pack_half2(clamp_half_range(f[6]), clamp_half_range(f[7])) & okmask;
+      qb[ks] = __builtin_bit_cast(half8_t, hb);
+    }
+  }
+
+  // Raw tile -> fp16 K [token][dim] and V^T [dim][position]; token t of the tile sits at position
+  // (t/16)*16 + ((t%8)/4)*8 + ((t/8)%2)*4 + t%4, the order in which the 32x32 S accumulator hands a
+  // lane its tokens.  One thread converts one 16-code K chunk and one 4-token x 4-dim V block.
   __device__ static __forceinline__ void expand(const uint8_t* raw, uint8_t* buf, int tid, float sc_mul, uint32_t l_sc) {
-    constexpr int KCH = D / 16;  // K chunks per token
+    constexpr int KCH = D / 16;
     if (tid < kTile * KCH) {
       const int tok = tid / KCH, ch = tid % KCH;
-      u32x4 w = *reinterpret_cast<const u32x4*>(raw + tok * RAW_PITCH + 16 * ch);
+      const u32x4 w = *reinterpret_cast<const u32x4*>(raw + tok * RAW_PITCH + 16 * ch);
       u32x4 lo, hi;
 #pragma unroll
       for (int i = 0; i < 2; ++i) {
@@ -358,19 +402,16 @@ struct FlashPrefill {
       *reinterpret_cast<u32x4*>(buf + tok * K_PITCH + 32 * ch) = lo;
       *reinterpret_cast<u32x4*>(buf + tok * K_PITCH + 32 * ch + 16) = hi;
     }
-    // with 8 waves the V blocks go to the upper four waves, so both halves of the work run side by side
-    const int vt = WAVES == 8 ? tid - 256 : tid;
-    if (vt >= 0 && vt < 8 * (D / 4)) {
-      const int tg = vt & 7, dq = vt >> 3;         // tokens 4tg .. 4tg+3, dims 4dq .. 4dq+3
+    if (tid < 8 * (D / 4)) {
+      const int tg = tid & 7, dq = tid >> 3;
       uint32_t t[4];
 #pragma unroll
       for (int a = 0; a < 4; ++a)
         t[a] = *reinterpret_cast<const uint32_t*>(raw + (4 * tg + a) * RAW_PITCH + (D + 4) + 4 * dq) ^ 0x80808080u;
-      // byte b of token a -> x01/x23 hold (tok0,tok1)/(tok2,tok3) interleaved per byte pair
       const uint32_t a01 = perm(t[1], t[0], 0x05010400u), b01 = perm(t[1], t[0], 0x07030602u);
       const uint32_t a23 = perm(t[3], t[2], 0x05010400u), b23 = perm(t[3], t[2], 0x07030602u);
-      // position of token 4tg in the P~ operand order: 8 * (tg % 4) + 4 * (tg / 4)
-      uint8_t* vrow = buf + K_BYTES + (4 * dq) * V_PITCH + 2 * (8 * (tg & 3) + 4 * (tg >> 2));
+      const int pos = (tg >> 2) * 16 + (tg & 1) * 8 + ((tg >> 1) & 1) * 4;
+      uint8_t* vrow = buf + K_BYTES + (4 * dq) * V_PITCH + 2 * pos;
 #pragma unroll
       for (int b = 0; b < 4; ++b) {
         const uint32_t p01 = (b < 2) ? a01 : b01, p23 = (b < 2) ? a23 : b23;
@@ -386,65 +427,60 @@ struct FlashPrefill {
     }
   }
 
+  // One tile for the wave's 32 columns.  S^T[32 tokens, 32 columns]: lane (c = column, g) holds
+  // token (i/4)*8 + 4g + i%4 in register i.
   template <bool MASK>
-  __device__ static __forceinline__ void compute(const uint8_t* buf, const half8_t (&qb)[NT][KSTEPS], const int (&limit)[NT], int t,
-                                 int lane, State& st) {
-    const int c = lane & 15, g = lane >> 4;
+  __device__ static __forceinline__ void compute(const uint8_t* buf, const half8_t (&qb)[KS], int limit, int t, int lane,
+                                                 floatx16 (&o)[MT], float& m, float& l) {
+    const int c = lane & 31, g = lane >> 5;
     const float* sc = reinterpret_cast<const float*>(buf + K_BYTES + V_BYTES);
-    const floatx4 ks0 = *reinterpret_cast<const floatx4*>(sc + 4 * g);
-    const floatx4 ks1 = *reinterpret_cast<const floatx4*>(sc + 16 + 4 * g);
-    const floatx4 vs0 = *reinterpret_cast<const floatx4*>(sc + 32 + 4 * g);
-    const floatx4 vs1 = *reinterpret_cast<const floatx4*>(sc + 48 + 4 * g);
+    floatx16 s;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) s[i] = 0.f;
+    const uint8_t* krow = buf + c * K_PITCH + g * 16;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const half8_t ka = *reinterpret_cast<const half8_t*>(krow + 32 * ks);
+      s = __builtin_amdgcn_mfma_f32_32x32x16_f16(ka, qb[ks], s, 0, 0, 0);
+    }
     const int tok_base = t * kTile + 4 * g;
-    half8_t p_op[NT];
-    // K operand of k-step kk: dims (kk>>1)*64 + g*16 + (kk&1)*8 .. +7, the order Q is held in
-    const uint8_t* krow = buf + c * K_PITCH + g * 32;
+    float mloc = -INFINITY;
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt) {
-      floatx4 s[2];
+    for (int q = 0; q < 4; ++q) {
+      const floatx4 ksc = *reinterpret_cast<const floatx4*>(sc + 8 * q + 4 * g);
 #pragma unroll
-      for (int mt = 0; mt < 2; ++mt) {
-        s[mt] = (floatx4){0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int kk = 0; kk < KSTEPS; ++kk) {
-          const half8_t ka = *reinterpret_cast<const half8_t*>(krow + mt * 16 * K_PITCH + (kk >> 1) * 128 + (kk & 1) * 16);
-          s[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka, qb[nt][kk], s[mt], 0, 0, 0);
-        }
+      for (int r = 0; r < 4; ++r) {
+        float x = s[4 * q + r] * ksc[r];
+        if constexpr (MASK) x = ((tok_base + q * 8 + r) < limit) ? x : -INFINITY;
+        s[4 * q + r] = x;
+        mloc = fmaxf(mloc, x);
       }
-      float logit[8];
-      float mloc = -INFINITY;
+    }
+    mloc = fmaxf(mloc, __shfl_xor(mloc, 32, kWave));
+    const float m_new = fmaxf(m, mloc);
+    const float m_ref = m_new == -INFINITY ? 0.f : m_new;  // see PrefillTile::qk_softmax
+    if (__builtin_amdgcn_ballot_w64(m_new > m) != 0) {
+      const float alpha = __builtin_amdgcn_exp2f(m - m_ref);
+      l *= alpha;
 #pragma unroll
-      for (int mt = 0; mt < 2; ++mt) {
+      for (int mt = 0; mt < MT; ++mt) o[mt] *= alpha;
+    }
+    m = m_new;
+    half8_t p_op[2];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          float x = s[mt][i] * (mt ? ks1 : ks0)[i];
-          if constexpr (MASK) x = ((tok_base + mt * 16 + i) < limit[nt]) ? x : -INFINITY;
-          logit[mt * 4 + i] = x;
-          mloc = fmaxf(mloc, x);
-        }
-      }
-      mloc = fmaxf(mloc, __shfl_xor(mloc, 16, kWave));
-      mloc = fmaxf(mloc, __shfl_xor(mloc, 32, kWave));
-      const float m_new = fmaxf(st.m[nt], mloc);
-      const float m_ref = m_new == -INFINITY ? 0.f : m_new;  // see PrefillTile::qk_softmax
-      if (__builtin_amdgcn_ballot_w64(m_new > st.m[nt]) != 0) {
-        const float alpha = __builtin_amdgcn_exp2f(st.m[nt] - m_ref);
-        st.l[nt] *= alpha;
-#pragma unroll
-        for (int dt = 0; dt < DT; ++dt) st.o[nt][dt] *= alpha;
-      }
-      st.m[nt] = m_new;
+    for (int kt = 0; kt < 2; ++kt) {
       float pt[8];
 #pragma unroll
-      for (int mt = 0; mt < 2; ++mt) {
+      for (int h = 0; h < 2; ++h) {
+        const int q = 2 * kt + h;
+        const floatx4 vsc = *reinterpret_cast<const floatx4*>(sc + 32 + 8 * q + 4 * g);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int j = mt * 4 + i;
-          const float p = __builtin_amdgcn_exp2f(logit[j] - m_ref);
-          st.l[nt] += p;
-          float x = p * (mt ? vs1 : vs0)[i];
-          if constexpr (MASK) x = ((tok_base + mt * 16 + i) < limit[nt]) ? x : 0.f;
-          pt[j] = x;
+        for (int r = 0; r < 4; ++r) {
+          const float p = __builtin_amdgcn_exp2f(s[4 * q + r] - m_ref);
+          l += p;
+          float x = p * vsc[r];
+          if constexpr (MASK) x = ((tok_base + q * 8 + r) < limit) ? x : 0.f;
+          pt[4 * h + r] = x;
         }
       }
       u32x4 pb;
@@ -452,55 +488,23 @@ struct FlashPrefill {
       pb.y = pack_half2(pt[2], pt[3]);
       pb.z = pack_half2(pt[4], pt[5]);
       pb.w = pack_half2(pt[6], pt[7]);
-      p_op[nt] = __builtin_bit_cast(half8_t, pb);
+      p_op[kt] = __builtin_bit_cast(half8_t, pb);
     }
-    // V^T operand of dim tile dt: row dt*16 + c, token positions 8g .. 8g+7
     const uint8_t* vrow = buf + K_BYTES + c * V_PITCH + g * 16;
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt) {
-      const half8_t va = *reinterpret_cast<const half8_t*>(vrow + dt * 16 * V_PITCH);
+    for (int mt = 0; mt < MT; ++mt) {
 #pragma unroll
-      for (int nt = 0; nt < NT; ++nt)
-        st.o[nt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va, p_op[nt], st.o[nt][dt], 0, 0, 0);
-    }
-  }
-
-  // Lane (c, g) holds O[column c][dim dt*16 + 4g + i] in o[dt][i].
-  __device__ static void emit(const AttnIO& io, int nt, int64_t row, int head, bool valid, int lane, const State& st) {
-    float l = st.l[nt];
-    l += __shfl_xor(l, 16, kWave);
-    l += __shfl_xor(l, 32, kWave);
-    if (!valid) return;
-    const int g = lane >> 4;
-    const float mul = l > 0.f ? 1.0f / (l * kPScale) : 0.f;
-    const int64_t base = row * io.out_stride_t + (int64_t)head * io.out_stride_h + 4 * g;
-#pragma unroll
-    for (int dt = 0; dt < DT; ++dt) {
-      const floatx4 v = st.o[nt][dt] * mul;
-      if constexpr (ODT == KVQ_F32) {
-        *reinterpret_cast<floatx4_a4*>(reinterpret_cast<float*>(io.out) + base + dt * 16) = v;
-      } else {
-        u32x2 pk;
-        if constexpr (ODT == KVQ_BF16) {
-          pk.x = (uint32_t)f32_to_bf16_bits(v.x) | ((uint32_t)f32_to_bf16_bits(v.y) << 16);
-          pk.y = (uint32_t)f32_to_bf16_bits(v.z) | ((uint32_t)f32_to_bf16_bits(v.w) << 16);
-        } else {
-          pk.x = pack_half2(v.x, v.y);
-          pk.y = pack_half2(v.z, v.w);
-        }
-        *reinterpret_cast<u32x2_a4*>(reinterpret_cast<uint16_t*>(io.out) + base + dt * 16) = pk;
+      for (int kt = 0; kt < 2; ++kt) {
+        const half8_t va = *reinterpret_cast<const half8_t*>(vrow + mt * 32 * V_PITCH + 32 * kt);
+        o[mt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(va, p_op[kt], o[mt], 0, 0, 0);
       }
     }
-    if (io.lse != nullptr && g == 0)
-      io.lse[row * io.num_q_heads + head] = l > 0.f ? (st.m[nt] + __builtin_amdgcn_logf(l)) * kLn2 : -INFINITY;
   }
 };
 
-// grid (query blocks of the longest run, sequences, kv heads), 4 waves.  Later query blocks see
-// more keys, so block index 0 is the LAST query block: the longest workgroups start first.
-template <int D, int QDT, int ODT, int NT, int OCC, int WAVES>
-__global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(OCC, OCC))) void paged_prefill_flash_kernel(PrefillArgs a) {
-  using FP = FlashPrefill<D, QDT, ODT, NT, WAVES>;
+template <int D, int QDT, int ODT>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void paged_prefill_flash32_kernel(PrefillArgs a) {
+  using FP = Flash32<D, QDT, ODT>;
   using DTile = typename FP::DTile;
   extern __shared__ __align__(16) uint8_t lds[];
   uint8_t* raws = lds;
@@ -516,68 +520,54 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(OCC,
   const int q0 = ((int)gridDim.x - 1 - (int)blockIdx.x) * a.q_tokens;
   if (q_len <= 1 || q0 >= q_len || len <= 0) return;   // uniform over the workgroup
 
-  const int c = lane & 15;
+  // column of this lane: (query token q0 + n / group, head n % group), n = wave * 32 + (lane & 31)
   const int ctx = len - q_len;
-  int limit[NT];
-  int64_t row[NT];
-  int head[NT];
-  bool valid[NT];
-  int wave_max_limit = 0, wave_min_limit = 0x7fffffff;
-#pragma unroll
-  for (int nt = 0; nt < NT; ++nt) {
-    const int n = (wave * NT + nt) * 16 + c;
-    const int qt = n / io.group;
-    const int qi = q0 + qt;
-    valid[nt] = qt < a.q_tokens && qi < q_len;
-    head[nt] = hkv * io.group + (n - qt * io.group);
-    row[nt] = q_begin + (valid[nt] ? qi : q0);
-    int lim = a.causal ? ctx + qi + 1 : len;
-    lim = lim < 0 ? 0 : (lim > len ? len : lim);
-    limit[nt] = valid[nt] ? lim : 0;
-    wave_max_limit = max(wave_max_limit, limit[nt]);
-    wave_min_limit = min(wave_min_limit, valid[nt] ? lim : 0x7fffffff);
-  }
-  wave_max_limit = wave_max_i32(wave_max_limit);
-  wave_min_limit = -wave_max_i32(-wave_min_limit);
-  // the workgroup's last query token bounds every wave's keys
+  const int n = wave * 32 + (lane & 31);
+  const int qt = n / io.group;
+  const int qi = q0 + qt;
+  const bool valid = qt < a.q_tokens && qi < q_len;
+  const int head = hkv * io.group + (n - qt * io.group);
+  const int64_t row = q_begin + (valid ? qi : q0);
+  int lim = a.causal ? ctx + qi + 1 : len;
+  lim = lim < 0 ? 0 : (lim > len ? len : lim);
+  const int limit = valid ? lim : 0;
+  const int wave_max_limit = wave_max_i32(limit);
+  const int wave_min_limit = -wave_max_i32(valid ? -lim : -0x7fffffff);
   int wg_limit = a.causal ? ctx + min(q0 + a.q_tokens, q_len) : len;
   wg_limit = wg_limit < 0 ? 0 : (wg_limit > len ? len : wg_limit);
   const int t_end = (wg_limit + kTile - 1) / kTile;
 
-  typename FP::State st;
+  floatx16 o[FP::MT];
 #pragma unroll
-  for (int nt = 0; nt < NT; ++nt) {
+  for (int mt = 0; mt < FP::MT; ++mt)
 #pragma unroll
-    for (int dt = 0; dt < FP::DT; ++dt) st.o[nt][dt] = (floatx4){0.f, 0.f, 0.f, 0.f};
-    st.m[nt] = -INFINITY;
-    st.l[nt] = 0.f;
-  }
+    for (int i = 0; i < 16; ++i) o[mt][i] = 0.f;
+  float m = -INFINITY, l = 0.f;
 
   if (t_end > 0) {
     const LaneOffsets lo = DTile::lane_offsets(io.g, lane);
     const int32_t* bt_row = io.block_table + (int64_t)seq * io.bt_stride;
     const int step = (64 / DTile::NCH) * (int)io.g.stride_slot;
-    // Every wave issues the same two loads per tile, unconditionally and in the same order in
-    // every step, so the wait before a tile's registers are used can leave the younger tile's
-    // loads in flight.  Wave w takes chunk load n = (w >> 1) % NLD of 16-token half h = w & 1
-    // (waves beyond 2 * NLD repeat one; harmless) and that half's record tails.
-    static_assert(WAVES == 8, "load distribution below assumes eight waves");
-    const int half = wave & 1, ld_n = (wave >> 1) % DTile::NLD;
+    // every wave: chunk load (wave % NLD) of both 16-token halves and the record tails of half
+    // (wave & 1), unconditionally and in the same order in every step
+    const int half = wave & 1;
+    const int ld_n = wave % DTile::NLD;
     struct Regs {
-      u32x4 c;
+      u32x4 c0, c1;
       u32x2 tail;
     };
     Regs A{}, B{};
     auto issue = [&](const TileBlocks& nb, int t, Regs& r) __attribute__((always_inline)) {
       const typename DTile::Window w = DTile::window(io, nb, t, hkv);
-      const __amdgpu_buffer_rsrc_t rs = half ? w.r1 : w.r0;
-      r.c = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rs, lo.g_chunk, ld_n * step, 0));
-      r.tail = __builtin_bit_cast(u32x2, __builtin_amdgcn_raw_buffer_load_b64(rs, lo.g_tail, 0, 0));
+      r.c0 = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(w.r0, lo.g_chunk, ld_n * step, 0));
+      r.c1 = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(w.r1, lo.g_chunk, ld_n * step, 0));
+      r.tail = __builtin_bit_cast(u32x2, __builtin_amdgcn_raw_buffer_load_b64(half ? w.r1 : w.r0, lo.g_tail, 0, 0));
     };
-    const uint32_t l_chunk = lo.l_chunk + (16 * half + ld_n * (64 / DTile::NCH)) * FP::RAW_PITCH;
+    const uint32_t l_chunk = lo.l_chunk + ld_n * (64 / DTile::NCH) * FP::RAW_PITCH;
     const uint32_t l_tail = (16 * half + (lane & 15)) * FP::RAW_PITCH + 2 * D;
-    auto drop = [&](const Regs& r, uint8_t* raw) __attribute__((always_inline)) {  // registers -> raw LDS window
-      *reinterpret_cast<u32x4*>(raw + l_chunk) = r.c;
+    auto drop = [&](const Regs& r, uint8_t* raw) __attribute__((always_inline)) {
+      *reinterpret_cast<u32x4*>(raw + l_chunk) = r.c0;
+      *reinterpret_cast<u32x4*>(raw + l_chunk + 16 * FP::RAW_PITCH) = r.c1;
       if (wave < 2 && lane < 16) *reinterpret_cast<u32x2*>(raw + l_tail) = r.tail;
     };
     TileBlocks nb = DTile::fetch_blocks(io, bt_row, len, 0);
@@ -586,52 +576,89 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(OCC,
     issue(nb, 1, B);
     nb = DTile::fetch_blocks(io, bt_row, len, 2);
 
-    half8_t qb[NT][FP::KSTEPS];
-#pragma unroll
-    for (int nt = 0; nt < NT; ++nt)
-      (void)DTile::load_q_row(io, row[nt] * io.q_stride_t + (int64_t)(valid[nt] ? head[nt] : hkv * io.group) * io.q_stride_h,
-                              valid[nt], lane, qb[nt]);
+    half8_t qb[FP::KS];
+    FP::load_q(io, row * io.q_stride_t + (int64_t)(valid ? head : hkv * io.group) * io.q_stride_h, valid, lane, qb);
     const float sc_mul = lane < 32 ? io.scale_log2 : kPScale;
 
     drop(A, raws);
-    issue(nb, 2, A);  // tiles past the end reread the last block (clamped); they are never expanded
+    issue(nb, 2, A);
     nb = DTile::fetch_blocks(io, bt_row, len, 3);
     lds_barrier();
     // Step t: expand raw tile t into fp16 buffer t&1, drop tile t+1 (held in `next`) into the other
-    // raw window and refill `next` with tile t+3, ONE barrier, then compute tile t.  Safe with one
-    // barrier because both the raw windows and the fp16 tiles are double-buffered: what a step
-    // writes is only read after that step's barrier, and was last read before the previous one.
-    auto step_fn = [&](int t, Regs& next) __attribute__((always_inline)) {
+    // raw window and refill `next` with tile t+3, ONE barrier, then compute tile t.
+    auto step_fn = [&](auto masked, int t, Regs& next) __attribute__((always_inline)) {
       uint8_t* buf = bufs + (t & 1) * FP::BUF_BYTES;
       FP::expand(raws + (t & 1) * FP::RAW_BYTES, buf, tid, sc_mul, lo.l_sc);
       drop(next, raws + ((t + 1) & 1) * FP::RAW_BYTES);
       issue(nb, t + 3, next);
       lds_barrier();
-      nb = DTile::fetch_blocks(io, bt_row, len, t + 4);  // after the barrier: its wait would expose this scalar load
-      if (t * kTile < wave_max_limit) {  // wave-uniform: tiles past this wave's last key are skipped
-        if ((t + 1) * kTile <= wave_min_limit) FP::template compute<false>(buf, qb, limit, t, lane, st);
-        else FP::template compute<true>(buf, qb, limit, t, lane, st);
+      nb = DTile::fetch_blocks(io, bt_row, len, t + 4);
+      if constexpr (decltype(masked)::value) {
+        if (t * kTile < wave_max_limit) FP::template compute<true>(buf, qb, limit, t, lane, o, m, l);
+      } else {
+        FP::template compute<false>(buf, qb, limit, t, lane, o, m, l);
       }
     };
-    for (int t = 0; t < t_end; t += 2) {  // an odd t_end runs one step past the end: it computes nothing
-      step_fn(t, B);
-      step_fn(t + 1, A);
+    // Tiles below every column's limit need no mask.  They and the masked tail are two separate
+    // loops (every wave runs the same number of steps, hence of barriers, whichever loop a step is
+    // in), so that the accumulators keep their registers across the loop instead of being merged
+    // at a branch inside it.
+    const int t_plain = min(t_end, wave_min_limit / kTile) & ~1;
+    int t = 0;
+    for (; t < t_plain; t += 2) {
+      step_fn(std::false_type{}, t, B);
+      step_fn(std::false_type{}, t + 1, A);
+    }
+    for (; t < t_end; t += 2) {  // an odd t_end runs one step past the end: it computes nothing
+      step_fn(std::true_type{}, t, B);
+      step_fn(std::true_type{}, t + 1, A);
     }
   }
+  // Lane (c, g) holds O[column][dim mt*32 + (i/4)*8 + 4g + i%4] in o[mt][i].
+  l += __shfl_xor(l, 32, kWave);
+  if (!valid) return;
+  const int g = lane >> 5;
+  const float mul = l > 0.f ? 1.0f / (l * kPScale) : 0.f;
+  const int64_t base = row * io.out_stride_t + (int64_t)head * io.out_stride_h + 4 * g;
 #pragma unroll
-  for (int nt = 0; nt < NT; ++nt) FP::emit(io, nt, row[nt], head[nt], valid[nt], lane, st);
+  for (int mt = 0; mt < FP::MT; ++mt) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      floatx4 v;
+      v.x = o[mt][4 * q + 0] * mul;
+      v.y = o[mt][4 * q + 1] * mul;
+      v.z = o[mt][4 * q + 2] * mul;
+      v.w = o[mt][4 * q + 3] * mul;
+      const int64_t at = base + mt * 32 + q * 8;
+      if constexpr (ODT == KVQ_F32) {
+        *reinterpret_cast<floatx4_a4*>(reinterpret_cast<float*>(io.out) + at) = v;
+      } else {
+        u32x2 pk;
+        if constexpr (ODT == KVQ_BF16) {
+          pk.x = (uint32_t)f32_to_bf16_bits(v.x) | ((uint32_t)f32_to_bf16_bits(v.y) << 16);
+          pk.y = (uint32_t)f32_to_bf16_bits(v.z) | ((uint32_t)f32_to_bf16_bits(v.w) << 16);
+        } else {
+          pk.x = pack_half2(v.x, v.y);
+          pk.y = pack_half2(v.z, v.w);
+        }
+        *reinterpret_cast<u32x2_a4*>(reinterpret_cast<uint16_t*>(io.out) + at) = pk;
+      }
+    }
+  }
+  if (io.lse != nullptr && g == 0)
+    io.lse[row * io.num_q_heads + head] = l > 0.f ? (m + __builtin_amdgcn_logf(l)) * kLn2 : -INFINITY;
 }
 
-template <int D, int QDT, int ODT, int NT, int OCC, int WAVES>
-static int launch_prefill_flash(PrefillArgs& a, int max_query_len, hipStream_t s) {
-  using FP = FlashPrefill<D, QDT, ODT, NT, WAVES>;
+template <int D, int QDT, int ODT>
+static int launch_prefill_flash32(PrefillArgs& a, int max_query_len, hipStream_t s) {
+  using FP = Flash32<D, QDT, ODT>;
   a.q_tokens = FP::COLS / a.io.group;
   const int blocks = (max_query_len + a.q_tokens - 1) / a.q_tokens;
   if (a.num_seqs > 65535 || a.io.g.num_kv_heads > 65535) return fail(KVQ_EINVAL, "paged_attn_int8: prefill grid out of range");
   static_assert(FP::LDS_BYTES <= 64 * 1024, "static LDS opt-in would be needed");
   dim3 grid(blocks, a.num_seqs, a.io.g.num_kv_heads);
-  hipLaunchKernelGGL((paged_prefill_flash_kernel<D, QDT, ODT, NT, OCC, WAVES>), grid, dim3(WAVES * 64), FP::LDS_BYTES, s, a);
-  return check_hip(hipGetLastError(), "paged_prefill_flash launch");
+  hipLaunchKernelGGL((paged_prefill_flash32_kernel<D, QDT, ODT>), grid, dim3(256), FP::LDS_BYTES, s, a);
+  return check_hip(hipGetLastError(), "paged_prefill_flash32 launch");
 }
 
 template <int D, int QDT, int ODT, int NT, int WPW>
@@ -648,9 +675,7 @@ static int launch_prefill_nt(PrefillArgs& a, int max_query_len, hipStream_t s) {
   constexpr int WPW = 4;
   // long runs: the workgroup-shared fp16 tile (compute-bound shape)
   if constexpr (D <= 128) {
-    if (max_query_len * a.io.group >= 64) {
-      return launch_prefill_flash<D, QDT, ODT, 2, 2, 8>(a, max_query_len, s);
-    }
+    if (max_query_len * a.io.group >= 64) return launch_prefill_flash32<D, QDT, ODT>(a, max_query_len, s);
   }
   // two column tiles per wave where the accumulators fit the register file next to a tile in flight
   if (D <= 128 && a.io.group * 2 <= 32 && max_query_len * a.io.group > 16) {
