@@ -341,9 +341,12 @@ struct Flash32 {
 
   // Q of the lane's column as the B operand: lane (c = lane & 31, g = lane >> 5) holds, for k-step
   // ks, dims 16 ks + 8 g + j.
-  __device__ static __forceinline__ void load_q(const AttnIO& io, int64_t elem, bool valid, int lane, half8_t (&qb)[KS]) {
+  // Returns -1152 * sum(q) of the column: the S accumulator's start value, which cancels the code
+  // bias that K keeps (V's is removed during the expansion).
+  __device__ static __forceinline__ float load_q(const AttnIO& io, int64_t elem, bool valid, int lane, half8_t (&qb)[KS]) {
     const int g = lane >> 5;
     const uint32_t okmask = valid ? 0xffffffffu : 0u;
+    float qsum = 0.f;
     u32x4 raw[QDT == KVQ_F32 ? 1 : KS];
     if constexpr (QDT != KVQ_F32) {
 #pragma unroll
@@ -378,10 +381,14 @@ struct Flash32 {
       hb.z = pack_half2(clamp_half_range(f[4]), clamp_half_range(f[5])) & okmask;
       hb.w = pack_half2(clamp_half_range(f[6]), clamp_half_range(f[7])) & okmask;
       qb[ks] = __builtin_bit_cast(half8_t, hb);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) qsum += (float)qb[ks][j];  // the sum of what the MFMA will actually see
     }
+    qsum += __shfl_xor(qsum, 32, kWave);
+    return -kCodeBias * qsum;
   }
 
-  // Raw tile -> fp16 K [token][dim] and V^T [dim][position]; token t of the tile sits at position
+  // Raw tile -> fp16 K [token][dim] (codes + 1152) and V^T [dim][position] (codes); token t of the tile sits at position
   // (t/16)*16 + ((t%8)/4)*8 + ((t/8)%2)*4 + t%4, the order in which the 32x32 S accumulator hands a
   // lane its tokens.  One thread converts one 16-code K chunk and one 4-token x 4-dim V block.
   __device__ static __forceinline__ void expand(const uint8_t* raw, uint8_t* buf, int tid, float sc_mul, uint32_t l_sc) {
@@ -393,11 +400,11 @@ struct Flash32 {
 #pragma unroll
       for (int i = 0; i < 2; ++i) {
         const uint32_t x = w[i] ^ 0x80808080u;
-        lo[2 * i] = to_half2(x, false);
-        lo[2 * i + 1] = to_half2(x, true);
+        lo[2 * i] = bytes_to_half2(x, false);
+        lo[2 * i + 1] = bytes_to_half2(x, true);
         const uint32_t y = w[2 + i] ^ 0x80808080u;
-        hi[2 * i] = to_half2(y, false);
-        hi[2 * i + 1] = to_half2(y, true);
+        hi[2 * i] = bytes_to_half2(y, false);
+        hi[2 * i + 1] = bytes_to_half2(y, true);
       }
       *reinterpret_cast<u32x4*>(buf + tok * K_PITCH + 32 * ch) = lo;
       *reinterpret_cast<u32x4*>(buf + tok * K_PITCH + 32 * ch + 16) = hi;
@@ -430,42 +437,49 @@ struct Flash32 {
   // One tile for the wave's 32 columns.  S^T[32 tokens, 32 columns]: lane (c = column, g) holds
   // token (i/4)*8 + 4g + i%4 in register i.
   template <bool MASK>
-  __device__ static __forceinline__ void compute(const uint8_t* buf, const half8_t (&qb)[KS], int limit, int t, int lane,
-                                                 floatx16 (&o)[MT], float& m, float& l) {
+  __device__ static __forceinline__ void compute(const uint8_t* buf, const half8_t (&qb)[KS], float s_init, int limit, int t,
+                                                 int lane, floatx16 (&o)[MT], float& m, float& l) {
     const int c = lane & 31, g = lane >> 5;
     const float* sc = reinterpret_cast<const float*>(buf + K_BYTES + V_BYTES);
     floatx16 s;
 #pragma unroll
-    for (int i = 0; i < 16; ++i) s[i] = 0.f;
+    for (int i = 0; i < 16; ++i) s[i] = s_init;
     const uint8_t* krow = buf + c * K_PITCH + g * 16;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       const half8_t ka = *reinterpret_cast<const half8_t*>(krow + 32 * ks);
       s = __builtin_amdgcn_mfma_f32_32x32x16_f16(ka, qb[ks], s, 0, 0, 0);
     }
+    // Logits are taken relative to the running maximum in the same multiply-add that applies the K
+    // scale: y = s * k_scale - m.  While no column's maximum moves (the usual case after the first
+    // tiles) p = exp2(y) needs no further subtraction.
     const int tok_base = t * kTile + 4 * g;
-    float mloc = -INFINITY;
+    const bool fresh = m == -INFINITY;          // the column has seen no visible token yet
+    const float mref = fresh ? 0.f : m;
+    float d = -INFINITY;
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
       const floatx4 ksc = *reinterpret_cast<const floatx4*>(sc + 8 * q + 4 * g);
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        float x = s[4 * q + r] * ksc[r];
-        if constexpr (MASK) x = ((tok_base + q * 8 + r) < limit) ? x : -INFINITY;
-        s[4 * q + r] = x;
-        mloc = fmaxf(mloc, x);
+        float y = __builtin_fmaf(s[4 * q + r], ksc[r], -mref);
+        if constexpr (MASK) y = ((tok_base + q * 8 + r) < limit) ? y : -INFINITY;
+        s[4 * q + r] = y;
+        d = fmaxf(d, y);
       }
     }
-    mloc = fmaxf(mloc, __shfl_xor(mloc, 32, kWave));
-    const float m_new = fmaxf(m, mloc);
-    const float m_ref = m_new == -INFINITY ? 0.f : m_new;  // see PrefillTile::qk_softmax
-    if (__builtin_amdgcn_ballot_w64(m_new > m) != 0) {
-      const float alpha = __builtin_amdgcn_exp2f(m - m_ref);
+    d = fmaxf(d, __shfl_xor(d, 32, kWave));
+    // how far the maximum moves: a fresh column takes d itself (0 while it still sees nothing)
+    const float up = fresh ? (d == -INFINITY ? 0.f : d) : fmaxf(d, 0.f);
+    if (__builtin_amdgcn_ballot_w64(up != 0.f) != 0) {
+      const float alpha = __builtin_amdgcn_exp2f(-up);  // a fresh column's o and l are still zero
       l *= alpha;
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) o[mt] *= alpha;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) s[i] -= up;
     }
-    m = m_new;
+    m = (fresh && d == -INFINITY) ? -INFINITY : mref + up;
     half8_t p_op[2];
 #pragma unroll
     for (int kt = 0; kt < 2; ++kt) {
@@ -476,7 +490,7 @@ struct Flash32 {
         const floatx4 vsc = *reinterpret_cast<const floatx4*>(sc + 32 + 8 * q + 4 * g);
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-          const float p = __builtin_amdgcn_exp2f(s[4 * q + r] - m_ref);
+          const float p = __builtin_amdgcn_exp2f(s[4 * q + r]);
           l += p;
           float x = p * vsc[r];
           if constexpr (MASK) x = ((tok_base + q * 8 + r) < limit) ? x : 0.f;
@@ -577,7 +591,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     nb = DTile::fetch_blocks(io, bt_row, len, 2);
 
     half8_t qb[FP::KS];
-    FP::load_q(io, row * io.q_stride_t + (int64_t)(valid ? head : hkv * io.group) * io.q_stride_h, valid, lane, qb);
+    const float s_init =
+        FP::load_q(io, row * io.q_stride_t + (int64_t)(valid ? head : hkv * io.group) * io.q_stride_h, valid, lane, qb);
     const float sc_mul = lane < 32 ? io.scale_log2 : kPScale;
 
     drop(A, raws);
@@ -594,9 +609,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       lds_barrier();
       nb = DTile::fetch_blocks(io, bt_row, len, t + 4);
       if constexpr (decltype(masked)::value) {
-        if (t * kTile < wave_max_limit) FP::template compute<true>(buf, qb, limit, t, lane, o, m, l);
+        if (t * kTile < wave_max_limit) FP::template compute<true>(buf, qb, s_init, limit, t, lane, o, m, l);
       } else {
-        FP::template compute<false>(buf, qb, limit, t, lane, o, m, l);
+        FP::template compute<false>(buf, qb, s_init, limit, t, lane, o, m, l);
       }
     };
     // Tiles below every column's limit need no mask.  They and the masked tail are two separate
