@@ -15,6 +15,8 @@
 // The token splits of a sequence are merged by the reduce kernel with the log-sum-exp algebra
 // (same two-stage shape as the reference's decode_attention_fwd); nothing is allocated here,
 // partials live in the caller's workspace.
+#include <atomic>
+
 #include "kvq_attn_core.cuh"
 
 namespace kvq {
@@ -410,12 +412,34 @@ static int mla_num_splits(int max_seq_hint, int num_seqs, int num_heads) {
   return splits;
 }
 
+// The decode kernel needs more dynamic LDS than the 64 KB a kernel gets by default.  The opt-in is a
+// per-device, per-kernel attribute; it is set for all three instantiations the first time either entry
+// point runs on a device -- the workspace query is the place a caller reaches before any stream
+// capture, so a captured decode call finds it done.
+static int mla_prepare_device() {
+  static std::atomic<uint64_t> done_mask{0};  // one bit per device id < 64
+  int dev = -1;
+  if (int e = check_hip(hipGetDevice(&dev), "hipGetDevice")) return e;
+  const uint64_t bit = dev >= 0 && dev < 64 ? (1ull << dev) : 0;
+  if (bit != 0 && (done_mask.load(std::memory_order_acquire) & bit)) return KVQ_OK;
+  const void* fns[3] = {reinterpret_cast<const void*>(&mla_decode_kernel<KVQ_F32>),
+                        reinterpret_cast<const void*>(&mla_decode_kernel<KVQ_BF16>),
+                        reinterpret_cast<const void*>(&mla_decode_kernel<KVQ_F16>)};
+  for (const void* f : fns)
+    if (int e = check_hip(hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, kMlaLdsBytes),
+                          "hipFuncSetAttribute(mla_decode_kernel)"))
+      return e;
+  done_mask.fetch_or(bit, std::memory_order_release);
+  return KVQ_OK;
+}
+
 }  // namespace kvq
 
 extern "C" {
 
 size_t kvq_mla_decode_workspace_bytes(int max_num_seqs, int num_heads, int kv_lora_rank) {
   if (max_num_seqs <= 0 || num_heads <= 0 || kv_lora_rank <= 0) return 0;
+  if (kvq::mla_prepare_device() != KVQ_OK) return 0;
   // sequences x splits stays below max(2 x resident workgroups per head group, sequences)
   const size_t groups = ((size_t)num_heads + 127) / 128;
   size_t items = 2 * (size_t)kvq::num_cus() / groups;
@@ -468,20 +492,8 @@ int kvq_mla_decode_int8(void* out, int out_dtype, float* lse, const void* q, int
   a.bs_magic = (uint32_t)((0x100000000ull + (uint64_t)g.block_size - 1) / (uint64_t)g.block_size);
   hipStream_t s = as_stream(stream);
   dim3 grid(splits, num_seqs, (num_heads + 127) / 128);
-#define KVQ_MLAD(T)                                                                                       \
-  do {                                                                                                  \
-    static int lds_ok_dev = -2;  /* the >64 KB dynamic LDS opt-in, once per device */                   \
-    int devid = -1;                                                                                     \
-    if (int e = check_hip(hipGetDevice(&devid), "hipGetDevice")) return e;                              \
-    if (lds_ok_dev != devid) {                                                                          \
-      if (int e = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(&mla_decode_kernel<T>),   \
-                                                hipFuncAttributeMaxDynamicSharedMemorySize, kMlaLdsBytes), \
-                            "hipFuncSetAttribute(mla_decode_kernel)"))                                  \
-        return e;                                                                                       \
-      lds_ok_dev = devid;                                                                               \
-    }                                                                                                   \
-    hipLaunchKernelGGL((mla_decode_kernel<T>), grid, dim3(kMlaThreads), kMlaLdsBytes, s, a);            \
-  } while (0)
+  if (int e = mla_prepare_device()) return e;
+#define KVQ_MLAD(T) hipLaunchKernelGGL((mla_decode_kernel<T>), grid, dim3(kMlaThreads), kMlaLdsBytes, s, a)
   switch (q_dtype) {
     case KVQ_F32: KVQ_MLAD(KVQ_F32); break;
     case KVQ_BF16: KVQ_MLAD(KVQ_BF16); break;
