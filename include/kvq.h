@@ -189,6 +189,24 @@ KVQ_API int kvq_concat_and_cache_mla_int8(const void* kv_c, const void* k_pe, in
                                   const kvq_mla_geom* geom, const int64_t* slot_mapping,
                                   int64_t num_tokens, float eps, kvq_stream_t stream);
 
+/*
+ * Gather + dequantise latent rows into a dense workspace.  Stands in for the
+ * quantised branch of gather_and_maybe_dequant_cache(src_cache, dst,
+ * block_table, cu_seq_lens, token_to_seq, num_tokens, kv_cache_dtype, scale,
+ * seq_starts), csrc/libtorch_stable/cache_kernels.cu:1072-1131, 1181-1247, which
+ * the MLA chunked-context prefill calls
+ * (vllm_metax/model_executor/layers/attention/mla_attention.py:2017-2140):
+ * destination row t belongs to sequence b = token_to_seq[t], position
+ * t - cu_seq_lens[b] (+ seq_starts[b] when given), and receives
+ * code * row_scale rounded once to `dst_dtype`.  dst [num_tokens, >= R+P],
+ * dst_stride in elements.  seq_starts may be NULL.
+ */
+KVQ_API int kvq_gather_and_dequant_mla_int8(void* dst, int dst_dtype, int64_t dst_stride, const void* cache,
+                                    const kvq_mla_geom* geom, const int32_t* block_table,
+                                    int64_t bt_stride, const int32_t* cu_seq_lens,
+                                    const int32_t* token_to_seq, const int32_t* seq_starts,
+                                    int64_t num_tokens, kvq_stream_t stream);
+
 KVQ_API size_t kvq_mla_decode_workspace_bytes(int max_num_seqs, int num_heads, int kv_lora_rank);
 
 /*

@@ -309,3 +309,20 @@ def mla_decode(q, cache, lay: MlaLayout, block_table, seq_lens, scale: float):
         "kvq_oracle_mla_decode",
     )
     return out, lse
+
+
+def mla_gather_dequant(cache, lay: MlaLayout, block_table, cu_seq_lens, token_to_seq, num_tokens, seq_starts=None):
+    """int8 latent cache -> fp32 [num_tokens, R+P] rows (code * row scale)."""
+    bt, cu, t2s = _i32c(block_table), _i32c(cu_seq_lens), _i32c(token_to_seq)
+    ss = _i32c(seq_starts) if seq_starts is not None else None
+    W = lay.kv_lora_rank + lay.rope_dim
+    dst = torch.zeros((num_tokens, W), dtype=torch.float32)
+    _check(
+        lib().kvq_oracle_mla_gather_dequant(
+            _p(dst), _i64(W), _p(cache), _i64(lay.stride_block), _i64(lay.stride_row), _i64(lay.scale_off),
+            _p(bt), _i64(bt.stride(0)), _p(cu), _p(t2s), _p(ss) if ss is not None else None,
+            ctypes.c_int(num_tokens), ctypes.c_int(W), ctypes.c_int(lay.block_size),
+        ),
+        "kvq_oracle_mla_gather_dequant",
+    )
+    return dst

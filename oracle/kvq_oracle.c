@@ -19,6 +19,8 @@
  *                                             passthrough)
  *   kvq_oracle_merge_attn_states    pinned   (torch restatement, +inf / -inf cases)
  *   kvq_oracle_mla_cache_write      pinned   (same quantiser, one group of 576)
+ *   kvq_oracle_mla_gather_dequant   pinned   (python gather loop, code * scale in numpy fp32,
+ *                                             round trip through the write)
  *   kvq_oracle_mla_decode           pinned   (torch SDPA enable_gqa + logsumexp)
  *
  * What no check available offline can pin (it lives in upstream vLLM's Triton
@@ -505,4 +507,39 @@ KVQ_EXPORT int kvq_oracle_num_threads(void) {
 #else
   return 1;
 #endif
+}
+
+
+/* ---------------------------------------------------------------------------
+ * Gather + dequantise rows of the int8 latent cache into a dense workspace:
+ * the int8 branch of gather_and_maybe_dequant_cache,
+ * csrc/libtorch_stable/cache_kernels.cu:1072-1131 (one destination row per
+ * token: batch = token_to_seq[token], position = token - cu_seq_lens[batch]
+ * + seq_starts[batch], block = block_table[batch, position / block_size],
+ * slot = position % block_size), used by the MLA chunked-context prefill
+ * (vllm_metax/model_executor/layers/attention/mla_attention.py:2017-2140).
+ * The reference converts with one per-tensor scale; here every row carries its
+ * own: dst[token, d] = (float)code * scale_of_row, one fp32 rounding.
+ * dst is fp32 [num_tokens, dst_stride]; the caller rounds to the output type.
+ * ------------------------------------------------------------------------- */
+KVQ_EXPORT int kvq_oracle_mla_gather_dequant(float* dst, int64_t dst_stride, const uint8_t* cache,
+                                             int64_t stride_block, int64_t stride_row, int64_t scale_off,
+                                             const int32_t* block_table, int64_t bt_stride,
+                                             const int32_t* cu_seq_lens, const int32_t* token_to_seq,
+                                             const int32_t* seq_starts, int num_tokens, int width,
+                                             int block_size) {
+  if (!dst || !cache || !block_table || !cu_seq_lens || !token_to_seq) return -1;
+  for (int t = 0; t < num_tokens; ++t) {
+    const int b = token_to_seq[t];
+    if (t >= cu_seq_lens[b + 1]) continue;
+    int pos = t - cu_seq_lens[b];
+    if (seq_starts) pos += seq_starts[b];
+    const int64_t blk = block_table[(int64_t)b * bt_stride + pos / block_size];
+    const int off = pos % block_size;
+    const int8_t* row = (const int8_t*)(cache + blk * stride_block + (int64_t)off * stride_row);
+    float scale;
+    memcpy(&scale, cache + blk * stride_block + scale_off + (int64_t)off * 4, 4);
+    for (int d = 0; d < width; ++d) dst[(int64_t)t * dst_stride + d] = (float)row[d] * scale;
+  }
+  return 0;
 }

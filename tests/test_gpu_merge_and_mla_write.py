@@ -93,3 +93,43 @@ def test_mla_write_errors(gpu_device):
         ops.concat_and_cache_mla(kv_c, k_pe[:, :32], cache, torch.zeros(4, device=dev, dtype=torch.int64))
     with pytest.raises(NotImplementedError):
         ops.concat_and_cache_mla(kv_c, k_pe, cache, torch.zeros(4, device=dev, dtype=torch.int64), kv_cache_dtype="fp8")
+
+
+@pytest.mark.parametrize("dst_dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("use_starts", [False, True])
+def test_mla_gather_and_dequant_bit_exact(gpu_device, dst_dtype, use_starts):
+    """Gather + dequantise for the chunked-context prefill: bit-exact against the oracle's
+    code * scale (one fp32 rounding, then one rounding to the output type), rows beyond a sequence's
+    end and beyond num_tokens untouched, and a round trip through the write."""
+    dev = gpu_device
+    R, P, bs, nb = 512, 64, 64, 12
+    g = torch.Generator().manual_seed(17)
+    ctx = [130, 64, 300]
+    bt = T.make_block_tables(ctx, bs, nb, g)
+    cpu = L.allocate_mla_cache(nb, bs, R + P, device="cpu", fill=0x33)
+    codes, scales = L.mla_cache_views(cpu)
+    lay = oracle.MlaLayout.from_views(cpu, codes, scales, R)
+    rows = []
+    for i, slots in enumerate(T.slots_for(bt, ctx, bs)):
+        kv_c = torch.randn((ctx[i], R), generator=g).to(torch.bfloat16)
+        k_pe = torch.randn((ctx[i], P), generator=g).to(torch.bfloat16)
+        oracle.mla_cache_write(kv_c, k_pe, cpu, lay, slots)
+        rows.append(torch.cat([kv_c, k_pe], -1).float())
+    # a chunk of every sequence: seq_starts[b] .. seq_starts[b] + chunk[b]
+    starts = [40, 0, 250] if use_starts else [0, 0, 0]
+    chunk = [70, 64, 50] if use_starts else ctx
+    cu = torch.tensor([0] + torch.tensor(chunk).cumsum(0).tolist(), dtype=torch.int32)
+    n = int(cu[-1])
+    t2s = torch.repeat_interleave(torch.arange(3, dtype=torch.int32), torch.tensor(chunk))
+    ss = torch.tensor(starts, dtype=torch.int32) if use_starts else None
+    want = oracle.mla_gather_dequant(cpu, lay, bt, cu, t2s, n, ss)
+    dst = torch.full((n + 3, R + P), 7.0, dtype=dst_dtype, device=dev)
+    ops.gather_and_maybe_dequant_cache(cpu.to(dev), dst, bt.to(dev), cu.to(dev), t2s.to(dev), n,
+                                       seq_starts=ss.to(dev) if ss is not None else None)
+    torch.cuda.synchronize()
+    assert torch.equal(dst[:n].cpu(), want.to(dst_dtype)), "gathered rows differ from the oracle"
+    assert bool((dst[n:] == 7.0).all()), "rows beyond num_tokens were written"
+    # the gathered rows are the written rows up to the quantisation step
+    src = torch.cat([rows[b][starts[b]:starts[b] + chunk[b]] for b in range(3)])
+    amax = src.abs().amax(-1, keepdim=True)
+    assert bool(((want - src).abs() <= amax / 127 * 0.5 * (1 + 1e-4)).all())

@@ -114,3 +114,32 @@ def test_within_one_code_of_reciprocal_formulation():
     codes, _ = oracle.quant_rows(x)
     alt, _ = torch_ref.dynamic_per_token_quant_int8_reciprocal(x)
     assert (codes.int() - alt.int()).abs().max() <= 1
+
+
+def test_mla_gather_dequant_is_the_python_gather_loop():
+    """The oracle's gather + dequantise against a gather written with the typed cache views
+    (the reference's test pattern for gather ops, tests/kernels/attention/test_cache.py:706-863:
+    per-sequence block lookup, then row copy), with and without seq_starts."""
+    import oracle
+    from vllm_metax_amd import layout as L
+
+    R, P, bs, nb = 512, 64, 16, 20
+    g = torch.Generator().manual_seed(2)
+    cache = L.allocate_mla_cache(nb, bs, R + P, device="cpu")
+    codes, scales = L.mla_cache_views(cache)
+    codes.copy_(torch.randint(-128, 128, codes.shape, generator=g, dtype=torch.int8))
+    scales.copy_(torch.rand(scales.shape, generator=g) * 0.05 + 1e-3)
+    lay = oracle.MlaLayout.from_views(cache, codes, scales, R)
+    bt = torch.randperm(nb, generator=g)[:18].to(torch.int32).reshape(3, 6)
+    for starts, chunk in (([0, 0, 0], [50, 96, 7]), ([30, 5, 90], [40, 16, 6])):
+        cu = torch.tensor([0] + torch.tensor(chunk).cumsum(0).tolist(), dtype=torch.int32)
+        n = int(cu[-1])
+        t2s = torch.repeat_interleave(torch.arange(3, dtype=torch.int32), torch.tensor(chunk))
+        got = oracle.mla_gather_dequant(cache, lay, bt, cu, t2s, n, torch.tensor(starts, dtype=torch.int32))
+        want = torch.empty((n, R + P))
+        for t in range(n):
+            b = int(t2s[t])
+            pos = t - int(cu[b]) + starts[b]
+            blk, off = int(bt[b, pos // bs]), pos % bs
+            want[t] = codes[blk, off].to(torch.float32) * scales[blk, off]
+        assert torch.equal(got, want)

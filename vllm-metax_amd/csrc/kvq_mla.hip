@@ -48,7 +48,83 @@ __global__ __launch_bounds__(256) void mla_quant_write_kernel(const void* __rest
   if (lane == 0) *reinterpret_cast<float*>(cache + blk * g.stride_block + g.scale_off + off * 4) = scale;
 }
 
+// Gather + dequantise latent rows into a dense [num_tokens, W] workspace (the chunked-context
+// prefill reads its cached context this way).  One wavefront per destination row: lanes 0 .. W/16-1
+// load 16 codes each (one coalesced run of W bytes), every lane reads the row's scale, and the 16
+// products code * scale go out as one or two 16-byte stores per lane.
+template <int DT>
+__global__ __launch_bounds__(256) void mla_gather_dequant_kernel(void* __restrict__ dst, int64_t dst_stride,
+                                                                 const uint8_t* __restrict__ cache, kvq_mla_geom g,
+                                                                 const int32_t* __restrict__ block_table,
+                                                                 int64_t bt_stride,
+                                                                 const int32_t* __restrict__ cu_seq_lens,
+                                                                 const int32_t* __restrict__ token_to_seq,
+                                                                 const int32_t* __restrict__ seq_starts,
+                                                                 int num_tokens) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int W = g.kv_lora_rank + g.rope_dim;
+  for (int64_t t = (int64_t)blockIdx.x * (blockDim.x / kWave) + (threadIdx.x / kWave); t < num_tokens;
+       t += (int64_t)gridDim.x * (blockDim.x / kWave)) {
+    const int b = token_to_seq[t];
+    if (t >= cu_seq_lens[b + 1]) continue;
+    int pos = (int)t - cu_seq_lens[b];
+    if (seq_starts != nullptr) pos += seq_starts[b];
+    const int e = pos / g.block_size;
+    const int off = pos - e * g.block_size;
+    const int64_t blk = block_table[(int64_t)b * bt_stride + e];
+    const uint8_t* base = cache + blk * g.stride_block;
+    const float scale = *reinterpret_cast<const float*>(base + g.scale_off + (int64_t)off * 4);
+    if (lane * 16 >= W) continue;
+    const u32x4 w = *reinterpret_cast<const u32x4_a4*>(base + (int64_t)off * g.stride_row + lane * 16);
+    float f[16];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const uint32_t x = w[i];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) f[4 * i + j] = (float)(int8_t)(x >> (8 * j)) * scale;
+    }
+    const int64_t at = t * dst_stride + lane * 16;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) store_act<DT>(dst, at + i, f[i]);
+  }
+}
+
 }  // namespace kvq
+
+extern "C" int kvq_gather_and_dequant_mla_int8(void* dst, int dst_dtype, int64_t dst_stride, const void* cache,
+                                               const kvq_mla_geom* geom, const int32_t* block_table,
+                                               int64_t bt_stride, const int32_t* cu_seq_lens,
+                                               const int32_t* token_to_seq, const int32_t* seq_starts,
+                                               int64_t num_tokens, kvq_stream_t stream) {
+  using namespace kvq;
+  const char* op = "gather_and_dequant_mla_int8";
+  KVQ_REQUIRE(geom != nullptr, "%s: geom is NULL", op);
+  KVQ_REQUIRE(num_tokens >= 0 && num_tokens <= 0x7fffffffLL, "%s: num_tokens out of range", op);
+  if (num_tokens == 0) return KVQ_OK;
+  KVQ_REQUIRE(dst && cache && block_table && cu_seq_lens && token_to_seq, "%s: NULL pointer", op);
+  const kvq_mla_geom& g = *geom;
+  const int W = g.kv_lora_rank + g.rope_dim;
+  KVQ_REQUIRE(g.kv_lora_rank > 0 && g.rope_dim >= 0 && g.block_size > 0, "%s: bad geometry", op);
+  KVQ_REQUIRE(W % 16 == 0 && W <= 1024, "%s: row width %d must be a multiple of 16, at most 1024", op, W);
+  KVQ_REQUIRE((g.stride_block | g.stride_row | g.scale_off) % 4 == 0 && ((uintptr_t)cache % 4) == 0,
+              "%s: cache strides must be 4-byte aligned", op);
+  KVQ_REQUIRE(dst_stride >= W, "%s: dst rows overlap", op);
+  hipStream_t s = as_stream(stream);
+  const int64_t want = (num_tokens + 3) / 4;
+  const unsigned blocks = (unsigned)(want < 65536 ? want : 65536);
+#define KVQ_MLAG(T)                                                                                      \
+  hipLaunchKernelGGL((mla_gather_dequant_kernel<T>), dim3(blocks), dim3(256), 0, s, dst, dst_stride,  \
+                     static_cast<const uint8_t*>(cache), g, block_table, bt_stride, cu_seq_lens,       \
+                     token_to_seq, seq_starts, (int)num_tokens)
+  switch (dst_dtype) {
+    case KVQ_F32: KVQ_MLAG(KVQ_F32); break;
+    case KVQ_BF16: KVQ_MLAG(KVQ_BF16); break;
+    case KVQ_F16: KVQ_MLAG(KVQ_F16); break;
+    default: return fail(KVQ_EINVAL, "%s: unknown dst_dtype %d", op, dst_dtype);
+  }
+#undef KVQ_MLAG
+  return check_hip(hipGetLastError(), "gather_and_dequant_mla_int8 launch");
+}
 
 extern "C" int kvq_concat_and_cache_mla_int8(const void* kv_c, const void* k_pe, int src_dtype,
                                              int64_t kv_c_stride, int64_t k_pe_stride, void* cache,

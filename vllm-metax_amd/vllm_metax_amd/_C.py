@@ -57,6 +57,7 @@ SIGNATURES = {
     "kvq_splitk_reduce": (_i, [_vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
     "kvq_merge_attn_states": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i64, _i, _i, _i64, _vp]),
     "kvq_concat_and_cache_mla_int8": (_i, [_vp, _vp, _i, _i64, _i64, _vp, _mla_p, _vp, _i64, _f, _vp]),
+    "kvq_gather_and_dequant_mla_int8": (_i, [_vp, _i, _i64, _vp, _mla_p, _vp, _i64, _vp, _vp, _vp, _i64, _vp]),
     "kvq_mla_decode_workspace_bytes": (_sz, [_i, _i, _i]),
     "kvq_mla_decode_int8": (_i, [_vp, _i, _vp, _vp, _i, _i64, _i64, _vp, _mla_p, _vp, _i64, _vp, _i, _i, _f,
                                  _vp, _sz, _vp]),

@@ -349,6 +349,39 @@ def concat_and_cache_mla(kv_c: torch.Tensor, k_pe: torch.Tensor, kv_cache: torch
     _C.check(rc, "concat_and_cache_mla")
 
 
+def gather_and_maybe_dequant_cache(src_cache: torch.Tensor, dst: torch.Tensor, block_table: torch.Tensor,
+                                   cu_seq_lens: torch.Tensor, token_to_seq: torch.Tensor, num_tokens: int,
+                                   kv_cache_dtype: str = "int8_per_token", scale: torch.Tensor | None = None,
+                                   seq_starts: torch.Tensor | None = None, kv_lora_rank: int = 512,
+                                   geometry: MlaGeometry | None = None) -> None:
+    """Argument order of ``gather_and_maybe_dequant_cache``
+    (csrc/libtorch_stable/cache_kernels.cu:1181-1247), for the int8 latent cache: ``dst[t] = code *
+    row scale`` of the row that token ``t`` of sequence ``token_to_seq[t]`` names.  ``scale`` (the
+    reference's per-tensor scale) is not used: every row carries its own."""
+    if kv_cache_dtype != "int8_per_token":
+        raise NotImplementedError(f"kv_cache_dtype {kv_cache_dtype!r}: only int8_per_token is built")
+    dev = _require_cuda(src_cache, dst, block_table, cu_seq_lens, token_to_seq, seq_starts)
+    geom = geometry or mla_geometry(src_cache, kv_lora_rank)
+    W = geom.kv_lora_rank + geom.rope_dim
+    if dst.dim() != 2 or dst.shape[1] != W or dst.stride(1) != 1 or dst.shape[0] < num_tokens:
+        raise RuntimeError(f"dst must be [>= num_tokens, {W}] with a contiguous last dim")
+    for name, t in (("block_table", block_table), ("cu_seq_lens", cu_seq_lens), ("token_to_seq", token_to_seq),
+                    ("seq_starts", seq_starts)):
+        if t is not None and t.dtype != torch.int32:
+            raise RuntimeError(f"{name} must be int32")
+    if block_table.stride(1) != 1 or not cu_seq_lens.is_contiguous() or not token_to_seq.is_contiguous():
+        raise RuntimeError("block_table rows, cu_seq_lens and token_to_seq must be contiguous")
+    if token_to_seq.numel() < num_tokens:
+        raise RuntimeError("token_to_seq is shorter than num_tokens")
+    g = geom.as_struct()
+    with torch.cuda.device(dev):
+        rc = _C.load().kvq_gather_and_dequant_mla_int8(
+            _ptr(dst), _dtype_code(dst, "dst"), dst.stride(0), ctypes.c_void_p(geom.base_ptr), ctypes.byref(g),
+            _ptr(block_table), block_table.stride(0), _ptr(cu_seq_lens), _ptr(token_to_seq), _ptr(seq_starts),
+            int(num_tokens), _stream(dev))
+    _C.check(rc, "gather_and_maybe_dequant_cache")
+
+
 def mla_decode_workspace_bytes(max_num_seqs: int, num_heads: int, kv_lora_rank: int) -> int:
     return int(_C.load().kvq_mla_decode_workspace_bytes(max_num_seqs, num_heads, kv_lora_rank))
 
