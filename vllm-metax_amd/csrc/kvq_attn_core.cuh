@@ -24,6 +24,7 @@
 namespace kvq {
 
 constexpr int kTile = 32;            // tokens per step
+constexpr int kSyncTiles = 2;        // workgroup rendezvous period of the decode stream, in tiles (power of two)
 constexpr float kPScale = 256.0f;    // P~ is kept 2^8 larger so small weights stay normal in fp16
 constexpr float kLn2 = 0.6931471805599453f;
 constexpr float kLog2e = 1.4426950408889634f;
@@ -459,6 +460,12 @@ struct DecodeTile {
       compute<false>(lo, qb, s_init, len, t, lane, lds, st);
       phase_fence();
       ++t;
+      // The waves of a workgroup read neighbouring records of the same tokens (one kv head each);
+      // the 128-byte lines at record boundaries are shared between them.  A rendezvous every few
+      // tiles keeps the waves within a few tiles of each other, so the second reader of such a
+      // line still finds it in L2 instead of fetching it from HBM again.  (Every wave of the
+      // workgroup runs the same tile range, so the barrier count is uniform.)
+      if ((t & (kSyncTiles - 1)) == 0) __builtin_amdgcn_s_barrier();
     }
     stage(a, lo, sc_mul, lane, lds);
     compute_any(lo, qb, s_init, len, t, lane, lds, st);
