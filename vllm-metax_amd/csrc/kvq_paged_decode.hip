@@ -149,6 +149,38 @@ __global__ __launch_bounds__(256) void paged_decode_streamk_reduce_kernel(Stream
   float m = -INFINITY, l = 0.f, acc[V];
 #pragma unroll
   for (int i = 0; i < V; ++i) acc[i] = 0.f;
+  // Few slots (the usual case: a sequence spans a handful of workgroups): the (m, l) pairs and ALL
+  // the partial outputs are requested in one go, so the kernel pays one memory round trip for them
+  // instead of two.
+  constexpr int kFew = 8;
+  if (w_last - w_first < kFew) {
+    const int w = w_first + lane;
+    const bool live = w <= w_last && wg_tile_begin(w, total, P) < wg_tile_begin(w + 1, total, P);
+    const int64_t slot = (int64_t)min(w, w_last) + seq;
+    const uint32_t keep = live ? 0xffffffffu : 0u;
+    const float mj_raw = a.part_ml[(slot * a.io.num_q_heads + head) * 2 + 0];
+    const float lj_raw = a.part_ml[(slot * a.io.num_q_heads + head) * 2 + 1];
+    float po[kFew][V];
+#pragma unroll
+    for (int k = 0; k < kFew; ++k) {
+      const int64_t sk = (int64_t)min(w_first + k, w_last) + seq;
+      const float* p = a.part_o + (sk * a.io.num_q_heads + head) * (int64_t)D + lane * V;
+#pragma unroll
+      for (int i = 0; i < V; ++i) po[k][i] = p[i];
+    }
+    const float mj = live ? as_f32(as_u32(mj_raw) & keep) : -INFINITY;
+    const float lj = as_f32(as_u32(lj_raw) & keep);
+    m = wave_max(mj);
+    const float ej = live ? __builtin_amdgcn_exp2f(mj - m) : 0.f;
+    l = wave_sum(lj * ej);
+#pragma unroll
+    for (int k = 0; k < kFew; ++k) {
+      const float wk = __shfl(ej, k, kWave);  // 0 for slots past the last and for empty ones
+      const uint32_t kk = wk != 0.f ? 0xffffffffu : 0u;
+#pragma unroll
+      for (int i = 0; i < V; ++i) acc[i] += as_f32(as_u32(po[k][i]) & kk) * wk;
+    }
+  } else
   for (int wb = w_first; wb <= w_last; wb += kWave) {
     const int w = wb + lane;
     const bool live = w <= w_last && wg_tile_begin(w, total, P) < wg_tile_begin(w + 1, total, P);
