@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define KVQ_ABI_VERSION 1
+#define KVQ_ABI_VERSION 2
 
 #define KVQ_OK 0
 #define KVQ_EINVAL (-22)
@@ -123,14 +123,22 @@ KVQ_API size_t kvq_paged_attn_workspace_bytes(int max_num_seqs, int num_q_heads,
  * rows of single-token sequences go to the bandwidth-bound split-K tile, longer
  * query runs to the MFMA prefill tile.  lse (optional, [num_tokens, num_q_heads]
  * fp32, natural log) may be NULL.
+ *
+ * window_size > 0: a query at position p sees keys p - window_size + 1 .. p only
+ * (the reference passes window_size = (sliding_window - 1, 0),
+ * vllm_metax/v1/attention/backends/triton_attn.py:507-512, 701; needs `causal`);
+ * 0 = no window.  softcap > 0: logits become softcap * tanh(scale * q.k / softcap)
+ * (triton_attn.py:703; semantics as in the reference's test oracle,
+ * tests/kernels/attention/test_triton_unified_attention.py:63-70); 0 = none.
  */
 KVQ_API int kvq_paged_attn_int8(void* out, int out_dtype, int64_t out_stride_t, int64_t out_stride_h,
                         const void* q, int q_dtype, int64_t q_stride_t, int64_t q_stride_h,
                         const void* cache, const kvq_cache_geom* geom,
                         const int32_t* block_table, int64_t bt_stride, const int32_t* seq_lens,
                         const int32_t* cu_seqlens_q, int num_seqs, int num_q_heads,
-                        int max_query_len, float scale, int causal, float* lse,
-                        void* workspace, size_t workspace_bytes, kvq_stream_t stream);
+                        int max_query_len, float scale, int causal, int window_size,
+                        float softcap, float* lse, void* workspace, size_t workspace_bytes,
+                        kvq_stream_t stream);
 
 /*
  * Fixed-partition split-K decode + reduce (one query row per sequence).

@@ -167,8 +167,10 @@ def cache_write(key, value, kv_cache, lay: RecordLayout, slot_mapping, eps: floa
 
 
 def paged_attn(q, kv_cache, lay: RecordLayout, block_table, seq_lens, cu_seqlens_q,
-               scale: float, causal: bool = True, return_lse: bool = False):
-    """q [N, Hq, D] -> out fp32 [N, Hq, D] (and lse fp32 [N, Hq])."""
+               scale: float, causal: bool = True, return_lse: bool = False, sliding_window: int = 0,
+               soft_cap: float = 0.0):
+    """q [N, Hq, D] -> out fp32 [N, Hq, D] (and lse fp32 [N, Hq]).  sliding_window > 0: a query sees its
+    last `sliding_window` keys (itself included); soft_cap > 0: logits -> cap * tanh(logit / cap)."""
     qf = _f32c(q)
     N, Hq, D = qf.shape
     bt, sl, cu = _i32c(block_table), _i32c(seq_lens), _i32c(cu_seqlens_q)
@@ -176,15 +178,16 @@ def paged_attn(q, kv_cache, lay: RecordLayout, block_table, seq_lens, cu_seqlens
     out = torch.empty((N, Hq, D), dtype=torch.float32)
     lse = torch.empty((N, Hq), dtype=torch.float32) if return_lse else None
     _check(
-        lib().kvq_oracle_paged_attn(
+        lib().kvq_oracle_paged_attn_ex(
             _p(out), _p(lse), _p(qf), _p(kv_cache),
             _i64(lay.k_off), _i64(lay.v_off), _i64(lay.ks_off), _i64(lay.vs_off),
             _i64(lay.stride_block), _i64(lay.stride_slot), _i64(lay.stride_head),
             _p(bt), _i64(bt.stride(0)), _p(sl), _p(cu),
             ctypes.c_int(B), ctypes.c_int(Hq), ctypes.c_int(lay.num_kv_heads), ctypes.c_int(D),
             ctypes.c_int(lay.block_size), ctypes.c_float(scale), ctypes.c_int(1 if causal else 0),
+            ctypes.c_int(int(sliding_window or 0)), ctypes.c_float(float(soft_cap or 0.0)),
         ),
-        "kvq_oracle_paged_attn",
+        "kvq_oracle_paged_attn_ex",
     )
     return (out, lse) if return_lse else out
 

@@ -130,7 +130,7 @@ static void attend_range(const float* q, int D, const uint8_t* cache,
                          int64_t k_off, int64_t v_off, int64_t ks_off, int64_t vs_off,
                          int64_t stride_block, int64_t stride_slot, int64_t stride_head,
                          const int32_t* bt_row, int block_size, int hkv,
-                         int64_t k_begin, int64_t k_end, double scale,
+                         int64_t k_begin, int64_t k_end, double scale, double softcap,
                          double* acc, double* m_out, double* l_out, double* logits) {
   double m = -INFINITY;
   for (int64_t j = k_begin; j < k_end; ++j) {
@@ -143,6 +143,7 @@ static void attend_range(const float* q, int D, const uint8_t* cache,
     double s = 0.0;
     for (int d = 0; d < D; ++d) s += (double)q[d] * ((double)kc[d] * (double)ks);
     s *= scale;
+    if (softcap > 0.0) s = softcap * tanh(s / softcap);
     logits[j - k_begin] = s;
     if (s > m) m = s;
   }
@@ -180,13 +181,16 @@ static void attend_range(const float* q, int D, const uint8_t* cache,
  * out [N, Hq, D] fp32; lse [N, Hq] fp32 or NULL (natural-log sum-exp of the
  * scaled logits).  Rows with no visible key produce zeros and lse = -inf.
  * ------------------------------------------------------------------------- */
-KVQ_EXPORT int kvq_oracle_paged_attn(
+/* window > 0: a query at position p sees keys p - window + 1 .. p only (the
+ * sliding_window mask of ref_paged_attn, :60-66).  softcap > 0: scaled logits
+ * become softcap * tanh(logit / softcap) before masking (:67-68).           */
+KVQ_EXPORT int kvq_oracle_paged_attn_ex(
     float* out, float* lse, const float* q, const uint8_t* cache,
     int64_t k_off, int64_t v_off, int64_t ks_off, int64_t vs_off,
     int64_t stride_block, int64_t stride_slot, int64_t stride_head,
     const int32_t* block_table, int64_t bt_stride, const int32_t* seq_lens,
     const int32_t* cu_seqlens_q, int B, int Hq, int Hkv, int D, int block_size,
-    float scale, int causal) {
+    float scale, int causal, int window, float softcap) {
   if (!out || !q || !cache || !block_table || !seq_lens || !cu_seqlens_q) return -1;
   if (Hkv <= 0 || Hq % Hkv != 0) return -1;
   const int G = Hq / Hkv;
@@ -210,8 +214,13 @@ KVQ_EXPORT int kvq_oracle_paged_attn(
           for (int64_t r = 0; r < qlen; ++r) {
             int64_t vis = causal ? (kvlen - qlen + r + 1) : kvlen;
             if (vis > kvlen) vis = kvlen;
+            int64_t first = 0;
+            if (window > 0) {
+              first = (kvlen - qlen + r + 1) - window;
+              if (first < 0) first = 0;
+            }
             float* o = out + ((q0 + r) * Hq + h) * (int64_t)D;
-            if (vis <= 0) {
+            if (vis <= first) {
               for (int d = 0; d < D; ++d) o[d] = 0.0f;
               if (lse) lse[(q0 + r) * Hq + h] = -INFINITY;
               continue;
@@ -219,8 +228,8 @@ KVQ_EXPORT int kvq_oracle_paged_attn(
             double m, l;
             attend_range(q + ((q0 + r) * Hq + h) * (int64_t)D, D, cache, k_off, v_off,
                          ks_off, vs_off, stride_block, stride_slot, stride_head,
-                         block_table + (int64_t)i * bt_stride, block_size, h / G, 0, vis,
-                         (double)scale, acc, &m, &l, logits);
+                         block_table + (int64_t)i * bt_stride, block_size, h / G, first, vis,
+                         (double)scale, (double)softcap, acc, &m, &l, logits);
             for (int d = 0; d < D; ++d) o[d] = (float)(acc[d] / l);
             if (lse) lse[(q0 + r) * Hq + h] = (float)(m + log(l));
           }
@@ -231,6 +240,18 @@ KVQ_EXPORT int kvq_oracle_paged_attn(
     free(logits);
   }
   return err ? -2 : 0;
+}
+
+KVQ_EXPORT int kvq_oracle_paged_attn(
+    float* out, float* lse, const float* q, const uint8_t* cache,
+    int64_t k_off, int64_t v_off, int64_t ks_off, int64_t vs_off,
+    int64_t stride_block, int64_t stride_slot, int64_t stride_head,
+    const int32_t* block_table, int64_t bt_stride, const int32_t* seq_lens,
+    const int32_t* cu_seqlens_q, int B, int Hq, int Hkv, int D, int block_size,
+    float scale, int causal) {
+  return kvq_oracle_paged_attn_ex(out, lse, q, cache, k_off, v_off, ks_off, vs_off, stride_block,
+                                  stride_slot, stride_head, block_table, bt_stride, seq_lens,
+                                  cu_seqlens_q, B, Hq, Hkv, D, block_size, scale, causal, 0, 0.0f);
 }
 
 /* ---------------------------------------------------------------------------
@@ -279,7 +300,7 @@ KVQ_EXPORT int kvq_oracle_paged_attn_partition(
             attend_range(q + ((int64_t)i * Hq + h) * D, D, cache, k_off, v_off, ks_off,
                          vs_off, stride_block, stride_slot, stride_head,
                          block_table + (int64_t)i * bt_stride, block_size, h / G, b0, b1,
-                         (double)scale, acc, &m, &l, logits);
+                         (double)scale, 0.0, acc, &m, &l, logits);
             int64_t idx = ((int64_t)i * Hq + h) * max_parts + j;
             for (int d = 0; d < D; ++d) tmp_out[idx * D + d] = (float)(acc[d] / l);
             max_logits[idx] = (float)m;

@@ -1,7 +1,8 @@
 """GPU parity of chunked prefill and mixed decode + prefill batches over the int8 cache, through
 the C ABI's varlen entry point, against the oracle (causal attention of a query run of q_len
 tokens that ends at the sequence end; the run's own K/V are already in the cache, as in the
-reference's unified kernel, vllm_metax/v1/attention/ops/triton_unified_attention.py:56-246)."""
+unified attention op the reference calls, vllm_metax/v1/attention/backends/triton_attn.py:688-725,
+and in its test oracle, tests/kernels/attention/test_triton_unified_attention.py:26-78)."""
 import math
 
 import pytest

@@ -81,6 +81,30 @@ def test_paged_attn_vs_as_written_reference_op():
     T.assert_close_attn(want16, out, what="as-written bf16 op vs oracle")
 
 
+@pytest.mark.parametrize("window,cap", [(16, 0.0), (64, 0.0), (1000, 0.0), (0, 30.0), (40, 5.0)])
+def test_sliding_window_and_soft_cap_vs_as_written_reference_op(window, cap):
+    """The same op with its sliding_window / soft_cap arguments
+    (tests/kernels/attention/test_triton_unified_attention.py:38-39,60-68), fp32 instance; and two
+    closed forms: a window at least as long as the sequence changes nothing, a huge cap changes nothing."""
+    hq, hkv, d, bs = 8, 2, 64, 16
+    ctx, ql = [100, 463, 18, 1], [1, 129, 5, 1]
+    kv, views, lay, bt, q, cu, sl = _build(ctx, ql, hq, hkv, d, bs, "NHD", 11)
+    q = q * 3.0                                    # logits large enough for the cap to bite
+    scale = d ** -0.5
+    out = oracle.paged_attn(q, T.storage_bytes(kv), lay, bt, sl, cu, scale, sliding_window=window, soft_cap=cap)
+    k, v, ks, vs = views
+    kd, vd = torch_ref.dequant_cache(k, v, ks, vs, d, torch.float32)
+    want = torch_ref.paged_attn(q.float(), kd, vd, ql, ctx, bt, scale, sliding_window=window or None, soft_cap=cap or None)
+    torch.testing.assert_close(out, want, atol=3e-5, rtol=1e-5)
+    plain = oracle.paged_attn(q, T.storage_bytes(kv), lay, bt, sl, cu, scale)
+    if window >= max(ctx) and cap == 0.0:
+        assert torch.equal(out, plain)
+    else:
+        assert not torch.equal(out, plain)
+    big = oracle.paged_attn(q, T.storage_bytes(kv), lay, bt, sl, cu, scale, soft_cap=1e6)
+    torch.testing.assert_close(big, plain, atol=1e-5, rtol=1e-5)
+
+
 def test_block_permutation_invariance_and_noncausal():
     hq, hkv, d, bs = 4, 2, 64, 16
     ctx, ql = [50, 33], [1, 3]

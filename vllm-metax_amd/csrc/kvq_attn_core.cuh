@@ -85,7 +85,20 @@ struct AttnIO {
   int group;  // q heads per kv head
   float scale_log2;  // softmax scale * log2(e)
   uint32_t bs_magic;  // ceil(2^32 / block_size): x / block_size == umulhi(x, bs_magic) for x < 2^22
+  int window;         // sliding window: a query sees its last `window` keys, itself included; 0 = all
+  float cap_c;        // logits soft cap in the log2 domain, cap * log2(e); 0 = none
+  float cap_k;        // 2 * log2(e) / cap_c
 };
+
+// cap * tanh(x / cap) for a log2-domain logit x: tanh(u) = 1 - 2 / (exp(2u) + 1).
+__device__ __forceinline__ float soft_cap(float x, float cap_c, float cap_k) {
+  return cap_c - 2.0f * cap_c * __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(x * cap_k) + 1.0f);
+}
+
+// First token a decode row of a `len`-token sequence sees.
+__device__ __forceinline__ int window_first(int len, int window) {
+  return window > 0 && len > window ? len - window : 0;
+}
 
 // One lane's share of a 32-token tile as it arrives from HBM: raw 16-byte chunks of records.
 template <int D>
@@ -302,9 +315,10 @@ struct DecodeTile {
   // Phase 1 of a tile: S^T = K . Q^T on the MFMA from the LDS window, online softmax.  Returns
   // P~^T as the MFMA B operand.  MASK: the tile holds the end of the sequence (tokens >= len must
   // not contribute).
-  template <bool MASK>
-  __device__ static half8_t qk_softmax(const LaneOffsets& lo, const half8_t (&qb)[KSTEPS], float s_init, int len,
-                                       int t, int lane, const uint8_t* lds, State& st) {
+  // CAP: logits pass through the soft cap.  Tokens outside [first, len) never contribute.
+  template <bool MASK, bool CAP>
+  __device__ static half8_t qk_softmax(const AttnIO& io, const LaneOffsets& lo, const half8_t (&qb)[KSTEPS], float s_init,
+                                       int len, int first, int t, int lane, const uint8_t* lds, State& st) {
     const int g = lane >> 4;
     const float* sc_lds = reinterpret_cast<const float*>(lds + LDS_TILE);
     const floatx4 ks0 = *reinterpret_cast<const floatx4*>(sc_lds + 4 * g);
@@ -332,7 +346,8 @@ struct DecodeTile {
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         float x = s[mt][i] * (mt ? ks1 : ks0)[i];
-        if constexpr (MASK) x = ((tok_base + mt * 16 + i) < len) ? x : -INFINITY;
+        if constexpr (CAP) x = soft_cap(x, io.cap_c, io.cap_k);
+        if constexpr (MASK) x = ((uint32_t)(tok_base + mt * 16 + i - first) < (uint32_t)(len - first)) ? x : -INFINITY;
         logit[mt * 4 + i] = x;
         mloc = fmaxf(mloc, x);
       }
@@ -359,7 +374,8 @@ struct DecodeTile {
         const float p = __builtin_amdgcn_exp2f(logit[j] - st.m);  // masked: exp2(-inf) = 0
         st.l += p;
         float x = p * (mt ? vs1 : vs0)[i];
-        if constexpr (MASK) x = ((tok_base + mt * 16 + i) < len) ? x : 0.f;  // garbage scales never enter
+        if constexpr (MASK)  // garbage scales never enter
+          x = ((uint32_t)(tok_base + mt * 16 + i - first) < (uint32_t)(len - first)) ? x : 0.f;
         pt[j] = x;
       }
     }
@@ -406,16 +422,17 @@ struct DecodeTile {
     }
   }
 
-  template <bool MASK>
-  __device__ static void compute(const LaneOffsets& lo, const half8_t (&qb)[KSTEPS], float s_init, int len, int t,
-                                 int lane, const uint8_t* lds, State& st) {
-    const half8_t p = qk_softmax<MASK>(lo, qb, s_init, len, t, lane, lds, st);
+  template <bool MASK, bool CAP>
+  __device__ static void compute(const AttnIO& io, const LaneOffsets& lo, const half8_t (&qb)[KSTEPS], float s_init, int len,
+                                 int first, int t, int lane, const uint8_t* lds, State& st) {
+    const half8_t p = qk_softmax<MASK, CAP>(io, lo, qb, s_init, len, first, t, lane, lds, st);
     pv(lo, p, lds, st);
   }
-  __device__ static void compute_any(const LaneOffsets& lo, const half8_t (&qb)[KSTEPS], float s_init, int len, int t,
-                                     int lane, const uint8_t* lds, State& st) {
-    if ((t + 1) * kTile > len) compute<true>(lo, qb, s_init, len, t, lane, lds, st);
-    else compute<false>(lo, qb, s_init, len, t, lane, lds, st);
+  template <bool CAP>
+  __device__ static void compute_any(const AttnIO& io, const LaneOffsets& lo, const half8_t (&qb)[KSTEPS], float s_init,
+                                     int len, int first, int t, int lane, const uint8_t* lds, State& st) {
+    if ((t + 1) * kTile > len || t * kTile < first) compute<true, CAP>(io, lo, qb, s_init, len, first, t, lane, lds, st);
+    else compute<false, CAP>(io, lo, qb, s_init, len, first, t, lane, lds, st);
   }
 
   // Keeps the instruction scheduler from moving work across the phase boundaries of the
@@ -429,7 +446,10 @@ struct DecodeTile {
   // next tile, so one tile of loads per wave is in flight while one is computed (measured on
   // MI355X: a second tile in flight per wave lowers the achieved HBM bandwidth).
   // `lds` is this wave's private LDS_WAVE-byte window.
-  __device__ static void run(const AttnIO& io, int seq, int64_t row, int len, int t_begin, int t_end, int hkv,
+  // Tokens before `first` (the sliding window's lower edge; 0 without a window) do not contribute;
+  // t_begin is then the tile that holds `first` or a later one.
+  template <bool CAP>
+  __device__ static void run(const AttnIO& io, int seq, int64_t row, int len, int first, int t_begin, int t_end, int hkv,
                              int lane, uint8_t* lds, State& st) {
     const LaneOffsets lo = lane_offsets(io.g, lane);
     const int32_t* bt_row = io.block_table + (int64_t)seq * io.bt_stride;
@@ -448,6 +468,19 @@ struct DecodeTile {
     st.psum = (floatx4){0.f, 0.f, 0.f, 0.f};
     st.m = -INFINITY;
     st.l = 0.f;
+    // a first tile that straddles the window's lower edge is masked; it is peeled off so that the
+    // steady loop below keeps a single, unmasked body
+    if (t + 1 < t_end && t * kTile < first) {
+      const Window w = window(io, nb, t + 1, hkv);
+      stage(a, lo, sc_mul, lane, lds);
+      phase_fence();
+      load_tile(io, w, lo, a);
+      phase_fence();
+      nb = fetch_blocks(io, bt_row, len, t + 2);
+      compute<true, CAP>(io, lo, qb, s_init, len, first, t, lane, lds, st);
+      phase_fence();
+      ++t;
+    }
     // steady state: tile t+1 exists, so the refill is unconditional and tile t does not end the
     // sequence
     while (t + 1 < t_end) {
@@ -457,7 +490,7 @@ struct DecodeTile {
       load_tile(io, w, lo, a);
       phase_fence();
       nb = fetch_blocks(io, bt_row, len, t + 2);
-      compute<false>(lo, qb, s_init, len, t, lane, lds, st);
+      compute<false, CAP>(io, lo, qb, s_init, len, first, t, lane, lds, st);
       phase_fence();
       ++t;
       // The waves of a workgroup read neighbouring records of the same tokens (one kv head each);
@@ -468,7 +501,7 @@ struct DecodeTile {
       if ((t & (kSyncTiles - 1)) == 0) __builtin_amdgcn_s_barrier();
     }
     stage(a, lo, sc_mul, lane, lds);
-    compute_any(lo, qb, s_init, len, t, lane, lds, st);
+    compute_any<CAP>(io, lo, qb, s_init, len, first, t, lane, lds, st);
   }
 
   // Sum of the lane-local l over the 4 lane groups of a head.

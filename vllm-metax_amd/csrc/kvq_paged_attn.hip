@@ -21,7 +21,7 @@ extern "C" int kvq_paged_attn_int8(void* out, int out_dtype, int64_t out_stride_
                                    const void* cache, const kvq_cache_geom* geom, const int32_t* block_table,
                                    int64_t bt_stride, const int32_t* seq_lens, const int32_t* cu_seqlens_q,
                                    int num_seqs, int num_q_heads, int max_query_len, float scale, int causal,
-                                   float* lse, void* workspace, size_t workspace_bytes, kvq_stream_t stream) {
+                                   int window_size, float softcap, float* lse, void* workspace, size_t workspace_bytes, kvq_stream_t stream) {
   using namespace kvq;
   const char* op = "paged_attn_int8";
   KVQ_REQUIRE(geom != nullptr, "%s: geom is NULL", op);
@@ -29,6 +29,9 @@ extern "C" int kvq_paged_attn_int8(void* out, int out_dtype, int64_t out_stride_
   KVQ_REQUIRE(num_seqs > 0 && num_q_heads > 0, "%s: num_seqs and num_q_heads must be positive", op);
   KVQ_REQUIRE(max_query_len >= 1, "%s: max_query_len must be >= 1", op);
   KVQ_REQUIRE(max_query_len == 1 || cu_seqlens_q != nullptr, "%s: cu_seqlens_q is required when max_query_len > 1", op);
+  KVQ_REQUIRE(window_size >= 0, "%s: window_size %d must be >= 0 (0 = no sliding window)", op, window_size);
+  KVQ_REQUIRE(window_size == 0 || causal, "%s: a sliding window needs causal attention", op);
+  KVQ_REQUIRE(softcap >= 0.f && softcap == softcap, "%s: softcap must be >= 0 (0 = none)", op);
   const kvq_cache_geom& g = *geom;
   KVQ_REQUIRE(g.num_kv_heads > 0 && num_q_heads % g.num_kv_heads == 0,
               "%s: num_q_heads %d is not a multiple of num_kv_heads %d", op, num_q_heads, g.num_kv_heads);
@@ -69,6 +72,9 @@ extern "C" int kvq_paged_attn_int8(void* out, int out_dtype, int64_t out_stride_
   a.io.group = num_q_heads / g.num_kv_heads;
   a.io.scale_log2 = scale * kLog2e;
   a.io.bs_magic = (uint32_t)((0x100000000ull + (uint64_t)geom->block_size - 1) / (uint64_t)geom->block_size);
+  a.io.window = window_size;
+  a.io.cap_c = softcap * kLog2e;
+  a.io.cap_k = softcap > 0.f ? 2.0f / softcap : 0.f;  // 2 log2(e) / cap_c
   a.seq_lens = seq_lens;
   a.cu_seqlens_q = cu_seqlens_q;
   a.num_seqs = num_seqs;

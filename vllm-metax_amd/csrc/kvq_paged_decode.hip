@@ -27,19 +27,21 @@ __device__ __forceinline__ int wave_incl_scan(int v, int lane) {
   return v;
 }
 
-// Tiles a sequence contributes to the decode tile line (0 for prefill sequences).
-__device__ __forceinline__ int decode_tiles(const int32_t* seq_lens, const int32_t* cu, int s, int num_seqs) {
+// Tiles a sequence contributes to the decode tile line (0 for prefill sequences): the tiles that
+// hold a token of the row's window, [window_first / 32, ceil(len / 32)).
+__device__ __forceinline__ int decode_tiles(const int32_t* seq_lens, const int32_t* cu, int s, int num_seqs,
+                                            int window) {
   if (s >= num_seqs) return 0;
   if (cu != nullptr && (cu[s + 1] - cu[s]) != 1) return 0;
   const int len = seq_lens[s];
-  return len > 0 ? (len + kTile - 1) / kTile : 0;
+  return len > 0 ? (len + kTile - 1) / kTile - window_first(len, window) / kTile : 0;
 }
 
 __device__ __forceinline__ int64_t wg_tile_begin(int w, int64_t total, int num_wg) {
   return ((int64_t)w * total) / num_wg;
 }
 
-template <int D, int QDT, int ODT, int WPW>
+template <int D, int QDT, int ODT, int WPW, bool CAP>
 __global__ __launch_bounds__(WPW * 64) void paged_decode_streamk_kernel(StreamKArgs a) {
   using DTile = DecodeTile<D, QDT, ODT>;
   __shared__ __align__(16) uint8_t lds[WPW][DTile::LDS_WAVE];
@@ -53,7 +55,7 @@ __global__ __launch_bounds__(WPW * 64) void paged_decode_streamk_kernel(StreamKA
   // total tiles (each wave redoes this tiny scan; no LDS, no barrier)
   int64_t total = 0;
   for (int base = 0; base < B; base += kWave) {
-    int n = decode_tiles(a.seq_lens, a.cu_seqlens_q, base + lane, B);
+    int n = decode_tiles(a.seq_lens, a.cu_seqlens_q, base + lane, B, a.io.window);
     n = wave_incl_scan(n, lane);
     total += __builtin_amdgcn_readlane(n, 63);
   }
@@ -67,7 +69,7 @@ __global__ __launch_bounds__(WPW * 64) void paged_decode_streamk_kernel(StreamKA
   {
     int64_t cum = 0;
     for (int base = 0; base < B; base += kWave) {
-      const int n = decode_tiles(a.seq_lens, a.cu_seqlens_q, base + lane, B);
+      const int n = decode_tiles(a.seq_lens, a.cu_seqlens_q, base + lane, B, a.io.window);
       const int incl = wave_incl_scan(n, lane);
       const int64_t first = cum + incl - n, last = cum + incl;
       const uint64_t hit = __builtin_amdgcn_ballot_w64(n > 0 && first <= lo && lo < last);
@@ -84,19 +86,21 @@ __global__ __launch_bounds__(WPW * 64) void paged_decode_streamk_kernel(StreamKA
 
   int64_t pos = lo;
   while (pos < hi && seq < B) {
-    const int ntiles = __builtin_amdgcn_readfirstlane(decode_tiles(a.seq_lens, a.cu_seqlens_q, seq, B));
+    const int ntiles = __builtin_amdgcn_readfirstlane(decode_tiles(a.seq_lens, a.cu_seqlens_q, seq, B, a.io.window));
     if (ntiles == 0) {
       ++seq;
       continue;
     }
     const int len = __builtin_amdgcn_readfirstlane(a.seq_lens[seq]);
     const int64_t row = a.cu_seqlens_q ? (int64_t)a.cu_seqlens_q[seq] : (int64_t)seq;
-    const int t_begin = __builtin_amdgcn_readfirstlane((int)(pos - seq_start));
+    const int first = window_first(len, a.io.window);  // tokens before it are outside the window
+    const int t0 = first / kTile;                      // the sequence's tile line starts at this tile
+    const int t_begin = __builtin_amdgcn_readfirstlane(t0 + (int)(pos - seq_start));
     const int64_t rem = hi - seq_start;
-    const int t_end = __builtin_amdgcn_readfirstlane(rem < ntiles ? (int)rem : ntiles);
+    const int t_end = __builtin_amdgcn_readfirstlane(t0 + (rem < ntiles ? (int)rem : ntiles));
     typename DTile::State st;
-    DTile::run(a.io, seq, row, len, t_begin, t_end, hkv, lane, lds[wave], st);
-    if (t_begin == 0 && t_end == ntiles) {
+    DTile::template run<CAP>(a.io, seq, row, len, first, t_begin, t_end, hkv, lane, lds[wave], st);
+    if (t_begin == t0 && t_end == t0 + ntiles) {
       DTile::emit_final(a.io, row, hkv, lane, st);
     } else {
       DTile::emit_partial(a.io, a.part_o, a.part_ml, (int64_t)w + seq, hkv, lane, st);
@@ -121,10 +125,10 @@ __global__ __launch_bounds__(256) void paged_decode_streamk_reduce_kernel(Stream
   const int q0 = a.cu_seqlens_q ? a.cu_seqlens_q[seq] : seq;
   const int q1 = a.cu_seqlens_q ? a.cu_seqlens_q[seq + 1] : seq + 1;
   const int len = a.seq_lens[seq];
-  int n_first = decode_tiles(a.seq_lens, a.cu_seqlens_q, lane, B);  // first 64 sequences of the scan
+  int n_first = decode_tiles(a.seq_lens, a.cu_seqlens_q, lane, B, a.io.window);  // first 64 sequences of the scan
   if (q1 - q0 != 1) return;
   const int64_t row = q0;
-  const int ntiles = len > 0 ? (len + kTile - 1) / kTile : 0;
+  const int ntiles = len > 0 ? (len + kTile - 1) / kTile - window_first(len, a.io.window) / kTile : 0;
   if (ntiles == 0) {  // empty sequence: defined output (zeros, lse = -inf)
     for (int i = 0; i < V; ++i)
       store_act<ODT>(a.io.out, row * a.io.out_stride_t + (int64_t)head * a.io.out_stride_h + lane * V + i, 0.f);
@@ -133,7 +137,7 @@ __global__ __launch_bounds__(256) void paged_decode_streamk_reduce_kernel(Stream
   }
   int64_t total = 0, start = 0;
   for (int base = 0; base < B; base += kWave) {
-    int n = base == 0 ? n_first : decode_tiles(a.seq_lens, a.cu_seqlens_q, base + lane, B);
+    int n = base == 0 ? n_first : decode_tiles(a.seq_lens, a.cu_seqlens_q, base + lane, B, a.io.window);
     const int incl = wave_incl_scan(n, lane);
     if (seq >= base && seq < base + kWave) start = total + __builtin_amdgcn_readlane(incl - n, seq - base);
     total += __builtin_amdgcn_readlane(incl, 63);
@@ -243,7 +247,7 @@ __global__ __launch_bounds__(WPW * 64) void paged_decode_v2_kernel(V2Args a) {
   if (t_begin >= ntiles) return;
   const int t_end = min(ntiles, t_begin + a.partition_tiles);
   typename DTile::State st;
-  DTile::run(a.io, seq, seq, len, t_begin, t_end, hkv, lane, lds[wave], st);
+  DTile::template run<false>(a.io, seq, seq, len, 0, t_begin, t_end, hkv, lane, lds[wave], st);
   DTile::emit_v2(a.io, a.tmp_out, a.max_logits, a.exp_sums, seq, part, a.max_parts, hkv, lane, st);
 }
 
@@ -327,12 +331,24 @@ static int launch_streamk(const StreamKArgs& a, hipStream_t s) {
   const int hkv = a.io.g.num_kv_heads;
   const int wpw = waves_per_wg(hkv);
   dim3 grid(a.num_wg, (hkv + wpw - 1) / wpw);
-  switch (wpw) {
-    case 8: hipLaunchKernelGGL((paged_decode_streamk_kernel<D, QDT, ODT, 8>), grid, dim3(512), 0, s, a); break;
-    case 4: hipLaunchKernelGGL((paged_decode_streamk_kernel<D, QDT, ODT, 4>), grid, dim3(256), 0, s, a); break;
-    case 2: hipLaunchKernelGGL((paged_decode_streamk_kernel<D, QDT, ODT, 2>), grid, dim3(128), 0, s, a); break;
-    default: hipLaunchKernelGGL((paged_decode_streamk_kernel<D, QDT, ODT, 1>), grid, dim3(64), 0, s, a); break;
+#define KVQ_SK(W, C) \
+  hipLaunchKernelGGL((paged_decode_streamk_kernel<D, QDT, ODT, W, C>), grid, dim3(W * 64), 0, s, a)
+  if (a.io.cap_c != 0.f) {
+    switch (wpw) {
+      case 8: KVQ_SK(8, true); break;
+      case 4: KVQ_SK(4, true); break;
+      case 2: KVQ_SK(2, true); break;
+      default: KVQ_SK(1, true); break;
+    }
+  } else {
+    switch (wpw) {
+      case 8: KVQ_SK(8, false); break;
+      case 4: KVQ_SK(4, false); break;
+      case 2: KVQ_SK(2, false); break;
+      default: KVQ_SK(1, false); break;
+    }
   }
+#undef KVQ_SK
   int rc = check_hip(hipGetLastError(), "paged_attn_int8 decode launch");
   if (rc) return rc;
   dim3 rgrid(a.num_seqs, (a.io.num_q_heads + 3) / 4);

@@ -1,9 +1,9 @@
 // Chunked-prefill tile over the int8 paged cache (gfx950, wave64, MFMA f16): query runs longer
 // than one token, causal, reading context and the run's own tokens from the cache.
 //
-// The MFMA N dimension carries (query token, q head of the group) pairs -- the BLOCK_M =
-// BLOCK_Q x queries-per-kv folding of the reference's unified kernel
-// (vllm_metax/v1/attention/ops/triton_unified_attention.py:56-246) -- so one pass over a kv head's
+// The MFMA N dimension carries (query token, q head of the group) pairs -- the
+// folding of query tokens and the q heads of a kv group that the unified attention op the reference
+// calls does (vllm_metax/v1/attention/backends/triton_attn.py:43, 688-725) -- so one pass over a kv head's
 // records serves 16 * NT columns: the records are read from HBM, dropped into the wave's LDS
 // window and turned into fp16 operands once per tile, and each operand feeds NT MFMAs.
 // One wavefront = one (sequence, query block, kv head); it streams tiles 0 .. last visible tile
@@ -39,10 +39,11 @@ struct PrefillTile {
   };
 
   // S^T = K . Q^T for NT column tiles, online softmax with a per-column visible-token limit.
+  // A column sees tokens [limit - wspan, limit): wspan is the sliding window, or 2^31 - 1 without one.
   template <bool MASK>
-  __device__ static void qk_softmax(const LaneOffsets& lo, const half8_t (&qb)[NT][KSTEPS], const float (&s_init)[NT],
-                                    const int (&limit)[NT], int t, int lane, const uint8_t* lds, State& st,
-                                    half8_t (&p_op)[NT]) {
+  __device__ static void qk_softmax(const AttnIO& io, const LaneOffsets& lo, const half8_t (&qb)[NT][KSTEPS],
+                                    const float (&s_init)[NT], const int (&limit)[NT], uint32_t wspan, int t, int lane,
+                                    const uint8_t* lds, State& st, half8_t (&p_op)[NT]) {
     const int g = lane >> 4;
     const float* sc_lds = reinterpret_cast<const float*>(lds + LDS_TILE);
     floatx4 s[NT][2];
@@ -69,6 +70,7 @@ struct PrefillTile {
     const floatx4 vs0 = *reinterpret_cast<const floatx4*>(sc_lds + 32 + 4 * g);
     const floatx4 vs1 = *reinterpret_cast<const floatx4*>(sc_lds + 48 + 4 * g);
     const int tok_base = t * kTile + 4 * g;
+    const bool capped = io.cap_c != 0.f;  // uniform
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
       float logit[8];
@@ -76,9 +78,18 @@ struct PrefillTile {
 #pragma unroll
       for (int mt = 0; mt < 2; ++mt) {
 #pragma unroll
+        for (int i = 0; i < 4; ++i) logit[mt * 4 + i] = s[nt][mt][i] * (mt ? ks1 : ks0)[i];
+      }
+      if (capped) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) logit[j] = soft_cap(logit[j], io.cap_c, io.cap_k);
+      }
+#pragma unroll
+      for (int mt = 0; mt < 2; ++mt) {
+#pragma unroll
         for (int i = 0; i < 4; ++i) {
-          float x = s[nt][mt][i] * (mt ? ks1 : ks0)[i];
-          if constexpr (MASK) x = ((tok_base + mt * 16 + i) < limit[nt]) ? x : -INFINITY;
+          float x = logit[mt * 4 + i];
+          if constexpr (MASK) x = ((uint32_t)(limit[nt] - 1 - (tok_base + mt * 16 + i)) < wspan) ? x : -INFINITY;
           logit[mt * 4 + i] = x;
           mloc = fmaxf(mloc, x);
         }
@@ -106,7 +117,7 @@ struct PrefillTile {
           const float p = __builtin_amdgcn_exp2f(logit[j] - m_ref);
           st.l[nt] += p;
           float x = p * (mt ? vs1 : vs0)[i];
-          if constexpr (MASK) x = ((tok_base + mt * 16 + i) < limit[nt]) ? x : 0.f;
+          if constexpr (MASK) x = ((uint32_t)(limit[nt] - 1 - (tok_base + mt * 16 + i)) < wspan) ? x : 0.f;
           pt[j] = x;
         }
       }
@@ -243,6 +254,12 @@ __global__ __launch_bounds__(WPW * 64) void paged_prefill_kernel(PrefillArgs a) 
   max_limit = wave_max_i32(max_limit);
   min_limit = -wave_max_i32(-min_limit);
   const int t_end = (max_limit + kTile - 1) / kTile;  // wave-uniform
+  // sliding window: a column sees [limit - window, limit); the wave starts at the tile that holds
+  // the earliest of these lower edges and masks tiles below the latest one
+  const uint32_t wspan = io.window > 0 ? (uint32_t)io.window : 0x7fffffffu;
+  const int min_first = io.window > 0 ? max(0, min(min_limit, max_limit) - io.window) : 0;
+  const int max_first = io.window > 0 ? max(0, max_limit - io.window) : 0;
+  const int t_start = min_first / kTile;
   if (t_end == 0) {  // nothing visible for any column (run longer than the sequence): defined zeros
     typename PT::State z;
 #pragma unroll
@@ -260,7 +277,7 @@ __global__ __launch_bounds__(WPW * 64) void paged_prefill_kernel(PrefillArgs a) 
   const LaneOffsets lo = DTile::lane_offsets(io.g, lane);
   const int32_t* bt_row = io.block_table + (int64_t)seq * io.bt_stride;
   typename DTile::Tile kv;
-  int t = 0;
+  int t = t_start;
   TileBlocks nb = DTile::fetch_blocks(io, bt_row, len, t);
   DTile::load_tile(io, DTile::window(io, nb, t, hkv), lo, kv);
   DTile::phase_fence();
@@ -290,14 +307,16 @@ __global__ __launch_bounds__(WPW * 64) void paged_prefill_kernel(PrefillArgs a) 
     DTile::load_tile(io, w, lo, kv);
     DTile::phase_fence();
     nb = DTile::fetch_blocks(io, bt_row, len, t + 2);
-    if ((t + 1) * kTile <= min_limit) PT::template qk_softmax<false>(lo, qb, s_init, limit, t, lane, lds, st, p_op);
-    else PT::template qk_softmax<true>(lo, qb, s_init, limit, t, lane, lds, st, p_op);
+    if ((t + 1) * kTile <= min_limit && t * kTile >= max_first)
+      PT::template qk_softmax<false>(io, lo, qb, s_init, limit, wspan, t, lane, lds, st, p_op);
+    else
+      PT::template qk_softmax<true>(io, lo, qb, s_init, limit, wspan, t, lane, lds, st, p_op);
     PT::pv(lo, p_op, lds, st);
     DTile::phase_fence();
     ++t;
   }
   DTile::stage(kv, lo, sc_mul, lane, lds);
-  PT::template qk_softmax<true>(lo, qb, s_init, limit, t, lane, lds, st, p_op);
+  PT::template qk_softmax<true>(io, lo, qb, s_init, limit, wspan, t, lane, lds, st, p_op);
   PT::pv(lo, p_op, lds, st);
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt) PT::emit(io, nt, row[nt], head[nt], valid[nt], lane, st);
@@ -436,9 +455,12 @@ struct Flash32 {
 
   // One tile for the wave's 32 columns.  S^T[32 tokens, 32 columns]: lane (c = column, g) holds
   // token (i/4)*8 + 4g + i%4 in register i.
-  template <bool MASK>
-  __device__ static __forceinline__ void compute(const uint8_t* buf, const half8_t (&qb)[KS], float s_init, int limit, int t,
-                                                 int lane, floatx16 (&o)[MT], float& m, float& l) {
+  // EXT: the column sees only tokens [limit - wspan, limit) (sliding window) and the logits may
+  // pass through the soft cap (cap_c != 0); without EXT wspan, cap_c and cap_k are not looked at.
+  template <bool MASK, bool EXT>
+  __device__ static __forceinline__ void compute(const uint8_t* buf, const half8_t (&qb)[KS], float s_init, int limit,
+                                                 uint32_t wspan, float cap_c, float cap_k, int t, int lane,
+                                                 floatx16 (&o)[MT], float& m, float& l) {
     const int c = lane & 31, g = lane >> 5;
     const float* sc = reinterpret_cast<const float*>(buf + K_BYTES + V_BYTES);
     floatx16 s;
@@ -457,13 +479,32 @@ struct Flash32 {
     const bool fresh = m == -INFINITY;          // the column has seen no visible token yet
     const float mref = fresh ? 0.f : m;
     float d = -INFINITY;
+    bool capped = false;
+    if constexpr (EXT) capped = cap_c != 0.f;  // uniform
+    if (capped) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const floatx4 ksc = *reinterpret_cast<const floatx4*>(sc + 8 * q + 4 * g);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) s[4 * q + r] = soft_cap(s[4 * q + r] * ksc[r], cap_c, cap_k) - mref;
+      }
+    } else {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const floatx4 ksc = *reinterpret_cast<const floatx4*>(sc + 8 * q + 4 * g);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) s[4 * q + r] = __builtin_fmaf(s[4 * q + r], ksc[r], -mref);
+      }
+    }
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
-      const floatx4 ksc = *reinterpret_cast<const floatx4*>(sc + 8 * q + 4 * g);
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        float y = __builtin_fmaf(s[4 * q + r], ksc[r], -mref);
-        if constexpr (MASK) y = ((tok_base + q * 8 + r) < limit) ? y : -INFINITY;
+        float y = s[4 * q + r];
+        if constexpr (MASK) {
+          if constexpr (EXT) y = ((uint32_t)(limit - 1 - (tok_base + q * 8 + r)) < wspan) ? y : -INFINITY;
+          else y = ((tok_base + q * 8 + r) < limit) ? y : -INFINITY;
+        }
         s[4 * q + r] = y;
         d = fmaxf(d, y);
       }
@@ -493,7 +534,10 @@ struct Flash32 {
           const float p = __builtin_amdgcn_exp2f(s[4 * q + r]);
           l += p;
           float x = p * vsc[r];
-          if constexpr (MASK) x = ((tok_base + q * 8 + r) < limit) ? x : 0.f;
+          if constexpr (MASK) {
+            if constexpr (EXT) x = ((uint32_t)(limit - 1 - (tok_base + q * 8 + r)) < wspan) ? x : 0.f;
+            else x = ((tok_base + q * 8 + r) < limit) ? x : 0.f;
+          }
           pt[4 * h + r] = x;
         }
       }
@@ -516,7 +560,8 @@ struct Flash32 {
   }
 };
 
-template <int D, int QDT, int ODT>
+// EXT adds the sliding window and the logits soft cap; the plain causal kernel carries neither.
+template <int D, int QDT, int ODT, bool EXT>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void paged_prefill_flash32_kernel(PrefillArgs a) {
   using FP = Flash32<D, QDT, ODT>;
   using DTile = typename FP::DTile;
@@ -550,6 +595,21 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   int wg_limit = a.causal ? ctx + min(q0 + a.q_tokens, q_len) : len;
   wg_limit = wg_limit < 0 ? 0 : (wg_limit > len ? len : wg_limit);
   const int t_end = (wg_limit + kTile - 1) / kTile;
+  // Sliding window: a column sees [limit - window, limit).  The workgroup starts at the (even) tile
+  // pair that holds the first query token's lower edge; a wave masks tiles below the latest lower
+  // edge among its columns and skips those that end before the earliest.
+  uint32_t wspan = 0x7fffffffu;
+  int t_first = 0, wave_min_first = 0, wave_max_first = 0;
+  if constexpr (EXT) {
+    if (io.window > 0) {
+      wspan = (uint32_t)io.window;
+      int wg_first = (a.causal ? ctx + q0 + 1 : len) - io.window;
+      wg_first = wg_first < 0 ? 0 : wg_first;
+      t_first = (wg_first / kTile) & ~1;
+      wave_min_first = max(0, wave_min_limit - io.window);
+      wave_max_first = max(0, wave_max_limit - io.window);
+    }
+  }
 
   floatx16 o[FP::MT];
 #pragma unroll
@@ -558,7 +618,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     for (int i = 0; i < 16; ++i) o[mt][i] = 0.f;
   float m = -INFINITY, l = 0.f;
 
-  if (t_end > 0) {
+  if (t_end > t_first) {
     const LaneOffsets lo = DTile::lane_offsets(io.g, lane);
     const int32_t* bt_row = io.block_table + (int64_t)seq * io.bt_stride;
     const int step = (64 / DTile::NCH) * (int)io.g.stride_slot;
@@ -584,20 +644,20 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       *reinterpret_cast<u32x4*>(raw + l_chunk + 16 * FP::RAW_PITCH) = r.c1;
       if (wave < 2 && lane < 16) *reinterpret_cast<u32x2*>(raw + l_tail) = r.tail;
     };
-    TileBlocks nb = DTile::fetch_blocks(io, bt_row, len, 0);
-    issue(nb, 0, A);
-    nb = DTile::fetch_blocks(io, bt_row, len, 1);
-    issue(nb, 1, B);
-    nb = DTile::fetch_blocks(io, bt_row, len, 2);
+    TileBlocks nb = DTile::fetch_blocks(io, bt_row, len, t_first);
+    issue(nb, t_first, A);
+    nb = DTile::fetch_blocks(io, bt_row, len, t_first + 1);
+    issue(nb, t_first + 1, B);
+    nb = DTile::fetch_blocks(io, bt_row, len, t_first + 2);
 
     half8_t qb[FP::KS];
     const float s_init =
         FP::load_q(io, row * io.q_stride_t + (int64_t)(valid ? head : hkv * io.group) * io.q_stride_h, valid, lane, qb);
     const float sc_mul = lane < 32 ? io.scale_log2 : kPScale;
 
-    drop(A, raws);
-    issue(nb, 2, A);
-    nb = DTile::fetch_blocks(io, bt_row, len, 3);
+    drop(A, raws);  // t_first is even: raw window 0
+    issue(nb, t_first + 2, A);
+    nb = DTile::fetch_blocks(io, bt_row, len, t_first + 3);
     lds_barrier();
     // Step t: expand raw tile t into fp16 buffer t&1, drop tile t+1 (held in `next`) into the other
     // raw window and refill `next` with tile t+3, ONE barrier, then compute tile t.
@@ -609,9 +669,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       lds_barrier();
       nb = DTile::fetch_blocks(io, bt_row, len, t + 4);
       if constexpr (decltype(masked)::value) {
-        if (t * kTile < wave_max_limit) FP::template compute<true>(buf, qb, s_init, limit, t, lane, o, m, l);
+        bool live = t * kTile < wave_max_limit;
+        if constexpr (EXT) live = live && (t + 1) * kTile > wave_min_first;
+        if (live) FP::template compute<true, EXT>(buf, qb, s_init, limit, wspan, io.cap_c, io.cap_k, t, lane, o, m, l);
       } else {
-        FP::template compute<false>(buf, qb, s_init, limit, t, lane, o, m, l);
+        FP::template compute<false, EXT>(buf, qb, s_init, limit, wspan, io.cap_c, io.cap_k, t, lane, o, m, l);
       }
     };
     // Tiles below every column's limit need no mask.  They and the masked tail are two separate
@@ -619,7 +681,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     // in), so that the accumulators keep their registers across the loop instead of being merged
     // at a branch inside it.
     const int t_plain = min(t_end, wave_min_limit / kTile) & ~1;
-    int t = 0;
+    int t = t_first;
+    if constexpr (EXT) {  // tiles that straddle a column's lower window edge
+      const int t_head = min(t_end, ((wave_max_first + kTile - 1) / kTile + 1) & ~1);
+      for (; t < t_head; t += 2) {
+        step_fn(std::true_type{}, t, B);
+        step_fn(std::true_type{}, t + 1, A);
+      }
+    }
     for (; t < t_plain; t += 2) {
       step_fn(std::false_type{}, t, B);
       step_fn(std::false_type{}, t + 1, A);
@@ -664,7 +733,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     io.lse[row * io.num_q_heads + head] = l > 0.f ? (m + __builtin_amdgcn_logf(l)) * kLn2 : -INFINITY;
 }
 
-template <int D, int QDT, int ODT>
+template <int D, int QDT, int ODT, bool EXT>
 static int launch_prefill_flash32(PrefillArgs& a, int max_query_len, hipStream_t s) {
   using FP = Flash32<D, QDT, ODT>;
   a.q_tokens = FP::COLS / a.io.group;
@@ -672,7 +741,7 @@ static int launch_prefill_flash32(PrefillArgs& a, int max_query_len, hipStream_t
   if (a.num_seqs > 65535 || a.io.g.num_kv_heads > 65535) return fail(KVQ_EINVAL, "paged_attn_int8: prefill grid out of range");
   static_assert(FP::LDS_BYTES <= 64 * 1024, "static LDS opt-in would be needed");
   dim3 grid(blocks, a.num_seqs, a.io.g.num_kv_heads);
-  hipLaunchKernelGGL((paged_prefill_flash32_kernel<D, QDT, ODT>), grid, dim3(256), FP::LDS_BYTES, s, a);
+  hipLaunchKernelGGL((paged_prefill_flash32_kernel<D, QDT, ODT, EXT>), grid, dim3(256), FP::LDS_BYTES, s, a);
   return check_hip(hipGetLastError(), "paged_prefill_flash32 launch");
 }
 
@@ -690,7 +759,10 @@ static int launch_prefill_nt(PrefillArgs& a, int max_query_len, hipStream_t s) {
   constexpr int WPW = 4;
   // long runs: the workgroup-shared fp16 tile (compute-bound shape)
   if constexpr (D <= 128) {
-    if (max_query_len * a.io.group >= 64) return launch_prefill_flash32<D, QDT, ODT>(a, max_query_len, s);
+    if (max_query_len * a.io.group >= 64) {
+      if (a.io.window > 0 || a.io.cap_c != 0.f) return launch_prefill_flash32<D, QDT, ODT, true>(a, max_query_len, s);
+      return launch_prefill_flash32<D, QDT, ODT, false>(a, max_query_len, s);
+    }
   }
   // two column tiles per wave where the accumulators fit the register file next to a tile in flight
   if (D <= 128 && a.io.group * 2 <= 32 && max_query_len * a.io.group > 16) {

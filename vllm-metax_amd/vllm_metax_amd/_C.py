@@ -13,7 +13,7 @@ _LIB_DIR = os.path.join(os.path.dirname(os.path.abspath(__file__)), "_lib")
 LIB_PATH = os.path.join(_LIB_DIR, "libkvq_hip.so")
 
 KVQ_F32, KVQ_BF16, KVQ_F16 = 0, 1, 2
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 
 class CacheGeom(ctypes.Structure):
@@ -51,7 +51,7 @@ SIGNATURES = {
     "kvq_reshape_and_cache_int8": (_i, [_vp, _vp, _i, _i64, _i64, _i64, _i64, _vp, _geom_p, _vp, _i64, _f, _vp]),
     "kvq_paged_attn_workspace_bytes": (_sz, [_i, _i, _i]),
     "kvq_paged_attn_int8": (_i, [_vp, _i, _i64, _i64, _vp, _i, _i64, _i64, _vp, _geom_p, _vp, _i64, _vp, _vp,
-                                 _i, _i, _i, _f, _i, _vp, _vp, _sz, _vp]),
+                                 _i, _i, _i, _f, _i, _i, _f, _vp, _vp, _sz, _vp]),
     "kvq_paged_attn_v2_int8": (_i, [_vp, _i, _vp, _vp, _vp, _vp, _i, _i64, _i64, _vp, _geom_p, _vp, _i64, _vp,
                                     _i, _i, _f, _i, _i, _vp]),
     "kvq_splitk_reduce": (_i, [_vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),

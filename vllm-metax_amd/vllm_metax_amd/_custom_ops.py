@@ -168,15 +168,26 @@ def unified_attention(
     int32 context lengths; ``cu_seqlens_q`` ``[B+1]`` int32; ``block_table`` ``[B, max_blocks]``
     int32.  Extra keyword arguments of the reference's call that only steer its Triton launch
     (``seq_threshold_3D``, ``softmax_segm_*``, ``use_td`` ...) are accepted and ignored; features
-    this path does not build raise ``NotImplementedError``."""
+    this path does not build raise ``NotImplementedError``.  ``window_size=(W - 1, 0)`` restricts a
+    query to its last W keys; ``softcap > 0`` maps logits through ``softcap * tanh(x / softcap)``."""
     if kv_quant_mode != KVQuantMode.INT8_PER_TOKEN_HEAD:
         raise NotImplementedError(f"kv_quant_mode {kv_quant_mode!r}: only INT8_PER_TOKEN_HEAD is built")
     if alibi_slopes is not None or sinks is not None or output_scale is not None or mm_prefix_range is not None:
         raise NotImplementedError("alibi, sinks, fused output quantisation and mm-prefix ranges are not built")
-    if softcap not in (0, 0.0, None):
-        raise NotImplementedError("logits soft cap is not built")
-    if tuple(window_size) != (-1, -1):
-        raise NotImplementedError("sliding window is not built")
+    softcap = float(softcap or 0.0)
+    if softcap < 0:
+        raise RuntimeError("softcap must be >= 0")
+    # (left, right) as the reference passes it (triton_attn.py:507-512): (-1, -1) = none,
+    # (W - 1, 0) = causal window of W keys ending at the query; two-sided windows are encoder-only
+    left, right = (int(x) for x in window_size)
+    if (left, right) == (-1, -1):
+        window = 0
+    elif left >= 0 and right == 0:
+        if not causal:
+            raise NotImplementedError("a sliding window needs causal attention")
+        window = left + 1
+    else:
+        raise NotImplementedError(f"window_size {(left, right)}: only (-1, -1) and (W - 1, 0) are built")
     if q_descale is not None:
         raise NotImplementedError("quantised query input is not built")
     if unused.get("rswa_window") is not None or unused.get("chunk_lookback", -1) not in (-1, None):
@@ -215,7 +226,7 @@ def unified_attention(
             _ptr(q), _dtype_code(q, "q"), q.stride(0), q.stride(1),
             ctypes.c_void_p(geom.base_ptr), ctypes.byref(g), _ptr(block_table), block_table.stride(0),
             _ptr(seqused_k), _ptr(cu_seqlens_q), num_seqs, num_q_heads, int(max_seqlen_q),
-            float(softmax_scale), 1 if causal else 0, _ptr(lse), _ptr(workspace),
+            float(softmax_scale), 1 if causal else 0, window, softcap, _ptr(lse), _ptr(workspace),
             workspace.numel() * workspace.element_size(), _stream(dev))
     _C.check(rc, "unified_attention")
 

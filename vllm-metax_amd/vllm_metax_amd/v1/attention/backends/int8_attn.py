@@ -176,7 +176,7 @@ class Int8AttentionBackend(_BackendBase):
 
     @classmethod
     def supports_sliding_window(cls) -> bool:
-        return False
+        return True
 
     @classmethod
     def supports_sink(cls) -> bool:
@@ -248,8 +248,7 @@ class Int8AttentionImpl(_ImplBase):
                  attn_type: str = AttentionType.DECODER, kv_sharing_target_layer_name: str | None = None,
                  sinks: torch.Tensor | None = None, use_alibi_sqrt: bool = False, chunk_lookback: int = -1) -> None:
         unsupported = {
-            "alibi_slopes": alibi_slopes is not None, "sliding_window": sliding_window is not None,
-            "logits_soft_cap": bool(logits_soft_cap), "sinks": sinks is not None,
+            "alibi_slopes": alibi_slopes is not None, "sinks": sinks is not None,
             "kv_sharing_target_layer_name": kv_sharing_target_layer_name is not None,
             "chunk_lookback": chunk_lookback not in (-1, None),
         }
@@ -270,8 +269,11 @@ class Int8AttentionImpl(_ImplBase):
         self.num_queries_per_kv = num_heads // num_kv_heads
         self.kv_cache_dtype = kv_cache_dtype
         self.attn_type = attn_type
-        self.sliding_window = (-1, -1)
-        self.logits_soft_cap = 0
+        # decoder attention only: (W - 1, 0), as at triton_attn.py:507-512; soft cap 0 = none (:536-539)
+        if sliding_window is not None and sliding_window < 1:
+            raise ValueError(f"sliding_window must be >= 1, got {sliding_window}")
+        self.sliding_window = (-1, -1) if sliding_window is None else (sliding_window - 1, 0)
+        self.logits_soft_cap = float(logits_soft_cap or 0)
         self._kv_quant_mode = get_kv_quant_mode(kv_cache_dtype)
         self._is_per_token_head_quant = True
         # per-cache views and byte geometry, built at first use (one cache tensor per layer)
