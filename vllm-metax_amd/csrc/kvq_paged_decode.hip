@@ -27,14 +27,29 @@ __device__ __forceinline__ int wave_incl_scan(int v, int lane) {
   return v;
 }
 
-// Tiles a sequence contributes to the decode tile line (0 for prefill sequences): the tiles that
-// hold a token of the row's window, [window_first / 32, ceil(len / 32)).
+// Starting on a sequence (query row, first tile with nothing in flight, storing the state of the
+// one before) costs a workgroup about as long as one tile takes; the work line that is cut into
+// equal shares therefore charges every sequence this many units before its tiles.  Measured on
+// MI355X at batch 64, 1k..8k tokens: workgroups whose share crossed a sequence boundary ran 2.9 us
+// (one tile time) longer than the others and were the last to finish; with the charge they get
+// one tile less.
+constexpr int kSetupUnits = 1;
+
+// Tiles of a decode sequence: those that hold a token of the row's window,
+// [window_first / 32, ceil(len / 32)).  0 for prefill sequences and empty ones.
 __device__ __forceinline__ int decode_tiles(const int32_t* seq_lens, const int32_t* cu, int s, int num_seqs,
                                             int window) {
   if (s >= num_seqs) return 0;
   if (cu != nullptr && (cu[s + 1] - cu[s]) != 1) return 0;
   const int len = seq_lens[s];
   return len > 0 ? (len + kTile - 1) / kTile - window_first(len, window) / kTile : 0;
+}
+
+// Units a sequence takes on the work line: its setup charge, then one unit per tile.
+__device__ __forceinline__ int decode_units(const int32_t* seq_lens, const int32_t* cu, int s, int num_seqs,
+                                            int window) {
+  const int n = decode_tiles(seq_lens, cu, s, num_seqs, window);
+  return n > 0 ? n + kSetupUnits : 0;
 }
 
 __device__ __forceinline__ int64_t wg_tile_begin(int w, int64_t total, int num_wg) {
@@ -52,10 +67,10 @@ __global__ __launch_bounds__(WPW * 64) void paged_decode_streamk_kernel(StreamKA
   const int w = blockIdx.x;
   const int B = a.num_seqs;
 
-  // total tiles (each wave redoes this tiny scan; no LDS, no barrier)
+  // total units of the work line (each wave redoes this tiny scan; no LDS, no barrier)
   int64_t total = 0;
   for (int base = 0; base < B; base += kWave) {
-    int n = decode_tiles(a.seq_lens, a.cu_seqlens_q, base + lane, B, a.io.window);
+    int n = decode_units(a.seq_lens, a.cu_seqlens_q, base + lane, B, a.io.window);
     n = wave_incl_scan(n, lane);
     total += __builtin_amdgcn_readlane(n, 63);
   }
@@ -63,13 +78,13 @@ __global__ __launch_bounds__(WPW * 64) void paged_decode_streamk_kernel(StreamKA
   const int64_t hi = wg_tile_begin(w + 1, total, a.num_wg);
   if (lo >= hi) return;
 
-  // locate the sequence holding tile `lo`
+  // locate the sequence holding unit `lo`
   int seq = 0;
-  int64_t seq_start = 0;  // global index of the sequence's tile 0
+  int64_t seq_start = 0;  // global index of the sequence's first unit
   {
     int64_t cum = 0;
     for (int base = 0; base < B; base += kWave) {
-      const int n = decode_tiles(a.seq_lens, a.cu_seqlens_q, base + lane, B, a.io.window);
+      const int n = decode_units(a.seq_lens, a.cu_seqlens_q, base + lane, B, a.io.window);
       const int incl = wave_incl_scan(n, lane);
       const int64_t first = cum + incl - n, last = cum + incl;
       const uint64_t hit = __builtin_amdgcn_ballot_w64(n > 0 && first <= lo && lo < last);
@@ -86,27 +101,34 @@ __global__ __launch_bounds__(WPW * 64) void paged_decode_streamk_kernel(StreamKA
 
   int64_t pos = lo;
   while (pos < hi && seq < B) {
-    const int ntiles = __builtin_amdgcn_readfirstlane(decode_tiles(a.seq_lens, a.cu_seqlens_q, seq, B, a.io.window));
-    if (ntiles == 0) {
+    const int units = __builtin_amdgcn_readfirstlane(decode_units(a.seq_lens, a.cu_seqlens_q, seq, B, a.io.window));
+    if (units == 0) {
       ++seq;
       continue;
     }
+    const int ntiles = units - kSetupUnits;
     const int len = __builtin_amdgcn_readfirstlane(a.seq_lens[seq]);
     const int64_t row = a.cu_seqlens_q ? (int64_t)a.cu_seqlens_q[seq] : (int64_t)seq;
     const int first = window_first(len, a.io.window);  // tokens before it are outside the window
     const int t0 = first / kTile;                      // the sequence's tile line starts at this tile
-    const int t_begin = __builtin_amdgcn_readfirstlane(t0 + (int)(pos - seq_start));
+    // units [pos, min(hi, end of the sequence)) of the line; the first kSetupUnits of a sequence
+    // stand for no tile
+    const int u_begin = (int)(pos - seq_start);
     const int64_t rem = hi - seq_start;
-    const int t_end = __builtin_amdgcn_readfirstlane(t0 + (rem < ntiles ? (int)rem : ntiles));
-    typename DTile::State st;
-    DTile::template run<CAP>(a.io, seq, row, len, first, t_begin, t_end, hkv, lane, lds[wave], st);
-    if (t_begin == t0 && t_end == t0 + ntiles) {
-      DTile::emit_final(a.io, row, hkv, lane, st);
-    } else {
-      DTile::emit_partial(a.io, a.part_o, a.part_ml, (int64_t)w + seq, hkv, lane, st);
+    const int u_end = rem < units ? (int)rem : units;
+    const int t_begin = __builtin_amdgcn_readfirstlane(t0 + (u_begin > kSetupUnits ? u_begin - kSetupUnits : 0));
+    const int t_end = __builtin_amdgcn_readfirstlane(t0 + u_end - kSetupUnits);
+    if (t_begin < t_end) {  // else: this share ends inside the setup charge and holds no tile
+      typename DTile::State st;
+      DTile::template run<CAP>(a.io, seq, row, len, first, t_begin, t_end, hkv, lane, lds[wave], st);
+      if (t_begin == t0 && t_end == t0 + ntiles) {
+        DTile::emit_final(a.io, row, hkv, lane, st);
+      } else {
+        DTile::emit_partial(a.io, a.part_o, a.part_ml, (int64_t)w + seq, hkv, lane, st);
+      }
     }
-    pos = seq_start + t_end;
-    seq_start += ntiles;
+    pos = seq_start + u_end;
+    seq_start += units;
     ++seq;
   }
 }
@@ -125,7 +147,7 @@ __global__ __launch_bounds__(256) void paged_decode_streamk_reduce_kernel(Stream
   const int q0 = a.cu_seqlens_q ? a.cu_seqlens_q[seq] : seq;
   const int q1 = a.cu_seqlens_q ? a.cu_seqlens_q[seq + 1] : seq + 1;
   const int len = a.seq_lens[seq];
-  int n_first = decode_tiles(a.seq_lens, a.cu_seqlens_q, lane, B, a.io.window);  // first 64 sequences of the scan
+  int n_first = decode_units(a.seq_lens, a.cu_seqlens_q, lane, B, a.io.window);  // first 64 sequences of the scan
   if (q1 - q0 != 1) return;
   const int64_t row = q0;
   const int ntiles = len > 0 ? (len + kTile - 1) / kTile - window_first(len, a.io.window) / kTile : 0;
@@ -137,15 +159,16 @@ __global__ __launch_bounds__(256) void paged_decode_streamk_reduce_kernel(Stream
   }
   int64_t total = 0, start = 0;
   for (int base = 0; base < B; base += kWave) {
-    int n = base == 0 ? n_first : decode_tiles(a.seq_lens, a.cu_seqlens_q, base + lane, B, a.io.window);
+    int n = base == 0 ? n_first : decode_units(a.seq_lens, a.cu_seqlens_q, base + lane, B, a.io.window);
     const int incl = wave_incl_scan(n, lane);
     if (seq >= base && seq < base + kWave) start = total + __builtin_amdgcn_readlane(incl - n, seq - base);
     total += __builtin_amdgcn_readlane(incl, 63);
   }
   const int P = a.num_wg;
-  // workgroup holding tile x: the largest w with floor(w*T/P) <= x
-  const int w_first = (int)(((start + 1) * P - 1) / total);
-  const int w_last = (int)(((start + ntiles) * P - 1) / total);
+  // workgroup holding unit x: the largest w with floor(w*T/P) <= x; the sequence's tiles are units
+  // start + kSetupUnits .. start + kSetupUnits + ntiles - 1
+  const int w_first = (int)(((start + kSetupUnits + 1) * P - 1) / total);
+  const int w_last = (int)(((start + kSetupUnits + ntiles) * P - 1) / total);
   if (w_first == w_last) return;  // written directly by the main kernel
 
   // pass 1: every lane takes one workgroup's (m, l); the wave agrees on the max and the weights

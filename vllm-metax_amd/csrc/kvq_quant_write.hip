@@ -20,29 +20,47 @@ __global__ __launch_bounds__(256) void quant_write_kernel(
   if (row >= num_rows) return;
   const int is_v = (int)(row & 1);
   const int64_t th = row >> 1;
-  const int h = (int)(th % g.num_kv_heads);
-  const int64_t t = th / g.num_kv_heads;
-  const int64_t slot = slot_mapping[t];
-  if (slot < 0) return;  // padding token
-  const int64_t blk = slot / g.block_size;
-  const int64_t off = slot - blk * g.block_size;
+  // 32-bit index arithmetic whenever the row count allows it (a 64-bit divide is a long routine)
+  int h;
+  int64_t t;
+  if (num_rows <= 0xffffffffLL) {
+    const uint32_t t32 = (uint32_t)th / (uint32_t)g.num_kv_heads;
+    h = (int)((uint32_t)th - t32 * (uint32_t)g.num_kv_heads);
+    t = t32;
+  } else {
+    h = (int)(th % g.num_kv_heads);
+    t = th / g.num_kv_heads;
+  }
   const int D = g.head_size;
-
   const void* src = is_v ? value : key;
   const int64_t src_base = is_v ? (t * value_stride_t + h * value_stride_h)
                                 : (t * key_stride_t + h * key_stride_h);
+  // The row's loads do not depend on the slot: they go out together with the slot's load, so the
+  // kernel pays one memory round trip before it can write instead of two.
+  const int64_t slot = slot_mapping[t];
+  float x[VEC > 0 ? VEC : 1];
+  if constexpr (VEC > 0) {
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) x[i] = load_act<DT>(src, src_base + lane * VEC + i);
+  }
+  if (slot < 0) return;  // padding token
+  int64_t blk, off;
+  if ((uint64_t)slot <= 0xffffffffull) {
+    const uint32_t b32 = (uint32_t)slot / (uint32_t)g.block_size;
+    blk = b32;
+    off = (uint32_t)slot - b32 * (uint32_t)g.block_size;
+  } else {
+    blk = slot / g.block_size;
+    off = slot - blk * g.block_size;
+  }
   uint8_t* rec = cache + blk * g.stride_block + off * g.stride_slot + (int64_t)h * g.stride_head;
   int8_t* codes = reinterpret_cast<int8_t*>(rec + (is_v ? g.v_off : g.k_off));
   float* scale_ptr = reinterpret_cast<float*>(rec + (is_v ? g.vs_off : g.ks_off));
 
   if constexpr (VEC > 0) {
-    float x[VEC];
     float amax = 0.f;
 #pragma unroll
-    for (int i = 0; i < VEC; ++i) {
-      x[i] = load_act<DT>(src, src_base + lane * VEC + i);
-      amax = fmaxf(amax, fabsf(x[i]));
-    }
+    for (int i = 0; i < VEC; ++i) amax = fmaxf(amax, fabsf(x[i]));
     amax = fmaxf(wave_max(amax), eps);  // eps may be 0 for fp16 sources (1e-10 underflows)
     const float scale = amax / 127.0f;
     int8_t c[VEC];
