@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define KVQ_ABI_VERSION 2
+#define KVQ_ABI_VERSION 3
 
 #define KVQ_OK 0
 #define KVQ_EINVAL (-22)
@@ -168,6 +168,39 @@ KVQ_API int kvq_splitk_reduce(void* out, int out_dtype, float* lse, const float*
                       const float* max_logits, const float* tmp_out, const int32_t* seq_lens,
                       int num_seqs, int num_q_heads, int head_size, int partition_size,
                       int max_num_partitions, kvq_stream_t stream);
+
+/* Directions of kvq_swap_blocks. */
+#define KVQ_DEVICE_TO_DEVICE 0
+#define KVQ_DEVICE_TO_HOST 1
+#define KVQ_HOST_TO_DEVICE 2
+
+/*
+ * Move whole cache blocks: dst block block_mapping[i][1] = src block
+ * block_mapping[i][0], block_bytes each.  Stands in for swap_blocks(src, dst,
+ * block_size_in_bytes, block_mapping), csrc/libtorch_stable/cache_kernels.cu:33-77
+ * (schema torch_bindings.cpp:816-818).  block_mapping is a HOST array of int64
+ * pairs with element strides map_stride0 / map_stride1, as the reference requires
+ * (cache_kernels.cu:51-55).  A block of the int8 layouts (kvq_cache_geom /
+ * kvq_mla_geom: block_bytes = stride_block) holds codes and scales together, so
+ * the move is self-contained.  Asynchronous on `stream`; host memory should be
+ * pinned.  Pairs must not overlap when src and dst are the same allocation.
+ */
+KVQ_API int kvq_swap_blocks(const void* src, void* dst, int64_t block_bytes,
+                    const int64_t* block_mapping, int64_t num_pairs, int64_t map_stride0,
+                    int64_t map_stride1, int direction, kvq_stream_t stream);
+
+/*
+ * n independent copies (src_ptrs[i] -> dst_ptrs[i], sizes[i] bytes), submitted
+ * together.  Stands in for swap_blocks_batch(src_ptrs, dst_ptrs, sizes, ...),
+ * csrc/libtorch_stable/cache_kernels.cu:79-178 (schema torch_bindings.cpp:821-823).
+ * The three arrays are HOST arrays of int64.  all_on_device != 0 promises that
+ * every pointer is device memory of the current device: the copies then run as
+ * one kernel launch per 64 entries; otherwise each entry is one asynchronous
+ * copy whose direction is taken from the pointers.
+ */
+KVQ_API int kvq_swap_blocks_batch(const int64_t* src_ptrs, const int64_t* dst_ptrs,
+                          const int64_t* sizes, int64_t n, int all_on_device,
+                          kvq_stream_t stream);
 
 /*
  * LSE merge of two partial attention states.  Stands in for merge_attn_states,

@@ -303,6 +303,78 @@ def splitk_reduce(out: torch.Tensor, exp_sums: torch.Tensor, max_logits: torch.T
     _C.check(rc, "splitk_reduce")
 
 
+def swap_blocks(src: torch.Tensor, dst: torch.Tensor, block_size_in_bytes: int, block_mapping: torch.Tensor) -> None:
+    """``swap_blocks(Tensor src, Tensor! dst, int block_size_in_bytes, Tensor block_mapping)``
+    (csrc/libtorch_stable/torch_bindings.cpp:816-818, cache_kernels.cu:33-77): dst block
+    ``block_mapping[i, 1]`` = src block ``block_mapping[i, 0]``.  ``block_mapping`` is a CPU int64
+    ``[n, 2]`` tensor (the reference refuses a GPU one, cache_kernels.cu:51-55); src / dst are cache
+    tensors of the int8 layouts (GQA or MLA) on the GPU or in (pinned) host memory, at least one of
+    them on the GPU, both on the same GPU if both are.  Asynchronous on the current stream."""
+    if block_mapping.is_cuda:
+        raise RuntimeError("block_mapping must be on CPU")
+    if block_mapping.dtype != torch.int64 or block_mapping.dim() != 2 or block_mapping.shape[1] != 2:
+        raise RuntimeError("block_mapping must be an int64 [n, 2] tensor")
+    if src.is_cuda and dst.is_cuda:
+        if src.device != dst.device:
+            raise RuntimeError("src and dst must be on the same GPU")
+        direction, dev = 0, src.device
+    elif src.is_cuda and not dst.is_cuda:
+        direction, dev = 1, src.device
+    elif dst.is_cuda and not src.is_cuda:
+        direction, dev = 2, dst.device
+    else:
+        raise RuntimeError("Invalid device combination")
+    n = block_mapping.shape[0]
+    if n == 0:
+        return
+    block_size_in_bytes = int(block_size_in_bytes)
+    hi = int(block_mapping.max()) + 1
+    lo = int(block_mapping.min())
+    for t, col, name in ((src, 0, "src"), (dst, 1, "dst")):
+        top = int(block_mapping[:, col].max()) + 1
+        if top * block_size_in_bytes > t.untyped_storage().nbytes() - t.storage_offset() * t.element_size():
+            raise RuntimeError(f"block_mapping names block {top - 1} beyond the end of {name}")
+    if lo < 0 or hi <= 0:
+        raise RuntimeError("block numbers must not be negative")
+    lib = _C.load()
+    with torch.cuda.device(dev):
+        rc = lib.kvq_swap_blocks(_ptr(src), _ptr(dst), block_size_in_bytes, _ptr(block_mapping), n,
+                                 block_mapping.stride(0), block_mapping.stride(1), direction, _stream(dev))
+    _C.check(rc, "swap_blocks")
+
+
+def swap_blocks_batch(src_ptrs: torch.Tensor, dst_ptrs: torch.Tensor, sizes: torch.Tensor,
+                      is_src_access_order_any: bool = False, all_on_device: bool = False) -> None:
+    """``swap_blocks_batch(Tensor src_ptrs, Tensor dst_ptrs, Tensor sizes, bool
+    is_src_access_order_any=False)`` (torch_bindings.cpp:821-823, cache_kernels.cu:79-178): ``n``
+    independent copies given as CPU int64 tensors of raw addresses and byte counts, submitted
+    together on the current stream.  ``is_src_access_order_any`` steers a driver hint of the
+    reference's batched memcpy and changes no result; it is accepted and ignored.
+    ``all_on_device=True`` promises that every address is memory of the current GPU: the batch then
+    runs as one kernel launch per 64 entries instead of one copy call per entry."""
+    for t, name in ((src_ptrs, "src_ptrs"), (dst_ptrs, "dst_ptrs"), (sizes, "sizes")):
+        if t.is_cuda:
+            raise RuntimeError(f"{name} must be on CPU")
+        if t.dtype != torch.int64:
+            raise RuntimeError(f"{name} must be int64")
+        if not t.is_contiguous() or t.dim() != 1:
+            raise RuntimeError(f"{name} must be a contiguous 1-D tensor")
+    n = src_ptrs.shape[0]
+    if dst_ptrs.shape[0] != n:
+        raise RuntimeError("dst_ptrs length must match src_ptrs")
+    if sizes.shape[0] != n:
+        raise RuntimeError("sizes length must match src_ptrs")
+    if n == 0:
+        return
+    if not torch.cuda.is_available():
+        raise RuntimeError("swap_blocks_batch needs a GPU (there is no CPU path)")
+    dev = torch.device("cuda", torch.cuda.current_device())
+    lib = _C.load()
+    rc = lib.kvq_swap_blocks_batch(_ptr(src_ptrs), _ptr(dst_ptrs), _ptr(sizes), n, 1 if all_on_device else 0,
+                                   _stream(dev))
+    _C.check(rc, "swap_blocks_batch")
+
+
 def merge_attn_states(output: torch.Tensor, prefix_output: torch.Tensor, prefix_lse: torch.Tensor,
                       suffix_output: torch.Tensor, suffix_lse: torch.Tensor,
                       output_lse: torch.Tensor | None = None, prefill_tokens_with_context: int | None = None) -> None:
