@@ -1,9 +1,10 @@
 // Paged decode attention over the int8 cache: work decomposition and reduce (gfx950).
 //
 // Balanced split-K ("stream-K" over tokens): the 32-token tiles of all decode
-// sequences form one global tile line; the launch has exactly as many workgroups as
-// the device keeps resident and workgroup w takes tiles [w*T/P, (w+1)*T/P), whatever
-// sequence boundaries fall inside.  A workgroup is one wave per KV head, so a block's
+// sequences form one global work line (one unit per tile, plus a small charge per
+// sequence start); the launch has exactly as many workgroups as the device keeps
+// resident and workgroup w takes units [w*T/P, (w+1)*T/P), whatever sequence
+// boundaries fall inside.  A workgroup is one wave per KV head, so a block's
 // bytes are read by one CU at the same time and each byte leaves HBM once.  A run of
 // tiles that covers a whole sequence writes the output row directly; otherwise it
 // stores an fp32 partial state (o, m, l) in slot w + seq (unique along the staircase of
@@ -63,7 +64,7 @@ __global__ __launch_bounds__(WPW * 64) void paged_decode_streamk_kernel(StreamKA
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int hkv = __builtin_amdgcn_readfirstlane(blockIdx.y * WPW + wave);
-  if (hkv >= a.io.g.num_kv_heads) return;  // no workgroup barriers below
+  if (hkv >= a.io.g.num_kv_heads) return;  // a finished wave no longer counts at the tile loop's barriers
   const int w = blockIdx.x;
   const int B = a.num_seqs;
 
