@@ -41,6 +41,26 @@ def _require_cuda(*tensors: torch.Tensor) -> torch.device:
     return dev
 
 
+class _on_device:
+    """``torch.cuda.device(dev)`` that does nothing when ``dev`` is already current (the usual case on
+    a per-step path; the context manager costs several microseconds of host time)."""
+
+    __slots__ = ("_ctx",)
+
+    def __init__(self, dev: torch.device):
+        idx = dev.index if dev.index is not None else torch.cuda.current_device()
+        self._ctx = None if idx == torch.cuda.current_device() else torch.cuda.device(idx)
+
+    def __enter__(self):
+        if self._ctx is not None:
+            self._ctx.__enter__()
+
+    def __exit__(self, *exc):
+        if self._ctx is not None:
+            return self._ctx.__exit__(*exc)
+        return False
+
+
 def _stream(dev: torch.device) -> ctypes.c_void_p:
     return ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
 
@@ -98,7 +118,7 @@ def reshape_and_cache_flash_per_token_head_quant(
         raise RuntimeError("slot_mapping is longer than key")
     lib = _C.load()
     g = geom.as_struct()
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         rc = lib.kvq_reshape_and_cache_int8(
             _ptr(key), _ptr(value), _dtype_code(key, "key"), key.stride(0), key.stride(1), value.stride(0),
             value.stride(1), ctypes.c_void_p(geom.base_ptr), ctypes.byref(g), _ptr(slot_mapping), num_tokens,
@@ -114,8 +134,17 @@ triton_reshape_and_cache_flash_per_token_head_quant = reshape_and_cache_flash_pe
 # attention
 # ---------------------------------------------------------------------------------------------
 
+_ws_bytes_cache: dict = {}
+
+
 def paged_attn_workspace_bytes(max_num_seqs: int, num_q_heads: int, head_size: int) -> int:
-    return int(_C.load().kvq_paged_attn_workspace_bytes(max_num_seqs, num_q_heads, head_size))
+    """Host query (depends on the current device's CU count); answers are remembered per device."""
+    key = (torch.cuda.current_device() if torch.cuda.is_available() else -1, max_num_seqs, num_q_heads, head_size)
+    got = _ws_bytes_cache.get(key)
+    if got is None:
+        got = int(_C.load().kvq_paged_attn_workspace_bytes(max_num_seqs, num_q_heads, head_size))
+        _ws_bytes_cache[key] = got
+    return got
 
 
 _ws_cache: dict = {}
@@ -220,7 +249,7 @@ def unified_attention(
                             or tuple(lse.shape) != (q.shape[0], num_q_heads)):
         raise RuntimeError("lse must be a contiguous float32 [num_tokens, num_q_heads] tensor")
     g = geom.as_struct()
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         rc = lib.kvq_paged_attn_int8(
             _ptr(out), _dtype_code(out, "out"), out.stride(0), out.stride(1),
             _ptr(q), _dtype_code(q, "q"), q.stride(0), q.stride(1),
@@ -277,7 +306,7 @@ def paged_attention_v2(
     if seq_lens.dtype != torch.int32 or block_tables.dtype != torch.int32 or block_tables.stride(1) != 1:
         raise RuntimeError("seq_lens and block_tables must be int32 (rows contiguous)")
     g = geom.as_struct()
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         rc = _C.load().kvq_paged_attn_v2_int8(
             _ptr(out), _dtype_code(out, "out"), _ptr(exp_sums), _ptr(max_logits), _ptr(tmp_out), _ptr(query),
             _dtype_code(query, "query"), query.stride(0), query.stride(1), ctypes.c_void_p(geom.base_ptr),
@@ -296,7 +325,7 @@ def splitk_reduce(out: torch.Tensor, exp_sums: torch.Tensor, max_logits: torch.T
             raise RuntimeError(f"{name} must be contiguous float32")
     if tuple(out.shape) != (B, Hq, D) or not out.is_contiguous() or seq_lens.dtype != torch.int32:
         raise RuntimeError("out must be contiguous [B, Hq, D] and seq_lens int32")
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         rc = _C.load().kvq_splitk_reduce(_ptr(out), _dtype_code(out, "out"), _ptr(lse), _ptr(exp_sums),
                                          _ptr(max_logits), _ptr(tmp_out), _ptr(seq_lens), B, Hq, D,
                                          int(partition_size), P, _stream(dev))
@@ -337,7 +366,7 @@ def swap_blocks(src: torch.Tensor, dst: torch.Tensor, block_size_in_bytes: int, 
     if lo < 0 or hi <= 0:
         raise RuntimeError("block numbers must not be negative")
     lib = _C.load()
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         rc = lib.kvq_swap_blocks(_ptr(src), _ptr(dst), block_size_in_bytes, _ptr(block_mapping), n,
                                  block_mapping.stride(0), block_mapping.stride(1), direction, _stream(dev))
     _C.check(rc, "swap_blocks")
@@ -392,7 +421,7 @@ def merge_attn_states(output: torch.Tensor, prefix_output: torch.Tensor, prefix_
     if prefix_lse.dtype != torch.float32 or suffix_lse.dtype != torch.float32 or tuple(prefix_lse.shape) != (H, T):
         raise RuntimeError("lse tensors must be float32 [num_heads, num_tokens]")
     n_prefix = T if prefill_tokens_with_context is None else int(prefill_tokens_with_context)
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         rc = _C.load().kvq_merge_attn_states(_ptr(output), _ptr(output_lse), _ptr(prefix_output), _ptr(prefix_lse),
                                              _ptr(suffix_output), _ptr(suffix_lse), _dtype_code(output, "output"),
                                              T, H, D, n_prefix, _stream(dev))
@@ -424,7 +453,7 @@ def concat_and_cache_mla(kv_c: torch.Tensor, k_pe: torch.Tensor, kv_cache: torch
     if T > kv_c.shape[0] or T > k_pe.shape[0]:
         raise RuntimeError("slot_mapping is longer than kv_c / k_pe")
     g = geom.as_struct()
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         rc = _C.load().kvq_concat_and_cache_mla_int8(_ptr(kv_c), _ptr(k_pe), _dtype_code(kv_c, "kv_c"),
                                                      kv_c.stride(0), k_pe.stride(0), ctypes.c_void_p(geom.base_ptr),
                                                      ctypes.byref(g), _ptr(slot_mapping), T,
@@ -457,7 +486,7 @@ def gather_and_maybe_dequant_cache(src_cache: torch.Tensor, dst: torch.Tensor, b
     if token_to_seq.numel() < num_tokens:
         raise RuntimeError("token_to_seq is shorter than num_tokens")
     g = geom.as_struct()
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         rc = _C.load().kvq_gather_and_dequant_mla_int8(
             _ptr(dst), _dtype_code(dst, "dst"), dst.stride(0), ctypes.c_void_p(geom.base_ptr), ctypes.byref(g),
             _ptr(block_table), block_table.stride(0), _ptr(cu_seq_lens), _ptr(token_to_seq), _ptr(seq_starts),
@@ -490,7 +519,7 @@ def mla_decode_int8(q: torch.Tensor, kv_cache: torch.Tensor, o: torch.Tensor, ls
     if workspace is None:
         workspace = _default_workspace(dev, need)
     g = geom.as_struct()
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         rc = _C.load().kvq_mla_decode_int8(_ptr(o), _dtype_code(o, "o"), _ptr(lse), _ptr(q), _dtype_code(q, "q"),
                                            q.stride(0), q.stride(1), ctypes.c_void_p(geom.base_ptr), ctypes.byref(g),
                                            _ptr(block_table), block_table.stride(0), _ptr(seq_lens), B, H,

@@ -142,9 +142,14 @@ class CacheGeometry:
     base_ptr: int
 
     def as_struct(self) -> "_C.CacheGeom":
-        return _C.CacheGeom(self.k_off, self.v_off, self.ks_off, self.vs_off, self.stride_block,
-                            self.stride_slot, self.stride_head, self.num_kv_heads, self.head_size,
-                            self.block_size, 0)
+        """The ctypes struct, built once per geometry object (it is read-only for the library)."""
+        st = self.__dict__.get("_struct")
+        if st is None:
+            st = _C.CacheGeom(self.k_off, self.v_off, self.ks_off, self.vs_off, self.stride_block,
+                              self.stride_slot, self.stride_head, self.num_kv_heads, self.head_size,
+                              self.block_size, 0)
+            object.__setattr__(self, "_struct", st)
+        return st
 
     @property
     def record_bytes(self) -> int:
@@ -240,8 +245,13 @@ class MlaGeometry:
     base_ptr: int
 
     def as_struct(self) -> "_C.MlaGeom":
-        return _C.MlaGeom(self.stride_block, self.stride_row, self.scale_off, self.kv_lora_rank,
-                          self.rope_dim, self.block_size, 0)
+        """The ctypes struct, built once per geometry object (it is read-only for the library)."""
+        st = self.__dict__.get("_struct")
+        if st is None:
+            st = _C.MlaGeom(self.stride_block, self.stride_row, self.scale_off, self.kv_lora_rank,
+                            self.rope_dim, self.block_size, 0)
+            object.__setattr__(self, "_struct", st)
+        return st
 
 
 def mla_geometry(cache: torch.Tensor, kv_lora_rank: int) -> MlaGeometry:
