@@ -1,20 +1,23 @@
-// MLA decode over the int8 latent cache (gfx950, wave64, MFMA 16x16x32 f16).
+// MLA decode over the int8 latent cache (gfx950, wave64; QK on the int8 MFMA 16x16x64, PV on the
+// f16 MFMA 16x16x32).
 //
 // All query heads of a sequence share ONE latent stream (576 int8 codes + one fp32 scale per
 // token), so this is a dense contraction: S^T[token, head] = C . Q^T over 576 dims and
 // O^T[dim, head] = C[:, :512]^T . P~^T, both on the MFMA with the heads as the N dimension.
 //
 // Work item = (sequence, token split); workgroup = 8 waves, wave w owns heads 16w .. 16w+15 of a
-// 128-head group and keeps their absorbed Q (18 k-steps) and their 512 x 16 output tile in
-// registers (a 32-head tile per wave would halve the dequantisation work per flop but needs
-// more than the 512 registers a lane can have).  The workgroup loads each 32-token tile once, as flat 16-byte chunks (every
-// quarter-wave reads 256 contiguous bytes), through registers into a double-buffered LDS window
-// (one barrier per tile); every wave then reads the int8 rows back in MFMA operand order and
-// turns codes into exact fp16 numbers code + 1152 with one byte permute per two codes -- the
-// constant is taken out again through the accumulator start value (QK) and a row of ones (PV).
+// 128-head group and keeps their 512 x 16 output tile in registers; their absorbed Q sits in LDS
+// (and 4 of its 18 operands in registers) as two int8 terms that a small kernel prepares once per
+// launch, so the QK product reads the cached code bytes as they are.  (A 32-head tile per wave
+// would halve the work per flop on the PV side but needs more than the 512 registers a lane can
+// have next to the rest.)  The workgroup loads each 32-token tile once, as flat 16-byte chunks
+// (every quarter-wave reads 256 contiguous bytes), through registers into a double-buffered LDS
+// window (one barrier per tile).  For PV every wave reads the int8 rows back transposed in
+// registers and turns codes into exact fp16 numbers code + 1152 with one byte permute per two
+// codes -- the constant is taken out again through a row of ones.
 // The token splits of a sequence are merged by the reduce kernel with the log-sum-exp algebra
 // (same two-stage shape as the reference's decode_attention_fwd); nothing is allocated here,
-// partials live in the caller's workspace.
+// partials and the int8 Q live in the caller's workspace.
 #include <atomic>
 
 #include "kvq_attn_core.cuh"
@@ -31,8 +34,11 @@ constexpr int kMlaVB = kMlaR / 16;                        // 32 V bytes per toke
 constexpr int kChunksPerRow = kMlaW / 16;                 // 36
 constexpr int kChunksPerHalf = 16 * kChunksPerRow;        // 576
 constexpr int kMlaThreads = 512;
-constexpr int kMlaQRegSteps = 4;                          // k-steps of Q kept in registers; the rest in LDS
-constexpr int kMlaQLdsBytes = (kMlaKSteps - kMlaQRegSteps) * kMlaThreads * 16;  // 114688
+constexpr int kMlaKSteps8 = kMlaW / 64;                   // 9 int8 k-steps of 64 dims
+constexpr int kMlaQOps = 2 * kMlaKSteps8;                 // B operands of Q: two int8 terms per k-step
+constexpr int kMlaQRegOps = 4;                            // operands of Q kept in registers; the rest in LDS
+constexpr int kMlaQLdsBytes = (kMlaQOps - kMlaQRegOps) * kMlaThreads * 16;  // 114688
+typedef int32_t i32x4 __attribute__((ext_vector_type(4)));
 constexpr int kMlaLdsBytes = 2 * kMlaBufBytes + kMlaQLdsBytes;                  // 153088 of 163840
 
 struct MlaArgs {
@@ -50,6 +56,10 @@ struct MlaArgs {
   // log2 domain, -inf for an empty split.
   uint16_t* part_o;
   float* part_lse;
+  // Q as the int8 MFMA wants it (written by mla_quant_q_kernel, read by every split of a sequence):
+  // q_ops [B, ceil(H/16)][18 operands][64 lanes][16 bytes], q_scale [B, 16 * ceil(H/16)] = s1 per head.
+  uint8_t* q_ops;
+  float* q_scale;
   int head_groups;  // ceil(H / 16)
   int num_heads;
   int num_splits;
@@ -63,11 +73,109 @@ __device__ __forceinline__ int mla_split_len(int len, int num_splits) {
   return ((per + kTile - 1) / kTile) * kTile;
 }
 
+// Q for the int8 MFMA.  The cache codes ARE int8, so the QK product can run on
+// v_mfma_i32_16x16x64_i8 straight from the cached bytes -- no conversion of K at all -- once Q is
+// int8 too: q = s1 * a + s2 * b with a = rint(q / s1), s1 = max|q| / 127 per head, and
+// b = rint((q - s1 a) / s2), s2 = s1 / 254.  The residual after two terms is at most
+// s2 / 2 = max|q| / 64516, finer than the fp16 rounding of q it replaces, and the integer dot
+// products are exact.  One wave per (sequence, 16 heads), once per launch (every token split of the
+// sequence reads the result): lane (c = head, g) produces, for k-step kk, dims 64 kk + 16 g + j
+// (j < 16) as 16 bytes, operand 2 kk = term a, operand 2 kk + 1 = term b.
 template <int QDT>
+__global__ __launch_bounds__(64) void mla_quant_q_kernel(MlaArgs a) {
+  const int lane = threadIdx.x;
+  const int c = lane & 15, g = lane >> 4;
+  const int seq = blockIdx.x, hgroup = blockIdx.y;
+  const int head = hgroup * 16 + c;
+  const bool head_ok = head < a.num_heads;
+  const int64_t qblock = (int64_t)seq * a.head_groups + hgroup;
+  u32x4* qdst = reinterpret_cast<u32x4*>(a.q_ops + qblock * (kMlaQOps * kWave * 16)) + lane;
+  float s1, s2;
+  {
+    const int64_t qbase = (int64_t)seq * a.q_stride_b + (int64_t)(head_ok ? head : 0) * a.q_stride_h + 16 * g;
+    u32x4 raw[QDT == KVQ_F32 ? 1 : kMlaKSteps8][2];
+    if constexpr (QDT != KVQ_F32) {  // all 18 loads in flight before the first conversion waits
+#pragma unroll
+      for (int kk = 0; kk < kMlaKSteps8; ++kk)
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+          raw[kk][h] = *reinterpret_cast<const u32x4_a4*>(reinterpret_cast<const uint16_t*>(a.q) + qbase + 64 * kk + 8 * h);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    // the 16 values of k-step kk as floats (fp32 queries are read again in the second pass)
+    auto values = [&](int kk, float (&f)[16]) __attribute__((always_inline)) {
+      if constexpr (QDT == KVQ_F32) {
+        const float* p = reinterpret_cast<const float*>(a.q) + qbase + 64 * kk;
+#pragma unroll
+        for (int i = 0; i < 16; i += 4) {
+          const floatx4 v = *reinterpret_cast<const floatx4_a4*>(p + i);
+          f[i] = v.x; f[i + 1] = v.y; f[i + 2] = v.z; f[i + 3] = v.w;
+        }
+      } else {
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          const u32x4 v = raw[kk][h];
+#pragma unroll
+          for (int w = 0; w < 4; ++w) {
+            const uint32_t e = v[w];
+            if constexpr (QDT == KVQ_BF16) {
+              f[8 * h + 2 * w] = as_f32(e << 16);
+              f[8 * h + 2 * w + 1] = as_f32(e & 0xffff0000u);
+            } else {
+              const half2_t hh = __builtin_bit_cast(half2_t, e);
+              f[8 * h + 2 * w] = (float)hh.x;
+              f[8 * h + 2 * w + 1] = (float)hh.y;
+            }
+          }
+        }
+      }
+    };
+    float amax = 0.f;
+#pragma unroll
+    for (int kk = 0; kk < kMlaKSteps8; ++kk) {
+      float f[16];
+      values(kk, f);
+#pragma unroll
+      for (int i = 0; i < 16; ++i) amax = fmaxf(amax, fabsf(f[i]));
+    }
+    amax = fmaxf(amax, __shfl_xor(amax, 16, kWave));
+    amax = fmaxf(amax, __shfl_xor(amax, 32, kWave));
+    amax = head_ok ? fminf(amax, 3.0e38f) : 0.f;      // heads past the end contribute zero columns
+    s1 = amax > 0.f ? amax / 127.0f : 1.0f;
+    s2 = s1 / 254.0f;
+    const float inv1 = 1.0f / s1, inv2 = 254.0f * inv1;
+#pragma unroll
+    for (int kk = 0; kk < kMlaKSteps8; ++kk) {
+      float f[16];
+      values(kk, f);
+      i32x4 ta, tb;
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        uint32_t pa = 0, pb = 0;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const float q = head_ok ? f[4 * w + j] : 0.f;
+          const float fa = fminf(fmaxf(rintf(q * inv1), -127.f), 127.f);
+          const float r = __builtin_fmaf(-fa, s1, q);
+          const float fb = fminf(fmaxf(rintf(r * inv2), -127.f), 127.f);
+          pa |= ((uint32_t)(int)fa & 0xffu) << (8 * j);
+          pb |= ((uint32_t)(int)fb & 0xffu) << (8 * j);
+        }
+        ta[w] = (int32_t)pa;
+        tb[w] = (int32_t)pb;
+      }
+      qdst[(2 * kk) * kWave] = __builtin_bit_cast(u32x4, ta);
+      qdst[(2 * kk + 1) * kWave] = __builtin_bit_cast(u32x4, tb);
+    }
+  }
+  if (g == 0) a.q_scale[qblock * 16 + c] = s1;
+  (void)s2;
+}
+
 __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
   extern __shared__ __align__(16) uint8_t lds_raw[];
   uint8_t(*lds)[kMlaBufBytes] = reinterpret_cast<uint8_t(*)[kMlaBufBytes]>(lds_raw);
-  // B operands of Q for k-steps >= kMlaQRegSteps: slot [kk][thread], written and read by the same lane
+  // B operands of Q from number kMlaQRegOps on: slot [operand][thread], written and read by the same lane
   u32x4* qlds = reinterpret_cast<u32x4*>(lds_raw + 2 * kMlaBufBytes) + threadIdx.x;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -153,57 +261,31 @@ __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
   issue_loads(fetch_blocks(t_begin));
   Blocks nb = fetch_blocks(t_begin + 1);
 
-  // ---- absorbed Q of this wave's 16 heads as the MFMA B operand: lane (c = head, g) holds, for
-  //      k-step kk, dims 32 kk + 8 g + j
-  half8_t qb[kMlaQRegSteps];
-  float qsum = 0.f;
-  {
-    const uint32_t okmask = head_ok ? 0xffffffffu : 0u;   // heads past the end contribute zero columns
-    const int64_t qbase = (int64_t)seq * a.q_stride_b + (int64_t)(head_ok ? hbase + c : 0) * a.q_stride_h + 8 * g;
-    u32x4 raw[QDT == KVQ_F32 ? 1 : kMlaKSteps];
-    if constexpr (QDT != KVQ_F32) {  // all 18 loads in flight before the first conversion waits
+  // ---- absorbed Q of this wave's 16 heads: the int8 B operands mla_quant_q_kernel prepared (operand
+  //      2 kk = first term, 2 kk + 1 = second term of k-step kk; lane (c = head, g) holds dims
+  //      64 kk + 16 g + j)
+  i32x4 qreg[kMlaQRegOps];
+  float s1 = 1.f, s2 = 0.f;
+  if (wave_ok) {
+    const int64_t qblock = (int64_t)seq * a.head_groups + hgroup;
+    const u32x4* qsrc = reinterpret_cast<const u32x4*>(a.q_ops + qblock * (kMlaQOps * kWave * 16)) + lane;
+    u32x4 raw[kMlaQOps];
 #pragma unroll
-      for (int kk = 0; kk < kMlaKSteps; ++kk)
-        raw[kk] = *reinterpret_cast<const u32x4_a4*>(reinterpret_cast<const uint16_t*>(a.q) + qbase + 32 * kk);
-      __builtin_amdgcn_sched_barrier(0);
+    for (int op = 0; op < kMlaQOps; ++op) raw[op] = qsrc[op * kWave];
+    s1 = a.q_scale[qblock * 16 + c];
+    s2 = s1 / 254.0f;
+#pragma unroll
+    for (int op = 0; op < kMlaQOps; ++op) {
+      if (op < kMlaQRegOps) qreg[op] = __builtin_bit_cast(i32x4, raw[op]);
+      else qlds[(op - kMlaQRegOps) * kMlaThreads] = raw[op];
     }
+  } else {
 #pragma unroll
-    for (int kk = 0; kk < kMlaKSteps; ++kk) {
-      float f[8];
-      if constexpr (QDT == KVQ_F32) {
-        const float* p = reinterpret_cast<const float*>(a.q) + qbase + 32 * kk;
-        const floatx4 v0 = *reinterpret_cast<const floatx4_a4*>(p), v1 = *reinterpret_cast<const floatx4_a4*>(p + 4);
-        f[0] = v0.x; f[1] = v0.y; f[2] = v0.z; f[3] = v0.w; f[4] = v1.x; f[5] = v1.y; f[6] = v1.z; f[7] = v1.w;
-      } else {
-        const u32x4 v = raw[kk];
-#pragma unroll
-        for (int w = 0; w < 4; ++w) {
-          const uint32_t e = v[w];
-          if constexpr (QDT == KVQ_BF16) {
-            f[2 * w] = as_f32(e << 16);
-            f[2 * w + 1] = as_f32(e & 0xffff0000u);
-          } else {
-            const half2_t hh = __builtin_bit_cast(half2_t, e);
-            f[2 * w] = (float)hh.x;
-            f[2 * w + 1] = (float)hh.y;
-          }
-        }
-      }
-      u32x4 hb;
-      hb.x = pack_half2(clamp_half_range(f[0]), clamp_half_range(f[1])) & okmask;
-      hb.y = pack_half2(clamp_half_range(f[2]), clamp_half_range(f[3])) & okmask;
-      hb.z = pack_half2(clamp_half_range(f[4]), clamp_half_range(f[5])) & okmask;
-      hb.w = pack_half2(clamp_half_range(f[6]), clamp_half_range(f[7])) & okmask;
-      const half8_t h8 = __builtin_bit_cast(half8_t, hb);
-#pragma unroll
-      for (int j = 0; j < 8; ++j) qsum += (float)h8[j];
-      if (kk < kMlaQRegSteps) qb[kk] = h8;
-      else qlds[(kk - kMlaQRegSteps) * kMlaThreads] = hb;
+    for (int op = 0; op < kMlaQOps; ++op) {
+      if (op < kMlaQRegOps) qreg[op] = (i32x4){0, 0, 0, 0};
+      else qlds[(op - kMlaQRegOps) * kMlaThreads] = (u32x4){0u, 0u, 0u, 0u};
     }
-    qsum += __shfl_xor(qsum, 16, kWave);
-    qsum += __shfl_xor(qsum, 32, kWave);
   }
-  const float s_init = -kCodeBias * qsum;
 
   floatx4 o[kMlaDT];
 #pragma unroll
@@ -220,19 +302,28 @@ __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
     const uint8_t* tile = lds[buf];
     const float* sck = reinterpret_cast<const float*>(tile + kMlaTileBytes);
 
-    // ---- S^T[32 tokens, 16 heads]: A = code rows, lane (r = token, g): bytes 32 kk + 8 g ..
-    floatx4 s[2];
-    s[0] = (floatx4){s_init, s_init, s_init, s_init};
-    s[1] = s[0];
+    // ---- S^T[32 tokens, 16 heads] on the int8 MFMA: A = the cached code bytes as they are, lane
+    //      (r = token, g): dims 64 kk + 16 g ..; one accumulator per term of Q
+    i32x4 acc[2][2];
 #pragma unroll
-    for (int kk = 0; kk < kMlaKSteps; ++kk) {
-      half8_t qop;
-      if (kk < kMlaQRegSteps) qop = qb[kk];
-      else qop = __builtin_bit_cast(half8_t, qlds[(kk - kMlaQRegSteps) * kMlaThreads]);
+    for (int term = 0; term < 2; ++term)
+#pragma unroll
+      for (int mt = 0; mt < 2; ++mt) acc[term][mt] = (i32x4){0, 0, 0, 0};
+#pragma unroll
+    for (int kk = 0; kk < kMlaKSteps8; ++kk) {
+      i32x4 qa, qb8;
+      if (2 * kk < kMlaQRegOps) {
+        qa = qreg[2 * kk];
+        qb8 = qreg[2 * kk + 1];
+      } else {
+        qa = __builtin_bit_cast(i32x4, qlds[(2 * kk - kMlaQRegOps) * kMlaThreads]);
+        qb8 = __builtin_bit_cast(i32x4, qlds[(2 * kk + 1 - kMlaQRegOps) * kMlaThreads]);
+      }
 #pragma unroll
       for (int mt = 0; mt < 2; ++mt) {
-        const u32x2 w = *reinterpret_cast<const u32x2*>(tile + (mt * 16 + c) * kMlaPitch + 32 * kk + 8 * g);
-        s[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(dequant8(w.x, w.y), qop, s[mt], 0, 0, 0);
+        const i32x4 ka = *reinterpret_cast<const i32x4*>(tile + (mt * 16 + c) * kMlaPitch + 64 * kk + 16 * g);
+        acc[0][mt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(ka, qa, acc[0][mt], 0, 0, 0);
+        acc[1][mt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(ka, qb8, acc[1][mt], 0, 0, 0);
       }
     }
 
@@ -245,7 +336,7 @@ __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int tok = t * kTile + 16 * mt + 4 * g + i;
-        float x = s[mt][i] * ks[i];
+        float x = __builtin_fmaf((float)acc[1][mt][i], s2, (float)acc[0][mt][i] * s1) * ks[i];
         x = tok < tok_end ? x : -INFINITY;
         logit[4 * mt + i] = x;
         mloc = fmaxf(mloc, x);
@@ -413,7 +504,7 @@ static int mla_num_splits(int max_seq_hint, int num_seqs, int num_heads) {
 }
 
 // The decode kernel needs more dynamic LDS than the 64 KB a kernel gets by default.  The opt-in is a
-// per-device, per-kernel attribute; it is set for all three instantiations the first time either entry
+// per-device, per-kernel attribute; it is set the first time either entry
 // point runs on a device -- the workspace query is the place a caller reaches before any stream
 // capture, so a captured decode call finds it done.
 static int mla_prepare_device() {
@@ -422,13 +513,10 @@ static int mla_prepare_device() {
   if (int e = check_hip(hipGetDevice(&dev), "hipGetDevice")) return e;
   const uint64_t bit = dev >= 0 && dev < 64 ? (1ull << dev) : 0;
   if (bit != 0 && (done_mask.load(std::memory_order_acquire) & bit)) return KVQ_OK;
-  const void* fns[3] = {reinterpret_cast<const void*>(&mla_decode_kernel<KVQ_F32>),
-                        reinterpret_cast<const void*>(&mla_decode_kernel<KVQ_BF16>),
-                        reinterpret_cast<const void*>(&mla_decode_kernel<KVQ_F16>)};
-  for (const void* f : fns)
-    if (int e = check_hip(hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, kMlaLdsBytes),
-                          "hipFuncSetAttribute(mla_decode_kernel)"))
-      return e;
+  if (int e = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(&mla_decode_kernel),
+                                            hipFuncAttributeMaxDynamicSharedMemorySize, kMlaLdsBytes),
+                        "hipFuncSetAttribute(mla_decode_kernel)"))
+    return e;
   done_mask.fetch_or(bit, std::memory_order_release);
   return KVQ_OK;
 }
@@ -445,7 +533,9 @@ size_t kvq_mla_decode_workspace_bytes(int max_num_seqs, int num_heads, int kv_lo
   size_t items = 2 * (size_t)kvq::num_cus() / groups;
   if (items < (size_t)max_num_seqs) items = (size_t)max_num_seqs;
   const size_t heads_padded = ((size_t)num_heads + 15) / 16 * 16;
-  return items * heads_padded * ((size_t)kv_lora_rank * sizeof(uint16_t) + sizeof(float));
+  // split states (fp16 outputs + fp32 lse) and, per sequence, Q as two int8 terms + one scale per head
+  return items * heads_padded * ((size_t)kv_lora_rank * sizeof(uint16_t) + sizeof(float)) +
+         (size_t)max_num_seqs * heads_padded * ((size_t)kvq::kMlaQOps * 64 + sizeof(float));
 }
 
 int kvq_mla_decode_int8(void* out, int out_dtype, float* lse, const void* q, int q_dtype, int64_t q_stride_b,
@@ -471,7 +561,9 @@ int kvq_mla_decode_int8(void* out, int out_dtype, float* lse, const void* q, int
   const int splits = mla_num_splits(0, num_seqs, num_heads);
   const int head_groups = (num_heads + 15) / 16;
   const size_t states = (size_t)num_seqs * head_groups * 16 * splits;
-  const size_t need = states * ((size_t)kMlaR * sizeof(uint16_t) + sizeof(float));
+  const size_t qheads = (size_t)num_seqs * head_groups * 16;
+  const size_t need = states * ((size_t)kMlaR * sizeof(uint16_t) + sizeof(float)) +
+                      qheads * ((size_t)kMlaQOps * 64 + sizeof(float));
   KVQ_REQUIRE(workspace != nullptr && workspace_bytes >= need && ((uintptr_t)workspace % 16) == 0,
               "%s: workspace of %zu bytes (16-byte aligned) required, got %zu", op, need, workspace_bytes);
   MlaArgs a{};
@@ -484,7 +576,9 @@ int kvq_mla_decode_int8(void* out, int out_dtype, float* lse, const void* q, int
   a.bt_stride = bt_stride;
   a.seq_lens = seq_lens;
   a.part_lse = static_cast<float*>(workspace);  // fp32 first, so both arrays keep their alignment
-  a.part_o = reinterpret_cast<uint16_t*>(a.part_lse + states);
+  a.q_scale = a.part_lse + states;
+  a.part_o = reinterpret_cast<uint16_t*>(a.q_scale + qheads);
+  a.q_ops = reinterpret_cast<uint8_t*>(a.part_o + states * kMlaR);   // 16-byte aligned: every part is a multiple of 64 bytes
   a.head_groups = head_groups;
   a.num_heads = num_heads;
   a.num_splits = splits;
@@ -493,14 +587,17 @@ int kvq_mla_decode_int8(void* out, int out_dtype, float* lse, const void* q, int
   hipStream_t s = as_stream(stream);
   dim3 grid(splits, num_seqs, (num_heads + 127) / 128);
   if (int e = mla_prepare_device()) return e;
-#define KVQ_MLAD(T) hipLaunchKernelGGL((mla_decode_kernel<T>), grid, dim3(kMlaThreads), kMlaLdsBytes, s, a)
+  dim3 qgrid(num_seqs, head_groups);
+#define KVQ_MLAQ(T) hipLaunchKernelGGL((mla_quant_q_kernel<T>), qgrid, dim3(64), 0, s, a)
   switch (q_dtype) {
-    case KVQ_F32: KVQ_MLAD(KVQ_F32); break;
-    case KVQ_BF16: KVQ_MLAD(KVQ_BF16); break;
-    case KVQ_F16: KVQ_MLAD(KVQ_F16); break;
+    case KVQ_F32: KVQ_MLAQ(KVQ_F32); break;
+    case KVQ_BF16: KVQ_MLAQ(KVQ_BF16); break;
+    case KVQ_F16: KVQ_MLAQ(KVQ_F16); break;
     default: return fail(KVQ_EINVAL, "%s: unknown q_dtype %d", op, q_dtype);
   }
-#undef KVQ_MLAD
+#undef KVQ_MLAQ
+  if (int e = check_hip(hipGetLastError(), "mla_decode_int8 query launch")) return e;
+  hipLaunchKernelGGL(mla_decode_kernel, grid, dim3(kMlaThreads), kMlaLdsBytes, s, a);
   int rc = check_hip(hipGetLastError(), "mla_decode_int8 launch");
   if (rc) return rc;
   dim3 rgrid(num_seqs, head_groups);
