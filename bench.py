@@ -30,7 +30,7 @@ import torch  # noqa: E402
 HBM_PEAK_GBPS = 8000.0
 # HBM bytes per decode attention launch, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by a plain
 # read / copy kernel of known size (factors 2.000 and 1.000); summaries under profiles/.
-MEASURED_TRAFFIC = {"llama3_8b_decode_b64_ctx1k-8k": 727.1e6, "mla_decode_b32_h128_ctx4096": 190.0e6}
+MEASURED_TRAFFIC = {"llama3_8b_decode_b64_ctx1k-8k": 727.1e6, "mla_decode_b32_h128_ctx4096": 199.6e6}
 METRIC = "int8-KV paged decode: achieved HBM GB/s (% peak), µs/layer @B=64 ctx=8k"
 
 
@@ -248,7 +248,7 @@ def mla_main(args, cfg, dev, ops):
         "roofline": {"bound": "mfma", "achieved": round(flops / attn_s / 1e12, 1), "peak": MFMA_F16_PEAK_TFLOPS,
                      "unit": "TFLOP/s", "frac": round(flops / attn_s / 1e12 / MFMA_F16_PEAK_TFLOPS, 4),
                      "traffic": MEASURED_TRAFFIC.get(args.workload),
-                     "kernel": "MLA decode launch = mla_decode_kernel + mla_reduce_kernel",
+                     "kernel": "MLA decode launch = mla_quant_q_kernel + mla_decode_kernel + mla_reduce_kernel",
                      "algorithmic_flops_per_launch": flops, "algorithmic_bytes_per_launch": nbytes,
                      "hbm_frac_of_peak": round(nbytes / attn_s / 1e9 / HBM_PEAK_GBPS, 4)},
     }

@@ -248,6 +248,13 @@ KVQ_API int kvq_gather_and_dequant_mla_int8(void* dst, int dst_dtype, int64_t ds
                                     const int32_t* token_to_seq, const int32_t* seq_starts,
                                     int64_t num_tokens, kvq_stream_t stream);
 
+/*
+ * Workspace for kvq_mla_decode_int8 (host query, depends on the device): the fp16
+ * split states and their lse values (counterpart of the reference's attn_logits
+ * buffer, vllm_metax/v1/attention/backends/mla/triton_mla.py:261-269) plus the
+ * query as two int8 terms per element, which the launch prepares once for all
+ * splits.  An upper bound for any batch of at most max_num_seqs sequences.
+ */
 KVQ_API size_t kvq_mla_decode_workspace_bytes(int max_num_seqs, int num_heads, int kv_lora_rank);
 
 /*

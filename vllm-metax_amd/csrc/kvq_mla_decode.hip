@@ -78,98 +78,96 @@ __device__ __forceinline__ int mla_split_len(int len, int num_splits) {
 // int8 too: q = s1 * a + s2 * b with a = rint(q / s1), s1 = max|q| / 127 per head, and
 // b = rint((q - s1 a) / s2), s2 = s1 / 254.  The residual after two terms is at most
 // s2 / 2 = max|q| / 64516, finer than the fp16 rounding of q it replaces, and the integer dot
-// products are exact.  One wave per (sequence, 16 heads), once per launch (every token split of the
+// products are exact.  One workgroup per (sequence, 16 heads), once per launch (every token split of the
 // sequence reads the result): lane (c = head, g) produces, for k-step kk, dims 64 kk + 16 g + j
 // (j < 16) as 16 bytes, operand 2 kk = term a, operand 2 kk + 1 = term b.
 template <int QDT>
-__global__ __launch_bounds__(64) void mla_quant_q_kernel(MlaArgs a) {
-  const int lane = threadIdx.x;
+__global__ __launch_bounds__(256) void mla_quant_q_kernel(MlaArgs a) {
+  // 4 waves share the 9 k-steps of a (sequence, 16 heads) block: wave v takes k-steps v, v + 4, v + 8
+  constexpr int kMine = 3;
+  __shared__ float part_max[4][16];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int c = lane & 15, g = lane >> 4;
   const int seq = blockIdx.x, hgroup = blockIdx.y;
   const int head = hgroup * 16 + c;
   const bool head_ok = head < a.num_heads;
   const int64_t qblock = (int64_t)seq * a.head_groups + hgroup;
   u32x4* qdst = reinterpret_cast<u32x4*>(a.q_ops + qblock * (kMlaQOps * kWave * 16)) + lane;
-  float s1, s2;
-  {
-    const int64_t qbase = (int64_t)seq * a.q_stride_b + (int64_t)(head_ok ? head : 0) * a.q_stride_h + 16 * g;
-    u32x4 raw[QDT == KVQ_F32 ? 1 : kMlaKSteps8][2];
-    if constexpr (QDT != KVQ_F32) {  // all 18 loads in flight before the first conversion waits
+  const int64_t qbase = (int64_t)seq * a.q_stride_b + (int64_t)(head_ok ? head : 0) * a.q_stride_h + 16 * g;
+  // the wave's values as floats: f[n][i] = dim 64 kk + 16 g + i of k-step kk = wave + 4 n (a k-step
+  // past the last rereads the last one and is not written)
+  float f[kMine][16];
 #pragma unroll
-      for (int kk = 0; kk < kMlaKSteps8; ++kk)
+  for (int n = 0; n < kMine; ++n) {
+    const int kk = min(wave + 4 * n, kMlaKSteps8 - 1);
+    if constexpr (QDT == KVQ_F32) {
+      const float* p = reinterpret_cast<const float*>(a.q) + qbase + 64 * kk;
 #pragma unroll
-        for (int h = 0; h < 2; ++h)
-          raw[kk][h] = *reinterpret_cast<const u32x4_a4*>(reinterpret_cast<const uint16_t*>(a.q) + qbase + 64 * kk + 8 * h);
-      __builtin_amdgcn_sched_barrier(0);
-    }
-    // the 16 values of k-step kk as floats (fp32 queries are read again in the second pass)
-    auto values = [&](int kk, float (&f)[16]) __attribute__((always_inline)) {
-      if constexpr (QDT == KVQ_F32) {
-        const float* p = reinterpret_cast<const float*>(a.q) + qbase + 64 * kk;
+      for (int i = 0; i < 16; i += 4) {
+        const floatx4 v = *reinterpret_cast<const floatx4_a4*>(p + i);
+        f[n][i] = v.x; f[n][i + 1] = v.y; f[n][i + 2] = v.z; f[n][i + 3] = v.w;
+      }
+    } else {
 #pragma unroll
-        for (int i = 0; i < 16; i += 4) {
-          const floatx4 v = *reinterpret_cast<const floatx4_a4*>(p + i);
-          f[i] = v.x; f[i + 1] = v.y; f[i + 2] = v.z; f[i + 3] = v.w;
-        }
-      } else {
+      for (int h = 0; h < 2; ++h) {
+        const u32x4 v = *reinterpret_cast<const u32x4_a4*>(reinterpret_cast<const uint16_t*>(a.q) + qbase + 64 * kk + 8 * h);
 #pragma unroll
-        for (int h = 0; h < 2; ++h) {
-          const u32x4 v = raw[kk][h];
-#pragma unroll
-          for (int w = 0; w < 4; ++w) {
-            const uint32_t e = v[w];
-            if constexpr (QDT == KVQ_BF16) {
-              f[8 * h + 2 * w] = as_f32(e << 16);
-              f[8 * h + 2 * w + 1] = as_f32(e & 0xffff0000u);
-            } else {
-              const half2_t hh = __builtin_bit_cast(half2_t, e);
-              f[8 * h + 2 * w] = (float)hh.x;
-              f[8 * h + 2 * w + 1] = (float)hh.y;
-            }
+        for (int w = 0; w < 4; ++w) {
+          const uint32_t e = v[w];
+          if constexpr (QDT == KVQ_BF16) {
+            f[n][8 * h + 2 * w] = as_f32(e << 16);
+            f[n][8 * h + 2 * w + 1] = as_f32(e & 0xffff0000u);
+          } else {
+            const half2_t hh = __builtin_bit_cast(half2_t, e);
+            f[n][8 * h + 2 * w] = (float)hh.x;
+            f[n][8 * h + 2 * w + 1] = (float)hh.y;
           }
         }
       }
-    };
-    float amax = 0.f;
-#pragma unroll
-    for (int kk = 0; kk < kMlaKSteps8; ++kk) {
-      float f[16];
-      values(kk, f);
-#pragma unroll
-      for (int i = 0; i < 16; ++i) amax = fmaxf(amax, fabsf(f[i]));
-    }
-    amax = fmaxf(amax, __shfl_xor(amax, 16, kWave));
-    amax = fmaxf(amax, __shfl_xor(amax, 32, kWave));
-    amax = head_ok ? fminf(amax, 3.0e38f) : 0.f;      // heads past the end contribute zero columns
-    s1 = amax > 0.f ? amax / 127.0f : 1.0f;
-    s2 = s1 / 254.0f;
-    const float inv1 = 1.0f / s1, inv2 = 254.0f * inv1;
-#pragma unroll
-    for (int kk = 0; kk < kMlaKSteps8; ++kk) {
-      float f[16];
-      values(kk, f);
-      i32x4 ta, tb;
-#pragma unroll
-      for (int w = 0; w < 4; ++w) {
-        uint32_t pa = 0, pb = 0;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const float q = head_ok ? f[4 * w + j] : 0.f;
-          const float fa = fminf(fmaxf(rintf(q * inv1), -127.f), 127.f);
-          const float r = __builtin_fmaf(-fa, s1, q);
-          const float fb = fminf(fmaxf(rintf(r * inv2), -127.f), 127.f);
-          pa |= ((uint32_t)(int)fa & 0xffu) << (8 * j);
-          pb |= ((uint32_t)(int)fb & 0xffu) << (8 * j);
-        }
-        ta[w] = (int32_t)pa;
-        tb[w] = (int32_t)pb;
-      }
-      qdst[(2 * kk) * kWave] = __builtin_bit_cast(u32x4, ta);
-      qdst[(2 * kk + 1) * kWave] = __builtin_bit_cast(u32x4, tb);
     }
   }
-  if (g == 0) a.q_scale[qblock * 16 + c] = s1;
-  (void)s2;
+  float amax = 0.f;
+#pragma unroll
+  for (int n = 0; n < kMine; ++n)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) amax = fmaxf(amax, fabsf(f[n][i]));
+  amax = fmaxf(amax, __shfl_xor(amax, 16, kWave));
+  amax = fmaxf(amax, __shfl_xor(amax, 32, kWave));
+  if (g == 0) part_max[wave][c] = amax;
+  __syncthreads();
+  amax = fmaxf(fmaxf(part_max[0][c], part_max[1][c]), fmaxf(part_max[2][c], part_max[3][c]));
+  amax = head_ok ? fminf(amax, 3.0e38f) : 0.f;      // heads past the end contribute zero columns
+  const float s1 = amax > 0.f ? amax / 127.0f : 1.0f;
+  const float inv1 = 1.0f / s1, inv2 = 254.0f * inv1;
+  // x + 1.5 * 2^23 rounds x to the nearest integer (ties to even) and leaves it, in two's complement,
+  // in the low mantissa bits: the low byte is the int8 code (|x| <= 127 here by construction)
+  constexpr float kMagic = 12582912.0f;
+#pragma unroll
+  for (int n = 0; n < kMine; ++n) {
+    const int kk = wave + 4 * n;
+    u32x4 ta, tb;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      uint32_t ba[4], bb[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float q = head_ok ? f[n][4 * w + j] : 0.f;
+        const float ra = __builtin_fmaf(q, inv1, kMagic);
+        const float r = __builtin_fmaf(-(ra - kMagic), s1, q);
+        const float rb = __builtin_fmaf(r, inv2, kMagic);
+        ba[j] = as_u32(ra);
+        bb[j] = as_u32(rb);
+      }
+      ta[w] = perm(ba[1], ba[0], 0x0c0c0400u) | perm(ba[3], ba[2], 0x04000c0cu);
+      tb[w] = perm(bb[1], bb[0], 0x0c0c0400u) | perm(bb[3], bb[2], 0x04000c0cu);
+    }
+    if (kk < kMlaKSteps8) {
+      qdst[(2 * kk) * kWave] = ta;
+      qdst[(2 * kk + 1) * kWave] = tb;
+    }
+  }
+  if (wave == 0 && g == 0) a.q_scale[qblock * 16 + c] = s1;
 }
 
 __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
@@ -588,7 +586,7 @@ int kvq_mla_decode_int8(void* out, int out_dtype, float* lse, const void* q, int
   dim3 grid(splits, num_seqs, (num_heads + 127) / 128);
   if (int e = mla_prepare_device()) return e;
   dim3 qgrid(num_seqs, head_groups);
-#define KVQ_MLAQ(T) hipLaunchKernelGGL((mla_quant_q_kernel<T>), qgrid, dim3(64), 0, s, a)
+#define KVQ_MLAQ(T) hipLaunchKernelGGL((mla_quant_q_kernel<T>), qgrid, dim3(256), 0, s, a)
   switch (q_dtype) {
     case KVQ_F32: KVQ_MLAQ(KVQ_F32); break;
     case KVQ_BF16: KVQ_MLAQ(KVQ_BF16); break;
