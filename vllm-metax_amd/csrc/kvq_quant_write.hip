@@ -95,11 +95,113 @@ __global__ __launch_bounds__(256) void quant_write_kernel(
   }
 }
 
+// The same arithmetic with D / 8 lanes per row and 8 elements per lane (one 16-byte load for 16-bit
+// sources), i.e. 512 / D rows per wave: four times fewer waves than one row per wave at D = 128 and
+// 16-byte instead of 4-byte accesses.  Rows past the end are clamped for the loads and masked for
+// the stores, so that every lane takes part in the shuffles.
+template <int DT, int D>
+__global__ __launch_bounds__(256) void quant_write_rows_kernel(
+    const void* __restrict__ key, const void* __restrict__ value, int64_t key_stride_t,
+    int64_t key_stride_h, int64_t value_stride_t, int64_t value_stride_h,
+    uint8_t* __restrict__ cache, kvq_cache_geom g, const int64_t* __restrict__ slot_mapping,
+    int64_t num_rows /* T * Hkv * 2 */, float eps) {
+  constexpr int LPR = D / 8;        // lanes per row
+  constexpr int RPW = kWave / LPR;  // rows per wave
+  const int lane = threadIdx.x & (kWave - 1);
+  const int li = lane % LPR;
+  const int64_t row_raw = ((int64_t)blockIdx.x * (blockDim.x / kWave) + (threadIdx.x / kWave)) * RPW + lane / LPR;
+  const bool live = row_raw < num_rows;
+  const int64_t row = live ? row_raw : num_rows - 1;
+  const int is_v = (int)(row & 1);
+  const int64_t th = row >> 1;
+  int h;
+  int64_t t;
+  if (num_rows <= 0xffffffffLL) {
+    const uint32_t t32 = (uint32_t)th / (uint32_t)g.num_kv_heads;
+    h = (int)((uint32_t)th - t32 * (uint32_t)g.num_kv_heads);
+    t = t32;
+  } else {
+    h = (int)(th % g.num_kv_heads);
+    t = th / g.num_kv_heads;
+  }
+  const void* src = is_v ? value : key;
+  const int64_t src_base = (is_v ? (t * value_stride_t + h * value_stride_h) : (t * key_stride_t + h * key_stride_h)) + li * 8;
+  const int64_t slot = slot_mapping[t];  // in flight together with the row's loads
+  float x[8];
+  if constexpr (DT == KVQ_F32) {
+    const float* p = reinterpret_cast<const float*>(src) + src_base;
+    const floatx4 a = *reinterpret_cast<const floatx4_a4*>(p), b = *reinterpret_cast<const floatx4_a4*>(p + 4);
+    x[0] = a.x; x[1] = a.y; x[2] = a.z; x[3] = a.w; x[4] = b.x; x[5] = b.y; x[6] = b.z; x[7] = b.w;
+  } else {
+    const u32x4 v = *reinterpret_cast<const u32x4_a4*>(reinterpret_cast<const uint16_t*>(src) + src_base);
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      const uint32_t e = v[w];
+      if constexpr (DT == KVQ_BF16) {
+        x[2 * w] = as_f32(e << 16);
+        x[2 * w + 1] = as_f32(e & 0xffff0000u);
+      } else {
+        const half2_t hh = __builtin_bit_cast(half2_t, e);
+        x[2 * w] = (float)hh.x;
+        x[2 * w + 1] = (float)hh.y;
+      }
+    }
+  }
+  float amax = 0.f;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf(x[i]));
+#pragma unroll
+  for (int o = LPR / 2; o >= 1; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o, kWave));
+  amax = fmaxf(amax, eps);  // eps may be 0 for fp16 sources (1e-10 underflows)
+  const float scale = amax / 127.0f;
+  uint32_t pk[2] = {0u, 0u};
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    float r = scale > 0.f ? rintf(x[i] / scale) : 0.f;  // scale == 0: all-zero fp16 row
+    r = fminf(fmaxf(r, -128.f), 127.f);
+    pk[i >> 2] |= ((uint32_t)(int)r & 0xffu) << (8 * (i & 3));
+  }
+  if (!live || slot < 0) return;  // padding token (after the shuffles: every lane took part)
+  int64_t blk, off;
+  if ((uint64_t)slot <= 0xffffffffull) {
+    const uint32_t b32 = (uint32_t)slot / (uint32_t)g.block_size;
+    blk = b32;
+    off = (uint32_t)slot - b32 * (uint32_t)g.block_size;
+  } else {
+    blk = slot / g.block_size;
+    off = slot - blk * g.block_size;
+  }
+  uint8_t* rec = cache + blk * g.stride_block + off * g.stride_slot + (int64_t)h * g.stride_head;
+  *reinterpret_cast<u32x2_a4*>(rec + (is_v ? g.v_off : g.k_off) + li * 8) = (u32x2){pk[0], pk[1]};
+  if (li == 0) *reinterpret_cast<float*>(rec + (is_v ? g.vs_off : g.ks_off)) = scale;
+}
+
 template <int DT>
 static int launch_quant_write(const void* key, const void* value, int64_t kst, int64_t ksh,
                               int64_t vst, int64_t vsh, uint8_t* cache, const kvq_cache_geom& g,
                               const int64_t* slot_mapping, int64_t T, float eps, hipStream_t s) {
   const int64_t rows = T * g.num_kv_heads * 2;
+  // several rows per wave where the rows can be read 8 elements at a time (4-byte aligned)
+  const int esz = DT == KVQ_F32 ? 4 : 2;
+  const bool vec_ok = (g.head_size == 64 || g.head_size == 128 || g.head_size == 256) &&
+                      ((uintptr_t)key % 4) == 0 && ((uintptr_t)value % 4) == 0 &&
+                      ((kst | ksh | vst | vsh) * esz) % 4 == 0;
+  if (vec_ok) {
+    const int rpw = 512 / g.head_size;
+    const int64_t vblocks = (rows + 4 * rpw - 1) / (4 * rpw);
+    if (vblocks > 0x7fffffffLL) return fail(KVQ_EINVAL, "reshape_and_cache_int8: too many tokens");
+    dim3 vgrid((unsigned)vblocks), vblock(256);
+#define KVQ_LAUNCH_ROWS(DD)                                                                          \
+  hipLaunchKernelGGL((quant_write_rows_kernel<DT, DD>), vgrid, vblock, 0, s, key, value, kst, ksh, \
+                     vst, vsh, cache, g, slot_mapping, rows, eps)
+    switch (g.head_size) {
+      case 64: KVQ_LAUNCH_ROWS(64); break;
+      case 128: KVQ_LAUNCH_ROWS(128); break;
+      default: KVQ_LAUNCH_ROWS(256); break;
+    }
+#undef KVQ_LAUNCH_ROWS
+    return check_hip(hipGetLastError(), "reshape_and_cache_int8 launch");
+  }
   const int64_t blocks = (rows + 3) / 4;
   if (blocks > 0x7fffffffLL) return fail(KVQ_EINVAL, "reshape_and_cache_int8: too many tokens");
   dim3 grid((unsigned)blocks), block(256);
