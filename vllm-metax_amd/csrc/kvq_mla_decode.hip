@@ -6,15 +6,16 @@
 // O^T[dim, head] = C[:, :512]^T . P~^T, both on the MFMA with the heads as the N dimension.
 //
 // Work item = (sequence, token split); workgroup = 8 waves, wave w owns heads 16w .. 16w+15 of a
-// 128-head group and keeps their 512 x 16 output tile in registers; their absorbed Q sits in LDS
-// (and 4 of its 18 operands in registers) as two int8 terms that a small kernel prepares once per
-// launch, so the QK product reads the cached code bytes as they are.  (A 32-head tile per wave
-// would halve the work per flop on the PV side but needs more than the 512 registers a lane can
-// have next to the rest.)  The workgroup loads each 32-token tile once, as flat 16-byte chunks
-// (every quarter-wave reads 256 contiguous bytes), through registers into a double-buffered LDS
-// window (one barrier per tile).  For PV every wave reads the int8 rows back transposed in
-// registers and turns codes into exact fp16 numbers code + 1152 with one byte permute per two
-// codes -- the constant is taken out again through a row of ones.
+// 128-head group and keeps their 512 x 16 output tile in registers; their absorbed Q sits in
+// registers (8 of its 18 operands) and LDS as two int8 terms that a small kernel prepares once per
+// launch, so the QK product reads the cached code bytes as they are.  The workgroup loads each
+// 32-token tile once, as flat 16-byte chunks (every quarter-wave reads 256 contiguous bytes),
+// through registers into a double-buffered LDS window, and transposes its V part ONCE, shared by
+// the eight waves, into an fp16 V^T tile (plain codes, byte permutes in registers); every wave
+// then feeds the PV MFMA with 16-byte LDS reads.  Two barriers per tile: V^T visible / V^T free.
+// (Before, each wave transposed and expanded the tile for itself: 8x the vector work, ~320
+// instructions per tile per wave.  A 32-head tile per wave would also halve the LDS reads per flop
+// but needs 400 of a lane's 512 registers for Q and O alone.)
 // The token splits of a sequence are merged by the reduce kernel with the log-sum-exp algebra
 // (same two-stage shape as the reference's decode_attention_fwd); nothing is allocated here,
 // partials and the int8 Q live in the caller's workspace.
@@ -36,10 +37,12 @@ constexpr int kChunksPerHalf = 16 * kChunksPerRow;        // 576
 constexpr int kMlaThreads = 512;
 constexpr int kMlaKSteps8 = kMlaW / 64;                   // 9 int8 k-steps of 64 dims
 constexpr int kMlaQOps = 2 * kMlaKSteps8;                 // B operands of Q: two int8 terms per k-step
-constexpr int kMlaQRegOps = 4;                            // operands of Q kept in registers; the rest in LDS
-constexpr int kMlaQLdsBytes = (kMlaQOps - kMlaQRegOps) * kMlaThreads * 16;  // 114688
+constexpr int kMlaQRegOps = 8;                            // operands of Q kept in registers; the rest in LDS
+constexpr int kMlaQLdsBytes = (kMlaQOps - kMlaQRegOps) * kMlaThreads * 16;  // 81920
+constexpr int kMlaVtPitch = 2 * kTile + 16;               // fp16 V^T row: 32 tokens (+ pad: conflict-free operand reads)
+constexpr int kMlaVtBytes = kMlaR * kMlaVtPitch;          // 40960
 typedef int32_t i32x4 __attribute__((ext_vector_type(4)));
-constexpr int kMlaLdsBytes = 2 * kMlaBufBytes + kMlaQLdsBytes;                  // 153088 of 163840
+constexpr int kMlaLdsBytes = 2 * kMlaBufBytes + kMlaVtBytes + kMlaQLdsBytes;                  // 153088 of 163840
 
 struct MlaArgs {
   const void* q;
@@ -66,6 +69,14 @@ struct MlaArgs {
   float scale_log2;
   uint32_t bs_magic;
 };
+
+// Bytes (0,1) or (2,3) of x (codes ^ 0x80) as two exact fp16 codes: 0x6400 | byte is 1024 + byte =
+// code + 1152; the constant is subtracted again (exact in fp16).
+__device__ __forceinline__ uint32_t mla_codes_to_half2(uint32_t x, bool upper) {
+  const half2_t bias = {(half_t)kCodeBias, (half_t)kCodeBias};
+  const half2_t v = __builtin_bit_cast(half2_t, bytes_to_half2(x, upper)) - bias;
+  return __builtin_bit_cast(uint32_t, v);
+}
 
 // tokens of a sequence per split, a whole number of tiles
 __device__ __forceinline__ int mla_split_len(int len, int num_splits) {
@@ -174,7 +185,8 @@ __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
   extern __shared__ __align__(16) uint8_t lds_raw[];
   uint8_t(*lds)[kMlaBufBytes] = reinterpret_cast<uint8_t(*)[kMlaBufBytes]>(lds_raw);
   // B operands of Q from number kMlaQRegOps on: slot [operand][thread], written and read by the same lane
-  u32x4* qlds = reinterpret_cast<u32x4*>(lds_raw + 2 * kMlaBufBytes) + threadIdx.x;
+  uint8_t* vt = lds_raw + 2 * kMlaBufBytes;  // fp16 V^T of the current tile
+  u32x4* qlds = reinterpret_cast<u32x4*>(lds_raw + 2 * kMlaBufBytes + kMlaVtBytes) + threadIdx.x;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -288,17 +300,47 @@ __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
   floatx4 o[kMlaDT];
 #pragma unroll
   for (int dt = 0; dt < kMlaDT; ++dt) o[dt] = (floatx4){0.f, 0.f, 0.f, 0.f};
-  floatx4 psum = {0.f, 0.f, 0.f, 0.f};
   float m = -INFINITY, l = 0.f;
+
+  // ---- V^T of the tile as fp16, made ONCE per workgroup: wave v transposes dims 64 v .. 64 v + 63.
+  //      A thread takes, twice, a block of 4 tokens x 4 dims (one dword per token row), transposes it
+  //      with byte permutes and writes, for each of the 4 dims, the 4 tokens' plain codes as fp16 (8
+  //      bytes).  Dim 64 w + 4 r' + b sits in row (4 w + b) * 16 + r' -- row r' of output tile 4 w + b --
+  //      and token 16 mt + 4 g' + i at position 8 g' + 4 mt + i, the order in which a lane of the P~
+  //      operand holds its 8 tokens.  Lanes = 8 consecutive rows x 8 token groups: the 8-byte writes
+  //      of a wave spread evenly over the LDS banks.
+  const int tr = lane & 7, tq = lane >> 3;
+  const uint32_t vt_src = (uint32_t)(4 * tq * kMlaPitch + 4 * (16 * wave + tr));
+  const uint32_t vt_dst = (uint32_t)((64 * wave + tr) * kMlaVtPitch + 2 * (8 * (tq & 3) + 4 * (tq >> 2)));
+  auto transpose_v = [&](const uint8_t* tile) __attribute__((always_inline)) {
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      uint32_t x[4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        x[r] = *reinterpret_cast<const uint32_t*>(tile + vt_src + r * kMlaPitch + 32 * u) ^ 0x80808080u;
+      const uint32_t a01 = perm(x[1], x[0], 0x05010400u), b01 = perm(x[1], x[0], 0x07030602u);
+      const uint32_t a23 = perm(x[3], x[2], 0x05010400u), b23 = perm(x[3], x[2], 0x07030602u);
+#pragma unroll
+      for (int b = 0; b < 4; ++b) {
+        u32x2 h;
+        h.x = mla_codes_to_half2(b < 2 ? a01 : b01, b & 1);
+        h.y = mla_codes_to_half2(b < 2 ? a23 : b23, b & 1);
+        *reinterpret_cast<u32x2*>(vt + vt_dst + (16 * b + 8 * u) * kMlaVtPitch) = h;
+      }
+    }
+  };
+
+  stage(lds[0]);
+  issue_loads(nb);  // unconditional: past the split's end it rereads a valid half that is never used
+  lds_barrier();
+  nb = fetch_blocks(t_begin + 2);  // after the barrier, whose wait would otherwise expose these scalar loads
 
   int buf = 0;
   for (int t = t_begin; t < t_end; ++t) {
-    stage(lds[buf]);
-    issue_loads(nb);  // unconditional: past the split's end it rereads a valid half that is never staged
-    lds_barrier();
-    nb = fetch_blocks(t + 2);  // after the barrier, whose wait would otherwise expose these scalar loads
     const uint8_t* tile = lds[buf];
     const float* sck = reinterpret_cast<const float*>(tile + kMlaTileBytes);
+    transpose_v(tile);
 
     // ---- S^T[32 tokens, 16 heads] on the int8 MFMA: A = the cached code bytes as they are, lane
     //      (r = token, g): dims 64 kk + 16 g ..; one accumulator per term of Q
@@ -347,7 +389,6 @@ __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
       const float alpha = __builtin_amdgcn_exp2f(m - m_new);
       m = m_new;
       l *= alpha;
-      psum *= alpha;
 #pragma unroll
       for (int dt = 0; dt < kMlaDT; ++dt) o[dt] *= alpha;
     }
@@ -370,40 +411,24 @@ __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
     pb.w = pack_half2(pt[6], pt[7]);
     const half8_t p_op = __builtin_bit_cast(half8_t, pb);
 
-    // ---- O^T[512 dims, 16 heads] += (C + 1152)^T . P~^T.  Lane (r, g) supplies, for w = 0..7, bytes
-    //      [64 w + 4 r, +4) of tokens 4g+j (j<4) and 16+4g+(j-4), transposed in registers: row r of
-    //      output tile 4w+b is dim 64 w + 4 r + b.  (Lanes r = 0..15 read 16 consecutive dwords of a
-    //      row, so the 64 lanes of a read spread over all LDS banks.)
-    {
-      const half_t one = (half_t)1.0f;
-      const half8_t ones = {one, one, one, one, one, one, one, one};
-      psum = __builtin_amdgcn_mfma_f32_16x16x32_f16(ones, p_op, psum, 0, 0, 0);
+    // the next tile goes into the other raw window (its last readers finished before the previous
+    // iteration's second barrier) and the loads of the tile after it are issued
+    if (t + 1 < t_end) {
+      stage(lds[buf ^ 1]);
+      issue_loads(nb);
     }
+    lds_barrier();  // V^T of this tile (and the next raw tile) is visible to every wave
+    nb = fetch_blocks(t + 3);
+
+    // ---- O^T[512 dims, 16 heads] += C^T . P~^T: A = fp16 V^T rows, lane (r = row of output tile dt,
+    //      g): positions 8 g .. 8 g + 7
+    const uint8_t* vrow = vt + c * kMlaVtPitch + 16 * g;
 #pragma unroll
-    for (int w = 0; w < kMlaVB / 4; ++w) {
-      uint32_t x0[4], x1[4];
-#pragma unroll
-      for (int pr = 0; pr < 4; ++pr) {
-        const int ja = 2 * pr, jb = 2 * pr + 1;
-        const int ta_tok = (ja & 3) + (ja >> 2) * 16 + 4 * g;
-        const int tb_tok = (jb & 3) + (jb >> 2) * 16 + 4 * g;
-        const uint32_t ta = *reinterpret_cast<const uint32_t*>(tile + ta_tok * kMlaPitch + 64 * w + 4 * c) ^ 0x80808080u;
-        const uint32_t tb = *reinterpret_cast<const uint32_t*>(tile + tb_tok * kMlaPitch + 64 * w + 4 * c) ^ 0x80808080u;
-        x0[pr] = perm(tb, ta, 0x05010400u);
-        x1[pr] = perm(tb, ta, 0x07030602u);
-      }
-#pragma unroll
-      for (int b = 0; b < 4; ++b) {
-        u32x4 av;
-        const uint32_t* x = (b < 2) ? x0 : x1;
-        av.x = bytes_to_half2(x[0], b & 1);
-        av.y = bytes_to_half2(x[1], b & 1);
-        av.z = bytes_to_half2(x[2], b & 1);
-        av.w = bytes_to_half2(x[3], b & 1);
-        const int dt = 4 * w + b;
-        o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, av), p_op, o[dt], 0, 0, 0);
-      }
+    for (int dt = 0; dt < kMlaDT; ++dt) {
+      const half8_t va = *reinterpret_cast<const half8_t*>(vrow + dt * 16 * kMlaVtPitch);
+      o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va, p_op, o[dt], 0, 0, 0);
     }
+    lds_barrier();  // every wave is done with V^T before the next tile's transposition overwrites it
     buf ^= 1;
   }
 
@@ -412,7 +437,6 @@ __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
   l += __shfl_xor(l, 16, kWave);
   l += __shfl_xor(l, 32, kWave);
   if (!wave_ok) return;
-  const float corr = kCodeBias * psum[0];
   const float inv = 1.0f / (l * kPScale);
   uint16_t* po = a.part_o + pblock * (16 * kMlaR) + lane * 4;
 #pragma unroll
@@ -420,8 +444,8 @@ __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       u32x2 v;  // a locally normalised output is a convex mix of dequantised rows: within fp16 range
-      v.x = pack_half2(clamp_half_range((o[4 * d4 + 0][i] - corr) * inv), clamp_half_range((o[4 * d4 + 1][i] - corr) * inv));
-      v.y = pack_half2(clamp_half_range((o[4 * d4 + 2][i] - corr) * inv), clamp_half_range((o[4 * d4 + 3][i] - corr) * inv));
+      v.x = pack_half2(clamp_half_range(o[4 * d4 + 0][i] * inv), clamp_half_range(o[4 * d4 + 1][i] * inv));
+      v.y = pack_half2(clamp_half_range(o[4 * d4 + 2][i] * inv), clamp_half_range(o[4 * d4 + 3][i] * inv));
       *reinterpret_cast<u32x2*>(po + (d4 * 4 + i) * 256) = v;
     }
   }
