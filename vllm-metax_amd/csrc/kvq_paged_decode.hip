@@ -14,6 +14,8 @@
 //
 // The fixed-partition entry point (512-token partitions, locally normalised partials)
 // reuses the same tile code with the reference's (partition, sequence) grid.
+#include <type_traits>
+
 #include "kvq_attn_core.cuh"
 
 namespace kvq {
@@ -193,17 +195,20 @@ __global__ __launch_bounds__(256) void paged_decode_streamk_reduce_kernel(Stream
   // Few slots (the usual case: a sequence spans a handful of workgroups): the (m, l) pairs and ALL
   // the partial outputs are requested in one go, so the kernel pays one memory round trip for them
   // instead of two.
-  constexpr int kFew = 16;
-  if (w_last - w_first < kFew) {
+  constexpr int kFew = 32;
+  // N = how many slots the one-round-trip path requests (all of them unconditionally: slots past the
+  // last reread the last one), in three sizes so that a short span does not fetch 32 rows
+  auto merge_few = [&](auto n_tag) __attribute__((always_inline)) {
+    constexpr int N = decltype(n_tag)::value;
     const int w = w_first + lane;
     const bool live = w <= w_last && wg_tile_begin(w, total, P) < wg_tile_begin(w + 1, total, P);
     const int64_t slot = (int64_t)min(w, w_last) + seq;
     const uint32_t keep = live ? 0xffffffffu : 0u;
     const float mj_raw = a.part_ml[(slot * a.io.num_q_heads + head) * 2 + 0];
     const float lj_raw = a.part_ml[(slot * a.io.num_q_heads + head) * 2 + 1];
-    float po[kFew][V];
+    float po[N][V];
 #pragma unroll
-    for (int k = 0; k < kFew; ++k) {
+    for (int k = 0; k < N; ++k) {
       const int64_t sk = (int64_t)min(w_first + k, w_last) + seq;
       const float* p = a.part_o + (sk * a.io.num_q_heads + head) * (int64_t)D + lane * V;
 #pragma unroll
@@ -215,12 +220,20 @@ __global__ __launch_bounds__(256) void paged_decode_streamk_reduce_kernel(Stream
     const float ej = live ? __builtin_amdgcn_exp2f(mj - m) : 0.f;
     l = wave_sum(lj * ej);
 #pragma unroll
-    for (int k = 0; k < kFew; ++k) {
+    for (int k = 0; k < N; ++k) {
       const float wk = __shfl(ej, k, kWave);  // 0 for slots past the last and for empty ones
       const uint32_t kk = wk != 0.f ? 0xffffffffu : 0u;
 #pragma unroll
       for (int i = 0; i < V; ++i) acc[i] += as_f32(as_u32(po[k][i]) & kk) * wk;
     }
+  };
+  const int span = w_last - w_first + 1;
+  if (span <= 4) {
+    merge_few(std::integral_constant<int, 4>{});
+  } else if (span <= 12) {
+    merge_few(std::integral_constant<int, 12>{});
+  } else if (span <= kFew) {
+    merge_few(std::integral_constant<int, kFew>{});
   } else
   for (int wb = w_first; wb <= w_last; wb += kWave) {
     const int w = wb + lane;
@@ -241,14 +254,25 @@ __global__ __launch_bounds__(256) void paged_decode_streamk_reduce_kernel(Stream
 #pragma unroll
     for (int i = 0; i < V; ++i) acc[i] *= ca;
     m = m_new;
+    // sixteen slots per round trip: the loads of a batch are unconditional (slots past the last reread
+    // the last one, weight 0) so that they all leave before the first is used
     const int count = min(kWave, w_last - wb + 1);
-#pragma unroll 4
-    for (int k = 0; k < count; ++k) {
-      const float wk = __shfl(ej, k, kWave);  // the partial outputs are unnormalised sums
-      const uint32_t kk = wk != 0.f ? 0xffffffffu : 0u;
-      const float* po = a.part_o + (((int64_t)(wb + k) + seq) * a.io.num_q_heads + head) * (int64_t)D + lane * V;
+    for (int k0 = 0; k0 < count; k0 += 16) {
+      float pv[16][V];
 #pragma unroll
-      for (int i = 0; i < V; ++i) acc[i] += as_f32(as_u32(po[i]) & kk) * wk;
+      for (int k = 0; k < 16; ++k) {
+        const int64_t sk = (int64_t)min(wb + k0 + k, w_last) + seq;
+        const float* po = a.part_o + (sk * a.io.num_q_heads + head) * (int64_t)D + lane * V;
+#pragma unroll
+        for (int i = 0; i < V; ++i) pv[k][i] = po[i];
+      }
+#pragma unroll
+      for (int k = 0; k < 16; ++k) {
+        const float wk = (k0 + k) < count ? __shfl(ej, (k0 + k) & (kWave - 1), kWave) : 0.f;  // unnormalised sums
+        const uint32_t kk = wk != 0.f ? 0xffffffffu : 0u;
+#pragma unroll
+        for (int i = 0; i < V; ++i) acc[i] += as_f32(as_u32(pv[k][i]) & kk) * wk;
+      }
     }
   }
   const float inv = 1.0f / l;
