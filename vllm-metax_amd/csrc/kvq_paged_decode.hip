@@ -42,10 +42,14 @@ constexpr int kSetupUnits = 1;
 // [window_first / 32, ceil(len / 32)).  0 for prefill sequences and empty ones.
 __device__ __forceinline__ int decode_tiles(const int32_t* seq_lens, const int32_t* cu, int s, int num_seqs,
                                             int window) {
-  if (s >= num_seqs) return 0;
-  if (cu != nullptr && (cu[s + 1] - cu[s]) != 1) return 0;
-  const int len = seq_lens[s];
-  return len > 0 ? (len + kTile - 1) / kTile - window_first(len, window) / kTile : 0;
+  // no data-dependent branches: the loads of a lane (and of the lanes' next chunks) all go out
+  // together; a lane past the last sequence rereads the last one and its result is dropped
+  const int sc = s < num_seqs ? s : num_seqs - 1;
+  const int len = seq_lens[sc];
+  int q_len = 1;
+  if (cu != nullptr) q_len = cu[sc + 1] - cu[sc];
+  const int n = (len + kTile - 1) / kTile - window_first(len, window) / kTile;
+  return (s < num_seqs && q_len == 1 && len > 0) ? n : 0;
 }
 
 // Units a sequence takes on the work line: its setup charge, then one unit per tile.
@@ -53,6 +57,78 @@ __device__ __forceinline__ int decode_units(const int32_t* seq_lens, const int32
                                             int window) {
   const int n = decode_tiles(seq_lens, cu, s, num_seqs, window);
   return n > 0 ? n + kSetupUnits : 0;
+}
+
+// The scans over the sequences work on chunks of 64 (one per lane).  Large batches take kScanBatch
+// chunks per step so that their loads are in flight together (batch 512: 16 dependent round trips
+// -> 4); a batch that fits one chunk keeps the single-chunk loop, which measured 3 us faster there.
+constexpr int kScanBatch = 4;
+
+// Total units of the work line.
+template <int BATCH>
+__device__ __forceinline__ int64_t scan_total(const StreamKArgs& a, int lane) {
+  const int B = a.num_seqs;
+  int64_t total = 0;
+  for (int base = 0; base < B; base += kWave * BATCH) {
+    int n[BATCH];
+#pragma unroll
+    for (int j = 0; j < BATCH; ++j)
+      n[j] = decode_units(a.seq_lens, a.cu_seqlens_q, base + kWave * j + lane, B, a.io.window);
+#pragma unroll
+    for (int j = 0; j < BATCH; ++j) total += __builtin_amdgcn_readlane(wave_incl_scan(n[j], lane), 63);
+  }
+  return total;
+}
+
+// The sequence that holds unit `lo` and the index of its first unit.
+template <int BATCH>
+__device__ __forceinline__ void scan_locate(const StreamKArgs& a, int lane, int64_t lo, int& seq, int64_t& seq_start) {
+  const int B = a.num_seqs;
+  int64_t cum = 0;
+  bool found = false;
+  for (int base = 0; base < B && !found; base += kWave * BATCH) {
+    int nn[BATCH];
+#pragma unroll
+    for (int j = 0; j < BATCH; ++j)
+      nn[j] = decode_units(a.seq_lens, a.cu_seqlens_q, base + kWave * j + lane, B, a.io.window);
+#pragma unroll
+    for (int j = 0; j < BATCH; ++j) {
+      const int n = nn[j];
+      const int incl = wave_incl_scan(n, lane);
+      const int64_t first = cum + incl - n, last = cum + incl;
+      const uint64_t hit = __builtin_amdgcn_ballot_w64(n > 0 && first <= lo && lo < last);
+      if (hit != 0 && !found) {
+        const int src = __builtin_ctzll(hit);
+        seq = base + kWave * j + src;
+        seq_start = cum + __builtin_amdgcn_readlane(incl - n, src);
+        found = true;
+      }
+      cum += __builtin_amdgcn_readlane(incl, 63);
+    }
+  }
+}
+
+// Total units and the first unit of sequence `seq`; n_first = the units of the first BATCH chunks,
+// loaded by the caller ahead of its first branch.
+template <int BATCH>
+__device__ __forceinline__ void scan_start(const StreamKArgs& a, int lane, int seq, const int (&n_first)[BATCH],
+                                           int64_t& total, int64_t& start) {
+  const int B = a.num_seqs;
+  total = 0;
+  start = 0;
+  for (int base = 0; base < B; base += kWave * BATCH) {
+    int nn[BATCH];
+#pragma unroll
+    for (int j = 0; j < BATCH; ++j)
+      nn[j] = base == 0 ? n_first[j] : decode_units(a.seq_lens, a.cu_seqlens_q, base + kWave * j + lane, B, a.io.window);
+#pragma unroll
+    for (int j = 0; j < BATCH; ++j) {
+      const int n = nn[j], b0 = base + kWave * j;
+      const int incl = wave_incl_scan(n, lane);
+      if (seq >= b0 && seq < b0 + kWave) start = total + __builtin_amdgcn_readlane(incl - n, seq - b0);
+      total += __builtin_amdgcn_readlane(incl, 63);
+    }
+  }
 }
 
 __device__ __forceinline__ int64_t wg_tile_begin(int w, int64_t total, int num_wg) {
@@ -82,12 +158,8 @@ __global__ __launch_bounds__(WPW * 64) void paged_decode_streamk_kernel(StreamKA
   const int B = a.num_seqs;
 
   // total units of the work line (each wave redoes this tiny scan; no LDS, no barrier)
-  int64_t total = 0;
-  for (int base = 0; base < B; base += kWave) {
-    int n = decode_units(a.seq_lens, a.cu_seqlens_q, base + lane, B, a.io.window);
-    n = wave_incl_scan(n, lane);
-    total += __builtin_amdgcn_readlane(n, 63);
-  }
+  const bool one_chunk = B <= kWave;
+  const int64_t total = one_chunk ? scan_total<1>(a, lane) : scan_total<kScanBatch>(a, lane);
   const int num_wg = active_workgroups(total, a.num_wg);
   if (w >= num_wg) return;
   const int64_t lo = wg_tile_begin(w, total, num_wg);
@@ -97,22 +169,8 @@ __global__ __launch_bounds__(WPW * 64) void paged_decode_streamk_kernel(StreamKA
   // locate the sequence holding unit `lo`
   int seq = 0;
   int64_t seq_start = 0;  // global index of the sequence's first unit
-  {
-    int64_t cum = 0;
-    for (int base = 0; base < B; base += kWave) {
-      const int n = decode_units(a.seq_lens, a.cu_seqlens_q, base + lane, B, a.io.window);
-      const int incl = wave_incl_scan(n, lane);
-      const int64_t first = cum + incl - n, last = cum + incl;
-      const uint64_t hit = __builtin_amdgcn_ballot_w64(n > 0 && first <= lo && lo < last);
-      if (hit != 0) {
-        const int src = __builtin_ctzll(hit);
-        seq = base + src;
-        seq_start = cum + __builtin_amdgcn_readlane(incl - n, src);
-        break;
-      }
-      cum += __builtin_amdgcn_readlane(incl, 63);
-    }
-  }
+  if (one_chunk) scan_locate<1>(a, lane, lo, seq, seq_start);
+  else scan_locate<kScanBatch>(a, lane, lo, seq, seq_start);
   seq = __builtin_amdgcn_readfirstlane(seq);
 
   int64_t pos = lo;
@@ -163,7 +221,14 @@ __global__ __launch_bounds__(256) void paged_decode_streamk_reduce_kernel(Stream
   const int q0 = a.cu_seqlens_q ? a.cu_seqlens_q[seq] : seq;
   const int q1 = a.cu_seqlens_q ? a.cu_seqlens_q[seq + 1] : seq + 1;
   const int len = a.seq_lens[seq];
-  int n_first = decode_units(a.seq_lens, a.cu_seqlens_q, lane, B, a.io.window);  // first 64 sequences of the scan
+  const bool one_chunk = B <= kWave;
+  int n_first[kScanBatch];  // first sequences of the scan
+  n_first[0] = decode_units(a.seq_lens, a.cu_seqlens_q, lane, B, a.io.window);
+  if (!one_chunk) {
+#pragma unroll
+    for (int j = 1; j < kScanBatch; ++j)
+      n_first[j] = decode_units(a.seq_lens, a.cu_seqlens_q, kWave * j + lane, B, a.io.window);
+  }
   if (q1 - q0 != 1) return;
   const int64_t row = q0;
   const int ntiles = len > 0 ? (len + kTile - 1) / kTile - window_first(len, a.io.window) / kTile : 0;
@@ -173,12 +238,12 @@ __global__ __launch_bounds__(256) void paged_decode_streamk_reduce_kernel(Stream
     if (a.io.lse != nullptr && lane == 0) a.io.lse[row * a.io.num_q_heads + head] = -INFINITY;
     return;
   }
-  int64_t total = 0, start = 0;
-  for (int base = 0; base < B; base += kWave) {
-    int n = base == 0 ? n_first : decode_units(a.seq_lens, a.cu_seqlens_q, base + lane, B, a.io.window);
-    const int incl = wave_incl_scan(n, lane);
-    if (seq >= base && seq < base + kWave) start = total + __builtin_amdgcn_readlane(incl - n, seq - base);
-    total += __builtin_amdgcn_readlane(incl, 63);
+  int64_t total, start;
+  if (one_chunk) {
+    const int n1[1] = {n_first[0]};
+    scan_start<1>(a, lane, seq, n1, total, start);
+  } else {
+    scan_start<kScanBatch>(a, lane, seq, n_first, total, start);
   }
   const int P = active_workgroups(total, a.num_wg);
   // workgroup holding unit x: the largest w with floor(w*T/P) <= x; the sequence's tiles are units
