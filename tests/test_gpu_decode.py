@@ -68,6 +68,35 @@ def test_ragged_lengths_fp32_out(gpu_device, ctx):
     T.assert_close_attn(got, want, atol=2e-3, rtol=2e-3, what=f"ctx={ctx[:5]}")
 
 
+@pytest.mark.parametrize("hkv", [1, 2, 8])
+def test_hundreds_of_short_sequences(gpu_device, hkv):
+    """300 sequences of 0 .. 200 tokens with prefill rows in between: the sequence scans run in
+    batches of several 64-sequence chunks, a workgroup's share crosses many sequence boundaries
+    (or, with one kv head, the work line is so short that not every workgroup gets a share), and
+    empty sequences must come out as zeros with lse = -inf."""
+    g = torch.Generator().manual_seed(hkv)
+    ctx = torch.randint(0, 201, (300,), generator=g).tolist()
+    qls = [1] * 300
+    for i in range(7, 300, 41):            # a few rows of another kind: short query runs
+        qls[i] = min(3, max(ctx[i], 1))
+        ctx[i] = max(ctx[i], qls[i])
+    from test_gpu_prefill import build
+    kv, lay, bt, q, sl, cu = build([max(c, 1) for c in ctx], qls, 2 * hkv, hkv, 128, 16, seed=hkv)
+    sl = torch.tensor(ctx, dtype=torch.int32)   # the true lengths, zeros included
+    scale = 1 / math.sqrt(128)
+    want, want_lse = oracle.paged_attn(q, T.storage_bytes(kv), lay, bt, sl, cu, scale, return_lse=True)
+    kvd = T.to_device_cache(kv, gpu_device, "NHD")
+    k, v = L.key_value_views(kvd)
+    ks, vs = L.scale_views(kvd)
+    out = torch.full(q.shape, float("nan"), dtype=torch.float32, device=gpu_device)
+    lse = torch.full(q.shape[:2], float("nan"), dtype=torch.float32, device=gpu_device)
+    ops.unified_attention(q.to(gpu_device), k, v, out, cu.to(gpu_device), max(qls), sl.to(gpu_device), max(ctx), scale,
+                          True, block_table=bt.to(gpu_device), k_scale_cache=ks, v_scale_cache=vs, lse=lse)
+    torch.cuda.synchronize()
+    T.assert_close_attn(out, want, atol=2e-3, rtol=2e-3, what=f"300 sequences, hkv={hkv}")
+    torch.testing.assert_close(lse.cpu(), want_lse, atol=5e-3, rtol=1e-3)
+
+
 @pytest.mark.parametrize("hq,hkv,d,bs", [(28, 4, 128, 16), (8, 8, 128, 16), (16, 1, 128, 32), (8, 2, 64, 16),
                                          (4, 2, 256, 16), (32, 16, 128, 64),
                                          # head counts of the reference's paged-attention grid
