@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define KVQ_ABI_VERSION 3
+#define KVQ_ABI_VERSION 4
 
 #define KVQ_OK 0
 #define KVQ_EINVAL (-22)
@@ -247,6 +247,24 @@ KVQ_API int kvq_gather_and_dequant_mla_int8(void* dst, int dst_dtype, int64_t ds
                                     int64_t bt_stride, const int32_t* cu_seq_lens,
                                     const int32_t* token_to_seq, const int32_t* seq_starts,
                                     int64_t num_tokens, kvq_stream_t stream);
+
+/*
+ * Gather the latent rows of `batch_size` sequences WITHOUT dequantising them.
+ * Stands in for cp_gather_cache(src_cache, dst, block_table, cu_seq_lens,
+ * batch_size, seq_starts), csrc/libtorch_stable/cache_kernels.cu:1316-1379,
+ * 1397-1462, over the int8 latent cache: destination row t (int8, dst_stride
+ * bytes apart) belongs to the sequence b with cu_seq_lens[b] <= t <
+ * cu_seq_lens[b+1], position t - cu_seq_lens[b] (+ seq_starts[b] when given, which
+ * need not be a multiple of the block size), and receives the row's
+ * kv_lora_rank + rope_dim code bytes followed by the 4 bytes of its fp32 scale:
+ * the token-major form of a cache whose blocks keep codes and scales apart.
+ * Rows >= cu_seq_lens[batch_size] are left untouched.
+ */
+KVQ_API int kvq_cp_gather_mla_int8(void* dst, int64_t dst_stride, const void* cache,
+                           const kvq_mla_geom* geom, const int32_t* block_table,
+                           int64_t bt_stride, const int32_t* cu_seq_lens,
+                           const int32_t* seq_starts, int batch_size, int64_t num_tokens,
+                           kvq_stream_t stream);
 
 /*
  * Workspace for kvq_mla_decode_int8 (host query, depends on the device): the fp16

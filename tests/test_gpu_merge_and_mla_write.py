@@ -133,3 +133,50 @@ def test_mla_gather_and_dequant_bit_exact(gpu_device, dst_dtype, use_starts):
     src = torch.cat([rows[b][starts[b]:starts[b] + chunk[b]] for b in range(3)])
     amax = src.abs().amax(-1, keepdim=True)
     assert bool(((want - src).abs() <= amax / 127 * 0.5 * (1 + 1e-4)).all())
+
+
+@pytest.mark.parametrize("use_starts", [False, True])
+def test_mla_cp_gather_bit_exact(gpu_device, use_starts):
+    """cp_gather_cache over the int8 latent cache (pattern of the reference's
+    tests/kernels/attention/test_cache.py:706-863 gather tests): every destination row is the
+    token's 576 code bytes followed by its 4 scale bytes, found with a plain python walk over the
+    block table; chunk starts that are no multiple of the block size; rows past the last sequence
+    untouched; and the rows dequantise to exactly what gather_and_maybe_dequant_cache returns."""
+    dev = gpu_device
+    R, P, bs, nb = 512, 64, 64, 12
+    W = R + P
+    g = torch.Generator().manual_seed(23)
+    ctx = [130, 64, 300]
+    bt = T.make_block_tables(ctx, bs, nb, g)
+    cpu = L.allocate_mla_cache(nb, bs, W, device="cpu", fill=0x33)
+    codes, scales = L.mla_cache_views(cpu)
+    lay = oracle.MlaLayout.from_views(cpu, codes, scales, R)
+    for i, slots in enumerate(T.slots_for(bt, ctx, bs)):
+        oracle.mla_cache_write(torch.randn((ctx[i], R), generator=g).to(torch.bfloat16),
+                               torch.randn((ctx[i], P), generator=g).to(torch.bfloat16), cpu, lay, slots)
+    starts = [41, 0, 250] if use_starts else [0, 0, 0]
+    chunk = [70, 64, 50] if use_starts else ctx
+    cu = torch.tensor([0] + torch.tensor(chunk).cumsum(0).tolist(), dtype=torch.int32)
+    n = int(cu[-1])
+    want = torch.empty((n, W + 4), dtype=torch.int8)
+    t = 0
+    for b in range(3):
+        for p in range(starts[b], starts[b] + chunk[b]):
+            blk, off = int(bt[b, p // bs]), p % bs
+            want[t, :W] = codes[blk, off]
+            want[t, W:] = scales[blk, off].reshape(1).view(torch.int8)
+            t += 1
+    ss = torch.tensor(starts, dtype=torch.int32).to(dev) if use_starts else None
+    dst = torch.full((n + 5, W + 4), 9, dtype=torch.int8, device=dev)
+    cache_d = cpu.to(dev)
+    ops.cp_gather_cache(cache_d, dst, bt.to(dev), cu.to(dev), 3, seq_starts=ss)
+    torch.cuda.synchronize()
+    assert torch.equal(dst[:n].cpu(), want), "gathered rows differ from the python walk"
+    assert bool((dst[n:] == 9).all()), "rows past the last sequence were written"
+    # the same rows, dequantised by the other gather
+    t2s = torch.repeat_interleave(torch.arange(3, dtype=torch.int32), torch.tensor(chunk)).to(dev)
+    deq = torch.empty((n, W), dtype=torch.float32, device=dev)
+    ops.gather_and_maybe_dequant_cache(cache_d, deq, bt.to(dev), cu.to(dev), t2s, n, seq_starts=ss)
+    torch.cuda.synchronize()
+    row_scale = dst[:n, W:].contiguous().view(torch.float32)            # [n, 1]
+    assert torch.equal(dst[:n, :W].float() * row_scale, deq)

@@ -89,7 +89,71 @@ __global__ __launch_bounds__(256) void mla_gather_dequant_kernel(void* __restric
   }
 }
 
+// Gather without dequantisation: row t of dst = the W code bytes of its token followed by the token's
+// 4 scale bytes (W + 4 bytes, the token-major form of the cache for copies and transfers).  One
+// wavefront per token finds its sequence by bisection over cu_seq_lens (uniform, scalar loads).
+__global__ __launch_bounds__(256) void mla_cp_gather_kernel(uint8_t* __restrict__ dst, int64_t dst_stride,
+                                                            const uint8_t* __restrict__ cache, kvq_mla_geom g,
+                                                            const int32_t* __restrict__ block_table, int64_t bt_stride,
+                                                            const int32_t* __restrict__ cu_seq_lens,
+                                                            const int32_t* __restrict__ seq_starts, int batch,
+                                                            int num_tokens) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int W = g.kv_lora_rank + g.rope_dim;
+  for (int64_t t = (int64_t)blockIdx.x * (blockDim.x / kWave) + (threadIdx.x / kWave); t < num_tokens;
+       t += (int64_t)gridDim.x * (blockDim.x / kWave)) {
+    int lo = 0, hi = batch - 1;  // the last sequence whose first row is <= t
+    while (lo < hi) {
+      const int mid = (lo + hi + 1) >> 1;
+      if (cu_seq_lens[mid] <= t) lo = mid;
+      else hi = mid - 1;
+    }
+    const int b = lo;
+    if (t >= cu_seq_lens[b + 1]) continue;  // rows past the last sequence stay untouched
+    int pos = (int)t - cu_seq_lens[b];
+    if (seq_starts != nullptr) pos += seq_starts[b];
+    const int e = pos / g.block_size;
+    const int off = pos - e * g.block_size;
+    const int64_t blk = block_table[(int64_t)b * bt_stride + e];
+    const uint8_t* base = cache + blk * g.stride_block;
+    uint8_t* out = dst + t * dst_stride;
+    if (lane * 16 < W) {
+      const u32x4 w = *reinterpret_cast<const u32x4_a4*>(base + (int64_t)off * g.stride_row + lane * 16);
+      *reinterpret_cast<u32x4_a4*>(out + lane * 16) = w;
+    } else if (lane * 16 == ((W + 15) & ~15)) {  // the first idle lane carries the scale
+      *reinterpret_cast<uint32_t*>(out + W) = *reinterpret_cast<const uint32_t*>(base + g.scale_off + (int64_t)off * 4);
+    }
+  }
+}
+
 }  // namespace kvq
+
+extern "C" int kvq_cp_gather_mla_int8(void* dst, int64_t dst_stride, const void* cache, const kvq_mla_geom* geom,
+                                      const int32_t* block_table, int64_t bt_stride, const int32_t* cu_seq_lens,
+                                      const int32_t* seq_starts, int batch_size, int64_t num_tokens,
+                                      kvq_stream_t stream) {
+  using namespace kvq;
+  const char* op = "cp_gather_mla_int8";
+  KVQ_REQUIRE(geom != nullptr, "%s: geom is NULL", op);
+  KVQ_REQUIRE(num_tokens >= 0 && num_tokens <= 0x7fffffffLL, "%s: num_tokens out of range", op);
+  if (num_tokens == 0) return KVQ_OK;
+  KVQ_REQUIRE(dst && cache && block_table && cu_seq_lens, "%s: NULL pointer", op);
+  KVQ_REQUIRE(batch_size > 0, "%s: batch_size must be positive", op);
+  const kvq_mla_geom& g = *geom;
+  const int W = g.kv_lora_rank + g.rope_dim;
+  KVQ_REQUIRE(g.kv_lora_rank > 0 && g.rope_dim >= 0 && g.block_size > 0 && W % 16 == 0 && W <= 1008,
+              "%s: rows must be a multiple of 16 bytes and at most 1008 wide (got %d)", op, W);
+  KVQ_REQUIRE((g.stride_block | g.stride_row | g.scale_off) % 4 == 0 && ((uintptr_t)cache % 4) == 0,
+              "%s: cache strides must be 4-byte aligned", op);
+  KVQ_REQUIRE(dst_stride >= W + 4 && dst_stride % 4 == 0 && ((uintptr_t)dst % 4) == 0,
+              "%s: dst rows must be 4-byte aligned and at least %d bytes apart", op, W + 4);
+  const int64_t want = (num_tokens + 3) / 4;
+  const unsigned blocks = (unsigned)(want < 65536 ? want : 65536);
+  hipLaunchKernelGGL(mla_cp_gather_kernel, dim3(blocks), dim3(256), 0, as_stream(stream), static_cast<uint8_t*>(dst),
+                     dst_stride, static_cast<const uint8_t*>(cache), g, block_table, bt_stride, cu_seq_lens, seq_starts,
+                     batch_size, (int)num_tokens);
+  return check_hip(hipGetLastError(), "cp_gather_mla_int8 launch");
+}
 
 extern "C" int kvq_gather_and_dequant_mla_int8(void* dst, int dst_dtype, int64_t dst_stride, const void* cache,
                                                const kvq_mla_geom* geom, const int32_t* block_table,

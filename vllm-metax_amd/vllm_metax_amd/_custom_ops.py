@@ -494,6 +494,38 @@ def gather_and_maybe_dequant_cache(src_cache: torch.Tensor, dst: torch.Tensor, b
     _C.check(rc, "gather_and_maybe_dequant_cache")
 
 
+def cp_gather_cache(src_cache: torch.Tensor, dst: torch.Tensor, block_table: torch.Tensor, cu_seq_lens: torch.Tensor,
+                    batch_size: int, seq_starts: torch.Tensor | None = None, kv_lora_rank: int = 512,
+                    geometry: MlaGeometry | None = None) -> None:
+    """Argument order of ``cp_gather_cache`` (csrc/libtorch_stable/cache_kernels.cu:1397-1462) over
+    the int8 latent cache: ``dst`` ``[tot_tokens, W + 4]`` int8/uint8 receives, for every token of the
+    ``batch_size`` sequences (rows ``cu_seq_lens[b] .. cu_seq_lens[b+1]-1``, cache positions
+    shifted by ``seq_starts[b]`` when given), its ``W`` code bytes followed by the 4 bytes of its
+    fp32 scale -- no dequantisation."""
+    dev = _require_cuda(src_cache, dst, block_table, cu_seq_lens, seq_starts)
+    geom = geometry or mla_geometry(src_cache, kv_lora_rank)
+    W = geom.kv_lora_rank + geom.rope_dim
+    if dst.dtype not in (torch.int8, torch.uint8) or dst.dim() != 2 or dst.shape[1] != W + 4 or dst.stride(1) != 1:
+        raise RuntimeError(f"dst must be an int8 [tot_tokens, {W + 4}] tensor with a contiguous last dim")
+    for name, t in (("block_table", block_table), ("cu_seq_lens", cu_seq_lens), ("seq_starts", seq_starts)):
+        if t is not None and t.dtype != torch.int32:
+            raise RuntimeError(f"{name} must be int32")
+    if block_table.stride(1) != 1 or not cu_seq_lens.is_contiguous():
+        raise RuntimeError("block_table rows and cu_seq_lens must be contiguous")
+    if cu_seq_lens.numel() < batch_size + 1 or block_table.shape[0] < batch_size:
+        raise RuntimeError("cu_seq_lens needs batch_size + 1 entries and block_table batch_size rows")
+    if seq_starts is not None and (seq_starts.numel() < batch_size or not seq_starts.is_contiguous()):
+        raise RuntimeError("seq_starts needs batch_size contiguous entries")
+    if batch_size == 0 or dst.shape[0] == 0:
+        return
+    g = geom.as_struct()
+    with _on_device(dev):
+        rc = _C.load().kvq_cp_gather_mla_int8(
+            _ptr(dst), dst.stride(0), ctypes.c_void_p(geom.base_ptr), ctypes.byref(g), _ptr(block_table),
+            block_table.stride(0), _ptr(cu_seq_lens), _ptr(seq_starts), int(batch_size), dst.shape[0], _stream(dev))
+    _C.check(rc, "cp_gather_cache")
+
+
 def mla_decode_workspace_bytes(max_num_seqs: int, num_heads: int, kv_lora_rank: int) -> int:
     return int(_C.load().kvq_mla_decode_workspace_bytes(max_num_seqs, num_heads, kv_lora_rank))
 
