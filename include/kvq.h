@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define KVQ_ABI_VERSION 4
+#define KVQ_ABI_VERSION 5
 
 #define KVQ_OK 0
 #define KVQ_EINVAL (-22)
@@ -247,6 +247,32 @@ KVQ_API int kvq_gather_and_dequant_mla_int8(void* dst, int dst_dtype, int64_t ds
                                     int64_t bt_stride, const int32_t* cu_seq_lens,
                                     const int32_t* token_to_seq, const int32_t* seq_starts,
                                     int64_t num_tokens, kvq_stream_t stream);
+
+/*
+ * Rotary embedding of q_pe and k_pe (in place) fused with the quantise-on-write
+ * of the latent row [kv_c | rotated k_pe].  Stands in for
+ * concat_and_cache_mla_rope_fused(positions, q_pe, k_pe, kv_c, cos_sin_cache,
+ * is_neox, slot_mapping, kv_cache, kv_cache_dtype, kv_cache_scale),
+ * csrc/libtorch_stable/cache_kernels_fused.cu:24-168 (schema
+ * torch_bindings.cpp:851-862), for the int8 latent cache.
+ * q_pe [T, num_q_heads, rot_dim], k_pe [T, rot_dim], kv_c [T, kv_lora_rank] of
+ * `dtype` (strides in elements, last dim contiguous); cos_sin_cache
+ * [max_position, rot_dim] of `cos_sin_dtype`: row p holds rot_dim/2 cosines, then
+ * rot_dim/2 sines.  Pair i of a row is (i, rot_dim/2 + i) when is_neox, else
+ * (2i, 2i+1); (x, y) -> (x cos - y sin, y cos + x sin) in `dtype` arithmetic, one
+ * rounding per operation.  Tokens with slot < 0 are left entirely untouched.  The
+ * row is quantised as by kvq_concat_and_cache_mla_int8 applied to the rotated
+ * k_pe: codes and scale are bit-identical to rotating first and writing second.
+ */
+KVQ_API int kvq_concat_and_cache_mla_rope_int8(const int64_t* positions, void* q_pe,
+                                       int64_t q_stride_t, int64_t q_stride_h,
+                                       int num_q_heads, void* k_pe, int64_t k_pe_stride,
+                                       const void* kv_c, int64_t kv_c_stride, int dtype,
+                                       const void* cos_sin_cache, int cos_sin_dtype,
+                                       int rot_dim, int is_neox, void* cache,
+                                       const kvq_mla_geom* geom,
+                                       const int64_t* slot_mapping, int64_t num_tokens,
+                                       float eps, kvq_stream_t stream);
 
 /*
  * Gather the latent rows of `batch_size` sequences WITHOUT dequantising them.

@@ -294,6 +294,59 @@ def mla_cache_write(kv_c, k_pe, cache, lay: MlaLayout, slot_mapping, eps: float 
     )
 
 
+def rope_rotate(x, positions, cos_sin_cache, is_neox: bool):
+    """Rotary embedding as the reference's fused kernel applies it
+    (csrc/libtorch_stable/cache_kernels_fused.cu:55-84 for q_pe, :90-117 for k_pe), restated with
+    torch ops in the tensor's own dtype: cos / sin are cast to it first, every product and every
+    sum is rounded to it on its own (the reference's ``qk_t`` operators; for float32 that means no
+    fused multiply-add; which rounding a 16-bit type's operators perform is spelled out below).  ``x`` ``[T, ..., rot_dim]``; ``cos_sin_cache`` ``[max_position, rot_dim]``
+    = ``rot_dim/2`` cosines then ``rot_dim/2`` sines per position.  Pair i is ``(i, rot_dim/2 + i)``
+    when ``is_neox`` else ``(2i, 2i + 1)``.  Returns a new tensor."""
+    rot = x.shape[-1]
+    embed = rot // 2
+    cs = cos_sin_cache[positions.long()].to(x.dtype)                  # [T, rot]
+    shape = [x.shape[0]] + [1] * (x.dim() - 2) + [embed]
+    cos, sin = cs[:, :embed].reshape(shape), cs[:, embed:].reshape(shape)
+    if is_neox:
+        xs, ys = x[..., :embed], x[..., embed:]
+    else:
+        xs, ys = x[..., 0::2], x[..., 1::2]
+    if x.dtype == torch.float16:
+        # native half operators: every result is the exact one rounded ONCE to fp16.  The exact
+        # products and sums of fp16 numbers fit a double; numpy converts double -> half directly.
+        import numpy as np
+
+        def once(t):
+            return torch.from_numpy(t.astype(np.float16))
+
+        d = lambda t: t.double().numpy()
+        xo = once(d(once(d(xs) * d(cos))) - d(once(d(ys) * d(sin))))
+        yo = once(d(once(d(ys) * d(cos))) + d(once(d(xs) * d(sin))))
+    else:
+        # bfloat16: torch's operators go through float and round after every operation, like the
+        # bf16 operators of hip_bf16.h that the reference's ROCm branch uses (:13-16); float32: plain
+        xo = xs * cos - ys * sin
+        yo = ys * cos + xs * sin
+    out = torch.empty_like(x)
+    if is_neox:
+        out[..., :embed], out[..., embed:] = xo, yo
+    else:
+        out[..., 0::2], out[..., 1::2] = xo, yo
+    return out
+
+
+def mla_rope_cache_write(positions, q_pe, k_pe, kv_c, cos_sin_cache, is_neox: bool, cache, lay: MlaLayout,
+                         slot_mapping, eps: float | None = None):
+    """``concat_and_cache_mla_rope_fused`` (csrc/libtorch_stable/cache_kernels_fused.cu:24-168) over
+    the int8 latent cache: rotates ``q_pe`` ``[T, Hq, rot]`` and ``k_pe`` ``[T, rot]`` IN PLACE for the
+    tokens whose slot is >= 0 (padded tokens are skipped before anything is touched, :42-46) and
+    writes ``[kv_c | rotated k_pe]`` through the latent quantiser."""
+    live = slot_mapping >= 0
+    q_pe[live] = rope_rotate(q_pe[live], positions[live], cos_sin_cache, is_neox)
+    k_pe[live] = rope_rotate(k_pe[live], positions[live], cos_sin_cache, is_neox)
+    mla_cache_write(kv_c, k_pe, cache, lay, slot_mapping, eps)
+
+
 def mla_decode(q, cache, lay: MlaLayout, block_table, seq_lens, scale: float):
     """q [B, H, R+P] -> (out fp32 [B, H, R], lse fp32 [B, H])."""
     qf = _f32c(q)

@@ -22,6 +22,8 @@
  *   kvq_oracle_mla_gather_dequant   pinned   (python gather loop, code * scale in numpy fp32,
  *                                             round trip through the write)
  *   kvq_oracle_mla_decode           pinned   (torch SDPA enable_gqa + logsumexp)
+ *   (python) rope_rotate            pinned for bf16 / fp16; PARITY UNPINNED for fp32 (whether
+ *                                   the reference's compiler fuses x cos - y sin is not in its source)
  *
  * What no check available offline can pin (it lives in upstream vLLM's Triton
  * sources, which the reference imports but does not vendor): whether the

@@ -180,3 +180,50 @@ def test_mla_cp_gather_bit_exact(gpu_device, use_starts):
     torch.cuda.synchronize()
     row_scale = dst[:n, W:].contiguous().view(torch.float32)            # [n, 1]
     assert torch.equal(dst[:n, :W].float() * row_scale, deq)
+
+
+def _cos_sin(max_pos, rot, dtype=torch.float32, base=10000.0):
+    inv = 1.0 / (base ** (torch.arange(0, rot, 2, dtype=torch.float64) / rot))
+    ang = torch.arange(max_pos, dtype=torch.float64)[:, None] * inv[None, :]
+    return torch.cat([ang.cos(), ang.sin()], -1).to(dtype)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("is_neox", [True, False])
+@pytest.mark.parametrize("cs_same_dtype", [False, True])
+def test_mla_rope_fused_write_bit_exact(gpu_device, dtype, is_neox, cs_same_dtype):
+    """concat_and_cache_mla_rope_fused over the int8 latent cache: rotated q_pe and k_pe (in place),
+    codes and scales all bit-identical to the oracle (the reference kernel's arithmetic restated with
+    per-operation rounding in the activation dtype); padded tokens untouched; q_pe given as a strided
+    slice of a wider tensor, as the caller's fused q projection leaves it."""
+    dev = gpu_device
+    R, P, bs, nb, H = 512, 64, 64, 6, 16
+    g = torch.Generator().manual_seed(31 + is_neox)
+    T_ = 150
+    cs = _cos_sin(4096, P, dtype if cs_same_dtype else torch.float32)
+    pos = torch.randint(0, 4096, (T_,), generator=g)
+    q_full = torch.randn((T_, H, 128 + P), generator=g).to(dtype)     # [nope | pe] per head
+    k_pe = torch.randn((T_, P), generator=g).to(dtype)
+    kv_c = (torch.randn((T_, R), generator=g) * 3).to(dtype)
+    slots = torch.randperm(nb * bs, generator=g)[:T_].to(torch.int64)
+    slots[[3, 77, 149]] = -1
+    cpu = L.allocate_mla_cache(nb, bs, R + P, device="cpu", fill=0x22)
+    lay = oracle.MlaLayout.from_views(cpu, *L.mla_cache_views(cpu), R)
+    want_q, want_k = q_full[..., 128:].clone(), k_pe.clone()
+    oracle.mla_rope_cache_write(pos, want_q, want_k, kv_c, cs, is_neox, cpu, lay, slots)
+
+    cache_d = L.allocate_mla_cache(nb, bs, R + P, device=dev, fill=0x22)
+    q_d = q_full.to(dev)
+    k_d = k_pe.to(dev)
+    ops.concat_and_cache_mla_rope_fused(pos.to(dev), q_d[..., 128:], k_d, kv_c.to(dev), cs.to(dev), is_neox,
+                                        slots.to(dev), cache_d)
+    torch.cuda.synchronize()
+    assert torch.equal(q_d[..., 128:].cpu(), want_q), "rotated q_pe differs"
+    assert torch.equal(q_d[..., :128].cpu(), q_full[..., :128]), "the nope part of q was touched"
+    assert torch.equal(k_d.cpu(), want_k), "rotated k_pe differs"
+    assert torch.equal(cache_d.cpu(), cpu), "cache bytes (codes / scales) differ"
+    # the fused op is rotation followed by the plain latent write
+    cache2 = L.allocate_mla_cache(nb, bs, R + P, device=dev, fill=0x22)
+    ops.concat_and_cache_mla(kv_c.to(dev), k_d, cache2, slots.to(dev))
+    torch.cuda.synchronize()
+    assert torch.equal(cache2, cache_d)

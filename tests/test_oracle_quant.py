@@ -143,3 +143,70 @@ def test_mla_gather_dequant_is_the_python_gather_loop():
             blk, off = int(bt[b, pos // bs]), pos % bs
             want[t] = codes[blk, off].to(torch.float32) * scales[blk, off]
         assert torch.equal(got, want)
+
+
+# ---- rotary embedding of the fused MLA write (oracle.rope_rotate) -------------------------------
+
+def _cos_sin(max_pos, rot, dtype=torch.float32, base=10000.0):
+    inv = 1.0 / (base ** (torch.arange(0, rot, 2, dtype=torch.float64) / rot))
+    ang = torch.arange(max_pos, dtype=torch.float64)[:, None] * inv[None, :]
+    return torch.cat([ang.cos(), ang.sin()], -1).to(dtype)
+
+
+def test_rope_quarter_turns_and_pair_layouts():
+    """Exact cases: cos = 0, sin = 1 sends (x, y) to (-y, x); the NeoX layout pairs (i, rot/2 + i), the
+    GPT-J layout pairs (2i, 2i + 1); position 0 (cos = 1, sin = 0) is the identity."""
+    x = torch.tensor([[1.0, 2.0, 3.0, 4.0]])
+    cs = torch.tensor([[1.0, 1.0, 0.0, 0.0], [0.0, 0.0, 1.0, 1.0]])        # pos 0: identity, pos 1: quarter turn
+    pos = torch.tensor([1])
+    assert oracle.rope_rotate(x, pos, cs, True).tolist() == [[-3.0, -4.0, 1.0, 2.0]]
+    assert oracle.rope_rotate(x, pos, cs, False).tolist() == [[-2.0, 1.0, -4.0, 3.0]]
+    assert torch.equal(oracle.rope_rotate(x, torch.tensor([0]), cs, True), x)
+    assert torch.equal(oracle.rope_rotate(x, torch.tensor([0]), cs, False), x)
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-6), (torch.bfloat16, 2e-2), (torch.float16, 3e-3)])
+@pytest.mark.parametrize("is_neox", [True, False])
+def test_rope_matches_complex_rotation(dtype, tol, is_neox):
+    """Against exact complex arithmetic in float64: each pair is multiplied by e^{i theta}; the norm of
+    every pair is preserved to rounding; heads of a token share the token's angles."""
+    g = torch.Generator().manual_seed(3)
+    T_, H, rot = 9, 5, 64
+    cs = _cos_sin(50, rot)
+    pos = torch.randint(0, 50, (T_,), generator=g)
+    x = torch.randn((T_, H, rot), generator=g).to(dtype)
+    got = oracle.rope_rotate(x, pos, cs, is_neox).double()
+    xd = x.double()
+    xs, ys = (xd[..., :rot // 2], xd[..., rot // 2:]) if is_neox else (xd[..., 0::2], xd[..., 1::2])
+    z = torch.complex(xs, ys) * torch.polar(torch.ones(T_, rot // 2, dtype=torch.float64),
+                                            torch.arange(0, rot, 2, dtype=torch.float64)[None, :].mul(0)
+                                            + pos[:, None].double() / (10000.0 ** (torch.arange(0, rot, 2, dtype=torch.float64) / rot)))[:, None, :]
+    gs, gy = (got[..., :rot // 2], got[..., rot // 2:]) if is_neox else (got[..., 0::2], got[..., 1::2])
+    assert float((gs - z.real).abs().max()) <= tol * 4 and float((gy - z.imag).abs().max()) <= tol * 4
+    assert float(((gs ** 2 + gy ** 2).sqrt() - (xs ** 2 + ys ** 2).sqrt()).abs().max()) <= tol * 4
+
+
+def test_rope_cache_write_is_rotate_then_write_and_skips_padding():
+    """The fused op equals rotation followed by the latent write; tokens with slot < 0 keep their
+    q_pe / k_pe and leave the cache alone."""
+    from vllm_metax_amd import layout as L
+    g = torch.Generator().manual_seed(5)
+    R, P, bs, nb, T_, H = 512, 64, 16, 4, 6, 3
+    cs = _cos_sin(64, P)
+    pos = torch.randint(0, 64, (T_,), generator=g)
+    q_pe = torch.randn((T_, H, P), generator=g).to(torch.bfloat16)
+    k_pe = torch.randn((T_, P), generator=g).to(torch.bfloat16)
+    kv_c = torch.randn((T_, R), generator=g).to(torch.bfloat16)
+    slots = torch.tensor([5, -1, 17, 0, 33, -1], dtype=torch.int64)
+    a = L.allocate_mla_cache(nb, bs, R + P, device="cpu", fill=0x11)
+    b = a.clone()
+    la = oracle.MlaLayout.from_views(a, *L.mla_cache_views(a), R)
+    lb = oracle.MlaLayout.from_views(b, *L.mla_cache_views(b), R)
+    q1, k1 = q_pe.clone(), k_pe.clone()
+    oracle.mla_rope_cache_write(pos, q1, k1, kv_c, cs, True, a, la, slots)
+    k2 = oracle.rope_rotate(k_pe, pos, cs, True)
+    oracle.mla_cache_write(kv_c, k2, b, lb, slots)
+    assert torch.equal(a, b)
+    live = slots >= 0
+    assert torch.equal(k1[live], k2[live]) and torch.equal(k1[~live], k_pe[~live]) and torch.equal(q1[~live], q_pe[~live])
+    assert torch.equal(q1[live], oracle.rope_rotate(q_pe, pos, cs, True)[live])

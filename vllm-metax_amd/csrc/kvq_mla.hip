@@ -48,6 +48,109 @@ __global__ __launch_bounds__(256) void mla_quant_write_kernel(const void* __rest
   if (lane == 0) *reinterpret_cast<float*>(cache + blk * g.stride_block + g.scale_off + off * 4) = scale;
 }
 
+// Round a float to the nearest value of the activation type (the arithmetic type of the rotary
+// embedding below is the activation type, one rounding per operation).
+template <int DT>
+__device__ __forceinline__ float round_act(float v) {
+  if constexpr (DT == KVQ_F32) return v;
+  if constexpr (DT == KVQ_BF16) return bf16_bits_to_f32(f32_to_bf16_bits(v));
+  return (float)(half_t)v;
+}
+
+// (x, y) -> (x cos - y sin, y cos + x sin) in the activation type: every product and every sum is
+// rounded on its own (no fused multiply-add), as the reference's operators on qk_t do
+// (csrc/libtorch_stable/cache_kernels_fused.cu:77-84).  fp16 uses the native half operators (each
+// result correctly rounded); bf16 goes through float and rounds after every operation, which is
+// what the bf16 operators of hip_bf16.h -- the type the reference's ROCm branch selects, :13-16 --
+// do; fp32 is plain fp32 without contraction.
+template <int DT>
+__device__ __forceinline__ void rotate_pair(float x, float y, float c, float s, float& xo, float& yo) {
+#pragma clang fp contract(off)  // the default for device code is to fuse a * b + c, also through __fmul_rn
+  if constexpr (DT == KVQ_F16) {
+    const half_t hx = (half_t)x, hy = (half_t)y, hc = (half_t)c, hs = (half_t)s;
+    const half_t a = hx * hc, b = hy * hs, d = hy * hc, e = hx * hs;
+    xo = (float)(half_t)(a - b);
+    yo = (float)(half_t)(d + e);
+  } else {
+    const float a = round_act<DT>(x * c), b = round_act<DT>(y * s), d = round_act<DT>(y * c), e = round_act<DT>(x * s);
+    xo = round_act<DT>(a - b);
+    yo = round_act<DT>(d + e);
+  }
+}
+
+// Rotary embedding of q_pe and k_pe (in place) fused with the quantise-on-write of the latent row
+// [kv_c | rotated k_pe].  One workgroup per token: all 256 threads rotate the (head, pair) items of
+// q_pe; wave 0 also rotates k_pe (one pair per lane), keeps the rotated values and quantises the
+// row with them, exactly as mla_quant_write_kernel would after a separate rotation.
+template <int DT, int CT, bool NEOX>
+__global__ __launch_bounds__(256) void mla_rope_quant_write_kernel(
+    const int64_t* __restrict__ positions, void* __restrict__ q_pe, int64_t q_stride_t, int64_t q_stride_h,
+    int num_q_heads, void* __restrict__ k_pe, int64_t k_pe_stride, const void* __restrict__ kv_c, int64_t kv_c_stride,
+    const void* __restrict__ cos_sin, int rot_dim, uint8_t* __restrict__ cache, kvq_mla_geom g,
+    const int64_t* __restrict__ slot_mapping, float eps) {
+  const int64_t t = blockIdx.x;
+  const int64_t slot = slot_mapping[t];
+  if (slot < 0) return;  // padding token: nothing is rotated, nothing is written (as the reference)
+  const int64_t pos = positions[t];
+  const int embed = rot_dim / 2;
+  const int64_t cs = pos * rot_dim;
+  // ---- q_pe: (head, pair) items over all threads
+  const int nq = num_q_heads * embed;
+  for (int i = threadIdx.x; i < nq; i += blockDim.x) {
+    const int head = i / embed, pair = i - head * embed;
+    const float c = round_act<DT>(load_act<CT>(cos_sin, cs + pair));
+    const float sn = round_act<DT>(load_act<CT>(cos_sin, cs + pair + embed));
+    const int ix = NEOX ? pair : 2 * pair, iy = NEOX ? embed + pair : 2 * pair + 1;
+    const int64_t base = t * q_stride_t + (int64_t)head * q_stride_h;
+    float xo, yo;
+    rotate_pair<DT>(load_act<DT>(q_pe, base + ix), load_act<DT>(q_pe, base + iy), c, sn, xo, yo);
+    store_act<DT>(q_pe, base + ix, xo);
+    store_act<DT>(q_pe, base + iy, yo);
+  }
+  if (threadIdx.x >= kWave) return;
+  // ---- wave 0: k_pe rotation (lane = pair) and the latent row
+  const int lane = threadIdx.x;
+  const int R = g.kv_lora_rank;
+  float kx = 0.f, ky = 0.f;
+  const int ix = NEOX ? lane : 2 * lane, iy = NEOX ? embed + lane : 2 * lane + 1;
+  if (lane < embed) {
+    const float c = round_act<DT>(load_act<CT>(cos_sin, cs + lane));
+    const float sn = round_act<DT>(load_act<CT>(cos_sin, cs + lane + embed));
+    rotate_pair<DT>(load_act<DT>(k_pe, t * k_pe_stride + ix), load_act<DT>(k_pe, t * k_pe_stride + iy), c, sn, kx, ky);
+    store_act<DT>(k_pe, t * k_pe_stride + ix, kx);
+    store_act<DT>(k_pe, t * k_pe_stride + iy, ky);
+  }
+  constexpr int kMaxPerLane = 16;  // kv_lora_rank up to 1024 stays in registers
+  float x[kMaxPerLane];
+  float amax = fmaxf(fabsf(kx), fabsf(ky));
+#pragma unroll
+  for (int i = 0; i < kMaxPerLane; ++i) {
+    const int d = lane + kWave * i;
+    x[i] = d < R ? load_act<DT>(kv_c, t * kv_c_stride + d) : 0.f;
+    amax = fmaxf(amax, fabsf(x[i]));
+  }
+  amax = fmaxf(wave_max(amax), eps);
+  const float scale = amax / 127.0f;
+  const int64_t blk = slot / g.block_size;
+  const int64_t off = slot - blk * g.block_size;
+  int8_t* row = reinterpret_cast<int8_t*>(cache + blk * g.stride_block + off * g.stride_row);
+  auto code = [&](float v) {
+    float r = scale > 0.f ? rintf(v / scale) : 0.f;
+    r = fminf(fmaxf(r, -128.f), 127.f);
+    return (int8_t)(int)r;
+  };
+#pragma unroll
+  for (int i = 0; i < kMaxPerLane; ++i) {
+    const int d = lane + kWave * i;
+    if (d < R) row[d] = code(x[i]);
+  }
+  if (lane < embed) {
+    row[R + ix] = code(kx);
+    row[R + iy] = code(ky);
+  }
+  if (lane == 0) *reinterpret_cast<float*>(cache + blk * g.stride_block + g.scale_off + off * 4) = scale;
+}
+
 // Gather + dequantise latent rows into a dense [num_tokens, W] workspace (the chunked-context
 // prefill reads its cached context this way).  One wavefront per destination row: lanes 0 .. W/16-1
 // load 16 codes each (one coalesced run of W bytes), every lane reads the row's scale, and the 16
@@ -188,6 +291,66 @@ extern "C" int kvq_gather_and_dequant_mla_int8(void* dst, int dst_dtype, int64_t
   }
 #undef KVQ_MLAG
   return check_hip(hipGetLastError(), "gather_and_dequant_mla_int8 launch");
+}
+
+namespace kvq {
+template <int DT, int CT>
+static void launch_rope_write(bool neox, unsigned tokens, hipStream_t s, const int64_t* positions, void* q_pe,
+                              int64_t qst, int64_t qsh, int hq, void* k_pe, int64_t kps, const void* kv_c, int64_t kcs,
+                              const void* cos_sin, int rot, uint8_t* cache, const kvq_mla_geom& g,
+                              const int64_t* slots, float eps) {
+  if (neox)
+    hipLaunchKernelGGL((mla_rope_quant_write_kernel<DT, CT, true>), dim3(tokens), dim3(256), 0, s, positions, q_pe, qst,
+                       qsh, hq, k_pe, kps, kv_c, kcs, cos_sin, rot, cache, g, slots, eps);
+  else
+    hipLaunchKernelGGL((mla_rope_quant_write_kernel<DT, CT, false>), dim3(tokens), dim3(256), 0, s, positions, q_pe, qst,
+                       qsh, hq, k_pe, kps, kv_c, kcs, cos_sin, rot, cache, g, slots, eps);
+}
+}  // namespace kvq
+
+extern "C" int kvq_concat_and_cache_mla_rope_int8(const int64_t* positions, void* q_pe, int64_t q_stride_t,
+                                                  int64_t q_stride_h, int num_q_heads, void* k_pe,
+                                                  int64_t k_pe_stride, const void* kv_c, int64_t kv_c_stride,
+                                                  int dtype, const void* cos_sin_cache, int cos_sin_dtype,
+                                                  int rot_dim, int is_neox, void* cache, const kvq_mla_geom* geom,
+                                                  const int64_t* slot_mapping, int64_t num_tokens, float eps,
+                                                  kvq_stream_t stream) {
+  using namespace kvq;
+  const char* op = "concat_and_cache_mla_rope_int8";
+  KVQ_REQUIRE(geom != nullptr, "%s: geom is NULL", op);
+  KVQ_REQUIRE(num_tokens >= 0 && num_tokens <= 0x7fffffffLL, "%s: num_tokens out of range", op);
+  if (num_tokens == 0) return KVQ_OK;
+  KVQ_REQUIRE(positions && q_pe && k_pe && kv_c && cos_sin_cache && cache && slot_mapping, "%s: NULL pointer", op);
+  const kvq_mla_geom& g = *geom;
+  KVQ_REQUIRE(g.kv_lora_rank > 0 && g.kv_lora_rank <= 1024 && g.block_size > 0, "%s: bad geometry", op);
+  KVQ_REQUIRE(rot_dim == g.rope_dim && rot_dim > 0 && rot_dim % 2 == 0 && rot_dim <= 128,
+              "%s: rot_dim %d must equal the cache's rope width %d, be even and at most 128", op, rot_dim, g.rope_dim);
+  KVQ_REQUIRE(num_q_heads >= 0, "%s: negative num_q_heads", op);
+  KVQ_REQUIRE((g.stride_block | g.scale_off) % 4 == 0 && ((uintptr_t)cache % 4) == 0,
+              "%s: block stride / scale offset must be 4-byte aligned", op);
+  KVQ_REQUIRE(eps >= 0.f, "%s: eps must not be negative", op);
+  hipStream_t s = as_stream(stream);
+  uint8_t* c = static_cast<uint8_t*>(cache);
+  const unsigned n = (unsigned)num_tokens;
+#define KVQ_ROPE(D, C)                                                                                          \
+  launch_rope_write<D, C>(is_neox != 0, n, s, positions, q_pe, q_stride_t, q_stride_h, num_q_heads, k_pe,    \
+                          k_pe_stride, kv_c, kv_c_stride, cos_sin_cache, rot_dim, c, g, slot_mapping, eps)
+#define KVQ_ROPE_C(D)                                                              \
+  switch (cos_sin_dtype) {                                                         \
+    case KVQ_F32: KVQ_ROPE(D, KVQ_F32); break;                                     \
+    case KVQ_BF16: KVQ_ROPE(D, KVQ_BF16); break;                                   \
+    case KVQ_F16: KVQ_ROPE(D, KVQ_F16); break;                                     \
+    default: return fail(KVQ_EINVAL, "%s: unknown cos_sin_dtype %d", op, cos_sin_dtype); \
+  }
+  switch (dtype) {
+    case KVQ_F32: KVQ_ROPE_C(KVQ_F32); break;
+    case KVQ_BF16: KVQ_ROPE_C(KVQ_BF16); break;
+    case KVQ_F16: KVQ_ROPE_C(KVQ_F16); break;
+    default: return fail(KVQ_EINVAL, "%s: unknown dtype %d", op, dtype);
+  }
+#undef KVQ_ROPE_C
+#undef KVQ_ROPE
+  return check_hip(hipGetLastError(), "concat_and_cache_mla_rope_int8 launch");
 }
 
 extern "C" int kvq_concat_and_cache_mla_int8(const void* kv_c, const void* k_pe, int src_dtype,

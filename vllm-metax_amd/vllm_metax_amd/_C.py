@@ -13,7 +13,7 @@ _LIB_DIR = os.path.join(os.path.dirname(os.path.abspath(__file__)), "_lib")
 LIB_PATH = os.path.join(_LIB_DIR, "libkvq_hip.so")
 
 KVQ_F32, KVQ_BF16, KVQ_F16 = 0, 1, 2
-ABI_VERSION = 4
+ABI_VERSION = 5
 
 
 class CacheGeom(ctypes.Structure):
@@ -60,6 +60,8 @@ SIGNATURES = {
     "kvq_merge_attn_states": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i64, _i, _i, _i64, _vp]),
     "kvq_concat_and_cache_mla_int8": (_i, [_vp, _vp, _i, _i64, _i64, _vp, _mla_p, _vp, _i64, _f, _vp]),
     "kvq_gather_and_dequant_mla_int8": (_i, [_vp, _i, _i64, _vp, _mla_p, _vp, _i64, _vp, _vp, _vp, _i64, _vp]),
+    "kvq_concat_and_cache_mla_rope_int8": (_i, [_vp, _vp, _i64, _i64, _i, _vp, _i64, _vp, _i64, _i, _vp, _i, _i, _i,
+                                                _vp, _mla_p, _vp, _i64, _f, _vp]),
     "kvq_cp_gather_mla_int8": (_i, [_vp, _i64, _vp, _mla_p, _vp, _i64, _vp, _vp, _i, _i64, _vp]),
     "kvq_mla_decode_workspace_bytes": (_sz, [_i, _i, _i]),
     "kvq_mla_decode_int8": (_i, [_vp, _i, _vp, _vp, _i, _i64, _i64, _vp, _mla_p, _vp, _i64, _vp, _i, _i, _f,

@@ -461,6 +461,45 @@ def concat_and_cache_mla(kv_c: torch.Tensor, k_pe: torch.Tensor, kv_cache: torch
     _C.check(rc, "concat_and_cache_mla")
 
 
+def concat_and_cache_mla_rope_fused(positions: torch.Tensor, q_pe: torch.Tensor, k_pe: torch.Tensor,
+                                    kv_c: torch.Tensor, cos_sin_cache: torch.Tensor, is_neox: bool,
+                                    slot_mapping: torch.Tensor, kv_cache: torch.Tensor,
+                                    kv_cache_dtype: str = "int8_per_token", kv_cache_scale: torch.Tensor | None = None,
+                                    geometry: MlaGeometry | None = None) -> None:
+    """Argument order of ``concat_and_cache_mla_rope_fused``
+    (csrc/libtorch_stable/torch_bindings.cpp:851-862, cache_kernels_fused.cu:24-168): rotary
+    embedding of ``q_pe`` ``[T, Hq, rot]`` and ``k_pe`` ``[T, rot]`` in place, then ``[kv_c | k_pe]`` into
+    the int8 latent cache.  ``kv_cache_scale`` (the reference's per-tensor fp8 scale) is not used:
+    every row carries its own scale."""
+    if kv_cache_dtype != "int8_per_token":
+        raise NotImplementedError(f"kv_cache_dtype {kv_cache_dtype!r}: only int8_per_token is built")
+    dev = _require_cuda(positions, q_pe, k_pe, kv_c, cos_sin_cache, slot_mapping, kv_cache)
+    geom = geometry or mla_geometry(kv_cache, kv_c.shape[-1])
+    if q_pe.dim() != 3 or k_pe.dim() != 2 or kv_c.dim() != 2 or not (q_pe.dtype == k_pe.dtype == kv_c.dtype):
+        raise RuntimeError("q_pe [T, Hq, rot], k_pe [T, rot] and kv_c [T, R] must share one dtype")
+    rot = k_pe.shape[1]
+    if q_pe.shape[2] != rot or rot != geom.rope_dim or kv_c.shape[1] != geom.kv_lora_rank:
+        raise RuntimeError("q_pe / k_pe / kv_c widths do not match the cache entry")
+    if cos_sin_cache.dim() != 2 or cos_sin_cache.shape[1] != rot or not cos_sin_cache.is_contiguous():
+        raise RuntimeError("cos_sin_cache must be a contiguous [max_position, rot_dim] tensor")
+    if q_pe.stride(2) != 1 or k_pe.stride(1) != 1 or kv_c.stride(1) != 1:
+        raise RuntimeError("q_pe / k_pe / kv_c rows must be contiguous")
+    for name, t in (("positions", positions), ("slot_mapping", slot_mapping)):
+        if t.dtype != torch.int64 or not t.is_contiguous():
+            raise RuntimeError(f"{name} must be contiguous int64")
+    T = slot_mapping.shape[0]
+    if positions.shape[0] < T or q_pe.shape[0] < T or k_pe.shape[0] < T or kv_c.shape[0] < T:
+        raise RuntimeError("slot_mapping is longer than positions / q_pe / k_pe / kv_c")
+    g = geom.as_struct()
+    with _on_device(dev):
+        rc = _C.load().kvq_concat_and_cache_mla_rope_int8(
+            _ptr(positions), _ptr(q_pe), q_pe.stride(0), q_pe.stride(1), q_pe.shape[1], _ptr(k_pe), k_pe.stride(0),
+            _ptr(kv_c), kv_c.stride(0), _dtype_code(kv_c, "kv_c"), _ptr(cos_sin_cache),
+            _dtype_code(cos_sin_cache, "cos_sin_cache"), rot, 1 if is_neox else 0, ctypes.c_void_p(geom.base_ptr),
+            ctypes.byref(g), _ptr(slot_mapping), T, eps_for_dtype(kv_c.dtype), _stream(dev))
+    _C.check(rc, "concat_and_cache_mla_rope_fused")
+
+
 def gather_and_maybe_dequant_cache(src_cache: torch.Tensor, dst: torch.Tensor, block_table: torch.Tensor,
                                    cu_seq_lens: torch.Tensor, token_to_seq: torch.Tensor, num_tokens: int,
                                    kv_cache_dtype: str = "int8_per_token", scale: torch.Tensor | None = None,
