@@ -118,6 +118,12 @@ def build_device_state(cfg, dev, layers, seed=0, layout="NHD", permute=True):
                 new_v=new_v, out=out, ws=ws, scale=1.0 / math.sqrt(d), max_ctx=max(ctx))
 
 
+def _window_kwargs(st):
+    """window_size / softcap keywords of the attention call (the plain causal call when neither is set)."""
+    w, cap = st.get("window", 0), st.get("softcap", 0.0)
+    return dict(window_size=(w - 1, 0) if w else (-1, -1), softcap=cap)
+
+
 def run_step(st, layer, ops, write=True, attn=True):
     c = st["caches"][layer]
     if write:
@@ -126,7 +132,7 @@ def run_step(st, layer, ops, write=True, attn=True):
     if attn:
         ops.unified_attention(st["q"], c["k"], c["v"], st["out"], st["cu_d"], 1, st["sl_d"], st["max_ctx"], st["scale"],
                               True, block_table=st["bt_d"], k_scale_cache=c["ks"], v_scale_cache=c["vs"],
-                              workspace=st["ws"], geometry=c["geom"])
+                              workspace=st["ws"], geometry=c["geom"], **_window_kwargs(st))
 
 
 MFMA_F16_PEAK_TFLOPS = 2500.0
@@ -312,7 +318,8 @@ def mixed_main(args, cfg, dev, ops):
                                                              geometry=c["geom"])
         if attn:
             ops.unified_attention(q, c["k"], c["v"], out, cu_d, max(qls), sl_d, max(ctx), scale, True, block_table=bt_d,
-                                  k_scale_cache=c["ks"], v_scale_cache=c["vs"], workspace=ws, geometry=c["geom"])
+                                  k_scale_cache=c["ks"], v_scale_cache=c["vs"], workspace=ws, geometry=c["geom"],
+                                  **_window_kwargs(dict(window=args.sliding_window, softcap=args.soft_cap)))
 
     Lr = args.layers
     for i in range(args.warmup):
@@ -343,7 +350,10 @@ def mixed_main(args, cfg, dev, ops):
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(dt * 1e3, 5), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None,
         "dtype": "int8 KV codes, fp16 MFMA operands, fp32 softmax/accumulate, bf16 Q/out", "data": "synthetic",
-        "config": {"workload": args.workload, "batch": B, "new_tokens": n_tok, "sum_ctx": sum(ctx), "q_heads": hq,
+        "config": {"workload": args.workload,
+                   **({"sliding_window": args.sliding_window} if args.sliding_window else {}),
+                   **({"soft_cap": args.soft_cap} if args.soft_cap else {}),
+                   "batch": B, "new_tokens": n_tok, "sum_ctx": sum(ctx), "q_heads": hq,
                    "kv_heads": hkv, "head_dim": d, "block_size": bs, "layer_caches_rotated": Lr},
         "attn_launch_us": round(attn_s * 1e6, 1),
         "roofline": {"bound": "mfma", "achieved": round(flops / attn_s / 1e12, 1), "peak": MFMA_F16_PEAK_TFLOPS,
@@ -400,6 +410,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=40)
     ap.add_argument("--workload", default="llama3_8b_decode_b64_ctx1k-8k")
     ap.add_argument("--layers", type=int, default=4, help="distinct layer caches the steps rotate over")
+    ap.add_argument("--sliding-window", type=int, default=0,
+                    help="GQA workloads: attend to the last N keys only (0 = full causal, the configured workloads)")
+    ap.add_argument("--soft-cap", type=float, default=0.0, help="GQA workloads: logits soft cap (0 = none)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=15.0)
     args = ap.parse_args()
@@ -416,7 +429,10 @@ def main():
     if cfg.get("mixed"):
         return mixed_main(args, cfg, dev, ops)
     st = build_device_state(cfg, dev, args.layers)
+    st["window"], st["softcap"] = args.sliding_window, args.soft_cap
     attn_bytes, write_bytes = algorithmic_bytes(cfg)
+    if args.sliding_window:  # a windowed decode row reads only its last `window` tokens
+        attn_bytes, _ = algorithmic_bytes(dict(cfg, ctx=[min(c, args.sliding_window) for c in cfg["ctx"]]))
     L = args.layers
 
     for i in range(args.warmup):
@@ -461,7 +477,9 @@ def main():
         "data": "synthetic",
         "config": {"workload": args.workload, "batch": len(cfg["ctx"]), "sum_ctx": sum(cfg["ctx"]),
                    "q_heads": cfg["hq"], "kv_heads": cfg["hkv"], "head_dim": cfg["d"], "block_size": cfg["bs"],
-                   "pool_blocks": cfg["pool"], "layer_caches_rotated": L, "kv_layout": "NHD"},
+                   "pool_blocks": cfg["pool"], "layer_caches_rotated": L, "kv_layout": "NHD",
+                   **({"sliding_window": args.sliding_window} if args.sliding_window else {}),
+                   **({"soft_cap": args.soft_cap} if args.soft_cap else {})},
         "pct_hbm_peak": round(100 * value / HBM_PEAK_GBPS, 2),
         "us_per_layer": round(ms_per_step * 1e3, 2),
         "decode_tokens_per_s": round(len(cfg["ctx"]) / (dt / args.steps), 1),
