@@ -357,14 +357,12 @@ def swap_blocks(src: torch.Tensor, dst: torch.Tensor, block_size_in_bytes: int, 
     if n == 0:
         return
     block_size_in_bytes = int(block_size_in_bytes)
-    hi = int(block_mapping.max()) + 1
-    lo = int(block_mapping.min())
+    if int(block_mapping.min()) < 0:
+        raise RuntimeError("block numbers must not be negative")
     for t, col, name in ((src, 0, "src"), (dst, 1, "dst")):
         top = int(block_mapping[:, col].max()) + 1
         if top * block_size_in_bytes > t.untyped_storage().nbytes() - t.storage_offset() * t.element_size():
             raise RuntimeError(f"block_mapping names block {top - 1} beyond the end of {name}")
-    if lo < 0 or hi <= 0:
-        raise RuntimeError("block numbers must not be negative")
     lib = _C.load()
     with _on_device(dev):
         rc = lib.kvq_swap_blocks(_ptr(src), _ptr(dst), block_size_in_bytes, _ptr(block_mapping), n,
