@@ -58,6 +58,7 @@ def _run(q, cache, bt, sl, scale, out_dtype=None, want_lse=True):
     (16, 16, [17, 33, 511]),
     (32, 128, [4096]),
     (64, 20, [5, 0, 95, 1000, 31, 32]),
+    (64, 160, [70, 300, 33]),          # a second 128-head group with only two of its eight 16-head blocks
 ])
 def test_mla_decode_matches_oracle(gpu_device, dtype, bs, heads, ctx):
     cache, lay, bt, sl = _build(ctx, bs, seed=bs + heads, dtype=torch.bfloat16)
