@@ -69,10 +69,17 @@ def _ptr(t) -> ctypes.c_void_p:
     return ctypes.c_void_p(t.data_ptr() if t is not None else 0)
 
 
+_eps_cache: dict = {}
+
+
 def eps_for_dtype(dtype: torch.dtype) -> float:
     """absmax floor as the reference's quantiser applies it: ``clamp(min=1e-10)`` in the
     SOURCE dtype, before the cast to fp32 (tests/kernels/quant_utils.py:212-213)."""
-    return float(torch.tensor(QUANT_EPS, dtype=torch.float64).to(dtype).to(torch.float32))
+    got = _eps_cache.get(dtype)
+    if got is None:
+        got = float(torch.tensor(QUANT_EPS, dtype=torch.float64).to(dtype).to(torch.float32))
+        _eps_cache[dtype] = got
+    return got
 
 
 def device_num_cus() -> int:
@@ -137,12 +144,22 @@ triton_reshape_and_cache_flash_per_token_head_quant = reshape_and_cache_flash_pe
 _ws_bytes_cache: dict = {}
 
 
-def paged_attn_workspace_bytes(max_num_seqs: int, num_q_heads: int, head_size: int) -> int:
-    """Host query (depends on the current device's CU count); answers are remembered per device."""
-    key = (torch.cuda.current_device() if torch.cuda.is_available() else -1, max_num_seqs, num_q_heads, head_size)
+def paged_attn_workspace_bytes(max_num_seqs: int, num_q_heads: int, head_size: int,
+                               device: torch.device | None = None) -> int:
+    """Host query (depends on the device's CU count); answers are remembered per device.
+    ``device`` defaults to the current one."""
+    if device is None or device.index is None:
+        idx = torch.cuda.current_device() if torch.cuda.is_available() else -1
+    else:
+        idx = device.index
+    key = (idx, max_num_seqs, num_q_heads, head_size)
     got = _ws_bytes_cache.get(key)
     if got is None:
-        got = int(_C.load().kvq_paged_attn_workspace_bytes(max_num_seqs, num_q_heads, head_size))
+        if idx >= 0 and idx != torch.cuda.current_device():
+            with torch.cuda.device(idx):
+                got = int(_C.load().kvq_paged_attn_workspace_bytes(max_num_seqs, num_q_heads, head_size))
+        else:
+            got = int(_C.load().kvq_paged_attn_workspace_bytes(max_num_seqs, num_q_heads, head_size))
         _ws_bytes_cache[key] = got
     return got
 
@@ -242,7 +259,7 @@ def unified_attention(
         return
     num_q_heads = q.shape[1]
     lib = _C.load()
-    need = paged_attn_workspace_bytes(num_seqs, num_q_heads, geom.head_size)
+    need = paged_attn_workspace_bytes(num_seqs, num_q_heads, geom.head_size, dev)
     if workspace is None:
         workspace = _default_workspace(dev, need)
     if lse is not None and (lse.dtype != torch.float32 or not lse.is_contiguous()
