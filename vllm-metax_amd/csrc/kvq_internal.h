@@ -71,6 +71,37 @@ __device__ __forceinline__ float wave_max(float v) {
   for (int o = 32; o >= 1; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, kWave));
   return v;
 }
+// Reductions over the four lanes l, l ^ 16, l ^ 32, l ^ 48 (one lane of each quarter-wave), result in
+// all four: two register swaps (v_permlane32_swap / v_permlane16_swap exchange half-waves / odd and
+// even rows of 16 between two registers), no trip through LDS.  The instruction swaps between TWO
+// registers; the empty asm keeps the compiler from handing it one register twice for equal values.
+__device__ __forceinline__ void swap_halves(uint32_t x, bool rows16, uint32_t& a, uint32_t& b) {
+  uint32_t y = x;
+  asm volatile("" : "+v"(y));
+  if (rows16) {
+    auto r = __builtin_amdgcn_permlane16_swap(x, y, false, false);
+    a = r[0];
+    b = r[1];
+  } else {
+    auto r = __builtin_amdgcn_permlane32_swap(x, y, false, false);
+    a = r[0];
+    b = r[1];
+  }
+}
+__device__ __forceinline__ float max_over_quarters(float v) {
+  uint32_t a, b;
+  swap_halves(__builtin_bit_cast(uint32_t, v), false, a, b);
+  v = fmaxf(__builtin_bit_cast(float, a), __builtin_bit_cast(float, b));
+  swap_halves(__builtin_bit_cast(uint32_t, v), true, a, b);
+  return fmaxf(__builtin_bit_cast(float, a), __builtin_bit_cast(float, b));
+}
+__device__ __forceinline__ float sum_over_quarters(float v) {
+  uint32_t a, b;
+  swap_halves(__builtin_bit_cast(uint32_t, v), false, a, b);
+  v = __builtin_bit_cast(float, a) + __builtin_bit_cast(float, b);
+  swap_halves(__builtin_bit_cast(uint32_t, v), true, a, b);
+  return __builtin_bit_cast(float, a) + __builtin_bit_cast(float, b);
+}
 // Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits for every global
 // load in flight (vmcnt(0)), which would drain the tile prefetch issued just before it; here the
 // loads stay in flight and the compiler's own wait before their first use still applies.

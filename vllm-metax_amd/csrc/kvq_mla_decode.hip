@@ -20,14 +20,15 @@
 // (same two-stage shape as the reference's decode_attention_fwd); nothing is allocated here,
 // partials and the int8 Q live in the caller's workspace.
 #include <atomic>
+#include <type_traits>
 
 #include "kvq_attn_core.cuh"
 
 namespace kvq {
 
 constexpr int kMlaR = 512, kMlaP = 64, kMlaW = kMlaR + kMlaP;
-constexpr int kMlaPitch = kMlaW + 16;                     // LDS row pitch: 16-byte aligned rows
-constexpr int kMlaTileBytes = kTile * kMlaPitch;          // 32 rows
+constexpr int kMlaPitch = kMlaW;                          // LDS rows are packed; the 16-byte chunks of a row are swizzled
+constexpr int kMlaTileBytes = kTile * kMlaPitch;          // 32 rows = 1152 chunks
 constexpr int kMlaBufBytes = kMlaTileBytes + 2 * kTile * 4;  // + 32 K-side and 32 V-side scales
 constexpr int kMlaKSteps = kMlaW / 32;                    // 18
 constexpr int kMlaDT = kMlaR / 16;                        // 32 output row tiles of 16 dims
@@ -37,12 +38,18 @@ constexpr int kChunksPerHalf = 16 * kChunksPerRow;        // 576
 constexpr int kMlaThreads = 512;
 constexpr int kMlaKSteps8 = kMlaW / 64;                   // 9 int8 k-steps of 64 dims
 constexpr int kMlaQOps = 2 * kMlaKSteps8;                 // B operands of Q: two int8 terms per k-step
-constexpr int kMlaQRegOps = 8;                            // operands of Q kept in registers; the rest in LDS
-constexpr int kMlaQLdsBytes = (kMlaQOps - kMlaQRegOps) * kMlaThreads * 16;  // 81920
-constexpr int kMlaVtPitch = 2 * kTile + 16;               // fp16 V^T row: 32 tokens (+ pad: conflict-free operand reads)
-constexpr int kMlaVtBytes = kMlaR * kMlaVtPitch;          // 40960
+constexpr int kMlaQRegOps = 10;                           // operands of Q kept in registers; the rest in LDS
+constexpr int kMlaQLdsBytes = (kMlaQOps - kMlaQRegOps) * kMlaThreads * 16;  // 65536
+constexpr int kMlaVtPitch = 2 * kTile;                    // fp16 V^T row: 32 tokens = 4 chunks of 16 bytes, swizzled
+constexpr int kMlaVtBytes = kMlaR * kMlaVtPitch;          // 32768
 typedef int32_t i32x4 __attribute__((ext_vector_type(4)));
-constexpr int kMlaLdsBytes = 2 * kMlaBufBytes + kMlaVtBytes + kMlaQLdsBytes;                  // 153088 of 163840
+constexpr float kMlaLazy = 8.0f;       // log2 of how far a logit may exceed the reference maximum
+constexpr float kMlaLazyVs = 255.0f;   // largest V-side scale (already times 2^8) with which 2^kMlaLazy * scale stays in fp16
+// What the head-owning waves hand to the others, per tile and double-buffered: the eight P~ operands
+// (64 lanes x 16 bytes each), one rescale factor per head and one "running max moved" byte per wave.
+constexpr int kMlaPBytes = 8 * kWave * 16;                // 8192
+constexpr int kMlaXchgBytes = kMlaPBytes + 128 * 4 + 16;  // 8720
+constexpr int kMlaLdsBytes = 2 * kMlaBufBytes + kMlaVtBytes + kMlaQLdsBytes + 2 * kMlaXchgBytes;  // 153120 of 163840
 
 struct MlaArgs {
   const void* q;
@@ -181,46 +188,55 @@ __global__ __launch_bounds__(256) void mla_quant_q_kernel(MlaArgs a) {
   if (wave == 0 && g == 0) a.q_scale[qblock * 16 + c] = s1;
 }
 
+// FULL: every 128-head block of the launch has its eight head tiles (num_heads a multiple of 128)
+template <bool FULL>
 __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
   extern __shared__ __align__(16) uint8_t lds_raw[];
   uint8_t(*lds)[kMlaBufBytes] = reinterpret_cast<uint8_t(*)[kMlaBufBytes]>(lds_raw);
+  uint8_t* vt = lds_raw + 2 * kMlaBufBytes;  // fp16 V^T of the current tile; rows 64 w .. 64 w + 63 belong to wave w
   // B operands of Q from number kMlaQRegOps on: slot [operand][thread], written and read by the same lane
-  uint8_t* vt = lds_raw + 2 * kMlaBufBytes;  // fp16 V^T of the current tile
   u32x4* qlds = reinterpret_cast<u32x4*>(lds_raw + 2 * kMlaBufBytes + kMlaVtBytes) + threadIdx.x;
+  uint8_t* xchg = lds_raw + 2 * kMlaBufBytes + kMlaVtBytes + kMlaQLdsBytes;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int c = lane & 15, g = lane >> 4;
   const int seq = blockIdx.y, split = blockIdx.x;
-  const int hbase = blockIdx.z * 128 + wave * 16;
   const int len = a.seq_lens[seq];
   const int slen = mla_split_len(len > 0 ? len : 0, a.num_splits);
   const int tok_begin = split * slen;
   const int tok_end = min(len, tok_begin + slen);
-  const bool head_ok = (hbase + c) < a.num_heads;
+  // head tiles (16 heads each) of this workgroup's 128-head block; wave w < nht owns tile w: it
+  // computes that tile's logits and softmax.  EVERY wave accumulates the outputs of all nht tiles,
+  // for its own 64 of the 512 dims.
+  const int nht = FULL ? 8 : min(8, a.head_groups - (int)blockIdx.z * 8);
   const int hgroup = blockIdx.z * 8 + wave;
-  const bool wave_ok = hgroup < a.head_groups;    // wave-uniform: this wave owns at least one head
-  const int64_t pblock = ((int64_t)seq * a.num_splits + split) * a.head_groups + hgroup;
+  const bool owner = wave < nht;                  // wave-uniform
+  const int64_t pblock0 = ((int64_t)seq * a.num_splits + split) * a.head_groups + blockIdx.z * 8;
   if (tok_begin >= tok_end) {  // empty split (uniform over the workgroup): mark it and leave
-    if (wave_ok && g == 0) a.part_lse[pblock * 16 + c] = -INFINITY;
+    if (owner && g == 0) a.part_lse[(pblock0 + wave) * 16 + c] = -INFINITY;
     return;
   }
   const int t_begin = tok_begin / kTile, t_end = (tok_end + kTile - 1) / kTile;
   const int bs = a.g.block_size;
   const int32_t* bt_row = a.block_table + (int64_t)seq * a.bt_stride;
 
-  // ---- cooperative tile load: thread tid takes chunk tid (and tid + 512 for tid < 64) of each
-  //      16-row half; 36 consecutive threads cover one 576-byte row
-  uint32_t goff[2], loff[2];
+  // ---- cooperative tile load, straight from global memory into LDS (no registers in between): a
+  //      wave's load instruction fills 1024 contiguous LDS bytes, lane i the 16-byte slot i, with
+  //      whatever global chunk the lane names.  Slot s of a 16-row half holds row s / 36, chunk
+  //      (s % 36) ^ swizzle(row) of that row (the two low bits of the chunk number xor bits 1..2 of
+  //      the row), so the rows need no padding for conflict-free operand reads: with 16 lanes reading
+  //      the same k-chunk of 16 consecutive rows, this swizzle measures free of bank conflicts, row
+  //      padding and the other two-bit swizzles cost every such read twice its cycles.  Thread tid
+  //      names the chunk of slot tid; the first wave also names slots 512 .. 575.
+  uint32_t goff[2];
 #pragma unroll
   for (int n = 0; n < 2; ++n) {
-    const int qi = tid + kMlaThreads * n;
-    const int row = qi / kChunksPerRow, col = qi % kChunksPerRow;
+    const int slot = n == 0 ? tid : kMlaThreads + lane;
+    const int row = slot / kChunksPerRow, pos = slot % kChunksPerRow;
+    const int col = (pos & ~3) | ((pos & 3) ^ ((row >> 1) & 3));
     goff[n] = (uint32_t)(row * a.g.stride_row + 16 * col);
-    loff[n] = (uint32_t)(row * kMlaPitch + 16 * col);
   }
-  const bool second = tid < kChunksPerHalf - kMlaThreads;
-  u32x4 cr[2][2];
   uint32_t scr[2];
   // Block ids of the two 16-token halves of tile t (scalar loads); a half past the end of the
   // sequence rereads its last valid half and is masked in the softmax.
@@ -240,7 +256,8 @@ __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
     }
     return r;
   };
-  auto issue_loads = [&](const Blocks& nb) __attribute__((always_inline)) {
+  typedef __attribute__((address_space(3))) void* lds_ptr_t;
+  auto issue_loads = [&](const Blocks& nb, uint8_t* buf) __attribute__((always_inline)) {
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
       const uint8_t* pb = a.cache + (int64_t)nb.b[h] * a.g.stride_block;
@@ -248,35 +265,38 @@ __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
           const_cast<uint8_t*>(pb + (int64_t)nb.s[h] * a.g.stride_row), 0, 0x7fffffff, 0x00020000);
       const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
           const_cast<uint8_t*>(pb + a.g.scale_off + (int64_t)nb.s[h] * 4), 0, 0x7fffffff, 0x00020000);
-      cr[h][0] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rr, goff[0], 0, 0));
-      if (second) cr[h][1] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rr, goff[1], 0, 0));
+      uint8_t* hb = buf + h * (kChunksPerHalf * 16);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rr, (lds_ptr_t)(hb + wave * (kWave * 16)), 16, goff[0], 0, 0, 0);
+      if (wave == 0)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rr, (lds_ptr_t)(hb + kMlaThreads * 16), 16, goff[1], 0, 0, 0);
       scr[h] = __builtin_amdgcn_raw_buffer_load_b32(rs, (uint32_t)((tid & 15) * 4), 0, 0);
     }
   };
-  auto stage = [&](uint8_t* buf) {
+  auto stage_scales = [&](uint8_t* buf) {
+    if (tid < 16) {
+      float* sc = reinterpret_cast<float*>(buf + kMlaTileBytes);
 #pragma unroll
-    for (int h = 0; h < 2; ++h) {
-      uint8_t* hb = buf + h * 16 * kMlaPitch;
-      *reinterpret_cast<u32x4*>(hb + loff[0]) = cr[h][0];
-      if (second) *reinterpret_cast<u32x4*>(hb + loff[1]) = cr[h][1];
-      if (tid < 16) {
-        float* sc = reinterpret_cast<float*>(buf + kMlaTileBytes);
+      for (int h = 0; h < 2; ++h) {
         const float v = as_f32(scr[h]);
         sc[h * 16 + tid] = v * a.scale_log2;                       // K side: scale * log2e folded in
         sc[kTile + h * 16 + tid] = fminf(v * kPScale, 65504.f);    // V side: 2^8, capped
       }
     }
   };
+  // Barrier that also waits for this wave's loads into LDS (they count as vector memory loads).
+  auto tile_barrier = [&]() __attribute__((always_inline)) {
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+  };
 
-  issue_loads(fetch_blocks(t_begin));
+  issue_loads(fetch_blocks(t_begin), lds[0]);
   Blocks nb = fetch_blocks(t_begin + 1);
 
-  // ---- absorbed Q of this wave's 16 heads: the int8 B operands mla_quant_q_kernel prepared (operand
-  //      2 kk = first term, 2 kk + 1 = second term of k-step kk; lane (c = head, g) holds dims
-  //      64 kk + 16 g + j)
+  // ---- absorbed Q of the 16 heads this wave owns: the int8 B operands mla_quant_q_kernel prepared
+  //      (operand 2 kk = first term, 2 kk + 1 = second term of k-step kk; lane (c = head, g) holds
+  //      dims 64 kk + 16 g + j)
   i32x4 qreg[kMlaQRegOps];
   float s1 = 1.f, s2 = 0.f;
-  if (wave_ok) {
+  if (owner) {
     const int64_t qblock = (int64_t)seq * a.head_groups + hgroup;
     const u32x4* qsrc = reinterpret_cast<const u32x4*>(a.q_ops + qblock * (kMlaQOps * kWave * 16)) + lane;
     u32x4 raw[kMlaQOps];
@@ -291,34 +311,42 @@ __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
     }
   } else {
 #pragma unroll
-    for (int op = 0; op < kMlaQOps; ++op) {
-      if (op < kMlaQRegOps) qreg[op] = (i32x4){0, 0, 0, 0};
-      else qlds[(op - kMlaQRegOps) * kMlaThreads] = (u32x4){0u, 0u, 0u, 0u};
-    }
+    for (int op = 0; op < kMlaQRegOps; ++op) qreg[op] = (i32x4){0, 0, 0, 0};
   }
 
-  floatx4 o[kMlaDT];
+  // o[ht][b][i]: head 16 ht + c, dim 64 wave + 16 g + 4 i + b
+  floatx4 o[8][4];
 #pragma unroll
-  for (int dt = 0; dt < kMlaDT; ++dt) o[dt] = (floatx4){0.f, 0.f, 0.f, 0.f};
+  for (int ht = 0; ht < 8; ++ht)
+#pragma unroll
+    for (int b = 0; b < 4; ++b) o[ht][b] = (floatx4){0.f, 0.f, 0.f, 0.f};
   float m = -INFINITY, l = 0.f;
 
-  // ---- V^T of the tile as fp16, made ONCE per workgroup: wave v transposes dims 64 v .. 64 v + 63.
+  // ---- V^T of the tile as fp16: wave v transposes dims 64 v .. 64 v + 63, the dims whose outputs
+  //      it accumulates, so this part of LDS is private to the wave (no barrier guards it).
   //      A thread takes, twice, a block of 4 tokens x 4 dims (one dword per token row), transposes it
   //      with byte permutes and writes, for each of the 4 dims, the 4 tokens' plain codes as fp16 (8
   //      bytes).  Dim 64 w + 4 r' + b sits in row (4 w + b) * 16 + r' -- row r' of output tile 4 w + b --
   //      and token 16 mt + 4 g' + i at position 8 g' + 4 mt + i, the order in which a lane of the P~
-  //      operand holds its 8 tokens.  Lanes = 8 consecutive rows x 8 token groups: the 8-byte writes
-  //      of a wave spread evenly over the LDS banks.
+  //      operand holds its 8 tokens; the four 16-byte chunks of a row are swizzled with bits 1..2 of
+  //      the row like the raw tile's.  Lanes = 8 consecutive rows x 8 token groups.
   const int tr = lane & 7, tq = lane >> 3;
-  const uint32_t vt_src = (uint32_t)(4 * tq * kMlaPitch + 4 * (16 * wave + tr));
-  const uint32_t vt_dst = (uint32_t)((64 * wave + tr) * kMlaVtPitch + 2 * (8 * (tq & 3) + 4 * (tq >> 2)));
+  // dword of dims 64 wave + 4 tr + 32 u .. + 3 in row 4 tq + r: chunk 4 wave + 2 u + (tr >> 2), swizzled with
+  // bits 1..2 of the row, which r >> 1 takes part in
+  uint32_t vt_src[2][2];
+#pragma unroll
+  for (int u = 0; u < 2; ++u)
+#pragma unroll
+    for (int rh = 0; rh < 2; ++rh)
+      vt_src[u][rh] = (uint32_t)(4 * tq * kMlaPitch + 16 * (4 * wave + ((2 * u + (tr >> 2)) ^ ((2 * tq + rh) & 3))) + 4 * (tr & 3));
+  const uint32_t vt_dst = (uint32_t)((64 * wave + tr) * kMlaVtPitch + 16 * ((tq & 3) ^ ((tr >> 1) & 3)) + 8 * (tq >> 2));
   auto transpose_v = [&](const uint8_t* tile) __attribute__((always_inline)) {
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
       uint32_t x[4];
 #pragma unroll
       for (int r = 0; r < 4; ++r)
-        x[r] = *reinterpret_cast<const uint32_t*>(tile + vt_src + r * kMlaPitch + 32 * u) ^ 0x80808080u;
+        x[r] = *reinterpret_cast<const uint32_t*>(tile + vt_src[u][r >> 1] + r * kMlaPitch) ^ 0x80808080u;
       const uint32_t a01 = perm(x[1], x[0], 0x05010400u), b01 = perm(x[1], x[0], 0x07030602u);
       const uint32_t a23 = perm(x[3], x[2], 0x05010400u), b23 = perm(x[3], x[2], 0x07030602u);
 #pragma unroll
@@ -331,125 +359,205 @@ __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
     }
   };
 
-  stage(lds[0]);
-  issue_loads(nb);  // unconditional: past the split's end it rereads a valid half that is never used
+  stage_scales(lds[0]);
+  // every load so far (Q operands, the first tile) has landed; said with the builtin so that the
+  // compiler knows it too and does not wait for loads again inside the loop, where a wait for
+  // "all loads" would also wait for the tile prefetch in flight
+  __builtin_amdgcn_s_waitcnt(0x0f70);   // vmcnt(0)
+  if (t_begin + 1 < t_end) issue_loads(nb, lds[1]);
+  nb = fetch_blocks(t_begin + 2);
   lds_barrier();
-  nb = fetch_blocks(t_begin + 2);  // after the barrier, whose wait would otherwise expose these scalar loads
 
+  const uint32_t ka_off = (uint32_t)(c * kMlaPitch + 16 * (g ^ ((c >> 1) & 3)));   // row c, chunk g of a k-step, swizzled
   int buf = 0;
   for (int t = t_begin; t < t_end; ++t) {
     const uint8_t* tile = lds[buf];
     const float* sck = reinterpret_cast<const float*>(tile + kMlaTileBytes);
+    uint8_t* xb = xchg + buf * kMlaXchgBytes;         // this tile's P~ operands, rescale factors, flags
+    float* x_alpha = reinterpret_cast<float*>(xb + kMlaPBytes);
+    uint8_t* x_flag = xb + kMlaPBytes + 128 * 4;
     transpose_v(tile);
 
-    // ---- S^T[32 tokens, 16 heads] on the int8 MFMA: A = the cached code bytes as they are, lane
-    //      (r = token, g): dims 64 kk + 16 g ..; one accumulator per term of Q
-    i32x4 acc[2][2];
+    if (owner) {
+      // ---- S^T[32 tokens, 16 heads] on the int8 MFMA: A = the cached code bytes as they are, lane
+      //      (r = token, g): dims 64 kk + 16 g ..; one accumulator per term of Q
+      i32x4 acc[2][2];
 #pragma unroll
-    for (int term = 0; term < 2; ++term)
+      for (int term = 0; term < 2; ++term)
 #pragma unroll
-      for (int mt = 0; mt < 2; ++mt) acc[term][mt] = (i32x4){0, 0, 0, 0};
+        for (int mt = 0; mt < 2; ++mt) acc[term][mt] = (i32x4){0, 0, 0, 0};
+      // the operands of k-step kk + 1 are fetched before the products of k-step kk are issued;
+      // the fences hold the compiler to that order
+      const uint8_t* kap = tile + ka_off;
+      i32x4 ka[2][2], ql[2][2];
+      ka[0][0] = *reinterpret_cast<const i32x4*>(kap);
+      ka[0][1] = *reinterpret_cast<const i32x4*>(kap + 16 * kMlaPitch);
 #pragma unroll
-    for (int kk = 0; kk < kMlaKSteps8; ++kk) {
-      i32x4 qa, qb8;
-      if (2 * kk < kMlaQRegOps) {
-        qa = qreg[2 * kk];
-        qb8 = qreg[2 * kk + 1];
-      } else {
-        qa = __builtin_bit_cast(i32x4, qlds[(2 * kk - kMlaQRegOps) * kMlaThreads]);
-        qb8 = __builtin_bit_cast(i32x4, qlds[(2 * kk + 1 - kMlaQRegOps) * kMlaThreads]);
+      for (int kk = 0; kk < kMlaKSteps8; ++kk) {
+        const int cur = kk & 1, nxt = cur ^ 1;
+        if (kk + 1 < kMlaKSteps8) {
+          ka[nxt][0] = *reinterpret_cast<const i32x4*>(kap + 64 * (kk + 1));
+          ka[nxt][1] = *reinterpret_cast<const i32x4*>(kap + 16 * kMlaPitch + 64 * (kk + 1));
+          if (2 * (kk + 1) >= kMlaQRegOps) {
+            ql[nxt][0] = __builtin_bit_cast(i32x4, qlds[(2 * (kk + 1) - kMlaQRegOps) * kMlaThreads]);
+            ql[nxt][1] = __builtin_bit_cast(i32x4, qlds[(2 * (kk + 1) + 1 - kMlaQRegOps) * kMlaThreads]);
+          }
+        }
+        const i32x4 qa = 2 * kk < kMlaQRegOps ? qreg[2 * kk < kMlaQRegOps ? 2 * kk : 0] : ql[cur][0];
+        const i32x4 qb8 = 2 * kk < kMlaQRegOps ? qreg[2 * kk < kMlaQRegOps ? 2 * kk + 1 : 0] : ql[cur][1];
+#pragma unroll
+        for (int mt = 0; mt < 2; ++mt) {
+          acc[0][mt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(ka[cur][mt], qa, acc[0][mt], 0, 0, 0);
+          acc[1][mt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(ka[cur][mt], qb8, acc[1][mt], 0, 0, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
       }
+
+      // ---- softmax, log2 domain; lane (c, g) holds tokens mt*16 + 4g + i of head c.  Only a split's
+      //      last tile can hold tokens past its end: every other tile takes the path without masks.
+      auto softmax = [&](auto masked_tag) __attribute__((always_inline)) {
+        constexpr bool MASKED = decltype(masked_tag)::value;
+        float logit[8];
+        float mloc = -INFINITY;
 #pragma unroll
-      for (int mt = 0; mt < 2; ++mt) {
-        const i32x4 ka = *reinterpret_cast<const i32x4*>(tile + (mt * 16 + c) * kMlaPitch + 64 * kk + 16 * g);
-        acc[0][mt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(ka, qa, acc[0][mt], 0, 0, 0);
-        acc[1][mt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(ka, qb8, acc[1][mt], 0, 0, 0);
-      }
+        for (int mt = 0; mt < 2; ++mt) {
+          const floatx4 ks = *reinterpret_cast<const floatx4*>(sck + 16 * mt + 4 * g);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            float x = __builtin_fmaf((float)acc[1][mt][i], s2, (float)acc[0][mt][i] * s1) * ks[i];
+            if constexpr (MASKED) x = t * kTile + 16 * mt + 4 * g + i < tok_end ? x : -INFINITY;
+            logit[4 * mt + i] = x;
+            mloc = fmaxf(mloc, x);
+          }
+        }
+        mloc = max_over_quarters(mloc);
+        // The reference maximum m of a head only has to keep 2^(logit - m) in range, it need not be the
+        // true maximum: it moves when some head of the tile outgrows it by more than 2^kMlaLazy (or at
+        // all, when a token's value scale is so large that p * scale could leave the fp16 range
+        // otherwise).  Moving m rescales what is accumulated so far, and the accumulators of these
+        // heads are spread over all waves, so the factors travel with the tile; with i.i.d. logits the
+        // true maximum moves in most of a split's first dozen tiles, the lazy one a few times.
+        floatx4 vs[2];
+#pragma unroll
+        for (int mt = 0; mt < 2; ++mt) vs[mt] = *reinterpret_cast<const floatx4*>(sck + kTile + 16 * mt + 4 * g);
+        const float vsmax = fmaxf(fmaxf(fmaxf(vs[0].x, vs[0].y), fmaxf(vs[0].z, vs[0].w)),
+                                  fmaxf(fmaxf(vs[1].x, vs[1].y), fmaxf(vs[1].z, vs[1].w)));
+        const float lim = vsmax > kMlaLazyVs ? m : m + kMlaLazy;
+        const bool moved = __builtin_amdgcn_ballot_w64(mloc > lim) != 0;
+        if (moved) {
+          const float m_new = fmaxf(m, mloc);
+          const float alpha = __builtin_amdgcn_exp2f(m - m_new);
+          m = m_new;
+          l *= alpha;
+          if (g == 0) x_alpha[wave * 16 + c] = alpha;
+        }
+        if (lane == 0) x_flag[wave] = moved ? 1 : 0;
+        float pt[8];
+#pragma unroll
+        for (int mt = 0; mt < 2; ++mt) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const float p = __builtin_amdgcn_exp2f(logit[4 * mt + i] - m);   // 0 for a masked token
+            l += p;
+            pt[4 * mt + i] = p * vs[mt][i];
+            // a slot past the end may hold any bit pattern as its scale: select, do not multiply by 0
+            if constexpr (MASKED) pt[4 * mt + i] = t * kTile + 16 * mt + 4 * g + i < tok_end ? pt[4 * mt + i] : 0.f;
+          }
+        }
+        u32x4 pb;
+        pb.x = pack_half2(pt[0], pt[1]);
+        pb.y = pack_half2(pt[2], pt[3]);
+        pb.z = pack_half2(pt[4], pt[5]);
+        pb.w = pack_half2(pt[6], pt[7]);
+        reinterpret_cast<u32x4*>(xb)[wave * kWave + lane] = pb;
+      };
+      if ((t + 1) * kTile > tok_end) softmax(std::true_type{});
+      else softmax(std::false_type{});
     }
 
-    // ---- softmax, log2 domain; lane (c, g) holds tokens mt*16 + 4g + i of head c
-    float logit[8];
-    float mloc = -INFINITY;
-#pragma unroll
-    for (int mt = 0; mt < 2; ++mt) {
-      const floatx4 ks = *reinterpret_cast<const floatx4*>(sck + 16 * mt + 4 * g);
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int tok = t * kTile + 16 * mt + 4 * g + i;
-        float x = __builtin_fmaf((float)acc[1][mt][i], s2, (float)acc[0][mt][i] * s1) * ks[i];
-        x = tok < tok_end ? x : -INFINITY;
-        logit[4 * mt + i] = x;
-        mloc = fmaxf(mloc, x);
-      }
-    }
-    mloc = fmaxf(mloc, __shfl_xor(mloc, 16, kWave));
-    mloc = fmaxf(mloc, __shfl_xor(mloc, 32, kWave));
-    if (__builtin_amdgcn_ballot_w64(mloc > m) != 0) {
-      const float m_new = fmaxf(m, mloc);
-      const float alpha = __builtin_amdgcn_exp2f(m - m_new);
-      m = m_new;
-      l *= alpha;
-#pragma unroll
-      for (int dt = 0; dt < kMlaDT; ++dt) o[dt] *= alpha;
-    }
-    float pt[8];
-#pragma unroll
-    for (int mt = 0; mt < 2; ++mt) {
-      const floatx4 vs = *reinterpret_cast<const floatx4*>(sck + kTile + 16 * mt + 4 * g);
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int tok = t * kTile + 16 * mt + 4 * g + i;
-        const float p = __builtin_amdgcn_exp2f(logit[4 * mt + i] - m);
-        l += p;
-        pt[4 * mt + i] = tok < tok_end ? p * vs[i] : 0.f;
-      }
-    }
-    u32x4 pb;
-    pb.x = pack_half2(pt[0], pt[1]);
-    pb.y = pack_half2(pt[2], pt[3]);
-    pb.z = pack_half2(pt[4], pt[5]);
-    pb.w = pack_half2(pt[6], pt[7]);
-    const half8_t p_op = __builtin_bit_cast(half8_t, pb);
-
-    // the next tile goes into the other raw window (its last readers finished before the previous
-    // iteration's second barrier) and the loads of the tile after it are issued
-    if (t + 1 < t_end) {
-      stage(lds[buf ^ 1]);
-      issue_loads(nb);
-    }
-    lds_barrier();  // V^T of this tile (and the next raw tile) is visible to every wave
+    if (t + 1 < t_end) stage_scales(lds[buf ^ 1]);
+    // The ONE barrier of a tile (it also waits for this wave's part of the next raw tile): P~, the
+    // rescale factors and the next raw tile are visible to every wave.  The exchange area is double-buffered, so a wave that runs ahead into the next tile
+    // writes the other half while slower waves still read this one.
+    tile_barrier();
+    // this tile's raw window is free now (its readers are past the barrier): the tile after the next
+    // streams into it, a whole tile time ahead of its use
+    if (t + 2 < t_end) issue_loads(nb, lds[buf]);
     nb = fetch_blocks(t + 3);
 
-    // ---- O^T[512 dims, 16 heads] += C^T . P~^T: A = fp16 V^T rows, lane (r = row of output tile dt,
-    //      g): positions 8 g .. 8 g + 7
-    const uint8_t* vrow = vt + c * kMlaVtPitch + 16 * g;
+    // ---- O^T[64 dims of this wave, 128 heads] += C^T . P~^T: A = fp16 V^T rows, lane (r = row of
+    //      output tile 4 wave + b, g): positions 8 g .. 8 g + 7; B = head tile ht's P~ operand
+    const u32x2 flags = *reinterpret_cast<const u32x2*>(x_flag);
+    half8_t va[4];
 #pragma unroll
-    for (int dt = 0; dt < kMlaDT; ++dt) {
-      const half8_t va = *reinterpret_cast<const half8_t*>(vrow + dt * 16 * kMlaVtPitch);
-      o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va, p_op, o[dt], 0, 0, 0);
+    for (int b = 0; b < 4; ++b)
+      va[b] = *reinterpret_cast<const half8_t*>(vt + ((4 * wave + b) * 16 + c) * kMlaVtPitch + 16 * (g ^ ((c >> 1) & 3)));
+    // (FULL) operand ht + 3 is fetched while tile ht multiplies; the first three leave with the
+    // flags, before anything waits
+    const u32x4* pl = reinterpret_cast<const u32x4*>(xb) + lane;
+    u32x4 pq[8];
+    if constexpr (FULL) {
+      pq[0] = pl[0];
+      pq[1] = pl[kWave];
+      pq[2] = pl[2 * kWave];
     }
-    lds_barrier();  // every wave is done with V^T before the next tile's transposition overwrites it
+    const uint32_t f_lo = __builtin_amdgcn_readfirstlane(flags.x), f_hi = __builtin_amdgcn_readfirstlane(flags.y);
+    if ((f_lo | f_hi) != 0) {   // some running maximum moved: rare after a split's first tiles
+#pragma unroll
+      for (int ht = 0; ht < 8; ++ht) {
+        const uint32_t f = ((ht < 4 ? f_lo : f_hi) >> (8 * (ht & 3))) & 0xffu;
+        if (ht < nht && f != 0) {
+          const float alpha = x_alpha[ht * 16 + c];
+#pragma unroll
+          for (int b = 0; b < 4; ++b) o[ht][b] *= alpha;
+        }
+      }
+    }
+    if constexpr (FULL) {   // one straight run of 8 operand reads and 32 MFMAs
+      // the fences keep the compiler from hoisting all eight fetches (it would spill)
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int ht = 0; ht < 8; ++ht) {
+        if (ht + 3 < 8) pq[ht + 3] = pl[(ht + 3) * kWave];
+        const half8_t p_op = __builtin_bit_cast(half8_t, pq[ht]);
+#pragma unroll
+        for (int b = 0; b < 4; ++b) o[ht][b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va[b], p_op, o[ht][b], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    } else {
+#pragma unroll
+      for (int ht = 0; ht < 8; ++ht) {
+        if (ht < nht) {
+          const half8_t p_op = __builtin_bit_cast(half8_t, reinterpret_cast<const u32x4*>(xb)[ht * kWave + lane]);
+#pragma unroll
+          for (int b = 0; b < 4; ++b) o[ht][b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va[b], p_op, o[ht][b], 0, 0, 0);
+        }
+      }
+    }
     buf ^= 1;
   }
 
-  // ---- emit the split's state: locally normalised output and its log2-domain lse.
-  //      Lane (c, g) holds O[head c][dim 64 w + 16 g + 4 i + b] in o[4w + b][i].
-  l += __shfl_xor(l, 16, kWave);
-  l += __shfl_xor(l, 32, kWave);
-  if (!wave_ok) return;
-  const float inv = 1.0f / (l * kPScale);
-  uint16_t* po = a.part_o + pblock * (16 * kMlaR) + lane * 4;
+  // ---- emit the split's state: locally normalised output and its log2-domain lse.  The owners pass
+  //      1 / l of their heads to every wave through the exchange half the last tile did not use.
+  l = sum_over_quarters(l);
+  float* x_inv = reinterpret_cast<float*>(xchg + buf * kMlaXchgBytes + kMlaPBytes);
+  if (owner && g == 0) x_inv[wave * 16 + c] = 1.0f / (l * kPScale);
+  lds_barrier();
 #pragma unroll
-  for (int d4 = 0; d4 < kMlaDT / 4; ++d4) {
+  for (int ht = 0; ht < 8; ++ht) {
+    if (ht < nht) {
+      const float inv = x_inv[ht * 16 + c];
+      uint16_t* po = a.part_o + (pblock0 + ht) * (16 * kMlaR) + lane * 4 + wave * 4 * 256;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      u32x2 v;  // a locally normalised output is a convex mix of dequantised rows: within fp16 range
-      v.x = pack_half2(clamp_half_range(o[4 * d4 + 0][i] * inv), clamp_half_range(o[4 * d4 + 1][i] * inv));
-      v.y = pack_half2(clamp_half_range(o[4 * d4 + 2][i] * inv), clamp_half_range(o[4 * d4 + 3][i] * inv));
-      *reinterpret_cast<u32x2*>(po + (d4 * 4 + i) * 256) = v;
+      for (int i = 0; i < 4; ++i) {
+        u32x2 v;  // a locally normalised output is a convex mix of dequantised rows: within fp16 range
+        v.x = pack_half2(clamp_half_range(o[ht][0][i] * inv), clamp_half_range(o[ht][1][i] * inv));
+        v.y = pack_half2(clamp_half_range(o[ht][2][i] * inv), clamp_half_range(o[ht][3][i] * inv));
+        *reinterpret_cast<u32x2*>(po + i * 256) = v;
+      }
     }
   }
-  if (g == 0) a.part_lse[pblock * 16 + c] = m + __builtin_amdgcn_logf(l);
+  if (owner && g == 0) a.part_lse[(pblock0 + wave) * 16 + c] = m + __builtin_amdgcn_logf(l);
 }
 
 // Stage 2: out = sum_j 2^(lse_j - max) o_j / sum_j 2^(lse_j - max); lse = ln 2 * (max + log2 sum).
@@ -535,7 +643,11 @@ static int mla_prepare_device() {
   if (int e = check_hip(hipGetDevice(&dev), "hipGetDevice")) return e;
   const uint64_t bit = dev >= 0 && dev < 64 ? (1ull << dev) : 0;
   if (bit != 0 && (done_mask.load(std::memory_order_acquire) & bit)) return KVQ_OK;
-  if (int e = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(&mla_decode_kernel),
+  if (int e = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(&mla_decode_kernel<true>),
+                                            hipFuncAttributeMaxDynamicSharedMemorySize, kMlaLdsBytes),
+                        "hipFuncSetAttribute(mla_decode_kernel)"))
+    return e;
+  if (int e = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(&mla_decode_kernel<false>),
                                             hipFuncAttributeMaxDynamicSharedMemorySize, kMlaLdsBytes),
                         "hipFuncSetAttribute(mla_decode_kernel)"))
     return e;
@@ -619,7 +731,10 @@ int kvq_mla_decode_int8(void* out, int out_dtype, float* lse, const void* q, int
   }
 #undef KVQ_MLAQ
   if (int e = check_hip(hipGetLastError(), "mla_decode_int8 query launch")) return e;
-  hipLaunchKernelGGL(mla_decode_kernel, grid, dim3(kMlaThreads), kMlaLdsBytes, s, a);
+  if (head_groups % 8 == 0)
+    hipLaunchKernelGGL(mla_decode_kernel<true>, grid, dim3(kMlaThreads), kMlaLdsBytes, s, a);
+  else
+    hipLaunchKernelGGL(mla_decode_kernel<false>, grid, dim3(kMlaThreads), kMlaLdsBytes, s, a);
   int rc = check_hip(hipGetLastError(), "mla_decode_int8 launch");
   if (rc) return rc;
   dim3 rgrid(num_seqs, head_groups);
