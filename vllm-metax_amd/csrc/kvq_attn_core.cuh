@@ -353,8 +353,7 @@ struct DecodeTile {
         mloc = fmaxf(mloc, x);
       }
     }
-    mloc = fmaxf(mloc, __shfl_xor(mloc, 16, kWave));
-    mloc = fmaxf(mloc, __shfl_xor(mloc, 32, kWave));
+    mloc = max_over_quarters(mloc);
     if (__builtin_amdgcn_ballot_w64(mloc > st.m) != 0) {  // rescale only when some head's max moved
       const float m_new = fmaxf(st.m, mloc);
       const float alpha = __builtin_amdgcn_exp2f(st.m - m_new);  // st.m = -inf -> 0

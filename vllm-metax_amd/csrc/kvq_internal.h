@@ -95,6 +95,12 @@ __device__ __forceinline__ float max_over_quarters(float v) {
   swap_halves(__builtin_bit_cast(uint32_t, v), true, a, b);
   return fmaxf(__builtin_bit_cast(float, a), __builtin_bit_cast(float, b));
 }
+// the same over the two lanes l, l ^ 32
+__device__ __forceinline__ float max_over_halves(float v) {
+  uint32_t a, b;
+  swap_halves(__builtin_bit_cast(uint32_t, v), false, a, b);
+  return fmaxf(__builtin_bit_cast(float, a), __builtin_bit_cast(float, b));
+}
 __device__ __forceinline__ float sum_over_quarters(float v) {
   uint32_t a, b;
   swap_halves(__builtin_bit_cast(uint32_t, v), false, a, b);

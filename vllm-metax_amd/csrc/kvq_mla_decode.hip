@@ -341,14 +341,18 @@ __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
       vt_src[u][rh] = (uint32_t)(4 * tq * kMlaPitch + 16 * (4 * wave + ((2 * u + (tr >> 2)) ^ ((2 * tq + rh) & 3))) + 4 * (tr & 3));
   const uint32_t vt_dst = (uint32_t)((64 * wave + tr) * kMlaVtPitch + 16 * ((tq & 3) ^ ((tr >> 1) & 3)) + 8 * (tq >> 2));
   auto transpose_v = [&](const uint8_t* tile) __attribute__((always_inline)) {
+    uint32_t x[2][4];   // all eight reads leave before the first permute waits
 #pragma unroll
-    for (int u = 0; u < 2; ++u) {
-      uint32_t x[4];
+    for (int u = 0; u < 2; ++u)
 #pragma unroll
       for (int r = 0; r < 4; ++r)
-        x[r] = *reinterpret_cast<const uint32_t*>(tile + vt_src[u][r >> 1] + r * kMlaPitch) ^ 0x80808080u;
-      const uint32_t a01 = perm(x[1], x[0], 0x05010400u), b01 = perm(x[1], x[0], 0x07030602u);
-      const uint32_t a23 = perm(x[3], x[2], 0x05010400u), b23 = perm(x[3], x[2], 0x07030602u);
+        x[u][r] = *reinterpret_cast<const uint32_t*>(tile + vt_src[u][r >> 1] + r * kMlaPitch);
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) x[u][r] ^= 0x80808080u;
+      const uint32_t a01 = perm(x[u][1], x[u][0], 0x05010400u), b01 = perm(x[u][1], x[u][0], 0x07030602u);
+      const uint32_t a23 = perm(x[u][3], x[u][2], 0x05010400u), b23 = perm(x[u][3], x[u][2], 0x07030602u);
 #pragma unroll
       for (int b = 0; b < 4; ++b) {
         u32x2 h;

@@ -94,8 +94,7 @@ struct PrefillTile {
           mloc = fmaxf(mloc, x);
         }
       }
-      mloc = fmaxf(mloc, __shfl_xor(mloc, 16, kWave));
-      mloc = fmaxf(mloc, __shfl_xor(mloc, 32, kWave));
+      mloc = max_over_quarters(mloc);
       const float m_new = fmaxf(st.m[nt], mloc);
       // a column that has seen no visible token yet keeps m = -inf; exponents are then taken
       // against 0 so that they come out as exp2(-inf) = 0 and never as (-inf) - (-inf)
@@ -509,7 +508,7 @@ struct Flash32 {
         d = fmaxf(d, y);
       }
     }
-    d = fmaxf(d, __shfl_xor(d, 32, kWave));
+    d = max_over_halves(d);
     // how far the maximum moves: a fresh column takes d itself (0 while it still sees nothing)
     const float up = fresh ? (d == -INFINITY ? 0.f : d) : fmaxf(d, 0.f);
     if (__builtin_amdgcn_ballot_w64(up != 0.f) != 0) {
