@@ -307,8 +307,8 @@ KVQ_API size_t kvq_mla_decode_workspace_bytes(int max_num_seqs, int num_heads, i
  * lse, block_table, seq_lens, attn_logits, num_kv_splits, sm_scale, page_size,
  * ..., is_mla=True), vllm_metax/v1/attention/backends/mla/triton_mla.py:226-295,
  * vllm_metax/v1/attention/ops/triton_decode_attention.py:763-825.
- * q [B, H, kv_lora_rank + rope_dim] (absorbed), out [B, H, kv_lora_rank],
- * lse [B, H] fp32 natural log (may be NULL).
+ * q [B, H, kv_lora_rank + rope_dim] (absorbed), out [B, H, kv_lora_rank]
+ * contiguous and 16-byte aligned, lse [B, H] fp32 natural log (may be NULL).
  */
 KVQ_API int kvq_mla_decode_int8(void* out, int out_dtype, float* lse, const void* q, int q_dtype,
                         int64_t q_stride_b, int64_t q_stride_h, const void* cache,

@@ -616,11 +616,21 @@ __global__ __launch_bounds__(512) void mla_reduce_kernel(void* out, float* lse, 
   const int64_t obase = ((int64_t)seq * num_heads + head) * kMlaR + 16 * g;
 #pragma unroll
   for (int r = 0; r < 4; ++r) {
-    const int64_t o = obase + 64 * wave + 4 * r;
-    store_act<ODT>(out, o + 0, acc[r].x * inv);
-    store_act<ODT>(out, o + 1, acc[r].y * inv);
-    store_act<ODT>(out, o + 2, acc[r].z * inv);
-    store_act<ODT>(out, o + 3, acc[r].w * inv);
+    const int64_t o = obase + 64 * wave + 4 * r;   // four consecutive dims: one store (rows are 1024 elements apart)
+    const floatx4 v = acc[r] * inv;
+    if constexpr (ODT == KVQ_F32) {
+      *reinterpret_cast<floatx4*>(reinterpret_cast<float*>(out) + o) = v;
+    } else if constexpr (ODT == KVQ_BF16) {
+      u32x2 w;
+      w.x = (uint32_t)f32_to_bf16_bits(v.x) | ((uint32_t)f32_to_bf16_bits(v.y) << 16);
+      w.y = (uint32_t)f32_to_bf16_bits(v.z) | ((uint32_t)f32_to_bf16_bits(v.w) << 16);
+      *reinterpret_cast<u32x2*>(reinterpret_cast<uint16_t*>(out) + o) = w;
+    } else {
+      u32x2 w;
+      w.x = pack_half2(v.x, v.y);
+      w.y = pack_half2(v.z, v.w);
+      *reinterpret_cast<u32x2*>(reinterpret_cast<uint16_t*>(out) + o) = w;
+    }
   }
   if (lse != nullptr && wave == 0 && g == 0)
     lse[(int64_t)seq * num_heads + head] = den > 0.f ? (mx + __builtin_amdgcn_logf(den)) * kLn2 : -INFINITY;
@@ -686,6 +696,7 @@ int kvq_mla_decode_int8(void* out, int out_dtype, float* lse, const void* q, int
   KVQ_REQUIRE(geom != nullptr, "%s: geom is NULL", op);
   KVQ_REQUIRE(out && q && cache && block_table && seq_lens, "%s: NULL pointer", op);
   KVQ_REQUIRE(num_seqs > 0 && num_seqs <= 65535 && num_heads > 0, "%s: num_seqs / num_heads out of range", op);
+  KVQ_REQUIRE(((uintptr_t)out % 16) == 0, "%s: out must be 16-byte aligned", op);
   const kvq_mla_geom& g = *geom;
   KVQ_REQUIRE(g.kv_lora_rank == kMlaR && g.rope_dim == kMlaP,
               "%s: only kv_lora_rank 512 + rope 64 is built (got %d + %d)", op, g.kv_lora_rank, g.rope_dim);
