@@ -26,6 +26,8 @@ namespace kvq {
 constexpr int kTile = 32;            // tokens per step
 constexpr int kSyncTiles = 2;        // workgroup rendezvous period of the decode stream, in tiles (power of two)
 constexpr float kPScale = 256.0f;    // P~ is kept 2^8 larger so small weights stay normal in fp16
+constexpr float kLazyMax = 8.0f;          // log2 of how far a logit may exceed the reference maximum of its row
+constexpr float kLazyScaleMax = 255.0f;   // largest V-side scale (already times 2^8) for which 2^kLazyMax * scale stays in fp16
 constexpr float kLn2 = 0.6931471805599453f;
 constexpr float kLog2e = 1.4426950408889634f;
 

@@ -43,8 +43,6 @@ constexpr int kMlaQLdsBytes = (kMlaQOps - kMlaQRegOps) * kMlaThreads * 16;  // 6
 constexpr int kMlaVtPitch = 2 * kTile;                    // fp16 V^T row: 32 tokens = 4 chunks of 16 bytes, swizzled
 constexpr int kMlaVtBytes = kMlaR * kMlaVtPitch;          // 32768
 typedef int32_t i32x4 __attribute__((ext_vector_type(4)));
-constexpr float kMlaLazy = 8.0f;       // log2 of how far a logit may exceed the reference maximum
-constexpr float kMlaLazyVs = 255.0f;   // largest V-side scale (already times 2^8) with which 2^kMlaLazy * scale stays in fp16
 // What the head-owning waves hand to the others, per tile and double-buffered: the eight P~ operands
 // (64 lanes x 16 bytes each), one rescale factor per head and one "running max moved" byte per wave.
 constexpr int kMlaPBytes = 8 * kWave * 16;                // 8192
@@ -436,7 +434,7 @@ __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
         }
         mloc = max_over_quarters(mloc);
         // The reference maximum m of a head only has to keep 2^(logit - m) in range, it need not be the
-        // true maximum: it moves when some head of the tile outgrows it by more than 2^kMlaLazy (or at
+        // true maximum: it moves when some head of the tile outgrows it by more than 2^kLazyMax (or at
         // all, when a token's value scale is so large that p * scale could leave the fp16 range
         // otherwise).  Moving m rescales what is accumulated so far, and the accumulators of these
         // heads are spread over all waves, so the factors travel with the tile; with i.i.d. logits the
@@ -446,7 +444,7 @@ __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
         for (int mt = 0; mt < 2; ++mt) vs[mt] = *reinterpret_cast<const floatx4*>(sck + kTile + 16 * mt + 4 * g);
         const float vsmax = fmaxf(fmaxf(fmaxf(vs[0].x, vs[0].y), fmaxf(vs[0].z, vs[0].w)),
                                   fmaxf(fmaxf(vs[1].x, vs[1].y), fmaxf(vs[1].z, vs[1].w)));
-        const float lim = vsmax > kMlaLazyVs ? m : m + kMlaLazy;
+        const float lim = vsmax > kLazyScaleMax ? m : m + kLazyMax;
         const bool moved = __builtin_amdgcn_ballot_w64(mloc > lim) != 0;
         if (moved) {
           const float m_new = fmaxf(m, mloc);

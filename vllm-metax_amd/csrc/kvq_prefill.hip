@@ -347,7 +347,7 @@ struct Flash32 {
   static constexpr int K_BYTES = kTile * K_PITCH;
   static constexpr int V_PITCH = 2 * kTile + 16;
   static constexpr int V_BYTES = D * V_PITCH;
-  static constexpr int BUF_BYTES = K_BYTES + V_BYTES + 64 * 4;
+  static constexpr int BUF_BYTES = K_BYTES + V_BYTES + 68 * 4;   // 32 K-side + 32 V-side scales + the tile's lazy-maximum allowance
   static constexpr int LDS_BYTES = 2 * RAW_BYTES + 2 * BUF_BYTES;
   static constexpr int COLS = 32 * WAVES;
 
@@ -448,7 +448,13 @@ struct Flash32 {
     }
     if (tid < 64) {
       const float sc = *reinterpret_cast<const float*>(raw + l_sc);
-      reinterpret_cast<float*>(buf + K_BYTES + V_BYTES)[tid] = fminf(sc * sc_mul, 65504.f);
+      const float val = fminf(sc * sc_mul, 65504.f);
+      reinterpret_cast<float*>(buf + K_BYTES + V_BYTES)[tid] = val;
+      // How far a logit may exceed a column's reference maximum in this tile before the maximum has
+      // to move: 2^kLazyMax * (largest V-side scale) must stay inside fp16, else nothing is allowed.
+      const bool big = tid >= 32 && val > kLazyScaleMax;
+      const bool any_big = __builtin_amdgcn_ballot_w64(big) != 0;
+      if (tid == 0) reinterpret_cast<float*>(buf + K_BYTES + V_BYTES)[64] = any_big ? 0.f : kLazyMax;
     }
   }
 
@@ -509,8 +515,13 @@ struct Flash32 {
       }
     }
     d = max_over_halves(d);
-    // how far the maximum moves: a fresh column takes d itself (0 while it still sees nothing)
-    const float up = fresh ? (d == -INFINITY ? 0.f : d) : fmaxf(d, 0.f);
+    // How far the reference maximum moves: a fresh column takes d itself (0 while it still sees
+    // nothing); otherwise it only has to keep 2^(logit - m) in range, not be the true maximum, and
+    // stays put while no logit exceeds it by more than the tile's allowance.  With 32 columns per
+    // wave SOME true maximum moves in most tiles of the first thousand tokens, and each move rescales
+    // every accumulator of the wave; the lazy reference moves a few times per column.
+    const float allow = sc[64];
+    const float up = fresh ? (d == -INFINITY ? 0.f : d) : (d > allow ? d : 0.f);
     if (__builtin_amdgcn_ballot_w64(up != 0.f) != 0) {
       const float alpha = __builtin_amdgcn_exp2f(-up);  // a fresh column's o and l are still zero
       l *= alpha;
