@@ -30,7 +30,7 @@ import torch  # noqa: E402
 HBM_PEAK_GBPS = 8000.0
 # HBM bytes per decode attention launch, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by a plain
 # read / copy kernel of known size (factors 2.000 and 1.000); summaries under profiles/.
-MEASURED_TRAFFIC = {"llama3_8b_decode_b64_ctx1k-8k": 727.1e6, "mla_decode_b32_h128_ctx4096": 199.6e6}
+MEASURED_TRAFFIC = {"llama3_8b_decode_b64_ctx1k-8k": 727.1e6, "mla_decode_b32_h128_ctx4096": 195.4e6}
 METRIC = "int8-KV paged decode: achieved HBM GB/s (% peak), µs/layer @B=64 ctx=8k"
 
 
