@@ -17,8 +17,9 @@ R, P = 512, 64
 GOLDEN = os.path.join(os.path.dirname(__file__), "golden", "kvq_golden_small.pt")
 
 
-def _build(ctx, bs, seed, dtype=torch.bfloat16, poison=True, amp=1.0):
-    """A latent cache written by the oracle for sequences of the given lengths, blocks shuffled."""
+def _build(ctx, bs, seed, dtype=torch.bfloat16, poison=True, amp=1.0, rows_fn=None):
+    """A latent cache written by the oracle for sequences of the given lengths, blocks shuffled.
+    ``rows_fn(kv_c, k_pe)`` may reshape the random rows of a sequence before they are quantised."""
     g = torch.Generator().manual_seed(seed)
     B = len(ctx)
     per = [(c + bs - 1) // bs for c in ctx]
@@ -36,6 +37,9 @@ def _build(ctx, bs, seed, dtype=torch.bfloat16, poison=True, amp=1.0):
             continue
         kv_c = (torch.randn((c, R), generator=g) * amp).to(dtype)
         k_pe = (torch.randn((c, P), generator=g) * amp).to(dtype)
+        if rows_fn is not None:
+            kv_c, k_pe = rows_fn(kv_c.float(), k_pe.float())
+            kv_c, k_pe = kv_c.to(dtype), k_pe.to(dtype)
         pos = torch.arange(c)
         slots = (bt[i, pos // bs].long() * bs + pos % bs)
         oracle.mla_cache_write(kv_c, k_pe, cache, lay, slots)
@@ -89,6 +93,55 @@ def test_mla_decode_peaked_softmax_and_large_values(gpu_device):
     got, lse = _run(q, cache, bt, sl, scale)
     T.assert_close_attn(got, want, atol=2e-2 * 8, rtol=1e-2, what="mla decode, peaked")  # atol scaled with |V|
     torch.testing.assert_close(lse.cpu(), want_lse, atol=5e-2, rtol=1e-3)
+
+
+@pytest.mark.parametrize("step", [0.1, 0.4, 3.0])
+def test_mla_decode_logits_that_keep_rising(gpu_device, step):
+    """Every head's logits grow along the sequence (a shared direction whose weight ramps up), by
+    ``step`` (log2 units) per 32-token tile: the softmax's reference maximum may lag the true one by
+    up to 2^8 before it moves, so a slow rise keeps it lagging for many tiles, a fast one moves it in
+    most tiles.  16 tiles per split (32 sequences x 8 splits x 512 tokens)."""
+    B, H, c = 32, 16, 4096
+    u = torch.randn(R, generator=torch.Generator().manual_seed(1))
+    u = u / u.norm()
+
+    def ramp(kv_c, k_pe):
+        n = kv_c.shape[0]
+        w = torch.arange(n, dtype=torch.float32) / 32.0 * step          # log2 units by token
+        return 0.3 * kv_c + w[:, None] * u[None, :] * 0.6931, 0.3 * k_pe   # q.u = 1 below, scale = 1
+
+    cache, lay, bt, sl = _build([c] * B, 64, seed=21, rows_fn=ramp)
+    g = torch.Generator().manual_seed(4)
+    q = torch.randn((B, H, R + P), generator=g) * 0.3
+    q[:, :, :R] += u                                    # unit projection on the ramp direction
+    q = q.to(torch.bfloat16)
+    want, want_lse = oracle.mla_decode(q, cache, lay, bt, sl, 1.0)
+    got, lse = _run(q, cache, bt, sl, 1.0)
+    vmax = float(want.abs().max())
+    T.assert_close_attn(got, want, atol=2e-2 * max(1.0, vmax), rtol=1e-2, what=f"mla decode, rising logits {step}")
+    torch.testing.assert_close(lse.cpu(), want_lse, atol=2e-2, rtol=1e-3)
+
+
+def test_mla_decode_huge_value_scales(gpu_device):
+    """Latent rows in the thousands: per-token scales above 1, where p * scale of a lagging
+    reference maximum could leave the fp16 range, so the kernel moves the maximum eagerly in such
+    tiles.  Some sequences mix ordinary and huge rows tile by tile."""
+    B, H = 16, 32
+
+    def huge_every_other_tile(kv_c, k_pe):
+        n = kv_c.shape[0]
+        big = ((torch.arange(n) // 32) % 2 == 1).float() * 1999.0 + 1.0
+        return kv_c * big[:, None], k_pe * big[:, None]
+
+    cache, lay, bt, sl = _build([2048] * B, 64, seed=33, rows_fn=huge_every_other_tile)
+    g = torch.Generator().manual_seed(6)
+    q = (torch.randn((B, H, R + P), generator=g) * 0.01).to(torch.bfloat16)
+    scale = 0.005
+    want, want_lse = oracle.mla_decode(q, cache, lay, bt, sl, scale)
+    got, lse = _run(q, cache, bt, sl, scale, out_dtype=torch.float32)
+    assert torch.isfinite(got).all()
+    T.assert_close_attn(got, want, atol=2e-2 * 2000, rtol=1e-2, what="mla decode, huge value scales")
+    torch.testing.assert_close(lse.cpu(), want_lse, atol=2e-2, rtol=1e-3)
 
 
 def test_mla_decode_strided_q_and_no_lse(gpu_device):

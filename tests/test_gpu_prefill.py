@@ -170,3 +170,42 @@ def test_backend_forward_mixed_batch(gpu_device, monkeypatch):
     want = oracle.paged_attn(q.view(n_tok, hq, d), T.storage_bytes(kv_cpu), lay, bt,
                              torch.tensor(ctx, dtype=torch.int32), cu, 0.0884)
     T.assert_close_attn(out.view(n_tok, hq, d), want, what="backend forward, mixed batch")
+
+
+@pytest.mark.parametrize("step", [0.2, 2.0])
+def test_prefill_logits_that_keep_rising(gpu_device, step):
+    """Keys whose logits grow along the sequence by ``step`` (log2 units) per 32-token tile: the
+    prefill tile's reference maximum may lag the true one by up to 2^8 before it moves.  A 300-token
+    chunk on 1500 cached tokens (workgroup-shared tile) plus short runs."""
+    hq, hkv, d, bs = 8, 2, 128, 16
+    ctx, qls = [1800, 400, 90], [300, 40, 1]
+    kv, lay, bt, q, sl, cu = build(ctx, qls, hq, hkv, d, bs, seed=12)
+    g = torch.Generator().manual_seed(13)
+    u = torch.randn(d, generator=g)
+    u = u / u.norm()
+    ks = [0.3 * torch.randn((c, hkv, d), generator=g) + (torch.arange(c) / 32.0 * step * 0.6931)[:, None, None] * u for c in ctx]
+    vs = [torch.randn((c, hkv, d), generator=g) for c in ctx]
+    T.fill_cache_from_sources(kv, lay, bt, ctx, bs, [k.to(torch.bfloat16) for k in ks], [v.to(torch.bfloat16) for v in vs])
+    q = (0.3 * q.float() + u).to(torch.bfloat16)          # unit projection on the ramp direction
+    want, want_lse = oracle.paged_attn(q, T.storage_bytes(kv), lay, bt, sl, cu, 1.0, return_lse=True)
+    got, lse = run(gpu_device, kv, "NHD", bt, q, sl, cu, max(qls), 1.0, want_lse=True)
+    T.assert_close_attn(got, want, what=f"prefill, rising logits {step}")
+    torch.testing.assert_close(lse.cpu(), want_lse, atol=2e-2, rtol=1e-3)
+
+
+def test_prefill_huge_value_scales(gpu_device):
+    """V rows in the thousands in every other tile: scales above 1, for which the tile moves its
+    reference maximum eagerly (p * scale must stay inside fp16)."""
+    hq, hkv, d, bs = 8, 2, 128, 16
+    ctx, qls = [1200, 64], [500, 64]
+    kv, lay, bt, q, sl, cu = build(ctx, qls, hq, hkv, d, bs, seed=14)
+    g = torch.Generator().manual_seed(15)
+    ks = [torch.randn((c, hkv, d), generator=g) for c in ctx]
+    vs = [torch.randn((c, hkv, d), generator=g) * (((torch.arange(c) // 32) % 2 == 1).float() * 1999.0 + 1.0)[:, None, None]
+          for c in ctx]
+    T.fill_cache_from_sources(kv, lay, bt, ctx, bs, [k.to(torch.bfloat16) for k in ks], [v.to(torch.bfloat16) for v in vs])
+    scale = 1 / math.sqrt(d)
+    want = oracle.paged_attn(q, T.storage_bytes(kv), lay, bt, sl, cu, scale)
+    got = run(gpu_device, kv, "NHD", bt, q, sl, cu, max(qls), scale, out_dtype=torch.float32)
+    assert torch.isfinite(got).all()
+    T.assert_close_attn(got, want, atol=2e-2 * 2000, rtol=1e-2, what="prefill, huge value scales")
