@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define KVQ_ABI_VERSION 5
+#define KVQ_ABI_VERSION 6
 
 #define KVQ_OK 0
 #define KVQ_EINVAL (-22)
@@ -293,6 +293,19 @@ KVQ_API int kvq_cp_gather_mla_int8(void* dst, int64_t dst_stride, const void* ca
                            kvq_stream_t stream);
 
 /*
+ * q_out[t, h, :] = [ql_nope[t, h, :] | q_pe[t, h, :]]: concat_mla_q(ql_nope,
+ * q_pe, q_out), csrc/libtorch_stable/cache_kernels.cu:1740-1783 (schema
+ * torch_bindings.cpp:893), the step before an MLA decode whose caller holds the
+ * absorbed query in two parts.  Strides in elements of `dtype`, last dims
+ * contiguous.  (kvq_mla_decode_int8 also takes the two parts directly.)
+ */
+KVQ_API int kvq_concat_mla_q(void* q_out, int64_t out_stride_t, int64_t out_stride_h,
+                             const void* ql_nope, int64_t nope_stride_t, int64_t nope_stride_h,
+                             const void* q_pe, int64_t pe_stride_t, int64_t pe_stride_h, int dtype,
+                             int64_t num_tokens, int num_heads, int nope_dim, int rope_dim,
+                             kvq_stream_t stream);
+
+/*
  * Workspace for kvq_mla_decode_int8 (host query, depends on the device): the fp16
  * split states and their lse values (counterpart of the reference's attn_logits
  * buffer, vllm_metax/v1/attention/backends/mla/triton_mla.py:261-269) plus the
@@ -307,11 +320,16 @@ KVQ_API size_t kvq_mla_decode_workspace_bytes(int max_num_seqs, int num_heads, i
  * lse, block_table, seq_lens, attn_logits, num_kv_splits, sm_scale, page_size,
  * ..., is_mla=True), vllm_metax/v1/attention/backends/mla/triton_mla.py:226-295,
  * vllm_metax/v1/attention/ops/triton_decode_attention.py:763-825.
- * q [B, H, kv_lora_rank + rope_dim] (absorbed), out [B, H, kv_lora_rank]
- * contiguous and 16-byte aligned, lse [B, H] fp32 natural log (may be NULL).
+ * q [B, H, kv_lora_rank + rope_dim] (absorbed) with q_pe NULL, or -- the
+ * (ql_nope, q_pe) form of forward_mqa's first argument, triton_mla.py:226-238,
+ * taken as it is, without the concatenation -- q = ql_nope [B, H, kv_lora_rank]
+ * and q_pe [B, H, rope_dim] of the same dtype (strides in elements); out
+ * [B, H, kv_lora_rank] contiguous and 16-byte aligned, lse [B, H] fp32 natural
+ * log (may be NULL).
  */
 KVQ_API int kvq_mla_decode_int8(void* out, int out_dtype, float* lse, const void* q, int q_dtype,
-                        int64_t q_stride_b, int64_t q_stride_h, const void* cache,
+                        int64_t q_stride_b, int64_t q_stride_h, const void* q_pe,
+                        int64_t q_pe_stride_b, int64_t q_pe_stride_h, const void* cache,
                         const kvq_mla_geom* geom, const int32_t* block_table,
                         int64_t bt_stride, const int32_t* seq_lens, int num_seqs,
                         int num_heads, float scale, void* workspace, size_t workspace_bytes,

@@ -158,6 +158,58 @@ def test_mla_decode_strided_q_and_no_lse(gpu_device):
     T.assert_close_attn(o, want, what="mla decode, strided q")
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_mla_decode_takes_the_query_in_two_parts(gpu_device, dtype):
+    """forward_mqa may receive (ql_nope, q_pe) (vllm_metax/v1/attention/backends/mla/triton_mla.py:226-238,
+    where the reference concatenates them): the kernel reads the two parts where they lie, and the
+    result is bit-identical to the call on the concatenated tensor.  The parts are strided views."""
+    ctx = [300, 64, 1000]
+    cache, lay, bt, sl = _build(ctx, 64, seed=17)
+    g = torch.Generator().manual_seed(3)
+    H = 48
+    nope_store = torch.randn((3, H, R + 32), generator=g).to(dtype)      # rows wider than the part they hold
+    pe_store = torch.randn((3, 2 * H, P), generator=g).to(dtype)         # every other head row is used
+    dev = gpu_device
+    ql_nope = nope_store.to(dev)[:, :, :R]
+    q_pe = pe_store.to(dev)[:, ::2, :]
+    joined = torch.cat([ql_nope, q_pe], dim=-1)
+    kv = cache.to(dev)
+    outs = []
+    for q in (joined, (ql_nope, q_pe)):
+        o = torch.full((3, H, R), float("nan"), dtype=dtype, device=dev)
+        lse = torch.full((3, H), float("nan"), dtype=torch.float32, device=dev)
+        ops.mla_decode_int8(q, kv, o, lse, bt.to(dev), sl.to(dev), 0.07, R)
+        torch.cuda.synchronize()
+        outs.append((o.cpu(), lse.cpu()))
+    assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[0][1], outs[1][1])
+    want, _ = oracle.mla_decode(joined.cpu(), cache, lay, bt, sl, 0.07)
+    tol = dict(atol=4e-3, rtol=4e-3) if dtype == torch.float32 else {}
+    T.assert_close_attn(outs[1][0], want, what="mla decode, two-part query", **tol)
+    with pytest.raises(RuntimeError):
+        ops.mla_decode_int8((ql_nope, q_pe[:, :, :32]), kv, o, lse, bt.to(dev), sl.to(dev), 0.07, R)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_concat_mla_q(gpu_device, dtype):
+    """ops.concat_mla_q(ql_nope, q_pe, q_out) == torch.cat((ql_nope, q_pe), dim=-1), which it replaces
+    (csrc/libtorch_stable/cache_kernels.cu:1738-1739); strided inputs and output, bytes must match."""
+    dev = gpu_device
+    g = torch.Generator().manual_seed(8)
+    for T_, H in [(1, 128), (37, 16), (300, 5), (0, 8)]:
+        a = torch.randn((T_, H, R + 64), generator=g).to(dtype).to(dev)[:, :, 64:]
+        b = torch.randn((T_, 2 * H, P), generator=g).to(dtype).to(dev)[:, 1::2, :]
+        out_store = torch.full((T_, H, R + P + 16), 7.0, dtype=dtype, device=dev)
+        out = out_store[:, :, : R + P]
+        ops.concat_mla_q(a, b, out)
+        torch.cuda.synchronize()
+        assert torch.equal(out, torch.cat((a, b), dim=-1))
+        assert bool((out_store[:, :, R + P:] == 7.0).all())          # nothing written past the rows
+    with pytest.raises(RuntimeError):
+        ops.concat_mla_q(a, b, out_store)                              # wrong output width
+    with pytest.raises(RuntimeError):
+        ops.concat_mla_q(a, b.float() if dtype != torch.float32 else b.half(), out)
+
+
 def test_mla_decode_golden(gpu_device):
     G = torch.load(GOLDEN, weights_only=True)
     cache = G["mla_cache"]

@@ -229,7 +229,54 @@ __global__ __launch_bounds__(256) void mla_cp_gather_kernel(uint8_t* __restrict_
   }
 }
 
+// q_out[t, h, :] = [ql_nope[t, h, :] | q_pe[t, h, :]], a byte move: one wave per (token, head) row, 4-byte
+// pieces (the reference's kernel has the same shape, one warp per row:
+// csrc/libtorch_stable/cache_kernels.cu:1769-1782).  Row lengths are in bytes.
+__global__ __launch_bounds__(256) void concat_mla_q_kernel(uint8_t* out, int64_t out_st, int64_t out_sh,
+                                                           const uint8_t* nope, int64_t nope_st, int64_t nope_sh,
+                                                           const uint8_t* pe, int64_t pe_st, int64_t pe_sh,
+                                                           int64_t rows, int num_heads, int nope_bytes, int pe_bytes) {
+  const int lane = threadIdx.x & 63;
+  const int64_t wave = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  for (int64_t row = wave; row < rows; row += (int64_t)gridDim.x * 4) {
+    const int64_t t = row / num_heads, h = row - t * num_heads;
+    uint8_t* o = out + t * out_st + h * out_sh;
+    const uint8_t* a = nope + t * nope_st + h * nope_sh;
+    const uint8_t* b = pe + t * pe_st + h * pe_sh;
+    for (int i = 4 * lane; i < nope_bytes; i += 256)
+      *reinterpret_cast<uint32_t*>(o + i) = *reinterpret_cast<const uint32_t*>(a + i);
+    for (int i = 4 * lane; i < pe_bytes; i += 256)
+      *reinterpret_cast<uint32_t*>(o + nope_bytes + i) = *reinterpret_cast<const uint32_t*>(b + i);
+  }
+}
+
 }  // namespace kvq
+
+extern "C" int kvq_concat_mla_q(void* q_out, int64_t out_stride_t, int64_t out_stride_h, const void* ql_nope,
+                                int64_t nope_stride_t, int64_t nope_stride_h, const void* q_pe,
+                                int64_t pe_stride_t, int64_t pe_stride_h, int dtype, int64_t num_tokens,
+                                int num_heads, int nope_dim, int rope_dim, kvq_stream_t stream) {
+  using namespace kvq;
+  const char* op = "concat_mla_q";
+  KVQ_REQUIRE(dtype == KVQ_F32 || dtype == KVQ_BF16 || dtype == KVQ_F16, "%s: unknown dtype %d", op, dtype);
+  KVQ_REQUIRE(num_tokens >= 0 && num_heads > 0 && nope_dim > 0 && rope_dim > 0, "%s: bad sizes", op);
+  if (num_tokens == 0) return KVQ_OK;
+  KVQ_REQUIRE(q_out && ql_nope && q_pe, "%s: NULL pointer", op);
+  const int64_t es = dtype == KVQ_F32 ? 4 : 2;
+  KVQ_REQUIRE((nope_dim * es) % 4 == 0 && (rope_dim * es) % 4 == 0, "%s: row parts must be whole 4-byte words", op);
+  KVQ_REQUIRE(((uintptr_t)q_out | (uintptr_t)ql_nope | (uintptr_t)q_pe) % 4 == 0 &&
+                  ((out_stride_t | out_stride_h | nope_stride_t | nope_stride_h | pe_stride_t | pe_stride_h) * es) % 4 == 0,
+              "%s: rows must be 4-byte aligned", op);
+  KVQ_REQUIRE(out_stride_h >= nope_dim + rope_dim || num_heads == 1, "%s: q_out rows overlap", op);
+  const int64_t rows = num_tokens * num_heads;
+  const int64_t want = (rows + 3) / 4;
+  const unsigned blocks = (unsigned)(want < 65536 ? want : 65536);
+  hipLaunchKernelGGL(concat_mla_q_kernel, dim3(blocks), dim3(256), 0, as_stream(stream), static_cast<uint8_t*>(q_out),
+                     out_stride_t * es, out_stride_h * es, static_cast<const uint8_t*>(ql_nope), nope_stride_t * es,
+                     nope_stride_h * es, static_cast<const uint8_t*>(q_pe), pe_stride_t * es, pe_stride_h * es, rows,
+                     num_heads, (int)(nope_dim * es), (int)(rope_dim * es));
+  return check_hip(hipGetLastError(), "concat_mla_q launch");
+}
 
 extern "C" int kvq_cp_gather_mla_int8(void* dst, int64_t dst_stride, const void* cache, const kvq_mla_geom* geom,
                                       const int32_t* block_table, int64_t bt_stride, const int32_t* cu_seq_lens,

@@ -50,8 +50,10 @@ constexpr int kMlaXchgBytes = kMlaPBytes + 128 * 4 + 16;  // 8720
 constexpr int kMlaLdsBytes = 2 * kMlaBufBytes + kMlaVtBytes + kMlaQLdsBytes + 2 * kMlaXchgBytes;  // 153120 of 163840
 
 struct MlaArgs {
-  const void* q;
+  const void* q;            // dims 0 .. 511 of the absorbed query (ql_nope) ...
   int64_t q_stride_b, q_stride_h;
+  const void* q_pe;         // ... and its 64 rope dims: q + 512 elements when the caller holds them joined
+  int64_t pe_stride_b, pe_stride_h;
   const uint8_t* cache;
   kvq_mla_geom g;
   const int32_t* block_table;
@@ -111,6 +113,7 @@ __global__ __launch_bounds__(256) void mla_quant_q_kernel(MlaArgs a) {
   const int64_t qblock = (int64_t)seq * a.head_groups + hgroup;
   u32x4* qdst = reinterpret_cast<u32x4*>(a.q_ops + qblock * (kMlaQOps * kWave * 16)) + lane;
   const int64_t qbase = (int64_t)seq * a.q_stride_b + (int64_t)(head_ok ? head : 0) * a.q_stride_h + 16 * g;
+  const int64_t pebase = (int64_t)seq * a.pe_stride_b + (int64_t)(head_ok ? head : 0) * a.pe_stride_h + 16 * g;
   // the wave's values as floats: f[n][i] = dim 64 kk + 16 g + i of k-step kk = wave + 4 n (a k-step
   // past the last rereads the last one and is not written)
   float f[kMine][16];
@@ -118,7 +121,9 @@ __global__ __launch_bounds__(256) void mla_quant_q_kernel(MlaArgs a) {
   for (int n = 0; n < kMine; ++n) {
     const int kk = min(wave + 4 * n, kMlaKSteps8 - 1);
     if constexpr (QDT == KVQ_F32) {
-      const float* p = reinterpret_cast<const float*>(a.q) + qbase + 64 * kk;
+      // k-step 8 is the rope part
+      const float* p = kk < kMlaR / 64 ? reinterpret_cast<const float*>(a.q) + qbase + 64 * kk
+                                       : reinterpret_cast<const float*>(a.q_pe) + pebase;
 #pragma unroll
       for (int i = 0; i < 16; i += 4) {
         const floatx4 v = *reinterpret_cast<const floatx4_a4*>(p + i);
@@ -127,7 +132,9 @@ __global__ __launch_bounds__(256) void mla_quant_q_kernel(MlaArgs a) {
     } else {
 #pragma unroll
       for (int h = 0; h < 2; ++h) {
-        const u32x4 v = *reinterpret_cast<const u32x4_a4*>(reinterpret_cast<const uint16_t*>(a.q) + qbase + 64 * kk + 8 * h);
+        const uint16_t* p = kk < kMlaR / 64 ? reinterpret_cast<const uint16_t*>(a.q) + qbase + 64 * kk
+                                            : reinterpret_cast<const uint16_t*>(a.q_pe) + pebase;
+        const u32x4 v = *reinterpret_cast<const u32x4_a4*>(p + 8 * h);
 #pragma unroll
         for (int w = 0; w < 4; ++w) {
           const uint32_t e = v[w];
@@ -685,7 +692,8 @@ size_t kvq_mla_decode_workspace_bytes(int max_num_seqs, int num_heads, int kv_lo
 }
 
 int kvq_mla_decode_int8(void* out, int out_dtype, float* lse, const void* q, int q_dtype, int64_t q_stride_b,
-                        int64_t q_stride_h, const void* cache, const kvq_mla_geom* geom,
+                        int64_t q_stride_h, const void* q_pe, int64_t q_pe_stride_b, int64_t q_pe_stride_h,
+                        const void* cache, const kvq_mla_geom* geom,
                         const int32_t* block_table, int64_t bt_stride, const int32_t* seq_lens, int num_seqs,
                         int num_heads, float scale, void* workspace, size_t workspace_bytes,
                         kvq_stream_t stream) {
@@ -705,6 +713,13 @@ int kvq_mla_decode_int8(void* out, int out_dtype, float* lse, const void* q, int
   const int qsz = q_dtype == KVQ_F32 ? 4 : 2;
   KVQ_REQUIRE(((uintptr_t)q % 4) == 0 && (q_stride_b * qsz) % 4 == 0 && (q_stride_h * qsz) % 4 == 0,
               "%s: q rows must be 4-byte aligned", op);
+  if (q_pe == nullptr) {   // joined [B, H, 576] rows
+    q_pe = static_cast<const char*>(q) + (size_t)kMlaR * qsz;
+    q_pe_stride_b = q_stride_b;
+    q_pe_stride_h = q_stride_h;
+  }
+  KVQ_REQUIRE(((uintptr_t)q_pe % 4) == 0 && (q_pe_stride_b * qsz) % 4 == 0 && (q_pe_stride_h * qsz) % 4 == 0,
+              "%s: q_pe rows must be 4-byte aligned", op);
   const int splits = mla_num_splits(0, num_seqs, num_heads);
   const int head_groups = (num_heads + 15) / 16;
   const size_t states = (size_t)num_seqs * head_groups * 16 * splits;
@@ -717,6 +732,9 @@ int kvq_mla_decode_int8(void* out, int out_dtype, float* lse, const void* q, int
   a.q = q;
   a.q_stride_b = q_stride_b;
   a.q_stride_h = q_stride_h;
+  a.q_pe = q_pe;
+  a.pe_stride_b = q_pe_stride_b;
+  a.pe_stride_h = q_pe_stride_h;
   a.cache = static_cast<const uint8_t*>(cache);
   a.g = g;
   a.block_table = block_table;

@@ -13,7 +13,7 @@ _LIB_DIR = os.path.join(os.path.dirname(os.path.abspath(__file__)), "_lib")
 LIB_PATH = os.path.join(_LIB_DIR, "libkvq_hip.so")
 
 KVQ_F32, KVQ_BF16, KVQ_F16 = 0, 1, 2
-ABI_VERSION = 5
+ABI_VERSION = 6
 
 
 class CacheGeom(ctypes.Structure):
@@ -64,8 +64,9 @@ SIGNATURES = {
                                                 _vp, _mla_p, _vp, _i64, _f, _vp]),
     "kvq_cp_gather_mla_int8": (_i, [_vp, _i64, _vp, _mla_p, _vp, _i64, _vp, _vp, _i, _i64, _vp]),
     "kvq_mla_decode_workspace_bytes": (_sz, [_i, _i, _i]),
-    "kvq_mla_decode_int8": (_i, [_vp, _i, _vp, _vp, _i, _i64, _i64, _vp, _mla_p, _vp, _i64, _vp, _i, _i, _f,
-                                 _vp, _sz, _vp]),
+    "kvq_mla_decode_int8": (_i, [_vp, _i, _vp, _vp, _i, _i64, _i64, _vp, _i64, _i64, _vp, _mla_p, _vp, _i64, _vp,
+                                 _i, _i, _f, _vp, _sz, _vp]),
+    "kvq_concat_mla_q": (_i, [_vp, _i64, _i64, _vp, _i64, _i64, _vp, _i64, _i64, _i, _i64, _i, _i, _i, _vp]),
 }
 
 _lib = None

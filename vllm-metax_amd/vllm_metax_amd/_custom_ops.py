@@ -584,17 +584,30 @@ def mla_decode_workspace_bytes(max_num_seqs: int, num_heads: int, kv_lora_rank: 
     return int(_C.load().kvq_mla_decode_workspace_bytes(max_num_seqs, num_heads, kv_lora_rank))
 
 
-def mla_decode_int8(q: torch.Tensor, kv_cache: torch.Tensor, o: torch.Tensor, lse: torch.Tensor | None,
+def mla_decode_int8(q, kv_cache: torch.Tensor, o: torch.Tensor, lse: torch.Tensor | None,
                     block_table: torch.Tensor, seq_lens: torch.Tensor, sm_scale: float, kv_lora_rank: int,
                     workspace: torch.Tensor | None = None, geometry: MlaGeometry | None = None) -> None:
     """MLA decode over the int8 latent cache: the job of ``decode_attention_fwd(..., is_mla=True)``
-    (vllm_metax/v1/attention/ops/triton_decode_attention.py:763-825).  q ``[B, H, R+P]``,
+    (vllm_metax/v1/attention/ops/triton_decode_attention.py:763-825).  q ``[B, H, R+P]`` or the pair
+    ``(ql_nope [B, H, R], q_pe [B, H, P])`` that ``forward_mqa`` may receive
+    (vllm_metax/v1/attention/backends/mla/triton_mla.py:226-238; read as it is, no concatenation),
     o ``[B, H, R]``, lse ``[B, H]`` fp32 or None."""
-    dev = _require_cuda(q, kv_cache, o, lse, block_table, seq_lens, workspace)
+    q_pe = None
+    if type(q) is tuple:
+        q, q_pe = q
+    dev = _require_cuda(q, q_pe, kv_cache, o, lse, block_table, seq_lens, workspace)
     geom = geometry or mla_geometry(kv_cache, kv_lora_rank)
     B, H, W = q.shape
-    if W != geom.kv_lora_rank + geom.rope_dim or tuple(o.shape) != (B, H, geom.kv_lora_rank):
-        raise RuntimeError("q must be [B, H, R+P] and o [B, H, R]")
+    if q_pe is None:
+        if W != geom.kv_lora_rank + geom.rope_dim:
+            raise RuntimeError("q must be [B, H, R+P]")
+    else:
+        if W != geom.kv_lora_rank or tuple(q_pe.shape) != (B, H, geom.rope_dim) or q_pe.dtype != q.dtype:
+            raise RuntimeError("(ql_nope, q_pe) must be [B, H, R] and [B, H, P] of one dtype")
+        if q_pe.stride(2) != 1:
+            raise RuntimeError("q_pe head dim must be contiguous")
+    if tuple(o.shape) != (B, H, geom.kv_lora_rank):
+        raise RuntimeError("o must be [B, H, R]")
     if q.stride(2) != 1 or not o.is_contiguous():
         raise RuntimeError("q head dim must be contiguous and o contiguous")
     if seq_lens.dtype != torch.int32 or block_table.dtype != torch.int32 or block_table.stride(1) != 1:
@@ -607,8 +620,34 @@ def mla_decode_int8(q: torch.Tensor, kv_cache: torch.Tensor, o: torch.Tensor, ls
     g = geom.as_struct()
     with _on_device(dev):
         rc = _C.load().kvq_mla_decode_int8(_ptr(o), _dtype_code(o, "o"), _ptr(lse), _ptr(q), _dtype_code(q, "q"),
-                                           q.stride(0), q.stride(1), ctypes.c_void_p(geom.base_ptr), ctypes.byref(g),
+                                           q.stride(0), q.stride(1), _ptr(q_pe),
+                                           q_pe.stride(0) if q_pe is not None else 0,
+                                           q_pe.stride(1) if q_pe is not None else 0,
+                                           ctypes.c_void_p(geom.base_ptr), ctypes.byref(g),
                                            _ptr(block_table), block_table.stride(0), _ptr(seq_lens), B, H,
                                            float(sm_scale), _ptr(workspace),
                                            workspace.numel() * workspace.element_size(), _stream(dev))
     _C.check(rc, "mla_decode_int8")
+
+
+def concat_mla_q(ql_nope: torch.Tensor, q_pe: torch.Tensor, q_out: torch.Tensor) -> None:
+    """``q_out[..., :R] = ql_nope; q_out[..., R:] = q_pe``: the reference's ``ops.concat_mla_q``
+    (csrc/libtorch_stable/cache_kernels.cu:1740-1783; call site
+    vllm_metax/v1/attention/backends/mla/flashmla_sparse.py:1100).  ``[T, H, R]``, ``[T, H, P]`` ->
+    ``[T, H, R+P]``, one dtype, last dims contiguous."""
+    dev = _require_cuda(ql_nope, q_pe, q_out)
+    if ql_nope.dim() != 3 or q_pe.dim() != 3 or q_out.dim() != 3:
+        raise RuntimeError("concat_mla_q takes [num_tokens, num_heads, dim] tensors")
+    T, H, R = ql_nope.shape
+    P = q_pe.shape[2]
+    if tuple(q_pe.shape[:2]) != (T, H) or tuple(q_out.shape) != (T, H, R + P):
+        raise RuntimeError("q_pe must be [T, H, P] and q_out [T, H, R+P]")
+    if not (ql_nope.dtype == q_pe.dtype == q_out.dtype):
+        raise RuntimeError("ql_nope, q_pe and q_out must share a dtype")
+    if ql_nope.stride(2) != 1 or q_pe.stride(2) != 1 or q_out.stride(2) != 1:
+        raise RuntimeError("last dims must be contiguous")
+    with _on_device(dev):
+        rc = _C.load().kvq_concat_mla_q(_ptr(q_out), q_out.stride(0), q_out.stride(1), _ptr(ql_nope),
+                                        ql_nope.stride(0), ql_nope.stride(1), _ptr(q_pe), q_pe.stride(0),
+                                        q_pe.stride(1), _dtype_code(ql_nope, "ql_nope"), T, H, R, P, _stream(dev))
+    _C.check(rc, "concat_mla_q")

@@ -132,11 +132,12 @@ class Int8MLAImpl:
         ``(o [B, H, kv_lora_rank], lse [B, H] float32)``."""
         assert kv_c_and_k_pe_cache.numel() > 0
         assert attn_metadata.decode is not None
-        if type(q) is tuple:
-            q = torch.cat(q, dim=-1)
-        B, H = q.shape[0], q.shape[1]
-        o = torch.empty((B, H, self.kv_lora_rank), dtype=q.dtype, device=q.device)
-        lse = torch.empty((B, H), dtype=torch.float32, device=q.device)
+        # a (ql_nope, q_pe) pair goes to the kernel as it is: the reference concatenates first
+        # (vllm_metax/v1/attention/backends/mla/triton_mla.py:236-237)
+        q0 = q[0] if type(q) is tuple else q
+        B, H = q0.shape[0], q0.shape[1]
+        o = torch.empty((B, H, self.kv_lora_rank), dtype=q0.dtype, device=q0.device)
+        lse = torch.empty((B, H), dtype=torch.float32, device=q0.device)
         ops.mla_decode_int8(q, kv_c_and_k_pe_cache, o, lse, attn_metadata.decode.block_table,
                             attn_metadata.decode.seq_lens, self.scale, self.kv_lora_rank,
                             workspace=getattr(attn_metadata, "workspace", None),
