@@ -256,6 +256,41 @@ def test_mla_backend_forward_mqa(gpu_device):
     torch.testing.assert_close(lse.cpu(), want_lse, atol=5e-3, rtol=1e-3)
 
 
+def test_mla_decode_caller_absorb_decode_up_proj(gpu_device):
+    """The steps either side of forward_mqa (vllm_metax/model_executor/layers/attention/mla_attention.py:
+    833-848, 874, 902, 1087-1110): q_nope x W_UK_T -> decode -> x W_UV, the query handed over as the
+    strided views the GEMM leaves.  Checked against the same chain in fp32 on the CPU with the
+    reference's bf16 roundings of ql_nope and of the decode output."""
+    from types import SimpleNamespace
+
+    from vllm_metax_amd.v1.attention.backends.mla.int8_mla import Int8MLADecodeCaller, Int8MLAImpl
+
+    dev = gpu_device
+    N, Pn, V = 16, 128, 128
+    ctx = [300, 1000, 64]
+    cache, lay, bt, sl = _build(ctx, 64, seed=41)
+    g = torch.Generator().manual_seed(42)
+    W_UK_T = (torch.randn((N, Pn, R), generator=g) / Pn ** 0.5).to(torch.bfloat16)
+    W_UV = (torch.randn((N, R, V), generator=g) / R ** 0.5).to(torch.bfloat16)
+    q_nope = torch.randn((3, N, Pn), generator=g).to(torch.bfloat16)
+    q_pe = torch.randn((3, N, P), generator=g).to(torch.bfloat16)
+    scale = (Pn + P) ** -0.5
+    impl = Int8MLAImpl(num_heads=N, head_size=R + P, scale=scale, num_kv_heads=1, kv_cache_dtype="int8_per_token",
+                       kv_lora_rank=R, qk_rope_head_dim=P)
+    caller = Int8MLADecodeCaller(impl, W_UK_T.to(dev), W_UV.to(dev))
+    md = SimpleNamespace(decode=SimpleNamespace(block_table=bt.to(dev), seq_lens=sl.to(dev)))
+    out = torch.full((3, N * V), float("nan"), dtype=torch.bfloat16, device=dev)
+    ql_view = caller.absorb_q(q_nope.to(dev))
+    assert ql_view.shape == (3, N, R) and not ql_view.is_contiguous()      # handed over as a view
+    lse = caller.forward_decode(q_nope.to(dev), q_pe.to(dev), cache.to(dev), md, out)
+    torch.cuda.synchronize()
+    ql = torch.einsum("bnp,npl->bnl", q_nope.float(), W_UK_T.float()).to(torch.bfloat16)
+    o_ref, lse_ref = oracle.mla_decode(torch.cat([ql, q_pe], -1), cache, lay, bt, sl, scale)
+    want = torch.einsum("bnl,nlv->bnv", o_ref.to(torch.bfloat16).float(), W_UV.float()).reshape(3, N * V)
+    torch.testing.assert_close(out.float().cpu(), want, atol=3e-2, rtol=2e-2)
+    torch.testing.assert_close(lse.cpu(), lse_ref, atol=2e-2, rtol=1e-3)
+
+
 def test_mla_decode_errors(gpu_device):
     dev = gpu_device
     cache = L.allocate_mla_cache(4, 64, R + P, device=dev)

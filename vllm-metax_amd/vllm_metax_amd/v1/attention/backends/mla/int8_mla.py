@@ -143,3 +143,49 @@ class Int8MLAImpl:
                             workspace=getattr(attn_metadata, "workspace", None),
                             geometry=self._geom(kv_c_and_k_pe_cache))
         return o, lse
+
+
+class Int8MLADecodeCaller:
+    """The steps either side of ``forward_mqa`` in the reference's MLA layer
+    (vllm_metax/model_executor/layers/attention/mla_attention.py:833-848, 857, 874, 902,
+    1087-1110), for the plain (unquantised-weight) branch: Q absorption
+    ``bmm(q_nope [N, B, P], W_UK_T [N, P, L])``, the decode, and the V up-projection
+    ``bmm(o [N, B, L], W_UV [N, L, V])``.  The two products are library GEMMs, as they are there.
+    What this path changes is the hand-off: the ``(ql_nope, q_pe)`` pair goes to the decode as the
+    strided views the GEMM leaves -- neither the transposed copy nor the concatenation is made --
+    and the decode's output feeds the second GEMM as a view as well."""
+
+    def __init__(self, impl: Int8MLAImpl, W_UK_T: torch.Tensor, W_UV: torch.Tensor) -> None:
+        N, P, L = W_UK_T.shape
+        if N != impl.num_heads or L != impl.kv_lora_rank or W_UV.shape[0] != N or W_UV.shape[1] != L:
+            raise ValueError("W_UK_T must be [num_heads, qk_nope_head_dim, kv_lora_rank] and W_UV "
+                             "[num_heads, kv_lora_rank, v_head_dim]")
+        self.impl = impl
+        self.W_UK_T = W_UK_T
+        self.W_UV = W_UV
+        self.num_heads = N
+        self.kv_lora_rank = L
+        self.v_head_dim = W_UV.shape[2]
+
+    def absorb_q(self, mqa_q_nope: torch.Tensor) -> torch.Tensor:
+        """``[B, N, P]`` -> ``[B, N, L]`` (a transposed view of the ``[N, B, L]`` product)."""
+        q = mqa_q_nope.transpose(0, 1)                       # (N, B, P)
+        ql = q.new_empty((self.num_heads, q.shape[1], self.kv_lora_rank))
+        torch.bmm(q, self.W_UK_T, out=ql)
+        return ql.transpose(0, 1)
+
+    def v_up_proj(self, x: torch.Tensor, out: torch.Tensor) -> None:
+        """``x [B, N, L]`` -> ``out [B, N * V]``."""
+        x = x.view(-1, self.num_heads, self.kv_lora_rank).transpose(0, 1)
+        out = out.view(-1, self.num_heads, self.v_head_dim)
+        torch.bmm(x, self.W_UV, out=out.transpose(0, 1))
+
+    def forward_decode(self, mqa_q_nope: torch.Tensor, mqa_q_pe: torch.Tensor, kv_cache: torch.Tensor,
+                       attn_metadata, out: torch.Tensor):
+        """q_nope ``[B, N, P]``, q_pe ``[B, N, rope]`` (already rotated), writes ``out [B, N * V]``;
+        returns the decode's ``lse [B, N]``."""
+        ql_nope = self.absorb_q(mqa_q_nope)
+        attn_out, lse = self.impl.forward_mqa((ql_nope, mqa_q_pe), kv_cache, attn_metadata)
+        self.v_up_proj(attn_out, out)
+        return lse
+
