@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define KVQ_ABI_VERSION 6
+#define KVQ_ABI_VERSION 7
 
 #define KVQ_OK 0
 #define KVQ_EINVAL (-22)
@@ -201,6 +201,23 @@ KVQ_API int kvq_swap_blocks(const void* src, void* dst, int64_t block_bytes,
 KVQ_API int kvq_swap_blocks_batch(const int64_t* src_ptrs, const int64_t* dst_ptrs,
                           const int64_t* sizes, int64_t n, int all_on_device,
                           kvq_stream_t stream);
+
+/*
+ * copy_blocks / copy_blocks_mla over the int8 format: for every (src, dst) row of
+ * block_mapping [num_pairs, 2] (int64, contiguous, ON THE DEVICE) and every
+ * layer, block dst of the layer's cache becomes a copy of block src -- the
+ * kernels of csrc/libtorch_stable/cache_kernels.cu:184-232, exercised by
+ * tests/kernels/attention/test_cache.py:55-110 and :592-650.  A block of these
+ * layouts holds keys, values and their scales, so one cache pointer per layer
+ * replaces the reference's key/value pointer pair.  cache_ptrs [num_layers]
+ * (int64 addresses, on the device); block_bytes = the cache's block stride;
+ * pairs naming a block outside [0, num_blocks) are skipped (the host cannot
+ * check a device-resident mapping without a synchronisation).  A source may be
+ * copied to several destinations; sources and destinations must not overlap.
+ */
+KVQ_API int kvq_copy_blocks(const int64_t* cache_ptrs, int num_layers, const int64_t* block_mapping,
+                            int64_t num_pairs, int64_t block_bytes, int64_t num_blocks,
+                            kvq_stream_t stream);
 
 /*
  * LSE merge of two partial attention states.  Stands in for merge_attn_states,

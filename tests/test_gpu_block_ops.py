@@ -151,6 +151,63 @@ def test_swap_blocks_batch(gpu_device, all_on_device):
         assert torch.equal(host[:5000], s_cpu[1234:6234]) and int(host[5000:].sum()) == 0
 
 
+@pytest.mark.parametrize("kind", ["gqa_nhd", "gqa_hnd", "mla"])
+@pytest.mark.parametrize("num_mappings,num_layers", [(1, 1), (7, 3), (60, 5)])
+def test_copy_blocks(gpu_device, kind, num_mappings, num_layers):
+    """The reference's test_copy_blocks / test_copy_blocks_mla (tests/kernels/attention/test_cache.py:
+    55-110, 592-650): every source block goes to TWO destinations, in every layer; compared with the
+    same copies done on clones.  Bytes must match, codes and scales alike."""
+    nb = 256
+    random.seed(num_mappings + num_layers)
+    src_blocks = random.sample(range(nb), num_mappings)
+    rest = list(set(range(nb)) - set(src_blocks))
+    dst_blocks = random.sample(rest, 2 * num_mappings)
+    mapping = []
+    for i, s_ in enumerate(src_blocks):
+        mapping += [(s_, dst_blocks[2 * i]), (s_, dst_blocks[2 * i + 1])]
+    caches = []
+    for _ in range(num_layers):
+        if kind == "mla":
+            kv = L.allocate_mla_cache(nb, 64, 576, device=gpu_device)
+            kv.view(torch.uint8).random_(0, 256)
+        else:
+            kv = L.allocate_kv_cache(nb, 16, 4, 128, device=gpu_device, layout="NHD" if kind == "gqa_nhd" else "HND", fill=None)
+            as_blocks(kv).random_(0, 256)
+        caches.append(kv)
+    raw = (lambda kv: kv.view(torch.uint8).reshape(nb, -1)) if kind == "mla" else as_blocks
+    want = [raw(kv).cpu().clone() for kv in caches]
+    for s_, d_ in mapping:
+        for w in want:
+            w[d_] = w[s_]
+    mapping_t = torch.tensor(mapping, dtype=torch.int64, device=gpu_device).view(-1, 2)
+    (ops.copy_blocks_mla if kind == "mla" else ops.copy_blocks)(caches, mapping_t)
+    torch.cuda.synchronize()
+    for kv, w in zip(caches, want):
+        assert torch.equal(raw(kv).cpu(), w)
+
+
+def test_copy_blocks_skips_bad_pairs_and_checks_arguments(gpu_device):
+    nb = 16
+    kv = L.allocate_kv_cache(nb, 16, 2, 64, device=gpu_device, fill=None)
+    as_blocks(kv).random_(0, 256)
+    before = as_blocks(kv).cpu().clone()
+    mapping = torch.tensor([[3, 5], [2, 99], [-1, 4], [7, 7]], dtype=torch.int64, device=gpu_device)
+    ops.copy_blocks([kv], mapping)                          # one valid pair; the others name no block
+    torch.cuda.synchronize()
+    want = before.clone()
+    want[5] = before[3]
+    assert torch.equal(as_blocks(kv).cpu(), want)
+    ops.copy_blocks([], mapping)
+    ops.copy_blocks([kv], torch.zeros((0, 2), dtype=torch.int64, device=gpu_device))
+    with pytest.raises(RuntimeError):                       # mapping on the CPU
+        ops.copy_blocks([kv], mapping.cpu())
+    with pytest.raises(RuntimeError):
+        ops.copy_blocks([kv], mapping.to(torch.int32))
+    other = L.allocate_kv_cache(nb + 1, 16, 2, 64, device=gpu_device, fill=None)
+    with pytest.raises(RuntimeError):                       # layers of different shapes
+        ops.copy_blocks([kv, other], mapping)
+
+
 def test_argument_errors(gpu_device):
     kv = L.allocate_kv_cache(8, 16, 2, 64, device=gpu_device)
     cpu = L.allocate_kv_cache(8, 16, 2, 64, device="cpu")

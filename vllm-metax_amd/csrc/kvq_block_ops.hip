@@ -55,9 +55,46 @@ __global__ __launch_bounds__(256) void copy_triples_kernel(CopyTriples t) {
   }
 }
 
+// copy_blocks: every (src, dst) pair of a device-resident mapping, in every layer's cache, in one
+// launch: grid (slices per block, pairs, layers).  num_blocks bounds the block numbers read from the
+// mapping (a pair outside it is skipped: the host cannot see the mapping without a synchronisation).
+__global__ __launch_bounds__(256) void copy_blocks_kernel(const int64_t* __restrict__ cache_ptrs,
+                                                          const int64_t* __restrict__ block_mapping,
+                                                          int64_t block_bytes, int64_t num_blocks, int vec16) {
+  uint8_t* cache = reinterpret_cast<uint8_t*>(cache_ptrs[blockIdx.z]);
+  const int64_t src = block_mapping[2 * (int64_t)blockIdx.y], dst = block_mapping[2 * (int64_t)blockIdx.y + 1];
+  if (src < 0 || dst < 0 || src >= num_blocks || dst >= num_blocks || src == dst) return;
+  const int64_t begin = (int64_t)blockIdx.x * kSliceBytes;
+  const int64_t end = begin + kSliceBytes < block_bytes ? begin + kSliceBytes : block_bytes;
+  const uint8_t* s = cache + src * block_bytes + begin;
+  uint8_t* d = cache + dst * block_bytes + begin;
+  if (vec16 && ((reinterpret_cast<uintptr_t>(cache) & 15) == 0)) {
+    const int n = (int)((end - begin) / 16);
+    for (int i = threadIdx.x; i < n; i += 256) reinterpret_cast<u32x4*>(d)[i] = reinterpret_cast<const u32x4*>(s)[i];
+  } else {
+    for (int64_t i = threadIdx.x; i < end - begin; i += 256) d[i] = s[i];
+  }
+}
+
 }  // namespace kvq
 
 extern "C" {
+
+int kvq_copy_blocks(const int64_t* cache_ptrs, int num_layers, const int64_t* block_mapping, int64_t num_pairs,
+                    int64_t block_bytes, int64_t num_blocks, kvq_stream_t stream) {
+  using namespace kvq;
+  const char* op = "copy_blocks";
+  KVQ_REQUIRE(num_layers >= 0 && num_pairs >= 0, "%s: negative count", op);
+  if (num_layers == 0 || num_pairs == 0) return KVQ_OK;
+  KVQ_REQUIRE(cache_ptrs && block_mapping, "%s: NULL pointer", op);
+  KVQ_REQUIRE(block_bytes > 0 && num_blocks > 0, "%s: block_bytes and num_blocks must be positive", op);
+  KVQ_REQUIRE(num_layers <= 65535 && num_pairs <= 65535, "%s: at most 65535 layers and 65535 pairs per call", op);
+  const int64_t slices = (block_bytes + kSliceBytes - 1) / kSliceBytes;
+  KVQ_REQUIRE(slices <= 0x7fffffff, "%s: block_bytes out of range", op);
+  hipLaunchKernelGGL(copy_blocks_kernel, dim3((unsigned)slices, (unsigned)num_pairs, (unsigned)num_layers), dim3(256), 0,
+                     as_stream(stream), cache_ptrs, block_mapping, block_bytes, num_blocks, block_bytes % 16 == 0 ? 1 : 0);
+  return check_hip(hipGetLastError(), "copy_blocks launch");
+}
 
 int kvq_swap_blocks(const void* src, void* dst, int64_t block_bytes, const int64_t* block_mapping,
                     int64_t num_pairs, int64_t map_stride0, int64_t map_stride1, int direction,

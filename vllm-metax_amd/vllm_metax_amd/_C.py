@@ -13,7 +13,7 @@ _LIB_DIR = os.path.join(os.path.dirname(os.path.abspath(__file__)), "_lib")
 LIB_PATH = os.path.join(_LIB_DIR, "libkvq_hip.so")
 
 KVQ_F32, KVQ_BF16, KVQ_F16 = 0, 1, 2
-ABI_VERSION = 6
+ABI_VERSION = 7
 
 
 class CacheGeom(ctypes.Structure):
@@ -57,6 +57,7 @@ SIGNATURES = {
     "kvq_splitk_reduce": (_i, [_vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
     "kvq_swap_blocks": (_i, [_vp, _vp, _i64, _vp, _i64, _i64, _i64, _i, _vp]),
     "kvq_swap_blocks_batch": (_i, [_vp, _vp, _vp, _i64, _i, _vp]),
+    "kvq_copy_blocks": (_i, [_vp, _i, _vp, _i64, _i64, _i64, _vp]),
     "kvq_merge_attn_states": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i64, _i, _i, _i64, _vp]),
     "kvq_concat_and_cache_mla_int8": (_i, [_vp, _vp, _i, _i64, _i64, _vp, _mla_p, _vp, _i64, _f, _vp]),
     "kvq_gather_and_dequant_mla_int8": (_i, [_vp, _i, _i64, _vp, _mla_p, _vp, _i64, _vp, _vp, _vp, _i64, _vp]),

@@ -419,6 +419,40 @@ def swap_blocks_batch(src_ptrs: torch.Tensor, dst_ptrs: torch.Tensor, sizes: tor
     _C.check(rc, "swap_blocks_batch")
 
 
+def copy_blocks(kv_caches: list[torch.Tensor], block_mapping: torch.Tensor) -> None:
+    """``copy_blocks`` / ``copy_blocks_mla`` over the int8 format (kernels
+    csrc/libtorch_stable/cache_kernels.cu:184-232; tests/kernels/attention/test_cache.py:55-110,
+    592-650): block ``dst`` of EVERY layer's cache becomes a copy of block ``src`` for every row
+    ``(src, dst)`` of ``block_mapping`` (``[num_pairs, 2]`` int64, on the GPU, as in the
+    reference's test).  A block of these layouts holds keys, values and scales, so one cache list
+    replaces the reference's key / value lists.  All caches share shape and block stride."""
+    if len(kv_caches) == 0:
+        return
+    dev = _require_cuda(*kv_caches, block_mapping)
+    if block_mapping.dtype != torch.int64 or block_mapping.dim() != 2 or block_mapping.shape[1] != 2 \
+            or not block_mapping.is_contiguous():
+        raise RuntimeError("block_mapping must be a contiguous [num_pairs, 2] int64 tensor")
+    first = kv_caches[0]
+    block_bytes = first.stride(0) * first.element_size()
+    for t in kv_caches:
+        if t.shape != first.shape or t.stride() != first.stride() or t.dtype != first.dtype:
+            raise RuntimeError("every layer's cache must have the same shape, strides and dtype")
+    num_pairs = block_mapping.shape[0]
+    if num_pairs == 0:
+        return
+    ptrs = torch.tensor([t.data_ptr() for t in kv_caches], dtype=torch.int64).to(dev)
+    with _on_device(dev):
+        rc = _C.load().kvq_copy_blocks(_ptr(ptrs), len(kv_caches), _ptr(block_mapping), num_pairs, block_bytes,
+                                       first.shape[0], _stream(dev))
+        # the pointer table must outlive the launch that reads it
+        ptrs.record_stream(torch.cuda.current_stream(dev))
+    _C.check(rc, "copy_blocks")
+
+
+# the latent cache is one joint tensor per layer as well
+copy_blocks_mla = copy_blocks
+
+
 def merge_attn_states(output: torch.Tensor, prefix_output: torch.Tensor, prefix_lse: torch.Tensor,
                       suffix_output: torch.Tensor, suffix_lse: torch.Tensor,
                       output_lse: torch.Tensor | None = None, prefill_tokens_with_context: int | None = None) -> None:
