@@ -129,3 +129,31 @@ def test_builder_packs_metadata_without_touching_the_gpu():
     c.num_reqs = 5
     with pytest.raises(RuntimeError):
         b.build(0, c)
+
+
+def test_ops_refuse_cpu_tensors_and_bad_shapes_before_touching_the_library():
+    """There is no CPU path: every op raises RuntimeError on host tensors (the product must fail
+    loudly, never fall back), and shape / dtype mistakes are reported by the wrappers themselves."""
+    import pytest
+    import torch
+
+    from vllm_metax_amd import _custom_ops as ops
+    from vllm_metax_amd import layout as L
+
+    a = torch.zeros((2, 4, 512), dtype=torch.bfloat16)
+    b = torch.zeros((2, 4, 64), dtype=torch.bfloat16)
+    out = torch.zeros((2, 4, 576), dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError):
+        ops.concat_mla_q(a, b, out)
+    kv = L.allocate_kv_cache(4, 16, 2, 64, device="cpu")
+    with pytest.raises(RuntimeError):
+        ops.copy_blocks([kv], torch.zeros((1, 2), dtype=torch.int64))
+    ops.copy_blocks([], torch.zeros((1, 2), dtype=torch.int64))          # nothing to do: no library call
+    cache = L.allocate_mla_cache(2, 64, 576, device="cpu")
+    o = torch.zeros((2, 4, 512), dtype=torch.bfloat16)
+    bt = torch.zeros((2, 1), dtype=torch.int32)
+    sl = torch.ones(2, dtype=torch.int32)
+    with pytest.raises(RuntimeError):
+        ops.mla_decode_int8((a, b), cache, o, None, bt, sl, 0.1, 512)
+    with pytest.raises(RuntimeError):
+        ops.mla_decode_int8(out, cache, o, None, bt, sl, 0.1, 512)
