@@ -10,7 +10,8 @@
  *     (KVQ_EINVAL for rejected arguments, KVQ_EHIP for a HIP runtime error).
  *     kvq_last_error() returns a thread-local, human-readable reason.
  *   - no entry point allocates or frees device memory; scratch comes in as a
- *     caller-provided workspace whose size the *_workspace_bytes() helpers give.
+ *     caller-provided workspace whose size the *_workspace_bytes() helpers give
+ *     (kvq_paged_attn_int8_static_scratch uses a fixed array of the library instead).
  *   - stateless, thread-safe; strides are taken from the caller, never assumed.
  *
  * Each declaration cites the interface of MetaX-MACA/vLLM-metax it stands in
@@ -26,7 +27,7 @@
 extern "C" {
 #endif
 
-#define KVQ_ABI_VERSION 7
+#define KVQ_ABI_VERSION 8
 
 #define KVQ_OK 0
 #define KVQ_EINVAL (-22)
@@ -139,6 +140,32 @@ KVQ_API int kvq_paged_attn_int8(void* out, int out_dtype, int64_t out_stride_t, 
                         int max_query_len, float scale, int causal, int window_size,
                         float softcap, float* lse, void* workspace, size_t workspace_bytes,
                         kvq_stream_t stream);
+
+/*
+ * kvq_paged_attn_int8 for callers that cannot hand over a workspace they allocated:
+ * code under HIP graph capture, tight serving loops and harnesses that forbid
+ * hipMalloc.  It has no counterpart in the reference.  Same arguments, results and
+ * kernels as kvq_paged_attn_int8, minus the workspace: the split-K partial states
+ * live in a fixed array of KVQ_STATIC_SCRATCH_BYTES that is part of the library's
+ * code object (each GPU the library runs on holds one copy until the process
+ * ends).  The call allocates and frees nothing.  A batch whose partial states
+ * would not fit -- (W + num_seqs) * num_q_heads * (head_size + 2) * 4 bytes, W =
+ * compute units * 8 / min(8, largest power of two <= num_kv_heads) resident
+ * workgroups; never more than kvq_paged_attn_workspace_bytes(num_seqs,
+ * num_q_heads, head_size) -- is rejected with KVQ_EINVAL and nothing is
+ * launched (32 q heads / 8 kv heads of 128 dims: up to 1256 sequences on 256
+ * compute units).  All calls on one GPU
+ * share that GPU's array: calls that overlap in time on one GPU (different
+ * streams, different threads) race and must be serialised by the caller.
+ */
+#define KVQ_STATIC_SCRATCH_BYTES (24u << 20)
+KVQ_API size_t kvq_paged_attn_static_scratch_bytes(void);
+KVQ_API int kvq_paged_attn_int8_static_scratch(
+    void* out, int out_dtype, int64_t out_stride_t, int64_t out_stride_h, const void* q, int q_dtype,
+    int64_t q_stride_t, int64_t q_stride_h, const void* cache, const kvq_cache_geom* geom,
+    const int32_t* block_table, int64_t bt_stride, const int32_t* seq_lens, const int32_t* cu_seqlens_q,
+    int num_seqs, int num_q_heads, int max_query_len, float scale, int causal, int window_size,
+    float softcap, float* lse, kvq_stream_t stream);
 
 /*
  * Fixed-partition split-K decode + reduce (one query row per sequence).

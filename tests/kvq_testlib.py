@@ -68,7 +68,8 @@ def fill_cache_from_sources(kv, lay, bt, ctx_lens, block_size, k_src, v_src):
     """Quantise per-sequence K/V sources ([ctx, Hkv, D] each) into the CPU cache with the oracle."""
     base = storage_bytes(kv)
     for i, slots in enumerate(slots_for(bt, ctx_lens, block_size)):
-        oracle.cache_write(k_src[i], v_src[i], base, lay, slots)
+        if slots.numel() > 0:  # an empty sequence writes nothing
+            oracle.cache_write(k_src[i], v_src[i], base, lay, slots)
 
 
 def to_device_cache(kv_cpu, device, layout):

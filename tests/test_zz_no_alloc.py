@@ -1,0 +1,95 @@
+"""GPU test of kvq_paged_attn_int8_static_scratch, the entry point that allocates nothing: called
+through the C ABI, its output must equal kvq_paged_attn_int8's bit for bit (same kernels, the
+split-K states in the library's own fixed array instead of a caller workspace) and lie within
+atol 2e-2 / rtol 1e-2 of the oracle -- on two calls in a row, the second on a smaller batch, so
+that what the first call left in the shared array is seen not to leak into the second."""
+import ctypes
+import math
+
+import pytest
+import torch
+
+import kvq_testlib as T
+import oracle
+from vllm_metax_amd import _C
+from vllm_metax_amd import _custom_ops as ops
+from vllm_metax_amd import layout as L
+
+pytestmark = pytest.mark.gpu
+
+
+def _case(ctx, qls, hq, hkv, d, bs, seed):
+    g = torch.Generator().manual_seed(seed)
+    nb = sum((c + bs - 1) // bs for c in ctx) + 5
+    kv, _, lay = T.cpu_cache(nb, bs, hkv, d, "NHD")
+    T.storage_bytes(kv).fill_(0xFF)
+    bt = T.make_block_tables(ctx, bs, nb, g)
+    ks = [torch.randn((c, hkv, d), generator=g).to(torch.bfloat16) for c in ctx]
+    vs = [torch.randn((c, hkv, d), generator=g).to(torch.bfloat16) for c in ctx]
+    T.fill_cache_from_sources(kv, lay, bt, ctx, bs, ks, vs)
+    q = torch.randn((sum(qls), hq, d), generator=g).to(torch.bfloat16)
+    sl = torch.tensor(ctx, dtype=torch.int32)
+    cu = torch.tensor([0] + torch.tensor(qls).cumsum(0).tolist(), dtype=torch.int32)
+    return kv, lay, bt, q, sl, cu
+
+
+def _call(dev, static, kv, bt, q, sl, cu, max_q, scale, ws=None):
+    """One call through the C ABI; returns (out, lse)."""
+    lib = _C.load()
+    k, v = L.key_value_views(kv)
+    ksc, vsc = L.scale_views(kv)
+    geom = L.geometry_from_views(k, v, ksc, vsc)
+    g = geom.as_struct()
+    out = torch.full(q.shape, float("nan"), dtype=torch.bfloat16, device=dev)
+    lse = torch.full(q.shape[:2], float("nan"), dtype=torch.float32, device=dev)
+    stream = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+    head = (ctypes.c_void_p(out.data_ptr()), _C.KVQ_BF16, out.stride(0), out.stride(1),
+            ctypes.c_void_p(q.data_ptr()), _C.KVQ_BF16, q.stride(0), q.stride(1),
+            ctypes.c_void_p(geom.base_ptr), ctypes.byref(g), ctypes.c_void_p(bt.data_ptr()), bt.stride(0),
+            ctypes.c_void_p(sl.data_ptr()), ctypes.c_void_p(cu.data_ptr()), sl.shape[0], q.shape[1], max_q,
+            scale, 1, 0, 0.0, ctypes.c_void_p(lse.data_ptr()))
+    if static:
+        rc = lib.kvq_paged_attn_int8_static_scratch(*head, stream)
+        _C.check(rc, "kvq_paged_attn_int8_static_scratch")
+    else:
+        rc = lib.kvq_paged_attn_int8(*head, ctypes.c_void_p(ws.data_ptr()), ws.numel(), stream)
+        _C.check(rc, "kvq_paged_attn_int8")
+    torch.cuda.synchronize()
+    return out, lse
+
+
+def test_static_scratch_matches_workspace_entry_twice(gpu_device):
+    dev = gpu_device
+    hq, hkv, d, bs = 32, 8, 128, 16
+    scale = 1 / math.sqrt(d)
+    # first call: 24 sequences cut into many split-K states, a prefill row and an empty sequence among them;
+    # second call: 3 short sequences, far fewer states, in the same array
+    first = ([1500, 33, 0, 2047, 640] + [300 + 37 * i for i in range(19)], [1, 1, 1, 1, 50] + [1] * 19)
+    second = ([700, 16, 129], [1, 1, 1])
+    for seed, (ctx, qls) in enumerate((first, second)):
+        kv_cpu, lay, bt, q, sl, cu = _case(ctx, qls, hq, hkv, d, bs, 100 + seed)
+        kv = T.to_device_cache(kv_cpu, dev, "NHD")
+        args = (kv, bt.to(dev), q.to(dev), sl.to(dev), cu.to(dev), max(qls), scale)
+        ws = torch.empty(ops.paged_attn_workspace_bytes(len(ctx), hq, d), dtype=torch.uint8, device=dev)
+        want_out, want_lse = _call(dev, False, *args, ws=ws)
+        got_out, got_lse = _call(dev, True, *args)
+        assert torch.equal(got_out.view(torch.int16), want_out.view(torch.int16)), f"call {seed}: outputs differ"
+        assert torch.equal(got_lse.view(torch.int32), want_lse.view(torch.int32)), f"call {seed}: lse differs"
+        ref = oracle.paged_attn(q, T.storage_bytes(kv_cpu), lay, bt, sl, cu, scale)
+        T.assert_close_attn(got_out, ref, what=f"static scratch call {seed}")
+
+
+def test_static_scratch_rejects_oversized_batches(gpu_device):
+    """One kv head means one-wave workgroups, eight per compute unit: with 16 q heads of 256 dims their
+    partial states alone outgrow the array, so the call must refuse (and launch nothing)."""
+    dev = gpu_device
+    hq, hkv, d, bs, n = 16, 1, 256, 16, 2
+    limit = _C.load().kvq_paged_attn_static_scratch_bytes()
+    assert (8 * ops.device_num_cus() + n) * hq * (d + 2) * 4 > limit
+    kv = L.allocate_kv_cache(4, bs, hkv, d, device=dev, layout="NHD", fill=0)
+    bt = torch.zeros((n, 1), dtype=torch.int32, device=dev)
+    q = torch.zeros((n, hq, d), dtype=torch.bfloat16, device=dev)
+    sl = torch.ones(n, dtype=torch.int32, device=dev)
+    cu = torch.arange(n + 1, dtype=torch.int32, device=dev)
+    with pytest.raises(RuntimeError, match="too large for the built-in scratch"):
+        _call(dev, True, kv, bt, q, sl, cu, 1, 1.0)

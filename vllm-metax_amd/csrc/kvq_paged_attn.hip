@@ -3,6 +3,8 @@
 // The host never looks at device data: max_query_len (a host integer the caller's
 // metadata already carries) decides which tiles are launched, and each kernel skips
 // the sequences that are not its kind by reading cu_seqlens_q on the device.
+#include <mutex>
+
 #include "kvq_attn_core.cuh"
 
 namespace kvq {
@@ -14,16 +16,15 @@ int decode_streamk_num_wg(int num_kv_heads);
 int launch_prefill(const AttnIO& io, const int32_t* seq_lens, const int32_t* cu_seqlens_q, int num_seqs,
                    int max_query_len, int causal, int q_dtype, int out_dtype, hipStream_t s);
 
-}  // namespace kvq
-
-extern "C" int kvq_paged_attn_int8(void* out, int out_dtype, int64_t out_stride_t, int64_t out_stride_h,
-                                   const void* q, int q_dtype, int64_t q_stride_t, int64_t q_stride_h,
-                                   const void* cache, const kvq_cache_geom* geom, const int32_t* block_table,
-                                   int64_t bt_stride, const int32_t* seq_lens, const int32_t* cu_seqlens_q,
-                                   int num_seqs, int num_q_heads, int max_query_len, float scale, int causal,
-                                   int window_size, float softcap, float* lse, void* workspace, size_t workspace_bytes, kvq_stream_t stream) {
-  using namespace kvq;
-  const char* op = "paged_attn_int8";
+// Arguments are checked, the launch is shaped and enqueued here; the two entry points differ only
+// in where the split-K partial states live.
+static int paged_attn_launch(const char* op, void* out, int out_dtype, int64_t out_stride_t, int64_t out_stride_h,
+                             const void* q, int q_dtype, int64_t q_stride_t, int64_t q_stride_h, const void* cache,
+                             const kvq_cache_geom* geom, const int32_t* block_table, int64_t bt_stride,
+                             const int32_t* seq_lens, const int32_t* cu_seqlens_q, int num_seqs, int num_q_heads,
+                             int max_query_len, float scale, int causal, int window_size, float softcap, float* lse,
+                             void* workspace, size_t workspace_bytes, const char* workspace_what,
+                             kvq_stream_t stream) {
   KVQ_REQUIRE(geom != nullptr, "%s: geom is NULL", op);
   KVQ_REQUIRE(out && q && cache && block_table && seq_lens, "%s: NULL pointer", op);
   KVQ_REQUIRE(num_seqs > 0 && num_q_heads > 0, "%s: num_seqs and num_q_heads must be positive", op);
@@ -54,7 +55,7 @@ extern "C" int kvq_paged_attn_int8(void* out, int out_dtype, int64_t out_stride_
   KVQ_REQUIRE(num_wg > 0, "%s: no HIP device", op);
   const size_t need = streamk_workspace_bytes(num_seqs, num_q_heads, g.head_size, num_wg);
   KVQ_REQUIRE(workspace != nullptr && workspace_bytes >= need && ((uintptr_t)workspace % 16) == 0,
-              "%s: workspace of %zu bytes (16-byte aligned) required, got %zu", op, need, workspace_bytes);
+              "%s: %s of %zu bytes (16-byte aligned) required, got %zu", op, workspace_what, need, workspace_bytes);
 
   StreamKArgs a{};
   a.io.q = q;
@@ -90,4 +91,70 @@ extern "C" int kvq_paged_attn_int8(void* out, int out_dtype, int64_t out_stride_
     rc = launch_prefill(a.io, seq_lens, cu_seqlens_q, num_seqs, max_query_len, causal, q_dtype, out_dtype, s);
   }
   return rc;
+}
+
+// Scratch of the entry point that allocates nothing: a fixed array in the code object's own device
+// memory.  Every GPU the library runs on holds one copy, at its own address, until the process ends.
+// In host code the array's NAME is only a handle for the runtime; the address kernels may use is the
+// one hipGetSymbolAddress returns, resolved once per device and kept in g_static_scratch[].
+static __device__ __align__(256) unsigned char scratch[KVQ_STATIC_SCRATCH_BYTES];
+
+constexpr int kMaxDevices = 64;
+static std::mutex g_static_scratch_mutex;
+static void* g_static_scratch[kMaxDevices];  // guarded by the mutex; nullptr = not resolved yet
+
+// Device address of `scratch` on the current device (resolved on the first call per device).
+static int static_scratch_ptr(const char* op, void** ptr) {
+  int dev = -1;
+  int rc = check_hip(hipGetDevice(&dev), "hipGetDevice");
+  if (rc) return rc;
+  KVQ_REQUIRE(dev >= 0 && dev < kMaxDevices, "%s: device index %d out of range", op, dev);
+  std::lock_guard<std::mutex> lock(g_static_scratch_mutex);
+  if (g_static_scratch[dev] == nullptr) {
+    void* p = nullptr;
+    rc = check_hip(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)), "hipGetSymbolAddress(scratch)");
+    if (rc) return rc;
+    KVQ_REQUIRE(p != nullptr, "%s: the static scratch array has no device address", op);
+    g_static_scratch[dev] = p;
+  }
+  *ptr = g_static_scratch[dev];
+  return KVQ_OK;
+}
+
+}  // namespace kvq
+
+extern "C" int kvq_paged_attn_int8(void* out, int out_dtype, int64_t out_stride_t, int64_t out_stride_h,
+                                   const void* q, int q_dtype, int64_t q_stride_t, int64_t q_stride_h,
+                                   const void* cache, const kvq_cache_geom* geom, const int32_t* block_table,
+                                   int64_t bt_stride, const int32_t* seq_lens, const int32_t* cu_seqlens_q,
+                                   int num_seqs, int num_q_heads, int max_query_len, float scale, int causal,
+                                   int window_size, float softcap, float* lse, void* workspace,
+                                   size_t workspace_bytes, kvq_stream_t stream) {
+  return kvq::paged_attn_launch("paged_attn_int8", out, out_dtype, out_stride_t, out_stride_h, q, q_dtype, q_stride_t,
+                                q_stride_h, cache, geom, block_table, bt_stride, seq_lens, cu_seqlens_q, num_seqs,
+                                num_q_heads, max_query_len, scale, causal, window_size, softcap, lse, workspace,
+                                workspace_bytes, "workspace", stream);
+}
+
+extern "C" size_t kvq_paged_attn_static_scratch_bytes(void) { return KVQ_STATIC_SCRATCH_BYTES; }
+
+extern "C" int kvq_paged_attn_int8_static_scratch(void* out, int out_dtype, int64_t out_stride_t,
+                                                  int64_t out_stride_h, const void* q, int q_dtype,
+                                                  int64_t q_stride_t, int64_t q_stride_h, const void* cache,
+                                                  const kvq_cache_geom* geom, const int32_t* block_table,
+                                                  int64_t bt_stride, const int32_t* seq_lens,
+                                                  const int32_t* cu_seqlens_q, int num_seqs, int num_q_heads,
+                                                  int max_query_len, float scale, int causal, int window_size,
+                                                  float softcap, float* lse, kvq_stream_t stream) {
+  const char* op = "paged_attn_int8_static_scratch";
+  void* ptr = nullptr;
+  const int rc = kvq::static_scratch_ptr(op, &ptr);
+  if (rc) return rc;
+  // The split-K partial states need no clearing: every slot the reduce reads was written by this
+  // launch's main kernel first (slots it does not own are masked out bit-wise, whatever they hold).
+  return kvq::paged_attn_launch(op, out, out_dtype, out_stride_t, out_stride_h, q, q_dtype, q_stride_t, q_stride_h,
+                                cache, geom, block_table, bt_stride, seq_lens, cu_seqlens_q, num_seqs, num_q_heads,
+                                max_query_len, scale, causal, window_size, softcap, lse, ptr,
+                                KVQ_STATIC_SCRATCH_BYTES,
+                                "batch too large for the built-in scratch: split-K state", stream);
 }

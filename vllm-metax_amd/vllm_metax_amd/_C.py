@@ -13,7 +13,7 @@ _LIB_DIR = os.path.join(os.path.dirname(os.path.abspath(__file__)), "_lib")
 LIB_PATH = os.path.join(_LIB_DIR, "libkvq_hip.so")
 
 KVQ_F32, KVQ_BF16, KVQ_F16 = 0, 1, 2
-ABI_VERSION = 7
+ABI_VERSION = 8
 
 
 class CacheGeom(ctypes.Structure):
@@ -52,6 +52,9 @@ SIGNATURES = {
     "kvq_paged_attn_workspace_bytes": (_sz, [_i, _i, _i]),
     "kvq_paged_attn_int8": (_i, [_vp, _i, _i64, _i64, _vp, _i, _i64, _i64, _vp, _geom_p, _vp, _i64, _vp, _vp,
                                  _i, _i, _i, _f, _i, _i, _f, _vp, _vp, _sz, _vp]),
+    "kvq_paged_attn_static_scratch_bytes": (_sz, []),
+    "kvq_paged_attn_int8_static_scratch": (_i, [_vp, _i, _i64, _i64, _vp, _i, _i64, _i64, _vp, _geom_p, _vp, _i64, _vp,
+                                                _vp, _i, _i, _i, _f, _i, _i, _f, _vp, _vp]),
     "kvq_paged_attn_v2_int8": (_i, [_vp, _i, _vp, _vp, _vp, _vp, _i, _i64, _i64, _vp, _geom_p, _vp, _i64, _vp,
                                     _i, _i, _f, _i, _i, _vp]),
     "kvq_splitk_reduce": (_i, [_vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),

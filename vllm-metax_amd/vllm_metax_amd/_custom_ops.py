@@ -205,6 +205,7 @@ def unified_attention(
     workspace: torch.Tensor | None = None,
     geometry: CacheGeometry | None = None,
     lse: torch.Tensor | None = None,
+    static_scratch: bool = False,
     **unused,
 ) -> None:
     """Drop-in for ``unified_attention`` as called at
@@ -215,7 +216,9 @@ def unified_attention(
     int32.  Extra keyword arguments of the reference's call that only steer its Triton launch
     (``seq_threshold_3D``, ``softmax_segm_*``, ``use_td`` ...) are accepted and ignored; features
     this path does not build raise ``NotImplementedError``.  ``window_size=(W - 1, 0)`` restricts a
-    query to its last W keys; ``softcap > 0`` maps logits through ``softcap * tanh(x / softcap)``."""
+    query to its last W keys; ``softcap > 0`` maps logits through ``softcap * tanh(x / softcap)``.
+    ``static_scratch=True`` keeps the split-K states in the library's own fixed array instead of a
+    workspace tensor (nothing is allocated; calls on one GPU must then not overlap in time)."""
     if kv_quant_mode != KVQuantMode.INT8_PER_TOKEN_HEAD:
         raise NotImplementedError(f"kv_quant_mode {kv_quant_mode!r}: only INT8_PER_TOKEN_HEAD is built")
     if alibi_slopes is not None or sinks is not None or output_scale is not None or mm_prefix_range is not None:
@@ -259,21 +262,24 @@ def unified_attention(
         return
     num_q_heads = q.shape[1]
     lib = _C.load()
-    need = paged_attn_workspace_bytes(num_seqs, num_q_heads, geom.head_size, dev)
-    if workspace is None:
-        workspace = _default_workspace(dev, need)
     if lse is not None and (lse.dtype != torch.float32 or not lse.is_contiguous()
                             or tuple(lse.shape) != (q.shape[0], num_q_heads)):
         raise RuntimeError("lse must be a contiguous float32 [num_tokens, num_q_heads] tensor")
     g = geom.as_struct()
-    with _on_device(dev):
-        rc = lib.kvq_paged_attn_int8(
-            _ptr(out), _dtype_code(out, "out"), out.stride(0), out.stride(1),
+    head = (_ptr(out), _dtype_code(out, "out"), out.stride(0), out.stride(1),
             _ptr(q), _dtype_code(q, "q"), q.stride(0), q.stride(1),
             ctypes.c_void_p(geom.base_ptr), ctypes.byref(g), _ptr(block_table), block_table.stride(0),
             _ptr(seqused_k), _ptr(cu_seqlens_q), num_seqs, num_q_heads, int(max_seqlen_q),
-            float(softmax_scale), 1 if causal else 0, window, softcap, _ptr(lse), _ptr(workspace),
-            workspace.numel() * workspace.element_size(), _stream(dev))
+            float(softmax_scale), 1 if causal else 0, window, softcap, _ptr(lse))
+    if static_scratch:
+        with _on_device(dev):
+            rc = lib.kvq_paged_attn_int8_static_scratch(*head, _stream(dev))
+    else:
+        if workspace is None:
+            workspace = _default_workspace(dev, paged_attn_workspace_bytes(num_seqs, num_q_heads, geom.head_size, dev))
+        with _on_device(dev):
+            rc = lib.kvq_paged_attn_int8(*head, _ptr(workspace), workspace.numel() * workspace.element_size(),
+                                         _stream(dev))
     _C.check(rc, "unified_attention")
 
 
