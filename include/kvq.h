@@ -149,12 +149,10 @@ KVQ_API int kvq_paged_attn_int8(void* out, int out_dtype, int64_t out_stride_t, 
  * live in a fixed array of KVQ_STATIC_SCRATCH_BYTES that is part of the library's
  * code object (each GPU the library runs on holds one copy until the process
  * ends).  The call allocates and frees nothing.  A batch whose partial states
- * would not fit -- (W + num_seqs) * num_q_heads * (head_size + 2) * 4 bytes, W =
- * compute units * 8 / min(8, largest power of two <= num_kv_heads) resident
- * workgroups; never more than kvq_paged_attn_workspace_bytes(num_seqs,
- * num_q_heads, head_size) -- is rejected with KVQ_EINVAL and nothing is
- * launched (32 q heads / 8 kv heads of 128 dims: up to 1256 sequences on 256
- * compute units).  All calls on one GPU
+ * would not fit -- kvq_paged_attn_workspace_bytes(num_seqs, num_q_heads,
+ * head_size) = (compute units + num_seqs) * num_q_heads * (head_size + 2) * 4
+ * bytes -- is rejected with KVQ_EINVAL and nothing is launched (32 q heads of
+ * 128 dims on 256 compute units: up to 1256 sequences).  All calls on one GPU
  * share that GPU's array: calls that overlap in time on one GPU (different
  * streams, different threads) race and must be serialised by the caller.
  */

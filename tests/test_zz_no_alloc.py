@@ -80,12 +80,11 @@ def test_static_scratch_matches_workspace_entry_twice(gpu_device):
 
 
 def test_static_scratch_rejects_oversized_batches(gpu_device):
-    """One kv head means one-wave workgroups, eight per compute unit: with 16 q heads of 256 dims their
-    partial states alone outgrow the array, so the call must refuse (and launch nothing)."""
+    """A batch whose split-K states outgrow the array must be refused (and nothing launched)."""
     dev = gpu_device
-    hq, hkv, d, bs, n = 16, 1, 256, 16, 2
+    hq, hkv, d, bs, n = 64, 8, 256, 16, 1200
     limit = _C.load().kvq_paged_attn_static_scratch_bytes()
-    assert (8 * ops.device_num_cus() + n) * hq * (d + 2) * 4 > limit
+    assert ops.paged_attn_workspace_bytes(n, hq, d) > limit
     kv = L.allocate_kv_cache(4, bs, hkv, d, device=dev, layout="NHD", fill=0)
     bt = torch.zeros((n, 1), dtype=torch.int32, device=dev)
     q = torch.zeros((n, hq, d), dtype=torch.bfloat16, device=dev)

@@ -77,6 +77,7 @@ struct AttnIO {
   int64_t q_stride_t, q_stride_h;
   void* out;
   int64_t out_stride_t, out_stride_h;
+  int out_dtype;  // read by kernels built for ODT == kRuntimeDtype
   float* lse;  // [rows, Hq] natural log, or nullptr
   // cache
   const uint8_t* cache;
@@ -160,7 +161,8 @@ struct DecodeTile {
   static constexpr int NCH = Tile::NCH;
   static constexpr int NLD = Tile::NLD;
   static constexpr int LDS_TILE = kTile * PITCH;          // bytes of the record window
-  static constexpr int LDS_WAVE = LDS_TILE + 64 * 4;      // + 64 staged scales
+  static constexpr int LDS_STATE = (DT + 1) * 1024;       // a wave's softmax state, dumped for a merge inside the workgroup
+  static constexpr int LDS_WAVE = LDS_TILE + 64 * 4 > LDS_STATE ? LDS_TILE + 64 * 4 : LDS_STATE;  // window + 64 staged scales
 
   __device__ static LaneOffsets lane_offsets(const kvq_cache_geom& G, int lane) {
     const int r = lane & 15, g = lane >> 4;
@@ -308,6 +310,11 @@ struct DecodeTile {
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    stage_scales(lo, sc_mul, lane, lds);
+  }
+
+  // The 64 scales of the window's 32 records, multiplied and capped, in the 256 bytes behind it.
+  __device__ static void stage_scales(const LaneOffsets& lo, float sc_mul, int lane, uint8_t* lds) {
     const float sc = *reinterpret_cast<const float*>(lds + lo.l_sc);
     reinterpret_cast<float*>(lds + LDS_TILE)[lane] = fminf(sc * sc_mul, 65504.f);
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -443,67 +450,111 @@ struct DecodeTile {
   // where it would wait on the newest loads instead of the oldest.
   __device__ static __forceinline__ void phase_fence() { __builtin_amdgcn_sched_barrier(0); }
 
-  // Run tiles [t_begin, t_end) of one sequence for kv head `hkv`; leaves the state in `st`.
+  // Run this wave's share of tiles [t_begin, t_end) of one sequence for kv head `hkv`; leaves the
+  // state in `st`.  The `nsub` waves that serve one kv head take the tiles in turn: wave `sub` owns
+  // tiles t_begin + sub, t_begin + sub + nsub, ... (one wave per kv head: nsub = 1, every tile).
   // One register buffer: as soon as a tile has been dropped into LDS its registers take the
-  // next tile, so one tile of loads per wave is in flight while one is computed (measured on
+  // wave's next tile, so one tile of loads per wave is in flight while one is computed (measured on
   // MI355X: a second tile in flight per wave lowers the achieved HBM bandwidth).
   // `lds` is this wave's private LDS_WAVE-byte window.
   // Tokens before `first` (the sliding window's lower edge; 0 without a window) do not contribute;
   // t_begin is then the tile that holds `first` or a later one.
+  // Every wave of the workgroup must call this with the same (t_begin, t_end, nsub): the rendezvous
+  // barriers inside are counted in rounds of nsub tiles, the same number for every wave, also for
+  // one that owns no tile of the range (its state stays empty: m = -inf).
   template <bool CAP>
   __device__ static void run(const AttnIO& io, int seq, int64_t row, int len, int first, int t_begin, int t_end, int hkv,
-                             int lane, uint8_t* lds, State& st) {
+                             int lane, uint8_t* lds, State& st, int sub = 0, int nsub = 1) {
     const LaneOffsets lo = lane_offsets(io.g, lane);
     const int32_t* bt_row = io.block_table + (int64_t)seq * io.bt_stride;
-    Tile a;
-    int t = t_begin;
-    // the first tile's loads go out before anything else of the run is touched
-    TileBlocks nb = fetch_blocks(io, bt_row, len, t);
-    load_tile(io, window(io, nb, t, hkv), lo, a);
-    phase_fence();
-    nb = fetch_blocks(io, bt_row, len, t + 1);  // block ids run one tile ahead of the loads
-    half8_t qb[KSTEPS];
-    const float s_init = load_q(io, row, hkv, lane, qb);
-    const float sc_mul = lane < 32 ? io.scale_log2 : kPScale;
+    const int rounds = (t_end - t_begin + nsub - 1) / nsub;
+    const int num_barriers = rounds / kSyncTiles;
+    int barriers = 0;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) st.o[dt] = (floatx4){0.f, 0.f, 0.f, 0.f};
     st.psum = (floatx4){0.f, 0.f, 0.f, 0.f};
     st.m = -INFINITY;
     st.l = 0.f;
-    // a first tile that straddles the window's lower edge is masked; it is peeled off so that the
-    // steady loop below keeps a single, unmasked body
-    if (t + 1 < t_end && t * kTile < first) {
-      const Window w = window(io, nb, t + 1, hkv);
+    int t = t_begin + sub;
+    if (t < t_end) {
+      Tile a;
+      // the first tile's loads go out before anything else of the run is touched
+      TileBlocks nb = fetch_blocks(io, bt_row, len, t);
+      load_tile(io, window(io, nb, t, hkv), lo, a);
+      phase_fence();
+      nb = fetch_blocks(io, bt_row, len, t + nsub);  // block ids run one tile ahead of the loads
+      half8_t qb[KSTEPS];
+      const float s_init = load_q(io, row, hkv, lane, qb);
+      const float sc_mul = lane < 32 ? io.scale_log2 : kPScale;
+      int r = 0;  // rounds this wave has finished
+      // a first tile that straddles the window's lower edge is masked; it is peeled off so that the
+      // steady loop below keeps a single, unmasked body
+      if (t + nsub < t_end && t * kTile < first) {
+        const Window w = window(io, nb, t + nsub, hkv);
+        stage(a, lo, sc_mul, lane, lds);
+        phase_fence();
+        load_tile(io, w, lo, a);
+        phase_fence();
+        nb = fetch_blocks(io, bt_row, len, t + 2 * nsub);
+        compute<true, CAP>(io, lo, qb, s_init, len, first, t, lane, lds, st);
+        phase_fence();
+        t += nsub;
+        ++r;
+        if ((r & (kSyncTiles - 1)) == 0) {
+          __builtin_amdgcn_s_barrier();
+          ++barriers;
+        }
+      }
+      // steady state: the wave's next tile exists, so the refill is unconditional and tile t does not
+      // end the sequence
+      while (t + nsub < t_end) {
+        const Window w = window(io, nb, t + nsub, hkv);
+        stage(a, lo, sc_mul, lane, lds);
+        phase_fence();
+        load_tile(io, w, lo, a);
+        phase_fence();
+        nb = fetch_blocks(io, bt_row, len, t + 2 * nsub);
+        compute<false, CAP>(io, lo, qb, s_init, len, first, t, lane, lds, st);
+        phase_fence();
+        t += nsub;
+        ++r;
+        // The waves of a workgroup read neighbouring records of the same tokens (one kv head each) or
+        // neighbouring tiles; the 128-byte lines at record boundaries are shared between them.  A
+        // rendezvous every few rounds keeps the waves within a few tiles of each other, so the second
+        // reader of such a line still finds it in L2 instead of fetching it from HBM again.
+        if ((r & (kSyncTiles - 1)) == 0) {
+          __builtin_amdgcn_s_barrier();
+          ++barriers;
+        }
+      }
       stage(a, lo, sc_mul, lane, lds);
-      phase_fence();
-      load_tile(io, w, lo, a);
-      phase_fence();
-      nb = fetch_blocks(io, bt_row, len, t + 2);
-      compute<true, CAP>(io, lo, qb, s_init, len, first, t, lane, lds, st);
-      phase_fence();
-      ++t;
+      compute_any<CAP>(io, lo, qb, s_init, len, first, t, lane, lds, st);
     }
-    // steady state: tile t+1 exists, so the refill is unconditional and tile t does not end the
-    // sequence
-    while (t + 1 < t_end) {
-      const Window w = window(io, nb, t + 1, hkv);
-      stage(a, lo, sc_mul, lane, lds);
-      phase_fence();
-      load_tile(io, w, lo, a);
-      phase_fence();
-      nb = fetch_blocks(io, bt_row, len, t + 2);
-      compute<false, CAP>(io, lo, qb, s_init, len, first, t, lane, lds, st);
-      phase_fence();
-      ++t;
-      // The waves of a workgroup read neighbouring records of the same tokens (one kv head each);
-      // the 128-byte lines at record boundaries are shared between them.  A rendezvous every few
-      // tiles keeps the waves within a few tiles of each other, so the second reader of such a
-      // line still finds it in L2 instead of fetching it from HBM again.  (Every wave of the
-      // workgroup runs the same tile range, so the barrier count is uniform.)
-      if ((t & (kSyncTiles - 1)) == 0) __builtin_amdgcn_s_barrier();
-    }
-    stage(a, lo, sc_mul, lane, lds);
-    compute_any<CAP>(io, lo, qb, s_init, len, first, t, lane, lds, st);
+    // the rendezvous count is the same for every wave of the workgroup, whatever its share of the tiles
+    for (; barriers < num_barriers; ++barriers) __builtin_amdgcn_s_barrier();
+  }
+
+  // ---- several waves per kv head: their states meet in LDS ------------------------------------
+  // Every wave but the head's first drops its state into its own LDS window (free once its tiles are
+  // done); after a workgroup barrier the first wave folds them into its own, in wave order.
+  __device__ static void dump_state(const State& st, int lane, uint8_t* lds) {
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) *reinterpret_cast<floatx4*>(lds + (dt * 64 + lane) * 16) = st.o[dt];
+    *reinterpret_cast<floatx4*>(lds + (DT * 64 + lane) * 16) = (floatx4){st.psum[0], st.m, st.l, 0.f};
+  }
+  __device__ static void fold_state(State& st, int lane, const uint8_t* lds) {
+    const floatx4 x = *reinterpret_cast<const floatx4*>(lds + (DT * 64 + lane) * 16);
+    const float mj = x.y;
+    const float m_new = fmaxf(st.m, mj);
+    // both states hold at least one token, so m_new is finite
+    const float a = __builtin_amdgcn_exp2f(st.m - m_new);
+    const float b = __builtin_amdgcn_exp2f(mj - m_new);
+    st.m = m_new;
+    st.l = st.l * a + x.z * b;
+    st.psum = st.psum * a + x.x * b;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+      st.o[dt] = st.o[dt] * a + *reinterpret_cast<const floatx4*>(lds + (dt * 64 + lane) * 16) * b;
   }
 
   // Sum of the lane-local l over the 4 lane groups of a head.
@@ -526,6 +577,16 @@ struct DecodeTile {
 
   // Whole sequence handled by this wave: normalise and write the output row (and lse).
   __device__ static void emit_final(const AttnIO& io, int64_t row, int hkv, int lane, const State& st) {
+    if constexpr (ODT == kRuntimeDtype) {
+      if (io.out_dtype == KVQ_F32) emit_final_as<KVQ_F32>(io, row, hkv, lane, st);
+      else if (io.out_dtype == KVQ_BF16) emit_final_as<KVQ_BF16>(io, row, hkv, lane, st);
+      else emit_final_as<KVQ_F16>(io, row, hkv, lane, st);
+    } else {
+      emit_final_as<ODT>(io, row, hkv, lane, st);
+    }
+  }
+  template <int OT>
+  __device__ static void emit_final_as(const AttnIO& io, int64_t row, int hkv, int lane, const State& st) {
     const float l = total_l(st);  // every lane takes part in the shuffles
     const int c = lane & 15, g = lane >> 4;
     if (c >= io.group) return;
@@ -533,7 +594,7 @@ struct DecodeTile {
     float v[D / 4];
     gather_row(st, 1.0f / (l * kPScale), v);
     const int64_t base = row * io.out_stride_t + (int64_t)head * io.out_stride_h + g * (D / 4);
-    if constexpr (ODT == KVQ_F32) {
+    if constexpr (OT == KVQ_F32) {
       float* o = reinterpret_cast<float*>(io.out) + base;
 #pragma unroll
       for (int i = 0; i < D / 4; i += 4) *reinterpret_cast<floatx4_a4*>(o + i) = (floatx4){v[i], v[i + 1], v[i + 2], v[i + 3]};
@@ -545,7 +606,7 @@ struct DecodeTile {
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           uint32_t w;
-          if constexpr (ODT == KVQ_BF16) {
+          if constexpr (OT == KVQ_BF16) {
             w = (uint32_t)f32_to_bf16_bits(v[i + 2 * j]) | ((uint32_t)f32_to_bf16_bits(v[i + 2 * j + 1]) << 16);
           } else {
             w = pack_half2(v[i + 2 * j], v[i + 2 * j + 1]);

@@ -66,6 +66,14 @@ __device__ __forceinline__ void store_act(void* p, int64_t i, float v) {
   else reinterpret_cast<half_t*>(p)[i] = (half_t)v;
 }
 
+// Output dtype known only at run time (one uniform branch per store).
+constexpr int kRuntimeDtype = -1;
+__device__ __forceinline__ void store_act_rt(int dtype, void* p, int64_t i, float v) {
+  if (dtype == KVQ_F32) store_act<KVQ_F32>(p, i, v);
+  else if (dtype == KVQ_BF16) store_act<KVQ_BF16>(p, i, v);
+  else store_act<KVQ_F16>(p, i, v);
+}
+
 __device__ __forceinline__ float wave_max(float v) {
 #pragma unroll
   for (int o = 32; o >= 1; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, kWave));

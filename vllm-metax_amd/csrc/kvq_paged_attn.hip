@@ -16,6 +16,37 @@ int decode_streamk_num_wg(int num_kv_heads);
 int launch_prefill(const AttnIO& io, const int32_t* seq_lens, const int32_t* cu_seqlens_q, int num_seqs,
                    int max_query_len, int causal, int q_dtype, int out_dtype, hipStream_t s);
 
+// Scratch of the entry point that allocates nothing: a fixed array in the code object's own device
+// memory.  Every GPU the library runs on holds one copy, at its own address, until the process ends.
+// In host code the array's NAME is only a handle for the runtime; the address kernels may use is the
+// one hipGetSymbolAddress returns, resolved once per device and kept in g_dev[].
+static __device__ __align__(256) unsigned char scratch[KVQ_STATIC_SCRATCH_BYTES];
+
+constexpr int kMaxDevices = 64;
+struct DeviceSymbols {
+  void* scratch = nullptr;
+};
+static std::mutex g_dev_mutex;
+static DeviceSymbols g_dev[kMaxDevices];  // guarded by the mutex; nullptr = not resolved yet
+
+// Device address of the array on the current device (resolved on the first call per device).
+static int device_symbols(const char* op, DeviceSymbols* out) {
+  int dev = -1;
+  int rc = check_hip(hipGetDevice(&dev), "hipGetDevice");
+  if (rc) return rc;
+  KVQ_REQUIRE(dev >= 0 && dev < kMaxDevices, "%s: device index %d out of range", op, dev);
+  std::lock_guard<std::mutex> lock(g_dev_mutex);
+  if (g_dev[dev].scratch == nullptr) {
+    void* p = nullptr;
+    rc = check_hip(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)), "hipGetSymbolAddress(scratch)");
+    if (rc) return rc;
+    KVQ_REQUIRE(p != nullptr, "%s: the static scratch array has no device address", op);
+    g_dev[dev].scratch = p;
+  }
+  *out = g_dev[dev];
+  return KVQ_OK;
+}
+
 // Arguments are checked, the launch is shaped and enqueued here; the two entry points differ only
 // in where the split-K partial states live.
 static int paged_attn_launch(const char* op, void* out, int out_dtype, int64_t out_stride_t, int64_t out_stride_h,
@@ -64,6 +95,7 @@ static int paged_attn_launch(const char* op, void* out, int out_dtype, int64_t o
   a.io.out = out;
   a.io.out_stride_t = out_stride_t;
   a.io.out_stride_h = out_stride_h;
+  a.io.out_dtype = out_dtype;
   a.io.lse = lse;
   a.io.cache = static_cast<const uint8_t*>(cache);
   a.io.g = g;
@@ -93,34 +125,6 @@ static int paged_attn_launch(const char* op, void* out, int out_dtype, int64_t o
   return rc;
 }
 
-// Scratch of the entry point that allocates nothing: a fixed array in the code object's own device
-// memory.  Every GPU the library runs on holds one copy, at its own address, until the process ends.
-// In host code the array's NAME is only a handle for the runtime; the address kernels may use is the
-// one hipGetSymbolAddress returns, resolved once per device and kept in g_static_scratch[].
-static __device__ __align__(256) unsigned char scratch[KVQ_STATIC_SCRATCH_BYTES];
-
-constexpr int kMaxDevices = 64;
-static std::mutex g_static_scratch_mutex;
-static void* g_static_scratch[kMaxDevices];  // guarded by the mutex; nullptr = not resolved yet
-
-// Device address of `scratch` on the current device (resolved on the first call per device).
-static int static_scratch_ptr(const char* op, void** ptr) {
-  int dev = -1;
-  int rc = check_hip(hipGetDevice(&dev), "hipGetDevice");
-  if (rc) return rc;
-  KVQ_REQUIRE(dev >= 0 && dev < kMaxDevices, "%s: device index %d out of range", op, dev);
-  std::lock_guard<std::mutex> lock(g_static_scratch_mutex);
-  if (g_static_scratch[dev] == nullptr) {
-    void* p = nullptr;
-    rc = check_hip(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)), "hipGetSymbolAddress(scratch)");
-    if (rc) return rc;
-    KVQ_REQUIRE(p != nullptr, "%s: the static scratch array has no device address", op);
-    g_static_scratch[dev] = p;
-  }
-  *ptr = g_static_scratch[dev];
-  return KVQ_OK;
-}
-
 }  // namespace kvq
 
 extern "C" int kvq_paged_attn_int8(void* out, int out_dtype, int64_t out_stride_t, int64_t out_stride_h,
@@ -147,9 +151,10 @@ extern "C" int kvq_paged_attn_int8_static_scratch(void* out, int out_dtype, int6
                                                   int max_query_len, float scale, int causal, int window_size,
                                                   float softcap, float* lse, kvq_stream_t stream) {
   const char* op = "paged_attn_int8_static_scratch";
-  void* ptr = nullptr;
-  const int rc = kvq::static_scratch_ptr(op, &ptr);
+  kvq::DeviceSymbols sym;
+  const int rc = kvq::device_symbols(op, &sym);
   if (rc) return rc;
+  void* ptr = sym.scratch;
   // The split-K partial states need no clearing: every slot the reduce reads was written by this
   // launch's main kernel first (slots it does not own are masked out bit-wise, whatever they hold).
   return kvq::paged_attn_launch(op, out, out_dtype, out_stride_t, out_stride_h, q, q_dtype, q_stride_t, q_stride_h,

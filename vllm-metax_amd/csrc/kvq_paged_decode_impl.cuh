@@ -1,0 +1,456 @@
+// Device code and launch templates of the paged decode kernels, instantiated once per head size in
+// kvq_paged_decode_d64.hip / _d128.hip / _d256.hip (one translation unit each, so they compile in parallel).
+#pragma once
+
+#include <type_traits>
+
+#include "kvq_attn_core.cuh"
+
+namespace kvq {
+
+int heads_per_wg(int num_kv_heads);
+
+
+
+__device__ __forceinline__ int wave_incl_scan(int v, int lane) {
+#pragma unroll
+  for (int o = 1; o < kWave; o <<= 1) {
+    int u = __shfl_up(v, o, kWave);
+    if (lane >= o) v += u;
+  }
+  return v;
+}
+
+// Starting on a sequence (query row, first tile with nothing in flight, storing the state of the
+// one before) costs a workgroup about as long as one tile takes; the work line that is cut into
+// equal shares therefore charges every sequence this many units before its tiles.  Measured on
+// MI355X at batch 64, 1k..8k tokens: workgroups whose share crossed a sequence boundary ran 2.9 us
+// (one tile time) longer than the others and were the last to finish; with the charge they get
+// one tile less.
+constexpr int kSetupUnits = 1;
+
+// Tiles of a decode sequence: those that hold a token of the row's window,
+// [window_first / 32, ceil(len / 32)).  0 for prefill sequences and empty ones.
+__device__ __forceinline__ int decode_tiles(const int32_t* seq_lens, const int32_t* cu, int s, int num_seqs,
+                                            int window) {
+  // no data-dependent branches: the loads of a lane (and of the lanes' next chunks) all go out
+  // together; a lane past the last sequence rereads the last one and its result is dropped
+  const int sc = s < num_seqs ? s : num_seqs - 1;
+  const int len = seq_lens[sc];
+  int q_len = 1;
+  if (cu != nullptr) q_len = cu[sc + 1] - cu[sc];
+  const int n = (len + kTile - 1) / kTile - window_first(len, window) / kTile;
+  return (s < num_seqs && q_len == 1 && len > 0) ? n : 0;
+}
+
+// Units a sequence takes on the work line: its setup charge, then one unit per tile.
+__device__ __forceinline__ int decode_units(const int32_t* seq_lens, const int32_t* cu, int s, int num_seqs,
+                                            int window) {
+  const int n = decode_tiles(seq_lens, cu, s, num_seqs, window);
+  return n > 0 ? n + kSetupUnits : 0;
+}
+
+// The scans over the sequences work on chunks of 64 (one per lane).  Large batches take kScanBatch
+// chunks per step so that their loads are in flight together (batch 512: 16 dependent round trips
+// -> 4); a batch that fits one chunk keeps the single-chunk loop, which measured 3 us faster there.
+constexpr int kScanBatch = 4;
+
+// Total units of the work line.
+template <int BATCH>
+__device__ __forceinline__ int64_t scan_total(const StreamKArgs& a, int lane) {
+  const int B = a.num_seqs;
+  int64_t total = 0;
+  for (int base = 0; base < B; base += kWave * BATCH) {
+    int n[BATCH];
+#pragma unroll
+    for (int j = 0; j < BATCH; ++j)
+      n[j] = decode_units(a.seq_lens, a.cu_seqlens_q, base + kWave * j + lane, B, a.io.window);
+#pragma unroll
+    for (int j = 0; j < BATCH; ++j) total += __builtin_amdgcn_readlane(wave_incl_scan(n[j], lane), 63);
+  }
+  return total;
+}
+
+// The sequence that holds unit `lo` and the index of its first unit.
+template <int BATCH>
+__device__ __forceinline__ void scan_locate(const StreamKArgs& a, int lane, int64_t lo, int& seq, int64_t& seq_start) {
+  const int B = a.num_seqs;
+  int64_t cum = 0;
+  bool found = false;
+  for (int base = 0; base < B && !found; base += kWave * BATCH) {
+    int nn[BATCH];
+#pragma unroll
+    for (int j = 0; j < BATCH; ++j)
+      nn[j] = decode_units(a.seq_lens, a.cu_seqlens_q, base + kWave * j + lane, B, a.io.window);
+#pragma unroll
+    for (int j = 0; j < BATCH; ++j) {
+      const int n = nn[j];
+      const int incl = wave_incl_scan(n, lane);
+      const int64_t first = cum + incl - n, last = cum + incl;
+      const uint64_t hit = __builtin_amdgcn_ballot_w64(n > 0 && first <= lo && lo < last);
+      if (hit != 0 && !found) {
+        const int src = __builtin_ctzll(hit);
+        seq = base + kWave * j + src;
+        seq_start = cum + __builtin_amdgcn_readlane(incl - n, src);
+        found = true;
+      }
+      cum += __builtin_amdgcn_readlane(incl, 63);
+    }
+  }
+}
+
+// Total units and the first unit of sequence `seq`; n_first = the units of the first BATCH chunks,
+// loaded by the caller ahead of its first branch.
+template <int BATCH>
+__device__ __forceinline__ void scan_start(const StreamKArgs& a, int lane, int seq, const int (&n_first)[BATCH],
+                                           int64_t& total, int64_t& start) {
+  const int B = a.num_seqs;
+  total = 0;
+  start = 0;
+  for (int base = 0; base < B; base += kWave * BATCH) {
+    int nn[BATCH];
+#pragma unroll
+    for (int j = 0; j < BATCH; ++j)
+      nn[j] = base == 0 ? n_first[j] : decode_units(a.seq_lens, a.cu_seqlens_q, base + kWave * j + lane, B, a.io.window);
+#pragma unroll
+    for (int j = 0; j < BATCH; ++j) {
+      const int n = nn[j], b0 = base + kWave * j;
+      const int incl = wave_incl_scan(n, lane);
+      if (seq >= b0 && seq < b0 + kWave) start = total + __builtin_amdgcn_readlane(incl - n, seq - b0);
+      total += __builtin_amdgcn_readlane(incl, 63);
+    }
+  }
+}
+
+__device__ __forceinline__ int64_t wg_tile_begin(int w, int64_t total, int num_wg) {
+  return ((int64_t)w * total) / num_wg;
+}
+
+// Workgroups that take a share of a line of `total` units: all that were launched, unless the line
+// is so short that a share would fall below kMinUnitsPerWg -- a small batch is then spread over
+// fewer workgroups, so that a sequence is not cut into dozens of one-tile partial states for the
+// reduce to merge.  Measured at batch 4 x 512 tokens (main + reduce kernel): 15.6 us with shares of
+// at least 2 units, 18.3 us with 4 (a tile at a time per wave: about 4 us per tile at low load).
+constexpr int kMinUnitsPerWg = 2;
+__device__ __forceinline__ int active_workgroups(int64_t total, int num_wg) {
+  const int64_t want = total / kMinUnitsPerWg;
+  return want >= num_wg ? num_wg : (want < 1 ? 1 : (int)want);
+}
+
+// HPW = kv heads per workgroup (1, 2, 4 or 8).  A workgroup always has eight waves: with fewer than
+// eight kv heads the 8 / HPW waves of a head take the tiles of a run in turn and their states are
+// folded together in LDS when the run ends, so a compute unit keeps eight tile streams in flight
+// whatever the head count and a sequence is cut into no more partial states than with eight heads.
+template <int D, int QDT, int HPW, bool CAP>
+__global__ __launch_bounds__(512) void paged_decode_streamk_kernel(StreamKArgs a) {
+  using DTile = DecodeTile<D, QDT, kRuntimeDtype>;
+  constexpr int NSUB = 8 / HPW;
+  __shared__ __align__(16) uint8_t lds[8][DTile::LDS_WAVE];
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int sub = wave % NSUB;
+  const int hkv = __builtin_amdgcn_readfirstlane(blockIdx.y * HPW + wave / NSUB);
+  if (hkv >= a.io.g.num_kv_heads) return;  // a finished wave no longer counts at the workgroup's barriers
+  const int w = blockIdx.x;
+  const int B = a.num_seqs;
+
+  // total units of the work line (each wave redoes this tiny scan; no LDS, no barrier)
+  const bool one_chunk = B <= kWave;
+  const int64_t total = one_chunk ? scan_total<1>(a, lane) : scan_total<kScanBatch>(a, lane);
+  const int num_wg = active_workgroups(total, a.num_wg);
+  if (w >= num_wg) return;
+  const int64_t lo = wg_tile_begin(w, total, num_wg);
+  const int64_t hi = wg_tile_begin(w + 1, total, num_wg);
+  if (lo >= hi) return;
+
+  // locate the sequence holding unit `lo`
+  int seq = 0;
+  int64_t seq_start = 0;  // global index of the sequence's first unit
+  if (one_chunk) scan_locate<1>(a, lane, lo, seq, seq_start);
+  else scan_locate<kScanBatch>(a, lane, lo, seq, seq_start);
+  seq = __builtin_amdgcn_readfirstlane(seq);
+
+  int64_t pos = lo;
+  while (pos < hi && seq < B) {
+    const int units = __builtin_amdgcn_readfirstlane(decode_units(a.seq_lens, a.cu_seqlens_q, seq, B, a.io.window));
+    if (units == 0) {
+      ++seq;
+      continue;
+    }
+    const int ntiles = units - kSetupUnits;
+    const int len = __builtin_amdgcn_readfirstlane(a.seq_lens[seq]);
+    const int64_t row = a.cu_seqlens_q ? (int64_t)a.cu_seqlens_q[seq] : (int64_t)seq;
+    const int first = window_first(len, a.io.window);  // tokens before it are outside the window
+    const int t0 = first / kTile;                      // the sequence's tile line starts at this tile
+    // units [pos, min(hi, end of the sequence)) of the line; the first kSetupUnits of a sequence
+    // stand for no tile
+    const int u_begin = (int)(pos - seq_start);
+    const int64_t rem = hi - seq_start;
+    const int u_end = rem < units ? (int)rem : units;
+    const int t_begin = __builtin_amdgcn_readfirstlane(t0 + (u_begin > kSetupUnits ? u_begin - kSetupUnits : 0));
+    const int t_end = __builtin_amdgcn_readfirstlane(t0 + u_end - kSetupUnits);
+    if (t_begin < t_end) {  // else: this share ends inside the setup charge and holds no tile
+      typename DTile::State st;
+      DTile::template run<CAP>(a.io, seq, row, len, first, t_begin, t_end, hkv, lane, lds[wave], st, sub, NSUB);
+      if constexpr (NSUB > 1) {
+        if (sub != 0) DTile::dump_state(st, lane, lds[wave]);
+        lds_barrier();
+        if (sub == 0) {
+#pragma unroll
+          for (int j = 1; j < NSUB; ++j)
+            if (t_begin + j < t_end) DTile::fold_state(st, lane, lds[wave + j]);  // wave j owned a tile
+        }
+        lds_barrier();  // the windows may be overwritten by the next run
+      }
+      if (sub == 0) {
+        if (t_begin == t0 && t_end == t0 + ntiles) {
+          DTile::emit_final(a.io, row, hkv, lane, st);
+        } else {
+          DTile::emit_partial(a.io, a.part_o, a.part_ml, (int64_t)w + seq, hkv, lane, st);
+        }
+      }
+    }
+    pos = seq_start + u_end;
+    seq_start += units;
+    ++seq;
+  }
+}
+
+// Merge the partial states of every decode sequence that more than one workgroup touched.
+// grid (num_seqs, ceil(Hq / 4)), 4 waves, one wave per q head, lane owns D/64 dims.
+template <int D>
+__global__ __launch_bounds__(256) void paged_decode_streamk_reduce_kernel(StreamKArgs a) {
+  constexpr int V = D / 64;
+  const int lane = threadIdx.x & 63;
+  const int head = blockIdx.y * 4 + (threadIdx.x >> 6);
+  const int seq = blockIdx.x;
+  const int B = a.num_seqs;
+  if (head >= a.io.num_q_heads) return;
+  // all the loads that depend on nothing but the arguments go out together, before the first branch
+  const int q0 = a.cu_seqlens_q ? a.cu_seqlens_q[seq] : seq;
+  const int q1 = a.cu_seqlens_q ? a.cu_seqlens_q[seq + 1] : seq + 1;
+  const int len = a.seq_lens[seq];
+  const bool one_chunk = B <= kWave;
+  int n_first[kScanBatch];  // first sequences of the scan
+  n_first[0] = decode_units(a.seq_lens, a.cu_seqlens_q, lane, B, a.io.window);
+  if (!one_chunk) {
+#pragma unroll
+    for (int j = 1; j < kScanBatch; ++j)
+      n_first[j] = decode_units(a.seq_lens, a.cu_seqlens_q, kWave * j + lane, B, a.io.window);
+  }
+  if (q1 - q0 != 1) return;
+  const int64_t row = q0;
+  const int ntiles = len > 0 ? (len + kTile - 1) / kTile - window_first(len, a.io.window) / kTile : 0;
+  if (ntiles == 0) {  // empty sequence: defined output (zeros, lse = -inf)
+    for (int i = 0; i < V; ++i)
+      store_act_rt(a.io.out_dtype, a.io.out, row * a.io.out_stride_t + (int64_t)head * a.io.out_stride_h + lane * V + i, 0.f);
+    if (a.io.lse != nullptr && lane == 0) a.io.lse[row * a.io.num_q_heads + head] = -INFINITY;
+    return;
+  }
+  int64_t total, start;
+  if (one_chunk) {
+    const int n1[1] = {n_first[0]};
+    scan_start<1>(a, lane, seq, n1, total, start);
+  } else {
+    scan_start<kScanBatch>(a, lane, seq, n_first, total, start);
+  }
+  const int P = active_workgroups(total, a.num_wg);
+  // workgroup holding unit x: the largest w with floor(w*T/P) <= x; the sequence's tiles are units
+  // start + kSetupUnits .. start + kSetupUnits + ntiles - 1
+  const int w_first = (int)(((start + kSetupUnits + 1) * P - 1) / total);
+  const int w_last = (int)(((start + kSetupUnits + ntiles) * P - 1) / total);
+  if (w_first == w_last) return;  // written directly by the main kernel
+
+  // pass 1: every lane takes one workgroup's (m, l); the wave agrees on the max and the weights
+  // pass 2: weighted sum of the partial outputs, all loads independent of each other
+  float m = -INFINITY, l = 0.f, acc[V];
+#pragma unroll
+  for (int i = 0; i < V; ++i) acc[i] = 0.f;
+  // Few slots (the usual case: a sequence spans a handful of workgroups): the (m, l) pairs and ALL
+  // the partial outputs are requested in one go, so the kernel pays one memory round trip for them
+  // instead of two.
+  constexpr int kFew = 32;
+  // N = how many slots the one-round-trip path requests (all of them unconditionally: slots past the
+  // last reread the last one), in three sizes so that a short span does not fetch 32 rows
+  auto merge_few = [&](auto n_tag) __attribute__((always_inline)) {
+    constexpr int N = decltype(n_tag)::value;
+    const int w = w_first + lane;
+    const bool live = w <= w_last && wg_tile_begin(w, total, P) < wg_tile_begin(w + 1, total, P);
+    const int64_t slot = (int64_t)min(w, w_last) + seq;
+    const uint32_t keep = live ? 0xffffffffu : 0u;
+    const float mj_raw = a.part_ml[(slot * a.io.num_q_heads + head) * 2 + 0];
+    const float lj_raw = a.part_ml[(slot * a.io.num_q_heads + head) * 2 + 1];
+    float po[N][V];
+#pragma unroll
+    for (int k = 0; k < N; ++k) {
+      const int64_t sk = (int64_t)min(w_first + k, w_last) + seq;
+      const float* p = a.part_o + (sk * a.io.num_q_heads + head) * (int64_t)D + lane * V;
+#pragma unroll
+      for (int i = 0; i < V; ++i) po[k][i] = p[i];
+    }
+    const float mj = live ? as_f32(as_u32(mj_raw) & keep) : -INFINITY;
+    const float lj = as_f32(as_u32(lj_raw) & keep);
+    m = wave_max(mj);
+    const float ej = live ? __builtin_amdgcn_exp2f(mj - m) : 0.f;
+    l = wave_sum(lj * ej);
+#pragma unroll
+    for (int k = 0; k < N; ++k) {
+      const float wk = __shfl(ej, k, kWave);  // 0 for slots past the last and for empty ones
+      const uint32_t kk = wk != 0.f ? 0xffffffffu : 0u;
+#pragma unroll
+      for (int i = 0; i < V; ++i) acc[i] += as_f32(as_u32(po[k][i]) & kk) * wk;
+    }
+  };
+  const int span = w_last - w_first + 1;
+  if (span <= 4) {
+    merge_few(std::integral_constant<int, 4>{});
+  } else if (span <= 12) {
+    merge_few(std::integral_constant<int, 12>{});
+  } else if (span <= kFew) {
+    merge_few(std::integral_constant<int, kFew>{});
+  } else
+  for (int wb = w_first; wb <= w_last; wb += kWave) {
+    const int w = wb + lane;
+    const bool live = w <= w_last && wg_tile_begin(w, total, P) < wg_tile_begin(w + 1, total, P);
+    // loads are unconditional (clamped to the sequence's last workgroup) and what they return is
+    // removed with a bit mask where the slot holds nothing: a select on the loaded value becomes a
+    // branch around the load, and the loads of successive slots would then run one after another
+    const int64_t slot = (int64_t)min(w, w_last) + seq;
+    const uint32_t keep = live ? 0xffffffffu : 0u;
+    const float mj_raw = a.part_ml[(slot * a.io.num_q_heads + head) * 2 + 0];
+    const float lj_raw = a.part_ml[(slot * a.io.num_q_heads + head) * 2 + 1];
+    const float mj = live ? as_f32(as_u32(mj_raw) & keep) : -INFINITY;
+    const float lj = as_f32(as_u32(lj_raw) & keep);
+    const float m_new = fmaxf(m, wave_max(mj));
+    const float ca = __builtin_amdgcn_exp2f(m - m_new);  // first chunk: exp2(-inf) = 0
+    const float ej = live ? __builtin_amdgcn_exp2f(mj - m_new) : 0.f;
+    l = l * ca + wave_sum(lj * ej);
+#pragma unroll
+    for (int i = 0; i < V; ++i) acc[i] *= ca;
+    m = m_new;
+    // sixteen slots per round trip: the loads of a batch are unconditional (slots past the last reread
+    // the last one, weight 0) so that they all leave before the first is used
+    const int count = min(kWave, w_last - wb + 1);
+    for (int k0 = 0; k0 < count; k0 += 16) {
+      float pv[16][V];
+#pragma unroll
+      for (int k = 0; k < 16; ++k) {
+        const int64_t sk = (int64_t)min(wb + k0 + k, w_last) + seq;
+        const float* po = a.part_o + (sk * a.io.num_q_heads + head) * (int64_t)D + lane * V;
+#pragma unroll
+        for (int i = 0; i < V; ++i) pv[k][i] = po[i];
+      }
+#pragma unroll
+      for (int k = 0; k < 16; ++k) {
+        const float wk = (k0 + k) < count ? __shfl(ej, (k0 + k) & (kWave - 1), kWave) : 0.f;  // unnormalised sums
+        const uint32_t kk = wk != 0.f ? 0xffffffffu : 0u;
+#pragma unroll
+        for (int i = 0; i < V; ++i) acc[i] += as_f32(as_u32(pv[k][i]) & kk) * wk;
+      }
+    }
+  }
+  const float inv = 1.0f / l;
+#pragma unroll
+  for (int i = 0; i < V; ++i)
+    store_act_rt(a.io.out_dtype, a.io.out, row * a.io.out_stride_t + (int64_t)head * a.io.out_stride_h + lane * V + i, acc[i] * inv);
+  if (a.io.lse != nullptr && lane == 0)
+    a.io.lse[row * a.io.num_q_heads + head] = (m + __builtin_amdgcn_logf(l)) * kLn2;
+}
+
+// ---- fixed partitions: grid (max_parts, num_seqs, head groups) --------------------------
+struct V2Args {
+  AttnIO io;
+  const int32_t* seq_lens;
+  float* tmp_out;
+  float* max_logits;
+  float* exp_sums;
+  int partition_tiles;  // partition_size / 32
+  int max_parts;
+};
+
+template <int D, int QDT, int WPW>
+__global__ __launch_bounds__(WPW * 64) void paged_decode_v2_kernel(V2Args a) {
+  using DTile = DecodeTile<D, QDT, KVQ_F32>;
+  __shared__ __align__(16) uint8_t lds[WPW][DTile::LDS_WAVE];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int hkv = __builtin_amdgcn_readfirstlane(blockIdx.z * WPW + wave);
+  if (hkv >= a.io.g.num_kv_heads) return;
+  const int part = blockIdx.x, seq = blockIdx.y;
+  const int len = a.seq_lens[seq];
+  const int ntiles = len > 0 ? (len + kTile - 1) / kTile : 0;
+  const int t_begin = part * a.partition_tiles;
+  if (t_begin >= ntiles) return;
+  const int t_end = min(ntiles, t_begin + a.partition_tiles);
+  typename DTile::State st;
+  DTile::template run<false>(a.io, seq, seq, len, 0, t_begin, t_end, hkv, lane, lds[wave], st);
+  DTile::emit_v2(a.io, a.tmp_out, a.max_logits, a.exp_sums, seq, part, a.max_parts, hkv, lane, st);
+}
+
+// out = sum_j w_j tmp_out_j / sum_j w_j, w_j = exp_sums_j * exp(max_logits_j - max).
+template <int D, int QDT>
+static int launch_streamk(const StreamKArgs& a, hipStream_t s) {
+  const int hkv = a.io.g.num_kv_heads;
+  const int hpw = heads_per_wg(hkv);
+  dim3 grid(a.num_wg, (hkv + hpw - 1) / hpw);
+#define KVQ_SK(H, C) hipLaunchKernelGGL((paged_decode_streamk_kernel<D, QDT, H, C>), grid, dim3(512), 0, s, a)
+  if (a.io.cap_c != 0.f) {
+    switch (hpw) {
+      case 8: KVQ_SK(8, true); break;
+      case 4: KVQ_SK(4, true); break;
+      case 2: KVQ_SK(2, true); break;
+      default: KVQ_SK(1, true); break;
+    }
+  } else {
+    switch (hpw) {
+      case 8: KVQ_SK(8, false); break;
+      case 4: KVQ_SK(4, false); break;
+      case 2: KVQ_SK(2, false); break;
+      default: KVQ_SK(1, false); break;
+    }
+  }
+#undef KVQ_SK
+  int rc = check_hip(hipGetLastError(), "paged_attn_int8 decode launch");
+  if (rc) return rc;
+  dim3 rgrid(a.num_seqs, (a.io.num_q_heads + 3) / 4);
+  hipLaunchKernelGGL((paged_decode_streamk_reduce_kernel<D>), rgrid, dim3(256), 0, s, a);
+  return check_hip(hipGetLastError(), "paged_attn_int8 reduce launch");
+}
+
+template <int D>
+int launch_streamk_q(const StreamKArgs& a, int q_dtype, int out_dtype, hipStream_t s) {
+  if (out_dtype != KVQ_F32 && out_dtype != KVQ_BF16 && out_dtype != KVQ_F16)
+    return fail(KVQ_EINVAL, "paged_attn_int8: unknown out_dtype %d", out_dtype);
+  switch (q_dtype) {
+    case KVQ_F32: return launch_streamk<D, KVQ_F32>(a, s);
+    case KVQ_BF16: return launch_streamk<D, KVQ_BF16>(a, s);
+    case KVQ_F16: return launch_streamk<D, KVQ_F16>(a, s);
+  }
+  return fail(KVQ_EINVAL, "paged_attn_int8: unknown q_dtype %d", q_dtype);
+}
+
+template <int D, int QDT>
+static int launch_v2(const V2Args& a, int num_seqs, hipStream_t s) {
+  const int hkv = a.io.g.num_kv_heads;
+  const int wpw = heads_per_wg(hkv);
+  dim3 grid(a.max_parts, num_seqs, (hkv + wpw - 1) / wpw);
+  switch (wpw) {
+    case 8: hipLaunchKernelGGL((paged_decode_v2_kernel<D, QDT, 8>), grid, dim3(512), 0, s, a); break;
+    case 4: hipLaunchKernelGGL((paged_decode_v2_kernel<D, QDT, 4>), grid, dim3(256), 0, s, a); break;
+    case 2: hipLaunchKernelGGL((paged_decode_v2_kernel<D, QDT, 2>), grid, dim3(128), 0, s, a); break;
+    default: hipLaunchKernelGGL((paged_decode_v2_kernel<D, QDT, 1>), grid, dim3(64), 0, s, a); break;
+  }
+  return check_hip(hipGetLastError(), "paged_attn_v2_int8 launch");
+}
+
+template <int D>
+int launch_v2_q(const V2Args& a, int num_seqs, int q_dtype, hipStream_t s) {
+  switch (q_dtype) {
+    case KVQ_F32: return launch_v2<D, KVQ_F32>(a, num_seqs, s);
+    case KVQ_BF16: return launch_v2<D, KVQ_BF16>(a, num_seqs, s);
+    case KVQ_F16: return launch_v2<D, KVQ_F16>(a, num_seqs, s);
+  }
+  return fail(KVQ_EINVAL, "paged_attn_v2_int8: unknown q_dtype %d", q_dtype);
+}
+
+
+}  // namespace kvq
