@@ -28,10 +28,55 @@ sys.path.insert(0, ROOT)
 import torch  # noqa: E402
 
 HBM_PEAK_GBPS = 8000.0
-# HBM bytes per decode attention launch, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by a plain
-# read / copy kernel of known size (factors 2.000 and 1.000); summaries under profiles/.
-MEASURED_TRAFFIC = {"llama3_8b_decode_b64_ctx1k-8k": 727.1e6, "mla_decode_b32_h128_ctx4096": 195.4e6}
 METRIC = "int8-KV paged decode: achieved HBM GB/s (% peak), µs/layer @B=64 ctx=8k"
+# Untimed steps run for this long before the counted warm-up, so that a short run (the driver's 20 steps) is
+# timed at the clocks a long one reaches; printed in the line as "prewarm_s".
+PREWARM_S = 0.5
+# rocprofv3 summaries that carry the measured HBM traffic of a workload's attention launch
+# (a line "traffic_bytes_per_launch: N" and a line "measured_at_commit: HASH")
+TRAFFIC_PROFILE = {"llama3_8b_decode_b64_ctx1k-8k": "paged_decode_streamk_llama3_8b_b64_ctx1k-8k.md",
+                   "mla_decode_b32_h128_ctx4096": "mla_decode_b32_h128_ctx4096.md"}
+
+
+def measured_traffic(workload):
+    """(bytes per launch, source) from the workload's rocprofv3 summary under profiles/, or (None, None): the
+    figure is what a profiler run measured at the named commit, never a constant of this file."""
+    name = TRAFFIC_PROFILE.get(workload)
+    path = os.path.join(ROOT, "profiles", name) if name else None
+    if not path or not os.path.exists(path):
+        return None, None
+    nbytes = commit = None
+    for line in open(path, encoding="utf-8"):
+        if line.startswith("traffic_bytes_per_launch:"):
+            nbytes = float(line.split(":", 1)[1].split()[0])
+        elif line.startswith("measured_at_commit:"):
+            commit = line.split(":", 1)[1].strip()
+    if nbytes is None:
+        return None, None
+    return nbytes, f"profiles/{name} (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, measured at commit {commit})"
+
+
+def prewarm(step, seconds=PREWARM_S):
+    """Run `step(i)` untimed for a fixed wall time."""
+    t0, i = time.perf_counter(), 0
+    while time.perf_counter() - t0 < seconds:
+        for _ in range(20):
+            step(i)
+            i += 1
+        torch.cuda.synchronize()
+
+
+def time_back_to_back(fn, n):
+    """Average duration of `fn(i)` over n launches issued back to back between two events on the launch
+    stream (torch's current stream, which the ops launch on)."""
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    e0.record()
+    for i in range(n):
+        fn(i)
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / n * 1e-3
 
 
 def make_batch(workload: str, seed: int = 0):
@@ -226,6 +271,7 @@ def mla_main(args, cfg, dev, ops):
     st = build_mla_state(cfg, dev, args.layers)
     nbytes, flops = mla_algorithmic(cfg)
     L = args.layers
+    prewarm(lambda i: run_mla_step(st, i % L, ops, cfg))
     for i in range(args.warmup):
         run_mla_step(st, i % L, ops, cfg)
     torch.cuda.synchronize()
@@ -234,15 +280,9 @@ def mla_main(args, cfg, dev, ops):
         run_mla_step(st, i % L, ops, cfg)
     torch.cuda.synchronize()
     dt = (time.perf_counter() - t0) / args.steps
-    n_ev = min(args.steps, 200)
-    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n_ev)]
-    for i in range(n_ev):
-        run_mla_step(st, i % L, ops, cfg, write=True, attn=False)
-        evs[i][0].record()
-        run_mla_step(st, i % L, ops, cfg, write=False, attn=True)
-        evs[i][1].record()
-    torch.cuda.synchronize()
-    attn_s = sum(a.elapsed_time(b) for a, b in evs) / n_ev * 1e-3
+    n_ev = max(args.steps, 100)
+    attn_s = time_back_to_back(lambda i: run_mla_step(st, i % L, ops, cfg, write=False, attn=True), n_ev)
+    traffic, traffic_source = measured_traffic(args.workload)
     res = {
         "metric": "int8 MLA latent-cache decode: achieved HBM GB/s, µs/layer @B=32 H=128 ctx=4096",
         "value": round(nbytes / dt / 1e9, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -250,11 +290,12 @@ def mla_main(args, cfg, dev, ops):
         "dtype": "int8 latent codes, fp16 MFMA operands, fp32 softmax/accumulate, bf16 Q/out", "data": "synthetic",
         "config": {"workload": args.workload, "batch": len(cfg["ctx"]), "sum_ctx": sum(cfg["ctx"]), "heads": cfg["heads"],
                    "kv_lora_rank": cfg["r"], "rope_dim": cfg["p"], "block_size": cfg["bs"], "layer_caches_rotated": L},
-        "us_per_layer": round(dt * 1e6, 2), "attn_launch_us": round(attn_s * 1e6, 2),
+        "prewarm_s": PREWARM_S, "us_per_layer": round(dt * 1e6, 2), "attn_launch_us": round(attn_s * 1e6, 2),
         "roofline": {"bound": "mfma", "achieved": round(flops / attn_s / 1e12, 1), "peak": MFMA_F16_PEAK_TFLOPS,
                      "unit": "TFLOP/s", "frac": round(flops / attn_s / 1e12 / MFMA_F16_PEAK_TFLOPS, 4),
-                     "traffic": MEASURED_TRAFFIC.get(args.workload),
+                     "traffic": traffic, "traffic_source": traffic_source,
                      "kernel": "MLA decode launch = mla_quant_q_kernel + mla_decode_kernel + mla_reduce_kernel",
+                     "timing": f"{n_ev} decode launches back to back between two events on the launch stream",
                      "algorithmic_flops_per_launch": flops, "algorithmic_bytes_per_launch": nbytes,
                      "hbm_frac_of_peak": round(nbytes / attn_s / 1e9 / HBM_PEAK_GBPS, 4)},
     }
@@ -322,6 +363,7 @@ def mixed_main(args, cfg, dev, ops):
                                   **_window_kwargs(dict(window=args.sliding_window, softcap=args.soft_cap)))
 
     Lr = args.layers
+    prewarm(lambda i: step(i % Lr))
     for i in range(args.warmup):
         step(i % Lr)
     torch.cuda.synchronize()
@@ -330,15 +372,8 @@ def mixed_main(args, cfg, dev, ops):
         step(i % Lr)
     torch.cuda.synchronize()
     dt = (time.perf_counter() - t0) / args.steps
-    n_ev = min(args.steps, 50)
-    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n_ev)]
-    for i in range(n_ev):
-        step(i % Lr, write=True, attn=False)
-        evs[i][0].record()
-        step(i % Lr, write=False, attn=True)
-        evs[i][1].record()
-    torch.cuda.synchronize()
-    attn_s = sum(a.elapsed_time(b) for a, b in evs) / n_ev * 1e-3
+    n_ev = min(max(args.steps, 20), 100)
+    attn_s = time_back_to_back(lambda i: step(i % Lr, write=False, attn=True), n_ev)
     # causal prefill flops: 4 D Hq (q_len * cached + q_len (q_len + 1) / 2); decode rows: 4 D Hq ctx
     flops = sum(4 * d * hq * (ql * (c - ql) + ql * (ql + 1) // 2) for c, ql in zip(ctx, qls))
     dec_bytes = sum(c for c, ql in zip(ctx, qls) if ql == 1) * hkv * 2 * (d + 4)
@@ -355,7 +390,7 @@ def mixed_main(args, cfg, dev, ops):
                    **({"soft_cap": args.soft_cap} if args.soft_cap else {}),
                    "batch": B, "new_tokens": n_tok, "sum_ctx": sum(ctx), "q_heads": hq,
                    "kv_heads": hkv, "head_dim": d, "block_size": bs, "layer_caches_rotated": Lr},
-        "attn_launch_us": round(attn_s * 1e6, 1),
+        "prewarm_s": PREWARM_S, "attn_launch_us": round(attn_s * 1e6, 1),
         "roofline": {"bound": "mfma", "achieved": round(flops / attn_s / 1e12, 1), "peak": MFMA_F16_PEAK_TFLOPS,
                      "unit": "TFLOP/s", "frac": round(flops / attn_s / 1e12 / MFMA_F16_PEAK_TFLOPS, 4), "traffic": None,
                      "kernel": "varlen attention launch = decode stream-K + reduce + paged_prefill_kernel",
@@ -403,6 +438,29 @@ def cpu_baseline(cfg, st, seconds_target=15.0):
                 us_per_layer_extrapolated=t_total / done_bytes * algorithmic_bytes(cfg, False)[0] * 1e6)
 
 
+def time_decode(cfg, st, args, ops):
+    """Pre-warm, W untimed and K timed steps (write + attention) on the host clock around a device
+    synchronisation; then the attention launch and the write launch on their own, back to back."""
+    attn_bytes, write_bytes = algorithmic_bytes(cfg)
+    if args.sliding_window:  # a windowed decode row reads only its last `window` tokens
+        attn_bytes, _ = algorithmic_bytes(dict(cfg, ctx=[min(c, args.sliding_window) for c in cfg["ctx"]]))
+    L = args.layers
+    prewarm(lambda i: run_step(st, i % L, ops))
+    for i in range(args.warmup):
+        run_step(st, i % L, ops)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        run_step(st, i % L, ops)
+    torch.cuda.synchronize()
+    step_s = (time.perf_counter() - t0) / args.steps
+    n = max(args.steps, 100)
+    attn_s = time_back_to_back(lambda i: run_step(st, i % L, ops, write=False, attn=True), n)
+    write_s = time_back_to_back(lambda i: run_step(st, i % L, ops, write=True, attn=False), n)
+    return dict(step_s=step_s, attn_s=attn_s, write_s=write_s, attn_bytes=attn_bytes, n_attn=n,
+                value=(attn_bytes + write_bytes) / step_s / 1e9)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -414,6 +472,8 @@ def main():
                     help="GQA workloads: attend to the last N keys only (0 = full causal, the configured workloads)")
     ap.add_argument("--soft-cap", type=float, default=0.0, help="GQA workloads: logits soft cap (0 = none)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-fixed-8k", action="store_true",
+                    help="default workload only: skip the extra fixed-context (64 x 8192) measurement")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     args = ap.parse_args()
     if args.gpus != 1:
@@ -430,46 +490,20 @@ def main():
         return mixed_main(args, cfg, dev, ops)
     st = build_device_state(cfg, dev, args.layers)
     st["window"], st["softcap"] = args.sliding_window, args.soft_cap
-    attn_bytes, write_bytes = algorithmic_bytes(cfg)
-    if args.sliding_window:  # a windowed decode row reads only its last `window` tokens
-        attn_bytes, _ = algorithmic_bytes(dict(cfg, ctx=[min(c, args.sliding_window) for c in cfg["ctx"]]))
     L = args.layers
-
-    for i in range(args.warmup):
-        run_step(st, i % L, ops)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for i in range(args.steps):
-        run_step(st, i % L, ops)
-    torch.cuda.synchronize()
-    dt = time.perf_counter() - t0
-    ms_per_step = dt / args.steps * 1e3
-    value = (attn_bytes + write_bytes) / (dt / args.steps) / 1e9
-
-    # the decode attention launch alone, events on the launch stream (torch's current stream)
-    n_ev = min(args.steps, 200)
-    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n_ev)]
-    wevs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n_ev)]
-    for i in range(n_ev):
-        wevs[i][0].record()
-        run_step(st, i % L, ops, write=True, attn=False)
-        wevs[i][1].record()
-        evs[i][0].record()
-        run_step(st, i % L, ops, write=False, attn=True)
-        evs[i][1].record()
-    torch.cuda.synchronize()
-    attn_ms = sum(a.elapsed_time(b) for a, b in evs) / n_ev
-    write_ms = sum(a.elapsed_time(b) for a, b in wevs) / n_ev
-    achieved = attn_bytes / (attn_ms * 1e-3) / 1e9
+    t = time_decode(cfg, st, args, ops)
+    traffic, traffic_source = measured_traffic(args.workload)
+    if args.sliding_window or args.soft_cap:
+        traffic, traffic_source = None, None
 
     res = {
         "metric": METRIC,
-        "value": round(value, 1),
+        "value": round(t["value"], 1),
         "unit": "GB/s",
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
-        "ms_per_step": round(ms_per_step, 5),
+        "ms_per_step": round(t["step_s"] * 1e3, 5),
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
@@ -480,16 +514,33 @@ def main():
                    "pool_blocks": cfg["pool"], "layer_caches_rotated": L, "kv_layout": "NHD",
                    **({"sliding_window": args.sliding_window} if args.sliding_window else {}),
                    **({"soft_cap": args.soft_cap} if args.soft_cap else {})},
-        "pct_hbm_peak": round(100 * value / HBM_PEAK_GBPS, 2),
-        "us_per_layer": round(ms_per_step * 1e3, 2),
-        "decode_tokens_per_s": round(len(cfg["ctx"]) / (dt / args.steps), 1),
-        "attn_launch_us": round(attn_ms * 1e3, 2),
-        "write_launch_us": round(write_ms * 1e3, 2),
-        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": MEASURED_TRAFFIC.get(args.workload),
+        "prewarm_s": PREWARM_S,
+        "pct_hbm_peak": round(100 * t["value"] / HBM_PEAK_GBPS, 2),
+        "us_per_layer": round(t["step_s"] * 1e6, 2),
+        "decode_tokens_per_s": round(len(cfg["ctx"]) / t["step_s"], 1),
+        "attn_launch_us": round(t["attn_s"] * 1e6, 2),
+        "write_launch_us": round(t["write_s"] * 1e6, 2),
+        "roofline": {"bound": "hbm", "achieved": round(t["attn_bytes"] / t["attn_s"] / 1e9, 1), "peak": HBM_PEAK_GBPS,
+                     "unit": "GB/s", "frac": round(t["attn_bytes"] / t["attn_s"] / 1e9 / HBM_PEAK_GBPS, 4),
+                     "traffic": traffic, "traffic_source": traffic_source,
                      "kernel": "paged decode attention launch = paged_decode_streamk_kernel + paged_decode_streamk_reduce_kernel",
-                     "algorithmic_bytes_per_launch": attn_bytes},
+                     "timing": f"{t['n_attn']} attention launches back to back between two events on the launch stream",
+                     "algorithmic_bytes_per_launch": t["attn_bytes"]},
     }
+    if args.workload == "llama3_8b_decode_b64_ctx1k-8k" and not (args.sliding_window or args.soft_cap or args.no_fixed_8k):
+        # the shape the metric's wording names (every context 8192), same steps, in the same line
+        cfg8 = make_batch("llama3_8b_decode_b64_ctx8k_fixed")
+        st8 = build_device_state(cfg8, dev, args.layers)
+        st8["window"], st8["softcap"] = 0, 0.0
+        t8 = time_decode(cfg8, st8, args, ops)
+        res["fixed_ctx_8192"] = {
+            "workload": "llama3_8b_decode_b64_ctx8k_fixed", "sum_ctx": sum(cfg8["ctx"]),
+            "value": round(t8["value"], 1), "unit": "GB/s", "pct_hbm_peak": round(100 * t8["value"] / HBM_PEAK_GBPS, 2),
+            "us_per_layer": round(t8["step_s"] * 1e6, 2), "decode_tokens_per_s": round(len(cfg8["ctx"]) / t8["step_s"], 1),
+            "attn_launch_us": round(t8["attn_s"] * 1e6, 2),
+            "roofline_frac": round(t8["attn_bytes"] / t8["attn_s"] / 1e9 / HBM_PEAK_GBPS, 4),
+            "algorithmic_bytes_per_launch": t8["attn_bytes"]}
+        del st8
     if not args.no_cpu_baseline:
         res["cpu_baseline"] = cpu_baseline(cfg, st, args.cpu_seconds)
     print(json.dumps(res))
