@@ -75,7 +75,71 @@ def test_selection_and_reasons():
         P.get_attn_backend_cls(**{**ok, "kv_cache_dtype": "auto"})
     with pytest.raises(ValueError):
         P.get_attn_backend_cls("FLASH_ATTN", **ok)
-    P.register_attention_backends()                    # no upstream vLLM here: must be a no-op
+    assert P.register_attention_backends() is False    # nothing is overwritten by default
+    assert P.register_attention_backends(replace_slots=True) is False   # no upstream vLLM here: a no-op
+
+
+def test_register_returns_the_platform_and_the_platform_routes_by_kv_dtype():
+    """register() names the platform class, as the reference's does (vllm_metax/__init__.py:14-16); the platform
+    sends int8 KV dtypes to this build's backends and refuses to swallow the others."""
+    import importlib
+
+    import vllm_metax_amd
+
+    path = vllm_metax_amd.register()
+    assert path == P.PLATFORM_PATH
+    module, _, cls = path.rpartition(".")
+    plat = getattr(importlib.import_module(module), cls)
+    sel = types.SimpleNamespace(kv_cache_dtype="int8_per_token_head", head_size=128, dtype=torch.bfloat16, block_size=16)
+    assert plat.get_attn_backend_cls(None, sel, 32) == P.INT8_ATTN_PATH
+    mla = types.SimpleNamespace(kv_cache_dtype="int8_per_token", dtype=torch.bfloat16, block_size=64, use_mla=True)
+    assert plat.get_attn_backend_cls(None, mla, 128) == P.INT8_MLA_PATH
+    with pytest.raises(ValueError, match="does not serve kv_cache_dtype"):
+        plat.get_attn_backend_cls("FLASH_ATTN", sel, 32)
+    with pytest.raises(ValueError, match="not served by this build"):          # no upstream platform to hand it to here
+        plat.get_attn_backend_cls(None, types.SimpleNamespace(kv_cache_dtype="auto"), 32)
+    vllm_metax_amd.register_out_of_tree()
+    toml = open(os.path.join(ROOT, "vllm-metax_amd", "pyproject.toml")).read()
+    assert 'vllm.platform_plugins' in toml and '"vllm_metax_amd:register"' in toml
+    assert 'vllm.general_plugins' in toml and '"vllm_metax_amd:register_out_of_tree"' in toml
+
+
+def test_mla_builder_splits_decodes_first_and_needs_no_gpu():
+    from vllm_metax_amd.v1.attention.backends.mla.int8_mla import Int8MLAMetadataBuilder
+
+    assert Int8MLABackend.get_builder_cls() is Int8MLAMetadataBuilder
+    assert Int8MLAMetadataBuilder._cudagraph_support.name == "UNIFORM_SINGLE_TOKEN_DECODE"
+    assert Int8AttentionMetadataBuilder._cudagraph_support.name == "ALWAYS"
+    spec = types.SimpleNamespace(block_size=64, num_kv_heads=1, head_size=576, num_heads=16)
+    cfg = types.SimpleNamespace(scheduler_config=types.SimpleNamespace(max_num_seqs=4))
+    b = Int8MLAMetadataBuilder(spec, ["l0"], cfg, "cpu")
+    c = types.SimpleNamespace(num_reqs=3, num_actual_tokens=7, max_query_len=5, max_seq_len=90,
+                              query_start_loc=torch.tensor([0, 1, 2, 7], dtype=torch.int32),
+                              seq_lens=torch.tensor([9, 4, 90], dtype=torch.int32),
+                              block_table_tensor=torch.zeros((3, 2), dtype=torch.int32),
+                              slot_mapping=torch.arange(7))
+    md = b.build(0, c)
+    assert (md.num_decodes, md.num_decode_tokens, md.num_prefills) == (2, 2, 1)
+    assert md.decode.seq_lens.tolist() == [9, 4] and md.decode.block_table.shape == (2, 2)
+    assert md.workspace is None and md.decode_out is None      # no GPU: nothing reserved
+    c.query_start_loc = torch.tensor([0, 5, 6, 7], dtype=torch.int32)           # a decode after a prefill
+    with pytest.raises(RuntimeError, match="decode requests must come first"):
+        b.build(0, c)
+
+
+def test_impl_fills_scale_views_once_per_cache_tensor():
+    impl = Int8AttentionImpl(8, 128, 0.09, 2)
+    from vllm_metax_amd import layout as L
+
+    a = L.allocate_kv_cache(4, 16, 2, 128, device="cpu")
+    b = L.allocate_kv_cache(4, 16, 2, 128, device="cpu")
+    impl._ensure_scale_caches(a)
+    ks, vs = L.scale_views(a)
+    assert bool((ks == 1).all()) and bool((vs == 1).all())
+    ks.fill_(0.5)                                              # scales a write has stored
+    impl._ensure_scale_caches(b)
+    impl._ensure_scale_caches(a)                               # back on A: must not be wiped
+    assert bool((L.scale_views(a)[0] == 0.5).all())
 
 
 def test_impl_constructor_errors():

@@ -68,3 +68,41 @@ def test_decode_step_through_the_backend(gpu_device, layout, monkeypatch):
                              torch.tensor(ctx, dtype=torch.int32), torch.arange(B + 1, dtype=torch.int32),
                              1 / math.sqrt(d))
     T.assert_close_attn(out[:B].view(B, hq, d), want, what=f"backend decode {layout}")
+
+
+def test_impl_keeps_the_scales_of_a_cache_it_comes_back_to(gpu_device):
+    """One impl, two cache tensors: write to A, touch B, attend on A.  The scale views are filled with 1.0
+    only the first time a tensor is seen, so A's stored scales survive the visit to B."""
+    dev = gpu_device
+    hq, hkv, d, bs, nb = 8, 2, 128, 16, 12
+    ctx = [70, 33]
+    B = len(ctx)
+    g = torch.Generator().manual_seed(3)
+    impl = Int8AttentionBackend.get_impl_cls()(hq, d, 0.09, hkv, kv_cache_dtype="int8_per_token_head")
+    kv_a = L.allocate_kv_cache(nb, bs, hkv, d, device=dev, layout="NHD")
+    kv_b = L.allocate_kv_cache(nb, bs, hkv, d, device=dev, layout="NHD")
+    kv_cpu, views, lay = T.cpu_cache(nb, bs, hkv, d, "NHD")
+    views[2].fill_(1.0)
+    views[3].fill_(1.0)
+    bt = T.make_block_tables(ctx, bs, nb, g)
+    slots = T.slots_for(bt, ctx, bs)
+    layer = types.SimpleNamespace()
+    for i, c in enumerate(ctx):
+        k = torch.randn((c, hkv, d), generator=g).to(torch.bfloat16)
+        v = torch.randn((c, hkv, d), generator=g).to(torch.bfloat16)
+        impl.do_kv_cache_update(layer, k.to(dev), v.to(dev), kv_a, slots[i].to(dev))
+        oracle.cache_write(k, v, T.storage_bytes(kv_cpu), lay, slots[i])
+    junk = torch.randn((5, hkv, d), generator=g).to(torch.bfloat16).to(dev)
+    impl.do_kv_cache_update(layer, junk, junk, kv_b, torch.arange(5, dtype=torch.int64, device=dev))   # touch B
+    q = torch.randn((B, hq * d), generator=g).to(torch.bfloat16)
+    md = types.SimpleNamespace(num_actual_tokens=B, max_query_len=1, max_seq_len=max(ctx), use_cascade=False,
+                               query_start_loc=torch.arange(B + 1, dtype=torch.int32, device=dev),
+                               seq_lens=torch.tensor(ctx, dtype=torch.int32, device=dev), causal=True,
+                               block_table=bt.to(dev), workspace=None)
+    out = torch.zeros((B, hq * d), dtype=torch.bfloat16, device=dev)
+    impl.forward(layer, q.to(dev), None, None, kv_a, md, out)                                            # back on A
+    torch.cuda.synchronize()
+    assert torch.equal(T.storage_bytes(kv_a).cpu(), T.storage_bytes(kv_cpu)), "A's bytes changed by the visit to B"
+    want = oracle.paged_attn(q.view(B, hq, d), T.storage_bytes(kv_cpu), lay, bt, torch.tensor(ctx, dtype=torch.int32),
+                             torch.arange(B + 1, dtype=torch.int32), 0.09)
+    T.assert_close_attn(out.view(B, hq, d), want, what="attend on A after touching B")

@@ -57,6 +57,39 @@ def test_config1_shape(gpu_device, layout):
     torch.testing.assert_close(lse.cpu(), want_lse, atol=2e-3, rtol=1e-3)
 
 
+def test_config1_as_worded_fp32_sources_written_on_the_gpu(gpu_device):
+    """The first configuration to the letter: K / V sources are fp32 N(0, 1), quantised per token and head by
+    the write kernel itself (bit-exact against the oracle's cache), block tables a seeded permutation of the
+    128-block pool, Q bf16, output bf16 [4, 32, 128]."""
+    dev = gpu_device
+    hq, hkv, d, bs, nb = 32, 8, 128, 16, 128
+    ctx = [512] * 4
+    g = torch.Generator().manual_seed(0)
+    bt = torch.randperm(nb, generator=g).to(torch.int32).view(4, 32)
+    kv_cpu, _, lay = T.cpu_cache(nb, bs, hkv, d, "NHD")
+    kv = L.allocate_kv_cache(nb, bs, hkv, d, device=dev, layout="NHD")
+    k, v = L.key_value_views(kv)
+    ks, vs = L.scale_views(kv)
+    for i, slots in enumerate(T.slots_for(bt, ctx, bs)):
+        key = torch.randn((ctx[i], hkv, d), generator=g, dtype=torch.float32)
+        val = torch.randn((ctx[i], hkv, d), generator=g, dtype=torch.float32)
+        oracle.cache_write(key, val, T.storage_bytes(kv_cpu), lay, slots)
+        ops.reshape_and_cache_flash_per_token_head_quant(key.to(dev), val.to(dev), k, v, ks, vs, slots.to(dev))
+    torch.cuda.synchronize()
+    assert torch.equal(T.storage_bytes(kv).cpu(), T.storage_bytes(kv_cpu)), "quantised cache differs from the oracle"
+    q = torch.randn((4, hq, d), generator=g).to(torch.bfloat16)
+    sl = torch.tensor(ctx, dtype=torch.int32)
+    cu = torch.arange(5, dtype=torch.int32)
+    scale = 1 / math.sqrt(d)
+    out = torch.full(q.shape, float("nan"), dtype=torch.bfloat16, device=dev)
+    ops.unified_attention(q.to(dev), k, v, out, cu.to(dev), 1, sl.to(dev), 512, scale, True, block_table=bt.to(dev),
+                          k_scale_cache=ks, v_scale_cache=vs)
+    torch.cuda.synchronize()
+    want = oracle.paged_attn(q, T.storage_bytes(kv_cpu), lay, bt, sl, cu, scale)
+    assert out.shape == (4, 32, 128) and out.dtype == torch.bfloat16
+    T.assert_close_attn(out, want, what="config 1 as worded")
+
+
 @pytest.mark.parametrize("ctx", [[1], [31, 32, 33], [15, 16, 17, 1, 2], [1000, 3, 517, 64, 4097], [700] * 70])
 def test_ragged_lengths_fp32_out(gpu_device, ctx):
     """Ragged and tiny contexts, sequence boundaries falling inside workgroup ranges, more

@@ -5,7 +5,7 @@
 // Per tile it
 //   * reads the 32 records as flat 16-byte chunks, consecutive lanes taking consecutive chunks
 //     of one record, so every quarter-wave touches 256 contiguous bytes of HBM; the chunks land
-//     in registers, two tiles ahead of the tile being computed;
+//     in registers, one tile ahead of the tile being computed;
 //   * drops the chunks into a wave-private LDS window (one record per row, 16-byte aligned,
 //     bank-conflict-free pitch) and reads them back in MFMA operand order: the transposition
 //     between "how memory is laid out" and "how the matrix core wants it" happens in LDS;
@@ -93,10 +93,16 @@ struct AttnIO {
   float cap_k;        // 2 * log2(e) / cap_c
 };
 
-// cap * tanh(x / cap) for a log2-domain logit x: tanh(u) = 1 - 2 / (exp(2u) + 1).  Saturates
-// cleanly at +-cap; the absolute error is about cap * 2^-23 (models use caps of 30 .. 50).
+// cap * tanh(x / cap) for a log2-domain logit x.  Away from zero tanh(u) = 1 - 2 / (exp(2u) + 1), which
+// saturates cleanly at +-cap but whose absolute error is about cap * 2^-23 whatever x is; for |u| < 1/8
+// the odd series u (1 - u^2/3 + 2 u^4/15) takes over (next term 17/315 u^6 < 2e-7), so the result is
+// accurate RELATIVE to x for every cap, and a cap far above the logits is the identity.
 __device__ __forceinline__ float soft_cap(float x, float cap_c, float cap_k) {
-  return cap_c - 2.0f * cap_c * __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(x * cap_k) + 1.0f);
+  const float big = cap_c - 2.0f * cap_c * __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(x * cap_k) + 1.0f);
+  const float u = x * cap_k * 0.34657359f;  // x / cap_c: cap_k = 2 log2(e) / cap_c
+  const float u2 = u * u;
+  const float small = x * (1.0f + u2 * (-0.33333334f + u2 * 0.13333334f));
+  return fabsf(u) < 0.125f ? small : big;
 }
 
 // First token a decode row of a `len`-token sequence sees.

@@ -5,17 +5,19 @@
 // token), so this is a dense contraction: S^T[token, head] = C . Q^T over 576 dims and
 // O^T[dim, head] = C[:, :512]^T . P~^T, both on the MFMA with the heads as the N dimension.
 //
-// Work item = (sequence, token split); workgroup = 8 waves, wave w owns heads 16w .. 16w+15 of a
-// 128-head group and keeps their 512 x 16 output tile in registers; their absorbed Q sits in
-// registers (8 of its 18 operands) and LDS as two int8 terms that a small kernel prepares once per
-// launch, so the QK product reads the cached code bytes as they are.  The workgroup loads each
-// 32-token tile once, as flat 16-byte chunks (every quarter-wave reads 256 contiguous bytes),
-// through registers into a double-buffered LDS window, and transposes its V part ONCE, shared by
-// the eight waves, into an fp16 V^T tile (plain codes, byte permutes in registers); every wave
-// then feeds the PV MFMA with 16-byte LDS reads.  Two barriers per tile: V^T visible / V^T free.
-// (Before, each wave transposed and expanded the tile for itself: 8x the vector work, ~320
-// instructions per tile per wave.  A 32-head tile per wave would also halve the LDS reads per flop
-// but needs 400 of a lane's 512 registers for Q and O alone.)
+// Work item = (sequence, token split, 128-head block); workgroup = 8 waves.  Each 32-token tile of
+// the latent stream goes from global memory STRAIGHT into a double-buffered LDS window
+// (buffer_load ... lds, no registers in between), a whole tile time ahead of its use; the 16-byte
+// chunks of a row are swizzled so that operand reads are free of bank conflicts without padding.
+// QK: wave w owns head tile w (16 heads) of the block and computes that tile's logits on the int8
+// MFMA straight from the cached code bytes; its absorbed Q sits in registers (10 of its 18
+// operands) and LDS (the other 8) as two int8 terms that a small kernel prepares once per launch.
+// It runs the tile's softmax (lazy reference maximum) and publishes the P~ operand, the rescale
+// factors and a "maximum moved" flag through a double-buffered LDS exchange.
+// PV is split over the waves by OUTPUT DIMS, not by heads: wave w accumulates dims 64 w .. 64 w + 63
+// of all 128 heads, so it transposes only those 64 dims of the tile into its own, wave-private
+// fp16 V^T (byte permutes in registers) and reads eight P~ operands per tile.  One workgroup
+// barrier per tile (P~ and the next raw tile visible).
 // The token splits of a sequence are merged by the reduce kernel with the log-sum-exp algebra
 // (same two-stage shape as the reference's decode_attention_fwd); nothing is allocated here,
 // partials and the int8 Q live in the caller's workspace.

@@ -13,6 +13,8 @@ namespace kvq {
 int launch_decode_streamk(const StreamKArgs& a, int q_dtype, int out_dtype, hipStream_t s);
 size_t streamk_workspace_bytes(int max_num_seqs, int num_q_heads, int head_size, int num_wg);
 int decode_streamk_num_wg(int num_kv_heads);
+int validate_common(const char* op, const void* q, const void* cache, const kvq_cache_geom* geom,
+                    const int32_t* block_table, const int32_t* seq_lens, int num_seqs, int num_q_heads);
 int launch_prefill(const AttnIO& io, const int32_t* seq_lens, const int32_t* cu_seqlens_q, int num_seqs,
                    int max_query_len, int causal, int q_dtype, int out_dtype, hipStream_t s);
 
@@ -56,29 +58,15 @@ static int paged_attn_launch(const char* op, void* out, int out_dtype, int64_t o
                              int max_query_len, float scale, int causal, int window_size, float softcap, float* lse,
                              void* workspace, size_t workspace_bytes, const char* workspace_what,
                              kvq_stream_t stream) {
-  KVQ_REQUIRE(geom != nullptr, "%s: geom is NULL", op);
-  KVQ_REQUIRE(out && q && cache && block_table && seq_lens, "%s: NULL pointer", op);
-  KVQ_REQUIRE(num_seqs > 0 && num_q_heads > 0, "%s: num_seqs and num_q_heads must be positive", op);
+  int rc0 = validate_common(op, q, cache, geom, block_table, seq_lens, num_seqs, num_q_heads);
+  if (rc0) return rc0;
+  KVQ_REQUIRE(out != nullptr, "%s: out is NULL", op);
   KVQ_REQUIRE(max_query_len >= 1, "%s: max_query_len must be >= 1", op);
   KVQ_REQUIRE(max_query_len == 1 || cu_seqlens_q != nullptr, "%s: cu_seqlens_q is required when max_query_len > 1", op);
   KVQ_REQUIRE(window_size >= 0, "%s: window_size %d must be >= 0 (0 = no sliding window)", op, window_size);
   KVQ_REQUIRE(window_size == 0 || causal, "%s: a sliding window needs causal attention", op);
   KVQ_REQUIRE(softcap >= 0.f && softcap == softcap, "%s: softcap must be >= 0 (0 = none)", op);
   const kvq_cache_geom& g = *geom;
-  KVQ_REQUIRE(g.num_kv_heads > 0 && num_q_heads % g.num_kv_heads == 0,
-              "%s: num_q_heads %d is not a multiple of num_kv_heads %d", op, num_q_heads, g.num_kv_heads);
-  KVQ_REQUIRE(num_q_heads / g.num_kv_heads <= 16, "%s: more than 16 q heads per kv head is not supported", op);
-  KVQ_REQUIRE(g.head_size == 64 || g.head_size == 128 || g.head_size == 256,
-              "%s: head_size %d not supported (64, 128, 256)", op, g.head_size);
-  KVQ_REQUIRE(g.block_size > 0 && g.block_size % 16 == 0, "%s: block_size %d must be a multiple of 16", op,
-              g.block_size);
-  KVQ_REQUIRE((g.k_off | g.v_off | g.ks_off | g.vs_off | g.stride_block | g.stride_slot | g.stride_head) % 4 == 0 &&
-                  ((uintptr_t)cache % 4) == 0,
-              "%s: cache offsets/strides must be 4-byte aligned", op);
-  KVQ_REQUIRE(g.ks_off - g.k_off == g.head_size && g.v_off - g.k_off == g.head_size + 4 &&
-                  g.vs_off - g.k_off == 2 * g.head_size + 4,
-              "%s: a cache record must be [K codes | K scale | V codes | V scale]", op);
-  KVQ_REQUIRE(g.stride_slot > 0 && g.stride_slot <= 0x7fffffff / 64, "%s: stride_slot out of range", op);
   const int osz = out_dtype == KVQ_F32 ? 4 : 2;
   KVQ_REQUIRE(((uintptr_t)out % 4) == 0 && (out_stride_t * osz) % 4 == 0 && (out_stride_h * osz) % 4 == 0,
               "%s: out rows must be 4-byte aligned", op);

@@ -75,7 +75,7 @@ int heads_per_wg(int num_kv_heads) {
 // Resident workgroups the stream-K launch uses: one eight-wave workgroup per compute unit.
 static int streamk_num_wg(int) { return num_cus(); }
 
-static int validate_common(const char* op, const void* q, const void* cache, const kvq_cache_geom* geom,
+int validate_common(const char* op, const void* q, const void* cache, const kvq_cache_geom* geom,
                            const int32_t* block_table, const int32_t* seq_lens, int num_seqs, int num_q_heads) {
   KVQ_REQUIRE(geom != nullptr, "%s: geom is NULL", op);
   KVQ_REQUIRE(q && cache && block_table && seq_lens, "%s: NULL pointer", op);

@@ -8,9 +8,17 @@ __version__ = "0.1.0"
 
 
 def register():
-    """vllm.platform_plugins entry point: registers the attention backends with upstream
-    vLLM's registry (when importable) and returns nothing else to override."""
+    """``vllm.platform_plugins`` entry point: the class path of the platform, as the reference's
+    ``register()`` returns ``"vllm_metax.platform.MacaPlatform"`` (vllm_metax/__init__.py:14-16)."""
+    from .platform import PLATFORM_PATH
+
+    return PLATFORM_PATH
+
+
+def register_out_of_tree():
+    """``vllm.general_plugins`` entry point (the reference's runs its patches and registry module,
+    vllm_metax/__init__.py:30-32): nothing is overwritten by default -- the platform routes the int8
+    KV-cache dtypes to this build's backends and leaves every other dtype to upstream's."""
     from .platform import register_attention_backends
 
-    register_attention_backends()
-    return None
+    register_attention_backends(replace_slots=False)

@@ -165,13 +165,22 @@ def paged_attn_workspace_bytes(max_num_seqs: int, num_q_heads: int, head_size: i
 
 
 _ws_cache: dict = {}
+_ws_retired: list = []
 
 
 def _default_workspace(dev: torch.device, nbytes: int) -> torch.Tensor:
     """Grow-only per-device scratch for callers that did not bring their own (tests, eager use).
-    The backend's metadata builder pre-sizes its own instead, so a captured step never lands here."""
+    The backends' metadata builders pre-size their own instead, so a captured step never lands here.
+    A buffer that is outgrown is kept alive, not freed: a HIP graph captured earlier may still hold
+    its address.  Growing while a capture is under way is refused (it would allocate inside the
+    capture and leave the graph with a buffer no later call uses)."""
     cur = _ws_cache.get(dev)
     if cur is None or cur.numel() < nbytes:
+        if torch.cuda.is_current_stream_capturing():
+            raise RuntimeError("the default workspace would have to grow during stream capture: pass a "
+                               "pre-sized workspace (the metadata builders hold one)")
+        if cur is not None:
+            _ws_retired.append(cur)
         cur = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=dev)
         _ws_cache[dev] = cur
     return cur

@@ -26,6 +26,19 @@ from ....layout import (
 )
 
 try:  # pragma: no cover - upstream vLLM is not installed in the build container
+    from vllm.v1.attention.backend import AttentionCGSupport  # type: ignore
+except Exception:  # noqa: BLE001
+    import enum as _enum
+
+    class AttentionCGSupport(_enum.Enum):
+        """Stand-in for upstream's enum of the same name (what a builder promises to graph capture)."""
+
+        ALWAYS = 3
+        UNIFORM_BATCH = 2
+        UNIFORM_SINGLE_TOKEN_DECODE = 1
+        NEVER = 0
+
+try:  # pragma: no cover - upstream vLLM is not installed in the build container
     from vllm.v1.attention.backend import (  # type: ignore
         AttentionBackend as _BackendBase,
         AttentionImpl as _ImplBase,
@@ -80,6 +93,9 @@ class Int8AttentionMetadataBuilder(_BuilderBase):
     """Counterpart of TritonAttentionMetadataBuilder
     (vllm_metax/v1/attention/backends/triton_attn.py:102-269): packs the common metadata and owns
     the scratch that ``forward`` uses, sized once so a captured decode step never allocates."""
+
+    # the kernels read lengths and tables on the device and nothing is allocated per step (:103)
+    _cudagraph_support: ClassVar[AttentionCGSupport] = AttentionCGSupport.ALWAYS
 
     def __init__(self, kv_cache_spec, layer_names, vllm_config, device):
         if _BuilderBase is not object:  # pragma: no cover
@@ -276,8 +292,9 @@ class Int8AttentionImpl(_ImplBase):
         self.logits_soft_cap = float(logits_soft_cap or 0)
         self._kv_quant_mode = get_kv_quant_mode(kv_cache_dtype)
         self._is_per_token_head_quant = True
-        # per-cache views and byte geometry, built at first use (one cache tensor per layer)
-        self._views_for: int | None = None
+        # per-cache views and byte geometry, built when a cache tensor is first seen
+        self._views: dict = {}
+        self._views_for = None
         self._key_cache = self._value_cache = None
         self._k_scale_cache = self._v_scale_cache = None
         self._geometry = None
@@ -290,17 +307,24 @@ class Int8AttentionImpl(_ImplBase):
 
     # -- cache views ---------------------------------------------------------------------------
     def _ensure_scale_caches(self, kv_cache: torch.Tensor) -> None:
-        """fp32 strided views over the inline scale bytes, filled with 1.0 at first use, as
-        vllm_metax/v1/attention/backends/triton_attn.py:418-479."""
+        """fp32 strided views over the inline scale bytes, as
+        vllm_metax/v1/attention/backends/triton_attn.py:418-479.  The reference builds them -- and
+        fills the scales with 1.0 -- once per impl, at first use; an impl here may meet several cache
+        tensors (tests, a re-bound cache), so the views are kept per tensor and the fill happens only
+        the first time a tensor is seen: coming back to a cache never wipes the scales written into it."""
         key = (kv_cache.data_ptr(), tuple(kv_cache.shape), tuple(kv_cache.stride()))
         if self._views_for == key:
             return
-        self._k_scale_cache, self._v_scale_cache = scale_views(kv_cache)
-        self._k_scale_cache.fill_(1.0)
-        self._v_scale_cache.fill_(1.0)
-        self._key_cache, self._value_cache = key_value_views(kv_cache)
-        self._geometry = geometry_from_views(self._key_cache, self._value_cache, self._k_scale_cache,
-                                             self._v_scale_cache)
+        got = self._views.get(key)
+        if got is None:
+            k_scale, v_scale = scale_views(kv_cache)
+            k_scale.fill_(1.0)
+            v_scale.fill_(1.0)
+            key_cache, value_cache = key_value_views(kv_cache)
+            got = (key_cache, value_cache, k_scale, v_scale,
+                   geometry_from_views(key_cache, value_cache, k_scale, v_scale))
+            self._views[key] = got
+        self._key_cache, self._value_cache, self._k_scale_cache, self._v_scale_cache, self._geometry = got
         self._views_for = key
 
     def _pth_key_value_caches(self, kv_cache: torch.Tensor):

@@ -9,6 +9,7 @@ region after them inside each block) is this build's: the reference's MLA backen
 """
 from __future__ import annotations
 
+from dataclasses import dataclass
 from typing import ClassVar
 
 import torch
@@ -16,7 +17,12 @@ import torch
 from ..... import _custom_ops as ops
 from .....kv_cache_interface import INT8_PER_TOKEN
 from .....layout import mla_cache_shape, mla_geometry
-from ..int8_attn import AttentionType, MultipleOf
+from ..int8_attn import AttentionCGSupport, AttentionType, MultipleOf, _BackendBase, _BuilderBase, _first_attr
+
+try:  # pragma: no cover - upstream vLLM is not installed in the build container
+    from vllm.v1.attention.backend import MLAAttentionImpl as _MLAImplBase  # type: ignore
+except Exception:  # noqa: BLE001
+    _MLAImplBase = object
 
 # num_kv_splits policy of the reference (vllm_metax/v1/attention/backends/mla/triton_mla.py:42-55)
 _MIN_WORK_PER_SPLIT = 512
@@ -32,7 +38,111 @@ def _compute_num_kv_splits(max_seq_len: int, sm_count: int) -> int:
     return min(ideal, sm_count * _SPLIT_OCCUPANCY_MULTIPLIER)
 
 
-class Int8MLABackend:
+@dataclass
+class Int8MLADecodeMetadata:
+    """The decode half of the MLA metadata, fields of MLACommonDecodeMetadata that ``forward_mqa`` reads
+    (vllm_metax/v1/attention/backends/mla/triton_mla.py:283-284)."""
+
+    block_table: torch.Tensor
+    seq_lens: torch.Tensor
+
+
+@dataclass
+class Int8MLAMetadata:
+    """What the MLA layer and ``forward_mqa`` read of MLACommonMetadata
+    (vllm_metax/model_executor/layers/attention/mla_attention.py:1384-1440): the split of the batch into
+    decode requests (first, one token each) and prefill requests, and the decode half; plus the buffers
+    the builder owns so that a decode step allocates nothing."""
+
+    num_actual_tokens: int
+    num_reqs: int
+    max_query_len: int
+    max_seq_len: int
+    query_start_loc: torch.Tensor
+    slot_mapping: torch.Tensor
+    num_decodes: int
+    num_decode_tokens: int
+    num_prefills: int
+    decode: Int8MLADecodeMetadata | None
+    workspace: torch.Tensor | None = None   # split states + int8 query terms of the decode launch
+    decode_out: torch.Tensor | None = None  # [max_num_seqs, H, kv_lora_rank]
+    decode_lse: torch.Tensor | None = None  # [max_num_seqs, H] fp32
+
+
+class Int8MLAMetadataBuilder(_BuilderBase):
+    """Counterpart of TritonMLAMetadataBuilder (vllm_metax/v1/attention/backends/mla/triton_mla.py:57-88) and
+    of the decode side of MLACommonMetadataBuilder.build (mla_attention.py:1753-1960): decode requests come
+    first in the batch (``reorder_batch_threshold = 1``, mla_attention.py:1546-1551) and are split off on
+    the host copy of the lengths, with no device synchronisation; the decode launch's scratch is reserved
+    once, at the worst case (``max_num_seqs`` decode tokens), as ``_reserve_attn_logits_workspace`` does,
+    so a step -- captured or not -- never allocates."""
+
+    _cudagraph_support: ClassVar[AttentionCGSupport] = AttentionCGSupport.UNIFORM_SINGLE_TOKEN_DECODE
+    reorder_batch_threshold: int = 1
+
+    def __init__(self, kv_cache_spec, layer_names, vllm_config, device):
+        if _BuilderBase is not object:  # pragma: no cover
+            super().__init__(kv_cache_spec, layer_names, vllm_config, device)
+        self.kv_cache_spec = kv_cache_spec
+        self.layer_names = layer_names
+        self.vllm_config = vllm_config
+        self.device = torch.device(device)
+        model_config = getattr(vllm_config, "model_config", None)
+        parallel_config = getattr(vllm_config, "parallel_config", None)
+        if model_config is not None and hasattr(model_config, "get_num_attention_heads"):
+            self.num_heads = model_config.get_num_attention_heads(parallel_config)
+        else:
+            self.num_heads = _first_attr(kv_cache_spec, "num_q_heads", "num_heads", default=None)
+        hf = getattr(getattr(model_config, "hf_text_config", None), "kv_lora_rank", None)
+        self.kv_lora_rank = int(hf or _first_attr(kv_cache_spec, "kv_lora_rank", default=512))
+        sched = getattr(vllm_config, "scheduler_config", None)
+        self.max_num_seqs = int(_first_attr(sched, "max_num_seqs", default=256)) if sched is not None else 256
+        self.dtype = _first_attr(model_config, "dtype", default=torch.bfloat16) if model_config is not None \
+            else torch.bfloat16
+        self._workspace = self._out = self._lse = None
+        self._reserve_decode_buffers()
+
+    def _reserve_decode_buffers(self) -> None:
+        if self.device.type != "cuda" or self.num_heads is None:
+            return
+        nbytes = ops.mla_decode_workspace_bytes(self.max_num_seqs, self.num_heads, self.kv_lora_rank)
+        self._workspace = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=self.device)
+        self._out = torch.empty((self.max_num_seqs, self.num_heads, self.kv_lora_rank), dtype=self.dtype,
+                                device=self.device)
+        self._lse = torch.empty((self.max_num_seqs, self.num_heads), dtype=torch.float32, device=self.device)
+
+    def build_for_cudagraph_capture(self, common_attn_metadata) -> Int8MLAMetadata:
+        md = self.build(0, common_attn_metadata)
+        if md.decode is not None:
+            md.decode.seq_lens.fill_(1)
+        return md
+
+    def build(self, common_prefix_len: int, common_attn_metadata, fast_build: bool = False) -> Int8MLAMetadata:
+        c = common_attn_metadata
+        if c.num_reqs > self.max_num_seqs:
+            raise RuntimeError(f"batch of {c.num_reqs} sequences exceeds max_num_seqs={self.max_num_seqs}")
+        qsl_cpu = getattr(c, "query_start_loc_cpu", None)
+        if qsl_cpu is None:
+            qsl_cpu = c.query_start_loc.cpu() if c.query_start_loc.is_cuda else c.query_start_loc
+        qlens = (qsl_cpu[1:c.num_reqs + 1] - qsl_cpu[:c.num_reqs]).tolist()
+        num_decodes = 0
+        while num_decodes < len(qlens) and qlens[num_decodes] <= self.reorder_batch_threshold:
+            num_decodes += 1
+        if any(q <= self.reorder_batch_threshold for q in qlens[num_decodes:]):
+            raise RuntimeError("decode requests must come first in the batch (reorder_batch_threshold = 1)")
+        num_decode_tokens = int(qsl_cpu[num_decodes])
+        decode = None
+        if num_decodes > 0:
+            decode = Int8MLADecodeMetadata(block_table=c.block_table_tensor[:num_decodes],
+                                           seq_lens=c.seq_lens[:num_decodes])
+        return Int8MLAMetadata(
+            num_actual_tokens=c.num_actual_tokens, num_reqs=c.num_reqs, max_query_len=c.max_query_len,
+            max_seq_len=c.max_seq_len, query_start_loc=c.query_start_loc, slot_mapping=c.slot_mapping,
+            num_decodes=num_decodes, num_decode_tokens=num_decode_tokens, num_prefills=c.num_reqs - num_decodes,
+            decode=decode, workspace=self._workspace, decode_out=self._out, decode_lse=self._lse)
+
+
+class Int8MLABackend(_BackendBase):
     supported_dtypes: ClassVar[list[torch.dtype]] = [torch.float16, torch.bfloat16]
     supported_kv_cache_dtypes: ClassVar[list[str]] = [INT8_PER_TOKEN]
 
@@ -83,8 +193,12 @@ class Int8MLABackend:
     def get_impl_cls():
         return Int8MLAImpl
 
+    @staticmethod
+    def get_builder_cls():
+        return Int8MLAMetadataBuilder
 
-class Int8MLAImpl:
+
+class Int8MLAImpl(_MLAImplBase):
     """Decode half of TritonMLAImpl (vllm_metax/v1/attention/backends/mla/triton_mla.py:140-295)."""
 
     can_return_lse_for_decode: bool = True
@@ -136,13 +250,24 @@ class Int8MLAImpl:
         # (vllm_metax/v1/attention/backends/mla/triton_mla.py:236-237)
         q0 = q[0] if type(q) is tuple else q
         B, H = q0.shape[0], q0.shape[1]
-        o = torch.empty((B, H, self.kv_lora_rank), dtype=q0.dtype, device=q0.device)
-        lse = torch.empty((B, H), dtype=torch.float32, device=q0.device)
+        # the builder's buffers when the metadata carries them (nothing is allocated then: the step can be
+        # captured in a graph); what is returned are views of them, valid until the next decode step
+        o_buf, lse_buf = getattr(attn_metadata, "decode_out", None), getattr(attn_metadata, "decode_lse", None)
+        if o_buf is not None and lse_buf is not None and o_buf.dtype == q0.dtype and o_buf.shape[0] >= B \
+                and o_buf.shape[1] == H and o_buf.shape[2] == self.kv_lora_rank:
+            o, lse = o_buf[:B], lse_buf[:B]
+        else:
+            o = torch.empty((B, H, self.kv_lora_rank), dtype=q0.dtype, device=q0.device)
+            lse = torch.empty((B, H), dtype=torch.float32, device=q0.device)
         ops.mla_decode_int8(q, kv_c_and_k_pe_cache, o, lse, attn_metadata.decode.block_table,
                             attn_metadata.decode.seq_lens, self.scale, self.kv_lora_rank,
                             workspace=getattr(attn_metadata, "workspace", None),
                             geometry=self._geom(kv_c_and_k_pe_cache))
         return o, lse
+
+    def forward_mha(self, *args, **kwargs):
+        raise NotImplementedError("this backend serves the decode half of the MLA layer (forward_mqa); prefill "
+                                  "tokens go through the layer's prefill backend, as in the reference")
 
 
 class Int8MLADecodeCaller:
