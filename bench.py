@@ -113,6 +113,12 @@ def algorithmic_bytes(cfg, include_write=True):
     return attn, write
 
 
+def _quant_mode(cfg):
+    from vllm_metax_amd.kv_cache_interface import KVQuantMode
+
+    return KVQuantMode.FP8_PER_TOKEN_HEAD if cfg.get("kv_dtype") == "fp8" else KVQuantMode.INT8_PER_TOKEN_HEAD
+
+
 def build_device_state(cfg, dev, layers, seed=0, layout="NHD", permute=True):
     from vllm_metax_amd import _custom_ops as ops
     from vllm_metax_amd import layout as L
@@ -142,7 +148,7 @@ def build_device_state(cfg, dev, layers, seed=0, layout="NHD", permute=True):
         ks, vs = L.scale_views(kv)
         ks.fill_(1.0)
         vs.fill_(1.0)
-        geom = L.geometry_from_views(k, v, ks, vs)
+        geom = L.geometry_from_views(k, v, ks, vs, L.code_type_of(_quant_mode(cfg)))
         # fill the context with N(0,1) bf16 sources through the quantise-on-write kernel itself
         for i, c in enumerate(ctx):
             pos = torch.arange(c, device=dev)
@@ -151,7 +157,8 @@ def build_device_state(cfg, dev, layers, seed=0, layout="NHD", permute=True):
                 n = min(32768, c - s0)
                 ksrc = torch.randn((n, hkv, d), device=dev, dtype=torch.float32).to(torch.bfloat16)
                 vsrc = torch.randn((n, hkv, d), device=dev, dtype=torch.float32).to(torch.bfloat16)
-                ops.reshape_and_cache_flash_per_token_head_quant(ksrc, vsrc, k, v, ks, vs, slots[s0:s0 + n], geometry=geom)
+                ops.reshape_and_cache_flash_per_token_head_quant(ksrc, vsrc, k, v, ks, vs, slots[s0:s0 + n],
+                                                                 kv_quant_mode=_quant_mode(cfg), geometry=geom)
         caches.append(dict(kv=kv, k=k, v=v, ks=ks, vs=vs, geom=geom))
     q = torch.randn((B, hq, d), device=dev, dtype=torch.float32).to(torch.bfloat16)
     new_k = torch.randn((B, hkv, d), device=dev, dtype=torch.float32).to(torch.bfloat16)
@@ -160,7 +167,7 @@ def build_device_state(cfg, dev, layers, seed=0, layout="NHD", permute=True):
     ws = torch.empty(ops.paged_attn_workspace_bytes(B, hq, d), dtype=torch.uint8, device=dev)
     torch.cuda.synchronize()
     return dict(bt=bt, bt_d=bt_d, sl_d=sl_d, cu_d=cu_d, slots_new=last.to(dev), caches=caches, q=q, new_k=new_k,
-                new_v=new_v, out=out, ws=ws, scale=1.0 / math.sqrt(d), max_ctx=max(ctx))
+                new_v=new_v, out=out, ws=ws, scale=1.0 / math.sqrt(d), max_ctx=max(ctx), mode=_quant_mode(cfg))
 
 
 def _window_kwargs(st):
@@ -173,11 +180,11 @@ def run_step(st, layer, ops, write=True, attn=True):
     c = st["caches"][layer]
     if write:
         ops.reshape_and_cache_flash_per_token_head_quant(st["new_k"], st["new_v"], c["k"], c["v"], c["ks"], c["vs"],
-                                                         st["slots_new"], geometry=c["geom"])
+                                                         st["slots_new"], kv_quant_mode=st["mode"], geometry=c["geom"])
     if attn:
         ops.unified_attention(st["q"], c["k"], c["v"], st["out"], st["cu_d"], 1, st["sl_d"], st["max_ctx"], st["scale"],
                               True, block_table=st["bt_d"], k_scale_cache=c["ks"], v_scale_cache=c["vs"],
-                              workspace=st["ws"], geometry=c["geom"], **_window_kwargs(st))
+                              workspace=st["ws"], geometry=c["geom"], kv_quant_mode=st["mode"], **_window_kwargs(st))
 
 
 MFMA_F16_PEAK_TFLOPS = 2500.0
@@ -471,6 +478,8 @@ def main():
     ap.add_argument("--sliding-window", type=int, default=0,
                     help="GQA workloads: attend to the last N keys only (0 = full causal, the configured workloads)")
     ap.add_argument("--soft-cap", type=float, default=0.0, help="GQA workloads: logits soft cap (0 = none)")
+    ap.add_argument("--kv-dtype", choices=["int8", "fp8"], default="int8",
+                    help="GQA decode workloads: code format of the cache (fp8 = e4m3fn per-token-head mode of the same layout)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-fixed-8k", action="store_true",
                     help="default workload only: skip the extra fixed-context (64 x 8192) measurement")
@@ -484,6 +493,7 @@ def main():
 
     dev = torch.device("cuda:0")
     cfg = make_batch(args.workload)
+    cfg["kv_dtype"] = args.kv_dtype
     if cfg.get("mla"):
         return mla_main(args, cfg, dev, ops)
     if cfg.get("mixed"):
@@ -493,7 +503,7 @@ def main():
     L = args.layers
     t = time_decode(cfg, st, args, ops)
     traffic, traffic_source = measured_traffic(args.workload)
-    if args.sliding_window or args.soft_cap:
+    if args.sliding_window or args.soft_cap or args.kv_dtype != "int8":
         traffic, traffic_source = None, None
 
     res = {
@@ -512,6 +522,7 @@ def main():
         "config": {"workload": args.workload, "batch": len(cfg["ctx"]), "sum_ctx": sum(cfg["ctx"]),
                    "q_heads": cfg["hq"], "kv_heads": cfg["hkv"], "head_dim": cfg["d"], "block_size": cfg["bs"],
                    "pool_blocks": cfg["pool"], "layer_caches_rotated": L, "kv_layout": "NHD",
+                   **({"kv_dtype": "fp8_per_token_head"} if args.kv_dtype == "fp8" else {}),
                    **({"sliding_window": args.sliding_window} if args.sliding_window else {}),
                    **({"soft_cap": args.soft_cap} if args.soft_cap else {})},
         "prewarm_s": PREWARM_S,
@@ -527,9 +538,11 @@ def main():
                      "timing": f"{t['n_attn']} attention launches back to back between two events on the launch stream",
                      "algorithmic_bytes_per_launch": t["attn_bytes"]},
     }
-    if args.workload == "llama3_8b_decode_b64_ctx1k-8k" and not (args.sliding_window or args.soft_cap or args.no_fixed_8k):
+    if args.workload == "llama3_8b_decode_b64_ctx1k-8k" and not (args.sliding_window or args.soft_cap or args.no_fixed_8k
+                                                                  or args.kv_dtype != "int8"):
         # the shape the metric's wording names (every context 8192), same steps, in the same line
         cfg8 = make_batch("llama3_8b_decode_b64_ctx8k_fixed")
+        cfg8["kv_dtype"] = "int8"
         st8 = build_device_state(cfg8, dev, args.layers)
         st8["window"], st8["softcap"] = 0, 0.0
         t8 = time_decode(cfg8, st8, args, ops)
@@ -541,7 +554,7 @@ def main():
             "roofline_frac": round(t8["attn_bytes"] / t8["attn_s"] / 1e9 / HBM_PEAK_GBPS, 4),
             "algorithmic_bytes_per_launch": t8["attn_bytes"]}
         del st8
-    if not args.no_cpu_baseline:
+    if not args.no_cpu_baseline and args.kv_dtype == "int8":
         res["cpu_baseline"] = cpu_baseline(cfg, st, args.cpu_seconds)
     print(json.dumps(res))
 

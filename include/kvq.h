@@ -27,7 +27,7 @@
 extern "C" {
 #endif
 
-#define KVQ_ABI_VERSION 8
+#define KVQ_ABI_VERSION 9
 
 #define KVQ_OK 0
 #define KVQ_EINVAL (-22)
@@ -62,8 +62,21 @@ typedef struct kvq_cache_geom {
   int64_t k_off, v_off, ks_off, vs_off;           /* bytes */
   int64_t stride_block, stride_slot, stride_head; /* bytes */
   int32_t num_kv_heads, head_size, block_size;
-  int32_t reserved;
+  int32_t code_type;                              /* KVQ_CODE_INT8 (0) or KVQ_CODE_FP8_E4M3 */
 } kvq_cache_geom;
+
+/*
+ * What a code byte of the cache is.  KVQ_CODE_INT8: the reference's
+ * int8_per_token_head mode, scale = absmax / 127, code = rint(x / scale).
+ * KVQ_CODE_FP8_E4M3: its fp8_per_token_head mode over the same record layout (the
+ * element is one byte either way, vllm_metax/v1/attention/backends/triton_attn.py:
+ * 336-348, 729-739): OCP e4m3fn bit patterns, scale = absmax / 448, code = the
+ * e4m3fn number nearest to x / scale (ties to even, saturating at +-448).  Served
+ * by kvq_reshape_and_cache_int8 and kvq_paged_attn_int8 (and its static-scratch
+ * form); the fixed-partition entry point is int8 only.
+ */
+#define KVQ_CODE_INT8 0
+#define KVQ_CODE_FP8_E4M3 1
 
 /* Byte geometry of the int8 MLA latent cache: per block, block_size code rows
  * of (kv_lora_rank + rope_dim) bytes followed by block_size fp32 scales. */

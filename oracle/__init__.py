@@ -146,7 +146,35 @@ def quant_rows(x: torch.Tensor, eps: float | None = None):
     return codes, scales
 
 
-def cache_write(key, value, kv_cache, lay: RecordLayout, slot_mapping, eps: float | None = None):
+CODE_INT8, CODE_FP8 = 0, 1
+
+
+def quant_rows_fp8(x: torch.Tensor, eps: float | None = None):
+    """x [..., D] (CPU) -> (codes uint8 [..., D] holding e4m3fn bit patterns, scales fp32 [...]):
+    scale = max(absmax, eps) / 448, code = nearest e4m3fn to x / scale (ties to even)."""
+    if eps is None:
+        eps = eps_for(x.dtype)
+    xf = _f32c(x)
+    D = xf.shape[-1]
+    rows = xf.numel() // D
+    codes = torch.empty(xf.shape, dtype=torch.uint8)
+    scales = torch.empty(xf.shape[:-1], dtype=torch.float32)
+    _check(
+        lib().kvq_oracle_quant_rows_fp8(_p(xf), _i64(rows), _i64(D), ctypes.c_float(eps), _p(codes), _p(scales)),
+        "kvq_oracle_quant_rows_fp8",
+    )
+    return codes, scales
+
+
+def e4m3fn_table() -> torch.Tensor:
+    """The 256 values of the e4m3fn byte (0x7f / 0xff, the format's NaN, read as +-480 and never produced)."""
+    fn = lib().kvq_oracle_e4m3fn_value
+    fn.restype = ctypes.c_float
+    return torch.tensor([fn(ctypes.c_int(i)) for i in range(256)], dtype=torch.float32)
+
+
+def cache_write(key, value, kv_cache, lay: RecordLayout, slot_mapping, eps: float | None = None,
+                code_type: int = CODE_INT8):
     """Quantise key/value [T', Hkv, D] into kv_cache (CPU int8 storage) in place."""
     if eps is None:
         eps = eps_for(key.dtype)
@@ -155,20 +183,20 @@ def cache_write(key, value, kv_cache, lay: RecordLayout, slot_mapping, eps: floa
     T = sm.shape[0]
     assert kf.shape[0] >= T and kf.shape[1] == lay.num_kv_heads and kf.shape[2] == lay.head_size
     _check(
-        lib().kvq_oracle_cache_write(
+        lib().kvq_oracle_cache_write_ex(
             _p(kf), _p(vf), _p(kv_cache),
             _i64(lay.k_off), _i64(lay.v_off), _i64(lay.ks_off), _i64(lay.vs_off),
             _i64(lay.stride_block), _i64(lay.stride_slot), _i64(lay.stride_head),
             _p(sm), _i64(T), ctypes.c_int(lay.num_kv_heads), ctypes.c_int(lay.head_size),
-            ctypes.c_int(lay.block_size), ctypes.c_float(eps),
+            ctypes.c_int(lay.block_size), ctypes.c_float(eps), ctypes.c_int(code_type),
         ),
-        "kvq_oracle_cache_write",
+        "kvq_oracle_cache_write_ex",
     )
 
 
 def paged_attn(q, kv_cache, lay: RecordLayout, block_table, seq_lens, cu_seqlens_q,
                scale: float, causal: bool = True, return_lse: bool = False, sliding_window: int = 0,
-               soft_cap: float = 0.0):
+               soft_cap: float = 0.0, code_type: int = CODE_INT8):
     """q [N, Hq, D] -> out fp32 [N, Hq, D] (and lse fp32 [N, Hq]).  sliding_window > 0: a query sees its
     last `sliding_window` keys (itself included); soft_cap > 0: logits -> cap * tanh(logit / cap)."""
     qf = _f32c(q)
@@ -178,7 +206,7 @@ def paged_attn(q, kv_cache, lay: RecordLayout, block_table, seq_lens, cu_seqlens
     out = torch.empty((N, Hq, D), dtype=torch.float32)
     lse = torch.empty((N, Hq), dtype=torch.float32) if return_lse else None
     _check(
-        lib().kvq_oracle_paged_attn_ex(
+        lib().kvq_oracle_paged_attn_ex2(
             _p(out), _p(lse), _p(qf), _p(kv_cache),
             _i64(lay.k_off), _i64(lay.v_off), _i64(lay.ks_off), _i64(lay.vs_off),
             _i64(lay.stride_block), _i64(lay.stride_slot), _i64(lay.stride_head),
@@ -186,8 +214,9 @@ def paged_attn(q, kv_cache, lay: RecordLayout, block_table, seq_lens, cu_seqlens
             ctypes.c_int(B), ctypes.c_int(Hq), ctypes.c_int(lay.num_kv_heads), ctypes.c_int(D),
             ctypes.c_int(lay.block_size), ctypes.c_float(scale), ctypes.c_int(1 if causal else 0),
             ctypes.c_int(int(sliding_window or 0)), ctypes.c_float(float(soft_cap or 0.0)),
+            ctypes.c_int(code_type),
         ),
-        "kvq_oracle_paged_attn_ex",
+        "kvq_oracle_paged_attn_ex2",
     )
     return (out, lse) if return_lse else out
 

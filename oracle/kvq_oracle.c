@@ -12,6 +12,8 @@
  *   kvq_oracle_quant_rows           pinned   (torch CPU round/div, closed forms,
  *                                             exact-rational brute force)
  *   kvq_oracle_cache_write          pinned   (layout algebra + python scatter loop)
+ *   kvq_oracle_quant_rows_fp8       pinned   (torch CPU float8_e4m3fn conversion on every fp32 in range,
+ *                                             the 256-entry decode table against torch, closed forms)
  *   kvq_oracle_paged_attn           pinned   (torch SDPA on gathered K/V, block
  *                                             permutation invariance)
  *   kvq_oracle_paged_attn_partition pinned   (equals unsplit attention for any
@@ -88,6 +90,67 @@ KVQ_EXPORT int kvq_oracle_quant_rows(const float* x, int64_t rows, int64_t D,
 }
 
 /* ---------------------------------------------------------------------------
+ * fp8 (OCP e4m3fn: 1 sign, 4 exponent bits with bias 7, 3 mantissa bits, no infinities, largest
+ * finite value 448) codes of the FP8_PER_TOKEN_HEAD mode of the same layout
+ * (vllm_metax/v1/attention/backends/triton_attn.py:336-348, 729-739: the element is one byte, so the
+ * record keeps its [K | scale | V | scale] shape).  The rule mirrors the int8 one with the format's
+ * maximum in the place of 127: scale = max(absmax, eps) / 448 (fp32 true division), code = the e4m3fn
+ * number nearest to x / scale, ties to even, saturating at +-448.
+ * ------------------------------------------------------------------------- */
+#define KVQ_CODE_INT8 0
+#define KVQ_CODE_FP8 1
+
+static float e4m3fn_value(uint8_t b) {
+  const int e = (b >> 3) & 15, m = b & 7;
+  float v = e == 0 ? ldexpf((float)m, -9) : ldexpf((float)(8 + m), e - 10);
+  return (b & 0x80) ? -v : v;
+}
+
+static uint8_t f32_to_e4m3fn(float y) {
+  const uint8_t sign = signbit(y) ? 0x80 : 0;
+  float a = fabsf(y);
+  if (!(a < 464.0f)) return sign | 0x7e;           /* rounds past 448 (or inf / nan): saturate */
+  if (a < 0.015625f) {                              /* below 2^-6: multiples of 2^-9 */
+    return sign | (uint8_t)nearbyintf(a * 512.0f);  /* 8 is the smallest normal, as it should be */
+  }
+  int e = ilogbf(a);                                /* a = f * 2^e, 1 <= f < 2 */
+  float q = nearbyintf(ldexpf(a, 3 - e));           /* 8 .. 16, ties to even */
+  if (q == 16.0f) {
+    q = 8.0f;
+    ++e;
+  }
+  return sign | (uint8_t)(((e + 7) << 3) | ((int)q - 8));
+}
+
+KVQ_EXPORT float kvq_oracle_e4m3fn_value(int code) { return e4m3fn_value((uint8_t)code); }
+
+KVQ_EXPORT int kvq_oracle_quant_rows_fp8(const float* x, int64_t rows, int64_t D, float eps,
+                                         uint8_t* codes, float* scales) {
+  if (!x || !codes || !scales || rows < 0 || D <= 0) return -1;
+#pragma omp parallel for schedule(static)
+  for (int64_t r = 0; r < rows; ++r) {
+    const float* xr = x + r * D;
+    float amax = 0.0f;
+    for (int64_t d = 0; d < D; ++d) {
+      float a = fabsf(xr[d]);
+      if (a > amax || a != a) amax = a;
+    }
+    if (amax < eps) amax = eps;
+    volatile float scale = amax / 448.0f;
+    scales[r] = scale;
+    for (int64_t d = 0; d < D; ++d) {
+      volatile float qf = scale > 0.0f ? xr[d] / scale : 0.0f;
+      codes[r * D + d] = f32_to_e4m3fn(qf);
+    }
+  }
+  return 0;
+}
+
+static inline double code_value(uint8_t b, int code_type) {
+  return code_type == KVQ_CODE_FP8 ? (double)e4m3fn_value(b) : (double)(int8_t)b;
+}
+
+/* ---------------------------------------------------------------------------
  * Quantise-on-write into the paged cache.
  * Layout follows vllm_metax/v1/attention/backends/triton_attn.py:318-348
  * (shape), :418-479 (scale views) and :729-739 (K/V views): a (slot, head)
@@ -98,14 +161,34 @@ KVQ_EXPORT int kvq_oracle_quant_rows(const float* x, int64_t rows, int64_t D,
  * csrc/libtorch_stable/cache_kernels.cu:321-339 (slot < 0 is padding: skip)
  * and :839-849 (token count comes from slot_mapping, not from key).
  * ------------------------------------------------------------------------- */
-KVQ_EXPORT int kvq_oracle_cache_write(
+KVQ_EXPORT int kvq_oracle_cache_write_ex(
     const float* key, const float* value, /* [T, Hkv, D] fp32, contiguous */
     uint8_t* cache, int64_t k_off, int64_t v_off, int64_t ks_off, int64_t vs_off,
     int64_t stride_block, int64_t stride_slot, int64_t stride_head,
     const int64_t* slot_mapping, int64_t T, int Hkv, int D, int block_size,
-    float eps) {
+    float eps, int code_type);
+
+KVQ_EXPORT int kvq_oracle_cache_write(
+    const float* key, const float* value, uint8_t* cache, int64_t k_off, int64_t v_off, int64_t ks_off,
+    int64_t vs_off, int64_t stride_block, int64_t stride_slot, int64_t stride_head,
+    const int64_t* slot_mapping, int64_t T, int Hkv, int D, int block_size, float eps) {
+  return kvq_oracle_cache_write_ex(key, value, cache, k_off, v_off, ks_off, vs_off, stride_block, stride_slot,
+                                   stride_head, slot_mapping, T, Hkv, D, block_size, eps, KVQ_CODE_INT8);
+}
+
+static int quant_row_any(const float* x, int D, float eps, uint8_t* codes, float* s, int code_type) {
+  return code_type == KVQ_CODE_FP8 ? kvq_oracle_quant_rows_fp8(x, 1, D, eps, codes, s)
+                                   : kvq_oracle_quant_rows(x, 1, D, eps, (int8_t*)codes, s);
+}
+
+KVQ_EXPORT int kvq_oracle_cache_write_ex(
+    const float* key, const float* value, /* [T, Hkv, D] fp32, contiguous */
+    uint8_t* cache, int64_t k_off, int64_t v_off, int64_t ks_off, int64_t vs_off,
+    int64_t stride_block, int64_t stride_slot, int64_t stride_head,
+    const int64_t* slot_mapping, int64_t T, int Hkv, int D, int block_size,
+    float eps, int code_type) {
   if (!key || !value || !cache || !slot_mapping) return -1;
-  int8_t* codes = (int8_t*)malloc((size_t)D);
+  uint8_t* codes = (uint8_t*)malloc((size_t)D);
   if (!codes) return -2;
   for (int64_t t = 0; t < T; ++t) {
     int64_t slot = slot_mapping[t];
@@ -114,10 +197,10 @@ KVQ_EXPORT int kvq_oracle_cache_write(
     for (int h = 0; h < Hkv; ++h) {
       uint8_t* rec = cache + blk * stride_block + off * stride_slot + (int64_t)h * stride_head;
       float s;
-      kvq_oracle_quant_rows(key + (t * Hkv + h) * (int64_t)D, 1, D, eps, codes, &s);
+      quant_row_any(key + (t * Hkv + h) * (int64_t)D, D, eps, codes, &s, code_type);
       memcpy(rec + k_off, codes, (size_t)D);
       memcpy(rec + ks_off, &s, 4);
-      kvq_oracle_quant_rows(value + (t * Hkv + h) * (int64_t)D, 1, D, eps, codes, &s);
+      quant_row_any(value + (t * Hkv + h) * (int64_t)D, D, eps, codes, &s, code_type);
       memcpy(rec + v_off, codes, (size_t)D);
       memcpy(rec + vs_off, &s, 4);
     }
@@ -133,17 +216,17 @@ static void attend_range(const float* q, int D, const uint8_t* cache,
                          int64_t stride_block, int64_t stride_slot, int64_t stride_head,
                          const int32_t* bt_row, int block_size, int hkv,
                          int64_t k_begin, int64_t k_end, double scale, double softcap,
-                         double* acc, double* m_out, double* l_out, double* logits) {
+                         double* acc, double* m_out, double* l_out, double* logits, int code_type) {
   double m = -INFINITY;
   for (int64_t j = k_begin; j < k_end; ++j) {
     int64_t blk = bt_row[j / block_size];
     const uint8_t* rec = cache + blk * stride_block + (j % block_size) * stride_slot +
                          (int64_t)hkv * stride_head;
-    const int8_t* kc = (const int8_t*)(rec + k_off);
+    const uint8_t* kc = rec + k_off;
     float ks;
     memcpy(&ks, rec + ks_off, 4);
     double s = 0.0;
-    for (int d = 0; d < D; ++d) s += (double)q[d] * ((double)kc[d] * (double)ks);
+    for (int d = 0; d < D; ++d) s += (double)q[d] * (code_value(kc[d], code_type) * (double)ks);
     s *= scale;
     if (softcap > 0.0) s = softcap * tanh(s / softcap);
     logits[j - k_begin] = s;
@@ -155,13 +238,13 @@ static void attend_range(const float* q, int D, const uint8_t* cache,
     int64_t blk = bt_row[j / block_size];
     const uint8_t* rec = cache + blk * stride_block + (j % block_size) * stride_slot +
                          (int64_t)hkv * stride_head;
-    const int8_t* vc = (const int8_t*)(rec + v_off);
+    const uint8_t* vc = rec + v_off;
     float vs;
     memcpy(&vs, rec + vs_off, 4);
     double p = exp(logits[j - k_begin] - m);
     l += p;
     double pv = p * (double)vs;
-    for (int d = 0; d < D; ++d) acc[d] += pv * (double)vc[d];
+    for (int d = 0; d < D; ++d) acc[d] += pv * code_value(vc[d], code_type);
   }
   *m_out = m;
   *l_out = l;
@@ -186,13 +269,13 @@ static void attend_range(const float* q, int D, const uint8_t* cache,
 /* window > 0: a query at position p sees keys p - window + 1 .. p only (the
  * sliding_window mask of ref_paged_attn, :60-66).  softcap > 0: scaled logits
  * become softcap * tanh(logit / softcap) before masking (:67-68).           */
-KVQ_EXPORT int kvq_oracle_paged_attn_ex(
+KVQ_EXPORT int kvq_oracle_paged_attn_ex2(
     float* out, float* lse, const float* q, const uint8_t* cache,
     int64_t k_off, int64_t v_off, int64_t ks_off, int64_t vs_off,
     int64_t stride_block, int64_t stride_slot, int64_t stride_head,
     const int32_t* block_table, int64_t bt_stride, const int32_t* seq_lens,
     const int32_t* cu_seqlens_q, int B, int Hq, int Hkv, int D, int block_size,
-    float scale, int causal, int window, float softcap) {
+    float scale, int causal, int window, float softcap, int code_type) {
   if (!out || !q || !cache || !block_table || !seq_lens || !cu_seqlens_q) return -1;
   if (Hkv <= 0 || Hq % Hkv != 0) return -1;
   const int G = Hq / Hkv;
@@ -231,7 +314,7 @@ KVQ_EXPORT int kvq_oracle_paged_attn_ex(
             attend_range(q + ((q0 + r) * Hq + h) * (int64_t)D, D, cache, k_off, v_off,
                          ks_off, vs_off, stride_block, stride_slot, stride_head,
                          block_table + (int64_t)i * bt_stride, block_size, h / G, first, vis,
-                         (double)scale, (double)softcap, acc, &m, &l, logits);
+                         (double)scale, (double)softcap, acc, &m, &l, logits, code_type);
             for (int d = 0; d < D; ++d) o[d] = (float)(acc[d] / l);
             if (lse) lse[(q0 + r) * Hq + h] = (float)(m + log(l));
           }
@@ -242,6 +325,19 @@ KVQ_EXPORT int kvq_oracle_paged_attn_ex(
     free(logits);
   }
   return err ? -2 : 0;
+}
+
+KVQ_EXPORT int kvq_oracle_paged_attn_ex(
+    float* out, float* lse, const float* q, const uint8_t* cache,
+    int64_t k_off, int64_t v_off, int64_t ks_off, int64_t vs_off,
+    int64_t stride_block, int64_t stride_slot, int64_t stride_head,
+    const int32_t* block_table, int64_t bt_stride, const int32_t* seq_lens,
+    const int32_t* cu_seqlens_q, int B, int Hq, int Hkv, int D, int block_size,
+    float scale, int causal, int window, float softcap) {
+  return kvq_oracle_paged_attn_ex2(out, lse, q, cache, k_off, v_off, ks_off, vs_off, stride_block,
+                                   stride_slot, stride_head, block_table, bt_stride, seq_lens,
+                                   cu_seqlens_q, B, Hq, Hkv, D, block_size, scale, causal, window,
+                                   softcap, KVQ_CODE_INT8);
 }
 
 KVQ_EXPORT int kvq_oracle_paged_attn(
@@ -302,7 +398,7 @@ KVQ_EXPORT int kvq_oracle_paged_attn_partition(
             attend_range(q + ((int64_t)i * Hq + h) * D, D, cache, k_off, v_off, ks_off,
                          vs_off, stride_block, stride_slot, stride_head,
                          block_table + (int64_t)i * bt_stride, block_size, h / G, b0, b1,
-                         (double)scale, 0.0, acc, &m, &l, logits);
+                         (double)scale, 0.0, acc, &m, &l, logits, KVQ_CODE_INT8);
             int64_t idx = ((int64_t)i * Hq + h) * max_parts + j;
             for (int d = 0; d < D; ++d) tmp_out[idx * D + d] = (float)(acc[d] / l);
             max_logits[idx] = (float)m;

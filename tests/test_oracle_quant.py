@@ -210,3 +210,58 @@ def test_rope_cache_write_is_rotate_then_write_and_skips_padding():
     live = slots >= 0
     assert torch.equal(k1[live], k2[live]) and torch.equal(k1[~live], k_pe[~live]) and torch.equal(q1[~live], q_pe[~live])
     assert torch.equal(q1[live], oracle.rope_rotate(q_pe, pos, cs, True)[live])
+
+
+# ---------------------------------------------------------------------------------------------
+# fp8 (e4m3fn) per-token-head mode of the same record layout
+# ---------------------------------------------------------------------------------------------
+
+def test_e4m3fn_table_matches_torch_for_every_code():
+    tab = oracle.e4m3fn_table()
+    ref = torch.arange(256, dtype=torch.uint8).view(torch.float8_e4m3fn).to(torch.float32)
+    finite = ~torch.isnan(ref)
+    assert finite.sum() == 254 and torch.equal(tab[finite], ref[finite])
+    assert tab[0x7e] == 448 and tab[0x08] == 2.0 ** -6 and tab[0x01] == 2.0 ** -9 and tab[0x80] == 0
+
+
+def test_fp8_conversion_matches_torch_on_a_dense_sweep_and_on_ties():
+    """Every fp32 whose low 12 mantissa bits are zero between 2^-12 and 448, both signs, plus all exact
+    midpoints between neighbouring codes (ties go to the even code): the oracle's conversion equals
+    torch's float8_e4m3fn cast (an independent implementation of round-to-nearest-even)."""
+    bits = torch.arange(0x39800000, 0x43e00001, 1 << 12, dtype=torch.int64).to(torch.int32)
+    y = bits.view(torch.float32)
+    y = torch.cat([y, -y])
+    codes, scales = oracle.quant_rows_fp8(torch.cat([y, torch.tensor([448.0])]).view(1, -1))   # absmax 448 -> scale 1
+    assert scales.item() == 1.0
+    want = y.to(torch.float8_e4m3fn).view(torch.uint8)
+    assert torch.equal(codes.view(-1)[:-1], want)
+    tab = oracle.e4m3fn_table()[:0x7f]                       # positive codes in increasing order
+    mid = (tab[:-1] + tab[1:]) / 2                            # exact in fp32
+    codes, _ = oracle.quant_rows_fp8(torch.cat([mid, torch.tensor([448.0])]).view(1, -1))
+    got = codes.view(-1)[:-1].to(torch.int64)
+    lower = torch.arange(0x7e)
+    assert torch.equal(got, torch.where(lower % 2 == 0, lower, lower + 1)), "ties must go to the even code"
+    assert torch.equal(got.to(torch.uint8), mid.to(torch.float8_e4m3fn).view(torch.uint8))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+def test_fp8_quant_rows_rule_and_closed_forms(dtype):
+    g = torch.Generator().manual_seed(11)
+    x = (torch.randn((300, 128), generator=g) * 3).to(dtype)
+    x[7] = 0                                                   # a zero row
+    codes, scales = oracle.quant_rows_fp8(x)
+    xf = x.to(torch.float32)
+    amax = xf.abs().amax(dim=-1).clamp(min=oracle.eps_for(dtype))
+    assert torch.equal(scales, amax / 448.0)                   # fp32 true division
+    safe = torch.where(scales > 0, scales, torch.ones_like(scales))
+    want = (xf / safe[:, None]).to(torch.float8_e4m3fn).view(torch.uint8)
+    assert torch.equal(codes, want)
+    assert bool((codes[7] == 0).all())
+    deq = oracle.e4m3fn_table()[codes.to(torch.int64)] * scales[:, None]
+    # the absmax element maps to +-448 exactly, and every element is within half a code step
+    idx = xf.abs().argmax(dim=-1)
+    rows = torch.arange(300)
+    live = amax > 1e-9
+    assert torch.equal(deq[rows, idx][live].abs(), (scales * 448.0)[live])
+    step = torch.maximum(deq.abs() / 16.0, scales[:, None] * 2.0 ** -10)   # half of 2^-3 relative / half the subnormal step
+    assert bool(((deq - xf).abs() <= step * 1.0001 + 1e-30).all())

@@ -47,15 +47,39 @@ __device__ __forceinline__ uint32_t bytes_to_half2(uint32_t x, bool upper) {
   return perm(0x64646464u, x, upper ? 0x04030402u : 0x04010400u);
 }
 
-// 8 consecutive code bytes (two dwords) -> 8 fp16 (code + 1152), one MFMA k-step operand.
+// Two e4m3fn code bytes of x -> two fp16 values code / 2^8: the byte's 7 magnitude bits sit in an fp16
+// pattern at bits 7 .. 13 and the sign at bit 15; as an fp16 number that pattern is the code's value
+// times 2^-8 (the exponent biases differ by 15 - 7), exactly, subnormal codes included.  The 2^8 is put
+// back with the scales.
+__device__ __forceinline__ uint32_t fp8_bytes_to_half2(uint32_t x, bool upper) {
+  const uint32_t y = perm(0u, x, upper ? 0x030c020cu : 0x010c000cu);   // the two bytes in the high byte of each half
+  return (y & 0x80008000u) | ((y >> 1) & 0x3f803f80u);
+}
+
+// Two code bytes -> the two fp16 numbers the MFMA sees, for either kind of code (int8 bytes are
+// expected already ^ 0x80, see prep_codes).
+template <bool FP8>
+__device__ __forceinline__ uint32_t codes_to_half2(uint32_t x, bool upper) {
+  if constexpr (FP8) return fp8_bytes_to_half2(x, upper);
+  else return bytes_to_half2(x, upper);
+}
+template <bool FP8>
+__device__ __forceinline__ uint32_t prep_codes(uint32_t x) {
+  if constexpr (FP8) return x;
+  else return x ^ 0x80808080u;
+}
+
+// 8 consecutive code bytes (two dwords) -> 8 fp16 (code + 1152, or code / 2^8 for fp8 codes), one MFMA
+// k-step operand.
+template <bool FP8 = false>
 __device__ __forceinline__ half8_t dequant8(uint32_t lo, uint32_t hi) {
-  lo ^= 0x80808080u;
-  hi ^= 0x80808080u;
+  lo = prep_codes<FP8>(lo);
+  hi = prep_codes<FP8>(hi);
   u32x4 r;
-  r.x = bytes_to_half2(lo, false);
-  r.y = bytes_to_half2(lo, true);
-  r.z = bytes_to_half2(hi, false);
-  r.w = bytes_to_half2(hi, true);
+  r.x = codes_to_half2<FP8>(lo, false);
+  r.y = codes_to_half2<FP8>(lo, true);
+  r.z = codes_to_half2<FP8>(hi, false);
+  r.w = codes_to_half2<FP8>(hi, true);
   return __builtin_bit_cast(half8_t, r);
 }
 
@@ -154,8 +178,14 @@ struct LaneOffsets {
   uint32_t l_sc;      // LDS: (lane & 31)*PITCH + (lane < 32 ? D : 2*D+4), the lane's scale
 };
 
-template <int D, int QDT, int ODT>
+// CODE: what a code byte is (KVQ_CODE_INT8 or KVQ_CODE_FP8_E4M3).  An int8 code enters the MFMA as
+// code + 1152 and the constant is taken out afterwards; an fp8 code enters as its value / 2^8 (exact in
+// fp16) and the 2^8 is put back with the K scale, while on the V side it cancels the 2^8 that P~ carries.
+template <int D, int QDT, int ODT, int CODE = KVQ_CODE_INT8>
 struct DecodeTile {
+  static constexpr bool FP8 = CODE == KVQ_CODE_FP8_E4M3;
+  static constexpr float kKScaleMul = FP8 ? 256.0f : 1.0f;   // on top of scale * log2(e)
+  static constexpr float kOutDiv = FP8 ? 1.0f : kPScale;      // what the accumulated output still carries
   static constexpr int KSTEPS = D / 32;
   static constexpr int DT = D / 16;
   static constexpr int VB = D / 16;  // V bytes per token per lane
@@ -247,7 +277,7 @@ struct DecodeTile {
     }
     qsum += __shfl_xor(qsum, 16, kWave);
     qsum += __shfl_xor(qsum, 32, kWave);
-    return -kCodeBias * qsum;
+    return FP8 ? 0.f : -kCodeBias * qsum;
   }
 
   // Token index -> block-table entry / slot, by multiplication (scalar ALU, no divide).
@@ -348,8 +378,8 @@ struct DecodeTile {
 #pragma unroll
       for (int i = 0; i < KSTEPS / 2; ++i) {
         const u32x4 w = *reinterpret_cast<const u32x4*>(lds + lo.l_k + mt * 16 * PITCH + i * 64);
-        s[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(dequant8(w.x, w.y), qb[2 * i], s[mt], 0, 0, 0);
-        s[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(dequant8(w.z, w.w), qb[2 * i + 1], s[mt], 0, 0, 0);
+        s[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(dequant8<FP8>(w.x, w.y), qb[2 * i], s[mt], 0, 0, 0);
+        s[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(dequant8<FP8>(w.z, w.w), qb[2 * i + 1], s[mt], 0, 0, 0);
       }
     }
 
@@ -406,7 +436,7 @@ struct DecodeTile {
   // tokens 4g+j (j<4) and 16+4g+(j-4) from the LDS window, transposes the 8 x VB byte block in
   // registers (byte permutes), one MFMA per 16-dim tile; sum(P~) comes from a row of ones.
   __device__ static void pv(const LaneOffsets& lo, half8_t p_op, const uint8_t* lds, State& st) {
-    {
+    if constexpr (!FP8) {  // fp8 codes carry no bias to take out again
       const half_t one = (half_t)1.0f;
       const half8_t ones = {one, one, one, one, one, one, one, one};
       st.psum = __builtin_amdgcn_mfma_f32_16x16x32_f16(ones, p_op, st.psum, 0, 0, 0);
@@ -418,8 +448,8 @@ struct DecodeTile {
 #pragma unroll
       for (int a = 0; a < 4; ++a) {
         const int ja = 2 * a, jb = 2 * a + 1;
-        const uint32_t ta = *reinterpret_cast<const uint32_t*>(lds + lo.l_v + ((ja & 3) + (ja >> 2) * 16) * PITCH + 4 * w) ^ 0x80808080u;
-        const uint32_t tb = *reinterpret_cast<const uint32_t*>(lds + lo.l_v + ((jb & 3) + (jb >> 2) * 16) * PITCH + 4 * w) ^ 0x80808080u;
+        const uint32_t ta = prep_codes<FP8>(*reinterpret_cast<const uint32_t*>(lds + lo.l_v + ((ja & 3) + (ja >> 2) * 16) * PITCH + 4 * w));
+        const uint32_t tb = prep_codes<FP8>(*reinterpret_cast<const uint32_t*>(lds + lo.l_v + ((jb & 3) + (jb >> 2) * 16) * PITCH + 4 * w));
         x0[a] = perm(tb, ta, 0x05010400u);
         x1[a] = perm(tb, ta, 0x07030602u);
       }
@@ -427,10 +457,10 @@ struct DecodeTile {
       for (int b = 0; b < 4; ++b) {
         u32x4 av;
         const uint32_t* x = (b < 2) ? x0 : x1;
-        av.x = bytes_to_half2(x[0], b & 1);
-        av.y = bytes_to_half2(x[1], b & 1);
-        av.z = bytes_to_half2(x[2], b & 1);
-        av.w = bytes_to_half2(x[3], b & 1);
+        av.x = codes_to_half2<FP8>(x[0], b & 1);
+        av.y = codes_to_half2<FP8>(x[1], b & 1);
+        av.z = codes_to_half2<FP8>(x[2], b & 1);
+        av.w = codes_to_half2<FP8>(x[3], b & 1);
         const int dt = 4 * w + b;
         st.o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, av), p_op, st.o[dt], 0, 0, 0);
       }
@@ -491,7 +521,7 @@ struct DecodeTile {
       nb = fetch_blocks(io, bt_row, len, t + nsub);  // block ids run one tile ahead of the loads
       half8_t qb[KSTEPS];
       const float s_init = load_q(io, row, hkv, lane, qb);
-      const float sc_mul = lane < 32 ? io.scale_log2 : kPScale;
+      const float sc_mul = lane < 32 ? io.scale_log2 * kKScaleMul : kPScale;
       int r = 0;  // rounds this wave has finished
       // a first tile that straddles the window's lower edge is masked; it is peeled off so that the
       // steady loop below keeps a single, unmasked body
@@ -574,7 +604,7 @@ struct DecodeTile {
   // Lane (c, g) holds O[head c][dim (4g+i)*VB + dt], i = 0..3, dt = 0..DT-1: D/4 contiguous
   // dims starting at g*D/4.  Gather them in order, code bias removed, scaled by `mul`.
   __device__ static void gather_row(const State& st, float mul, float (&v)[D / 4]) {
-    const float corr = kCodeBias * st.psum[0];
+    const float corr = FP8 ? 0.f : kCodeBias * st.psum[0];
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
@@ -598,7 +628,7 @@ struct DecodeTile {
     if (c >= io.group) return;
     const int head = hkv * io.group + c;
     float v[D / 4];
-    gather_row(st, 1.0f / (l * kPScale), v);
+    gather_row(st, 1.0f / (l * kOutDiv), v);
     const int64_t base = row * io.out_stride_t + (int64_t)head * io.out_stride_h + g * (D / 4);
     if constexpr (OT == KVQ_F32) {
       float* o = reinterpret_cast<float*>(io.out) + base;
@@ -634,7 +664,7 @@ struct DecodeTile {
     if (c >= io.group) return;
     const int head = hkv * io.group + c;
     float v[D / 4];
-    gather_row(st, 1.0f / kPScale, v);
+    gather_row(st, 1.0f / kOutDiv, v);
     float* o = part_o + (slot * io.num_q_heads + head) * (int64_t)D + g * (D / 4);
 #pragma unroll
     for (int i = 0; i < D / 4; i += 4) *reinterpret_cast<floatx4*>(o + i) = (floatx4){v[i], v[i + 1], v[i + 2], v[i + 3]};
@@ -652,7 +682,7 @@ struct DecodeTile {
     if (c >= io.group) return;
     const int head = hkv * io.group + c;
     float v[D / 4];
-    gather_row(st, 1.0f / (l * kPScale), v);
+    gather_row(st, 1.0f / (l * kOutDiv), v);
     const int64_t idx = (seq * io.num_q_heads + head) * (int64_t)max_parts + part;
     float* o = tmp_out + idx * D + g * (D / 4);
 #pragma unroll

@@ -66,6 +66,24 @@ __device__ __forceinline__ void store_act(void* p, int64_t i, float v) {
   else reinterpret_cast<half_t*>(p)[i] = (half_t)v;
 }
 
+// fp32 -> OCP e4m3fn bit pattern (1 sign, 4 exponent bits with bias 7, 3 mantissa bits; largest finite
+// value 448, no infinities), round to nearest even, saturating: in integer arithmetic, so that the codes
+// are the same bits on every path that produces them.
+__device__ __forceinline__ uint32_t f32_to_e4m3fn_bits(float y) {
+  uint32_t u = __builtin_bit_cast(uint32_t, y);
+  const uint32_t sign = (u >> 24) & 0x80u;
+  u &= 0x7fffffffu;
+  uint32_t code;
+  if (u < 0x3c800000u) {                       // below 2^-6: multiples of 2^-9 (8 = the smallest normal)
+    code = (uint32_t)__builtin_rintf(__builtin_bit_cast(float, u) * 512.0f);
+  } else {
+    const uint32_t r = u + 0x7ffffu + ((u >> 20) & 1u);   // nearest even at mantissa bit 20
+    code = (r >> 20) - ((127u - 7u) << 3);
+    code = code > 0x7eu ? 0x7eu : code;        // past 448 (also inf / nan): the largest finite code
+  }
+  return sign | code;
+}
+
 // Output dtype known only at run time (one uniform branch per store).
 constexpr int kRuntimeDtype = -1;
 __device__ __forceinline__ void store_act_rt(int dtype, void* p, int64_t i, float v) {

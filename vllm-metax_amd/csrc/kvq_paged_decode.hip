@@ -95,6 +95,8 @@ int validate_common(const char* op, const void* q, const void* cache, const kvq_
                   g.vs_off - g.k_off == 2 * g.head_size + 4,
               "%s: a cache record must be [K codes | K scale | V codes | V scale]", op);
   KVQ_REQUIRE(g.stride_slot > 0 && g.stride_slot <= 0x7fffffff / 64, "%s: stride_slot out of range", op);
+  KVQ_REQUIRE(g.code_type == KVQ_CODE_INT8 || g.code_type == KVQ_CODE_FP8_E4M3, "%s: unknown code_type %d", op,
+              g.code_type);
   return KVQ_OK;
 }
 
@@ -150,6 +152,7 @@ int kvq_paged_attn_v2_int8(void* out, int out_dtype, float* exp_sums, float* max
   int rc = validate_common("paged_attn_v2_int8", q, cache, geom, block_table, seq_lens, num_seqs, num_q_heads);
   if (rc) return rc;
   KVQ_REQUIRE(out && exp_sums && max_logits && tmp_out, "paged_attn_v2_int8: NULL output pointer");
+  KVQ_REQUIRE(geom->code_type == KVQ_CODE_INT8, "paged_attn_v2_int8: int8 codes only");
   KVQ_REQUIRE(partition_size > 0 && partition_size % kTile == 0,
               "paged_attn_v2_int8: partition_size %d must be a positive multiple of %d", partition_size, kTile);
   KVQ_REQUIRE(max_num_partitions > 0 && max_num_partitions <= 65535,

@@ -141,9 +141,9 @@ __device__ __forceinline__ int active_workgroups(int64_t total, int num_wg) {
 // eight kv heads the 8 / HPW waves of a head take the tiles of a run in turn and their states are
 // folded together in LDS when the run ends, so a compute unit keeps eight tile streams in flight
 // whatever the head count and a sequence is cut into no more partial states than with eight heads.
-template <int D, int QDT, int HPW, bool CAP>
+template <int D, int QDT, int HPW, bool CAP, int CODE>
 __global__ __launch_bounds__(512) void paged_decode_streamk_kernel(StreamKArgs a) {
-  using DTile = DecodeTile<D, QDT, kRuntimeDtype>;
+  using DTile = DecodeTile<D, QDT, kRuntimeDtype, CODE>;
   constexpr int NSUB = 8 / HPW;
   __shared__ __align__(16) uint8_t lds[8][DTile::LDS_WAVE];
   const int lane = threadIdx.x & 63;
@@ -392,7 +392,13 @@ static int launch_streamk(const StreamKArgs& a, hipStream_t s) {
   const int hkv = a.io.g.num_kv_heads;
   const int hpw = heads_per_wg(hkv);
   dim3 grid(a.num_wg, (hkv + hpw - 1) / hpw);
-#define KVQ_SK(H, C) hipLaunchKernelGGL((paged_decode_streamk_kernel<D, QDT, H, C>), grid, dim3(512), 0, s, a)
+#define KVQ_SK(H, C)                                                                                              \
+  do {                                                                                                            \
+    if (a.io.g.code_type == KVQ_CODE_FP8_E4M3)                                                                    \
+      hipLaunchKernelGGL((paged_decode_streamk_kernel<D, QDT, H, C, KVQ_CODE_FP8_E4M3>), grid, dim3(512), 0, s, a); \
+    else                                                                                                          \
+      hipLaunchKernelGGL((paged_decode_streamk_kernel<D, QDT, H, C, KVQ_CODE_INT8>), grid, dim3(512), 0, s, a);     \
+  } while (0)
   if (a.io.cap_c != 0.f) {
     switch (hpw) {
       case 8: KVQ_SK(8, true); break;

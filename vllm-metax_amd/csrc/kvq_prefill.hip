@@ -23,9 +23,10 @@ struct PrefillArgs {
   int q_tokens;  // query tokens per block: (16 * NT) / group
 };
 
-template <int D, int QDT, int ODT, int NT>
+template <int D, int QDT, int ODT, int NT, int CODE = KVQ_CODE_INT8>
 struct PrefillTile {
-  using DTile = DecodeTile<D, QDT, ODT>;
+  using DTile = DecodeTile<D, QDT, ODT, CODE>;
+  static constexpr bool FP8 = DTile::FP8;
   static constexpr int KSTEPS = DTile::KSTEPS;
   static constexpr int DT = DTile::DT;
   static constexpr int VB = DTile::VB;
@@ -57,7 +58,7 @@ struct PrefillTile {
 #pragma unroll
       for (int i = 0; i < KSTEPS / 2; ++i) {
         const u32x4 w = *reinterpret_cast<const u32x4*>(lds + lo.l_k + mt * 16 * PITCH + i * 64);
-        const half8_t a0 = dequant8(w.x, w.y), a1 = dequant8(w.z, w.w);
+        const half8_t a0 = dequant8<FP8>(w.x, w.y), a1 = dequant8<FP8>(w.z, w.w);
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) {
           s[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a0, qb[nt][2 * i], s[nt][mt], 0, 0, 0);
@@ -131,7 +132,7 @@ struct PrefillTile {
 
   // O^T += (V + 1152)^T . P~^T: every converted V operand feeds the NT column tiles.
   __device__ static void pv(const LaneOffsets& lo, const half8_t (&p_op)[NT], const uint8_t* lds, State& st) {
-    {
+    if constexpr (!FP8) {
       const half_t one = (half_t)1.0f;
       const half8_t ones = {one, one, one, one, one, one, one, one};
 #pragma unroll
@@ -144,8 +145,8 @@ struct PrefillTile {
 #pragma unroll
       for (int a = 0; a < 4; ++a) {
         const int ja = 2 * a, jb = 2 * a + 1;
-        const uint32_t ta = *reinterpret_cast<const uint32_t*>(lds + lo.l_v + ((ja & 3) + (ja >> 2) * 16) * PITCH + 4 * w) ^ 0x80808080u;
-        const uint32_t tb = *reinterpret_cast<const uint32_t*>(lds + lo.l_v + ((jb & 3) + (jb >> 2) * 16) * PITCH + 4 * w) ^ 0x80808080u;
+        const uint32_t ta = prep_codes<FP8>(*reinterpret_cast<const uint32_t*>(lds + lo.l_v + ((ja & 3) + (ja >> 2) * 16) * PITCH + 4 * w));
+        const uint32_t tb = prep_codes<FP8>(*reinterpret_cast<const uint32_t*>(lds + lo.l_v + ((jb & 3) + (jb >> 2) * 16) * PITCH + 4 * w));
         x0[a] = perm(tb, ta, 0x05010400u);
         x1[a] = perm(tb, ta, 0x07030602u);
       }
@@ -153,10 +154,10 @@ struct PrefillTile {
       for (int b = 0; b < 4; ++b) {
         u32x4 av;
         const uint32_t* x = (b < 2) ? x0 : x1;
-        av.x = bytes_to_half2(x[0], b & 1);
-        av.y = bytes_to_half2(x[1], b & 1);
-        av.z = bytes_to_half2(x[2], b & 1);
-        av.w = bytes_to_half2(x[3], b & 1);
+        av.x = codes_to_half2<FP8>(x[0], b & 1);
+        av.y = codes_to_half2<FP8>(x[1], b & 1);
+        av.z = codes_to_half2<FP8>(x[2], b & 1);
+        av.w = codes_to_half2<FP8>(x[3], b & 1);
         const half8_t a_op = __builtin_bit_cast(half8_t, av);
         const int dt = 4 * w + b;
 #pragma unroll
@@ -173,8 +174,8 @@ struct PrefillTile {
     l += __shfl_xor(l, 32, kWave);
     if (!valid) return;
     const int g = lane >> 4;
-    const float mul = l > 0.f ? 1.0f / (l * kPScale) : 0.f;   // no visible key: zeros
-    const float corr = kCodeBias * st.psum[nt][0];
+    const float mul = l > 0.f ? 1.0f / (l * DTile::kOutDiv) : 0.f;   // no visible key: zeros
+    const float corr = FP8 ? 0.f : kCodeBias * st.psum[nt][0];
     float v[D / 4];
 #pragma unroll
     for (int i = 0; i < 4; ++i)
@@ -210,9 +211,9 @@ struct PrefillTile {
 
 // grid (query blocks of the longest run, sequences, ceil(Hkv / WPW)); wave w of a workgroup owns
 // kv head blockIdx.z * WPW + w.  Sequences with a one-token run belong to the decode kernel.
-template <int D, int QDT, int ODT, int NT, int WPW>
+template <int D, int QDT, int ODT, int NT, int WPW, int CODE = KVQ_CODE_INT8>
 __global__ __launch_bounds__(WPW * 64) void paged_prefill_kernel(PrefillArgs a) {
-  using PT = PrefillTile<D, QDT, ODT, NT>;
+  using PT = PrefillTile<D, QDT, ODT, NT, CODE>;
   using DTile = typename PT::DTile;
   __shared__ __align__(16) uint8_t lds_all[WPW][DTile::LDS_WAVE];
   const int lane = threadIdx.x & 63;
@@ -288,7 +289,7 @@ __global__ __launch_bounds__(WPW * 64) void paged_prefill_kernel(PrefillArgs a) 
   for (int nt = 0; nt < NT; ++nt)
     s_init[nt] = DTile::load_q_row(io, row[nt] * io.q_stride_t + (int64_t)(valid[nt] ? head[nt] : hkv * io.group) * io.q_stride_h,
                                    valid[nt], lane, qb[nt]);
-  const float sc_mul = lane < 32 ? io.scale_log2 : kPScale;
+  const float sc_mul = lane < 32 ? io.scale_log2 * DTile::kKScaleMul : kPScale;
   typename PT::State st;
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt) {
@@ -755,18 +756,22 @@ static int launch_prefill_flash32(PrefillArgs& a, int max_query_len, hipStream_t
   return check_hip(hipGetLastError(), "paged_prefill_flash32 launch");
 }
 
-template <int D, int QDT, int ODT, int NT, int WPW>
+template <int D, int QDT, int ODT, int NT, int WPW, int CODE = KVQ_CODE_INT8>
 static int launch_prefill_cfg(const PrefillArgs& a, int max_query_len, hipStream_t s) {
   const int blocks = (max_query_len + a.q_tokens - 1) / a.q_tokens;
   if (blocks > 0x7fffffff / 2 || a.num_seqs > 65535) return fail(KVQ_EINVAL, "paged_attn_int8: prefill grid out of range");
   dim3 grid(blocks, a.num_seqs, (a.io.g.num_kv_heads + WPW - 1) / WPW);
-  hipLaunchKernelGGL((paged_prefill_kernel<D, QDT, ODT, NT, WPW>), grid, dim3(WPW * 64), 0, s, a);
+  hipLaunchKernelGGL((paged_prefill_kernel<D, QDT, ODT, NT, WPW, CODE>), grid, dim3(WPW * 64), 0, s, a);
   return check_hip(hipGetLastError(), "paged_prefill launch");
 }
 
 template <int D, int QDT, int ODT>
 static int launch_prefill_nt(PrefillArgs& a, int max_query_len, hipStream_t s) {
   constexpr int WPW = 4;
+  if (a.io.g.code_type == KVQ_CODE_FP8_E4M3) {  // fp8 codes: the per-wave tile, one column tile per wave
+    a.q_tokens = 16 / a.io.group;
+    return launch_prefill_cfg<D, QDT, ODT, 1, WPW, KVQ_CODE_FP8_E4M3>(a, max_query_len, s);
+  }
   // long runs: the workgroup-shared fp16 tile (compute-bound shape)
   if constexpr (D <= 128) {
     if (max_query_len * a.io.group >= 64) {

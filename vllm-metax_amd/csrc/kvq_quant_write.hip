@@ -4,7 +4,8 @@
 // coalesced loads, the absmax is reduced across the 64 lanes, and codes plus the
 // fp32 scale go straight into the (block, slot, head) record.  The arithmetic is
 // the bit-exact contract: scale = max(absmax, eps) / 127 (IEEE fp32 division),
-// code = clamp(rint(x / scale), -128, 127) with round-half-to-even.
+// code = clamp(rint(x / scale), -128, 127) with round-half-to-even.  A cache whose geometry says
+// KVQ_CODE_FP8_E4M3 gets scale = max(absmax, eps) / 448 and the nearest e4m3fn code instead.
 #include "kvq_internal.h"
 
 namespace kvq {
@@ -62,13 +63,18 @@ __global__ __launch_bounds__(256) void quant_write_kernel(
 #pragma unroll
     for (int i = 0; i < VEC; ++i) amax = fmaxf(amax, fabsf(x[i]));
     amax = fmaxf(wave_max(amax), eps);  // eps may be 0 for fp16 sources (1e-10 underflows)
-    const float scale = amax / 127.0f;
+    const bool fp8 = g.code_type == KVQ_CODE_FP8_E4M3;
+    const float scale = fp8 ? amax / 448.0f : amax / 127.0f;
     int8_t c[VEC];
 #pragma unroll
     for (int i = 0; i < VEC; ++i) {
-      float r = scale > 0.f ? rintf(x[i] / scale) : 0.f;  // scale == 0: all-zero fp16 row
-      r = fminf(fmaxf(r, -128.f), 127.f);
-      c[i] = (int8_t)(int)r;
+      const float y = scale > 0.f ? x[i] / scale : 0.f;  // scale == 0: all-zero fp16 row
+      if (fp8) {
+        c[i] = (int8_t)f32_to_e4m3fn_bits(y);
+      } else {
+        const float r = fminf(fmaxf(rintf(y), -128.f), 127.f);
+        c[i] = (int8_t)(int)r;
+      }
     }
     if constexpr (VEC == 1) {
       codes[lane] = c[0];
@@ -85,11 +91,16 @@ __global__ __launch_bounds__(256) void quant_write_kernel(
     float amax = 0.f;
     for (int d = lane; d < D; d += kWave) amax = fmaxf(amax, fabsf(load_act<DT>(src, src_base + d)));
     amax = fmaxf(wave_max(amax), eps);  // eps may be 0 for fp16 sources (1e-10 underflows)
-    const float scale = amax / 127.0f;
+    const bool fp8 = g.code_type == KVQ_CODE_FP8_E4M3;
+    const float scale = fp8 ? amax / 448.0f : amax / 127.0f;
     for (int d = lane; d < D; d += kWave) {
-      float r = scale > 0.f ? rintf(load_act<DT>(src, src_base + d) / scale) : 0.f;
-      r = fminf(fmaxf(r, -128.f), 127.f);
-      codes[d] = (int8_t)(int)r;
+      const float y = scale > 0.f ? load_act<DT>(src, src_base + d) / scale : 0.f;
+      if (fp8) {
+        codes[d] = (int8_t)f32_to_e4m3fn_bits(y);
+      } else {
+        const float r = fminf(fmaxf(rintf(y), -128.f), 127.f);
+        codes[d] = (int8_t)(int)r;
+      }
     }
     if (lane == 0) *scale_ptr = scale;
   }
@@ -153,13 +164,20 @@ __global__ __launch_bounds__(256) void quant_write_rows_kernel(
 #pragma unroll
   for (int o = LPR / 2; o >= 1; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o, kWave));
   amax = fmaxf(amax, eps);  // eps may be 0 for fp16 sources (1e-10 underflows)
-  const float scale = amax / 127.0f;
+  const bool fp8 = g.code_type == KVQ_CODE_FP8_E4M3;
+  const float scale = fp8 ? amax / 448.0f : amax / 127.0f;
   uint32_t pk[2] = {0u, 0u};
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
-    float r = scale > 0.f ? rintf(x[i] / scale) : 0.f;  // scale == 0: all-zero fp16 row
-    r = fminf(fmaxf(r, -128.f), 127.f);
-    pk[i >> 2] |= ((uint32_t)(int)r & 0xffu) << (8 * (i & 3));
+    const float y = scale > 0.f ? x[i] / scale : 0.f;  // scale == 0: all-zero fp16 row
+    uint32_t code;
+    if (fp8) {
+      code = f32_to_e4m3fn_bits(y);
+    } else {
+      const float r = fminf(fmaxf(rintf(y), -128.f), 127.f);
+      code = (uint32_t)(int)r & 0xffu;
+    }
+    pk[i >> 2] |= code << (8 * (i & 3));
   }
   if (!live || slot < 0) return;  // padding token (after the shuffles: every lane took part)
   int64_t blk, off;
@@ -241,6 +259,8 @@ extern "C" int kvq_reshape_and_cache_int8(const void* key, const void* value, in
                g.stride_head) % 4 == 0 && ((uintptr_t)cache % 4) == 0,
               "reshape_and_cache_int8: cache offsets/strides must be 4-byte aligned");
   KVQ_REQUIRE(eps >= 0.f, "reshape_and_cache_int8: eps must not be negative");
+  KVQ_REQUIRE(g.code_type == KVQ_CODE_INT8 || g.code_type == KVQ_CODE_FP8_E4M3,
+              "reshape_and_cache_int8: unknown code_type %d", g.code_type);
   hipStream_t s = as_stream(stream);
   uint8_t* c = static_cast<uint8_t*>(cache);
   switch (src_dtype) {

@@ -13,7 +13,8 @@ _LIB_DIR = os.path.join(os.path.dirname(os.path.abspath(__file__)), "_lib")
 LIB_PATH = os.path.join(_LIB_DIR, "libkvq_hip.so")
 
 KVQ_F32, KVQ_BF16, KVQ_F16 = 0, 1, 2
-ABI_VERSION = 8
+KVQ_CODE_INT8, KVQ_CODE_FP8_E4M3 = 0, 1
+ABI_VERSION = 9
 
 
 class CacheGeom(ctypes.Structure):
@@ -25,7 +26,7 @@ class CacheGeom(ctypes.Structure):
         ("stride_block", ctypes.c_int64), ("stride_slot", ctypes.c_int64),
         ("stride_head", ctypes.c_int64),
         ("num_kv_heads", ctypes.c_int32), ("head_size", ctypes.c_int32),
-        ("block_size", ctypes.c_int32), ("reserved", ctypes.c_int32),
+        ("block_size", ctypes.c_int32), ("code_type", ctypes.c_int32),
     ]
 
 

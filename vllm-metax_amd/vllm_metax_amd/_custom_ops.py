@@ -15,7 +15,7 @@ import torch
 
 from . import _C
 from .kv_cache_interface import KVQuantMode
-from .layout import QUANT_EPS, CacheGeometry, MlaGeometry, geometry_from_views, mla_geometry
+from .layout import QUANT_EPS, CacheGeometry, MlaGeometry, code_type_of, geometry_from_views, mla_geometry
 
 _DTYPE_CODE = {torch.float32: _C.KVQ_F32, torch.bfloat16: _C.KVQ_BF16, torch.float16: _C.KVQ_F16}
 
@@ -107,11 +107,12 @@ def reshape_and_cache_flash_per_token_head_quant(
     key/value ``[>= T, Hkv, D]``; key_cache/value_cache ``(nb, bs, Hkv, D+4)`` int8 views and
     k/v_scale_cache ``(nb, bs, Hkv)`` fp32 views of one cache; slot_mapping ``[T]`` int64
     (negative = padding, skipped).  ``geometry`` may carry the precomputed byte geometry of
-    the four views so the per-step call does no view arithmetic."""
-    if kv_quant_mode != KVQuantMode.INT8_PER_TOKEN_HEAD:
-        raise NotImplementedError(f"kv_quant_mode {kv_quant_mode!r}: only INT8_PER_TOKEN_HEAD is built")
+    the four views so the per-step call does no view arithmetic.  ``kv_quant_mode``
+    INT8_PER_TOKEN_HEAD (scale = absmax / 127, codes rint(x / scale)) or FP8_PER_TOKEN_HEAD
+    (scale = absmax / 448, e4m3fn codes) -- the two one-byte modes of this record layout."""
+    code_type = code_type_of(kv_quant_mode)   # int8, or the fp8 mode of the same record layout
     dev = _require_cuda(key, value, key_cache, value_cache, k_scale_cache, v_scale_cache, slot_mapping)
-    geom = geometry or geometry_from_views(key_cache, value_cache, k_scale_cache, v_scale_cache)
+    geom = (geometry or geometry_from_views(key_cache, value_cache, k_scale_cache, v_scale_cache)).with_code_type(code_type)
     if key.dim() != 3 or value.shape != key.shape or key.dtype != value.dtype:
         raise RuntimeError("key/value must be [num_tokens, num_kv_heads, head_size] of one dtype")
     if key.shape[1] != geom.num_kv_heads or key.shape[2] != geom.head_size:
@@ -228,8 +229,7 @@ def unified_attention(
     query to its last W keys; ``softcap > 0`` maps logits through ``softcap * tanh(x / softcap)``.
     ``static_scratch=True`` keeps the split-K states in the library's own fixed array instead of a
     workspace tensor (nothing is allocated; calls on one GPU must then not overlap in time)."""
-    if kv_quant_mode != KVQuantMode.INT8_PER_TOKEN_HEAD:
-        raise NotImplementedError(f"kv_quant_mode {kv_quant_mode!r}: only INT8_PER_TOKEN_HEAD is built")
+    code_type = code_type_of(kv_quant_mode)
     if alibi_slopes is not None or sinks is not None or output_scale is not None or mm_prefix_range is not None:
         raise NotImplementedError("alibi, sinks, fused output quantisation and mm-prefix ranges are not built")
     softcap = float(softcap or 0.0)
@@ -253,7 +253,7 @@ def unified_attention(
     if block_table is None or k_scale_cache is None or v_scale_cache is None:
         raise RuntimeError("block_table, k_scale_cache and v_scale_cache are required")
     dev = _require_cuda(q, k, v, out, cu_seqlens_q, seqused_k, block_table, k_scale_cache, v_scale_cache, workspace, lse)
-    geom = geometry or geometry_from_views(k, v, k_scale_cache, v_scale_cache)
+    geom = (geometry or geometry_from_views(k, v, k_scale_cache, v_scale_cache)).with_code_type(code_type)
     if q.dim() != 3 or out.shape != q.shape or q.shape[2] != geom.head_size:
         raise RuntimeError("q/out must be [num_tokens, num_q_heads, head_size] matching the cache head size")
     if q.stride(2) != 1 or out.stride(2) != 1:

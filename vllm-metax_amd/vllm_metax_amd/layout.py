@@ -24,7 +24,13 @@ from dataclasses import dataclass
 import torch
 
 from . import _C
-from .kv_cache_interface import INT8_PER_TOKEN, INT8_PER_TOKEN_HEAD, kv_cache_uses_per_token_head_scales
+from .kv_cache_interface import (
+    FP8_PER_TOKEN_HEAD,
+    INT8_PER_TOKEN,
+    INT8_PER_TOKEN_HEAD,
+    KVQuantMode,
+    kv_cache_uses_per_token_head_scales,
+)
 
 SCALE_BYTES = 4  # one fp32 scale
 # absmax floor of the quantiser (tests/kernels/quant_utils.py:194: eps=1e-10)
@@ -54,9 +60,10 @@ def kv_cache_shape(num_blocks: int, block_size: int, num_kv_heads: int, head_siz
     if block_size % 16 != 0:
         raise ValueError("Block size must be a multiple of 16.")
     if kv_cache_uses_per_token_head_scales(cache_dtype_str):
-        if cache_dtype_str != INT8_PER_TOKEN_HEAD:
-            raise NotImplementedError(f"kv cache dtype {cache_dtype_str!r}: only {INT8_PER_TOKEN_HEAD!r} is built")
-        scale_pad = SCALE_BYTES // torch.int8.itemsize
+        if cache_dtype_str not in (INT8_PER_TOKEN_HEAD, FP8_PER_TOKEN_HEAD):
+            raise NotImplementedError(f"kv cache dtype {cache_dtype_str!r}: only {INT8_PER_TOKEN_HEAD!r} and "
+                                      f"{FP8_PER_TOKEN_HEAD!r} are built (one-byte elements)")
+        scale_pad = SCALE_BYTES // torch.int8.itemsize   # fp8 elements are one byte as well
         return (num_blocks, num_kv_heads, block_size, 2 * (head_size + scale_pad))
     return (num_blocks, num_kv_heads, block_size, 2 * head_size)
 
@@ -140,6 +147,19 @@ class CacheGeometry:
     block_size: int
     num_blocks: int
     base_ptr: int
+    code_type: int = _C.KVQ_CODE_INT8   # what a code byte is: int8, or an e4m3fn bit pattern
+
+    def with_code_type(self, code_type: int) -> "CacheGeometry":
+        """The same bytes read as another kind of code (the geometry of a cache does not depend on it)."""
+        if code_type == self.code_type:
+            return self
+        got = self.__dict__.get("_other")
+        if got is None:
+            d = {k: v for k, v in self.__dict__.items() if not k.startswith("_")}
+            d["code_type"] = code_type
+            got = CacheGeometry(**d)
+            object.__setattr__(self, "_other", got)
+        return got
 
     def as_struct(self) -> "_C.CacheGeom":
         """The ctypes struct, built once per geometry object (it is read-only for the library)."""
@@ -147,7 +167,7 @@ class CacheGeometry:
         if st is None:
             st = _C.CacheGeom(self.k_off, self.v_off, self.ks_off, self.vs_off, self.stride_block,
                               self.stride_slot, self.stride_head, self.num_kv_heads, self.head_size,
-                              self.block_size, 0)
+                              self.block_size, self.code_type)
             object.__setattr__(self, "_struct", st)
         return st
 
@@ -156,14 +176,28 @@ class CacheGeometry:
         return 2 * (self.head_size + SCALE_BYTES)
 
 
+_ONE_BYTE_DTYPES = tuple(d for d in (torch.int8, torch.uint8, getattr(torch, "float8_e4m3fn", None)) if d is not None)
+
+
+def code_type_of(kv_quant_mode) -> int:
+    """``kvq_cache_geom.code_type`` of a KV quantisation mode."""
+    if kv_quant_mode == KVQuantMode.INT8_PER_TOKEN_HEAD:
+        return _C.KVQ_CODE_INT8
+    if kv_quant_mode == KVQuantMode.FP8_PER_TOKEN_HEAD:
+        return _C.KVQ_CODE_FP8_E4M3
+    raise NotImplementedError(f"kv_quant_mode {kv_quant_mode!r}: INT8_PER_TOKEN_HEAD and FP8_PER_TOKEN_HEAD are built")
+
+
 def geometry_from_views(key_cache: torch.Tensor, value_cache: torch.Tensor,
-                        k_scale_cache: torch.Tensor, v_scale_cache: torch.Tensor) -> CacheGeometry:
+                        k_scale_cache: torch.Tensor, v_scale_cache: torch.Tensor,
+                        code_type: int = _C.KVQ_CODE_INT8) -> CacheGeometry:
     """Validate the four views and reduce them to one base pointer + byte geometry.
 
-    key_cache / value_cache: ``(nb, bs, Hkv, D+4)`` int8; scale caches ``(nb, bs, Hkv)`` fp32
-    over the same storage, all four with identical block/slot/head byte strides."""
-    if key_cache.dtype != torch.int8 or value_cache.dtype != torch.int8:
-        raise ValueError("key_cache/value_cache must be int8")
+    key_cache / value_cache: ``(nb, bs, Hkv, D+4)`` of a one-byte dtype (int8; uint8 or float8_e4m3fn
+    for fp8 codes); scale caches ``(nb, bs, Hkv)`` fp32 over the same storage, all four with identical
+    block/slot/head byte strides."""
+    if key_cache.dtype not in _ONE_BYTE_DTYPES or value_cache.dtype != key_cache.dtype:
+        raise ValueError("key_cache/value_cache must share a one-byte dtype (int8, uint8 or float8_e4m3fn)")
     if k_scale_cache.dtype != torch.float32 or v_scale_cache.dtype != torch.float32:
         raise ValueError("scale caches must be float32")
     if key_cache.dim() != 4 or key_cache.shape != value_cache.shape:
@@ -183,6 +217,7 @@ def geometry_from_views(key_cache: torch.Tensor, value_cache: torch.Tensor,
         ks_off=k_scale_cache.data_ptr() - base, vs_off=v_scale_cache.data_ptr() - base,
         stride_block=sb, stride_slot=ss, stride_head=sh,
         num_kv_heads=hkv, head_size=padded - SCALE_BYTES, block_size=bs, num_blocks=nb, base_ptr=base,
+        code_type=code_type,
     )
     if any(v % 4 for v in (geom.k_off, geom.v_off, geom.ks_off, geom.vs_off, sb, ss, sh, base)):
         raise ValueError("cache views must be 4-byte aligned")
@@ -243,6 +278,19 @@ class MlaGeometry:
     block_size: int
     num_blocks: int
     base_ptr: int
+    code_type: int = _C.KVQ_CODE_INT8   # what a code byte is: int8, or an e4m3fn bit pattern
+
+    def with_code_type(self, code_type: int) -> "CacheGeometry":
+        """The same bytes read as another kind of code (the geometry of a cache does not depend on it)."""
+        if code_type == self.code_type:
+            return self
+        got = self.__dict__.get("_other")
+        if got is None:
+            d = {k: v for k, v in self.__dict__.items() if not k.startswith("_")}
+            d["code_type"] = code_type
+            got = CacheGeometry(**d)
+            object.__setattr__(self, "_other", got)
+        return got
 
     def as_struct(self) -> "_C.MlaGeom":
         """The ctypes struct, built once per geometry object (it is read-only for the library)."""

@@ -15,10 +15,10 @@ from __future__ import annotations
 
 import importlib
 
-from .kv_cache_interface import INT8_PER_TOKEN, INT8_PER_TOKEN_HEAD
+from .kv_cache_interface import FP8_PER_TOKEN_HEAD, INT8_PER_TOKEN, INT8_PER_TOKEN_HEAD
 
 PLATFORM_PATH = "vllm_metax_amd.platform.Int8KVPlatform"
-INT8_KV_DTYPES = (INT8_PER_TOKEN_HEAD, INT8_PER_TOKEN)
+INT8_KV_DTYPES = (INT8_PER_TOKEN_HEAD, FP8_PER_TOKEN_HEAD, INT8_PER_TOKEN)   # the inline-scale dtypes this build serves
 
 INT8_ATTN_PATH = "vllm_metax_amd.v1.attention.backends.int8_attn.Int8AttentionBackend"
 INT8_MLA_PATH = "vllm_metax_amd.v1.attention.backends.mla.int8_mla.Int8MLABackend"

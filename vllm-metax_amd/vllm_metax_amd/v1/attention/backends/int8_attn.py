@@ -18,6 +18,7 @@ import torch
 from .... import _custom_ops as ops
 from ....kv_cache_interface import KVQuantMode, get_kv_quant_mode, kv_cache_uses_per_token_head_scales
 from ....layout import (
+    code_type_of,
     geometry_from_views,
     key_value_views,
     kv_cache_shape,
@@ -155,7 +156,7 @@ class Int8AttentionBackend(_BackendBase):
     (vllm_metax/v1/attention/backends/triton_attn.py:272-410)."""
 
     supported_dtypes: ClassVar[list[torch.dtype]] = [torch.float16, torch.bfloat16, torch.float32]
-    supported_kv_cache_dtypes: ClassVar[list[str]] = ["int8_per_token_head"]
+    supported_kv_cache_dtypes: ClassVar[list[str]] = ["int8_per_token_head", "fp8_per_token_head"]
     forward_includes_kv_cache_update: bool = False
 
     @staticmethod
@@ -273,9 +274,10 @@ class Int8AttentionImpl(_ImplBase):
             raise NotImplementedError(f"Int8AttentionImpl does not support: {', '.join(bad)}")
         if attn_type != AttentionType.DECODER:
             raise NotImplementedError("quantized KV cache is not supported for encoder attention")
-        if not kv_cache_uses_per_token_head_scales(kv_cache_dtype) or \
-                get_kv_quant_mode(kv_cache_dtype) != KVQuantMode.INT8_PER_TOKEN_HEAD:
-            raise ValueError(f"Int8AttentionImpl needs kv_cache_dtype 'int8_per_token_head', got {kv_cache_dtype!r}")
+        if not kv_cache_uses_per_token_head_scales(kv_cache_dtype) or get_kv_quant_mode(kv_cache_dtype) not in (
+                KVQuantMode.INT8_PER_TOKEN_HEAD, KVQuantMode.FP8_PER_TOKEN_HEAD):
+            raise ValueError("Int8AttentionImpl needs kv_cache_dtype 'int8_per_token_head' or 'fp8_per_token_head', "
+                             f"got {kv_cache_dtype!r}")
         if num_heads % num_kv_heads:
             raise ValueError("num_heads must be a multiple of num_kv_heads")
         self.num_heads = num_heads
@@ -322,7 +324,7 @@ class Int8AttentionImpl(_ImplBase):
             v_scale.fill_(1.0)
             key_cache, value_cache = key_value_views(kv_cache)
             got = (key_cache, value_cache, k_scale, v_scale,
-                   geometry_from_views(key_cache, value_cache, k_scale, v_scale))
+                   geometry_from_views(key_cache, value_cache, k_scale, v_scale, code_type_of(self._kv_quant_mode)))
             self._views[key] = got
         self._key_cache, self._value_cache, self._k_scale_cache, self._v_scale_cache, self._geometry = got
         self._views_for = key
