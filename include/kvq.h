@@ -27,7 +27,7 @@
 extern "C" {
 #endif
 
-#define KVQ_ABI_VERSION 9
+#define KVQ_ABI_VERSION 10
 
 #define KVQ_OK 0
 #define KVQ_EINVAL (-22)
@@ -389,6 +389,39 @@ KVQ_API int kvq_mla_decode_int8(void* out, int out_dtype, float* lse, const void
                         int64_t bt_stride, const int32_t* seq_lens, int num_seqs,
                         int num_heads, float scale, void* workspace, size_t workspace_bytes,
                         kvq_stream_t stream);
+
+/*
+ * Varlen attention with LSE output over dense K and V: the attention step of
+ * the MLA prefill.  Stands in for the two flash_attn_varlen_func calls of
+ * vllm_metax/v1/attention/backends/mla/prefill/flash_attn.py:176-221
+ * (run_prefill_new_tokens: causal, keys = the new tokens; run_prefill_context_chunk:
+ * unmasked, keys = one gathered chunk of the cached context, LSE returned), which
+ * vllm_metax/model_executor/layers/attention/mla_attention.py:2017-2140 and
+ * 2298-2378 call between gather_and_maybe_dequant_cache + kv_b_proj and
+ * merge_attn_states.  The key is taken in the two pieces the layer holds,
+ * k_nope [S, H, nope_dim] (a strided view of kv_b_proj's output) and
+ * k_pe [S, rope_dim] shared by all heads, instead of the concatenated tensor of
+ * mla_attention.py:1995-2015; v [S, H, v_dim] is read at its own head size (no
+ * padding to the qk head size, flash_attn.py:138-143).
+ * q [T, H, nope_dim + rope_dim]; out [T, H, v_dim]; lse [H, total_q] fp32 natural
+ * log, may be NULL.  All of `dtype` KVQ_BF16 or KVQ_F16, strides in elements and
+ * multiples of 8, pointers 16-byte aligned.  cu_seqlens_q / cu_seqlens_k
+ * [num_seqs + 1] int32 on the device; a sequence longer than max_seqlen_q is
+ * only attended for its first max_seqlen_q rows.  With `causal`, key j of a
+ * sequence is visible to its query row i iff j <= i + (k_len - q_len).  A row
+ * with no visible key gets out = 0 and lse = -inf (what mask_empty_context of
+ * mla_attention.py:2104-2110 forces).  Built head dims (nope, rope, v):
+ * (128, 64, 128), (64, 32, 64), (128, 0, 128).
+ */
+KVQ_API int kvq_mla_prefill_attn(const void* q, int dtype, int64_t q_stride_tok, int64_t q_stride_head,
+                         const void* k_nope, int64_t kn_stride_tok, int64_t kn_stride_head,
+                         const void* k_pe, int64_t kpe_stride_tok, const void* v,
+                         int64_t v_stride_tok, int64_t v_stride_head,
+                         const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k, int num_seqs,
+                         int max_seqlen_q, int64_t total_q, int num_heads, int nope_dim,
+                         int rope_dim, int v_dim, float scale, int causal, void* out,
+                         int64_t out_stride_tok, int64_t out_stride_head, float* lse,
+                         kvq_stream_t stream);
 
 #ifdef __cplusplus
 }

@@ -138,3 +138,55 @@ def merge_attn_states(prefix_output, prefix_lse, suffix_output, suffix_lse):
     pw = (pe / tot).T.unsqueeze(2)
     sw = (se / tot).T.unsqueeze(2)
     return prefix_output * pw + suffix_output * sw, out_lse
+
+
+def varlen_attn_lse(q, k_nope, k_pe, v, cu_q, cu_k, scale, causal):
+    """fp32 statement of the varlen attention the MLA prefill calls
+    (vllm_metax/v1/attention/backends/mla/prefill/flash_attn.py:176-221 ->
+    flash_attn_varlen_func with return_softmax_lse): q [T, H, nope + rope], k_nope [S, H, nope],
+    k_pe [S, rope] shared by the heads (the broadcast of mla_attention.py:1995-2015), v [S, H, dv].
+    With ``causal``, key j is visible to query row i iff j <= i + (k_len - q_len).  Returns
+    out [T, H, dv] fp32 and lse [H, T] fp32 (natural log); a row without visible keys gets 0 / -inf."""
+    T, H, _ = q.shape
+    out = torch.zeros(T, H, v.shape[2], dtype=torch.float32)
+    lse = torch.full((H, T), -torch.inf, dtype=torch.float32)
+    for b in range(len(cu_q) - 1):
+        qs, qe, ks, ke = int(cu_q[b]), int(cu_q[b + 1]), int(cu_k[b]), int(cu_k[b + 1])
+        if qe == qs or ke == ks:
+            continue
+        kk = k_nope[ks:ke].float()
+        if k_pe is not None:
+            kk = torch.cat([kk, k_pe[ks:ke].float()[:, None].expand(-1, H, -1)], dim=-1)
+        s = torch.einsum("qhd,khd->hqk", q[qs:qe].float(), kk) * scale
+        if causal:
+            i = torch.arange(qe - qs)[:, None]
+            j = torch.arange(ke - ks)[None]
+            s = s.masked_fill(j > i + (ke - ks) - (qe - qs), -torch.inf)
+        l = torch.logsumexp(s, dim=-1)
+        p = torch.nan_to_num(torch.exp(s - l[..., None]), nan=0.0)
+        out[qs:qe] = torch.einsum("hqk,khd->qhd", p, v[ks:ke].float())
+        lse[:, qs:qe] = l
+    return out, lse
+
+
+def mla_prefill_unchunked(q, kv_c_new, k_pe_new, context_rows, w_kv_b, query_lens, context_lens, kv_lora_rank,
+                          nope, scale, act_dtype):
+    """What the chunked-context prefill of the MLA layer must equal
+    (vllm_metax/model_executor/layers/attention/mla_attention.py:2017-2140, 2298-2378), stated without
+    chunks: every prefill attends, causally and in one pass, to its cached context followed by its new
+    tokens.  ``context_rows[b]`` are the dequantised latent rows [context_len, R + P] of prefill b, the
+    new tokens come as (kv_c_new [T, R], k_pe_new [T, P]); both are up-projected with ``w_kv_b``
+    [R, H * (nope + dv)] and the products rounded to ``act_dtype`` as the layer's GEMM output is.
+    Returns out [T, H, dv] fp32."""
+    T, H, _ = q.shape
+    hd = w_kv_b.shape[1] // H
+    outs = []
+    t0 = 0
+    for b, (ql, cl) in enumerate(zip(query_lens, context_lens)):
+        lat = torch.cat([context_rows[b][:, :kv_lora_rank].to(act_dtype).float(), kv_c_new[t0:t0 + ql].float()])
+        pe = torch.cat([context_rows[b][:, kv_lora_rank:].to(act_dtype).float(), k_pe_new[t0:t0 + ql].float()])
+        kv = (lat @ w_kv_b.float()).to(act_dtype).float().view(cl + ql, H, hd)
+        o, _ = varlen_attn_lse(q[t0:t0 + ql], kv[..., :nope], pe, kv[..., nope:], [0, ql], [0, cl + ql], scale, True)
+        outs.append(o)
+        t0 += ql
+    return torch.cat(outs)

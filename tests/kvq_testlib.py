@@ -99,3 +99,32 @@ def assert_close_attn(got, want, atol=2e-2, rtol=1e-2, what=""):
     bound = atol + rtol * want.abs()
     worst = (err - bound).max().item()
     assert worst <= 0, f"{what}: max |err| {err.max().item():.4g}, worst excess over atol+rtol*|ref| {worst:.4g}"
+
+
+def build_mla_cache(ctx, bs, seed, dtype=torch.bfloat16, poison=True, amp=1.0, rows_fn=None, R=512, P=64):
+    """A latent cache written by the oracle for sequences of the given lengths, blocks shuffled.
+    ``rows_fn(kv_c, k_pe)`` may reshape the random rows of a sequence before they are quantised."""
+    g = torch.Generator().manual_seed(seed)
+    B = len(ctx)
+    per = [(c + bs - 1) // bs for c in ctx]
+    nb = sum(per) + 3
+    order = torch.randperm(nb, generator=g).tolist()
+    cache = L.allocate_mla_cache(nb, bs, R + P, device="cpu", fill=-1 if poison else 0)  # all-ones bytes: unwritten scales read as NaN
+    codes, scales = L.mla_cache_views(cache)
+    lay = oracle.MlaLayout.from_views(cache, codes, scales, R)
+    bt = torch.zeros((B, max(max(per), 1)), dtype=torch.int32)
+    it = iter(order)
+    for i, c in enumerate(ctx):
+        blocks = [next(it) for _ in range(per[i])]
+        bt[i, : per[i]] = torch.tensor(blocks, dtype=torch.int32)
+        if c == 0:
+            continue
+        kv_c = (torch.randn((c, R), generator=g) * amp).to(dtype)
+        k_pe = (torch.randn((c, P), generator=g) * amp).to(dtype)
+        if rows_fn is not None:
+            kv_c, k_pe = rows_fn(kv_c.float(), k_pe.float())
+            kv_c, k_pe = kv_c.to(dtype), k_pe.to(dtype)
+        pos = torch.arange(c)
+        slots = (bt[i, pos // bs].long() * bs + pos % bs)
+        oracle.mla_cache_write(kv_c, k_pe, cache, lay, slots)
+    return cache, lay, bt, torch.tensor(ctx, dtype=torch.int32)

@@ -700,3 +700,55 @@ def concat_mla_q(ql_nope: torch.Tensor, q_pe: torch.Tensor, q_out: torch.Tensor)
                                         ql_nope.stride(0), ql_nope.stride(1), _ptr(q_pe), q_pe.stride(0),
                                         q_pe.stride(1), _dtype_code(ql_nope, "ql_nope"), T, H, R, P, _stream(dev))
     _C.check(rc, "concat_mla_q")
+
+
+def mla_prefill_attention(q: torch.Tensor, k_nope: torch.Tensor, k_pe: torch.Tensor | None, v: torch.Tensor,
+                          cu_seqlens_q: torch.Tensor, cu_seqlens_k: torch.Tensor, max_seqlen_q: int,
+                          softmax_scale: float, causal: bool, out: torch.Tensor | None = None,
+                          lse: torch.Tensor | None = None, return_softmax_lse: bool = False):
+    """Varlen attention of the MLA prefill with the LSE the chunked-context merge needs: the role of
+    ``flash_attn_varlen_func`` in vllm_metax/v1/attention/backends/mla/prefill/flash_attn.py:128-221 (keyword
+    names kept), except that the key comes in the two pieces the layer holds -- ``k_nope [S, H, nope]`` and
+    ``k_pe [S, rope]`` or ``[S, 1, rope]``, shared by the heads -- and ``v [S, H, v_dim]`` keeps its own
+    head size.  ``q [T, H, nope + rope]``; returns ``out [T, H, v_dim]``, and ``(out, lse [H, T] fp32)`` with
+    ``return_softmax_lse``.  ``out`` / ``lse`` may be passed in to avoid the allocation."""
+    dev = _require_cuda(q, k_nope, k_pe, v, cu_seqlens_q, cu_seqlens_k, out, lse)
+    if q.dim() != 3 or k_nope.dim() != 3 or v.dim() != 3:
+        raise RuntimeError("q, k_nope and v must be [tokens, heads, dim]")
+    T, H, Dqk = q.shape
+    S, _, nope = k_nope.shape
+    rope = Dqk - nope
+    dv = v.shape[2]
+    if k_pe is not None and k_pe.dim() == 3:
+        if k_pe.shape[1] != 1:
+            raise RuntimeError("k_pe must be shared by the heads: [S, rope] or [S, 1, rope]")
+        k_pe = k_pe[:, 0]
+    if rope < 0 or (rope > 0 and (k_pe is None or tuple(k_pe.shape) != (S, rope))):
+        raise RuntimeError(f"k_pe must be [{S}, {rope}] for q of head size {Dqk} and k_nope of {nope}")
+    if k_nope.shape[1] != H or tuple(v.shape[:2]) != (S, H):
+        raise RuntimeError("k_nope and v must have q's head count and one row per key")
+    for name, t in (("q", q), ("k_nope", k_nope), ("k_pe", k_pe), ("v", v)):
+        if t is not None and (t.dtype != q.dtype or t.stride(-1) != 1):
+            raise RuntimeError(f"{name}: one dtype and contiguous last dims are required")
+    for name, t in (("cu_seqlens_q", cu_seqlens_q), ("cu_seqlens_k", cu_seqlens_k)):
+        if t.dtype != torch.int32 or not t.is_contiguous():
+            raise RuntimeError(f"{name} must be contiguous int32")
+    B = cu_seqlens_q.numel() - 1
+    if cu_seqlens_k.numel() != B + 1:
+        raise RuntimeError("cu_seqlens_q and cu_seqlens_k must have the same length")
+    if out is None:
+        out = torch.empty(T, H, dv, dtype=q.dtype, device=dev)
+    elif tuple(out.shape) != (T, H, dv) or out.dtype != q.dtype or out.stride(2) != 1:
+        raise RuntimeError(f"out must be [{T}, {H}, {dv}] of q's dtype with a contiguous last dim")
+    if lse is None and return_softmax_lse:
+        lse = torch.empty(H, T, dtype=torch.float32, device=dev)
+    if lse is not None and (tuple(lse.shape) != (H, T) or lse.dtype != torch.float32 or not lse.is_contiguous()):
+        raise RuntimeError(f"lse must be contiguous float32 [{H}, {T}]")
+    with _on_device(dev):
+        rc = _C.load().kvq_mla_prefill_attn(
+            _ptr(q), _dtype_code(q, "q"), q.stride(0), q.stride(1), _ptr(k_nope), k_nope.stride(0), k_nope.stride(1),
+            _ptr(k_pe), k_pe.stride(0) if k_pe is not None else 0, _ptr(v), v.stride(0), v.stride(1),
+            _ptr(cu_seqlens_q), _ptr(cu_seqlens_k), B, int(max_seqlen_q), T, H, nope, rope, dv, float(softmax_scale),
+            1 if causal else 0, _ptr(out), out.stride(0), out.stride(1), _ptr(lse), _stream(dev))
+    _C.check(rc, "mla_prefill_attention")
+    return (out, lse) if return_softmax_lse else out

@@ -1,9 +1,10 @@
-"""MLA decode backend over the int8 latent cache on MI355X.
+"""MLA backend over the int8 latent cache on MI355X.
 
-Host-side mirror of the reference's TRITON_MLA backend for the decode path
+Host-side mirror of the reference's TRITON_MLA backend
 (vllm_metax/v1/attention/backends/mla/triton_mla.py): ``forward_mqa`` has the reference's
 signature and returns ``(o, lse)``; the cache write keeps ``concat_and_cache_mla``'s argument
-order.  The int8 latent entry (576 codes + one fp32 scale per token, rows first and the scale
+order; ``forward_mha`` is the prefill half of the MLA layer with its chunked context
+(vllm_metax/model_executor/layers/attention/mla_attention.py:2298-2378).  The int8 latent entry (576 codes + one fp32 scale per token, rows first and the scale
 region after them inside each block) is this build's: the reference's MLA backends stop at fp8
 (:94-100).
 """
@@ -18,6 +19,8 @@ from ..... import _custom_ops as ops
 from .....kv_cache_interface import INT8_PER_TOKEN
 from .....layout import mla_cache_shape, mla_geometry
 from ..int8_attn import AttentionCGSupport, AttentionType, MultipleOf, _BackendBase, _BuilderBase, _first_attr
+from .prefill import (Int8MLAPrefillBackend, Int8MLAPrefillMetadata, build_mla_chunked_context_metadata,
+                      compute_prefill_context, determine_chunked_prefill_workspace_size)
 
 try:  # pragma: no cover - upstream vLLM is not installed in the build container
     from vllm.v1.attention.backend import MLAAttentionImpl as _MLAImplBase  # type: ignore
@@ -64,6 +67,7 @@ class Int8MLAMetadata:
     num_decode_tokens: int
     num_prefills: int
     decode: Int8MLADecodeMetadata | None
+    prefill: Int8MLAPrefillMetadata | None = None
     workspace: torch.Tensor | None = None   # split states + int8 query terms of the decode launch
     decode_out: torch.Tensor | None = None  # [max_num_seqs, H, kv_lora_rank]
     decode_lse: torch.Tensor | None = None  # [max_num_seqs, H] fp32
@@ -101,6 +105,23 @@ class Int8MLAMetadataBuilder(_BuilderBase):
             else torch.bfloat16
         self._workspace = self._out = self._lse = None
         self._reserve_decode_buffers()
+        # prefill side: the context workspace (mla_attention.py:1554-1582, 1668-1690) and the attention calls
+        hf_cfg = getattr(model_config, "hf_text_config", None)
+        self.qk_nope_head_dim = int(getattr(hf_cfg, "qk_nope_head_dim", 128) or 128)
+        self.qk_rope_head_dim = int(getattr(hf_cfg, "qk_rope_head_dim", 64) or 64)
+        self.v_head_dim = int(getattr(hf_cfg, "v_head_dim", 128) or 128)
+        self.block_size = int(_first_attr(kv_cache_spec, "block_size", default=64))
+        max_model_len = int(_first_attr(model_config, "max_model_len", default=0) or 0) if model_config is not None else 0
+        self.chunked_prefill_workspace_size = int(
+            _first_attr(vllm_config, "mla_chunked_prefill_workspace_size", default=0)
+            or determine_chunked_prefill_workspace_size(max_model_len or 8192, self.max_num_seqs, self.block_size))
+        self._chunked_prefill_workspace = None
+        self._prefill_backend = None
+        if self.num_heads is not None:
+            scale = (self.qk_nope_head_dim + self.qk_rope_head_dim) ** -0.5
+            self._prefill_backend = Int8MLAPrefillBackend(self.num_heads, scale, self.kv_lora_rank,
+                                                          self.qk_nope_head_dim, self.qk_rope_head_dim,
+                                                          self.v_head_dim, vllm_config)
 
     def _reserve_decode_buffers(self) -> None:
         if self.device.type != "cuda" or self.num_heads is None:
@@ -135,11 +156,43 @@ class Int8MLAMetadataBuilder(_BuilderBase):
         if num_decodes > 0:
             decode = Int8MLADecodeMetadata(block_table=c.block_table_tensor[:num_decodes],
                                            seq_lens=c.seq_lens[:num_decodes])
+        prefill = None
+        if c.num_reqs > num_decodes:
+            prefill = self._build_prefill(c, qsl_cpu, num_decodes)
         return Int8MLAMetadata(
             num_actual_tokens=c.num_actual_tokens, num_reqs=c.num_reqs, max_query_len=c.max_query_len,
             max_seq_len=c.max_seq_len, query_start_loc=c.query_start_loc, slot_mapping=c.slot_mapping,
             num_decodes=num_decodes, num_decode_tokens=num_decode_tokens, num_prefills=c.num_reqs - num_decodes,
-            decode=decode, workspace=self._workspace, decode_out=self._out, decode_lse=self._lse)
+            decode=decode, prefill=prefill, workspace=self._workspace, decode_out=self._out, decode_lse=self._lse)
+
+    def _build_prefill(self, c, qsl_cpu: torch.Tensor, start: int) -> Int8MLAPrefillMetadata:
+        """The prefill half of MLACommonMetadataBuilder.build (mla_attention.py:1784-1830): offsets relative
+        to the first prefill token, context lengths from the host copy of the sequence lengths."""
+        n = c.num_reqs
+        seq_lens_cpu = _first_attr(c, "seq_lens_cpu_upper_bound", "seq_lens_cpu", default=None)
+        if seq_lens_cpu is None:
+            seq_lens_cpu = c.seq_lens.cpu()
+        qlens = qsl_cpu[start + 1:n + 1] - qsl_cpu[start:n]
+        context_lens = seq_lens_cpu[start:n].to(qlens.dtype) - qlens
+        qsl_rel_cpu = (qsl_cpu[start:n + 1] - qsl_cpu[start]).to(torch.int32)
+        qsl_rel = (c.query_start_loc[start:n + 1] - c.query_start_loc[start]).to(torch.int32)
+        chunked = None
+        if int(context_lens.max()) > 0:
+            if self._chunked_prefill_workspace is None:
+                self._chunked_prefill_workspace = torch.empty(
+                    (self.chunked_prefill_workspace_size, self.kv_lora_rank + self.qk_rope_head_dim),
+                    dtype=self.dtype, device=self.device)
+            chunked = build_mla_chunked_context_metadata(
+                context_lens_cpu=context_lens, prefill_query_start_loc_cpu=qsl_rel_cpu, num_prefills=n - start,
+                chunked_prefill_workspace=self._chunked_prefill_workspace,
+                chunked_prefill_workspace_size=self.chunked_prefill_workspace_size, block_size=self.block_size,
+                align_chunk_to_block=True, device=self.device)
+        md = Int8MLAPrefillMetadata(block_table=c.block_table_tensor[start:n], query_start_loc=qsl_rel,
+                                    max_query_len=int(qlens.max()), chunked_context=chunked,
+                                    prefill_backend=self._prefill_backend)
+        if self._prefill_backend is not None:
+            self._prefill_backend.prepare_metadata(md)
+        return md
 
 
 class Int8MLABackend(_BackendBase):
@@ -207,7 +260,7 @@ class Int8MLAImpl(_MLAImplBase):
                  alibi_slopes=None, sliding_window=None, kv_cache_dtype: str = INT8_PER_TOKEN,
                  logits_soft_cap=None, attn_type: str = AttentionType.DECODER,
                  kv_sharing_target_layer_name=None, kv_lora_rank: int = 512, qk_rope_head_dim: int = 64,
-                 **mla_args) -> None:
+                 qk_nope_head_dim: int = 128, v_head_dim: int = 128, kv_b_proj=None, **mla_args) -> None:
         if any([alibi_slopes, sliding_window, logits_soft_cap]):
             raise NotImplementedError(
                 "Int8MLAImpl does not support one of the following: alibi_slopes, sliding_window, logits_soft_cap")
@@ -221,6 +274,9 @@ class Int8MLAImpl(_MLAImplBase):
         self.scale = float(scale)
         self.kv_lora_rank = kv_lora_rank
         self.qk_rope_head_dim = qk_rope_head_dim
+        self.qk_nope_head_dim = qk_nope_head_dim
+        self.v_head_dim = v_head_dim
+        self.kv_b_proj = kv_b_proj
         self.kv_cache_dtype = kv_cache_dtype
         self.supports_quant_query_input = False
         self._geometry = None
@@ -265,9 +321,48 @@ class Int8MLAImpl(_MLAImplBase):
                             geometry=self._geom(kv_c_and_k_pe_cache))
         return o, lse
 
-    def forward_mha(self, *args, **kwargs):
-        raise NotImplementedError("this backend serves the decode half of the MLA layer (forward_mqa); prefill "
-                                  "tokens go through the layer's prefill backend, as in the reference")
+    def _kv_up_proj(self, kv_c: torch.Tensor) -> torch.Tensor:
+        if self.kv_b_proj is None:
+            raise RuntimeError("forward_mha needs the layer's kv_b_proj (pass kv_b_proj= to the impl)")
+        y = self.kv_b_proj(kv_c)
+        y = y[0] if type(y) is tuple else y    # the reference's linear layers return (output, bias)
+        return y.view(-1, self.num_heads, self.qk_nope_head_dim + self.v_head_dim)
+
+    def forward_mha(self, q: torch.Tensor, kv_c_normed: torch.Tensor, k_pe: torch.Tensor,
+                    kv_c_and_k_pe_cache: torch.Tensor, attn_metadata, k_scale=None,
+                    output: torch.Tensor | None = None, output_scale=None) -> torch.Tensor:
+        """Prefill tokens, signature of MLACommonImpl.forward_mha (mla_attention.py:2298-2378): ``q
+        [T, H, nope + rope]``, ``kv_c_normed [T, kv_lora_rank]`` and ``k_pe [T, 1, rope]`` (or ``[T, rope]``)
+        of the new tokens, ``output [T, H * v_head_dim]``.  The causal pass over the new tokens is merged
+        with the attention over the cached context, which is read back from the int8 latent cache chunk by
+        chunk (``compute_prefill_context``)."""
+        prefill = attn_metadata.prefill
+        assert prefill is not None and prefill.prefill_backend is not None
+        if output_scale is not None:
+            raise NotImplementedError("quantised attention output is not built")
+        T = q.shape[0]
+        if output is None:
+            output = torch.empty((T, self.num_heads * self.v_head_dim), dtype=q.dtype, device=q.device)
+        out3 = output.view(T, self.num_heads, self.v_head_dim)
+        kv_nope = self._kv_up_proj(kv_c_normed)
+        k_nope, v = kv_nope[..., :self.qk_nope_head_dim], kv_nope[..., self.qk_nope_head_dim:]
+        k_pe2 = k_pe.reshape(T, -1)
+        has_context = prefill.chunked_context is not None
+        if not has_context:
+            prefill.prefill_backend.run_prefill_new_tokens(q=q, k=(k_nope, k_pe2), v=v, return_softmax_lse=False,
+                                                           out=out3)
+            return output
+        suffix_output, suffix_lse = prefill.prefill_backend.run_prefill_new_tokens(
+            q=q, k=(k_nope, k_pe2), v=v, return_softmax_lse=True)
+        context_output, context_lse = compute_prefill_context(
+            q, kv_c_and_k_pe_cache, prefill, self._kv_up_proj, self.num_heads, self.kv_lora_rank,
+            self.qk_nope_head_dim, self.v_head_dim, geometry=self._geom(kv_c_and_k_pe_cache))
+        if not out3.is_contiguous():
+            raise RuntimeError("output must be contiguous")
+        ops.merge_attn_states(output=out3, prefix_output=context_output, prefix_lse=context_lse,
+                              suffix_output=suffix_output, suffix_lse=suffix_lse,
+                              prefill_tokens_with_context=prefill.chunked_context.prefill_tokens_with_context)
+        return output
 
 
 class Int8MLADecodeCaller:
