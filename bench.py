@@ -301,14 +301,50 @@ def mla_main(args, cfg, dev, ops):
         "roofline": {"bound": "mfma", "achieved": round(flops / attn_s / 1e12, 1), "peak": MFMA_F16_PEAK_TFLOPS,
                      "unit": "TFLOP/s", "frac": round(flops / attn_s / 1e12 / MFMA_F16_PEAK_TFLOPS, 4),
                      "traffic": traffic, "traffic_source": traffic_source,
-                     "kernel": "MLA decode launch = mla_quant_q_kernel + mla_decode_kernel + mla_reduce_kernel",
+                     "kernel": "MLA decode launch on an absorbed query = mla_quant_q_kernel + mla_decode_kernel + mla_reduce_kernel",
                      "timing": f"{n_ev} decode launches back to back between two events on the launch stream",
                      "algorithmic_flops_per_launch": flops, "algorithmic_bytes_per_launch": nbytes,
                      "hbm_frac_of_peak": round(nbytes / attn_s / 1e9 / HBM_PEAK_GBPS, 4)},
     }
+    res["decode_caller"] = mla_caller_chain(cfg, st, dev, ops, n_ev)
     if not args.no_cpu_baseline:
         res["cpu_baseline"] = mla_cpu_baseline(cfg, st, args.cpu_seconds)
     print(json.dumps(res))
+
+
+def mla_caller_chain(cfg, st, dev, ops, n):
+    """The layer-level decode step around the launch above, from the un-absorbed query (q_nope x W_UK_T ->
+    decode -> x W_UV, mla_attention.py:835-848, 902): with the absorption inside the decode launch, and as
+    the reference's three steps (library GEMM, decode of the bf16 product, library GEMM)."""
+    from types import SimpleNamespace
+
+    from vllm_metax_amd.v1.attention.backends.mla.int8_mla import Int8MLADecodeCaller, Int8MLAImpl
+
+    H, R, P, B, Pn, V = cfg["heads"], cfg["r"], cfg["p"], len(cfg["ctx"]), 128, 128
+    impl = Int8MLAImpl(num_heads=H, head_size=R + P, scale=st["scale"], kv_lora_rank=R, qk_rope_head_dim=P)
+    w_uk_t = (torch.randn((H, Pn, R), device=dev) / Pn ** 0.5).to(torch.bfloat16)
+    w_uv = (torch.randn((H, R, V), device=dev) / R ** 0.5).to(torch.bfloat16)
+    caller = Int8MLADecodeCaller(impl, w_uk_t, w_uv)
+    q_nope = (torch.randn((B, H, Pn), device=dev) * 0.5).to(torch.bfloat16)
+    q_pe = (torch.randn((B, H, P), device=dev) * 0.5).to(torch.bfloat16)
+    out = torch.empty((B, H * V), dtype=torch.bfloat16, device=dev)
+    md = SimpleNamespace(decode=SimpleNamespace(block_table=st["bt_d"], seq_lens=st["sl_d"]), workspace=st["ws"],
+                         decode_out=st["out"], decode_lse=st["lse"])
+    L = len(st["caches"])
+
+    def fused(i):
+        caller.forward_decode(q_nope, q_pe, st["caches"][i % L], md, out)
+
+    def three_steps(i):
+        attn_out, _ = impl.forward_mqa((caller.absorb_q(q_nope), q_pe), st["caches"][i % L], md)
+        caller.v_up_proj(attn_out, out)
+
+    res = {}
+    for name, fn in (("absorb_in_launch_us", fused), ("library_gemm_then_decode_us", three_steps)):
+        prewarm(fn, 0.2)
+        res[name] = round(time_back_to_back(fn, n) * 1e6, 2)
+    res["steps"] = "q_nope [B,H,128] x W_UK_T -> decode -> x W_UV [H,512,128] -> out [B, H*128], bf16"
+    return res
 
 
 def mixed_main(args, cfg, dev, ops):

@@ -391,6 +391,28 @@ KVQ_API int kvq_mla_decode_int8(void* out, int out_dtype, float* lse, const void
                         kvq_stream_t stream);
 
 /*
+ * MLA decode with the query absorption fused in: the first bmm of the
+ * reference's MLA layer, ql_nope = q_nope x W_UK_T
+ * (vllm_metax/model_executor/layers/attention/mla_attention.py:835-848), runs on
+ * the MFMA inside the launch and its result goes straight into the decode's
+ * int8 operand layout; the absorbed query is never written to memory in the
+ * activation type.  Same results contract, cache, workspace and outputs as
+ * kvq_mla_decode_int8 (whose q = ql_nope, q_pe form this replaces).
+ * q_nope [B, H, nope_dim] and q_pe [B, H, rope_dim] (strides in elements,
+ * 4-byte aligned rows), w_uk_t [H, nope_dim, kv_lora_rank] with contiguous last
+ * dim, 16-byte aligned rows (strides multiples of 8); all three KVQ_BF16 or
+ * KVQ_F16; nope_dim a multiple of 32.
+ */
+KVQ_API int kvq_mla_decode_absorb_int8(void* out, int out_dtype, float* lse, const void* q_nope, int q_dtype,
+                               int64_t qn_stride_b, int64_t qn_stride_h, int nope_dim,
+                               const void* w_uk_t, int64_t w_stride_h, int64_t w_stride_p,
+                               const void* q_pe, int64_t q_pe_stride_b, int64_t q_pe_stride_h,
+                               const void* cache, const kvq_mla_geom* geom,
+                               const int32_t* block_table, int64_t bt_stride,
+                               const int32_t* seq_lens, int num_seqs, int num_heads, float scale,
+                               void* workspace, size_t workspace_bytes, kvq_stream_t stream);
+
+/*
  * Varlen attention with LSE output over dense K and V: the attention step of
  * the MLA prefill.  Stands in for the two flash_attn_varlen_func calls of
  * vllm_metax/v1/attention/backends/mla/prefill/flash_attn.py:176-221

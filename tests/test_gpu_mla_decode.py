@@ -265,6 +265,65 @@ def test_mla_decode_caller_absorb_decode_up_proj(gpu_device):
     torch.testing.assert_close(lse.cpu(), lse_ref, atol=2e-2, rtol=1e-3)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("N,Pn,ctx", [
+    (16, 128, [300, 1000, 64]),
+    (128, 128, [700] * 5 + [33]),
+    (20, 64, [5, 0, 95, 1000, 31, 32] * 7),      # 42 sequences: a second block of 32, a last tile of 10; 20 heads: a group of 4
+])
+def test_mla_decode_with_fused_absorption(gpu_device, dtype, N, Pn, ctx):
+    """kvq_mla_decode_absorb_int8: q_nope x W_UK_T on the MFMA inside the launch, written as the decode's int8
+    operands (vllm_metax/model_executor/layers/attention/mla_attention.py:835-848 + the decode).  Checked
+    against the oracle's decode of the fp32 product -- the fused path never rounds it to the activation type."""
+    dev = gpu_device
+    B = len(ctx)
+    cache, lay, bt, sl = _build(ctx, 64, seed=51, dtype=dtype)
+    g = torch.Generator().manual_seed(52)
+    W_UK_T = (torch.randn((N, Pn, R), generator=g) / Pn ** 0.5).to(dtype)
+    q_nope = torch.randn((B, N, Pn), generator=g).to(dtype)
+    q_pe = torch.randn((B, N, P), generator=g).to(dtype)
+    scale = (Pn + P) ** -0.5
+    o = torch.full((B, N, R), float("nan"), dtype=dtype, device=dev)
+    lse = torch.full((B, N), float("nan"), dtype=torch.float32, device=dev)
+    # q_nope as the strided view a fused q projection leaves: the nope slice of [B, N, Pn + P]
+    q_full = torch.cat([q_nope, q_pe], dim=-1).to(dev)
+    ops.mla_decode_absorb_int8(q_full[..., :Pn], W_UK_T.to(dev), q_full[..., Pn:], cache.to(dev), o, lse, bt.to(dev),
+                               sl.to(dev), scale, R)
+    torch.cuda.synchronize()
+    ql = torch.einsum("bnp,npl->bnl", q_nope.float(), W_UK_T.float())
+    want, want_lse = oracle.mla_decode(torch.cat([ql, q_pe.float()], -1), cache, lay, bt, sl, scale)
+    live = sl > 0
+    T.assert_close_attn(o[live.to(dev)], want[live], what="fused absorption")
+    assert torch.all(o[(~live).to(dev)] == 0)
+    torch.testing.assert_close(lse.cpu()[live], want_lse[live], atol=5e-3, rtol=1e-3)
+
+
+def test_decode_caller_makes_one_library_gemm(gpu_device, monkeypatch):
+    """The Q side of Int8MLADecodeCaller.forward_decode runs in the decode launch: the only torch.bmm left is
+    the V up-projection (mla_attention.py:902, 1087-1110)."""
+    from types import SimpleNamespace
+
+    from vllm_metax_amd.v1.attention.backends.mla.int8_mla import Int8MLADecodeCaller, Int8MLAImpl
+
+    dev = gpu_device
+    N, Pn, V = 16, 128, 128
+    cache, lay, bt, sl = _build([100, 40], 64, seed=61)
+    g = torch.Generator().manual_seed(62)
+    W_UK_T = (torch.randn((N, Pn, R), generator=g) / Pn ** 0.5).to(torch.bfloat16).to(dev)
+    W_UV = (torch.randn((N, R, V), generator=g) / R ** 0.5).to(torch.bfloat16).to(dev)
+    impl = Int8MLAImpl(num_heads=N, head_size=R + P, scale=0.07, kv_lora_rank=R, qk_rope_head_dim=P)
+    caller = Int8MLADecodeCaller(impl, W_UK_T, W_UV)
+    md = SimpleNamespace(decode=SimpleNamespace(block_table=bt.to(dev), seq_lens=sl.to(dev)))
+    calls = []
+    real_bmm = torch.bmm
+    monkeypatch.setattr(torch, "bmm", lambda *a, **k: (calls.append(a[0].shape), real_bmm(*a, **k))[1])
+    out = torch.empty((2, N * V), dtype=torch.bfloat16, device=dev)
+    caller.forward_decode(torch.randn((2, N, Pn), generator=g).to(torch.bfloat16).to(dev),
+                          torch.randn((2, N, P), generator=g).to(torch.bfloat16).to(dev), cache.to(dev), md, out)
+    torch.cuda.synchronize()
+    assert calls == [torch.Size([N, 2, R])]
+
+
 def test_mla_decode_errors(gpu_device):
     dev = gpu_device
     cache = L.allocate_mla_cache(4, 64, R + P, device=dev)

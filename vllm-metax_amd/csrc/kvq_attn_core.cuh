@@ -92,6 +92,33 @@ __device__ __forceinline__ float clamp_half_range(float x) {
   return fminf(fmaxf(x, -65504.f), 65504.f);
 }
 
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float floatx2 __attribute__((ext_vector_type(2)));
+
+// 16x16x32 MFMA of the activation type (fp16 or bf16 operands as four dwords, fp32 accumulate).
+template <int DT>
+__device__ __forceinline__ floatx4 mfma16(u32x4 a, u32x4 b, floatx4 c) {
+  if constexpr (DT == KVQ_F16)
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, a), __builtin_bit_cast(half8_t, b), c, 0, 0, 0);
+  else
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+}
+
+// Two floats rounded to the activation type, packed into one dword.
+template <int DT>
+__device__ __forceinline__ uint32_t pack2(float a, float b) {
+  if constexpr (DT == KVQ_F16) {
+    return pack_half2(a, b);
+  } else {
+    const floatx2 f = {a, b};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2_t));
+  }
+}
+
+// Selectors that build one dword of a register transposition: the low (or high) halves of two dwords.
+constexpr uint32_t kPermLowHalves = 0x05040100u, kPermHighHalves = 0x07060302u;
+
 // What a finished run of tiles turns into.
 enum class Emit { kFinal, kStreamPartial, kV2Partial };
 

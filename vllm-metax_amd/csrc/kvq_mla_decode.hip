@@ -93,6 +93,30 @@ __device__ __forceinline__ int mla_split_len(int len, int num_splits) {
   return ((per + kTile - 1) / kTile) * kTile;
 }
 
+// 16 values of one head -> the 16 bytes of each of the two int8 terms (see mla_quant_q_kernel): a =
+// rint(q / s1), b = rint((q - s1 a) * 254 / s1).  `live` false gives zero bytes (heads past the end).
+__device__ __forceinline__ void mla_two_int8_terms(const float (&f)[16], float s1, bool live, u32x4& ta, u32x4& tb) {
+  const float inv1 = 1.0f / s1, inv2 = 254.0f * inv1;
+  // x + 1.5 * 2^23 rounds x to the nearest integer (ties to even) and leaves it, in two's complement,
+  // in the low mantissa bits: the low byte is the int8 code (|x| <= 127 here by construction)
+  constexpr float kMagic = 12582912.0f;
+#pragma unroll
+  for (int w = 0; w < 4; ++w) {
+    uint32_t ba[4], bb[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const float q = live ? f[4 * w + j] : 0.f;
+      const float ra = __builtin_fmaf(q, inv1, kMagic);
+      const float r = __builtin_fmaf(-(ra - kMagic), s1, q);
+      const float rb = __builtin_fmaf(r, inv2, kMagic);
+      ba[j] = as_u32(ra);
+      bb[j] = as_u32(rb);
+    }
+    ta[w] = perm(ba[1], ba[0], 0x0c0c0400u) | perm(ba[3], ba[2], 0x04000c0cu);
+    tb[w] = perm(bb[1], bb[0], 0x0c0c0400u) | perm(bb[3], bb[2], 0x04000c0cu);
+  }
+}
+
 // Q for the int8 MFMA.  The cache codes ARE int8, so the QK product can run on
 // v_mfma_i32_16x16x64_i8 straight from the cached bytes -- no conversion of K at all -- once Q is
 // int8 too: q = s1 * a + s2 * b with a = rint(q / s1), s1 = max|q| / 127 per head, and
@@ -164,35 +188,168 @@ __global__ __launch_bounds__(256) void mla_quant_q_kernel(MlaArgs a) {
   amax = fmaxf(fmaxf(part_max[0][c], part_max[1][c]), fmaxf(part_max[2][c], part_max[3][c]));
   amax = head_ok ? fminf(amax, 3.0e38f) : 0.f;      // heads past the end contribute zero columns
   const float s1 = amax > 0.f ? amax / 127.0f : 1.0f;
-  const float inv1 = 1.0f / s1, inv2 = 254.0f * inv1;
-  // x + 1.5 * 2^23 rounds x to the nearest integer (ties to even) and leaves it, in two's complement,
-  // in the low mantissa bits: the low byte is the int8 code (|x| <= 127 here by construction)
-  constexpr float kMagic = 12582912.0f;
 #pragma unroll
   for (int n = 0; n < kMine; ++n) {
     const int kk = wave + 4 * n;
     u32x4 ta, tb;
-#pragma unroll
-    for (int w = 0; w < 4; ++w) {
-      uint32_t ba[4], bb[4];
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const float q = head_ok ? f[n][4 * w + j] : 0.f;
-        const float ra = __builtin_fmaf(q, inv1, kMagic);
-        const float r = __builtin_fmaf(-(ra - kMagic), s1, q);
-        const float rb = __builtin_fmaf(r, inv2, kMagic);
-        ba[j] = as_u32(ra);
-        bb[j] = as_u32(rb);
-      }
-      ta[w] = perm(ba[1], ba[0], 0x0c0c0400u) | perm(ba[3], ba[2], 0x04000c0cu);
-      tb[w] = perm(bb[1], bb[0], 0x0c0c0400u) | perm(bb[3], bb[2], 0x04000c0cu);
-    }
+    mla_two_int8_terms(f[n], s1, head_ok, ta, tb);
     if (kk < kMlaKSteps8) {
       qdst[(2 * kk) * kWave] = ta;
       qdst[(2 * kk + 1) * kWave] = tb;
     }
   }
   if (wave == 0 && g == 0) a.q_scale[qblock * 16 + c] = s1;
+}
+
+// Q absorption fused with the int8 preparation: ql[b, h, :] = q_nope[b, h, :] . W_UK_T[h] (the first
+// bmm of the reference's MLA layer, mla_attention.py:835-848) computed on the MFMA and written
+// STRAIGHT into the decode's operand layout as two int8 terms + s1 -- the absorbed query never exists
+// in HBM as bf16 and mla_quant_q_kernel does not run.
+// Workgroup = (head, 16 sequences), 4 waves; wave w owns latent dims 128 w .. 128 w + 127.  The product
+// is taken transposed, ql^T = W^T q^T: B = q_nope rows (lane = sequence, 8 consecutive p), A = W^T needs 8
+// p of one dim per lane while W_UK_T [P, L] keeps 8 dims of one p together, so each lane loads the
+// slice [its 8 p] x [8 consecutive dims] and transposes it in registers (one v_perm_b32 per dword), as
+// the prefill attention does for V.  Block i of a wave's output then holds dims 8 lane + i: a lane ends
+// with 32 consecutive dims of its own sequence, i.e. two of the 16-byte pieces of the operand layout.
+// The row maximum (all 576 dims, rope included) crosses the four waves through LDS.
+constexpr int kMlaAbsorbTiles = 1;   // tiles of 16 sequences per workgroup (at most 4: wave t brings tile t's rope dims)
+struct MlaAbsorbArgs {
+  const void* q_nope;   // [B, H, P]
+  int64_t qn_sb, qn_sh;
+  const void* w;        // W_UK_T [H, P, 512], dims contiguous
+  int64_t w_sh, w_sp;
+  const void* q_pe;     // [B, H, 64]
+  int64_t pe_sb, pe_sh;
+  uint8_t* q_ops;
+  float* q_scale;
+  int head_groups, num_heads, num_seqs, ksteps;   // ksteps = P / 32
+};
+
+// KSTEPS = P / 32 when known at compile time (the loop is unrolled and every load of W is in flight at
+// once: the kernel is one memory round trip long), 0 = read it from the arguments.
+template <int QDT, int KSTEPS>
+__global__ __launch_bounds__(256) void mla_absorb_q_kernel(MlaAbsorbArgs a) {
+  constexpr int NB = kMlaAbsorbTiles;
+  __shared__ float part_max[4][NB][16];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int c = lane & 15, g = lane >> 4;
+  const int head = blockIdx.x, b0 = blockIdx.y * (16 * NB);
+  const bool head_ok = head < a.num_heads;
+  const int hsrc = head_ok ? head : 0;
+  floatx4 acc[NB][8];
+#pragma unroll
+  for (int t = 0; t < NB; ++t)
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[t][i] = (floatx4){0.f, 0.f, 0.f, 0.f};
+  int brow[NB];
+#pragma unroll
+  for (int t = 0; t < NB; ++t) brow[t] = min(b0 + 16 * t + c, a.num_seqs - 1);   // rows past the end: a copy, not written
+  const uint16_t* wp = static_cast<const uint16_t*>(a.w) + (int64_t)hsrc * a.w_sh + (int64_t)(8 * g) * a.w_sp + 128 * wave + 8 * c;
+  const uint16_t* qp = static_cast<const uint16_t*>(a.q_nope) + (int64_t)hsrc * a.qn_sh + 8 * g;
+  auto step = [&](const u32x4 (&rows)[8], const u32x4 (&qop)[NB]) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const uint32_t sel = (i & 1) ? kPermHighHalves : kPermLowHalves;
+      u32x4 wt;
+      wt.x = perm(rows[1][i >> 1], rows[0][i >> 1], sel);
+      wt.y = perm(rows[3][i >> 1], rows[2][i >> 1], sel);
+      wt.z = perm(rows[5][i >> 1], rows[4][i >> 1], sel);
+      wt.w = perm(rows[7][i >> 1], rows[6][i >> 1], sel);
+#pragma unroll
+      for (int t = 0; t < NB; ++t) acc[t][i] = mfma16<QDT>(wt, qop[t], acc[t][i]);
+    }
+  };
+  if constexpr (KSTEPS > 0) {
+    // every load of the kernel first, then the arithmetic
+    u32x4 rows[KSTEPS][8], qop[KSTEPS][NB];
+#pragma unroll
+    for (int s = 0; s < KSTEPS; ++s) {
+#pragma unroll
+      for (int t = 0; t < NB; ++t) qop[s][t] = *reinterpret_cast<const u32x4_a4*>(qp + (int64_t)brow[t] * a.qn_sb + 32 * s);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) rows[s][j] = *reinterpret_cast<const u32x4*>(wp + (int64_t)(32 * s + j) * a.w_sp);
+    }
+    __builtin_amdgcn_sched_barrier(0);   // keep the scheduler from sinking the loads back to their uses
+#pragma unroll
+    for (int s = 0; s < KSTEPS; ++s) step(rows[s], qop[s]);
+  } else {
+    for (int s = 0; s < a.ksteps; ++s) {
+      u32x4 rows[8], qop[NB];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) rows[j] = *reinterpret_cast<const u32x4*>(wp + (int64_t)(32 * s + j) * a.w_sp);
+#pragma unroll
+      for (int t = 0; t < NB; ++t) qop[t] = *reinterpret_cast<const u32x4_a4*>(qp + (int64_t)brow[t] * a.qn_sb + 32 * s);
+      step(rows, qop);
+    }
+  }
+  // lane (sequence c, quarter g) of wave w holds dims 128 w + 32 g + 8 r + i of its sequence in acc[t][i][r]
+  float pe[16];   // wave t also brings the rope dims 16 g .. 16 g + 15 of tile t
+  {
+    const int t = wave < NB ? wave : 0;
+    const uint16_t* pp = static_cast<const uint16_t*>(a.q_pe) + (int64_t)brow[t] * a.pe_sb + (int64_t)hsrc * a.pe_sh + 16 * g;
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const u32x4 v = *reinterpret_cast<const u32x4_a4*>(pp + 8 * h);
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        const uint32_t e = v[w];
+        if constexpr (QDT == KVQ_BF16) {
+          pe[8 * h + 2 * w] = as_f32(e << 16);
+          pe[8 * h + 2 * w + 1] = as_f32(e & 0xffff0000u);
+        } else {
+          const half2_t hh = __builtin_bit_cast(half2_t, e);
+          pe[8 * h + 2 * w] = (float)hh.x;
+          pe[8 * h + 2 * w + 1] = (float)hh.y;
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int t = 0; t < NB; ++t) {
+    float amax = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) amax = fmaxf(amax, fabsf(acc[t][i][r]));
+    if (wave == t) {
+#pragma unroll
+      for (int j = 0; j < 16; ++j) amax = fmaxf(amax, fabsf(pe[j]));
+    }
+    amax = max_over_quarters(amax);
+    if (g == 0) part_max[wave][t][c] = amax;
+  }
+  __syncthreads();
+  const int hgroup = head >> 4, hc = head & 15;
+#pragma unroll
+  for (int t = 0; t < NB; ++t) {
+    const int b = b0 + 16 * t + c;
+    if (b >= a.num_seqs) continue;
+    float amax = fmaxf(fmaxf(part_max[0][t][c], part_max[1][t][c]), fmaxf(part_max[2][t][c], part_max[3][t][c]));
+    amax = head_ok ? fminf(amax, 3.0e38f) : 0.f;   // heads past the end contribute zero columns
+    const float s1 = amax > 0.f ? amax / 127.0f : 1.0f;
+    const int64_t qblock = (int64_t)b * a.head_groups + hgroup;
+    u32x4* qdst = reinterpret_cast<u32x4*>(a.q_ops + qblock * (kMlaQOps * kWave * 16)) + hc;
+    // the lane's 32 dims are the 16-dim pieces u = 0, 1: k-step kk = 2 w + g / 2, piece 2 (g % 2) + u of it
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      float f[16];
+#pragma unroll
+      for (int j = 0; j < 16; ++j) f[j] = acc[t][j & 7][2 * u + (j >> 3)];
+      u32x4 ta, tb;
+      mla_two_int8_terms(f, s1, head_ok, ta, tb);
+      const int kk = 2 * wave + (g >> 1), piece = 2 * (g & 1) + u;
+      qdst[(2 * kk) * kWave + 16 * piece] = ta;
+      qdst[(2 * kk + 1) * kWave + 16 * piece] = tb;
+    }
+    if (wave == t) {
+      u32x4 ta, tb;
+      mla_two_int8_terms(pe, s1, head_ok, ta, tb);
+      qdst[(2 * (kMlaKSteps8 - 1)) * kWave + 16 * g] = ta;
+      qdst[(2 * (kMlaKSteps8 - 1) + 1) * kWave + 16 * g] = tb;
+      if (g == 0) a.q_scale[qblock * 16 + hc] = s1;
+    }
+  }
 }
 
 // FULL: every 128-head block of the launch has its eight head tiles (num_heads a multiple of 128)
@@ -678,31 +835,17 @@ static int mla_prepare_device() {
 
 }  // namespace kvq
 
-extern "C" {
-
-size_t kvq_mla_decode_workspace_bytes(int max_num_seqs, int num_heads, int kv_lora_rank) {
-  if (max_num_seqs <= 0 || num_heads <= 0 || kv_lora_rank <= 0) return 0;
-  if (kvq::mla_prepare_device() != KVQ_OK) return 0;
-  // sequences x splits stays below max(2 x resident workgroups per head group, sequences)
-  const size_t groups = ((size_t)num_heads + 127) / 128;
-  size_t items = 2 * (size_t)kvq::num_cus() / groups;
-  if (items < (size_t)max_num_seqs) items = (size_t)max_num_seqs;
-  const size_t heads_padded = ((size_t)num_heads + 15) / 16 * 16;
-  // split states (fp16 outputs + fp32 lse) and, per sequence, Q as two int8 terms + one scale per head
-  return items * heads_padded * ((size_t)kv_lora_rank * sizeof(uint16_t) + sizeof(float)) +
-         (size_t)max_num_seqs * heads_padded * ((size_t)kvq::kMlaQOps * 64 + sizeof(float));
-}
-
-int kvq_mla_decode_int8(void* out, int out_dtype, float* lse, const void* q, int q_dtype, int64_t q_stride_b,
-                        int64_t q_stride_h, const void* q_pe, int64_t q_pe_stride_b, int64_t q_pe_stride_h,
-                        const void* cache, const kvq_mla_geom* geom,
-                        const int32_t* block_table, int64_t bt_stride, const int32_t* seq_lens, int num_seqs,
-                        int num_heads, float scale, void* workspace, size_t workspace_bytes,
-                        kvq_stream_t stream) {
+// Both entry points: `absorb` NULL = q holds the absorbed query (prepared by mla_quant_q_kernel), else q
+// is unused and the absorb kernel prepares the operands from (q_nope, W_UK_T, q_pe).
+static int mla_decode_run(const char* op, void* out, int out_dtype, float* lse, const void* q, int q_dtype,
+                          int64_t q_stride_b, int64_t q_stride_h, const void* q_pe, int64_t q_pe_stride_b,
+                          int64_t q_pe_stride_h, kvq::MlaAbsorbArgs* absorb, const void* cache,
+                          const kvq_mla_geom* geom, const int32_t* block_table, int64_t bt_stride,
+                          const int32_t* seq_lens, int num_seqs, int num_heads, float scale, void* workspace,
+                          size_t workspace_bytes, kvq_stream_t stream) {
   using namespace kvq;
-  const char* op = "mla_decode_int8";
   KVQ_REQUIRE(geom != nullptr, "%s: geom is NULL", op);
-  KVQ_REQUIRE(out && q && cache && block_table && seq_lens, "%s: NULL pointer", op);
+  KVQ_REQUIRE(out && (q || absorb) && cache && block_table && seq_lens, "%s: NULL pointer", op);
   KVQ_REQUIRE(num_seqs > 0 && num_seqs <= 65535 && num_heads > 0, "%s: num_seqs / num_heads out of range", op);
   KVQ_REQUIRE(((uintptr_t)out % 16) == 0, "%s: out must be 16-byte aligned", op);
   const kvq_mla_geom& g = *geom;
@@ -715,7 +858,7 @@ int kvq_mla_decode_int8(void* out, int out_dtype, float* lse, const void* q, int
   const int qsz = q_dtype == KVQ_F32 ? 4 : 2;
   KVQ_REQUIRE(((uintptr_t)q % 4) == 0 && (q_stride_b * qsz) % 4 == 0 && (q_stride_h * qsz) % 4 == 0,
               "%s: q rows must be 4-byte aligned", op);
-  if (q_pe == nullptr) {   // joined [B, H, 576] rows
+  if (q_pe == nullptr && absorb == nullptr) {   // joined [B, H, 576] rows
     q_pe = static_cast<const char*>(q) + (size_t)kMlaR * qsz;
     q_pe_stride_b = q_stride_b;
     q_pe_stride_h = q_stride_h;
@@ -754,15 +897,33 @@ int kvq_mla_decode_int8(void* out, int out_dtype, float* lse, const void* q, int
   hipStream_t s = as_stream(stream);
   dim3 grid(splits, num_seqs, (num_heads + 127) / 128);
   if (int e = mla_prepare_device()) return e;
-  dim3 qgrid(num_seqs, head_groups);
+  if (absorb != nullptr) {
+    absorb->q_ops = a.q_ops;
+    absorb->q_scale = a.q_scale;
+    absorb->head_groups = head_groups;
+    absorb->num_heads = num_heads;
+    absorb->num_seqs = num_seqs;
+    dim3 agrid(head_groups * 16, (num_seqs + 16 * kMlaAbsorbTiles - 1) / (16 * kMlaAbsorbTiles));
+#define KVQ_MLAA(T, K) hipLaunchKernelGGL((mla_absorb_q_kernel<T, K>), agrid, dim3(256), 0, s, *absorb)
+    if (q_dtype == KVQ_BF16) {
+      if (absorb->ksteps == 4) KVQ_MLAA(KVQ_BF16, 4);
+      else KVQ_MLAA(KVQ_BF16, 0);
+    } else {
+      if (absorb->ksteps == 4) KVQ_MLAA(KVQ_F16, 4);
+      else KVQ_MLAA(KVQ_F16, 0);
+    }
+#undef KVQ_MLAA
+  } else {
+    dim3 qgrid(num_seqs, head_groups);
 #define KVQ_MLAQ(T) hipLaunchKernelGGL((mla_quant_q_kernel<T>), qgrid, dim3(256), 0, s, a)
-  switch (q_dtype) {
-    case KVQ_F32: KVQ_MLAQ(KVQ_F32); break;
-    case KVQ_BF16: KVQ_MLAQ(KVQ_BF16); break;
-    case KVQ_F16: KVQ_MLAQ(KVQ_F16); break;
-    default: return fail(KVQ_EINVAL, "%s: unknown q_dtype %d", op, q_dtype);
-  }
+    switch (q_dtype) {
+      case KVQ_F32: KVQ_MLAQ(KVQ_F32); break;
+      case KVQ_BF16: KVQ_MLAQ(KVQ_BF16); break;
+      case KVQ_F16: KVQ_MLAQ(KVQ_F16); break;
+      default: return fail(KVQ_EINVAL, "%s: unknown q_dtype %d", op, q_dtype);
+    }
 #undef KVQ_MLAQ
+  }
   if (int e = check_hip(hipGetLastError(), "mla_decode_int8 query launch")) return e;
   if (head_groups % 8 == 0)
     hipLaunchKernelGGL(mla_decode_kernel<true>, grid, dim3(kMlaThreads), kMlaLdsBytes, s, a);
@@ -782,6 +943,64 @@ int kvq_mla_decode_int8(void* out, int out_dtype, float* lse, const void* q, int
   }
 #undef KVQ_MLAR
   return check_hip(hipGetLastError(), "mla_decode_int8 reduce launch");
+}
+
+extern "C" {
+
+size_t kvq_mla_decode_workspace_bytes(int max_num_seqs, int num_heads, int kv_lora_rank) {
+  if (max_num_seqs <= 0 || num_heads <= 0 || kv_lora_rank <= 0) return 0;
+  if (kvq::mla_prepare_device() != KVQ_OK) return 0;
+  // sequences x splits stays below max(2 x resident workgroups per head group, sequences)
+  const size_t groups = ((size_t)num_heads + 127) / 128;
+  size_t items = 2 * (size_t)kvq::num_cus() / groups;
+  if (items < (size_t)max_num_seqs) items = (size_t)max_num_seqs;
+  const size_t heads_padded = ((size_t)num_heads + 15) / 16 * 16;
+  // split states (fp16 outputs + fp32 lse) and, per sequence, Q as two int8 terms + one scale per head
+  return items * heads_padded * ((size_t)kv_lora_rank * sizeof(uint16_t) + sizeof(float)) +
+         (size_t)max_num_seqs * heads_padded * ((size_t)kvq::kMlaQOps * 64 + sizeof(float));
+}
+
+int kvq_mla_decode_int8(void* out, int out_dtype, float* lse, const void* q, int q_dtype, int64_t q_stride_b,
+                        int64_t q_stride_h, const void* q_pe, int64_t q_pe_stride_b, int64_t q_pe_stride_h,
+                        const void* cache, const kvq_mla_geom* geom,
+                        const int32_t* block_table, int64_t bt_stride, const int32_t* seq_lens, int num_seqs,
+                        int num_heads, float scale, void* workspace, size_t workspace_bytes,
+                        kvq_stream_t stream) {
+  return mla_decode_run("mla_decode_int8", out, out_dtype, lse, q, q_dtype, q_stride_b, q_stride_h, q_pe, q_pe_stride_b,
+                        q_pe_stride_h, nullptr, cache, geom, block_table, bt_stride, seq_lens, num_seqs, num_heads,
+                        scale, workspace, workspace_bytes, stream);
+}
+
+int kvq_mla_decode_absorb_int8(void* out, int out_dtype, float* lse, const void* q_nope, int q_dtype,
+                               int64_t qn_stride_b, int64_t qn_stride_h, int nope_dim, const void* w_uk_t,
+                               int64_t w_stride_h, int64_t w_stride_p, const void* q_pe, int64_t q_pe_stride_b,
+                               int64_t q_pe_stride_h, const void* cache, const kvq_mla_geom* geom,
+                               const int32_t* block_table, int64_t bt_stride, const int32_t* seq_lens,
+                               int num_seqs, int num_heads, float scale, void* workspace, size_t workspace_bytes,
+                               kvq_stream_t stream) {
+  using namespace kvq;
+  const char* op = "mla_decode_absorb_int8";
+  KVQ_REQUIRE(q_nope && w_uk_t && q_pe, "%s: NULL pointer", op);
+  KVQ_REQUIRE(q_dtype == KVQ_BF16 || q_dtype == KVQ_F16, "%s: q_nope, W_UK_T and q_pe must be bf16 or fp16 (dtype %d)", op, q_dtype);
+  KVQ_REQUIRE(nope_dim > 0 && nope_dim % 32 == 0, "%s: qk_nope_head_dim %d must be a multiple of 32", op, nope_dim);
+  KVQ_REQUIRE(((uintptr_t)w_uk_t % 16) == 0 && w_stride_h % 8 == 0 && w_stride_p % 8 == 0 && w_stride_p >= kMlaR,
+              "%s: W_UK_T rows must be 16-byte aligned and hold 512 contiguous dims", op);
+  KVQ_REQUIRE(((uintptr_t)q_nope % 4) == 0 && qn_stride_b % 2 == 0 && qn_stride_h % 2 == 0 && ((uintptr_t)q_pe % 4) == 0 &&
+                  q_pe_stride_b % 2 == 0 && q_pe_stride_h % 2 == 0, "%s: q_nope / q_pe rows must be 4-byte aligned", op);
+  MlaAbsorbArgs ab{};
+  ab.q_nope = q_nope;
+  ab.qn_sb = qn_stride_b;
+  ab.qn_sh = qn_stride_h;
+  ab.w = w_uk_t;
+  ab.w_sh = w_stride_h;
+  ab.w_sp = w_stride_p;
+  ab.q_pe = q_pe;
+  ab.pe_sb = q_pe_stride_b;
+  ab.pe_sh = q_pe_stride_h;
+  ab.ksteps = nope_dim / 32;
+  return mla_decode_run(op, out, out_dtype, lse, nullptr, q_dtype, 0, 0, q_pe, q_pe_stride_b, q_pe_stride_h, &ab, cache,
+                        geom, block_table, bt_stride, seq_lens, num_seqs, num_heads, scale, workspace, workspace_bytes,
+                        stream);
 }
 
 }  // extern "C"

@@ -23,10 +23,6 @@
 
 namespace kvq {
 
-typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
-typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
-typedef float floatx2 __attribute__((ext_vector_type(2)));
-
 struct VarlenArgs {
   const void* q;
   const void* k_nope;
@@ -40,24 +36,6 @@ struct VarlenArgs {
   int causal;
   float scale_log2;
 };
-
-template <int DT>
-__device__ __forceinline__ floatx4 mfma16(u32x4 a, u32x4 b, floatx4 c) {
-  if constexpr (DT == KVQ_F16)
-    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, a), __builtin_bit_cast(half8_t, b), c, 0, 0, 0);
-  else
-    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
-}
-
-template <int DT>
-__device__ __forceinline__ uint32_t pack2(float a, float b) {
-  if constexpr (DT == KVQ_F16) {
-    return pack_half2(a, b);
-  } else {
-    const floatx2 f = {a, b};
-    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2_t));
-  }
-}
 
 template <int NDW>
 struct Words {
@@ -174,7 +152,7 @@ __global__ __launch_bounds__(256) void varlen_attn_kernel(VarlenArgs a) {
 #pragma unroll
     for (int i = 0; i < DPL; ++i) {
       u32x4 vt;
-      const uint32_t sel = (i & 1) ? 0x07060302u : 0x05040100u;
+      const uint32_t sel = (i & 1) ? kPermHighHalves : kPermLowHalves;
       vt.x = perm(vrow[1].w[i >> 1], vrow[0].w[i >> 1], sel);
       vt.y = perm(vrow[3].w[i >> 1], vrow[2].w[i >> 1], sel);
       vt.z = perm(vrow[5].w[i >> 1], vrow[4].w[i >> 1], sel);

@@ -71,6 +71,8 @@ SIGNATURES = {
     "kvq_mla_decode_workspace_bytes": (_sz, [_i, _i, _i]),
     "kvq_mla_decode_int8": (_i, [_vp, _i, _vp, _vp, _i, _i64, _i64, _vp, _i64, _i64, _vp, _mla_p, _vp, _i64, _vp,
                                  _i, _i, _f, _vp, _sz, _vp]),
+    "kvq_mla_decode_absorb_int8": (_i, [_vp, _i, _vp, _vp, _i, _i64, _i64, _i, _vp, _i64, _i64, _vp, _i64, _i64, _vp,
+                                        _mla_p, _vp, _i64, _vp, _i, _i, _f, _vp, _sz, _vp]),
     "kvq_concat_mla_q": (_i, [_vp, _i64, _i64, _vp, _i64, _i64, _vp, _i64, _i64, _i, _i64, _i, _i, _i, _vp]),
     "kvq_mla_prefill_attn": (_i, [_vp, _i, _i64, _i64, _vp, _i64, _i64, _vp, _i64, _vp, _i64, _i64, _vp, _vp, _i, _i,
                                   _i64, _i, _i, _i, _i, _f, _i, _vp, _i64, _i64, _vp, _vp]),

@@ -679,6 +679,42 @@ def mla_decode_int8(q, kv_cache: torch.Tensor, o: torch.Tensor, lse: torch.Tenso
     _C.check(rc, "mla_decode_int8")
 
 
+def mla_decode_absorb_int8(q_nope: torch.Tensor, W_UK_T: torch.Tensor, q_pe: torch.Tensor, kv_cache: torch.Tensor,
+                           o: torch.Tensor, lse: torch.Tensor | None, block_table: torch.Tensor,
+                           seq_lens: torch.Tensor, sm_scale: float, kv_lora_rank: int,
+                           workspace: torch.Tensor | None = None, geometry: MlaGeometry | None = None) -> None:
+    """``mla_decode_int8`` with the absorption ``ql_nope = bmm(q_nope, W_UK_T)`` of the MLA layer
+    (vllm_metax/model_executor/layers/attention/mla_attention.py:835-848) done inside the launch: q_nope
+    ``[B, H, P]``, W_UK_T ``[H, P, R]``, q_pe ``[B, H, rope]`` (bf16 or fp16, one dtype); the product is
+    written directly as the decode's int8 query operands.  o ``[B, H, R]``, lse ``[B, H]`` fp32 or None."""
+    dev = _require_cuda(q_nope, W_UK_T, q_pe, kv_cache, o, lse, block_table, seq_lens, workspace)
+    geom = geometry or mla_geometry(kv_cache, kv_lora_rank)
+    B, H, P = q_nope.shape
+    if tuple(W_UK_T.shape) != (H, P, geom.kv_lora_rank) or tuple(q_pe.shape) != (B, H, geom.rope_dim):
+        raise RuntimeError("W_UK_T must be [H, P, R] and q_pe [B, H, rope]")
+    if not (q_nope.dtype == W_UK_T.dtype == q_pe.dtype):
+        raise RuntimeError("q_nope, W_UK_T and q_pe must share a dtype")
+    if q_nope.stride(2) != 1 or W_UK_T.stride(2) != 1 or q_pe.stride(2) != 1:
+        raise RuntimeError("last dims must be contiguous")
+    if tuple(o.shape) != (B, H, geom.kv_lora_rank) or not o.is_contiguous():
+        raise RuntimeError("o must be contiguous [B, H, R]")
+    if seq_lens.dtype != torch.int32 or block_table.dtype != torch.int32 or block_table.stride(1) != 1:
+        raise RuntimeError("seq_lens and block_table must be int32")
+    if lse is not None and (lse.dtype != torch.float32 or tuple(lse.shape) != (B, H) or not lse.is_contiguous()):
+        raise RuntimeError("lse must be contiguous float32 [B, H]")
+    if workspace is None:
+        workspace = _default_workspace(dev, mla_decode_workspace_bytes(B, H, geom.kv_lora_rank))
+    g = geom.as_struct()
+    with _on_device(dev):
+        rc = _C.load().kvq_mla_decode_absorb_int8(
+            _ptr(o), _dtype_code(o, "o"), _ptr(lse), _ptr(q_nope), _dtype_code(q_nope, "q_nope"), q_nope.stride(0),
+            q_nope.stride(1), P, _ptr(W_UK_T), W_UK_T.stride(0), W_UK_T.stride(1), _ptr(q_pe), q_pe.stride(0),
+            q_pe.stride(1), ctypes.c_void_p(geom.base_ptr), ctypes.byref(g), _ptr(block_table), block_table.stride(0),
+            _ptr(seq_lens), B, H, float(sm_scale), _ptr(workspace), workspace.numel() * workspace.element_size(),
+            _stream(dev))
+    _C.check(rc, "mla_decode_absorb_int8")
+
+
 def concat_mla_q(ql_nope: torch.Tensor, q_pe: torch.Tensor, q_out: torch.Tensor) -> None:
     """``q_out[..., :R] = ql_nope; q_out[..., R:] = q_pe``: the reference's ``ops.concat_mla_q``
     (csrc/libtorch_stable/cache_kernels.cu:1740-1783; call site

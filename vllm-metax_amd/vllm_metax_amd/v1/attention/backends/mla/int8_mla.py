@@ -370,10 +370,11 @@ class Int8MLADecodeCaller:
     (vllm_metax/model_executor/layers/attention/mla_attention.py:833-848, 857, 874, 902,
     1087-1110), for the plain (unquantised-weight) branch: Q absorption
     ``bmm(q_nope [N, B, P], W_UK_T [N, P, L])``, the decode, and the V up-projection
-    ``bmm(o [N, B, L], W_UV [N, L, V])``.  The two products are library GEMMs, as they are there.
-    What this path changes is the hand-off: the ``(ql_nope, q_pe)`` pair goes to the decode as the
-    strided views the GEMM leaves -- neither the transposed copy nor the concatenation is made --
-    and the decode's output feeds the second GEMM as a view as well."""
+    ``bmm(o [N, B, L], W_UV [N, L, V])``.  The absorption runs inside the decode launch
+    (``kvq_mla_decode_absorb_int8``): its product lands in the decode's int8 operand layout and is
+    never stored in the activation type.  The up-projection stays the library GEMM it is in the
+    reference and reads the decode's output as a strided view, without a transposed copy.  fp32
+    activations (not a serving dtype) take the two-step path ``absorb_q`` + ``forward_mqa``."""
 
     def __init__(self, impl: Int8MLAImpl, W_UK_T: torch.Tensor, W_UV: torch.Tensor) -> None:
         N, P, L = W_UK_T.shape
@@ -388,7 +389,8 @@ class Int8MLADecodeCaller:
         self.v_head_dim = W_UV.shape[2]
 
     def absorb_q(self, mqa_q_nope: torch.Tensor) -> torch.Tensor:
-        """``[B, N, P]`` -> ``[B, N, L]`` (a transposed view of the ``[N, B, L]`` product)."""
+        """``[B, N, P]`` -> ``[B, N, L]`` as the library GEMM (a transposed view of the ``[N, B, L]``
+        product): the separate first step of the reference, kept for fp32 and for comparison."""
         q = mqa_q_nope.transpose(0, 1)                       # (N, B, P)
         ql = q.new_empty((self.num_heads, q.shape[1], self.kv_lora_rank))
         torch.bmm(q, self.W_UK_T, out=ql)
@@ -400,12 +402,29 @@ class Int8MLADecodeCaller:
         out = out.view(-1, self.num_heads, self.v_head_dim)
         torch.bmm(x, self.W_UV, out=out.transpose(0, 1))
 
+    def decode_absorbed(self, mqa_q_nope: torch.Tensor, mqa_q_pe: torch.Tensor, kv_cache: torch.Tensor, attn_metadata):
+        """Absorption + decode in one launch; returns ``(o [B, N, L], lse [B, N])`` like ``forward_mqa``."""
+        impl = self.impl
+        B = mqa_q_nope.shape[0]
+        o_buf, lse_buf = getattr(attn_metadata, "decode_out", None), getattr(attn_metadata, "decode_lse", None)
+        if o_buf is not None and lse_buf is not None and o_buf.dtype == mqa_q_nope.dtype and o_buf.shape[0] >= B \
+                and o_buf.shape[1] == self.num_heads and o_buf.shape[2] == self.kv_lora_rank:
+            o, lse = o_buf[:B], lse_buf[:B]
+        else:
+            o = torch.empty((B, self.num_heads, self.kv_lora_rank), dtype=mqa_q_nope.dtype, device=mqa_q_nope.device)
+            lse = torch.empty((B, self.num_heads), dtype=torch.float32, device=mqa_q_nope.device)
+        ops.mla_decode_absorb_int8(mqa_q_nope, self.W_UK_T, mqa_q_pe, kv_cache, o, lse, attn_metadata.decode.block_table,
+                                   attn_metadata.decode.seq_lens, impl.scale, self.kv_lora_rank,
+                                   workspace=getattr(attn_metadata, "workspace", None), geometry=impl._geom(kv_cache))
+        return o, lse
+
     def forward_decode(self, mqa_q_nope: torch.Tensor, mqa_q_pe: torch.Tensor, kv_cache: torch.Tensor,
                        attn_metadata, out: torch.Tensor):
         """q_nope ``[B, N, P]``, q_pe ``[B, N, rope]`` (already rotated), writes ``out [B, N * V]``;
         returns the decode's ``lse [B, N]``."""
-        ql_nope = self.absorb_q(mqa_q_nope)
-        attn_out, lse = self.impl.forward_mqa((ql_nope, mqa_q_pe), kv_cache, attn_metadata)
+        if mqa_q_nope.dtype == torch.float32:
+            attn_out, lse = self.impl.forward_mqa((self.absorb_q(mqa_q_nope), mqa_q_pe), kv_cache, attn_metadata)
+        else:
+            attn_out, lse = self.decode_absorbed(mqa_q_nope, mqa_q_pe, kv_cache, attn_metadata)
         self.v_up_proj(attn_out, out)
         return lse
-
