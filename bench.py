@@ -516,6 +516,10 @@ def main():
     ap.add_argument("--soft-cap", type=float, default=0.0, help="GQA workloads: logits soft cap (0 = none)")
     ap.add_argument("--kv-dtype", choices=["int8", "fp8"], default="int8",
                     help="GQA decode workloads: code format of the cache (fp8 = e4m3fn per-token-head mode of the same layout)")
+    ap.add_argument("--kv-layout", choices=["HND", "NHD"], default="HND",
+                    help="GQA decode workloads: memory order of the cache tensor, both of which the reference defines "
+                         "(triton_attn.py:350-372, VLLM_KV_CACHE_LAYOUT).  HND keeps a head's records of a block back to "
+                         "back, which lets the decode loads stream; the default workload reports the other order too")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-fixed-8k", action="store_true",
                     help="default workload only: skip the extra fixed-context (64 x 8192) measurement")
@@ -534,7 +538,7 @@ def main():
         return mla_main(args, cfg, dev, ops)
     if cfg.get("mixed"):
         return mixed_main(args, cfg, dev, ops)
-    st = build_device_state(cfg, dev, args.layers)
+    st = build_device_state(cfg, dev, args.layers, layout=args.kv_layout)
     st["window"], st["softcap"] = args.sliding_window, args.soft_cap
     L = args.layers
     t = time_decode(cfg, st, args, ops)
@@ -557,7 +561,7 @@ def main():
         "data": "synthetic",
         "config": {"workload": args.workload, "batch": len(cfg["ctx"]), "sum_ctx": sum(cfg["ctx"]),
                    "q_heads": cfg["hq"], "kv_heads": cfg["hkv"], "head_dim": cfg["d"], "block_size": cfg["bs"],
-                   "pool_blocks": cfg["pool"], "layer_caches_rotated": L, "kv_layout": "NHD",
+                   "pool_blocks": cfg["pool"], "layer_caches_rotated": L, "kv_layout": args.kv_layout,
                    **({"kv_dtype": "fp8_per_token_head"} if args.kv_dtype == "fp8" else {}),
                    **({"sliding_window": args.sliding_window} if args.sliding_window else {}),
                    **({"soft_cap": args.soft_cap} if args.soft_cap else {})},
@@ -579,7 +583,7 @@ def main():
         # the shape the metric's wording names (every context 8192), same steps, in the same line
         cfg8 = make_batch("llama3_8b_decode_b64_ctx8k_fixed")
         cfg8["kv_dtype"] = "int8"
-        st8 = build_device_state(cfg8, dev, args.layers)
+        st8 = build_device_state(cfg8, dev, args.layers, layout=args.kv_layout)
         st8["window"], st8["softcap"] = 0, 0.0
         t8 = time_decode(cfg8, st8, args, ops)
         res["fixed_ctx_8192"] = {
@@ -590,6 +594,17 @@ def main():
             "roofline_frac": round(t8["attn_bytes"] / t8["attn_s"] / 1e9 / HBM_PEAK_GBPS, 4),
             "algorithmic_bytes_per_launch": t8["attn_bytes"]}
         del st8
+        # the same workload in the other memory order of the cache, same steps
+        other = "NHD" if args.kv_layout == "HND" else "HND"
+        sto = build_device_state(cfg, dev, args.layers, layout=other)
+        sto["window"], sto["softcap"] = 0, 0.0
+        to = time_decode(cfg, sto, args, ops)
+        res["other_kv_layout"] = {
+            "kv_layout": other, "value": round(to["value"], 1), "unit": "GB/s",
+            "pct_hbm_peak": round(100 * to["value"] / HBM_PEAK_GBPS, 2), "us_per_layer": round(to["step_s"] * 1e6, 2),
+            "attn_launch_us": round(to["attn_s"] * 1e6, 2),
+            "roofline_frac": round(to["attn_bytes"] / to["attn_s"] / 1e9 / HBM_PEAK_GBPS, 4)}
+        del sto
     if not args.no_cpu_baseline and args.kv_dtype == "int8":
         res["cpu_baseline"] = cpu_baseline(cfg, st, args.cpu_seconds)
     print(json.dumps(res))

@@ -141,7 +141,7 @@ __device__ __forceinline__ int active_workgroups(int64_t total, int num_wg) {
 // eight kv heads the 8 / HPW waves of a head take the tiles of a run in turn and their states are
 // folded together in LDS when the run ends, so a compute unit keeps eight tile streams in flight
 // whatever the head count and a sequence is cut into no more partial states than with eight heads.
-template <int D, int QDT, int HPW, bool CAP, int CODE>
+template <int D, int QDT, int HPW, bool CAP, int CODE, bool STREAM>
 __global__ __launch_bounds__(512) void paged_decode_streamk_kernel(StreamKArgs a) {
   using DTile = DecodeTile<D, QDT, kRuntimeDtype, CODE>;
   constexpr int NSUB = 8 / HPW;
@@ -191,7 +191,7 @@ __global__ __launch_bounds__(512) void paged_decode_streamk_kernel(StreamKArgs a
     const int t_end = __builtin_amdgcn_readfirstlane(t0 + u_end - kSetupUnits);
     if (t_begin < t_end) {  // else: this share ends inside the setup charge and holds no tile
       typename DTile::State st;
-      DTile::template run<CAP>(a.io, seq, row, len, first, t_begin, t_end, hkv, lane, lds[wave], st, sub, NSUB);
+      DTile::template run<CAP, STREAM>(a.io, seq, row, len, first, t_begin, t_end, hkv, lane, lds[wave], st, sub, NSUB);
       if constexpr (NSUB > 1) {
         if (sub != 0) DTile::dump_state(st, lane, lds[wave]);
         lds_barrier();
@@ -395,10 +395,14 @@ static int launch_streamk(const StreamKArgs& a, hipStream_t s) {
 #define KVQ_SK(H, C)                                                                                              \
   do {                                                                                                            \
     if (a.io.g.code_type == KVQ_CODE_FP8_E4M3)                                                                    \
-      hipLaunchKernelGGL((paged_decode_streamk_kernel<D, QDT, H, C, KVQ_CODE_FP8_E4M3>), grid, dim3(512), 0, s, a); \
+      hipLaunchKernelGGL((paged_decode_streamk_kernel<D, QDT, H, C, KVQ_CODE_FP8_E4M3, false>), grid, dim3(512), 0, s, a); \
+    else if (!C && stream)                                                                                        \
+      hipLaunchKernelGGL((paged_decode_streamk_kernel<D, QDT, H, false, KVQ_CODE_INT8, true>), grid, dim3(512), 0, s, a); \
     else                                                                                                          \
-      hipLaunchKernelGGL((paged_decode_streamk_kernel<D, QDT, H, C, KVQ_CODE_INT8>), grid, dim3(512), 0, s, a);     \
+      hipLaunchKernelGGL((paged_decode_streamk_kernel<D, QDT, H, C, KVQ_CODE_INT8, false>), grid, dim3(512), 0, s, a); \
   } while (0)
+  // a head's records of a block back to back (HND order): the tile loads may stream past the caches
+  const bool stream = a.io.g.stride_slot == 2 * (D + 4) && a.io.g.block_size >= 16;
   if (a.io.cap_c != 0.f) {
     switch (hpw) {
       case 8: KVQ_SK(8, true); break;
