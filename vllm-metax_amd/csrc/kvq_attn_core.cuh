@@ -168,6 +168,7 @@ struct KVTile {
   static constexpr int NLD = NCH / 4;      // wave-wide chunk loads per 16-token half
   u32x4 c[2][NLD];                         // chunk (n*64 + lane) of half 0 / half 1
   u32x2 tail0, tail1;                      // last 8 bytes of record (lane & 15) of half 0 / half 1
+  u32x4 e[2];                              // streamed loads only: chunk NLD*64 + (lane & 7), the run's last 128 bytes
 };
 
 template <int D>
@@ -203,6 +204,11 @@ struct LaneOffsets {
   uint32_t l_k;       // LDS: r*PITCH + g*16, K operand chunk of token r
   uint32_t l_v;       // LDS: 4g*PITCH + (D+4) + r*VB, V operand bytes of token 4g
   uint32_t l_sc;      // LDS: (lane & 31)*PITCH + (lane < 32 ? D : 2*D+4), the lane's scale
+  // streamed loads: where the 16-byte chunk n*64 + lane of a 16-record run lands in the window (its first 8
+  // bytes; the other 8 follow, or open the next row when bit n of l_flat_split is set)
+  uint32_t g_flat;    // HBM: 16 * lane
+  uint32_t l_flat[9];
+  uint32_t l_flat_split;
 };
 
 // CODE: what a code byte is (KVQ_CODE_INT8 or KVQ_CODE_FP8_E4M3).  An int8 code enters the MFMA as
@@ -237,6 +243,15 @@ struct DecodeTile {
     o.l_k = (uint32_t)(r * PITCH + g * 16);
     o.l_v = (uint32_t)(4 * g * PITCH + (D + 4) + r * VB);
     o.l_sc = (uint32_t)((lane & 31) * PITCH + (lane < 32 ? D : 2 * D + 4));
+    o.g_flat = (uint32_t)(16 * lane);
+    o.l_flat_split = 0;
+#pragma unroll
+    for (int n = 0; n <= NLD; ++n) {
+      const int q = n < NLD ? n * 64 + lane : NLD * 64 + (lane & 7);   // chunk of the run
+      const int rec = (16 * q) / R, off = 16 * q - rec * R;            // its record and the offset inside it
+      o.l_flat[n] = (uint32_t)(rec * PITCH + off);
+      if (off == R - 8) o.l_flat_split |= 1u << n;
+    }
     return o;
   }
 
@@ -349,14 +364,29 @@ struct DecodeTile {
 
   // Issue the HBM loads of one tile: 2*NLD chunk loads (lane n*64+l takes chunk (n*64+l) % NCH of
   // record (n*64+l) / NCH of the half) and the two 8-byte record tails.
-  // STREAM: the loads carry the non-temporal hint.  Right only where a head's records of a block lie
-  // back to back (the HND order: a wave then reads whole runs of 16 x 2(D+4) bytes and nothing it skips
-  // shares a cache line with what it reads): there the hint raises the achieved HBM rate by 8 %; in the
-  // NHD order, where the 128-byte lines at a record's ends belong half to a neighbouring head's wave, it
-  // makes both waves fetch them and costs 9 %.
+  // STREAM: for a cache in which a head's records of a block lie back to back (the HND order).  A half
+  // tile is then ONE run of 16 R bytes, read as aligned 16-byte chunks with the non-temporal hint (scales
+  // included: no 8-byte tail loads) -- measured on MI355X, reads of this shape reach 6.8 TB/s against 6.0
+  // without the hint.  The hint is wrong for the NHD order: there the 128-byte lines at a record's ends
+  // belong half to a neighbouring head's wave, a line that is not kept in L2 is fetched by both, and the
+  // rate drops by 9 %.
   template <bool STREAM = false>
   __device__ static void load_tile(const AttnIO& io, const Window& w, const LaneOffsets& lo, Tile& kv) {
     constexpr int AUX = STREAM ? 2 : 0;
+    if constexpr (STREAM) {
+      // the half's 16 records are one run of 16 R bytes: read it as R aligned 16-byte chunks, scales and all
+      // (NLD full wave-loads and the last 8 chunks, which every lane names so that the load is unconditional)
+      const uint32_t f = lo.g_flat;
+#pragma unroll
+      for (int n = 0; n < NLD; ++n) {
+        kv.c[0][n] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(w.r0, f, n * 1024, AUX));
+        kv.c[1][n] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(w.r1, f, n * 1024, AUX));
+      }
+      const uint32_t fe = (f & 127u) + NLD * 1024;
+      kv.e[0] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(w.r0, fe, 0, AUX));
+      kv.e[1] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(w.r1, fe, 0, AUX));
+      return;
+    }
     const int step = (64 / NCH) * (int)io.g.stride_slot;  // records advanced per wave-wide load
 #pragma unroll
     for (int n = 0; n < NLD; ++n) {
@@ -370,7 +400,32 @@ struct DecodeTile {
   // Drop a loaded tile into the wave's LDS window, one record per PITCH-byte row, then stage the
   // 64 scales (K scales pre-multiplied by scale*log2e, V scales by 2^8, capped so P~ stays finite).
   // After this the tile's registers are free for the next prefetch.
+  template <bool STREAM = false>
   __device__ static void stage(const Tile& kv, const LaneOffsets& lo, float sc_mul, int lane, uint8_t* lds) {
+    if constexpr (STREAM) {
+      // a chunk of the run is 8-byte aligned inside its record and may end one record and begin the next:
+      // two 8-byte writes each
+      auto put = [&](const u32x4& v, uint32_t at, bool split) __attribute__((always_inline)) {
+        *reinterpret_cast<u32x2*>(lds + at) = (u32x2){v.x, v.y};
+        *reinterpret_cast<u32x2*>(lds + at + (split ? 8 + (PITCH - R) : 8)) = (u32x2){v.z, v.w};
+      };
+#pragma unroll
+      for (int n = 0; n < NLD; ++n) {
+        const bool split = (lo.l_flat_split >> n) & 1;
+        put(kv.c[0][n], lo.l_flat[n], split);
+        put(kv.c[1][n], lo.l_flat[n] + 16 * PITCH, split);
+      }
+      if (lane < 8) {
+        const bool split = (lo.l_flat_split >> NLD) & 1;
+        put(kv.e[0], lo.l_flat[NLD], split);
+        put(kv.e[1], lo.l_flat[NLD] + 16 * PITCH, split);
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      stage_scales(lo, sc_mul, lane, lds);
+      return;
+    }
 #pragma unroll
     for (int n = 0; n < NLD; ++n) {
       *reinterpret_cast<u32x4*>(lds + lo.l_chunk + n * (64 / NCH) * PITCH) = kv.c[0][n];
@@ -538,7 +593,7 @@ struct DecodeTile {
     const LaneOffsets lo = lane_offsets(io.g, lane);
     const int32_t* bt_row = io.block_table + (int64_t)seq * io.bt_stride;
     const int rounds = (t_end - t_begin + nsub - 1) / nsub;
-    const int num_barriers = rounds / kSyncTiles;
+    const int num_barriers = STREAM ? 0 : rounds / kSyncTiles;
     int barriers = 0;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) st.o[dt] = (floatx4){0.f, 0.f, 0.f, 0.f};
@@ -561,7 +616,7 @@ struct DecodeTile {
       // steady loop below keeps a single, unmasked body
       if (t + nsub < t_end && t * kTile < first) {
         const Window w = window(io, nb, t + nsub, hkv);
-        stage(a, lo, sc_mul, lane, lds);
+        stage<STREAM>(a, lo, sc_mul, lane, lds);
         phase_fence();
         load_tile<STREAM>(io, w, lo, a);
         phase_fence();
@@ -570,16 +625,28 @@ struct DecodeTile {
         phase_fence();
         t += nsub;
         ++r;
-        if ((r & (kSyncTiles - 1)) == 0) {
+        if (!STREAM && (r & (kSyncTiles - 1)) == 0) {
           __builtin_amdgcn_s_barrier();
           ++barriers;
         }
       }
+      auto rendezvous = [&]() __attribute__((always_inline)) {
+        ++r;
+        // The waves of a workgroup read neighbouring records of the same tokens (one kv head each) or
+        // neighbouring tiles; the 128-byte lines at record boundaries are shared between them.  A
+        // rendezvous every few rounds keeps the waves within a few tiles of each other, so the second
+        // reader of such a line still finds it in L2 instead of fetching it from HBM again.  Streamed loads
+        // (whole runs per wave, nothing kept in L2) have no such lines to share and skip the rendezvous.
+        if (!STREAM && (r & (kSyncTiles - 1)) == 0) {
+          __builtin_amdgcn_s_barrier();
+          ++barriers;
+        }
+      };
       // steady state: the wave's next tile exists, so the refill is unconditional and tile t does not
       // end the sequence
       while (t + nsub < t_end) {
         const Window w = window(io, nb, t + nsub, hkv);
-        stage(a, lo, sc_mul, lane, lds);
+        stage<STREAM>(a, lo, sc_mul, lane, lds);
         phase_fence();
         load_tile<STREAM>(io, w, lo, a);
         phase_fence();
@@ -587,17 +654,9 @@ struct DecodeTile {
         compute<false, CAP>(io, lo, qb, s_init, len, first, t, lane, lds, st);
         phase_fence();
         t += nsub;
-        ++r;
-        // The waves of a workgroup read neighbouring records of the same tokens (one kv head each) or
-        // neighbouring tiles; the 128-byte lines at record boundaries are shared between them.  A
-        // rendezvous every few rounds keeps the waves within a few tiles of each other, so the second
-        // reader of such a line still finds it in L2 instead of fetching it from HBM again.
-        if ((r & (kSyncTiles - 1)) == 0) {
-          __builtin_amdgcn_s_barrier();
-          ++barriers;
-        }
+        rendezvous();
       }
-      stage(a, lo, sc_mul, lane, lds);
+      stage<STREAM>(a, lo, sc_mul, lane, lds);
       compute_any<CAP>(io, lo, qb, s_init, len, first, t, lane, lds, st);
     }
     // the rendezvous count is the same for every wave of the workgroup, whatever its share of the tiles
