@@ -394,15 +394,21 @@ static int launch_streamk(const StreamKArgs& a, hipStream_t s) {
   dim3 grid(a.num_wg, (hkv + hpw - 1) / hpw);
 #define KVQ_SK(H, C)                                                                                              \
   do {                                                                                                            \
-    if (a.io.g.code_type == KVQ_CODE_FP8_E4M3)                                                                    \
-      hipLaunchKernelGGL((paged_decode_streamk_kernel<D, QDT, H, C, KVQ_CODE_FP8_E4M3, false>), grid, dim3(512), 0, s, a); \
-    else if (!C && stream)                                                                                        \
+    if (a.io.g.code_type == KVQ_CODE_FP8_E4M3) {                                                                  \
+      if (!C && stream)                                                                                           \
+        hipLaunchKernelGGL((paged_decode_streamk_kernel<D, QDT, H, false, KVQ_CODE_FP8_E4M3, true>), grid, dim3(512), 0, s, a); \
+      else                                                                                                        \
+        hipLaunchKernelGGL((paged_decode_streamk_kernel<D, QDT, H, C, KVQ_CODE_FP8_E4M3, false>), grid, dim3(512), 0, s, a); \
+    } else if (!C && stream) {                                                                                    \
       hipLaunchKernelGGL((paged_decode_streamk_kernel<D, QDT, H, false, KVQ_CODE_INT8, true>), grid, dim3(512), 0, s, a); \
-    else                                                                                                          \
+    } else {                                                                                                      \
       hipLaunchKernelGGL((paged_decode_streamk_kernel<D, QDT, H, C, KVQ_CODE_INT8, false>), grid, dim3(512), 0, s, a); \
+    }                                                                                                             \
   } while (0)
   // a head's records of a block back to back (HND order): the tile loads may stream past the caches
-  const bool stream = a.io.g.stride_slot == 2 * (D + 4) && a.io.g.block_size >= 16;
+  // (not at head size 256, where the second register image of a 16 KB tile costs more than the loads gain:
+  // 293 against 279 us on 64 x 1k-8k tokens)
+  const bool stream = D <= 128 && a.io.g.stride_slot == 2 * (D + 4) && a.io.g.block_size >= 16;
   if (a.io.cap_c != 0.f) {
     switch (hpw) {
       case 8: KVQ_SK(8, true); break;
