@@ -406,8 +406,7 @@ static int launch_streamk(const StreamKArgs& a, hipStream_t s) {
     }                                                                                                             \
   } while (0)
   // a head's records of a block back to back (HND order): the tile loads may stream past the caches
-  // (not at head size 256, where the second register image of a 16 KB tile costs more than the loads gain:
-  // 293 against 279 us on 64 x 1k-8k tokens)
+  // (not at head size 256, where it measured slower: 293 against 279 us on 64 x 1k-8k tokens)
   const bool stream = D <= 128 && a.io.g.stride_slot == 2 * (D + 4) && a.io.g.block_size >= 16;
   if (a.io.cap_c != 0.f) {
     switch (hpw) {
