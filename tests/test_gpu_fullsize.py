@@ -28,10 +28,10 @@ def _tables(ctx, bs, pool, g):
     return bt
 
 
-def _fill_gqa(dev, ctx, bt, hkv, d, bs, pool, outlier=False):
+def _fill_gqa(dev, ctx, bt, hkv, d, bs, pool, outlier=False, layout="NHD"):
     """Cache filled on the GPU through the quantise-on-write kernel (bit-exactness of that kernel
     is its own test); sources N(0,1) bf16, optionally with 1 % of the channels scaled x20."""
-    kv = L.allocate_kv_cache(pool, bs, hkv, d, device=dev, layout="NHD", fill=0)
+    kv = L.allocate_kv_cache(pool, bs, hkv, d, device=dev, layout=layout, fill=0)
     k, v = L.key_value_views(kv)
     ks, vs = L.scale_views(kv)
     ks.fill_(1.0)
@@ -55,10 +55,10 @@ def _fill_gqa(dev, ctx, bt, hkv, d, bs, pool, outlier=False):
     return kv, k, v, ks, vs
 
 
-def _gather_to_cpu(kv, bt, seqs, ctx, hkv, d, bs):
+def _gather_to_cpu(kv, bt, seqs, ctx, hkv, d, bs, layout="NHD"):
     """The blocks of the chosen sequences as a small CPU cache with a renumbered block table."""
     per = [(ctx[i] + bs - 1) // bs for i in seqs]
-    cpu, _views, lay = T.cpu_cache(sum(per) + 1, bs, hkv, d, "NHD")
+    cpu, _views, lay = T.cpu_cache(sum(per) + 1, bs, hkv, d, layout)
     big = T.storage_bytes(kv).view(kv.shape[0], -1)
     small = T.storage_bytes(cpu).view(sum(per) + 1, -1)
     bt2 = torch.zeros((len(seqs), max(per)), dtype=torch.int32)
@@ -89,13 +89,14 @@ def _decode_both_ways(dev, q, k, v, ks, vs, bt, ctx, hq, hkv, d, bs, scale):
     return a, b, lse
 
 
-def test_config2_llama3_8b_b64_ctx1k_8k(gpu_device):
+@pytest.mark.parametrize("layout", ["NHD", "HND"])   # HND: the streamed run loads of the decode kernel
+def test_config2_llama3_8b_b64_ctx1k_8k(gpu_device, layout):
     dev = gpu_device
     hq, hkv, d, bs, pool = 32, 8, 128, 16, 40000
     g = torch.Generator().manual_seed(0)
     ctx = torch.randint(1024, 8193, (64,), generator=g).tolist()
     bt = _tables(ctx, bs, pool, g)
-    kv, k, v, ks, vs = _fill_gqa(dev, ctx, bt, hkv, d, bs, pool)
+    kv, k, v, ks, vs = _fill_gqa(dev, ctx, bt, hkv, d, bs, pool, layout=layout)
     q = torch.randn((64, hq, d), device=dev).to(torch.bfloat16)
     scale = 1 / math.sqrt(d)
     a, b, lse = _decode_both_ways(dev, q, k, v, ks, vs, bt, ctx, hq, hkv, d, bs, scale)
@@ -103,7 +104,7 @@ def test_config2_llama3_8b_b64_ctx1k_8k(gpu_device):
     T.assert_close_attn(a, b, atol=2e-3, rtol=2e-3, what="balanced split-K vs 512-token partitions")
     order = sorted(range(64), key=lambda i: ctx[i])
     seqs = [order[0], order[32], order[63]]
-    cpu, lay, bt2 = _gather_to_cpu(kv, bt, seqs, ctx, hkv, d, bs)
+    cpu, lay, bt2 = _gather_to_cpu(kv, bt, seqs, ctx, hkv, d, bs, layout)
     sl2 = torch.tensor([ctx[i] for i in seqs], dtype=torch.int32)
     want, want_lse = oracle.paged_attn(q[seqs].cpu(), T.storage_bytes(cpu), lay, bt2, sl2,
                                        torch.arange(4, dtype=torch.int32), scale, return_lse=True)
