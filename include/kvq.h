@@ -144,6 +144,12 @@ KVQ_API size_t kvq_paged_attn_workspace_bytes(int max_num_seqs, int num_q_heads,
  * 0 = no window.  softcap > 0: logits become softcap * tanh(scale * q.k / softcap)
  * (triton_attn.py:703; semantics as in the reference's test oracle,
  * tests/kernels/attention/test_triton_unified_attention.py:63-70); 0 = none.
+ *
+ * Value range: the weights enter the second product as fp16 numbers
+ * p * v_scale * 2^8, so a V row whose scale exceeds 255.8 (int8 codes: absmax
+ * above 32 500; fp8 codes: above 114 000) is attended as if its scale were 255.8.
+ * Small values need no care: with V of magnitude 1e-3 spread over 8192 keys the
+ * result is within 3e-4 relative of the fp32 result.
  */
 KVQ_API int kvq_paged_attn_int8(void* out, int out_dtype, int64_t out_stride_t, int64_t out_stride_h,
                         const void* q, int q_dtype, int64_t q_stride_t, int64_t q_stride_h,
