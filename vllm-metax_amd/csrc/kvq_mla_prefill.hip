@@ -4,20 +4,25 @@
 // the rope part k_pe [S, ROPE] shared by all heads -- so the concatenated [S, H, NOPE + ROPE] tensor is
 // never built.
 //
-// One wave owns 16 query rows of one (sequence, head) and walks the keys 32 at a time; nothing goes
-// through LDS.  Both products are computed transposed so that every per-row quantity is lane-local:
+// Workgroup = 128 query rows of one (sequence, head): 4 waves x 2 blocks of 16 rows.  The keys are walked 32
+// at a time; a tile's K rows (NOPE + ROPE wide) and V rows are brought into LDS once per workgroup
+// (registers in between, one tile ahead, double-buffered: one barrier per tile) and every wave feeds its two
+// row blocks from there, so a K or V byte is fetched from L2 once per 128 rows.  K rows are stored with
+// their 16-byte chunks xor-swizzled by the row number, which makes the operand reads (16 rows x the same
+// chunk) free of bank conflicts without padding.
+// Both products are computed transposed so that every per-row quantity is lane-local:
 //   S^T = K Q^T   A = K rows (lane = key, 8 consecutive d), B = Q (lane = query row): 16x16x32 MFMA of the
 //                 input type; a lane ends up with 8 keys of ITS query row, so the row maximum is a
 //                 reduction over the four quarter-waves and alpha / l stay in the lane.
 //   O^T = V^T P^T B = P~ straight from the S^T registers (k slot j of quarter g is key 16 (j / 4) + 4 g +
 //                 j % 4; any order works as long as V uses the same one).  A = V^T needs 8 keys of one
-//                 dim per lane while memory holds 8 dims of one key: each lane loads the slice
+//                 dim per lane while a V row holds 8 dims of one key together: each lane reads the slice
 //                 [its 8 keys] x [DV / 16 consecutive dims] and transposes it in registers with one
-//                 v_perm_b32 per output dword.  Output block i then holds dims (DV/16) * lane + i, which
-//                 leaves every lane with 4 runs of DV/16 consecutive dims of its own query row: 16-byte
-//                 stores.
+//                 v_perm_b32 per output dword (once per tile, for both row blocks).  Output block i then
+//                 holds dims (DV/16) * lane + i, which leaves every lane with 4 runs of DV/16 consecutive
+//                 dims of its own query row: 16-byte stores.
 // Masked keys (beyond the sequence, or above the causal diagonal, which is aligned to the END of the
-// keys as flash-attention does) get weight 0; their loads are clamped to the last valid key.
+// keys as flash-attention does) get weight 0; their rows are clamped copies of the last valid key.
 #include "kvq_attn_core.cuh"
 #include "kvq_internal.h"
 
@@ -66,127 +71,201 @@ __global__ __launch_bounds__(256) void varlen_attn_kernel(VarlenArgs a) {
   constexpr int KSN = NOPE / 32, KSR = ROPE / 32, KS = KSN + KSR;   // k-steps of the QK product
   constexpr int DPL = DV / 16;                                      // dims per lane and output block
   constexpr int VR = DPL / 2;                                       // dwords of one key's slice
+  constexpr int RB = 2;                                             // row blocks of 16 per wave
+  constexpr int KC = (NOPE + ROPE) / 8, KCN = NOPE / 8;             // 16-byte chunks of a K row / of its nope part
+  constexpr int VC = DV / 8;                                        // chunks of a V row
+  constexpr int K_BYTES = 32 * KC * 16, V_BYTES = 32 * VC * 16;
+  constexpr int KLD = (32 * KC + 255) / 256, VLD = (32 * VC + 255) / 256;   // chunk loads per thread and tile
   // fp16 weights are kept 2^8 larger so that small ones stay normal; l carries the same factor
   constexpr float kShift = DT == KVQ_F16 ? 8.f : 0.f;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  __shared__ __align__(16) uint8_t lds[2][K_BYTES + V_BYTES];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
   const int seq = blockIdx.z, head = blockIdx.y;
   const int q_begin = a.cu_q[seq], q_len = a.cu_q[seq + 1] - q_begin;
   const int k_begin = a.cu_k[seq], k_len = a.cu_k[seq + 1] - k_begin;
-  const int q0 = (blockIdx.x * 4 + wave) * 16;
-  if (q0 >= q_len) return;
+  // the last query blocks see the most keys under the causal mask: they are launched first
+  const int q0wg = ((int)gridDim.x - 1 - (int)blockIdx.x) * (64 * RB);
+  if (q0wg >= q_len) return;   // uniform over the workgroup
   const int c = lane & 15, g = lane >> 4;
-  const int qrow = min(q0 + c, q_len - 1);   // rows past the end compute on a copy and are not stored
-
-  u32x4 qop[KS];
-  {
-    const uint16_t* qp = static_cast<const uint16_t*>(a.q) + (int64_t)(q_begin + qrow) * a.q_st + (int64_t)head * a.q_sh + 8 * g;
-#pragma unroll
-    for (int s = 0; s < KS; ++s) qop[s] = *reinterpret_cast<const u32x4*>(qp + 32 * s);
-  }
-
   // key j is visible to query row i iff j <= i + (k_len - q_len)
   const int diag = k_len - q_len;
-  const int my_limit = a.causal ? max(0, min(k_len, q0 + c + diag + 1)) : k_len;
-  const int k_end = a.causal ? max(0, min(k_len, q0 + 15 + diag + 1)) : k_len;
-  const int num_tiles = (k_end + 31) / 32;
+  const int wg_rows_end = min(q_len, q0wg + 64 * RB);
+  const int wg_k_end = a.causal ? max(0, min(k_len, wg_rows_end - 1 + diag + 1)) : k_len;
+  const int num_tiles = (wg_k_end + 31) / 32;
 
-  floatx4 oacc[DPL];
+  // ---- the wave's rows
+  int q0[RB], my_limit[RB], blk_k_end[RB];
+  u32x4 qop[RB][KS];
 #pragma unroll
-  for (int i = 0; i < DPL; ++i) oacc[i] = (floatx4){0.f, 0.f, 0.f, 0.f};
-  float m = -INFINITY, l = 0.f;
+  for (int rb = 0; rb < RB; ++rb) {
+    q0[rb] = q0wg + (wave * RB + rb) * 16;
+    const int qrow = min(q0[rb] + c, q_len - 1);   // rows past the end compute on a copy and are not stored
+    const uint16_t* qp = static_cast<const uint16_t*>(a.q) + (int64_t)(q_begin + qrow) * a.q_st + (int64_t)head * a.q_sh + 8 * g;
+#pragma unroll
+    for (int s = 0; s < KS; ++s) qop[rb][s] = *reinterpret_cast<const u32x4*>(qp + 32 * s);
+    my_limit[rb] = a.causal ? max(0, min(k_len, q0[rb] + c + diag + 1)) : k_len;
+    blk_k_end[rb] = q0[rb] >= q_len ? 0 : (a.causal ? max(0, min(k_len, q0[rb] + 15 + diag + 1)) : k_len);
+  }
+  const int wave_tiles = (max(blk_k_end[0], blk_k_end[1]) + 31) / 32;   // tiles this wave has anything to do in
 
-  const uint16_t* kn_base = static_cast<const uint16_t*>(a.k_nope) + (int64_t)head * a.kn_sh + 8 * g;
-  const uint16_t* kpe_base = static_cast<const uint16_t*>(a.k_pe) + 8 * g;
-  const uint16_t* v_base = static_cast<const uint16_t*>(a.v) + (int64_t)head * a.v_sh + DPL * c;
+  floatx4 oacc[RB][DPL];
+  float m[RB], l[RB];
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) {
+#pragma unroll
+    for (int i = 0; i < DPL; ++i) oacc[rb][i] = (floatx4){0.f, 0.f, 0.f, 0.f};
+    m[rb] = -INFINITY;
+    l[rb] = 0.f;
+  }
 
+  // ---- cooperative tile copy: thread tid owns chunks tid + 256 i of the K tile and of the V tile
+  const uint16_t* kn_base = static_cast<const uint16_t*>(a.k_nope) + (int64_t)head * a.kn_sh;
+  const uint16_t* kpe_base = static_cast<const uint16_t*>(a.k_pe);
+  const uint16_t* v_base = static_cast<const uint16_t*>(a.v) + (int64_t)head * a.v_sh;
+  u32x4 kreg[KLD], vreg[VLD];
+  auto fetch = [&](int t) __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = 0; i < KLD; ++i) {
+      const int q = min(tid + 256 * i, 32 * KC - 1);
+      const int row = q / KC, ch = q - row * KC;
+      const int64_t krow = k_begin + min(t * 32 + row, k_len - 1);
+      const uint16_t* p = ch < KCN ? kn_base + krow * a.kn_st + 8 * ch : kpe_base + krow * a.kpe_st + 8 * (ch - KCN);
+      kreg[i] = *reinterpret_cast<const u32x4*>(p);
+    }
+#pragma unroll
+    for (int i = 0; i < VLD; ++i) {
+      const int q = min(tid + 256 * i, 32 * VC - 1);
+      const int row = q / VC, ch = q - row * VC;
+      const int64_t vrow = k_begin + min(t * 32 + row, k_len - 1);
+      vreg[i] = *reinterpret_cast<const u32x4*>(v_base + vrow * a.v_st + 8 * ch);
+    }
+  };
+  auto swz = [](int row, int ch) { return KC % 8 == 0 ? (ch ^ (row & 7)) : (ch ^ ((row >> 1) & 3)); };
+  auto drop = [&](uint8_t* buf) __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = 0; i < KLD; ++i) {
+      const int q = tid + 256 * i;
+      if (q < 32 * KC) {
+        const int row = q / KC, ch = q - row * KC;
+        *reinterpret_cast<u32x4*>(buf + (row * KC + swz(row, ch)) * 16) = kreg[i];
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < VLD; ++i) {
+      const int q = tid + 256 * i;
+      if (q < 32 * VC) *reinterpret_cast<u32x4*>(buf + K_BYTES + q * 16) = vreg[i];
+    }
+  };
+
+  if (num_tiles > 0) {
+    fetch(0);
+    drop(lds[0]);
+    __syncthreads();
+  }
   for (int t = 0; t < num_tiles; ++t) {
-    // ---- S^T = K Q^T for the tile's two blocks of 16 keys
-    floatx4 sacc[2];
+    const uint8_t* buf = lds[t & 1];
+    if (t + 1 < num_tiles) fetch(t + 1);
+    if (t < wave_tiles) {
+      // ---- S^T = K Q^T for the tile's two blocks of 16 keys, both row blocks off one operand read
+      floatx4 sacc[RB][2];
 #pragma unroll
-    for (int blk = 0; blk < 2; ++blk) {
-      const int64_t krow = k_begin + min(t * 32 + 16 * blk + c, k_len - 1);
-      const uint16_t* kn = kn_base + krow * a.kn_st;
-      const uint16_t* kp = kpe_base + krow * a.kpe_st;
-      floatx4 acc = {0.f, 0.f, 0.f, 0.f};
+      for (int rb = 0; rb < RB; ++rb) sacc[rb][0] = sacc[rb][1] = (floatx4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int s = 0; s < KSN; ++s) acc = mfma16<DT>(*reinterpret_cast<const u32x4*>(kn + 32 * s), qop[s], acc);
+      for (int blk = 0; blk < 2; ++blk) {
+        const int row = 16 * blk + c;
+        const uint8_t* krow = buf + row * (KC * 16);
 #pragma unroll
-      for (int s = 0; s < KSR; ++s) acc = mfma16<DT>(*reinterpret_cast<const u32x4*>(kp + 32 * s), qop[KSN + s], acc);
-      sacc[blk] = acc;
+        for (int s = 0; s < KS; ++s) {
+          const u32x4 ka = *reinterpret_cast<const u32x4*>(krow + swz(row, 4 * s + g) * 16);
+#pragma unroll
+          for (int rb = 0; rb < RB; ++rb) sacc[rb][blk] = mfma16<DT>(ka, qop[rb][s], sacc[rb][blk]);
+        }
+      }
+      // ---- the lane's 8 keys' slices of V (k slot j = 4 blk + r is key 16 blk + 4 g + r)
+      Words<VR> vrow[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        vrow[j] = load_words<VR>(reinterpret_cast<const uint16_t*>(buf + K_BYTES + (16 * (j >> 2) + 4 * g + (j & 3)) * (VC * 16)) + DPL * c);
+      // ---- online softmax in base 2, per row block
+      u32x4 pk[RB];
+      float alpha[RB];
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb) {
+        float sc[8];
+        float mx = -INFINITY;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const int key = t * 32 + 16 * (j >> 2) + 4 * g + (j & 3);
+          const float sv = sacc[rb][j >> 2][j & 3] * a.scale_log2;
+          sc[j] = key < my_limit[rb] ? sv : -INFINITY;
+          mx = fmaxf(mx, sc[j]);
+        }
+        mx = max_over_quarters(mx);
+        const float m_new = fmaxf(m[rb], mx);
+        const float m_use = m_new == -INFINITY ? 0.f : m_new;
+        alpha[rb] = __builtin_amdgcn_exp2f(m[rb] - m_use);
+        float p[8], psum = 0.f;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          p[j] = __builtin_amdgcn_exp2f(sc[j] - m_use + kShift);
+          psum += p[j];
+        }
+        l[rb] = l[rb] * alpha[rb] + psum;
+        m[rb] = m_new;
+        pk[rb].x = pack2<DT>(p[0], p[1]);
+        pk[rb].y = pack2<DT>(p[2], p[3]);
+        pk[rb].z = pack2<DT>(p[4], p[5]);
+        pk[rb].w = pack2<DT>(p[6], p[7]);
+      }
+      // ---- O^T = alpha O^T + V^T P^T
+#pragma unroll
+      for (int i = 0; i < DPL; ++i) {
+        u32x4 vt;
+        const uint32_t sel = (i & 1) ? kPermHighHalves : kPermLowHalves;
+        vt.x = perm(vrow[1].w[i >> 1], vrow[0].w[i >> 1], sel);
+        vt.y = perm(vrow[3].w[i >> 1], vrow[2].w[i >> 1], sel);
+        vt.z = perm(vrow[5].w[i >> 1], vrow[4].w[i >> 1], sel);
+        vt.w = perm(vrow[7].w[i >> 1], vrow[6].w[i >> 1], sel);
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) {
+          floatx4 o = oacc[rb][i];
+          o.x *= alpha[rb];
+          o.y *= alpha[rb];
+          o.z *= alpha[rb];
+          o.w *= alpha[rb];
+          oacc[rb][i] = mfma16<DT>(vt, pk[rb], o);
+        }
+      }
     }
-    // ---- the lane's 8 keys' slices of V (k slot j = 4 blk + r is key 16 blk + 4 g + r)
-    Words<VR> vrow[8];
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const int64_t vr = k_begin + min(t * 32 + 16 * (j >> 2) + 4 * g + (j & 3), k_len - 1);
-      vrow[j] = load_words<VR>(v_base + vr * a.v_st);
-    }
-    // ---- online softmax in base 2
-    float sc[8];
-    float mx = -INFINITY;
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const int key = t * 32 + 16 * (j >> 2) + 4 * g + (j & 3);
-      const float sv = sacc[j >> 2][j & 3] * a.scale_log2;
-      sc[j] = key < my_limit ? sv : -INFINITY;
-      mx = fmaxf(mx, sc[j]);
-    }
-    mx = max_over_quarters(mx);
-    const float m_new = fmaxf(m, mx);
-    const float m_use = m_new == -INFINITY ? 0.f : m_new;
-    const float alpha = __builtin_amdgcn_exp2f(m - m_use);
-    float p[8], psum = 0.f;
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      p[j] = __builtin_amdgcn_exp2f(sc[j] - m_use + kShift);
-      psum += p[j];
-    }
-    l = l * alpha + psum;
-    m = m_new;
-    u32x4 pk;
-    pk.x = pack2<DT>(p[0], p[1]);
-    pk.y = pack2<DT>(p[2], p[3]);
-    pk.z = pack2<DT>(p[4], p[5]);
-    pk.w = pack2<DT>(p[6], p[7]);
-    // ---- O^T = alpha O^T + V^T P^T
-#pragma unroll
-    for (int i = 0; i < DPL; ++i) {
-      u32x4 vt;
-      const uint32_t sel = (i & 1) ? kPermHighHalves : kPermLowHalves;
-      vt.x = perm(vrow[1].w[i >> 1], vrow[0].w[i >> 1], sel);
-      vt.y = perm(vrow[3].w[i >> 1], vrow[2].w[i >> 1], sel);
-      vt.z = perm(vrow[5].w[i >> 1], vrow[4].w[i >> 1], sel);
-      vt.w = perm(vrow[7].w[i >> 1], vrow[6].w[i >> 1], sel);
-      floatx4 o = oacc[i];
-      o.x *= alpha;
-      o.y *= alpha;
-      o.z *= alpha;
-      o.w *= alpha;
-      oacc[i] = mfma16<DT>(vt, pk, o);
-    }
+    if (t + 1 < num_tiles) drop(lds[(t + 1) & 1]);
+    __syncthreads();
   }
 
-  const float l_tot = sum_over_quarters(l);
-  const bool live = l_tot > 0.f;
-  const float inv = live ? 1.f / l_tot : 0.f;
-  if (q0 + c >= q_len) return;
-  const int64_t tok = q_begin + q0 + c;
-  uint16_t* op = static_cast<uint16_t*>(a.out) + tok * a.out_st + (int64_t)head * a.out_sh;
 #pragma unroll
-  for (int r = 0; r < 4; ++r) {
-    uint32_t w[VR];
+  for (int rb = 0; rb < RB; ++rb) {
+    const float l_tot = sum_over_quarters(l[rb]);
+    const bool live = l_tot > 0.f;
+    const float inv = live ? 1.f / l_tot : 0.f;
+    if (q0[rb] + c >= q_len) continue;
+    const int64_t tok = q_begin + q0[rb] + c;
+    uint16_t* op = static_cast<uint16_t*>(a.out) + tok * a.out_st + (int64_t)head * a.out_sh;
 #pragma unroll
-    for (int i = 0; i < VR; ++i) w[i] = pack2<DT>(oacc[2 * i][r] * inv, oacc[2 * i + 1][r] * inv);
-    uint16_t* dst = op + DPL * (4 * g + r);
-    if constexpr (VR == 2) {
-      *reinterpret_cast<u32x2*>(dst) = (u32x2){w[0], w[1]};
-    } else {
+    for (int r = 0; r < 4; ++r) {
+      uint32_t w[VR];
 #pragma unroll
-      for (int i = 0; i < VR / 4; ++i) reinterpret_cast<u32x4*>(dst)[i] = (u32x4){w[4 * i], w[4 * i + 1], w[4 * i + 2], w[4 * i + 3]};
+      for (int i = 0; i < VR; ++i) w[i] = pack2<DT>(oacc[rb][2 * i][r] * inv, oacc[rb][2 * i + 1][r] * inv);
+      uint16_t* dst = op + DPL * (4 * g + r);
+      if constexpr (VR == 2) {
+        *reinterpret_cast<u32x2*>(dst) = (u32x2){w[0], w[1]};
+      } else {
+#pragma unroll
+        for (int i = 0; i < VR / 4; ++i) reinterpret_cast<u32x4*>(dst)[i] = (u32x4){w[4 * i], w[4 * i + 1], w[4 * i + 2], w[4 * i + 3]};
+      }
     }
+    if (a.lse != nullptr && g == 0)
+      a.lse[(int64_t)head * a.total_q + tok] = live ? (m[rb] - kShift) * kLn2 + __logf(l_tot) : -INFINITY;
   }
-  if (a.lse != nullptr && g == 0)
-    a.lse[(int64_t)head * a.total_q + tok] = live ? (m - kShift) * kLn2 + __logf(l_tot) : -INFINITY;
 }
 
 template <int NOPE, int ROPE, int DV>
@@ -229,7 +308,7 @@ extern "C" int kvq_mla_prefill_attn(const void* q, int dtype, int64_t q_stride_t
   a.out_st = out_stride_tok; a.out_sh = out_stride_head; a.total_q = total_q;
   a.causal = causal != 0;
   a.scale_log2 = scale * kLog2e;
-  const dim3 grid((unsigned)((max_seqlen_q + 63) / 64), (unsigned)num_heads, (unsigned)num_seqs);
+  const dim3 grid((unsigned)((max_seqlen_q + 127) / 128), (unsigned)num_heads, (unsigned)num_seqs);
   hipStream_t s = as_stream(stream);
   if (nope_dim == 128 && rope_dim == 64 && v_dim == 128) return launch_varlen<128, 64, 128>(dtype, a, grid, s);
   if (nope_dim == 64 && rope_dim == 32 && v_dim == 64) return launch_varlen<64, 32, 64>(dtype, a, grid, s);
