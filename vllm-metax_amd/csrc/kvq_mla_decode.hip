@@ -6,7 +6,7 @@
 // O^T[dim, head] = C[:, :512]^T . P~^T, both on the MFMA with the heads as the N dimension.
 //
 // Work item = (sequence, token split, 128-head block); workgroup = 8 waves.  Each 32-token tile of
-// the latent stream goes from global memory STRAIGHT into a double-buffered LDS window
+// the latent stream goes from global memory STRAIGHT into one of three LDS windows
 // (buffer_load ... lds, no registers in between), a whole tile time ahead of its use; the 16-byte
 // chunks of a row are swizzled so that operand reads are free of bank conflicts without padding.
 // QK: wave w owns head tile w (16 heads) of the block and computes that tile's logits on the int8
@@ -15,9 +15,11 @@
 // It runs the tile's softmax (lazy reference maximum) and publishes the P~ operand, the rescale
 // factors and a "maximum moved" flag through a double-buffered LDS exchange.
 // PV is split over the waves by OUTPUT DIMS, not by heads: wave w accumulates dims 64 w .. 64 w + 63
-// of all 128 heads, so it transposes only those 64 dims of the tile into its own, wave-private
-// fp16 V^T (byte permutes in registers) and reads eight P~ operands per tile.  One workgroup
-// barrier per tile (P~ and the next raw tile visible).
+// of all 128 heads, so it needs only those 64 dims of the tile as fp16 V^T: a lane reads one dword
+// from each of its 8 token rows of the raw tile and transposes in registers (byte permutes), no
+// second copy of the tile in LDS; it reads eight P~ operands per tile.  One workgroup barrier per
+// tile (P~ and the next raw tile visible); the third window is what lets the P~V read the raw tile
+// after that barrier while the tile after the next already streams in.
 // The token splits of a sequence are merged by the reduce kernel with the log-sum-exp algebra
 // (same two-stage shape as the reference's decode_attention_fwd); nothing is allocated here,
 // partials and the int8 Q live in the caller's workspace.
@@ -42,14 +44,13 @@ constexpr int kMlaKSteps8 = kMlaW / 64;                   // 9 int8 k-steps of 6
 constexpr int kMlaQOps = 2 * kMlaKSteps8;                 // B operands of Q: two int8 terms per k-step
 constexpr int kMlaQRegOps = 10;                           // operands of Q kept in registers; the rest in LDS
 constexpr int kMlaQLdsBytes = (kMlaQOps - kMlaQRegOps) * kMlaThreads * 16;  // 65536
-constexpr int kMlaVtPitch = 2 * kTile;                    // fp16 V^T row: 32 tokens = 4 chunks of 16 bytes, swizzled
-constexpr int kMlaVtBytes = kMlaR * kMlaVtPitch;          // 32768
+constexpr int kMlaRing = 3;                               // raw tile windows: tile t is read (QK, then PV) while t + 1 and t + 2 stream in
 typedef int32_t i32x4 __attribute__((ext_vector_type(4)));
 // What the head-owning waves hand to the others, per tile and double-buffered: the eight P~ operands
 // (64 lanes x 16 bytes each), one rescale factor per head and one "running max moved" byte per wave.
 constexpr int kMlaPBytes = 8 * kWave * 16;                // 8192
 constexpr int kMlaXchgBytes = kMlaPBytes + 128 * 4 + 16;  // 8720
-constexpr int kMlaLdsBytes = 2 * kMlaBufBytes + kMlaVtBytes + kMlaQLdsBytes + 2 * kMlaXchgBytes;  // 153120 of 163840
+constexpr int kMlaLdsBytes = kMlaRing * kMlaBufBytes + kMlaQLdsBytes + 2 * kMlaXchgBytes;  // 139296 of 163840
 
 struct MlaArgs {
   const void* q;            // dims 0 .. 511 of the absorbed query (ql_nope) ...
@@ -356,11 +357,10 @@ __global__ __launch_bounds__(256) void mla_absorb_q_kernel(MlaAbsorbArgs a) {
 template <bool FULL>
 __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
   extern __shared__ __align__(16) uint8_t lds_raw[];
-  uint8_t(*lds)[kMlaBufBytes] = reinterpret_cast<uint8_t(*)[kMlaBufBytes]>(lds_raw);
-  uint8_t* vt = lds_raw + 2 * kMlaBufBytes;  // fp16 V^T of the current tile; rows 64 w .. 64 w + 63 belong to wave w
+  uint8_t(*lds)[kMlaBufBytes] = reinterpret_cast<uint8_t(*)[kMlaBufBytes]>(lds_raw);   // kMlaRing raw windows
   // B operands of Q from number kMlaQRegOps on: slot [operand][thread], written and read by the same lane
-  u32x4* qlds = reinterpret_cast<u32x4*>(lds_raw + 2 * kMlaBufBytes + kMlaVtBytes) + threadIdx.x;
-  uint8_t* xchg = lds_raw + 2 * kMlaBufBytes + kMlaVtBytes + kMlaQLdsBytes;
+  u32x4* qlds = reinterpret_cast<u32x4*>(lds_raw + kMlaRing * kMlaBufBytes) + threadIdx.x;
+  uint8_t* xchg = lds_raw + kMlaRing * kMlaBufBytes + kMlaQLdsBytes;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -486,44 +486,33 @@ __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
     for (int b = 0; b < 4; ++b) o[ht][b] = (floatx4){0.f, 0.f, 0.f, 0.f};
   float m = -INFINITY, l = 0.f;
 
-  // ---- V^T of the tile as fp16: wave v transposes dims 64 v .. 64 v + 63, the dims whose outputs
-  //      it accumulates, so this part of LDS is private to the wave (no barrier guards it).
-  //      A thread takes, twice, a block of 4 tokens x 4 dims (one dword per token row), transposes it
-  //      with byte permutes and writes, for each of the 4 dims, the 4 tokens' plain codes as fp16 (8
-  //      bytes).  Dim 64 w + 4 r' + b sits in row (4 w + b) * 16 + r' -- row r' of output tile 4 w + b --
-  //      and token 16 mt + 4 g' + i at position 8 g' + 4 mt + i, the order in which a lane of the P~
-  //      operand holds its 8 tokens; the four 16-byte chunks of a row are swizzled with bits 1..2 of
-  //      the row like the raw tile's.  Lanes = 8 consecutive rows x 8 token groups.
-  const int tr = lane & 7, tq = lane >> 3;
-  // dword of dims 64 wave + 4 tr + 32 u .. + 3 in row 4 tq + r: chunk 4 wave + 2 u + (tr >> 2), swizzled with
-  // bits 1..2 of the row, which r >> 1 takes part in
-  uint32_t vt_src[2][2];
+  // ---- V^T operands of the tile, built in registers from the raw tile.  Wave w accumulates dims
+  //      64 w .. 64 w + 63 of all heads; output tile 4 w + b, row r' is dim 64 w + 4 r' + b.  A lane (r', g)
+  //      reads one dword -- its four dims -- from each of the 8 token rows its P~ operand holds (k slot j of
+  //      quarter g is token 16 (j / 4) + 4 g + j % 4), transposes the 8 x 4 byte block with byte permutes and
+  //      turns each dim's 8 codes into one fp16 A operand.  Rows 4 g + i and 16 + 4 g + i share their swizzle
+  //      in pairs: two loop-invariant offsets, the rest are immediates.
+  const uint32_t vo_a = (uint32_t)(4 * g * kMlaPitch + 16 * (4 * wave + ((c >> 2) ^ ((2 * g) & 3))) + 4 * (c & 3));
+  const uint32_t vo_b = (uint32_t)(4 * g * kMlaPitch + 16 * (4 * wave + ((c >> 2) ^ ((2 * g + 1) & 3))) + 4 * (c & 3));
+  auto v_operands = [&](const uint8_t* tile, half8_t (&va)[4]) __attribute__((always_inline)) {
+    uint32_t x[8];
 #pragma unroll
-  for (int u = 0; u < 2; ++u)
+    for (int j = 0; j < 8; ++j)
+      x[j] = *reinterpret_cast<const uint32_t*>(tile + ((j & 2) ? vo_b : vo_a) + (16 * (j >> 2) + (j & 3)) * kMlaPitch) ^ 0x80808080u;
+    uint32_t lo[4], hi[4];   // token pairs (0,1) (2,3) (4,5) (6,7): dims 0,1 interleaved / dims 2,3 interleaved
 #pragma unroll
-    for (int rh = 0; rh < 2; ++rh)
-      vt_src[u][rh] = (uint32_t)(4 * tq * kMlaPitch + 16 * (4 * wave + ((2 * u + (tr >> 2)) ^ ((2 * tq + rh) & 3))) + 4 * (tr & 3));
-  const uint32_t vt_dst = (uint32_t)((64 * wave + tr) * kMlaVtPitch + 16 * ((tq & 3) ^ ((tr >> 1) & 3)) + 8 * (tq >> 2));
-  auto transpose_v = [&](const uint8_t* tile) __attribute__((always_inline)) {
-    uint32_t x[2][4];   // all eight reads leave before the first permute waits
+    for (int q = 0; q < 4; ++q) {
+      lo[q] = perm(x[2 * q + 1], x[2 * q], 0x05010400u);
+      hi[q] = perm(x[2 * q + 1], x[2 * q], 0x07030602u);
+    }
 #pragma unroll
-    for (int u = 0; u < 2; ++u)
-#pragma unroll
-      for (int r = 0; r < 4; ++r)
-        x[u][r] = *reinterpret_cast<const uint32_t*>(tile + vt_src[u][r >> 1] + r * kMlaPitch);
-#pragma unroll
-    for (int u = 0; u < 2; ++u) {
-#pragma unroll
-      for (int r = 0; r < 4; ++r) x[u][r] ^= 0x80808080u;
-      const uint32_t a01 = perm(x[u][1], x[u][0], 0x05010400u), b01 = perm(x[u][1], x[u][0], 0x07030602u);
-      const uint32_t a23 = perm(x[u][3], x[u][2], 0x05010400u), b23 = perm(x[u][3], x[u][2], 0x07030602u);
-#pragma unroll
-      for (int b = 0; b < 4; ++b) {
-        u32x2 h;
-        h.x = mla_codes_to_half2(b < 2 ? a01 : b01, b & 1);
-        h.y = mla_codes_to_half2(b < 2 ? a23 : b23, b & 1);
-        *reinterpret_cast<u32x2*>(vt + vt_dst + (16 * b + 8 * u) * kMlaVtPitch) = h;
-      }
+    for (int b = 0; b < 4; ++b) {
+      u32x4 h;
+      h.x = mla_codes_to_half2(b < 2 ? lo[0] : hi[0], b & 1);
+      h.y = mla_codes_to_half2(b < 2 ? lo[1] : hi[1], b & 1);
+      h.z = mla_codes_to_half2(b < 2 ? lo[2] : hi[2], b & 1);
+      h.w = mla_codes_to_half2(b < 2 ? lo[3] : hi[3], b & 1);
+      va[b] = __builtin_bit_cast(half8_t, h);
     }
   };
 
@@ -537,14 +526,16 @@ __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
   lds_barrier();
 
   const uint32_t ka_off = (uint32_t)(c * kMlaPitch + 16 * (g ^ ((c >> 1) & 3)));   // row c, chunk g of a k-step, swizzled
-  int buf = 0;
+  int buf = 0;   // parity of the exchange area
+  int cur = 0;   // raw window of tile t; t + 1 is in cur + 1, t + 2 streams into cur + 2 (mod 3)
   for (int t = t_begin; t < t_end; ++t) {
-    const uint8_t* tile = lds[buf];
+    const uint8_t* tile = lds[cur];
+    const int nxt = cur == kMlaRing - 1 ? 0 : cur + 1;
+    const int nxt2 = nxt == kMlaRing - 1 ? 0 : nxt + 1;
     const float* sck = reinterpret_cast<const float*>(tile + kMlaTileBytes);
     uint8_t* xb = xchg + buf * kMlaXchgBytes;         // this tile's P~ operands, rescale factors, flags
     float* x_alpha = reinterpret_cast<float*>(xb + kMlaPBytes);
     uint8_t* x_flag = xb + kMlaPBytes + 128 * 4;
-    transpose_v(tile);
 
     if (owner) {
       // ---- S^T[32 tokens, 16 heads] on the int8 MFMA: A = the cached code bytes as they are, lane
@@ -643,23 +634,21 @@ __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
       else softmax(std::false_type{});
     }
 
-    if (t + 1 < t_end) stage_scales(lds[buf ^ 1]);
+    if (t + 1 < t_end) stage_scales(lds[nxt]);
     // The ONE barrier of a tile (it also waits for this wave's part of the next raw tile): P~, the
     // rescale factors and the next raw tile are visible to every wave.  The exchange area is double-buffered, so a wave that runs ahead into the next tile
     // writes the other half while slower waves still read this one.
     tile_barrier();
-    // this tile's raw window is free now (its readers are past the barrier): the tile after the next
-    // streams into it, a whole tile time ahead of its use
-    if (t + 2 < t_end) issue_loads(nb, lds[buf]);
+    // the window of tile t - 1 is free now (every wave is past its P~V): the tile after the next streams
+    // into it, a whole tile time ahead of its use, while this tile's window still feeds the P~V below
+    if (t + 2 < t_end) issue_loads(nb, lds[nxt2]);
     nb = fetch_blocks(t + 3);
 
-    // ---- O^T[64 dims of this wave, 128 heads] += C^T . P~^T: A = fp16 V^T rows, lane (r = row of
-    //      output tile 4 wave + b, g): positions 8 g .. 8 g + 7; B = head tile ht's P~ operand
+    // ---- O^T[64 dims of this wave, 128 heads] += C^T . P~^T: A = the wave's four fp16 V^T operands, built
+    //      from the raw tile in registers; B = head tile ht's P~ operand
     const u32x2 flags = *reinterpret_cast<const u32x2*>(x_flag);
     half8_t va[4];
-#pragma unroll
-    for (int b = 0; b < 4; ++b)
-      va[b] = *reinterpret_cast<const half8_t*>(vt + ((4 * wave + b) * 16 + c) * kMlaVtPitch + 16 * (g ^ ((c >> 1) & 3)));
+    v_operands(tile, va);
     // (FULL) operand ht + 3 is fetched while tile ht multiplies; the first three leave with the
     // flags, before anything waits
     const u32x4* pl = reinterpret_cast<const u32x4*>(xb) + lane;
@@ -703,6 +692,7 @@ __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
       }
     }
     buf ^= 1;
+    cur = nxt;
   }
 
   // ---- emit the split's state: locally normalised output and its log2-domain lse.  The owners pass
