@@ -101,8 +101,9 @@ def test_ragged_lengths_fp32_out(gpu_device, ctx):
     T.assert_close_attn(got, want, atol=2e-3, rtol=2e-3, what=f"ctx={ctx[:5]}")
 
 
+@pytest.mark.parametrize("layout", ["NHD", "HND"])
 @pytest.mark.parametrize("hkv", [1, 2, 8])
-def test_hundreds_of_short_sequences(gpu_device, hkv):
+def test_hundreds_of_short_sequences(gpu_device, hkv, layout):
     """300 sequences of 0 .. 200 tokens with prefill rows in between: the sequence scans run in
     batches of several 64-sequence chunks, a workgroup's share crosses many sequence boundaries
     (or, with one kv head, the work line is so short that not every workgroup gets a share), and
@@ -114,11 +115,11 @@ def test_hundreds_of_short_sequences(gpu_device, hkv):
         qls[i] = min(3, max(ctx[i], 1))
         ctx[i] = max(ctx[i], qls[i])
     from test_gpu_prefill import build
-    kv, lay, bt, q, sl, cu = build([max(c, 1) for c in ctx], qls, 2 * hkv, hkv, 128, 16, seed=hkv)
+    kv, lay, bt, q, sl, cu = build([max(c, 1) for c in ctx], qls, 2 * hkv, hkv, 128, 16, seed=hkv, layout=layout)
     sl = torch.tensor(ctx, dtype=torch.int32)   # the true lengths, zeros included
     scale = 1 / math.sqrt(128)
     want, want_lse = oracle.paged_attn(q, T.storage_bytes(kv), lay, bt, sl, cu, scale, return_lse=True)
-    kvd = T.to_device_cache(kv, gpu_device, "NHD")
+    kvd = T.to_device_cache(kv, gpu_device, layout)
     k, v = L.key_value_views(kvd)
     ks, vs = L.scale_views(kvd)
     out = torch.full(q.shape, float("nan"), dtype=torch.float32, device=gpu_device)
@@ -138,13 +139,14 @@ def test_hundreds_of_short_sequences(gpu_device, hkv):
                                          # kv head counts that leave the last workgroup partly empty (its
                                          # spare waves exit before the stream loop's rendezvous)
                                          (24, 12, 128, 16), (6, 3, 64, 16), (10, 5, 128, 32)])
-def test_head_and_block_shapes(gpu_device, hq, hkv, d, bs):
+@pytest.mark.parametrize("layout", ["NHD", "HND"])   # HND: the streamed run loads (head sizes 64 and 128)
+def test_head_and_block_shapes(gpu_device, hq, hkv, d, bs, layout):
     ctx = [200, 77, 1025, 48]
-    kv, lay, bt, q, sl, cu = build_case(ctx, hq, hkv, d, bs, "NHD", hq + d)
+    kv, lay, bt, q, sl, cu = build_case(ctx, hq, hkv, d, bs, layout, hq + d)
     scale = d ** -0.5
     want = oracle.paged_attn(q, T.storage_bytes(kv), lay, bt, sl, cu, scale)
-    got = run_unified(gpu_device, kv, "NHD", bt, q, sl, cu, scale)
-    T.assert_close_attn(got, want, what=f"hq={hq} hkv={hkv} d={d} bs={bs}")
+    got = run_unified(gpu_device, kv, layout, bt, q, sl, cu, scale)
+    T.assert_close_attn(got, want, what=f"hq={hq} hkv={hkv} d={d} bs={bs} {layout}")
 
 
 @pytest.mark.parametrize("q_dtype", [torch.float16, torch.float32])

@@ -18,8 +18,8 @@ from vllm_metax_amd import layout as L
 pytestmark = pytest.mark.gpu
 
 
-def run(dev, kv_cpu, bt, q, sl, cu, max_q, scale, window, cap, want_lse=False, out_dtype=None):
-    kv = T.to_device_cache(kv_cpu, dev, "NHD")
+def run(dev, kv_cpu, bt, q, sl, cu, max_q, scale, window, cap, want_lse=False, out_dtype=None, layout="NHD"):
+    kv = T.to_device_cache(kv_cpu, dev, layout)
     k, v = L.key_value_views(kv)
     ks, vs = L.scale_views(kv)
     out = torch.full(q.shape, float("nan"), dtype=out_dtype or q.dtype, device=dev)
@@ -31,25 +31,26 @@ def run(dev, kv_cpu, bt, q, sl, cu, max_q, scale, window, cap, want_lse=False, o
     return (out, lse) if want_lse else out
 
 
-def check(dev, ctx, qls, hq, hkv, d, bs, window, cap, seed, scale=None, q_dtype=torch.bfloat16, what=""):
-    kv, lay, bt, q, sl, cu = build(ctx, qls, hq, hkv, d, bs, seed=seed, q_dtype=q_dtype)
+def check(dev, ctx, qls, hq, hkv, d, bs, window, cap, seed, scale=None, q_dtype=torch.bfloat16, what="", layout="NHD"):
+    kv, lay, bt, q, sl, cu = build(ctx, qls, hq, hkv, d, bs, seed=seed, q_dtype=q_dtype, layout=layout)
     scale = scale if scale is not None else 1 / math.sqrt(d)
     want, want_lse = oracle.paged_attn(q, T.storage_bytes(kv), lay, bt, sl, cu, scale, return_lse=True,
                                        sliding_window=window or 0, soft_cap=cap or 0.0)
-    got, lse = run(dev, kv, bt, q, sl, cu, max(qls), scale, window, cap, want_lse=True)
-    T.assert_close_attn(got, want, what=f"{what} window={window} cap={cap}")
+    got, lse = run(dev, kv, bt, q, sl, cu, max(qls), scale, window, cap, want_lse=True, layout=layout)
+    T.assert_close_attn(got, want, what=f"{what} window={window} cap={cap} {layout}")
     torch.testing.assert_close(lse.cpu(), want_lse, atol=5e-3, rtol=1e-3)
 
 
+@pytest.mark.parametrize("layout", ["NHD", "HND"])   # HND without a cap: the streamed run loads, first tile peeled
 @pytest.mark.parametrize("window", [None, 1, 31, 32, 33, 256, 5000])
 @pytest.mark.parametrize("cap", [None, 50.0])
-def test_decode_rows(gpu_device, window, cap):
+def test_decode_rows(gpu_device, window, cap, layout):
     """Windows that start inside the first tile, on a tile edge, deep inside a long sequence (so
     that most tiles never enter the tile line) and beyond every sequence (no effect)."""
     if window is None and cap is None:
         pytest.skip("covered by the plain decode tests")
     ctx = [1, 31, 32, 33, 257, 1000, 4097, 300, 64]
-    check(gpu_device, ctx, [1] * len(ctx), 32, 8, 128, 16, window, cap, seed=3, what="decode")
+    check(gpu_device, ctx, [1] * len(ctx), 32, 8, 128, 16, window, cap, seed=3, what="decode", layout=layout)
 
 
 @pytest.mark.parametrize("hq,hkv,d,bs", [(28, 4, 128, 16), (8, 8, 64, 32), (4, 2, 256, 16), (16, 1, 128, 16)])
