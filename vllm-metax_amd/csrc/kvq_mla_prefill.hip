@@ -124,22 +124,32 @@ __global__ __launch_bounds__(256) void varlen_attn_kernel(VarlenArgs a) {
   const uint16_t* kpe_base = static_cast<const uint16_t*>(a.k_pe);
   const uint16_t* v_base = static_cast<const uint16_t*>(a.v) + (int64_t)head * a.v_sh;
   u32x4 kreg[KLD], vreg[VLD];
+  // per chunk, fixed for the whole run: its row in the tile, the tensor it comes from and the offset inside a row
+  int k_row[KLD], v_row[VLD];
+  const uint16_t* k_src[KLD];
+  int64_t k_stride[KLD];
+  const uint16_t* v_src[VLD];
+#pragma unroll
+  for (int i = 0; i < KLD; ++i) {
+    const int q = min(tid + 256 * i, 32 * KC - 1);
+    k_row[i] = q / KC;
+    const int ch = q - k_row[i] * KC;
+    k_src[i] = ch < KCN ? kn_base + 8 * ch : kpe_base + 8 * (ch - KCN);
+    k_stride[i] = ch < KCN ? a.kn_st : a.kpe_st;
+  }
+#pragma unroll
+  for (int i = 0; i < VLD; ++i) {
+    const int q = min(tid + 256 * i, 32 * VC - 1);
+    v_row[i] = q / VC;
+    v_src[i] = v_base + 8 * (q - v_row[i] * VC);
+  }
   auto fetch = [&](int t) __attribute__((always_inline)) {
 #pragma unroll
-    for (int i = 0; i < KLD; ++i) {
-      const int q = min(tid + 256 * i, 32 * KC - 1);
-      const int row = q / KC, ch = q - row * KC;
-      const int64_t krow = k_begin + min(t * 32 + row, k_len - 1);
-      const uint16_t* p = ch < KCN ? kn_base + krow * a.kn_st + 8 * ch : kpe_base + krow * a.kpe_st + 8 * (ch - KCN);
-      kreg[i] = *reinterpret_cast<const u32x4*>(p);
-    }
+    for (int i = 0; i < KLD; ++i)
+      kreg[i] = *reinterpret_cast<const u32x4*>(k_src[i] + (int64_t)(k_begin + min(t * 32 + k_row[i], k_len - 1)) * k_stride[i]);
 #pragma unroll
-    for (int i = 0; i < VLD; ++i) {
-      const int q = min(tid + 256 * i, 32 * VC - 1);
-      const int row = q / VC, ch = q - row * VC;
-      const int64_t vrow = k_begin + min(t * 32 + row, k_len - 1);
-      vreg[i] = *reinterpret_cast<const u32x4*>(v_base + vrow * a.v_st + 8 * ch);
-    }
+    for (int i = 0; i < VLD; ++i)
+      vreg[i] = *reinterpret_cast<const u32x4*>(v_src[i] + (int64_t)(k_begin + min(t * 32 + v_row[i], k_len - 1)) * a.v_st);
   };
   auto swz = [](int row, int ch) { return KC % 8 == 0 ? (ch ^ (row & 7)) : (ch ^ ((row >> 1) & 3)); };
   auto drop = [&](uint8_t* buf) __attribute__((always_inline)) {
@@ -190,6 +200,7 @@ __global__ __launch_bounds__(256) void varlen_attn_kernel(VarlenArgs a) {
       // ---- online softmax in base 2, per row block
       u32x4 pk[RB];
       float alpha[RB];
+      bool moved = false;
 #pragma unroll
       for (int rb = 0; rb < RB; ++rb) {
         float sc[8];
@@ -205,6 +216,7 @@ __global__ __launch_bounds__(256) void varlen_attn_kernel(VarlenArgs a) {
         const float m_new = fmaxf(m[rb], mx);
         const float m_use = m_new == -INFINITY ? 0.f : m_new;
         alpha[rb] = __builtin_amdgcn_exp2f(m[rb] - m_use);
+        moved = moved || m_new > m[rb];
         float p[8], psum = 0.f;
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
@@ -218,7 +230,15 @@ __global__ __launch_bounds__(256) void varlen_attn_kernel(VarlenArgs a) {
         pk[rb].z = pack2<DT>(p[4], p[5]);
         pk[rb].w = pack2<DT>(p[6], p[7]);
       }
-      // ---- O^T = alpha O^T + V^T P^T
+      // ---- O^T = alpha O^T + V^T P^T.  The accumulators are rescaled only in the tiles in which some row's
+      //      maximum moved (they live in accumulation registers: a rescale is a read, a multiply and a write
+      //      of each); after a sequence's first tiles that is rare.
+      if (__builtin_amdgcn_ballot_w64(moved) != 0) {
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+          for (int i = 0; i < DPL; ++i) oacc[rb][i] *= alpha[rb];
+      }
 #pragma unroll
       for (int i = 0; i < DPL; ++i) {
         u32x4 vt;
@@ -228,14 +248,7 @@ __global__ __launch_bounds__(256) void varlen_attn_kernel(VarlenArgs a) {
         vt.z = perm(vrow[5].w[i >> 1], vrow[4].w[i >> 1], sel);
         vt.w = perm(vrow[7].w[i >> 1], vrow[6].w[i >> 1], sel);
 #pragma unroll
-        for (int rb = 0; rb < RB; ++rb) {
-          floatx4 o = oacc[rb][i];
-          o.x *= alpha[rb];
-          o.y *= alpha[rb];
-          o.z *= alpha[rb];
-          o.w *= alpha[rb];
-          oacc[rb][i] = mfma16<DT>(vt, pk[rb], o);
-        }
+        for (int rb = 0; rb < RB; ++rb) oacc[rb][i] = mfma16<DT>(vt, pk[rb], oacc[rb][i]);
       }
     }
     if (t + 1 < num_tiles) drop(lds[(t + 1) & 1]);
