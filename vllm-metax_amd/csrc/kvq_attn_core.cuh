@@ -354,8 +354,12 @@ struct DecodeTile {
     // past the end of the sequence rereads the first half and is masked in compute
     const int s0 = mod_bs(io, tok0);
     const int s1 = tb.s1_same ? s0 : mod_bs(io, tok0 + 16);
-    const uint8_t* p0 = io.cache + G.k_off + (int64_t)tb.b0 * G.stride_block + (int64_t)s0 * G.stride_slot + (int64_t)hkv * G.stride_head;
-    const uint8_t* p1 = io.cache + G.k_off + (int64_t)tb.b1 * G.stride_block + (int64_t)s1 * G.stride_slot + (int64_t)hkv * G.stride_head;
+    // strides are below 2^31 (checked on the host): block number x block stride is one 32 x 32 -> 64 bit
+    // multiply, the offset inside the block stays in 32 bits
+    const uint8_t* head = io.cache + G.k_off + (uint64_t)((uint32_t)hkv * (uint32_t)G.stride_head);
+    const uint32_t sb = (uint32_t)G.stride_block, ss = (uint32_t)G.stride_slot;
+    const uint8_t* p0 = head + (uint64_t)(uint32_t)tb.b0 * sb + (uint32_t)s0 * ss;
+    const uint8_t* p1 = head + (uint64_t)(uint32_t)tb.b1 * sb + (uint32_t)s1 * ss;
     Window w;
     w.r0 = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(p0), 0, 0x7fffffff, 0x00020000);
     w.r1 = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(p1), 0, 0x7fffffff, 0x00020000);
