@@ -34,9 +34,6 @@ constexpr int kMlaR = 512, kMlaP = 64, kMlaW = kMlaR + kMlaP;
 constexpr int kMlaPitch = kMlaW;                          // LDS rows are packed; the 16-byte chunks of a row are swizzled
 constexpr int kMlaTileBytes = kTile * kMlaPitch;          // 32 rows = 1152 chunks
 constexpr int kMlaBufBytes = kMlaTileBytes + 2 * kTile * 4;  // + 32 K-side and 32 V-side scales
-constexpr int kMlaKSteps = kMlaW / 32;                    // 18
-constexpr int kMlaDT = kMlaR / 16;                        // 32 output row tiles of 16 dims
-constexpr int kMlaVB = kMlaR / 16;                        // 32 V bytes per token per lane
 constexpr int kChunksPerRow = kMlaW / 16;                 // 36
 constexpr int kChunksPerHalf = 16 * kChunksPerRow;        // 576
 constexpr int kMlaThreads = 512;
@@ -86,6 +83,26 @@ __device__ __forceinline__ uint32_t mla_codes_to_half2(uint32_t x, bool upper) {
   const half2_t bias = {(half_t)kCodeBias, (half_t)kCodeBias};
   const half2_t v = __builtin_bit_cast(half2_t, bytes_to_half2(x, upper)) - bias;
   return __builtin_bit_cast(uint32_t, v);
+}
+
+// Byte B of x0 and of x1, each a signed code, as the fp16 pair (x0.B, x1.B): the conversion reads its
+// byte through the operand's sub-dword select with sign extension and writes one half of the result, so
+// a pair costs two instructions and no shuffles.
+template <int B>
+__device__ __forceinline__ uint32_t mla_code_pair_to_half2(uint32_t x0, uint32_t x1) {
+  uint32_t r;
+  asm("v_cvt_f16_i16_sdwa %0, sext(%1) dst_sel:WORD_0 dst_unused:UNUSED_PAD src0_sel:BYTE_%2" : "=v"(r) : "v"(x0), "n"(B));
+  asm("v_cvt_f16_i16_sdwa %0, sext(%1) dst_sel:WORD_1 dst_unused:UNUSED_PRESERVE src0_sel:BYTE_%2" : "+v"(r) : "v"(x1), "n"(B));
+  return r;
+}
+template <int B>
+__device__ __forceinline__ half8_t mla_code_rows_to_operand(const uint32_t (&x)[8]) {
+  u32x4 h;
+  h.x = mla_code_pair_to_half2<B>(x[0], x[1]);
+  h.y = mla_code_pair_to_half2<B>(x[2], x[3]);
+  h.z = mla_code_pair_to_half2<B>(x[4], x[5]);
+  h.w = mla_code_pair_to_half2<B>(x[6], x[7]);
+  return __builtin_bit_cast(half8_t, h);
 }
 
 // tokens of a sequence per split, a whole number of tiles
@@ -718,6 +735,269 @@ __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
   if (owner && g == 0) a.part_lse[(pblock0 + wave) * 16 + c] = m + __builtin_amdgcn_logf(l);
 }
 
+// ---------------------------------------------------------------------------------------------
+// At most 16 heads (one head tile: a tensor-parallel shard of a 128-head model, or a small model).
+//
+// With one head tile the kernel above has one wave computing logits while seven wait, and a tile takes
+// as long as with 128 heads.  Here every wave streams its OWN tiles (wave w of four: tiles t_begin + w, + 4, ...)
+// and nothing is exchanged inside the tile loop: the wave loads a tile's rows from global memory straight
+// into registers in the int8 MFMA's A layout (lane = token, 16 consecutive dims: every byte is loaded
+// once, by the lane that multiplies it), computes the logits of its 16 heads against the Q operands it
+// keeps in registers, runs the softmax -- whose result already IS the P~ operand of the second product -- and copies
+// the rows' first 512 bytes into a wave-private, chunk-swizzled LDS window, from which it builds the fp16
+// V^T operands of all 512 output dims with dword reads and byte permutes (as the kernel above does for
+// its 64).  At the end the eight waves' states are summed through the (then idle) windows, each wave
+// adding up and emitting the 64 output dims of its number.
+constexpr int kMlaSmallWin = kTile * kMlaR;                                   // 16384: a tile's V part
+constexpr int kMlaSmallQBytes = 4096;                                         // (m, l) of the waves at the end
+constexpr int kMlaSmallWaves = 4;   // one wave per SIMD: a wave may then use the whole register file (512 per lane)
+constexpr int kMlaSmallThreads = kMlaSmallWaves * kWave;
+constexpr int kMlaSmallLdsBytes = kMlaSmallWaves * kMlaSmallWin + kMlaSmallQBytes;         // 69632
+
+__global__ __launch_bounds__(kMlaSmallThreads) void mla_decode_small_kernel(MlaArgs a) {
+  extern __shared__ __align__(16) uint8_t lds_raw[];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int c = lane & 15, g = lane >> 4;
+  uint8_t* win = lds_raw + wave * kMlaSmallWin;
+  const int seq = blockIdx.y, split = blockIdx.x;
+  const int len = a.seq_lens[seq];
+  const int slen = mla_split_len(len > 0 ? len : 0, a.num_splits);
+  const int tok_begin = split * slen;
+  const int tok_end = min(len, tok_begin + slen);
+  const int64_t pblock = ((int64_t)seq * a.num_splits + split) * a.head_groups;
+  if (tok_begin >= tok_end) {  // empty split (uniform over the workgroup): mark it and leave
+    if (wave == 0 && g == 0) a.part_lse[pblock * 16 + c] = -INFINITY;
+    return;
+  }
+  const int t_begin = tok_begin / kTile, t_end = (tok_end + kTile - 1) / kTile;
+  const int bs = a.g.block_size;
+  const int32_t* bt_row = a.block_table + (int64_t)seq * a.bt_stride;
+
+  // ---- Q operands of the sequence's heads in registers (a wave owns the whole register file), s1 per head
+  const int64_t qblock = (int64_t)seq * a.head_groups;
+  i32x4 qreg[kMlaQOps];
+  {
+    const u32x4* qsrc = reinterpret_cast<const u32x4*>(a.q_ops + qblock * (kMlaQOps * kWave * 16)) + lane;
+#pragma unroll
+    for (int op = 0; op < kMlaQOps; ++op) qreg[op] = __builtin_bit_cast(i32x4, qsrc[op * kWave]);
+  }
+  const float s1 = a.q_scale[qblock * 16 + c], s2 = s1 / 254.0f;
+
+  // ---- one tile's rows in registers: kreg[mt][kk] = row 16 mt + c, dims 64 kk + 16 g .. + 15; ks[mt] = the
+  //      scales of tokens 16 mt + 4 g .. + 3 (the four logits a lane holds per half)
+  struct Rows {
+    u32x4 k[2][kMlaKSteps8];
+    floatx4 ks[2];
+  };
+  // Block numbers are read one tile ahead of the rows that need them: a block-table read that misses the
+  // scalar cache costs a trip to memory, and the row loads behind it cannot leave before it returns.
+  struct TileIds {
+    int blk[2];
+  };
+  auto tile_tok = [&](int t, int h) __attribute__((always_inline)) {
+    const int tok = t * kTile + 16 * h;
+    return tok < len ? tok : ((len - 1) & ~15);   // a half past the end rereads the last valid half and is masked
+  };
+  auto load_ids = [&](int t, TileIds& ids) __attribute__((always_inline)) {
+#pragma unroll
+    for (int h = 0; h < 2; ++h) ids.blk[h] = scalar_load_i32(bt_row, (int)__umulhi((uint32_t)tile_tok(t, h), a.bs_magic));
+  };
+  auto load_rows = [&](int t, Rows& rr, const TileIds& ids) __attribute__((always_inline)) {
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const int tok = tile_tok(t, h);
+      const int slot = tok - (int)__umulhi((uint32_t)tok, a.bs_magic) * bs;
+      const uint8_t* pb = a.cache + (int64_t)ids.blk[h] * a.g.stride_block;
+      const uint8_t* row = pb + (int64_t)(slot + c) * a.g.stride_row + 16 * g;
+#pragma unroll
+      for (int kk = 0; kk < kMlaKSteps8; ++kk) rr.k[h][kk] = *reinterpret_cast<const u32x4_a4*>(row + 64 * kk);
+      rr.ks[h] = *reinterpret_cast<const floatx4_a4*>(pb + a.g.scale_off + (int64_t)(slot + 4 * g) * 4);
+    }
+  };
+
+  floatx4 o[32];   // o[4 d4 + b][i]: head c, dim 64 d4 + 16 g + 4 i + b
+#pragma unroll
+  for (int j = 0; j < 32; ++j) o[j] = (floatx4){0.f, 0.f, 0.f, 0.f};
+  float m = -INFINITY, l = 0.f;
+
+  // V dwords of the lane's 8 tokens (k slot j of quarter g is token 16 (j / 4) + 4 g + j % 4) for the dims
+  // 64 d4 + 4 c .. + 3: row pitch 512, 16-byte chunk number xor (row & 7)
+  uint32_t vrow_off[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const int row = 16 * (j >> 2) + 4 * g + (j & 3);
+    vrow_off[j] = (uint32_t)(row * kMlaR + 16 * ((c >> 2) ^ (row & 3)) + 4 * (c & 3));
+  }
+  const int vflip = g & 1;   // bit 2 of every one of the lane's rows: it toggles the low bit of the 64-dim group
+
+  auto tile_step = [&](Rows& rr, TileIds& ids, int t) __attribute__((always_inline)) {
+    // ---- S^T[32 tokens, 16 heads] on the int8 MFMA, one accumulator per term of Q
+    i32x4 acc[2][2];
+#pragma unroll
+    for (int term = 0; term < 2; ++term)
+#pragma unroll
+      for (int mt = 0; mt < 2; ++mt) acc[term][mt] = (i32x4){0, 0, 0, 0};
+#pragma unroll
+    for (int kk = 0; kk < kMlaKSteps8; ++kk) {
+      const i32x4 qa = qreg[2 * kk], qb8 = qreg[2 * kk + 1];
+#pragma unroll
+      for (int mt = 0; mt < 2; ++mt) {
+        const i32x4 ka = __builtin_bit_cast(i32x4, rr.k[mt][kk]);
+        acc[0][mt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(ka, qa, acc[0][mt], 0, 0, 0);
+        acc[1][mt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(ka, qb8, acc[1][mt], 0, 0, 0);
+      }
+    }
+    // ---- the rows' first 512 bytes into the window (chunk 4 kk + g of row 16 mt + c, swizzled)
+#pragma unroll
+    for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+      for (int kk = 0; kk < kMlaR / 64; ++kk)
+        *reinterpret_cast<u32x4*>(win + (16 * mt + c) * kMlaR + 16 * ((4 * kk + g) ^ (c & 7))) = rr.k[mt][kk];
+    const floatx4 sc0 = rr.ks[0], sc1 = rr.ks[1];
+    // the row registers are free: the wave's next tile streams in under the rest of this one
+    if (t + kMlaSmallWaves < t_end) {
+      load_rows(t + kMlaSmallWaves, rr, ids);
+      load_ids(t + 2 * kMlaSmallWaves, ids);
+    }
+
+    // ---- softmax, log2 domain; lane (c, g) holds tokens 16 mt + 4 g + i of head c
+    float logit[8];
+    float mloc = -INFINITY;
+#pragma unroll
+    for (int mt = 0; mt < 2; ++mt) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        float x = __builtin_fmaf((float)acc[1][mt][i], s2, (float)acc[0][mt][i] * s1) * ((mt ? sc1 : sc0)[i] * a.scale_log2);
+        x = t * kTile + 16 * mt + 4 * g + i < tok_end ? x : -INFINITY;
+        logit[4 * mt + i] = x;
+        mloc = fmaxf(mloc, x);
+      }
+    }
+    mloc = max_over_quarters(mloc);
+    if (__builtin_amdgcn_ballot_w64(mloc > m) != 0) {   // some head's maximum moved
+      const float m_new = fmaxf(m, mloc);
+      const float alpha = __builtin_amdgcn_exp2f(m - m_new);
+      const bool started = __builtin_amdgcn_ballot_w64(m != -INFINITY) != 0;
+      m = m_new;
+      l *= alpha;
+      if (started) {   // before the wave's first tile the accumulators are zero
+#pragma unroll
+        for (int j = 0; j < 32; ++j) o[j] *= alpha;
+      }
+    }
+    float pt[8];
+#pragma unroll
+    for (int mt = 0; mt < 2; ++mt) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float p = __builtin_amdgcn_exp2f(logit[4 * mt + i] - m);   // 0 for a masked token
+        l += p;
+        const float vs = fminf((mt ? sc1 : sc0)[i] * kPScale, 65504.f);
+        // a slot past the end may hold any bit pattern as its scale: select, do not multiply by 0
+        pt[4 * mt + i] = t * kTile + 16 * mt + 4 * g + i < tok_end ? p * vs : 0.f;
+      }
+    }
+    u32x4 pb;
+    pb.x = pack_half2(pt[0], pt[1]);
+    pb.y = pack_half2(pt[2], pt[3]);
+    pb.z = pack_half2(pt[4], pt[5]);
+    pb.w = pack_half2(pt[6], pt[7]);
+    const half8_t p_op = __builtin_bit_cast(half8_t, pb);
+
+    // ---- O^T[512 dims, 16 heads] += C^T . P~^T, 64 dims (four output tiles) at a time
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    // the dword reads of group d4 + 1 leave before group d4 is converted and multiplied
+    uint32_t xq[2][8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) xq[0][j] = *reinterpret_cast<const uint32_t*>(win + vrow_off[j] + 64 * (0 ^ vflip));
+#pragma unroll
+    for (int d4 = 0; d4 < 8; ++d4) {
+      if (d4 + 1 < 8) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+          xq[(d4 + 1) & 1][j] = *reinterpret_cast<const uint32_t*>(win + vrow_off[j] + 64 * ((d4 + 1) ^ vflip));
+      }
+      const uint32_t (&x)[8] = xq[d4 & 1];
+      o[4 * d4 + 0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(mla_code_rows_to_operand<0>(x), p_op, o[4 * d4 + 0], 0, 0, 0);
+      o[4 * d4 + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(mla_code_rows_to_operand<1>(x), p_op, o[4 * d4 + 1], 0, 0, 0);
+      o[4 * d4 + 2] = __builtin_amdgcn_mfma_f32_16x16x32_f16(mla_code_rows_to_operand<2>(x), p_op, o[4 * d4 + 2], 0, 0, 0);
+      o[4 * d4 + 3] = __builtin_amdgcn_mfma_f32_16x16x32_f16(mla_code_rows_to_operand<3>(x), p_op, o[4 * d4 + 3], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();   // the window is rewritten by the next tile
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  };
+  {
+    Rows rr;
+    TileIds ids;
+    int t = t_begin + wave;
+    if (t < t_end) {
+      load_ids(t, ids);
+      load_rows(t, rr, ids);
+      load_ids(t + kMlaSmallWaves, ids);
+    }
+    for (; t < t_end; t += kMlaSmallWaves) tile_step(rr, ids, t);
+  }
+
+  // ---- the waves' states become one.  (m, l) of every wave meet in the Q area; each wave rescales its
+  //      accumulators to the common maximum and drops them, 16 output tiles (16 KB) at a time, into its own
+  //      window; wave w then adds up, over the windows, the eight output tiles of ITS 128 dims (d4 = 2 w,
+  //      2 w + 1), normalises and emits them: the same split-state layout as the kernel above writes.
+  float* ml = reinterpret_cast<float*>(lds_raw + kMlaSmallWaves * kMlaSmallWin);   // [wave][m: 64 lanes | l: 64 lanes]
+  __syncthreads();                                                   // every wave is done with Q and with its window
+  ml[wave * 128 + lane] = m;
+  ml[wave * 128 + 64 + lane] = l;
+  __syncthreads();
+  float m_all = -INFINITY;
+#pragma unroll
+  for (int w = 0; w < kMlaSmallWaves; ++w) m_all = fmaxf(m_all, ml[w * 128 + lane]);
+  float l_all = 0.f;
+#pragma unroll
+  for (int w = 0; w < kMlaSmallWaves; ++w) {
+    const float mw = ml[w * 128 + lane];
+    l_all += mw == -INFINITY ? 0.f : ml[w * 128 + 64 + lane] * __builtin_amdgcn_exp2f(mw - m_all);
+  }
+  const float mine = m == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m - m_all);   // this wave's weight
+  floatx4 sum[8];
+#pragma unroll
+  for (int pass = 0; pass < 2; ++pass) {
+    floatx4* mywin = reinterpret_cast<floatx4*>(win);
+#pragma unroll
+    for (int j = 0; j < 16; ++j) mywin[j * kWave + lane] = o[16 * pass + j] * mine;
+    __syncthreads();
+    if ((wave >> 1) == pass) {   // output tiles 8 w .. 8 w + 7 are in this half
+#pragma unroll
+      for (int b = 0; b < 8; ++b) {
+        floatx4 acc4 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int w = 0; w < kMlaSmallWaves; ++w)
+          acc4 += reinterpret_cast<const floatx4*>(lds_raw + w * kMlaSmallWin)[(8 * (wave & 1) + b) * kWave + lane];
+        sum[b] = acc4;
+      }
+    }
+    __syncthreads();
+  }
+  l_all = sum_over_quarters(l_all);
+  const float inv = 1.0f / (l_all * kPScale);
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    uint16_t* po = a.part_o + pblock * (16 * kMlaR) + lane * 4 + (2 * wave + h) * 4 * 256;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      u32x2 v;  // a locally normalised output is a convex mix of dequantised rows: within fp16 range
+      v.x = pack_half2(clamp_half_range(sum[4 * h + 0][i] * inv), clamp_half_range(sum[4 * h + 1][i] * inv));
+      v.y = pack_half2(clamp_half_range(sum[4 * h + 2][i] * inv), clamp_half_range(sum[4 * h + 3][i] * inv));
+      *reinterpret_cast<u32x2*>(po + i * 256) = v;
+    }
+  }
+  if (wave == 0 && g == 0) a.part_lse[pblock * 16 + c] = m_all + __builtin_amdgcn_logf(l_all);
+}
+
 // Stage 2: out = sum_j 2^(lse_j - max) o_j / sum_j 2^(lse_j - max); lse = ln 2 * (max + log2 sum).
 // grid (B, ceil(H/16)), 8 waves; wave w combines the d4 = w slice of the block's 16 heads, lane (c, g)
 // as in the split state layout.
@@ -819,6 +1099,10 @@ static int mla_prepare_device() {
                                             hipFuncAttributeMaxDynamicSharedMemorySize, kMlaLdsBytes),
                         "hipFuncSetAttribute(mla_decode_kernel)"))
     return e;
+  if (int e = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(&mla_decode_small_kernel),
+                                            hipFuncAttributeMaxDynamicSharedMemorySize, kMlaSmallLdsBytes),
+                        "hipFuncSetAttribute(mla_decode_small_kernel)"))
+    return e;
   done_mask.fetch_or(bit, std::memory_order_release);
   return KVQ_OK;
 }
@@ -915,7 +1199,9 @@ static int mla_decode_run(const char* op, void* out, int out_dtype, float* lse, 
 #undef KVQ_MLAQ
   }
   if (int e = check_hip(hipGetLastError(), "mla_decode_int8 query launch")) return e;
-  if (head_groups % 8 == 0)
+  if (head_groups == 1)   // one head tile: every wave streams its own tiles
+    hipLaunchKernelGGL(mla_decode_small_kernel, dim3(splits, num_seqs), dim3(kMlaSmallThreads), kMlaSmallLdsBytes, s, a);
+  else if (head_groups % 8 == 0)
     hipLaunchKernelGGL(mla_decode_kernel<true>, grid, dim3(kMlaThreads), kMlaLdsBytes, s, a);
   else
     hipLaunchKernelGGL(mla_decode_kernel<false>, grid, dim3(kMlaThreads), kMlaLdsBytes, s, a);
