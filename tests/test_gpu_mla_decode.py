@@ -37,6 +37,9 @@ def _run(q, cache, bt, sl, scale, out_dtype=None, want_lse=True):
     (32, 128, [4096]),
     (64, 20, [5, 0, 95, 1000, 31, 32]),
     (64, 160, [70, 300, 33]),          # a second 128-head group with only two of its eight 16-head blocks
+    (64, 5, [5, 0, 95, 1000, 31, 32, 4097]),   # one head tile, partly filled; splits with fewer tiles than waves
+    (16, 16, [700] * 70),              # one head tile, more sequences than compute units / 4: one split each
+    (32, 8, [16384]),                  # one head tile, one long sequence: 64 splits
 ])
 def test_mla_decode_matches_oracle(gpu_device, dtype, bs, heads, ctx):
     cache, lay, bt, sl = _build(ctx, bs, seed=bs + heads, dtype=torch.bfloat16)

@@ -22,6 +22,7 @@ inline hipStream_t as_stream(kvq_stream_t s) { return reinterpret_cast<hipStream
 // ---- device side -----------------------------------------------------------
 typedef _Float16 half_t;
 typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
 typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));

@@ -135,6 +135,58 @@ __device__ __forceinline__ void mla_two_int8_terms(const float (&f)[16], float s
   }
 }
 
+// Dims 64 kk + 16 g .. + 15 of one head's query (k-step 8 is the rope part), as loaded -- four 16-byte words
+// for fp32 rows, two for 16-bit rows -- and as floats.  `qbase` / `pebase` are the element offsets of the
+// lane's head row plus 16 g.  Load and conversion are apart so that a caller can put other loads between.
+template <int QDT>
+struct MlaQRaw {
+  u32x4 w[QDT == KVQ_F32 ? 4 : 2];
+};
+template <int QDT>
+__device__ __forceinline__ MlaQRaw<QDT> mla_load_q16_raw(const MlaArgs& a, int64_t qbase, int64_t pebase, int kk) {
+  MlaQRaw<QDT> r;
+  if constexpr (QDT == KVQ_F32) {
+    const float* p = kk < kMlaR / 64 ? reinterpret_cast<const float*>(a.q) + qbase + 64 * kk
+                                     : reinterpret_cast<const float*>(a.q_pe) + pebase;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) r.w[i] = *reinterpret_cast<const u32x4_a4*>(p + 4 * i);
+  } else {
+    const uint16_t* p = kk < kMlaR / 64 ? reinterpret_cast<const uint16_t*>(a.q) + qbase + 64 * kk
+                                        : reinterpret_cast<const uint16_t*>(a.q_pe) + pebase;
+#pragma unroll
+    for (int h = 0; h < 2; ++h) r.w[h] = *reinterpret_cast<const u32x4_a4*>(p + 8 * h);
+  }
+  return r;
+}
+template <int QDT>
+__device__ __forceinline__ void mla_q16_to_float(const MlaQRaw<QDT>& r, float (&f)[16]) {
+  if constexpr (QDT == KVQ_F32) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) f[4 * i + j] = as_f32(r.w[i][j]);
+  } else {
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        const uint32_t e = r.w[h][w];
+        if constexpr (QDT == KVQ_BF16) {
+          f[8 * h + 2 * w] = as_f32(e << 16);
+          f[8 * h + 2 * w + 1] = as_f32(e & 0xffff0000u);
+        } else {
+          const half2_t hh = __builtin_bit_cast(half2_t, e);
+          f[8 * h + 2 * w] = (float)hh.x;
+          f[8 * h + 2 * w + 1] = (float)hh.y;
+        }
+      }
+  }
+}
+template <int QDT>
+__device__ __forceinline__ void mla_load_q16(const MlaArgs& a, int64_t qbase, int64_t pebase, int kk, float (&f)[16]) {
+  mla_q16_to_float<QDT>(mla_load_q16_raw<QDT>(a, qbase, pebase, kk), f);
+}
+
 // Q for the int8 MFMA.  The cache codes ARE int8, so the QK product can run on
 // v_mfma_i32_16x16x64_i8 straight from the cached bytes -- no conversion of K at all -- once Q is
 // int8 too: q = s1 * a + s2 * b with a = rint(q / s1), s1 = max|q| / 127 per head, and
@@ -162,38 +214,7 @@ __global__ __launch_bounds__(256) void mla_quant_q_kernel(MlaArgs a) {
   // past the last rereads the last one and is not written)
   float f[kMine][16];
 #pragma unroll
-  for (int n = 0; n < kMine; ++n) {
-    const int kk = min(wave + 4 * n, kMlaKSteps8 - 1);
-    if constexpr (QDT == KVQ_F32) {
-      // k-step 8 is the rope part
-      const float* p = kk < kMlaR / 64 ? reinterpret_cast<const float*>(a.q) + qbase + 64 * kk
-                                       : reinterpret_cast<const float*>(a.q_pe) + pebase;
-#pragma unroll
-      for (int i = 0; i < 16; i += 4) {
-        const floatx4 v = *reinterpret_cast<const floatx4_a4*>(p + i);
-        f[n][i] = v.x; f[n][i + 1] = v.y; f[n][i + 2] = v.z; f[n][i + 3] = v.w;
-      }
-    } else {
-#pragma unroll
-      for (int h = 0; h < 2; ++h) {
-        const uint16_t* p = kk < kMlaR / 64 ? reinterpret_cast<const uint16_t*>(a.q) + qbase + 64 * kk
-                                            : reinterpret_cast<const uint16_t*>(a.q_pe) + pebase;
-        const u32x4 v = *reinterpret_cast<const u32x4_a4*>(p + 8 * h);
-#pragma unroll
-        for (int w = 0; w < 4; ++w) {
-          const uint32_t e = v[w];
-          if constexpr (QDT == KVQ_BF16) {
-            f[n][8 * h + 2 * w] = as_f32(e << 16);
-            f[n][8 * h + 2 * w + 1] = as_f32(e & 0xffff0000u);
-          } else {
-            const half2_t hh = __builtin_bit_cast(half2_t, e);
-            f[n][8 * h + 2 * w] = (float)hh.x;
-            f[n][8 * h + 2 * w + 1] = (float)hh.y;
-          }
-        }
-      }
-    }
-  }
+  for (int n = 0; n < kMine; ++n) mla_load_q16<QDT>(a, qbase, pebase, min(wave + 4 * n, kMlaKSteps8 - 1), f[n]);
   float amax = 0.f;
 #pragma unroll
   for (int n = 0; n < kMine; ++n)
@@ -746,14 +767,18 @@ __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
 // keeps in registers, runs the softmax -- whose result already IS the P~ operand of the second product -- and copies
 // the rows' first 512 bytes into a wave-private, chunk-swizzled LDS window, from which it builds the fp16
 // V^T operands of all 512 output dims with dword reads and byte permutes (as the kernel above does for
-// its 64).  At the end the eight waves' states are summed through the (then idle) windows, each wave
-// adding up and emitting the 64 output dims of its number.
+// its 64).  At the end the four waves' states are summed through the (then idle) windows, each wave
+// adding up and emitting the 128 output dims of its number.
 constexpr int kMlaSmallWin = kTile * kMlaR;                                   // 16384: a tile's V part
-constexpr int kMlaSmallQBytes = 4096;                                         // (m, l) of the waves at the end
+constexpr int kMlaSmallQBytes = kMlaQOps * kWave * 16 + 256 + 2048;           // Q operands, the waves' maxima of |q|, (m, l) of the waves
 constexpr int kMlaSmallWaves = 4;   // one wave per SIMD: a wave may then use the whole register file (512 per lane)
 constexpr int kMlaSmallThreads = kMlaSmallWaves * kWave;
-constexpr int kMlaSmallLdsBytes = kMlaSmallWaves * kMlaSmallWin + kMlaSmallQBytes;         // 69632
+constexpr int kMlaSmallLdsBytes = kMlaSmallWaves * kMlaSmallWin + kMlaSmallQBytes;         // 86272
 
+// QDT >= 0: the kernel prepares the int8 operands of Q itself from the query rows of that type (every wave
+// for itself, in registers, under the latency of its first tile); QDT < 0: they were prepared by the
+// absorption kernel and are read from the workspace.
+template <int QDT>
 __global__ __launch_bounds__(kMlaSmallThreads) void mla_decode_small_kernel(MlaArgs a) {
   extern __shared__ __align__(16) uint8_t lds_raw[];
   const int tid = threadIdx.x;
@@ -775,17 +800,7 @@ __global__ __launch_bounds__(kMlaSmallThreads) void mla_decode_small_kernel(MlaA
   const int bs = a.g.block_size;
   const int32_t* bt_row = a.block_table + (int64_t)seq * a.bt_stride;
 
-  // ---- Q operands of the sequence's heads in registers (a wave owns the whole register file), s1 per head
-  const int64_t qblock = (int64_t)seq * a.head_groups;
-  i32x4 qreg[kMlaQOps];
-  {
-    const u32x4* qsrc = reinterpret_cast<const u32x4*>(a.q_ops + qblock * (kMlaQOps * kWave * 16)) + lane;
-#pragma unroll
-    for (int op = 0; op < kMlaQOps; ++op) qreg[op] = __builtin_bit_cast(i32x4, qsrc[op * kWave]);
-  }
-  const float s1 = a.q_scale[qblock * 16 + c], s2 = s1 / 254.0f;
-
-  // ---- one tile's rows in registers: kreg[mt][kk] = row 16 mt + c, dims 64 kk + 16 g .. + 15; ks[mt] = the
+  // ---- one tile's rows in registers: k[mt][kk] = row 16 mt + c, dims 64 kk + 16 g .. + 15; ks[mt] = the
   //      scales of tokens 16 mt + 4 g .. + 3 (the four logits a lane holds per half)
   struct Rows {
     u32x4 k[2][kMlaKSteps8];
@@ -804,18 +819,102 @@ __global__ __launch_bounds__(kMlaSmallThreads) void mla_decode_small_kernel(MlaA
 #pragma unroll
     for (int h = 0; h < 2; ++h) ids.blk[h] = scalar_load_i32(bt_row, (int)__umulhi((uint32_t)tile_tok(t, h), a.bs_magic));
   };
-  auto load_rows = [&](int t, Rows& rr, const TileIds& ids) __attribute__((always_inline)) {
+  // Where a tile's rows start for this lane; the loads themselves leave in pieces (a k-step of both halves at
+  // a time), spread over the arithmetic of the tile before: four waves that issue 18 KB each at the same
+  // moment queue up behind the CU's one address unit.
+  struct RowPtrs {
+    const uint8_t* row[2];
+    const uint8_t* sc[2];
+  };
+  auto row_ptrs = [&](int t, const TileIds& ids) __attribute__((always_inline)) {
+    RowPtrs rp;
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
       const int tok = tile_tok(t, h);
       const int slot = tok - (int)__umulhi((uint32_t)tok, a.bs_magic) * bs;
       const uint8_t* pb = a.cache + (int64_t)ids.blk[h] * a.g.stride_block;
-      const uint8_t* row = pb + (int64_t)(slot + c) * a.g.stride_row + 16 * g;
-#pragma unroll
-      for (int kk = 0; kk < kMlaKSteps8; ++kk) rr.k[h][kk] = *reinterpret_cast<const u32x4_a4*>(row + 64 * kk);
-      rr.ks[h] = *reinterpret_cast<const floatx4_a4*>(pb + a.g.scale_off + (int64_t)(slot + 4 * g) * 4);
+      rp.row[h] = pb + (int64_t)(slot + c) * a.g.stride_row + 16 * g;
+      rp.sc[h] = pb + a.g.scale_off + (int64_t)(slot + 4 * g) * 4;
     }
+    return rp;
   };
+  auto load_scales = [&](const RowPtrs& rp, Rows& rr) __attribute__((always_inline)) {
+#pragma unroll
+    for (int h = 0; h < 2; ++h) rr.ks[h] = *reinterpret_cast<const floatx4_a4*>(rp.sc[h]);
+  };
+  auto load_ksteps = [&](const RowPtrs& rp, Rows& rr, int kk0, int kk1) __attribute__((always_inline)) {
+#pragma unroll
+    for (int kk = kk0; kk < kk1; ++kk)
+#pragma unroll
+      for (int h = 0; h < 2; ++h) rr.k[h][kk] = *reinterpret_cast<const u32x4_a4*>(rp.row[h] + 64 * kk);
+  };
+
+  // ---- Q operands of the sequence's heads in registers (a wave owns the whole register file), s1 per head.
+  //      Order of the prologue: the loads of Q leave first (they need nothing but the sequence number), the
+  //      wave's first tile follows as soon as its block numbers are known, and the arithmetic on Q runs while
+  //      the tile is on its way.  The four waves share that arithmetic as the four waves of
+  //      mla_quant_q_kernel do (wave v: k-steps v, v + 4, v + 8) and pass the operands round through LDS.
+  constexpr int kMine = 3;
+  const int64_t qblock = (int64_t)seq * a.head_groups;
+  i32x4 qreg[kMlaQOps];
+  float s1;
+  MlaQRaw<(QDT < 0 ? KVQ_BF16 : QDT)> qraw[kMine];
+  const bool head_ok = c < a.num_heads;
+  if constexpr (QDT < 0) {
+    const u32x4* qsrc = reinterpret_cast<const u32x4*>(a.q_ops + qblock * (kMlaQOps * kWave * 16)) + lane;
+#pragma unroll
+    for (int op = 0; op < kMlaQOps; ++op) qreg[op] = __builtin_bit_cast(i32x4, qsrc[op * kWave]);
+    s1 = a.q_scale[qblock * 16 + c];
+  } else {
+    const int64_t qbase = (int64_t)seq * a.q_stride_b + (int64_t)(head_ok ? c : 0) * a.q_stride_h + 16 * g;
+    const int64_t pebase = (int64_t)seq * a.pe_stride_b + (int64_t)(head_ok ? c : 0) * a.pe_stride_h + 16 * g;
+#pragma unroll
+    for (int n = 0; n < kMine; ++n) qraw[n] = mla_load_q16_raw<QDT>(a, qbase, pebase, min(wave + 4 * n, kMlaKSteps8 - 1));
+  }
+  __builtin_amdgcn_sched_barrier(0);
+  Rows rr;
+  TileIds ids;
+  {  // unconditional (a wave without a tile reads rows it will not use; the addresses are clamped to the
+     // sequence): behind a branch, the wait for Q below would have to be a wait for every load
+    load_ids(t_begin + wave, ids);
+    const RowPtrs rp = row_ptrs(t_begin + wave, ids);
+    load_scales(rp, rr);
+    load_ksteps(rp, rr, 0, kMlaKSteps8);
+    load_ids(t_begin + wave + kMlaSmallWaves, ids);
+  }
+  __builtin_amdgcn_sched_barrier(0);
+  if constexpr (QDT >= 0) {
+    u32x4* qstage = reinterpret_cast<u32x4*>(lds_raw + kMlaSmallWaves * kMlaSmallWin);     // [18 operands][64 lanes]
+    float* part_max = reinterpret_cast<float*>(lds_raw + kMlaSmallWaves * kMlaSmallWin + kMlaQOps * kWave * 16);
+    float f[kMine][16];
+#pragma unroll
+    for (int n = 0; n < kMine; ++n) mla_q16_to_float<QDT>(qraw[n], f[n]);
+    float amax = 0.f;
+#pragma unroll
+    for (int n = 0; n < kMine; ++n)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) amax = fmaxf(amax, fabsf(f[n][i]));
+    amax = max_over_quarters(amax);
+    if (g == 0) part_max[wave * 16 + c] = amax;
+    lds_barrier();   // LDS only: the tile's loads stay in flight
+    amax = fmaxf(fmaxf(part_max[c], part_max[16 + c]), fmaxf(part_max[32 + c], part_max[48 + c]));
+    amax = head_ok ? fminf(amax, 3.0e38f) : 0.f;      // heads past the end contribute zero columns
+    s1 = amax > 0.f ? amax / 127.0f : 1.0f;
+#pragma unroll
+    for (int n = 0; n < kMine; ++n) {
+      const int kk = wave + 4 * n;
+      u32x4 ta, tb;
+      mla_two_int8_terms(f[n], s1, head_ok, ta, tb);
+      if (kk < kMlaKSteps8) {
+        qstage[(2 * kk) * kWave + lane] = ta;
+        qstage[(2 * kk + 1) * kWave + lane] = tb;
+      }
+    }
+    lds_barrier();
+#pragma unroll
+    for (int op = 0; op < kMlaQOps; ++op) qreg[op] = __builtin_bit_cast(i32x4, qstage[op * kWave + lane]);
+  }
+  const float s2 = s1 / 254.0f;
 
   floatx4 o[32];   // o[4 d4 + b][i]: head c, dim 64 d4 + 16 g + 4 i + b
 #pragma unroll
@@ -823,14 +922,15 @@ __global__ __launch_bounds__(kMlaSmallThreads) void mla_decode_small_kernel(MlaA
   float m = -INFINITY, l = 0.f;
 
   // V dwords of the lane's 8 tokens (k slot j of quarter g is token 16 (j / 4) + 4 g + j % 4) for the dims
-  // 64 d4 + 4 c .. + 3: row pitch 512, 16-byte chunk number xor (row & 7)
+  // 64 d4 + 4 c .. + 3: row pitch 512, 16-byte chunk number xor (row & 15), so that the four quarters of a
+  // wave read four different quarters of the banks
   uint32_t vrow_off[8];
 #pragma unroll
   for (int j = 0; j < 8; ++j) {
     const int row = 16 * (j >> 2) + 4 * g + (j & 3);
     vrow_off[j] = (uint32_t)(row * kMlaR + 16 * ((c >> 2) ^ (row & 3)) + 4 * (c & 3));
   }
-  const int vflip = g & 1;   // bit 2 of every one of the lane's rows: it toggles the low bit of the 64-dim group
+  const int vflip = g;   // bits 2-3 of every one of the lane's rows: they toggle the low bits of the 64-dim group
 
   auto tile_step = [&](Rows& rr, TileIds& ids, int t) __attribute__((always_inline)) {
     // ---- S^T[32 tokens, 16 heads] on the int8 MFMA, one accumulator per term of Q
@@ -854,13 +954,18 @@ __global__ __launch_bounds__(kMlaSmallThreads) void mla_decode_small_kernel(MlaA
     for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
       for (int kk = 0; kk < kMlaR / 64; ++kk)
-        *reinterpret_cast<u32x4*>(win + (16 * mt + c) * kMlaR + 16 * ((4 * kk + g) ^ (c & 7))) = rr.k[mt][kk];
+        *reinterpret_cast<u32x4*>(win + (16 * mt + c) * kMlaR + 16 * ((4 * kk + g) ^ c)) = rr.k[mt][kk];
     const floatx4 sc0 = rr.ks[0], sc1 = rr.ks[1];
     // the row registers are free: the wave's next tile streams in under the rest of this one
-    if (t + kMlaSmallWaves < t_end) {
-      load_rows(t + kMlaSmallWaves, rr, ids);
+    const bool more = t + kMlaSmallWaves < t_end;
+    RowPtrs rp;
+    if (more) {
+      rp = row_ptrs(t + kMlaSmallWaves, ids);
       load_ids(t + 2 * kMlaSmallWaves, ids);
+      load_scales(rp, rr);
+      load_ksteps(rp, rr, 0, 2);
     }
+    __builtin_amdgcn_sched_barrier(0);
 
     // ---- softmax, log2 domain; lane (c, g) holds tokens 16 mt + 4 g + i of head c
     float logit[8];
@@ -905,54 +1010,56 @@ __global__ __launch_bounds__(kMlaSmallThreads) void mla_decode_small_kernel(MlaA
     pb.z = pack_half2(pt[4], pt[5]);
     pb.w = pack_half2(pt[6], pt[7]);
     const half8_t p_op = __builtin_bit_cast(half8_t, pb);
+    __builtin_amdgcn_sched_barrier(0);
+    if (more) load_ksteps(rp, rr, 2, 4);
 
     // ---- O^T[512 dims, 16 heads] += C^T . P~^T, 64 dims (four output tiles) at a time
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    // the dword reads of group d4 + 1 leave before group d4 is converted and multiplied
+    // group d4's four operands are converted while the products of group d4 - 1 run, from dwords read a
+    // group earlier still
     uint32_t xq[2][8];
+    half8_t va[2][4];
+    auto read_group = [&](int d4) __attribute__((always_inline)) {
 #pragma unroll
-    for (int j = 0; j < 8; ++j) xq[0][j] = *reinterpret_cast<const uint32_t*>(win + vrow_off[j] + 64 * (0 ^ vflip));
+      for (int j = 0; j < 8; ++j) xq[d4 & 1][j] = *reinterpret_cast<const uint32_t*>(win + vrow_off[j] + 64 * (d4 ^ vflip));
+    };
+    auto convert_group = [&](int d4) __attribute__((always_inline)) {
+      const uint32_t (&x)[8] = xq[d4 & 1];
+      va[d4 & 1][0] = mla_code_rows_to_operand<0>(x);
+      va[d4 & 1][1] = mla_code_rows_to_operand<1>(x);
+      va[d4 & 1][2] = mla_code_rows_to_operand<2>(x);
+      va[d4 & 1][3] = mla_code_rows_to_operand<3>(x);
+    };
+    read_group(0);
+    read_group(1);
+    convert_group(0);
 #pragma unroll
     for (int d4 = 0; d4 < 8; ++d4) {
-      if (d4 + 1 < 8) {
+      if (d4 + 2 < 8) read_group(d4 + 2);
+      if (d4 < 5 && more) load_ksteps(rp, rr, 4 + d4, 5 + d4);
 #pragma unroll
-        for (int j = 0; j < 8; ++j)
-          xq[(d4 + 1) & 1][j] = *reinterpret_cast<const uint32_t*>(win + vrow_off[j] + 64 * ((d4 + 1) ^ vflip));
-      }
-      const uint32_t (&x)[8] = xq[d4 & 1];
-      o[4 * d4 + 0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(mla_code_rows_to_operand<0>(x), p_op, o[4 * d4 + 0], 0, 0, 0);
-      o[4 * d4 + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(mla_code_rows_to_operand<1>(x), p_op, o[4 * d4 + 1], 0, 0, 0);
-      o[4 * d4 + 2] = __builtin_amdgcn_mfma_f32_16x16x32_f16(mla_code_rows_to_operand<2>(x), p_op, o[4 * d4 + 2], 0, 0, 0);
-      o[4 * d4 + 3] = __builtin_amdgcn_mfma_f32_16x16x32_f16(mla_code_rows_to_operand<3>(x), p_op, o[4 * d4 + 3], 0, 0, 0);
+      for (int b = 0; b < 4; ++b)
+        o[4 * d4 + b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va[d4 & 1][b], p_op, o[4 * d4 + b], 0, 0, 0);
+      if (d4 + 1 < 8) convert_group(d4 + 1);
       __builtin_amdgcn_sched_barrier(0);
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();   // the window is rewritten by the next tile
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
   };
-  {
-    Rows rr;
-    TileIds ids;
-    int t = t_begin + wave;
-    if (t < t_end) {
-      load_ids(t, ids);
-      load_rows(t, rr, ids);
-      load_ids(t + kMlaSmallWaves, ids);
-    }
-    for (; t < t_end; t += kMlaSmallWaves) tile_step(rr, ids, t);
-  }
+  for (int t = t_begin + wave; t < t_end; t += kMlaSmallWaves) tile_step(rr, ids, t);
 
-  // ---- the waves' states become one.  (m, l) of every wave meet in the Q area; each wave rescales its
-  //      accumulators to the common maximum and drops them, 16 output tiles (16 KB) at a time, into its own
+  // ---- the waves' states become one.  (m, l) of every wave meet behind the windows; each wave brings its
+  //      accumulators to the common maximum and the common sum and drops them as fp16 (its share of a convex
+  //      mix of dequantised rows: within fp16 range, and the state is emitted in fp16 anyway) into its own
   //      window; wave w then adds up, over the windows, the eight output tiles of ITS 128 dims (d4 = 2 w,
-  //      2 w + 1), normalises and emits them: the same split-state layout as the kernel above writes.
-  float* ml = reinterpret_cast<float*>(lds_raw + kMlaSmallWaves * kMlaSmallWin);   // [wave][m: 64 lanes | l: 64 lanes]
-  __syncthreads();                                                   // every wave is done with Q and with its window
+  //      2 w + 1) and emits them: the same split-state layout as the kernel above writes.
+  float* ml = reinterpret_cast<float*>(lds_raw + kMlaSmallWaves * kMlaSmallWin + kMlaQOps * kWave * 16 + 256);   // [wave][m: 64 lanes | l: 64 lanes]
   ml[wave * 128 + lane] = m;
   ml[wave * 128 + 64 + lane] = l;
-  __syncthreads();
+  __syncthreads();                                                   // ... and every wave is done with its window
   float m_all = -INFINITY;
 #pragma unroll
   for (int w = 0; w < kMlaSmallWaves; ++w) m_all = fmaxf(m_all, ml[w * 128 + lane]);
@@ -962,36 +1069,40 @@ __global__ __launch_bounds__(kMlaSmallThreads) void mla_decode_small_kernel(MlaA
     const float mw = ml[w * 128 + lane];
     l_all += mw == -INFINITY ? 0.f : ml[w * 128 + 64 + lane] * __builtin_amdgcn_exp2f(mw - m_all);
   }
-  const float mine = m == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m - m_all);   // this wave's weight
+  l_all = sum_over_quarters(l_all);
+  // this wave's weight, with the normalisation folded in
+  const float mine = m == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m - m_all) / (l_all * kPScale);
+  {
+    u32x2* mywin = reinterpret_cast<u32x2*>(win);
+#pragma unroll
+    for (int j = 0; j < 32; ++j) {
+      u32x2 v;
+      v.x = pack_half2(clamp_half_range(o[j][0] * mine), clamp_half_range(o[j][1] * mine));
+      v.y = pack_half2(clamp_half_range(o[j][2] * mine), clamp_half_range(o[j][3] * mine));
+      mywin[j * kWave + lane] = v;
+    }
+  }
+  __syncthreads();
   floatx4 sum[8];
 #pragma unroll
-  for (int pass = 0; pass < 2; ++pass) {
-    floatx4* mywin = reinterpret_cast<floatx4*>(win);
+  for (int b = 0; b < 8; ++b) {
+    floatx4 acc4 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int j = 0; j < 16; ++j) mywin[j * kWave + lane] = o[16 * pass + j] * mine;
-    __syncthreads();
-    if ((wave >> 1) == pass) {   // output tiles 8 w .. 8 w + 7 are in this half
-#pragma unroll
-      for (int b = 0; b < 8; ++b) {
-        floatx4 acc4 = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int w = 0; w < kMlaSmallWaves; ++w)
-          acc4 += reinterpret_cast<const floatx4*>(lds_raw + w * kMlaSmallWin)[(8 * (wave & 1) + b) * kWave + lane];
-        sum[b] = acc4;
-      }
+    for (int w = 0; w < kMlaSmallWaves; ++w) {
+      const uint64_t v = reinterpret_cast<const uint64_t*>(lds_raw + w * kMlaSmallWin)[(8 * wave + b) * kWave + lane];
+      const half4_t h = __builtin_bit_cast(half4_t, v);
+      acc4 += (floatx4){(float)h[0], (float)h[1], (float)h[2], (float)h[3]};
     }
-    __syncthreads();
+    sum[b] = acc4;
   }
-  l_all = sum_over_quarters(l_all);
-  const float inv = 1.0f / (l_all * kPScale);
 #pragma unroll
   for (int h = 0; h < 2; ++h) {
     uint16_t* po = a.part_o + pblock * (16 * kMlaR) + lane * 4 + (2 * wave + h) * 4 * 256;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      u32x2 v;  // a locally normalised output is a convex mix of dequantised rows: within fp16 range
-      v.x = pack_half2(clamp_half_range(sum[4 * h + 0][i] * inv), clamp_half_range(sum[4 * h + 1][i] * inv));
-      v.y = pack_half2(clamp_half_range(sum[4 * h + 2][i] * inv), clamp_half_range(sum[4 * h + 3][i] * inv));
+      u32x2 v;
+      v.x = pack_half2(clamp_half_range(sum[4 * h + 0][i]), clamp_half_range(sum[4 * h + 1][i]));
+      v.y = pack_half2(clamp_half_range(sum[4 * h + 2][i]), clamp_half_range(sum[4 * h + 3][i]));
       *reinterpret_cast<u32x2*>(po + i * 256) = v;
     }
   }
@@ -1099,10 +1210,14 @@ static int mla_prepare_device() {
                                             hipFuncAttributeMaxDynamicSharedMemorySize, kMlaLdsBytes),
                         "hipFuncSetAttribute(mla_decode_kernel)"))
     return e;
-  if (int e = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(&mla_decode_small_kernel),
-                                            hipFuncAttributeMaxDynamicSharedMemorySize, kMlaSmallLdsBytes),
-                        "hipFuncSetAttribute(mla_decode_small_kernel)"))
-    return e;
+  const void* small[4] = {reinterpret_cast<const void*>(&mla_decode_small_kernel<-1>),
+                          reinterpret_cast<const void*>(&mla_decode_small_kernel<KVQ_F32>),
+                          reinterpret_cast<const void*>(&mla_decode_small_kernel<KVQ_BF16>),
+                          reinterpret_cast<const void*>(&mla_decode_small_kernel<KVQ_F16>)};
+  for (const void* k : small)
+    if (int e = check_hip(hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, kMlaSmallLdsBytes),
+                          "hipFuncSetAttribute(mla_decode_small_kernel)"))
+      return e;
   done_mask.fetch_or(bit, std::memory_order_release);
   return KVQ_OK;
 }
@@ -1187,7 +1302,7 @@ static int mla_decode_run(const char* op, void* out, int out_dtype, float* lse, 
       else KVQ_MLAA(KVQ_F16, 0);
     }
 #undef KVQ_MLAA
-  } else {
+  } else if (head_groups > 1) {   // the kernel for one head tile prepares its operands itself
     dim3 qgrid(num_seqs, head_groups);
 #define KVQ_MLAQ(T) hipLaunchKernelGGL((mla_quant_q_kernel<T>), qgrid, dim3(256), 0, s, a)
     switch (q_dtype) {
@@ -1199,9 +1314,16 @@ static int mla_decode_run(const char* op, void* out, int out_dtype, float* lse, 
 #undef KVQ_MLAQ
   }
   if (int e = check_hip(hipGetLastError(), "mla_decode_int8 query launch")) return e;
-  if (head_groups == 1)   // one head tile: every wave streams its own tiles
-    hipLaunchKernelGGL(mla_decode_small_kernel, dim3(splits, num_seqs), dim3(kMlaSmallThreads), kMlaSmallLdsBytes, s, a);
-  else if (head_groups % 8 == 0)
+  if (head_groups == 1) {   // one head tile: every wave streams its own tiles
+#define KVQ_MLAS(T) \
+  hipLaunchKernelGGL((mla_decode_small_kernel<T>), dim3(splits, num_seqs), dim3(kMlaSmallThreads), kMlaSmallLdsBytes, s, a)
+    if (absorb != nullptr) KVQ_MLAS(-1);
+    else if (q_dtype == KVQ_F32) KVQ_MLAS(KVQ_F32);
+    else if (q_dtype == KVQ_BF16) KVQ_MLAS(KVQ_BF16);
+    else if (q_dtype == KVQ_F16) KVQ_MLAS(KVQ_F16);
+    else return fail(KVQ_EINVAL, "%s: unknown q_dtype %d", op, q_dtype);
+#undef KVQ_MLAS
+  } else if (head_groups % 8 == 0)
     hipLaunchKernelGGL(mla_decode_kernel<true>, grid, dim3(kMlaThreads), kMlaLdsBytes, s, a);
   else
     hipLaunchKernelGGL(mla_decode_kernel<false>, grid, dim3(kMlaThreads), kMlaLdsBytes, s, a);
