@@ -1130,30 +1130,49 @@ __global__ __launch_bounds__(512) void mla_reduce_kernel(void* out, float* lse, 
   for (int r = 0; r < 4; ++r) acc[r] = (floatx4){0.f, 0.f, 0.f, 0.f};
   float mx = -INFINITY;
   const bool live = seq_lens[seq] > 0;
-#pragma unroll 8
-  for (int j = 0; j < num_splits; ++j) mx = fmaxf(mx, pl[j * lstride]);
-  mx = live ? mx : -INFINITY;
-  const float mref = mx == -INFINITY ? 0.f : mx;
   float den = 0.f;
-  // every load below is unconditional and a split that holds nothing (lse = -inf; its state rows were
-  // never written) is removed with a bit mask on the loaded words: a select on the value would be
-  // turned into a branch around the load, and the loads of successive splits would run one by one
-#pragma unroll 8
-  for (int j = 0; j < num_splits; ++j) {
-    const float lj = pl[j * lstride];
-    const float wj = (live && lj != -INFINITY) ? __builtin_amdgcn_exp2f(lj - mref) : 0.f;
-    const uint32_t keep = wj != 0.f ? 0xffffffffu : 0u;
-    den += wj;
-    const uint16_t* pj = po + j * ostride;
+  // Eight splits at a time, and all loads of a group -- the eight lse values and the eight states -- leave
+  // before anything is computed from them: one trip to memory per group instead of two (the maximum first,
+  // then the states).  The running maximum moves between groups, with the usual rescaling.
+  // Every load is unconditional and a split that holds nothing (lse = -inf; its state rows were never
+  // written) is removed with a bit mask on the loaded words: a select on the value would be turned into
+  // a branch around the load, and the loads of successive splits would run one by one.
+  for (int j0 = 0; j0 < num_splits; j0 += 8) {
+    float lj[8];
+    u32x2 hv[8][4];
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      const u32x2 hv = *reinterpret_cast<const u32x2*>(pj + r * 256);
-      const uint32_t h0 = hv.x & keep, h1 = hv.y & keep;
-      const half2_t a0 = __builtin_bit_cast(half2_t, h0), a1 = __builtin_bit_cast(half2_t, h1);
-      acc[r].x += (float)a0.x * wj;
-      acc[r].y += (float)a0.y * wj;
-      acc[r].z += (float)a1.x * wj;
-      acc[r].w += (float)a1.y * wj;
+    for (int u = 0; u < 8; ++u) {
+      const int j = min(j0 + u, num_splits - 1);   // a slot past the last split rereads the last one and weighs 0
+      lj[u] = pl[j * lstride];
+      const uint16_t* pj = po + j * ostride;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) hv[u][r] = *reinterpret_cast<const u32x2*>(pj + r * 256);
+    }
+    float cm = -INFINITY;
+#pragma unroll
+    for (int u = 0; u < 8; ++u) cm = fmaxf(cm, (live && j0 + u < num_splits) ? lj[u] : -INFINITY);
+    const float m_new = fmaxf(mx, cm);
+    const float mref = m_new == -INFINITY ? 0.f : m_new;
+    const float alpha = mx == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mx - mref);
+    mx = m_new;
+    den *= alpha;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) acc[r] *= alpha;
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const bool on = live && j0 + u < num_splits && lj[u] != -INFINITY;
+      const float wj = on ? __builtin_amdgcn_exp2f(lj[u] - mref) : 0.f;
+      const uint32_t keep = wj != 0.f ? 0xffffffffu : 0u;
+      den += wj;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const uint32_t h0 = hv[u][r].x & keep, h1 = hv[u][r].y & keep;
+        const half2_t a0 = __builtin_bit_cast(half2_t, h0), a1 = __builtin_bit_cast(half2_t, h1);
+        acc[r].x += (float)a0.x * wj;
+        acc[r].y += (float)a0.y * wj;
+        acc[r].z += (float)a1.x * wj;
+        acc[r].w += (float)a1.y * wj;
+      }
     }
   }
   if (!head_ok) return;
