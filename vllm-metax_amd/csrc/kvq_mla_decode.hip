@@ -187,6 +187,26 @@ __device__ __forceinline__ void mla_load_q16(const MlaArgs& a, int64_t qbase, in
   mla_q16_to_float<QDT>(mla_load_q16_raw<QDT>(a, qbase, pebase, kk), f);
 }
 
+// Which (sequence, split) a workgroup of the (splits, sequences) grid takes.  Workgroups go to the eight XCDs
+// (each with an L2 of its own) round-robin in launch order, so with the plain mapping the splits of one
+// sequence sit on eight different XCDs: each fetches the sequence's query operands for itself, and the
+// reduce kernel finds none of the sequence's split states in its L2.  Here all splits of a sequence share
+// the XCD "sequence mod 8" -- the one that mla_quant_q_kernel and mla_reduce_kernel (grids with the
+// sequence as x) run that sequence on.  Sequences past the last multiple of eight keep the plain mapping.
+__device__ __forceinline__ void mla_seq_split_of_block(int num_seqs, int num_splits, int& seq, int& split) {
+  const int n = blockIdx.x + gridDim.x * blockIdx.y;
+  const int seqs8 = num_seqs & ~7;
+  if (n < seqs8 * num_splits) {
+    const int xcd = n & 7, k = n >> 3;
+    seq = (k / num_splits) * 8 + xcd;
+    split = k % num_splits;
+  } else {
+    const int r = n - seqs8 * num_splits;
+    seq = seqs8 + r / num_splits;
+    split = r % num_splits;
+  }
+}
+
 // Q for the int8 MFMA.  The cache codes ARE int8, so the QK product can run on
 // v_mfma_i32_16x16x64_i8 straight from the cached bytes -- no conversion of K at all -- once Q is
 // int8 too: q = s1 * a + s2 * b with a = rint(q / s1), s1 = max|q| / 127 per head, and
@@ -403,7 +423,8 @@ __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int c = lane & 15, g = lane >> 4;
-  const int seq = blockIdx.y, split = blockIdx.x;
+  int seq, split;
+  mla_seq_split_of_block(gridDim.y, a.num_splits, seq, split);
   const int len = a.seq_lens[seq];
   const int slen = mla_split_len(len > 0 ? len : 0, a.num_splits);
   const int tok_begin = split * slen;
@@ -786,7 +807,8 @@ __global__ __launch_bounds__(kMlaSmallThreads) void mla_decode_small_kernel(MlaA
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int c = lane & 15, g = lane >> 4;
   uint8_t* win = lds_raw + wave * kMlaSmallWin;
-  const int seq = blockIdx.y, split = blockIdx.x;
+  int seq, split;
+  mla_seq_split_of_block(gridDim.y, a.num_splits, seq, split);
   const int len = a.seq_lens[seq];
   const int slen = mla_split_len(len > 0 ? len : 0, a.num_splits);
   const int tok_begin = split * slen;
