@@ -20,8 +20,12 @@
 // second copy of the tile in LDS; it reads eight P~ operands per tile.  One workgroup barrier per
 // tile (P~ and the next raw tile visible); the third window is what lets the P~V read the raw tile
 // after that barrier while the tile after the next already streams in.
+// With at most 16 heads (one head tile, the shape of a tensor-parallel shard) a second kernel takes
+// over, mla_decode_small_kernel: four waves, each streaming its own tiles straight from global memory
+// into the int8 MFMA's operand order, with the query quantised inside the kernel.
 // The token splits of a sequence are merged by the reduce kernel with the log-sum-exp algebra
-// (same two-stage shape as the reference's decode_attention_fwd); nothing is allocated here,
+// (same two-stage shape as the reference's decode_attention_fwd); all splits of a sequence run on the
+// XCD that prepares its query and reduces it (mla_seq_split_of_block).  Nothing is allocated here,
 // partials and the int8 Q live in the caller's workspace.
 #include <atomic>
 #include <type_traits>
