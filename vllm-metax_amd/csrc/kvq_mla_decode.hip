@@ -10,8 +10,8 @@
 // (buffer_load ... lds, no registers in between), a whole tile time ahead of its use; the 16-byte
 // chunks of a row are swizzled so that operand reads are free of bank conflicts without padding.
 // QK: wave w owns head tile w (16 heads) of the block and computes that tile's logits on the int8
-// MFMA straight from the cached code bytes; its absorbed Q sits in registers (10 of its 18
-// operands) and LDS (the other 8) as two int8 terms that a small kernel prepares once per launch.
+// MFMA straight from the cached code bytes; its absorbed Q sits in registers (16 of its 18
+// operands) and LDS (the other 2) as two int8 terms that a small kernel prepares once per launch.
 // It runs the tile's softmax (lazy reference maximum) and publishes the P~ operand, the rescale
 // factors and a "maximum moved" flag through a double-buffered LDS exchange.
 // PV is split over the waves by OUTPUT DIMS, not by heads: wave w accumulates dims 64 w .. 64 w + 63
@@ -43,8 +43,8 @@ constexpr int kChunksPerHalf = 16 * kChunksPerRow;        // 576
 constexpr int kMlaThreads = 512;
 constexpr int kMlaKSteps8 = kMlaW / 64;                   // 9 int8 k-steps of 64 dims
 constexpr int kMlaQOps = 2 * kMlaKSteps8;                 // B operands of Q: two int8 terms per k-step
-constexpr int kMlaQRegOps = 10;                           // operands of Q kept in registers; the rest in LDS
-constexpr int kMlaQLdsBytes = (kMlaQOps - kMlaQRegOps) * kMlaThreads * 16;  // 65536
+constexpr int kMlaQRegOps = 16;                           // operands of Q kept in registers; the rest in LDS
+constexpr int kMlaQLdsBytes = (kMlaQOps - kMlaQRegOps) * kMlaThreads * 16;  // 16384
 constexpr int kMlaRing = 3;                               // raw tile windows: tile t is read (QK, then PV) while t + 1 and t + 2 stream in
 typedef int32_t i32x4 __attribute__((ext_vector_type(4)));
 // What the head-owning waves hand to the others, per tile and double-buffered: the eight P~ operands
