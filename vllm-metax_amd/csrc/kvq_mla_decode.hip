@@ -81,14 +81,6 @@ struct MlaArgs {
   uint32_t bs_magic;
 };
 
-// Bytes (0,1) or (2,3) of x (codes ^ 0x80) as two exact fp16 codes: 0x6400 | byte is 1024 + byte =
-// code + 1152; the constant is subtracted again (exact in fp16).
-__device__ __forceinline__ uint32_t mla_codes_to_half2(uint32_t x, bool upper) {
-  const half2_t bias = {(half_t)kCodeBias, (half_t)kCodeBias};
-  const half2_t v = __builtin_bit_cast(half2_t, bytes_to_half2(x, upper)) - bias;
-  return __builtin_bit_cast(uint32_t, v);
-}
-
 // Byte B of x0 and of x1, each a signed code, as the fp16 pair (x0.B, x1.B): the conversion reads its
 // byte through the operand's sub-dword select with sign extension and writes one half of the result, so
 // a pair costs two instructions and no shuffles.
@@ -552,8 +544,8 @@ __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
   // ---- V^T operands of the tile, built in registers from the raw tile.  Wave w accumulates dims
   //      64 w .. 64 w + 63 of all heads; output tile 4 w + b, row r' is dim 64 w + 4 r' + b.  A lane (r', g)
   //      reads one dword -- its four dims -- from each of the 8 token rows its P~ operand holds (k slot j of
-  //      quarter g is token 16 (j / 4) + 4 g + j % 4), transposes the 8 x 4 byte block with byte permutes and
-  //      turns each dim's 8 codes into one fp16 A operand.  Rows 4 g + i and 16 + 4 g + i share their swizzle
+  //      quarter g is token 16 (j / 4) + 4 g + j % 4) and turns each dim's 8 codes into one fp16 A operand
+  //      with sign-extending sub-dword conversions (two instructions per pair of codes, no shuffles).  Rows 4 g + i and 16 + 4 g + i share their swizzle
   //      in pairs: two loop-invariant offsets, the rest are immediates.
   const uint32_t vo_a = (uint32_t)(4 * g * kMlaPitch + 16 * (4 * wave + ((c >> 2) ^ ((2 * g) & 3))) + 4 * (c & 3));
   const uint32_t vo_b = (uint32_t)(4 * g * kMlaPitch + 16 * (4 * wave + ((c >> 2) ^ ((2 * g + 1) & 3))) + 4 * (c & 3));
@@ -561,22 +553,11 @@ __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
     uint32_t x[8];
 #pragma unroll
     for (int j = 0; j < 8; ++j)
-      x[j] = *reinterpret_cast<const uint32_t*>(tile + ((j & 2) ? vo_b : vo_a) + (16 * (j >> 2) + (j & 3)) * kMlaPitch) ^ 0x80808080u;
-    uint32_t lo[4], hi[4];   // token pairs (0,1) (2,3) (4,5) (6,7): dims 0,1 interleaved / dims 2,3 interleaved
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      lo[q] = perm(x[2 * q + 1], x[2 * q], 0x05010400u);
-      hi[q] = perm(x[2 * q + 1], x[2 * q], 0x07030602u);
-    }
-#pragma unroll
-    for (int b = 0; b < 4; ++b) {
-      u32x4 h;
-      h.x = mla_codes_to_half2(b < 2 ? lo[0] : hi[0], b & 1);
-      h.y = mla_codes_to_half2(b < 2 ? lo[1] : hi[1], b & 1);
-      h.z = mla_codes_to_half2(b < 2 ? lo[2] : hi[2], b & 1);
-      h.w = mla_codes_to_half2(b < 2 ? lo[3] : hi[3], b & 1);
-      va[b] = __builtin_bit_cast(half8_t, h);
-    }
+      x[j] = *reinterpret_cast<const uint32_t*>(tile + ((j & 2) ? vo_b : vo_a) + (16 * (j >> 2) + (j & 3)) * kMlaPitch);
+    va[0] = mla_code_rows_to_operand<0>(x);
+    va[1] = mla_code_rows_to_operand<1>(x);
+    va[2] = mla_code_rows_to_operand<2>(x);
+    va[3] = mla_code_rows_to_operand<3>(x);
   };
 
   stage_scales(lds[0]);
