@@ -309,7 +309,7 @@ def mla_main(args, cfg, dev, ops):
         "prewarm_s": PREWARM_S, "us_per_layer": round(dt * 1e6, 2), "attn_launch_us": round(attn_s * 1e6, 2),
         "roofline": {**roof, "traffic": traffic, "traffic_source": traffic_source,
                      "kernel": ("MLA decode launch on an absorbed query = mla_decode_small_kernel + mla_reduce_kernel" if small else
-                                "MLA decode launch on an absorbed query = mla_quant_q_kernel + mla_decode_kernel + mla_reduce_kernel"),
+                                "MLA decode launch on an absorbed query = mla_decode_kernel (quantises the query itself) + mla_reduce_kernel"),
                      "timing": f"{n_ev} decode launches back to back between two events on the launch stream",
                      "algorithmic_flops_per_launch": flops, "algorithmic_bytes_per_launch": nbytes,
                      "hbm_frac_of_peak": round(nbytes / attn_s / 1e9 / HBM_PEAK_GBPS, 4)},

@@ -70,7 +70,7 @@ struct MlaArgs {
   // log2 domain, -inf for an empty split.
   uint16_t* part_o;
   float* part_lse;
-  // Q as the int8 MFMA wants it (written by mla_quant_q_kernel, read by every split of a sequence):
+  // Q as the int8 MFMA wants it (written by mla_absorb_q_kernel, read by every split of a sequence):
   // q_ops [B, ceil(H/16)][18 operands][64 lanes][16 bytes], q_scale [B, 16 * ceil(H/16)] = s1 per head.
   uint8_t* q_ops;
   float* q_scale;
@@ -107,7 +107,7 @@ __device__ __forceinline__ int mla_split_len(int len, int num_splits) {
   return ((per + kTile - 1) / kTile) * kTile;
 }
 
-// 16 values of one head -> the 16 bytes of each of the two int8 terms (see mla_quant_q_kernel): a =
+// 16 values of one head -> the 16 bytes of each of the two int8 terms: a =
 // rint(q / s1), b = rint((q - s1 a) * 254 / s1).  `live` false gives zero bytes (heads past the end).
 __device__ __forceinline__ void mla_two_int8_terms(const float (&f)[16], float s1, bool live, u32x4& ta, u32x4& tb) {
   const float inv1 = 1.0f / s1, inv2 = 254.0f * inv1;
@@ -178,17 +178,12 @@ __device__ __forceinline__ void mla_q16_to_float(const MlaQRaw<QDT>& r, float (&
       }
   }
 }
-template <int QDT>
-__device__ __forceinline__ void mla_load_q16(const MlaArgs& a, int64_t qbase, int64_t pebase, int kk, float (&f)[16]) {
-  mla_q16_to_float<QDT>(mla_load_q16_raw<QDT>(a, qbase, pebase, kk), f);
-}
-
 // Which (sequence, split) a workgroup of the (splits, sequences) grid takes.  Workgroups go to the eight XCDs
 // (each with an L2 of its own) round-robin in launch order, so with the plain mapping the splits of one
 // sequence sit on eight different XCDs: each fetches the sequence's query operands for itself, and the
 // reduce kernel finds none of the sequence's split states in its L2.  Here all splits of a sequence share
-// the XCD "sequence mod 8" -- the one that mla_quant_q_kernel and mla_reduce_kernel (grids with the
-// sequence as x) run that sequence on.  Sequences past the last multiple of eight keep the plain mapping.
+// the XCD "sequence mod 8" -- the one that mla_reduce_kernel (a grid with the sequence as x) runs that
+// sequence on.  Sequences past the last multiple of eight keep the plain mapping.
 __device__ __forceinline__ void mla_seq_split_of_block(int num_seqs, int num_splits, int& seq, int& split) {
   const int n = blockIdx.x + gridDim.x * blockIdx.y;
   const int seqs8 = num_seqs & ~7;
@@ -208,58 +203,15 @@ __device__ __forceinline__ void mla_seq_split_of_block(int num_seqs, int num_spl
 // int8 too: q = s1 * a + s2 * b with a = rint(q / s1), s1 = max|q| / 127 per head, and
 // b = rint((q - s1 a) / s2), s2 = s1 / 254.  The residual after two terms is at most
 // s2 / 2 = max|q| / 64516, finer than the fp16 rounding of q it replaces, and the integer dot
-// products are exact.  One workgroup per (sequence, 16 heads), once per launch (every token split of the
-// sequence reads the result): lane (c = head, g) produces, for k-step kk, dims 64 kk + 16 g + j
-// (j < 16) as 16 bytes, operand 2 kk = term a, operand 2 kk + 1 = term b.
-template <int QDT>
-__global__ __launch_bounds__(256) void mla_quant_q_kernel(MlaArgs a) {
-  // 4 waves share the 9 k-steps of a (sequence, 16 heads) block: wave v takes k-steps v, v + 4, v + 8
-  constexpr int kMine = 3;
-  __shared__ float part_max[4][16];
-  const int lane = threadIdx.x & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int c = lane & 15, g = lane >> 4;
-  const int seq = blockIdx.x, hgroup = blockIdx.y;
-  const int head = hgroup * 16 + c;
-  const bool head_ok = head < a.num_heads;
-  const int64_t qblock = (int64_t)seq * a.head_groups + hgroup;
-  u32x4* qdst = reinterpret_cast<u32x4*>(a.q_ops + qblock * (kMlaQOps * kWave * 16)) + lane;
-  const int64_t qbase = (int64_t)seq * a.q_stride_b + (int64_t)(head_ok ? head : 0) * a.q_stride_h + 16 * g;
-  const int64_t pebase = (int64_t)seq * a.pe_stride_b + (int64_t)(head_ok ? head : 0) * a.pe_stride_h + 16 * g;
-  // the wave's values as floats: f[n][i] = dim 64 kk + 16 g + i of k-step kk = wave + 4 n (a k-step
-  // past the last rereads the last one and is not written)
-  float f[kMine][16];
-#pragma unroll
-  for (int n = 0; n < kMine; ++n) mla_load_q16<QDT>(a, qbase, pebase, min(wave + 4 * n, kMlaKSteps8 - 1), f[n]);
-  float amax = 0.f;
-#pragma unroll
-  for (int n = 0; n < kMine; ++n)
-#pragma unroll
-    for (int i = 0; i < 16; ++i) amax = fmaxf(amax, fabsf(f[n][i]));
-  amax = fmaxf(amax, __shfl_xor(amax, 16, kWave));
-  amax = fmaxf(amax, __shfl_xor(amax, 32, kWave));
-  if (g == 0) part_max[wave][c] = amax;
-  __syncthreads();
-  amax = fmaxf(fmaxf(part_max[0][c], part_max[1][c]), fmaxf(part_max[2][c], part_max[3][c]));
-  amax = head_ok ? fminf(amax, 3.0e38f) : 0.f;      // heads past the end contribute zero columns
-  const float s1 = amax > 0.f ? amax / 127.0f : 1.0f;
-#pragma unroll
-  for (int n = 0; n < kMine; ++n) {
-    const int kk = wave + 4 * n;
-    u32x4 ta, tb;
-    mla_two_int8_terms(f[n], s1, head_ok, ta, tb);
-    if (kk < kMlaKSteps8) {
-      qdst[(2 * kk) * kWave] = ta;
-      qdst[(2 * kk + 1) * kWave] = tb;
-    }
-  }
-  if (wave == 0 && g == 0) a.q_scale[qblock * 16 + c] = s1;
-}
+// products are exact.  For a (sequence, 16 heads) block, lane (c = head, g) holds, for k-step kk, dims
+// 64 kk + 16 g + j (j < 16) as 16 bytes, operand 2 kk = term a, operand 2 kk + 1 = term b.  The decode
+// kernels build these operands in their prologues (mla_two_int8_terms); only the absorption kernel below
+// writes them to the workspace.
 
 // Q absorption fused with the int8 preparation: ql[b, h, :] = q_nope[b, h, :] . W_UK_T[h] (the first
 // bmm of the reference's MLA layer, mla_attention.py:835-848) computed on the MFMA and written
 // STRAIGHT into the decode's operand layout as two int8 terms + s1 -- the absorbed query never exists
-// in HBM as bf16 and mla_quant_q_kernel does not run.
+// in HBM as bf16.
 // Workgroup = (head, 16 sequences), 4 waves; wave w owns latent dims 128 w .. 128 w + 127.  The product
 // is taken transposed, ql^T = W^T q^T: B = q_nope rows (lane = sequence, 8 consecutive p), A = W^T needs 8
 // p of one dim per lane while W_UK_T [P, L] keeps 8 dims of one p together, so each lane loads the
@@ -408,7 +360,10 @@ __global__ __launch_bounds__(256) void mla_absorb_q_kernel(MlaAbsorbArgs a) {
 }
 
 // FULL: every 128-head block of the launch has its eight head tiles (num_heads a multiple of 128)
-template <bool FULL>
+// QDT >= 0: every owner wave quantises the query of its 16 heads itself, from rows of that type (its loads leave
+// before the first tile's, its arithmetic runs while the tile streams in); QDT < 0: the operands were prepared
+// by the absorption kernel and are read from the workspace.
+template <bool FULL, int QDT>
 __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
   extern __shared__ __align__(16) uint8_t lds_raw[];
   uint8_t(*lds)[kMlaBufBytes] = reinterpret_cast<uint8_t(*)[kMlaBufBytes]>(lds_raw);   // kMlaRing raw windows
@@ -507,27 +462,65 @@ __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
   };
 
+  // ---- Q of the 16 heads this wave owns as int8 B operands (operand 2 kk = first term, 2 kk + 1 = second term
+  //      of k-step kk; lane (c = head, g) holds dims 64 kk + 16 g + j)
+  const int own_head = hgroup * 16 + c;
+  const bool head_ok = own_head < a.num_heads;
+  MlaQRaw<(QDT < 0 ? KVQ_BF16 : QDT)> qraw[QDT < 0 ? 1 : kMlaKSteps8];
+  if constexpr (QDT >= 0) {
+    if (owner) {
+      const int64_t qbase = (int64_t)seq * a.q_stride_b + (int64_t)(head_ok ? own_head : 0) * a.q_stride_h + 16 * g;
+      const int64_t pebase = (int64_t)seq * a.pe_stride_b + (int64_t)(head_ok ? own_head : 0) * a.pe_stride_h + 16 * g;
+#pragma unroll
+      for (int kk = 0; kk < kMlaKSteps8; ++kk) qraw[kk] = mla_load_q16_raw<QDT>(a, qbase, pebase, kk);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  }
   issue_loads(fetch_blocks(t_begin), lds[0]);
   Blocks nb = fetch_blocks(t_begin + 1);
+  __builtin_amdgcn_sched_barrier(0);
 
-  // ---- absorbed Q of the 16 heads this wave owns: the int8 B operands mla_quant_q_kernel prepared
-  //      (operand 2 kk = first term, 2 kk + 1 = second term of k-step kk; lane (c = head, g) holds
-  //      dims 64 kk + 16 g + j)
   i32x4 qreg[kMlaQRegOps];
   float s1 = 1.f, s2 = 0.f;
   if (owner) {
-    const int64_t qblock = (int64_t)seq * a.head_groups + hgroup;
-    const u32x4* qsrc = reinterpret_cast<const u32x4*>(a.q_ops + qblock * (kMlaQOps * kWave * 16)) + lane;
-    u32x4 raw[kMlaQOps];
+    if constexpr (QDT < 0) {
+      const int64_t qblock = (int64_t)seq * a.head_groups + hgroup;
+      const u32x4* qsrc = reinterpret_cast<const u32x4*>(a.q_ops + qblock * (kMlaQOps * kWave * 16)) + lane;
+      u32x4 raw[kMlaQOps];
 #pragma unroll
-    for (int op = 0; op < kMlaQOps; ++op) raw[op] = qsrc[op * kWave];
-    s1 = a.q_scale[qblock * 16 + c];
-    s2 = s1 / 254.0f;
+      for (int op = 0; op < kMlaQOps; ++op) raw[op] = qsrc[op * kWave];
+      s1 = a.q_scale[qblock * 16 + c];
 #pragma unroll
-    for (int op = 0; op < kMlaQOps; ++op) {
-      if (op < kMlaQRegOps) qreg[op] = __builtin_bit_cast(i32x4, raw[op]);
-      else qlds[(op - kMlaQRegOps) * kMlaThreads] = raw[op];
+      for (int op = 0; op < kMlaQOps; ++op) {
+        if (op < kMlaQRegOps) qreg[op] = __builtin_bit_cast(i32x4, raw[op]);
+        else qlds[(op - kMlaQRegOps) * kMlaThreads] = raw[op];
+      }
+    } else {   // the two int8 terms of the wave's own 16 heads
+      float f[kMlaKSteps8][16];
+#pragma unroll
+      for (int kk = 0; kk < kMlaKSteps8; ++kk) mla_q16_to_float<QDT>(qraw[kk], f[kk]);
+      float amax = 0.f;
+#pragma unroll
+      for (int kk = 0; kk < kMlaKSteps8; ++kk)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) amax = fmaxf(amax, fabsf(f[kk][i]));
+      amax = max_over_quarters(amax);
+      amax = head_ok ? fminf(amax, 3.0e38f) : 0.f;      // heads past the end contribute zero columns
+      s1 = amax > 0.f ? amax / 127.0f : 1.0f;
+#pragma unroll
+      for (int kk = 0; kk < kMlaKSteps8; ++kk) {
+        u32x4 ta, tb;
+        mla_two_int8_terms(f[kk], s1, head_ok, ta, tb);
+        if (2 * kk < kMlaQRegOps) {
+          qreg[2 * kk] = __builtin_bit_cast(i32x4, ta);
+          qreg[2 * kk + 1] = __builtin_bit_cast(i32x4, tb);
+        } else {
+          qlds[(2 * kk - kMlaQRegOps) * kMlaThreads] = ta;
+          qlds[(2 * kk + 1 - kMlaQRegOps) * kMlaThreads] = tb;
+        }
+      }
     }
+    s2 = s1 / 254.0f;
   } else {
 #pragma unroll
     for (int op = 0; op < kMlaQRegOps; ++op) qreg[op] = (i32x4){0, 0, 0, 0};
@@ -859,8 +852,8 @@ __global__ __launch_bounds__(kMlaSmallThreads) void mla_decode_small_kernel(MlaA
   // ---- Q operands of the sequence's heads in registers (a wave owns the whole register file), s1 per head.
   //      Order of the prologue: the loads of Q leave first (they need nothing but the sequence number), the
   //      wave's first tile follows as soon as its block numbers are known, and the arithmetic on Q runs while
-  //      the tile is on its way.  The four waves share that arithmetic as the four waves of
-  //      mla_quant_q_kernel do (wave v: k-steps v, v + 4, v + 8) and pass the operands round through LDS.
+  //      the tile is on its way.  The four waves share that arithmetic (wave v: k-steps v, v + 4, v + 8) and
+  //      pass the operands round through LDS.
   constexpr int kMine = 3;
   const int64_t qblock = (int64_t)seq * a.head_groups;
   i32x4 qreg[kMlaQOps];
@@ -1228,14 +1221,18 @@ static int mla_prepare_device() {
   if (int e = check_hip(hipGetDevice(&dev), "hipGetDevice")) return e;
   const uint64_t bit = dev >= 0 && dev < 64 ? (1ull << dev) : 0;
   if (bit != 0 && (done_mask.load(std::memory_order_acquire) & bit)) return KVQ_OK;
-  if (int e = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(&mla_decode_kernel<true>),
-                                            hipFuncAttributeMaxDynamicSharedMemorySize, kMlaLdsBytes),
-                        "hipFuncSetAttribute(mla_decode_kernel)"))
-    return e;
-  if (int e = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(&mla_decode_kernel<false>),
-                                            hipFuncAttributeMaxDynamicSharedMemorySize, kMlaLdsBytes),
-                        "hipFuncSetAttribute(mla_decode_kernel)"))
-    return e;
+  const void* big[8] = {reinterpret_cast<const void*>(&mla_decode_kernel<true, -1>),
+                        reinterpret_cast<const void*>(&mla_decode_kernel<true, KVQ_F32>),
+                        reinterpret_cast<const void*>(&mla_decode_kernel<true, KVQ_BF16>),
+                        reinterpret_cast<const void*>(&mla_decode_kernel<true, KVQ_F16>),
+                        reinterpret_cast<const void*>(&mla_decode_kernel<false, -1>),
+                        reinterpret_cast<const void*>(&mla_decode_kernel<false, KVQ_F32>),
+                        reinterpret_cast<const void*>(&mla_decode_kernel<false, KVQ_BF16>),
+                        reinterpret_cast<const void*>(&mla_decode_kernel<false, KVQ_F16>)};
+  for (const void* k : big)
+    if (int e = check_hip(hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, kMlaLdsBytes),
+                          "hipFuncSetAttribute(mla_decode_kernel)"))
+      return e;
   const void* small[4] = {reinterpret_cast<const void*>(&mla_decode_small_kernel<-1>),
                           reinterpret_cast<const void*>(&mla_decode_small_kernel<KVQ_F32>),
                           reinterpret_cast<const void*>(&mla_decode_small_kernel<KVQ_BF16>),
@@ -1250,7 +1247,7 @@ static int mla_prepare_device() {
 
 }  // namespace kvq
 
-// Both entry points: `absorb` NULL = q holds the absorbed query (prepared by mla_quant_q_kernel), else q
+// Both entry points: `absorb` NULL = q holds the absorbed query (quantised by the decode kernel itself), else q
 // is unused and the absorb kernel prepares the operands from (q_nope, W_UK_T, q_pe).
 static int mla_decode_run(const char* op, void* out, int out_dtype, float* lse, const void* q, int q_dtype,
                           int64_t q_stride_b, int64_t q_stride_h, const void* q_pe, int64_t q_pe_stride_b,
@@ -1328,17 +1325,9 @@ static int mla_decode_run(const char* op, void* out, int out_dtype, float* lse, 
       else KVQ_MLAA(KVQ_F16, 0);
     }
 #undef KVQ_MLAA
-  } else if (head_groups > 1) {   // the kernel for one head tile prepares its operands itself
-    dim3 qgrid(num_seqs, head_groups);
-#define KVQ_MLAQ(T) hipLaunchKernelGGL((mla_quant_q_kernel<T>), qgrid, dim3(256), 0, s, a)
-    switch (q_dtype) {
-      case KVQ_F32: KVQ_MLAQ(KVQ_F32); break;
-      case KVQ_BF16: KVQ_MLAQ(KVQ_BF16); break;
-      case KVQ_F16: KVQ_MLAQ(KVQ_F16); break;
-      default: return fail(KVQ_EINVAL, "%s: unknown q_dtype %d", op, q_dtype);
-    }
-#undef KVQ_MLAQ
-  }
+  } else if (q_dtype != KVQ_F32 && q_dtype != KVQ_BF16 && q_dtype != KVQ_F16) {
+    return fail(KVQ_EINVAL, "%s: unknown q_dtype %d", op, q_dtype);
+  }   // without absorption the decode kernels quantise the query themselves
   if (int e = check_hip(hipGetLastError(), "mla_decode_int8 query launch")) return e;
   if (head_groups == 1) {   // one head tile: every wave streams its own tiles
 #define KVQ_MLAS(T) \
@@ -1349,10 +1338,20 @@ static int mla_decode_run(const char* op, void* out, int out_dtype, float* lse, 
     else if (q_dtype == KVQ_F16) KVQ_MLAS(KVQ_F16);
     else return fail(KVQ_EINVAL, "%s: unknown q_dtype %d", op, q_dtype);
 #undef KVQ_MLAS
-  } else if (head_groups % 8 == 0)
-    hipLaunchKernelGGL(mla_decode_kernel<true>, grid, dim3(kMlaThreads), kMlaLdsBytes, s, a);
-  else
-    hipLaunchKernelGGL(mla_decode_kernel<false>, grid, dim3(kMlaThreads), kMlaLdsBytes, s, a);
+  } else {
+#define KVQ_MLAB(F, T) hipLaunchKernelGGL((mla_decode_kernel<F, T>), grid, dim3(kMlaThreads), kMlaLdsBytes, s, a)
+#define KVQ_MLABQ(F)                              \
+  do {                                            \
+    if (absorb != nullptr) KVQ_MLAB(F, -1);       \
+    else if (q_dtype == KVQ_F32) KVQ_MLAB(F, KVQ_F32);   \
+    else if (q_dtype == KVQ_BF16) KVQ_MLAB(F, KVQ_BF16); \
+    else KVQ_MLAB(F, KVQ_F16);                    \
+  } while (0)
+    if (head_groups % 8 == 0) KVQ_MLABQ(true);
+    else KVQ_MLABQ(false);
+#undef KVQ_MLABQ
+#undef KVQ_MLAB
+  }
   int rc = check_hip(hipGetLastError(), "mla_decode_int8 launch");
   if (rc) return rc;
   dim3 rgrid(num_seqs, head_groups);
