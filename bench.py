@@ -179,8 +179,14 @@ def _window_kwargs(st):
     return dict(window_size=(w - 1, 0) if w else (-1, -1), softcap=cap)
 
 
-def run_step(st, layer, ops, write=True, attn=True):
+def run_step(st, layer, ops, write=True, attn=True, fused=False):
     c = st["caches"][layer]
+    if fused:   # the same step in one launch: the attention kernel writes the new tokens itself
+        ops.decode_attention_with_cache_update(st["q"], st["new_k"], st["new_v"], c["k"], c["v"], st["out"], st["sl_d"],
+                                               st["max_ctx"], st["scale"], st["bt_d"], c["ks"], c["vs"],
+                                               workspace=st["ws"], geometry=c["geom"], kv_quant_mode=st["mode"],
+                                               **_window_kwargs(st))
+        return
     if write:
         ops.reshape_and_cache_flash_per_token_head_quant(st["new_k"], st["new_v"], c["k"], c["v"], c["ks"], c["vs"],
                                                          st["slots_new"], kv_quant_mode=st["mode"], geometry=c["geom"])
@@ -508,8 +514,18 @@ def time_decode(cfg, st, args, ops):
     n = max(args.steps, 100)
     attn_s = time_back_to_back(lambda i: run_step(st, i % L, ops, write=False, attn=True), n)
     write_s = time_back_to_back(lambda i: run_step(st, i % L, ops, write=True, attn=False), n)
+    # the same step as ONE launch (the decode kernel writes the new tokens), timed like the two-launch step
+    for i in range(args.warmup):
+        run_step(st, i % L, ops, fused=True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        run_step(st, i % L, ops, fused=True)
+    torch.cuda.synchronize()
+    fused_s = (time.perf_counter() - t0) / args.steps
     return dict(step_s=step_s, attn_s=attn_s, write_s=write_s, attn_bytes=attn_bytes, n_attn=n,
-                value=(attn_bytes + write_bytes) / step_s / 1e9)
+                value=(attn_bytes + write_bytes) / step_s / 1e9, fused_s=fused_s,
+                fused_value=(attn_bytes + write_bytes) / fused_s / 1e9)
 
 
 def main():
@@ -579,6 +595,10 @@ def main():
         "decode_tokens_per_s": round(len(cfg["ctx"]) / t["step_s"], 1),
         "attn_launch_us": round(t["attn_s"] * 1e6, 2),
         "write_launch_us": round(t["write_s"] * 1e6, 2),
+        "one_launch_step": {"what": "the same step with the cache update inside the attention launch "
+                                    "(kvq_paged_attn_int8_fused_write; a backend with forward_includes_kv_cache_update)",
+                            "us_per_layer": round(t["fused_s"] * 1e6, 2), "value": round(t["fused_value"], 1), "unit": "GB/s",
+                            "pct_hbm_peak": round(100 * t["fused_value"] / HBM_PEAK_GBPS, 2)},
         "roofline": {"bound": "hbm", "achieved": round(t["attn_bytes"] / t["attn_s"] / 1e9, 1), "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": round(t["attn_bytes"] / t["attn_s"] / 1e9 / HBM_PEAK_GBPS, 4),
                      "traffic": traffic, "traffic_source": traffic_source,

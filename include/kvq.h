@@ -27,7 +27,7 @@
 extern "C" {
 #endif
 
-#define KVQ_ABI_VERSION 10
+#define KVQ_ABI_VERSION 11
 
 #define KVQ_OK 0
 #define KVQ_EINVAL (-22)
@@ -157,6 +157,31 @@ KVQ_API int kvq_paged_attn_int8(void* out, int out_dtype, int64_t out_stride_t, 
                         const int32_t* block_table, int64_t bt_stride, const int32_t* seq_lens,
                         const int32_t* cu_seqlens_q, int num_seqs, int num_q_heads,
                         int max_query_len, float scale, int causal, int window_size,
+                        float softcap, float* lse, void* workspace, size_t workspace_bytes,
+                        kvq_stream_t stream);
+
+/*
+ * A decode step in ONE launch: the cache update of the step's new tokens and the attention
+ * over the updated cache -- kvq_reshape_and_cache_int8 followed by kvq_paged_attn_int8 with
+ * max_query_len == 1, same bytes in the cache and same output.  For a backend that sets
+ * forward_includes_kv_cache_update (the reference's attribute of that name,
+ * vllm_metax/v1/attention/backends/triton_attn.py:296; its forward then receives key and
+ * value and owns the update that do_kv_cache_update, triton_attn.py:788-840, does otherwise).
+ * Row i of key / value [num_seqs, Hkv, D] (src_dtype, element strides) is the token at
+ * position seq_lens[i] - 1 of sequence i; its slot comes from the block table.  The
+ * workgroup that streams a sequence's last tile quantises the row (the write kernel's
+ * arithmetic) and stores the record before it loads the tile.  Decode rows only: every
+ * sequence has exactly one query row (row i); sequences of length 0 are skipped.  eps as in
+ * kvq_reshape_and_cache_int8.  Workspace as for kvq_paged_attn_int8.
+ */
+KVQ_API int kvq_paged_attn_int8_fused_write(void* out, int out_dtype, int64_t out_stride_t, int64_t out_stride_h,
+                        const void* q, int q_dtype, int64_t q_stride_t, int64_t q_stride_h,
+                        const void* key, const void* value, int src_dtype,
+                        int64_t key_stride_t, int64_t key_stride_h,
+                        int64_t value_stride_t, int64_t value_stride_h, float eps,
+                        void* cache, const kvq_cache_geom* geom,
+                        const int32_t* block_table, int64_t bt_stride, const int32_t* seq_lens,
+                        int num_seqs, int num_q_heads, float scale, int window_size,
                         float softcap, float* lse, void* workspace, size_t workspace_bytes,
                         kvq_stream_t stream);
 

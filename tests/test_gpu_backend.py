@@ -11,13 +11,17 @@ import torch
 import kvq_testlib as T
 import oracle
 from vllm_metax_amd import layout as L
-from vllm_metax_amd.v1.attention.backends.int8_attn import Int8AttentionBackend
+from vllm_metax_amd.v1.attention.backends.int8_attn import Int8AttentionBackend, Int8FusedUpdateAttentionBackend
 
 pytestmark = pytest.mark.gpu
 
 
+@pytest.mark.parametrize("backend", [Int8AttentionBackend, Int8FusedUpdateAttentionBackend],
+                         ids=["two_calls", "forward_includes_kv_cache_update"])
 @pytest.mark.parametrize("layout", ["NHD", "HND"])
-def test_decode_step_through_the_backend(gpu_device, layout, monkeypatch):
+def test_decode_step_through_the_backend(gpu_device, layout, backend, monkeypatch):
+    """With ``forward_includes_kv_cache_update`` the layer skips ``do_kv_cache_update`` and ``forward`` writes the
+    step's tokens itself (one launch for a decode step); cache bytes and output are the same either way."""
     monkeypatch.setenv("VLLM_KV_CACHE_LAYOUT", layout)
     dev = gpu_device
     hq, hkv, d, bs, nb = 32, 8, 128, 16, 200
@@ -32,7 +36,7 @@ def test_decode_step_through_the_backend(gpu_device, layout, monkeypatch):
     views[2].fill_(1.0)                            # the impl fills the scale views with 1.0 at first use
     views[3].fill_(1.0)
     bt = T.make_block_tables(ctx, bs, nb, g)
-    impl = Int8AttentionBackend.get_impl_cls()(hq, d, 1 / math.sqrt(d), hkv, kv_cache_dtype="int8_per_token_head")
+    impl = backend.get_impl_cls()(hq, d, 1 / math.sqrt(d), hkv, kv_cache_dtype="int8_per_token_head")
     spec = types.SimpleNamespace(block_size=bs, num_kv_heads=hkv, head_size=d, num_q_heads=hq)
     cfg = types.SimpleNamespace(scheduler_config=types.SimpleNamespace(max_num_seqs=16))
     builder = Int8AttentionBackend.get_builder_cls()(spec, ["layer.0"], cfg, dev)
@@ -57,7 +61,8 @@ def test_decode_step_through_the_backend(gpu_device, layout, monkeypatch):
         seq_lens=torch.tensor(ctx, dtype=torch.int32, device=dev), block_table_tensor=bt.to(dev),
         slot_mapping=slot_new.to(dev), causal=True)
     md = builder.build(0, common)
-    impl.do_kv_cache_update(layer, k_new.to(dev), v_new.to(dev), kv_cache, md.slot_mapping)
+    if not backend.forward_includes_kv_cache_update:
+        impl.do_kv_cache_update(layer, k_new.to(dev), v_new.to(dev), kv_cache, md.slot_mapping)
     out = torch.full((B + pad, hq * d), 7.0, dtype=torch.bfloat16, device=dev)
     ret = impl.forward(layer, q.to(dev), k_new.to(dev), v_new.to(dev), kv_cache, md, out)
     torch.cuda.synchronize()

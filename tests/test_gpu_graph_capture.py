@@ -16,7 +16,8 @@ from vllm_metax_amd import layout as L
 pytestmark = pytest.mark.gpu
 
 
-def test_decode_step_replays_correctly(gpu_device):
+@pytest.mark.parametrize("one_launch", [False, True], ids=["write_then_attention", "one_launch_step"])
+def test_decode_step_replays_correctly(gpu_device, one_launch):
     dev = gpu_device
     hq, hkv, d, bs, nb, B = 32, 8, 128, 16, 120, 4
     max_len = 400
@@ -46,6 +47,10 @@ def test_decode_step_replays_correctly(gpu_device):
     scale = 1 / math.sqrt(d)
 
     def step():
+        if one_launch:   # the attention launch writes the new tokens itself
+            ops.decode_attention_with_cache_update(q, new_k, new_v, k, v, out, seq_lens, max_len, scale, bt_d, ksc, vsc,
+                                                   workspace=ws, geometry=geom)
+            return
         ops.reshape_and_cache_flash_per_token_head_quant(new_k, new_v, k, v, ksc, vsc, slots, geometry=geom)
         ops.unified_attention(q, k, v, out, cu, 1, seq_lens, max_len, scale, True, block_table=bt_d,
                               k_scale_cache=ksc, v_scale_cache=vsc, workspace=ws, geometry=geom)

@@ -800,6 +800,42 @@ struct StreamKArgs {
   float* part_ml;               // [(P + B), Hq, 2]
   int num_seqs;
   int num_wg;  // P
+  // Fused write of the step's new tokens (decode rows only; k_new == nullptr: the cache already holds them):
+  // row i of k_new / v_new is the token at position seq_lens[i] - 1 of sequence i.
+  const void* k_new;
+  const void* v_new;
+  int64_t kn_stride_t, kn_stride_h, vn_stride_t, vn_stride_h;  // elements
+  int new_dtype;
+  float new_eps;
 };
+
+// The decode kernel's fused cache update: the wave that owns kv head `hkv` of the run that holds a sequence's
+// LAST tile quantises that sequence's new K and V rows (the arithmetic of the write kernel, quant_row8) into
+// the record at position len - 1 before it streams the run's tiles.  D / 8 lanes per row: lanes
+// [0, D/8) take the K row, [D/8, D/4) the V row; the rest repeat them and store nothing.
+template <int D>
+__device__ __forceinline__ void write_new_token(const StreamKArgs& a, int seq, int64_t row, int len, int hkv, int lane) {
+  constexpr int LPR = D / 8;
+  const kvq_cache_geom& g = a.io.g;
+  const int is_v = (lane / LPR) & 1;
+  const int li = lane % LPR;
+  const void* src = is_v ? a.v_new : a.k_new;
+  const int64_t elem = (is_v ? row * a.vn_stride_t + (int64_t)hkv * a.vn_stride_h
+                             : row * a.kn_stride_t + (int64_t)hkv * a.kn_stride_h) + li * 8;
+  float x[8];
+  load_row8(src, a.new_dtype, elem, x);
+  uint32_t pk[2];
+  float scale;
+  quant_row8<LPR>(x, a.new_eps, g.code_type == KVQ_CODE_FP8_E4M3, pk, scale);
+  const int pos = len - 1;
+  const int e = (int)__umulhi((uint32_t)pos, a.io.bs_magic);
+  const int off = pos - e * g.block_size;
+  const int64_t blk = a.io.block_table[(int64_t)seq * a.io.bt_stride + e];
+  uint8_t* rec = const_cast<uint8_t*>(a.io.cache) + blk * g.stride_block + (int64_t)off * g.stride_slot + (int64_t)hkv * g.stride_head;
+  if (lane < 2 * LPR) {
+    *reinterpret_cast<u32x2_a4*>(rec + (is_v ? g.v_off : g.k_off) + li * 8) = (u32x2){pk[0], pk[1]};
+    if (li == 0) *reinterpret_cast<float*>(rec + (is_v ? g.vs_off : g.ks_off)) = scale;
+  }
+}
 
 }  // namespace kvq

@@ -138,6 +138,57 @@ __device__ __forceinline__ float sum_over_quarters(float v) {
 // Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits for every global
 // load in flight (vmcnt(0)), which would drain the tile prefetch issued just before it; here the
 // loads stay in flight and the compiler's own wait before their first use still applies.
+// One cache row's quantisation with 8 elements per lane and LPR lanes per row (every lane of the wave takes
+// part in the shuffles): scale = max(amax, eps) / 127 (448 for fp8 codes), code = rint(x / scale) clamped.
+// Shared by the write kernel and by the decode kernel's fused write, so that both store the same bytes.
+template <int LPR>
+__device__ __forceinline__ void quant_row8(const float (&x)[8], float eps, bool fp8, uint32_t (&pk)[2], float& scale) {
+  float amax = 0.f;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf(x[i]));
+#pragma unroll
+  for (int o = LPR / 2; o >= 1; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o, kWave));
+  amax = fmaxf(amax, eps);  // eps may be 0 for fp16 sources (1e-10 underflows)
+  scale = fp8 ? amax / 448.0f : amax / 127.0f;
+  pk[0] = 0u;
+  pk[1] = 0u;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const float y = scale > 0.f ? x[i] / scale : 0.f;  // scale == 0: all-zero fp16 row
+    uint32_t code;
+    if (fp8) {
+      code = f32_to_e4m3fn_bits(y);
+    } else {
+      const float r = fminf(fmaxf(rintf(y), -128.f), 127.f);
+      code = (uint32_t)(int)r & 0xffu;
+    }
+    pk[i >> 2] |= code << (8 * (i & 3));
+  }
+}
+
+// Eight consecutive elements of a row of runtime type `dt`, as floats (`elem` = element offset; 4-byte aligned).
+__device__ __forceinline__ void load_row8(const void* src, int dt, int64_t elem, float (&x)[8]) {
+  if (dt == KVQ_F32) {
+    const float* p = reinterpret_cast<const float*>(src) + elem;
+    const floatx4 a = *reinterpret_cast<const floatx4_a4*>(p), b = *reinterpret_cast<const floatx4_a4*>(p + 4);
+    x[0] = a.x; x[1] = a.y; x[2] = a.z; x[3] = a.w; x[4] = b.x; x[5] = b.y; x[6] = b.z; x[7] = b.w;
+  } else {
+    const u32x4 v = *reinterpret_cast<const u32x4_a4*>(reinterpret_cast<const uint16_t*>(src) + elem);
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      const uint32_t e = v[w];
+      if (dt == KVQ_BF16) {
+        x[2 * w] = as_f32(e << 16);
+        x[2 * w + 1] = as_f32(e & 0xffff0000u);
+      } else {
+        const half2_t hh = __builtin_bit_cast(half2_t, e);
+        x[2 * w] = (float)hh.x;
+        x[2 * w + 1] = (float)hh.y;
+      }
+    }
+  }
+}
+
 __device__ __forceinline__ void lds_barrier() {
   asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }

@@ -49,15 +49,24 @@ static int device_symbols(const char* op, DeviceSymbols* out) {
   return KVQ_OK;
 }
 
-// Arguments are checked, the launch is shaped and enqueued here; the two entry points differ only
-// in where the split-K partial states live.
+// The new tokens of a decode step, for the entry point that writes them into the cache inside the launch.
+struct NewTokens {
+  const void* key;
+  const void* value;
+  int dtype;
+  int64_t key_stride_t, key_stride_h, value_stride_t, value_stride_h;
+  float eps;
+};
+
+// Arguments are checked, the launch is shaped and enqueued here; the entry points differ only
+// in where the split-K partial states live and in whether the launch also writes the step's new tokens.
 static int paged_attn_launch(const char* op, void* out, int out_dtype, int64_t out_stride_t, int64_t out_stride_h,
                              const void* q, int q_dtype, int64_t q_stride_t, int64_t q_stride_h, const void* cache,
                              const kvq_cache_geom* geom, const int32_t* block_table, int64_t bt_stride,
                              const int32_t* seq_lens, const int32_t* cu_seqlens_q, int num_seqs, int num_q_heads,
                              int max_query_len, float scale, int causal, int window_size, float softcap, float* lse,
                              void* workspace, size_t workspace_bytes, const char* workspace_what,
-                             kvq_stream_t stream) {
+                             kvq_stream_t stream, const NewTokens* fresh = nullptr) {
   int rc0 = validate_common(op, q, cache, geom, block_table, seq_lens, num_seqs, num_q_heads);
   if (rc0) return rc0;
   KVQ_REQUIRE(out != nullptr, "%s: out is NULL", op);
@@ -104,6 +113,27 @@ static int paged_attn_launch(const char* op, void* out, int out_dtype, int64_t o
   a.part_o = static_cast<float*>(workspace);
   a.part_ml = a.part_o + slots * (size_t)num_q_heads * (size_t)g.head_size;
 
+  if (fresh != nullptr) {
+    KVQ_REQUIRE(max_query_len == 1, "%s: the fused write takes decode rows only (max_query_len == 1)", op);
+    KVQ_REQUIRE(fresh->key != nullptr && fresh->value != nullptr, "%s: key / value is NULL", op);
+    KVQ_REQUIRE(fresh->dtype == KVQ_F32 || fresh->dtype == KVQ_BF16 || fresh->dtype == KVQ_F16,
+                "%s: unknown src_dtype %d", op, fresh->dtype);
+    KVQ_REQUIRE(fresh->eps >= 0.f, "%s: eps must not be negative", op);
+    KVQ_REQUIRE(g.head_size == 64 || g.head_size == 128 || g.head_size == 256,
+                "%s: head_size %d is not built", op, g.head_size);
+    const int esz = fresh->dtype == KVQ_F32 ? 4 : 2;
+    KVQ_REQUIRE(((uintptr_t)fresh->key % 4) == 0 && ((uintptr_t)fresh->value % 4) == 0 &&
+                    ((fresh->key_stride_t | fresh->key_stride_h | fresh->value_stride_t | fresh->value_stride_h) * esz) % 4 == 0,
+                "%s: key / value rows must be 4-byte aligned", op);
+    a.k_new = fresh->key;
+    a.v_new = fresh->value;
+    a.kn_stride_t = fresh->key_stride_t;
+    a.kn_stride_h = fresh->key_stride_h;
+    a.vn_stride_t = fresh->value_stride_t;
+    a.vn_stride_h = fresh->value_stride_h;
+    a.new_dtype = fresh->dtype;
+    a.new_eps = fresh->eps;
+  }
   hipStream_t s = as_stream(stream);
   int rc = launch_decode_streamk(a, q_dtype, out_dtype, s);
   if (rc) return rc;
@@ -126,6 +156,23 @@ extern "C" int kvq_paged_attn_int8(void* out, int out_dtype, int64_t out_stride_
                                 q_stride_h, cache, geom, block_table, bt_stride, seq_lens, cu_seqlens_q, num_seqs,
                                 num_q_heads, max_query_len, scale, causal, window_size, softcap, lse, workspace,
                                 workspace_bytes, "workspace", stream);
+}
+
+extern "C" int kvq_paged_attn_int8_fused_write(void* out, int out_dtype, int64_t out_stride_t, int64_t out_stride_h,
+                                               const void* q, int q_dtype, int64_t q_stride_t, int64_t q_stride_h,
+                                               const void* key, const void* value, int src_dtype,
+                                               int64_t key_stride_t, int64_t key_stride_h, int64_t value_stride_t,
+                                               int64_t value_stride_h, float eps, void* cache,
+                                               const kvq_cache_geom* geom, const int32_t* block_table,
+                                               int64_t bt_stride, const int32_t* seq_lens, int num_seqs,
+                                               int num_q_heads, float scale, int window_size, float softcap,
+                                               float* lse, void* workspace, size_t workspace_bytes,
+                                               kvq_stream_t stream) {
+  const kvq::NewTokens fresh{key, value, src_dtype, key_stride_t, key_stride_h, value_stride_t, value_stride_h, eps};
+  return kvq::paged_attn_launch("paged_attn_int8_fused_write", out, out_dtype, out_stride_t, out_stride_h, q, q_dtype,
+                                q_stride_t, q_stride_h, cache, geom, block_table, bt_stride, seq_lens, nullptr, num_seqs,
+                                num_q_heads, 1, scale, 1, window_size, softcap, lse, workspace, workspace_bytes,
+                                "workspace", stream, &fresh);
 }
 
 extern "C" size_t kvq_paged_attn_static_scratch_bytes(void) { return KVQ_STATIC_SCRATCH_BYTES; }

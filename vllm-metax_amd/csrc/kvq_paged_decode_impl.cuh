@@ -190,6 +190,12 @@ __global__ __launch_bounds__(512) void paged_decode_streamk_kernel(StreamKArgs a
     const int t_begin = __builtin_amdgcn_readfirstlane(t0 + (u_begin > kSetupUnits ? u_begin - kSetupUnits : 0));
     const int t_end = __builtin_amdgcn_readfirstlane(t0 + u_end - kSetupUnits);
     if (t_begin < t_end) {  // else: this share ends inside the setup charge and holds no tile
+      if (a.k_new != nullptr && t_end == t0 + ntiles) {   // uniform over the workgroup: the run holds the last tile
+        if (sub == 0) write_new_token<D>(a, seq, row, len, hkv, lane);
+        // the record is in memory before any wave of the workgroup loads the tile that holds it
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        if constexpr (NSUB > 1) lds_barrier();
+      }
       typename DTile::State st;
       DTile::template run<CAP, STREAM>(a.io, seq, row, len, first, t_begin, t_end, hkv, lane, lds[wave], st, sub, NSUB);
       if constexpr (NSUB > 1) {

@@ -158,27 +158,9 @@ __global__ __launch_bounds__(256) void quant_write_rows_kernel(
       }
     }
   }
-  float amax = 0.f;
-#pragma unroll
-  for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf(x[i]));
-#pragma unroll
-  for (int o = LPR / 2; o >= 1; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o, kWave));
-  amax = fmaxf(amax, eps);  // eps may be 0 for fp16 sources (1e-10 underflows)
-  const bool fp8 = g.code_type == KVQ_CODE_FP8_E4M3;
-  const float scale = fp8 ? amax / 448.0f : amax / 127.0f;
-  uint32_t pk[2] = {0u, 0u};
-#pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    const float y = scale > 0.f ? x[i] / scale : 0.f;  // scale == 0: all-zero fp16 row
-    uint32_t code;
-    if (fp8) {
-      code = f32_to_e4m3fn_bits(y);
-    } else {
-      const float r = fminf(fmaxf(rintf(y), -128.f), 127.f);
-      code = (uint32_t)(int)r & 0xffu;
-    }
-    pk[i >> 2] |= code << (8 * (i & 3));
-  }
+  uint32_t pk[2];
+  float scale;
+  quant_row8<LPR>(x, eps, g.code_type == KVQ_CODE_FP8_E4M3, pk, scale);
   if (!live || slot < 0) return;  // padding token (after the shuffles: every lane took part)
   int64_t blk, off;
   if ((uint64_t)slot <= 0xffffffffull) {

@@ -292,6 +292,86 @@ def unified_attention(
     _C.check(rc, "unified_attention")
 
 
+def decode_attention_with_cache_update(
+    q: torch.Tensor,
+    key: torch.Tensor,
+    value: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    out: torch.Tensor,
+    seqused_k: torch.Tensor,
+    max_seqlen_k: int,
+    softmax_scale: float,
+    block_table: torch.Tensor,
+    k_scale_cache: torch.Tensor,
+    v_scale_cache: torch.Tensor,
+    window_size=(-1, -1),
+    softcap: float = 0.0,
+    kv_quant_mode: KVQuantMode = KVQuantMode.INT8_PER_TOKEN_HEAD,
+    workspace: torch.Tensor | None = None,
+    geometry: CacheGeometry | None = None,
+    lse: torch.Tensor | None = None,
+) -> None:
+    """A decode step in one launch: the cache update of ``reshape_and_cache_flash_per_token_head_quant`` and the
+    attention of ``unified_attention`` with one query row per sequence, for a backend whose ``forward`` includes
+    the KV cache update (``forward_includes_kv_cache_update``, vllm_metax/v1/attention/backends/triton_attn.py:296).
+
+    ``q``/``out`` ``[B, Hq, D]``; ``key``/``value`` ``[B, Hkv, D]``: row ``i`` is the token at position
+    ``seqused_k[i] - 1`` of sequence ``i`` (the block table gives its slot); ``k``/``v`` and the scale views as in
+    ``unified_attention``.  The cache ends up with the same bytes and ``out`` with the same values as the two
+    calls give."""
+    code_type = code_type_of(kv_quant_mode)
+    softcap = float(softcap or 0.0)
+    if softcap < 0:
+        raise RuntimeError("softcap must be >= 0")
+    left, right = (int(x) for x in window_size)
+    if (left, right) == (-1, -1):
+        window = 0
+    elif left >= 0 and right == 0:
+        window = left + 1
+    else:
+        raise NotImplementedError(f"window_size {(left, right)}: only (-1, -1) and (W - 1, 0) are built")
+    dev = _require_cuda(q, key, value, k, v, out, seqused_k, block_table, k_scale_cache, v_scale_cache, workspace, lse)
+    geom = (geometry or geometry_from_views(k, v, k_scale_cache, v_scale_cache)).with_code_type(code_type)
+    num_seqs = seqused_k.shape[0]
+    if q.dim() != 3 or out.shape != q.shape or q.shape[2] != geom.head_size or q.shape[0] != num_seqs:
+        raise RuntimeError("q/out must be [num_seqs, num_q_heads, head_size] matching the cache head size")
+    if q.stride(2) != 1 or out.stride(2) != 1:
+        raise RuntimeError("q/out head dim must be contiguous")
+    if key.dim() != 3 or value.shape != key.shape or key.dtype != value.dtype or key.shape[0] < num_seqs:
+        raise RuntimeError("key/value must be [num_seqs, num_kv_heads, head_size] of one dtype")
+    if key.shape[1] != geom.num_kv_heads or key.shape[2] != geom.head_size:
+        raise RuntimeError(f"key shape {tuple(key.shape)} does not match cache (Hkv={geom.num_kv_heads}, D={geom.head_size})")
+    if key.stride(2) != 1 or value.stride(2) != 1:
+        raise RuntimeError("key/value head dim must be contiguous")
+    if seqused_k.dtype != torch.int32 or block_table.dtype != torch.int32 or not seqused_k.is_contiguous():
+        raise RuntimeError("seqused_k (contiguous) and block_table must be int32")
+    if block_table.shape[0] < num_seqs or block_table.stride(1) != 1:
+        raise RuntimeError("block_table needs num_seqs contiguous rows")
+    if block_table.shape[1] * geom.block_size < int(max_seqlen_k):
+        raise RuntimeError("block_table rows are too short for max_seqlen_k")
+    if num_seqs == 0:
+        return
+    num_q_heads = q.shape[1]
+    if lse is not None and (lse.dtype != torch.float32 or not lse.is_contiguous()
+                            or tuple(lse.shape) != (num_seqs, num_q_heads)):
+        raise RuntimeError("lse must be a contiguous float32 [num_seqs, num_q_heads] tensor")
+    lib = _C.load()
+    g = geom.as_struct()
+    if workspace is None:
+        workspace = _default_workspace(dev, paged_attn_workspace_bytes(num_seqs, num_q_heads, geom.head_size, dev))
+    with _on_device(dev):
+        rc = lib.kvq_paged_attn_int8_fused_write(
+            _ptr(out), _dtype_code(out, "out"), out.stride(0), out.stride(1),
+            _ptr(q), _dtype_code(q, "q"), q.stride(0), q.stride(1),
+            _ptr(key), _ptr(value), _dtype_code(key, "key"), key.stride(0), key.stride(1), value.stride(0),
+            value.stride(1), eps_for_dtype(key.dtype), ctypes.c_void_p(geom.base_ptr), ctypes.byref(g),
+            _ptr(block_table), block_table.stride(0), _ptr(seqused_k), num_seqs, num_q_heads,
+            float(softmax_scale), window, softcap, _ptr(lse), _ptr(workspace),
+            workspace.numel() * workspace.element_size(), _stream(dev))
+    _C.check(rc, "decode_attention_with_cache_update")
+
+
 def paged_attention_v2(
     out: torch.Tensor,
     exp_sums: torch.Tensor,

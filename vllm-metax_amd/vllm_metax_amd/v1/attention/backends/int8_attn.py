@@ -370,3 +370,48 @@ class Int8AttentionImpl(_ImplBase):
             kv_quant_mode=self._kv_quant_mode, k_scale_cache=self._k_scale_cache, v_scale_cache=self._v_scale_cache,
             workspace=attn_metadata.workspace, geometry=self._geometry)
         return output
+
+
+class Int8FusedUpdateAttentionImpl(Int8AttentionImpl):
+    """The same layer with the KV cache update inside ``forward``: a decode-only step is ONE launch (the
+    attention kernel quantises each sequence's new token into the cache before it streams the tile that holds
+    it); a step with prefill rows falls back to the two calls, in this order, inside ``forward``."""
+
+    def forward(self, layer, query: torch.Tensor, key: torch.Tensor, value: torch.Tensor, kv_cache: torch.Tensor,
+                attn_metadata: Int8AttentionMetadata | None, output: torch.Tensor,
+                output_scale: torch.Tensor | None = None, output_block_scale: torch.Tensor | None = None) -> torch.Tensor:
+        if output_scale is not None or output_block_scale is not None:
+            raise NotImplementedError("fused output quantization is not supported")
+        if attn_metadata is None:  # profiling run
+            return output.fill_(0)
+        if attn_metadata.use_cascade:
+            raise NotImplementedError("cascade attention is not supported")
+        n = attn_metadata.num_actual_tokens
+        num_seqs = attn_metadata.seq_lens.shape[0]
+        if attn_metadata.max_query_len != 1 or n != num_seqs or key is None or value is None:
+            if key is not None and value is not None:
+                self.do_kv_cache_update(layer, key[:n], value[:n], kv_cache, attn_metadata.slot_mapping[:n])
+            return super().forward(layer, query, key, value, kv_cache, attn_metadata, output)
+        key_cache, value_cache = self._pth_key_value_caches(kv_cache)
+        ops.decode_attention_with_cache_update(
+            q=query[:n].view(n, self.num_heads, self.head_size),
+            key=key[:n].view(n, self.num_kv_heads, self.head_size),
+            value=value[:n].view(n, self.num_kv_heads, self.head_size),
+            k=key_cache, v=value_cache, out=output[:n].view(n, self.num_heads, self.head_size),
+            seqused_k=attn_metadata.seq_lens, max_seqlen_k=attn_metadata.max_seq_len, softmax_scale=self.scale,
+            block_table=attn_metadata.block_table, k_scale_cache=self._k_scale_cache, v_scale_cache=self._v_scale_cache,
+            window_size=self.sliding_window, softcap=self.logits_soft_cap, kv_quant_mode=self._kv_quant_mode,
+            workspace=attn_metadata.workspace, geometry=self._geometry)
+        return output
+
+
+class Int8FusedUpdateAttentionBackend(Int8AttentionBackend):
+    """``Int8AttentionBackend`` with ``forward_includes_kv_cache_update`` set (the reference's attribute of that
+    name, vllm_metax/v1/attention/backends/triton_attn.py:296): the layer then does not call
+    ``do_kv_cache_update`` and hands key and value to ``forward``."""
+
+    forward_includes_kv_cache_update: bool = True
+
+    @staticmethod
+    def get_impl_cls():
+        return Int8FusedUpdateAttentionImpl
