@@ -48,6 +48,58 @@ __global__ __launch_bounds__(256) void mla_quant_write_kernel(const void* __rest
   if (lane == 0) *reinterpret_cast<float*>(cache + blk * g.stride_block + g.scale_off + off * 4) = scale;
 }
 
+// The same arithmetic, eight consecutive elements per lane and load (rows whose two parts are multiples of 8
+// wide and 4-byte aligned; at most 1024 wide): one wave per token, lane l takes the 8-element pieces l and
+// 64 + l of the row [kv_c | k_pe], 16-byte loads (two for fp32 sources) that leave before the slot is known --
+// one trip to memory instead of two -- and 8-byte stores of packed codes instead of byte stores.
+__global__ __launch_bounds__(256) void mla_quant_write_rows8_kernel(const void* __restrict__ kv_c,
+                                                                    const void* __restrict__ k_pe, int dt,
+                                                                    int64_t kv_c_stride, int64_t k_pe_stride,
+                                                                    uint8_t* __restrict__ cache, kvq_mla_geom g,
+                                                                    const int64_t* __restrict__ slot_mapping,
+                                                                    int64_t num_tokens, float eps) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int64_t t_raw = (int64_t)blockIdx.x * (blockDim.x / kWave) + (threadIdx.x / kWave);
+  const bool live = t_raw < num_tokens;
+  const int64_t t = live ? t_raw : num_tokens - 1;
+  const int rp = g.kv_lora_rank / 8, np = (g.kv_lora_rank + g.rope_dim) / 8;   // pieces of kv_c, of the row
+  const int64_t slot = slot_mapping[t];  // in flight together with the row's loads
+  float x[2][8];
+  bool have[2];
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const int piece = lane + kWave * j;
+    have[j] = piece < np;
+    const int pc = have[j] ? piece : 0;
+    if (pc < rp) load_row8(kv_c, dt, t * kv_c_stride + 8 * pc, x[j]);
+    else load_row8(k_pe, dt, t * k_pe_stride + 8 * (pc - rp), x[j]);
+  }
+  float amax = 0.f;
+#pragma unroll
+  for (int j = 0; j < 2; ++j)
+#pragma unroll
+    for (int i = 0; i < 8; ++i) amax = fmaxf(amax, have[j] ? fabsf(x[j][i]) : 0.f);
+  amax = fmaxf(wave_max(amax), eps);
+  const float scale = amax / 127.0f;
+  if (!live || slot < 0) return;  // padding token (after the shuffles: every lane took part)
+  const int64_t blk = slot / g.block_size;
+  const int64_t off = slot - blk * g.block_size;
+  uint8_t* row = cache + blk * g.stride_block + off * g.stride_row;
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    if (!have[j]) continue;
+    uint32_t pk[2] = {0u, 0u};
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      float r = scale > 0.f ? rintf(x[j][i] / scale) : 0.f;
+      r = fminf(fmaxf(r, -128.f), 127.f);
+      pk[i >> 2] |= ((uint32_t)(int)r & 0xffu) << (8 * (i & 3));
+    }
+    *reinterpret_cast<u32x2_a4*>(row + 8 * (lane + kWave * j)) = (u32x2){pk[0], pk[1]};
+  }
+  if (lane == 0) *reinterpret_cast<float*>(cache + blk * g.stride_block + g.scale_off + off * 4) = scale;
+}
+
 // Round a float to the nearest value of the activation type (the arithmetic type of the rotary
 // embedding below is the activation type, one rounding per operation).
 template <int DT>
@@ -420,6 +472,14 @@ extern "C" int kvq_concat_and_cache_mla_int8(const void* kv_c, const void* k_pe,
   KVQ_REQUIRE(blocks <= 0x7fffffffLL, "%s: too many tokens", op);
   hipStream_t s = as_stream(stream);
   uint8_t* c = static_cast<uint8_t*>(cache);
+  const int esz = src_dtype == KVQ_F32 ? 4 : 2;
+  if ((src_dtype == KVQ_F32 || src_dtype == KVQ_BF16 || src_dtype == KVQ_F16) && g.kv_lora_rank % 8 == 0 &&
+      g.rope_dim % 8 == 0 && g.stride_row % 4 == 0 && ((uintptr_t)kv_c % 4) == 0 && ((uintptr_t)k_pe % 4) == 0 &&
+      (kv_c_stride * esz) % 4 == 0 && (k_pe_stride * esz) % 4 == 0) {
+    hipLaunchKernelGGL(mla_quant_write_rows8_kernel, dim3((unsigned)blocks), dim3(256), 0, s, kv_c, k_pe, src_dtype,
+                       kv_c_stride, k_pe_stride, c, g, slot_mapping, num_tokens, eps);
+    return check_hip(hipGetLastError(), "concat_and_cache_mla_int8 launch");
+  }
 #define KVQ_MLAW(T)                                                                                       \
   hipLaunchKernelGGL((mla_quant_write_kernel<T>), dim3((unsigned)blocks), dim3(256), 0, s, kv_c, k_pe, \
                      kv_c_stride, k_pe_stride, c, g, slot_mapping, num_tokens, eps)
