@@ -765,8 +765,8 @@ __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
 // once, by the lane that multiplies it), computes the logits of its 16 heads against the Q operands it
 // keeps in registers, runs the softmax -- whose result already IS the P~ operand of the second product -- and copies
 // the rows' first 512 bytes into a wave-private, chunk-swizzled LDS window, from which it builds the fp16
-// V^T operands of all 512 output dims with dword reads and byte permutes (as the kernel above does for
-// its 64).  At the end the four waves' states are summed through the (then idle) windows, each wave
+// V^T operands of all 512 output dims with dword reads and sub-dword conversions (as the kernel above does
+// for its 64).  At the end the four waves' states are summed through the (then idle) windows, each wave
 // adding up and emitting the 128 output dims of its number.
 constexpr int kMlaSmallWin = kTile * kMlaR;                                   // 16384: a tile's V part
 constexpr int kMlaSmallQBytes = kMlaQOps * kWave * 16 + 256 + 2048;           // Q operands, the waves' maxima of |q|, (m, l) of the waves
