@@ -27,7 +27,7 @@
 extern "C" {
 #endif
 
-#define KVQ_ABI_VERSION 11
+#define KVQ_ABI_VERSION 12
 
 #define KVQ_OK 0
 #define KVQ_EINVAL (-22)
@@ -416,6 +416,29 @@ KVQ_API size_t kvq_mla_decode_workspace_bytes(int max_num_seqs, int num_heads, i
 KVQ_API int kvq_mla_decode_int8(void* out, int out_dtype, float* lse, const void* q, int q_dtype,
                         int64_t q_stride_b, int64_t q_stride_h, const void* q_pe,
                         int64_t q_pe_stride_b, int64_t q_pe_stride_h, const void* cache,
+                        const kvq_mla_geom* geom, const int32_t* block_table,
+                        int64_t bt_stride, const int32_t* seq_lens, int num_seqs,
+                        int num_heads, float scale, void* workspace, size_t workspace_bytes,
+                        kvq_stream_t stream);
+
+/*
+ * An MLA decode step in ONE launch: kvq_concat_and_cache_mla_int8 for the step's new
+ * tokens followed by kvq_mla_decode_int8, same bytes in the cache and same output
+ * (do_kv_cache_update and forward_mqa of the reference's MLA backend,
+ * vllm_metax/v1/attention/backends/mla/triton_mla.py:226-295, which a backend with
+ * forward_includes_kv_cache_update may do in one step).  Row i of kv_c
+ * [num_seqs, kv_lora_rank] / k_pe [num_seqs, rope_dim] (src_dtype, row strides in
+ * elements, rows 4-byte aligned) is the token at position seq_lens[i] - 1 of sequence i;
+ * its slot comes from the block table.  The wave that streams the sequence's last tile
+ * quantises the row (the write kernel's arithmetic) and stores it before that tile is
+ * requested.  Sequences of length 0 are skipped.  eps as in
+ * kvq_concat_and_cache_mla_int8; everything else as in kvq_mla_decode_int8.
+ */
+KVQ_API int kvq_mla_decode_int8_fused_write(void* out, int out_dtype, float* lse, const void* q,
+                        int q_dtype, int64_t q_stride_b, int64_t q_stride_h, const void* q_pe,
+                        int64_t q_pe_stride_b, int64_t q_pe_stride_h, const void* kv_c,
+                        const void* k_pe, int src_dtype, int64_t kv_c_stride,
+                        int64_t k_pe_stride, float eps, void* cache,
                         const kvq_mla_geom* geom, const int32_t* block_table,
                         int64_t bt_stride, const int32_t* seq_lens, int num_seqs,
                         int num_heads, float scale, void* workspace, size_t workspace_bytes,

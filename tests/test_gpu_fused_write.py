@@ -117,3 +117,101 @@ def test_fused_write_strided_sources_and_full_size(gpu_device):
     (cache_a, out_a, _), (cache_b, out_b, _) = _both_ways(dev, kv, "HND", bt, q, sl, ctx, key, value, 0.088)
     assert torch.equal(cache_a, cache_b)
     assert torch.equal(out_a.view(torch.int16), out_b.view(torch.int16))
+
+
+# ---------------------------------------------------------------------------------------------
+# MLA: kvq_mla_decode_int8_fused_write against concat_and_cache_mla + mla_decode_int8
+# (vllm_metax/v1/attention/backends/mla/triton_mla.py:226-295 does the two in two steps)
+# ---------------------------------------------------------------------------------------------
+R, P = 512, 64
+
+
+def _mla_both_ways(dev, cache_cpu, bt, sl, ctx, bs, q, kv_c, k_pe, scale):
+    res = []
+    for fused in (False, True):
+        cache = cache_cpu.clone().to(dev)
+        B, H, _ = q.shape
+        o = torch.full((B, H, R), float("nan"), dtype=q.dtype, device=dev)
+        lse = torch.full((B, H), float("nan"), dtype=torch.float32, device=dev)
+        if fused:
+            ops.mla_decode_with_cache_update(q.to(dev), kv_c.to(dev), k_pe.to(dev), cache, o, lse, bt.to(dev),
+                                             sl.to(dev), scale, R)
+        else:
+            ops.concat_and_cache_mla(kv_c.to(dev), k_pe.to(dev), cache, _last_slots(bt, ctx, bs).to(dev))
+            ops.mla_decode_int8(q.to(dev), cache, o, lse, bt.to(dev), sl.to(dev), scale, R)
+        torch.cuda.synchronize()
+        res.append((T.storage_bytes(cache).cpu(), o.cpu(), lse.cpu()))
+    return res
+
+
+def _same_bits(a, b):
+    return torch.equal(a.contiguous().view(torch.uint8), b.contiguous().view(torch.uint8))
+
+
+@pytest.mark.parametrize("bs,heads,ctx", [
+    (64, 128, [300, 1, 64, 2049, 65, 33, 32]),      # many splits per sequence: the row is written before the tiles
+    (16, 16, [17, 33, 511, 1, 16, 32, 64, 97]),     # one head tile; lengths that end at the first / last row of a tile
+    (64, 20, [5, 0, 95, 1000, 31, 0, 32]),          # empty sequences next to live ones; part-filled 128-head block
+    (64, 160, [70, 300, 33, 129]),                  # two 128-head blocks write the same row
+    (16, 5, [5, 95, 1000, 31, 32, 4097]),
+    (32, 8, [16384, 16385]),                        # one head tile, 64 splits
+    (16, 16, [700, 701, 672, 673, 641, 400] * 44),  # one split per sequence: a wave has many tiles, the row is written late
+    (16, 16, [2000, 2017, 1985, 3000] * 18),        # four splits of 16 tiles and more
+    (32, 128, [2048, 4096, 4065, 3000] * 9),        # 128 heads, 36 sequences: long splits, the row is written late
+])
+def test_mla_fused_write_equals_write_then_decode(gpu_device, bs, heads, ctx):
+    cache, lay, bt, sl = T.build_mla_cache(ctx, bs, seed=bs + heads, dtype=torch.bfloat16, poison=False)
+    g = torch.Generator().manual_seed(13)
+    B = len(ctx)
+    q = torch.randn((B, heads, R + P), generator=g).to(torch.bfloat16)
+    kv_c = (torch.randn((B, R), generator=g) * 2).to(torch.bfloat16)
+    k_pe = (torch.randn((B, P), generator=g) * 2).to(torch.bfloat16)
+    scale = (128 + 64) ** -0.5
+    (cache_a, out_a, lse_a), (cache_b, out_b, lse_b) = _mla_both_ways(gpu_device, cache, bt, sl, ctx, bs, q, kv_c, k_pe, scale)
+    assert torch.equal(cache_a, cache_b), "the fused write left other bytes in the cache than the write kernel"
+    live = torch.tensor([i for i, c in enumerate(ctx) if c > 0])
+    assert _same_bits(out_a[live], out_b[live]), "outputs differ"
+    assert _same_bits(lse_a[live], lse_b[live]), "lse differs"
+    # the cache against the oracle's write, and (where the oracle is quick) the output against its decode
+    ref = cache.clone()
+    oracle.mla_cache_write(kv_c[live], k_pe[live], ref, lay, _last_slots(bt, ctx, bs)[live])
+    assert torch.equal(cache_b, T.storage_bytes(ref)), "the fused write's cache differs from the oracle's"
+    if sum(ctx) * heads <= 1 << 20:
+        want, want_lse = oracle.mla_decode(q, ref, lay, bt, sl, scale)
+        T.assert_close_attn(out_b[live], want[live], what="mla fused write + decode")
+        torch.testing.assert_close(lse_b[live], want_lse[live], atol=5e-3, rtol=1e-3)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+@pytest.mark.parametrize("heads", [16, 128])
+def test_mla_fused_write_source_types_and_strides(gpu_device, dtype, heads):
+    """fp16 / fp32 rows (the query has the rows' type), an all-zero row, kv_c and k_pe as two slices of one
+    projection output (row stride R + P)."""
+    ctx = [333, 16, 1, 2000, 3000, 777] * 8
+    bs = 16
+    cache, lay, bt, sl = T.build_mla_cache(ctx, bs, seed=3, dtype=torch.bfloat16, poison=False)
+    g = torch.Generator().manual_seed(9)
+    B = len(ctx)
+    q = torch.randn((B, heads, R + P), generator=g).to(dtype)
+    proj = torch.randn((B, R + P), generator=g).to(dtype)
+    proj[1] = 0
+    kv_c, k_pe = proj[:, :R], proj[:, R:]
+    (cache_a, out_a, lse_a), (cache_b, out_b, lse_b) = _mla_both_ways(gpu_device, cache, bt, sl, ctx, bs, q, kv_c, k_pe, 0.072)
+    assert torch.equal(cache_a, cache_b)
+    assert _same_bits(out_a, out_b) and _same_bits(lse_a, lse_b)
+
+
+def test_mla_fused_write_rejects_bad_arguments(gpu_device):
+    dev = gpu_device
+    cache, lay, bt, sl = T.build_mla_cache([40, 50], 16, seed=1, poison=False)
+    q = torch.zeros((2, 16, R + P), dtype=torch.bfloat16, device=dev)
+    o = torch.zeros((2, 16, R), dtype=torch.bfloat16, device=dev)
+    kv_c = torch.zeros((2, R), dtype=torch.bfloat16, device=dev)
+    k_pe = torch.zeros((2, P), dtype=torch.bfloat16, device=dev)
+    args = (cache.to(dev), o, None, bt.to(dev), sl.to(dev), 0.1, R)
+    with pytest.raises(RuntimeError, match="one row per sequence"):
+        ops.mla_decode_with_cache_update(q, kv_c[:1], k_pe, *args)
+    with pytest.raises(RuntimeError, match="one dtype"):
+        ops.mla_decode_with_cache_update(q, kv_c, k_pe.float(), *args)
+    with pytest.raises(RuntimeError, match="4-byte aligned"):
+        ops.mla_decode_with_cache_update(q, torch.zeros((2, R + 1), dtype=torch.bfloat16, device=dev)[:, 1:], k_pe, *args)

@@ -189,6 +189,85 @@ __device__ __forceinline__ void load_row8(const void* src, int dt, int64_t elem,
   }
 }
 
+// One MLA latent row [kv_c | k_pe] quantised by ONE wave, eight elements per lane and piece: lane l takes the
+// 8-element pieces l and 64 + l of the row (rp pieces of kv_c, np pieces in all, np <= 128).  Loading,
+// converting and quantising are apart so that a caller can put other work between them (a conversion right
+// behind the loads would make the wave wait for them there).  Shared by the write kernel and by the decode
+// kernels' fused write, so that both store the same bytes.
+struct MlaRowRaw {
+  u32x4 w[2][2];   // 8 elements: one 16-byte word of 16-bit elements, two of fp32
+  bool have[2];
+};
+struct MlaRowPieces {
+  float x[2][8];
+  bool have[2];
+};
+__device__ __forceinline__ void mla_row_load_raw(const void* kv_c, const void* k_pe, int dt, int64_t kvc_elem,
+                                                 int64_t kpe_elem, int rp, int np, int lane, MlaRowRaw& r) {
+  const int64_t esz = dt == KVQ_F32 ? 4 : 2;
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const int piece = lane + kWave * j;
+    r.have[j] = piece < np;
+    const int pc = r.have[j] ? piece : 0;
+    const uint8_t* p = pc < rp ? static_cast<const uint8_t*>(kv_c) + (kvc_elem + 8 * pc) * esz
+                               : static_cast<const uint8_t*>(k_pe) + (kpe_elem + 8 * (pc - rp)) * esz;
+    r.w[j][0] = *reinterpret_cast<const u32x4_a4*>(p);
+    if (dt == KVQ_F32) r.w[j][1] = *reinterpret_cast<const u32x4_a4*>(p + 16);   // uniform
+    else r.w[j][1] = (u32x4){0u, 0u, 0u, 0u};
+  }
+}
+__device__ __forceinline__ void mla_row_convert(const MlaRowRaw& raw, int dt, MlaRowPieces& r) {
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    r.have[j] = raw.have[j];
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      const uint32_t e = raw.w[j][0][w];
+      const half2_t hh = __builtin_bit_cast(half2_t, e);
+      const float lo16 = dt == KVQ_BF16 ? as_f32(e << 16) : (float)hh.x;
+      const float hi16 = dt == KVQ_BF16 ? as_f32(e & 0xffff0000u) : (float)hh.y;
+      // fp32: elements 0-3 in word 0, 4-7 in word 1
+      r.x[j][2 * w] = dt == KVQ_F32 ? as_f32(raw.w[j][w >> 1][(2 * w) & 3]) : lo16;
+      r.x[j][2 * w + 1] = dt == KVQ_F32 ? as_f32(raw.w[j][w >> 1][(2 * w + 1) & 3]) : hi16;
+    }
+  }
+}
+__device__ __forceinline__ void mla_row_load(const void* kv_c, const void* k_pe, int dt, int64_t kvc_elem,
+                                             int64_t kpe_elem, int rp, int np, int lane, MlaRowPieces& r) {
+  MlaRowRaw raw;
+  mla_row_load_raw(kv_c, k_pe, dt, kvc_elem, kpe_elem, rp, np, lane, raw);
+  mla_row_convert(raw, dt, r);
+}
+// scale = max(amax, eps) / 127 (every lane of the wave takes part in the maximum)
+__device__ __forceinline__ float mla_row_scale(const MlaRowPieces& r, float eps) {
+  float amax = 0.f;
+#pragma unroll
+  for (int j = 0; j < 2; ++j)
+#pragma unroll
+    for (int i = 0; i < 8; ++i) amax = fmaxf(amax, r.have[j] ? fabsf(r.x[j][i]) : 0.f);
+#pragma unroll
+  for (int o = 32; o >= 1; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o, kWave));
+  return fmaxf(amax, eps) / 127.0f;
+}
+__device__ __forceinline__ void mla_row_store(const MlaRowPieces& r, float scale, uint8_t* row, float* scale_ptr, int lane) {
+  const bool pos = scale > 0.f;   // scale == 0: an all-zero row with eps 0
+  const float div = pos ? scale : 1.f;
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    if (!r.have[j]) continue;
+    uint32_t pk[2] = {0u, 0u};
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      float q = rintf(r.x[j][i] / div);
+      q = pos ? fminf(fmaxf(q, -128.f), 127.f) : 0.f;
+      pk[i >> 2] |= ((uint32_t)(int)q & 0xffu) << (8 * (i & 3));
+    }
+    *reinterpret_cast<u32x2_a4*>(row + 8 * (lane + kWave * j)) = (u32x2){pk[0], pk[1]};
+  }
+  if (lane == 0) *scale_ptr = scale;
+}
+
 __device__ __forceinline__ void lds_barrier() {
   asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }

@@ -64,40 +64,14 @@ __global__ __launch_bounds__(256) void mla_quant_write_rows8_kernel(const void* 
   const int64_t t = live ? t_raw : num_tokens - 1;
   const int rp = g.kv_lora_rank / 8, np = (g.kv_lora_rank + g.rope_dim) / 8;   // pieces of kv_c, of the row
   const int64_t slot = slot_mapping[t];  // in flight together with the row's loads
-  float x[2][8];
-  bool have[2];
-#pragma unroll
-  for (int j = 0; j < 2; ++j) {
-    const int piece = lane + kWave * j;
-    have[j] = piece < np;
-    const int pc = have[j] ? piece : 0;
-    if (pc < rp) load_row8(kv_c, dt, t * kv_c_stride + 8 * pc, x[j]);
-    else load_row8(k_pe, dt, t * k_pe_stride + 8 * (pc - rp), x[j]);
-  }
-  float amax = 0.f;
-#pragma unroll
-  for (int j = 0; j < 2; ++j)
-#pragma unroll
-    for (int i = 0; i < 8; ++i) amax = fmaxf(amax, have[j] ? fabsf(x[j][i]) : 0.f);
-  amax = fmaxf(wave_max(amax), eps);
-  const float scale = amax / 127.0f;
+  MlaRowPieces r;
+  mla_row_load(kv_c, k_pe, dt, t * kv_c_stride, t * k_pe_stride, rp, np, lane, r);
+  const float scale = mla_row_scale(r, eps);
   if (!live || slot < 0) return;  // padding token (after the shuffles: every lane took part)
   const int64_t blk = slot / g.block_size;
   const int64_t off = slot - blk * g.block_size;
-  uint8_t* row = cache + blk * g.stride_block + off * g.stride_row;
-#pragma unroll
-  for (int j = 0; j < 2; ++j) {
-    if (!have[j]) continue;
-    uint32_t pk[2] = {0u, 0u};
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      float r = scale > 0.f ? rintf(x[j][i] / scale) : 0.f;
-      r = fminf(fmaxf(r, -128.f), 127.f);
-      pk[i >> 2] |= ((uint32_t)(int)r & 0xffu) << (8 * (i & 3));
-    }
-    *reinterpret_cast<u32x2_a4*>(row + 8 * (lane + kWave * j)) = (u32x2){pk[0], pk[1]};
-  }
-  if (lane == 0) *reinterpret_cast<float*>(cache + blk * g.stride_block + g.scale_off + off * 4) = scale;
+  mla_row_store(r, scale, cache + blk * g.stride_block + off * g.stride_row,
+                reinterpret_cast<float*>(cache + blk * g.stride_block + g.scale_off + off * 4), lane);
 }
 
 // Round a float to the nearest value of the activation type (the arithmetic type of the rotary

@@ -79,7 +79,31 @@ struct MlaArgs {
   int num_splits;
   float scale_log2;
   uint32_t bs_magic;
+  // Fused write of the step's new latent rows (kvc_new == nullptr: the cache already holds them): row i of
+  // kvc_new [B, 512] / kpe_new [B, 64] is the token at position seq_lens[i] - 1 of sequence i.
+  const void* kvc_new;
+  const void* kpe_new;
+  int64_t kvc_stride, kpe_stride;  // elements
+  int new_dtype;
+  float new_eps;
 };
+
+// The fused cache update of the decode kernels: ONE wave loads (mla_new_row_load) and later quantises and stores
+// (mla_new_row_store) the sequence's new latent row at position len - 1, with the write kernel's arithmetic.
+__device__ __forceinline__ void mla_new_row_load(const MlaArgs& a, int seq, int lane, MlaRowRaw& raw) {
+  mla_row_load_raw(a.kvc_new, a.kpe_new, a.new_dtype, (int64_t)seq * a.kvc_stride, (int64_t)seq * a.kpe_stride,
+                   kMlaR / 8, kMlaW / 8, lane, raw);
+}
+__device__ __forceinline__ void mla_new_row_store(const MlaArgs& a, int seq, int len, int lane, const MlaRowRaw& raw) {
+  MlaRowPieces r;
+  mla_row_convert(raw, a.new_dtype, r);
+  const float scale = mla_row_scale(r, a.new_eps);
+  const int pos = len - 1;
+  const int e = (int)__umulhi((uint32_t)pos, a.bs_magic);
+  const int off = pos - e * a.g.block_size;
+  uint8_t* blk = const_cast<uint8_t*>(a.cache) + (int64_t)a.block_table[(int64_t)seq * a.bt_stride + e] * a.g.stride_block;
+  mla_row_store(r, scale, blk + (int64_t)off * a.g.stride_row, reinterpret_cast<float*>(blk + a.g.scale_off + (int64_t)off * 4), lane);
+}
 
 // Byte B of x0 and of x1, each a signed code, as the fp16 pair (x0.B, x1.B): the conversion reads its
 // byte through the operand's sub-dword select with sign extension and writes one half of the result, so
@@ -394,6 +418,23 @@ __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
   const int t_begin = tok_begin / kTile, t_end = (tok_end + kTile - 1) / kTile;
   const int bs = a.g.block_size;
   const int32_t* bt_row = a.block_table + (int64_t)seq * a.bt_stride;
+  // Fused write: the workgroup whose split holds the sequence's end stores the new row (its last wave does;
+  // every 128-head block of the sequence stores the same bytes).  The tile that holds the row must be loaded
+  // after the store has completed.  With three tiles or more that tile is requested inside the loop, after a
+  // tile barrier that follows the writer's wait for its own memory operations, so the row's loads may leave
+  // with the prologue's and its store after the query arithmetic; with fewer the write comes first and blocks.
+  const bool writes = a.kvc_new != nullptr && tok_end == len;
+  const bool write_first = writes && t_end - t_begin < 3;
+  if (write_first) {   // uniform over the workgroup
+    if (wave == 7) {
+      MlaRowRaw r;
+      mla_new_row_load(a, seq, lane, r);
+      mla_new_row_store(a, seq, len, lane, r);
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    lds_barrier();
+  }
+  const bool write_late = writes && !write_first && wave == 7;
 
   // ---- cooperative tile load, straight from global memory into LDS (no registers in between): a
   //      wave's load instruction fills 1024 contiguous LDS bytes, lane i the 16-byte slot i, with
@@ -478,6 +519,8 @@ __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
   }
   issue_loads(fetch_blocks(t_begin), lds[0]);
   Blocks nb = fetch_blocks(t_begin + 1);
+  MlaRowRaw new_row;
+  if (write_late) mla_new_row_load(a, seq, lane, new_row);
   __builtin_amdgcn_sched_barrier(0);
 
   i32x4 qreg[kMlaQRegOps];
@@ -525,6 +568,8 @@ __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
 #pragma unroll
     for (int op = 0; op < kMlaQRegOps; ++op) qreg[op] = (i32x4){0, 0, 0, 0};
   }
+
+  if (write_late) mla_new_row_store(a, seq, len, lane, new_row);
 
   // o[ht][b][i]: head 16 ht + c, dim 64 wave + 16 g + 4 i + b
   floatx4 o[8][4];
@@ -799,6 +844,19 @@ __global__ __launch_bounds__(kMlaSmallThreads) void mla_decode_small_kernel(MlaA
   const int t_begin = tok_begin / kTile, t_end = (tok_end + kTile - 1) / kTile;
   const int bs = a.g.block_size;
   const int32_t* bt_row = a.block_table + (int64_t)seq * a.bt_stride;
+  // Fused write: the wave that streams the sequence's last tile stores the new row.  A wave's tiles are its own;
+  // with three tiles or more of its own, the last one is requested after waits that cover the store, so the
+  // row's loads leave with the prologue's and its store after the query arithmetic; with fewer the write comes
+  // first and blocks.
+  const int my_tiles = t_begin + wave < t_end ? (t_end - 1 - (t_begin + wave)) / kMlaSmallWaves + 1 : 0;
+  const bool writes = a.kvc_new != nullptr && tok_end == len && wave == ((t_end - 1 - t_begin) & (kMlaSmallWaves - 1));
+  const bool write_late = writes && my_tiles >= 3;
+  if (writes && !write_late) {   // uniform over the wave
+    MlaRowRaw r;
+    mla_new_row_load(a, seq, lane, r);
+    mla_new_row_store(a, seq, len, lane, r);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  }
 
   // ---- one tile's rows in registers: k[mt][kk] = row 16 mt + c, dims 64 kk + 16 g .. + 15; ks[mt] = the
   //      scales of tokens 16 mt + 4 g .. + 3 (the four logits a lane holds per half)
@@ -882,6 +940,8 @@ __global__ __launch_bounds__(kMlaSmallThreads) void mla_decode_small_kernel(MlaA
     load_ksteps(rp, rr, 0, kMlaKSteps8);
     load_ids(t_begin + wave + kMlaSmallWaves, ids);
   }
+  MlaRowRaw new_row;
+  if (write_late) mla_new_row_load(a, seq, lane, new_row);
   __builtin_amdgcn_sched_barrier(0);
   if constexpr (QDT >= 0) {
     u32x4* qstage = reinterpret_cast<u32x4*>(lds_raw + kMlaSmallWaves * kMlaSmallWin);     // [18 operands][64 lanes]
@@ -915,6 +975,7 @@ __global__ __launch_bounds__(kMlaSmallThreads) void mla_decode_small_kernel(MlaA
     for (int op = 0; op < kMlaQOps; ++op) qreg[op] = __builtin_bit_cast(i32x4, qstage[op * kWave + lane]);
   }
   const float s2 = s1 / 254.0f;
+  if (write_late) mla_new_row_store(a, seq, len, lane, new_row);
 
   floatx4 o[32];   // o[4 d4 + b][i]: head c, dim 64 d4 + 16 g + 4 i + b
 #pragma unroll
@@ -1245,19 +1306,39 @@ static int mla_prepare_device() {
   return KVQ_OK;
 }
 
+// The step's new latent rows for the fused write: row i belongs to sequence i, position seq_lens[i] - 1.
+struct MlaNewRows {
+  const void* kv_c;
+  const void* k_pe;
+  int64_t kv_c_stride, k_pe_stride;  // elements
+  int dtype;
+  float eps;
+};
+
 }  // namespace kvq
 
-// Both entry points: `absorb` NULL = q holds the absorbed query (quantised by the decode kernel itself), else q
-// is unused and the absorb kernel prepares the operands from (q_nope, W_UK_T, q_pe).
+// All entry points: `absorb` NULL = q holds the absorbed query (quantised by the decode kernel itself), else q
+// is unused and the absorb kernel prepares the operands from (q_nope, W_UK_T, q_pe).  `fresh` non-NULL: the
+// decode launch also writes the step's new rows into the cache.
 static int mla_decode_run(const char* op, void* out, int out_dtype, float* lse, const void* q, int q_dtype,
                           int64_t q_stride_b, int64_t q_stride_h, const void* q_pe, int64_t q_pe_stride_b,
                           int64_t q_pe_stride_h, kvq::MlaAbsorbArgs* absorb, const void* cache,
                           const kvq_mla_geom* geom, const int32_t* block_table, int64_t bt_stride,
                           const int32_t* seq_lens, int num_seqs, int num_heads, float scale, void* workspace,
-                          size_t workspace_bytes, kvq_stream_t stream) {
+                          size_t workspace_bytes, kvq_stream_t stream, const kvq::MlaNewRows* fresh = nullptr) {
   using namespace kvq;
   KVQ_REQUIRE(geom != nullptr, "%s: geom is NULL", op);
   KVQ_REQUIRE(out && (q || absorb) && cache && block_table && seq_lens, "%s: NULL pointer", op);
+  if (fresh != nullptr) {
+    KVQ_REQUIRE(fresh->kv_c && fresh->k_pe, "%s: NULL kv_c / k_pe", op);
+    KVQ_REQUIRE(fresh->dtype == KVQ_F32 || fresh->dtype == KVQ_BF16 || fresh->dtype == KVQ_F16,
+                "%s: unknown src_dtype %d", op, fresh->dtype);
+    const int esz = fresh->dtype == KVQ_F32 ? 4 : 2;
+    KVQ_REQUIRE(((uintptr_t)fresh->kv_c % 4) == 0 && ((uintptr_t)fresh->k_pe % 4) == 0 &&
+                    (fresh->kv_c_stride * esz) % 4 == 0 && (fresh->k_pe_stride * esz) % 4 == 0,
+                "%s: kv_c / k_pe rows must be 4-byte aligned", op);
+    KVQ_REQUIRE(fresh->eps >= 0.f, "%s: eps must not be negative", op);
+  }
   KVQ_REQUIRE(num_seqs > 0 && num_seqs <= 65535 && num_heads > 0, "%s: num_seqs / num_heads out of range", op);
   KVQ_REQUIRE(((uintptr_t)out % 16) == 0, "%s: out must be 16-byte aligned", op);
   const kvq_mla_geom& g = *geom;
@@ -1306,6 +1387,14 @@ static int mla_decode_run(const char* op, void* out, int out_dtype, float* lse, 
   a.num_splits = splits;
   a.scale_log2 = scale * kLog2e;
   a.bs_magic = (uint32_t)((0x100000000ull + (uint64_t)g.block_size - 1) / (uint64_t)g.block_size);
+  if (fresh != nullptr) {
+    a.kvc_new = fresh->kv_c;
+    a.kpe_new = fresh->k_pe;
+    a.kvc_stride = fresh->kv_c_stride;
+    a.kpe_stride = fresh->k_pe_stride;
+    a.new_dtype = fresh->dtype;
+    a.new_eps = fresh->eps;
+  }
   hipStream_t s = as_stream(stream);
   dim3 grid(splits, num_seqs, (num_heads + 127) / 128);
   if (int e = mla_prepare_device()) return e;
@@ -1392,6 +1481,19 @@ int kvq_mla_decode_int8(void* out, int out_dtype, float* lse, const void* q, int
   return mla_decode_run("mla_decode_int8", out, out_dtype, lse, q, q_dtype, q_stride_b, q_stride_h, q_pe, q_pe_stride_b,
                         q_pe_stride_h, nullptr, cache, geom, block_table, bt_stride, seq_lens, num_seqs, num_heads,
                         scale, workspace, workspace_bytes, stream);
+}
+
+int kvq_mla_decode_int8_fused_write(void* out, int out_dtype, float* lse, const void* q, int q_dtype,
+                                    int64_t q_stride_b, int64_t q_stride_h, const void* q_pe, int64_t q_pe_stride_b,
+                                    int64_t q_pe_stride_h, const void* kv_c, const void* k_pe, int src_dtype,
+                                    int64_t kv_c_stride, int64_t k_pe_stride, float eps, void* cache,
+                                    const kvq_mla_geom* geom, const int32_t* block_table, int64_t bt_stride,
+                                    const int32_t* seq_lens, int num_seqs, int num_heads, float scale,
+                                    void* workspace, size_t workspace_bytes, kvq_stream_t stream) {
+  const kvq::MlaNewRows fresh{kv_c, k_pe, kv_c_stride, k_pe_stride, src_dtype, eps};
+  return mla_decode_run("mla_decode_int8_fused_write", out, out_dtype, lse, q, q_dtype, q_stride_b, q_stride_h, q_pe,
+                        q_pe_stride_b, q_pe_stride_h, nullptr, cache, geom, block_table, bt_stride, seq_lens, num_seqs,
+                        num_heads, scale, workspace, workspace_bytes, stream, &fresh);
 }
 
 int kvq_mla_decode_absorb_int8(void* out, int out_dtype, float* lse, const void* q_nope, int q_dtype,

@@ -14,7 +14,7 @@ LIB_PATH = os.path.join(_LIB_DIR, "libkvq_hip.so")
 
 KVQ_F32, KVQ_BF16, KVQ_F16 = 0, 1, 2
 KVQ_CODE_INT8, KVQ_CODE_FP8_E4M3 = 0, 1
-ABI_VERSION = 11
+ABI_VERSION = 12
 
 
 class CacheGeom(ctypes.Structure):
@@ -73,6 +73,8 @@ SIGNATURES = {
     "kvq_mla_decode_workspace_bytes": (_sz, [_i, _i, _i]),
     "kvq_mla_decode_int8": (_i, [_vp, _i, _vp, _vp, _i, _i64, _i64, _vp, _i64, _i64, _vp, _mla_p, _vp, _i64, _vp,
                                  _i, _i, _f, _vp, _sz, _vp]),
+    "kvq_mla_decode_int8_fused_write": (_i, [_vp, _i, _vp, _vp, _i, _i64, _i64, _vp, _i64, _i64, _vp, _vp, _i, _i64,
+                                             _i64, _f, _vp, _mla_p, _vp, _i64, _vp, _i, _i, _f, _vp, _sz, _vp]),
     "kvq_mla_decode_absorb_int8": (_i, [_vp, _i, _vp, _vp, _i, _i64, _i64, _i, _vp, _i64, _i64, _vp, _i64, _i64, _vp,
                                         _mla_p, _vp, _i64, _vp, _i, _i, _f, _vp, _sz, _vp]),
     "kvq_concat_mla_q": (_i, [_vp, _i64, _i64, _vp, _i64, _i64, _vp, _i64, _i64, _i, _i64, _i, _i, _i, _vp]),

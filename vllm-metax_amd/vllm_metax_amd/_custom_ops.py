@@ -715,18 +715,28 @@ def mla_decode_workspace_bytes(max_num_seqs: int, num_heads: int, kv_lora_rank: 
 
 def mla_decode_int8(q, kv_cache: torch.Tensor, o: torch.Tensor, lse: torch.Tensor | None,
                     block_table: torch.Tensor, seq_lens: torch.Tensor, sm_scale: float, kv_lora_rank: int,
-                    workspace: torch.Tensor | None = None, geometry: MlaGeometry | None = None) -> None:
+                    workspace: torch.Tensor | None = None, geometry: MlaGeometry | None = None,
+                    new_rows: tuple[torch.Tensor, torch.Tensor] | None = None) -> None:
     """MLA decode over the int8 latent cache: the job of ``decode_attention_fwd(..., is_mla=True)``
     (vllm_metax/v1/attention/ops/triton_decode_attention.py:763-825).  q ``[B, H, R+P]`` or the pair
     ``(ql_nope [B, H, R], q_pe [B, H, P])`` that ``forward_mqa`` may receive
     (vllm_metax/v1/attention/backends/mla/triton_mla.py:226-238; read as it is, no concatenation),
-    o ``[B, H, R]``, lse ``[B, H]`` fp32 or None."""
+    o ``[B, H, R]``, lse ``[B, H]`` fp32 or None.  ``new_rows`` = (kv_c ``[B, R]``, k_pe ``[B, P]``): see
+    :func:`mla_decode_with_cache_update`."""
     q_pe = None
     if type(q) is tuple:
         q, q_pe = q
-    dev = _require_cuda(q, q_pe, kv_cache, o, lse, block_table, seq_lens, workspace)
+    kv_c, k_pe = new_rows if new_rows is not None else (None, None)
+    dev = _require_cuda(q, q_pe, kv_cache, o, lse, block_table, seq_lens, workspace, kv_c, k_pe)
     geom = geometry or mla_geometry(kv_cache, kv_lora_rank)
     B, H, W = q.shape
+    if new_rows is not None:
+        if kv_c.dim() != 2 or k_pe.dim() != 2 or kv_c.dtype != k_pe.dtype:
+            raise RuntimeError("kv_c [B, R] and k_pe [B, P] must be 2-D of one dtype")
+        if tuple(kv_c.shape) != (B, geom.kv_lora_rank) or tuple(k_pe.shape) != (B, geom.rope_dim):
+            raise RuntimeError("kv_c / k_pe must hold one row per sequence, as wide as the cache entry")
+        if kv_c.stride(1) != 1 or k_pe.stride(1) != 1:
+            raise RuntimeError("kv_c / k_pe rows must be contiguous")
     if q_pe is None:
         if W != geom.kv_lora_rank + geom.rope_dim:
             raise RuntimeError("q must be [B, H, R+P]")
@@ -747,16 +757,33 @@ def mla_decode_int8(q, kv_cache: torch.Tensor, o: torch.Tensor, lse: torch.Tenso
     if workspace is None:
         workspace = _default_workspace(dev, need)
     g = geom.as_struct()
+    head = (_ptr(o), _dtype_code(o, "o"), _ptr(lse), _ptr(q), _dtype_code(q, "q"), q.stride(0), q.stride(1), _ptr(q_pe),
+            q_pe.stride(0) if q_pe is not None else 0, q_pe.stride(1) if q_pe is not None else 0)
     with _on_device(dev):
-        rc = _C.load().kvq_mla_decode_int8(_ptr(o), _dtype_code(o, "o"), _ptr(lse), _ptr(q), _dtype_code(q, "q"),
-                                           q.stride(0), q.stride(1), _ptr(q_pe),
-                                           q_pe.stride(0) if q_pe is not None else 0,
-                                           q_pe.stride(1) if q_pe is not None else 0,
-                                           ctypes.c_void_p(geom.base_ptr), ctypes.byref(g),
-                                           _ptr(block_table), block_table.stride(0), _ptr(seq_lens), B, H,
-                                           float(sm_scale), _ptr(workspace),
-                                           workspace.numel() * workspace.element_size(), _stream(dev))
-    _C.check(rc, "mla_decode_int8")
+        tail = (ctypes.c_void_p(geom.base_ptr), ctypes.byref(g), _ptr(block_table), block_table.stride(0),
+                _ptr(seq_lens), B, H, float(sm_scale), _ptr(workspace),
+                workspace.numel() * workspace.element_size(), _stream(dev))
+        if new_rows is None:
+            rc = _C.load().kvq_mla_decode_int8(*head, *tail)
+        else:
+            rc = _C.load().kvq_mla_decode_int8_fused_write(*head, _ptr(kv_c), _ptr(k_pe), _dtype_code(kv_c, "kv_c"),
+                                                           kv_c.stride(0), k_pe.stride(0),
+                                                           eps_for_dtype(kv_c.dtype), *tail)
+    _C.check(rc, "mla_decode_int8" if new_rows is None else "mla_decode_int8_fused_write")
+
+
+def mla_decode_with_cache_update(q, kv_c: torch.Tensor, k_pe: torch.Tensor, kv_cache: torch.Tensor, o: torch.Tensor,
+                                 lse: torch.Tensor | None, block_table: torch.Tensor, seq_lens: torch.Tensor,
+                                 sm_scale: float, kv_lora_rank: int, workspace: torch.Tensor | None = None,
+                                 geometry: MlaGeometry | None = None) -> None:
+    """One decode step of an MLA layer in one launch: ``concat_and_cache_mla(kv_c, k_pe, kv_cache, slot_mapping)``
+    followed by :func:`mla_decode_int8`, for a batch that holds one new token per sequence (row i of kv_c / k_pe is
+    the token at position ``seq_lens[i] - 1`` of sequence i; its slot comes from the block table, as
+    ``slot_mapping`` would name it).  What ``do_kv_cache_update`` + ``forward_mqa`` do in two steps
+    (vllm_metax/v1/attention/backends/mla/triton_mla.py:226-295); cache bytes and outputs are those of the two
+    calls."""
+    mla_decode_int8(q, kv_cache, o, lse, block_table, seq_lens, sm_scale, kv_lora_rank, workspace, geometry,
+                    new_rows=(kv_c, k_pe))
 
 
 def mla_decode_absorb_int8(q_nope: torch.Tensor, W_UK_T: torch.Tensor, q_pe: torch.Tensor, kv_cache: torch.Tensor,
