@@ -246,8 +246,12 @@ def build_mla_state(cfg, dev, layers, seed=0):
     return st
 
 
-def run_mla_step(st, layer, ops, cfg, write=True, attn=True):
+def run_mla_step(st, layer, ops, cfg, write=True, attn=True, fused=False):
     cache = st["caches"][layer]
+    if fused:   # the same step in one launch: the decode kernel writes the new rows itself
+        ops.mla_decode_with_cache_update(st["q"], st["new_c"], st["new_pe"], cache, st["out"], st["lse"], st["bt_d"],
+                                         st["sl_d"], st["scale"], cfg["r"], workspace=st["ws"])
+        return
     if write:
         ops.concat_and_cache_mla(st["new_c"], st["new_pe"], cache, st["slots_new"])
     if attn:
@@ -298,6 +302,14 @@ def mla_main(args, cfg, dev, ops):
     dt = (time.perf_counter() - t0) / args.steps
     n_ev = max(args.steps, 100)
     attn_s = time_back_to_back(lambda i: run_mla_step(st, i % L, ops, cfg, write=False, attn=True), n_ev)
+    for i in range(args.warmup):
+        run_mla_step(st, i % L, ops, cfg, fused=True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        run_mla_step(st, i % L, ops, cfg, fused=True)
+    torch.cuda.synchronize()
+    fused_s = (time.perf_counter() - t0) / args.steps
     traffic, traffic_source = measured_traffic(args.workload)
     small = cfg["heads"] <= 16   # one head tile: a kernel of its own, which also prepares the query
     # at 16 heads the launch moves few flops per byte: the HBM roof is the one that binds
@@ -320,6 +332,10 @@ def mla_main(args, cfg, dev, ops):
                      "algorithmic_flops_per_launch": flops, "algorithmic_bytes_per_launch": nbytes,
                      "hbm_frac_of_peak": round(nbytes / attn_s / 1e9 / HBM_PEAK_GBPS, 4)},
     }
+    res["one_launch_step"] = {"what": "the same layer step with the latent write inside the decode launch "
+                                      "(kvq_mla_decode_int8_fused_write)",
+                              "us_per_layer": round(fused_s * 1e6, 2), "value": round(nbytes / fused_s / 1e9, 1),
+                              "unit": "GB/s"}
     res["decode_caller"] = mla_caller_chain(cfg, st, dev, ops, n_ev)
     if not args.no_cpu_baseline:
         res["cpu_baseline"] = mla_cpu_baseline(cfg, st, args.cpu_seconds)

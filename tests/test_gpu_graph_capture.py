@@ -97,7 +97,8 @@ def test_decode_step_replays_correctly(gpu_device, one_launch):
         assert torch.equal(eager, out), f"replay {it}: graph and eager outputs differ"
 
 
-def test_mla_decode_replays_correctly(gpu_device):
+@pytest.mark.parametrize("one_launch", [False, True], ids=["write_then_decode", "one_launch_step"])
+def test_mla_decode_replays_correctly(gpu_device, one_launch):
     dev = gpu_device
     R, P, H, bs, nb, B = 512, 64, 16, 64, 12, 2
     g = torch.Generator().manual_seed(8)
@@ -125,6 +126,10 @@ def test_mla_decode_replays_correctly(gpu_device):
     geom = L.mla_geometry(cache, R)
 
     def step():
+        if one_launch:
+            ops.mla_decode_with_cache_update(q, kv_c, k_pe, cache, o, lse, bt_d, seq_lens, 0.0722, R, workspace=ws,
+                                             geometry=geom)
+            return
         ops.concat_and_cache_mla(kv_c, k_pe, cache, slots, geometry=geom)
         ops.mla_decode_int8(q, cache, o, lse, bt_d, seq_lens, 0.0722, R, workspace=ws, geometry=geom)
 

@@ -231,6 +231,19 @@ def test_mla_backend_forward_mqa(gpu_device):
     want, want_lse = oracle.mla_decode(torch.cat([ql, qp], -1), cpu_cache, lay, bt, torch.tensor(ctx, dtype=torch.int32), 0.0722)
     T.assert_close_attn(o, want, what="forward_mqa")
     torch.testing.assert_close(lse.cpu(), want_lse, atol=5e-3, rtol=1e-3)
+    # the next step as one call: cache update and decode in one launch
+    ctx2 = [c + 1 for c in ctx]
+    new_c = torch.randn((2, R), generator=g).to(torch.bfloat16)
+    new_pe = torch.randn((2, 1, P), generator=g).to(torch.bfloat16)
+    slots = torch.tensor([int(bt[i, (c - 1) // bs]) * bs + (c - 1) % bs for i, c in enumerate(ctx2)])
+    oracle.mla_cache_write(new_c, new_pe.reshape(2, P), cpu_cache, lay, slots)
+    md.decode.seq_lens = torch.tensor(ctx2, dtype=torch.int32, device=dev)
+    o, lse = impl.forward_mqa_with_cache_update((ql.to(dev), qp.to(dev)), new_c.to(dev), new_pe.to(dev), cache, md)
+    torch.cuda.synchronize()
+    assert torch.equal(cache.cpu(), cpu_cache)
+    want, want_lse = oracle.mla_decode(torch.cat([ql, qp], -1), cpu_cache, lay, bt, torch.tensor(ctx2, dtype=torch.int32), 0.0722)
+    T.assert_close_attn(o, want, what="forward_mqa_with_cache_update")
+    torch.testing.assert_close(lse.cpu(), want_lse, atol=5e-3, rtol=1e-3)
 
 
 def test_mla_decode_caller_absorb_decode_up_proj(gpu_device):

@@ -297,9 +297,10 @@ class Int8MLAImpl(_MLAImplBase):
         ops.concat_and_cache_mla(kv_c_normed, k_pe.reshape(k_pe.shape[0], -1), kv_cache, slot_mapping,
                                  kv_cache_dtype or self.kv_cache_dtype, k_scale, geometry=self._geom(kv_cache))
 
-    def forward_mqa(self, q, kv_c_and_k_pe_cache: torch.Tensor, attn_metadata, layer=None):
+    def forward_mqa(self, q, kv_c_and_k_pe_cache: torch.Tensor, attn_metadata, layer=None, new_rows=None):
         """``q`` [B, H, 576] or ``(ql_nope [B, H, 512], q_pe [B, H, 64])``; returns
-        ``(o [B, H, kv_lora_rank], lse [B, H] float32)``."""
+        ``(o [B, H, kv_lora_rank], lse [B, H] float32)``.  ``new_rows`` = (kv_c_normed [B, R], k_pe [B, P]):
+        the launch also writes the step's rows (see ``forward_mqa_with_cache_update``)."""
         assert kv_c_and_k_pe_cache.numel() > 0
         assert attn_metadata.decode is not None
         # a (ql_nope, q_pe) pair goes to the kernel as it is: the reference concatenates first
@@ -318,8 +319,21 @@ class Int8MLAImpl(_MLAImplBase):
         ops.mla_decode_int8(q, kv_c_and_k_pe_cache, o, lse, attn_metadata.decode.block_table,
                             attn_metadata.decode.seq_lens, self.scale, self.kv_lora_rank,
                             workspace=getattr(attn_metadata, "workspace", None),
-                            geometry=self._geom(kv_c_and_k_pe_cache))
+                            geometry=self._geom(kv_c_and_k_pe_cache), new_rows=new_rows)
         return o, lse
+
+    def forward_mqa_with_cache_update(self, q, kv_c_normed: torch.Tensor, k_pe: torch.Tensor,
+                                      kv_c_and_k_pe_cache: torch.Tensor, attn_metadata, layer=None):
+        """``do_kv_cache_update`` + ``forward_mqa`` of a decode-only batch (one new token per sequence, row i
+        of ``kv_c_normed`` / ``k_pe`` at position ``seq_lens[i] - 1`` of sequence i) in one launch: the two
+        calls the reference's MLA layer makes for such a batch
+        (vllm_metax/model_executor/layers/attention/mla_attention.py:633-640, then forward_mqa,
+        vllm_metax/v1/attention/backends/mla/triton_mla.py:226-295).  Same cache bytes, same result."""
+        B = (q[0] if type(q) is tuple else q).shape[0]
+        if kv_c_normed.shape[0] != B:
+            raise RuntimeError("one new token per sequence: a batch with prefill tokens takes the two calls")
+        return self.forward_mqa(q, kv_c_and_k_pe_cache, attn_metadata, layer,
+                                new_rows=(kv_c_normed, k_pe.reshape(B, -1)))
 
     def _kv_up_proj(self, kv_c: torch.Tensor) -> torch.Tensor:
         if self.kv_b_proj is None:
