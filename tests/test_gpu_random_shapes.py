@@ -136,3 +136,65 @@ def test_mla_decode_random_cases(gpu_device, block):
         torch.testing.assert_close(lse.cpu()[live], want_lse[live], atol=5e-3, rtol=1e-3, msg=what)
         if (~live).any():
             assert torch.equal(o.float().cpu()[~live], torch.zeros_like(want[~live])), what
+
+
+def _draw_write(case):
+    rng = random.Random(7717 * case + 5)
+    return dict(hkv=rng.choice([1, 2, 3, 4, 8, 16]), d=rng.choice([64, 80, 96, 112, 128, 128, 256]),
+                bs=rng.choice([16, 32, 64]), layout=rng.choice(["NHD", "HND"]),
+                dtype=rng.choice([torch.bfloat16, torch.float16, torch.float32]), fp8=rng.random() < 0.25,
+                tokens=rng.choice([1, 2, 63, 64, 65, rng.randint(1, 400), rng.randint(1, 3000)]),
+                mag=rng.choice([1e-12, 1e-6, 1e-3, 1.0, 1.0, 30.0, 3000.0]), zero_rows=rng.random() < 0.3,
+                strided=rng.random() < 0.3)
+
+
+@pytest.mark.parametrize("block", range(6))
+def test_cache_write_random_cases_bit_exact(gpu_device, block):
+    """Quantise-on-write: every byte of the cache (codes, scales, untouched slots) equals the oracle's, for shapes,
+    source types, magnitudes (down to rows below the scale floor) and slot patterns drawn at random; MLA rows too."""
+    dev = gpu_device
+    for case in range(10 * block, 10 * block + 10):
+        c = _draw_write(case)
+        what = f"case {case}: {c}"
+        g = torch.Generator().manual_seed(case)
+        hkv, d, bs, n = c["hkv"], c["d"], c["bs"], c["tokens"]
+        nb = (n + bs - 1) // bs + 3
+        src = (torch.randn((n, 2, hkv, d), generator=g) * c["mag"]).to(c["dtype"])
+        if c["zero_rows"]:
+            src[::3, 0] = 0
+            src[1::4, 1, hkv - 1] = 0
+        if c["strided"]:
+            key, val = src[:, 0], src[:, 1]                  # the two halves of one projection output
+        else:
+            key, val = src[:, 0].contiguous(), src[:, 1].contiguous()
+        slots = torch.randperm(nb * bs, generator=g)[:n].to(torch.int64)
+        slots[torch.rand(n, generator=g) < 0.1] = -1
+        code = oracle.CODE_FP8 if c["fp8"] else oracle.CODE_INT8
+        kv_cpu, _, lay = T.cpu_cache(nb, bs, hkv, d, c["layout"], fill=0x11)
+        oracle.cache_write(key, val, T.storage_bytes(kv_cpu), lay, slots, code_type=code)
+        kv = L.allocate_kv_cache(nb, bs, hkv, d, device=dev, layout=c["layout"], fill=0x11)
+        k, v = L.key_value_views(kv)
+        ks, vs = L.scale_views(kv)
+        srcd = src.to(dev)
+        kd, vd = (srcd[:, 0], srcd[:, 1]) if c["strided"] else (srcd[:, 0].contiguous(), srcd[:, 1].contiguous())
+        mode = KVQuantMode.FP8_PER_TOKEN_HEAD if c["fp8"] else KVQuantMode.INT8_PER_TOKEN_HEAD
+        ops.reshape_and_cache_flash_per_token_head_quant(kd, vd, k, v, ks, vs, slots.to(dev), kv_quant_mode=mode)
+        torch.cuda.synchronize()
+        assert torch.equal(T.storage_bytes(kv).cpu(), T.storage_bytes(kv_cpu)), what
+        # the MLA latent row of the same case: [kv_c | k_pe], one scale per row
+        R, P = 512, 64
+        rows = (torch.randn((n, R + P), generator=g) * c["mag"]).to(c["dtype"])
+        if c["zero_rows"]:
+            rows[::5] = 0
+        cache_cpu = L.allocate_mla_cache(nb, bs, R + P, device="cpu", fill=0x11)
+        codes, scales = L.mla_cache_views(cache_cpu)
+        mlay = oracle.MlaLayout.from_views(cache_cpu, codes, scales, R)
+        oracle.mla_cache_write(rows[:, :R], rows[:, R:], cache_cpu, mlay, slots)
+        cache = L.allocate_mla_cache(nb, bs, R + P, device=dev, fill=0x11)
+        rd = rows.to(dev)
+        if c["strided"]:
+            ops.concat_and_cache_mla(rd[:, :R], rd[:, R:], cache, slots.to(dev))
+        else:
+            ops.concat_and_cache_mla(rd[:, :R].contiguous(), rd[:, R:].contiguous(), cache, slots.to(dev))
+        torch.cuda.synchronize()
+        assert torch.equal(T.storage_bytes(cache).cpu(), T.storage_bytes(cache_cpu)), what + " (MLA rows)"
