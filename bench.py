@@ -383,6 +383,7 @@ def mixed_main(args, cfg, dev, ops):
     from vllm_metax_amd import layout as L
 
     hq, hkv, d, bs, ctx, qls, pool = (cfg[k] for k in ("hq", "hkv", "d", "bs", "ctx", "qlens", "pool"))
+    mode = _quant_mode(cfg)
     B = len(ctx)
     g = torch.Generator().manual_seed(0)
     need = [(c + bs - 1) // bs for c in ctx]
@@ -416,7 +417,7 @@ def mixed_main(args, cfg, dev, ops):
             slots = bt_d[i, pos // bs].to(torch.int64) * bs + pos % bs
             ops.reshape_and_cache_flash_per_token_head_quant(
                 torch.randn((c, hkv, d), device=dev).to(torch.bfloat16), torch.randn((c, hkv, d), device=dev).to(torch.bfloat16),
-                k, v, ks, vs, slots, geometry=geom)
+                k, v, ks, vs, slots, geometry=geom, kv_quant_mode=mode)
         caches.append(dict(k=k, v=v, ks=ks, vs=vs, geom=geom, kv=kv))
     q = torch.randn((n_tok, hq, d), device=dev).to(torch.bfloat16)
     new_k = torch.randn((n_tok, hkv, d), device=dev).to(torch.bfloat16)
@@ -429,10 +430,11 @@ def mixed_main(args, cfg, dev, ops):
         c = caches[layer]
         if write:
             ops.reshape_and_cache_flash_per_token_head_quant(new_k, new_v, c["k"], c["v"], c["ks"], c["vs"], new_slots,
-                                                             geometry=c["geom"])
+                                                             geometry=c["geom"], kv_quant_mode=mode)
         if attn:
             ops.unified_attention(q, c["k"], c["v"], out, cu_d, max(qls), sl_d, max(ctx), scale, True, block_table=bt_d,
                                   k_scale_cache=c["ks"], v_scale_cache=c["vs"], workspace=ws, geometry=c["geom"],
+                                  kv_quant_mode=mode,
                                   **_window_kwargs(dict(window=args.sliding_window, softcap=args.soft_cap)))
 
     Lr = args.layers
@@ -453,12 +455,13 @@ def mixed_main(args, cfg, dev, ops):
     pre_bytes = sum(c for c, ql in zip(ctx, qls) if ql > 1) * hkv * 2 * (d + 4) + 2 * n_tok * hq * d * 2
     write_bytes = n_tok * hkv * (2 * d * 2 + 2 * (d + 4))
     res = {
-        "metric": "int8-KV mixed batch (4 x 2048-token prefill chunks + 60 decode rows): ms per layer",
+        "metric": f"{cfg.get('kv_dtype', 'int8')}-KV mixed batch (4 x 2048-token prefill chunks + 60 decode rows): ms per layer",
         "value": round((dec_bytes + pre_bytes + write_bytes) / dt / 1e9, 1), "unit": "GB/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(dt * 1e3, 5), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None,
-        "dtype": "int8 KV codes, fp16 MFMA operands, fp32 softmax/accumulate, bf16 Q/out", "data": "synthetic",
+        "dtype": f"{cfg.get('kv_dtype', 'int8')} KV codes, fp16 MFMA operands, fp32 softmax/accumulate, bf16 Q/out", "data": "synthetic",
         "config": {"workload": args.workload,
+                   **({"kv_dtype": "fp8_per_token_head"} if cfg.get("kv_dtype") == "fp8" else {}),
                    **({"sliding_window": args.sliding_window} if args.sliding_window else {}),
                    **({"soft_cap": args.soft_cap} if args.soft_cap else {}),
                    "batch": B, "new_tokens": n_tok, "sum_ctx": sum(ctx), "q_heads": hq,

@@ -131,6 +131,35 @@ def test_mixed_batch_matches_oracle(gpu_device):
     T.assert_close_attn(got, want, what="fp8 mixed batch")
 
 
+@pytest.mark.parametrize("hq,hkv,d,qls,window,cap", [
+    (32, 8, 128, [300, 1, 64, 2048], 0, 0.0),      # long chunks: the workgroup-shared fp16 tile expands fp8 codes
+    (28, 4, 128, [257, 33, 1, 700], 0, 0.0),       # 7 q heads per kv head
+    (16, 8, 64, [500, 100, 1, 90], 0, 0.0),
+    (32, 8, 128, [300, 1, 64, 900], 128, 0.0),     # its window / soft-cap instantiation
+    (32, 8, 128, [300, 1, 64, 900], 0, 30.0),
+    (8, 8, 128, [40, 1, 63, 17], 0, 0.0),          # fewer than 64 columns: the per-wave tile
+])
+def test_prefill_chunks_both_tiles(gpu_device, hq, hkv, d, qls, window, cap):
+    """fp8 codes through both prefill kernels, outlier-heavy sources (large scales, many subnormal codes)."""
+    ctx = [q + extra for q, extra in zip(qls, [700, 2000, 0, 133])]
+    kv, lay, bt, q, sl, cu = _fp8_case(ctx, qls, hq, hkv, d, 16, seed=hq + d + window, outlier=True)
+    scale = 1 / math.sqrt(d)
+    want, want_lse = oracle.paged_attn(q, T.storage_bytes(kv), lay, bt, sl, cu, scale, return_lse=True,
+                                       sliding_window=window, soft_cap=cap, code_type=oracle.CODE_FP8)
+    dev = gpu_device
+    kvd = T.to_device_cache(kv, dev, "NHD")
+    k, v = L.key_value_views(kvd)
+    ks, vs = L.scale_views(kvd)
+    out = torch.full(q.shape, float("nan"), dtype=torch.bfloat16, device=dev)
+    lse = torch.full(q.shape[:2], float("nan"), dtype=torch.float32, device=dev)
+    ops.unified_attention(q.to(dev), k, v, out, cu.to(dev), max(qls), sl.to(dev), int(sl.max()), scale, True,
+                          window_size=(window - 1, 0) if window else (-1, -1), softcap=cap, block_table=bt.to(dev),
+                          k_scale_cache=ks, v_scale_cache=vs, kv_quant_mode=FP8, lse=lse)
+    torch.cuda.synchronize()
+    T.assert_close_attn(out, want, what=f"fp8 prefill {hq}/{hkv} d{d} window {window} cap {cap}")
+    torch.testing.assert_close(lse.cpu(), want_lse, atol=5e-3, rtol=1e-3)
+
+
 def test_backend_serves_fp8_per_token_head(gpu_device):
     dev = gpu_device
     hq, hkv, d, bs, nb = 32, 8, 128, 16, 60

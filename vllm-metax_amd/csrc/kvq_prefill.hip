@@ -336,9 +336,10 @@ __global__ __launch_bounds__(WPW * 64) void paged_prefill_kernel(PrefillArgs a) 
 // the other's ALU- and MFMA-bound phases.
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
-template <int D, int QDT, int ODT>
+template <int D, int QDT, int ODT, int CODE = KVQ_CODE_INT8>
 struct Flash32 {
-  using DTile = DecodeTile<D, QDT, ODT>;
+  using DTile = DecodeTile<D, QDT, ODT, CODE>;
+  static constexpr bool FP8 = DTile::FP8;   // e4m3fn codes: they enter the MFMA as value / 2^8, without a bias
   static constexpr int WAVES = 4;
   static constexpr int KS = D / 16;                      // k-steps of the QK product
   static constexpr int MT = D / 32;                      // 32-dim row tiles of O^T
@@ -353,6 +354,7 @@ struct Flash32 {
   static constexpr int COLS = 32 * WAVES;
 
   __device__ static __forceinline__ uint32_t to_half2(uint32_t x, bool upper) {
+    if constexpr (FP8) return fp8_bytes_to_half2(x, upper);
     const half2_t bias = {(half_t)kCodeBias, (half_t)kCodeBias};
     const half2_t v = __builtin_bit_cast(half2_t, bytes_to_half2(x, upper)) - bias;
     return __builtin_bit_cast(uint32_t, v);
@@ -404,7 +406,7 @@ struct Flash32 {
       for (int j = 0; j < 8; ++j) qsum += (float)qb[ks][j];  // the sum of what the MFMA will actually see
     }
     qsum += __shfl_xor(qsum, 32, kWave);
-    return -kCodeBias * qsum;
+    return FP8 ? 0.f : -kCodeBias * qsum;
   }
 
   // Raw tile -> fp16 K [token][dim] (codes + 1152) and V^T [dim][position] (codes); token t of the tile sits at position
@@ -418,12 +420,12 @@ struct Flash32 {
       u32x4 lo, hi;
 #pragma unroll
       for (int i = 0; i < 2; ++i) {
-        const uint32_t x = w[i] ^ 0x80808080u;
-        lo[2 * i] = bytes_to_half2(x, false);
-        lo[2 * i + 1] = bytes_to_half2(x, true);
-        const uint32_t y = w[2 + i] ^ 0x80808080u;
-        hi[2 * i] = bytes_to_half2(y, false);
-        hi[2 * i + 1] = bytes_to_half2(y, true);
+        const uint32_t x = prep_codes<FP8>(w[i]);
+        lo[2 * i] = codes_to_half2<FP8>(x, false);
+        lo[2 * i + 1] = codes_to_half2<FP8>(x, true);
+        const uint32_t y = prep_codes<FP8>(w[2 + i]);
+        hi[2 * i] = codes_to_half2<FP8>(y, false);
+        hi[2 * i + 1] = codes_to_half2<FP8>(y, true);
       }
       *reinterpret_cast<u32x4*>(buf + tok * K_PITCH + 32 * ch) = lo;
       *reinterpret_cast<u32x4*>(buf + tok * K_PITCH + 32 * ch + 16) = hi;
@@ -433,7 +435,7 @@ struct Flash32 {
       uint32_t t[4];
 #pragma unroll
       for (int a = 0; a < 4; ++a)
-        t[a] = *reinterpret_cast<const uint32_t*>(raw + (4 * tg + a) * RAW_PITCH + (D + 4) + 4 * dq) ^ 0x80808080u;
+        t[a] = prep_codes<FP8>(*reinterpret_cast<const uint32_t*>(raw + (4 * tg + a) * RAW_PITCH + (D + 4) + 4 * dq));
       const uint32_t a01 = perm(t[1], t[0], 0x05010400u), b01 = perm(t[1], t[0], 0x07030602u);
       const uint32_t a23 = perm(t[3], t[2], 0x05010400u), b23 = perm(t[3], t[2], 0x07030602u);
       const int pos = (tg >> 2) * 16 + (tg & 1) * 8 + ((tg >> 1) & 1) * 4;
@@ -572,9 +574,9 @@ struct Flash32 {
 };
 
 // EXT adds the sliding window and the logits soft cap; the plain causal kernel carries neither.
-template <int D, int QDT, int ODT, bool EXT>
+template <int D, int QDT, int ODT, bool EXT, int CODE = KVQ_CODE_INT8>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void paged_prefill_flash32_kernel(PrefillArgs a) {
-  using FP = Flash32<D, QDT, ODT>;
+  using FP = Flash32<D, QDT, ODT, CODE>;
   using DTile = typename FP::DTile;
   extern __shared__ __align__(16) uint8_t lds[];
   uint8_t* raws = lds;
@@ -664,7 +666,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     half8_t qb[FP::KS];
     const float s_init =
         FP::load_q(io, row * io.q_stride_t + (int64_t)(valid ? head : hkv * io.group) * io.q_stride_h, valid, lane, qb);
-    const float sc_mul = lane < 32 ? io.scale_log2 : kPScale;
+    const float sc_mul = lane < 32 ? io.scale_log2 * DTile::kKScaleMul : kPScale;
 
     drop(A, raws);  // t_first is even: raw window 0
     issue(nb, t_first + 2, A);
@@ -713,7 +715,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   l += __shfl_xor(l, 32, kWave);
   if (!valid) return;
   const int g = lane >> 5;
-  const float mul = l > 0.f ? 1.0f / (l * kPScale) : 0.f;
+  const float mul = l > 0.f ? 1.0f / (l * DTile::kOutDiv) : 0.f;
   const int64_t base = row * io.out_stride_t + (int64_t)head * io.out_stride_h + 4 * g;
 #pragma unroll
   for (int mt = 0; mt < FP::MT; ++mt) {
@@ -744,15 +746,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     io.lse[row * io.num_q_heads + head] = l > 0.f ? (m + __builtin_amdgcn_logf(l)) * kLn2 : -INFINITY;
 }
 
-template <int D, int QDT, int ODT, bool EXT>
+template <int D, int QDT, int ODT, bool EXT, int CODE = KVQ_CODE_INT8>
 static int launch_prefill_flash32(PrefillArgs& a, int max_query_len, hipStream_t s) {
-  using FP = Flash32<D, QDT, ODT>;
+  using FP = Flash32<D, QDT, ODT, CODE>;
   a.q_tokens = FP::COLS / a.io.group;
   const int blocks = (max_query_len + a.q_tokens - 1) / a.q_tokens;
   if (a.num_seqs > 65535 || a.io.g.num_kv_heads > 65535) return fail(KVQ_EINVAL, "paged_attn_int8: prefill grid out of range");
   static_assert(FP::LDS_BYTES <= 64 * 1024, "static LDS opt-in would be needed");
   dim3 grid(blocks, a.num_seqs, a.io.g.num_kv_heads);
-  hipLaunchKernelGGL((paged_prefill_flash32_kernel<D, QDT, ODT, EXT>), grid, dim3(256), FP::LDS_BYTES, s, a);
+  hipLaunchKernelGGL((paged_prefill_flash32_kernel<D, QDT, ODT, EXT, CODE>), grid, dim3(256), FP::LDS_BYTES, s, a);
   return check_hip(hipGetLastError(), "paged_prefill_flash32 launch");
 }
 
@@ -768,16 +770,22 @@ static int launch_prefill_cfg(const PrefillArgs& a, int max_query_len, hipStream
 template <int D, int QDT, int ODT>
 static int launch_prefill_nt(PrefillArgs& a, int max_query_len, hipStream_t s) {
   constexpr int WPW = 4;
-  if (a.io.g.code_type == KVQ_CODE_FP8_E4M3) {  // fp8 codes: the per-wave tile, one column tile per wave
-    a.q_tokens = 16 / a.io.group;
-    return launch_prefill_cfg<D, QDT, ODT, 1, WPW, KVQ_CODE_FP8_E4M3>(a, max_query_len, s);
-  }
-  // long runs: the workgroup-shared fp16 tile (compute-bound shape)
+  const bool fp8 = a.io.g.code_type == KVQ_CODE_FP8_E4M3;
+  // long runs: the workgroup-shared fp16 tile (compute-bound shape), for either kind of code
   if constexpr (D <= 128) {
     if (max_query_len * a.io.group >= 64) {
-      if (a.io.window > 0 || a.io.cap_c != 0.f) return launch_prefill_flash32<D, QDT, ODT, true>(a, max_query_len, s);
+      const bool ext = a.io.window > 0 || a.io.cap_c != 0.f;
+      if (fp8) {
+        if (ext) return launch_prefill_flash32<D, QDT, ODT, true, KVQ_CODE_FP8_E4M3>(a, max_query_len, s);
+        return launch_prefill_flash32<D, QDT, ODT, false, KVQ_CODE_FP8_E4M3>(a, max_query_len, s);
+      }
+      if (ext) return launch_prefill_flash32<D, QDT, ODT, true>(a, max_query_len, s);
       return launch_prefill_flash32<D, QDT, ODT, false>(a, max_query_len, s);
     }
+  }
+  if (fp8) {  // short runs of fp8 codes: the per-wave tile, one column tile per wave
+    a.q_tokens = 16 / a.io.group;
+    return launch_prefill_cfg<D, QDT, ODT, 1, WPW, KVQ_CODE_FP8_E4M3>(a, max_query_len, s);
   }
   // two column tiles per wave where the accumulators fit the register file next to a tile in flight
   if (D <= 128 && a.io.group * 2 <= 32 && max_query_len * a.io.group > 16) {
