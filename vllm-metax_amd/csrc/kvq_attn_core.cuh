@@ -798,6 +798,11 @@ struct StreamKArgs {
   const int32_t* cu_seqlens_q;  // nullptr: row i belongs to sequence i
   float* part_o;                // [(P + B), Hq, D]
   float* part_ml;               // [(P + B), Hq, 2]
+  // [2 P + 2], what the main kernel leaves for the reduce kernel, whose waves would otherwise each rescan all
+  // sequence lengths: [0] = length of the work line; [2 w + 2], [2 w + 3] = the sequence that holds workgroup w's
+  // first unit and that sequence's own first unit (workgroups without a share write nothing).
+  int64_t* wg_info;
+  int64_t* seq_first_unit;      // [B]: the first unit of every decode sequence that has a tile (same purpose)
   int num_seqs;
   int num_wg;  // P
   // Fused write of the step's new tokens (decode rows only; k_new == nullptr: the cache already holds them):

@@ -112,6 +112,9 @@ static int paged_attn_launch(const char* op, void* out, int out_dtype, int64_t o
   const size_t slots = (size_t)num_wg + (size_t)num_seqs;
   a.part_o = static_cast<float*>(workspace);
   a.part_ml = a.part_o + slots * (size_t)num_q_heads * (size_t)g.head_size;
+  // 8-byte aligned: a slot's (D + 2) floats are a multiple of 8 bytes
+  a.wg_info = reinterpret_cast<int64_t*>(a.part_ml + slots * (size_t)num_q_heads * 2);
+  a.seq_first_unit = a.wg_info + 2 * (size_t)num_wg + 2;
 
   if (fresh != nullptr) {
     KVQ_REQUIRE(max_query_len == 1, "%s: the fused write takes decode rows only (max_query_len == 1)", op);

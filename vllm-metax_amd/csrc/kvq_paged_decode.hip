@@ -133,7 +133,8 @@ static int launch_reduce(void* out, int out_dtype, float* lse, const float* exp_
 // Workspace layout of the stream-K partials.
 size_t streamk_workspace_bytes(int max_num_seqs, int num_q_heads, int head_size, int num_wg) {
   const size_t slots = (size_t)num_wg + (size_t)max_num_seqs;
-  return slots * (size_t)num_q_heads * ((size_t)head_size + 2) * sizeof(float);
+  return slots * (size_t)num_q_heads * ((size_t)head_size + 2) * sizeof(float) +
+         (2 * (size_t)num_wg + 2 + (size_t)max_num_seqs) * sizeof(int64_t);   // where every workgroup's share begins on the work line
 }
 
 int decode_streamk_num_wg(int num_kv_heads) { return streamk_num_wg(num_kv_heads); }

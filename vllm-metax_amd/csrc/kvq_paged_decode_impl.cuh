@@ -99,29 +99,6 @@ __device__ __forceinline__ void scan_locate(const StreamKArgs& a, int lane, int6
   }
 }
 
-// Total units and the first unit of sequence `seq`; n_first = the units of the first BATCH chunks,
-// loaded by the caller ahead of its first branch.
-template <int BATCH>
-__device__ __forceinline__ void scan_start(const StreamKArgs& a, int lane, int seq, const int (&n_first)[BATCH],
-                                           int64_t& total, int64_t& start) {
-  const int B = a.num_seqs;
-  total = 0;
-  start = 0;
-  for (int base = 0; base < B; base += kWave * BATCH) {
-    int nn[BATCH];
-#pragma unroll
-    for (int j = 0; j < BATCH; ++j)
-      nn[j] = base == 0 ? n_first[j] : decode_units(a.seq_lens, a.cu_seqlens_q, base + kWave * j + lane, B, a.io.window);
-#pragma unroll
-    for (int j = 0; j < BATCH; ++j) {
-      const int n = nn[j], b0 = base + kWave * j;
-      const int incl = wave_incl_scan(n, lane);
-      if (seq >= b0 && seq < b0 + kWave) start = total + __builtin_amdgcn_readlane(incl - n, seq - b0);
-      total += __builtin_amdgcn_readlane(incl, 63);
-    }
-  }
-}
-
 __device__ __forceinline__ int64_t wg_tile_begin(int w, int64_t total, int num_wg) {
   return ((int64_t)w * total) / num_wg;
 }
@@ -161,7 +138,10 @@ __global__ __launch_bounds__(512) void paged_decode_streamk_kernel(StreamKArgs a
   if (w >= num_wg) return;
   const int64_t lo = wg_tile_begin(w, total, num_wg);
   const int64_t hi = wg_tile_begin(w + 1, total, num_wg);
-  if (lo >= hi) return;
+  if (lo >= hi) {   // an empty work line: workgroup 0 still reports its length
+    if (w == 0 && blockIdx.y == 0 && wave == 0 && lane == 0) a.wg_info[0] = total;
+    return;
+  }
 
   // locate the sequence holding unit `lo`
   int seq = 0;
@@ -169,6 +149,11 @@ __global__ __launch_bounds__(512) void paged_decode_streamk_kernel(StreamKArgs a
   if (one_chunk) scan_locate<1>(a, lane, lo, seq, seq_start);
   else scan_locate<kScanBatch>(a, lane, lo, seq, seq_start);
   seq = __builtin_amdgcn_readfirstlane(seq);
+  // Where the share begins (the reduce kernel's key to the span): noted in the first round of the loop, stored
+  // after the last.  A store ahead of the tile loads would sit before them in the wave's in-order memory
+  // counter, and the first tile would wait for the store's acknowledgement (measured: 0.6 us per launch).
+  int info_seq = -1;
+  int64_t info_start = 0;
 
   int64_t pos = lo;
   while (pos < hi && seq < B) {
@@ -180,6 +165,10 @@ __global__ __launch_bounds__(512) void paged_decode_streamk_kernel(StreamKArgs a
     const int ntiles = units - kSetupUnits;
     const int len = __builtin_amdgcn_readfirstlane(a.seq_lens[seq]);
     const int64_t row = a.cu_seqlens_q ? (int64_t)a.cu_seqlens_q[seq] : (int64_t)seq;
+    if (info_seq < 0) {
+      info_seq = seq;
+      info_start = seq_start;
+    }
     const int first = window_first(len, a.io.window);  // tokens before it are outside the window
     const int t0 = first / kTile;                      // the sequence's tile line starts at this tile
     // units [pos, min(hi, end of the sequence)) of the line; the first kSetupUnits of a sequence
@@ -198,6 +187,8 @@ __global__ __launch_bounds__(512) void paged_decode_streamk_kernel(StreamKArgs a
       }
       typename DTile::State st;
       DTile::template run<CAP, STREAM>(a.io, seq, row, len, first, t_begin, t_end, hkv, lane, lds[wave], st, sub, NSUB);
+      // the run holds the sequence's first tile: its place on the line, for the reduce kernel (behind the run's loads)
+      if (t_begin == t0 && blockIdx.y == 0 && wave == 0 && lane == 0) a.seq_first_unit[seq] = seq_start;
       if constexpr (NSUB > 1) {
         if (sub != 0) DTile::dump_state(st, lane, lds[wave]);
         lds_barrier();
@@ -220,30 +211,216 @@ __global__ __launch_bounds__(512) void paged_decode_streamk_kernel(StreamKArgs a
     seq_start += units;
     ++seq;
   }
+  if (blockIdx.y == 0 && wave == 0 && lane == 0) {   // this lane leaves the reduce kernel its notes
+    if (w == 0) a.wg_info[0] = total;
+    if (info_seq >= 0) {
+      a.wg_info[2 * w + 2] = info_seq;
+      a.wg_info[2 * w + 3] = info_start;
+    }
+  }
 }
 
-// Merge the partial states of every decode sequence that more than one workgroup touched.
-// grid (num_seqs, ceil(Hq / 4)), 4 waves, one wave per q head, lane owns D/64 dims.
+// Merge the partial states of every decode sequence that more than one workgroup touched, and give empty decode
+// sequences their defined output.  grid (P, ceil(Hq / 16)), 4 waves; a wave takes four q heads, 16 lanes each, a
+// lane D/16 dims.
+// A sequence is cut only where a workgroup's share begins inside it, so the grid runs over the P workgroups of
+// the main kernel, not over the sequences: block w looks at the sequence in which share w begins (the main
+// kernel left its number and its place on the work line) and merges it if share w is the
+// FIRST to begin inside it; a sequence cut several times is thus merged once, and one that is not cut costs a
+// block one round trip.  (A grid over the sequences, every wave scanning all sequence lengths for its place on
+// the line, took 44 us at 512 sequences; with one q head per wave the P x Hq waves of this grid, 8192 at 32
+// heads, did not fit the chip at once and took 11-13 us.)
 template <int D>
 __global__ __launch_bounds__(256) void paged_decode_streamk_reduce_kernel(StreamKArgs a) {
+  constexpr int V = D / 16;
+  const int lane = threadIdx.x & 63;
+  const int sub = lane & 15;           // lane within the head's group of 16
+  const int grp = lane & 48;           // first lane of that group
+  const int Hq = a.io.num_q_heads;
+  const int head_raw = (blockIdx.y * 4 + (threadIdx.x >> 6)) * 4 + (lane >> 4);
+  const bool head_ok = head_raw < Hq;
+  const int head = head_ok ? head_raw : Hq - 1;   // lanes past the last head repeat it and store nothing
+  const int w = blockIdx.x;
+  const int B = a.num_seqs;
+  // the loads that depend on nothing but the arguments go out before the first branch
+  const int64_t total = a.wg_info[0];
+  // (the share's sequence is undefined for a workgroup without a share: clamped here, looked at only if w < P)
+  const int seq = min(max((int)a.wg_info[2 * w + 2], 0), B - 1);
+  const int64_t start = a.wg_info[2 * w + 3];
+  auto store_dims = [&](int64_t r, const float (&x)[V]) __attribute__((always_inline)) {
+    if (!head_ok) return;
+    const int64_t at = r * a.io.out_stride_t + (int64_t)head * a.io.out_stride_h + sub * V;
+#pragma unroll
+    for (int i = 0; i < V; ++i) store_act_rt(a.io.out_dtype, a.io.out, at + i, x[i]);
+  };
+  // empty decode sequences (no tile: length 0): zeros, lse = -inf; the blocks share them out
+  for (int s = w; s < B; s += (int)gridDim.x) {
+    const int q0e = a.cu_seqlens_q ? a.cu_seqlens_q[s] : s;
+    const int q1e = a.cu_seqlens_q ? a.cu_seqlens_q[s + 1] : s + 1;
+    if (q1e - q0e == 1 && a.seq_lens[s] <= 0) {
+      float z[V];
+#pragma unroll
+      for (int i = 0; i < V; ++i) z[i] = 0.f;
+      store_dims(q0e, z);
+      if (a.io.lse != nullptr && sub == 0 && head_ok) a.io.lse[(int64_t)q0e * Hq + head] = -INFINITY;
+    }
+  }
+  const int P = active_workgroups(total, a.num_wg);
+  if (w == 0 || w >= P) return;
+  const int len = a.seq_lens[seq];
+  const int64_t row = a.cu_seqlens_q ? a.cu_seqlens_q[seq] : seq;
+  const int ntiles = (len + kTile - 1) / kTile - window_first(len, a.io.window) / kTile;   // a decode sequence with tiles
+  // workgroup holding unit x: the largest w with floor(w*T/P) <= x; the sequence's tiles are units
+  // start + kSetupUnits .. start + kSetupUnits + ntiles - 1
+  const int w_first = (int)(((start + kSetupUnits + 1) * P - 1) / total);
+  const int w_last = (int)(((start + kSetupUnits + ntiles) * P - 1) / total);
+  if (w_first == w_last) return;  // not cut
+  const int span = w_last - w_first + 1;
+  if (span > 16) {
+    // A long span (one sequence over dozens of workgroups): a whole wave per q head, 64 slots per pass, and the
+    // block's 16 heads spread over the first four blocks that begin inside the sequence (there are span - 1).
+    constexpr int V2 = D / 64;
+    const int j = w - (w_first + 1);
+    const int h1 = (blockIdx.y * 4 + j) * 4 + (threadIdx.x >> 6);
+    if (j < 0 || j >= 4 || h1 >= Hq) return;   // j < 0: the share begins with the sequence, not inside it
+    float m = -INFINITY, l = 0.f, acc[V2];
+#pragma unroll
+    for (int i = 0; i < V2; ++i) acc[i] = 0.f;
+    for (int wb = w_first; wb <= w_last; wb += kWave) {
+      const int wj = wb + lane;
+      const bool live = wj <= w_last && wg_tile_begin(wj, total, P) < wg_tile_begin(wj + 1, total, P);
+      // loads are unconditional (clamped to the sequence's last workgroup) and what they return is removed with
+      // a bit mask where the slot holds nothing
+      const int64_t slot = (int64_t)min(wj, w_last) + seq;
+      const uint32_t keep = live ? 0xffffffffu : 0u;
+      const float mj_raw = a.part_ml[(slot * Hq + h1) * 2 + 0];
+      const float lj_raw = a.part_ml[(slot * Hq + h1) * 2 + 1];
+      const float mj = live ? as_f32(as_u32(mj_raw) & keep) : -INFINITY;
+      const float lj = as_f32(as_u32(lj_raw) & keep);
+      const float m_new = fmaxf(m, wave_max(mj));
+      const float ca = __builtin_amdgcn_exp2f(m - m_new);  // first chunk: exp2(-inf) = 0
+      const float ej = live ? __builtin_amdgcn_exp2f(mj - m_new) : 0.f;
+      l = l * ca + wave_sum(lj * ej);
+#pragma unroll
+      for (int i = 0; i < V2; ++i) acc[i] *= ca;
+      m = m_new;
+      // up to sixty-four slots per round trip (128 registers of partial outputs in flight per lane)
+      constexpr int kBatch = V2 <= 2 ? 64 : 128 / V2;
+      const int count = min(kWave, w_last - wb + 1);
+      for (int k0 = 0; k0 < count; k0 += kBatch) {
+        float pv[kBatch][V2];
+#pragma unroll
+        for (int k = 0; k < kBatch; ++k) {
+          const int64_t sk = (int64_t)min(wb + k0 + k, w_last) + seq;
+          const float* po = a.part_o + (sk * Hq + h1) * (int64_t)D + lane * V2;
+#pragma unroll
+          for (int i = 0; i < V2; ++i) pv[k][i] = po[i];
+        }
+#pragma unroll
+        for (int k = 0; k < kBatch; ++k) {
+          const float wk = (k0 + k) < count ? __shfl(ej, (k0 + k) & (kWave - 1), kWave) : 0.f;  // unnormalised sums
+          const uint32_t kk = wk != 0.f ? 0xffffffffu : 0u;
+#pragma unroll
+          for (int i = 0; i < V2; ++i) acc[i] += as_f32(as_u32(pv[k][i]) & kk) * wk;
+        }
+      }
+    }
+    const float inv = 1.0f / l;
+#pragma unroll
+    for (int i = 0; i < V2; ++i)
+      store_act_rt(a.io.out_dtype, a.io.out, row * a.io.out_stride_t + (int64_t)h1 * a.io.out_stride_h + lane * V2 + i, acc[i] * inv);
+    if (a.io.lse != nullptr && lane == 0) a.io.lse[row * Hq + h1] = (m + __builtin_amdgcn_logf(l)) * kLn2;
+    return;
+  }
+  if (w != w_first + 1) return;  // another block's to merge
+
+  auto group_max = [&](float x) __attribute__((always_inline)) {
+#pragma unroll
+    for (int o = 8; o >= 1; o >>= 1) x = fmaxf(x, __shfl_xor(x, o, kWave));
+    return x;
+  };
+  auto group_sum = [&](float x) __attribute__((always_inline)) {
+#pragma unroll
+    for (int o = 8; o >= 1; o >>= 1) x += __shfl_xor(x, o, kWave);
+    return x;
+  };
+  const float* po_head = a.part_o + (int64_t)head * D + sub * V;
+  const float* ml_head = a.part_ml + (int64_t)head * 2;
+  // lane `sub` of a group takes slot wb + sub's (m, l); the group agrees on the maximum and the weights, then
+  // every lane adds up its dims over the slots.  All loads of a pass are unconditional (slots past the last
+  // reread the last one and get weight 0; a select on a loaded value would become a branch around the load) and
+  // leave before the first is used.  N slots per pass.
+  float m = -INFINITY, l = 0.f, acc[V];
+#pragma unroll
+  for (int i = 0; i < V; ++i) acc[i] = 0.f;
+  auto pass = [&](int wb, auto n_tag) __attribute__((always_inline)) {
+    constexpr int N = decltype(n_tag)::value;   // <= 16
+    const int wj = wb + sub;
+    const bool live = sub < N && wj <= w_last && wg_tile_begin(wj, total, P) < wg_tile_begin(wj + 1, total, P);
+    const int64_t slot = (int64_t)min(wj, w_last) + seq;
+    const float mj_raw = ml_head[slot * Hq * 2 + 0];
+    const float lj_raw = ml_head[slot * Hq * 2 + 1];
+    float po[N][V];
+#pragma unroll
+    for (int k = 0; k < N; ++k) {
+      const int64_t sk = (int64_t)min(wb + k, w_last) + seq;
+      const float* p = po_head + sk * Hq * (int64_t)D;
+#pragma unroll
+      for (int i = 0; i < V; i += 4) {
+        const floatx4 x = *reinterpret_cast<const floatx4*>(p + i);
+        po[k][i] = x.x; po[k][i + 1] = x.y; po[k][i + 2] = x.z; po[k][i + 3] = x.w;
+      }
+    }
+    const uint32_t keep = live ? 0xffffffffu : 0u;
+    const float mj = live ? as_f32(as_u32(mj_raw) & keep) : -INFINITY;
+    const float lj = as_f32(as_u32(lj_raw) & keep);
+    const float m_new = fmaxf(m, group_max(mj));
+    const float ca = __builtin_amdgcn_exp2f(m - m_new);  // first pass: exp2(-inf) = 0
+    const float ej = live ? __builtin_amdgcn_exp2f(mj - m_new) : 0.f;
+    l = l * ca + group_sum(lj * ej);
+    m = m_new;
+#pragma unroll
+    for (int i = 0; i < V; ++i) acc[i] *= ca;
+#pragma unroll
+    for (int k = 0; k < N; ++k) {
+      const float wk = __shfl(ej, grp + k, kWave);  // 0 for slots past the last and for empty ones
+      const uint32_t kk = wk != 0.f ? 0xffffffffu : 0u;
+#pragma unroll
+      for (int i = 0; i < V; ++i) acc[i] += as_f32(as_u32(po[k][i]) & kk) * wk;
+    }
+  };
+  constexpr int kLong = V <= 8 ? 16 : 8;   // 128 registers of partial outputs in flight per lane
+  if (span <= 4) {
+    pass(w_first, std::integral_constant<int, 4>{});
+  } else if (span <= 8) {
+    pass(w_first, std::integral_constant<int, 8>{});
+  } else {
+    for (int wb = w_first; wb <= w_last; wb += kLong) pass(wb, std::integral_constant<int, kLong>{});
+  }
+  const float inv = 1.0f / l;
+#pragma unroll
+  for (int i = 0; i < V; ++i) acc[i] *= inv;
+  store_dims(row, acc);
+  if (a.io.lse != nullptr && sub == 0 && head_ok)
+    a.io.lse[row * Hq + head] = (m + __builtin_amdgcn_logf(l)) * kLn2;
+}
+
+// The same merge with a grid over the sequences, for batches of few sequences (every one of which is cut, most
+// of them several times): grid (num_seqs, ceil(Hq / 4)), 4 waves, one wave per q head, lane owns D/64 dims.  The
+// sequence's place on the work line comes from the main kernel (seq_first_unit).
+template <int D>
+__global__ __launch_bounds__(256) void paged_decode_streamk_reduce_by_seq_kernel(StreamKArgs a) {
   constexpr int V = D / 64;
   const int lane = threadIdx.x & 63;
   const int head = blockIdx.y * 4 + (threadIdx.x >> 6);
   const int seq = blockIdx.x;
-  const int B = a.num_seqs;
   if (head >= a.io.num_q_heads) return;
   // all the loads that depend on nothing but the arguments go out together, before the first branch
   const int q0 = a.cu_seqlens_q ? a.cu_seqlens_q[seq] : seq;
   const int q1 = a.cu_seqlens_q ? a.cu_seqlens_q[seq + 1] : seq + 1;
   const int len = a.seq_lens[seq];
-  const bool one_chunk = B <= kWave;
-  int n_first[kScanBatch];  // first sequences of the scan
-  n_first[0] = decode_units(a.seq_lens, a.cu_seqlens_q, lane, B, a.io.window);
-  if (!one_chunk) {
-#pragma unroll
-    for (int j = 1; j < kScanBatch; ++j)
-      n_first[j] = decode_units(a.seq_lens, a.cu_seqlens_q, kWave * j + lane, B, a.io.window);
-  }
+  const int64_t total = a.wg_info[0];
+  const int64_t start = a.seq_first_unit[seq];   // defined for every decode sequence that has a tile
   if (q1 - q0 != 1) return;
   const int64_t row = q0;
   const int ntiles = len > 0 ? (len + kTile - 1) / kTile - window_first(len, a.io.window) / kTile : 0;
@@ -252,13 +429,6 @@ __global__ __launch_bounds__(256) void paged_decode_streamk_reduce_kernel(Stream
       store_act_rt(a.io.out_dtype, a.io.out, row * a.io.out_stride_t + (int64_t)head * a.io.out_stride_h + lane * V + i, 0.f);
     if (a.io.lse != nullptr && lane == 0) a.io.lse[row * a.io.num_q_heads + head] = -INFINITY;
     return;
-  }
-  int64_t total, start;
-  if (one_chunk) {
-    const int n1[1] = {n_first[0]};
-    scan_start<1>(a, lane, seq, n1, total, start);
-  } else {
-    scan_start<kScanBatch>(a, lane, seq, n_first, total, start);
   }
   const int P = active_workgroups(total, a.num_wg);
   // workgroup holding unit x: the largest w with floor(w*T/P) <= x; the sequence's tiles are units
@@ -435,8 +605,16 @@ static int launch_streamk(const StreamKArgs& a, hipStream_t s) {
 #undef KVQ_SK
   int rc = check_hip(hipGetLastError(), "paged_attn_int8 decode launch");
   if (rc) return rc;
-  dim3 rgrid(a.num_seqs, (a.io.num_q_heads + 3) / 4);
-  hipLaunchKernelGGL((paged_decode_streamk_reduce_kernel<D>), rgrid, dim3(256), 0, s, a);
+  // a sequence is cut where a share begins inside it: a batch of few sequences has most of them cut several
+  // times (grid over the sequences, a wave per q head), a large batch has at most one cut per share and many
+  // sequences with none (grid over the shares, four q heads per wave)
+  if (2 * a.num_seqs <= a.num_wg) {
+    dim3 rgrid(a.num_seqs, (a.io.num_q_heads + 3) / 4);
+    hipLaunchKernelGGL((paged_decode_streamk_reduce_by_seq_kernel<D>), rgrid, dim3(256), 0, s, a);
+  } else {
+    dim3 rgrid(a.num_wg, (a.io.num_q_heads + 15) / 16);
+    hipLaunchKernelGGL((paged_decode_streamk_reduce_kernel<D>), rgrid, dim3(256), 0, s, a);
+  }
   return check_hip(hipGetLastError(), "paged_attn_int8 reduce launch");
 }
 
