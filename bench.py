@@ -621,7 +621,7 @@ def main():
         "roofline": {"bound": "hbm", "achieved": round(t["attn_bytes"] / t["attn_s"] / 1e9, 1), "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": round(t["attn_bytes"] / t["attn_s"] / 1e9 / HBM_PEAK_GBPS, 4),
                      "traffic": traffic, "traffic_source": traffic_source,
-                     "kernel": "paged decode attention launch = paged_decode_streamk_kernel + paged_decode_streamk_reduce_by_seq_kernel (up to 128 sequences; beyond: paged_decode_streamk_reduce_kernel)",
+                     "kernel": "paged decode attention launch = paged_decode_streamk_kernel + a reduce kernel (paged_decode_streamk_reduce_split4_kernel up to 16 sequences, _reduce_by_seq_kernel up to 96, _reduce_kernel beyond)",
                      "timing": f"{t['n_attn']} attention launches back to back between two events on the launch stream",
                      "algorithmic_bytes_per_launch": t["attn_bytes"]},
     }

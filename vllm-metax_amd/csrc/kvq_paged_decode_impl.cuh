@@ -536,6 +536,119 @@ __global__ __launch_bounds__(256) void paged_decode_streamk_reduce_by_seq_kernel
     a.io.lse[row * a.io.num_q_heads + head] = (m + __builtin_amdgcn_logf(l)) * kLn2;
 }
 
+// The same merge for a handful of sequences, each cut dozens or hundreds of times (long contexts): grid
+// (num_seqs, Hq), the block's four waves share ONE q head's span -- wave p takes the span's slots p, p + 4, ... --
+// and their four states meet in LDS.  (With a wave per head a 256-slot span was a chain of eight round trips:
+// 20.8 us for one 128k-token sequence, next to a 48 us main kernel.)
+template <int D>
+__global__ __launch_bounds__(256) void paged_decode_streamk_reduce_split4_kernel(StreamKArgs a) {
+  constexpr int V = D / 64;
+  __shared__ float sh_acc[3][V][kWave];
+  __shared__ float sh_ml[3][2];
+  const int lane = threadIdx.x & 63;
+  const int part = threadIdx.x >> 6;
+  const int head = blockIdx.y;
+  const int seq = blockIdx.x;
+  const int Hq = a.io.num_q_heads;
+  const int q0 = a.cu_seqlens_q ? a.cu_seqlens_q[seq] : seq;
+  const int q1 = a.cu_seqlens_q ? a.cu_seqlens_q[seq + 1] : seq + 1;
+  const int len = a.seq_lens[seq];
+  const int64_t total = a.wg_info[0];
+  const int64_t start = a.seq_first_unit[seq];   // defined for every decode sequence that has a tile
+  if (q1 - q0 != 1) return;                      // every branch down to the barrier is uniform over the block
+  const int64_t row = q0;
+  const int ntiles = len > 0 ? (len + kTile - 1) / kTile - window_first(len, a.io.window) / kTile : 0;
+  if (ntiles == 0) {  // empty sequence: defined output (zeros, lse = -inf)
+    if (part == 0) {
+      for (int i = 0; i < V; ++i)
+        store_act_rt(a.io.out_dtype, a.io.out, row * a.io.out_stride_t + (int64_t)head * a.io.out_stride_h + lane * V + i, 0.f);
+      if (a.io.lse != nullptr && lane == 0) a.io.lse[row * Hq + head] = -INFINITY;
+    }
+    return;
+  }
+  const int P = active_workgroups(total, a.num_wg);
+  const int w_first = (int)(((start + kSetupUnits + 1) * P - 1) / total);
+  const int w_last = (int)(((start + kSetupUnits + ntiles) * P - 1) / total);
+  if (w_first == w_last) return;  // written directly by the main kernel
+  // this wave's slots: w_first + part + 4 i, i = 0 .. n - 1 (n = 0 for a span shorter than its number)
+  const int span = w_last - w_first + 1;
+  const int n = span > part ? (span - part + 3) / 4 : 0;
+  float m = -INFINITY, l = 0.f, acc[V];
+#pragma unroll
+  for (int i = 0; i < V; ++i) acc[i] = 0.f;
+  // one pass = N of the wave's slots from index i0 on: lane j takes slot j's (m, l), the wave agrees on the
+  // maximum and the weights, every lane adds up its dims.  All loads are unconditional (indices past the last
+  // reread the span's last slot and get weight 0) and leave before the first is used.
+  auto pass = [&](int i0, auto n_tag) __attribute__((always_inline)) {
+    constexpr int N = decltype(n_tag)::value;   // <= 64
+    const int i = i0 + lane;
+    const int wj = w_first + part + 4 * i;
+    const bool live = lane < N && i < n && wg_tile_begin(wj, total, P) < wg_tile_begin(wj + 1, total, P);
+    const int64_t slot = (int64_t)min(wj, w_last) + seq;
+    const float mj_raw = a.part_ml[(slot * Hq + head) * 2 + 0];
+    const float lj_raw = a.part_ml[(slot * Hq + head) * 2 + 1];
+    float po[N][V];
+#pragma unroll
+    for (int k = 0; k < N; ++k) {
+      const int64_t sk = (int64_t)min(w_first + part + 4 * (i0 + k), w_last) + seq;
+      const float* p = a.part_o + (sk * Hq + head) * (int64_t)D + lane * V;
+#pragma unroll
+      for (int x = 0; x < V; ++x) po[k][x] = p[x];
+    }
+    const uint32_t keep = live ? 0xffffffffu : 0u;
+    const float mj = live ? as_f32(as_u32(mj_raw) & keep) : -INFINITY;
+    const float lj = as_f32(as_u32(lj_raw) & keep);
+    const float m_new = fmaxf(m, wave_max(mj));
+    const float ca = m_new == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m - m_new);   // a wave without a slot stays empty
+    const float ej = live ? __builtin_amdgcn_exp2f(mj - m_new) : 0.f;
+    l = l * ca + wave_sum(lj * ej);
+    m = m_new;
+#pragma unroll
+    for (int x = 0; x < V; ++x) acc[x] *= ca;
+#pragma unroll
+    for (int k = 0; k < N; ++k) {
+      const float wk = __shfl(ej, k, kWave);
+      const uint32_t kk = wk != 0.f ? 0xffffffffu : 0u;
+#pragma unroll
+      for (int x = 0; x < V; ++x) acc[x] += as_f32(as_u32(po[k][x]) & kk) * wk;
+    }
+  };
+  constexpr int kLong = V <= 2 ? 64 : 128 / V;   // 128 registers of partial outputs in flight per lane
+  if (n <= 4) {
+    pass(0, std::integral_constant<int, 4>{});
+  } else if (n <= 16) {
+    pass(0, std::integral_constant<int, 16>{});
+  } else {
+    for (int i0 = 0; i0 < n; i0 += kLong) pass(i0, std::integral_constant<int, kLong>{});
+  }
+  if (part > 0) {
+#pragma unroll
+    for (int x = 0; x < V; ++x) sh_acc[part - 1][x][lane] = acc[x];
+    if (lane == 0) {
+      sh_ml[part - 1][0] = m;
+      sh_ml[part - 1][1] = l;
+    }
+  }
+  __syncthreads();
+  if (part > 0) return;
+#pragma unroll
+  for (int p = 0; p < 3; ++p) {
+    const float mp = sh_ml[p][0], lp = sh_ml[p][1];
+    if (mp == -INFINITY) continue;   // that wave had no slot (uniform)
+    const float m_new = fmaxf(m, mp);   // wave 0 always holds the span's first slot: m is finite
+    const float ca = __builtin_amdgcn_exp2f(m - m_new), cb = __builtin_amdgcn_exp2f(mp - m_new);
+    l = l * ca + lp * cb;
+    m = m_new;
+#pragma unroll
+    for (int x = 0; x < V; ++x) acc[x] = acc[x] * ca + sh_acc[p][x][lane] * cb;
+  }
+  const float inv = 1.0f / l;
+#pragma unroll
+  for (int x = 0; x < V; ++x)
+    store_act_rt(a.io.out_dtype, a.io.out, row * a.io.out_stride_t + (int64_t)head * a.io.out_stride_h + lane * V + x, acc[x] * inv);
+  if (a.io.lse != nullptr && lane == 0) a.io.lse[row * Hq + head] = (m + __builtin_amdgcn_logf(l)) * kLn2;
+}
+
 // ---- fixed partitions: grid (max_parts, num_seqs, head groups) --------------------------
 struct V2Args {
   AttnIO io;
@@ -608,7 +721,10 @@ static int launch_streamk(const StreamKArgs& a, hipStream_t s) {
   // a sequence is cut where a share begins inside it: a batch of few sequences has most of them cut several
   // times (grid over the sequences, a wave per q head), a large batch has at most one cut per share and many
   // sequences with none (grid over the shares, four q heads per wave)
-  if (2 * a.num_seqs <= a.num_wg) {
+  if (16 * a.num_seqs <= a.num_wg) {   // a handful of sequences, each cut many times: four waves per q head
+    dim3 rgrid(a.num_seqs, a.io.num_q_heads);
+    hipLaunchKernelGGL((paged_decode_streamk_reduce_split4_kernel<D>), rgrid, dim3(256), 0, s, a);
+  } else if (8 * a.num_seqs <= 3 * a.num_wg) {
     dim3 rgrid(a.num_seqs, (a.io.num_q_heads + 3) / 4);
     hipLaunchKernelGGL((paged_decode_streamk_reduce_by_seq_kernel<D>), rgrid, dim3(256), 0, s, a);
   } else {
