@@ -187,6 +187,34 @@ def test_concat_mla_q(gpu_device, dtype):
         ops.concat_mla_q(a, b.float() if dtype != torch.float32 else b.half(), out)
 
 
+@pytest.mark.parametrize("heads,nseq,dtype", [
+    (128, 260, torch.bfloat16),     # one split per sequence: the decode kernel stores the result itself, no reduce
+    (160, 130, torch.float16),      # two 128-head blocks per sequence, the second partly filled
+    (20, 257, torch.float32),
+    (16, 300, torch.bfloat16),      # the one-head-tile kernel
+    (5, 256, torch.float32),
+])
+def test_mla_decode_one_split_per_sequence(gpu_device, heads, nseq, dtype):
+    g = torch.Generator().manual_seed(heads + nseq)
+    ctx = torch.randint(1, 200, (nseq,), generator=g).tolist()
+    ctx[3] = 0
+    ctx[nseq - 1] = 0                # empty sequences: zeros and lse = -inf, written by the decode kernel too
+    ctx[7] = 33
+    cache, lay, bt, sl = _build(ctx, 16, seed=nseq, dtype=torch.bfloat16)
+    q = torch.randn((nseq, heads, R + P), generator=g).to(dtype)
+    scale = (128 + 64) ** -0.5
+    want, want_lse = oracle.mla_decode(q, cache, lay, bt, sl, scale)
+    got, lse = _run(q, cache, bt, sl, scale)
+    live = sl > 0
+    if dtype == torch.float32:
+        T.assert_close_attn(got[live], want[live], atol=4e-3, rtol=4e-3, what="mla decode, one split, fp32")
+    else:
+        T.assert_close_attn(got[live], want[live], what="mla decode, one split")
+    torch.testing.assert_close(lse.cpu()[live], want_lse[live], atol=5e-3, rtol=1e-3)
+    assert torch.equal(got.float().cpu()[~live], torch.zeros_like(want[~live]))
+    assert torch.isinf(lse.cpu()[~live]).all() and (lse.cpu()[~live] < 0).all()
+
+
 def test_mla_decode_golden(gpu_device):
     G = torch.load(GOLDEN, weights_only=True)
     cache = G["mla_cache"]

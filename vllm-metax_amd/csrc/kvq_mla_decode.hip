@@ -86,7 +86,30 @@ struct MlaArgs {
   int64_t kvc_stride, kpe_stride;  // elements
   int new_dtype;
   float new_eps;
+  // One split per sequence (out != nullptr): the split's state IS the result, and the decode kernels write it
+  // themselves -- out [B, H, 512] in out_dtype, lse_out [B, H] natural log (may be NULL) -- instead of leaving a
+  // state for a reduce kernel that would only convert and copy it.
+  void* out;
+  float* lse_out;
+  int out_dtype;
 };
+
+// Four consecutive output dims of one head in the caller's output type (`elem` = element offset, a multiple of 4).
+__device__ __forceinline__ void mla_store_out4(const MlaArgs& a, int64_t elem, floatx4 v) {
+  if (a.out_dtype == KVQ_F32) {
+    *reinterpret_cast<floatx4*>(reinterpret_cast<float*>(a.out) + elem) = v;
+  } else {
+    u32x2 w;
+    if (a.out_dtype == KVQ_BF16) {
+      w.x = (uint32_t)f32_to_bf16_bits(v.x) | ((uint32_t)f32_to_bf16_bits(v.y) << 16);
+      w.y = (uint32_t)f32_to_bf16_bits(v.z) | ((uint32_t)f32_to_bf16_bits(v.w) << 16);
+    } else {
+      w.x = pack_half2(v.x, v.y);
+      w.y = pack_half2(v.z, v.w);
+    }
+    *reinterpret_cast<u32x2*>(reinterpret_cast<uint16_t*>(a.out) + elem) = w;
+  }
+}
 
 // The fused cache update of the decode kernels: ONE wave loads (mla_new_row_load) and later quantises and stores
 // (mla_new_row_store) the sequence's new latent row at position len - 1, with the write kernel's arithmetic.
@@ -412,6 +435,20 @@ __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
   const bool owner = wave < nht;                  // wave-uniform
   const int64_t pblock0 = ((int64_t)seq * a.num_splits + split) * a.head_groups + blockIdx.z * 8;
   if (tok_begin >= tok_end) {  // empty split (uniform over the workgroup): mark it and leave
+    if (a.out != nullptr) {    // the sequence's only split: an empty sequence, zeros and lse = -inf
+#pragma unroll
+      for (int ht = 0; ht < 8; ++ht) {
+        const int head = (blockIdx.z * 8 + ht) * 16 + c;
+        if (ht < nht && head < a.num_heads) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            mla_store_out4(a, ((int64_t)seq * a.num_heads + head) * kMlaR + 64 * wave + 16 * g + 4 * i, (floatx4){0.f, 0.f, 0.f, 0.f});
+        }
+      }
+      if (owner && g == 0 && hgroup * 16 + c < a.num_heads && a.lse_out != nullptr)
+        a.lse_out[(int64_t)seq * a.num_heads + hgroup * 16 + c] = -INFINITY;
+      return;
+    }
     if (owner && g == 0) a.part_lse[(pblock0 + wave) * 16 + c] = -INFINITY;
     return;
   }
@@ -783,6 +820,22 @@ __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
   float* x_inv = reinterpret_cast<float*>(xchg + buf * kMlaXchgBytes + kMlaPBytes);
   if (owner && g == 0) x_inv[wave * 16 + c] = 1.0f / (l * kPScale);
   lds_barrier();
+  if (a.out != nullptr) {   // one split per sequence: the state is the result
+#pragma unroll
+    for (int ht = 0; ht < 8; ++ht) {
+      const int head = (blockIdx.z * 8 + ht) * 16 + c;
+      if (ht < nht && head < a.num_heads) {
+        const float inv = x_inv[ht * 16 + c];
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          mla_store_out4(a, ((int64_t)seq * a.num_heads + head) * kMlaR + 64 * wave + 16 * g + 4 * i,
+                         (floatx4){o[ht][0][i] * inv, o[ht][1][i] * inv, o[ht][2][i] * inv, o[ht][3][i] * inv});
+      }
+    }
+    if (owner && g == 0 && hgroup * 16 + c < a.num_heads && a.lse_out != nullptr)
+      a.lse_out[(int64_t)seq * a.num_heads + hgroup * 16 + c] = (m + __builtin_amdgcn_logf(l)) * kLn2;
+    return;
+  }
 #pragma unroll
   for (int ht = 0; ht < 8; ++ht) {
     if (ht < nht) {
@@ -838,6 +891,17 @@ __global__ __launch_bounds__(kMlaSmallThreads) void mla_decode_small_kernel(MlaA
   const int tok_end = min(len, tok_begin + slen);
   const int64_t pblock = ((int64_t)seq * a.num_splits + split) * a.head_groups;
   if (tok_begin >= tok_end) {  // empty split (uniform over the workgroup): mark it and leave
+    if (a.out != nullptr) {    // the sequence's only split: an empty sequence, zeros and lse = -inf
+      if (c < a.num_heads) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            mla_store_out4(a, ((int64_t)seq * a.num_heads + c) * kMlaR + 64 * (2 * wave + h) + 16 * g + 4 * i, (floatx4){0.f, 0.f, 0.f, 0.f});
+        if (wave == 0 && g == 0 && a.lse_out != nullptr) a.lse_out[(int64_t)seq * a.num_heads + c] = -INFINITY;
+      }
+      return;
+    }
     if (wave == 0 && g == 0) a.part_lse[pblock * 16 + c] = -INFINITY;
     return;
   }
@@ -1156,6 +1220,19 @@ __global__ __launch_bounds__(kMlaSmallThreads) void mla_decode_small_kernel(MlaA
     }
     sum[b] = acc4;
   }
+  if (a.out != nullptr) {   // one split per sequence: the state is the result
+    if (c < a.num_heads) {
+#pragma unroll
+      for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          mla_store_out4(a, ((int64_t)seq * a.num_heads + c) * kMlaR + 64 * (2 * wave + h) + 16 * g + 4 * i,
+                         (floatx4){sum[4 * h + 0][i], sum[4 * h + 1][i], sum[4 * h + 2][i], sum[4 * h + 3][i]});
+      if (wave == 0 && g == 0 && a.lse_out != nullptr)
+        a.lse_out[(int64_t)seq * a.num_heads + c] = (m_all + __builtin_amdgcn_logf(l_all)) * kLn2;
+    }
+    return;
+  }
 #pragma unroll
   for (int h = 0; h < 2; ++h) {
     uint16_t* po = a.part_o + pblock * (16 * kMlaR) + lane * 4 + (2 * wave + h) * 4 * 256;
@@ -1172,11 +1249,16 @@ __global__ __launch_bounds__(kMlaSmallThreads) void mla_decode_small_kernel(MlaA
 
 // Stage 2: out = sum_j 2^(lse_j - max) o_j / sum_j 2^(lse_j - max); lse = ln 2 * (max + log2 sum).
 // grid (B, ceil(H/16)), 8 waves; wave w combines the d4 = w slice of the block's 16 heads, lane (c, g)
-// as in the split state layout.
-template <int ODT>
+// as in the split state layout.  RPT = 4: a thread takes its four 4-dim pieces of every split, eight splits per
+// trip to memory.  RPT = 1 (grid.z = 4): one piece per thread and 32 splits per trip, for a few sequences cut
+// into dozens of splits -- their grid is a handful of blocks, and eight splits per trip made 64 splits a chain
+// of eight round trips (20 us for one 32k-token sequence, half as long as its decode kernel).
+template <int ODT, int RPT>
 __global__ __launch_bounds__(512) void mla_reduce_kernel(void* out, float* lse, const uint16_t* part_o,
                                                          const float* part_lse, const int32_t* seq_lens,
                                                          int num_heads, int head_groups, int num_splits) {
+  constexpr int SPT = RPT == 4 ? 8 : 32;           // splits per trip
+  const int r0 = RPT == 4 ? 0 : (int)blockIdx.z;   // the thread's first piece
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int c = lane & 15, g = lane >> 4;
   const int seq = blockIdx.x, hgroup = blockIdx.y;
@@ -1184,11 +1266,11 @@ __global__ __launch_bounds__(512) void mla_reduce_kernel(void* out, float* lse, 
   const bool head_ok = head < num_heads;
   const int64_t lstride = (int64_t)head_groups * 16;                    // part_lse stride between splits
   const float* pl = part_lse + ((int64_t)seq * num_splits * head_groups + hgroup) * 16 + c;
-  const uint16_t* po = part_o + ((int64_t)seq * num_splits * head_groups + hgroup) * (16 * kMlaR) + (wave * 4 * 64 + lane) * 4;
+  const uint16_t* po = part_o + ((int64_t)seq * num_splits * head_groups + hgroup) * (16 * kMlaR) + (wave * 4 * 64 + lane) * 4 + r0 * 256;
   const int64_t ostride = (int64_t)head_groups * 16 * kMlaR;            // part_o stride between splits
-  floatx4 acc[4];
+  floatx4 acc[RPT];
 #pragma unroll
-  for (int r = 0; r < 4; ++r) acc[r] = (floatx4){0.f, 0.f, 0.f, 0.f};
+  for (int r = 0; r < RPT; ++r) acc[r] = (floatx4){0.f, 0.f, 0.f, 0.f};
   float mx = -INFINITY;
   const bool live = seq_lens[seq] > 0;
   float den = 0.f;
@@ -1198,35 +1280,35 @@ __global__ __launch_bounds__(512) void mla_reduce_kernel(void* out, float* lse, 
   // Every load is unconditional and a split that holds nothing (lse = -inf; its state rows were never
   // written) is removed with a bit mask on the loaded words: a select on the value would be turned into
   // a branch around the load, and the loads of successive splits would run one by one.
-  for (int j0 = 0; j0 < num_splits; j0 += 8) {
-    float lj[8];
-    u32x2 hv[8][4];
+  for (int j0 = 0; j0 < num_splits; j0 += SPT) {
+    float lj[SPT];
+    u32x2 hv[SPT][RPT];
 #pragma unroll
-    for (int u = 0; u < 8; ++u) {
+    for (int u = 0; u < SPT; ++u) {
       const int j = min(j0 + u, num_splits - 1);   // a slot past the last split rereads the last one and weighs 0
       lj[u] = pl[j * lstride];
       const uint16_t* pj = po + j * ostride;
 #pragma unroll
-      for (int r = 0; r < 4; ++r) hv[u][r] = *reinterpret_cast<const u32x2*>(pj + r * 256);
+      for (int r = 0; r < RPT; ++r) hv[u][r] = *reinterpret_cast<const u32x2*>(pj + r * 256);
     }
     float cm = -INFINITY;
 #pragma unroll
-    for (int u = 0; u < 8; ++u) cm = fmaxf(cm, (live && j0 + u < num_splits) ? lj[u] : -INFINITY);
+    for (int u = 0; u < SPT; ++u) cm = fmaxf(cm, (live && j0 + u < num_splits) ? lj[u] : -INFINITY);
     const float m_new = fmaxf(mx, cm);
     const float mref = m_new == -INFINITY ? 0.f : m_new;
     const float alpha = mx == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mx - mref);
     mx = m_new;
     den *= alpha;
 #pragma unroll
-    for (int r = 0; r < 4; ++r) acc[r] *= alpha;
+    for (int r = 0; r < RPT; ++r) acc[r] *= alpha;
 #pragma unroll
-    for (int u = 0; u < 8; ++u) {
+    for (int u = 0; u < SPT; ++u) {
       const bool on = live && j0 + u < num_splits && lj[u] != -INFINITY;
       const float wj = on ? __builtin_amdgcn_exp2f(lj[u] - mref) : 0.f;
       const uint32_t keep = wj != 0.f ? 0xffffffffu : 0u;
       den += wj;
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
+      for (int r = 0; r < RPT; ++r) {
         const uint32_t h0 = hv[u][r].x & keep, h1 = hv[u][r].y & keep;
         const half2_t a0 = __builtin_bit_cast(half2_t, h0), a1 = __builtin_bit_cast(half2_t, h1);
         acc[r].x += (float)a0.x * wj;
@@ -1240,8 +1322,8 @@ __global__ __launch_bounds__(512) void mla_reduce_kernel(void* out, float* lse, 
   const float inv = den > 0.f ? 1.0f / den : 0.f;                       // nothing attended: zeros
   const int64_t obase = ((int64_t)seq * num_heads + head) * kMlaR + 16 * g;
 #pragma unroll
-  for (int r = 0; r < 4; ++r) {
-    const int64_t o = obase + 64 * wave + 4 * r;   // four consecutive dims: one store (rows are 1024 elements apart)
+  for (int r = 0; r < RPT; ++r) {
+    const int64_t o = obase + 64 * wave + 4 * (r0 + r);   // four consecutive dims: one store (rows are 1024 elements apart)
     const floatx4 v = acc[r] * inv;
     if constexpr (ODT == KVQ_F32) {
       *reinterpret_cast<floatx4*>(reinterpret_cast<float*>(out) + o) = v;
@@ -1257,7 +1339,7 @@ __global__ __launch_bounds__(512) void mla_reduce_kernel(void* out, float* lse, 
       *reinterpret_cast<u32x2*>(reinterpret_cast<uint16_t*>(out) + o) = w;
     }
   }
-  if (lse != nullptr && wave == 0 && g == 0)
+  if (lse != nullptr && wave == 0 && g == 0 && r0 == 0)
     lse[(int64_t)seq * num_heads + head] = den > 0.f ? (mx + __builtin_amdgcn_logf(den)) * kLn2 : -INFINITY;
 }
 
@@ -1387,6 +1469,12 @@ static int mla_decode_run(const char* op, void* out, int out_dtype, float* lse, 
   a.num_splits = splits;
   a.scale_log2 = scale * kLog2e;
   a.bs_magic = (uint32_t)((0x100000000ull + (uint64_t)g.block_size - 1) / (uint64_t)g.block_size);
+  if (splits == 1) {   // nothing to merge: the decode kernel converts and stores its one state as the result
+    KVQ_REQUIRE(out_dtype == KVQ_F32 || out_dtype == KVQ_BF16 || out_dtype == KVQ_F16, "%s: unknown out_dtype %d", op, out_dtype);
+    a.out = out;
+    a.lse_out = lse;
+    a.out_dtype = out_dtype;
+  }
   if (fresh != nullptr) {
     a.kvc_new = fresh->kv_c;
     a.kpe_new = fresh->k_pe;
@@ -1443,10 +1531,19 @@ static int mla_decode_run(const char* op, void* out, int out_dtype, float* lse, 
   }
   int rc = check_hip(hipGetLastError(), "mla_decode_int8 launch");
   if (rc) return rc;
-  dim3 rgrid(num_seqs, head_groups);
-#define KVQ_MLAR(T)                                                                                           \
-  hipLaunchKernelGGL((mla_reduce_kernel<T>), rgrid, dim3(512), 0, s, out, lse, a.part_o, a.part_lse, seq_lens, \
-                     num_heads, head_groups, splits)
+  if (splits == 1) return KVQ_OK;   // the decode kernel wrote the result itself
+  // a few blocks and dozens of splits: a piece per thread, 32 splits per trip, four times the blocks
+  const bool fine = splits > 8 && 4 * num_seqs * head_groups <= num_cus();
+  dim3 rgrid(num_seqs, head_groups, fine ? 4 : 1);
+#define KVQ_MLAR(T)                                                                                                \
+  do {                                                                                                             \
+    if (fine)                                                                                                      \
+      hipLaunchKernelGGL((mla_reduce_kernel<T, 1>), rgrid, dim3(512), 0, s, out, lse, a.part_o, a.part_lse,        \
+                         seq_lens, num_heads, head_groups, splits);                                                \
+    else                                                                                                           \
+      hipLaunchKernelGGL((mla_reduce_kernel<T, 4>), rgrid, dim3(512), 0, s, out, lse, a.part_o, a.part_lse,        \
+                         seq_lens, num_heads, head_groups, splits);                                                \
+  } while (0)
   switch (out_dtype) {
     case KVQ_F32: KVQ_MLAR(KVQ_F32); break;
     case KVQ_BF16: KVQ_MLAR(KVQ_BF16); break;
