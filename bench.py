@@ -469,7 +469,7 @@ def mixed_main(args, cfg, dev, ops):
         "prewarm_s": PREWARM_S, "attn_launch_us": round(attn_s * 1e6, 1),
         "roofline": {"bound": "mfma", "achieved": round(flops / attn_s / 1e12, 1), "peak": MFMA_F16_PEAK_TFLOPS,
                      "unit": "TFLOP/s", "frac": round(flops / attn_s / 1e12 / MFMA_F16_PEAK_TFLOPS, 4), "traffic": None,
-                     "kernel": "varlen attention launch = decode stream-K + reduce + paged_prefill_kernel",
+                     "kernel": "varlen attention launch = paged_decode_streamk_kernel + reduce + prefill_plan_kernel + paged_prefill_flash32_kernel",
                      "algorithmic_flops_per_launch": flops, "algorithmic_bytes_per_launch": dec_bytes + pre_bytes},
     }
     print(json.dumps(res))

@@ -81,11 +81,25 @@ __global__ __launch_bounds__(256) void varlen_attn_kernel(VarlenArgs a) {
   __shared__ __align__(16) uint8_t lds[2][K_BYTES + V_BYTES];
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
-  const int seq = blockIdx.z, head = blockIdx.y;
+  // Workgroups go to the eight XCDs in turn by their linear number, and every XCD has its own L2.  The query
+  // blocks of one (sequence, head) all stream the same keys: numbered so that they land on ONE XCD (possible when
+  // the (sequence, head) pairs divide by eight), its L2 serves all but the first reader of a tile.
+  int seq = blockIdx.z, head = blockIdx.y, qb = blockIdx.x;
+  {
+    const unsigned pairs = gridDim.y * gridDim.z;
+    if ((pairs & 7u) == 0) {
+      const unsigned lin = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
+      const unsigned j = lin >> 3;                             // the XCD's j-th workgroup
+      const unsigned pair = (j / gridDim.x) * 8 + (lin & 7u);  // every eighth pair is this XCD's
+      qb = (int)(j % gridDim.x);
+      head = (int)(pair % gridDim.y);
+      seq = (int)(pair / gridDim.y);
+    }
+  }
   const int q_begin = a.cu_q[seq], q_len = a.cu_q[seq + 1] - q_begin;
   const int k_begin = a.cu_k[seq], k_len = a.cu_k[seq + 1] - k_begin;
   // the last query blocks see the most keys under the causal mask: they are launched first
-  const int q0wg = ((int)gridDim.x - 1 - (int)blockIdx.x) * (64 * RB);
+  const int q0wg = ((int)gridDim.x - 1 - qb) * (64 * RB);
   if (q0wg >= q_len) return;   // uniform over the workgroup
   const int c = lane & 15, g = lane >> 4;
   // key j is visible to query row i iff j <= i + (k_len - q_len)

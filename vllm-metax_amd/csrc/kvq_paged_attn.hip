@@ -16,7 +16,7 @@ int decode_streamk_num_wg(int num_kv_heads);
 int validate_common(const char* op, const void* q, const void* cache, const kvq_cache_geom* geom,
                     const int32_t* block_table, const int32_t* seq_lens, int num_seqs, int num_q_heads);
 int launch_prefill(const AttnIO& io, const int32_t* seq_lens, const int32_t* cu_seqlens_q, int num_seqs,
-                   int max_query_len, int causal, int q_dtype, int out_dtype, hipStream_t s);
+                   int max_query_len, int causal, int q_dtype, int out_dtype, int32_t* plan, hipStream_t s);
 
 // Scratch of the entry point that allocates nothing: a fixed array in the code object's own device
 // memory.  Every GPU the library runs on holds one copy, at its own address, until the process ends.
@@ -141,7 +141,9 @@ static int paged_attn_launch(const char* op, void* out, int out_dtype, int64_t o
   int rc = launch_decode_streamk(a, q_dtype, out_dtype, s);
   if (rc) return rc;
   if (max_query_len > 1) {
-    rc = launch_prefill(a.io, seq_lens, cu_seqlens_q, num_seqs, max_query_len, causal, q_dtype, out_dtype, s);
+    // the list of the sequences that have a query run sits behind the decode kernels' notes in the workspace
+    int32_t* plan = reinterpret_cast<int32_t*>(a.seq_first_unit + num_seqs);
+    rc = launch_prefill(a.io, seq_lens, cu_seqlens_q, num_seqs, max_query_len, causal, q_dtype, out_dtype, plan, s);
   }
   return rc;
 }

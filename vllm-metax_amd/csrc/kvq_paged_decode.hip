@@ -134,7 +134,8 @@ static int launch_reduce(void* out, int out_dtype, float* lse, const float* exp_
 size_t streamk_workspace_bytes(int max_num_seqs, int num_q_heads, int head_size, int num_wg) {
   const size_t slots = (size_t)num_wg + (size_t)max_num_seqs;
   return slots * (size_t)num_q_heads * ((size_t)head_size + 2) * sizeof(float) +
-         (2 * (size_t)num_wg + 2 + (size_t)max_num_seqs) * sizeof(int64_t);   // where every workgroup's share begins on the work line
+         (2 * (size_t)num_wg + 2 + (size_t)max_num_seqs) * sizeof(int64_t) +   // where the shares and the sequences begin
+         ((size_t)max_num_seqs + 2) / 2 * 2 * sizeof(int32_t);                  // the prefill kernels' list of sequences   // where every workgroup's share begins on the work line
 }
 
 int decode_streamk_num_wg(int num_kv_heads) { return streamk_num_wg(num_kv_heads); }
