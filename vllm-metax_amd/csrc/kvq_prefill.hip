@@ -244,7 +244,7 @@ struct PrefillTile {
 };
 
 // grid (query blocks of the longest run, sequences, ceil(Hkv / WPW)); wave w of a workgroup owns
-// kv head blockIdx.z * WPW + w.  Sequences with a one-token run belong to the decode kernel.
+// kv head (head group) * WPW + w.  Sequences with a one-token run belong to the decode kernel.
 template <int D, int QDT, int ODT, int NT, int WPW, int CODE = KVQ_CODE_INT8>
 __global__ __launch_bounds__(WPW * 64) void paged_prefill_kernel(PrefillArgs a) {
   using PT = PrefillTile<D, QDT, ODT, NT, CODE>;
@@ -252,14 +252,21 @@ __global__ __launch_bounds__(WPW * 64) void paged_prefill_kernel(PrefillArgs a) 
   __shared__ __align__(16) uint8_t lds_all[WPW][DTile::LDS_WAVE];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int seq = blockIdx.y;
-  const int hkv = blockIdx.z * WPW + wave;
+  // which sequence, head group and query block: the linear workgroup number read over the plan's sequences,
+  // sequence by sequence (longest first), inside a sequence query-block-major over the head groups, longest
+  // block first, the head group shifted by the block number (see paged_prefill_flash32_kernel)
+  const unsigned nqb = gridDim.x, hz = gridDim.z, per_seq = nqb * hz;
+  const unsigned lin = blockIdx.x + nqb * (blockIdx.y + gridDim.y * blockIdx.z);
+  if (lin >= per_seq * (unsigned)a.plan[0]) return;   // uniform over the workgroup
+  const unsigned rem = lin % per_seq, qbi = rem / hz;
+  const int seq = a.plan[1 + lin / per_seq];
+  const int hkv = (int)((rem % hz + qbi) % hz) * WPW + wave;
   const AttnIO& io = a.io;
   if (hkv >= io.g.num_kv_heads) return;
   const int q_begin = a.cu_seqlens_q[seq];
   const int q_len = a.cu_seqlens_q[seq + 1] - q_begin;
   const int len = a.seq_lens[seq];
-  const int q0 = blockIdx.x * a.q_tokens;           // first query token of this block within the run
+  const int q0 = (int)(nqb - 1 - qbi) * a.q_tokens;   // first query token of this block within the run
   if (q_len <= 1 || q0 >= q_len || len <= 0) return;
   uint8_t* lds = lds_all[wave];
 
