@@ -131,6 +131,33 @@ def test_hundreds_of_short_sequences(gpu_device, hkv, layout):
     torch.testing.assert_close(lse.cpu(), want_lse, atol=5e-3, rtol=1e-3)
 
 
+@pytest.mark.parametrize("where", [0, 77, 139])
+@pytest.mark.parametrize("hq,hkv", [(32, 8), (8, 2)])
+def test_one_long_sequence_among_many_short(gpu_device, hq, hkv, where):
+    """140 sequences of a few dozen tokens and one of 30000: the batch is large enough for the
+    reduce that runs one block per share of the work line, and the long sequence alone covers
+    far more than sixteen shares, so its partial results are merged by the long-span path of that
+    kernel, whether it comes first, in the middle or last."""
+    g = torch.Generator().manual_seed(hq + where)
+    ctx = torch.randint(1, 97, (140,), generator=g).tolist()
+    ctx[where] = 30000
+    qls = [1] * 140
+    from test_gpu_prefill import build
+    kv, lay, bt, q, sl, cu = build(ctx, qls, hq, hkv, 128, 16, seed=where + 1)
+    scale = 1 / math.sqrt(128)
+    want, want_lse = oracle.paged_attn(q, T.storage_bytes(kv), lay, bt, sl, cu, scale, return_lse=True)
+    kvd = T.to_device_cache(kv, gpu_device, "NHD")
+    k, v = L.key_value_views(kvd)
+    ks, vs = L.scale_views(kvd)
+    out = torch.full(q.shape, float("nan"), dtype=torch.float32, device=gpu_device)
+    lse = torch.full(q.shape[:2], float("nan"), dtype=torch.float32, device=gpu_device)
+    ops.unified_attention(q.to(gpu_device), k, v, out, cu.to(gpu_device), 1, sl.to(gpu_device), max(ctx), scale,
+                          True, block_table=bt.to(gpu_device), k_scale_cache=ks, v_scale_cache=vs, lse=lse)
+    torch.cuda.synchronize()
+    T.assert_close_attn(out, want, atol=2e-3, rtol=2e-3, what=f"long sequence at {where}")
+    torch.testing.assert_close(lse.cpu(), want_lse, atol=5e-3, rtol=1e-3)
+
+
 @pytest.mark.parametrize("hq,hkv,d,bs", [(28, 4, 128, 16), (8, 8, 128, 16), (16, 1, 128, 32), (8, 2, 64, 16),
                                          (4, 2, 256, 16), (32, 16, 128, 64),
                                          # head counts of the reference's paged-attention grid
