@@ -406,7 +406,7 @@ def mixed_main(args, cfg, dev, ops):
         new_slots.append(bt[i, pos // bs].long() * bs + pos % bs)
     new_slots = torch.cat(new_slots).to(dev)
     for _ in range(args.layers):
-        kv = L.allocate_kv_cache(pool, bs, hkv, d, device=dev, layout="NHD", fill=0)
+        kv = L.allocate_kv_cache(pool, bs, hkv, d, device=dev, layout=args.kv_layout, fill=0)
         k, v = L.key_value_views(kv)
         ks, vs = L.scale_views(kv)
         ks.fill_(1.0)
@@ -465,7 +465,8 @@ def mixed_main(args, cfg, dev, ops):
                    **({"sliding_window": args.sliding_window} if args.sliding_window else {}),
                    **({"soft_cap": args.soft_cap} if args.soft_cap else {}),
                    "batch": B, "new_tokens": n_tok, "sum_ctx": sum(ctx), "q_heads": hq,
-                   "kv_heads": hkv, "head_dim": d, "block_size": bs, "layer_caches_rotated": Lr},
+                   "kv_heads": hkv, "head_dim": d, "block_size": bs, "layer_caches_rotated": Lr,
+                   "kv_layout": args.kv_layout},
         "prewarm_s": PREWARM_S, "attn_launch_us": round(attn_s * 1e6, 1),
         "roofline": {"bound": "mfma", "achieved": round(flops / attn_s / 1e12, 1), "peak": MFMA_F16_PEAK_TFLOPS,
                      "unit": "TFLOP/s", "frac": round(flops / attn_s / 1e12 / MFMA_F16_PEAK_TFLOPS, 4), "traffic": None,
