@@ -171,8 +171,13 @@ KVQ_API int kvq_paged_attn_int8(void* out, int out_dtype, int64_t out_stride_t, 
  * position seq_lens[i] - 1 of sequence i; its slot comes from the block table.  The
  * workgroup that streams a sequence's last tile quantises the row (the write kernel's
  * arithmetic) and stores the record before it loads the tile.  Decode rows only: every
- * sequence has exactly one query row (row i); sequences of length 0 are skipped.  eps as in
- * kvq_reshape_and_cache_int8.  Workspace as for kvq_paged_attn_int8.
+ * sequence has exactly one query row (row i); sequences of length 0 are skipped.
+ * slot_mapping (int64 [num_seqs], may be NULL) is the step's slot mapping as the write
+ * kernel takes it: a row whose entry is negative is a padding row and is NOT written
+ * (cache_kernels.cu:322-326), whatever its sequence length says; a row with a
+ * non-negative entry is written at the place the block table gives, which the caller's
+ * metadata makes the same slot.  NULL: every row of a non-empty sequence is written.
+ * eps as in kvq_reshape_and_cache_int8.  Workspace as for kvq_paged_attn_int8.
  */
 KVQ_API int kvq_paged_attn_int8_fused_write(void* out, int out_dtype, int64_t out_stride_t, int64_t out_stride_h,
                         const void* q, int q_dtype, int64_t q_stride_t, int64_t q_stride_h,
@@ -181,6 +186,7 @@ KVQ_API int kvq_paged_attn_int8_fused_write(void* out, int out_dtype, int64_t ou
                         int64_t value_stride_t, int64_t value_stride_h, float eps,
                         void* cache, const kvq_cache_geom* geom,
                         const int32_t* block_table, int64_t bt_stride, const int32_t* seq_lens,
+                        const int64_t* slot_mapping,
                         int num_seqs, int num_q_heads, float scale, int window_size,
                         float softcap, float* lse, void* workspace, size_t workspace_bytes,
                         kvq_stream_t stream);
@@ -192,13 +198,18 @@ KVQ_API int kvq_paged_attn_int8_fused_write(void* out, int out_dtype, int64_t ou
  * kernels as kvq_paged_attn_int8, minus the workspace: the split-K partial states
  * live in a fixed array of KVQ_STATIC_SCRATCH_BYTES that is part of the library's
  * code object (each GPU the library runs on holds one copy until the process
- * ends).  The call allocates and frees nothing.  A batch whose partial states
- * would not fit -- kvq_paged_attn_workspace_bytes(num_seqs, num_q_heads,
- * head_size) = (compute units + num_seqs) * num_q_heads * (head_size + 2) * 4
- * bytes -- is rejected with KVQ_EINVAL and nothing is launched (32 q heads of
- * 128 dims on 256 compute units: up to 1256 sequences).  All calls on one GPU
+ * ends).  The call allocates and frees nothing.  A batch is served if
+ * kvq_paged_attn_workspace_bytes(num_seqs, num_q_heads, head_size) <=
+ * KVQ_STATIC_SCRATCH_BYTES (the partial states plus the kernels' notes: 32 q
+ * heads of 128 dims on 256 compute units: up to 1255 sequences); a larger one
+ * is rejected with KVQ_EINVAL and nothing is launched.  All calls on one GPU
  * share that GPU's array: calls that overlap in time on one GPU (different
  * streams, different threads) race and must be serialised by the caller.
+ * kvq_paged_attn_static_scratch_bytes() returns the array's size and is the
+ * set-up hook: called once per device, with that device current and outside any
+ * stream capture, it resolves the array's device address, so that calls under
+ * capture make no runtime query (the entry point resolves it on its first call
+ * on a device otherwise).
  */
 #define KVQ_STATIC_SCRATCH_BYTES (24u << 20)
 KVQ_API size_t kvq_paged_attn_static_scratch_bytes(void);

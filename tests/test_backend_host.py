@@ -44,12 +44,23 @@ def test_backend_statics_match_the_reference_surface():
     assert B.get_kv_cache_shape(40000, 16, 8, 128, "int8_per_token_head") == (40000, 8, 16, 264)
     with pytest.raises(ValueError):
         B.get_kv_cache_shape(10, 8, 8, 128)
+    # no setting: the order the decode kernel streams (a head's records of a block back to back)
     os.environ.pop("VLLM_KV_CACHE_LAYOUT", None)
-    assert B.get_kv_cache_stride_order() == (0, 2, 1, 3)
-    os.environ["VLLM_KV_CACHE_LAYOUT"] = "HND"
+    assert B.get_kv_cache_stride_order() == (0, 1, 2, 3)
+    assert B.get_kv_cache_stride_order(include_num_layers_dimension=True) == (1, 2, 0, 3, 4)
+    # an explicit setting is honoured either way (vllm_metax/v1/attention/backends/triton_attn.py:350-372)
+    for asked, order, order5 in (("NHD", (0, 2, 1, 3), (1, 0, 3, 2, 4)), ("HND", (0, 1, 2, 3), (1, 2, 0, 3, 4)),
+                                 ("nhd", (0, 2, 1, 3), (1, 0, 3, 2, 4))):
+        os.environ["VLLM_KV_CACHE_LAYOUT"] = asked
+        try:
+            assert B.get_kv_cache_stride_order() == order
+            assert B.get_kv_cache_stride_order(include_num_layers_dimension=True) == order5
+        finally:
+            os.environ.pop("VLLM_KV_CACHE_LAYOUT")
+    os.environ["VLLM_KV_CACHE_LAYOUT"] = "DHN"
     try:
-        assert B.get_kv_cache_stride_order() == (0, 1, 2, 3)
-        assert B.get_kv_cache_stride_order(include_num_layers_dimension=True) == (1, 2, 0, 3, 4)
+        with pytest.raises(ValueError):
+            B.get_kv_cache_stride_order()
     finally:
         os.environ.pop("VLLM_KV_CACHE_LAYOUT")
     assert B.use_cascade_attention() is False
@@ -140,6 +151,39 @@ def test_impl_fills_scale_views_once_per_cache_tensor():
     impl._ensure_scale_caches(b)
     impl._ensure_scale_caches(a)                               # back on A: must not be wiped
     assert bool((L.scale_views(a)[0] == 0.5).all())
+    impl._ensure_scale_caches(a.view(a.shape))                 # another tensor object over the same cache
+    assert bool((L.scale_views(a)[0] == 0.5).all())
+
+
+def test_impl_does_not_pin_replaced_caches_and_refills_a_new_cache_at_a_reused_address():
+    import gc
+    import weakref
+
+    from vllm_metax_amd import layout as L
+
+    impl = Int8AttentionImpl(8, 128, 0.09, 2)
+    a = L.allocate_kv_cache(4, 16, 2, 128, device="cpu")
+    b = L.allocate_kv_cache(4, 16, 2, 128, device="cpu")
+    impl._ensure_scale_caches(a)
+    dead = weakref.ref(a.untyped_storage())
+    addr = a.data_ptr()
+    impl._ensure_scale_caches(b)                               # the impl moves on to another cache ...
+    del a
+    gc.collect()
+    assert dead() is None                                      # ... and the first one is free to go
+    assert len(impl._filled) == 1
+    # allocations of the freed size until one lands on the freed address (the allocator usually hands it
+    # straight back); whichever address it gets, a cache never seen before must come out with scales 1.0
+    for _ in range(16):
+        c = L.allocate_kv_cache(4, 16, 2, 128, device="cpu", fill=None)
+        L.scale_views(c)[0].fill_(7.0)
+        L.scale_views(c)[1].fill_(7.0)
+        same = c.data_ptr() == addr
+        impl._ensure_scale_caches(c)
+        ks, vs = L.scale_views(c)
+        assert bool((ks == 1).all()) and bool((vs == 1).all())
+        if same:
+            break
 
 
 def test_impl_constructor_errors():

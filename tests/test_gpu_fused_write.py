@@ -24,8 +24,12 @@ def _last_slots(bt, ctx, bs):
 
 
 def _both_ways(dev, kv_cpu, layout, bt, q, sl, ctx, key, value, scale, mode=KVQuantMode.INT8_PER_TOKEN_HEAD,
-               window=(-1, -1), softcap=0.0, out_dtype=torch.bfloat16):
+               window=(-1, -1), softcap=0.0, out_dtype=torch.bfloat16, padding=()):
+    """`padding`: rows whose slot mapping entry is -1 (cudagraph padding): neither way may write them."""
     bs = L.key_value_views(T.to_device_cache(kv_cpu, dev, layout))[0].shape[1]
+    slots = _last_slots(bt, ctx, bs)
+    for i in padding:
+        slots[i] = -1
     res = []
     for fused in (False, True):
         kv = T.to_device_cache(kv_cpu, dev, layout)
@@ -37,10 +41,11 @@ def _both_ways(dev, kv_cpu, layout, bt, q, sl, ctx, key, value, scale, mode=KVQu
                       window_size=window, kv_quant_mode=mode)
         if fused:
             ops.decode_attention_with_cache_update(q.to(dev), key.to(dev), value.to(dev), k, v, out, sl.to(dev),
-                                                   int(sl.max()), scale, **common)
+                                                   int(sl.max()), scale, **common,
+                                                   slot_mapping=slots.to(dev) if padding else None)
         else:
             ops.reshape_and_cache_flash_per_token_head_quant(key.to(dev), value.to(dev), k, v, ks, vs,
-                                                             _last_slots(bt, ctx, bs).to(dev), kv_quant_mode=mode)
+                                                             slots.to(dev), kv_quant_mode=mode)
             cu = torch.arange(len(ctx) + 1, dtype=torch.int32, device=dev)
             ops.unified_attention(q.to(dev), k, v, out, cu, 1, sl.to(dev), int(sl.max()), scale, True, **common)
         torch.cuda.synchronize()
@@ -76,6 +81,23 @@ def test_fused_write_equals_write_then_attention(gpu_device, layout, hq, hkv, d,
     want = oracle.paged_attn(q, ref, lay, bt, sl, cu, scale)
     rows = torch.tensor(live)
     T.assert_close_attn(out_b[rows], want[rows], what="fused write + decode")
+
+
+@pytest.mark.parametrize("hkv", [8, 2])
+def test_fused_write_skips_padding_rows(gpu_device, hkv):
+    """Rows whose slot_mapping entry is negative are padding (cache_kernels.cu:322-326): their sequence length
+    may still be positive, and the cache bytes at their last position must stay what they were."""
+    ctx = [300, 48, 1000, 17, 64]
+    kv, lay, bt, q, sl, cu = build_case(ctx, 16, hkv, 128, 16, "HND", seed=21, poison=False)
+    g = torch.Generator().manual_seed(4)
+    key = torch.randn((len(ctx), hkv, 128), generator=g).to(torch.bfloat16)
+    value = torch.randn((len(ctx), hkv, 128), generator=g).to(torch.bfloat16)
+    before = T.storage_bytes(kv).clone()
+    (cache_a, out_a, _), (cache_b, out_b, _) = _both_ways(gpu_device, kv, "HND", bt, q, sl, ctx, key, value, 0.088,
+                                                          padding=(1, 4))
+    assert torch.equal(cache_a, cache_b), "a padding row was written (or a live one was not)"
+    assert not torch.equal(cache_b, before)
+    assert torch.equal(out_a.view(torch.int16), out_b.view(torch.int16))
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.float32])

@@ -812,6 +812,7 @@ struct StreamKArgs {
   int64_t kn_stride_t, kn_stride_h, vn_stride_t, vn_stride_h;  // elements
   int new_dtype;
   float new_eps;
+  const int64_t* new_slots;  // the step's slot mapping or nullptr: a row with a negative entry is padding, not written
 };
 
 // The decode kernel's fused cache update: the wave that owns kv head `hkv` of the run that holds a sequence's

@@ -56,6 +56,7 @@ struct NewTokens {
   int dtype;
   int64_t key_stride_t, key_stride_h, value_stride_t, value_stride_h;
   float eps;
+  const int64_t* slot_mapping;  // may be nullptr; a negative entry marks a padding row that is not written
 };
 
 // Arguments are checked, the launch is shaped and enqueued here; the entry points differ only
@@ -136,6 +137,7 @@ static int paged_attn_launch(const char* op, void* out, int out_dtype, int64_t o
     a.vn_stride_h = fresh->value_stride_h;
     a.new_dtype = fresh->dtype;
     a.new_eps = fresh->eps;
+    a.new_slots = fresh->slot_mapping;
   }
   hipStream_t s = as_stream(stream);
   int rc = launch_decode_streamk(a, q_dtype, out_dtype, s);
@@ -169,18 +171,26 @@ extern "C" int kvq_paged_attn_int8_fused_write(void* out, int out_dtype, int64_t
                                                int64_t key_stride_t, int64_t key_stride_h, int64_t value_stride_t,
                                                int64_t value_stride_h, float eps, void* cache,
                                                const kvq_cache_geom* geom, const int32_t* block_table,
-                                               int64_t bt_stride, const int32_t* seq_lens, int num_seqs,
+                                               int64_t bt_stride, const int32_t* seq_lens,
+                                               const int64_t* slot_mapping, int num_seqs,
                                                int num_q_heads, float scale, int window_size, float softcap,
                                                float* lse, void* workspace, size_t workspace_bytes,
                                                kvq_stream_t stream) {
-  const kvq::NewTokens fresh{key, value, src_dtype, key_stride_t, key_stride_h, value_stride_t, value_stride_h, eps};
+  const kvq::NewTokens fresh{key, value, src_dtype, key_stride_t, key_stride_h, value_stride_t, value_stride_h, eps,
+                             slot_mapping};
   return kvq::paged_attn_launch("paged_attn_int8_fused_write", out, out_dtype, out_stride_t, out_stride_h, q, q_dtype,
                                 q_stride_t, q_stride_h, cache, geom, block_table, bt_stride, seq_lens, nullptr, num_seqs,
                                 num_q_heads, 1, scale, 1, window_size, softcap, lse, workspace, workspace_bytes,
                                 "workspace", stream, &fresh);
 }
 
-extern "C" size_t kvq_paged_attn_static_scratch_bytes(void) { return KVQ_STATIC_SCRATCH_BYTES; }
+// Also the set-up hook: resolves the array's address on the current device, so that a first call of the
+// entry point below inside a stream capture finds it resolved and makes no runtime query there.
+extern "C" size_t kvq_paged_attn_static_scratch_bytes(void) {
+  kvq::DeviceSymbols sym;
+  (void)kvq::device_symbols("paged_attn_static_scratch_bytes", &sym);  // without a device: the size alone
+  return KVQ_STATIC_SCRATCH_BYTES;
+}
 
 extern "C" int kvq_paged_attn_int8_static_scratch(void* out, int out_dtype, int64_t out_stride_t,
                                                   int64_t out_stride_h, const void* q, int q_dtype,

@@ -180,7 +180,8 @@ __global__ __launch_bounds__(512) void paged_decode_streamk_kernel(StreamKArgs a
     const int t_end = __builtin_amdgcn_readfirstlane(t0 + u_end - kSetupUnits);
     if (t_begin < t_end) {  // else: this share ends inside the setup charge and holds no tile
       if (a.k_new != nullptr && t_end == t0 + ntiles) {   // uniform over the workgroup: the run holds the last tile
-        if (sub == 0) write_new_token<D>(a, seq, row, len, hkv, lane);
+        const bool padding = a.new_slots != nullptr && a.new_slots[row] < 0;   // uniform: a scalar load
+        if (sub == 0 && !padding) write_new_token<D>(a, seq, row, len, hkv, lane);
         // the record is in memory before any wave of the workgroup loads the tile that holds it
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         if constexpr (NSUB > 1) lds_barrier();

@@ -54,7 +54,7 @@ SIGNATURES = {
     "kvq_paged_attn_int8": (_i, [_vp, _i, _i64, _i64, _vp, _i, _i64, _i64, _vp, _geom_p, _vp, _i64, _vp, _vp,
                                  _i, _i, _i, _f, _i, _i, _f, _vp, _vp, _sz, _vp]),
     "kvq_paged_attn_int8_fused_write": (_i, [_vp, _i, _i64, _i64, _vp, _i, _i64, _i64, _vp, _vp, _i, _i64, _i64, _i64, _i64,
-                                             _f, _vp, _geom_p, _vp, _i64, _vp, _i, _i, _f, _i, _f, _vp, _vp, _sz, _vp]),
+                                             _f, _vp, _geom_p, _vp, _i64, _vp, _vp, _i, _i, _f, _i, _f, _vp, _vp, _sz, _vp]),
     "kvq_paged_attn_static_scratch_bytes": (_sz, []),
     "kvq_paged_attn_int8_static_scratch": (_i, [_vp, _i, _i64, _i64, _vp, _i, _i64, _i64, _vp, _geom_p, _vp, _i64, _vp,
                                                 _vp, _i, _i, _i, _f, _i, _i, _f, _vp, _vp]),

@@ -318,6 +318,7 @@ def decode_attention_with_cache_update(
     workspace: torch.Tensor | None = None,
     geometry: CacheGeometry | None = None,
     lse: torch.Tensor | None = None,
+    slot_mapping: torch.Tensor | None = None,
 ) -> None:
     """A decode step in one launch: the cache update of ``reshape_and_cache_flash_per_token_head_quant`` and the
     attention of ``unified_attention`` with one query row per sequence, for a backend whose ``forward`` includes
@@ -325,8 +326,10 @@ def decode_attention_with_cache_update(
 
     ``q``/``out`` ``[B, Hq, D]``; ``key``/``value`` ``[B, Hkv, D]``: row ``i`` is the token at position
     ``seqused_k[i] - 1`` of sequence ``i`` (the block table gives its slot); ``k``/``v`` and the scale views as in
-    ``unified_attention``.  The cache ends up with the same bytes and ``out`` with the same values as the two
-    calls give."""
+    ``unified_attention``.  ``slot_mapping`` (int64 ``[B]``, optional) is the step's slot mapping: a row whose
+    entry is negative is a padding row and is not written, as in the write kernel; the slot of every other row
+    comes from the block table.  The cache ends up with the same bytes and ``out`` with the same values as the
+    two calls give."""
     code_type = code_type_of(kv_quant_mode)
     softcap = float(softcap or 0.0)
     if softcap < 0:
@@ -357,6 +360,11 @@ def decode_attention_with_cache_update(
         raise RuntimeError("block_table needs num_seqs contiguous rows")
     if block_table.shape[1] * geom.block_size < int(max_seqlen_k):
         raise RuntimeError("block_table rows are too short for max_seqlen_k")
+    if slot_mapping is not None:
+        _require_cuda(slot_mapping)
+        if slot_mapping.dtype != torch.int64 or slot_mapping.dim() != 1 or slot_mapping.shape[0] < num_seqs \
+                or not slot_mapping.is_contiguous():
+            raise RuntimeError("slot_mapping must be a contiguous int64 tensor with one entry per sequence")
     if num_seqs == 0:
         return
     num_q_heads = q.shape[1]
@@ -373,7 +381,7 @@ def decode_attention_with_cache_update(
             _ptr(q), _dtype_code(q, "q"), q.stride(0), q.stride(1),
             _ptr(key), _ptr(value), _dtype_code(key, "key"), key.stride(0), key.stride(1), value.stride(0),
             value.stride(1), eps_for_dtype(key.dtype), ctypes.c_void_p(geom.base_ptr), ctypes.byref(g),
-            _ptr(block_table), block_table.stride(0), _ptr(seqused_k), num_seqs, num_q_heads,
+            _ptr(block_table), block_table.stride(0), _ptr(seqused_k), _ptr(slot_mapping), num_seqs, num_q_heads,
             float(softmax_scale), window, softcap, _ptr(lse), _ptr(workspace),
             workspace.numel() * workspace.element_size(), _stream(dev))
     _C.check(rc, "decode_attention_with_cache_update")

@@ -37,21 +37,41 @@ SCALE_BYTES = 4  # one fp32 scale
 QUANT_EPS = 1e-10
 
 
+def _explicit_kv_cache_layout() -> str | None:
+    """The memory order a deployment has ASKED for, or None: the ``VLLM_KV_CACHE_LAYOUT`` environment
+    variable, or upstream's programmatic override where upstream vLLM is importable."""
+    layout = os.environ.get("VLLM_KV_CACHE_LAYOUT")
+    if layout is None:
+        try:  # pragma: no cover - upstream vLLM is not installed in the build container
+            from vllm.v1.attention.backends import utils as upstream
+
+            layout = getattr(upstream, "_KV_CACHE_LAYOUT_OVERRIDE", None)
+        except Exception:  # noqa: BLE001
+            layout = None
+    if layout is None:
+        return None
+    layout = str(layout).upper()
+    if layout not in ("NHD", "HND"):
+        raise ValueError(f"Unknown cache layout: {layout}")
+    return layout
+
+
+# The order this backend allocates its cache in when nobody has asked for one.  On MI355X a kv head's
+# records of a block lying back to back (HND) let the decode kernel stream whole aligned runs past the
+# caches; token-major blocks (NHD) read 10 % slower.
+DEFAULT_KV_CACHE_LAYOUT = "HND"
+
+
 def get_kv_cache_layout() -> str:
-    """Physical order of the cache, "NHD" (default) or "HND".
+    """Physical order of the per-token-head cache, "HND" or "NHD".
 
     The reference asks upstream ``get_kv_cache_layout()``
-    (vllm_metax/v1/attention/backends/triton_attn.py:356); upstream reads the
-    ``VLLM_KV_CACHE_LAYOUT`` environment variable, which is honoured here too."""
-    try:  # pragma: no cover - upstream vLLM is not installed in the build container
-        from vllm.v1.attention.backends.utils import get_kv_cache_layout as upstream
-
-        return upstream()
-    except Exception:  # noqa: BLE001
-        layout = os.environ.get("VLLM_KV_CACHE_LAYOUT", "NHD").upper()
-        if layout not in ("NHD", "HND"):
-            raise ValueError(f"Unknown cache layout: {layout}")
-        return layout
+    (vllm_metax/v1/attention/backends/triton_attn.py:356), which reads the ``VLLM_KV_CACHE_LAYOUT``
+    environment variable; an explicit setting is honoured here the same way.  With no setting the
+    reference's backend gets upstream's default; this backend owns the static that answers
+    (``get_kv_cache_stride_order``, :350-372) and answers ``DEFAULT_KV_CACHE_LAYOUT``, the order its
+    kernels read fastest.  Both orders are served by every kernel."""
+    return _explicit_kv_cache_layout() or DEFAULT_KV_CACHE_LAYOUT
 
 
 def kv_cache_shape(num_blocks: int, block_size: int, num_kv_heads: int, head_size: int,
@@ -270,6 +290,9 @@ def mla_cache_views(cache: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
 
 @dataclass(frozen=True)
 class MlaGeometry:
+    """Byte geometry of the int8 latent cache handed to the C ABI (``kvq_mla_geom``); the codes are int8
+    only, so there is no code type to carry."""
+
     stride_block: int
     stride_row: int
     scale_off: int
@@ -278,19 +301,6 @@ class MlaGeometry:
     block_size: int
     num_blocks: int
     base_ptr: int
-    code_type: int = _C.KVQ_CODE_INT8   # what a code byte is: int8, or an e4m3fn bit pattern
-
-    def with_code_type(self, code_type: int) -> "CacheGeometry":
-        """The same bytes read as another kind of code (the geometry of a cache does not depend on it)."""
-        if code_type == self.code_type:
-            return self
-        got = self.__dict__.get("_other")
-        if got is None:
-            d = {k: v for k, v in self.__dict__.items() if not k.startswith("_")}
-            d["code_type"] = code_type
-            got = CacheGeometry(**d)
-            object.__setattr__(self, "_other", got)
-        return got
 
     def as_struct(self) -> "_C.MlaGeom":
         """The ctypes struct, built once per geometry object (it is read-only for the library)."""

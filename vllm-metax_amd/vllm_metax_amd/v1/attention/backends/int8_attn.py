@@ -10,6 +10,7 @@ from ``vllm_config`` / ``kv_cache_spec`` only the attributes the reference reads
 """
 from __future__ import annotations
 
+import weakref
 from dataclasses import dataclass
 from typing import ClassVar
 
@@ -295,8 +296,9 @@ class Int8AttentionImpl(_ImplBase):
         self._kv_quant_mode = get_kv_quant_mode(kv_cache_dtype)
         self._is_per_token_head_quant = True
         # per-cache views and byte geometry, built when a cache tensor is first seen
-        self._views: dict = {}
+        self._filled: dict = {}          # (storage id, offset, shape, strides) -> weak reference to the storage
         self._views_for = None
+        self._views_storage = None
         self._key_cache = self._value_cache = None
         self._k_scale_cache = self._v_scale_cache = None
         self._geometry = None
@@ -312,22 +314,26 @@ class Int8AttentionImpl(_ImplBase):
         """fp32 strided views over the inline scale bytes, as
         vllm_metax/v1/attention/backends/triton_attn.py:418-479.  The reference builds them -- and
         fills the scales with 1.0 -- once per impl, at first use; an impl here may meet several cache
-        tensors (tests, a re-bound cache), so the views are kept per tensor and the fill happens only
-        the first time a tensor is seen: coming back to a cache never wipes the scales written into it."""
-        key = (kv_cache.data_ptr(), tuple(kv_cache.shape), tuple(kv_cache.stride()))
-        if self._views_for == key:
+        tensors (tests, a re-bound cache).  Views are held for the cache in use only, so a cache that
+        was replaced is not kept alive; which caches have had their scales filled is remembered by
+        the identity of their storage through weak references, so coming back to a cache never wipes
+        the scales written into it, and a new allocation that lands on a freed cache's address is
+        filled like any new cache."""
+        storage = kv_cache.untyped_storage()
+        key = (storage._cdata, kv_cache.storage_offset(), tuple(kv_cache.shape), tuple(kv_cache.stride()))
+        if self._views_for == key and self._views_storage is storage:
             return
-        got = self._views.get(key)
-        if got is None:
-            k_scale, v_scale = scale_views(kv_cache)
+        seen = self._filled.get(key)
+        k_scale, v_scale = scale_views(kv_cache)
+        if seen is None or seen() is not storage:
             k_scale.fill_(1.0)
             v_scale.fill_(1.0)
-            key_cache, value_cache = key_value_views(kv_cache)
-            got = (key_cache, value_cache, k_scale, v_scale,
-                   geometry_from_views(key_cache, value_cache, k_scale, v_scale, code_type_of(self._kv_quant_mode)))
-            self._views[key] = got
-        self._key_cache, self._value_cache, self._k_scale_cache, self._v_scale_cache, self._geometry = got
-        self._views_for = key
+            filled = self._filled
+            self._filled[key] = weakref.ref(storage, lambda _r, key=key: filled.pop(key, None))
+        key_cache, value_cache = key_value_views(kv_cache)
+        self._key_cache, self._value_cache, self._k_scale_cache, self._v_scale_cache = key_cache, value_cache, k_scale, v_scale
+        self._geometry = geometry_from_views(key_cache, value_cache, k_scale, v_scale, code_type_of(self._kv_quant_mode))
+        self._views_for, self._views_storage = key, storage
 
     def _pth_key_value_caches(self, kv_cache: torch.Tensor):
         """(nb, bs, Hkv, D+4) int8 views of the K and V halves (:729-739)."""
@@ -375,7 +381,9 @@ class Int8AttentionImpl(_ImplBase):
 class Int8FusedUpdateAttentionImpl(Int8AttentionImpl):
     """The same layer with the KV cache update inside ``forward``: a decode-only step is ONE launch (the
     attention kernel quantises each sequence's new token into the cache before it streams the tile that holds
-    it); a step with prefill rows falls back to the two calls, in this order, inside ``forward``."""
+    it; the slot comes from the block table and the sequence length, and a row whose ``slot_mapping`` entry is
+    negative -- cudagraph padding -- is not written, as in the write kernel); a step with prefill rows falls
+    back to the two calls, in this order, inside ``forward``."""
 
     def forward(self, layer, query: torch.Tensor, key: torch.Tensor, value: torch.Tensor, kv_cache: torch.Tensor,
                 attn_metadata: Int8AttentionMetadata | None, output: torch.Tensor,
@@ -401,7 +409,8 @@ class Int8FusedUpdateAttentionImpl(Int8AttentionImpl):
             seqused_k=attn_metadata.seq_lens, max_seqlen_k=attn_metadata.max_seq_len, softmax_scale=self.scale,
             block_table=attn_metadata.block_table, k_scale_cache=self._k_scale_cache, v_scale_cache=self._v_scale_cache,
             window_size=self.sliding_window, softcap=self.logits_soft_cap, kv_quant_mode=self._kv_quant_mode,
-            workspace=attn_metadata.workspace, geometry=self._geometry)
+            workspace=attn_metadata.workspace, geometry=self._geometry,
+            slot_mapping=attn_metadata.slot_mapping[:n] if attn_metadata.slot_mapping is not None else None)
         return output
 
 

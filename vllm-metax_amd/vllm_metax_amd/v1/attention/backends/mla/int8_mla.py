@@ -299,7 +299,8 @@ class Int8MLAImpl(_MLAImplBase):
 
     def forward_mqa(self, q, kv_c_and_k_pe_cache: torch.Tensor, attn_metadata, layer=None, new_rows=None):
         """``q`` [B, H, 576] or ``(ql_nope [B, H, 512], q_pe [B, H, 64])``; returns
-        ``(o [B, H, kv_lora_rank], lse [B, H] float32)``.  ``new_rows`` = (kv_c_normed [B, R], k_pe [B, P]):
+        ``(o [B, H, kv_lora_rank], lse [B, H] float32)``, valid until the next decode call on the same
+        metadata (see below).  ``new_rows`` = (kv_c_normed [B, R], k_pe [B, P]):
         the launch also writes the step's rows (see ``forward_mqa_with_cache_update``)."""
         assert kv_c_and_k_pe_cache.numel() > 0
         assert attn_metadata.decode is not None
@@ -308,7 +309,10 @@ class Int8MLAImpl(_MLAImplBase):
         q0 = q[0] if type(q) is tuple else q
         B, H = q0.shape[0], q0.shape[1]
         # the builder's buffers when the metadata carries them (nothing is allocated then: the step can be
-        # captured in a graph); what is returned are views of them, valid until the next decode step
+        # captured in a graph).  What is returned are views of them, and every layer of the KV-cache group
+        # shares them through the same metadata: they are valid until the NEXT forward_mqa / decode_absorbed
+        # call on this metadata -- the next layer's, in the same step.  A caller that keeps (o, lse) across
+        # layers (a deferred merge) must copy them, or pass metadata without decode_out / decode_lse.
         o_buf, lse_buf = getattr(attn_metadata, "decode_out", None), getattr(attn_metadata, "decode_lse", None)
         if o_buf is not None and lse_buf is not None and o_buf.dtype == q0.dtype and o_buf.shape[0] >= B \
                 and o_buf.shape[1] == H and o_buf.shape[2] == self.kv_lora_rank:
@@ -417,7 +421,9 @@ class Int8MLADecodeCaller:
         torch.bmm(x, self.W_UV, out=out.transpose(0, 1))
 
     def decode_absorbed(self, mqa_q_nope: torch.Tensor, mqa_q_pe: torch.Tensor, kv_cache: torch.Tensor, attn_metadata):
-        """Absorption + decode in one launch; returns ``(o [B, N, L], lse [B, N])`` like ``forward_mqa``."""
+        """Absorption + decode in one launch; returns ``(o [B, N, L], lse [B, N])`` like ``forward_mqa``
+        (views of the builder's buffers when the metadata carries them: valid until the next decode call on
+        this metadata, the next layer's included)."""
         impl = self.impl
         B = mqa_q_nope.shape[0]
         o_buf, lse_buf = getattr(attn_metadata, "decode_out", None), getattr(attn_metadata, "decode_lse", None)
