@@ -45,6 +45,8 @@ constexpr int kMlaKSteps8 = kMlaW / 64;                   // 9 int8 k-steps of 6
 constexpr int kMlaQOps = 2 * kMlaKSteps8;                 // B operands of Q: two int8 terms per k-step
 constexpr int kMlaQRegOps = 16;                           // operands of Q kept in registers; the rest in LDS
 constexpr int kMlaQLdsBytes = (kMlaQOps - kMlaQRegOps) * kMlaThreads * 16;  // 16384
+constexpr float kMlaQ2 = 256.0f;                          // ratio of the scales of the query's two int8 terms
+constexpr float kMlaQ1Max = 16383.5f / kMlaQ2;            // largest first term: s1 = max|q| / kMlaQ1Max
 constexpr int kMlaRing = 3;                               // raw tile windows: tile t is read (QK, then PV) while t + 1 and t + 2 stream in
 typedef int32_t i32x4 __attribute__((ext_vector_type(4)));
 // What the head-owning waves hand to the others, per tile and double-buffered: the eight P~ operands
@@ -154,27 +156,26 @@ __device__ __forceinline__ int mla_split_len(int len, int num_splits) {
   return ((per + kTile - 1) / kTile) * kTile;
 }
 
-// 16 values of one head -> the 16 bytes of each of the two int8 terms: a =
-// rint(q / s1), b = rint((q - s1 a) * 254 / s1).  `live` false gives zero bytes (heads past the end).
+// 16 values of one head -> the 16 bytes of each of the two int8 terms, q ~ s1 a + s2 b with s2 = s1 / 256:
+// w = rint(q / s2) is a 15-bit integer (|w| <= 16384 because s1 = max|q| / kMlaQ1Max), and w = 256 a + b with
+// b in [-128, 127] splits it: a is the high byte of w + 128, b its low byte with the top bit flipped.  One
+// normalised 16-bit conversion quantises two values, one packed add and three byte permutes per four values
+// do the rest.  `live` false gives zero bytes (heads past the end).
+typedef uint16_t u16x2_t __attribute__((ext_vector_type(2)));
+typedef short s16x2_t __attribute__((__vector_size__(2 * sizeof(short))));
 __device__ __forceinline__ void mla_two_int8_terms(const float (&f)[16], float s1, bool live, u32x4& ta, u32x4& tb) {
-  const float inv1 = 1.0f / s1, inv2 = 254.0f * inv1;
-  // x + 1.5 * 2^23 rounds x to the nearest integer (ties to even) and leaves it, in two's complement,
-  // in the low mantissa bits: the low byte is the int8 code (|x| <= 127 here by construction)
-  constexpr float kMagic = 12582912.0f;
+  // the conversion multiplies by 32767: q * inv * 32767 = q / s2
+  const float inv = live ? kMlaQ2 / (s1 * 32767.0f) : 0.f;
 #pragma unroll
   for (int w = 0; w < 4; ++w) {
-    uint32_t ba[4], bb[4];
+    uint32_t t[2];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const float q = live ? f[4 * w + j] : 0.f;
-      const float ra = __builtin_fmaf(q, inv1, kMagic);
-      const float r = __builtin_fmaf(-(ra - kMagic), s1, q);
-      const float rb = __builtin_fmaf(r, inv2, kMagic);
-      ba[j] = as_u32(ra);
-      bb[j] = as_u32(rb);
+    for (int j = 0; j < 2; ++j) {
+      const s16x2_t pk = __builtin_amdgcn_cvt_pknorm_i16(f[4 * w + 2 * j] * inv, f[4 * w + 2 * j + 1] * inv);
+      t[j] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(u16x2_t, pk) + (u16x2_t){128, 128});
     }
-    ta[w] = perm(ba[1], ba[0], 0x0c0c0400u) | perm(ba[3], ba[2], 0x04000c0cu);
-    tb[w] = perm(bb[1], bb[0], 0x0c0c0400u) | perm(bb[3], bb[2], 0x04000c0cu);
+    ta[w] = perm(t[1], t[0], 0x07050301u);                  // the four high bytes
+    tb[w] = perm(t[1], t[0], 0x06040200u) ^ 0x80808080u;    // the four low bytes, as signed numbers
   }
 }
 
@@ -247,9 +248,10 @@ __device__ __forceinline__ void mla_seq_split_of_block(int num_seqs, int num_spl
 
 // Q for the int8 MFMA.  The cache codes ARE int8, so the QK product can run on
 // v_mfma_i32_16x16x64_i8 straight from the cached bytes -- no conversion of K at all -- once Q is
-// int8 too: q = s1 * a + s2 * b with a = rint(q / s1), s1 = max|q| / 127 per head, and
-// b = rint((q - s1 a) / s2), s2 = s1 / 254.  The residual after two terms is at most
-// s2 / 2 = max|q| / 64516, finer than the fp16 rounding of q it replaces, and the integer dot
+// int8 too: q = s1 * a + s2 * b with a the nearest multiple of s1 = max|q| / 64 per head (about), and
+// b the rest in units of s2 = s1 / 256, where 256 a + b = rint(q / s2) is a 15-bit integer (|a| <= 64, so that
+// 256 a . k + b . k, the two integer sums joined with one shift-add, stays below 2^31 for any codes).  The
+// residual after two terms is at most s2 / 2 = max|q| / 32767, finer than the fp16 rounding of q it replaces, and the integer dot
 // products are exact.  For a (sequence, 16 heads) block, lane (c = head, g) holds, for k-step kk, dims
 // 64 kk + 16 g + j (j < 16) as 16 bytes, operand 2 kk = term a, operand 2 kk + 1 = term b.  The decode
 // kernels build these operands in their prologues (mla_two_int8_terms); only the absorption kernel below
@@ -381,7 +383,7 @@ __global__ __launch_bounds__(256) void mla_absorb_q_kernel(MlaAbsorbArgs a) {
     if (b >= a.num_seqs) continue;
     float amax = fmaxf(fmaxf(part_max[0][t][c], part_max[1][t][c]), fmaxf(part_max[2][t][c], part_max[3][t][c]));
     amax = head_ok ? fminf(amax, 3.0e38f) : 0.f;   // heads past the end contribute zero columns
-    const float s1 = amax > 0.f ? amax / 127.0f : 1.0f;
+    const float s1 = amax > 0.f ? amax / kMlaQ1Max : 1.0f;
     const int64_t qblock = (int64_t)b * a.head_groups + hgroup;
     u32x4* qdst = reinterpret_cast<u32x4*>(a.q_ops + qblock * (kMlaQOps * kWave * 16)) + hc;
     // the lane's 32 dims are the 16-dim pieces u = 0, 1: k-step kk = 2 w + g / 2, piece 2 (g % 2) + u of it
@@ -586,7 +588,7 @@ __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
         for (int i = 0; i < 16; ++i) amax = fmaxf(amax, fabsf(f[kk][i]));
       amax = max_over_quarters(amax);
       amax = head_ok ? fminf(amax, 3.0e38f) : 0.f;      // heads past the end contribute zero columns
-      s1 = amax > 0.f ? amax / 127.0f : 1.0f;
+      s1 = amax > 0.f ? amax / kMlaQ1Max : 1.0f;
 #pragma unroll
       for (int kk = 0; kk < kMlaKSteps8; ++kk) {
         u32x4 ta, tb;
@@ -600,7 +602,7 @@ __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
         }
       }
     }
-    s2 = s1 / 254.0f;
+    s2 = s1 / kMlaQ2;
   } else {
 #pragma unroll
     for (int op = 0; op < kMlaQRegOps; ++op) qreg[op] = (i32x4){0, 0, 0, 0};
@@ -695,39 +697,45 @@ __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
       //      last tile can hold tokens past its end: every other tile takes the path without masks.
       auto softmax = [&](auto masked_tag) __attribute__((always_inline)) {
         constexpr bool MASKED = decltype(masked_tag)::value;
-        float logit[8];
-        float mloc = -INFINITY;
+        // The two integer sums are joined with one shift-add (256 a.k + b.k, below 2^31 for any codes) and the
+        // exponents formed straight away against the reference maximum as it stands -- which is right whenever
+        // it does not move, and it rarely does: the reference maximum m of a head only has to keep 2^(logit - m)
+        // in range, it need not be the true maximum.  It moves when some head of the tile outgrows it by more
+        // than 2^kLazyMax (or at all, when a token's value scale is so large that p * scale could leave the fp16
+        // range otherwise).  Moving m rescales what is accumulated so far, and the accumulators of these
+        // heads are spread over all waves, so the factors travel with the tile.
+        const bool first = m == -INFINITY;
+        const float mref = first ? 0.f : m;   // while there is no maximum yet: the logits themselves
+        float e[8];
+        float emax = -INFINITY;
 #pragma unroll
         for (int mt = 0; mt < 2; ++mt) {
           const floatx4 ks = *reinterpret_cast<const floatx4*>(sck + 16 * mt + 4 * g);
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
-            float x = __builtin_fmaf((float)acc[1][mt][i], s2, (float)acc[0][mt][i] * s1) * ks[i];
+            float x = __builtin_fmaf((float)((acc[0][mt][i] << 8) + acc[1][mt][i]), s2 * ks[i], -mref);
             if constexpr (MASKED) x = t * kTile + 16 * mt + 4 * g + i < tok_end ? x : -INFINITY;
-            logit[4 * mt + i] = x;
-            mloc = fmaxf(mloc, x);
+            e[4 * mt + i] = x;
+            emax = fmaxf(emax, x);
           }
         }
-        mloc = max_over_quarters(mloc);
-        // The reference maximum m of a head only has to keep 2^(logit - m) in range, it need not be the
-        // true maximum: it moves when some head of the tile outgrows it by more than 2^kLazyMax (or at
-        // all, when a token's value scale is so large that p * scale could leave the fp16 range
-        // otherwise).  Moving m rescales what is accumulated so far, and the accumulators of these
-        // heads are spread over all waves, so the factors travel with the tile; with i.i.d. logits the
-        // true maximum moves in most of a split's first dozen tiles, the lazy one a few times.
+        emax = max_over_quarters(emax);
         floatx4 vs[2];
 #pragma unroll
         for (int mt = 0; mt < 2; ++mt) vs[mt] = *reinterpret_cast<const floatx4*>(sck + kTile + 16 * mt + 4 * g);
         const float vsmax = fmaxf(fmaxf(fmaxf(vs[0].x, vs[0].y), fmaxf(vs[0].z, vs[0].w)),
                                   fmaxf(fmaxf(vs[1].x, vs[1].y), fmaxf(vs[1].z, vs[1].w)));
-        const float lim = vsmax > kLazyScaleMax ? m : m + kLazyMax;
-        const bool moved = __builtin_amdgcn_ballot_w64(mloc > lim) != 0;
-        if (moved) {
-          const float m_new = fmaxf(m, mloc);
+        const float lim = vsmax > kLazyScaleMax ? 0.f : kLazyMax;
+        const bool moved = __builtin_amdgcn_ballot_w64(first || emax > lim) != 0;
+        if (moved) {   // the new reference is the largest logit, emax + mref; the exponents shift by the difference
+          const float m_new = fmaxf(m, emax + mref);
           const float alpha = __builtin_amdgcn_exp2f(m - m_new);
+          const float shift = m_new - mref;
           m = m_new;
           l *= alpha;
           if (g == 0) x_alpha[wave * 16 + c] = alpha;
+#pragma unroll
+          for (int i = 0; i < 8; ++i) e[i] -= shift;   // a masked token's exponent stays -inf
         }
         if (lane == 0) x_flag[wave] = moved ? 1 : 0;
         float pt[8];
@@ -735,7 +743,7 @@ __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
         for (int mt = 0; mt < 2; ++mt) {
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
-            const float p = __builtin_amdgcn_exp2f(logit[4 * mt + i] - m);   // 0 for a masked token
+            const float p = __builtin_amdgcn_exp2f(e[4 * mt + i]);   // 0 for a masked token
             l += p;
             pt[4 * mt + i] = p * vs[mt][i];
             // a slot past the end may hold any bit pattern as its scale: select, do not multiply by 0
@@ -1023,7 +1031,7 @@ __global__ __launch_bounds__(kMlaSmallThreads) void mla_decode_small_kernel(MlaA
     lds_barrier();   // LDS only: the tile's loads stay in flight
     amax = fmaxf(fmaxf(part_max[c], part_max[16 + c]), fmaxf(part_max[32 + c], part_max[48 + c]));
     amax = head_ok ? fminf(amax, 3.0e38f) : 0.f;      // heads past the end contribute zero columns
-    s1 = amax > 0.f ? amax / 127.0f : 1.0f;
+    s1 = amax > 0.f ? amax / kMlaQ1Max : 1.0f;
 #pragma unroll
     for (int n = 0; n < kMine; ++n) {
       const int kk = wave + 4 * n;
@@ -1038,7 +1046,7 @@ __global__ __launch_bounds__(kMlaSmallThreads) void mla_decode_small_kernel(MlaA
 #pragma unroll
     for (int op = 0; op < kMlaQOps; ++op) qreg[op] = __builtin_bit_cast(i32x4, qstage[op * kWave + lane]);
   }
-  const float s2 = s1 / 254.0f;
+  const float s2 = s1 / kMlaQ2;
   if (write_late) mla_new_row_store(a, seq, len, lane, new_row);
 
   floatx4 o[32];   // o[4 d4 + b][i]: head c, dim 64 d4 + 16 g + 4 i + b
