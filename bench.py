@@ -35,6 +35,8 @@ PREWARM_S = 0.5
 # rocprofv3 summaries that carry the measured HBM traffic of a workload's attention launch
 # (a line "traffic_bytes_per_launch: N" and a line "measured_at_commit: HASH")
 TRAFFIC_PROFILE = {"llama3_8b_decode_b64_ctx1k-8k": "paged_decode_streamk_llama3_8b_b64_ctx1k-8k.md",
+                   "longctx_splitk_b8_32k-128k": "paged_decode_streamk_longctx_b8_32k-128k.md",
+                   "qwen2_7b_mixed_4x2048_prefill_60_decode": "paged_prefill_flash_qwen2_7b_mixed_4x2048_prefill_60_decode.md",
                    "mla_decode_b32_h128_ctx4096": "mla_decode_b32_h128_ctx4096.md",
                    "mla_decode_b32_h16_ctx4096": "mla_decode_b32_h16_ctx4096.md"}
 
@@ -80,6 +82,32 @@ def time_back_to_back(fn, n):
     return e0.elapsed_time(e1) / n * 1e-3
 
 
+def time_graph_replay(fn, n, replays=5):
+    """GPU time of one `fn(i)`: n of them captured into one HIP graph, the graph replayed and timed between two
+    events.  Inside a graph the launches follow each other without the host in between, so a kernel far shorter
+    than a host-side call (the decode write) is timed as what the GPU spends on it."""
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for i in range(n):
+            fn(i)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        for i in range(n):
+            fn(i)
+    graph.replay()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(replays):
+        graph.replay()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / (n * replays) * 1e-3
+
+
 def make_batch(workload: str, seed: int = 0):
     """Context lengths and pool size of the named workload (BASELINE.json configs)."""
     g = torch.Generator().manual_seed(seed)
@@ -99,6 +127,8 @@ def make_batch(workload: str, seed: int = 0):
                     qlens=[2048] * 4 + [1] * 60, pool=12000)
     if workload == "mla_decode_b32_h128_ctx4096":        # configs[3]: DeepSeek-V2 MLA decode
         return dict(mla=True, heads=128, r=512, p=64, bs=64, ctx=[4096] * 32, pool=32 * 64 + 8)
+    if workload == "mla_prefill_h128":                   # the MLA layer's prefill attention calls, DeepSeek-V2 shapes
+        return dict(mla_prefill=True, heads=128, nope=128, rope=64, dv=128)
     if workload == "mla_decode_b32_h16_ctx4096":         # the same step on one of eight tensor-parallel shards
         return dict(mla=True, heads=16, r=512, p=64, bs=64, ctx=[4096] * 32, pool=32 * 64 + 8)
     raise SystemExit(f"unknown workload {workload}")
@@ -302,14 +332,16 @@ def mla_main(args, cfg, dev, ops):
     dt = (time.perf_counter() - t0) / args.steps
     n_ev = max(args.steps, 100)
     attn_s = time_back_to_back(lambda i: run_mla_step(st, i % L, ops, cfg, write=False, attn=True), n_ev)
-    for i in range(args.warmup):
-        run_mla_step(st, i % L, ops, cfg, fused=True)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for i in range(args.steps):
-        run_mla_step(st, i % L, ops, cfg, fused=True)
-    torch.cuda.synchronize()
-    fused_s = (time.perf_counter() - t0) / args.steps
+    fused_s = None
+    if not args.no_one_launch:
+        for i in range(args.warmup):
+            run_mla_step(st, i % L, ops, cfg, fused=True)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(args.steps):
+            run_mla_step(st, i % L, ops, cfg, fused=True)
+        torch.cuda.synchronize()
+        fused_s = (time.perf_counter() - t0) / args.steps
     traffic, traffic_source = measured_traffic(args.workload)
     small = cfg["heads"] <= 16   # one head tile: a kernel of its own, which also prepares the query
     # at 16 heads the launch moves few flops per byte: the HBM roof is the one that binds
@@ -332,11 +364,12 @@ def mla_main(args, cfg, dev, ops):
                      "algorithmic_flops_per_launch": flops, "algorithmic_bytes_per_launch": nbytes,
                      "hbm_frac_of_peak": round(nbytes / attn_s / 1e9 / HBM_PEAK_GBPS, 4)},
     }
-    res["one_launch_step"] = {"what": "the same layer step with the latent write inside the decode launch "
-                                      "(kvq_mla_decode_int8_fused_write)",
-                              "us_per_layer": round(fused_s * 1e6, 2), "value": round(nbytes / fused_s / 1e9, 1),
-                              "unit": "GB/s"}
-    res["decode_caller"] = mla_caller_chain(cfg, st, dev, ops, n_ev)
+    if fused_s is not None:
+        res["one_launch_step"] = {"what": "the same layer step with the latent write inside the decode launch "
+                                          "(kvq_mla_decode_int8_fused_write)",
+                                  "us_per_layer": round(fused_s * 1e6, 2), "value": round(nbytes / fused_s / 1e9, 1),
+                                  "unit": "GB/s"}
+        res["decode_caller"] = mla_caller_chain(cfg, st, dev, ops, n_ev)
     if not args.no_cpu_baseline:
         res["cpu_baseline"] = mla_cpu_baseline(cfg, st, args.cpu_seconds)
     print(json.dumps(res))
@@ -375,6 +408,130 @@ def mla_caller_chain(cfg, st, dev, ops, n):
         res[name] = round(time_back_to_back(fn, n) * 1e6, 2)
     res["steps"] = "q_nope [B,H,128] x W_UK_T -> decode -> x W_UV [H,512,128] -> out [B, H*128], bf16"
     return res
+
+
+MLA_PREFILL_SHAPES = (("context chunk: 4 x 2048 queries, 8192 keys each, unmasked", 4, 2048, 8192, False),
+                      ("new tokens: 4 x 2048 causal", 4, 2048, 2048, True),
+                      ("new tokens: 1 x 8192 causal", 1, 8192, 8192, True))
+
+
+def mla_prefill_main(args, cfg, dev, ops):
+    """The attention call of the MLA layer's prefill (kvq_mla_prefill_attn: dense bf16 K / V behind the gather
+    and the up-projection) at DeepSeek-V2 shapes.  A step is one call of the first shape; the other two are
+    timed the same way and reported beside it.  --steps 1 --warmup 0 makes one call per shape (counter runs)."""
+    H, nope, rope, dv = cfg["heads"], cfg["nope"], cfg["rope"], cfg["dv"]
+    rows = []
+    for name, B, ql, kl, causal in MLA_PREFILL_SHAPES:
+        T, S = B * ql, B * kl
+        q = torch.randn(T, H, nope + rope, device=dev, dtype=torch.bfloat16)
+        kv = torch.randn(S, H, nope + dv, device=dev, dtype=torch.bfloat16)
+        kpe = torch.randn(S, rope, device=dev, dtype=torch.bfloat16)
+        cuq = torch.arange(0, T + 1, ql, dtype=torch.int32, device=dev)
+        cuk = torch.arange(0, S + 1, kl, dtype=torch.int32, device=dev)
+        out = torch.empty(T, H, dv, device=dev, dtype=torch.bfloat16)
+        lse = torch.empty(H, T, device=dev)
+
+        def call(_i=0):
+            ops.mla_prefill_attention(q, kv[..., :nope], kpe, kv[..., nope:], cuq, cuk, ql, (nope + rope) ** -0.5,
+                                      causal, out=out, lse=lse)
+
+        n = min(args.steps, 10)
+        for _ in range(min(args.warmup, 3)):
+            call()
+        s = time_back_to_back(call, n)
+        flops = B * ql * kl * (0.5 if causal else 1.0) * H * (nope + rope + dv) * 2
+        nbytes = (q.numel() + kv.numel() + kpe.numel() + out.numel()) * 2 + lse.numel() * 4
+        rows.append(dict(shape=name, ms_per_call=round(s * 1e3, 4), tflops=round(flops / s / 1e12, 1),
+                         frac=round(flops / s / 1e12 / MFMA_F16_PEAK_TFLOPS, 4), calls_timed=n,
+                         algorithmic_flops=int(flops), algorithmic_bytes=nbytes))
+        if name == MLA_PREFILL_SHAPES[0][0] and not args.no_cpu_baseline:
+            cpu = mla_prefill_cpu_baseline(q, kv, kpe, nope, ql, kl, args.cpu_seconds)
+        del q, kv, kpe, out, lse
+    r0 = rows[0]
+    res = {
+        "metric": "MLA prefill attention (bf16 K/V behind the latent gather): TFLOP/s over visible (query, key) pairs, 128 heads",
+        "value": r0["tflops"], "unit": "TFLOP/s", "n_gpus": 1, "steps": r0["calls_timed"], "warmup": min(args.warmup, 3),
+        "ms_per_step": r0["ms_per_call"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16 Q/K/V, fp16-range MFMA operands, fp32 softmax/accumulate", "data": "synthetic",
+        "config": {"workload": args.workload, "heads": H, "qk_nope_head_dim": nope, "qk_rope_head_dim": rope,
+                   "v_head_dim": dv, "shape": r0["shape"]},
+        "roofline": {"bound": "mfma", "achieved": r0["tflops"], "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": r0["frac"], "traffic": None, "kernel": "varlen_attn_kernel<1, 128, 64, 128>",
+                     "timing": f"{r0['calls_timed']} calls back to back between two events on the launch stream",
+                     "algorithmic_flops_per_launch": r0["algorithmic_flops"],
+                     "algorithmic_bytes_per_launch": r0["algorithmic_bytes"]},
+        "shapes": rows,
+    }
+    if not args.no_cpu_baseline:
+        res["cpu_baseline"] = cpu
+    print(json.dumps(res))
+
+
+def mla_prefill_cpu_baseline(q, kv, kpe, nope, ql, kl, seconds_target):
+    """fp32 torch statement of the same varlen attention on the host, on a slice of the first shape: the first
+    sequence, its last 128 query rows, a few heads at a time until the time is spent."""
+    from oracle import torch_ref
+
+    rows, hb = 128, 8
+    kn = kv[:kl, :, :nope].float().cpu()
+    vv = kv[:kl, :, nope:].float().cpu()
+    pe = kpe[:kl].float().cpu()
+    cu_q, cu_k = torch.tensor([0, rows], dtype=torch.int32), torch.tensor([0, kl], dtype=torch.int32)
+    t_total, blocks, r1 = 0.0, 0, ql
+    while t_total < seconds_target and r1 >= rows:       # row blocks from the end of the sequence backwards
+        qs = q[r1 - rows:r1].float().cpu()
+        for h in range(0, q.shape[1], hb):
+            t0 = time.perf_counter()
+            torch_ref.varlen_attn_lse(qs[:, h:h + hb], kn[:, h:h + hb], pe, vv[:, h:h + hb], cu_q, cu_k,
+                                      q.shape[-1] ** -0.5, False)
+            t_total += time.perf_counter() - t0
+            blocks += 1
+            if t_total >= seconds_target:
+                break
+        r1 -= rows
+    flops = blocks * rows * kl * hb * (q.shape[-1] + vv.shape[-1]) * 2
+    return dict(value=flops / t_total / 1e12, unit="TFLOP/s", cores=torch.get_num_threads(), kind="port",
+                sample=f"{blocks} blocks of {rows} query rows x {kl} keys x {hb} heads of the first shape's first sequence, "
+                       f"oracle/torch_ref.py varlen_attn_lse (fp32), {t_total:.1f} s, torch threads={torch.get_num_threads()}")
+
+
+def mixed_cpu_baseline(cfg, caches, bt, q, cu, scale, seconds_target):
+    """The reference's CPU path (as-written torch ops of its unified-attention test) on a bounded sample of the
+    mixed batch: the decode rows one after the other, then the last 64 query rows of each prefill chunk, in whole
+    passes until the time is spent.  Reported in the line's unit over the sample's algorithmic bytes, with its flops."""
+    from oracle import torch_ref
+
+    hq, hkv, d, bs, ctx, qls = (cfg[k] for k in ("hq", "hkv", "d", "bs", "ctx", "qlens"))
+    c0 = caches[0]
+    threads = torch.get_num_threads()
+    done_bytes = done_flops = 0
+    t_total, reps = 0.0, 0
+    order = [i for i, ql in enumerate(qls) if ql == 1] + [i for i, ql in enumerate(qls) if ql > 1]
+    host, idx = {}, 0
+    while t_total < seconds_target:                        # whole passes over the sample until the time is spent
+        i = order[idx % len(order)]
+        idx += 1
+        n = (ctx[i] + bs - 1) // bs
+        rows = min(qls[i], 64)
+        if i not in host:                                  # gathered to the host untimed: the reference's cache lives there
+            blocks = bt[i, :n].long().to(c0["k"].device)
+            host[i] = tuple(c0[name][blocks].cpu() for name in ("k", "v", "ks", "vs")) + (
+                q[int(cu[i + 1]) - rows:int(cu[i + 1])].cpu(),)
+        kb, vb, ksb, vsb, qi = host[i]
+        t0 = time.perf_counter()
+        kd, vd = torch_ref.dequant_cache(kb, vb, ksb, vsb, d, torch.bfloat16)
+        torch_ref.paged_attn(qi, kd, vd, [rows], [ctx[i]], torch.arange(n, dtype=torch.int32)[None], scale)
+        t_total += time.perf_counter() - t0
+        done_bytes += ctx[i] * hkv * 2 * (d + 4) + 2 * rows * hq * d * 2
+        done_flops += 4 * d * hq * (rows * (ctx[i] - rows) + rows * (rows + 1) // 2)
+        reps += 1
+        if idx % len(order) == 0 and t_total > 0.6 * seconds_target:
+            break
+    return dict(value=done_bytes / t_total / 1e9, unit="GB/s", cores=threads, kind="port",
+                tflops=done_flops / t_total / 1e12,
+                sample=f"{reps} sequence runs = {reps / len(order):.2f} passes over the 60 decode rows and the last 64 query rows of each of the four chunks ("
+                       f"{done_bytes / 1e6:.1f} MB of algorithmic bytes, {done_flops / 1e9:.1f} GFLOP), oracle/torch_ref.py "
+                       f"dequant_cache + paged_attn (bf16, as-written), {t_total:.1f} s, torch threads={threads}")
 
 
 def mixed_main(args, cfg, dev, ops):
@@ -454,6 +611,9 @@ def mixed_main(args, cfg, dev, ops):
     dec_bytes = sum(c for c, ql in zip(ctx, qls) if ql == 1) * hkv * 2 * (d + 4)
     pre_bytes = sum(c for c, ql in zip(ctx, qls) if ql > 1) * hkv * 2 * (d + 4) + 2 * n_tok * hq * d * 2
     write_bytes = n_tok * hkv * (2 * d * 2 + 2 * (d + 4))
+    traffic, traffic_source = measured_traffic(args.workload)
+    if args.sliding_window or args.soft_cap or cfg.get("kv_dtype") == "fp8" or args.kv_layout != "HND":
+        traffic, traffic_source = None, None
     res = {
         "metric": f"{cfg.get('kv_dtype', 'int8')}-KV mixed batch (4 x 2048-token prefill chunks + 60 decode rows): ms per layer",
         "value": round((dec_bytes + pre_bytes + write_bytes) / dt / 1e9, 1), "unit": "GB/s", "n_gpus": 1,
@@ -469,10 +629,14 @@ def mixed_main(args, cfg, dev, ops):
                    "kv_layout": args.kv_layout},
         "prewarm_s": PREWARM_S, "attn_launch_us": round(attn_s * 1e6, 1),
         "roofline": {"bound": "mfma", "achieved": round(flops / attn_s / 1e12, 1), "peak": MFMA_F16_PEAK_TFLOPS,
-                     "unit": "TFLOP/s", "frac": round(flops / attn_s / 1e12 / MFMA_F16_PEAK_TFLOPS, 4), "traffic": None,
+                     "unit": "TFLOP/s", "frac": round(flops / attn_s / 1e12 / MFMA_F16_PEAK_TFLOPS, 4),
+                     "traffic": traffic, "traffic_source": traffic_source,
+                     "timing": f"{n_ev} attention launches back to back between two events on the launch stream",
                      "kernel": "varlen attention launch = paged_decode_streamk_kernel + reduce + prefill_plan_kernel + paged_prefill_flash32_kernel",
                      "algorithmic_flops_per_launch": flops, "algorithmic_bytes_per_launch": dec_bytes + pre_bytes},
     }
+    if not args.no_cpu_baseline and cfg.get("kv_dtype") != "fp8":
+        res["cpu_baseline"] = mixed_cpu_baseline(cfg, caches, bt, q, cu, scale, args.cpu_seconds)
     print(json.dumps(res))
 
 
@@ -533,19 +697,25 @@ def time_decode(cfg, st, args, ops):
     step_s = (time.perf_counter() - t0) / args.steps
     n = max(args.steps, 100)
     attn_s = time_back_to_back(lambda i: run_step(st, i % L, ops, write=False, attn=True), n)
-    write_s = time_back_to_back(lambda i: run_step(st, i % L, ops, write=True, attn=False), n)
-    # the same step as ONE launch (the decode kernel writes the new tokens), timed like the two-launch step
-    for i in range(args.warmup):
-        run_step(st, i % L, ops, fused=True)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for i in range(args.steps):
-        run_step(st, i % L, ops, fused=True)
-    torch.cuda.synchronize()
-    fused_s = (time.perf_counter() - t0) / args.steps
-    return dict(step_s=step_s, attn_s=attn_s, write_s=write_s, attn_bytes=attn_bytes, n_attn=n,
-                value=(attn_bytes + write_bytes) / step_s / 1e9, fused_s=fused_s,
-                fused_value=(attn_bytes + write_bytes) / fused_s / 1e9)
+    write_host_s = time_back_to_back(lambda i: run_step(st, i % L, ops, write=True, attn=False), n)
+    write_s = time_graph_replay(lambda i: run_step(st, i % L, ops, write=True, attn=False), 100)
+    # the attention launch as GPU time only (50 launches in one HIP graph): differs from attn_s where the launch is
+    # shorter than the host's call (small batches)
+    attn_graph_s = time_graph_replay(lambda i: run_step(st, i % L, ops, write=False, attn=True), 50)
+    fused_s = None
+    if not args.no_one_launch:
+        # the same step as ONE launch (the decode kernel writes the new tokens), timed like the two-launch step
+        for i in range(args.warmup):
+            run_step(st, i % L, ops, fused=True)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(args.steps):
+            run_step(st, i % L, ops, fused=True)
+        torch.cuda.synchronize()
+        fused_s = (time.perf_counter() - t0) / args.steps
+    return dict(step_s=step_s, attn_s=attn_s, write_s=write_s, write_host_s=write_host_s, attn_bytes=attn_bytes, n_attn=n,
+                value=(attn_bytes + write_bytes) / step_s / 1e9, fused_s=fused_s, attn_graph_s=attn_graph_s,
+                fused_value=(attn_bytes + write_bytes) / fused_s / 1e9 if fused_s else None)
 
 
 def main():
@@ -560,11 +730,16 @@ def main():
     ap.add_argument("--soft-cap", type=float, default=0.0, help="GQA workloads: logits soft cap (0 = none)")
     ap.add_argument("--kv-dtype", choices=["int8", "fp8"], default="int8",
                     help="GQA decode workloads: code format of the cache (fp8 = e4m3fn per-token-head mode of the same layout)")
-    ap.add_argument("--kv-layout", choices=["HND", "NHD"], default="HND",
-                    help="GQA decode workloads: memory order of the cache tensor, both of which the reference defines "
-                         "(triton_attn.py:350-372, VLLM_KV_CACHE_LAYOUT).  HND keeps a head's records of a block back to "
-                         "back, which lets the decode loads stream; the default workload reports the other order too")
+    ap.add_argument("--kv-layout", choices=["HND", "NHD"], default=None,
+                    help="GQA workloads: memory order of the cache tensor, both of which the reference defines "
+                         "(triton_attn.py:350-372, VLLM_KV_CACHE_LAYOUT).  Default: what the backend itself asks for "
+                         "(vllm_metax_amd.layout.get_kv_cache_layout(): HND unless the environment says otherwise), "
+                         "so that the headline is the order a deployment gets; the default workload reports the other "
+                         "order too")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-one-launch", action="store_true",
+                    help="skip the one-launch variant of the step (write inside the decode launch): for profiler runs, "
+                         "where its dispatches would be averaged into the decode kernel's row")
     ap.add_argument("--no-fixed-8k", action="store_true",
                     help="default workload only: skip the extra fixed-context (64 x 8192) measurement")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
@@ -574,10 +749,15 @@ def main():
     if not torch.cuda.is_available():
         raise SystemExit("bench.py: no GPU visible; the HIP kernels have no CPU fallback")
     from vllm_metax_amd import _custom_ops as ops
+    from vllm_metax_amd.layout import get_kv_cache_layout
 
+    if args.kv_layout is None:
+        args.kv_layout = get_kv_cache_layout()
     dev = torch.device("cuda:0")
     cfg = make_batch(args.workload)
     cfg["kv_dtype"] = args.kv_dtype
+    if cfg.get("mla_prefill"):
+        return mla_prefill_main(args, cfg, dev, ops)
     if cfg.get("mla"):
         return mla_main(args, cfg, dev, ops)
     if cfg.get("mixed"):
@@ -587,8 +767,8 @@ def main():
     L = args.layers
     t = time_decode(cfg, st, args, ops)
     traffic, traffic_source = measured_traffic(args.workload)
-    if args.sliding_window or args.soft_cap or args.kv_dtype != "int8":
-        traffic, traffic_source = None, None
+    if args.sliding_window or args.soft_cap or args.kv_dtype != "int8" or args.kv_layout != "HND":
+        traffic, traffic_source = None, None   # the profiles were taken on the plain int8 workload in HND order
 
     res = {
         "metric": METRIC,
@@ -614,11 +794,16 @@ def main():
         "us_per_layer": round(t["step_s"] * 1e6, 2),
         "decode_tokens_per_s": round(len(cfg["ctx"]) / t["step_s"], 1),
         "attn_launch_us": round(t["attn_s"] * 1e6, 2),
+        # GPU time of the write kernel (100 launches in one HIP graph, replayed between two events), and what one
+        # call costs when the host issues them one by one (bound by the host, not by the kernel)
         "write_launch_us": round(t["write_s"] * 1e6, 2),
-        "one_launch_step": {"what": "the same step with the cache update inside the attention launch "
-                                    "(kvq_paged_attn_int8_fused_write; a backend with forward_includes_kv_cache_update)",
-                            "us_per_layer": round(t["fused_s"] * 1e6, 2), "value": round(t["fused_value"], 1), "unit": "GB/s",
-                            "pct_hbm_peak": round(100 * t["fused_value"] / HBM_PEAK_GBPS, 2)},
+        "write_call_host_us": round(t["write_host_s"] * 1e6, 2),
+        "attn_launch_in_graph_us": round(t["attn_graph_s"] * 1e6, 2),
+        "one_launch_step": None if t["fused_s"] is None else {
+            "what": "the same step with the cache update inside the attention launch "
+                    "(kvq_paged_attn_int8_fused_write; a backend with forward_includes_kv_cache_update)",
+            "us_per_layer": round(t["fused_s"] * 1e6, 2), "value": round(t["fused_value"], 1), "unit": "GB/s",
+            "pct_hbm_peak": round(100 * t["fused_value"] / HBM_PEAK_GBPS, 2)},
         "roofline": {"bound": "hbm", "achieved": round(t["attn_bytes"] / t["attn_s"] / 1e9, 1), "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": round(t["attn_bytes"] / t["attn_s"] / 1e9 / HBM_PEAK_GBPS, 4),
                      "traffic": traffic, "traffic_source": traffic_source,

@@ -60,7 +60,26 @@ def test_kernels_reproduce_golden(G, gpu_device):
                           block_table=G["block_table"].to(dev), k_scale_cache=ks, v_scale_cache=vs)
     torch.cuda.synchronize()
     T.assert_close_attn(out, G["part_reduced"], atol=2e-3, rtol=2e-3, what="golden decode")
+    # the fixture's whole mixed batch (decode rows and a prefill chunk through the one varlen entry point),
+    # output rows and log-sum-exp
+    qm = G["q"].to(dev)
+    outm = torch.empty(tuple(G["q"].shape), dtype=torch.float32, device=dev)
+    lsem = torch.empty(tuple(G["q"].shape[:2]), dtype=torch.float32, device=dev)
+    ops.unified_attention(qm, k, v, outm, G["cu"].to(dev), int(G["qlens"].max()), G["ctx"].to(dev), int(G["ctx"].max()),
+                          float(G["scale"]), True, block_table=G["block_table"].to(dev), k_scale_cache=ks,
+                          v_scale_cache=vs, lse=lsem)
+    torch.cuda.synchronize()
+    T.assert_close_attn(outm, G["out"], atol=4e-3, rtol=4e-3, what="golden mixed batch")
+    torch.testing.assert_close(lsem.cpu(), G["lse"], atol=5e-3, rtol=1e-3)
     mc = L.allocate_mla_cache(int(G["mla_nb"]), int(G["mla_bs"]), 576, device=dev)
     ops.concat_and_cache_mla(G["mla_kv_c"].to(dev), G["mla_k_pe"].to(dev), mc, G["mla_slots"].to(dev))
     torch.cuda.synchronize()
     assert torch.equal(mc.cpu(), G["mla_cache"]), "MLA latent cache differs from the golden bytes"
+    # MLA decode over the latent cache just written: output and log-sum-exp of the fixture
+    mq = G["mla_q"].to(dev)
+    mo = torch.empty(tuple(G["mla_out"].shape), dtype=torch.float32, device=dev)
+    mlse = torch.empty(tuple(G["mla_lse"].shape), dtype=torch.float32, device=dev)
+    ops.mla_decode_int8(mq, mc, mo, mlse, G["mla_block_table"].to(dev), G["mla_ctx"].to(dev), 192 ** -0.5, 512)
+    torch.cuda.synchronize()
+    T.assert_close_attn(mo, G["mla_out"], atol=4e-3, rtol=4e-3, what="golden mla decode")
+    torch.testing.assert_close(mlse.cpu(), G["mla_lse"], atol=5e-3, rtol=1e-3)

@@ -122,20 +122,21 @@ def test_config2_llama3_8b_b64_ctx1k_8k(gpu_device, layout):
     assert torch.equal(v.reshape(-1, hkv, d + 4)[last][..., :d], vc_before)
 
 
-def test_config3_long_context_split_k(gpu_device):
+@pytest.mark.parametrize("layout", ["NHD", "HND"])
+def test_config3_long_context_split_k(gpu_device, layout):
     dev = gpu_device
     hq, hkv, d, bs, pool = 32, 8, 128, 16, 66000
     g = torch.Generator().manual_seed(0)
     ctx = torch.randint(32768, 131073, (8,), generator=g).tolist()
     bt = _tables(ctx, bs, pool, g)
-    kv, k, v, ks, vs = _fill_gqa(dev, ctx, bt, hkv, d, bs, pool, outlier=True)
+    kv, k, v, ks, vs = _fill_gqa(dev, ctx, bt, hkv, d, bs, pool, outlier=True, layout=layout)
     q = torch.randn((8, hq, d), device=dev).to(torch.bfloat16)
     scale = 1 / math.sqrt(d)
     a, b, lse = _decode_both_ways(dev, q, k, v, ks, vs, bt, ctx, hq, hkv, d, bs, scale)
     assert torch.isfinite(a).all()
     T.assert_close_attn(a, b, atol=2e-3 * 20, rtol=2e-3, what="balanced split-K vs 512-token partitions")
     i = min(range(8), key=lambda j: ctx[j])
-    cpu, lay, bt2 = _gather_to_cpu(kv, bt, [i], ctx, hkv, d, bs)
+    cpu, lay, bt2 = _gather_to_cpu(kv, bt, [i], ctx, hkv, d, bs, layout)
     want, want_lse = oracle.paged_attn(q[[i]].cpu(), T.storage_bytes(cpu), lay, bt2,
                                        torch.tensor([ctx[i]], dtype=torch.int32), torch.arange(2, dtype=torch.int32),
                                        scale, return_lse=True)
@@ -187,7 +188,8 @@ def test_config4_mla_b32_ctx4096(gpu_device):
     torch.testing.assert_close(lse[seqs].cpu(), want_lse, atol=5e-3, rtol=1e-3)
 
 
-def test_config5_mixed_prefill_and_decode(gpu_device):
+@pytest.mark.parametrize("layout", ["NHD", "HND"])
+def test_config5_mixed_prefill_and_decode(gpu_device, layout):
     dev = gpu_device
     hq, hkv, d, bs, pool = 28, 4, 128, 16, 12000
     g = torch.Generator().manual_seed(0)
@@ -195,7 +197,7 @@ def test_config5_mixed_prefill_and_decode(gpu_device):
     ctx = [2048, 4096, 6144, 8192] + dctx            # lengths including the run's own tokens
     qls = [2048] * 4 + [1] * 60
     bt = _tables(ctx, bs, pool, g)
-    kv, k, v, ks, vs = _fill_gqa(dev, ctx, bt, hkv, d, bs, pool)
+    kv, k, v, ks, vs = _fill_gqa(dev, ctx, bt, hkv, d, bs, pool, layout=layout)
     n_tok = sum(qls)
     q = torch.randn((n_tok, hq, d), device=dev).to(torch.bfloat16)
     cu = torch.tensor([0] + torch.tensor(qls).cumsum(0).tolist(), dtype=torch.int32)
@@ -210,14 +212,14 @@ def test_config5_mixed_prefill_and_decode(gpu_device):
     cases = [(0, 0), (1, 1000), (3, 2016), (2, 37)]
     for i, r0 in cases:
         trunc = ctx[i] - qls[i] + r0 + 32
-        cpu, lay, bt2 = _gather_to_cpu(kv, bt, [i], [trunc if j == i else c for j, c in enumerate(ctx)], hkv, d, bs)
+        cpu, lay, bt2 = _gather_to_cpu(kv, bt, [i], [trunc if j == i else c for j, c in enumerate(ctx)], hkv, d, bs, layout)
         rows = slice(int(cu[i]) + r0, int(cu[i]) + r0 + 32)
         want = oracle.paged_attn(q[rows].cpu(), T.storage_bytes(cpu), lay, bt2, torch.tensor([trunc], dtype=torch.int32),
                                  torch.tensor([0, 32], dtype=torch.int32), scale)
         T.assert_close_attn(out[rows], want, atol=4e-3, rtol=4e-3, what=f"chunk {i} rows {r0}..")
     # decode rows of the same call
     seqs = [4, 33, 63]
-    cpu, lay, bt2 = _gather_to_cpu(kv, bt, seqs, ctx, hkv, d, bs)
+    cpu, lay, bt2 = _gather_to_cpu(kv, bt, seqs, ctx, hkv, d, bs, layout)
     rows = [int(cu[i]) for i in seqs]
     want = oracle.paged_attn(q[rows].cpu(), T.storage_bytes(cpu), lay, bt2, torch.tensor([ctx[i] for i in seqs], dtype=torch.int32),
                              torch.arange(4, dtype=torch.int32), scale)
