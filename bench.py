@@ -355,7 +355,8 @@ def mla_main(args, cfg, dev, ops):
         "ms_per_step": round(dt * 1e3, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "int8 latent codes, fp16 MFMA operands, fp32 softmax/accumulate, bf16 Q/out", "data": "synthetic",
         "config": {"workload": args.workload, "batch": len(cfg["ctx"]), "sum_ctx": sum(cfg["ctx"]), "heads": cfg["heads"],
-                   "kv_lora_rank": cfg["r"], "rope_dim": cfg["p"], "block_size": cfg["bs"], "layer_caches_rotated": L},
+                   "kv_lora_rank": cfg["r"], "rope_dim": cfg["p"], "block_size": cfg["bs"], "layer_caches_rotated": L,
+                   **({"batch_invariant": True} if ops.batch_invariant() else {})},
         "prewarm_s": PREWARM_S, "us_per_layer": round(dt * 1e6, 2), "attn_launch_us": round(attn_s * 1e6, 2),
         "roofline": {**roof, "traffic": traffic, "traffic_source": traffic_source,
                      "kernel": ("MLA decode launch on an absorbed query = mla_decode_small_kernel + mla_reduce_kernel" if small else
@@ -767,7 +768,7 @@ def main():
     L = args.layers
     t = time_decode(cfg, st, args, ops)
     traffic, traffic_source = measured_traffic(args.workload)
-    if args.sliding_window or args.soft_cap or args.kv_dtype != "int8" or args.kv_layout != "HND":
+    if args.sliding_window or args.soft_cap or args.kv_dtype != "int8" or args.kv_layout != "HND" or ops.batch_invariant():
         traffic, traffic_source = None, None   # the profiles were taken on the plain int8 workload in HND order
 
     res = {
@@ -786,6 +787,7 @@ def main():
         "config": {"workload": args.workload, "batch": len(cfg["ctx"]), "sum_ctx": sum(cfg["ctx"]),
                    "q_heads": cfg["hq"], "kv_heads": cfg["hkv"], "head_dim": cfg["d"], "block_size": cfg["bs"],
                    "pool_blocks": cfg["pool"], "layer_caches_rotated": L, "kv_layout": args.kv_layout,
+                   **({"batch_invariant": True} if ops.batch_invariant() else {}),
                    **({"kv_dtype": "fp8_per_token_head"} if args.kv_dtype == "fp8" else {}),
                    **({"sliding_window": args.sliding_window} if args.sliding_window else {}),
                    **({"soft_cap": args.soft_cap} if args.soft_cap else {})},

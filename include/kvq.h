@@ -27,7 +27,7 @@
 extern "C" {
 #endif
 
-#define KVQ_ABI_VERSION 12
+#define KVQ_ABI_VERSION 13
 
 #define KVQ_OK 0
 #define KVQ_EINVAL (-22)
@@ -91,6 +91,19 @@ KVQ_API const char* kvq_last_error(void);
 
 /* Number of compute units of the current device (host query, cached). */
 KVQ_API int kvq_device_num_cus(void);
+
+/*
+ * Batch-invariant mode, process-wide: the switch the reference reads from envs.VLLM_BATCH_INVARIANT
+ * (vllm_metax/v1/attention/backends/mla/triton_mla.py:247-253: one KV split; triton_attn.py:310-312:
+ * supports_batch_invariance).  While it is on, every decode sequence is cut into splits by its OWN length
+ * alone and its split states are merged in split order, so the bits of a row do not depend on what else the
+ * batch holds, on the batch size or on the device's CU count: kvq_paged_attn_int8* cut a sequence into at
+ * most 32 equal spans of at least 512 tokens, kvq_mla_decode_* into 8 splits.  Prefill rows never depend on
+ * their neighbours.  The workspace queries return what the mode needs, so set it before sizing workspaces
+ * and not while launches are being enqueued.  Returns the previous setting.
+ */
+KVQ_API int kvq_set_batch_invariant(int on);
+KVQ_API int kvq_get_batch_invariant(void);
 
 /*
  * Quantise-on-write of new K/V tokens into the paged cache.

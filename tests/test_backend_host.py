@@ -12,7 +12,7 @@ from vllm_metax_amd import _C, platform as P
 from vllm_metax_amd.kv_cache_interface import KVQuantMode, get_kv_quant_mode, kv_cache_uses_per_token_head_scales
 from vllm_metax_amd.v1.attention.backends.int8_attn import (
     AttentionType, Int8AttentionBackend, Int8AttentionImpl, Int8AttentionMetadataBuilder, MultipleOf)
-from vllm_metax_amd.v1.attention.backends.mla.int8_mla import Int8MLABackend, Int8MLAImpl, _compute_num_kv_splits
+from vllm_metax_amd.v1.attention.backends.mla.int8_mla import Int8MLABackend, Int8MLAImpl
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
@@ -213,11 +213,15 @@ def test_impl_constructor_errors():
         Int8MLAImpl(128, 576, 0.07, kv_cache_dtype="fp8")
 
 
-def test_num_kv_splits_policy():
-    assert _compute_num_kv_splits(4096, 256) == 8
-    assert _compute_num_kv_splits(100, 256) == 1
-    assert _compute_num_kv_splits(1 << 20, 4) == 8
-    assert _compute_num_kv_splits(5000, 256) == 16
+def test_backends_serve_batch_invariance_and_the_switch_is_the_librarys():
+    """triton_attn.py:310-312; the mode itself is a process-wide switch of the library (no GPU needed to flip it)."""
+    assert Int8AttentionBackend.supports_batch_invariance() is True
+    assert Int8MLABackend.supports_batch_invariance() is True
+    lib = _C.load()
+    before = lib.kvq_set_batch_invariant(1)
+    assert lib.kvq_get_batch_invariant() == 1 and lib.kvq_set_batch_invariant(0) == 1
+    assert lib.kvq_get_batch_invariant() == 0
+    lib.kvq_set_batch_invariant(before)
 
 
 def test_builder_packs_metadata_without_touching_the_gpu():

@@ -813,6 +813,9 @@ struct StreamKArgs {
   int new_dtype;
   float new_eps;
   const int64_t* new_slots;  // the step's slot mapping or nullptr: a row with a negative entry is padding, not written
+  // != 0: the batch-invariant cutting (every sequence cut by its own length alone); the partial states then take
+  // kFixedSpans slots per sequence and wg_info / seq_first_unit are not used
+  int fixed_spans;
 };
 
 // The decode kernel's fused cache update: the wave that owns kv head `hkv` of the run that holds a sequence's

@@ -2,6 +2,8 @@
 #include <stdarg.h>
 #include <stdio.h>
 
+#include <atomic>
+
 #include "kvq_internal.h"
 
 namespace kvq {
@@ -35,9 +37,15 @@ int num_cus() {
   return cached_cus;
 }
 
+static std::atomic<int> g_batch_invariant{0};
+bool batch_invariant() { return g_batch_invariant.load(std::memory_order_relaxed) != 0; }
+
 }  // namespace kvq
 
 extern "C" {
+
+int kvq_set_batch_invariant(int on) { return kvq::g_batch_invariant.exchange(on != 0 ? 1 : 0); }
+int kvq_get_batch_invariant(void) { return kvq::batch_invariant() ? 1 : 0; }
 
 int kvq_abi_version(void) { return KVQ_ABI_VERSION; }
 const char* kvq_last_error(void) { return kvq::g_err; }

@@ -12,6 +12,7 @@ namespace kvq {
 int fail(int code, const char* fmt, ...);  // records kvq_last_error(), returns code
 int check_hip(hipError_t e, const char* what);
 int num_cus();
+bool batch_invariant();  // the process-wide mode of kvq_set_batch_invariant()
 inline hipStream_t as_stream(kvq_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
 
 #define KVQ_REQUIRE(cond, ...)                      \

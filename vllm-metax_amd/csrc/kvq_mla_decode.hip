@@ -1353,8 +1353,12 @@ __global__ __launch_bounds__(512) void mla_reduce_kernel(void* out, float* lse, 
 
 // num_kv_splits policy of the reference (vllm_metax/v1/attention/backends/mla/triton_mla.py:45-55),
 // additionally bounded so that (sequences x splits) does not far exceed the resident workgroups.
+// In the batch-invariant mode every sequence is cut into kMlaInvariantSplits whatever the batch holds (the
+// reference takes one split there, triton_mla.py:247-253; any count that does not depend on the batch serves).
+constexpr int kMlaInvariantSplits = 8;
 static int mla_num_splits(int max_seq_hint, int num_seqs, int num_heads) {
   (void)max_seq_hint;
+  if (batch_invariant()) return kMlaInvariantSplits;
   const int cus = num_cus();
   const int groups = (num_heads + 127) / 128;
   int splits = 1;
@@ -1541,6 +1545,8 @@ static int mla_decode_run(const char* op, void* out, int out_dtype, float* lse, 
   if (rc) return rc;
   if (splits == 1) return KVQ_OK;   // the decode kernel wrote the result itself
   // a few blocks and dozens of splits: a piece per thread, 32 splits per trip, four times the blocks
+  // (never in the batch-invariant mode, whose eight splits are merged in one trip by either kernel: the choice must
+  // not depend on the batch)
   const bool fine = splits > 8 && 4 * num_seqs * head_groups <= num_cus();
   dim3 rgrid(num_seqs, head_groups, fine ? 4 : 1);
 #define KVQ_MLAR(T)                                                                                                \
@@ -1571,6 +1577,7 @@ size_t kvq_mla_decode_workspace_bytes(int max_num_seqs, int num_heads, int kv_lo
   const size_t groups = ((size_t)num_heads + 127) / 128;
   size_t items = 2 * (size_t)kvq::num_cus() / groups;
   if (items < (size_t)max_num_seqs) items = (size_t)max_num_seqs;
+  if (kvq::batch_invariant()) items = (size_t)kvq::kMlaInvariantSplits * (size_t)max_num_seqs;
   const size_t heads_padded = ((size_t)num_heads + 15) / 16 * 16;
   // split states (fp16 outputs + fp32 lse) and, per sequence, Q as two int8 terms + one scale per head
   return items * heads_padded * ((size_t)kv_lora_rank * sizeof(uint16_t) + sizeof(float)) +

@@ -12,6 +12,7 @@ namespace kvq {
 
 int launch_decode_streamk(const StreamKArgs& a, int q_dtype, int out_dtype, hipStream_t s);
 size_t streamk_workspace_bytes(int max_num_seqs, int num_q_heads, int head_size, int num_wg);
+size_t streamk_slots(int max_num_seqs, int num_wg);
 int decode_streamk_num_wg(int num_kv_heads);
 int validate_common(const char* op, const void* q, const void* cache, const kvq_cache_geom* geom,
                     const int32_t* block_table, const int32_t* seq_lens, int num_seqs, int num_q_heads);
@@ -110,7 +111,8 @@ static int paged_attn_launch(const char* op, void* out, int out_dtype, int64_t o
   a.cu_seqlens_q = cu_seqlens_q;
   a.num_seqs = num_seqs;
   a.num_wg = num_wg;
-  const size_t slots = (size_t)num_wg + (size_t)num_seqs;
+  const size_t slots = streamk_slots(num_seqs, num_wg);
+  a.fixed_spans = batch_invariant() ? 1 : 0;
   a.part_o = static_cast<float*>(workspace);
   a.part_ml = a.part_o + slots * (size_t)num_q_heads * (size_t)g.head_size;
   // 8-byte aligned: a slot's (D + 2) floats are a multiple of 8 bytes

@@ -130,12 +130,20 @@ static int launch_reduce(void* out, int out_dtype, float* lse, const float* exp_
   return check_hip(hipGetLastError(), "splitk_reduce launch");
 }
 
+// Slots of partial states a launch may fill: one per (workgroup, sequence) step of the balanced cutting's staircase,
+// or kFixedSpans per sequence with the batch-invariant cutting.
+size_t streamk_slots(int max_num_seqs, int num_wg) {
+  const size_t stair = (size_t)num_wg + (size_t)max_num_seqs;
+  const size_t fixed = (size_t)kFixedSpans * (size_t)max_num_seqs;
+  return batch_invariant() && fixed > stair ? fixed : stair;
+}
+
 // Workspace layout of the stream-K partials.
 size_t streamk_workspace_bytes(int max_num_seqs, int num_q_heads, int head_size, int num_wg) {
-  const size_t slots = (size_t)num_wg + (size_t)max_num_seqs;
+  const size_t slots = streamk_slots(max_num_seqs, num_wg);
   return slots * (size_t)num_q_heads * ((size_t)head_size + 2) * sizeof(float) +
          (2 * (size_t)num_wg + 2 + (size_t)max_num_seqs) * sizeof(int64_t) +   // where the shares and the sequences begin
-         ((size_t)max_num_seqs + 2) / 2 * 2 * sizeof(int32_t);                  // the prefill kernels' list of sequences   // where every workgroup's share begins on the work line
+         ((size_t)max_num_seqs + 2) / 2 * 2 * sizeof(int32_t);                  // the prefill kernels' list of sequences
 }
 
 int decode_streamk_num_wg(int num_kv_heads) { return streamk_num_wg(num_kv_heads); }

@@ -114,11 +114,25 @@ __device__ __forceinline__ int active_workgroups(int64_t total, int num_wg) {
   return want >= num_wg ? num_wg : (want < 1 ? 1 : (int)want);
 }
 
+// Batch-invariant cutting (StreamKArgs::fixed_spans): a sequence is cut at places that depend on nothing but its
+// own length -- into at most kFixedSpans spans of equal size, none shorter than kMinSpanTiles tiles -- and
+// workgroup w takes the (sequence, span) pairs w, w + P, w + 2 P, ... one after the other.  The states of a
+// sequence's spans lie in slots seq * kFixedSpans + span and are merged in span order, so a row's bits are the same
+// whatever else the batch holds and however many workgroups the device runs.
+constexpr int kFixedSpans = 32;
+constexpr int kMinSpanTiles = 16;
+__device__ __forceinline__ int fixed_span_tiles(int ntiles) {
+  const int per = (ntiles + kFixedSpans - 1) / kFixedSpans;
+  return per > kMinSpanTiles ? per : kMinSpanTiles;
+}
+
 // HPW = kv heads per workgroup (1, 2, 4 or 8).  A workgroup always has eight waves: with fewer than
 // eight kv heads the 8 / HPW waves of a head take the tiles of a run in turn and their states are
 // folded together in LDS when the run ends, so a compute unit keeps eight tile streams in flight
 // whatever the head count and a sequence is cut into no more partial states than with eight heads.
-template <int D, int QDT, int HPW, bool CAP, int CODE, bool STREAM>
+// FIXED: the batch-invariant cutting instead of the balanced one (a template argument, so that the balanced
+// kernel carries none of it: as a run-time branch it cost the headline launch 0.6 us).
+template <int D, int QDT, int HPW, bool CAP, int CODE, bool STREAM, bool FIXED = false>
 __global__ __launch_bounds__(512) void paged_decode_streamk_kernel(StreamKArgs a) {
   using DTile = DecodeTile<D, QDT, kRuntimeDtype, CODE>;
   constexpr int NSUB = 8 / HPW;
@@ -131,29 +145,86 @@ __global__ __launch_bounds__(512) void paged_decode_streamk_kernel(StreamKArgs a
   const int w = blockIdx.x;
   const int B = a.num_seqs;
 
-  // total units of the work line (each wave redoes this tiny scan; no LDS, no barrier)
-  const bool one_chunk = B <= kWave;
-  const int64_t total = one_chunk ? scan_total<1>(a, lane) : scan_total<kScanBatch>(a, lane);
-  const int num_wg = active_workgroups(total, a.num_wg);
-  if (w >= num_wg) return;
-  const int64_t lo = wg_tile_begin(w, total, num_wg);
-  const int64_t hi = wg_tile_begin(w + 1, total, num_wg);
-  if (lo >= hi) {   // an empty work line: workgroup 0 still reports its length
-    if (w == 0 && blockIdx.y == 0 && wave == 0 && lane == 0) a.wg_info[0] = total;
-    return;
-  }
+  constexpr bool fixed = FIXED;
 
-  // locate the sequence holding unit `lo`
+  // the balanced cutting: total units of the work line (each wave redoes this tiny scan; no LDS, no barrier)
+  const bool one_chunk = B <= kWave;
+  int64_t total = 0, lo = 0, hi = 0;
   int seq = 0;
   int64_t seq_start = 0;  // global index of the sequence's first unit
-  if (one_chunk) scan_locate<1>(a, lane, lo, seq, seq_start);
-  else scan_locate<kScanBatch>(a, lane, lo, seq, seq_start);
-  seq = __builtin_amdgcn_readfirstlane(seq);
+  if constexpr (!fixed) {
+    total = one_chunk ? scan_total<1>(a, lane) : scan_total<kScanBatch>(a, lane);
+    const int num_wg = active_workgroups(total, a.num_wg);
+    if (w >= num_wg) return;
+    lo = wg_tile_begin(w, total, num_wg);
+    hi = wg_tile_begin(w + 1, total, num_wg);
+    if (lo >= hi) {   // an empty work line: workgroup 0 still reports its length
+      if (w == 0 && blockIdx.y == 0 && wave == 0 && lane == 0) a.wg_info[0] = total;
+      return;
+    }
+    // locate the sequence holding unit `lo`
+    if (one_chunk) scan_locate<1>(a, lane, lo, seq, seq_start);
+    else scan_locate<kScanBatch>(a, lane, lo, seq, seq_start);
+    seq = __builtin_amdgcn_readfirstlane(seq);
+  }
   // Where the share begins (the reduce kernel's key to the span): noted in the first round of the loop, stored
   // after the last.  A store ahead of the tile loads would sit before them in the wave's in-order memory
   // counter, and the first tile would wait for the store's acknowledgement (measured: 0.6 us per launch).
   int info_seq = -1;
   int64_t info_start = 0;
+
+  // One run of tiles [t_begin, t_end) of sequence `cur` (ntiles tiles from tile t0 on), its state to `slot` unless
+  // the run is the whole sequence.
+  auto process = [&](int cur, int64_t cur_start, int64_t row, int len, int first, int t0, int ntiles, int t_begin,
+                     int t_end, int64_t slot) __attribute__((always_inline)) {
+    if (a.k_new != nullptr && t_end == t0 + ntiles) {   // uniform over the workgroup: the run holds the last tile
+      const bool padding = a.new_slots != nullptr && a.new_slots[row] < 0;   // uniform: a scalar load
+      if (sub == 0 && !padding) write_new_token<D>(a, cur, row, len, hkv, lane);
+      // the record is in memory before any wave of the workgroup loads the tile that holds it
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      if constexpr (NSUB > 1) lds_barrier();
+    }
+    typename DTile::State st;
+    DTile::template run<CAP, STREAM>(a.io, cur, row, len, first, t_begin, t_end, hkv, lane, lds[wave], st, sub, NSUB);
+    // the run holds the sequence's first tile: its place on the line, for the reduce kernel (behind the run's loads)
+    if (!fixed && t_begin == t0 && blockIdx.y == 0 && wave == 0 && lane == 0) a.seq_first_unit[cur] = cur_start;
+    if constexpr (NSUB > 1) {
+      if (sub != 0) DTile::dump_state(st, lane, lds[wave]);
+      lds_barrier();
+      if (sub == 0) {
+#pragma unroll
+        for (int j = 1; j < NSUB; ++j)
+          if (t_begin + j < t_end) DTile::fold_state(st, lane, lds[wave + j]);  // wave j owned a tile
+      }
+      lds_barrier();  // the windows may be overwritten by the next run
+    }
+    if (sub == 0) {
+      if (t_begin == t0 && t_end == t0 + ntiles) {
+        DTile::emit_final(a.io, row, hkv, lane, st);
+      } else {
+        DTile::emit_partial(a.io, a.part_o, a.part_ml, slot, hkv, lane, st);
+      }
+    }
+  };
+
+  if constexpr (fixed) {
+    // the (sequence, span) pairs w, w + P, ...
+    for (int item = w; item < B * kFixedSpans; item += (int)gridDim.x) {
+      const int cur = item / kFixedSpans;
+      const int span = item % kFixedSpans;
+      const int ntiles = __builtin_amdgcn_readfirstlane(decode_tiles(a.seq_lens, a.cu_seqlens_q, cur, B, a.io.window));
+      const int per = fixed_span_tiles(ntiles);
+      if (span * per >= ntiles) continue;   // also: no tiles at all
+      const int len = __builtin_amdgcn_readfirstlane(a.seq_lens[cur]);
+      const int64_t row = a.cu_seqlens_q ? (int64_t)a.cu_seqlens_q[cur] : (int64_t)cur;
+      const int first = window_first(len, a.io.window);
+      const int t0 = first / kTile;
+      const int t_begin = t0 + span * per;
+      const int t_end = min(t0 + ntiles, t_begin + per);
+      process(cur, 0, row, len, first, t0, ntiles, t_begin, t_end, (int64_t)cur * kFixedSpans + span);
+    }
+    return;
+  }
 
   int64_t pos = lo;
   while (pos < hi && seq < B) {
@@ -178,36 +249,8 @@ __global__ __launch_bounds__(512) void paged_decode_streamk_kernel(StreamKArgs a
     const int u_end = rem < units ? (int)rem : units;
     const int t_begin = __builtin_amdgcn_readfirstlane(t0 + (u_begin > kSetupUnits ? u_begin - kSetupUnits : 0));
     const int t_end = __builtin_amdgcn_readfirstlane(t0 + u_end - kSetupUnits);
-    if (t_begin < t_end) {  // else: this share ends inside the setup charge and holds no tile
-      if (a.k_new != nullptr && t_end == t0 + ntiles) {   // uniform over the workgroup: the run holds the last tile
-        const bool padding = a.new_slots != nullptr && a.new_slots[row] < 0;   // uniform: a scalar load
-        if (sub == 0 && !padding) write_new_token<D>(a, seq, row, len, hkv, lane);
-        // the record is in memory before any wave of the workgroup loads the tile that holds it
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        if constexpr (NSUB > 1) lds_barrier();
-      }
-      typename DTile::State st;
-      DTile::template run<CAP, STREAM>(a.io, seq, row, len, first, t_begin, t_end, hkv, lane, lds[wave], st, sub, NSUB);
-      // the run holds the sequence's first tile: its place on the line, for the reduce kernel (behind the run's loads)
-      if (t_begin == t0 && blockIdx.y == 0 && wave == 0 && lane == 0) a.seq_first_unit[seq] = seq_start;
-      if constexpr (NSUB > 1) {
-        if (sub != 0) DTile::dump_state(st, lane, lds[wave]);
-        lds_barrier();
-        if (sub == 0) {
-#pragma unroll
-          for (int j = 1; j < NSUB; ++j)
-            if (t_begin + j < t_end) DTile::fold_state(st, lane, lds[wave + j]);  // wave j owned a tile
-        }
-        lds_barrier();  // the windows may be overwritten by the next run
-      }
-      if (sub == 0) {
-        if (t_begin == t0 && t_end == t0 + ntiles) {
-          DTile::emit_final(a.io, row, hkv, lane, st);
-        } else {
-          DTile::emit_partial(a.io, a.part_o, a.part_ml, (int64_t)w + seq, hkv, lane, st);
-        }
-      }
-    }
+    if (t_begin < t_end)  // else: this share ends inside the setup charge and holds no tile
+      process(seq, seq_start, row, len, first, t0, ntiles, t_begin, t_end, (int64_t)w + seq);
     pos = seq_start + u_end;
     seq_start += units;
     ++seq;
@@ -219,6 +262,69 @@ __global__ __launch_bounds__(512) void paged_decode_streamk_kernel(StreamKArgs a
       a.wg_info[2 * w + 3] = info_start;
     }
   }
+}
+
+// The merge of the batch-invariant cutting: grid (num_seqs, ceil(Hq / 4)), a wave per q head, a lane owns D / 64
+// dims.  Lane j takes span j's (m, l); the wave agrees on the maximum and the weights; the spans' outputs are added
+// in span order.  Empty decode sequences get their defined output here as well.
+template <int D>
+__global__ __launch_bounds__(256) void paged_decode_fixed_spans_reduce_kernel(StreamKArgs a) {
+  constexpr int V = D / 64;
+  static_assert(kFixedSpans <= kWave, "one lane per span");
+  const int lane = threadIdx.x & 63;
+  const int head = blockIdx.y * 4 + (threadIdx.x >> 6);
+  const int seq = blockIdx.x;
+  const int Hq = a.io.num_q_heads;
+  if (head >= Hq) return;
+  const int q0 = a.cu_seqlens_q ? a.cu_seqlens_q[seq] : seq;
+  const int q1 = a.cu_seqlens_q ? a.cu_seqlens_q[seq + 1] : seq + 1;
+  const int len = a.seq_lens[seq];
+  if (q1 - q0 != 1) return;
+  const int64_t row = q0;
+  const int ntiles = len > 0 ? (len + kTile - 1) / kTile - window_first(len, a.io.window) / kTile : 0;
+  if (ntiles == 0) {  // empty sequence: defined output (zeros, lse = -inf)
+    for (int i = 0; i < V; ++i)
+      store_act_rt(a.io.out_dtype, a.io.out, row * a.io.out_stride_t + (int64_t)head * a.io.out_stride_h + lane * V + i, 0.f);
+    if (a.io.lse != nullptr && lane == 0) a.io.lse[row * Hq + head] = -INFINITY;
+    return;
+  }
+  const int per = fixed_span_tiles(ntiles);
+  const int spans = (ntiles + per - 1) / per;
+  if (spans == 1) return;  // written directly by the main kernel
+  const int64_t slot0 = (int64_t)seq * kFixedSpans;
+  const bool live = lane < spans;
+  const int64_t mine = slot0 + (live ? lane : spans - 1);
+  const float mj_raw = a.part_ml[(mine * Hq + head) * 2 + 0];
+  const float lj_raw = a.part_ml[(mine * Hq + head) * 2 + 1];
+  const float mj = live ? mj_raw : -INFINITY;
+  const float m = wave_max(mj);
+  const float ej = live ? __builtin_amdgcn_exp2f(mj - m) : 0.f;
+  const float l = wave_sum(live ? lj_raw * ej : 0.f);
+  float acc[V];
+#pragma unroll
+  for (int i = 0; i < V; ++i) acc[i] = 0.f;
+  for (int k0 = 0; k0 < spans; k0 += 8) {   // eight spans per trip to memory, added in span order
+    float po[8][V];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      const int64_t sk = slot0 + min(k0 + k, spans - 1);
+      const float* p = a.part_o + (sk * Hq + head) * (int64_t)D + lane * V;
+#pragma unroll
+      for (int i = 0; i < V; ++i) po[k][i] = p[i];
+    }
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      const float wk = k0 + k < spans ? __shfl(ej, k0 + k, kWave) : 0.f;
+      const uint32_t kk = wk != 0.f ? 0xffffffffu : 0u;
+#pragma unroll
+      for (int i = 0; i < V; ++i) acc[i] += as_f32(as_u32(po[k][i]) & kk) * wk;
+    }
+  }
+  const float inv = 1.0f / l;
+#pragma unroll
+  for (int i = 0; i < V; ++i)
+    store_act_rt(a.io.out_dtype, a.io.out, row * a.io.out_stride_t + (int64_t)head * a.io.out_stride_h + lane * V + i, acc[i] * inv);
+  if (a.io.lse != nullptr && lane == 0) a.io.lse[row * Hq + head] = (m + __builtin_amdgcn_logf(l)) * kLn2;
 }
 
 // Merge the partial states of every decode sequence that more than one workgroup touched, and give empty decode
@@ -687,7 +793,12 @@ static int launch_streamk(const StreamKArgs& a, hipStream_t s) {
   dim3 grid(a.num_wg, (hkv + hpw - 1) / hpw);
 #define KVQ_SK(H, C)                                                                                              \
   do {                                                                                                            \
-    if (a.io.g.code_type == KVQ_CODE_FP8_E4M3) {                                                                  \
+    if (a.fixed_spans) {                                                                                          \
+      if (a.io.g.code_type == KVQ_CODE_FP8_E4M3)                                                                  \
+        hipLaunchKernelGGL((paged_decode_streamk_kernel<D, QDT, H, C, KVQ_CODE_FP8_E4M3, false, true>), grid, dim3(512), 0, s, a); \
+      else                                                                                                        \
+        hipLaunchKernelGGL((paged_decode_streamk_kernel<D, QDT, H, C, KVQ_CODE_INT8, false, true>), grid, dim3(512), 0, s, a); \
+    } else if (a.io.g.code_type == KVQ_CODE_FP8_E4M3) {                                                           \
       if (!C && stream)                                                                                           \
         hipLaunchKernelGGL((paged_decode_streamk_kernel<D, QDT, H, false, KVQ_CODE_FP8_E4M3, true>), grid, dim3(512), 0, s, a); \
       else                                                                                                        \
@@ -719,6 +830,11 @@ static int launch_streamk(const StreamKArgs& a, hipStream_t s) {
 #undef KVQ_SK
   int rc = check_hip(hipGetLastError(), "paged_attn_int8 decode launch");
   if (rc) return rc;
+  if (a.fixed_spans) {
+    dim3 rgrid(a.num_seqs, (a.io.num_q_heads + 3) / 4);
+    hipLaunchKernelGGL((paged_decode_fixed_spans_reduce_kernel<D>), rgrid, dim3(256), 0, s, a);
+    return check_hip(hipGetLastError(), "paged_attn_int8 reduce launch");
+  }
   // a sequence is cut where a share begins inside it: a batch of few sequences has most of them cut several
   // times (grid over the sequences, a wave per q head), a large batch has at most one cut per share and many
   // sequences with none (grid over the shares, four q heads per wave)

@@ -14,7 +14,7 @@ LIB_PATH = os.path.join(_LIB_DIR, "libkvq_hip.so")
 
 KVQ_F32, KVQ_BF16, KVQ_F16 = 0, 1, 2
 KVQ_CODE_INT8, KVQ_CODE_FP8_E4M3 = 0, 1
-ABI_VERSION = 12
+ABI_VERSION = 13
 
 
 class CacheGeom(ctypes.Structure):
@@ -49,6 +49,8 @@ SIGNATURES = {
     "kvq_abi_version": (_i, []),
     "kvq_last_error": (ctypes.c_char_p, []),
     "kvq_device_num_cus": (_i, []),
+    "kvq_set_batch_invariant": (_i, [_i]),
+    "kvq_get_batch_invariant": (_i, []),
     "kvq_reshape_and_cache_int8": (_i, [_vp, _vp, _i, _i64, _i64, _i64, _i64, _vp, _geom_p, _vp, _i64, _f, _vp]),
     "kvq_paged_attn_workspace_bytes": (_sz, [_i, _i, _i]),
     "kvq_paged_attn_int8": (_i, [_vp, _i, _i64, _i64, _vp, _i, _i64, _i64, _vp, _geom_p, _vp, _i64, _vp, _vp,
@@ -104,6 +106,9 @@ def load() -> ctypes.CDLL:
     got = lib.kvq_abi_version()
     if got != ABI_VERSION:
         raise RuntimeError(f"libkvq_hip.so ABI version {got}, expected {ABI_VERSION}")
+    # the switch the reference reads as envs.VLLM_BATCH_INVARIANT, taken from the same variable
+    if os.environ.get("VLLM_BATCH_INVARIANT", "0").strip().lower() in ("1", "true", "yes", "on"):
+        lib.kvq_set_batch_invariant(1)
     _lib = lib
     return lib
 

@@ -93,6 +93,20 @@ def device_num_cus() -> int:
     return int(_C.load().kvq_device_num_cus())
 
 
+def set_batch_invariant(on: bool) -> bool:
+    """Turn the library's batch-invariant mode on or off (process-wide; on at load time when the environment
+    sets ``VLLM_BATCH_INVARIANT``, the variable the reference reads: mla/triton_mla.py:247-253).  While on, a
+    decode row's bits depend on its own sequence only.  Workspaces must be sized AFTER the mode is set
+    (``paged_attn_workspace_bytes`` / ``mla_decode_workspace_bytes`` return what the mode needs).  Returns the
+    previous setting."""
+    _ws_bytes_cache.clear()   # the remembered workspace sizes are those of the other mode
+    return bool(_C.load().kvq_set_batch_invariant(1 if on else 0))
+
+
+def batch_invariant() -> bool:
+    return bool(_C.load().kvq_get_batch_invariant())
+
+
 # ---------------------------------------------------------------------------------------------
 # quantise-on-write
 # ---------------------------------------------------------------------------------------------

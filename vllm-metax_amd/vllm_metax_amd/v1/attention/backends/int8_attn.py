@@ -202,7 +202,10 @@ class Int8AttentionBackend(_BackendBase):
 
     @classmethod
     def supports_batch_invariance(cls) -> bool:
-        return False  # the split depends on the batch's total length
+        """triton_attn.py:310-312.  Served by the library's batch-invariant mode (on when VLLM_BATCH_INVARIANT
+        is set, or through _custom_ops.set_batch_invariant): decode sequences are then cut by their own length
+        alone, and prefill rows never depend on their neighbours."""
+        return True
 
     @classmethod
     def supports_compute_capability(cls, capability) -> bool:

@@ -27,18 +27,9 @@ try:  # pragma: no cover - upstream vLLM is not installed in the build container
 except Exception:  # noqa: BLE001
     _MLAImplBase = object
 
-# num_kv_splits policy of the reference (vllm_metax/v1/attention/backends/mla/triton_mla.py:42-55)
-_MIN_WORK_PER_SPLIT = 512
-_SPLIT_OCCUPANCY_MULTIPLIER = 2
-
-
-def _next_power_of_2(n: int) -> int:
-    return 1 if n <= 1 else 1 << (n - 1).bit_length()
-
-
-def _compute_num_kv_splits(max_seq_len: int, sm_count: int) -> int:
-    ideal = _next_power_of_2(max(1, max_seq_len // _MIN_WORK_PER_SPLIT))
-    return min(ideal, sm_count * _SPLIT_OCCUPANCY_MULTIPLIER)
+# The number of KV splits (the reference's _compute_num_kv_splits, mla/triton_mla.py:42-55, and its one split
+# under VLLM_BATCH_INVARIANT, :247-253) is chosen inside the library: by the batch and the device's CUs, or, in
+# the batch-invariant mode (_custom_ops.set_batch_invariant), a fixed count that depends on nothing.
 
 
 @dataclass
@@ -214,6 +205,12 @@ class Int8MLABackend(_BackendBase):
     @classmethod
     def get_supported_head_sizes(cls) -> list[int]:
         return [576]
+
+    @classmethod
+    def supports_batch_invariance(cls) -> bool:
+        """Served by the library's batch-invariant mode (VLLM_BATCH_INVARIANT, as mla/triton_mla.py:247-253 reads
+        it): a fixed number of KV splits per sequence, merged in split order."""
+        return True
 
     @staticmethod
     def get_kv_cache_shape(num_blocks: int, block_size: int, num_kv_heads: int, head_size: int,
