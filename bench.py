@@ -141,15 +141,21 @@ def algorithmic_bytes(cfg, include_write=True):
     hq, hkv, d, bs = cfg["hq"], cfg["hkv"], cfg["d"], cfg["bs"]
     ctx = cfg["ctx"]
     B = len(ctx)
-    attn = sum(ctx) * hkv * 2 * (d + 4) + 2 * B * hq * d * 2 + sum((c + bs - 1) // bs for c in ctx) * 4 + 4 * B
-    write = B * hkv * (2 * d * 2 + 2 * (d + 4)) if include_write else 0
+    cb = d // 2 if cfg.get("kv_dtype") == "int4" else d   # code bytes of a half record (int4: two codes per byte)
+    attn = sum(ctx) * hkv * 2 * (cb + 4) + 2 * B * hq * d * 2 + sum((c + bs - 1) // bs for c in ctx) * 4 + 4 * B
+    write = B * hkv * (2 * d * 2 + 2 * (cb + 4)) if include_write else 0
     return attn, write
 
 
 def _quant_mode(cfg):
     from vllm_metax_amd.kv_cache_interface import KVQuantMode
 
-    return KVQuantMode.FP8_PER_TOKEN_HEAD if cfg.get("kv_dtype") == "fp8" else KVQuantMode.INT8_PER_TOKEN_HEAD
+    return {"fp8": KVQuantMode.FP8_PER_TOKEN_HEAD, "int4": KVQuantMode.INT4_PER_TOKEN_HEAD}.get(
+        cfg.get("kv_dtype"), KVQuantMode.INT8_PER_TOKEN_HEAD)
+
+
+def _cache_dtype_str(cfg):
+    return {"fp8": "fp8_per_token_head", "int4": "int4_per_token_head"}.get(cfg.get("kv_dtype"), "int8_per_token_head")
 
 
 def build_device_state(cfg, dev, layers, seed=0, layout="NHD", permute=True):
@@ -176,7 +182,7 @@ def build_device_state(cfg, dev, layers, seed=0, layout="NHD", permute=True):
     caches = []
     torch.manual_seed(seed)
     for _ in range(layers):
-        kv = L.allocate_kv_cache(pool, bs, hkv, d, device=dev, layout=layout, fill=0)
+        kv = L.allocate_kv_cache(pool, bs, hkv, d, device=dev, layout=layout, fill=0, cache_dtype_str=_cache_dtype_str(cfg))
         k, v = L.key_value_views(kv)
         ks, vs = L.scale_views(kv)
         ks.fill_(1.0)
@@ -564,12 +570,13 @@ def mixed_main(args, cfg, dev, ops):
         new_slots.append(bt[i, pos // bs].long() * bs + pos % bs)
     new_slots = torch.cat(new_slots).to(dev)
     for _ in range(args.layers):
-        kv = L.allocate_kv_cache(pool, bs, hkv, d, device=dev, layout=args.kv_layout, fill=0)
+        kv = L.allocate_kv_cache(pool, bs, hkv, d, device=dev, layout=args.kv_layout, fill=0,
+                                 cache_dtype_str=_cache_dtype_str(cfg))
         k, v = L.key_value_views(kv)
         ks, vs = L.scale_views(kv)
         ks.fill_(1.0)
         vs.fill_(1.0)
-        geom = L.geometry_from_views(k, v, ks, vs)
+        geom = L.geometry_from_views(k, v, ks, vs, L.code_type_of(mode))
         for i, c in enumerate(ctx):
             pos = torch.arange(c, device=dev)
             slots = bt_d[i, pos // bs].to(torch.int64) * bs + pos % bs
@@ -609,11 +616,12 @@ def mixed_main(args, cfg, dev, ops):
     attn_s = time_back_to_back(lambda i: step(i % Lr, write=False, attn=True), n_ev)
     # causal prefill flops: 4 D Hq (q_len * cached + q_len (q_len + 1) / 2); decode rows: 4 D Hq ctx
     flops = sum(4 * d * hq * (ql * (c - ql) + ql * (ql + 1) // 2) for c, ql in zip(ctx, qls))
-    dec_bytes = sum(c for c, ql in zip(ctx, qls) if ql == 1) * hkv * 2 * (d + 4)
-    pre_bytes = sum(c for c, ql in zip(ctx, qls) if ql > 1) * hkv * 2 * (d + 4) + 2 * n_tok * hq * d * 2
-    write_bytes = n_tok * hkv * (2 * d * 2 + 2 * (d + 4))
+    cb = d // 2 if cfg.get("kv_dtype") == "int4" else d
+    dec_bytes = sum(c for c, ql in zip(ctx, qls) if ql == 1) * hkv * 2 * (cb + 4)
+    pre_bytes = sum(c for c, ql in zip(ctx, qls) if ql > 1) * hkv * 2 * (cb + 4) + 2 * n_tok * hq * d * 2
+    write_bytes = n_tok * hkv * (2 * d * 2 + 2 * (cb + 4))
     traffic, traffic_source = measured_traffic(args.workload)
-    if args.sliding_window or args.soft_cap or cfg.get("kv_dtype") == "fp8" or args.kv_layout != "HND":
+    if args.sliding_window or args.soft_cap or cfg.get("kv_dtype") != "int8" or args.kv_layout != "HND":
         traffic, traffic_source = None, None
     res = {
         "metric": f"{cfg.get('kv_dtype', 'int8')}-KV mixed batch (4 x 2048-token prefill chunks + 60 decode rows): ms per layer",
@@ -622,7 +630,7 @@ def mixed_main(args, cfg, dev, ops):
         "scaling": "weak", "vs_baseline": None,
         "dtype": f"{cfg.get('kv_dtype', 'int8')} KV codes, fp16 MFMA operands, fp32 softmax/accumulate, bf16 Q/out", "data": "synthetic",
         "config": {"workload": args.workload,
-                   **({"kv_dtype": "fp8_per_token_head"} if cfg.get("kv_dtype") == "fp8" else {}),
+                   **({"kv_dtype": cfg["kv_dtype"] + "_per_token_head"} if cfg.get("kv_dtype") != "int8" else {}),
                    **({"sliding_window": args.sliding_window} if args.sliding_window else {}),
                    **({"soft_cap": args.soft_cap} if args.soft_cap else {}),
                    "batch": B, "new_tokens": n_tok, "sum_ctx": sum(ctx), "q_heads": hq,
@@ -636,7 +644,7 @@ def mixed_main(args, cfg, dev, ops):
                      "kernel": "varlen attention launch = paged_decode_streamk_kernel + reduce + prefill_plan_kernel + paged_prefill_flash32_kernel",
                      "algorithmic_flops_per_launch": flops, "algorithmic_bytes_per_launch": dec_bytes + pre_bytes},
     }
-    if not args.no_cpu_baseline and cfg.get("kv_dtype") != "fp8":
+    if not args.no_cpu_baseline and cfg.get("kv_dtype") == "int8":
         res["cpu_baseline"] = mixed_cpu_baseline(cfg, caches, bt, q, cu, scale, args.cpu_seconds)
     print(json.dumps(res))
 
@@ -729,8 +737,9 @@ def main():
     ap.add_argument("--sliding-window", type=int, default=0,
                     help="GQA workloads: attend to the last N keys only (0 = full causal, the configured workloads)")
     ap.add_argument("--soft-cap", type=float, default=0.0, help="GQA workloads: logits soft cap (0 = none)")
-    ap.add_argument("--kv-dtype", choices=["int8", "fp8"], default="int8",
-                    help="GQA decode workloads: code format of the cache (fp8 = e4m3fn per-token-head mode of the same layout)")
+    ap.add_argument("--kv-dtype", choices=["int8", "fp8", "int4"], default="int8",
+                    help="GQA workloads: code format of the cache (fp8 = e4m3fn per-token-head mode of the same layout; "
+                         "int4 = two 4-bit codes per byte, half the code bytes)")
     ap.add_argument("--kv-layout", choices=["HND", "NHD"], default=None,
                     help="GQA workloads: memory order of the cache tensor, both of which the reference defines "
                          "(triton_attn.py:350-372, VLLM_KV_CACHE_LAYOUT).  Default: what the backend itself asks for "
@@ -782,13 +791,13 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "int8 KV codes, fp16 MFMA operands, fp32 softmax/accumulate, bf16 Q/out",
+        "dtype": f"{args.kv_dtype} KV codes, fp16 MFMA operands, fp32 softmax/accumulate, bf16 Q/out",
         "data": "synthetic",
         "config": {"workload": args.workload, "batch": len(cfg["ctx"]), "sum_ctx": sum(cfg["ctx"]),
                    "q_heads": cfg["hq"], "kv_heads": cfg["hkv"], "head_dim": cfg["d"], "block_size": cfg["bs"],
                    "pool_blocks": cfg["pool"], "layer_caches_rotated": L, "kv_layout": args.kv_layout,
                    **({"batch_invariant": True} if ops.batch_invariant() else {}),
-                   **({"kv_dtype": "fp8_per_token_head"} if args.kv_dtype == "fp8" else {}),
+                   **({"kv_dtype": args.kv_dtype + "_per_token_head"} if args.kv_dtype != "int8" else {}),
                    **({"sliding_window": args.sliding_window} if args.sliding_window else {}),
                    **({"soft_cap": args.soft_cap} if args.soft_cap else {})},
         "prewarm_s": PREWARM_S,

@@ -27,7 +27,7 @@
 extern "C" {
 #endif
 
-#define KVQ_ABI_VERSION 13
+#define KVQ_ABI_VERSION 14
 
 #define KVQ_OK 0
 #define KVQ_EINVAL (-22)
@@ -49,8 +49,8 @@ typedef void* kvq_stream_t;
 
 /*
  * Byte geometry of the paged int8 cache with inline per-(token, head) scales.
- * One (block, slot, head) record is [K codes (head_size) | K scale fp32 |
- * V codes (head_size) | V scale fp32]; the four offsets locate those pieces
+ * One (block, slot, head) record is [K codes | K scale fp32 | V codes | V scale fp32],
+ * the codes of a half taking head_size bytes (head_size / 2 for KVQ_CODE_INT4); the four offsets locate those pieces
  * relative to the cache base for block 0 / slot 0 / head 0, the three strides
  * step to the next block / slot / head.  This is exactly the information the
  * reference's typed views carry: key_cache / value_cache =
@@ -62,7 +62,7 @@ typedef struct kvq_cache_geom {
   int64_t k_off, v_off, ks_off, vs_off;           /* bytes */
   int64_t stride_block, stride_slot, stride_head; /* bytes */
   int32_t num_kv_heads, head_size, block_size;
-  int32_t code_type;                              /* KVQ_CODE_INT8 (0) or KVQ_CODE_FP8_E4M3 */
+  int32_t code_type;                              /* KVQ_CODE_INT8 (0), KVQ_CODE_FP8_E4M3 or KVQ_CODE_INT4 */
 } kvq_cache_geom;
 
 /*
@@ -74,9 +74,18 @@ typedef struct kvq_cache_geom {
  * e4m3fn number nearest to x / scale (ties to even, saturating at +-448).  Served
  * by kvq_reshape_and_cache_int8 and kvq_paged_attn_int8 (and its static-scratch
  * form); the fixed-partition entry point is int8 only.
+ *
+ * KVQ_CODE_INT4: the int4_per_token_head mode, of which the reference states only the record width
+ * (triton_attn.py:336-348: two values per byte, head_size / 2 code bytes + the 4 scale bytes per half;
+ * the arithmetic lives in upstream Triton kernels it does not vendor).  This library's rule, a decision
+ * of this build: scale = max(absmax, eps) / 7 (fp32 division), code = clamp(rint(x / scale), -8, 7)
+ * (ties to even) as a 4-bit two's-complement number, dim 2 i in the low nibble of byte i and dim 2 i + 1
+ * in the high one.  Served by kvq_reshape_and_cache_int8, kvq_paged_attn_int8 and its fused-write and
+ * static-scratch forms (head sizes 64, 128, 256).
  */
 #define KVQ_CODE_INT8 0
 #define KVQ_CODE_FP8_E4M3 1
+#define KVQ_CODE_INT4 2
 
 /* Byte geometry of the int8 MLA latent cache: per block, block_size code rows
  * of (kv_lora_rank + rope_dim) bytes followed by block_size fp32 scales. */

@@ -74,7 +74,7 @@ class RecordLayout:
     num_kv_heads: int
 
     @staticmethod
-    def from_views(kv_cache, key_cache, value_cache, k_scale_cache, v_scale_cache):
+    def from_views(kv_cache, key_cache, value_cache, k_scale_cache, v_scale_cache, code_type: int = 0):
         """Derive the geometry from the typed views alone (data_ptr differences
         and strides), independent of how the views were constructed.
 
@@ -96,7 +96,7 @@ class RecordLayout:
             stride_block=sb,
             stride_slot=ss,
             stride_head=sh,
-            head_size=padded - 4,
+            head_size=(padded - 4) * (2 if code_type == 2 else 1),   # int4: two codes per byte
             block_size=bs,
             num_kv_heads=hkv,
         )
@@ -146,7 +146,33 @@ def quant_rows(x: torch.Tensor, eps: float | None = None):
     return codes, scales
 
 
-CODE_INT8, CODE_FP8 = 0, 1
+CODE_INT8, CODE_FP8, CODE_INT4 = 0, 1, 2
+
+
+def quant_rows_int4(x: torch.Tensor, eps: float | None = None):
+    """x [..., D] (CPU) -> (packed codes uint8 [..., D/2], scales fp32 [...]): scale = max(absmax, eps) / 7,
+    code = clamp(rint(x / scale), -8, 7) as a 4-bit two's-complement number, the even dim in the low nibble."""
+    if eps is None:
+        eps = eps_for(x.dtype)
+    xf = _f32c(x)
+    D = xf.shape[-1]
+    rows = xf.numel() // D
+    codes = torch.empty(xf.shape[:-1] + (D // 2,), dtype=torch.uint8)
+    scales = torch.empty(xf.shape[:-1], dtype=torch.float32)
+    lib().kvq_oracle_quant_rows_int4.restype = ctypes.c_int
+    _check(
+        lib().kvq_oracle_quant_rows_int4(_p(xf), _i64(rows), _i64(D), ctypes.c_float(eps), _p(codes), _p(scales)),
+        "kvq_oracle_quant_rows_int4",
+    )
+    return codes, scales
+
+
+def unpack_int4(codes: torch.Tensor) -> torch.Tensor:
+    """Packed int4 codes uint8 [..., D/2] -> their values int8 [..., D] (pure torch, for the tests)."""
+    c = codes.to(torch.int16)
+    lo, hi = c & 15, (c >> 4) & 15
+    both = torch.stack((lo, hi), dim=-1).reshape(codes.shape[:-1] + (codes.shape[-1] * 2,))
+    return torch.where(both >= 8, both - 16, both).to(torch.int8)
 
 
 def quant_rows_fp8(x: torch.Tensor, eps: float | None = None):

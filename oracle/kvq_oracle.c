@@ -14,6 +14,13 @@
  *   kvq_oracle_cache_write          pinned   (layout algebra + python scatter loop)
  *   kvq_oracle_quant_rows_fp8       pinned   (torch CPU float8_e4m3fn conversion on every fp32 in range,
  *                                             the 256-entry decode table against torch, closed forms)
+ *   kvq_oracle_quant_rows_int4      pinned against ITSELF only (closed forms: every value k * scale maps to k,
+ *                                             midpoints go to the even neighbour, brute force against exact
+ *                                             rationals, pack / unpack round trip); PARITY UNPINNED against
+ *                                             upstream: the reference states the record width of its int4 mode
+ *                                             (vllm_metax/v1/attention/backends/triton_attn.py:336-348) and nothing
+ *                                             of its arithmetic -- scale rule, rounding and nibble order are this
+ *                                             build's decision
  *   kvq_oracle_paged_attn           pinned   (torch SDPA on gathered K/V, block
  *                                             permutation invariance)
  *   kvq_oracle_paged_attn_partition pinned   (equals unsplit attention for any
@@ -146,8 +153,53 @@ KVQ_EXPORT int kvq_oracle_quant_rows_fp8(const float* x, int64_t rows, int64_t D
   return 0;
 }
 
-static inline double code_value(uint8_t b, int code_type) {
-  return code_type == KVQ_CODE_FP8 ? (double)e4m3fn_value(b) : (double)(int8_t)b;
+/* ---------------------------------------------------------------------------
+ * int4 codes of the INT4_PER_TOKEN_HEAD mode.  The reference fixes the record: two values per byte, so a
+ * half record is head_size / 2 code bytes + the fp32 scale
+ * (vllm_metax/v1/attention/backends/triton_attn.py:332-346).  The arithmetic is this build's decision,
+ * the int8 rule with the format's maximum in the place of 127: scale = max(absmax, eps) / 7 (fp32 true
+ * division), code = clamp(rint(x / scale), -8, 7) with ties to even, stored as a 4-bit two's-complement
+ * number; dim 2 i sits in the low nibble of byte i, dim 2 i + 1 in the high one.
+ * codes [rows, D / 2] bytes, scales [rows] fp32.
+ * ------------------------------------------------------------------------- */
+#define KVQ_CODE_INT4 2
+
+KVQ_EXPORT int kvq_oracle_quant_rows_int4(const float* x, int64_t rows, int64_t D, float eps,
+                                          uint8_t* codes, float* scales) {
+  if (!x || !codes || !scales || rows < 0 || D <= 0 || (D & 1)) return -1;
+#pragma omp parallel for schedule(static)
+  for (int64_t r = 0; r < rows; ++r) {
+    const float* xr = x + r * D;
+    float amax = 0.0f;
+    for (int64_t d = 0; d < D; ++d) {
+      float a = fabsf(xr[d]);
+      if (a > amax || a != a) amax = a;
+    }
+    if (amax < eps) amax = eps;
+    volatile float scale = amax / 7.0f;
+    scales[r] = scale;
+    for (int64_t d = 0; d < D; d += 2) {
+      unsigned byte = 0;
+      for (int j = 0; j < 2; ++j) {
+        volatile float qf = scale > 0.0f ? xr[d + j] / scale : 0.0f;
+        float rr = nearbyintf(qf);
+        if (rr < -8.0f) rr = -8.0f;
+        if (rr > 7.0f) rr = 7.0f;
+        byte |= ((unsigned)(int)rr & 0xfu) << (4 * j);
+      }
+      codes[r * (D / 2) + d / 2] = (uint8_t)byte;
+    }
+  }
+  return 0;
+}
+
+/* Value of code `d` of a half record whose code bytes start at `codes`. */
+static inline double code_at(const uint8_t* codes, int d, int code_type) {
+  if (code_type == KVQ_CODE_INT4) {
+    const int n = (codes[d >> 1] >> (4 * (d & 1))) & 0xf;
+    return (double)(n >= 8 ? n - 16 : n);
+  }
+  return code_type == KVQ_CODE_FP8 ? (double)e4m3fn_value(codes[d]) : (double)(int8_t)codes[d];
 }
 
 /* ---------------------------------------------------------------------------
@@ -177,6 +229,7 @@ KVQ_EXPORT int kvq_oracle_cache_write(
 }
 
 static int quant_row_any(const float* x, int D, float eps, uint8_t* codes, float* s, int code_type) {
+  if (code_type == KVQ_CODE_INT4) return kvq_oracle_quant_rows_int4(x, 1, D, eps, codes, s);
   return code_type == KVQ_CODE_FP8 ? kvq_oracle_quant_rows_fp8(x, 1, D, eps, codes, s)
                                    : kvq_oracle_quant_rows(x, 1, D, eps, (int8_t*)codes, s);
 }
@@ -197,11 +250,12 @@ KVQ_EXPORT int kvq_oracle_cache_write_ex(
     for (int h = 0; h < Hkv; ++h) {
       uint8_t* rec = cache + blk * stride_block + off * stride_slot + (int64_t)h * stride_head;
       float s;
+      const size_t nbytes = code_type == KVQ_CODE_INT4 ? (size_t)D / 2 : (size_t)D;
       quant_row_any(key + (t * Hkv + h) * (int64_t)D, D, eps, codes, &s, code_type);
-      memcpy(rec + k_off, codes, (size_t)D);
+      memcpy(rec + k_off, codes, nbytes);
       memcpy(rec + ks_off, &s, 4);
       quant_row_any(value + (t * Hkv + h) * (int64_t)D, D, eps, codes, &s, code_type);
-      memcpy(rec + v_off, codes, (size_t)D);
+      memcpy(rec + v_off, codes, nbytes);
       memcpy(rec + vs_off, &s, 4);
     }
   }
@@ -226,7 +280,7 @@ static void attend_range(const float* q, int D, const uint8_t* cache,
     float ks;
     memcpy(&ks, rec + ks_off, 4);
     double s = 0.0;
-    for (int d = 0; d < D; ++d) s += (double)q[d] * (code_value(kc[d], code_type) * (double)ks);
+    for (int d = 0; d < D; ++d) s += (double)q[d] * (code_at(kc, d, code_type) * (double)ks);
     s *= scale;
     if (softcap > 0.0) s = softcap * tanh(s / softcap);
     logits[j - k_begin] = s;
@@ -244,7 +298,7 @@ static void attend_range(const float* q, int D, const uint8_t* cache,
     double p = exp(logits[j - k_begin] - m);
     l += p;
     double pv = p * (double)vs;
-    for (int d = 0; d < D; ++d) acc[d] += pv * code_value(vc[d], code_type);
+    for (int d = 0; d < D; ++d) acc[d] += pv * code_at(vc, d, code_type);
   }
   *m_out = m;
   *l_out = l;

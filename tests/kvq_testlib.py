@@ -39,11 +39,17 @@ def slots_for(bt, ctx_lens, block_size):
     return out
 
 
-def cpu_cache(num_blocks, block_size, hkv, d, layout="NHD", fill=0):
-    kv = L.allocate_kv_cache(num_blocks, block_size, hkv, d, device="cpu", layout=layout, fill=fill)
+def _dtype_str(code_type):
+    return {oracle.CODE_INT8: "int8_per_token_head", oracle.CODE_FP8: "fp8_per_token_head",
+            oracle.CODE_INT4: "int4_per_token_head"}[code_type]
+
+
+def cpu_cache(num_blocks, block_size, hkv, d, layout="NHD", fill=0, code_type=oracle.CODE_INT8):
+    kv = L.allocate_kv_cache(num_blocks, block_size, hkv, d, device="cpu", layout=layout, fill=fill,
+                             cache_dtype_str=_dtype_str(code_type))
     k, v = L.key_value_views(kv)
     ks, vs = L.scale_views(kv)
-    lay = oracle.RecordLayout.from_views(_storage_base(kv), k, v, ks, vs)
+    lay = oracle.RecordLayout.from_views(_storage_base(kv), k, v, ks, vs, code_type)
     return kv, (k, v, ks, vs), lay
 
 
@@ -64,18 +70,20 @@ def storage_bytes(t):
     return torch.tensor([], dtype=torch.uint8, device=t.device).set_(t.untyped_storage())
 
 
-def fill_cache_from_sources(kv, lay, bt, ctx_lens, block_size, k_src, v_src):
+def fill_cache_from_sources(kv, lay, bt, ctx_lens, block_size, k_src, v_src, code_type=oracle.CODE_INT8):
     """Quantise per-sequence K/V sources ([ctx, Hkv, D] each) into the CPU cache with the oracle."""
     base = storage_bytes(kv)
     for i, slots in enumerate(slots_for(bt, ctx_lens, block_size)):
         if slots.numel() > 0:  # an empty sequence writes nothing
-            oracle.cache_write(k_src[i], v_src[i], base, lay, slots)
+            oracle.cache_write(k_src[i], v_src[i], base, lay, slots, code_type=code_type)
 
 
-def to_device_cache(kv_cpu, device, layout):
+def to_device_cache(kv_cpu, device, layout, code_type=oracle.CODE_INT8):
     """Same bytes, same layout, on the GPU; returns the logical-shape tensor."""
     nb, hkv, bs, content = kv_cpu.shape
-    kv = L.allocate_kv_cache(nb, bs, hkv, content // 2 - 4, device=device, layout=layout, fill=None)
+    d = (content // 2 - 4) * (2 if code_type == oracle.CODE_INT4 else 1)
+    kv = L.allocate_kv_cache(nb, bs, hkv, d, device=device, layout=layout, fill=None,
+                             cache_dtype_str=_dtype_str(code_type))
     storage_bytes(kv).copy_(storage_bytes(kv_cpu).to(device))
     return kv
 

@@ -265,3 +265,92 @@ def test_fp8_quant_rows_rule_and_closed_forms(dtype):
     assert torch.equal(deq[rows, idx][live].abs(), (scales * 448.0)[live])
     step = torch.maximum(deq.abs() / 16.0, scales[:, None] * 2.0 ** -10)   # half of 2^-3 relative / half the subnormal step
     assert bool(((deq - xf).abs() <= step * 1.0001 + 1e-30).all())
+
+
+# ---- int4 per-token-head codes (kvq_oracle_quant_rows_int4): the rule is this build's decision (the reference
+# states the record width only), so these pin the oracle against what the stated rule fixes, not against upstream
+
+def test_int4_closed_forms_and_nibble_order():
+    # a row whose absmax is 7 has scale 1: every integer in [-7, 7] is its own code; +-0.5 ties go to the even
+    # neighbour; values beyond the range clamp; dim 2 i sits in the low nibble of byte i
+    x = torch.tensor([[7.0, -7.0, 3.0, -3.0, 0.5, 1.5, 2.5, -0.5, -1.5, -2.5, 6.49, 6.51, 0.0, -6.5, 5.5, 1.0]])
+    codes, scales = oracle.quant_rows_int4(x)
+    assert scales.item() == 1.0
+    want = torch.tensor([7, -7, 3, -3, 0, 2, 2, 0, -2, -2, 6, 7, 0, -6, 6, 1], dtype=torch.int8)
+    assert torch.equal(oracle.unpack_int4(codes)[0], want)
+    assert codes[0, 0].item() == (7 | ((-7 & 15) << 4)) and codes[0, 7].item() == (6 | (1 << 4))
+    # -8 is reachable only through rounding past the symmetric range: the scale is absmax / 7, so it is not
+    x = torch.tensor([[-10.0, 10.0, 9.99, -9.99]])
+    codes, scales = oracle.quant_rows_int4(x)
+    assert torch.equal(oracle.unpack_int4(codes)[0], torch.tensor([-7, 7, 7, -7], dtype=torch.int8))
+    assert scales.item() == np.float32(10.0) / np.float32(7.0)
+
+
+def test_int4_zero_rows_and_floor():
+    z = torch.zeros((3, 64), dtype=torch.bfloat16)
+    codes, scales = oracle.quant_rows_int4(z)
+    assert torch.equal(codes, torch.zeros_like(codes))
+    assert torch.all(scales == np.float32(oracle.eps_for(torch.bfloat16)) / np.float32(7.0))
+    codes, scales = oracle.quant_rows_int4(torch.zeros((2, 64), dtype=torch.float16))   # 1e-10 underflows in fp16
+    assert torch.equal(codes, torch.zeros_like(codes)) and torch.all(scales == 0)
+
+
+def test_int4_bruteforce_exact_rational():
+    g = torch.Generator().manual_seed(4)
+    x = torch.randn((40, 32), generator=g, dtype=torch.float32)
+    x[:, 5] *= 9
+    codes, scales = oracle.quant_rows_int4(x)
+    vals = oracle.unpack_int4(codes)
+    for r in range(x.shape[0]):
+        amax = max(abs(float(v)) for v in x[r])
+        s32 = np.float32(amax) / np.float32(7.0)
+        assert scales[r].item() == s32
+        for d in range(x.shape[1]):
+            y = np.float32(np.float32(x[r, d].item()) / s32)          # the fp32 quotient the rule rounds
+            f = Fraction(float(y))
+            lo = f.numerator // f.denominator
+            frac = f - lo
+            k = lo + (1 if frac > Fraction(1, 2) or (frac == Fraction(1, 2) and lo % 2) else 0)
+            assert vals[r, d].item() == max(-8, min(7, k)), (r, d)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+def test_int4_matches_torch_round_div(dtype):
+    """The same rule in torch's CPU ops (a library routine's division and rounding)."""
+    x = _rand((64, 128), dtype, 11, "outlier")
+    codes, scales = oracle.quant_rows_int4(x)
+    xf = x.to(torch.float32)
+    amax = xf.abs().amax(-1).clamp(min=oracle.eps_for(dtype))
+    s = amax / 7.0
+    q = torch.clamp(torch.round(xf / s[:, None]), -8, 7).to(torch.int8)
+    assert torch.equal(scales, s) and torch.equal(oracle.unpack_int4(codes), q)
+
+
+def test_int4_cache_write_and_attention_read_the_same_nibbles():
+    """Write through the oracle, then attend: the result equals attention over code * scale computed in torch
+    from the unpacked bytes of the cache (pins the write's packing against the read's unpacking)."""
+    import kvq_testlib as T
+    hq, hkv, d, bs = 4, 2, 64, 16
+    ctx = [37, 5]
+    g = torch.Generator().manual_seed(3)
+    nb = 8
+    kv, (k, v, ks, vs), lay = T.cpu_cache(nb, bs, hkv, d, "NHD", code_type=oracle.CODE_INT4)
+    assert k.shape[-1] == d // 2 + 4 and lay.head_size == d
+    bt = T.make_block_tables(ctx, bs, nb, g)
+    srcs = [(torch.randn((c, hkv, d), generator=g), torch.randn((c, hkv, d), generator=g)) for c in ctx]
+    T.fill_cache_from_sources(kv, lay, bt, ctx, bs, [a for a, _ in srcs], [b for _, b in srcs], code_type=oracle.CODE_INT4)
+    q = torch.randn((2, hq, d), generator=g)
+    sl = torch.tensor(ctx, dtype=torch.int32)
+    cu = torch.arange(3, dtype=torch.int32)
+    got = oracle.paged_attn(q, T.storage_bytes(kv), lay, bt, sl, cu, 0.125, code_type=oracle.CODE_INT4)
+    for i, c in enumerate(ctx):
+        slots = T.slots_for(bt, ctx, bs)[i]
+        kc = oracle.unpack_int4(k.reshape(-1, hkv, d // 2 + 4)[slots][..., : d // 2].contiguous().view(torch.uint8))
+        vc = oracle.unpack_int4(v.reshape(-1, hkv, d // 2 + 4)[slots][..., : d // 2].contiguous().view(torch.uint8))
+        kd = kc.float() * ks.reshape(-1, hkv)[slots][..., None]
+        vd = vc.float() * vs.reshape(-1, hkv)[slots][..., None]
+        # the written codes are the quantiser's
+        wc, wscale = oracle.quant_rows_int4(srcs[i][0])
+        assert torch.equal(oracle.unpack_int4(wc), kc) and torch.equal(wscale, ks.reshape(-1, hkv)[slots])
+        want = torch_ref.sdpa_gathered(q[i:i + 1], kd, vd, 0.125)
+        torch.testing.assert_close(got[i:i + 1], want, atol=1e-5, rtol=1e-5)

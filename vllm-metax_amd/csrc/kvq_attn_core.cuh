@@ -83,6 +83,27 @@ __device__ __forceinline__ half8_t dequant8(uint32_t lo, uint32_t hi) {
   return __builtin_bit_cast(half8_t, r);
 }
 
+// int4 codes: a nibble n = code ^ 8 (0 .. 15) enters the MFMA as the fp16 number 0x6400 | n = code + 1032, exact;
+// the constant is taken out afterwards like the int8 path's 1152.  One and-or per two nibbles: with y = the dword
+// of four code bytes ^ 0x88888888, ((y >> 4 k) & 0x000f000f) | 0x64006400 holds nibbles k and k + 4 of the dword,
+// so the eight dims of a dword come out in the order 0 4 1 5 2 6 3 7 -- the order in which the query operand of an
+// int4 tile is laid out as well (nibble_order).
+constexpr float kCodeBiasInt4 = 1032.0f;
+__device__ __forceinline__ uint32_t nibbles_to_half2(uint32_t y, int k) {
+  return ((y >> (4 * k)) & 0x000f000fu) | 0x64006400u;
+}
+__device__ __forceinline__ half8_t dequant8_int4(uint32_t x) {
+  const uint32_t y = x ^ 0x88888888u;
+  u32x4 r;
+  r.x = nibbles_to_half2(y, 0);
+  r.y = nibbles_to_half2(y, 1);
+  r.z = nibbles_to_half2(y, 2);
+  r.w = nibbles_to_half2(y, 3);
+  return __builtin_bit_cast(half8_t, r);
+}
+// MFMA k position j of an int4 operand holds dim nibble_order(j) of the dword's eight.
+__host__ __device__ constexpr int nibble_order(int j) { return (j >> 1) + 4 * (j & 1); }
+
 __device__ __forceinline__ uint32_t pack_half2(float a, float b) {
   half2_t v = {(half_t)a, (half_t)b};
   return __builtin_bit_cast(uint32_t, v);
@@ -217,15 +238,20 @@ struct LaneOffsets {
 template <int D, int QDT, int ODT, int CODE = KVQ_CODE_INT8>
 struct DecodeTile {
   static constexpr bool FP8 = CODE == KVQ_CODE_FP8_E4M3;
+  // int4 codes: a record of head size D has the bytes of an int8 record of head size D / 2, so the tile is loaded
+  // and staged as that one; only the operand conversions and the query's dim order differ
+  static constexpr bool INT4 = CODE == KVQ_CODE_INT4;
+  static constexpr int DB = INT4 ? D / 2 : D;                 // code bytes of a half record
+  static constexpr float kBias = INT4 ? kCodeBiasInt4 : kCodeBias;
   static constexpr float kKScaleMul = FP8 ? 256.0f : 1.0f;   // on top of scale * log2(e)
   static constexpr float kOutDiv = FP8 ? 1.0f : kPScale;      // what the accumulated output still carries
   static constexpr int KSTEPS = D / 32;
   static constexpr int DT = D / 16;
-  static constexpr int VB = D / 16;  // V bytes per token per lane
-  using Tile = KVTile<D>;
+  static constexpr int VB = DB / 16;  // V bytes per token per lane
+  using Tile = KVTile<DB>;
   using State = DecodeState<D>;
 
-  static constexpr int R = 2 * (D + 4);      // record bytes
+  static constexpr int R = 2 * (DB + 4);     // record bytes
   static constexpr int PITCH = R + 8;        // LDS row pitch: 16-byte aligned rows, conflict-free operand reads
   static constexpr int NCH = Tile::NCH;
   static constexpr int NLD = Tile::NLD;
@@ -237,12 +263,12 @@ struct DecodeTile {
     const int r = lane & 15, g = lane >> 4;
     LaneOffsets o;
     o.g_chunk = (uint32_t)((lane / NCH) * G.stride_slot + 16 * (lane % NCH));
-    o.g_tail = (uint32_t)((lane & 15) * G.stride_slot + 2 * D);
+    o.g_tail = (uint32_t)((lane & 15) * G.stride_slot + 2 * DB);
     o.l_chunk = (uint32_t)((lane / NCH) * PITCH + 16 * (lane % NCH));
-    o.l_tail = (uint32_t)((lane & 31) * PITCH + 2 * D);
-    o.l_k = (uint32_t)(r * PITCH + g * 16);
-    o.l_v = (uint32_t)(4 * g * PITCH + (D + 4) + r * VB);
-    o.l_sc = (uint32_t)((lane & 31) * PITCH + (lane < 32 ? D : 2 * D + 4));
+    o.l_tail = (uint32_t)((lane & 31) * PITCH + 2 * DB);
+    o.l_k = (uint32_t)(r * PITCH + (INT4 ? g * (DB / 4) : g * 16));   // int4: the lane's D / 4 dims are DB / 4 bytes in a row
+    o.l_v = (uint32_t)(4 * g * PITCH + (DB + 4) + r * VB);
+    o.l_sc = (uint32_t)((lane & 31) * PITCH + (lane < 32 ? DB : 2 * DB + 4));
     o.g_flat = (uint32_t)(16 * lane);
     o.l_flat_split = 0;
 #pragma unroll
@@ -271,19 +297,22 @@ struct DecodeTile {
   // query row (it must be readable also when !valid; the operand is then zero).
   __device__ static float load_q_row(const AttnIO& io, int64_t elem, bool valid, int lane, half8_t (&qb)[KSTEPS]) {
     const int g = lane >> 4;
-    const int64_t base = elem + g * 16;
+    // int8 / fp8: 16 dims of every 64-dim chunk; int4: the D / 4 dims from g D / 4 on, in a row (the same loads,
+    // chunk `ch` then standing for the ch-th run of 16 of them)
+    constexpr int kChunkStep = INT4 ? 16 : 64;
+    const int64_t base = elem + (INT4 ? g * (D / 4) : g * 16);
     float f[D / 4];
 #pragma unroll
     for (int ch = 0; ch < D / 64; ++ch) {
       if constexpr (QDT == KVQ_F32) {
-        const float* p = reinterpret_cast<const float*>(io.q) + base + ch * 64;
+        const float* p = reinterpret_cast<const float*>(io.q) + base + ch * kChunkStep;
 #pragma unroll
         for (int i = 0; i < 16; i += 4) {
           const floatx4 v = *reinterpret_cast<const floatx4_a4*>(p + i);
           f[ch * 16 + i] = v.x; f[ch * 16 + i + 1] = v.y; f[ch * 16 + i + 2] = v.z; f[ch * 16 + i + 3] = v.w;
         }
       } else {
-        const uint16_t* p = reinterpret_cast<const uint16_t*>(io.q) + base + ch * 64;
+        const uint16_t* p = reinterpret_cast<const uint16_t*>(io.q) + base + ch * kChunkStep;
 #pragma unroll
         for (int i = 0; i < 16; i += 8) {
           const u32x4 v = *reinterpret_cast<const u32x4_a4*>(p + i);
@@ -306,12 +335,19 @@ struct DecodeTile {
     const uint32_t okmask = valid ? 0xffffffffu : 0u;  // a mask, not a select: no branches around the converts
 #pragma unroll
     for (int kk = 0; kk < KSTEPS; ++kk) {
-      const int b = (kk >> 1) * 16 + (kk & 1) * 8;
+      const int b = INT4 ? kk * 8 : (kk >> 1) * 16 + (kk & 1) * 8;
       u32x4 hb;
+      if constexpr (INT4) {   // the k positions follow the nibble conversion's dim order
+        hb.x = pack_half2(clamp_half_range(f[b + nibble_order(0)]), clamp_half_range(f[b + nibble_order(1)])) & okmask;
+        hb.y = pack_half2(clamp_half_range(f[b + nibble_order(2)]), clamp_half_range(f[b + nibble_order(3)])) & okmask;
+        hb.z = pack_half2(clamp_half_range(f[b + nibble_order(4)]), clamp_half_range(f[b + nibble_order(5)])) & okmask;
+        hb.w = pack_half2(clamp_half_range(f[b + nibble_order(6)]), clamp_half_range(f[b + nibble_order(7)])) & okmask;
+      } else {
       hb.x = pack_half2(clamp_half_range(f[b + 0]), clamp_half_range(f[b + 1])) & okmask;
       hb.y = pack_half2(clamp_half_range(f[b + 2]), clamp_half_range(f[b + 3])) & okmask;
       hb.z = pack_half2(clamp_half_range(f[b + 4]), clamp_half_range(f[b + 5])) & okmask;
       hb.w = pack_half2(clamp_half_range(f[b + 6]), clamp_half_range(f[b + 7])) & okmask;
+      }
       const half8_t h = __builtin_bit_cast(half8_t, hb);
 #pragma unroll
       for (int j = 0; j < 8; ++j) qsum += (float)h[j];  // the sum of what the MFMA will actually see
@@ -319,7 +355,49 @@ struct DecodeTile {
     }
     qsum += __shfl_xor(qsum, 16, kWave);
     qsum += __shfl_xor(qsum, 32, kWave);
-    return FP8 ? 0.f : -kCodeBias * qsum;
+    return FP8 ? 0.f : -kBias * qsum;
+  }
+
+  // The KSTEPS operands of K tokens (M-tile mt) of the lane, int4 codes: DB / 4 bytes in a row, a dword per k-step.
+  __device__ static void k_operands_int4(const LaneOffsets& lo, int mt, const uint8_t* lds, half8_t (&ka)[KSTEPS]) {
+    const uint8_t* p = lds + lo.l_k + mt * 16 * PITCH;
+    if constexpr (KSTEPS == 2) {
+      const u32x2 w = *reinterpret_cast<const u32x2*>(p);
+      ka[0] = dequant8_int4(w.x);
+      ka[1] = dequant8_int4(w.y);
+    } else {
+#pragma unroll
+      for (int i = 0; i < KSTEPS / 4; ++i) {
+        const u32x4 w = *reinterpret_cast<const u32x4*>(p + 16 * i);
+        ka[4 * i] = dequant8_int4(w.x);
+        ka[4 * i + 1] = dequant8_int4(w.y);
+        ka[4 * i + 2] = dequant8_int4(w.z);
+        ka[4 * i + 3] = dequant8_int4(w.w);
+      }
+    }
+  }
+
+  // The V^T operands of the lane's 8 tokens for the four 16-dim tiles that two code bytes hold (unit u = bytes
+  // 2 u, 2 u + 1 of the lane's VB: dims 4 u .. 4 u + 3 of its 2 VB, tile 4 u + n = nibble n), int4 codes.
+  __device__ static void v_operands_int4(const LaneOffsets& lo, int u, const uint8_t* lds, half8_t (&va)[4]) {
+    uint32_t y[4];
+#pragma unroll
+    for (int a = 0; a < 4; ++a) {
+      const int ja = 2 * a, jb = 2 * a + 1;
+      const uint8_t* pa = lds + lo.l_v + ((ja & 3) + (ja >> 2) * 16) * PITCH + 2 * u;
+      const uint8_t* pb = lds + lo.l_v + ((jb & 3) + (jb >> 2) * 16) * PITCH + 2 * u;
+      const uint32_t ta = *reinterpret_cast<const uint16_t*>(pa), tb = *reinterpret_cast<const uint16_t*>(pb);
+      y[a] = (ta | (tb << 16)) ^ 0x88888888u;   // token ja's two bytes below token jb's
+    }
+#pragma unroll
+    for (int n = 0; n < 4; ++n) {
+      u32x4 av;
+      av.x = nibbles_to_half2(y[0], n);
+      av.y = nibbles_to_half2(y[1], n);
+      av.z = nibbles_to_half2(y[2], n);
+      av.w = nibbles_to_half2(y[3], n);
+      va[n] = __builtin_bit_cast(half8_t, av);
+    }
   }
 
   // Token index -> block-table entry / slot, by multiplication (scalar ALU, no divide).
@@ -468,11 +546,18 @@ struct DecodeTile {
 #pragma unroll
     for (int mt = 0; mt < 2; ++mt) {
       s[mt] = (floatx4){s_init, s_init, s_init, s_init};
+      if constexpr (INT4) {
+        half8_t ka[KSTEPS];
+        k_operands_int4(lo, mt, lds, ka);
+#pragma unroll
+        for (int kk = 0; kk < KSTEPS; ++kk) s[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka[kk], qb[kk], s[mt], 0, 0, 0);
+      } else {
 #pragma unroll
       for (int i = 0; i < KSTEPS / 2; ++i) {
         const u32x4 w = *reinterpret_cast<const u32x4*>(lds + lo.l_k + mt * 16 * PITCH + i * 64);
         s[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(dequant8<FP8>(w.x, w.y), qb[2 * i], s[mt], 0, 0, 0);
         s[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(dequant8<FP8>(w.z, w.w), qb[2 * i + 1], s[mt], 0, 0, 0);
+      }
       }
     }
 
@@ -533,6 +618,17 @@ struct DecodeTile {
       const half_t one = (half_t)1.0f;
       const half8_t ones = {one, one, one, one, one, one, one, one};
       st.psum = __builtin_amdgcn_mfma_f32_16x16x32_f16(ones, p_op, st.psum, 0, 0, 0);
+    }
+    if constexpr (INT4) {
+#pragma unroll
+      for (int u = 0; u < VB / 2; ++u) {
+        half8_t va[4];
+        v_operands_int4(lo, u, lds, va);
+#pragma unroll
+        for (int n = 0; n < 4; ++n)
+          st.o[4 * u + n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va[n], p_op, st.o[4 * u + n], 0, 0, 0);
+      }
+      return;
     }
     constexpr int VW = VB / 4;
 #pragma unroll
@@ -698,14 +794,14 @@ struct DecodeTile {
     return l;
   }
 
-  // Lane (c, g) holds O[head c][dim (4g+i)*VB + dt], i = 0..3, dt = 0..DT-1: D/4 contiguous
+  // Lane (c, g) holds O[head c][dim (4g+i)*DT + dt], i = 0..3, dt = 0..DT-1: D/4 contiguous
   // dims starting at g*D/4.  Gather them in order, code bias removed, scaled by `mul`.
   __device__ static void gather_row(const State& st, float mul, float (&v)[D / 4]) {
-    const float corr = FP8 ? 0.f : kCodeBias * st.psum[0];
+    const float corr = FP8 ? 0.f : kBias * st.psum[0];
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
-      for (int dt = 0; dt < DT; ++dt) v[i * VB + dt] = (st.o[dt][i] - corr) * mul;
+      for (int dt = 0; dt < DT; ++dt) v[i * DT + dt] = (st.o[dt][i] - corr) * mul;
   }
 
   // Whole sequence handled by this wave: normalise and write the output row (and lse).
@@ -835,14 +931,15 @@ __device__ __forceinline__ void write_new_token(const StreamKArgs& a, int seq, i
   load_row8(src, a.new_dtype, elem, x);
   uint32_t pk[2];
   float scale;
-  quant_row8<LPR>(x, a.new_eps, g.code_type == KVQ_CODE_FP8_E4M3, pk, scale);
+  quant_row8<LPR>(x, a.new_eps, g.code_type, pk, scale);
   const int pos = len - 1;
   const int e = (int)__umulhi((uint32_t)pos, a.io.bs_magic);
   const int off = pos - e * g.block_size;
   const int64_t blk = a.io.block_table[(int64_t)seq * a.io.bt_stride + e];
   uint8_t* rec = const_cast<uint8_t*>(a.io.cache) + blk * g.stride_block + (int64_t)off * g.stride_slot + (int64_t)hkv * g.stride_head;
   if (lane < 2 * LPR) {
-    *reinterpret_cast<u32x2_a4*>(rec + (is_v ? g.v_off : g.k_off) + li * 8) = (u32x2){pk[0], pk[1]};
+    if (g.code_type == KVQ_CODE_INT4) *reinterpret_cast<uint32_t*>(rec + (is_v ? g.v_off : g.k_off) + li * 4) = pk[0];
+    else *reinterpret_cast<u32x2_a4*>(rec + (is_v ? g.v_off : g.k_off) + li * 8) = (u32x2){pk[0], pk[1]};
     if (li == 0) *reinterpret_cast<float*>(rec + (is_v ? g.vs_off : g.ks_off)) = scale;
   }
 }

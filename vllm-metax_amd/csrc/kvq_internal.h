@@ -139,25 +139,37 @@ __device__ __forceinline__ float sum_over_quarters(float v) {
 // Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits for every global
 // load in flight (vmcnt(0)), which would drain the tile prefetch issued just before it; here the
 // loads stay in flight and the compiler's own wait before their first use still applies.
+// Code bytes of one half (K or V) of a record.
+__host__ __device__ inline int code_bytes(const kvq_cache_geom& g) {
+  return g.code_type == KVQ_CODE_INT4 ? g.head_size / 2 : g.head_size;
+}
+
 // One cache row's quantisation with 8 elements per lane and LPR lanes per row (every lane of the wave takes
-// part in the shuffles): scale = max(amax, eps) / 127 (448 for fp8 codes), code = rint(x / scale) clamped.
+// part in the shuffles): scale = max(amax, eps) / 127 (448 for fp8 codes, 7 for int4), code = rint(x / scale)
+// clamped.  int8 / fp8: the lane's 8 code bytes in pk[0], pk[1]; int4: its 8 nibbles in pk[0] (element i in
+// bits 4 i .. 4 i + 3: an even dim in the low nibble of its byte).
 // Shared by the write kernel and by the decode kernel's fused write, so that both store the same bytes.
 template <int LPR>
-__device__ __forceinline__ void quant_row8(const float (&x)[8], float eps, bool fp8, uint32_t (&pk)[2], float& scale) {
+__device__ __forceinline__ void quant_row8(const float (&x)[8], float eps, int code_type, uint32_t (&pk)[2], float& scale) {
   float amax = 0.f;
 #pragma unroll
   for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf(x[i]));
 #pragma unroll
   for (int o = LPR / 2; o >= 1; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o, kWave));
   amax = fmaxf(amax, eps);  // eps may be 0 for fp16 sources (1e-10 underflows)
-  scale = fp8 ? amax / 448.0f : amax / 127.0f;
+  scale = code_type == KVQ_CODE_FP8_E4M3 ? amax / 448.0f : (code_type == KVQ_CODE_INT4 ? amax / 7.0f : amax / 127.0f);
   pk[0] = 0u;
   pk[1] = 0u;
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
     const float y = scale > 0.f ? x[i] / scale : 0.f;  // scale == 0: all-zero fp16 row
+    if (code_type == KVQ_CODE_INT4) {
+      const float r = fminf(fmaxf(rintf(y), -8.f), 7.f);
+      pk[0] |= ((uint32_t)(int)r & 0xfu) << (4 * i);
+      continue;
+    }
     uint32_t code;
-    if (fp8) {
+    if (code_type == KVQ_CODE_FP8_E4M3) {
       code = f32_to_e4m3fn_bits(y);
     } else {
       const float r = fminf(fmaxf(rintf(y), -128.f), 127.f);

@@ -91,16 +91,16 @@ int validate_common(const char* op, const void* q, const void* cache, const kvq_
   KVQ_REQUIRE((g.k_off | g.v_off | g.ks_off | g.vs_off | g.stride_block | g.stride_slot | g.stride_head) % 4 == 0 &&
                   ((uintptr_t)cache % 4) == 0,
               "%s: cache offsets/strides must be 4-byte aligned", op);
-  KVQ_REQUIRE(g.ks_off - g.k_off == g.head_size && g.v_off - g.k_off == g.head_size + 4 &&
-                  g.vs_off - g.k_off == 2 * g.head_size + 4,
+  KVQ_REQUIRE(g.code_type == KVQ_CODE_INT8 || g.code_type == KVQ_CODE_FP8_E4M3 || g.code_type == KVQ_CODE_INT4,
+              "%s: unknown code_type %d", op, g.code_type);
+  const int cb = code_bytes(g);
+  KVQ_REQUIRE(g.ks_off - g.k_off == cb && g.v_off - g.k_off == cb + 4 && g.vs_off - g.k_off == 2 * cb + 4,
               "%s: a cache record must be [K codes | K scale | V codes | V scale]", op);
   KVQ_REQUIRE(g.stride_slot > 0 && g.stride_slot <= 0x7fffffff / 64, "%s: stride_slot out of range", op);
   // the kernels multiply block numbers and slots by these as 32-bit numbers
   KVQ_REQUIRE(g.stride_block > 0 && g.stride_block <= 0x7fffffff && g.stride_head >= 0 && g.stride_head <= 0x7fffffff &&
                   (int64_t)g.block_size * g.stride_slot <= 0x7fffffff,
               "%s: a cache block of 2 GiB or more is not supported", op);
-  KVQ_REQUIRE(g.code_type == KVQ_CODE_INT8 || g.code_type == KVQ_CODE_FP8_E4M3, "%s: unknown code_type %d", op,
-              g.code_type);
   return KVQ_OK;
 }
 

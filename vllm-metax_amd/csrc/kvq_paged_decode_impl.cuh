@@ -791,27 +791,24 @@ static int launch_streamk(const StreamKArgs& a, hipStream_t s) {
   const int hkv = a.io.g.num_kv_heads;
   const int hpw = heads_per_wg(hkv);
   dim3 grid(a.num_wg, (hkv + hpw - 1) / hpw);
+#define KVQ_SK_CODE(H, C, CODE)                                                                                   \
+  do {                                                                                                            \
+    if (a.fixed_spans)                                                                                            \
+      hipLaunchKernelGGL((paged_decode_streamk_kernel<D, QDT, H, C, CODE, false, true>), grid, dim3(512), 0, s, a); \
+    else if (!C && stream)                                                                                        \
+      hipLaunchKernelGGL((paged_decode_streamk_kernel<D, QDT, H, false, CODE, true>), grid, dim3(512), 0, s, a);  \
+    else                                                                                                          \
+      hipLaunchKernelGGL((paged_decode_streamk_kernel<D, QDT, H, C, CODE, false>), grid, dim3(512), 0, s, a);     \
+  } while (0)
 #define KVQ_SK(H, C)                                                                                              \
   do {                                                                                                            \
-    if (a.fixed_spans) {                                                                                          \
-      if (a.io.g.code_type == KVQ_CODE_FP8_E4M3)                                                                  \
-        hipLaunchKernelGGL((paged_decode_streamk_kernel<D, QDT, H, C, KVQ_CODE_FP8_E4M3, false, true>), grid, dim3(512), 0, s, a); \
-      else                                                                                                        \
-        hipLaunchKernelGGL((paged_decode_streamk_kernel<D, QDT, H, C, KVQ_CODE_INT8, false, true>), grid, dim3(512), 0, s, a); \
-    } else if (a.io.g.code_type == KVQ_CODE_FP8_E4M3) {                                                           \
-      if (!C && stream)                                                                                           \
-        hipLaunchKernelGGL((paged_decode_streamk_kernel<D, QDT, H, false, KVQ_CODE_FP8_E4M3, true>), grid, dim3(512), 0, s, a); \
-      else                                                                                                        \
-        hipLaunchKernelGGL((paged_decode_streamk_kernel<D, QDT, H, C, KVQ_CODE_FP8_E4M3, false>), grid, dim3(512), 0, s, a); \
-    } else if (!C && stream) {                                                                                    \
-      hipLaunchKernelGGL((paged_decode_streamk_kernel<D, QDT, H, false, KVQ_CODE_INT8, true>), grid, dim3(512), 0, s, a); \
-    } else {                                                                                                      \
-      hipLaunchKernelGGL((paged_decode_streamk_kernel<D, QDT, H, C, KVQ_CODE_INT8, false>), grid, dim3(512), 0, s, a); \
-    }                                                                                                             \
+    if (a.io.g.code_type == KVQ_CODE_FP8_E4M3) KVQ_SK_CODE(H, C, KVQ_CODE_FP8_E4M3);                              \
+    else if (a.io.g.code_type == KVQ_CODE_INT4) KVQ_SK_CODE(H, C, KVQ_CODE_INT4);                                 \
+    else KVQ_SK_CODE(H, C, KVQ_CODE_INT8);                                                                        \
   } while (0)
   // a head's records of a block back to back (HND order): the tile loads may stream past the caches
   // (not at head size 256, where it measured slower: 293 against 279 us on 64 x 1k-8k tokens)
-  const bool stream = D <= 128 && a.io.g.stride_slot == 2 * (D + 4) && a.io.g.block_size >= 16;
+  const bool stream = D <= 128 && a.io.g.stride_slot == 2 * (code_bytes(a.io.g) + 4) && a.io.g.block_size >= 16;
   if (a.io.cap_c != 0.f) {
     switch (hpw) {
       case 8: KVQ_SK(8, true); break;
@@ -828,6 +825,7 @@ static int launch_streamk(const StreamKArgs& a, hipStream_t s) {
     }
   }
 #undef KVQ_SK
+#undef KVQ_SK_CODE
   int rc = check_hip(hipGetLastError(), "paged_attn_int8 decode launch");
   if (rc) return rc;
   if (a.fixed_spans) {

@@ -61,6 +61,7 @@ template <int D, int QDT, int ODT, int NT, int CODE = KVQ_CODE_INT8>
 struct PrefillTile {
   using DTile = DecodeTile<D, QDT, ODT, CODE>;
   static constexpr bool FP8 = DTile::FP8;
+  static constexpr bool INT4 = DTile::INT4;
   static constexpr int KSTEPS = DTile::KSTEPS;
   static constexpr int DT = DTile::DT;
   static constexpr int VB = DTile::VB;
@@ -89,6 +90,15 @@ struct PrefillTile {
     }
 #pragma unroll
     for (int mt = 0; mt < 2; ++mt) {
+      if constexpr (INT4) {
+        half8_t ka[KSTEPS];
+        DTile::k_operands_int4(lo, mt, lds, ka);
+#pragma unroll
+        for (int kk = 0; kk < KSTEPS; ++kk)
+#pragma unroll
+          for (int nt = 0; nt < NT; ++nt)
+            s[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka[kk], qb[nt][kk], s[nt][mt], 0, 0, 0);
+      } else {
 #pragma unroll
       for (int i = 0; i < KSTEPS / 2; ++i) {
         const u32x4 w = *reinterpret_cast<const u32x4*>(lds + lo.l_k + mt * 16 * PITCH + i * 64);
@@ -98,6 +108,7 @@ struct PrefillTile {
           s[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a0, qb[nt][2 * i], s[nt][mt], 0, 0, 0);
           s[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a1, qb[nt][2 * i + 1], s[nt][mt], 0, 0, 0);
         }
+      }
       }
     }
     const floatx4 ks0 = *reinterpret_cast<const floatx4*>(sc_lds + 4 * g);
@@ -173,6 +184,19 @@ struct PrefillTile {
       for (int nt = 0; nt < NT; ++nt)
         st.psum[nt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ones, p_op[nt], st.psum[nt], 0, 0, 0);
     }
+    if constexpr (INT4) {
+#pragma unroll
+      for (int u = 0; u < VB / 2; ++u) {
+        half8_t va[4];
+        DTile::v_operands_int4(lo, u, lds, va);
+#pragma unroll
+        for (int n = 0; n < 4; ++n)
+#pragma unroll
+          for (int nt = 0; nt < NT; ++nt)
+            st.o[nt][4 * u + n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va[n], p_op[nt], st.o[nt][4 * u + n], 0, 0, 0);
+      }
+      return;
+    }
 #pragma unroll
     for (int w = 0; w < VB / 4; ++w) {
       uint32_t x0[4], x1[4];
@@ -209,12 +233,12 @@ struct PrefillTile {
     if (!valid) return;
     const int g = lane >> 4;
     const float mul = l > 0.f ? 1.0f / (l * DTile::kOutDiv) : 0.f;   // no visible key: zeros
-    const float corr = FP8 ? 0.f : kCodeBias * st.psum[nt][0];
+    const float corr = FP8 ? 0.f : DTile::kBias * st.psum[nt][0];
     float v[D / 4];
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
-      for (int dt = 0; dt < DT; ++dt) v[i * VB + dt] = (st.o[nt][dt][i] - corr) * mul;
+      for (int dt = 0; dt < DT; ++dt) v[i * DT + dt] = (st.o[nt][dt][i] - corr) * mul;
     const int64_t base = row * io.out_stride_t + (int64_t)head * io.out_stride_h + g * (D / 4);
     if constexpr (ODT == KVQ_F32) {
       float* o = reinterpret_cast<float*>(io.out) + base;
@@ -838,7 +862,11 @@ template <int D, int QDT, int ODT>
 static int launch_prefill_nt(PrefillArgs& a, int max_query_len, hipStream_t s) {
   constexpr int WPW = 4;
   const bool fp8 = a.io.g.code_type == KVQ_CODE_FP8_E4M3;
-  // long runs: the workgroup-shared fp16 tile (compute-bound shape), for either kind of code
+  if (a.io.g.code_type == KVQ_CODE_INT4) {   // int4 codes: the per-wave tile for runs of any length
+    a.q_tokens = 16 / a.io.group;
+    return launch_prefill_cfg<D, QDT, ODT, 1, WPW, KVQ_CODE_INT4>(a, max_query_len, s);
+  }
+  // long runs: the workgroup-shared fp16 tile (compute-bound shape), for either kind of one-byte code
   if constexpr (D <= 128) {
     if (max_query_len * a.io.group >= 64) {
       const bool ext = a.io.window > 0 || a.io.cap_c != 0.f;

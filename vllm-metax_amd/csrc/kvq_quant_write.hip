@@ -5,7 +5,8 @@
 // fp32 scale go straight into the (block, slot, head) record.  The arithmetic is
 // the bit-exact contract: scale = max(absmax, eps) / 127 (IEEE fp32 division),
 // code = clamp(rint(x / scale), -128, 127) with round-half-to-even.  A cache whose geometry says
-// KVQ_CODE_FP8_E4M3 gets scale = max(absmax, eps) / 448 and the nearest e4m3fn code instead.
+// KVQ_CODE_FP8_E4M3 gets scale = max(absmax, eps) / 448 and the nearest e4m3fn code instead; KVQ_CODE_INT4
+// scale = max(absmax, eps) / 7 and 4-bit codes in [-8, 7], two per byte (the even dim in the low nibble).
 #include "kvq_internal.h"
 
 namespace kvq {
@@ -92,6 +93,20 @@ __global__ __launch_bounds__(256) void quant_write_kernel(
     for (int d = lane; d < D; d += kWave) amax = fmaxf(amax, fabsf(load_act<DT>(src, src_base + d)));
     amax = fmaxf(wave_max(amax), eps);  // eps may be 0 for fp16 sources (1e-10 underflows)
     const bool fp8 = g.code_type == KVQ_CODE_FP8_E4M3;
+    if (g.code_type == KVQ_CODE_INT4) {   // a byte per two dims: the even one in the low nibble
+      const float scale = amax / 7.0f;
+      for (int b = lane; b < D / 2; b += kWave) {
+        uint32_t byte = 0;
+        for (int j = 0; j < 2; ++j) {
+          const float y = scale > 0.f ? load_act<DT>(src, src_base + 2 * b + j) / scale : 0.f;
+          const float r = fminf(fmaxf(rintf(y), -8.f), 7.f);
+          byte |= ((uint32_t)(int)r & 0xfu) << (4 * j);
+        }
+        codes[b] = (int8_t)byte;
+      }
+      if (lane == 0) *scale_ptr = scale;
+      return;
+    }
     const float scale = fp8 ? amax / 448.0f : amax / 127.0f;
     for (int d = lane; d < D; d += kWave) {
       const float y = scale > 0.f ? load_act<DT>(src, src_base + d) / scale : 0.f;
@@ -160,7 +175,7 @@ __global__ __launch_bounds__(256) void quant_write_rows_kernel(
   }
   uint32_t pk[2];
   float scale;
-  quant_row8<LPR>(x, eps, g.code_type == KVQ_CODE_FP8_E4M3, pk, scale);
+  quant_row8<LPR>(x, eps, g.code_type, pk, scale);
   if (!live || slot < 0) return;  // padding token (after the shuffles: every lane took part)
   int64_t blk, off;
   if ((uint64_t)slot <= 0xffffffffull) {
@@ -172,7 +187,8 @@ __global__ __launch_bounds__(256) void quant_write_rows_kernel(
     off = slot - blk * g.block_size;
   }
   uint8_t* rec = cache + blk * g.stride_block + off * g.stride_slot + (int64_t)h * g.stride_head;
-  *reinterpret_cast<u32x2_a4*>(rec + (is_v ? g.v_off : g.k_off) + li * 8) = (u32x2){pk[0], pk[1]};
+  if (g.code_type == KVQ_CODE_INT4) *reinterpret_cast<uint32_t*>(rec + (is_v ? g.v_off : g.k_off) + li * 4) = pk[0];
+  else *reinterpret_cast<u32x2_a4*>(rec + (is_v ? g.v_off : g.k_off) + li * 8) = (u32x2){pk[0], pk[1]};
   if (li == 0) *reinterpret_cast<float*>(rec + (is_v ? g.vs_off : g.ks_off)) = scale;
 }
 
@@ -208,7 +224,7 @@ static int launch_quant_write(const void* key, const void* value, int64_t kst, i
 #define KVQ_LAUNCH(V)                                                                     \
   hipLaunchKernelGGL((quant_write_kernel<DT, V>), grid, block, 0, s, key, value, kst, ksh, \
                      vst, vsh, cache, g, slot_mapping, rows, eps)
-  switch (g.head_size) {
+  switch (g.code_type == KVQ_CODE_INT4 ? 0 : g.head_size) {   // nibbles: the any-size loop packs two dims per lane
     case 64: KVQ_LAUNCH(1); break;
     case 128: KVQ_LAUNCH(2); break;
     case 256: KVQ_LAUNCH(4); break;
@@ -241,7 +257,7 @@ extern "C" int kvq_reshape_and_cache_int8(const void* key, const void* value, in
                g.stride_head) % 4 == 0 && ((uintptr_t)cache % 4) == 0,
               "reshape_and_cache_int8: cache offsets/strides must be 4-byte aligned");
   KVQ_REQUIRE(eps >= 0.f, "reshape_and_cache_int8: eps must not be negative");
-  KVQ_REQUIRE(g.code_type == KVQ_CODE_INT8 || g.code_type == KVQ_CODE_FP8_E4M3,
+  KVQ_REQUIRE(g.code_type == KVQ_CODE_INT8 || g.code_type == KVQ_CODE_FP8_E4M3 || g.code_type == KVQ_CODE_INT4,
               "reshape_and_cache_int8: unknown code_type %d", g.code_type);
   hipStream_t s = as_stream(stream);
   uint8_t* c = static_cast<uint8_t*>(cache);

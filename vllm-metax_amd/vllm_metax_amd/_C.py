@@ -13,8 +13,8 @@ _LIB_DIR = os.path.join(os.path.dirname(os.path.abspath(__file__)), "_lib")
 LIB_PATH = os.path.join(_LIB_DIR, "libkvq_hip.so")
 
 KVQ_F32, KVQ_BF16, KVQ_F16 = 0, 1, 2
-KVQ_CODE_INT8, KVQ_CODE_FP8_E4M3 = 0, 1
-ABI_VERSION = 13
+KVQ_CODE_INT8, KVQ_CODE_FP8_E4M3, KVQ_CODE_INT4 = 0, 1, 2
+ABI_VERSION = 14
 
 
 class CacheGeom(ctypes.Structure):

@@ -58,6 +58,9 @@ except Exception:  # noqa: BLE001
 INT8_PER_TOKEN_HEAD = "int8_per_token_head"
 # the fp8 mode of the same inline-scale record layout (vllm_metax/v1/attention/backends/triton_attn.py:336-348)
 FP8_PER_TOKEN_HEAD = "fp8_per_token_head"
+# the int4 mode of the same layout: two codes per byte, head_size / 2 code bytes + the scale per half
+# (vllm_metax/v1/attention/backends/triton_attn.py:332-346)
+INT4_PER_TOKEN_HEAD = "int4_per_token_head"
 # MLA latent cache with one fp32 scale per token (this build's addition; the
 # reference's MLA backends stop at fp8, vllm_metax/v1/attention/backends/mla/triton_mla.py:94-100).
 INT8_PER_TOKEN = "int8_per_token"

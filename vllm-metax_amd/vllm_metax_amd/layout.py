@@ -26,6 +26,7 @@ import torch
 from . import _C
 from .kv_cache_interface import (
     FP8_PER_TOKEN_HEAD,
+    INT4_PER_TOKEN_HEAD,
     INT8_PER_TOKEN,
     INT8_PER_TOKEN_HEAD,
     KVQuantMode,
@@ -80,11 +81,15 @@ def kv_cache_shape(num_blocks: int, block_size: int, num_kv_heads: int, head_siz
     if block_size % 16 != 0:
         raise ValueError("Block size must be a multiple of 16.")
     if kv_cache_uses_per_token_head_scales(cache_dtype_str):
-        if cache_dtype_str not in (INT8_PER_TOKEN_HEAD, FP8_PER_TOKEN_HEAD):
-            raise NotImplementedError(f"kv cache dtype {cache_dtype_str!r}: only {INT8_PER_TOKEN_HEAD!r} and "
-                                      f"{FP8_PER_TOKEN_HEAD!r} are built (one-byte elements)")
-        scale_pad = SCALE_BYTES // torch.int8.itemsize   # fp8 elements are one byte as well
-        return (num_blocks, num_kv_heads, block_size, 2 * (head_size + scale_pad))
+        if cache_dtype_str not in (INT8_PER_TOKEN_HEAD, FP8_PER_TOKEN_HEAD, INT4_PER_TOKEN_HEAD):
+            raise NotImplementedError(f"kv cache dtype {cache_dtype_str!r}: {INT8_PER_TOKEN_HEAD!r}, "
+                                      f"{FP8_PER_TOKEN_HEAD!r} and {INT4_PER_TOKEN_HEAD!r} are built")
+        scale_pad = SCALE_BYTES // torch.int8.itemsize   # fp8 and packed int4 elements are one byte as well
+        # INT4 packs two values per byte, so the data occupies only head_size // 2 bytes (:332-346)
+        data_head_size = head_size // 2 if cache_dtype_str == INT4_PER_TOKEN_HEAD else head_size
+        if cache_dtype_str == INT4_PER_TOKEN_HEAD and head_size % 8:
+            raise ValueError("int4 codes need a head size that is a multiple of 8 (4-byte aligned records)")
+        return (num_blocks, num_kv_heads, block_size, 2 * (data_head_size + scale_pad))
     return (num_blocks, num_kv_heads, block_size, 2 * head_size)
 
 
@@ -100,10 +105,12 @@ def kv_cache_stride_order(include_num_layers_dimension: bool = False, layout: st
 
 
 def allocate_kv_cache(num_blocks: int, block_size: int, num_kv_heads: int, head_size: int,
-                      device="cuda", layout: str | None = None, fill: int | None = 0) -> torch.Tensor:
+                      device="cuda", layout: str | None = None, fill: int | None = 0,
+                      cache_dtype_str: str = INT8_PER_TOKEN_HEAD) -> torch.Tensor:
     """Allocate the cache the way the model runner does: physical tensor in stride
-    order, returned permuted back to the logical ``(nb, Hkv, bs, 2*(D+4))`` shape."""
-    shape = kv_cache_shape(num_blocks, block_size, num_kv_heads, head_size)
+    order, returned permuted back to the logical ``(nb, Hkv, bs, 2*(D+4))`` shape
+    (``2*(D/2+4)`` for int4 codes)."""
+    shape = kv_cache_shape(num_blocks, block_size, num_kv_heads, head_size, cache_dtype_str)
     order = kv_cache_stride_order(layout=layout)
     phys_shape = tuple(shape[i] for i in order)
     phys = torch.empty(phys_shape, dtype=torch.int8, device=device)
@@ -170,16 +177,27 @@ class CacheGeometry:
     code_type: int = _C.KVQ_CODE_INT8   # what a code byte is: int8, or an e4m3fn bit pattern
 
     def with_code_type(self, code_type: int) -> "CacheGeometry":
-        """The same bytes read as another kind of code (the geometry of a cache does not depend on it)."""
+        """The same bytes read as another kind of code.  Offsets and strides do not depend on it; the head
+        size does for int4 codes, two of which share a byte."""
         if code_type == self.code_type:
             return self
-        got = self.__dict__.get("_other")
+        others = self.__dict__.get("_others")
+        if others is None:
+            others = {}
+            object.__setattr__(self, "_others", others)
+        got = others.get(code_type)
         if got is None:
             d = {k: v for k, v in self.__dict__.items() if not k.startswith("_")}
             d["code_type"] = code_type
+            d["head_size"] = self.code_bytes * 2 if code_type == _C.KVQ_CODE_INT4 else self.code_bytes
             got = CacheGeometry(**d)
-            object.__setattr__(self, "_other", got)
+            others[code_type] = got
         return got
+
+    @property
+    def code_bytes(self) -> int:
+        """Code bytes of one half (K or V) of a record."""
+        return self.head_size // 2 if self.code_type == _C.KVQ_CODE_INT4 else self.head_size
 
     def as_struct(self) -> "_C.CacheGeom":
         """The ctypes struct, built once per geometry object (it is read-only for the library)."""
@@ -193,7 +211,7 @@ class CacheGeometry:
 
     @property
     def record_bytes(self) -> int:
-        return 2 * (self.head_size + SCALE_BYTES)
+        return 2 * (self.code_bytes + SCALE_BYTES)
 
 
 _ONE_BYTE_DTYPES = tuple(d for d in (torch.int8, torch.uint8, getattr(torch, "float8_e4m3fn", None)) if d is not None)
@@ -205,7 +223,9 @@ def code_type_of(kv_quant_mode) -> int:
         return _C.KVQ_CODE_INT8
     if kv_quant_mode == KVQuantMode.FP8_PER_TOKEN_HEAD:
         return _C.KVQ_CODE_FP8_E4M3
-    raise NotImplementedError(f"kv_quant_mode {kv_quant_mode!r}: INT8_PER_TOKEN_HEAD and FP8_PER_TOKEN_HEAD are built")
+    if kv_quant_mode == KVQuantMode.INT4_PER_TOKEN_HEAD:
+        return _C.KVQ_CODE_INT4
+    raise NotImplementedError(f"kv_quant_mode {kv_quant_mode!r}: the per-token-head modes (int8, fp8, int4) are built")
 
 
 def geometry_from_views(key_cache: torch.Tensor, value_cache: torch.Tensor,
@@ -214,8 +234,8 @@ def geometry_from_views(key_cache: torch.Tensor, value_cache: torch.Tensor,
     """Validate the four views and reduce them to one base pointer + byte geometry.
 
     key_cache / value_cache: ``(nb, bs, Hkv, D+4)`` of a one-byte dtype (int8; uint8 or float8_e4m3fn
-    for fp8 codes); scale caches ``(nb, bs, Hkv)`` fp32 over the same storage, all four with identical
-    block/slot/head byte strides."""
+    for fp8 codes; ``D/2+4`` bytes for int4 codes); scale caches ``(nb, bs, Hkv)`` fp32 over the same
+    storage, all four with identical block/slot/head byte strides."""
     if key_cache.dtype not in _ONE_BYTE_DTYPES or value_cache.dtype != key_cache.dtype:
         raise ValueError("key_cache/value_cache must share a one-byte dtype (int8, uint8 or float8_e4m3fn)")
     if k_scale_cache.dtype != torch.float32 or v_scale_cache.dtype != torch.float32:
@@ -236,8 +256,8 @@ def geometry_from_views(key_cache: torch.Tensor, value_cache: torch.Tensor,
         k_off=key_cache.data_ptr() - base, v_off=value_cache.data_ptr() - base,
         ks_off=k_scale_cache.data_ptr() - base, vs_off=v_scale_cache.data_ptr() - base,
         stride_block=sb, stride_slot=ss, stride_head=sh,
-        num_kv_heads=hkv, head_size=padded - SCALE_BYTES, block_size=bs, num_blocks=nb, base_ptr=base,
-        code_type=code_type,
+        num_kv_heads=hkv, head_size=(padded - SCALE_BYTES) * (2 if code_type == _C.KVQ_CODE_INT4 else 1),
+        block_size=bs, num_blocks=nb, base_ptr=base, code_type=code_type,
     )
     if any(v % 4 for v in (geom.k_off, geom.v_off, geom.ks_off, geom.vs_off, sb, ss, sh, base)):
         raise ValueError("cache views must be 4-byte aligned")

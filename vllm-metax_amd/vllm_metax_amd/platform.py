@@ -6,7 +6,7 @@ candidate, in priority order, for the reasons it cannot serve a configuration.  
 this build stand in the registry slots TRITON_ATTN (per-token-head int8 cache) and TRITON_MLA (int8
 latent cache) -- but ONLY for those two KV-cache dtypes: ``Int8KVPlatform.get_attn_backend_cls``
 routes a layer here when its ``kv_cache_dtype`` is one of them and hands every other dtype (auto,
-bf16, fp8, the reference's fp8 / int4 per-token-head modes ...) to the platform it derives from, so a
+bf16, per-tensor fp8 ...) to the platform it derives from, so a
 deployment that mixes cache dtypes keeps upstream's own backends for the rest.  Overwriting the two
 registry slots globally is possible (``register_attention_backends(replace_slots=True)``) and then
 removes those dtypes from the slots.
@@ -15,10 +15,10 @@ from __future__ import annotations
 
 import importlib
 
-from .kv_cache_interface import FP8_PER_TOKEN_HEAD, INT8_PER_TOKEN, INT8_PER_TOKEN_HEAD
+from .kv_cache_interface import FP8_PER_TOKEN_HEAD, INT4_PER_TOKEN_HEAD, INT8_PER_TOKEN, INT8_PER_TOKEN_HEAD
 
 PLATFORM_PATH = "vllm_metax_amd.platform.Int8KVPlatform"
-INT8_KV_DTYPES = (INT8_PER_TOKEN_HEAD, FP8_PER_TOKEN_HEAD, INT8_PER_TOKEN)   # the inline-scale dtypes this build serves
+INT8_KV_DTYPES = (INT8_PER_TOKEN_HEAD, FP8_PER_TOKEN_HEAD, INT4_PER_TOKEN_HEAD, INT8_PER_TOKEN)   # the inline-scale dtypes this build serves
 
 INT8_ATTN_PATH = "vllm_metax_amd.v1.attention.backends.int8_attn.Int8AttentionBackend"
 INT8_MLA_PATH = "vllm_metax_amd.v1.attention.backends.mla.int8_mla.Int8MLABackend"

@@ -157,7 +157,7 @@ class Int8AttentionBackend(_BackendBase):
     (vllm_metax/v1/attention/backends/triton_attn.py:272-410)."""
 
     supported_dtypes: ClassVar[list[torch.dtype]] = [torch.float16, torch.bfloat16, torch.float32]
-    supported_kv_cache_dtypes: ClassVar[list[str]] = ["int8_per_token_head", "fp8_per_token_head"]
+    supported_kv_cache_dtypes: ClassVar[list[str]] = ["int8_per_token_head", "fp8_per_token_head", "int4_per_token_head"]
     forward_includes_kv_cache_update: bool = False
 
     @staticmethod
@@ -279,8 +279,8 @@ class Int8AttentionImpl(_ImplBase):
         if attn_type != AttentionType.DECODER:
             raise NotImplementedError("quantized KV cache is not supported for encoder attention")
         if not kv_cache_uses_per_token_head_scales(kv_cache_dtype) or get_kv_quant_mode(kv_cache_dtype) not in (
-                KVQuantMode.INT8_PER_TOKEN_HEAD, KVQuantMode.FP8_PER_TOKEN_HEAD):
-            raise ValueError("Int8AttentionImpl needs kv_cache_dtype 'int8_per_token_head' or 'fp8_per_token_head', "
+                KVQuantMode.INT8_PER_TOKEN_HEAD, KVQuantMode.FP8_PER_TOKEN_HEAD, KVQuantMode.INT4_PER_TOKEN_HEAD):
+            raise ValueError("Int8AttentionImpl needs kv_cache_dtype 'int8_per_token_head', 'fp8_per_token_head' or 'int4_per_token_head', "
                              f"got {kv_cache_dtype!r}")
         if num_heads % num_kv_heads:
             raise ValueError("num_heads must be a multiple of num_kv_heads")
