@@ -87,6 +87,10 @@ typedef struct kvq_cache_geom {
 #define KVQ_CODE_FP8_E4M3 1
 #define KVQ_CODE_INT4 2
 
+/* flags of the `causal` argument of kvq_paged_attn_int8 and its static-scratch form */
+#define KVQ_ATTN_CAUSAL 1
+#define KVQ_ATTN_NO_DECODE_ROWS 2
+
 /* Byte geometry of the int8 MLA latent cache: per block, block_size code rows
  * of (kv_lora_rank + rope_dim) bytes followed by block_size fp32 scales. */
 typedef struct kvq_mla_geom {
@@ -166,6 +170,12 @@ KVQ_API size_t kvq_paged_attn_workspace_bytes(int max_num_seqs, int num_q_heads,
  * 0 = no window.  softcap > 0: logits become softcap * tanh(scale * q.k / softcap)
  * (triton_attn.py:703; semantics as in the reference's test oracle,
  * tests/kernels/attention/test_triton_unified_attention.py:63-70); 0 = none.
+ *
+ * `causal` is a set of flags: KVQ_ATTN_CAUSAL (1, the reference's causal=True) and, optionally,
+ * KVQ_ATTN_NO_DECODE_ROWS (2): the caller's promise that no sequence of this batch has exactly one query
+ * row (a pure prefill batch; a metadata builder knows it from the host copy of query_start_loc).  The
+ * split-K decode kernel and its reduce are then not launched at all; with a one-row sequence in the batch
+ * after all, that row's output is left unwritten.
  *
  * Value range: the weights enter the second product as fp16 numbers
  * p * v_scale * 2^8, so a V row whose scale exceeds 255.8 (int8 codes: absmax

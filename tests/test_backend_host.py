@@ -236,6 +236,13 @@ def test_builder_packs_metadata_without_touching_the_gpu():
     md = b.build(0, c)
     assert md.num_actual_tokens == 2 and md.workspace is None and md.use_cascade is False
     assert b.build_for_cudagraph_capture(c).seq_lens.tolist() == [1, 1]
+    assert md.has_decode_rows is True
+    # the host copy of query_start_loc tells a pure prefill batch from a mixed one
+    c2 = types.SimpleNamespace(**{**c.__dict__, "max_query_len": 7, "num_actual_tokens": 10,
+                                  "query_start_loc_cpu": torch.tensor([0, 3, 10], dtype=torch.int32)})
+    assert b.build(0, c2).has_decode_rows is False
+    c2.query_start_loc_cpu = torch.tensor([0, 1, 8], dtype=torch.int32)
+    assert b.build(0, c2).has_decode_rows is True
     with pytest.raises(NotImplementedError):
         b.build(4, c)
     c.num_reqs = 5

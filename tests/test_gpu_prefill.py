@@ -209,3 +209,27 @@ def test_prefill_huge_value_scales(gpu_device):
     got = run(gpu_device, kv, "NHD", bt, q, sl, cu, max(qls), scale, out_dtype=torch.float32)
     assert torch.isfinite(got).all()
     T.assert_close_attn(got, want, atol=2e-2 * 2000, rtol=1e-2, what="prefill, huge value scales")
+
+
+def test_pure_prefill_batch_with_the_no_decode_rows_promise(gpu_device):
+    """has_decode_rows=False (KVQ_ATTN_NO_DECODE_ROWS): the decode kernels are skipped; a batch without one-row
+    sequences gives the same bits either way, for both prefill tiles."""
+    dev = gpu_device
+    for hq, hkv, qls in ((32, 8, [300, 64, 2048]), (8, 8, [5, 33, 2])):
+        ctx = [q + extra for q, extra in zip(qls, [700, 0, 133])]
+        kv_cpu, lay, bt, q, sl, cu = build(ctx, qls, hq, hkv, 128, 16, seed=21)
+        kv = T.to_device_cache(kv_cpu, dev, "NHD")
+        k, v = L.key_value_views(kv)
+        ks, vs = L.scale_views(kv)
+        outs = []
+        for promise in (True, False):
+            out = torch.full(q.shape, float("nan"), dtype=torch.bfloat16, device=dev)
+            lse = torch.full(q.shape[:2], float("nan"), dtype=torch.float32, device=dev)
+            ops.unified_attention(q.to(dev), k, v, out, cu.to(dev), max(qls), sl.to(dev), int(sl.max()), 0.0884, True,
+                                  block_table=bt.to(dev), k_scale_cache=ks, v_scale_cache=vs, lse=lse,
+                                  has_decode_rows=promise)
+            torch.cuda.synchronize()
+            outs.append((out.cpu(), lse.cpu()))
+        assert torch.equal(outs[0][0].view(torch.int16), outs[1][0].view(torch.int16)) and torch.equal(outs[0][1], outs[1][1])
+        want = oracle.paged_attn(q, T.storage_bytes(kv_cpu), lay, bt, sl, cu, 0.0884)
+        T.assert_close_attn(outs[1][0], want, what="pure prefill batch")

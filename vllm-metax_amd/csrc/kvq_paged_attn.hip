@@ -71,6 +71,9 @@ static int paged_attn_launch(const char* op, void* out, int out_dtype, int64_t o
                              kvq_stream_t stream, const NewTokens* fresh = nullptr) {
   int rc0 = validate_common(op, q, cache, geom, block_table, seq_lens, num_seqs, num_q_heads);
   if (rc0) return rc0;
+  KVQ_REQUIRE((causal & ~(KVQ_ATTN_CAUSAL | KVQ_ATTN_NO_DECODE_ROWS)) == 0, "%s: unknown flag in causal (%d)", op, causal);
+  const bool no_decode_rows = (causal & KVQ_ATTN_NO_DECODE_ROWS) != 0;
+  causal &= KVQ_ATTN_CAUSAL;
   KVQ_REQUIRE(out != nullptr, "%s: out is NULL", op);
   KVQ_REQUIRE(max_query_len >= 1, "%s: max_query_len must be >= 1", op);
   KVQ_REQUIRE(max_query_len == 1 || cu_seqlens_q != nullptr, "%s: cu_seqlens_q is required when max_query_len > 1", op);
@@ -142,7 +145,9 @@ static int paged_attn_launch(const char* op, void* out, int out_dtype, int64_t o
     a.new_slots = fresh->slot_mapping;
   }
   hipStream_t s = as_stream(stream);
-  int rc = launch_decode_streamk(a, q_dtype, out_dtype, s);
+  int rc = KVQ_OK;
+  // a batch that the caller knows to hold no one-row sequence has nothing for the decode kernel and its reduce
+  if (!(no_decode_rows && max_query_len > 1)) rc = launch_decode_streamk(a, q_dtype, out_dtype, s);
   if (rc) return rc;
   if (max_query_len > 1) {
     // the list of the sequences that have a query run sits behind the decode kernels' notes in the workspace

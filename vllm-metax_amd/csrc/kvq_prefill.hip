@@ -405,6 +405,8 @@ template <int D, int QDT, int ODT, int CODE = KVQ_CODE_INT8>
 struct Flash32 {
   using DTile = DecodeTile<D, QDT, ODT, CODE>;
   static constexpr bool FP8 = DTile::FP8;   // e4m3fn codes: they enter the MFMA as value / 2^8, without a bias
+  static constexpr bool INT4 = DTile::INT4; // two codes per byte: only the expansion of the raw tile differs
+  static constexpr int DB = DTile::DB;      // code bytes of a half record
   static constexpr int WAVES = 4;
   static constexpr int KS = D / 16;                      // k-steps of the QK product
   static constexpr int MT = D / 32;                      // 32-dim row tiles of O^T
@@ -471,7 +473,53 @@ struct Flash32 {
       for (int j = 0; j < 8; ++j) qsum += (float)qb[ks][j];  // the sum of what the MFMA will actually see
     }
     qsum += __shfl_xor(qsum, 32, kWave);
-    return FP8 ? 0.f : -kCodeBias * qsum;
+    return FP8 ? 0.f : -DTile::kBias * qsum;
+  }
+
+  // Two nibbles of y (= code bytes ^ 0x88..., see nibbles_to_half2) as two fp16 codes, bias taken out.
+  __device__ static __forceinline__ uint32_t nibbles_to_codes(uint32_t y, int k) {
+    const half2_t bias = {(half_t)kCodeBiasInt4, (half_t)kCodeBiasInt4};
+    const half2_t v = __builtin_bit_cast(half2_t, nibbles_to_half2(y, k)) - bias;
+    return __builtin_bit_cast(uint32_t, v);
+  }
+
+  // The int4 form of expand(): one thread converts one 16-byte K chunk (32 codes, put back into dim order: the
+  // and-or conversion yields dims 0 4 1 5 2 6 3 7 of a dword) and one 4-token x 4-dim V block (two bytes per token).
+  __device__ static __forceinline__ void expand_int4(const uint8_t* raw, uint8_t* buf, int tid) {
+    constexpr int KCH = DB / 16;
+    if (tid < kTile * KCH) {
+      const int tok = tid / KCH, ch = tid % KCH;
+      const u32x4 w = *reinterpret_cast<const u32x4*>(raw + tok * RAW_PITCH + 16 * ch);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const uint32_t y = w[i] ^ 0x88888888u;
+        const uint32_t h0 = nibbles_to_half2(y, 0), h1 = nibbles_to_half2(y, 1);   // dims (0, 4), (1, 5)
+        const uint32_t h2 = nibbles_to_half2(y, 2), h3 = nibbles_to_half2(y, 3);   // dims (2, 6), (3, 7)
+        u32x4 o;
+        o.x = perm(h1, h0, kPermLowHalves);
+        o.y = perm(h3, h2, kPermLowHalves);
+        o.z = perm(h1, h0, kPermHighHalves);
+        o.w = perm(h3, h2, kPermHighHalves);
+        *reinterpret_cast<u32x4*>(buf + tok * K_PITCH + 64 * ch + 16 * i) = o;
+      }
+    }
+    if (tid < 8 * (D / 4)) {
+      const int tg = tid & 7, dq = tid >> 3;
+      uint32_t t[4];
+#pragma unroll
+      for (int a = 0; a < 4; ++a)
+        t[a] = *reinterpret_cast<const uint16_t*>(raw + (4 * tg + a) * RAW_PITCH + (DB + 4) + 2 * dq);
+      const uint32_t y01 = (t[0] | (t[1] << 16)) ^ 0x88888888u, y23 = (t[2] | (t[3] << 16)) ^ 0x88888888u;
+      const int pos = (tg >> 2) * 16 + (tg & 1) * 8 + ((tg >> 1) & 1) * 4;
+      uint8_t* vrow = buf + K_BYTES + (4 * dq) * V_PITCH + 2 * pos;
+#pragma unroll
+      for (int b = 0; b < 4; ++b) {
+        u32x2 o;
+        o.x = nibbles_to_codes(y01, b);
+        o.y = nibbles_to_codes(y23, b);
+        *reinterpret_cast<u32x2*>(vrow + b * V_PITCH) = o;
+      }
+    }
   }
 
   // Raw tile -> fp16 K [token][dim] (codes + 1152) and V^T [dim][position] (codes); token t of the tile sits at position
@@ -479,6 +527,9 @@ struct Flash32 {
   // lane its tokens.  One thread converts one 16-code K chunk and one 4-token x 4-dim V block.
   __device__ static __forceinline__ void expand(const uint8_t* raw, uint8_t* buf, int tid, float sc_mul, uint32_t l_sc) {
     constexpr int KCH = D / 16;
+    if constexpr (INT4) {
+      expand_int4(raw, buf, tid);
+    } else {
     if (tid < kTile * KCH) {
       const int tok = tid / KCH, ch = tid % KCH;
       const u32x4 w = *reinterpret_cast<const u32x4*>(raw + tok * RAW_PITCH + 16 * ch);
@@ -513,6 +564,7 @@ struct Flash32 {
         o.y = to_half2(p23, b & 1);
         *reinterpret_cast<u32x2*>(vrow + b * V_PITCH) = o;
       }
+    }
     }
     if (tid < 64) {
       const float sc = *reinterpret_cast<const float*>(raw + l_sc);
@@ -742,7 +794,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       r.tail = __builtin_bit_cast(u32x2, __builtin_amdgcn_raw_buffer_load_b64(half ? w.r1 : w.r0, lo.g_tail, 0, 0));
     };
     const uint32_t l_chunk = lo.l_chunk + ld_n * (64 / DTile::NCH) * FP::RAW_PITCH;
-    const uint32_t l_tail = (16 * half + (lane & 15)) * FP::RAW_PITCH + 2 * D;
+    const uint32_t l_tail = (16 * half + (lane & 15)) * FP::RAW_PITCH + 2 * FP::DB;
     auto drop = [&](const Regs& r, uint8_t* raw) __attribute__((always_inline)) {
       *reinterpret_cast<u32x4*>(raw + l_chunk) = r.c0;
       *reinterpret_cast<u32x4*>(raw + l_chunk + 16 * FP::RAW_PITCH) = r.c1;
@@ -862,14 +914,15 @@ template <int D, int QDT, int ODT>
 static int launch_prefill_nt(PrefillArgs& a, int max_query_len, hipStream_t s) {
   constexpr int WPW = 4;
   const bool fp8 = a.io.g.code_type == KVQ_CODE_FP8_E4M3;
-  if (a.io.g.code_type == KVQ_CODE_INT4) {   // int4 codes: the per-wave tile for runs of any length
-    a.q_tokens = 16 / a.io.group;
-    return launch_prefill_cfg<D, QDT, ODT, 1, WPW, KVQ_CODE_INT4>(a, max_query_len, s);
-  }
-  // long runs: the workgroup-shared fp16 tile (compute-bound shape), for either kind of one-byte code
+  const bool int4 = a.io.g.code_type == KVQ_CODE_INT4;
+  // long runs: the workgroup-shared fp16 tile (compute-bound shape), for every kind of code
   if constexpr (D <= 128) {
     if (max_query_len * a.io.group >= 64) {
       const bool ext = a.io.window > 0 || a.io.cap_c != 0.f;
+      if (int4) {
+        if (ext) return launch_prefill_flash32<D, QDT, ODT, true, KVQ_CODE_INT4>(a, max_query_len, s);
+        return launch_prefill_flash32<D, QDT, ODT, false, KVQ_CODE_INT4>(a, max_query_len, s);
+      }
       if (fp8) {
         if (ext) return launch_prefill_flash32<D, QDT, ODT, true, KVQ_CODE_FP8_E4M3>(a, max_query_len, s);
         return launch_prefill_flash32<D, QDT, ODT, false, KVQ_CODE_FP8_E4M3>(a, max_query_len, s);
@@ -881,6 +934,10 @@ static int launch_prefill_nt(PrefillArgs& a, int max_query_len, hipStream_t s) {
   if (fp8) {  // short runs of fp8 codes: the per-wave tile, one column tile per wave
     a.q_tokens = 16 / a.io.group;
     return launch_prefill_cfg<D, QDT, ODT, 1, WPW, KVQ_CODE_FP8_E4M3>(a, max_query_len, s);
+  }
+  if (int4) {
+    a.q_tokens = 16 / a.io.group;
+    return launch_prefill_cfg<D, QDT, ODT, 1, WPW, KVQ_CODE_INT4>(a, max_query_len, s);
   }
   // two column tiles per wave where the accumulators fit the register file next to a tile in flight
   if (D <= 128 && a.io.group * 2 <= 32 && max_query_len * a.io.group > 16) {

@@ -237,6 +237,7 @@ def unified_attention(
     geometry: CacheGeometry | None = None,
     lse: torch.Tensor | None = None,
     static_scratch: bool = False,
+    has_decode_rows: bool = True,
     **unused,
 ) -> None:
     """Drop-in for ``unified_attention`` as called at
@@ -249,7 +250,9 @@ def unified_attention(
     this path does not build raise ``NotImplementedError``.  ``window_size=(W - 1, 0)`` restricts a
     query to its last W keys; ``softcap > 0`` maps logits through ``softcap * tanh(x / softcap)``.
     ``static_scratch=True`` keeps the split-K states in the library's own fixed array instead of a
-    workspace tensor (nothing is allocated; calls on one GPU must then not overlap in time)."""
+    workspace tensor (nothing is allocated; calls on one GPU must then not overlap in time).
+    ``has_decode_rows=False`` is the caller's promise that no sequence of the batch has exactly one query row (a
+    pure prefill batch): the decode kernel and its reduce are then not launched."""
     code_type = code_type_of(kv_quant_mode)
     if alibi_slopes is not None or sinks is not None or output_scale is not None or mm_prefix_range is not None:
         raise NotImplementedError("alibi, sinks, fused output quantisation and mm-prefix ranges are not built")
@@ -300,7 +303,7 @@ def unified_attention(
             _ptr(q), _dtype_code(q, "q"), q.stride(0), q.stride(1),
             ctypes.c_void_p(geom.base_ptr), ctypes.byref(g), _ptr(block_table), block_table.stride(0),
             _ptr(seqused_k), _ptr(cu_seqlens_q), num_seqs, num_q_heads, int(max_seqlen_q),
-            float(softmax_scale), 1 if causal else 0, window, softcap, _ptr(lse))
+            float(softmax_scale), (1 if causal else 0) | (0 if has_decode_rows else 2), window, softcap, _ptr(lse))
     if static_scratch:
         with _on_device(dev):
             rc = lib.kvq_paged_attn_int8_static_scratch(*head, _stream(dev))

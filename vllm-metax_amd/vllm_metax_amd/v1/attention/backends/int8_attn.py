@@ -81,6 +81,9 @@ class Int8AttentionMetadata:
     causal: bool = True
     use_cascade: bool = False
     common_prefix_len: int = 0
+    # False when the builder KNOWS (from the host copy of query_start_loc) that no sequence has exactly one query
+    # row: the attention call then skips its decode kernels
+    has_decode_rows: bool = True
 
 
 def _first_attr(obj, *names, default=None):
@@ -139,7 +142,12 @@ class Int8AttentionMetadataBuilder(_BuilderBase):
         c = common_attn_metadata
         if c.num_reqs > self.max_num_seqs:
             raise RuntimeError(f"batch of {c.num_reqs} sequences exceeds max_num_seqs={self.max_num_seqs}")
+        has_decode_rows = True
+        qsl_cpu = getattr(c, "query_start_loc_cpu", None)
+        if qsl_cpu is not None and c.max_query_len > 1 and qsl_cpu.numel() > 1:
+            has_decode_rows = bool((qsl_cpu[1:] - qsl_cpu[:-1] == 1).any())
         return Int8AttentionMetadata(
+            has_decode_rows=has_decode_rows,
             num_actual_tokens=c.num_actual_tokens,
             max_query_len=c.max_query_len,
             query_start_loc=c.query_start_loc,
@@ -377,7 +385,8 @@ class Int8AttentionImpl(_ImplBase):
             max_seqlen_k=attn_metadata.max_seq_len, softmax_scale=self.scale, causal=attn_metadata.causal,
             window_size=self.sliding_window, block_table=attn_metadata.block_table, softcap=self.logits_soft_cap,
             kv_quant_mode=self._kv_quant_mode, k_scale_cache=self._k_scale_cache, v_scale_cache=self._v_scale_cache,
-            workspace=attn_metadata.workspace, geometry=self._geometry)
+            workspace=attn_metadata.workspace, geometry=self._geometry,
+            has_decode_rows=getattr(attn_metadata, "has_decode_rows", True))
         return output
 
 
