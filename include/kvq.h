@@ -111,7 +111,7 @@ KVQ_API int kvq_device_num_cus(void);
  * supports_batch_invariance).  While it is on, every decode sequence is cut into splits by its OWN length
  * alone and its split states are merged in split order, so the bits of a row do not depend on what else the
  * batch holds, on the batch size or on the device's CU count: kvq_paged_attn_int8* cut a sequence into at
- * most 32 equal spans of at least 512 tokens, kvq_mla_decode_* into 8 splits.  Prefill rows never depend on
+ * most 32 equal spans of at least 256 tokens, kvq_mla_decode_* into 8 splits.  Prefill rows never depend on
  * their neighbours.  The workspace queries return what the mode needs, so set it before sizing workspaces
  * and not while launches are being enqueued.  Returns the previous setting.
  */

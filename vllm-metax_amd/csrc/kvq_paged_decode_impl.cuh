@@ -43,11 +43,34 @@ __device__ __forceinline__ int decode_tiles(const int32_t* seq_lens, const int32
   return (s < num_seqs && q_len == 1 && len > 0) ? n : 0;
 }
 
+// Batch-invariant cutting (StreamKArgs::fixed_spans): a sequence is cut at places that depend on nothing but its
+// own length -- into at most kFixedSpans spans of equal size, none shorter than kMinSpanTiles tiles.  The spans of
+// all decode sequences form one line (a unit per span) that is cut into equal shares like the balanced line, so
+// WHICH workgroup computes a span depends on the batch, but not what it computes: the states of a sequence's
+// spans lie in slots seq * kFixedSpans + span and are merged in span order, so a row's bits are the same
+// whatever else the batch holds and however many workgroups the device runs.
+constexpr int kFixedSpans = 32;
+constexpr int kMinSpanTiles = 8;
+__device__ __forceinline__ int fixed_span_tiles(int ntiles) {
+  const int per = (ntiles + kFixedSpans - 1) / kFixedSpans;
+  return per > kMinSpanTiles ? per : kMinSpanTiles;
+}
+__device__ __forceinline__ int fixed_span_count(int ntiles) {
+  const int per = fixed_span_tiles(ntiles);
+  return (ntiles + per - 1) / per;   // 0 for no tiles
+}
+
 // Units a sequence takes on the work line: its setup charge, then one unit per tile.
 __device__ __forceinline__ int decode_units(const int32_t* seq_lens, const int32_t* cu, int s, int num_seqs,
                                             int window) {
   const int n = decode_tiles(seq_lens, cu, s, num_seqs, window);
   return n > 0 ? n + kSetupUnits : 0;
+}
+// Units of a sequence on the line the launch cuts: tiles + setup charge, or (FIXED) its spans.
+template <bool FIXED>
+__device__ __forceinline__ int line_units(const int32_t* seq_lens, const int32_t* cu, int s, int num_seqs, int window) {
+  if constexpr (FIXED) return fixed_span_count(decode_tiles(seq_lens, cu, s, num_seqs, window));
+  else return decode_units(seq_lens, cu, s, num_seqs, window);
 }
 
 // The scans over the sequences work on chunks of 64 (one per lane).  Large batches take kScanBatch
@@ -56,7 +79,7 @@ __device__ __forceinline__ int decode_units(const int32_t* seq_lens, const int32
 constexpr int kScanBatch = 4;
 
 // Total units of the work line.
-template <int BATCH>
+template <int BATCH, bool FIXED = false>
 __device__ __forceinline__ int64_t scan_total(const StreamKArgs& a, int lane) {
   const int B = a.num_seqs;
   int64_t total = 0;
@@ -64,7 +87,7 @@ __device__ __forceinline__ int64_t scan_total(const StreamKArgs& a, int lane) {
     int n[BATCH];
 #pragma unroll
     for (int j = 0; j < BATCH; ++j)
-      n[j] = decode_units(a.seq_lens, a.cu_seqlens_q, base + kWave * j + lane, B, a.io.window);
+      n[j] = line_units<FIXED>(a.seq_lens, a.cu_seqlens_q, base + kWave * j + lane, B, a.io.window);
 #pragma unroll
     for (int j = 0; j < BATCH; ++j) total += __builtin_amdgcn_readlane(wave_incl_scan(n[j], lane), 63);
   }
@@ -72,7 +95,7 @@ __device__ __forceinline__ int64_t scan_total(const StreamKArgs& a, int lane) {
 }
 
 // The sequence that holds unit `lo` and the index of its first unit.
-template <int BATCH>
+template <int BATCH, bool FIXED = false>
 __device__ __forceinline__ void scan_locate(const StreamKArgs& a, int lane, int64_t lo, int& seq, int64_t& seq_start) {
   const int B = a.num_seqs;
   int64_t cum = 0;
@@ -81,7 +104,7 @@ __device__ __forceinline__ void scan_locate(const StreamKArgs& a, int lane, int6
     int nn[BATCH];
 #pragma unroll
     for (int j = 0; j < BATCH; ++j)
-      nn[j] = decode_units(a.seq_lens, a.cu_seqlens_q, base + kWave * j + lane, B, a.io.window);
+      nn[j] = line_units<FIXED>(a.seq_lens, a.cu_seqlens_q, base + kWave * j + lane, B, a.io.window);
 #pragma unroll
     for (int j = 0; j < BATCH; ++j) {
       const int n = nn[j];
@@ -114,18 +137,6 @@ __device__ __forceinline__ int active_workgroups(int64_t total, int num_wg) {
   return want >= num_wg ? num_wg : (want < 1 ? 1 : (int)want);
 }
 
-// Batch-invariant cutting (StreamKArgs::fixed_spans): a sequence is cut at places that depend on nothing but its
-// own length -- into at most kFixedSpans spans of equal size, none shorter than kMinSpanTiles tiles -- and
-// workgroup w takes the (sequence, span) pairs w, w + P, w + 2 P, ... one after the other.  The states of a
-// sequence's spans lie in slots seq * kFixedSpans + span and are merged in span order, so a row's bits are the same
-// whatever else the batch holds and however many workgroups the device runs.
-constexpr int kFixedSpans = 32;
-constexpr int kMinSpanTiles = 16;
-__device__ __forceinline__ int fixed_span_tiles(int ntiles) {
-  const int per = (ntiles + kFixedSpans - 1) / kFixedSpans;
-  return per > kMinSpanTiles ? per : kMinSpanTiles;
-}
-
 // HPW = kv heads per workgroup (1, 2, 4 or 8).  A workgroup always has eight waves: with fewer than
 // eight kv heads the 8 / HPW waves of a head take the tiles of a run in turn and their states are
 // folded together in LDS when the run ends, so a compute unit keeps eight tile streams in flight
@@ -152,19 +163,21 @@ __global__ __launch_bounds__(512) void paged_decode_streamk_kernel(StreamKArgs a
   int64_t total = 0, lo = 0, hi = 0;
   int seq = 0;
   int64_t seq_start = 0;  // global index of the sequence's first unit
-  if constexpr (!fixed) {
-    total = one_chunk ? scan_total<1>(a, lane) : scan_total<kScanBatch>(a, lane);
-    const int num_wg = active_workgroups(total, a.num_wg);
+  {
+    total = one_chunk ? scan_total<1, fixed>(a, lane) : scan_total<kScanBatch, fixed>(a, lane);
+    // (the batch-invariant line is short -- a unit is a span of at least kMinSpanTiles tiles -- and is always shared
+    // out over every workgroup there is a unit for)
+    const int num_wg = fixed ? (total < a.num_wg ? (total < 1 ? 1 : (int)total) : a.num_wg) : active_workgroups(total, a.num_wg);
     if (w >= num_wg) return;
     lo = wg_tile_begin(w, total, num_wg);
     hi = wg_tile_begin(w + 1, total, num_wg);
     if (lo >= hi) {   // an empty work line: workgroup 0 still reports its length
-      if (w == 0 && blockIdx.y == 0 && wave == 0 && lane == 0) a.wg_info[0] = total;
+      if (!fixed && w == 0 && blockIdx.y == 0 && wave == 0 && lane == 0) a.wg_info[0] = total;
       return;
     }
     // locate the sequence holding unit `lo`
-    if (one_chunk) scan_locate<1>(a, lane, lo, seq, seq_start);
-    else scan_locate<kScanBatch>(a, lane, lo, seq, seq_start);
+    if (one_chunk) scan_locate<1, fixed>(a, lane, lo, seq, seq_start);
+    else scan_locate<kScanBatch, fixed>(a, lane, lo, seq, seq_start);
     seq = __builtin_amdgcn_readfirstlane(seq);
   }
   // Where the share begins (the reduce kernel's key to the span): noted in the first round of the loop, stored
@@ -208,20 +221,26 @@ __global__ __launch_bounds__(512) void paged_decode_streamk_kernel(StreamKArgs a
   };
 
   if constexpr (fixed) {
-    // the (sequence, span) pairs w, w + P, ...
-    for (int item = w; item < B * kFixedSpans; item += (int)gridDim.x) {
-      const int cur = item / kFixedSpans;
-      const int span = item % kFixedSpans;
-      const int ntiles = __builtin_amdgcn_readfirstlane(decode_tiles(a.seq_lens, a.cu_seqlens_q, cur, B, a.io.window));
+    // the spans [lo, hi) of the span line, sequence by sequence
+    int64_t at = lo;
+    while (at < hi && seq < B) {
+      const int ntiles = __builtin_amdgcn_readfirstlane(decode_tiles(a.seq_lens, a.cu_seqlens_q, seq, B, a.io.window));
+      const int spans = fixed_span_count(ntiles);
+      const int span = (int)(at - seq_start);
+      if (span >= spans) {   // also: a sequence without tiles
+        seq_start += spans;
+        ++seq;
+        continue;
+      }
       const int per = fixed_span_tiles(ntiles);
-      if (span * per >= ntiles) continue;   // also: no tiles at all
-      const int len = __builtin_amdgcn_readfirstlane(a.seq_lens[cur]);
-      const int64_t row = a.cu_seqlens_q ? (int64_t)a.cu_seqlens_q[cur] : (int64_t)cur;
+      const int len = __builtin_amdgcn_readfirstlane(a.seq_lens[seq]);
+      const int64_t row = a.cu_seqlens_q ? (int64_t)a.cu_seqlens_q[seq] : (int64_t)seq;
       const int first = window_first(len, a.io.window);
       const int t0 = first / kTile;
       const int t_begin = t0 + span * per;
       const int t_end = min(t0 + ntiles, t_begin + per);
-      process(cur, 0, row, len, first, t0, ntiles, t_begin, t_end, (int64_t)cur * kFixedSpans + span);
+      process(seq, 0, row, len, first, t0, ntiles, t_begin, t_end, (int64_t)seq * kFixedSpans + span);
+      ++at;
     }
     return;
   }
@@ -793,7 +812,9 @@ static int launch_streamk(const StreamKArgs& a, hipStream_t s) {
   dim3 grid(a.num_wg, (hkv + hpw - 1) / hpw);
 #define KVQ_SK_CODE(H, C, CODE)                                                                                   \
   do {                                                                                                            \
-    if (a.fixed_spans)                                                                                            \
+    if (a.fixed_spans && !C && stream)                                                                            \
+      hipLaunchKernelGGL((paged_decode_streamk_kernel<D, QDT, H, false, CODE, true, true>), grid, dim3(512), 0, s, a); \
+    else if (a.fixed_spans)                                                                                       \
       hipLaunchKernelGGL((paged_decode_streamk_kernel<D, QDT, H, C, CODE, false, true>), grid, dim3(512), 0, s, a); \
     else if (!C && stream)                                                                                        \
       hipLaunchKernelGGL((paged_decode_streamk_kernel<D, QDT, H, false, CODE, true>), grid, dim3(512), 0, s, a);  \
