@@ -27,7 +27,7 @@
 extern "C" {
 #endif
 
-#define KVQ_ABI_VERSION 14
+#define KVQ_ABI_VERSION 15
 
 #define KVQ_OK 0
 #define KVQ_EINVAL (-22)
@@ -147,6 +147,27 @@ KVQ_API int kvq_reshape_and_cache_int8(const void* key, const void* value, int s
  * vllm_metax/v1/attention/backends/triton_attn.py:155-176.
  */
 KVQ_API size_t kvq_paged_attn_workspace_bytes(int max_num_seqs, int num_q_heads, int head_size);
+
+/*
+ * Rotary embedding of the step's query and key rows fused with the quantise-on-write of the step's K / V:
+ * the body of do_rope_and_kv_cache_update(layer, query, key, value, positions, cos_sin_cache, is_neox,
+ * kv_cache, layer_slot_mapping), which the reference's backend declares and refuses
+ * (vllm_metax/v1/attention/backends/triton_attn.py:833-848: fused_rope_kvcache_supported() is False and the
+ * method raises "Not supported on Maca").  query [T, Hq, D] and key [T, Hkv, D] are rotated IN PLACE over their
+ * first rot_dim dims (pair i = (i, rot_dim/2 + i) when is_neox, else (2i, 2i+1); cos_sin_cache
+ * [max_position, rot_dim] = rot_dim/2 cosines then rot_dim/2 sines; the arithmetic of the reference's fused
+ * MLA kernel, csrc/libtorch_stable/cache_kernels_fused.cu:55-117: every product and sum rounded on its own in
+ * the activation type); the rotated K rows and the V rows are then quantised into the cache exactly as
+ * kvq_reshape_and_cache_int8 would.  A token whose slot is negative is padding: neither rotated nor written.
+ * Head sizes up to 256; every code type.
+ */
+KVQ_API int kvq_rope_and_cache_int8(const int64_t* positions, void* query, int64_t q_stride_t, int64_t q_stride_h,
+                            int num_q_heads, void* key, int64_t key_stride_t, int64_t key_stride_h,
+                            const void* value, int64_t value_stride_t, int64_t value_stride_h,
+                            int src_dtype, const void* cos_sin_cache, int cos_sin_dtype, int rot_dim,
+                            int is_neox, void* cache, const kvq_cache_geom* geom,
+                            const int64_t* slot_mapping, int64_t num_tokens, float eps,
+                            kvq_stream_t stream);
 
 /*
  * Varlen paged attention over the int8 cache: decode rows and chunked-prefill

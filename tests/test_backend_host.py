@@ -189,7 +189,7 @@ def test_impl_does_not_pin_replaced_caches_and_refills_a_new_cache_at_a_reused_a
 def test_impl_constructor_errors():
     mk = lambda **kw: Int8AttentionImpl(32, 128, 0.088, 8, **kw)
     impl = mk()
-    assert impl.num_queries_per_kv == 4 and impl.fused_rope_kvcache_supported() is False
+    assert impl.num_queries_per_kv == 4 and impl.fused_rope_kvcache_supported() is True   # built here; the reference answers False
     for kw in (dict(alibi_slopes=[1.0] * 32), dict(sinks=torch.zeros(32)), dict(attn_type=AttentionType.ENCODER_ONLY)):
         with pytest.raises(NotImplementedError):
             mk(**kw)

@@ -113,3 +113,53 @@ def test_errors_are_loud(gpu_device):
     with pytest.raises(RuntimeError):
         ops.reshape_and_cache_flash_per_token_head_quant(key.cpu(), key.cpu(), k, v, ks, vs,
                                                          torch.zeros(4, dtype=torch.int64))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("is_neox", [True, False])
+@pytest.mark.parametrize("hq,hkv,d,rot,mode", [
+    (32, 8, 128, 128, "int8"), (28, 4, 128, 64, "int8"), (8, 2, 64, 64, "fp8"), (4, 1, 256, 128, "int4"),
+    (6, 3, 80, 32, "int8"),
+])
+def test_fused_rope_and_write_is_rotate_then_write(gpu_device, dtype, is_neox, hq, hkv, d, rot, mode):
+    """do_rope_and_kv_cache_update in one launch (the reference declares it and raises,
+    vllm_metax/v1/attention/backends/triton_attn.py:833-848): query and key rotated in place bit for bit as the
+    oracle's statement of the reference's rotary arithmetic rotates them, cache bytes equal to the oracle's write of
+    the rotated key and the value; padded tokens untouched."""
+    import oracle
+    from vllm_metax_amd.kv_cache_interface import KVQuantMode
+
+    dev = gpu_device
+    code = {"int8": oracle.CODE_INT8, "fp8": oracle.CODE_FP8, "int4": oracle.CODE_INT4}[mode]
+    qmode = {"int8": KVQuantMode.INT8_PER_TOKEN_HEAD, "fp8": KVQuantMode.FP8_PER_TOKEN_HEAD,
+             "int4": KVQuantMode.INT4_PER_TOKEN_HEAD}[mode]
+    dstr = {"int8": "int8_per_token_head", "fp8": "fp8_per_token_head", "int4": "int4_per_token_head"}[mode]
+    bs, nb, n = 16, 12, 70
+    g = torch.Generator().manual_seed(hq + d + rot)
+    q = torch.randn((n, hq, d), generator=g).to(dtype)
+    k = (torch.randn((n, hkv, d), generator=g) * 2).to(dtype)
+    v = torch.randn((n, hkv, d), generator=g).to(dtype)
+    positions = torch.randint(0, 500, (n,), generator=g, dtype=torch.int64)
+    ang = torch.rand((500, rot // 2), generator=g, dtype=torch.float64) * 6.283
+    cos_sin = torch.cat([ang.cos(), ang.sin()], dim=1).to(dtype)
+    slots = torch.randperm(nb * bs, generator=g)[:n].to(torch.int64)
+    slots[torch.rand(n, generator=g) < 0.15] = -1
+    live = slots >= 0
+    # the oracle: rotate the live tokens' first `rot` dims, then write
+    q_want, k_want = q.clone(), k.clone()
+    q_want[live, :, :rot] = oracle.rope_rotate(q[live][..., :rot].contiguous(), positions[live], cos_sin, is_neox)
+    k_want[live, :, :rot] = oracle.rope_rotate(k[live][..., :rot].contiguous(), positions[live], cos_sin, is_neox)
+    kv_cpu, _, lay = T.cpu_cache(nb, bs, hkv, d, "HND", fill=0x22, code_type=code)
+    oracle.cache_write(k_want, v, T.storage_bytes(kv_cpu), lay, slots, code_type=code)
+    kv = L.allocate_kv_cache(nb, bs, hkv, d, device=dev, layout="HND", fill=0x22, cache_dtype_str=dstr)
+    kc, vc = L.key_value_views(kv)
+    ks, vs = L.scale_views(kv)
+    qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
+    ops.rope_and_cache_per_token_head_quant(positions.to(dev), qd, kd, vd, cos_sin.to(dev), is_neox, kc, vc, ks, vs,
+                                            slots.to(dev), kv_quant_mode=qmode)
+    torch.cuda.synchronize()
+    assert torch.equal(qd.cpu(), q_want), "rotated query differs"
+    assert torch.equal(kd.cpu(), k_want), "rotated key differs"
+    assert torch.equal(vd.cpu(), v)
+    got, want = T.storage_bytes(kv).cpu(), T.storage_bytes(kv_cpu)
+    assert torch.equal(got, want), f"{(got != want).sum().item()} cache bytes differ"

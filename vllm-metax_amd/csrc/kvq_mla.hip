@@ -74,36 +74,6 @@ __global__ __launch_bounds__(256) void mla_quant_write_rows8_kernel(const void* 
                 reinterpret_cast<float*>(cache + blk * g.stride_block + g.scale_off + off * 4), lane);
 }
 
-// Round a float to the nearest value of the activation type (the arithmetic type of the rotary
-// embedding below is the activation type, one rounding per operation).
-template <int DT>
-__device__ __forceinline__ float round_act(float v) {
-  if constexpr (DT == KVQ_F32) return v;
-  if constexpr (DT == KVQ_BF16) return bf16_bits_to_f32(f32_to_bf16_bits(v));
-  return (float)(half_t)v;
-}
-
-// (x, y) -> (x cos - y sin, y cos + x sin) in the activation type: every product and every sum is
-// rounded on its own (no fused multiply-add), as the reference's operators on qk_t do
-// (csrc/libtorch_stable/cache_kernels_fused.cu:77-84).  fp16 uses the native half operators (each
-// result correctly rounded); bf16 goes through float and rounds after every operation, which is
-// what the bf16 operators of hip_bf16.h -- the type the reference's ROCm branch selects, :13-16 --
-// do; fp32 is plain fp32 without contraction.
-template <int DT>
-__device__ __forceinline__ void rotate_pair(float x, float y, float c, float s, float& xo, float& yo) {
-#pragma clang fp contract(off)  // the default for device code is to fuse a * b + c, also through __fmul_rn
-  if constexpr (DT == KVQ_F16) {
-    const half_t hx = (half_t)x, hy = (half_t)y, hc = (half_t)c, hs = (half_t)s;
-    const half_t a = hx * hc, b = hy * hs, d = hy * hc, e = hx * hs;
-    xo = (float)(half_t)(a - b);
-    yo = (float)(half_t)(d + e);
-  } else {
-    const float a = round_act<DT>(x * c), b = round_act<DT>(y * s), d = round_act<DT>(y * c), e = round_act<DT>(x * s);
-    xo = round_act<DT>(a - b);
-    yo = round_act<DT>(d + e);
-  }
-}
-
 // Rotary embedding of q_pe and k_pe (in place) fused with the quantise-on-write of the latent row
 // [kv_c | rotated k_pe].  One workgroup per token: all 256 threads rotate the (head, pair) items of
 // q_pe; wave 0 also rotates k_pe (one pair per lane), keeps the rotated values and quantises the

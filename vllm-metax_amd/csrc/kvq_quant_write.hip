@@ -192,6 +192,100 @@ __global__ __launch_bounds__(256) void quant_write_rows_kernel(
   if (li == 0) *reinterpret_cast<float*>(rec + (is_v ? g.vs_off : g.ks_off)) = scale;
 }
 
+// Rotary embedding of the step's query and key rows (in place, the first rot_dim dims of every head) fused with
+// the quantise-on-write of the rotated K rows and the V rows: the work of do_rope_and_kv_cache_update.  One
+// workgroup per token.  All threads rotate the (q head, pair) items; then wave w takes the rows (kv head, K | V)
+// w, w + 4, ...: a lane owns the dim pairs (2 b, 2 b + 1), b = lane, lane + 64, and computes the rotated value of
+// each of its dims from the ORIGINAL row (so no lane reads what another wrote), stores it back into `key` and
+// quantises the row from those values -- the bytes the write kernel would store after a separate rotation.
+// The rotation arithmetic is rotate_pair's (one rounding per operation in the activation type).
+template <int DT, int CT, bool NEOX>
+__global__ __launch_bounds__(256) void rope_quant_write_kernel(
+    const int64_t* __restrict__ positions, void* __restrict__ query, int64_t q_stride_t, int64_t q_stride_h,
+    int num_q_heads, void* __restrict__ key, int64_t k_stride_t, int64_t k_stride_h, const void* __restrict__ value,
+    int64_t v_stride_t, int64_t v_stride_h, const void* __restrict__ cos_sin, int rot_dim,
+    uint8_t* __restrict__ cache, kvq_cache_geom g, const int64_t* __restrict__ slot_mapping, float eps) {
+  const int64_t t = blockIdx.x;
+  const int64_t slot = slot_mapping[t];
+  if (slot < 0) return;  // padding token: nothing is rotated, nothing is written
+  const int64_t pos = positions[t];
+  const int embed = rot_dim / 2;
+  const int64_t cs = pos * rot_dim;
+  auto cosine = [&](int pair) { return round_act<DT>(load_act<CT>(cos_sin, cs + pair)); };
+  auto sine = [&](int pair) { return round_act<DT>(load_act<CT>(cos_sin, cs + pair + embed)); };
+  // ---- query: (head, pair) items over all threads
+  const int nq = num_q_heads * embed;
+  for (int i = threadIdx.x; i < nq; i += blockDim.x) {
+    const int head = i / embed, pair = i - head * embed;
+    const int ix = NEOX ? pair : 2 * pair, iy = NEOX ? embed + pair : 2 * pair + 1;
+    const int64_t base = t * q_stride_t + (int64_t)head * q_stride_h;
+    float xo, yo;
+    rotate_pair<DT>(load_act<DT>(query, base + ix), load_act<DT>(query, base + iy), cosine(pair), sine(pair), xo, yo);
+    store_act<DT>(query, base + ix, xo);
+    store_act<DT>(query, base + iy, yo);
+  }
+  // ---- key / value rows
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x >> 6;
+  const int D = g.head_size;
+  const int64_t blk = slot / g.block_size;
+  const int64_t off = slot - blk * g.block_size;
+  constexpr int kMaxPairs = 2;   // head sizes up to 256
+  for (int r = wave; r < 2 * g.num_kv_heads; r += 4) {
+    const int h = r >> 1, is_v = r & 1;
+    const void* src = is_v ? value : key;
+    const int64_t base = is_v ? t * v_stride_t + (int64_t)h * v_stride_h : t * k_stride_t + (int64_t)h * k_stride_h;
+    // the value of dim d after the rotation (K rows, d < rot_dim) or as it is
+    auto dim_value = [&](int d) -> float {
+      if (is_v || d >= rot_dim) return load_act<DT>(src, base + d);
+      const int pair = NEOX ? (d < embed ? d : d - embed) : d >> 1;
+      const int ix = NEOX ? pair : 2 * pair, iy = NEOX ? embed + pair : 2 * pair + 1;
+      float xo, yo;
+      rotate_pair<DT>(load_act<DT>(src, base + ix), load_act<DT>(src, base + iy), cosine(pair), sine(pair), xo, yo);
+      return d == ix ? xo : yo;
+    };
+    float x[kMaxPairs][2];
+    float amax = 0.f;
+#pragma unroll
+    for (int i = 0; i < kMaxPairs; ++i) {
+      const int b = lane + kWave * i;
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        x[i][j] = 2 * b + j < D ? dim_value(2 * b + j) : 0.f;
+        amax = fmaxf(amax, fabsf(x[i][j]));
+      }
+    }
+    // every lane has read the original row before any lane overwrites it
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    amax = fmaxf(wave_max(amax), eps);
+    const int ct = g.code_type;
+    const float scale = ct == KVQ_CODE_FP8_E4M3 ? amax / 448.0f : (ct == KVQ_CODE_INT4 ? amax / 7.0f : amax / 127.0f);
+    uint8_t* rec = cache + blk * g.stride_block + off * g.stride_slot + (int64_t)h * g.stride_head;
+    uint8_t* codes = rec + (is_v ? g.v_off : g.k_off);
+#pragma unroll
+    for (int i = 0; i < kMaxPairs; ++i) {
+      const int b = lane + kWave * i;
+      if (2 * b >= D) continue;
+      uint32_t c[2];
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const float y = scale > 0.f ? x[i][j] / scale : 0.f;
+        if (ct == KVQ_CODE_FP8_E4M3) c[j] = f32_to_e4m3fn_bits(y);
+        else if (ct == KVQ_CODE_INT4) c[j] = (uint32_t)(int)fminf(fmaxf(rintf(y), -8.f), 7.f) & 0xfu;
+        else c[j] = (uint32_t)(int)fminf(fmaxf(rintf(y), -128.f), 127.f) & 0xffu;
+      }
+      if (ct == KVQ_CODE_INT4) codes[b] = (uint8_t)(c[0] | (c[1] << 4));
+      else *reinterpret_cast<uint16_t*>(codes + 2 * b) = (uint16_t)(c[0] | (c[1] << 8));
+      if (!is_v && 2 * b < rot_dim) {   // the rotated key goes back in place
+        store_act<DT>(key, base + 2 * b, x[i][0]);
+        store_act<DT>(key, base + 2 * b + 1, x[i][1]);
+      }
+    }
+    if (lane == 0) *reinterpret_cast<float*>(rec + (is_v ? g.vs_off : g.ks_off)) = scale;
+  }
+}
+
+
 template <int DT>
 static int launch_quant_write(const void* key, const void* value, int64_t kst, int64_t ksh,
                               int64_t vst, int64_t vsh, uint8_t* cache, const kvq_cache_geom& g,
@@ -274,4 +368,61 @@ extern "C" int kvq_reshape_and_cache_int8(const void* key, const void* value, in
     default:
       return fail(KVQ_EINVAL, "reshape_and_cache_int8: unknown src_dtype %d", src_dtype);
   }
+}
+
+extern "C" int kvq_rope_and_cache_int8(const int64_t* positions, void* query, int64_t q_stride_t, int64_t q_stride_h,
+                                       int num_q_heads, void* key, int64_t key_stride_t, int64_t key_stride_h,
+                                       const void* value, int64_t value_stride_t, int64_t value_stride_h,
+                                       int src_dtype, const void* cos_sin_cache, int cos_sin_dtype, int rot_dim,
+                                       int is_neox, void* cache, const kvq_cache_geom* geom,
+                                       const int64_t* slot_mapping, int64_t num_tokens, float eps,
+                                       kvq_stream_t stream) {
+  using namespace kvq;
+  const char* op = "rope_and_cache_int8";
+  KVQ_REQUIRE(geom != nullptr, "%s: geom is NULL", op);
+  KVQ_REQUIRE(num_tokens >= 0 && num_tokens <= 0x7fffffffLL, "%s: num_tokens out of range", op);
+  if (num_tokens == 0) return KVQ_OK;
+  KVQ_REQUIRE(positions && query && key && value && cos_sin_cache && cache && slot_mapping, "%s: NULL pointer", op);
+  const kvq_cache_geom& g = *geom;
+  KVQ_REQUIRE(g.num_kv_heads > 0 && g.block_size > 0 && g.head_size > 0 && g.head_size % 2 == 0 && g.head_size <= 256,
+              "%s: bad geometry (heads=%d head_size=%d block_size=%d; head sizes up to 256)", op, g.num_kv_heads,
+              g.head_size, g.block_size);
+  KVQ_REQUIRE(num_q_heads > 0, "%s: num_q_heads must be positive", op);
+  KVQ_REQUIRE(rot_dim > 0 && rot_dim % 2 == 0 && rot_dim <= g.head_size, "%s: rot_dim %d must be even and at most the head size %d",
+              op, rot_dim, g.head_size);
+  KVQ_REQUIRE((g.k_off | g.v_off | g.ks_off | g.vs_off | g.stride_block | g.stride_slot | g.stride_head) % 4 == 0 &&
+                  ((uintptr_t)cache % 4) == 0, "%s: cache offsets/strides must be 4-byte aligned", op);
+  KVQ_REQUIRE(g.code_type == KVQ_CODE_INT8 || g.code_type == KVQ_CODE_FP8_E4M3 || g.code_type == KVQ_CODE_INT4,
+              "%s: unknown code_type %d", op, g.code_type);
+  KVQ_REQUIRE(eps >= 0.f, "%s: eps must not be negative", op);
+  hipStream_t s = as_stream(stream);
+  uint8_t* c = static_cast<uint8_t*>(cache);
+  const dim3 grid((unsigned)num_tokens), block(256);
+#define KVQ_ROPE(D, C)                                                                                              \
+  do {                                                                                                              \
+    if (is_neox)                                                                                                    \
+      hipLaunchKernelGGL((rope_quant_write_kernel<D, C, true>), grid, block, 0, s, positions, query, q_stride_t,   \
+                         q_stride_h, num_q_heads, key, key_stride_t, key_stride_h, value, value_stride_t,           \
+                         value_stride_h, cos_sin_cache, rot_dim, c, g, slot_mapping, eps);                          \
+    else                                                                                                            \
+      hipLaunchKernelGGL((rope_quant_write_kernel<D, C, false>), grid, block, 0, s, positions, query, q_stride_t,  \
+                         q_stride_h, num_q_heads, key, key_stride_t, key_stride_h, value, value_stride_t,           \
+                         value_stride_h, cos_sin_cache, rot_dim, c, g, slot_mapping, eps);                          \
+  } while (0)
+#define KVQ_ROPE_C(D)                                                                        \
+  switch (cos_sin_dtype) {                                                                   \
+    case KVQ_F32: KVQ_ROPE(D, KVQ_F32); break;                                               \
+    case KVQ_BF16: KVQ_ROPE(D, KVQ_BF16); break;                                             \
+    case KVQ_F16: KVQ_ROPE(D, KVQ_F16); break;                                               \
+    default: return fail(KVQ_EINVAL, "%s: unknown cos_sin_dtype %d", op, cos_sin_dtype);     \
+  }
+  switch (src_dtype) {
+    case KVQ_F32: KVQ_ROPE_C(KVQ_F32); break;
+    case KVQ_BF16: KVQ_ROPE_C(KVQ_BF16); break;
+    case KVQ_F16: KVQ_ROPE_C(KVQ_F16); break;
+    default: return fail(KVQ_EINVAL, "%s: unknown src_dtype %d", op, src_dtype);
+  }
+#undef KVQ_ROPE_C
+#undef KVQ_ROPE
+  return check_hip(hipGetLastError(), "rope_and_cache_int8 launch");
 }

@@ -159,6 +159,59 @@ def reshape_and_cache_flash_per_token_head_quant(
 triton_reshape_and_cache_flash_per_token_head_quant = reshape_and_cache_flash_per_token_head_quant
 
 
+def rope_and_cache_per_token_head_quant(
+    positions: torch.Tensor,
+    query: torch.Tensor,
+    key: torch.Tensor,
+    value: torch.Tensor,
+    cos_sin_cache: torch.Tensor,
+    is_neox: bool,
+    key_cache: torch.Tensor,
+    value_cache: torch.Tensor,
+    k_scale_cache: torch.Tensor,
+    v_scale_cache: torch.Tensor,
+    slot_mapping: torch.Tensor,
+    kv_quant_mode: KVQuantMode = KVQuantMode.INT8_PER_TOKEN_HEAD,
+    geometry: CacheGeometry | None = None,
+) -> None:
+    """Rotary embedding of ``query`` ``[T, Hq, D]`` and ``key`` ``[T, Hkv, D]`` (in place, their first ``rot_dim =
+    cos_sin_cache.shape[1]`` dims) and the quantise-on-write of the rotated ``key`` and of ``value`` in ONE launch:
+    the work of ``do_rope_and_kv_cache_update``, which the reference's backend declares and refuses
+    (vllm_metax/v1/attention/backends/triton_attn.py:833-848).  Same results as the rotary embedding followed by
+    ``reshape_and_cache_flash_per_token_head_quant``; tokens whose slot is negative are neither rotated nor
+    written."""
+    code_type = code_type_of(kv_quant_mode)
+    dev = _require_cuda(positions, query, key, value, cos_sin_cache, key_cache, value_cache, k_scale_cache,
+                        v_scale_cache, slot_mapping)
+    geom = (geometry or geometry_from_views(key_cache, value_cache, k_scale_cache, v_scale_cache)).with_code_type(code_type)
+    if query.dim() != 3 or key.dim() != 3 or value.dim() != 3 or not (query.dtype == key.dtype == value.dtype):
+        raise RuntimeError("query [T, Hq, D], key and value [T, Hkv, D] must share one dtype")
+    if key.shape != value.shape or key.shape[1] != geom.num_kv_heads or key.shape[2] != geom.head_size \
+            or query.shape[2] != geom.head_size:
+        raise RuntimeError(f"query / key / value shapes do not match the cache (Hkv={geom.num_kv_heads}, D={geom.head_size})")
+    if query.stride(2) != 1 or key.stride(2) != 1 or value.stride(2) != 1:
+        raise RuntimeError("query / key / value rows must be contiguous")
+    if cos_sin_cache.dim() != 2 or not cos_sin_cache.is_contiguous():
+        raise RuntimeError("cos_sin_cache must be a contiguous [max_position, rot_dim] tensor")
+    rot = cos_sin_cache.shape[1]
+    if rot % 2 or rot > geom.head_size:
+        raise RuntimeError("rot_dim must be even and at most the head size")
+    for name, t in (("positions", positions), ("slot_mapping", slot_mapping)):
+        if t.dtype != torch.int64 or not t.is_contiguous():
+            raise RuntimeError(f"{name} must be contiguous int64")
+    T = slot_mapping.shape[0]
+    if positions.shape[0] < T or query.shape[0] < T or key.shape[0] < T:
+        raise RuntimeError("slot_mapping is longer than positions / query / key")
+    g = geom.as_struct()
+    with _on_device(dev):
+        rc = _C.load().kvq_rope_and_cache_int8(
+            _ptr(positions), _ptr(query), query.stride(0), query.stride(1), query.shape[1], _ptr(key), key.stride(0),
+            key.stride(1), _ptr(value), value.stride(0), value.stride(1), _dtype_code(key, "key"), _ptr(cos_sin_cache),
+            _dtype_code(cos_sin_cache, "cos_sin_cache"), rot, 1 if is_neox else 0, ctypes.c_void_p(geom.base_ptr),
+            ctypes.byref(g), _ptr(slot_mapping), T, eps_for_dtype(key.dtype), _stream(dev))
+    _C.check(rc, "rope_and_cache_per_token_head_quant")
+
+
 # ---------------------------------------------------------------------------------------------
 # attention
 # ---------------------------------------------------------------------------------------------

@@ -318,7 +318,24 @@ class Int8AttentionImpl(_ImplBase):
         return False
 
     def fused_rope_kvcache_supported(self) -> bool:
-        return False
+        """The reference answers False and raises in the method below (triton_attn.py:833-848); here the rotary
+        embedding and the cache update are one launch."""
+        return True
+
+    def do_rope_and_kv_cache_update(self, layer, query: torch.Tensor, key: torch.Tensor, value: torch.Tensor,
+                                    positions: torch.Tensor, cos_sin_cache: torch.Tensor, is_neox: bool,
+                                    kv_cache: torch.Tensor, layer_slot_mapping: torch.Tensor) -> None:
+        """Signature of triton_attn.py:836-848.  ``query`` / ``key`` ``[T, H * D]`` or ``[T, H, D]`` are rotated in
+        place, the rotated ``key`` and ``value`` quantised into ``kv_cache``."""
+        if self.attn_type in (AttentionType.ENCODER_ONLY, AttentionType.ENCODER):
+            return
+        key_cache, value_cache = self._pth_key_value_caches(kv_cache)
+        n = query.shape[0]
+        ops.rope_and_cache_per_token_head_quant(
+            positions, query.view(n, self.num_heads, self.head_size), key.view(n, self.num_kv_heads, self.head_size),
+            value.view(n, self.num_kv_heads, self.head_size), cos_sin_cache, is_neox, key_cache, value_cache,
+            self._k_scale_cache, self._v_scale_cache, layer_slot_mapping, kv_quant_mode=self._kv_quant_mode,
+            geometry=self._geometry)
 
     # -- cache views ---------------------------------------------------------------------------
     def _ensure_scale_caches(self, kv_cache: torch.Tensor) -> None:
