@@ -27,7 +27,7 @@
 extern "C" {
 #endif
 
-#define KVQ_ABI_VERSION 15
+#define KVQ_ABI_VERSION 16
 
 #define KVQ_OK 0
 #define KVQ_EINVAL (-22)
@@ -192,6 +192,11 @@ KVQ_API int kvq_rope_and_cache_int8(const int64_t* positions, void* query, int64
  * (triton_attn.py:703; semantics as in the reference's test oracle,
  * tests/kernels/attention/test_triton_unified_attention.py:63-70); 0 = none.
  *
+ * sinks (optional, [num_q_heads] fp32, may be NULL): attention sinks, the `sinks` argument of the reference's
+ * unified_attention call (triton_attn.py:712, 784; supports_sink(), :390-392).  Head h's softmax runs over its
+ * keys' logits and one more logit, sinks[h] (as given: not multiplied by `scale`), whose value row is zero:
+ * out = sum_j exp(s_j) v_j / (exp(sinks[h]) + sum_j exp(s_j)); lse includes the sink's term.
+ *
  * `causal` is a set of flags: KVQ_ATTN_CAUSAL (1, the reference's causal=True) and, optionally,
  * KVQ_ATTN_NO_DECODE_ROWS (2): the caller's promise that no sequence of this batch has exactly one query
  * row (a pure prefill batch; a metadata builder knows it from the host copy of query_start_loc).  The
@@ -210,7 +215,7 @@ KVQ_API int kvq_paged_attn_int8(void* out, int out_dtype, int64_t out_stride_t, 
                         const int32_t* block_table, int64_t bt_stride, const int32_t* seq_lens,
                         const int32_t* cu_seqlens_q, int num_seqs, int num_q_heads,
                         int max_query_len, float scale, int causal, int window_size,
-                        float softcap, float* lse, void* workspace, size_t workspace_bytes,
+                        float softcap, const float* sinks, float* lse, void* workspace, size_t workspace_bytes,
                         kvq_stream_t stream);
 
 /*
@@ -241,7 +246,7 @@ KVQ_API int kvq_paged_attn_int8_fused_write(void* out, int out_dtype, int64_t ou
                         const int32_t* block_table, int64_t bt_stride, const int32_t* seq_lens,
                         const int64_t* slot_mapping,
                         int num_seqs, int num_q_heads, float scale, int window_size,
-                        float softcap, float* lse, void* workspace, size_t workspace_bytes,
+                        float softcap, const float* sinks, float* lse, void* workspace, size_t workspace_bytes,
                         kvq_stream_t stream);
 
 /*
@@ -271,7 +276,7 @@ KVQ_API int kvq_paged_attn_int8_static_scratch(
     int64_t q_stride_t, int64_t q_stride_h, const void* cache, const kvq_cache_geom* geom,
     const int32_t* block_table, int64_t bt_stride, const int32_t* seq_lens, const int32_t* cu_seqlens_q,
     int num_seqs, int num_q_heads, int max_query_len, float scale, int causal, int window_size,
-    float softcap, float* lse, kvq_stream_t stream);
+    float softcap, const float* sinks, float* lse, kvq_stream_t stream);
 
 /*
  * Fixed-partition split-K decode + reduce (one query row per sequence).

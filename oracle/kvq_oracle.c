@@ -323,6 +323,18 @@ static void attend_range(const float* q, int D, const uint8_t* cache,
 /* window > 0: a query at position p sees keys p - window + 1 .. p only (the
  * sliding_window mask of ref_paged_attn, :60-66).  softcap > 0: scaled logits
  * become softcap * tanh(logit / softcap) before masking (:67-68).           */
+/* sinks != NULL: attention sinks, [Hq] fp32.  Head h's softmax gets one more logit, sinks[h] (not scaled), with a
+ * zero value row: out = sum_j exp(s_j) v_j / (exp(sinks[h]) + sum_j exp(s_j)), lse = log of that denominator.
+ * The definition of the `sinks` argument of upstream's unified_attention, which the reference passes through
+ * (vllm_metax/v1/attention/backends/triton_attn.py:712, 784); rows without a visible key stay zeros / -inf.  */
+KVQ_EXPORT int kvq_oracle_paged_attn_ex3(
+    float* out, float* lse, const float* q, const uint8_t* cache,
+    int64_t k_off, int64_t v_off, int64_t ks_off, int64_t vs_off,
+    int64_t stride_block, int64_t stride_slot, int64_t stride_head,
+    const int32_t* block_table, int64_t bt_stride, const int32_t* seq_lens,
+    const int32_t* cu_seqlens_q, int B, int Hq, int Hkv, int D, int block_size,
+    float scale, int causal, int window, float softcap, int code_type, const float* sinks);
+
 KVQ_EXPORT int kvq_oracle_paged_attn_ex2(
     float* out, float* lse, const float* q, const uint8_t* cache,
     int64_t k_off, int64_t v_off, int64_t ks_off, int64_t vs_off,
@@ -330,6 +342,18 @@ KVQ_EXPORT int kvq_oracle_paged_attn_ex2(
     const int32_t* block_table, int64_t bt_stride, const int32_t* seq_lens,
     const int32_t* cu_seqlens_q, int B, int Hq, int Hkv, int D, int block_size,
     float scale, int causal, int window, float softcap, int code_type) {
+  return kvq_oracle_paged_attn_ex3(out, lse, q, cache, k_off, v_off, ks_off, vs_off, stride_block, stride_slot,
+                                   stride_head, block_table, bt_stride, seq_lens, cu_seqlens_q, B, Hq, Hkv, D,
+                                   block_size, scale, causal, window, softcap, code_type, NULL);
+}
+
+KVQ_EXPORT int kvq_oracle_paged_attn_ex3(
+    float* out, float* lse, const float* q, const uint8_t* cache,
+    int64_t k_off, int64_t v_off, int64_t ks_off, int64_t vs_off,
+    int64_t stride_block, int64_t stride_slot, int64_t stride_head,
+    const int32_t* block_table, int64_t bt_stride, const int32_t* seq_lens,
+    const int32_t* cu_seqlens_q, int B, int Hq, int Hkv, int D, int block_size,
+    float scale, int causal, int window, float softcap, int code_type, const float* sinks) {
   if (!out || !q || !cache || !block_table || !seq_lens || !cu_seqlens_q) return -1;
   if (Hkv <= 0 || Hq % Hkv != 0) return -1;
   const int G = Hq / Hkv;
@@ -369,6 +393,17 @@ KVQ_EXPORT int kvq_oracle_paged_attn_ex2(
                          ks_off, vs_off, stride_block, stride_slot, stride_head,
                          block_table + (int64_t)i * bt_stride, block_size, h / G, first, vis,
                          (double)scale, (double)softcap, acc, &m, &l, logits, code_type);
+            if (sinks) {   /* one more logit with a zero value row */
+              const double sk = (double)sinks[h];
+              if (sk > m) {
+                const double f = exp(m - sk);
+                for (int d = 0; d < D; ++d) acc[d] *= f;
+                l = l * f + 1.0;
+                m = sk;
+              } else {
+                l += exp(sk - m);
+              }
+            }
             for (int d = 0; d < D; ++d) o[d] = (float)(acc[d] / l);
             if (lse) lse[(q0 + r) * Hq + h] = (float)(m + log(l));
           }

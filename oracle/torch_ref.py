@@ -50,8 +50,10 @@ def dequant_cache(key_cache, value_cache, k_scale_cache, v_scale_cache, head_siz
 
 
 def paged_attn(query, key_cache, value_cache, query_lens, kv_lens, block_tables, scale,
-               sliding_window=None, soft_cap=None):
+               sliding_window=None, soft_cap=None, sinks=None):
     """tests/kernels/attention/test_triton_unified_attention.py:26-78 (ref_paged_attn).
+    ``sinks`` ``[Hq]`` (not in the reference's copy of that test; the definition of upstream's argument): the
+    softmax runs over the masked logits and one more column holding ``sinks[h]``, which is dropped afterwards.
 
     key_cache/value_cache: dequantised (nb, bs, Hkv, D) in the query dtype.
     The reference op scales ``query`` in place; a scaled copy is used instead so the
@@ -77,7 +79,11 @@ def paged_attn(query, key_cache, value_cache, query_lens, kv_lens, block_tables,
         if soft_cap:
             logits = soft_cap * torch.tanh(logits / soft_cap)
         logits.masked_fill_(hide, float("-inf"))
-        probs = torch.softmax(logits, dim=-1).to(v.dtype)
+        if sinks is not None:
+            col = sinks.float().reshape(-1, 1, 1).expand(-1, ql, 1)
+            probs = torch.softmax(torch.cat([logits, col], dim=-1), dim=-1)[..., :-1].to(v.dtype)
+        else:
+            probs = torch.softmax(logits, dim=-1).to(v.dtype)
         outs.append(torch.einsum("hqk,khd->qhd", probs, v))
     return torch.cat(outs, dim=0)
 

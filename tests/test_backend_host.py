@@ -190,9 +190,13 @@ def test_impl_constructor_errors():
     mk = lambda **kw: Int8AttentionImpl(32, 128, 0.088, 8, **kw)
     impl = mk()
     assert impl.num_queries_per_kv == 4 and impl.fused_rope_kvcache_supported() is True   # built here; the reference answers False
-    for kw in (dict(alibi_slopes=[1.0] * 32), dict(sinks=torch.zeros(32)), dict(attn_type=AttentionType.ENCODER_ONLY)):
+    for kw in (dict(alibi_slopes=[1.0] * 32), dict(attn_type=AttentionType.ENCODER_ONLY)):
         with pytest.raises(NotImplementedError):
             mk(**kw)
+    # attention sinks: one per q head, kept as float32 (triton_attn.py:548-554)
+    assert mk(sinks=torch.zeros(32, dtype=torch.bfloat16)).sinks.dtype == torch.float32
+    with pytest.raises(ValueError):
+        mk(sinks=torch.zeros(8))
     # the reference's mapping of the two knobs (triton_attn.py:507-512, 536-539)
     assert impl.sliding_window == (-1, -1) and impl.logits_soft_cap == 0
     w = mk(sliding_window=128, logits_soft_cap=30.0)

@@ -105,6 +105,41 @@ def test_sliding_window_and_soft_cap_vs_as_written_reference_op(window, cap):
     torch.testing.assert_close(big, plain, atol=1e-5, rtol=1e-5)
 
 
+@pytest.mark.parametrize("window,cap", [(0, 0.0), (40, 0.0), (0, 20.0)])
+def test_attention_sinks_vs_softmax_over_one_more_column(window, cap):
+    """Attention sinks (the `sinks` argument the reference passes to unified_attention,
+    vllm_metax/v1/attention/backends/triton_attn.py:712): the oracle against torch's softmax over the logits and
+    one more column that is dropped afterwards; closed forms: a sink of -inf changes nothing, a sink equal to a
+    single key's logit halves that row, a huge sink empties the output; lse = logsumexp over logits and sink."""
+    hq, hkv, d, bs = 8, 2, 64, 16
+    ctx, ql = [100, 463, 18, 1], [1, 129, 5, 1]
+    kv, views, lay, bt, q, cu, sl = _build(ctx, ql, hq, hkv, d, bs, "NHD", 23)
+    scale = d ** -0.5
+    sinks = torch.linspace(-3.0, 4.0, hq)
+    out, lse = oracle.paged_attn(q, T.storage_bytes(kv), lay, bt, sl, cu, scale, sliding_window=window, soft_cap=cap,
+                                 sinks=sinks, return_lse=True)
+    k, v, ks, vs = views
+    kd, vd = torch_ref.dequant_cache(k, v, ks, vs, d, torch.float32)
+    want = torch_ref.paged_attn(q.float(), kd, vd, ql, ctx, bt, scale, sliding_window=window or None,
+                                soft_cap=cap or None, sinks=sinks)
+    torch.testing.assert_close(out, want, atol=3e-5, rtol=1e-5)
+    plain, plain_lse = oracle.paged_attn(q, T.storage_bytes(kv), lay, bt, sl, cu, scale, sliding_window=window,
+                                         soft_cap=cap, return_lse=True)
+    # out = plain * exp(plain_lse - lse), lse = logaddexp(plain_lse, sink): the sink only enlarges the denominator
+    torch.testing.assert_close(lse, torch.logaddexp(plain_lse, sinks[None, :].expand_as(plain_lse)), atol=2e-5, rtol=1e-5)
+    torch.testing.assert_close(out, plain * torch.exp(plain_lse - lse)[..., None], atol=3e-5, rtol=1e-5)
+    none = oracle.paged_attn(q, T.storage_bytes(kv), lay, bt, sl, cu, scale, sliding_window=window, soft_cap=cap,
+                             sinks=torch.full((hq,), float("-inf")))
+    assert torch.equal(none, plain)
+    huge = oracle.paged_attn(q, T.storage_bytes(kv), lay, bt, sl, cu, scale, sliding_window=window, soft_cap=cap,
+                             sinks=torch.full((hq,), 80.0))
+    assert huge.abs().max() < 1e-20
+    # the last sequence has ONE key: with the sink equal to that key's logit the row is half the value row
+    one = oracle.paged_attn(q[-1:], T.storage_bytes(kv), lay, bt[-1:], sl[-1:], torch.tensor([0, 1], dtype=torch.int32),
+                            scale, sliding_window=window, soft_cap=cap, sinks=plain_lse[-1])
+    torch.testing.assert_close(one, plain[-1:] * 0.5, atol=1e-6, rtol=1e-5)
+
+
 def test_block_permutation_invariance_and_noncausal():
     hq, hkv, d, bs = 4, 2, 64, 16
     ctx, ql = [50, 33], [1, 3]

@@ -161,6 +161,7 @@ struct AttnIO {
   float scale_log2;  // softmax scale * log2(e)
   uint32_t bs_magic;  // ceil(2^32 / block_size): x / block_size == umulhi(x, bs_magic) for x < 2^22
   int window;         // sliding window: a query sees its last `window` keys, itself included; 0 = all
+  const float* sinks; // [num_q_heads] attention sinks (natural-log logits) or nullptr
   float cap_c;        // logits soft cap in the log2 domain, cap * log2(e); 0 = none
   float cap_k;        // 2 * log2(e) / cap_c
 };
@@ -180,6 +181,12 @@ __device__ __forceinline__ float soft_cap(float x, float cap_c, float cap_k) {
 // First token a decode row of a `len`-token sequence sees.
 __device__ __forceinline__ int window_first(int len, int window) {
   return window > 0 && len > window ? len - window : 0;
+}
+
+// The sink's share of a head's softmax sum: exp(sink - max) with the running maximum `m` in the log2 domain
+// (0 without sinks).  Added once, where a row's sum is final.
+__device__ __forceinline__ float sink_term(const float* sinks, int head, float m) {
+  return sinks != nullptr ? __builtin_amdgcn_exp2f(sinks[head] * kLog2e - m) : 0.f;
 }
 
 // One lane's share of a 32-token tile as it arrives from HBM: raw 16-byte chunks of records.
@@ -816,10 +823,11 @@ struct DecodeTile {
   }
   template <int OT>
   __device__ static void emit_final_as(const AttnIO& io, int64_t row, int hkv, int lane, const State& st) {
-    const float l = total_l(st);  // every lane takes part in the shuffles
+    float l = total_l(st);  // every lane takes part in the shuffles
     const int c = lane & 15, g = lane >> 4;
     if (c >= io.group) return;
     const int head = hkv * io.group + c;
+    l += sink_term(io.sinks, head, st.m);
     float v[D / 4];
     gather_row(st, 1.0f / (l * kOutDiv), v);
     const int64_t base = row * io.out_stride_t + (int64_t)head * io.out_stride_h + g * (D / 4);

@@ -66,8 +66,8 @@ static int paged_attn_launch(const char* op, void* out, int out_dtype, int64_t o
                              const void* q, int q_dtype, int64_t q_stride_t, int64_t q_stride_h, const void* cache,
                              const kvq_cache_geom* geom, const int32_t* block_table, int64_t bt_stride,
                              const int32_t* seq_lens, const int32_t* cu_seqlens_q, int num_seqs, int num_q_heads,
-                             int max_query_len, float scale, int causal, int window_size, float softcap, float* lse,
-                             void* workspace, size_t workspace_bytes, const char* workspace_what,
+                             int max_query_len, float scale, int causal, int window_size, float softcap,
+                             const float* sinks, float* lse, void* workspace, size_t workspace_bytes, const char* workspace_what,
                              kvq_stream_t stream, const NewTokens* fresh = nullptr) {
   int rc0 = validate_common(op, q, cache, geom, block_table, seq_lens, num_seqs, num_q_heads);
   if (rc0) return rc0;
@@ -108,6 +108,7 @@ static int paged_attn_launch(const char* op, void* out, int out_dtype, int64_t o
   a.io.scale_log2 = scale * kLog2e;
   a.io.bs_magic = (uint32_t)((0x100000000ull + (uint64_t)geom->block_size - 1) / (uint64_t)geom->block_size);
   a.io.window = window_size;
+  a.io.sinks = sinks;
   a.io.cap_c = softcap * kLog2e;
   a.io.cap_k = softcap > 0.f ? 2.0f / softcap : 0.f;  // 2 log2(e) / cap_c
   a.seq_lens = seq_lens;
@@ -164,11 +165,11 @@ extern "C" int kvq_paged_attn_int8(void* out, int out_dtype, int64_t out_stride_
                                    const void* cache, const kvq_cache_geom* geom, const int32_t* block_table,
                                    int64_t bt_stride, const int32_t* seq_lens, const int32_t* cu_seqlens_q,
                                    int num_seqs, int num_q_heads, int max_query_len, float scale, int causal,
-                                   int window_size, float softcap, float* lse, void* workspace,
+                                   int window_size, float softcap, const float* sinks, float* lse, void* workspace,
                                    size_t workspace_bytes, kvq_stream_t stream) {
   return kvq::paged_attn_launch("paged_attn_int8", out, out_dtype, out_stride_t, out_stride_h, q, q_dtype, q_stride_t,
                                 q_stride_h, cache, geom, block_table, bt_stride, seq_lens, cu_seqlens_q, num_seqs,
-                                num_q_heads, max_query_len, scale, causal, window_size, softcap, lse, workspace,
+                                num_q_heads, max_query_len, scale, causal, window_size, softcap, sinks, lse, workspace,
                                 workspace_bytes, "workspace", stream);
 }
 
@@ -181,13 +182,13 @@ extern "C" int kvq_paged_attn_int8_fused_write(void* out, int out_dtype, int64_t
                                                int64_t bt_stride, const int32_t* seq_lens,
                                                const int64_t* slot_mapping, int num_seqs,
                                                int num_q_heads, float scale, int window_size, float softcap,
-                                               float* lse, void* workspace, size_t workspace_bytes,
+                                               const float* sinks, float* lse, void* workspace, size_t workspace_bytes,
                                                kvq_stream_t stream) {
   const kvq::NewTokens fresh{key, value, src_dtype, key_stride_t, key_stride_h, value_stride_t, value_stride_h, eps,
                              slot_mapping};
   return kvq::paged_attn_launch("paged_attn_int8_fused_write", out, out_dtype, out_stride_t, out_stride_h, q, q_dtype,
                                 q_stride_t, q_stride_h, cache, geom, block_table, bt_stride, seq_lens, nullptr, num_seqs,
-                                num_q_heads, 1, scale, 1, window_size, softcap, lse, workspace, workspace_bytes,
+                                num_q_heads, 1, scale, 1, window_size, softcap, sinks, lse, workspace, workspace_bytes,
                                 "workspace", stream, &fresh);
 }
 
@@ -206,7 +207,8 @@ extern "C" int kvq_paged_attn_int8_static_scratch(void* out, int out_dtype, int6
                                                   int64_t bt_stride, const int32_t* seq_lens,
                                                   const int32_t* cu_seqlens_q, int num_seqs, int num_q_heads,
                                                   int max_query_len, float scale, int causal, int window_size,
-                                                  float softcap, float* lse, kvq_stream_t stream) {
+                                                  float softcap, const float* sinks, float* lse,
+                                                  kvq_stream_t stream) {
   const char* op = "paged_attn_int8_static_scratch";
   kvq::DeviceSymbols sym;
   const int rc = kvq::device_symbols(op, &sym);
@@ -216,7 +218,7 @@ extern "C" int kvq_paged_attn_int8_static_scratch(void* out, int out_dtype, int6
   // launch's main kernel first (slots it does not own are masked out bit-wise, whatever they hold).
   return kvq::paged_attn_launch(op, out, out_dtype, out_stride_t, out_stride_h, q, q_dtype, q_stride_t, q_stride_h,
                                 cache, geom, block_table, bt_stride, seq_lens, cu_seqlens_q, num_seqs, num_q_heads,
-                                max_query_len, scale, causal, window_size, softcap, lse, ptr,
+                                max_query_len, scale, causal, window_size, softcap, sinks, lse, ptr,
                                 KVQ_STATIC_SCRATCH_BYTES,
                                 "batch too large for the built-in scratch: split-K state", stream);
 }

@@ -339,11 +339,12 @@ __global__ __launch_bounds__(256) void paged_decode_fixed_spans_reduce_kernel(St
       for (int i = 0; i < V; ++i) acc[i] += as_f32(as_u32(po[k][i]) & kk) * wk;
     }
   }
-  const float inv = 1.0f / l;
+  const float lt = l + sink_term(a.io.sinks, head, m);
+  const float inv = 1.0f / lt;
 #pragma unroll
   for (int i = 0; i < V; ++i)
     store_act_rt(a.io.out_dtype, a.io.out, row * a.io.out_stride_t + (int64_t)head * a.io.out_stride_h + lane * V + i, acc[i] * inv);
-  if (a.io.lse != nullptr && lane == 0) a.io.lse[row * Hq + head] = (m + __builtin_amdgcn_logf(l)) * kLn2;
+  if (a.io.lse != nullptr && lane == 0) a.io.lse[row * Hq + head] = (m + __builtin_amdgcn_logf(lt)) * kLn2;
 }
 
 // Merge the partial states of every decode sequence that more than one workgroup touched, and give empty decode
@@ -451,6 +452,7 @@ __global__ __launch_bounds__(256) void paged_decode_streamk_reduce_kernel(Stream
         }
       }
     }
+    l += sink_term(a.io.sinks, h1, m);
     const float inv = 1.0f / l;
 #pragma unroll
     for (int i = 0; i < V2; ++i)
@@ -523,6 +525,7 @@ __global__ __launch_bounds__(256) void paged_decode_streamk_reduce_kernel(Stream
   } else {
     for (int wb = w_first; wb <= w_last; wb += kLong) pass(wb, std::integral_constant<int, kLong>{});
   }
+  l += sink_term(a.io.sinks, head, m);
   const float inv = 1.0f / l;
 #pragma unroll
   for (int i = 0; i < V; ++i) acc[i] *= inv;
@@ -654,6 +657,7 @@ __global__ __launch_bounds__(256) void paged_decode_streamk_reduce_by_seq_kernel
       }
     }
   }
+  l += sink_term(a.io.sinks, head, m);
   const float inv = 1.0f / l;
 #pragma unroll
   for (int i = 0; i < V; ++i)
@@ -768,6 +772,7 @@ __global__ __launch_bounds__(256) void paged_decode_streamk_reduce_split4_kernel
 #pragma unroll
     for (int x = 0; x < V; ++x) acc[x] = acc[x] * ca + sh_acc[p][x][lane] * cb;
   }
+  l += sink_term(a.io.sinks, head, m);
   const float inv = 1.0f / l;
 #pragma unroll
   for (int x = 0; x < V; ++x)

@@ -231,6 +231,7 @@ struct PrefillTile {
     l += __shfl_xor(l, 16, kWave);
     l += __shfl_xor(l, 32, kWave);
     if (!valid) return;
+    if (l > 0.f) l += sink_term(io.sinks, head, st.m[nt]);   // a row without a visible key keeps its zeros
     const int g = lane >> 4;
     const float mul = l > 0.f ? 1.0f / (l * DTile::kOutDiv) : 0.f;   // no visible key: zeros
     const float corr = FP8 ? 0.f : DTile::kBias * st.psum[nt][0];
@@ -857,6 +858,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   // Lane (c, g) holds O[column][dim mt*32 + (i/4)*8 + 4g + i%4] in o[mt][i].
   l += __shfl_xor(l, 32, kWave);
   if (!valid) return;
+  if (l > 0.f) l += sink_term(io.sinks, head, m);   // a row without a visible key keeps its zeros
   const int g = lane >> 5;
   const float mul = l > 0.f ? 1.0f / (l * DTile::kOutDiv) : 0.f;
   const int64_t base = row * io.out_stride_t + (int64_t)head * io.out_stride_h + 4 * g;

@@ -206,7 +206,7 @@ class Int8AttentionBackend(_BackendBase):
 
     @classmethod
     def supports_sink(cls) -> bool:
-        return False
+        return True   # triton_attn.py:390-392
 
     @classmethod
     def supports_batch_invariance(cls) -> bool:
@@ -241,8 +241,6 @@ class Int8AttentionBackend(_BackendBase):
             reasons.append("block_size not supported")
         if not cls.supports_attn_type(attn_type):
             reasons.append("attention type not supported")
-        if has_sink:
-            reasons.append("sink setting not supported")
         return reasons
 
     @staticmethod
@@ -277,7 +275,7 @@ class Int8AttentionImpl(_ImplBase):
                  attn_type: str = AttentionType.DECODER, kv_sharing_target_layer_name: str | None = None,
                  sinks: torch.Tensor | None = None, use_alibi_sqrt: bool = False, chunk_lookback: int = -1) -> None:
         unsupported = {
-            "alibi_slopes": alibi_slopes is not None, "sinks": sinks is not None,
+            "alibi_slopes": alibi_slopes is not None,
             "kv_sharing_target_layer_name": kv_sharing_target_layer_name is not None,
             "chunk_lookback": chunk_lookback not in (-1, None),
         }
@@ -292,6 +290,11 @@ class Int8AttentionImpl(_ImplBase):
                              f"got {kv_cache_dtype!r}")
         if num_heads % num_kv_heads:
             raise ValueError("num_heads must be a multiple of num_kv_heads")
+        if sinks is not None and sinks.shape[0] != num_heads:   # the reference's check, triton_attn.py:548-554
+            raise ValueError(f"Sinks must have the same number of heads as the number of heads in the layer. "
+                             f"Sinks shape: {tuple(sinks.shape)}, num_heads: {num_heads}.")
+        # the kernels read the sinks as float32; converted once (a parameter in the model's dtype otherwise)
+        self.sinks = None if sinks is None else sinks.detach().to(torch.float32).contiguous()
         self.num_heads = num_heads
         self.head_size = head_size
         self.scale = float(scale)
@@ -336,6 +339,11 @@ class Int8AttentionImpl(_ImplBase):
             value.view(n, self.num_kv_heads, self.head_size), cos_sin_cache, is_neox, key_cache, value_cache,
             self._k_scale_cache, self._v_scale_cache, layer_slot_mapping, kv_quant_mode=self._kv_quant_mode,
             geometry=self._geometry)
+
+    def _sinks_on(self, device):
+        if self.sinks is not None and self.sinks.device != device:
+            self.sinks = self.sinks.to(device)
+        return self.sinks
 
     # -- cache views ---------------------------------------------------------------------------
     def _ensure_scale_caches(self, kv_cache: torch.Tensor) -> None:
@@ -403,7 +411,7 @@ class Int8AttentionImpl(_ImplBase):
             window_size=self.sliding_window, block_table=attn_metadata.block_table, softcap=self.logits_soft_cap,
             kv_quant_mode=self._kv_quant_mode, k_scale_cache=self._k_scale_cache, v_scale_cache=self._v_scale_cache,
             workspace=attn_metadata.workspace, geometry=self._geometry,
-            has_decode_rows=getattr(attn_metadata, "has_decode_rows", True))
+            has_decode_rows=getattr(attn_metadata, "has_decode_rows", True), sinks=self._sinks_on(q.device))
         return output
 
 
@@ -439,7 +447,8 @@ class Int8FusedUpdateAttentionImpl(Int8AttentionImpl):
             block_table=attn_metadata.block_table, k_scale_cache=self._k_scale_cache, v_scale_cache=self._v_scale_cache,
             window_size=self.sliding_window, softcap=self.logits_soft_cap, kv_quant_mode=self._kv_quant_mode,
             workspace=attn_metadata.workspace, geometry=self._geometry,
-            slot_mapping=attn_metadata.slot_mapping[:n] if attn_metadata.slot_mapping is not None else None)
+            slot_mapping=attn_metadata.slot_mapping[:n] if attn_metadata.slot_mapping is not None else None,
+            sinks=self._sinks_on(query.device))
         return output
 
 
