@@ -40,10 +40,14 @@ def _draw_paged(case):
     if sum(ctx) == 0:
         ctx[0] = 5
     cfg.update(ctx=ctx, qls=qls)
+    # later additions draw last, so that the cases above keep the shapes they always had
+    cfg["int4"] = (not cfg["fp8"]) and rng.random() < 0.25
+    cfg["sinks"] = rng.random() < 0.25
+    cfg["invariant"] = rng.random() < 0.15
     return cfg
 
 
-@pytest.mark.parametrize("block", range(8))
+@pytest.mark.parametrize("block", range(12))
 def test_paged_attention_random_cases(gpu_device, block):
     dev = gpu_device
     for case in range(12 * block, 12 * block + 12):
@@ -52,11 +56,11 @@ def test_paged_attention_random_cases(gpu_device, block):
         ctx, qls, bs, hkv, d = c["ctx"], c["qls"], c["bs"], c["hkv"], c["d"]
         g = torch.Generator().manual_seed(case)
         nb = sum((n + bs - 1) // bs for n in ctx) + 5
-        kv, views, lay = T.cpu_cache(nb, bs, hkv, d, c["layout"])
+        code = oracle.CODE_FP8 if c["fp8"] else (oracle.CODE_INT4 if c["int4"] else oracle.CODE_INT8)
+        kv, views, lay = T.cpu_cache(nb, bs, hkv, d, c["layout"], code_type=code)
         base = T.storage_bytes(kv)
         base.fill_(0xFF)                                     # NaN scales wherever nothing is written
         bt = T.make_block_tables(ctx, bs, nb, g)
-        code = oracle.CODE_FP8 if c["fp8"] else oracle.CODE_INT8
         for i, slots in enumerate(T.slots_for(bt, ctx, bs)):
             if slots.numel() > 0:
                 ksrc = torch.randn((ctx[i], hkv, d), generator=g).to(torch.bfloat16)
@@ -66,18 +70,25 @@ def test_paged_attention_random_cases(gpu_device, block):
         sl = torch.tensor(ctx, dtype=torch.int32)
         cu = torch.tensor([0] + torch.tensor(qls).cumsum(0).tolist(), dtype=torch.int32)
         scale = 1 / math.sqrt(d)
+        sinks = (torch.randn(c["hq"], generator=g) * 2).float() if c["sinks"] else None
         want, want_lse = oracle.paged_attn(q, base, lay, bt, sl, cu, scale, return_lse=True,
-                                           sliding_window=c["window"], soft_cap=c["cap"], code_type=code)
-        kvd = T.to_device_cache(kv, dev, c["layout"])
+                                           sliding_window=c["window"], soft_cap=c["cap"], code_type=code, sinks=sinks)
+        kvd = T.to_device_cache(kv, dev, c["layout"], code_type=code)
         k, v = L.key_value_views(kvd)
         ks, vs = L.scale_views(kvd)
         out = torch.full(q.shape, float("nan"), dtype=c["odt"], device=dev)
         lse = torch.full(q.shape[:2], float("nan"), dtype=torch.float32, device=dev)
-        mode = KVQuantMode.FP8_PER_TOKEN_HEAD if c["fp8"] else KVQuantMode.INT8_PER_TOKEN_HEAD
-        ops.unified_attention(q.to(dev), k, v, out, cu.to(dev), max(qls), sl.to(dev), int(sl.max()), scale, True,
-                              window_size=(c["window"] - 1, 0) if c["window"] else (-1, -1), softcap=c["cap"],
-                              block_table=bt.to(dev), k_scale_cache=ks, v_scale_cache=vs, lse=lse, kv_quant_mode=mode)
-        torch.cuda.synchronize()
+        mode = KVQuantMode.FP8_PER_TOKEN_HEAD if c["fp8"] else (
+            KVQuantMode.INT4_PER_TOKEN_HEAD if c["int4"] else KVQuantMode.INT8_PER_TOKEN_HEAD)
+        before = ops.set_batch_invariant(c["invariant"])
+        try:
+            ops.unified_attention(q.to(dev), k, v, out, cu.to(dev), max(qls), sl.to(dev), int(sl.max()), scale, True,
+                                  window_size=(c["window"] - 1, 0) if c["window"] else (-1, -1), softcap=c["cap"],
+                                  block_table=bt.to(dev), k_scale_cache=ks, v_scale_cache=vs, lse=lse,
+                                  kv_quant_mode=mode, sinks=None if sinks is None else sinks.to(dev))
+            torch.cuda.synchronize()
+        finally:
+            ops.set_batch_invariant(before)
         live = torch.tensor([ctx[i] > 0 for i in range(len(ctx)) for _ in range(qls[i])])
         T.assert_close_attn(out[live], want[live], what=what)        # atol 2e-2, rtol 1e-2
         torch.testing.assert_close(lse.cpu()[live], want_lse[live], atol=5e-3, rtol=1e-3, msg=what)
