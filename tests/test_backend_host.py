@@ -280,3 +280,37 @@ def test_ops_refuse_cpu_tensors_and_bad_shapes_before_touching_the_library():
         ops.mla_decode_int8((a, b), cache, o, None, bt, sl, 0.1, 512)
     with pytest.raises(RuntimeError):
         ops.mla_decode_int8(out, cache, o, None, bt, sl, 0.1, 512)
+
+
+def test_c_abi_rejects_bad_arguments_of_the_newer_entry_points_without_a_gpu():
+    """Argument checks run before anything is launched: the entry points return KVQ_EINVAL (-22) and leave a
+    message, also on a machine without a GPU."""
+    import ctypes
+
+    lib = _C.load()
+    g = _C.CacheGeom(0, 132, 128, 260, 16 * 8 * 264, 8 * 264, 264, 8, 128, 16, _C.KVQ_CODE_INT8)
+    null = ctypes.c_void_p(0)
+    one = ctypes.c_void_p(16)   # any non-NULL address: nothing is dereferenced on the host
+    # rope + write: NULL pointers, an odd rotary width, a rotary width beyond the head size, an unknown code type
+    assert lib.kvq_rope_and_cache_int8(null, one, 0, 0, 32, one, 0, 0, one, 0, 0, _C.KVQ_BF16, one, _C.KVQ_BF16, 64, 1,
+                                       one, ctypes.byref(g), one, 4, 0.0, null) == -22
+    assert b"NULL" in lib.kvq_last_error()
+    for rot in (63, 130):
+        assert lib.kvq_rope_and_cache_int8(one, one, 0, 0, 32, one, 0, 0, one, 0, 0, _C.KVQ_BF16, one, _C.KVQ_BF16, rot,
+                                           1, one, ctypes.byref(g), one, 4, 0.0, null) == -22
+        assert b"rot_dim" in lib.kvq_last_error()
+    bad = _C.CacheGeom(0, 132, 128, 260, 16 * 8 * 264, 8 * 264, 264, 8, 128, 16, 7)
+    assert lib.kvq_rope_and_cache_int8(one, one, 0, 0, 32, one, 0, 0, one, 0, 0, _C.KVQ_BF16, one, _C.KVQ_BF16, 64, 1,
+                                       one, ctypes.byref(bad), one, 4, 0.0, null) == -22
+    assert b"code_type" in lib.kvq_last_error()
+    assert lib.kvq_rope_and_cache_int8(one, one, 0, 0, 32, one, 0, 0, one, 0, 0, _C.KVQ_BF16, one, _C.KVQ_BF16, 64, 1,
+                                       one, ctypes.byref(g), one, 0, 0.0, null) == 0      # no tokens: nothing to do
+    # an int4 geometry whose record is not [D/2 codes | scale | D/2 codes | scale] is refused by the attention entry
+    g4 = _C.CacheGeom(0, 132, 128, 260, 16 * 8 * 264, 8 * 264, 264, 8, 128, 16, _C.KVQ_CODE_INT4)
+    rc = lib.kvq_paged_attn_int8(one, _C.KVQ_BF16, 4096, 128, one, _C.KVQ_BF16, 4096, 128, one, ctypes.byref(g4), one, 8,
+                                 one, null, 2, 32, 1, 0.1, 1, 0, 0.0, null, null, one, 1 << 20, null)
+    assert rc == -22 and b"record" in lib.kvq_last_error()
+    # an unknown flag in `causal`
+    rc = lib.kvq_paged_attn_int8(one, _C.KVQ_BF16, 4096, 128, one, _C.KVQ_BF16, 4096, 128, one, ctypes.byref(g), one, 8,
+                                 one, null, 2, 32, 1, 0.1, 9, 0, 0.0, null, null, one, 1 << 20, null)
+    assert rc == -22 and b"flag" in lib.kvq_last_error()
