@@ -27,7 +27,7 @@
 extern "C" {
 #endif
 
-#define KVQ_ABI_VERSION 16
+#define KVQ_ABI_VERSION 17
 
 #define KVQ_OK 0
 #define KVQ_EINVAL (-22)
@@ -197,6 +197,15 @@ KVQ_API int kvq_rope_and_cache_int8(const int64_t* positions, void* query, int64
  * keys' logits and one more logit, sinks[h] (as given: not multiplied by `scale`), whose value row is zero:
  * out = sum_j exp(s_j) v_j / (exp(sinks[h]) + sum_j exp(s_j)); lse includes the sink's term.
  *
+ * alibi_slopes (optional, [num_q_heads] fp32, may be NULL; needs `causal`): ALiBi, the alibi_slopes of the
+ * reference's attention op (triton_attn.py:504-506, 699; paged_attention_v2's alibi_slopes,
+ * csrc/libtorch_stable/torch_bindings.cpp:631-641).  The scaled (and capped) logit of the query at position p
+ * and the key at position j gets alibi_slopes[h] * (j - p) added: for a decode row, the
+ * alibi_slope * (token_idx - seq_len + 1) of the native kernel (csrc/libtorch_stable/attention/
+ * attention_kernels.cuh) and of its test oracle (tests/kernels/attention/test_attention.py:109-117); for a query
+ * run, each row with its own position.  lse is that of the biased logits.  The square-root form
+ * (use_alibi_sqrt, triton_attn.py:405-407, 700) is not built.
+ *
  * `causal` is a set of flags: KVQ_ATTN_CAUSAL (1, the reference's causal=True) and, optionally,
  * KVQ_ATTN_NO_DECODE_ROWS (2): the caller's promise that no sequence of this batch has exactly one query
  * row (a pure prefill batch; a metadata builder knows it from the host copy of query_start_loc).  The
@@ -215,7 +224,7 @@ KVQ_API int kvq_paged_attn_int8(void* out, int out_dtype, int64_t out_stride_t, 
                         const int32_t* block_table, int64_t bt_stride, const int32_t* seq_lens,
                         const int32_t* cu_seqlens_q, int num_seqs, int num_q_heads,
                         int max_query_len, float scale, int causal, int window_size,
-                        float softcap, const float* sinks, float* lse, void* workspace, size_t workspace_bytes,
+                        float softcap, const float* sinks, const float* alibi_slopes, float* lse, void* workspace, size_t workspace_bytes,
                         kvq_stream_t stream);
 
 /*
@@ -246,7 +255,7 @@ KVQ_API int kvq_paged_attn_int8_fused_write(void* out, int out_dtype, int64_t ou
                         const int32_t* block_table, int64_t bt_stride, const int32_t* seq_lens,
                         const int64_t* slot_mapping,
                         int num_seqs, int num_q_heads, float scale, int window_size,
-                        float softcap, const float* sinks, float* lse, void* workspace, size_t workspace_bytes,
+                        float softcap, const float* sinks, const float* alibi_slopes, float* lse, void* workspace, size_t workspace_bytes,
                         kvq_stream_t stream);
 
 /*
@@ -276,7 +285,7 @@ KVQ_API int kvq_paged_attn_int8_static_scratch(
     int64_t q_stride_t, int64_t q_stride_h, const void* cache, const kvq_cache_geom* geom,
     const int32_t* block_table, int64_t bt_stride, const int32_t* seq_lens, const int32_t* cu_seqlens_q,
     int num_seqs, int num_q_heads, int max_query_len, float scale, int causal, int window_size,
-    float softcap, const float* sinks, float* lse, kvq_stream_t stream);
+    float softcap, const float* sinks, const float* alibi_slopes, float* lse, kvq_stream_t stream);
 
 /*
  * Fixed-partition split-K decode + reduce (one query row per sequence).

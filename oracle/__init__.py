@@ -222,19 +222,21 @@ def cache_write(key, value, kv_cache, lay: RecordLayout, slot_mapping, eps: floa
 
 def paged_attn(q, kv_cache, lay: RecordLayout, block_table, seq_lens, cu_seqlens_q,
                scale: float, causal: bool = True, return_lse: bool = False, sliding_window: int = 0,
-               soft_cap: float = 0.0, code_type: int = CODE_INT8, sinks=None):
+               soft_cap: float = 0.0, code_type: int = CODE_INT8, sinks=None, alibi_slopes=None):
     """q [N, Hq, D] -> out fp32 [N, Hq, D] (and lse fp32 [N, Hq]).  sliding_window > 0: a query sees its
     last `sliding_window` keys (itself included); soft_cap > 0: logits -> cap * tanh(logit / cap);
-    sinks [Hq]: one more logit per head with a zero value row (attention sinks)."""
+    sinks [Hq]: one more logit per head with a zero value row (attention sinks); alibi_slopes [Hq]: the logit
+    of query position p and key position j gets slope * (j - p) added."""
     qf = _f32c(q)
     sk = _f32c(sinks) if sinks is not None else None
+    al = _f32c(alibi_slopes) if alibi_slopes is not None else None
     N, Hq, D = qf.shape
     bt, sl, cu = _i32c(block_table), _i32c(seq_lens), _i32c(cu_seqlens_q)
     B = sl.shape[0]
     out = torch.empty((N, Hq, D), dtype=torch.float32)
     lse = torch.empty((N, Hq), dtype=torch.float32) if return_lse else None
     _check(
-        lib().kvq_oracle_paged_attn_ex3(
+        lib().kvq_oracle_paged_attn_ex4(
             _p(out), _p(lse), _p(qf), _p(kv_cache),
             _i64(lay.k_off), _i64(lay.v_off), _i64(lay.ks_off), _i64(lay.vs_off),
             _i64(lay.stride_block), _i64(lay.stride_slot), _i64(lay.stride_head),
@@ -242,9 +244,9 @@ def paged_attn(q, kv_cache, lay: RecordLayout, block_table, seq_lens, cu_seqlens
             ctypes.c_int(B), ctypes.c_int(Hq), ctypes.c_int(lay.num_kv_heads), ctypes.c_int(D),
             ctypes.c_int(lay.block_size), ctypes.c_float(scale), ctypes.c_int(1 if causal else 0),
             ctypes.c_int(int(sliding_window or 0)), ctypes.c_float(float(soft_cap or 0.0)),
-            ctypes.c_int(code_type), _p(sk),
+            ctypes.c_int(code_type), _p(sk), _p(al),
         ),
-        "kvq_oracle_paged_attn_ex3",
+        "kvq_oracle_paged_attn_ex4",
     )
     return (out, lse) if return_lse else out
 

@@ -270,7 +270,8 @@ static void attend_range(const float* q, int D, const uint8_t* cache,
                          int64_t stride_block, int64_t stride_slot, int64_t stride_head,
                          const int32_t* bt_row, int block_size, int hkv,
                          int64_t k_begin, int64_t k_end, double scale, double softcap,
-                         double* acc, double* m_out, double* l_out, double* logits, int code_type) {
+                         double* acc, double* m_out, double* l_out, double* logits, int code_type,
+                         double alibi_slope, int64_t q_pos) {
   double m = -INFINITY;
   for (int64_t j = k_begin; j < k_end; ++j) {
     int64_t blk = bt_row[j / block_size];
@@ -283,6 +284,7 @@ static void attend_range(const float* q, int D, const uint8_t* cache,
     for (int d = 0; d < D; ++d) s += (double)q[d] * (code_at(kc, d, code_type) * (double)ks);
     s *= scale;
     if (softcap > 0.0) s = softcap * tanh(s / softcap);
+    s += alibi_slope * (double)(j - q_pos);   /* ALiBi: after the cap, on the scaled logit; 0 for the query's own key */
     logits[j - k_begin] = s;
     if (s > m) m = s;
   }
@@ -327,13 +329,31 @@ static void attend_range(const float* q, int D, const uint8_t* cache,
  * zero value row: out = sum_j exp(s_j) v_j / (exp(sinks[h]) + sum_j exp(s_j)), lse = log of that denominator.
  * The definition of the `sinks` argument of upstream's unified_attention, which the reference passes through
  * (vllm_metax/v1/attention/backends/triton_attn.py:712, 784); rows without a visible key stay zeros / -inf.  */
+/* alibi_slopes != NULL: ALiBi, [Hq] fp32.  The scaled (and capped) logit of query position p and key position j
+ * gets slope[h] * (j - p) added: the bias alibi_slopes * (position_ids - seq_len + 1) of
+ * ref_single_query_cached_kv_attention for a decode row (tests/kernels/attention/test_attention.py:109-117, the
+ * query standing at seq_len - 1) and `alibi_slope * (token_idx - seq_len + 1)` of the native kernel
+ * (csrc/libtorch_stable/attention/attention_kernels.cuh); for a query run, the same with each row's own position.  */
+KVQ_EXPORT int kvq_oracle_paged_attn_ex4(
+    float* out, float* lse, const float* q, const uint8_t* cache,
+    int64_t k_off, int64_t v_off, int64_t ks_off, int64_t vs_off,
+    int64_t stride_block, int64_t stride_slot, int64_t stride_head,
+    const int32_t* block_table, int64_t bt_stride, const int32_t* seq_lens,
+    const int32_t* cu_seqlens_q, int B, int Hq, int Hkv, int D, int block_size,
+    float scale, int causal, int window, float softcap, int code_type, const float* sinks,
+    const float* alibi_slopes);
+
 KVQ_EXPORT int kvq_oracle_paged_attn_ex3(
     float* out, float* lse, const float* q, const uint8_t* cache,
     int64_t k_off, int64_t v_off, int64_t ks_off, int64_t vs_off,
     int64_t stride_block, int64_t stride_slot, int64_t stride_head,
     const int32_t* block_table, int64_t bt_stride, const int32_t* seq_lens,
     const int32_t* cu_seqlens_q, int B, int Hq, int Hkv, int D, int block_size,
-    float scale, int causal, int window, float softcap, int code_type, const float* sinks);
+    float scale, int causal, int window, float softcap, int code_type, const float* sinks) {
+  return kvq_oracle_paged_attn_ex4(out, lse, q, cache, k_off, v_off, ks_off, vs_off, stride_block, stride_slot,
+                                   stride_head, block_table, bt_stride, seq_lens, cu_seqlens_q, B, Hq, Hkv, D,
+                                   block_size, scale, causal, window, softcap, code_type, sinks, NULL);
+}
 
 KVQ_EXPORT int kvq_oracle_paged_attn_ex2(
     float* out, float* lse, const float* q, const uint8_t* cache,
@@ -347,13 +367,14 @@ KVQ_EXPORT int kvq_oracle_paged_attn_ex2(
                                    block_size, scale, causal, window, softcap, code_type, NULL);
 }
 
-KVQ_EXPORT int kvq_oracle_paged_attn_ex3(
+KVQ_EXPORT int kvq_oracle_paged_attn_ex4(
     float* out, float* lse, const float* q, const uint8_t* cache,
     int64_t k_off, int64_t v_off, int64_t ks_off, int64_t vs_off,
     int64_t stride_block, int64_t stride_slot, int64_t stride_head,
     const int32_t* block_table, int64_t bt_stride, const int32_t* seq_lens,
     const int32_t* cu_seqlens_q, int B, int Hq, int Hkv, int D, int block_size,
-    float scale, int causal, int window, float softcap, int code_type, const float* sinks) {
+    float scale, int causal, int window, float softcap, int code_type, const float* sinks,
+    const float* alibi_slopes) {
   if (!out || !q || !cache || !block_table || !seq_lens || !cu_seqlens_q) return -1;
   if (Hkv <= 0 || Hq % Hkv != 0) return -1;
   const int G = Hq / Hkv;
@@ -392,7 +413,8 @@ KVQ_EXPORT int kvq_oracle_paged_attn_ex3(
             attend_range(q + ((q0 + r) * Hq + h) * (int64_t)D, D, cache, k_off, v_off,
                          ks_off, vs_off, stride_block, stride_slot, stride_head,
                          block_table + (int64_t)i * bt_stride, block_size, h / G, first, vis,
-                         (double)scale, (double)softcap, acc, &m, &l, logits, code_type);
+                         (double)scale, (double)softcap, acc, &m, &l, logits, code_type,
+                         alibi_slopes ? (double)alibi_slopes[h] : 0.0, kvlen - qlen + r);
             if (sinks) {   /* one more logit with a zero value row */
               const double sk = (double)sinks[h];
               if (sk > m) {
@@ -487,7 +509,7 @@ KVQ_EXPORT int kvq_oracle_paged_attn_partition(
             attend_range(q + ((int64_t)i * Hq + h) * D, D, cache, k_off, v_off, ks_off,
                          vs_off, stride_block, stride_slot, stride_head,
                          block_table + (int64_t)i * bt_stride, block_size, h / G, b0, b1,
-                         (double)scale, 0.0, acc, &m, &l, logits, KVQ_CODE_INT8);
+                         (double)scale, 0.0, acc, &m, &l, logits, KVQ_CODE_INT8, 0.0, 0);
             int64_t idx = ((int64_t)i * Hq + h) * max_parts + j;
             for (int d = 0; d < D; ++d) tmp_out[idx * D + d] = (float)(acc[d] / l);
             max_logits[idx] = (float)m;

@@ -50,8 +50,11 @@ def dequant_cache(key_cache, value_cache, k_scale_cache, v_scale_cache, head_siz
 
 
 def paged_attn(query, key_cache, value_cache, query_lens, kv_lens, block_tables, scale,
-               sliding_window=None, soft_cap=None, sinks=None):
+               sliding_window=None, soft_cap=None, sinks=None, alibi_slopes=None):
     """tests/kernels/attention/test_triton_unified_attention.py:26-78 (ref_paged_attn).
+    ``alibi_slopes`` ``[Hq]`` (not in that test either): the bias matrix ``slope * (key position - query position)``
+    is added to the scaled, capped logits -- ``alibi_slopes.view(-1, 1, 1) * (position_ids - seq_len + 1)`` of
+    tests/kernels/attention/test_attention.py:109-117 for the last position, the same for every row of a run.
     ``sinks`` ``[Hq]`` (not in the reference's copy of that test; the definition of upstream's argument): the
     softmax runs over the masked logits and one more column holding ``sinks[h]``, which is dropped afterwards.
 
@@ -78,6 +81,9 @@ def paged_attn(query, key_cache, value_cache, query_lens, kv_lens, block_tables,
             hide |= torch.triu(ones, diagonal=kl - (ql + sliding_window) + 1).bool().logical_not()
         if soft_cap:
             logits = soft_cap * torch.tanh(logits / soft_cap)
+        if alibi_slopes is not None:
+            rel = torch.arange(kl).view(1, kl) - (kl - ql + torch.arange(ql)).view(ql, 1)
+            logits = logits + alibi_slopes.float().view(-1, 1, 1) * rel.float()
         logits.masked_fill_(hide, float("-inf"))
         if sinks is not None:
             col = sinks.float().reshape(-1, 1, 1).expand(-1, ql, 1)

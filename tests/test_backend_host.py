@@ -190,9 +190,14 @@ def test_impl_constructor_errors():
     mk = lambda **kw: Int8AttentionImpl(32, 128, 0.088, 8, **kw)
     impl = mk()
     assert impl.num_queries_per_kv == 4 and impl.fused_rope_kvcache_supported() is True   # built here; the reference answers False
-    for kw in (dict(alibi_slopes=[1.0] * 32), dict(attn_type=AttentionType.ENCODER_ONLY)):
+    for kw in (dict(use_alibi_sqrt=True), dict(attn_type=AttentionType.ENCODER_ONLY)):
         with pytest.raises(NotImplementedError):
             mk(**kw)
+    # ALiBi slopes: a float32 tensor with one slope per head, as the reference keeps them (triton_attn.py:504-506)
+    al = mk(alibi_slopes=[0.5] * 32).alibi_slopes
+    assert al.dtype == torch.float32 and tuple(al.shape) == (32,) and mk().alibi_slopes is None
+    with pytest.raises(ValueError):
+        mk(alibi_slopes=[0.5] * 8)
     # attention sinks: one per q head, kept as float32 (triton_attn.py:548-554)
     assert mk(sinks=torch.zeros(32, dtype=torch.bfloat16)).sinks.dtype == torch.float32
     with pytest.raises(ValueError):
@@ -308,9 +313,9 @@ def test_c_abi_rejects_bad_arguments_of_the_newer_entry_points_without_a_gpu():
     # an int4 geometry whose record is not [D/2 codes | scale | D/2 codes | scale] is refused by the attention entry
     g4 = _C.CacheGeom(0, 132, 128, 260, 16 * 8 * 264, 8 * 264, 264, 8, 128, 16, _C.KVQ_CODE_INT4)
     rc = lib.kvq_paged_attn_int8(one, _C.KVQ_BF16, 4096, 128, one, _C.KVQ_BF16, 4096, 128, one, ctypes.byref(g4), one, 8,
-                                 one, null, 2, 32, 1, 0.1, 1, 0, 0.0, null, null, one, 1 << 20, null)
+                                 one, null, 2, 32, 1, 0.1, 1, 0, 0.0, null, null, null, one, 1 << 20, null)
     assert rc == -22 and b"record" in lib.kvq_last_error()
     # an unknown flag in `causal`
     rc = lib.kvq_paged_attn_int8(one, _C.KVQ_BF16, 4096, 128, one, _C.KVQ_BF16, 4096, 128, one, ctypes.byref(g), one, 8,
-                                 one, null, 2, 32, 1, 0.1, 9, 0, 0.0, null, null, one, 1 << 20, null)
+                                 one, null, 2, 32, 1, 0.1, 9, 0, 0.0, null, null, null, one, 1 << 20, null)
     assert rc == -22 and b"flag" in lib.kvq_last_error()

@@ -44,6 +44,7 @@ def _draw_paged(case):
     cfg["int4"] = (not cfg["fp8"]) and rng.random() < 0.25
     cfg["sinks"] = rng.random() < 0.25
     cfg["invariant"] = rng.random() < 0.15
+    cfg["alibi"] = rng.random() < 0.2
     return cfg
 
 
@@ -71,8 +72,11 @@ def test_paged_attention_random_cases(gpu_device, block):
         cu = torch.tensor([0] + torch.tensor(qls).cumsum(0).tolist(), dtype=torch.int32)
         scale = 1 / math.sqrt(d)
         sinks = (torch.randn(c["hq"], generator=g) * 2).float() if c["sinks"] else None
+        # ALiBi slopes between 2^-8 and 2 (drawn after everything else, so that the other cases keep their data)
+        slopes = torch.exp2(torch.rand(c["hq"], generator=g) * 9 - 8).float() if c["alibi"] else None
         want, want_lse = oracle.paged_attn(q, base, lay, bt, sl, cu, scale, return_lse=True,
-                                           sliding_window=c["window"], soft_cap=c["cap"], code_type=code, sinks=sinks)
+                                           sliding_window=c["window"], soft_cap=c["cap"], code_type=code, sinks=sinks,
+                                           alibi_slopes=slopes)
         kvd = T.to_device_cache(kv, dev, c["layout"], code_type=code)
         k, v = L.key_value_views(kvd)
         ks, vs = L.scale_views(kvd)
@@ -85,7 +89,8 @@ def test_paged_attention_random_cases(gpu_device, block):
             ops.unified_attention(q.to(dev), k, v, out, cu.to(dev), max(qls), sl.to(dev), int(sl.max()), scale, True,
                                   window_size=(c["window"] - 1, 0) if c["window"] else (-1, -1), softcap=c["cap"],
                                   block_table=bt.to(dev), k_scale_cache=ks, v_scale_cache=vs, lse=lse,
-                                  kv_quant_mode=mode, sinks=None if sinks is None else sinks.to(dev))
+                                  kv_quant_mode=mode, sinks=None if sinks is None else sinks.to(dev),
+                                  alibi_slopes=None if slopes is None else slopes.to(dev))
             torch.cuda.synchronize()
         finally:
             ops.set_batch_invariant(before)

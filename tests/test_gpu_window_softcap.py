@@ -207,3 +207,90 @@ def test_attention_sinks_decode_prefill_and_mixed(gpu_device, hq, hkv, d, layout
 def ks_last(rows):
     """The last token's row of every sequence, [B, Hkv, D]."""
     return torch.stack([r[-1] for r in rows])
+
+
+@pytest.mark.parametrize("hq,hkv,d,layout,code", [(32, 8, 128, "HND", "int8"), (28, 4, 128, "NHD", "int8"),
+                                                  (8, 2, 64, "HND", "fp8"), (4, 1, 256, "NHD", "int4"),
+                                                  (16, 8, 128, "HND", "int4"), (16, 1, 128, "HND", "int8")])
+@pytest.mark.parametrize("window,cap,with_sinks", [(0, 0.0, False), (200, 25.0, True)])
+def test_alibi_decode_prefill_and_mixed(gpu_device, hq, hkv, d, layout, code, window, cap, with_sinks):
+    """ALiBi (alibi_slopes of the reference's attention op, triton_attn.py:504-506, 699; the bias of
+    tests/kernels/attention/test_attention.py:109-117): decode rows whole and cut, both prefill tiles, a mixed
+    batch and the one-launch decode step, alone and on top of window + soft cap + sinks, output and lse against
+    the oracle; the batch-invariant cutting as well."""
+    import oracle
+    from vllm_metax_amd.kv_cache_interface import KVQuantMode
+    ct = {"int8": oracle.CODE_INT8, "fp8": oracle.CODE_FP8, "int4": oracle.CODE_INT4}[code]
+    mode = {"int8": KVQuantMode.INT8_PER_TOKEN_HEAD, "fp8": KVQuantMode.FP8_PER_TOKEN_HEAD,
+            "int4": KVQuantMode.INT4_PER_TOKEN_HEAD}[code]
+    dev = gpu_device
+    bs = 16
+    g = torch.Generator().manual_seed(hq * 11 + d + window)
+    # the usual geometric slopes, and a steep and a zero one
+    slopes = torch.tensor([2.0 ** (-8.0 * (i + 1) / hq) for i in range(hq)], dtype=torch.float32)
+    slopes[0], slopes[-1] = 1.5, 0.0
+    sinks = (torch.randn(hq, generator=g) * 2).float() if with_sinks else None
+    scale = 1 / math.sqrt(d)
+    for ctx, qls in (([1000, 3, 517, 64, 9000, 33], [1] * 6),          # decode rows: whole sequences and cut ones
+                     ([40000, 700], [1, 1]),                           # a handful of sequences, dozens of cuts
+                     ([900, 2300, 33, 257], [300, 1, 33, 2]),          # both prefill tiles beside a decode row
+                     ([700, 1500], [700, 1100])):                      # long runs: the workgroup-shared tile
+        nb = sum((c + bs - 1) // bs for c in ctx) + 5
+        kv_cpu, _, lay = T.cpu_cache(nb, bs, hkv, d, layout, code_type=ct)
+        bt = T.make_block_tables(ctx, bs, nb, g)
+        ks = [torch.randn((c, hkv, d), generator=g).to(torch.bfloat16) for c in ctx]
+        vs_ = [torch.randn((c, hkv, d), generator=g).to(torch.bfloat16) for c in ctx]
+        T.fill_cache_from_sources(kv_cpu, lay, bt, ctx, bs, ks, vs_, code_type=ct)
+        q = torch.randn((sum(qls), hq, d), generator=g).to(torch.bfloat16)
+        sl = torch.tensor(ctx, dtype=torch.int32)
+        cu = torch.tensor([0] + torch.tensor(qls).cumsum(0).tolist(), dtype=torch.int32)
+        want, want_lse = oracle.paged_attn(q, T.storage_bytes(kv_cpu), lay, bt, sl, cu, scale, return_lse=True,
+                                           sliding_window=window, soft_cap=cap, code_type=ct, sinks=sinks,
+                                           alibi_slopes=slopes)
+        plain = oracle.paged_attn(q, T.storage_bytes(kv_cpu), lay, bt, sl, cu, scale, sliding_window=window,
+                                  soft_cap=cap, code_type=ct, sinks=sinks)
+        assert not torch.allclose(want, plain, atol=5e-2)      # the bias matters in this case
+        kv = T.to_device_cache(kv_cpu, dev, layout, code_type=ct)
+        k, v = L.key_value_views(kv)
+        ksc, vsc = L.scale_views(kv)
+        sk = sinks.to(dev) if with_sinks else None
+        for invariant in (False, True):
+            before = ops.set_batch_invariant(invariant)
+            try:
+                out = torch.full(q.shape, float("nan"), dtype=torch.bfloat16, device=dev)
+                lse = torch.full(q.shape[:2], float("nan"), dtype=torch.float32, device=dev)
+                ops.unified_attention(q.to(dev), k, v, out, cu.to(dev), max(qls), sl.to(dev), max(ctx), scale, True,
+                                      window_size=(window - 1, 0) if window else (-1, -1), softcap=cap,
+                                      block_table=bt.to(dev), k_scale_cache=ksc, v_scale_cache=vsc, kv_quant_mode=mode,
+                                      lse=lse, sinks=sk, alibi_slopes=slopes.to(dev))
+                torch.cuda.synchronize()
+            finally:
+                ops.set_batch_invariant(before)
+            T.assert_close_attn(out, want, what=f"alibi {code} ctx {ctx} invariant={invariant}")
+            torch.testing.assert_close(lse.cpu(), want_lse, atol=5e-3, rtol=1e-3)
+        if max(qls) == 1:   # the one-launch step: same rows (the new token rewrites the last record with its own bytes)
+            out2 = torch.full(q.shape, float("nan"), dtype=torch.bfloat16, device=dev)
+            ops.decode_attention_with_cache_update(q.to(dev), ks_last(ks).to(dev), ks_last(vs_).to(dev), k, v, out2,
+                                                   sl.to(dev), max(ctx), scale, bt.to(dev), ksc, vsc,
+                                                   window_size=(window - 1, 0) if window else (-1, -1), softcap=cap,
+                                                   kv_quant_mode=mode, sinks=sk, alibi_slopes=slopes.to(dev))
+            torch.cuda.synchronize()
+            T.assert_close_attn(out2, want, what=f"alibi fused write {code}")
+
+
+def test_alibi_is_refused_without_causal_and_in_its_sqrt_form(gpu_device):
+    dev = gpu_device
+    kv = L.allocate_kv_cache(4, 16, 2, 64, device=dev)
+    k, v = L.key_value_views(kv)
+    ksc, vsc = L.scale_views(kv)
+    q = torch.zeros((1, 4, 64), dtype=torch.bfloat16, device=dev)
+    args = (q, k, v, torch.empty_like(q), torch.tensor([0, 1], dtype=torch.int32, device=dev), 1,
+            torch.tensor([5], dtype=torch.int32, device=dev), 5, 0.1)
+    kw = dict(block_table=torch.zeros((1, 1), dtype=torch.int32, device=dev), k_scale_cache=ksc, v_scale_cache=vsc)
+    sl = torch.ones(4, device=dev)
+    with pytest.raises(NotImplementedError):
+        ops.unified_attention(*args, False, alibi_slopes=sl, **kw)
+    with pytest.raises(NotImplementedError):
+        ops.unified_attention(*args, True, alibi_slopes=sl, use_alibi_sqrt=True, **kw)
+    with pytest.raises(RuntimeError):
+        ops.unified_attention(*args, True, alibi_slopes=torch.ones(3, device=dev), **kw)

@@ -140,6 +140,79 @@ def test_attention_sinks_vs_softmax_over_one_more_column(window, cap):
     torch.testing.assert_close(one, plain[-1:] * 0.5, atol=1e-6, rtol=1e-5)
 
 
+@pytest.mark.parametrize("window,cap", [(0, 0.0), (40, 0.0), (0, 20.0)])
+def test_alibi_vs_explicit_bias_matrix_sdpa_and_closed_forms(window, cap):
+    """ALiBi (alibi_slopes of the reference's attention op, vllm_metax/v1/attention/backends/triton_attn.py:699; the
+    bias of tests/kernels/attention/test_attention.py:109-117): the oracle against the restated reference op with
+    the explicit bias matrix, against torch's scaled_dot_product_attention fed the same matrix as attn_mask, and
+    closed forms: zero slopes change nothing; with equal keys the weights are a geometric series in the slope;
+    a one-token run equals a decode row; a huge slope leaves the query's own key."""
+    hq, hkv, d, bs = 8, 2, 64, 16
+    ctx, ql = [100, 463, 18, 1], [1, 129, 5, 1]
+    kv, views, lay, bt, q, cu, sl = _build(ctx, ql, hq, hkv, d, bs, "NHD", 29)
+    scale = d ** -0.5
+    slopes = torch.tensor([2.0 ** -(i + 1) for i in range(hq)])     # the usual ALiBi slopes of 8 heads
+    base = T.storage_bytes(kv)
+    kw = dict(sliding_window=window, soft_cap=cap)
+    out, lse = oracle.paged_attn(q, base, lay, bt, sl, cu, scale, alibi_slopes=slopes, return_lse=True, **kw)
+    k, v, ks, vs = views
+    kd, vd = torch_ref.dequant_cache(k, v, ks, vs, d, torch.float32)
+    want = torch_ref.paged_attn(q.float(), kd, vd, ql, ctx, bt, scale, sliding_window=window or None,
+                                soft_cap=cap or None, alibi_slopes=slopes)
+    torch.testing.assert_close(out, want, atol=3e-5, rtol=1e-5)
+    plain, plain_lse = oracle.paged_attn(q, base, lay, bt, sl, cu, scale, return_lse=True, **kw)
+    zero = oracle.paged_attn(q, base, lay, bt, sl, cu, scale, alibi_slopes=torch.zeros(hq), **kw)
+    assert torch.equal(zero, plain)
+    assert not torch.allclose(out, plain, atol=1e-3)
+    if not cap and not window:
+        # a library routine with the bias as an additive mask: sequence 1 (129 rows on 463 keys)
+        kl, n = ctx[1], ql[1]
+        blocks = bt[1, : (kl + bs - 1) // bs].long()
+        kk = kd[blocks].reshape(-1, hkv, d)[:kl].repeat_interleave(hq // hkv, dim=1).permute(1, 0, 2)
+        vv = vd[blocks].reshape(-1, hkv, d)[:kl].repeat_interleave(hq // hkv, dim=1).permute(1, 0, 2)
+        qq = q[int(cu[1]):int(cu[2])].float().permute(1, 0, 2)
+        rel = (torch.arange(kl).view(1, kl) - (kl - n + torch.arange(n)).view(n, 1)).float()
+        mask = slopes.view(-1, 1, 1) * rel
+        mask = mask.masked_fill(rel > 0, float("-inf"))
+        ref = torch.nn.functional.scaled_dot_product_attention(qq, kk, vv, attn_mask=mask, scale=scale)
+        torch.testing.assert_close(out[int(cu[1]):int(cu[2])], ref.permute(1, 0, 2), atol=3e-5, rtol=1e-5)
+        # the bias of the query's own key is zero and every other is negative: lse <= the plain lse
+        assert bool((lse <= plain_lse + 1e-6).all())
+    # a huge slope leaves the query's own key: the row is that key's value row (sequence 0, a decode row of 100 keys)
+    big = oracle.paged_attn(q[:1], base, lay, bt[:1], sl[:1], torch.tensor([0, 1], dtype=torch.int32), scale,
+                            alibi_slopes=torch.full((hq,), 1000.0), **kw)
+    last = vd[bt[0, (ctx[0] - 1) // bs].long(), (ctx[0] - 1) % bs].repeat_interleave(hq // hkv, dim=0)
+    torch.testing.assert_close(big[0], last, atol=1e-6, rtol=1e-6)
+
+
+def test_alibi_with_equal_keys_is_a_geometric_series():
+    """Every key and value record of the sequence is the same except the value's first element, which is the
+    position: the logits are then equal, the weights are exp(slope * (j - p)) / sum, and out[0] is the
+    slope-weighted mean position -- a closed form that a wrong sign or a wrong origin of the positions fails."""
+    hq, hkv, d, bs = 4, 1, 64, 16
+    n = 77
+    kvc, views, lay = T.cpu_cache(8, bs, hkv, d, "NHD")
+    g = torch.Generator().manual_seed(3)
+    krow = torch.randn((1, hkv, d), generator=g).expand(n, hkv, d).contiguous()
+    vrow = torch.zeros((n, hkv, d))
+    vrow[:, 0, 0] = torch.arange(n, dtype=torch.float32)
+    vrow[:, 0, 1] = 127.0                         # keeps every row's scale at 1: codes are the positions
+    bt = torch.arange(5, dtype=torch.int32).view(1, 5)
+    slots = torch.arange(n, dtype=torch.int64)
+    oracle.cache_write(krow, vrow, T.storage_bytes(kvc), lay, slots)
+    q = torch.randn((3, hq, d), generator=g)
+    slopes = torch.tensor([0.5, 0.1, 0.01, 0.0])
+    out = oracle.paged_attn(q, T.storage_bytes(kvc), lay, bt, torch.tensor([n], dtype=torch.int32),
+                            torch.tensor([0, 3], dtype=torch.int32), 0.3, alibi_slopes=slopes)
+    for r in range(3):
+        p = n - 3 + r                             # the row's position; it sees keys 0..p
+        j = torch.arange(p + 1, dtype=torch.float64)
+        for h in range(hq):
+            w = torch.exp(slopes[h].double() * (j - p))
+            want = float((w * j).sum() / w.sum())
+            assert abs(float(out[r, h, 0]) - want) < 1e-4 * max(1.0, want), (r, h, float(out[r, h, 0]), want)
+
+
 def test_block_permutation_invariance_and_noncausal():
     hq, hkv, d, bs = 4, 2, 64, 16
     ctx, ql = [50, 33], [1, 3]

@@ -49,7 +49,7 @@ def _enqueue(dev, static, kv, bt, q, sl, cu, max_q, scale, out, lse, ws=None, ge
             ctypes.c_void_p(q.data_ptr()), _C.KVQ_BF16, q.stride(0), q.stride(1),
             ctypes.c_void_p(geom.base_ptr), ctypes.byref(g), ctypes.c_void_p(bt.data_ptr()), bt.stride(0),
             ctypes.c_void_p(sl.data_ptr()), ctypes.c_void_p(cu.data_ptr()), sl.shape[0], q.shape[1], max_q,
-            scale, 1, 0, 0.0, ctypes.c_void_p(0), ctypes.c_void_p(lse.data_ptr()))   # no window, cap or sinks
+            scale, 1, 0, 0.0, ctypes.c_void_p(0), ctypes.c_void_p(0), ctypes.c_void_p(lse.data_ptr()))   # no window, cap, sinks or ALiBi
     if static:
         rc = lib.kvq_paged_attn_int8_static_scratch(*head, stream)
         _C.check(rc, "kvq_paged_attn_int8_static_scratch")

@@ -162,6 +162,7 @@ struct AttnIO {
   uint32_t bs_magic;  // ceil(2^32 / block_size): x / block_size == umulhi(x, bs_magic) for x < 2^22
   int window;         // sliding window: a query sees its last `window` keys, itself included; 0 = all
   const float* sinks; // [num_q_heads] attention sinks (natural-log logits) or nullptr
+  const float* alibi; // [num_q_heads] ALiBi slopes or nullptr: logit += slope * (key position - query position)
   float cap_c;        // logits soft cap in the log2 domain, cap * log2(e); 0 = none
   float cap_k;        // 2 * log2(e) / cap_c
 };
@@ -187,6 +188,11 @@ __device__ __forceinline__ int window_first(int len, int window) {
 // (0 without sinks).  Added once, where a row's sum is final.
 __device__ __forceinline__ float sink_term(const float* sinks, int head, float m) {
   return sinks != nullptr ? __builtin_amdgcn_exp2f(sinks[head] * kLog2e - m) : 0.f;
+}
+
+// A head's ALiBi slope in the log2 domain (0 without ALiBi).
+__device__ __forceinline__ float alibi_slope(const float* alibi, int head) {
+  return alibi != nullptr ? alibi[head] * kLog2e : 0.f;
 }
 
 // One lane's share of a 32-token tile as it arrives from HBM: raw 16-byte chunks of records.
@@ -539,10 +545,12 @@ struct DecodeTile {
   // Phase 1 of a tile: S^T = K . Q^T on the MFMA from the LDS window, online softmax.  Returns
   // P~^T as the MFMA B operand.  MASK: the tile holds the end of the sequence (tokens >= len must
   // not contribute).
-  // CAP: logits pass through the soft cap.  Tokens outside [first, len) never contribute.
+  // CAP: logits pass through the soft cap (the identity when cap_c = cap_k = 0) and take the ALiBi bias
+  // `ali` x (token - (len - 1)) of the lane's head (the query of a decode row stands at len - 1).
+  // Tokens outside [first, len) never contribute.
   template <bool MASK, bool CAP>
   __device__ static half8_t qk_softmax(const AttnIO& io, const LaneOffsets& lo, const half8_t (&qb)[KSTEPS], float s_init,
-                                       int len, int first, int t, int lane, const uint8_t* lds, State& st) {
+                                       int len, int first, int t, int lane, const uint8_t* lds, State& st, float ali) {
     const int g = lane >> 4;
     const float* sc_lds = reinterpret_cast<const float*>(lds + LDS_TILE);
     const floatx4 ks0 = *reinterpret_cast<const floatx4*>(sc_lds + 4 * g);
@@ -571,13 +579,14 @@ struct DecodeTile {
     // softmax in the log2 domain; lane holds tokens 32t + mt*16 + 4g + i of head (lane & 15)
     float logit[8];
     const int tok_base = t * kTile + 4 * g;
+    const float rel0 = (float)(tok_base - (len - 1));
     float mloc = -INFINITY;
 #pragma unroll
     for (int mt = 0; mt < 2; ++mt) {
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         float x = s[mt][i] * (mt ? ks1 : ks0)[i];
-        if constexpr (CAP) x = soft_cap(x, io.cap_c, io.cap_k);
+        if constexpr (CAP) x = __builtin_fmaf(ali, rel0 + (float)(mt * 16 + i), soft_cap(x, io.cap_c, io.cap_k));
         if constexpr (MASK) x = ((uint32_t)(tok_base + mt * 16 + i - first) < (uint32_t)(len - first)) ? x : -INFINITY;
         logit[mt * 4 + i] = x;
         mloc = fmaxf(mloc, x);
@@ -665,15 +674,15 @@ struct DecodeTile {
 
   template <bool MASK, bool CAP>
   __device__ static void compute(const AttnIO& io, const LaneOffsets& lo, const half8_t (&qb)[KSTEPS], float s_init, int len,
-                                 int first, int t, int lane, const uint8_t* lds, State& st) {
-    const half8_t p = qk_softmax<MASK, CAP>(io, lo, qb, s_init, len, first, t, lane, lds, st);
+                                 int first, int t, int lane, const uint8_t* lds, State& st, float ali) {
+    const half8_t p = qk_softmax<MASK, CAP>(io, lo, qb, s_init, len, first, t, lane, lds, st, ali);
     pv(lo, p, lds, st);
   }
   template <bool CAP>
   __device__ static void compute_any(const AttnIO& io, const LaneOffsets& lo, const half8_t (&qb)[KSTEPS], float s_init,
-                                     int len, int first, int t, int lane, const uint8_t* lds, State& st) {
-    if ((t + 1) * kTile > len || t * kTile < first) compute<true, CAP>(io, lo, qb, s_init, len, first, t, lane, lds, st);
-    else compute<false, CAP>(io, lo, qb, s_init, len, first, t, lane, lds, st);
+                                     int len, int first, int t, int lane, const uint8_t* lds, State& st, float ali) {
+    if ((t + 1) * kTile > len || t * kTile < first) compute<true, CAP>(io, lo, qb, s_init, len, first, t, lane, lds, st, ali);
+    else compute<false, CAP>(io, lo, qb, s_init, len, first, t, lane, lds, st, ali);
   }
 
   // Keeps the instruction scheduler from moving work across the phase boundaries of the
@@ -718,6 +727,8 @@ struct DecodeTile {
       half8_t qb[KSTEPS];
       const float s_init = load_q(io, row, hkv, lane, qb);
       const float sc_mul = lane < 32 ? io.scale_log2 * kKScaleMul : kPScale;
+      float ali = 0.f;
+      if constexpr (CAP) ali = alibi_slope(io.alibi, hkv * io.group + min(lane & 15, io.group - 1));
       int r = 0;  // rounds this wave has finished
       // a first tile that straddles the window's lower edge is masked; it is peeled off so that the
       // steady loop below keeps a single, unmasked body
@@ -728,7 +739,7 @@ struct DecodeTile {
         load_tile<STREAM>(io, w, lo, a);
         phase_fence();
         nb = fetch_blocks(io, bt_row, len, t + 2 * nsub);
-        compute<true, CAP>(io, lo, qb, s_init, len, first, t, lane, lds, st);
+        compute<true, CAP>(io, lo, qb, s_init, len, first, t, lane, lds, st, ali);
         phase_fence();
         t += nsub;
         ++r;
@@ -758,13 +769,13 @@ struct DecodeTile {
         load_tile<STREAM>(io, w, lo, a);
         phase_fence();
         nb = fetch_blocks(io, bt_row, len, t + 2 * nsub);
-        compute<false, CAP>(io, lo, qb, s_init, len, first, t, lane, lds, st);
+        compute<false, CAP>(io, lo, qb, s_init, len, first, t, lane, lds, st, ali);
         phase_fence();
         t += nsub;
         rendezvous();
       }
       stage<STREAM>(a, lo, sc_mul, lane, lds);
-      compute_any<CAP>(io, lo, qb, s_init, len, first, t, lane, lds, st);
+      compute_any<CAP>(io, lo, qb, s_init, len, first, t, lane, lds, st, ali);
     }
     // the rendezvous count is the same for every wave of the workgroup, whatever its share of the tiles
     for (; barriers < num_barriers; ++barriers) __builtin_amdgcn_s_barrier();

@@ -67,7 +67,7 @@ static int paged_attn_launch(const char* op, void* out, int out_dtype, int64_t o
                              const kvq_cache_geom* geom, const int32_t* block_table, int64_t bt_stride,
                              const int32_t* seq_lens, const int32_t* cu_seqlens_q, int num_seqs, int num_q_heads,
                              int max_query_len, float scale, int causal, int window_size, float softcap,
-                             const float* sinks, float* lse, void* workspace, size_t workspace_bytes, const char* workspace_what,
+                             const float* sinks, const float* alibi_slopes, float* lse, void* workspace, size_t workspace_bytes, const char* workspace_what,
                              kvq_stream_t stream, const NewTokens* fresh = nullptr) {
   int rc0 = validate_common(op, q, cache, geom, block_table, seq_lens, num_seqs, num_q_heads);
   if (rc0) return rc0;
@@ -80,6 +80,7 @@ static int paged_attn_launch(const char* op, void* out, int out_dtype, int64_t o
   KVQ_REQUIRE(window_size >= 0, "%s: window_size %d must be >= 0 (0 = no sliding window)", op, window_size);
   KVQ_REQUIRE(window_size == 0 || causal, "%s: a sliding window needs causal attention", op);
   KVQ_REQUIRE(softcap >= 0.f && softcap == softcap, "%s: softcap must be >= 0 (0 = none)", op);
+  KVQ_REQUIRE(alibi_slopes == nullptr || causal, "%s: alibi_slopes need causal attention", op);
   const kvq_cache_geom& g = *geom;
   const int osz = out_dtype == KVQ_F32 ? 4 : 2;
   KVQ_REQUIRE(((uintptr_t)out % 4) == 0 && (out_stride_t * osz) % 4 == 0 && (out_stride_h * osz) % 4 == 0,
@@ -109,6 +110,7 @@ static int paged_attn_launch(const char* op, void* out, int out_dtype, int64_t o
   a.io.bs_magic = (uint32_t)((0x100000000ull + (uint64_t)geom->block_size - 1) / (uint64_t)geom->block_size);
   a.io.window = window_size;
   a.io.sinks = sinks;
+  a.io.alibi = alibi_slopes;
   a.io.cap_c = softcap * kLog2e;
   a.io.cap_k = softcap > 0.f ? 2.0f / softcap : 0.f;  // 2 log2(e) / cap_c
   a.seq_lens = seq_lens;
@@ -165,11 +167,11 @@ extern "C" int kvq_paged_attn_int8(void* out, int out_dtype, int64_t out_stride_
                                    const void* cache, const kvq_cache_geom* geom, const int32_t* block_table,
                                    int64_t bt_stride, const int32_t* seq_lens, const int32_t* cu_seqlens_q,
                                    int num_seqs, int num_q_heads, int max_query_len, float scale, int causal,
-                                   int window_size, float softcap, const float* sinks, float* lse, void* workspace,
+                                   int window_size, float softcap, const float* sinks, const float* alibi_slopes, float* lse, void* workspace,
                                    size_t workspace_bytes, kvq_stream_t stream) {
   return kvq::paged_attn_launch("paged_attn_int8", out, out_dtype, out_stride_t, out_stride_h, q, q_dtype, q_stride_t,
                                 q_stride_h, cache, geom, block_table, bt_stride, seq_lens, cu_seqlens_q, num_seqs,
-                                num_q_heads, max_query_len, scale, causal, window_size, softcap, sinks, lse, workspace,
+                                num_q_heads, max_query_len, scale, causal, window_size, softcap, sinks, alibi_slopes, lse, workspace,
                                 workspace_bytes, "workspace", stream);
 }
 
@@ -182,13 +184,13 @@ extern "C" int kvq_paged_attn_int8_fused_write(void* out, int out_dtype, int64_t
                                                int64_t bt_stride, const int32_t* seq_lens,
                                                const int64_t* slot_mapping, int num_seqs,
                                                int num_q_heads, float scale, int window_size, float softcap,
-                                               const float* sinks, float* lse, void* workspace, size_t workspace_bytes,
+                                               const float* sinks, const float* alibi_slopes, float* lse, void* workspace, size_t workspace_bytes,
                                                kvq_stream_t stream) {
   const kvq::NewTokens fresh{key, value, src_dtype, key_stride_t, key_stride_h, value_stride_t, value_stride_h, eps,
                              slot_mapping};
   return kvq::paged_attn_launch("paged_attn_int8_fused_write", out, out_dtype, out_stride_t, out_stride_h, q, q_dtype,
                                 q_stride_t, q_stride_h, cache, geom, block_table, bt_stride, seq_lens, nullptr, num_seqs,
-                                num_q_heads, 1, scale, 1, window_size, softcap, sinks, lse, workspace, workspace_bytes,
+                                num_q_heads, 1, scale, 1, window_size, softcap, sinks, alibi_slopes, lse, workspace, workspace_bytes,
                                 "workspace", stream, &fresh);
 }
 
@@ -207,7 +209,7 @@ extern "C" int kvq_paged_attn_int8_static_scratch(void* out, int out_dtype, int6
                                                   int64_t bt_stride, const int32_t* seq_lens,
                                                   const int32_t* cu_seqlens_q, int num_seqs, int num_q_heads,
                                                   int max_query_len, float scale, int causal, int window_size,
-                                                  float softcap, const float* sinks, float* lse,
+                                                  float softcap, const float* sinks, const float* alibi_slopes, float* lse,
                                                   kvq_stream_t stream) {
   const char* op = "paged_attn_int8_static_scratch";
   kvq::DeviceSymbols sym;
@@ -218,7 +220,7 @@ extern "C" int kvq_paged_attn_int8_static_scratch(void* out, int out_dtype, int6
   // launch's main kernel first (slots it does not own are masked out bit-wise, whatever they hold).
   return kvq::paged_attn_launch(op, out, out_dtype, out_stride_t, out_stride_h, q, q_dtype, q_stride_t, q_stride_h,
                                 cache, geom, block_table, bt_stride, seq_lens, cu_seqlens_q, num_seqs, num_q_heads,
-                                max_query_len, scale, causal, window_size, softcap, sinks, lse, ptr,
+                                max_query_len, scale, causal, window_size, softcap, sinks, alibi_slopes, lse, ptr,
                                 KVQ_STATIC_SCRATCH_BYTES,
                                 "batch too large for the built-in scratch: split-K state", stream);
 }

@@ -835,7 +835,7 @@ static int launch_streamk(const StreamKArgs& a, hipStream_t s) {
   // a head's records of a block back to back (HND order): the tile loads may stream past the caches
   // (not at head size 256, where it measured slower: 293 against 279 us on 64 x 1k-8k tokens)
   const bool stream = D <= 128 && a.io.g.stride_slot == 2 * (code_bytes(a.io.g) + 4) && a.io.g.block_size >= 16;
-  if (a.io.cap_c != 0.f) {
+  if (a.io.cap_c != 0.f || a.io.alibi != nullptr) {   // the instantiation with the extras: soft cap and ALiBi
     switch (hpw) {
       case 8: KVQ_SK(8, true); break;
       case 4: KVQ_SK(4, true); break;

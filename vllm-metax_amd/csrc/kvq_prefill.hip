@@ -79,7 +79,7 @@ struct PrefillTile {
   template <bool MASK>
   __device__ static void qk_softmax(const AttnIO& io, const LaneOffsets& lo, const half8_t (&qb)[NT][KSTEPS],
                                     const float (&s_init)[NT], const int (&limit)[NT], uint32_t wspan, int t, int lane,
-                                    const uint8_t* lds, State& st, half8_t (&p_op)[NT]) {
+                                    const uint8_t* lds, State& st, half8_t (&p_op)[NT], const float (&ali)[NT]) {
     const int g = lane >> 4;
     const float* sc_lds = reinterpret_cast<const float*>(lds + LDS_TILE);
     floatx4 s[NT][2];
@@ -129,6 +129,11 @@ struct PrefillTile {
       if (capped) {
 #pragma unroll
         for (int j = 0; j < 8; ++j) logit[j] = soft_cap(logit[j], io.cap_c, io.cap_k);
+      }
+      if (io.alibi != nullptr) {   // uniform; the column's query stands at limit - 1
+        const float rel0 = (float)(tok_base - (limit[nt] - 1));
+#pragma unroll
+        for (int j = 0; j < 8; ++j) logit[j] = __builtin_fmaf(ali[nt], rel0 + (float)((j >> 2) * 16 + (j & 3)), logit[j]);
       }
 #pragma unroll
       for (int mt = 0; mt < 2; ++mt) {
@@ -350,7 +355,9 @@ __global__ __launch_bounds__(WPW * 64) void paged_prefill_kernel(PrefillArgs a) 
   nb = DTile::fetch_blocks(io, bt_row, len, t + 1);
 
   half8_t qb[NT][PT::KSTEPS];
-  float s_init[NT];
+  float s_init[NT], ali[NT];
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt) ali[nt] = alibi_slope(io.alibi, valid[nt] ? head[nt] : hkv * io.group);
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt)
     s_init[nt] = DTile::load_q_row(io, row[nt] * io.q_stride_t + (int64_t)(valid[nt] ? head[nt] : hkv * io.group) * io.q_stride_h,
@@ -374,15 +381,15 @@ __global__ __launch_bounds__(WPW * 64) void paged_prefill_kernel(PrefillArgs a) 
     DTile::phase_fence();
     nb = DTile::fetch_blocks(io, bt_row, len, t + 2);
     if ((t + 1) * kTile <= min_limit && t * kTile >= max_first)
-      PT::template qk_softmax<false>(io, lo, qb, s_init, limit, wspan, t, lane, lds, st, p_op);
+      PT::template qk_softmax<false>(io, lo, qb, s_init, limit, wspan, t, lane, lds, st, p_op, ali);
     else
-      PT::template qk_softmax<true>(io, lo, qb, s_init, limit, wspan, t, lane, lds, st, p_op);
+      PT::template qk_softmax<true>(io, lo, qb, s_init, limit, wspan, t, lane, lds, st, p_op, ali);
     PT::pv(lo, p_op, lds, st);
     DTile::phase_fence();
     ++t;
   }
   DTile::stage(kv, lo, sc_mul, lane, lds);
-  PT::template qk_softmax<true>(io, lo, qb, s_init, limit, wspan, t, lane, lds, st, p_op);
+  PT::template qk_softmax<true>(io, lo, qb, s_init, limit, wspan, t, lane, lds, st, p_op, ali);
   PT::pv(lo, p_op, lds, st);
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt) PT::emit(io, nt, row[nt], head[nt], valid[nt], lane, st);
@@ -581,12 +588,14 @@ struct Flash32 {
 
   // One tile for the wave's 32 columns.  S^T[32 tokens, 32 columns]: lane (c = column, g) holds
   // token (i/4)*8 + 4g + i%4 in register i.
-  // EXT: the column sees only tokens [limit - wspan, limit) (sliding window) and the logits may
-  // pass through the soft cap (cap_c != 0); without EXT wspan, cap_c and cap_k are not looked at.
+  // EXT: the column sees only tokens [limit - wspan, limit) (sliding window), the logits may
+  // pass through the soft cap (cap_c != 0) and take the ALiBi bias ali x (token - (limit - 1)) when `biased` (uniform;
+  // the column's query stands at limit - 1); without EXT wspan, cap_c, cap_k, ali and biased are not looked at.
   template <bool MASK, bool EXT>
   __device__ static __forceinline__ void compute(const uint8_t* buf, const half8_t (&qb)[KS], float s_init, int limit,
                                                  uint32_t wspan, float cap_c, float cap_k, int t, int lane,
-                                                 floatx16 (&o)[MT], float& m, float& l) {
+                                                 floatx16 (&o)[MT], float& m, float& l, float ali = 0.f,
+                                                 bool biased = false) {
     const int c = lane & 31, g = lane >> 5;
     const float* sc = reinterpret_cast<const float*>(buf + K_BYTES + V_BYTES);
     floatx16 s;
@@ -628,6 +637,13 @@ struct Flash32 {
         for (int r = 0; r < 4; ++r) s[4 * q + r] = __builtin_fmaf(s[4 * q + r], ksc[r], -mref);
       }
     }
+    if constexpr (EXT) {
+      if (biased) {
+        const float rel0 = (float)(tok_base - (limit - 1));
+#pragma unroll
+        for (int i = 0; i < 16; ++i) s[i] = __builtin_fmaf(ali, rel0 + (float)((i >> 2) * 8 + (i & 3)), s[i]);
+      }
+    }
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
 #pragma unroll
@@ -650,7 +666,9 @@ struct Flash32 {
     const float allow = sc[64];
     const float up = fresh ? (d == -INFINITY ? 0.f : d) : (d > allow ? d : 0.f);
     if (__builtin_amdgcn_ballot_w64(up != 0.f) != 0) {
-      const float alpha = __builtin_amdgcn_exp2f(-up);  // a fresh column's o and l are still zero
+      // a fresh column's o and l are still zero and stay so (its first logits may lie so far below zero, under an
+      // ALiBi bias, that 2^-up is no finite number)
+      const float alpha = fresh ? 0.f : __builtin_amdgcn_exp2f(-up);
       l *= alpha;
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) o[mt] *= alpha;
@@ -811,6 +829,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const float s_init =
         FP::load_q(io, row * io.q_stride_t + (int64_t)(valid ? head : hkv * io.group) * io.q_stride_h, valid, lane, qb);
     const float sc_mul = lane < 32 ? io.scale_log2 * DTile::kKScaleMul : kPScale;
+    float ali = 0.f;
+    bool biased = false;
+    if constexpr (EXT) {
+      biased = io.alibi != nullptr;
+      ali = alibi_slope(io.alibi, valid ? head : hkv * io.group);
+    }
 
     drop(A, raws);  // t_first is even: raw window 0
     issue(nb, t_first + 2, A);
@@ -828,9 +852,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       if constexpr (decltype(masked)::value) {
         bool live = t * kTile < wave_max_limit;
         if constexpr (EXT) live = live && (t + 1) * kTile > wave_min_first;
-        if (live) FP::template compute<true, EXT>(buf, qb, s_init, limit, wspan, io.cap_c, io.cap_k, t, lane, o, m, l);
+        if (live)
+          FP::template compute<true, EXT>(buf, qb, s_init, limit, wspan, io.cap_c, io.cap_k, t, lane, o, m, l, ali, biased);
       } else {
-        FP::template compute<false, EXT>(buf, qb, s_init, limit, wspan, io.cap_c, io.cap_k, t, lane, o, m, l);
+        FP::template compute<false, EXT>(buf, qb, s_init, limit, wspan, io.cap_c, io.cap_k, t, lane, o, m, l, ali, biased);
       }
     };
     // Tiles below every column's limit need no mask.  They and the masked tail are two separate
@@ -920,7 +945,7 @@ static int launch_prefill_nt(PrefillArgs& a, int max_query_len, hipStream_t s) {
   // long runs: the workgroup-shared fp16 tile (compute-bound shape), for every kind of code
   if constexpr (D <= 128) {
     if (max_query_len * a.io.group >= 64) {
-      const bool ext = a.io.window > 0 || a.io.cap_c != 0.f;
+      const bool ext = a.io.window > 0 || a.io.cap_c != 0.f || a.io.alibi != nullptr;
       if (int4) {
         if (ext) return launch_prefill_flash32<D, QDT, ODT, true, KVQ_CODE_INT4>(a, max_query_len, s);
         return launch_prefill_flash32<D, QDT, ODT, false, KVQ_CODE_INT4>(a, max_query_len, s);

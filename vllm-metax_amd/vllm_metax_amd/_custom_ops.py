@@ -89,13 +89,14 @@ def eps_for_dtype(dtype: torch.dtype) -> float:
     return got
 
 
-def _check_sinks(sinks, num_q_heads: int, dev) -> None:
-    """Attention sinks as the library takes them: contiguous float32 ``[num_q_heads]`` on the call's device."""
+def _check_sinks(sinks, num_q_heads: int, dev, what: str = "sinks") -> None:
+    """Attention sinks (or ALiBi slopes) as the library takes them: contiguous float32 ``[num_q_heads]`` on the
+    call's device."""
     if sinks is None:
         return
     if sinks.dtype != torch.float32 or not sinks.is_contiguous() or tuple(sinks.shape) != (num_q_heads,) \
             or sinks.device != dev:
-        raise RuntimeError("sinks must be a contiguous float32 [num_q_heads] tensor on the device of q")
+        raise RuntimeError(f"{what} must be a contiguous float32 [num_q_heads] tensor on the device of q")
 
 
 def device_num_cus() -> int:
@@ -315,11 +316,17 @@ def unified_attention(
     workspace tensor (nothing is allocated; calls on one GPU must then not overlap in time).
     ``sinks`` ``[Hq]`` float32: attention sinks, one more logit per head with a zero value row (the reference
     passes them through, triton_attn.py:712).
+    ``alibi_slopes`` ``[Hq]`` float32: the logit of query position p and key position j gets ``slope * (j - p)``
+    added (triton_attn.py:699; causal attention only); the square-root form (``use_alibi_sqrt``) is not built.
     ``has_decode_rows=False`` is the caller's promise that no sequence of the batch has exactly one query row (a
     pure prefill batch): the decode kernel and its reduce are then not launched."""
     code_type = code_type_of(kv_quant_mode)
-    if alibi_slopes is not None or output_scale is not None or mm_prefix_range is not None:
-        raise NotImplementedError("alibi, fused output quantisation and mm-prefix ranges are not built")
+    if output_scale is not None or mm_prefix_range is not None:
+        raise NotImplementedError("fused output quantisation and mm-prefix ranges are not built")
+    if use_alibi_sqrt:
+        raise NotImplementedError("the square-root form of ALiBi is not built")
+    if alibi_slopes is not None and not causal:
+        raise NotImplementedError("ALiBi needs causal attention")
     softcap = float(softcap or 0.0)
     if softcap < 0:
         raise RuntimeError("softcap must be >= 0")
@@ -359,6 +366,7 @@ def unified_attention(
         return
     num_q_heads = q.shape[1]
     _check_sinks(sinks, num_q_heads, q.device)
+    _check_sinks(alibi_slopes, num_q_heads, q.device, "alibi_slopes")
     lib = _C.load()
     if lse is not None and (lse.dtype != torch.float32 or not lse.is_contiguous()
                             or tuple(lse.shape) != (q.shape[0], num_q_heads)):
@@ -369,7 +377,7 @@ def unified_attention(
             ctypes.c_void_p(geom.base_ptr), ctypes.byref(g), _ptr(block_table), block_table.stride(0),
             _ptr(seqused_k), _ptr(cu_seqlens_q), num_seqs, num_q_heads, int(max_seqlen_q),
             float(softmax_scale), (1 if causal else 0) | (0 if has_decode_rows else 2), window, softcap,
-            _ptr(sinks), _ptr(lse))
+            _ptr(sinks), _ptr(alibi_slopes), _ptr(lse))
     if static_scratch:
         with _on_device(dev):
             rc = lib.kvq_paged_attn_int8_static_scratch(*head, _stream(dev))
@@ -403,6 +411,7 @@ def decode_attention_with_cache_update(
     lse: torch.Tensor | None = None,
     slot_mapping: torch.Tensor | None = None,
     sinks: torch.Tensor | None = None,
+    alibi_slopes: torch.Tensor | None = None,
 ) -> None:
     """A decode step in one launch: the cache update of ``reshape_and_cache_flash_per_token_head_quant`` and the
     attention of ``unified_attention`` with one query row per sequence, for a backend whose ``forward`` includes
@@ -456,6 +465,7 @@ def decode_attention_with_cache_update(
                             or tuple(lse.shape) != (num_seqs, num_q_heads)):
         raise RuntimeError("lse must be a contiguous float32 [num_seqs, num_q_heads] tensor")
     _check_sinks(sinks, num_q_heads, q.device)
+    _check_sinks(alibi_slopes, num_q_heads, q.device, "alibi_slopes")
     lib = _C.load()
     g = geom.as_struct()
     if workspace is None:
@@ -467,7 +477,7 @@ def decode_attention_with_cache_update(
             _ptr(key), _ptr(value), _dtype_code(key, "key"), key.stride(0), key.stride(1), value.stride(0),
             value.stride(1), eps_for_dtype(key.dtype), ctypes.c_void_p(geom.base_ptr), ctypes.byref(g),
             _ptr(block_table), block_table.stride(0), _ptr(seqused_k), _ptr(slot_mapping), num_seqs, num_q_heads,
-            float(softmax_scale), window, softcap, _ptr(sinks), _ptr(lse), _ptr(workspace),
+            float(softmax_scale), window, softcap, _ptr(sinks), _ptr(alibi_slopes), _ptr(lse), _ptr(workspace),
             workspace.numel() * workspace.element_size(), _stream(dev))
     _C.check(rc, "decode_attention_with_cache_update")
 

@@ -275,7 +275,7 @@ class Int8AttentionImpl(_ImplBase):
                  attn_type: str = AttentionType.DECODER, kv_sharing_target_layer_name: str | None = None,
                  sinks: torch.Tensor | None = None, use_alibi_sqrt: bool = False, chunk_lookback: int = -1) -> None:
         unsupported = {
-            "alibi_slopes": alibi_slopes is not None,
+            "use_alibi_sqrt": bool(use_alibi_sqrt),
             "kv_sharing_target_layer_name": kv_sharing_target_layer_name is not None,
             "chunk_lookback": chunk_lookback not in (-1, None),
         }
@@ -295,6 +295,12 @@ class Int8AttentionImpl(_ImplBase):
                              f"Sinks shape: {tuple(sinks.shape)}, num_heads: {num_heads}.")
         # the kernels read the sinks as float32; converted once (a parameter in the model's dtype otherwise)
         self.sinks = None if sinks is None else sinks.detach().to(torch.float32).contiguous()
+        # ALiBi slopes as a float32 tensor, as the reference keeps them (triton_attn.py:504-506)
+        if alibi_slopes is not None:
+            alibi_slopes = torch.as_tensor(alibi_slopes, dtype=torch.float32).contiguous()
+            if tuple(alibi_slopes.shape) != (num_heads,):
+                raise ValueError(f"alibi_slopes must have one slope per head ({num_heads}), got {tuple(alibi_slopes.shape)}")
+        self.alibi_slopes = alibi_slopes
         self.num_heads = num_heads
         self.head_size = head_size
         self.scale = float(scale)
@@ -344,6 +350,11 @@ class Int8AttentionImpl(_ImplBase):
         if self.sinks is not None and self.sinks.device != device:
             self.sinks = self.sinks.to(device)
         return self.sinks
+
+    def _alibi_on(self, device):
+        if self.alibi_slopes is not None and self.alibi_slopes.device != device:
+            self.alibi_slopes = self.alibi_slopes.to(device)
+        return self.alibi_slopes
 
     # -- cache views ---------------------------------------------------------------------------
     def _ensure_scale_caches(self, kv_cache: torch.Tensor) -> None:
@@ -411,7 +422,8 @@ class Int8AttentionImpl(_ImplBase):
             window_size=self.sliding_window, block_table=attn_metadata.block_table, softcap=self.logits_soft_cap,
             kv_quant_mode=self._kv_quant_mode, k_scale_cache=self._k_scale_cache, v_scale_cache=self._v_scale_cache,
             workspace=attn_metadata.workspace, geometry=self._geometry,
-            has_decode_rows=getattr(attn_metadata, "has_decode_rows", True), sinks=self._sinks_on(q.device))
+            has_decode_rows=getattr(attn_metadata, "has_decode_rows", True), sinks=self._sinks_on(q.device),
+            alibi_slopes=self._alibi_on(q.device))
         return output
 
 
@@ -448,7 +460,7 @@ class Int8FusedUpdateAttentionImpl(Int8AttentionImpl):
             window_size=self.sliding_window, softcap=self.logits_soft_cap, kv_quant_mode=self._kv_quant_mode,
             workspace=attn_metadata.workspace, geometry=self._geometry,
             slot_mapping=attn_metadata.slot_mapping[:n] if attn_metadata.slot_mapping is not None else None,
-            sinks=self._sinks_on(query.device))
+            sinks=self._sinks_on(query.device), alibi_slopes=self._alibi_on(query.device))
         return output
 
 
