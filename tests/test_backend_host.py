@@ -193,6 +193,10 @@ def test_impl_constructor_errors():
     for kw in (dict(use_alibi_sqrt=True), dict(attn_type=AttentionType.ENCODER_ONLY)):
         with pytest.raises(NotImplementedError):
             mk(**kw)
+    # cross-attention goes through the cache like decoder self-attention (triton_attn.py:394-402, 796-799)
+    assert mk(attn_type=AttentionType.ENCODER_DECODER).attn_type == AttentionType.ENCODER_DECODER
+    assert Int8AttentionBackend.supports_attn_type(AttentionType.ENCODER_DECODER)
+    assert not Int8AttentionBackend.supports_attn_type(AttentionType.ENCODER)
     # ALiBi slopes: a float32 tensor with one slope per head, as the reference keeps them (triton_attn.py:504-506)
     al = mk(alibi_slopes=[0.5] * 32).alibi_slopes
     assert al.dtype == torch.float32 and tuple(al.shape) == (32,) and mk().alibi_slopes is None

@@ -233,3 +233,26 @@ def test_pure_prefill_batch_with_the_no_decode_rows_promise(gpu_device):
         assert torch.equal(outs[0][0].view(torch.int16), outs[1][0].view(torch.int16)) and torch.equal(outs[0][1], outs[1][1])
         want = oracle.paged_attn(q, T.storage_bytes(kv_cpu), lay, bt, sl, cu, 0.0884)
         T.assert_close_attn(outs[1][0], want, what="pure prefill batch")
+
+
+@pytest.mark.parametrize("hq,hkv,d,layout", [(32, 8, 128, "HND"), (28, 4, 128, "NHD"), (8, 2, 64, "HND"), (4, 2, 256, "NHD")])
+def test_non_causal_rows_see_every_key(gpu_device, hq, hkv, d, layout):
+    """causal=False, the cross-attention form of the reference's call (`causal=attn_metadata.causal`,
+    vllm_metax/v1/attention/backends/triton_attn.py:698; AttentionType.ENCODER_DECODER goes through the cached
+    path, :394-402): every query row of a run attends all `seq_len` keys, whatever its place in the run -- decode
+    rows, short runs (the per-wave tile), long runs (the workgroup-shared tile), output and lse against the oracle,
+    and every row of a run of copies of one query gets the same bits."""
+    ctx = [700, 33, 1500, 64, 257, 5, 900]
+    qls = [1, 33, 300, 1, 17, 5, 70]
+    kv, lay, bt, q, sl, cu = build(ctx, qls, hq, hkv, d, 16, layout=layout, seed=hq + d + 1)
+    # the last run: copies of one query row
+    q[int(cu[-2]):] = q[int(cu[-2])].clone()
+    scale = 1 / math.sqrt(d)
+    want, want_lse = oracle.paged_attn(q, T.storage_bytes(kv), lay, bt, sl, cu, scale, causal=False, return_lse=True)
+    causal = oracle.paged_attn(q, T.storage_bytes(kv), lay, bt, sl, cu, scale, causal=True)
+    assert not torch.allclose(want, causal, atol=5e-2)
+    got, lse = run(gpu_device, kv, layout, bt, q, sl, cu, max(qls), scale, want_lse=True, causal=False)
+    T.assert_close_attn(got, want, what=f"non-causal {hq}/{hkv} d{d}")
+    torch.testing.assert_close(lse.cpu(), want_lse, atol=5e-3, rtol=1e-3)
+    tail = got[int(cu[-2]):].cpu()
+    assert torch.equal(tail.view(torch.int16), tail[:1].expand_as(tail).contiguous().view(torch.int16))

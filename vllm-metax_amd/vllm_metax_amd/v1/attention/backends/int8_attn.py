@@ -194,7 +194,9 @@ class Int8AttentionBackend(_BackendBase):
 
     @classmethod
     def supports_attn_type(cls, attn_type: str) -> bool:
-        return attn_type == AttentionType.DECODER
+        """Decoder self-attention and cross-attention, the two types that go through the cache; the reference
+        refuses a quantised cache for the encoder types too (triton_attn.py:759-764)."""
+        return attn_type in (AttentionType.DECODER, AttentionType.ENCODER_DECODER)
 
     @classmethod
     def supports_non_causal(cls) -> bool:
@@ -282,8 +284,10 @@ class Int8AttentionImpl(_ImplBase):
         bad = [k for k, v in unsupported.items() if v]
         if bad:  # the way TritonMLAImpl refuses features it lacks (mla/triton_mla.py:177-190)
             raise NotImplementedError(f"Int8AttentionImpl does not support: {', '.join(bad)}")
-        if attn_type != AttentionType.DECODER:
+        if attn_type not in (AttentionType.DECODER, AttentionType.ENCODER_DECODER):   # triton_attn.py:759-764
             raise NotImplementedError("quantized KV cache is not supported for encoder attention")
+        if attn_type == AttentionType.ENCODER_DECODER and alibi_slopes is not None:
+            raise NotImplementedError("ALiBi needs causal attention")
         if not kv_cache_uses_per_token_head_scales(kv_cache_dtype) or get_kv_quant_mode(kv_cache_dtype) not in (
                 KVQuantMode.INT8_PER_TOKEN_HEAD, KVQuantMode.FP8_PER_TOKEN_HEAD, KVQuantMode.INT4_PER_TOKEN_HEAD):
             raise ValueError("Int8AttentionImpl needs kv_cache_dtype 'int8_per_token_head', 'fp8_per_token_head' or 'int4_per_token_head', "
