@@ -296,13 +296,18 @@ KVQ_API int kvq_paged_attn_int8_static_scratch(
  * locally normalised tmp_out[b, h, j, :], max_logits[b, h, j] and
  * exp_sums[b, h, j] (all fp32 here); the reduce then writes out.
  * max_num_partitions = ceil(max_seq_len / partition_size).
+ * alibi_slopes ([num_q_heads] fp32 or NULL): the op's alibi_slopes argument; a key at position j gets
+ * alibi_slopes[h] * (j - seq_len + 1) on its scaled logit before the partition's maximum is taken
+ * (csrc/libtorch_stable/attention/attention_kernels.cuh), so max_logits and exp_sums are those of the
+ * biased logits.
  */
 KVQ_API int kvq_paged_attn_v2_int8(void* out, int out_dtype, float* exp_sums, float* max_logits,
                            float* tmp_out, const void* q, int q_dtype, int64_t q_stride_t,
                            int64_t q_stride_h, const void* cache, const kvq_cache_geom* geom,
                            const int32_t* block_table, int64_t bt_stride,
                            const int32_t* seq_lens, int num_seqs, int num_q_heads, float scale,
-                           int partition_size, int max_num_partitions, kvq_stream_t stream);
+                           const float* alibi_slopes, int partition_size, int max_num_partitions,
+                           kvq_stream_t stream);
 
 /*
  * The reduce stage on its own.  Stands in for paged_attention_v2_reduce_kernel,

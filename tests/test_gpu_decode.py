@@ -245,6 +245,41 @@ def test_fixed_partitions_v2_contract(gpu_device):
     torch.testing.assert_close(lse.cpu(), wl2, atol=1e-4, rtol=1e-5)
 
 
+@pytest.mark.parametrize("hq,hkv,d", [(32, 8, 128), (8, 2, 64), (4, 1, 256)])
+def test_fixed_partitions_v2_with_alibi(gpu_device, hq, hkv, d):
+    """alibi_slopes of paged_attention_v2 (csrc/libtorch_stable/torch_bindings.cpp:631-641; the bias
+    alibi_slopes * (position - seq_len + 1) of tests/kernels/attention/test_attention.py:109-117): the reduced
+    output matches the oracle's biased attention, and the per-partition tmp_out / max_logits / exp_sums are a
+    consistent stage 1 -- the oracle's reduce over them gives the same rows and the biased lse."""
+    dev = gpu_device
+    ctx = [1500, 512, 513, 30, 2048]
+    bs = 16
+    kv_cpu, lay, bt, q, sl, cu = build_case(ctx, hq, hkv, d, bs, "HND", 21)
+    scale = d ** -0.5
+    slopes = torch.tensor([2.0 ** (-8.0 * (i + 1) / hq) for i in range(hq)], dtype=torch.float32)
+    slopes[0] = 1.0
+    P = (max(ctx) + 511) // 512
+    kv = T.to_device_cache(kv_cpu, dev, "HND")
+    k, v = L.key_value_views(kv)
+    ks, vs = L.scale_views(kv)
+    B = len(ctx)
+    out = torch.empty((B, hq, d), dtype=torch.bfloat16, device=dev)
+    es = torch.zeros((B, hq, P), dtype=torch.float32, device=dev)
+    ml = torch.zeros((B, hq, P), dtype=torch.float32, device=dev)
+    tmp = torch.zeros((B, hq, P, d), dtype=torch.float32, device=dev)
+    ops.paged_attention_v2(out, es, ml, tmp, q.to(dev), k, v, hkv, scale, bt.to(dev), sl.to(dev), bs, max(ctx),
+                           alibi_slopes=slopes.to(dev), k_scale=ks, v_scale=vs)
+    torch.cuda.synchronize()
+    base = T.storage_bytes(kv_cpu)
+    want, want_lse = oracle.paged_attn(q, base, lay, bt, sl, cu, scale, alibi_slopes=slopes, return_lse=True)
+    plain = oracle.paged_attn(q, base, lay, bt, sl, cu, scale)
+    assert not torch.allclose(want, plain, atol=5e-2)
+    T.assert_close_attn(out, want, what="v2 with alibi")
+    red, red_lse = oracle.splitk_reduce(tmp.cpu(), ml.cpu(), es.cpu(), sl, 512, return_lse=True)
+    T.assert_close_attn(red, want, atol=2e-3, rtol=2e-3, what="v2 stage 1 with alibi, reduced by the oracle")
+    torch.testing.assert_close(red_lse, want_lse, atol=2e-3, rtol=1e-3)
+
+
 @pytest.mark.parametrize("q_lens", [[1, 1, 1], [1, 5, 129]])
 def test_block_size_does_not_change_the_result(gpu_device, q_lens):
     """The same tokens paged with 16-, 32-, 64- and 128-token blocks give bit-identical outputs (the

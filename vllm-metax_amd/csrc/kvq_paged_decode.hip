@@ -161,7 +161,8 @@ int kvq_paged_attn_v2_int8(void* out, int out_dtype, float* exp_sums, float* max
                            const void* q, int q_dtype, int64_t q_stride_t, int64_t q_stride_h,
                            const void* cache, const kvq_cache_geom* geom, const int32_t* block_table,
                            int64_t bt_stride, const int32_t* seq_lens, int num_seqs, int num_q_heads,
-                           float scale, int partition_size, int max_num_partitions, kvq_stream_t stream) {
+                           float scale, const float* alibi_slopes, int partition_size, int max_num_partitions,
+                           kvq_stream_t stream) {
   using namespace kvq;
   int rc = validate_common("paged_attn_v2_int8", q, cache, geom, block_table, seq_lens, num_seqs, num_q_heads);
   if (rc) return rc;
@@ -183,6 +184,7 @@ int kvq_paged_attn_v2_int8(void* out, int out_dtype, float* exp_sums, float* max
   a.io.num_q_heads = num_q_heads;
   a.io.group = num_q_heads / geom->num_kv_heads;
   a.io.scale_log2 = scale * kLog2e;
+  a.io.alibi = alibi_slopes;
   a.io.bs_magic = (uint32_t)((0x100000000ull + (uint64_t)geom->block_size - 1) / (uint64_t)geom->block_size);
   a.seq_lens = seq_lens;
   a.tmp_out = tmp_out;

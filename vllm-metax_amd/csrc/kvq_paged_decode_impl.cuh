@@ -791,7 +791,8 @@ struct V2Args {
   int max_parts;
 };
 
-template <int D, int QDT, int WPW>
+// BIAS: the instantiation with the ALiBi bias (DecodeTile's form with the extras; the soft cap stays the identity).
+template <int D, int QDT, int WPW, bool BIAS>
 __global__ __launch_bounds__(WPW * 64) void paged_decode_v2_kernel(V2Args a) {
   using DTile = DecodeTile<D, QDT, KVQ_F32>;
   __shared__ __align__(16) uint8_t lds[WPW][DTile::LDS_WAVE];
@@ -805,7 +806,7 @@ __global__ __launch_bounds__(WPW * 64) void paged_decode_v2_kernel(V2Args a) {
   if (t_begin >= ntiles) return;
   const int t_end = min(ntiles, t_begin + a.partition_tiles);
   typename DTile::State st;
-  DTile::template run<false>(a.io, seq, seq, len, 0, t_begin, t_end, hkv, lane, lds[wave], st);
+  DTile::template run<BIAS>(a.io, seq, seq, len, 0, t_begin, t_end, hkv, lane, lds[wave], st);
   DTile::emit_v2(a.io, a.tmp_out, a.max_logits, a.exp_sums, seq, part, a.max_parts, hkv, lane, st);
 }
 
@@ -892,12 +893,23 @@ static int launch_v2(const V2Args& a, int num_seqs, hipStream_t s) {
   const int hkv = a.io.g.num_kv_heads;
   const int wpw = heads_per_wg(hkv);
   dim3 grid(a.max_parts, num_seqs, (hkv + wpw - 1) / wpw);
-  switch (wpw) {
-    case 8: hipLaunchKernelGGL((paged_decode_v2_kernel<D, QDT, 8>), grid, dim3(512), 0, s, a); break;
-    case 4: hipLaunchKernelGGL((paged_decode_v2_kernel<D, QDT, 4>), grid, dim3(256), 0, s, a); break;
-    case 2: hipLaunchKernelGGL((paged_decode_v2_kernel<D, QDT, 2>), grid, dim3(128), 0, s, a); break;
-    default: hipLaunchKernelGGL((paged_decode_v2_kernel<D, QDT, 1>), grid, dim3(64), 0, s, a); break;
+#define KVQ_V2(W, BIAS) hipLaunchKernelGGL((paged_decode_v2_kernel<D, QDT, W, BIAS>), grid, dim3(W * 64), 0, s, a)
+  if (a.io.alibi != nullptr) {
+    switch (wpw) {
+      case 8: KVQ_V2(8, true); break;
+      case 4: KVQ_V2(4, true); break;
+      case 2: KVQ_V2(2, true); break;
+      default: KVQ_V2(1, true); break;
+    }
+  } else {
+    switch (wpw) {
+      case 8: KVQ_V2(8, false); break;
+      case 4: KVQ_V2(4, false); break;
+      case 2: KVQ_V2(2, false); break;
+      default: KVQ_V2(1, false); break;
+    }
   }
+#undef KVQ_V2
   return check_hip(hipGetLastError(), "paged_attn_v2_int8 launch");
 }
 

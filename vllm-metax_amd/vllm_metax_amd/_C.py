@@ -62,7 +62,7 @@ SIGNATURES = {
     "kvq_paged_attn_int8_static_scratch": (_i, [_vp, _i, _i64, _i64, _vp, _i, _i64, _i64, _vp, _geom_p, _vp, _i64, _vp,
                                                 _vp, _i, _i, _i, _f, _i, _i, _f, _vp, _vp, _vp, _vp]),
     "kvq_paged_attn_v2_int8": (_i, [_vp, _i, _vp, _vp, _vp, _vp, _i, _i64, _i64, _vp, _geom_p, _vp, _i64, _vp,
-                                    _i, _i, _f, _i, _i, _vp]),
+                                    _i, _i, _f, _vp, _i, _i, _vp]),
     "kvq_splitk_reduce": (_i, [_vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
     "kvq_swap_blocks": (_i, [_vp, _vp, _i64, _vp, _i64, _i64, _i64, _i, _vp]),
     "kvq_swap_blocks_batch": (_i, [_vp, _vp, _vp, _i64, _i, _vp]),

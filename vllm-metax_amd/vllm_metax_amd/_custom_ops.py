@@ -506,11 +506,11 @@ def paged_attention_v2(
     """Fixed-partition split-K decode, argument order of ``paged_attention_v2``
     (csrc/libtorch_stable/torch_bindings.cpp:631-641).  key_cache/value_cache are the int8 cache
     views and k_scale/v_scale the per-(token, head) fp32 scale views; exp_sums / max_logits
-    ``[B, Hq, P]`` and tmp_out ``[B, Hq, P, D]`` are fp32, P = ceil(max_seq_len / partition_size)."""
+    ``[B, Hq, P]`` and tmp_out ``[B, Hq, P, D]`` are fp32, P = ceil(max_seq_len / partition_size).
+    ``alibi_slopes`` ``[Hq]`` float32 as in the reference op: the key at position j gets
+    ``slope * (j - seq_len + 1)`` on its scaled logit."""
     if kv_cache_dtype != "int8_per_token_head":
         raise NotImplementedError(f"kv_cache_dtype {kv_cache_dtype!r}: only int8_per_token_head is built")
-    if alibi_slopes is not None:
-        raise NotImplementedError("alibi is not built")
     if k_scale is None or v_scale is None:
         raise RuntimeError("k_scale / v_scale (the per-token-head scale views) are required")
     dev = _require_cuda(out, exp_sums, max_logits, tmp_out, query, key_cache, value_cache, block_tables, seq_lens, k_scale, v_scale)
@@ -527,13 +527,14 @@ def paged_attention_v2(
         raise RuntimeError("out must be contiguous [B, Hq, D]; query head dim contiguous")
     if seq_lens.dtype != torch.int32 or block_tables.dtype != torch.int32 or block_tables.stride(1) != 1:
         raise RuntimeError("seq_lens and block_tables must be int32 (rows contiguous)")
+    _check_sinks(alibi_slopes, Hq, query.device, "alibi_slopes")
     g = geom.as_struct()
     with _on_device(dev):
         rc = _C.load().kvq_paged_attn_v2_int8(
             _ptr(out), _dtype_code(out, "out"), _ptr(exp_sums), _ptr(max_logits), _ptr(tmp_out), _ptr(query),
             _dtype_code(query, "query"), query.stride(0), query.stride(1), ctypes.c_void_p(geom.base_ptr),
             ctypes.byref(g), _ptr(block_tables), block_tables.stride(0), _ptr(seq_lens), B, Hq, float(scale),
-            int(partition_size), int(P), _stream(dev))
+            _ptr(alibi_slopes), int(partition_size), int(P), _stream(dev))
     _C.check(rc, "paged_attention_v2")
 
 
