@@ -746,6 +746,8 @@ def main():
                          "(vllm_metax_amd.layout.get_kv_cache_layout(): HND unless the environment says otherwise), "
                          "so that the headline is the order a deployment gets; the default workload reports the other "
                          "order too")
+    ap.add_argument("--seed", type=int, default=0,
+                    help="draw of the workload's random context lengths (0 = the draw every published figure uses)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-one-launch", action="store_true",
                     help="skip the one-launch variant of the step (write inside the decode launch): for profiler runs, "
@@ -764,7 +766,7 @@ def main():
     if args.kv_layout is None:
         args.kv_layout = get_kv_cache_layout()
     dev = torch.device("cuda:0")
-    cfg = make_batch(args.workload)
+    cfg = make_batch(args.workload, args.seed)
     cfg["kv_dtype"] = args.kv_dtype
     if cfg.get("mla_prefill"):
         return mla_prefill_main(args, cfg, dev, ops)
@@ -797,6 +799,7 @@ def main():
                    "q_heads": cfg["hq"], "kv_heads": cfg["hkv"], "head_dim": cfg["d"], "block_size": cfg["bs"],
                    "pool_blocks": cfg["pool"], "layer_caches_rotated": L, "kv_layout": args.kv_layout,
                    **({"batch_invariant": True} if ops.batch_invariant() else {}),
+                   **({"lengths_seed": args.seed} if args.seed else {}),
                    **({"kv_dtype": args.kv_dtype + "_per_token_head"} if args.kv_dtype != "int8" else {}),
                    **({"sliding_window": args.sliding_window} if args.sliding_window else {}),
                    **({"soft_cap": args.soft_cap} if args.soft_cap else {})},
