@@ -42,6 +42,19 @@ struct VarlenArgs {
   float scale_log2;
 };
 
+// acc + the two 16-bit floats of `pair` (fp16 or bf16).
+template <int DT>
+__device__ __forceinline__ float pair_sum(uint32_t pair, float acc) {
+  if constexpr (DT == KVQ_F16) {
+    const half2_t one = {(half_t)1.0f, (half_t)1.0f};
+    return __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, pair), one, acc, false);
+  } else {
+    typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+    const bf16x2_t one = {(__bf16)1.0f, (__bf16)1.0f};
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, pair), one, acc, false);
+  }
+}
+
 template <int NDW>
 struct Words {
   uint32_t w[NDW];
@@ -122,6 +135,8 @@ __global__ __launch_bounds__(256) void varlen_attn_kernel(VarlenArgs a) {
     blk_k_end[rb] = q0[rb] >= q_len ? 0 : (a.causal ? max(0, min(k_len, q0[rb] + 15 + diag + 1)) : k_len);
   }
   const int wave_tiles = (max(blk_k_end[0], blk_k_end[1]) + 31) / 32;   // tiles this wave has anything to do in
+  // the smallest limit among the wave's rows: tiles that end at or below it are visible to every row
+  const int wave_min_limit = -wave_max_i32(-min(my_limit[0], my_limit[1]));
 
   floatx4 oacc[RB][DPL];
   float m[RB], l[RB];
@@ -221,32 +236,45 @@ __global__ __launch_bounds__(256) void varlen_attn_kernel(VarlenArgs a) {
       bool moved = false;
 #pragma unroll
       for (int rb = 0; rb < RB; ++rb) {
+        // the maximum is taken over the raw products (the scale is positive and the same for every key), so that
+        // scale and maximum enter each logit in ONE multiply-add
+        // only a tile that reaches past some row's limit (the causal diagonal, the end of the keys) is masked: a
+        // uniform branch round the compares and selects, which work on the products where they lie
+        if ((t + 1) * 32 > wave_min_limit) {
+#pragma unroll
+          for (int j = 0; j < 8; ++j) {
+            const int key = t * 32 + 16 * (j >> 2) + 4 * g + (j & 3);
+            sacc[rb][j >> 2][j & 3] = key < my_limit[rb] ? sacc[rb][j >> 2][j & 3] : -INFINITY;
+          }
+        }
         float sc[8];
         float mx = -INFINITY;
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
-          const int key = t * 32 + 16 * (j >> 2) + 4 * g + (j & 3);
-          const float sv = sacc[rb][j >> 2][j & 3] * a.scale_log2;
-          sc[j] = key < my_limit[rb] ? sv : -INFINITY;
+          sc[j] = sacc[rb][j >> 2][j & 3];
           mx = fmaxf(mx, sc[j]);
         }
-        mx = max_over_quarters(mx);
+        mx = max_over_quarters(mx) * a.scale_log2;
         const float m_new = fmaxf(m[rb], mx);
         const float m_use = m_new == -INFINITY ? 0.f : m_new;
         alpha[rb] = __builtin_amdgcn_exp2f(m[rb] - m_use);
         moved = moved || m_new > m[rb];
-        float p[8], psum = 0.f;
+        const float off = kShift - m_use;
+        float p[8];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          p[j] = __builtin_amdgcn_exp2f(sc[j] - m_use + kShift);
-          psum += p[j];
-        }
-        l[rb] = l[rb] * alpha[rb] + psum;
+        for (int j = 0; j < 8; ++j)
+          p[j] = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[j], a.scale_log2, off));   // a masked key: 2^-inf = 0
         m[rb] = m_new;
         pk[rb].x = pack2<DT>(p[0], p[1]);
         pk[rb].y = pack2<DT>(p[2], p[3]);
         pk[rb].z = pack2<DT>(p[4], p[5]);
         pk[rb].w = pack2<DT>(p[6], p[7]);
+        // the row sum is that of the weights as the second product sees them (rounded to the input type): one
+        // two-element dot product with ones per packed pair instead of two additions
+        float psum = 0.f;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) psum = pair_sum<DT>(pk[rb][w], psum);
+        l[rb] = l[rb] * alpha[rb] + psum;
       }
       // ---- O^T = alpha O^T + V^T P^T.  The accumulators are rescaled only in the tiles in which some row's
       //      maximum moved (they live in accumulation registers: a rescale is a read, a multiply and a write
@@ -324,6 +352,7 @@ extern "C" int kvq_mla_prefill_attn(const void* q, int dtype, int64_t q_stride_t
   KVQ_REQUIRE(num_seqs >= 0 && max_seqlen_q >= 0 && total_q >= 0 && num_heads > 0, "%s: bad sizes", op);
   if (num_seqs == 0 || max_seqlen_q == 0 || total_q == 0) return KVQ_OK;
   KVQ_REQUIRE(dtype == KVQ_BF16 || dtype == KVQ_F16, "%s: q, k and v must be bf16 or fp16 (dtype %d)", op, dtype);
+  KVQ_REQUIRE(scale > 0.f && scale < INFINITY, "%s: scale must be positive and finite", op);   // the kernel takes row maxima before scaling
   KVQ_REQUIRE(q && k_nope && v && out && cu_seqlens_q && cu_seqlens_k, "%s: NULL pointer", op);
   KVQ_REQUIRE(rope_dim == 0 || k_pe != nullptr, "%s: k_pe is NULL with rope_dim %d", op, rope_dim);
   KVQ_REQUIRE(num_heads <= 65535 && num_seqs <= 65535, "%s: more than 65535 heads or sequences", op);
