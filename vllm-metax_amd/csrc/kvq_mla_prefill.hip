@@ -16,11 +16,10 @@
 //                 reduction over the four quarter-waves and alpha / l stay in the lane.
 //   O^T = V^T P^T B = P~ straight from the S^T registers (k slot j of quarter g is key 16 (j / 4) + 4 g +
 //                 j % 4; any order works as long as V uses the same one).  A = V^T needs 8 keys of one
-//                 dim per lane while a V row holds 8 dims of one key together: each lane reads the slice
-//                 [its 8 keys] x [DV / 16 consecutive dims] and transposes it in registers with one
-//                 v_perm_b32 per output dword (once per tile, for both row blocks).  Output block i then
-//                 holds dims (DV/16) * lane + i, which leaves every lane with 4 runs of DV/16 consecutive
-//                 dims of its own query row: 16-byte stores.
+//                 dim per lane while a V row holds the dims of one key together: the LDS's transposing read
+//                 (ds_read_b64_tr_b16) hands a lane four keys of one dim out of four rows, two of them make an
+//                 operand, no register shuffles.  Output block i holds dims 16 i .. 16 i + 15; a lane ends
+//                 with dims 16 i + 4 g .. + 3 of its own query row: 8-byte stores.
 // Masked keys (beyond the sequence, or above the causal diagonal, which is aligned to the END of the
 // keys as flash-attention does) get weight 0; their rows are clamped copies of the last valid key.
 #include "kvq_attn_core.cuh"
@@ -55,39 +54,17 @@ __device__ __forceinline__ float pair_sum(uint32_t pair, float acc) {
   }
 }
 
-template <int NDW>
-struct Words {
-  uint32_t w[NDW];
-};
-template <int NDW>
-__device__ __forceinline__ Words<NDW> load_words(const uint16_t* p) {
-  Words<NDW> r;
-  if constexpr (NDW == 2) {
-    const u32x2 v = *reinterpret_cast<const u32x2*>(p);
-    r.w[0] = v.x;
-    r.w[1] = v.y;
-  } else {
-#pragma unroll
-    for (int i = 0; i < NDW / 4; ++i) {
-      const u32x4 v = reinterpret_cast<const u32x4*>(p)[i];
-      r.w[4 * i] = v.x;
-      r.w[4 * i + 1] = v.y;
-      r.w[4 * i + 2] = v.z;
-      r.w[4 * i + 3] = v.w;
-    }
-  }
-  return r;
-}
-
 template <int DT, int NOPE, int ROPE, int DV>
 __global__ __launch_bounds__(256) void varlen_attn_kernel(VarlenArgs a) {
   constexpr int KSN = NOPE / 32, KSR = ROPE / 32, KS = KSN + KSR;   // k-steps of the QK product
   constexpr int DPL = DV / 16;                                      // dims per lane and output block
-  constexpr int VR = DPL / 2;                                       // dwords of one key's slice
   constexpr int RB = 2;                                             // row blocks of 16 per wave
   constexpr int KC = (NOPE + ROPE) / 8, KCN = NOPE / 8;             // 16-byte chunks of a K row / of its nope part
   constexpr int VC = DV / 8;                                        // chunks of a V row
-  constexpr int K_BYTES = 32 * KC * 16, V_BYTES = 32 * VC * 16;
+  // V rows carry 32 bytes of padding: the transposing reads of a quarter-wave take 32 bytes from each of four
+  // successive rows, which the padding puts on different banks
+  constexpr int V_PITCH = VC * 16 + 32;
+  constexpr int K_BYTES = 32 * KC * 16, V_BYTES = 32 * V_PITCH;
   constexpr int KLD = (32 * KC + 255) / 256, VLD = (32 * VC + 255) / 256;   // chunk loads per thread and tile
   // fp16 weights are kept 2^8 larger so that small ones stay normal; l carries the same factor
   constexpr float kShift = DT == KVQ_F16 ? 8.f : 0.f;
@@ -193,7 +170,7 @@ __global__ __launch_bounds__(256) void varlen_attn_kernel(VarlenArgs a) {
 #pragma unroll
     for (int i = 0; i < VLD; ++i) {
       const int q = tid + 256 * i;
-      if (q < 32 * VC) *reinterpret_cast<u32x4*>(buf + K_BYTES + q * 16) = vreg[i];
+      if (q < 32 * VC) *reinterpret_cast<u32x4*>(buf + K_BYTES + (q / VC) * V_PITCH + (q % VC) * 16) = vreg[i];
     }
   };
 
@@ -225,11 +202,6 @@ __global__ __launch_bounds__(256) void varlen_attn_kernel(VarlenArgs a) {
           for (int rb = 0; rb < RB; ++rb) sacc[rb][blk] = mfma16<DT>(ka, qop[rb][s], sacc[rb][blk]);
         }
       }
-      // ---- the lane's 8 keys' slices of V (k slot j = 4 blk + r is key 16 blk + 4 g + r)
-      Words<VR> vrow[8];
-#pragma unroll
-      for (int j = 0; j < 8; ++j)
-        vrow[j] = load_words<VR>(reinterpret_cast<const uint16_t*>(buf + K_BYTES + (16 * (j >> 2) + 4 * g + (j & 3)) * (VC * 16)) + DPL * c);
       // ---- online softmax in base 2, per row block
       u32x4 pk[RB];
       float alpha[RB];
@@ -285,16 +257,22 @@ __global__ __launch_bounds__(256) void varlen_attn_kernel(VarlenArgs a) {
 #pragma unroll
           for (int i = 0; i < DPL; ++i) oacc[rb][i] *= alpha[rb];
       }
+      // V^T operands straight from the row-major tile with the LDS's transposing read (ds_read_b64_tr_b16): lane s
+      // of a quarter-wave names the 8 bytes [key kb + s / 4][dims 16 i + 4 (s % 4) .. + 3] and receives
+      // [keys kb .. kb + 3][dim 16 i + s]; two reads (kb = 4 g and 16 + 4 g, the keys of the lane's k slots) make
+      // the A operand of output block i = dims 16 i .. 16 i + 15.
+      {
+        typedef short s4_t __attribute__((ext_vector_type(4)));
+        typedef __attribute__((address_space(3))) s4_t* lds_s4_ptr;
+        const uint8_t* v0 = buf + K_BYTES + (4 * g + (c >> 2)) * V_PITCH + 8 * (c & 3);
 #pragma unroll
-      for (int i = 0; i < DPL; ++i) {
-        u32x4 vt;
-        const uint32_t sel = (i & 1) ? kPermHighHalves : kPermLowHalves;
-        vt.x = perm(vrow[1].w[i >> 1], vrow[0].w[i >> 1], sel);
-        vt.y = perm(vrow[3].w[i >> 1], vrow[2].w[i >> 1], sel);
-        vt.z = perm(vrow[5].w[i >> 1], vrow[4].w[i >> 1], sel);
-        vt.w = perm(vrow[7].w[i >> 1], vrow[6].w[i >> 1], sel);
+        for (int i = 0; i < DPL; ++i) {
+          const u32x2 lo = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4_ptr)(v0 + 32 * i)));
+          const u32x2 hi = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4_ptr)(v0 + 16 * V_PITCH + 32 * i)));
+          const u32x4 vt = {lo.x, lo.y, hi.x, hi.y};
 #pragma unroll
-        for (int rb = 0; rb < RB; ++rb) oacc[rb][i] = mfma16<DT>(vt, pk[rb], oacc[rb][i]);
+          for (int rb = 0; rb < RB; ++rb) oacc[rb][i] = mfma16<DT>(vt, pk[rb], oacc[rb][i]);
+        }
       }
       __builtin_amdgcn_s_setprio(0);
     }
@@ -310,18 +288,13 @@ __global__ __launch_bounds__(256) void varlen_attn_kernel(VarlenArgs a) {
     if (q0[rb] + c >= q_len) continue;
     const int64_t tok = q_begin + q0[rb] + c;
     uint16_t* op = static_cast<uint16_t*>(a.out) + tok * a.out_st + (int64_t)head * a.out_sh;
+    // block i: the lane holds dims 16 i + 4 g .. + 3 of its row
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      uint32_t w[VR];
-#pragma unroll
-      for (int i = 0; i < VR; ++i) w[i] = pack2<DT>(oacc[rb][2 * i][r] * inv, oacc[rb][2 * i + 1][r] * inv);
-      uint16_t* dst = op + DPL * (4 * g + r);
-      if constexpr (VR == 2) {
-        *reinterpret_cast<u32x2*>(dst) = (u32x2){w[0], w[1]};
-      } else {
-#pragma unroll
-        for (int i = 0; i < VR / 4; ++i) reinterpret_cast<u32x4*>(dst)[i] = (u32x4){w[4 * i], w[4 * i + 1], w[4 * i + 2], w[4 * i + 3]};
-      }
+    for (int i = 0; i < DPL; ++i) {
+      u32x2 w;
+      w.x = pack2<DT>(oacc[rb][i][0] * inv, oacc[rb][i][1] * inv);
+      w.y = pack2<DT>(oacc[rb][i][2] * inv, oacc[rb][i][3] * inv);
+      *reinterpret_cast<u32x2*>(op + 16 * i + 4 * g) = w;
     }
     if (a.lse != nullptr && g == 0)
       a.lse[(int64_t)head * a.total_q + tok] = live ? (m[rb] - kShift) * kLn2 + __logf(l_tot) : -INFINITY;
