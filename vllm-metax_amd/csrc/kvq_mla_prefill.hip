@@ -125,53 +125,67 @@ __global__ __launch_bounds__(256) void varlen_attn_kernel(VarlenArgs a) {
     l[rb] = 0.f;
   }
 
-  // ---- cooperative tile copy: thread tid owns chunks tid + 256 i of the K tile and of the V tile
-  const uint16_t* kn_base = static_cast<const uint16_t*>(a.k_nope) + (int64_t)head * a.kn_sh;
-  const uint16_t* kpe_base = static_cast<const uint16_t*>(a.k_pe);
-  const uint16_t* v_base = static_cast<const uint16_t*>(a.v) + (int64_t)head * a.v_sh;
-  u32x4 kreg[KLD], vreg[VLD];
-  // per chunk, fixed for the whole run: its row in the tile, the tensor it comes from and the offset inside a row
-  int k_row[KLD], v_row[VLD];
-  const uint16_t* k_src[KLD];
-  int64_t k_stride[KLD];
-  const uint16_t* v_src[VLD];
+  // ---- cooperative tile copy.  Every load is "buffer resource + a lane offset that never changes": the resources
+  //      (scalar registers) are re-based on the tile's first key with scalar arithmetic, so the tile loop spends no
+  //      vector instruction on addresses (as 64-bit pointers per chunk they were 64 of the ~230 vector instructions
+  //      of a tile).  A resource ends with the sequence's last key: rows past it read as zeros and are masked.
+  //      Thread tid owns chunks tid + 256 i of the tile's k_nope part, of its k_pe part and of its V rows.
+  constexpr int KCR = KC - KCN;
+  constexpr int NLD = (32 * KCN + 255) / 256, RLD = (32 * KCR + 255) / 256;
+  static_assert(NLD + RLD >= KLD, "chunk loads");
+  const uint8_t* kn_base = reinterpret_cast<const uint8_t*>(static_cast<const uint16_t*>(a.k_nope) + (int64_t)head * a.kn_sh);
+  const uint8_t* kpe_base = reinterpret_cast<const uint8_t*>(a.k_pe);
+  const uint8_t* v_base = reinterpret_cast<const uint8_t*>(static_cast<const uint16_t*>(a.v) + (int64_t)head * a.v_sh);
+  const int64_t kn_row = a.kn_st * 2, kpe_row = a.kpe_st * 2, v_row_bytes = a.v_st * 2;   // bytes per key
+  u32x4 nreg[NLD], rreg[RLD > 0 ? RLD : 1], vreg[VLD];
+  uint32_t n_off[NLD], r_off[RLD > 0 ? RLD : 1], v_off[VLD];         // global: byte offset from the tile's first key
+  uint32_t n_lds[NLD], r_lds[RLD > 0 ? RLD : 1], v_lds[VLD];         // LDS: byte offset in the tile's buffer
+  auto swz = [](int row, int ch) { return KC % 8 == 0 ? (ch ^ (row & 7)) : (ch ^ ((row >> 1) & 3)); };
 #pragma unroll
-  for (int i = 0; i < KLD; ++i) {
-    const int q = min(tid + 256 * i, 32 * KC - 1);
-    k_row[i] = q / KC;
-    const int ch = q - k_row[i] * KC;
-    k_src[i] = ch < KCN ? kn_base + 8 * ch : kpe_base + 8 * (ch - KCN);
-    k_stride[i] = ch < KCN ? a.kn_st : a.kpe_st;
+  for (int i = 0; i < NLD; ++i) {
+    const int q = min(tid + 256 * i, 32 * KCN - 1), row = q / KCN, ch = q - row * KCN;
+    n_off[i] = (uint32_t)(row * (int)kn_row + 16 * ch);
+    n_lds[i] = (uint32_t)((row * KC + swz(row, ch)) * 16);
+  }
+#pragma unroll
+  for (int i = 0; i < RLD; ++i) {
+    const int q = min(tid + 256 * i, 32 * KCR - 1), row = q / KCR, ch = q - row * KCR;
+    r_off[i] = (uint32_t)(row * (int)kpe_row + 16 * ch);
+    r_lds[i] = (uint32_t)((row * KC + swz(row, KCN + ch)) * 16);
   }
 #pragma unroll
   for (int i = 0; i < VLD; ++i) {
-    const int q = min(tid + 256 * i, 32 * VC - 1);
-    v_row[i] = q / VC;
-    v_src[i] = v_base + 8 * (q - v_row[i] * VC);
+    const int q = min(tid + 256 * i, 32 * VC - 1), row = q / VC, ch = q - row * VC;
+    v_off[i] = (uint32_t)(row * (int)v_row_bytes + 16 * ch);
+    v_lds[i] = (uint32_t)(K_BYTES + row * V_PITCH + 16 * ch);
   }
-  auto fetch = [&](int t) __attribute__((always_inline)) {
-#pragma unroll
-    for (int i = 0; i < KLD; ++i)
-      kreg[i] = *reinterpret_cast<const u32x4*>(k_src[i] + (int64_t)(k_begin + min(t * 32 + k_row[i], k_len - 1)) * k_stride[i]);
-#pragma unroll
-    for (int i = 0; i < VLD; ++i)
-      vreg[i] = *reinterpret_cast<const u32x4*>(v_src[i] + (int64_t)(k_begin + min(t * 32 + v_row[i], k_len - 1)) * a.v_st);
+  auto tile_rsrc = [&](const uint8_t* base, int64_t row_bytes, int t) __attribute__((always_inline)) {
+    const int64_t left = (int64_t)(k_len - 32 * t) * row_bytes;     // bytes up to the end of the sequence's keys
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(base + (int64_t)(k_begin + 32 * t) * row_bytes), 0,
+                                             (int)(left < 0x7fffffff ? left : 0x7fffffff), 0x00020000);
   };
-  auto swz = [](int row, int ch) { return KC % 8 == 0 ? (ch ^ (row & 7)) : (ch ^ ((row >> 1) & 3)); };
+  auto fetch = [&](int t) __attribute__((always_inline)) {
+    const __amdgpu_buffer_rsrc_t rn = tile_rsrc(kn_base, kn_row, t), rv = tile_rsrc(v_base, v_row_bytes, t);
+#pragma unroll
+    for (int i = 0; i < NLD; ++i) nreg[i] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rn, n_off[i], 0, 0));
+    if constexpr (RLD > 0) {
+      const __amdgpu_buffer_rsrc_t rr = tile_rsrc(kpe_base, kpe_row, t);
+#pragma unroll
+      for (int i = 0; i < RLD; ++i) rreg[i] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rr, r_off[i], 0, 0));
+    }
+#pragma unroll
+    for (int i = 0; i < VLD; ++i) vreg[i] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rv, v_off[i], 0, 0));
+  };
   auto drop = [&](uint8_t* buf) __attribute__((always_inline)) {
 #pragma unroll
-    for (int i = 0; i < KLD; ++i) {
-      const int q = tid + 256 * i;
-      if (q < 32 * KC) {
-        const int row = q / KC, ch = q - row * KC;
-        *reinterpret_cast<u32x4*>(buf + (row * KC + swz(row, ch)) * 16) = kreg[i];
-      }
-    }
+    for (int i = 0; i < NLD; ++i)
+      if (tid + 256 * i < 32 * KCN) *reinterpret_cast<u32x4*>(buf + n_lds[i]) = nreg[i];
 #pragma unroll
-    for (int i = 0; i < VLD; ++i) {
-      const int q = tid + 256 * i;
-      if (q < 32 * VC) *reinterpret_cast<u32x4*>(buf + K_BYTES + (q / VC) * V_PITCH + (q % VC) * 16) = vreg[i];
-    }
+    for (int i = 0; i < RLD; ++i)
+      if (tid + 256 * i < 32 * KCR) *reinterpret_cast<u32x4*>(buf + r_lds[i]) = rreg[i];
+#pragma unroll
+    for (int i = 0; i < VLD; ++i)
+      if (tid + 256 * i < 32 * VC) *reinterpret_cast<u32x4*>(buf + v_lds[i]) = vreg[i];
   };
 
   if (num_tiles > 0) {
@@ -332,6 +346,9 @@ extern "C" int kvq_mla_prefill_attn(const void* q, int dtype, int64_t q_stride_t
   const int64_t strides[] = {q_stride_tok, q_stride_head, kn_stride_tok, kn_stride_head, kpe_stride_tok,
                              v_stride_tok, v_stride_head, out_stride_tok, out_stride_head};
   for (int64_t st : strides) KVQ_REQUIRE(st >= 0 && st % 8 == 0, "%s: strides must be multiples of 8 elements (got %lld)", op, (long long)st);
+  // a tile's 32 rows are addressed with 32-bit offsets from its first key
+  KVQ_REQUIRE(kn_stride_tok < (1 << 24) && kpe_stride_tok < (1 << 24) && v_stride_tok < (1 << 24),
+              "%s: token strides must be below 2^24 elements", op);
   KVQ_REQUIRE(((uintptr_t)q | (uintptr_t)k_nope | (uintptr_t)k_pe | (uintptr_t)v | (uintptr_t)out) % 16 == 0,
               "%s: tensors must be 16-byte aligned", op);
   VarlenArgs a{};
