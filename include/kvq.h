@@ -564,7 +564,8 @@ KVQ_API int kvq_mla_decode_absorb_int8(void* out, int out_dtype, float* lse, con
  * padding to the qk head size, flash_attn.py:138-143).
  * q [T, H, nope_dim + rope_dim]; out [T, H, v_dim]; lse [H, total_q] fp32 natural
  * log, may be NULL.  All of `dtype` KVQ_BF16 or KVQ_F16, strides in elements and
- * multiples of 8, pointers 16-byte aligned.  cu_seqlens_q / cu_seqlens_k
+ * multiples of 8 (the token strides of k_nope, k_pe and v below 2^24), pointers
+ * 16-byte aligned, `scale` positive and finite.  cu_seqlens_q / cu_seqlens_k
  * [num_seqs + 1] int32 on the device; a sequence longer than max_seqlen_q is
  * only attended for its first max_seqlen_q rows.  With `causal`, key j of a
  * sequence is visible to its query row i iff j <= i + (k_len - q_len).  A row
