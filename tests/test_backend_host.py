@@ -323,3 +323,22 @@ def test_c_abi_rejects_bad_arguments_of_the_newer_entry_points_without_a_gpu():
     rc = lib.kvq_paged_attn_int8(one, _C.KVQ_BF16, 4096, 128, one, _C.KVQ_BF16, 4096, 128, one, ctypes.byref(g), one, 8,
                                  one, null, 2, 32, 1, 0.1, 9, 0, 0.0, null, null, null, one, 1 << 20, null)
     assert rc == -22 and b"flag" in lib.kvq_last_error()
+
+
+def test_mla_prefill_entry_checks_scale_and_strides_without_a_gpu():
+    """The kernel takes row maxima before scaling and addresses a tile's rows with 32-bit offsets: a scale that is
+    not positive and a token stride of 2^24 elements or more are refused before anything is launched."""
+    import ctypes
+
+    lib = _C.load()
+    p = ctypes.c_void_p(256)    # any non-NULL, 16-byte aligned address: nothing is dereferenced on the host
+    null = ctypes.c_void_p(0)
+
+    def call(scale=0.1, kn_stride=128 * 128, v_stride=128 * 128):
+        return lib.kvq_mla_prefill_attn(p, _C.KVQ_BF16, 128 * 192, 192, p, kn_stride, 128, p, 64, p, v_stride, 128, p, p,
+                                        1, 64, 64, 128, 128, 64, 128, scale, 1, p, 128 * 128, 128, null, null)
+
+    for bad in (0.0, -0.1, float("inf"), float("nan")):
+        assert call(scale=bad) == -22 and b"scale" in lib.kvq_last_error()
+    assert call(kn_stride=1 << 24) == -22 and b"stride" in lib.kvq_last_error()
+    assert call(v_stride=1 << 24) == -22 and b"stride" in lib.kvq_last_error()
