@@ -125,6 +125,9 @@ def make_batch(workload: str, seed: int = 0):
         dctx = torch.randint(512, 4097, (60,), generator=g).tolist()
         return dict(mixed=True, hq=28, hkv=4, d=128, bs=16, ctx=[2048, 4096, 6144, 8192] + dctx,
                     qlens=[2048] * 4 + [1] * 60, pool=12000)
+    if workload == "llama3_8b_spec_decode_b64_q4_ctx1k-8k":   # configs[1]'s batch in a speculative-decoding step: 1 + 3 query tokens per sequence
+        ctx = torch.randint(1024, 8193, (64,), generator=g).tolist()
+        return dict(mixed=True, spec=True, hq=32, hkv=8, d=128, bs=16, ctx=ctx, qlens=[4] * 64, pool=40000)
     if workload == "mla_decode_b32_h128_ctx4096":        # configs[3]: DeepSeek-V2 MLA decode
         return dict(mla=True, heads=128, r=512, p=64, bs=64, ctx=[4096] * 32, pool=32 * 64 + 8)
     if workload == "mla_prefill_h128":                   # the MLA layer's prefill attention calls, DeepSeek-V2 shapes
@@ -623,6 +626,27 @@ def mixed_main(args, cfg, dev, ops):
     traffic, traffic_source = measured_traffic(args.workload)
     if args.sliding_window or args.soft_cap or cfg.get("kv_dtype") != "int8" or args.kv_layout != "HND":
         traffic, traffic_source = None, None
+    if cfg.get("spec"):
+        # a memory-bound step: every record of every context is read once, as in a decode step
+        res = {
+            "metric": f"{cfg.get('kv_dtype', 'int8')}-KV speculative-decoding step ({B} sequences x {qls[0]} query tokens): achieved HBM GB/s",
+            "value": round(pre_bytes / attn_s / 1e9, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
+            "warmup": args.warmup, "ms_per_step": round(dt * 1e3, 5), "higher_is_better": True, "scaling": "weak",
+            "vs_baseline": None,
+            "dtype": f"{cfg.get('kv_dtype', 'int8')} KV codes, fp16 MFMA operands, fp32 softmax/accumulate, bf16 Q/out",
+            "data": "synthetic",
+            "config": {"workload": args.workload, "batch": B, "new_tokens": n_tok, "sum_ctx": sum(ctx), "q_heads": hq,
+                       "kv_heads": hkv, "head_dim": d, "block_size": bs, "layer_caches_rotated": Lr,
+                       "kv_layout": args.kv_layout},
+            "prewarm_s": PREWARM_S, "attn_launch_us": round(attn_s * 1e6, 1),
+            "roofline": {"bound": "hbm", "achieved": round(pre_bytes / attn_s / 1e9, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                         "frac": round(pre_bytes / attn_s / 1e9 / HBM_PEAK_GBPS, 4), "traffic": None,
+                         "timing": f"{n_ev} attention launches back to back between two events on the launch stream",
+                         "kernel": "varlen attention launch = prefill_plan_kernel + paged_prefill_kernel (an item's tiles spread over a workgroup's waves)",
+                         "algorithmic_bytes_per_launch": pre_bytes},
+        }
+        print(json.dumps(res))
+        return
     res = {
         "metric": f"{cfg.get('kv_dtype', 'int8')}-KV mixed batch (4 x 2048-token prefill chunks + 60 decode rows): ms per layer",
         "value": round((dec_bytes + pre_bytes + write_bytes) / dt / 1e9, 1), "unit": "GB/s", "n_gpus": 1,

@@ -256,3 +256,53 @@ def test_non_causal_rows_see_every_key(gpu_device, hq, hkv, d, layout):
     torch.testing.assert_close(lse.cpu(), want_lse, atol=5e-3, rtol=1e-3)
     tail = got[int(cu[-2]):].cpu()
     assert torch.equal(tail.view(torch.int16), tail[:1].expand_as(tail).contiguous().view(torch.int16))
+
+
+@pytest.mark.parametrize("hq,hkv,d,layout,qmax", [(32, 8, 128, "HND", 4), (32, 8, 128, "NHD", 8), (28, 4, 128, "HND", 2),
+                                                  (8, 8, 64, "HND", 16), (16, 2, 256, "NHD", 2), (16, 1, 128, "HND", 1)])
+def test_short_runs_on_long_contexts_spread_over_a_workgroup(gpu_device, hq, hkv, d, layout, qmax):
+    """A speculative-decoding step: every sequence brings a few query tokens (1 + k) on a long context.  With few
+    items per launch the short-run kernel spreads an item's tiles over the waves of a workgroup and folds their
+    states; contexts shorter than the waves' stride (waves without a tile), one-token sequences next to them (the
+    decode kernel's) and a sliding window are in the batch.  Output and lse against the oracle."""
+    ctx = [9000, 37, 2500, 300, 64, 5000, 1, 700]
+    qls = [min(c, q) for c, q in zip(ctx, [qmax, 2, qmax, 1, 3, qmax, 1, 2])]
+    kv, lay, bt, q, sl, cu = build(ctx, qls, hq, hkv, d, 16, layout=layout, seed=hq + qmax)
+    scale = 1 / math.sqrt(d)
+    for window in (0, 1000):
+        want, want_lse = oracle.paged_attn(q, T.storage_bytes(kv), lay, bt, sl, cu, scale, return_lse=True,
+                                           sliding_window=window)
+        dev = gpu_device
+        kvd = T.to_device_cache(kv, dev, layout)
+        k, v = L.key_value_views(kvd)
+        ks, vs = L.scale_views(kvd)
+        out = torch.full(q.shape, float("nan"), dtype=q.dtype, device=dev)
+        lse = torch.full(q.shape[:2], float("nan"), dtype=torch.float32, device=dev)
+        ops.unified_attention(q.to(dev), k, v, out, cu.to(dev), max(qls), sl.to(dev), int(sl.max()), scale, True,
+                              window_size=(window - 1, 0) if window else (-1, -1), block_table=bt.to(dev),
+                              k_scale_cache=ks, v_scale_cache=vs, lse=lse)
+        torch.cuda.synchronize()
+        T.assert_close_attn(out, want, what=f"short runs {hq}/{hkv} d{d} q<={qmax} window {window}")
+        torch.testing.assert_close(lse.cpu(), want_lse, atol=5e-3, rtol=1e-3)
+
+
+def test_many_short_runs_take_one_wave_per_item(gpu_device):
+    """Beyond a few thousand items per launch an item stays with one wave (300 sequences x 8 kv heads here): the
+    same rows as the oracle's, also when the batch is cut in three launches that spread their items over
+    workgroups."""
+    hq, hkv, d = 32, 8, 128
+    g = torch.Generator().manual_seed(17)
+    n = 300
+    ctx = torch.randint(20, 400, (n,), generator=g).tolist()
+    qls = [min(c, int(x)) for c, x in zip(ctx, torch.randint(1, 5, (n,), generator=g).tolist())]
+    kv, lay, bt, q, sl, cu = build(ctx, qls, hq, hkv, d, 16, layout="HND", seed=3)
+    scale = 1 / math.sqrt(d)
+    want = oracle.paged_attn(q, T.storage_bytes(kv), lay, bt, sl, cu, scale)
+    got = run(gpu_device, kv, "HND", bt, q, sl, cu, max(qls), scale)
+    T.assert_close_attn(got, want, what="300 short runs, one wave per item")
+    parts = []
+    for lo_, hi_ in ((0, 100), (100, 200), (200, 300)):
+        qq = q[int(cu[lo_]):int(cu[hi_])]
+        cc = (cu[lo_:hi_ + 1] - cu[lo_]).contiguous()
+        parts.append(run(gpu_device, kv, "HND", bt[lo_:hi_].contiguous(), qq, sl[lo_:hi_].contiguous(), cc, max(qls), scale))
+    T.assert_close_attn(torch.cat(parts), want, what="the same runs in three launches")

@@ -230,6 +230,29 @@ struct PrefillTile {
     }
   }
 
+  // ---- several waves on one item: their states meet in LDS, one column tile at a time.  A wave drops the tile's
+  //      state into its own window (free once its tiles are done); the item's first wave folds them into its own.
+  //      A column may have seen nothing in a wave's tiles (m = -inf): its weight is then 0, never 2^(-inf + inf).
+  __device__ static void dump_state(const State& st, int nt, int lane, uint8_t* lds) {
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) *reinterpret_cast<floatx4*>(lds + (dt * 64 + lane) * 16) = st.o[nt][dt];
+    *reinterpret_cast<floatx4*>(lds + (DT * 64 + lane) * 16) = (floatx4){st.psum[nt][0], st.m[nt], st.l[nt], 0.f};
+  }
+  __device__ static void fold_state(State& st, int nt, int lane, const uint8_t* lds) {
+    const floatx4 x = *reinterpret_cast<const floatx4*>(lds + (DT * 64 + lane) * 16);
+    const float mj = x.y;
+    const float m_new = fmaxf(st.m[nt], mj);
+    const float m_ref = m_new == -INFINITY ? 0.f : m_new;
+    const float a = __builtin_amdgcn_exp2f(st.m[nt] - m_ref);
+    const float b = __builtin_amdgcn_exp2f(mj - m_ref);
+    st.m[nt] = m_new;
+    st.l[nt] = st.l[nt] * a + x.z * b;
+    st.psum[nt] = st.psum[nt] * a + x.x * b;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+      st.o[nt][dt] = st.o[nt][dt] * a + *reinterpret_cast<const floatx4*>(lds + (dt * 64 + lane) * 16) * b;
+  }
+
   // Normalise column tile `nt` and write the lane's quarter of its output row.
   __device__ static void emit(const AttnIO& io, int nt, int64_t row, int head, bool valid, int lane, const State& st) {
     float l = st.l[nt];
@@ -275,7 +298,12 @@ struct PrefillTile {
 
 // grid (query blocks of the longest run, sequences, ceil(Hkv / WPW)); wave w of a workgroup owns
 // kv head (head group) * WPW + w.  Sequences with a one-token run belong to the decode kernel.
-template <int D, int QDT, int ODT, int NT, int WPW, int CODE = KVQ_CODE_INT8>
+// SPLIT: grid z = Hkv and ALL waves of the workgroup serve one kv head, taking the
+// item's tiles in turn (wave w: tiles t_start + w, + WPW, ...); their states are folded in LDS at the end.  For
+// launches with few items and long contexts -- a handful of query tokens per sequence, as a speculative-decoding
+// step has them: one wave per item leaves most of the chip's waves idle (measured on MI355X, 64 sequences of
+// 1k-8k tokens with 2 or 4 query tokens each: 280 us per call that way against 118 us for one query token).
+template <int D, int QDT, int ODT, int NT, int WPW, int CODE = KVQ_CODE_INT8, bool SPLIT = false>
 __global__ __launch_bounds__(WPW * 64) void paged_prefill_kernel(PrefillArgs a) {
   using PT = PrefillTile<D, QDT, ODT, NT, CODE>;
   using DTile = typename PT::DTile;
@@ -290,7 +318,8 @@ __global__ __launch_bounds__(WPW * 64) void paged_prefill_kernel(PrefillArgs a) 
   if (lin >= per_seq * (unsigned)a.plan[0]) return;   // uniform over the workgroup
   const unsigned rem = lin % per_seq, qbi = rem / hz;
   const int seq = a.plan[1 + lin / per_seq];
-  const int hkv = (int)((rem % hz + qbi) % hz) * WPW + wave;
+  const int hkv = SPLIT ? (int)((rem % hz + qbi) % hz) : (int)((rem % hz + qbi) % hz) * WPW + wave;
+  constexpr int STEP = SPLIT ? WPW : 1;          // tiles between two of this wave's
   const AttnIO& io = a.io;
   if (hkv >= io.g.num_kv_heads) return;
   const int q_begin = a.cu_seqlens_q[seq];
@@ -340,7 +369,7 @@ __global__ __launch_bounds__(WPW * 64) void paged_prefill_kernel(PrefillArgs a) 
       z.psum[nt] = (floatx4){0.f, 0.f, 0.f, 0.f};
       z.m[nt] = -INFINITY;
       z.l[nt] = 0.f;
-      PT::emit(io, nt, row[nt], head[nt], valid[nt], lane, z);
+      if (!SPLIT || wave == 0) PT::emit(io, nt, row[nt], head[nt], valid[nt], lane, z);
     }
     return;
   }
@@ -348,11 +377,13 @@ __global__ __launch_bounds__(WPW * 64) void paged_prefill_kernel(PrefillArgs a) 
   const LaneOffsets lo = DTile::lane_offsets(io.g, lane);
   const int32_t* bt_row = io.block_table + (int64_t)seq * io.bt_stride;
   typename DTile::Tile kv;
-  int t = t_start;
+  int t = t_start + (SPLIT ? wave : 0);
+  const bool has_tiles = t < t_end;              // without the split: always
+  // (a wave without a tile still loads one -- the block table is read clamped into the sequence -- and uses nothing)
   TileBlocks nb = DTile::fetch_blocks(io, bt_row, len, t);
   DTile::load_tile(io, DTile::window(io, nb, t, hkv), lo, kv);
   DTile::phase_fence();
-  nb = DTile::fetch_blocks(io, bt_row, len, t + 1);
+  nb = DTile::fetch_blocks(io, bt_row, len, t + STEP);
 
   half8_t qb[NT][PT::KSTEPS];
   float s_init[NT], ali[NT];
@@ -373,24 +404,41 @@ __global__ __launch_bounds__(WPW * 64) void paged_prefill_kernel(PrefillArgs a) 
     st.l[nt] = 0.f;
   }
   half8_t p_op[NT];
-  while (t + 1 < t_end) {
-    const typename DTile::Window w = DTile::window(io, nb, t + 1, hkv);
+  if (has_tiles) {
+    while (t + STEP < t_end) {
+      const typename DTile::Window w = DTile::window(io, nb, t + STEP, hkv);
+      DTile::stage(kv, lo, sc_mul, lane, lds);
+      DTile::phase_fence();
+      DTile::load_tile(io, w, lo, kv);
+      DTile::phase_fence();
+      nb = DTile::fetch_blocks(io, bt_row, len, t + 2 * STEP);
+      if ((t + 1) * kTile <= min_limit && t * kTile >= max_first)
+        PT::template qk_softmax<false>(io, lo, qb, s_init, limit, wspan, t, lane, lds, st, p_op, ali);
+      else
+        PT::template qk_softmax<true>(io, lo, qb, s_init, limit, wspan, t, lane, lds, st, p_op, ali);
+      PT::pv(lo, p_op, lds, st);
+      DTile::phase_fence();
+      t += STEP;
+    }
     DTile::stage(kv, lo, sc_mul, lane, lds);
-    DTile::phase_fence();
-    DTile::load_tile(io, w, lo, kv);
-    DTile::phase_fence();
-    nb = DTile::fetch_blocks(io, bt_row, len, t + 2);
-    if ((t + 1) * kTile <= min_limit && t * kTile >= max_first)
-      PT::template qk_softmax<false>(io, lo, qb, s_init, limit, wspan, t, lane, lds, st, p_op, ali);
-    else
-      PT::template qk_softmax<true>(io, lo, qb, s_init, limit, wspan, t, lane, lds, st, p_op, ali);
+    PT::template qk_softmax<true>(io, lo, qb, s_init, limit, wspan, t, lane, lds, st, p_op, ali);
     PT::pv(lo, p_op, lds, st);
-    DTile::phase_fence();
-    ++t;
   }
-  DTile::stage(kv, lo, sc_mul, lane, lds);
-  PT::template qk_softmax<true>(io, lo, qb, s_init, limit, wspan, t, lane, lds, st, p_op, ali);
-  PT::pv(lo, p_op, lds, st);
+  if constexpr (SPLIT) {
+    // every wave of the workgroup arrives here (the returns above are uniform over it)
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+      if (nt > 0) lds_barrier();   // the windows are read no more: they take the next column tile's states
+      if (wave != 0 && has_tiles) PT::dump_state(st, nt, lane, lds);
+      lds_barrier();
+      if (wave == 0) {
+#pragma unroll
+        for (int j = 1; j < WPW; ++j)
+          if (t_start + j < t_end) PT::fold_state(st, nt, lane, lds_all[j]);   // wave j owned a tile
+      }
+    }
+    if (wave != 0) return;
+  }
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt) PT::emit(io, nt, row[nt], head[nt], valid[nt], lane, st);
 }
@@ -928,10 +976,21 @@ static int launch_prefill_flash32(PrefillArgs& a, int max_query_len, hipStream_t
   return check_hip(hipGetLastError(), "paged_prefill_flash32 launch");
 }
 
+// Launches with this many items (query block x sequence x kv head) or fewer spread each item over a workgroup's waves.
+constexpr int64_t kSplitItems = 2048;
+
 template <int D, int QDT, int ODT, int NT, int WPW, int CODE = KVQ_CODE_INT8>
 static int launch_prefill_cfg(const PrefillArgs& a, int max_query_len, hipStream_t s) {
   const int blocks = (max_query_len + a.q_tokens - 1) / a.q_tokens;
   if (blocks > 0x7fffffff / 2 || a.num_seqs > 65535) return fail(KVQ_EINVAL, "paged_attn_int8: prefill grid out of range");
+  if ((int64_t)blocks * a.num_seqs * a.io.g.num_kv_heads <= kSplitItems && a.io.g.num_kv_heads <= 65535) {
+    // waves per item: eight with one column tile per wave; four with two (their accumulators need the registers
+    // of a 256-thread workgroup)
+    constexpr int SW = NT == 1 ? 8 : 4;
+    dim3 grid(blocks, a.num_seqs, a.io.g.num_kv_heads);
+    hipLaunchKernelGGL((paged_prefill_kernel<D, QDT, ODT, NT, SW, CODE, true>), grid, dim3(SW * 64), 0, s, a);
+    return check_hip(hipGetLastError(), "paged_prefill launch");
+  }
   dim3 grid(blocks, a.num_seqs, (a.io.g.num_kv_heads + WPW - 1) / WPW);
   hipLaunchKernelGGL((paged_prefill_kernel<D, QDT, ODT, NT, WPW, CODE>), grid, dim3(WPW * 64), 0, s, a);
   return check_hip(hipGetLastError(), "paged_prefill launch");
