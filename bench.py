@@ -125,6 +125,8 @@ def make_batch(workload: str, seed: int = 0):
         dctx = torch.randint(512, 4097, (60,), generator=g).tolist()
         return dict(mixed=True, hq=28, hkv=4, d=128, bs=16, ctx=[2048, 4096, 6144, 8192] + dctx,
                     qlens=[2048] * 4 + [1] * 60, pool=12000)
+    if workload == "llama3_8b_chunk512_ctx32k":          # one request's 512-token prefill chunk on 32k cached tokens
+        return dict(mixed=True, chunk=True, hq=32, hkv=8, d=128, bs=16, ctx=[32768 + 512], qlens=[512], pool=2200)
     if workload == "llama3_8b_spec_decode_b64_q4_ctx1k-8k":   # configs[1]'s batch in a speculative-decoding step: 1 + 3 query tokens per sequence
         ctx = torch.randint(1024, 8193, (64,), generator=g).tolist()
         return dict(mixed=True, spec=True, hq=32, hkv=8, d=128, bs=16, ctx=ctx, qlens=[4] * 64, pool=40000)
@@ -594,7 +596,12 @@ def mixed_main(args, cfg, dev, ops):
     ws = torch.empty(ops.paged_attn_workspace_bytes(B, hq, d), dtype=torch.uint8, device=dev)
     scale = 1.0 / math.sqrt(d)
 
-    def step(layer, write=True, attn=True):
+    # context splits of the long runs, as the metadata builder proposes them from the run lengths
+    splits = ops.prefill_context_splits(qls, max(ctx), hq, hkv) if cfg.get("chunk") else 1
+    if splits > 1:
+        ws = torch.empty(ops.split_prefill_workspace_bytes(B, hq, d, n_tok, splits), dtype=torch.uint8, device=dev)
+
+    def step(layer, write=True, attn=True, splits=splits):
         c = caches[layer]
         if write:
             ops.reshape_and_cache_flash_per_token_head_quant(new_k, new_v, c["k"], c["v"], c["ks"], c["vs"], new_slots,
@@ -602,7 +609,7 @@ def mixed_main(args, cfg, dev, ops):
         if attn:
             ops.unified_attention(q, c["k"], c["v"], out, cu_d, max(qls), sl_d, max(ctx), scale, True, block_table=bt_d,
                                   k_scale_cache=c["ks"], v_scale_cache=c["vs"], workspace=ws, geometry=c["geom"],
-                                  kv_quant_mode=mode,
+                                  kv_quant_mode=mode, prefill_splits=splits,
                                   **_window_kwargs(dict(window=args.sliding_window, softcap=args.soft_cap)))
 
     Lr = args.layers
@@ -626,6 +633,28 @@ def mixed_main(args, cfg, dev, ops):
     traffic, traffic_source = measured_traffic(args.workload)
     if args.sliding_window or args.soft_cap or cfg.get("kv_dtype") != "int8" or args.kv_layout != "HND":
         traffic, traffic_source = None, None
+    if cfg.get("chunk"):
+        unsplit_s = time_back_to_back(lambda i: step(i % Lr, write=False, attn=True, splits=1), min(n_ev, 20))
+        res = {
+            "metric": f"{cfg.get('kv_dtype', 'int8')}-KV prefill chunk of one request ({qls[0]} tokens on {ctx[0] - qls[0]} cached): TFLOP/s of the attention launch",
+            "value": round(flops / attn_s / 1e12, 1), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
+            "warmup": args.warmup, "ms_per_step": round(dt * 1e3, 5), "higher_is_better": True, "scaling": "weak",
+            "vs_baseline": None,
+            "dtype": f"{cfg.get('kv_dtype', 'int8')} KV codes, fp16 MFMA operands, fp32 softmax/accumulate, bf16 Q/out",
+            "data": "synthetic",
+            "config": {"workload": args.workload, "batch": B, "new_tokens": n_tok, "sum_ctx": sum(ctx), "q_heads": hq,
+                       "kv_heads": hkv, "head_dim": d, "block_size": bs, "layer_caches_rotated": Lr,
+                       "kv_layout": args.kv_layout, "context_splits": splits},
+            "prewarm_s": PREWARM_S, "attn_launch_us": round(attn_s * 1e6, 1),
+            "attn_launch_us_without_context_splits": round(unsplit_s * 1e6, 1),
+            "roofline": {"bound": "mfma", "achieved": round(flops / attn_s / 1e12, 1), "peak": MFMA_F16_PEAK_TFLOPS,
+                         "unit": "TFLOP/s", "frac": round(flops / attn_s / 1e12 / MFMA_F16_PEAK_TFLOPS, 4), "traffic": None,
+                         "timing": f"{n_ev} attention launches back to back between two events on the launch stream",
+                         "kernel": "varlen attention launch = prefill_plan_kernel + paged_prefill_flash32_kernel (context splits) + prefill_split_merge_kernel",
+                         "algorithmic_flops_per_launch": flops},
+        }
+        print(json.dumps(res))
+        return
     if cfg.get("spec"):
         # a memory-bound step: every record of every context is read once, as in a decode step
         res = {

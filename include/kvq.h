@@ -27,7 +27,7 @@
 extern "C" {
 #endif
 
-#define KVQ_ABI_VERSION 17
+#define KVQ_ABI_VERSION 18
 
 #define KVQ_OK 0
 #define KVQ_EINVAL (-22)
@@ -225,6 +225,32 @@ KVQ_API int kvq_paged_attn_int8(void* out, int out_dtype, int64_t out_stride_t, 
                         const int32_t* cu_seqlens_q, int num_seqs, int num_q_heads,
                         int max_query_len, float scale, int causal, int window_size,
                         float softcap, const float* sinks, const float* alibi_slopes, float* lse, void* workspace, size_t workspace_bytes,
+                        kvq_stream_t stream);
+
+/*
+ * kvq_paged_attn_int8 with the long runs' CONTEXT cut into `prefill_splits` ranges (1..8; 1 = the plain call).
+ * It has no counterpart in the reference's call (its Triton kernel chooses its own decomposition): the caller's
+ * metadata builder knows what a launch holds.  For a launch whose long query runs make few workgroups on a long
+ * context -- one request's small prefill chunk: 512 tokens on 32k cached ones are 128 workgroups that each walk
+ * the whole context, 1.2 ms whatever the chunk size -- every (query block, kv head) item becomes `prefill_splits`
+ * workgroups that each take a range of the context's tiles and leave a partial state per (query row, q head); a
+ * merge kernel combines them with the log-sum-exp algebra of merge_attn_states (sinks and lse as in the plain
+ * call).  Only the workgroup-shared tile takes part (head sizes up to 128, max_query_len x group >= 64); one-token
+ * sequences, short runs and head size 256 are served as in the plain call.  Same results within the tolerance of
+ * the plain call (the order of the additions differs).  num_tokens = the rows of q; the workspace must hold
+ * kvq_paged_attn_split_prefill_workspace_bytes(num_seqs, num_q_heads, head_size, num_tokens, prefill_splits)
+ * bytes (the plain workspace + num_tokens x num_q_heads x prefill_splits x (head_size + 2) floats).
+ */
+KVQ_API size_t kvq_paged_attn_split_prefill_workspace_bytes(int max_num_seqs, int num_q_heads, int head_size,
+                                                            int num_tokens, int prefill_splits);
+KVQ_API int kvq_paged_attn_int8_split_prefill(void* out, int out_dtype, int64_t out_stride_t, int64_t out_stride_h,
+                        const void* q, int q_dtype, int64_t q_stride_t, int64_t q_stride_h,
+                        const void* cache, const kvq_cache_geom* geom,
+                        const int32_t* block_table, int64_t bt_stride, const int32_t* seq_lens,
+                        const int32_t* cu_seqlens_q, int num_seqs, int num_q_heads,
+                        int max_query_len, float scale, int causal, int window_size,
+                        float softcap, const float* sinks, const float* alibi_slopes, float* lse,
+                        int num_tokens, int prefill_splits, void* workspace, size_t workspace_bytes,
                         kvq_stream_t stream);
 
 /*

@@ -342,3 +342,19 @@ def test_mla_prefill_entry_checks_scale_and_strides_without_a_gpu():
         assert call(scale=bad) == -22 and b"scale" in lib.kvq_last_error()
     assert call(kn_stride=1 << 24) == -22 and b"stride" in lib.kvq_last_error()
     assert call(v_stride=1 << 24) == -22 and b"stride" in lib.kvq_last_error()
+
+
+def test_context_split_proposal_follows_the_launch_shape():
+    """prefill_context_splits: what a metadata builder asks for from the host copy of the query lengths."""
+    from vllm_metax_amd._custom_ops import prefill_context_splits as f
+    # one request's small chunk on a long context: 512 tokens x 8 kv heads = 128 workgroups on 256 CUs
+    assert f([512], 32768, 32, 8) == 4
+    assert f([512] + [1] * 60, 32768, 32, 8) == 4          # decode rows do not count
+    assert f([256], 32768, 32, 8) == 8
+    assert f([2048], 32768, 32, 8) == 1                    # fills the chip as it is
+    assert f([512], 2048, 32, 8) == 1                      # a short context is walked quickly anyway
+    assert f([1] * 64, 32768, 32, 8) == 1                  # decode only
+    assert f([4] * 64, 32768, 32, 8) == 1                  # short runs: the other kernel
+    assert f([2048], 131072, 32, 8, max_split_tokens=4096) == 1
+    assert f([1024], 131072, 32, 8, max_split_tokens=4096) == 2    # 256 workgroups: two ranges fill the chip's 512 places
+    assert f(torch.tensor([300, 1, 1]), 8192, 28, 4) == 4          # the context allows one split per 2048 tokens

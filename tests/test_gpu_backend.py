@@ -10,6 +10,7 @@ import torch
 
 import kvq_testlib as T
 import oracle
+from vllm_metax_amd import _custom_ops as ops
 from vllm_metax_amd import layout as L
 from vllm_metax_amd.v1.attention.backends.int8_attn import Int8AttentionBackend, Int8FusedUpdateAttentionBackend
 
@@ -111,3 +112,48 @@ def test_impl_keeps_the_scales_of_a_cache_it_comes_back_to(gpu_device):
     want = oracle.paged_attn(q.view(B, hq, d), T.storage_bytes(kv_cpu), lay, bt, torch.tensor(ctx, dtype=torch.int32),
                              torch.arange(B + 1, dtype=torch.int32), 0.09)
     T.assert_close_attn(out.view(B, hq, d), want, what="attend on A after touching B")
+
+
+def test_small_chunk_on_a_long_context_goes_through_context_splits(gpu_device):
+    """A step with one request's 160-token prefill chunk on 9000 cached tokens and two decode rows: the builder
+    proposes context splits from the host copy of query_start_loc, reserves their room in its workspace, and the
+    layer's forward gives the oracle's rows."""
+    dev = gpu_device
+    hq, hkv, d, bs, nb = 32, 8, 128, 16, 700
+    ctx = [9160, 300, 41]
+    qls = [160, 1, 1]
+    B = len(ctx)
+    g = torch.Generator().manual_seed(11)
+    kv_cache = L.allocate_kv_cache(nb, bs, hkv, d, device=dev)
+    layout = "HND" if Int8AttentionBackend.get_kv_cache_stride_order() != (0, 1, 2, 3) else "NHD"
+    kv_cpu, views, lay = T.cpu_cache(nb, bs, hkv, d, layout)
+    views[2].fill_(1.0)
+    views[3].fill_(1.0)
+    bt = T.make_block_tables(ctx, bs, nb, g)
+    impl = Int8AttentionBackend.get_impl_cls()(hq, d, 1 / math.sqrt(d), hkv, kv_cache_dtype="int8_per_token_head")
+    spec = types.SimpleNamespace(block_size=bs, num_kv_heads=hkv, head_size=d, num_q_heads=hq)
+    cfg = types.SimpleNamespace(scheduler_config=types.SimpleNamespace(max_num_seqs=16))
+    builder = Int8AttentionBackend.get_builder_cls()(spec, ["layer.0"], cfg, dev)
+    layer = types.SimpleNamespace()
+    slots = T.slots_for(bt, ctx, bs)
+    for i, c in enumerate(ctx):
+        k = torch.randn((c, hkv, d), generator=g).to(torch.bfloat16)
+        v = torch.randn((c, hkv, d), generator=g).to(torch.bfloat16)
+        impl.do_kv_cache_update(layer, k.to(dev), v.to(dev), kv_cache, slots[i].to(dev))
+        oracle.cache_write(k, v, T.storage_bytes(kv_cpu), lay, slots[i])
+    n = sum(qls)
+    cu = torch.tensor([0] + torch.tensor(qls).cumsum(0).tolist(), dtype=torch.int32)
+    common = types.SimpleNamespace(
+        num_reqs=B, num_actual_tokens=n, max_query_len=max(qls), max_seq_len=max(ctx), query_start_loc=cu.to(dev),
+        query_start_loc_cpu=cu, seq_lens=torch.tensor(ctx, dtype=torch.int32, device=dev),
+        block_table_tensor=bt.to(dev), slot_mapping=torch.zeros(n, dtype=torch.int64, device=dev), causal=True)
+    md = builder.build(0, common)
+    assert md.prefill_splits == 4 and md.has_decode_rows          # 5 query blocks x 8 kv heads; 9160 // 2048 = 4
+    assert md.workspace.numel() >= ops.split_prefill_workspace_bytes(16, hq, d, n, md.prefill_splits)
+    q = torch.randn((n, hq * d), generator=g).to(torch.bfloat16)
+    out = torch.zeros((n, hq * d), dtype=torch.bfloat16, device=dev)
+    impl.forward(layer, q.to(dev), None, None, kv_cache, md, out)
+    torch.cuda.synchronize()
+    want = oracle.paged_attn(q.view(n, hq, d), T.storage_bytes(kv_cpu), lay, bt, torch.tensor(ctx, dtype=torch.int32),
+                             cu, 1 / math.sqrt(d))
+    T.assert_close_attn(out.view(n, hq, d), want, what="chunk on a long context through the backend")

@@ -306,3 +306,75 @@ def test_many_short_runs_take_one_wave_per_item(gpu_device):
         cc = (cu[lo_:hi_ + 1] - cu[lo_]).contiguous()
         parts.append(run(gpu_device, kv, "HND", bt[lo_:hi_].contiguous(), qq, sl[lo_:hi_].contiguous(), cc, max(qls), scale))
     T.assert_close_attn(torch.cat(parts), want, what="the same runs in three launches")
+
+
+@pytest.mark.parametrize("hq,hkv,d,layout,code", [(32, 8, 128, "HND", "int8"), (28, 4, 128, "NHD", "int8"),
+                                                  (8, 2, 64, "HND", "fp8"), (16, 8, 128, "HND", "int4")])
+@pytest.mark.parametrize("window,cap,extras", [(0, 0.0, False), (1500, 30.0, True)])
+def test_context_splits_of_long_runs(gpu_device, hq, hkv, d, layout, code, window, cap, extras):
+    """kvq_paged_attn_int8_split_prefill: the context of the long query runs in 2..8 ranges, merged afterwards.  A
+    small chunk on a long context, a run that starts its sequence, a decode row and a short run (both served as in
+    the plain call) in one batch; ranges without a visible tile (window, causal limit); sinks and ALiBi on top.
+    Output and lse against the oracle for every split count, and within 1e-2 of the plain call."""
+    from vllm_metax_amd.kv_cache_interface import KVQuantMode
+    ct = {"int8": oracle.CODE_INT8, "fp8": oracle.CODE_FP8, "int4": oracle.CODE_INT4}[code]
+    mode = {"int8": KVQuantMode.INT8_PER_TOKEN_HEAD, "fp8": KVQuantMode.FP8_PER_TOKEN_HEAD,
+            "int4": KVQuantMode.INT4_PER_TOKEN_HEAD}[code]
+    dev = gpu_device
+    bs = 16
+    ctx = [6000, 700, 200, 64, 3000]
+    qls = [200, 1, 200, 3, 77]
+    g = torch.Generator().manual_seed(hq + d + window)
+    nb = sum((c + bs - 1) // bs for c in ctx) + 5
+    kv_cpu, _, lay = T.cpu_cache(nb, bs, hkv, d, layout, code_type=ct)
+    bt = T.make_block_tables(ctx, bs, nb, g)
+    ks = [torch.randn((c, hkv, d), generator=g).to(torch.bfloat16) for c in ctx]
+    vs_ = [torch.randn((c, hkv, d), generator=g).to(torch.bfloat16) for c in ctx]
+    T.fill_cache_from_sources(kv_cpu, lay, bt, ctx, bs, ks, vs_, code_type=ct)
+    q = torch.randn((sum(qls), hq, d), generator=g).to(torch.bfloat16)
+    sl = torch.tensor(ctx, dtype=torch.int32)
+    cu = torch.tensor([0] + torch.tensor(qls).cumsum(0).tolist(), dtype=torch.int32)
+    scale = 1 / math.sqrt(d)
+    sinks = (torch.randn(hq, generator=g) * 2).float() if extras else None
+    slopes = torch.tensor([2.0 ** (-8.0 * (i + 1) / hq) for i in range(hq)], dtype=torch.float32) if extras else None
+    want, want_lse = oracle.paged_attn(q, T.storage_bytes(kv_cpu), lay, bt, sl, cu, scale, return_lse=True,
+                                       sliding_window=window, soft_cap=cap, code_type=ct, sinks=sinks, alibi_slopes=slopes)
+    kv = T.to_device_cache(kv_cpu, dev, layout, code_type=ct)
+    k, v = L.key_value_views(kv)
+    ksc, vsc = L.scale_views(kv)
+    plain = None
+    for splits in (1, 2, 3, 5, 8):
+        out = torch.full(q.shape, float("nan"), dtype=torch.bfloat16, device=dev)
+        lse = torch.full(q.shape[:2], float("nan"), dtype=torch.float32, device=dev)
+        ops.unified_attention(q.to(dev), k, v, out, cu.to(dev), max(qls), sl.to(dev), max(ctx), scale, True,
+                              window_size=(window - 1, 0) if window else (-1, -1), softcap=cap, block_table=bt.to(dev),
+                              k_scale_cache=ksc, v_scale_cache=vsc, kv_quant_mode=mode, lse=lse,
+                              sinks=None if sinks is None else sinks.to(dev),
+                              alibi_slopes=None if slopes is None else slopes.to(dev), prefill_splits=splits)
+        torch.cuda.synchronize()
+        T.assert_close_attn(out, want, what=f"{splits} context splits, {code}")
+        torch.testing.assert_close(lse.cpu(), want_lse, atol=5e-3, rtol=1e-3)
+        if plain is None:
+            plain = out.float().cpu()
+        else:
+            torch.testing.assert_close(out.float().cpu(), plain, atol=1e-2, rtol=1e-2)
+
+
+def test_context_splits_need_their_workspace(gpu_device):
+    dev = gpu_device
+    kv = L.allocate_kv_cache(40, 16, 2, 128, device=dev)
+    k, v = L.key_value_views(kv)
+    ks, vs = L.scale_views(kv)
+    q = torch.zeros((64, 8, 128), dtype=torch.bfloat16, device=dev)
+    cu = torch.tensor([0, 64], dtype=torch.int32, device=dev)
+    sl = torch.tensor([500], dtype=torch.int32, device=dev)
+    bt = torch.arange(32, dtype=torch.int32, device=dev).view(1, 32)
+    small = torch.empty(ops.paged_attn_workspace_bytes(1, 8, 128), dtype=torch.uint8, device=dev)
+    need = ops.split_prefill_workspace_bytes(1, 8, 128, 64, 4)
+    assert need >= small.numel() + 64 * 8 * 4 * 130 * 4
+    with pytest.raises(RuntimeError, match="workspace"):
+        ops.unified_attention(q, k, v, torch.empty_like(q), cu, 64, sl, 500, 0.1, True, block_table=bt,
+                              k_scale_cache=ks, v_scale_cache=vs, workspace=small, prefill_splits=4)
+    with pytest.raises(RuntimeError):
+        ops.unified_attention(q, k, v, torch.empty_like(q), cu, 64, sl, 500, 0.1, True, block_table=bt,
+                              k_scale_cache=ks, v_scale_cache=vs, prefill_splits=9)

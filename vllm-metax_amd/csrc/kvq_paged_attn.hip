@@ -17,7 +17,15 @@ int decode_streamk_num_wg(int num_kv_heads);
 int validate_common(const char* op, const void* q, const void* cache, const kvq_cache_geom* geom,
                     const int32_t* block_table, const int32_t* seq_lens, int num_seqs, int num_q_heads);
 int launch_prefill(const AttnIO& io, const int32_t* seq_lens, const int32_t* cu_seqlens_q, int num_seqs,
-                   int max_query_len, int causal, int q_dtype, int out_dtype, int32_t* plan, hipStream_t s);
+                   int max_query_len, int causal, int q_dtype, int out_dtype, int32_t* plan, hipStream_t s,
+                   int ksplit, float* part);
+
+// Where the context splits' partial states begin in a workspace, and how many bytes they take.
+static size_t split_part_offset(size_t streamk_bytes) { return (streamk_bytes + 255) & ~(size_t)255; }
+static size_t split_part_bytes(int num_tokens, int num_q_heads, int head_size, int splits) {
+  return (size_t)num_tokens * (size_t)num_q_heads * (size_t)splits * (size_t)(head_size + 2) * sizeof(float);
+}
+constexpr int kMaxPrefillSplits = 8;
 
 // Scratch of the entry point that allocates nothing: a fixed array in the code object's own device
 // memory.  Every GPU the library runs on holds one copy, at its own address, until the process ends.
@@ -68,7 +76,8 @@ static int paged_attn_launch(const char* op, void* out, int out_dtype, int64_t o
                              const int32_t* seq_lens, const int32_t* cu_seqlens_q, int num_seqs, int num_q_heads,
                              int max_query_len, float scale, int causal, int window_size, float softcap,
                              const float* sinks, const float* alibi_slopes, float* lse, void* workspace, size_t workspace_bytes, const char* workspace_what,
-                             kvq_stream_t stream, const NewTokens* fresh = nullptr) {
+                             kvq_stream_t stream, const NewTokens* fresh = nullptr, int prefill_splits = 1,
+                             int num_tokens = 0) {
   int rc0 = validate_common(op, q, cache, geom, block_table, seq_lens, num_seqs, num_q_heads);
   if (rc0) return rc0;
   KVQ_REQUIRE((causal & ~(KVQ_ATTN_CAUSAL | KVQ_ATTN_NO_DECODE_ROWS)) == 0, "%s: unknown flag in causal (%d)", op, causal);
@@ -87,7 +96,14 @@ static int paged_attn_launch(const char* op, void* out, int out_dtype, int64_t o
               "%s: out rows must be 4-byte aligned", op);
   const int num_wg = decode_streamk_num_wg(g.num_kv_heads);
   KVQ_REQUIRE(num_wg > 0, "%s: no HIP device", op);
-  const size_t need = streamk_workspace_bytes(num_seqs, num_q_heads, g.head_size, num_wg);
+  size_t need = streamk_workspace_bytes(num_seqs, num_q_heads, g.head_size, num_wg);
+  const size_t part_at = split_part_offset(need);
+  KVQ_REQUIRE(prefill_splits >= 1 && prefill_splits <= kMaxPrefillSplits, "%s: prefill_splits %d must be 1..%d", op,
+              prefill_splits, kMaxPrefillSplits);
+  if (prefill_splits > 1) {
+    KVQ_REQUIRE(num_tokens >= 1, "%s: num_tokens (the rows of q) is required with prefill_splits > 1", op);
+    need = part_at + split_part_bytes(num_tokens, num_q_heads, g.head_size, prefill_splits);
+  }
   KVQ_REQUIRE(workspace != nullptr && workspace_bytes >= need && ((uintptr_t)workspace % 16) == 0,
               "%s: %s of %zu bytes (16-byte aligned) required, got %zu", op, workspace_what, need, workspace_bytes);
 
@@ -155,7 +171,8 @@ static int paged_attn_launch(const char* op, void* out, int out_dtype, int64_t o
   if (max_query_len > 1) {
     // the list of the sequences that have a query run sits behind the decode kernels' notes in the workspace
     int32_t* plan = reinterpret_cast<int32_t*>(a.seq_first_unit + num_seqs);
-    rc = launch_prefill(a.io, seq_lens, cu_seqlens_q, num_seqs, max_query_len, causal, q_dtype, out_dtype, plan, s);
+    rc = launch_prefill(a.io, seq_lens, cu_seqlens_q, num_seqs, max_query_len, causal, q_dtype, out_dtype, plan, s,
+                        prefill_splits, reinterpret_cast<float*>(static_cast<uint8_t*>(workspace) + part_at));
   }
   return rc;
 }
@@ -173,6 +190,31 @@ extern "C" int kvq_paged_attn_int8(void* out, int out_dtype, int64_t out_stride_
                                 q_stride_h, cache, geom, block_table, bt_stride, seq_lens, cu_seqlens_q, num_seqs,
                                 num_q_heads, max_query_len, scale, causal, window_size, softcap, sinks, alibi_slopes, lse, workspace,
                                 workspace_bytes, "workspace", stream);
+}
+
+extern "C" size_t kvq_paged_attn_split_prefill_workspace_bytes(int max_num_seqs, int num_q_heads, int head_size,
+                                                              int num_tokens, int prefill_splits) {
+  if (max_num_seqs <= 0 || num_q_heads <= 0 || head_size <= 0) return 0;
+  const size_t base = kvq::streamk_workspace_bytes(max_num_seqs, num_q_heads, head_size, kvq::num_cus());
+  if (prefill_splits <= 1 || num_tokens <= 0) return base;
+  return kvq::split_part_offset(base) + kvq::split_part_bytes(num_tokens, num_q_heads, head_size, prefill_splits);
+}
+
+extern "C" int kvq_paged_attn_int8_split_prefill(void* out, int out_dtype, int64_t out_stride_t, int64_t out_stride_h,
+                                                 const void* q, int q_dtype, int64_t q_stride_t, int64_t q_stride_h,
+                                                 const void* cache, const kvq_cache_geom* geom,
+                                                 const int32_t* block_table, int64_t bt_stride,
+                                                 const int32_t* seq_lens, const int32_t* cu_seqlens_q, int num_seqs,
+                                                 int num_q_heads, int max_query_len, float scale, int causal,
+                                                 int window_size, float softcap, const float* sinks,
+                                                 const float* alibi_slopes, float* lse, int num_tokens,
+                                                 int prefill_splits, void* workspace, size_t workspace_bytes,
+                                                 kvq_stream_t stream) {
+  return kvq::paged_attn_launch("paged_attn_int8_split_prefill", out, out_dtype, out_stride_t, out_stride_h, q, q_dtype,
+                                q_stride_t, q_stride_h, cache, geom, block_table, bt_stride, seq_lens, cu_seqlens_q,
+                                num_seqs, num_q_heads, max_query_len, scale, causal, window_size, softcap, sinks,
+                                alibi_slopes, lse, workspace, workspace_bytes, "workspace", stream, nullptr,
+                                prefill_splits, num_tokens);
 }
 
 extern "C" int kvq_paged_attn_int8_fused_write(void* out, int out_dtype, int64_t out_stride_t, int64_t out_stride_h,

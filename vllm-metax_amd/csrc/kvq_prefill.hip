@@ -24,6 +24,13 @@ struct PrefillArgs {
   // [1 + B]: how many sequences of the batch have a query run (q_len > 1, len > 0), then their numbers in batch
   // order; written by prefill_plan_kernel ahead of the attention kernel of the same call.
   const int32_t* plan;
+  // Context splits of the workgroup-shared tile (1 = none).  With S > 1 an item's tiles are cut into S ranges, each
+  // range is a workgroup of its own that leaves a partial state per (query row, q head) in `part`
+  // ([row][q head][split][D + 2] fp32: the accumulated row, the reference maximum, the sum), and a merge kernel
+  // combines them: a launch with few items on a long context (a small prefill chunk of one long request) would
+  // otherwise walk the whole context in a handful of workgroups, one tile after the other.
+  int ksplit;
+  float* part;
 };
 
 // One workgroup lists the sequences that have work for the prefill kernels.  A mixed batch is mostly decode rows;
@@ -765,8 +772,11 @@ struct Flash32 {
 };
 
 // EXT adds the sliding window and the logits soft cap; the plain causal kernel carries neither.
-template <int D, int QDT, int ODT, bool EXT, int CODE = KVQ_CODE_INT8>
+// KSPLIT (with EXT only): the grid's x dimension carries a.ksplit context splits per query block; a workgroup takes
+// one range of its item's tiles and writes a partial state instead of the rows.
+template <int D, int QDT, int ODT, bool EXT, int CODE = KVQ_CODE_INT8, bool KSPLIT = false>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void paged_prefill_flash32_kernel(PrefillArgs a) {
+  static_assert(!KSPLIT || EXT, "the context split is built into the kernel with the extras only");
   using FP = Flash32<D, QDT, ODT, CODE>;
   using DTile = typename FP::DTile;
   extern __shared__ __align__(16) uint8_t lds[];
@@ -787,9 +797,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   // of every eight of every pair), 4 x 1024 new tokens on 8k-32k cached ones 2.43 -> 2.02 ms.  Query-block-major
   // over ALL pairs was better still for short prompts from scratch (16 x 512: 103 against 113 us) and much worse
   // with long contexts (the mixed batch 959 us: sixteen streams of keys at once, six times the HBM fetches).
-  const unsigned nqb = gridDim.x, hk = gridDim.z, per_seq = nqb * hk;
+  const unsigned nsplit = KSPLIT ? (unsigned)a.ksplit : 1u;
+  const unsigned nqb = gridDim.x / nsplit, hk = gridDim.z, per_seq = nqb * hk;
   const unsigned nseq = (unsigned)a.plan[0];
-  const unsigned lin = blockIdx.x + nqb * (blockIdx.y + gridDim.y * blockIdx.z);
+  const unsigned lin_all = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
+  const unsigned split = KSPLIT ? lin_all % nsplit : 0u;   // the splits of an item are neighbours in launch order
+  const unsigned lin = KSPLIT ? lin_all / nsplit : lin_all;
   if (lin >= per_seq * nseq) return;   // uniform over the workgroup
   const unsigned rem = lin % per_seq;
   const int qb = (int)(rem / hk);
@@ -841,7 +854,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     for (int i = 0; i < 16; ++i) o[mt][i] = 0.f;
   float m = -INFINITY, l = 0.f;
 
-  if (t_end > t_first) {
+  // this workgroup's tiles: all of the item's, or one of nsplit ranges of an even number of tiles
+  int t_lo = t_first, t_hi = t_end;
+  if constexpr (KSPLIT) {
+    const int per = (((t_end - t_first) + (int)nsplit - 1) / (int)nsplit + 1) & ~1;
+    t_lo = t_first + (int)split * per;
+    t_hi = min(t_end, t_lo + per);
+  }
+  if (t_hi > t_lo) {
     const LaneOffsets lo = DTile::lane_offsets(io.g, lane);
     const int32_t* bt_row = io.block_table + (int64_t)seq * io.bt_stride;
     const int step = (64 / DTile::NCH) * (int)io.g.stride_slot;
@@ -867,11 +887,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       *reinterpret_cast<u32x4*>(raw + l_chunk + 16 * FP::RAW_PITCH) = r.c1;
       if (wave < 2 && lane < 16) *reinterpret_cast<u32x2*>(raw + l_tail) = r.tail;
     };
-    TileBlocks nb = DTile::fetch_blocks(io, bt_row, len, t_first);
-    issue(nb, t_first, A);
-    nb = DTile::fetch_blocks(io, bt_row, len, t_first + 1);
-    issue(nb, t_first + 1, B);
-    nb = DTile::fetch_blocks(io, bt_row, len, t_first + 2);
+    TileBlocks nb = DTile::fetch_blocks(io, bt_row, len, t_lo);
+    issue(nb, t_lo, A);
+    nb = DTile::fetch_blocks(io, bt_row, len, t_lo + 1);
+    issue(nb, t_lo + 1, B);
+    nb = DTile::fetch_blocks(io, bt_row, len, t_lo + 2);
 
     half8_t qb[FP::KS];
     const float s_init =
@@ -884,9 +904,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       ali = alibi_slope(io.alibi, valid ? head : hkv * io.group);
     }
 
-    drop(A, raws);  // t_first is even: raw window 0
-    issue(nb, t_first + 2, A);
-    nb = DTile::fetch_blocks(io, bt_row, len, t_first + 3);
+    drop(A, raws);  // t_lo is even: raw window 0
+    issue(nb, t_lo + 2, A);
+    nb = DTile::fetch_blocks(io, bt_row, len, t_lo + 3);
     lds_barrier();
     // Step t: expand raw tile t into fp16 buffer t&1, drop tile t+1 (held in `next`) into the other
     // raw window and refill `next` with tile t+3, ONE barrier, then compute tile t.
@@ -910,10 +930,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     // loops (every wave runs the same number of steps, hence of barriers, whichever loop a step is
     // in), so that the accumulators keep their registers across the loop instead of being merged
     // at a branch inside it.
-    const int t_plain = min(t_end, wave_min_limit / kTile) & ~1;
-    int t = t_first;
+    const int t_plain = min(t_hi, wave_min_limit / kTile) & ~1;
+    int t = t_lo;
     if constexpr (EXT) {  // tiles that straddle a column's lower window edge
-      const int t_head = min(t_end, ((wave_max_first + kTile - 1) / kTile + 1) & ~1);
+      const int t_head = min(t_hi, ((wave_max_first + kTile - 1) / kTile + 1) & ~1);
       for (; t < t_head; t += 2) {
         step_fn(std::true_type{}, t, B);
         step_fn(std::true_type{}, t + 1, A);
@@ -923,7 +943,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       step_fn(std::false_type{}, t, B);
       step_fn(std::false_type{}, t + 1, A);
     }
-    for (; t < t_end; t += 2) {  // an odd t_end runs one step past the end: it computes nothing
+    for (; t < t_hi; t += 2) {  // an odd end runs one step past it: that step computes nothing
       step_fn(std::true_type{}, t, B);
       step_fn(std::true_type{}, t + 1, A);
     }
@@ -931,6 +951,23 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   // Lane (c, g) holds O[column][dim mt*32 + (i/4)*8 + 4g + i%4] in o[mt][i].
   l += __shfl_xor(l, 32, kWave);
   if (!valid) return;
+  if constexpr (KSPLIT) {
+    // the range's state: the row as accumulated (without the factor the weights carry), the reference maximum, the sum
+    float* p = a.part + (((int64_t)row * io.num_q_heads + head) * nsplit + split) * (D + 2);
+    const float unit = 1.0f / DTile::kOutDiv;
+    const int gg = lane >> 5;
+#pragma unroll
+    for (int mt = 0; mt < FP::MT; ++mt)
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+        *reinterpret_cast<floatx4_a4*>(p + mt * 32 + q * 8 + 4 * gg) =
+            (floatx4){o[mt][4 * q] * unit, o[mt][4 * q + 1] * unit, o[mt][4 * q + 2] * unit, o[mt][4 * q + 3] * unit};
+    if (gg == 0) {
+      p[D] = m;
+      p[D + 1] = l;
+    }
+    return;
+  }
   if (l > 0.f) l += sink_term(io.sinks, head, m);   // a row without a visible key keeps its zeros
   const int g = lane >> 5;
   const float mul = l > 0.f ? 1.0f / (l * DTile::kOutDiv) : 0.f;
@@ -964,6 +1001,53 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     io.lse[row * io.num_q_heads + head] = l > 0.f ? (m + __builtin_amdgcn_logf(l)) * kLn2 : -INFINITY;
 }
 
+// The merge of the context splits: grid (query token of a run, sequence of the plan), 4 waves; a wave takes q heads
+// wave, wave + 4, ... of its row, a lane D / 64 dims.  out = sum_s w_s o_s / sum_s w_s l_s with w_s = 2^(m_s - max m):
+// the algebra of merge_attn_states over the splits' states; the sink's term and the row's lse as in the unsplit kernel.
+template <int D, int ODT>
+__global__ __launch_bounds__(256) void prefill_split_merge_kernel(PrefillArgs a) {
+  constexpr int V = D / 64;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  if (blockIdx.y >= (unsigned)a.plan[0]) return;
+  const int seq = a.plan[1 + blockIdx.y];
+  const int q_begin = a.cu_seqlens_q[seq];
+  const int q_len = a.cu_seqlens_q[seq + 1] - q_begin;
+  const int qi = blockIdx.x;
+  if (q_len <= 1 || qi >= q_len || a.seq_lens[seq] <= 0) return;
+  const AttnIO& io = a.io;
+  const int64_t row = q_begin + qi;
+  const int S = a.ksplit;
+  for (int head = wave; head < io.num_q_heads; head += 4) {
+    const float* p = a.part + ((row * io.num_q_heads + head) * S) * (D + 2);
+    float mmax = -INFINITY;
+    for (int s = 0; s < S; ++s) mmax = fmaxf(mmax, p[s * (D + 2) + D]);
+    const float mref = mmax == -INFINITY ? 0.f : mmax;
+    float acc[V];
+#pragma unroll
+    for (int i = 0; i < V; ++i) acc[i] = 0.f;
+    float l = 0.f;
+    for (int s = 0; s < S; ++s) {
+      const float* ps = p + s * (D + 2);
+      const float w = __builtin_amdgcn_exp2f(ps[D] - mref);   // an empty range: 2^-inf = 0
+      l += w * ps[D + 1];
+#pragma unroll
+      for (int i = 0; i < V; ++i) acc[i] += w * ps[V * lane + i];
+    }
+    if (l > 0.f) l += sink_term(io.sinks, head, mmax);   // a row without a visible key keeps its zeros
+    const float mul = l > 0.f ? 1.0f / l : 0.f;
+    const int64_t at = row * io.out_stride_t + (int64_t)head * io.out_stride_h + V * lane;
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+      const float v = acc[i] * mul;
+      if constexpr (ODT == KVQ_F32) reinterpret_cast<float*>(io.out)[at + i] = v;
+      else if constexpr (ODT == KVQ_BF16) reinterpret_cast<uint16_t*>(io.out)[at + i] = f32_to_bf16_bits(v);
+      else reinterpret_cast<uint16_t*>(io.out)[at + i] = (uint16_t)(pack_half2(v, 0.f) & 0xffffu);
+    }
+    if (io.lse != nullptr && lane == 0)
+      io.lse[row * io.num_q_heads + head] = l > 0.f ? (mmax + __builtin_amdgcn_logf(l)) * kLn2 : -INFINITY;
+  }
+}
+
 template <int D, int QDT, int ODT, bool EXT, int CODE = KVQ_CODE_INT8>
 static int launch_prefill_flash32(PrefillArgs& a, int max_query_len, hipStream_t s) {
   using FP = Flash32<D, QDT, ODT, CODE>;
@@ -971,6 +1055,16 @@ static int launch_prefill_flash32(PrefillArgs& a, int max_query_len, hipStream_t
   const int blocks = (max_query_len + a.q_tokens - 1) / a.q_tokens;
   if (a.num_seqs > 65535 || a.io.g.num_kv_heads > 65535) return fail(KVQ_EINVAL, "paged_attn_int8: prefill grid out of range");
   static_assert(FP::LDS_BYTES <= 64 * 1024, "static LDS opt-in would be needed");
+  if constexpr (EXT) {
+    if (a.ksplit > 1) {
+      dim3 grid(blocks * a.ksplit, a.num_seqs, a.io.g.num_kv_heads);
+      hipLaunchKernelGGL((paged_prefill_flash32_kernel<D, QDT, ODT, true, CODE, true>), grid, dim3(256), FP::LDS_BYTES, s, a);
+      if (int e = check_hip(hipGetLastError(), "paged_prefill_flash32 launch")) return e;
+      dim3 mgrid(max_query_len, a.num_seqs);
+      hipLaunchKernelGGL((prefill_split_merge_kernel<D, ODT>), mgrid, dim3(256), 0, s, a);
+      return check_hip(hipGetLastError(), "prefill split merge launch");
+    }
+  }
   dim3 grid(blocks, a.num_seqs, a.io.g.num_kv_heads);
   hipLaunchKernelGGL((paged_prefill_flash32_kernel<D, QDT, ODT, EXT, CODE>), grid, dim3(256), FP::LDS_BYTES, s, a);
   return check_hip(hipGetLastError(), "paged_prefill_flash32 launch");
@@ -1004,7 +1098,7 @@ static int launch_prefill_nt(PrefillArgs& a, int max_query_len, hipStream_t s) {
   // long runs: the workgroup-shared fp16 tile (compute-bound shape), for every kind of code
   if constexpr (D <= 128) {
     if (max_query_len * a.io.group >= 64) {
-      const bool ext = a.io.window > 0 || a.io.cap_c != 0.f || a.io.alibi != nullptr;
+      const bool ext = a.io.window > 0 || a.io.cap_c != 0.f || a.io.alibi != nullptr || a.ksplit > 1;
       if (int4) {
         if (ext) return launch_prefill_flash32<D, QDT, ODT, true, KVQ_CODE_INT4>(a, max_query_len, s);
         return launch_prefill_flash32<D, QDT, ODT, false, KVQ_CODE_INT4>(a, max_query_len, s);
@@ -1055,8 +1149,11 @@ static int launch_prefill_q(PrefillArgs& a, int max_query_len, int q_dtype, int 
 }
 
 int launch_prefill(const AttnIO& io, const int32_t* seq_lens, const int32_t* cu_seqlens_q, int num_seqs,
-                   int max_query_len, int causal, int q_dtype, int out_dtype, int32_t* plan, hipStream_t s) {
+                   int max_query_len, int causal, int q_dtype, int out_dtype, int32_t* plan, hipStream_t s,
+                   int ksplit, float* part) {
   PrefillArgs a{};
+  a.ksplit = ksplit;
+  a.part = part;
   a.io = io;
   a.seq_lens = seq_lens;
   a.cu_seqlens_q = cu_seqlens_q;

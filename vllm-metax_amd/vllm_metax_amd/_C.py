@@ -14,7 +14,7 @@ LIB_PATH = os.path.join(_LIB_DIR, "libkvq_hip.so")
 
 KVQ_F32, KVQ_BF16, KVQ_F16 = 0, 1, 2
 KVQ_CODE_INT8, KVQ_CODE_FP8_E4M3, KVQ_CODE_INT4 = 0, 1, 2
-ABI_VERSION = 17
+ABI_VERSION = 18
 
 
 class CacheGeom(ctypes.Structure):
@@ -58,6 +58,9 @@ SIGNATURES = {
     "kvq_paged_attn_int8_fused_write": (_i, [_vp, _i, _i64, _i64, _vp, _i, _i64, _i64, _vp, _vp, _i, _i64, _i64, _i64, _i64,
                                              _f, _vp, _geom_p, _vp, _i64, _vp, _vp, _i, _i, _f, _i, _f, _vp, _vp, _vp, _vp, _sz,
                                              _vp]),
+    "kvq_paged_attn_split_prefill_workspace_bytes": (_sz, [_i, _i, _i, _i, _i]),
+    "kvq_paged_attn_int8_split_prefill": (_i, [_vp, _i, _i64, _i64, _vp, _i, _i64, _i64, _vp, _geom_p, _vp, _i64, _vp, _vp,
+                                               _i, _i, _i, _f, _i, _i, _f, _vp, _vp, _vp, _i, _i, _vp, _sz, _vp]),
     "kvq_paged_attn_static_scratch_bytes": (_sz, []),
     "kvq_paged_attn_int8_static_scratch": (_i, [_vp, _i, _i64, _i64, _vp, _i, _i64, _i64, _vp, _geom_p, _vp, _i64, _vp,
                                                 _vp, _i, _i, _i, _f, _i, _i, _f, _vp, _vp, _vp, _vp]),

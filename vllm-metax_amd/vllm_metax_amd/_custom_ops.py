@@ -301,6 +301,7 @@ def unified_attention(
     lse: torch.Tensor | None = None,
     static_scratch: bool = False,
     has_decode_rows: bool = True,
+    prefill_splits: int = 1,
     **unused,
 ) -> None:
     """Drop-in for ``unified_attention`` as called at
@@ -319,7 +320,11 @@ def unified_attention(
     ``alibi_slopes`` ``[Hq]`` float32: the logit of query position p and key position j gets ``slope * (j - p)``
     added (triton_attn.py:699; causal attention only); the square-root form (``use_alibi_sqrt``) is not built.
     ``has_decode_rows=False`` is the caller's promise that no sequence of the batch has exactly one query row (a
-    pure prefill batch): the decode kernel and its reduce are then not launched."""
+    pure prefill batch): the decode kernel and its reduce are then not launched.
+    ``prefill_splits`` (1..8): the context of the long query runs is cut into that many ranges, each a workgroup of
+    its own, and merged (``prefill_context_splits`` proposes a value): for launches whose long runs make few
+    workgroups on a long context, e.g. one request's small prefill chunk.  The workspace must then hold
+    ``split_prefill_workspace_bytes(...)``; the default workspace is grown as needed."""
     code_type = code_type_of(kv_quant_mode)
     if output_scale is not None or mm_prefix_range is not None:
         raise NotImplementedError("fused output quantisation and mm-prefix ranges are not built")
@@ -378,9 +383,19 @@ def unified_attention(
             _ptr(seqused_k), _ptr(cu_seqlens_q), num_seqs, num_q_heads, int(max_seqlen_q),
             float(softmax_scale), (1 if causal else 0) | (0 if has_decode_rows else 2), window, softcap,
             _ptr(sinks), _ptr(alibi_slopes), _ptr(lse))
+    prefill_splits = int(prefill_splits)
+    if not 1 <= prefill_splits <= 8:
+        raise RuntimeError("prefill_splits must be 1..8")
     if static_scratch:
         with _on_device(dev):
             rc = lib.kvq_paged_attn_int8_static_scratch(*head, _stream(dev))
+    elif prefill_splits > 1 and int(max_seqlen_q) > 1:
+        need = split_prefill_workspace_bytes(num_seqs, num_q_heads, geom.head_size, q.shape[0], prefill_splits, dev)
+        if workspace is None:
+            workspace = _default_workspace(dev, need)
+        with _on_device(dev):
+            rc = lib.kvq_paged_attn_int8_split_prefill(*head, q.shape[0], prefill_splits, _ptr(workspace),
+                                                       workspace.numel() * workspace.element_size(), _stream(dev))
     else:
         if workspace is None:
             workspace = _default_workspace(dev, paged_attn_workspace_bytes(num_seqs, num_q_heads, geom.head_size, dev))
@@ -388,6 +403,35 @@ def unified_attention(
             rc = lib.kvq_paged_attn_int8(*head, _ptr(workspace), workspace.numel() * workspace.element_size(),
                                          _stream(dev))
     _C.check(rc, "unified_attention")
+
+
+def split_prefill_workspace_bytes(max_num_seqs: int, num_q_heads: int, head_size: int, num_tokens: int,
+                                  prefill_splits: int, device: torch.device | None = None) -> int:
+    """Workspace of ``unified_attention(..., prefill_splits=n)``: the plain workspace plus the partial states of
+    ``num_tokens`` query rows."""
+    idx = torch.cuda.current_device() if device is None or device.index is None else device.index
+    with torch.cuda.device(idx):
+        return int(_C.load().kvq_paged_attn_split_prefill_workspace_bytes(max_num_seqs, num_q_heads, head_size,
+                                                                         num_tokens, prefill_splits))
+
+
+def prefill_context_splits(query_lens, max_seq_len: int, num_q_heads: int, num_kv_heads: int, num_cus: int = 256,
+                           max_split_tokens: int = 4096) -> int:
+    """How many context splits a launch should ask for, from what a metadata builder knows on the host: the query
+    run lengths of the batch (``query_lens``: a list or CPU tensor; one-token runs do not count), the longest
+    sequence, the head counts.  A run of q tokens makes ceil(q / (128 / group)) x Hkv workgroups of the
+    workgroup-shared tile; when the launch's workgroups do not fill the chip's two per compute unit and the context
+    is long, the context is cut so that they do -- as long as the partial states stay small (splits x run tokens
+    <= ``max_split_tokens``)."""
+    group = max(1, num_q_heads // max(1, num_kv_heads))
+    lens = [int(x) for x in (query_lens.tolist() if hasattr(query_lens, "tolist") else query_lens)]
+    runs = [x for x in lens if x > 1]
+    if not runs or max(runs) * group < 64 or max_seq_len < 4096:
+        return 1
+    q_tokens = max(1, 128 // group)
+    wgs = sum((x + q_tokens - 1) // q_tokens for x in runs) * num_kv_heads
+    splits = min(8, (2 * num_cus) // max(1, wgs), max_split_tokens // max(1, sum(runs)), max_seq_len // 2048)
+    return max(1, splits)
 
 
 def decode_attention_with_cache_update(

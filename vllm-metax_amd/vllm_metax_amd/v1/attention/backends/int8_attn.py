@@ -79,6 +79,7 @@ class Int8AttentionMetadata:
     slot_mapping: torch.Tensor
     workspace: torch.Tensor | None
     causal: bool = True
+    prefill_splits: int = 1      # context splits of the long query runs (the builder's proposal for this launch)
     use_cascade: bool = False
     common_prefix_len: int = 0
     # False when the builder KNOWS (from the host copy of query_start_loc) that no sequence has exactly one query
@@ -124,9 +125,15 @@ class Int8AttentionMetadataBuilder(_BuilderBase):
         self.max_num_seqs = int(_first_attr(sched, "max_num_seqs", default=256)) if sched is not None else 256
         self._workspace: torch.Tensor | None = None
 
+    # query rows x context splits whose partial states the workspace has room for (a launch is split only when its
+    # long runs are few: a small prefill chunk of a long request)
+    MAX_SPLIT_TOKENS: ClassVar[int] = 4096
+
     def _get_workspace(self) -> torch.Tensor | None:
         if self._workspace is None and self.device.type == "cuda":
-            nbytes = ops.paged_attn_workspace_bytes(self.max_num_seqs, self.num_heads_q, self.headdim)
+            # the plain workspace + the partial states of MAX_SPLIT_TOKENS (rows x splits)
+            nbytes = ops.split_prefill_workspace_bytes(self.max_num_seqs, self.num_heads_q, self.headdim,
+                                                       self.MAX_SPLIT_TOKENS // 2, 2)
             self._workspace = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=self.device)
         return self._workspace
 
@@ -143,11 +150,20 @@ class Int8AttentionMetadataBuilder(_BuilderBase):
         if c.num_reqs > self.max_num_seqs:
             raise RuntimeError(f"batch of {c.num_reqs} sequences exceeds max_num_seqs={self.max_num_seqs}")
         has_decode_rows = True
+        prefill_splits = 1
         qsl_cpu = getattr(c, "query_start_loc_cpu", None)
         if qsl_cpu is not None and c.max_query_len > 1 and qsl_cpu.numel() > 1:
-            has_decode_rows = bool((qsl_cpu[1:] - qsl_cpu[:-1] == 1).any())
+            qlens = qsl_cpu[1:] - qsl_cpu[:-1]
+            has_decode_rows = bool((qlens == 1).any())
+            # a launch whose long runs make too few workgroups for the chip walks a long context in context splits;
+            # the partial states are indexed by the query row, so every row of the batch counts against the room
+            prefill_splits = ops.prefill_context_splits(qlens, int(c.max_seq_len), self.num_heads_q, self.num_heads_kv,
+                                                        max_split_tokens=self.MAX_SPLIT_TOKENS)
+            while prefill_splits > 1 and prefill_splits * int(c.num_actual_tokens) > self.MAX_SPLIT_TOKENS:
+                prefill_splits -= 1
         return Int8AttentionMetadata(
             has_decode_rows=has_decode_rows,
+            prefill_splits=prefill_splits,
             num_actual_tokens=c.num_actual_tokens,
             max_query_len=c.max_query_len,
             query_start_loc=c.query_start_loc,
@@ -427,7 +443,7 @@ class Int8AttentionImpl(_ImplBase):
             kv_quant_mode=self._kv_quant_mode, k_scale_cache=self._k_scale_cache, v_scale_cache=self._v_scale_cache,
             workspace=attn_metadata.workspace, geometry=self._geometry,
             has_decode_rows=getattr(attn_metadata, "has_decode_rows", True), sinks=self._sinks_on(q.device),
-            alibi_slopes=self._alibi_on(q.device))
+            alibi_slopes=self._alibi_on(q.device), prefill_splits=getattr(attn_metadata, "prefill_splits", 1))
         return output
 
 
