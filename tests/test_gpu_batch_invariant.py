@@ -201,3 +201,39 @@ def test_mla_decode_rows_do_not_depend_on_the_batch(gpu_device, invariant_mode, 
     live = sl > 0
     T.assert_close_attn(got[live], want[live], what="batch-invariant mla decode vs oracle")
     torch.testing.assert_close(got_lse[live], want_lse[live], atol=5e-3, rtol=1e-3)
+
+
+def test_short_runs_and_context_splits_keep_their_bits_in_the_mode(gpu_device, invariant_mode):
+    """Short query runs alone (a launch with few items) and among 300 sequences (a launch with many), and a long run
+    with and without a proposal of context splits: the mode keeps one way of cutting, so the bits do not move."""
+    dev = gpu_device
+    hq, hkv, d, bs = 32, 8, 128, 16
+    g = torch.Generator().manual_seed(4)
+    n = 300
+    ctx = [3000, 900] + torch.randint(20, 200, (n - 2,), generator=g).tolist()
+    qls = [3, 150] + torch.randint(1, 4, (n - 2,), generator=g).tolist()
+    qls = [min(c, x) for c, x in zip(ctx, qls)]
+    kv_cpu, lay, bt, _, sl, _ = build_case(ctx, hq, hkv, d, bs, "HND", 6, poison=False)
+    kv = T.to_device_cache(kv_cpu, dev, "HND")
+    k, v = L.key_value_views(kv)
+    ks, vs = L.scale_views(kv)
+    qs = [torch.randn((x, hq, d), generator=g).to(torch.bfloat16) for x in qls]
+    scale = 1 / math.sqrt(d)
+
+    def run(idx, splits=1):
+        q = torch.cat([qs[i] for i in idx]).to(dev)
+        cu = torch.tensor([0] + torch.tensor([qls[i] for i in idx]).cumsum(0).tolist(), dtype=torch.int32, device=dev)
+        ii = torch.tensor(idx)
+        out = torch.full(q.shape, float("nan"), dtype=torch.bfloat16, device=dev)
+        ops.unified_attention(q, k, v, out, cu, max(qls[i] for i in idx), sl[ii].to(dev), int(sl[ii].max()), scale, True,
+                              block_table=bt[ii].contiguous().to(dev), k_scale_cache=ks, v_scale_cache=vs,
+                              prefill_splits=splits)
+        torch.cuda.synchronize()
+        cu = cu.cpu()
+        return {i: out[int(cu[j]):int(cu[j + 1])].cpu() for j, i in enumerate(idx)}
+
+    whole = run(list(range(n)))
+    for idx, splits in (([0], 1), ([1], 1), ([1], 4), ([0, 1, 5], 2), (list(range(0, n, 3)), 1)):
+        got = run(idx, splits)
+        for i in idx:
+            assert torch.equal(got[i].view(torch.int16), whole[i].view(torch.int16)), f"sequence {i} in batch {idx[:4]} x{splits}"

@@ -171,8 +171,10 @@ static int paged_attn_launch(const char* op, void* out, int out_dtype, int64_t o
   if (max_query_len > 1) {
     // the list of the sequences that have a query run sits behind the decode kernels' notes in the workspace
     int32_t* plan = reinterpret_cast<int32_t*>(a.seq_first_unit + num_seqs);
+    // (the batch-invariant mode keeps one cut of the context whatever the caller proposes for this launch)
     rc = launch_prefill(a.io, seq_lens, cu_seqlens_q, num_seqs, max_query_len, causal, q_dtype, out_dtype, plan, s,
-                        prefill_splits, reinterpret_cast<float*>(static_cast<uint8_t*>(workspace) + part_at));
+                        batch_invariant() ? 1 : prefill_splits,
+                        reinterpret_cast<float*>(static_cast<uint8_t*>(workspace) + part_at));
   }
   return rc;
 }

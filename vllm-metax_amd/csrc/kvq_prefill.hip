@@ -31,6 +31,10 @@ struct PrefillArgs {
   // otherwise walk the whole context in a handful of workgroups, one tile after the other.
   int ksplit;
   float* part;
+  // Batch-invariant mode: which runs a kernel of this launch takes -- 0 all, 1 only those that fill the
+  // workgroup-shared tile by themselves (q_len x group >= 64), 2 only the others.  Without the mode the batch's
+  // longest run chooses ONE kernel for every run of the launch, so a short run's bits would depend on its company.
+  int route;
 };
 
 // One workgroup lists the sequences that have work for the prefill kernels.  A mixed batch is mostly decode rows;
@@ -334,6 +338,7 @@ __global__ __launch_bounds__(WPW * 64) void paged_prefill_kernel(PrefillArgs a) 
   const int len = a.seq_lens[seq];
   const int q0 = (int)(nqb - 1 - qbi) * a.q_tokens;   // first query token of this block within the run
   if (q_len <= 1 || q0 >= q_len || len <= 0) return;
+  if (a.route == 2 && q_len * io.group >= 64) return;   // the workgroup-shared tile's (uniform over the workgroup)
   uint8_t* lds = lds_all[wave];
 
   // ---- columns: n = nt * 16 + c  ->  (query token q0 + n / group, head n % group)
@@ -814,6 +819,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   const int len = a.seq_lens[seq];
   const int q0 = ((int)nqb - 1 - qb) * a.q_tokens;
   if (q_len <= 1 || q0 >= q_len || len <= 0) return;   // uniform over the workgroup
+  if (a.route == 1 && q_len * io.group < 64) return;    // the per-wave tile's
 
   // column of this lane: (query token q0 + n / group, head n % group), n = wave * 32 + (lane & 31)
   const int ctx = len - q_len;
@@ -1077,7 +1083,9 @@ template <int D, int QDT, int ODT, int NT, int WPW, int CODE = KVQ_CODE_INT8>
 static int launch_prefill_cfg(const PrefillArgs& a, int max_query_len, hipStream_t s) {
   const int blocks = (max_query_len + a.q_tokens - 1) / a.q_tokens;
   if (blocks > 0x7fffffff / 2 || a.num_seqs > 65535) return fail(KVQ_EINVAL, "paged_attn_int8: prefill grid out of range");
-  if ((int64_t)blocks * a.num_seqs * a.io.g.num_kv_heads <= kSplitItems && a.io.g.num_kv_heads <= 65535) {
+  // (not in the batch-invariant mode: how an item is cut would depend on what else the launch holds)
+  if (!batch_invariant() && (int64_t)blocks * a.num_seqs * a.io.g.num_kv_heads <= kSplitItems &&
+      a.io.g.num_kv_heads <= 65535) {
     // waves per item: eight with one column tile per wave; four with two (their accumulators need the registers
     // of a 256-thread workgroup)
     constexpr int SW = NT == 1 ? 8 : 4;
@@ -1091,13 +1099,34 @@ static int launch_prefill_cfg(const PrefillArgs& a, int max_query_len, hipStream
 }
 
 template <int D, int QDT, int ODT>
+static int launch_prefill_nt(PrefillArgs& a, int max_query_len, hipStream_t s);
+
+// Batch-invariant mode: every run goes to the kernel its OWN length chooses.  Runs that fill the workgroup-shared
+// tile by themselves take it; the others take the per-wave tile with one column tile per wave -- in a second launch
+// when the batch holds both kinds.
+template <int D, int QDT, int ODT>
+static int launch_prefill_invariant(PrefillArgs& a, int max_query_len, hipStream_t s) {
+  const int group = a.io.group;
+  if (D <= 128 && max_query_len * group >= 64) {
+    a.route = 1;
+    if (int e = launch_prefill_nt<D, QDT, ODT>(a, max_query_len, s)) return e;
+    a.route = 2;
+    const int longest_short = (63 / group);        // q_len x group < 64
+    if (longest_short < 2) return KVQ_OK;           // no run of two tokens or more is short
+    return launch_prefill_nt<D, QDT, ODT>(a, longest_short, s);
+  }
+  a.route = 0;
+  return launch_prefill_nt<D, QDT, ODT>(a, max_query_len, s);
+}
+
+template <int D, int QDT, int ODT>
 static int launch_prefill_nt(PrefillArgs& a, int max_query_len, hipStream_t s) {
   constexpr int WPW = 4;
   const bool fp8 = a.io.g.code_type == KVQ_CODE_FP8_E4M3;
   const bool int4 = a.io.g.code_type == KVQ_CODE_INT4;
   // long runs: the workgroup-shared fp16 tile (compute-bound shape), for every kind of code
   if constexpr (D <= 128) {
-    if (max_query_len * a.io.group >= 64) {
+    if (max_query_len * a.io.group >= 64 && a.route != 2) {
       const bool ext = a.io.window > 0 || a.io.cap_c != 0.f || a.io.alibi != nullptr || a.ksplit > 1;
       if (int4) {
         if (ext) return launch_prefill_flash32<D, QDT, ODT, true, KVQ_CODE_INT4>(a, max_query_len, s);
@@ -1120,7 +1149,7 @@ static int launch_prefill_nt(PrefillArgs& a, int max_query_len, hipStream_t s) {
     return launch_prefill_cfg<D, QDT, ODT, 1, WPW, KVQ_CODE_INT4>(a, max_query_len, s);
   }
   // two column tiles per wave where the accumulators fit the register file next to a tile in flight
-  if (D <= 128 && a.io.group * 2 <= 32 && max_query_len * a.io.group > 16) {
+  if (D <= 128 && a.io.group * 2 <= 32 && max_query_len * a.io.group > 16 && !batch_invariant()) {
     a.q_tokens = 32 / a.io.group;
     return launch_prefill_cfg<D, QDT, ODT, (D <= 128 ? 2 : 1), WPW>(a, max_query_len, s);
   }
@@ -1131,9 +1160,12 @@ static int launch_prefill_nt(PrefillArgs& a, int max_query_len, hipStream_t s) {
 template <int D, int QDT>
 static int launch_prefill_o(PrefillArgs& a, int max_query_len, int out_dtype, hipStream_t s) {
   switch (out_dtype) {
-    case KVQ_F32: return launch_prefill_nt<D, QDT, KVQ_F32>(a, max_query_len, s);
-    case KVQ_BF16: return launch_prefill_nt<D, QDT, KVQ_BF16>(a, max_query_len, s);
-    case KVQ_F16: return launch_prefill_nt<D, QDT, KVQ_F16>(a, max_query_len, s);
+    case KVQ_F32: return batch_invariant() ? launch_prefill_invariant<D, QDT, KVQ_F32>(a, max_query_len, s)
+                                           : launch_prefill_nt<D, QDT, KVQ_F32>(a, max_query_len, s);
+    case KVQ_BF16: return batch_invariant() ? launch_prefill_invariant<D, QDT, KVQ_BF16>(a, max_query_len, s)
+                                            : launch_prefill_nt<D, QDT, KVQ_BF16>(a, max_query_len, s);
+    case KVQ_F16: return batch_invariant() ? launch_prefill_invariant<D, QDT, KVQ_F16>(a, max_query_len, s)
+                                           : launch_prefill_nt<D, QDT, KVQ_F16>(a, max_query_len, s);
     default: return fail(KVQ_EINVAL, "paged_attn_int8: unknown out_dtype %d", out_dtype);
   }
 }
