@@ -412,7 +412,7 @@ def mla_caller_chain(cfg, st, dev, ops, n):
 
     def three_steps(i):
         attn_out, _ = impl.forward_mqa((caller.absorb_q(q_nope), q_pe), st["caches"][i % L], md)
-        caller.v_up_proj(attn_out, out)
+        caller.v_up_proj_library(attn_out, out)
 
     res = {}
     for name, fn in (("absorb_in_launch_us", fused), ("library_gemm_then_decode_us", three_steps)):

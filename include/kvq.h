@@ -27,7 +27,7 @@
 extern "C" {
 #endif
 
-#define KVQ_ABI_VERSION 18
+#define KVQ_ABI_VERSION 19
 
 #define KVQ_OK 0
 #define KVQ_EINVAL (-22)
@@ -574,6 +574,25 @@ KVQ_API int kvq_mla_decode_absorb_int8(void* out, int out_dtype, float* lse, con
                                const int32_t* block_table, int64_t bt_stride,
                                const int32_t* seq_lens, int num_seqs, int num_heads, float scale,
                                void* workspace, size_t workspace_bytes, kvq_stream_t stream);
+
+/*
+ * The V up-projection behind the MLA decode: out[b, h, :] = x[b, h, :] . W_UV[h],
+ * the second bmm of the reference's MLA layer (`_v_up_proj`,
+ * vllm_metax/model_executor/layers/attention/mla_attention.py:1087-1109: x [B, N, L]
+ * transposed to [N, B, L], bmm with W_UV [N, L, V], back to [B, N * V]; the plain
+ * branch, without quantised weights).  x [num_seqs, num_heads, kv_lora_rank] is
+ * what kvq_mla_decode_int8 / _absorb_int8 wrote, w_uv [num_heads, kv_lora_rank,
+ * v_head_dim] with the output dims contiguous, out [num_seqs, num_heads,
+ * v_head_dim] (a view of [num_seqs, num_heads * v_head_dim]).  All three of
+ * `dtype` KVQ_BF16 or KVQ_F16, fp32 accumulation, one rounding at the store;
+ * strides in elements.  kv_lora_rank and v_head_dim multiples of 128, W_UV and
+ * out rows 16-byte aligned, x rows 4-byte aligned.
+ */
+KVQ_API int kvq_mla_v_up_proj(void* out, int64_t out_stride_b, int64_t out_stride_h,
+                              const void* x, int dtype, int64_t x_stride_b, int64_t x_stride_h,
+                              const void* w_uv, int64_t w_stride_h, int64_t w_stride_l,
+                              int num_seqs, int num_heads, int kv_lora_rank, int v_head_dim,
+                              kvq_stream_t stream);
 
 /*
  * Varlen attention with LSE output over dense K and V: the attention step of

@@ -344,9 +344,9 @@ def test_mla_decode_with_fused_absorption(gpu_device, dtype, N, Pn, ctx):
     torch.testing.assert_close(lse.cpu()[live], want_lse[live], atol=5e-3, rtol=1e-3)
 
 
-def test_decode_caller_makes_one_library_gemm(gpu_device, monkeypatch):
-    """The Q side of Int8MLADecodeCaller.forward_decode runs in the decode launch: the only torch.bmm left is
-    the V up-projection (mla_attention.py:902, 1087-1110)."""
+def test_decode_caller_makes_no_library_gemm(gpu_device, monkeypatch):
+    """Int8MLADecodeCaller.forward_decode in a serving dtype: the Q absorption runs in the decode launch and the V
+    up-projection (mla_attention.py:902, 1087-1110) is kvq_mla_v_up_proj -- no torch.bmm is left."""
     from types import SimpleNamespace
 
     from vllm_metax_amd.v1.attention.backends.mla.int8_mla import Int8MLADecodeCaller, Int8MLAImpl
@@ -367,7 +367,57 @@ def test_decode_caller_makes_one_library_gemm(gpu_device, monkeypatch):
     caller.forward_decode(torch.randn((2, N, Pn), generator=g).to(torch.bfloat16).to(dev),
                           torch.randn((2, N, P), generator=g).to(torch.bfloat16).to(dev), cache.to(dev), md, out)
     torch.cuda.synchronize()
-    assert calls == [torch.Size([N, 2, R])]
+    assert calls == []
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("B,N,L,V", [
+    (32, 128, 512, 128),     # the decode batch of the 128-head configuration
+    (3, 16, 512, 128),       # a tensor-parallel shard, a tile of 3 live rows
+    (17, 20, 512, 128),      # a second sequence tile of one row; heads that do not fill the last XCD round
+    (1, 5, 256, 256),        # another latent width (run-time step count), two blocks of output dims
+    (70, 9, 384, 128),
+])
+def test_v_up_proj_matches_the_fp32_product(gpu_device, dtype, B, N, L, V):
+    """kvq_mla_v_up_proj against the product in fp32 (the reference's _v_up_proj is a bmm over [N, B, L] x
+    [N, L, V], vllm_metax/model_executor/layers/attention/mla_attention.py:1087-1109): fp32 accumulation and one
+    rounding to the activation type, so the result is within one rounding step of the exact product."""
+    dev = gpu_device
+    g = torch.Generator().manual_seed(B * 131 + N)
+    x_full = torch.randn((B, N, L + 64), generator=g).to(dtype)          # x as a strided view: rows L + 64 apart
+    W = (torch.randn((N, L, V), generator=g) / L ** 0.5).to(dtype)
+    out = torch.full((B, N * V), float("nan"), dtype=dtype, device=dev)
+    ops.mla_v_up_proj(x_full.to(dev)[..., :L], W.to(dev), out)
+    torch.cuda.synchronize()
+    want = torch.einsum("bnl,nlv->bnv", x_full[..., :L].float(), W.float()).reshape(B, N * V)
+    eps = 2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -11
+    torch.testing.assert_close(out.float().cpu(), want, atol=5e-5, rtol=eps)
+    # a few exactly representable cases: x = one-hot rows pick rows of W
+    x1 = torch.zeros((B, N, L), dtype=dtype)
+    pick = torch.randint(0, L, (B, N), generator=g)
+    x1.scatter_(2, pick.unsqueeze(-1), 1.0)
+    out3 = torch.empty((B, N, V), dtype=dtype, device=dev)
+    ops.mla_v_up_proj(x1.to(dev), W.to(dev), out3)
+    torch.cuda.synchronize()
+    want1 = W[torch.arange(N).unsqueeze(0).expand(B, N), pick]            # [B, N, V]
+    assert torch.equal(out3.cpu(), want1)
+
+
+def test_v_up_proj_errors(gpu_device):
+    dev = gpu_device
+    x = torch.zeros((2, 4, 512), dtype=torch.bfloat16, device=dev)
+    W = torch.zeros((4, 512, 128), dtype=torch.bfloat16, device=dev)
+    out = torch.zeros((2, 4 * 128), dtype=torch.bfloat16, device=dev)
+    with pytest.raises(RuntimeError):
+        ops.mla_v_up_proj(x, W.half(), out)                      # mixed dtypes
+    with pytest.raises(RuntimeError):
+        ops.mla_v_up_proj(x[..., :500], W[:, :500], out)         # latent width not a multiple of 128
+    with pytest.raises(RuntimeError):
+        ops.mla_v_up_proj(x, W[..., :64], out[:, :4 * 64])       # 64 output dims
+    with pytest.raises(RuntimeError):
+        ops.mla_v_up_proj(x.float(), W.float(), out.float())     # fp32 goes to the library GEMM in the caller
+    with pytest.raises(RuntimeError):
+        ops.mla_v_up_proj(x, W, out[:, :-1])
 
 
 def test_mla_decode_errors(gpu_device):

@@ -279,6 +279,7 @@ struct MlaAbsorbArgs {
   uint8_t* q_ops;
   float* q_scale;
   int head_groups, num_heads, num_seqs, ksteps;   // ksteps = P / 32
+  int seq_tiles, group_major;                     // tiles of 16 * kMlaAbsorbTiles sequences; how workgroups are numbered
 };
 
 // KSTEPS = P / 32 when known at compile time (the loop is unrolled and every load of W is in flight at
@@ -290,7 +291,20 @@ __global__ __launch_bounds__(256) void mla_absorb_q_kernel(MlaAbsorbArgs a) {
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int c = lane & 15, g = lane >> 4;
-  const int head = blockIdx.x, b0 = blockIdx.y * (16 * NB);
+  // Workgroups go to the eight XCDs round-robin in launch order.  With a multiple of eight head groups a group's
+  // workgroups (16 heads x the tiles of sequences) are numbered onto ONE XCD: the 16-byte pieces that 16 heads
+  // write into an operand block then meet in that XCD's L2 as whole lines (and the tiles of a head still share
+  // its weights there); otherwise heads are numbered first, which keeps the tiles of a head on one XCD.
+  int head, b0;
+  if (a.group_major) {
+    const int per_group = 16 * a.seq_tiles;
+    const int q = blockIdx.x >> 3, r = q % per_group;
+    head = ((q / per_group) * 8 + (blockIdx.x & 7)) * 16 + (r & 15);
+    b0 = (r >> 4) * (16 * NB);
+  } else {
+    head = blockIdx.x % (a.head_groups * 16);
+    b0 = blockIdx.x / (a.head_groups * 16) * (16 * NB);
+  }
   const bool head_ok = head < a.num_heads;
   const int hsrc = head_ok ? head : 0;
   floatx4 acc[NB][8];
@@ -1504,7 +1518,9 @@ static int mla_decode_run(const char* op, void* out, int out_dtype, float* lse, 
     absorb->head_groups = head_groups;
     absorb->num_heads = num_heads;
     absorb->num_seqs = num_seqs;
-    dim3 agrid(head_groups * 16, (num_seqs + 16 * kMlaAbsorbTiles - 1) / (16 * kMlaAbsorbTiles));
+    absorb->seq_tiles = (num_seqs + 16 * kMlaAbsorbTiles - 1) / (16 * kMlaAbsorbTiles);
+    absorb->group_major = head_groups % 8 == 0;
+    dim3 agrid(head_groups * 16 * absorb->seq_tiles);
 #define KVQ_MLAA(T, K) hipLaunchKernelGGL((mla_absorb_q_kernel<T, K>), agrid, dim3(256), 0, s, *absorb)
     if (q_dtype == KVQ_BF16) {
       if (absorb->ksteps == 4) KVQ_MLAA(KVQ_BF16, 4);

@@ -14,7 +14,7 @@ LIB_PATH = os.path.join(_LIB_DIR, "libkvq_hip.so")
 
 KVQ_F32, KVQ_BF16, KVQ_F16 = 0, 1, 2
 KVQ_CODE_INT8, KVQ_CODE_FP8_E4M3, KVQ_CODE_INT4 = 0, 1, 2
-ABI_VERSION = 18
+ABI_VERSION = 19
 
 
 class CacheGeom(ctypes.Structure):
@@ -86,6 +86,7 @@ SIGNATURES = {
     "kvq_rope_and_cache_int8": (_i, [_vp, _vp, _i64, _i64, _i, _vp, _i64, _i64, _vp, _i64, _i64, _i, _vp, _i, _i, _i, _vp,
                                      _geom_p, _vp, _i64, _f, _vp]),
     "kvq_concat_mla_q": (_i, [_vp, _i64, _i64, _vp, _i64, _i64, _vp, _i64, _i64, _i, _i64, _i, _i, _i, _vp]),
+    "kvq_mla_v_up_proj": (_i, [_vp, _i64, _i64, _vp, _i, _i64, _i64, _vp, _i64, _i64, _i, _i, _i, _i, _vp]),
     "kvq_mla_prefill_attn": (_i, [_vp, _i, _i64, _i64, _vp, _i64, _i64, _vp, _i64, _vp, _i64, _i64, _vp, _vp, _i, _i,
                                   _i64, _i, _i, _i, _i, _f, _i, _vp, _i64, _i64, _vp, _vp]),
 }

@@ -977,6 +977,36 @@ def mla_decode_absorb_int8(q_nope: torch.Tensor, W_UK_T: torch.Tensor, q_pe: tor
     _C.check(rc, "mla_decode_absorb_int8")
 
 
+def mla_v_up_proj(x: torch.Tensor, W_UV: torch.Tensor, out: torch.Tensor) -> None:
+    """``out[b, h, :] = x[b, h, :] @ W_UV[h]``: the V up-projection behind the MLA decode, the
+    reference's ``_v_up_proj`` (vllm_metax/model_executor/layers/attention/mla_attention.py:1087-1109)
+    for unquantised weights.  x ``[B, H, L]``, W_UV ``[H, L, V]``, out ``[B, H, V]`` or ``[B, H * V]``;
+    bf16 or fp16, one dtype; L and V multiples of 128."""
+    dev = _require_cuda(x, W_UV, out)
+    if x.dim() != 3 or W_UV.dim() != 3:
+        raise RuntimeError("mla_v_up_proj takes x [B, H, L] and W_UV [H, L, V]")
+    B, H, L = x.shape
+    V = W_UV.shape[2]
+    if tuple(W_UV.shape) != (H, L, V):
+        raise RuntimeError("W_UV must be [H, L, V]")
+    if out.dim() == 2:
+        if tuple(out.shape) != (B, H * V) or out.stride(1) != 1:
+            raise RuntimeError("out must be [B, H * V] with a contiguous last dim")
+        o_sb, o_sh = out.stride(0), V
+    else:
+        if tuple(out.shape) != (B, H, V) or out.stride(2) != 1:
+            raise RuntimeError("out must be [B, H, V] with a contiguous last dim")
+        o_sb, o_sh = out.stride(0), out.stride(1)
+    if not (x.dtype == W_UV.dtype == out.dtype):
+        raise RuntimeError("x, W_UV and out must share a dtype")
+    if x.stride(2) != 1 or W_UV.stride(2) != 1:
+        raise RuntimeError("last dims must be contiguous")
+    with _on_device(dev):
+        rc = _C.load().kvq_mla_v_up_proj(_ptr(out), o_sb, o_sh, _ptr(x), _dtype_code(x, "x"), x.stride(0), x.stride(1),
+                                         _ptr(W_UV), W_UV.stride(0), W_UV.stride(1), B, H, L, V, _stream(dev))
+    _C.check(rc, "mla_v_up_proj")
+
+
 def concat_mla_q(ql_nope: torch.Tensor, q_pe: torch.Tensor, q_out: torch.Tensor) -> None:
     """``q_out[..., :R] = ql_nope; q_out[..., R:] = q_pe``: the reference's ``ops.concat_mla_q``
     (csrc/libtorch_stable/cache_kernels.cu:1740-1783; call site

@@ -387,9 +387,9 @@ class Int8MLADecodeCaller:
     ``bmm(q_nope [N, B, P], W_UK_T [N, P, L])``, the decode, and the V up-projection
     ``bmm(o [N, B, L], W_UV [N, L, V])``.  The absorption runs inside the decode launch
     (``kvq_mla_decode_absorb_int8``): its product lands in the decode's int8 operand layout and is
-    never stored in the activation type.  The up-projection stays the library GEMM it is in the
-    reference and reads the decode's output as a strided view, without a transposed copy.  fp32
-    activations (not a serving dtype) take the two-step path ``absorb_q`` + ``forward_mqa``."""
+    never stored in the activation type.  The up-projection is ``kvq_mla_v_up_proj``, a stream of the
+    weights with the handful of decode rows as the MFMA's other operand.  fp32 activations (not a
+    serving dtype) take the library GEMMs and the two-step path ``absorb_q`` + ``forward_mqa``."""
 
     def __init__(self, impl: Int8MLAImpl, W_UK_T: torch.Tensor, W_UV: torch.Tensor) -> None:
         N, P, L = W_UK_T.shape
@@ -411,11 +411,20 @@ class Int8MLADecodeCaller:
         torch.bmm(q, self.W_UK_T, out=ql)
         return ql.transpose(0, 1)
 
-    def v_up_proj(self, x: torch.Tensor, out: torch.Tensor) -> None:
-        """``x [B, N, L]`` -> ``out [B, N * V]``."""
+    def v_up_proj_library(self, x: torch.Tensor, out: torch.Tensor) -> None:
+        """``x [B, N, L]`` -> ``out [B, N * V]`` as the library GEMM of the reference (strided views, no
+        transposed copies): fp32 activations, shapes the kernel does not take, and comparison."""
         x = x.view(-1, self.num_heads, self.kv_lora_rank).transpose(0, 1)
         out = out.view(-1, self.num_heads, self.v_head_dim)
         torch.bmm(x, self.W_UV, out=out.transpose(0, 1))
+
+    def v_up_proj(self, x: torch.Tensor, out: torch.Tensor) -> None:
+        """``x [B, N, L]`` -> ``out [B, N * V]``."""
+        if x.dtype == torch.float32 or self.kv_lora_rank % 128 != 0 or self.v_head_dim % 128 != 0:
+            self.v_up_proj_library(x, out)
+            return
+        ops.mla_v_up_proj(x.view(-1, self.num_heads, self.kv_lora_rank), self.W_UV,
+                          out.view(-1, self.num_heads, self.v_head_dim))
 
     def decode_absorbed(self, mqa_q_nope: torch.Tensor, mqa_q_pe: torch.Tensor, kv_cache: torch.Tensor, attn_metadata):
         """Absorption + decode in one launch; returns ``(o [B, N, L], lse [B, N])`` like ``forward_mqa``
