@@ -931,6 +931,7 @@ struct StreamKArgs {
   // != 0: the batch-invariant cutting (every sequence cut by its own length alone); the partial states then take
   // kFixedSpans slots per sequence and wg_info / seq_first_unit are not used
   int fixed_spans;
+  int setup_units;   // units a sequence is charged on the balanced work line before its tiles
 };
 
 // The decode kernel's fused cache update: the wave that owns kv head `hkv` of the run that holds a sequence's

@@ -21,13 +21,15 @@ __device__ __forceinline__ int wave_incl_scan(int v, int lane) {
   return v;
 }
 
-// Starting on a sequence (query row, first tile with nothing in flight, storing the state of the
-// one before) costs a workgroup about as long as one tile takes; the work line that is cut into
-// equal shares therefore charges every sequence this many units before its tiles.  Measured on
-// MI355X at batch 64, 1k..8k tokens: workgroups whose share crossed a sequence boundary ran 2.9 us
-// (one tile time) longer than the others and were the last to finish; with the charge they get
-// one tile less.
-constexpr int kSetupUnits = 1;
+// Starting on a sequence (query row, first tile with nothing in flight, folding and storing the state of the
+// one before) costs a workgroup 4 - 5 us, whatever the number of kv heads it serves; the work line that is cut into
+// equal shares therefore charges every sequence StreamKArgs::setup_units units before its tiles.  A unit is a
+// tile of the workgroup's run, and the 8 / HPW waves of a head take a run's tiles in turn, so a unit lasts
+// 2.9 us / (8 / HPW) and the charge grows with the waves per head (setup_units_for).  Measured on MI355X at batch 64,
+// 1k..8k tokens: with eight kv heads and no charge, workgroups whose share crossed a sequence boundary ran 2.9 us
+// (one tile time) longer than the others and were the last to finish; with one kv head and a charge of one unit
+// they ran 23.0 us against 18.2 us and the launch waited for them.
+constexpr int setup_units_for(int waves_per_head) { return waves_per_head == 1 ? 1 : 3 * waves_per_head / 2; }
 
 // Tiles of a decode sequence: those that hold a token of the row's window,
 // [window_first / 32, ceil(len / 32)).  0 for prefill sequences and empty ones.
@@ -62,15 +64,16 @@ __device__ __forceinline__ int fixed_span_count(int ntiles) {
 
 // Units a sequence takes on the work line: its setup charge, then one unit per tile.
 __device__ __forceinline__ int decode_units(const int32_t* seq_lens, const int32_t* cu, int s, int num_seqs,
-                                            int window) {
+                                            int window, int setup) {
   const int n = decode_tiles(seq_lens, cu, s, num_seqs, window);
-  return n > 0 ? n + kSetupUnits : 0;
+  return n > 0 ? n + setup : 0;
 }
 // Units of a sequence on the line the launch cuts: tiles + setup charge, or (FIXED) its spans.
 template <bool FIXED>
-__device__ __forceinline__ int line_units(const int32_t* seq_lens, const int32_t* cu, int s, int num_seqs, int window) {
+__device__ __forceinline__ int line_units(const int32_t* seq_lens, const int32_t* cu, int s, int num_seqs, int window,
+                                          int setup) {
   if constexpr (FIXED) return fixed_span_count(decode_tiles(seq_lens, cu, s, num_seqs, window));
-  else return decode_units(seq_lens, cu, s, num_seqs, window);
+  else return decode_units(seq_lens, cu, s, num_seqs, window, setup);
 }
 
 // The scans over the sequences work on chunks of 64 (one per lane).  Large batches take kScanBatch
@@ -87,7 +90,7 @@ __device__ __forceinline__ int64_t scan_total(const StreamKArgs& a, int lane) {
     int n[BATCH];
 #pragma unroll
     for (int j = 0; j < BATCH; ++j)
-      n[j] = line_units<FIXED>(a.seq_lens, a.cu_seqlens_q, base + kWave * j + lane, B, a.io.window);
+      n[j] = line_units<FIXED>(a.seq_lens, a.cu_seqlens_q, base + kWave * j + lane, B, a.io.window, a.setup_units);
 #pragma unroll
     for (int j = 0; j < BATCH; ++j) total += __builtin_amdgcn_readlane(wave_incl_scan(n[j], lane), 63);
   }
@@ -104,7 +107,7 @@ __device__ __forceinline__ void scan_locate(const StreamKArgs& a, int lane, int6
     int nn[BATCH];
 #pragma unroll
     for (int j = 0; j < BATCH; ++j)
-      nn[j] = line_units<FIXED>(a.seq_lens, a.cu_seqlens_q, base + kWave * j + lane, B, a.io.window);
+      nn[j] = line_units<FIXED>(a.seq_lens, a.cu_seqlens_q, base + kWave * j + lane, B, a.io.window, a.setup_units);
 #pragma unroll
     for (int j = 0; j < BATCH; ++j) {
       const int n = nn[j];
@@ -247,12 +250,13 @@ __global__ __launch_bounds__(512) void paged_decode_streamk_kernel(StreamKArgs a
 
   int64_t pos = lo;
   while (pos < hi && seq < B) {
-    const int units = __builtin_amdgcn_readfirstlane(decode_units(a.seq_lens, a.cu_seqlens_q, seq, B, a.io.window));
+    const int units = __builtin_amdgcn_readfirstlane(decode_units(a.seq_lens, a.cu_seqlens_q, seq, B, a.io.window, a.setup_units));
     if (units == 0) {
       ++seq;
       continue;
     }
-    const int ntiles = units - kSetupUnits;
+    const int setup = a.setup_units;
+    const int ntiles = units - setup;
     const int len = __builtin_amdgcn_readfirstlane(a.seq_lens[seq]);
     const int64_t row = a.cu_seqlens_q ? (int64_t)a.cu_seqlens_q[seq] : (int64_t)seq;
     if (info_seq < 0) {
@@ -261,13 +265,13 @@ __global__ __launch_bounds__(512) void paged_decode_streamk_kernel(StreamKArgs a
     }
     const int first = window_first(len, a.io.window);  // tokens before it are outside the window
     const int t0 = first / kTile;                      // the sequence's tile line starts at this tile
-    // units [pos, min(hi, end of the sequence)) of the line; the first kSetupUnits of a sequence
+    // units [pos, min(hi, end of the sequence)) of the line; the first setup_units of a sequence
     // stand for no tile
     const int u_begin = (int)(pos - seq_start);
     const int64_t rem = hi - seq_start;
     const int u_end = rem < units ? (int)rem : units;
-    const int t_begin = __builtin_amdgcn_readfirstlane(t0 + (u_begin > kSetupUnits ? u_begin - kSetupUnits : 0));
-    const int t_end = __builtin_amdgcn_readfirstlane(t0 + u_end - kSetupUnits);
+    const int t_begin = __builtin_amdgcn_readfirstlane(t0 + (u_begin > setup ? u_begin - setup : 0));
+    const int t_end = __builtin_amdgcn_readfirstlane(t0 + u_end - setup);
     if (t_begin < t_end)  // else: this share ends inside the setup charge and holds no tile
       process(seq, seq_start, row, len, first, t0, ntiles, t_begin, t_end, (int64_t)w + seq);
     pos = seq_start + u_end;
@@ -398,9 +402,9 @@ __global__ __launch_bounds__(256) void paged_decode_streamk_reduce_kernel(Stream
   const int64_t row = a.cu_seqlens_q ? a.cu_seqlens_q[seq] : seq;
   const int ntiles = (len + kTile - 1) / kTile - window_first(len, a.io.window) / kTile;   // a decode sequence with tiles
   // workgroup holding unit x: the largest w with floor(w*T/P) <= x; the sequence's tiles are units
-  // start + kSetupUnits .. start + kSetupUnits + ntiles - 1
-  const int w_first = (int)(((start + kSetupUnits + 1) * P - 1) / total);
-  const int w_last = (int)(((start + kSetupUnits + ntiles) * P - 1) / total);
+  // start + setup_units .. start + setup_units + ntiles - 1
+  const int w_first = (int)(((start + a.setup_units + 1) * P - 1) / total);
+  const int w_last = (int)(((start + a.setup_units + ntiles) * P - 1) / total);
   if (w_first == w_last) return;  // not cut
   const int span = w_last - w_first + 1;
   if (span > 16) {
@@ -561,9 +565,9 @@ __global__ __launch_bounds__(256) void paged_decode_streamk_reduce_by_seq_kernel
   }
   const int P = active_workgroups(total, a.num_wg);
   // workgroup holding unit x: the largest w with floor(w*T/P) <= x; the sequence's tiles are units
-  // start + kSetupUnits .. start + kSetupUnits + ntiles - 1
-  const int w_first = (int)(((start + kSetupUnits + 1) * P - 1) / total);
-  const int w_last = (int)(((start + kSetupUnits + ntiles) * P - 1) / total);
+  // start + setup_units .. start + setup_units + ntiles - 1
+  const int w_first = (int)(((start + a.setup_units + 1) * P - 1) / total);
+  const int w_last = (int)(((start + a.setup_units + ntiles) * P - 1) / total);
   if (w_first == w_last) return;  // written directly by the main kernel
 
   // pass 1: every lane takes one workgroup's (m, l); the wave agrees on the max and the weights
@@ -697,8 +701,8 @@ __global__ __launch_bounds__(256) void paged_decode_streamk_reduce_split4_kernel
     return;
   }
   const int P = active_workgroups(total, a.num_wg);
-  const int w_first = (int)(((start + kSetupUnits + 1) * P - 1) / total);
-  const int w_last = (int)(((start + kSetupUnits + ntiles) * P - 1) / total);
+  const int w_first = (int)(((start + a.setup_units + 1) * P - 1) / total);
+  const int w_last = (int)(((start + a.setup_units + ntiles) * P - 1) / total);
   if (w_first == w_last) return;  // written directly by the main kernel
   // this wave's slots: w_first + part + 4 i, i = 0 .. n - 1 (n = 0 for a span shorter than its number)
   const int span = w_last - w_first + 1;
@@ -812,9 +816,11 @@ __global__ __launch_bounds__(WPW * 64) void paged_decode_v2_kernel(V2Args a) {
 
 // out = sum_j w_j tmp_out_j / sum_j w_j, w_j = exp_sums_j * exp(max_logits_j - max).
 template <int D, int QDT>
-static int launch_streamk(const StreamKArgs& a, hipStream_t s) {
-  const int hkv = a.io.g.num_kv_heads;
+static int launch_streamk(const StreamKArgs& args, hipStream_t s) {
+  const int hkv = args.io.g.num_kv_heads;
   const int hpw = heads_per_wg(hkv);
+  StreamKArgs a = args;
+  a.setup_units = setup_units_for(8 / hpw);
   dim3 grid(a.num_wg, (hkv + hpw - 1) / hpw);
 #define KVQ_SK_CODE(H, C, CODE)                                                                                   \
   do {                                                                                                            \
