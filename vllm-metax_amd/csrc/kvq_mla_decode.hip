@@ -330,6 +330,15 @@ __global__ __launch_bounds__(256) void mla_absorb_q_kernel(MlaAbsorbArgs a) {
       for (int t = 0; t < NB; ++t) acc[t][i] = mfma16<QDT>(wt, qop[t], acc[t][i]);
     }
   };
+  // wave t also brings the rope dims 16 g .. 16 g + 15 of tile t: requested with everything else, so that the
+  // kernel stays one trip to memory long
+  u32x4 pe_raw[2];
+  {
+    const int t = wave < NB ? wave : 0;
+    const uint16_t* pp = static_cast<const uint16_t*>(a.q_pe) + (int64_t)brow[t] * a.pe_sb + (int64_t)hsrc * a.pe_sh + 16 * g;
+#pragma unroll
+    for (int h = 0; h < 2; ++h) pe_raw[h] = *reinterpret_cast<const u32x4_a4*>(pp + 8 * h);
+  }
   if constexpr (KSTEPS > 0) {
     // every load of the kernel first, then the arithmetic
     u32x4 rows[KSTEPS][8], qop[KSTEPS][NB];
@@ -354,13 +363,11 @@ __global__ __launch_bounds__(256) void mla_absorb_q_kernel(MlaAbsorbArgs a) {
     }
   }
   // lane (sequence c, quarter g) of wave w holds dims 128 w + 32 g + 8 r + i of its sequence in acc[t][i][r]
-  float pe[16];   // wave t also brings the rope dims 16 g .. 16 g + 15 of tile t
+  float pe[16];
   {
-    const int t = wave < NB ? wave : 0;
-    const uint16_t* pp = static_cast<const uint16_t*>(a.q_pe) + (int64_t)brow[t] * a.pe_sb + (int64_t)hsrc * a.pe_sh + 16 * g;
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
-      const u32x4 v = *reinterpret_cast<const u32x4_a4*>(pp + 8 * h);
+      const u32x4 v = pe_raw[h];
 #pragma unroll
       for (int w = 0; w < 4; ++w) {
         const uint32_t e = v[w];
