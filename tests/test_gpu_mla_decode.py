@@ -376,7 +376,9 @@ def test_decode_caller_makes_no_library_gemm(gpu_device, monkeypatch):
     (3, 16, 512, 128),       # a tensor-parallel shard, a tile of 3 live rows
     (17, 20, 512, 128),      # a second sequence tile of one row; heads that do not fill the last XCD round
     (1, 5, 256, 256),        # another latent width (run-time step count), two blocks of output dims
-    (70, 9, 384, 128),
+    (70, 9, 384, 128),       # 5 tiles of 16 sequences: two per workgroup
+    (130, 16, 512, 128),
+    (300, 8, 512, 128),      # 19 tiles: four per workgroup, the last workgroup with three of which one is partial
 ])
 def test_v_up_proj_matches_the_fp32_product(gpu_device, dtype, B, N, L, V):
     """kvq_mla_v_up_proj against the product in fp32 (the reference's _v_up_proj is a bmm over [N, B, L] x

@@ -3,8 +3,8 @@
 // W_UV [N, L, V], back to [B, N * V]) for the handful of rows a decode step has.
 //
 // The product is a stream of the weights (128 KB per head at L = 512, V = 128, next to 16 KB of x for 16
-// sequences): the kernel is one round trip to memory long.  Workgroup = (head, 16 sequences, 128 output
-// dims), 4 waves, wave w contracting over the latent dims L/4 * w .. L/4 * (w + 1) - 1; every load of a wave
+// sequences): the kernel is one round trip to memory long.  Workgroup = (head, 16 sequences -- 32 or 64 in
+// large batches --, 128 output dims), 4 waves, wave w contracting over the latent dims L/4 * w .. L/4 * (w + 1) - 1; every load of a wave
 // is issued before its first product, the four partial sums meet in LDS and wave 0 stores the result.
 // The product is taken transposed, out^T = W^T x^T, as the absorption kernel takes its own: B = x rows (lane =
 // sequence, 8 consecutive latent dims: one 16-byte load), A = W^T needs 8 latent dims of one output dim per
@@ -31,8 +31,10 @@ struct MlaUpProjArgs {
 constexpr int kXcds = 8;
 
 // KSTEPS = L / 128 when known at compile time (every load of the wave in flight at once), 0 = read it from
-// the arguments.
-template <int DT, int KSTEPS>
+// the arguments.  NB = tiles of 16 sequences per workgroup: the weights a wave has loaded and transposed serve NB
+// products, so a large batch reads them NB times less often through the L2 (NB = 1 up to 64 sequences, where the
+// launch should fill the chip; 2 up to 256; 4 beyond).
+template <int DT, int KSTEPS, int NB>
 __global__ __launch_bounds__(256) void mla_v_up_proj_kernel(MlaUpProjArgs a) {
   __shared__ floatx4 red[3][8][64];
   const int lane = threadIdx.x & 63;
@@ -44,16 +46,22 @@ __global__ __launch_bounds__(256) void mla_v_up_proj_kernel(MlaUpProjArgs a) {
   const int head = (q / per_head) * kXcds + blockIdx.x % kXcds;
   if (head >= a.num_heads) return;   // uniform over the workgroup
   const int rem = q % per_head;
-  const int n0 = (rem / a.seq_tiles) * 128, b0 = (rem % a.seq_tiles) * 16;
+  const int n0 = (rem / a.seq_tiles) * 128, b0 = (rem % a.seq_tiles) * (16 * NB);
   const int ksteps = KSTEPS > 0 ? KSTEPS : a.ksteps;
   const int k0 = wave * ksteps * 32;
-  const int brow = min(b0 + c, a.num_seqs - 1);   // rows past the end: a copy, not written
   const uint16_t* wp = static_cast<const uint16_t*>(a.w) + (int64_t)head * a.w_sh + (int64_t)(k0 + 8 * g) * a.w_sl + n0 + 8 * c;
-  const uint16_t* xp = static_cast<const uint16_t*>(a.x) + (int64_t)brow * a.x_sb + (int64_t)head * a.x_sh + k0 + 8 * g;
-  floatx4 acc[8];
+  const uint16_t* xp[NB];
 #pragma unroll
-  for (int i = 0; i < 8; ++i) acc[i] = (floatx4){0.f, 0.f, 0.f, 0.f};
-  auto step = [&](const u32x4 (&rows)[8], const u32x4& xop) {
+  for (int t = 0; t < NB; ++t) {
+    const int brow = min(b0 + 16 * t + c, a.num_seqs - 1);   // rows past the end: a copy, not written
+    xp[t] = static_cast<const uint16_t*>(a.x) + (int64_t)brow * a.x_sb + (int64_t)head * a.x_sh + k0 + 8 * g;
+  }
+  floatx4 acc[NB][8];
+#pragma unroll
+  for (int t = 0; t < NB; ++t)
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[t][i] = (floatx4){0.f, 0.f, 0.f, 0.f};
+  auto step = [&](const u32x4 (&rows)[8], const u32x4 (&xop)[NB]) {
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       const uint32_t sel = (i & 1) ? kPermHighHalves : kPermLowHalves;
@@ -62,14 +70,16 @@ __global__ __launch_bounds__(256) void mla_v_up_proj_kernel(MlaUpProjArgs a) {
       wt.y = perm(rows[3][i >> 1], rows[2][i >> 1], sel);
       wt.z = perm(rows[5][i >> 1], rows[4][i >> 1], sel);
       wt.w = perm(rows[7][i >> 1], rows[6][i >> 1], sel);
-      acc[i] = mfma16<DT>(wt, xop, acc[i]);
+#pragma unroll
+      for (int t = 0; t < NB; ++t) acc[t][i] = mfma16<DT>(wt, xop[t], acc[t][i]);
     }
   };
   if constexpr (KSTEPS > 0) {
-    u32x4 rows[KSTEPS][8], xop[KSTEPS];
+    u32x4 rows[KSTEPS][8], xop[KSTEPS][NB];
 #pragma unroll
     for (int s = 0; s < KSTEPS; ++s) {
-      xop[s] = *reinterpret_cast<const u32x4_a4*>(xp + 32 * s);
+#pragma unroll
+      for (int t = 0; t < NB; ++t) xop[s][t] = *reinterpret_cast<const u32x4_a4*>(xp[t] + 32 * s);
 #pragma unroll
       for (int j = 0; j < 8; ++j) rows[s][j] = *reinterpret_cast<const u32x4*>(wp + (int64_t)(32 * s + j) * a.w_sl);
     }
@@ -78,33 +88,41 @@ __global__ __launch_bounds__(256) void mla_v_up_proj_kernel(MlaUpProjArgs a) {
     for (int s = 0; s < KSTEPS; ++s) step(rows[s], xop[s]);
   } else {
     for (int s = 0; s < ksteps; ++s) {
-      u32x4 rows[8];
+      u32x4 rows[8], xop[NB];
 #pragma unroll
       for (int j = 0; j < 8; ++j) rows[j] = *reinterpret_cast<const u32x4*>(wp + (int64_t)(32 * s + j) * a.w_sl);
-      const u32x4 xop = *reinterpret_cast<const u32x4_a4*>(xp + 32 * s);
+#pragma unroll
+      for (int t = 0; t < NB; ++t) xop[t] = *reinterpret_cast<const u32x4_a4*>(xp[t] + 32 * s);
       step(rows, xop);
     }
   }
-  // lane (sequence c, quarter g) holds output dims n0 + 32 g + 8 r + i of its sequence in acc[i][r]
-  if (wave > 0) {
+  // lane (sequence c, quarter g) holds output dims n0 + 32 g + 8 r + i of its sequence of tile t in acc[t][i][r];
+  // the tiles pass through the one LDS area in turn
 #pragma unroll
-    for (int i = 0; i < 8; ++i) red[wave - 1][i][lane] = acc[i];
-  }
-  __syncthreads();
-  if (wave > 0 || b0 + c >= a.num_seqs) return;
+  for (int t = 0; t < NB; ++t) {
+    if (t > 0) __syncthreads();   // wave 0 has read tile t - 1
+    if (wave > 0) {
 #pragma unroll
-  for (int w = 0; w < 3; ++w)
+      for (int i = 0; i < 8; ++i) red[wave - 1][i][lane] = acc[t][i];
+    }
+    __syncthreads();
+    const int b = b0 + 16 * t + c;
+    if (wave == 0 && b < a.num_seqs) {
 #pragma unroll
-    for (int i = 0; i < 8; ++i) acc[i] += red[w][i][lane];
-  uint16_t* op = static_cast<uint16_t*>(a.out) + (int64_t)(b0 + c) * a.o_sb + (int64_t)head * a.o_sh + n0 + 32 * g;
+      for (int w = 0; w < 3; ++w)
 #pragma unroll
-  for (int r = 0; r < 4; ++r) {
-    u32x4 v;
-    v.x = pack2<DT>(acc[0][r], acc[1][r]);
-    v.y = pack2<DT>(acc[2][r], acc[3][r]);
-    v.z = pack2<DT>(acc[4][r], acc[5][r]);
-    v.w = pack2<DT>(acc[6][r], acc[7][r]);
-    *reinterpret_cast<u32x4*>(op + 8 * r) = v;
+        for (int i = 0; i < 8; ++i) acc[t][i] += red[w][i][lane];
+      uint16_t* op = static_cast<uint16_t*>(a.out) + (int64_t)b * a.o_sb + (int64_t)head * a.o_sh + n0 + 32 * g;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        u32x4 v;
+        v.x = pack2<DT>(acc[t][0][r], acc[t][1][r]);
+        v.y = pack2<DT>(acc[t][2][r], acc[t][3][r]);
+        v.z = pack2<DT>(acc[t][4][r], acc[t][5][r]);
+        v.w = pack2<DT>(acc[t][6][r], acc[t][7][r]);
+        *reinterpret_cast<u32x4*>(op + 8 * r) = v;
+      }
+    }
   }
 }
 
@@ -141,14 +159,22 @@ int kvq_mla_v_up_proj(void* out, int64_t out_stride_b, int64_t out_stride_h, con
   a.o_sh = out_stride_h;
   a.num_seqs = num_seqs;
   a.num_heads = num_heads;
-  a.seq_tiles = (num_seqs + 15) / 16;
+  const int tiles16 = (num_seqs + 15) / 16;
+  const int nb = tiles16 <= 4 ? 1 : (tiles16 <= 16 ? 2 : 4);
+  a.seq_tiles = (tiles16 + nb - 1) / nb;
   a.v_blocks = v_head_dim / 128;
   a.ksteps = kv_lora_rank / 128;
   const int64_t blocks = (int64_t)((num_heads + kXcds - 1) / kXcds) * kXcds * a.seq_tiles * a.v_blocks;
   KVQ_REQUIRE(blocks < (1ll << 31), "%s: %lld workgroups do not fit a grid", op, (long long)blocks);
   hipStream_t s = as_stream(stream);
   const dim3 grid((unsigned)blocks), block(256);
-#define KVQ_UPPROJ(T, K) hipLaunchKernelGGL((mla_v_up_proj_kernel<T, K>), grid, block, 0, s, a)
+#define KVQ_UPPROJ_NB(T, K, N) hipLaunchKernelGGL((mla_v_up_proj_kernel<T, K, N>), grid, block, 0, s, a)
+#define KVQ_UPPROJ(T, K)              \
+  do {                                \
+    if (nb == 1) KVQ_UPPROJ_NB(T, K, 1);      \
+    else if (nb == 2) KVQ_UPPROJ_NB(T, K, 2); \
+    else KVQ_UPPROJ_NB(T, K, 4);              \
+  } while (0)
   if (dtype == KVQ_BF16) {
     if (a.ksteps == 4) KVQ_UPPROJ(KVQ_BF16, 4);
     else KVQ_UPPROJ(KVQ_BF16, 0);
@@ -157,6 +183,7 @@ int kvq_mla_v_up_proj(void* out, int64_t out_stride_b, int64_t out_stride_h, con
     else KVQ_UPPROJ(KVQ_F16, 0);
   }
 #undef KVQ_UPPROJ
+#undef KVQ_UPPROJ_NB
   return check_hip(hipGetLastError(), "mla_v_up_proj launch");
 }
 
