@@ -316,6 +316,7 @@ def test_mla_decode_caller_absorb_decode_up_proj(gpu_device):
     (20, 64, [5, 0, 95, 1000, 31, 32] * 7),      # 42 sequences: a second block of 32, a last tile of 10; 20 heads: a group of 4
     (128, 128, [70, 0, 130, 33] * 65),           # 260 sequences: one split each, the decode kernel stores the result itself
     (16, 128, [50, 120, 1, 0, 64] * 60),         # the same through the one-head-tile kernel
+    (32, 128, [40, 7, 90] * 30),                 # 90 sequences: two tiles of 16 per absorption workgroup
 ])
 def test_mla_decode_with_fused_absorption(gpu_device, dtype, N, Pn, ctx):
     """kvq_mla_decode_absorb_int8: q_nope x W_UK_T on the MFMA inside the launch, written as the decode's int8

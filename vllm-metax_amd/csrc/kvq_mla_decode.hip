@@ -268,7 +268,11 @@ __device__ __forceinline__ void mla_seq_split_of_block(int num_seqs, int num_spl
 // the prefill attention does for V.  Block i of a wave's output then holds dims 8 lane + i: a lane ends
 // with 32 consecutive dims of its own sequence, i.e. two of the 16-byte pieces of the operand layout.
 // The row maximum (all 576 dims, rope included) crosses the four waves through LDS.
-constexpr int kMlaAbsorbTiles = 1;   // tiles of 16 sequences per workgroup (at most 4: wave t brings tile t's rope dims)
+// Tiles of 16 sequences per workgroup (at most 4: wave t brings tile t's rope dims): the weights a wave has loaded
+// and transposed serve all of them.  One tile while that fills the chip; a workgroup is one trip to memory long
+// whatever its tiles, so a large batch takes fewer rounds of workgroups with more of them (library GEMM of the same
+// product at 128 heads: 10.5 / 15.3 / 26.0 us at 128 / 256 / 512 sequences; one tile per workgroup: 17.7 / 28.8 / 51.9 us).
+__host__ __device__ constexpr int mla_absorb_tiles(int num_seqs) { return num_seqs <= 64 ? 1 : (num_seqs <= 128 ? 2 : 4); }
 struct MlaAbsorbArgs {
   const void* q_nope;   // [B, H, P]
   int64_t qn_sb, qn_sh;
@@ -279,14 +283,13 @@ struct MlaAbsorbArgs {
   uint8_t* q_ops;
   float* q_scale;
   int head_groups, num_heads, num_seqs, ksteps;   // ksteps = P / 32
-  int seq_tiles, group_major;                     // tiles of 16 * kMlaAbsorbTiles sequences; how workgroups are numbered
+  int seq_tiles, group_major;                     // tiles of 16 * NB sequences; how workgroups are numbered
 };
 
 // KSTEPS = P / 32 when known at compile time (the loop is unrolled and every load of W is in flight at
 // once: the kernel is one memory round trip long), 0 = read it from the arguments.
-template <int QDT, int KSTEPS>
+template <int QDT, int KSTEPS, int NB>
 __global__ __launch_bounds__(256) void mla_absorb_q_kernel(MlaAbsorbArgs a) {
-  constexpr int NB = kMlaAbsorbTiles;
   __shared__ float part_max[4][NB][16];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -1525,10 +1528,17 @@ static int mla_decode_run(const char* op, void* out, int out_dtype, float* lse, 
     absorb->head_groups = head_groups;
     absorb->num_heads = num_heads;
     absorb->num_seqs = num_seqs;
-    absorb->seq_tiles = (num_seqs + 16 * kMlaAbsorbTiles - 1) / (16 * kMlaAbsorbTiles);
+    const int atiles = mla_absorb_tiles(num_seqs);
+    absorb->seq_tiles = (num_seqs + 16 * atiles - 1) / (16 * atiles);
     absorb->group_major = head_groups % 8 == 0;
     dim3 agrid(head_groups * 16 * absorb->seq_tiles);
-#define KVQ_MLAA(T, K) hipLaunchKernelGGL((mla_absorb_q_kernel<T, K>), agrid, dim3(256), 0, s, *absorb)
+#define KVQ_MLAA_NB(T, K, N) hipLaunchKernelGGL((mla_absorb_q_kernel<T, K, N>), agrid, dim3(256), 0, s, *absorb)
+#define KVQ_MLAA(T, K)                        \
+  do {                                        \
+    if (atiles == 1) KVQ_MLAA_NB(T, K, 1);      \
+    else if (atiles == 2) KVQ_MLAA_NB(T, K, 2); \
+    else KVQ_MLAA_NB(T, K, 4);                  \
+  } while (0)
     if (q_dtype == KVQ_BF16) {
       if (absorb->ksteps == 4) KVQ_MLAA(KVQ_BF16, 4);
       else KVQ_MLAA(KVQ_BF16, 0);
@@ -1537,6 +1547,7 @@ static int mla_decode_run(const char* op, void* out, int out_dtype, float* lse, 
       else KVQ_MLAA(KVQ_F16, 0);
     }
 #undef KVQ_MLAA
+#undef KVQ_MLAA_NB
   } else if (q_dtype != KVQ_F32 && q_dtype != KVQ_BF16 && q_dtype != KVQ_F16) {
     return fail(KVQ_EINVAL, "%s: unknown q_dtype %d", op, q_dtype);
   }   // without absorption the decode kernels quantise the query themselves

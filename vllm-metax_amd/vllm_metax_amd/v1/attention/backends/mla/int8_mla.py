@@ -422,6 +422,11 @@ class Int8MLADecodeCaller:
     # replays at 128 heads, 5.8 against 8.8 us at 32 rows, 15.3 against 16.4 us at 256, 32.8 against 19.5 us at 512
     # (there the activations, not the weights, are the larger stream); at 16 heads it is ahead or level up to 1024.
     KERNEL_MAX_ROWS_X_HEADS = 256 * 128
+    # Rows x heads up to which the absorption inside the decode launch is level with or ahead of the library GEMM
+    # + decode (whole chain, 128 heads: 78.4 against 77.4 us at 64 rows, 129 against 118 us at 256; 16 heads:
+    # 33.9 against 47.2 us at 64 rows, 89.8 against 90.6 us at 512, 117.4 against 110.8 us at 1024): the kernel
+    # writes the int8 operands as 16-byte pieces of lines that 16 heads share, which a large batch pays for.
+    ABSORB_MAX_ROWS_X_HEADS = 64 * 128
 
     def v_up_proj(self, x: torch.Tensor, out: torch.Tensor) -> None:
         """``x [B, N, L]`` -> ``out [B, N * V]``."""
@@ -455,7 +460,7 @@ class Int8MLADecodeCaller:
                        attn_metadata, out: torch.Tensor):
         """q_nope ``[B, N, P]``, q_pe ``[B, N, rope]`` (already rotated), writes ``out [B, N * V]``;
         returns the decode's ``lse [B, N]``."""
-        if mqa_q_nope.dtype == torch.float32:
+        if mqa_q_nope.dtype == torch.float32 or mqa_q_nope.shape[0] * self.num_heads > self.ABSORB_MAX_ROWS_X_HEADS:
             attn_out, lse = self.impl.forward_mqa((self.absorb_q(mqa_q_nope), mqa_q_pe), kv_cache, attn_metadata)
         else:
             attn_out, lse = self.decode_absorbed(mqa_q_nope, mqa_q_pe, kv_cache, attn_metadata)
