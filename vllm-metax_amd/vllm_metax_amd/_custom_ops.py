@@ -1001,6 +1001,8 @@ def mla_v_up_proj(x: torch.Tensor, W_UV: torch.Tensor, out: torch.Tensor) -> Non
         raise RuntimeError("x, W_UV and out must share a dtype")
     if x.stride(2) != 1 or W_UV.stride(2) != 1:
         raise RuntimeError("last dims must be contiguous")
+    if B == 0:
+        return
     with _on_device(dev):
         rc = _C.load().kvq_mla_v_up_proj(_ptr(out), o_sb, o_sh, _ptr(x), _dtype_code(x, "x"), x.stride(0), x.stride(1),
                                          _ptr(W_UV), W_UV.stride(0), W_UV.stride(1), B, H, L, V, _stream(dev))
