@@ -317,6 +317,7 @@ def test_mla_decode_caller_absorb_decode_up_proj(gpu_device):
     (128, 128, [70, 0, 130, 33] * 65),           # 260 sequences: one split each, the decode kernel stores the result itself
     (16, 128, [50, 120, 1, 0, 64] * 60),         # the same through the one-head-tile kernel
     (32, 128, [40, 7, 90] * 30),                 # 90 sequences: two tiles of 16 per absorption workgroup
+    (256, 128, [100, 33, 70]),                   # 16 head groups: two of them per XCD in the absorption's numbering
 ])
 def test_mla_decode_with_fused_absorption(gpu_device, dtype, N, Pn, ctx):
     """kvq_mla_decode_absorb_int8: q_nope x W_UK_T on the MFMA inside the launch, written as the decode's int8
@@ -380,6 +381,7 @@ def test_decode_caller_makes_no_library_gemm(gpu_device, monkeypatch):
     (70, 9, 384, 128),       # 5 tiles of 16 sequences: two per workgroup
     (130, 16, 512, 128),
     (300, 8, 512, 128),      # 19 tiles: four per workgroup, the last workgroup with three of which one is partial
+    (40, 256, 512, 128),
 ])
 def test_v_up_proj_matches_the_fp32_product(gpu_device, dtype, B, N, L, V):
     """kvq_mla_v_up_proj against the product in fp32 (the reference's _v_up_proj is a bmm over [N, B, L] x
