@@ -73,7 +73,9 @@ struct MlaArgs {
   uint16_t* part_o;
   float* part_lse;
   // Q as the int8 MFMA wants it (written by mla_absorb_q_kernel, read by every split of a sequence):
-  // q_ops [B, ceil(H/16)][18 operands][64 lanes][16 bytes], q_scale [B, 16 * ceil(H/16)] = s1 per head.
+  // q_ops [B, ceil(H/16)][18 operands][64 slots][16 bytes], lane (c = head, g)'s piece in slot 4 c + g (a head's four
+  // pieces together: the absorption kernel, a workgroup per head, writes 64 contiguous bytes per operand);
+  // q_scale [B, 16 * ceil(H/16)] = s1 per head.
   uint8_t* q_ops;
   float* q_scale;
   int head_groups;  // ceil(H / 16)
@@ -409,7 +411,7 @@ __global__ __launch_bounds__(256) void mla_absorb_q_kernel(MlaAbsorbArgs a) {
     amax = head_ok ? fminf(amax, 3.0e38f) : 0.f;   // heads past the end contribute zero columns
     const float s1 = amax > 0.f ? amax / kMlaQ1Max : 1.0f;
     const int64_t qblock = (int64_t)b * a.head_groups + hgroup;
-    u32x4* qdst = reinterpret_cast<u32x4*>(a.q_ops + qblock * (kMlaQOps * kWave * 16)) + hc;
+    u32x4* qdst = reinterpret_cast<u32x4*>(a.q_ops + qblock * (kMlaQOps * kWave * 16)) + 4 * hc;   // a head's four pieces of an operand lie together
     // the lane's 32 dims are the 16-dim pieces u = 0, 1: k-step kk = 2 w + g / 2, piece 2 (g % 2) + u of it
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
@@ -419,14 +421,14 @@ __global__ __launch_bounds__(256) void mla_absorb_q_kernel(MlaAbsorbArgs a) {
       u32x4 ta, tb;
       mla_two_int8_terms(f, s1, head_ok, ta, tb);
       const int kk = 2 * wave + (g >> 1), piece = 2 * (g & 1) + u;
-      qdst[(2 * kk) * kWave + 16 * piece] = ta;
-      qdst[(2 * kk + 1) * kWave + 16 * piece] = tb;
+      qdst[(2 * kk) * kWave + piece] = ta;
+      qdst[(2 * kk + 1) * kWave + piece] = tb;
     }
     if (wave == t) {
       u32x4 ta, tb;
       mla_two_int8_terms(pe, s1, head_ok, ta, tb);
-      qdst[(2 * (kMlaKSteps8 - 1)) * kWave + 16 * g] = ta;
-      qdst[(2 * (kMlaKSteps8 - 1) + 1) * kWave + 16 * g] = tb;
+      qdst[(2 * (kMlaKSteps8 - 1)) * kWave + g] = ta;
+      qdst[(2 * (kMlaKSteps8 - 1) + 1) * kWave + g] = tb;
       if (g == 0) a.q_scale[qblock * 16 + hc] = s1;
     }
   }
@@ -591,7 +593,7 @@ __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
   if (owner) {
     if constexpr (QDT < 0) {
       const int64_t qblock = (int64_t)seq * a.head_groups + hgroup;
-      const u32x4* qsrc = reinterpret_cast<const u32x4*>(a.q_ops + qblock * (kMlaQOps * kWave * 16)) + lane;
+      const u32x4* qsrc = reinterpret_cast<const u32x4*>(a.q_ops + qblock * (kMlaQOps * kWave * 16)) + (4 * c + g);
       u32x4 raw[kMlaQOps];
 #pragma unroll
       for (int op = 0; op < kMlaQOps; ++op) raw[op] = qsrc[op * kWave];
@@ -1015,7 +1017,7 @@ __global__ __launch_bounds__(kMlaSmallThreads) void mla_decode_small_kernel(MlaA
   MlaQRaw<(QDT < 0 ? KVQ_BF16 : QDT)> qraw[kMine];
   const bool head_ok = c < a.num_heads;
   if constexpr (QDT < 0) {
-    const u32x4* qsrc = reinterpret_cast<const u32x4*>(a.q_ops + qblock * (kMlaQOps * kWave * 16)) + lane;
+    const u32x4* qsrc = reinterpret_cast<const u32x4*>(a.q_ops + qblock * (kMlaQOps * kWave * 16)) + (4 * c + g);
 #pragma unroll
     for (int op = 0; op < kMlaQOps; ++op) qreg[op] = __builtin_bit_cast(i32x4, qsrc[op * kWave]);
     s1 = a.q_scale[qblock * 16 + c];
