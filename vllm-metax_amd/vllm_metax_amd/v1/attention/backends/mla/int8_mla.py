@@ -423,10 +423,10 @@ class Int8MLADecodeCaller:
     # (there the activations, not the weights, are the larger stream); at 16 heads it is ahead or level up to 1024.
     KERNEL_MAX_ROWS_X_HEADS = 256 * 128
     # Rows x heads up to which the absorption inside the decode launch is level with or ahead of the library GEMM
-    # + decode (whole chain, 128 heads: 78.4 against 77.4 us at 64 rows, 129 against 118 us at 256; 16 heads:
-    # 33.9 against 47.2 us at 64 rows, 89.8 against 90.6 us at 512, 117.4 against 110.8 us at 1024): the kernel
-    # writes the int8 operands as 16-byte pieces of lines that 16 heads share, which a large batch pays for.
-    ABSORB_MAX_ROWS_X_HEADS = 64 * 128
+    # + decode (whole chain, 128 heads: 78.1 against 78.4 us at 64 rows, 116.9 against 116.2 us at 128, 124.9 against
+    # 118.2 us at 256; 16 heads: 32.7 against 44.7 us at 64 rows, 107.6 against 110.2 us at 1024): the kernel writes
+    # the int8 operands as 64-byte pieces of lines that two heads share, which a large batch of many heads pays for.
+    ABSORB_MAX_ROWS_X_HEADS = 128 * 128
 
     def v_up_proj(self, x: torch.Tensor, out: torch.Tensor) -> None:
         """``x [B, N, L]`` -> ``out [B, N * V]``."""
