@@ -380,7 +380,7 @@ def test_decode_caller_makes_no_library_gemm(gpu_device, monkeypatch):
     (1, 5, 256, 256),        # another latent width (run-time step count), two blocks of output dims
     (70, 9, 384, 128),       # 5 tiles of 16 sequences: two per workgroup
     (130, 16, 512, 128),
-    (300, 8, 512, 128),      # 19 tiles: four per workgroup, the last workgroup with three of which one is partial
+    (300, 8, 512, 128),      # 19 tiles: the last workgroup with one, partial
     (40, 256, 512, 128),
 ])
 def test_v_up_proj_matches_the_fp32_product(gpu_device, dtype, B, N, L, V):

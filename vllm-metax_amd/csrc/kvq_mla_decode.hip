@@ -270,11 +270,12 @@ __device__ __forceinline__ void mla_seq_split_of_block(int num_seqs, int num_spl
 // the prefill attention does for V.  Block i of a wave's output then holds dims 8 lane + i: a lane ends
 // with 32 consecutive dims of its own sequence, i.e. two of the 16-byte pieces of the operand layout.
 // The row maximum (all 576 dims, rope included) crosses the four waves through LDS.
-// Tiles of 16 sequences per workgroup (at most 4: wave t brings tile t's rope dims): the weights a wave has loaded
-// and transposed serve all of them.  One tile while that fills the chip; a workgroup is one trip to memory long
-// whatever its tiles, so a large batch takes fewer rounds of workgroups with more of them (library GEMM of the same
-// product at 128 heads: 10.5 / 15.3 / 26.0 us at 128 / 256 / 512 sequences; one tile per workgroup: 17.7 / 28.8 / 51.9 us).
-__host__ __device__ constexpr int mla_absorb_tiles(int num_seqs) { return num_seqs <= 64 ? 1 : (num_seqs <= 128 ? 2 : 4); }
+// Tiles of 16 sequences per workgroup (the kernel takes up to 4: wave t brings tile t's rope dims): the weights a wave
+// has loaded and transposed serve all of them.  One tile while that fills the chip, two beyond 64 sequences; with
+// four, a workgroup's registers leave one workgroup per CU and it measured slower (library GEMM of the same product
+// at 128 heads: 10.5 / 15.3 / 26.0 us at 128 / 256 / 512 sequences; one tile: 17.7 / 28.8 / 51.9 us; two tiles and
+// the operand slots of MlaArgs::q_ops: 13.5 / 20.4 / 35.7 us; four tiles: 23.1 / 41.5 us at 256 / 512).
+__host__ __device__ constexpr int mla_absorb_tiles(int num_seqs) { return num_seqs <= 64 ? 1 : 2; }
 struct MlaAbsorbArgs {
   const void* q_nope;   // [B, H, P]
   int64_t qn_sb, qn_sh;
@@ -1538,8 +1539,7 @@ static int mla_decode_run(const char* op, void* out, int out_dtype, float* lse, 
 #define KVQ_MLAA(T, K)                        \
   do {                                        \
     if (atiles == 1) KVQ_MLAA_NB(T, K, 1);      \
-    else if (atiles == 2) KVQ_MLAA_NB(T, K, 2); \
-    else KVQ_MLAA_NB(T, K, 4);                  \
+    else KVQ_MLAA_NB(T, K, 2);                  \
   } while (0)
     if (q_dtype == KVQ_BF16) {
       if (absorb->ksteps == 4) KVQ_MLAA(KVQ_BF16, 4);

@@ -419,7 +419,7 @@ class Int8MLADecodeCaller:
         torch.bmm(x, self.W_UV, out=out.transpose(0, 1))
 
     # Rows x heads up to which the weight stream (kvq_mla_v_up_proj) beats the library GEMM: measured through graph
-    # replays at 128 heads, 5.8 against 8.8 us at 32 rows, 15.3 against 16.4 us at 256, 32.8 against 19.5 us at 512
+    # replays at 128 heads, 5.9 against 8.8 us at 32 rows, 15.5 against 16.6 us at 256, 26.6 against 19.5 us at 512
     # (there the activations, not the weights, are the larger stream); at 16 heads it is ahead or level up to 1024.
     KERNEL_MAX_ROWS_X_HEADS = 256 * 128
     # Rows x heads up to which the absorption inside the decode launch is level with or ahead of the library GEMM
