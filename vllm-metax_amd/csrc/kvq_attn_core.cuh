@@ -703,19 +703,44 @@ struct DecodeTile {
   // Every wave of the workgroup must call this with the same (t_begin, t_end, nsub): the rendezvous
   // barriers inside are counted in rounds of nsub tiles, the same number for every wave, also for
   // one that owns no tile of the range (its state stays empty: m = -inf).
-  template <bool CAP, bool STREAM = false>
-  __device__ static void run(const AttnIO& io, int seq, int64_t row, int len, int first, int t_begin, int t_end, int hkv,
-                             int lane, uint8_t* lds, State& st, int sub = 0, int nsub = 1) {
-    const LaneOffsets lo = lane_offsets(io.g, lane);
-    const int32_t* bt_row = io.block_table + (int64_t)seq * io.bt_stride;
-    const int rounds = (t_end - t_begin + nsub - 1) / nsub;
-    const int num_barriers = STREAM ? 0 : rounds / kSyncTiles;
-    int barriers = 0;
+  // SPANS (one wave per kv head only: nsub = 1): the run covers several consecutive spans of `sp.per` tiles of the
+  // batch-invariant cutting.  The tile stream -- query registers, block numbers, the tile in flight -- goes on across
+  // a span's edge; there the state is stored as the span's partial state (slot sp.slot) and started afresh, so every
+  // span's state holds exactly what a run over that span alone would have computed, in the same order.  The state of
+  // the run's last span is left to the caller (sp.slot names it on return).
+  struct SpanEdges {
+    float* part_o;
+    float* part_ml;
+    int64_t slot;   // of the span the next tile belongs to
+    int per;        // tiles per span
+    int left;       // tiles of the current span still to come
+  };
+  __device__ static void reset_state(State& st) {
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) st.o[dt] = (floatx4){0.f, 0.f, 0.f, 0.f};
     st.psum = (floatx4){0.f, 0.f, 0.f, 0.f};
     st.m = -INFINITY;
     st.l = 0.f;
+  }
+  template <bool CAP, bool STREAM = false, bool SPANS = false>
+  __device__ static void run(const AttnIO& io, int seq, int64_t row, int len, int first, int t_begin, int t_end, int hkv,
+                             int lane, uint8_t* lds, State& st, int sub = 0, int nsub = 1, SpanEdges* sp = nullptr) {
+    const LaneOffsets lo = lane_offsets(io.g, lane);
+    const int32_t* bt_row = io.block_table + (int64_t)seq * io.bt_stride;
+    const int rounds = (t_end - t_begin + nsub - 1) / nsub;
+    const int num_barriers = STREAM ? 0 : rounds / kSyncTiles;
+    int barriers = 0;
+    reset_state(st);
+    auto span_edge = [&]() __attribute__((always_inline)) {
+      if constexpr (SPANS) {
+        if (--sp->left == 0) {   // uniform over the wave
+          emit_partial(io, sp->part_o, sp->part_ml, sp->slot, hkv, lane, st);
+          reset_state(st);
+          ++sp->slot;
+          sp->left = sp->per;
+        }
+      }
+    };
     int t = t_begin + sub;
     if (t < t_end) {
       Tile a;
@@ -741,6 +766,7 @@ struct DecodeTile {
         nb = fetch_blocks(io, bt_row, len, t + 2 * nsub);
         compute<true, CAP>(io, lo, qb, s_init, len, first, t, lane, lds, st, ali);
         phase_fence();
+        span_edge();
         t += nsub;
         ++r;
         if (!STREAM && (r & (kSyncTiles - 1)) == 0) {
@@ -771,6 +797,7 @@ struct DecodeTile {
         nb = fetch_blocks(io, bt_row, len, t + 2 * nsub);
         compute<false, CAP>(io, lo, qb, s_init, len, first, t, lane, lds, st, ali);
         phase_fence();
+        span_edge();
         t += nsub;
         rendezvous();
       }

@@ -223,6 +223,23 @@ __global__ __launch_bounds__(512) void paged_decode_streamk_kernel(StreamKArgs a
     }
   };
 
+  // (batch-invariant cutting, one wave per kv head) `count` consecutive spans of one sequence as ONE run of tiles: the
+  // stream goes on across the spans' edges, where DecodeTile::run stores and restarts the state, so a span's state
+  // holds the same bits as if it had been computed alone -- without a query reload and a first tile that nothing
+  // prefetched per span.
+  auto process_spans = [&](int cur, int64_t row, int len, int first, int t0, int ntiles, int t_begin, int t_end, int per,
+                           int span) __attribute__((always_inline)) {
+    if (a.k_new != nullptr && t_end == t0 + ntiles) {   // uniform over the workgroup: the run holds the last tile
+      const bool padding = a.new_slots != nullptr && a.new_slots[row] < 0;
+      if (!padding) write_new_token<D>(a, cur, row, len, hkv, lane);
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    }
+    typename DTile::State st;
+    typename DTile::SpanEdges sp{a.part_o, a.part_ml, (int64_t)cur * kFixedSpans + span, per, per};
+    DTile::template run<CAP, STREAM, true>(a.io, cur, row, len, first, t_begin, t_end, hkv, lane, lds[wave], st, 0, 1, &sp);
+    DTile::emit_partial(a.io, a.part_o, a.part_ml, sp.slot, hkv, lane, st);
+  };
+
   if constexpr (fixed) {
     // the spans [lo, hi) of the span line, sequence by sequence
     int64_t at = lo;
@@ -241,6 +258,15 @@ __global__ __launch_bounds__(512) void paged_decode_streamk_kernel(StreamKArgs a
       const int first = window_first(len, a.io.window);
       const int t0 = first / kTile;
       const int t_begin = t0 + span * per;
+      if constexpr (NSUB == 1) {
+        const int64_t rest = hi - at;
+        const int count = rest < spans - span ? (int)rest : spans - span;   // the sequence's spans inside this share
+        if (count > 1) {
+          process_spans(seq, row, len, first, t0, ntiles, t_begin, min(t0 + ntiles, t_begin + count * per), per, span);
+          at += count;
+          continue;
+        }
+      }
       const int t_end = min(t0 + ntiles, t_begin + per);
       process(seq, 0, row, len, first, t0, ntiles, t_begin, t_end, (int64_t)seq * kFixedSpans + span);
       ++at;
